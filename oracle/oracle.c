@@ -1,0 +1,765 @@
+/*
+ * CPU oracle -- TEST INFRASTRUCTURE ONLY (see oracle.h).  Plain C restatement
+ * of the reference interpreter's scalar arithmetic for the quantized-matmul
+ * path.  Citations are file:line under the reference tree.
+ */
+#include "oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ======================================================================== */
+/* integer rounding helpers                                                  */
+/* ======================================================================== */
+
+/* RightShiftRound<T>, lib/Support/MathUtils.cpp:474-514.
+ * Arithmetic shift; the discarded low bits ("mant") are compared with one
+ * half.  Modes outside the listed seven fall through to floor. */
+int64_t orc_right_shift_round(int64_t src, int shift_num, int round_mode) {
+  if (shift_num == 0)
+    return src;
+  if (shift_num > 63)
+    shift_num = 63;
+  if (shift_num < 0)
+    return (int64_t)((uint64_t)src << (-shift_num));
+  int64_t val = src >> shift_num;
+  int64_t res = val;
+  int64_t lo_mask = (int64_t)((1ull << shift_num) - 1);
+  int64_t mant = src & lo_mask;
+  int64_t half = (int64_t)(1ull << (shift_num - 1));
+  switch (round_mode) {
+  case ORC_ROUNDING_HALF_TO_EVEN:
+    if (mant == half)
+      res = val + (val & 1);
+    else if (mant > half)
+      res = val + 1;
+    break;
+  case ORC_ROUNDING_HALF_AWAY_FROM_ZERO:
+    if (src >= 0 && mant >= half)
+      res = val + 1;
+    else if (src < 0 && mant > half)
+      res = val + 1;
+    break;
+  case ORC_ROUNDING_TOWARDS_ZERO:
+    if (src < 0)
+      res = val + (mant != 0);
+    break;
+  case ORC_ROUNDING_DOWN:
+    res = val;
+    break;
+  case ORC_ROUNDING_UP:
+    res = val + (mant != 0);
+    break;
+  case ORC_ROUNDING_HALF_UP:
+    if (mant >= half)
+      res = val + 1;
+    break;
+  case ORC_ROUNDING_HALF_DOWN:
+    if (mant > half)
+      res = val + 1;
+    break;
+  default:
+    break;
+  }
+  return res;
+}
+
+/* MultiplyByQuantizedMultiplier, lib/Support/MathUtils.cpp:523-536.
+ * The optional left shift is done in 32 bits (as the reference's `x << shift`
+ * on an int32_t), the product and the Q31 rounding in 64 bits. */
+int32_t orc_multiply_by_quantized_multiplier(int32_t x, int32_t multiplier,
+                                             int shift, int round_mode) {
+  int64_t value = shift > 0 ? (int32_t)((uint32_t)x << shift) : x;
+  value = orc_right_shift_round(value * (int64_t)multiplier, 31,
+                                ORC_ROUNDING_HALF_UP);
+  if (value > 2147483647ll)
+    value = 2147483647ll;
+  else if (value < -2147483648ll)
+    value = -2147483648ll;
+  if (shift < 0)
+    value = orc_right_shift_round(value, -shift, round_mode);
+  return (int32_t)value;
+}
+
+/* to_int<T>, lib/Support/MathUtils.cpp:179-213 */
+int64_t orc_to_int_f64(double v, int round_mode) {
+  switch (round_mode) {
+  case ORC_ROUNDING_HALF_AWAY_FROM_ZERO:
+    return (int64_t)round(v);
+  case ORC_ROUNDING_UP:
+    return (int64_t)ceil(v);
+  case ORC_ROUNDING_DOWN:
+    return (int64_t)floor(v);
+  case ORC_ROUNDING_HALF_TO_EVEN: {
+    /* the reference narrows to float here (MathUtils.cpp:189-191) */
+    float integer;
+    float abs_v = (float)fabs(v);
+    float fraction = modff(abs_v, &integer);
+    int64_t r = (int64_t)integer;
+    if (fraction > 0.5f)
+      r += 1;
+    else if (fraction == 0.5f && (r & 1))
+      r += 1;
+    return v < 0 ? -r : r;
+  }
+  case ORC_ROUNDING_HALF_UP:
+    return (int64_t)floor(v + 0.5);
+  case ORC_ROUNDING_HALF_DOWN:
+    return (int64_t)ceil(v - 0.5);
+  case ORC_ROUNDING_TOWARDS_ZERO:
+    return (int64_t)v;
+  default:
+    return (int64_t)round(v);
+  }
+}
+
+int64_t orc_to_int_f32(float v, int round_mode) {
+  switch (round_mode) {
+  case ORC_ROUNDING_HALF_AWAY_FROM_ZERO:
+    return (int64_t)roundf(v);
+  case ORC_ROUNDING_UP:
+    return (int64_t)ceilf(v);
+  case ORC_ROUNDING_DOWN:
+    return (int64_t)floorf(v);
+  case ORC_ROUNDING_HALF_UP:
+    /* `v + 0.5` promotes to double in the reference (MathUtils.cpp:203) */
+    return (int64_t)floor((double)v + 0.5);
+  case ORC_ROUNDING_HALF_DOWN:
+    return (int64_t)ceil((double)v - 0.5);
+  case ORC_ROUNDING_TOWARDS_ZERO:
+    return (int64_t)v;
+  default:
+    return orc_to_int_f64((double)v, round_mode);
+  }
+}
+
+/* applyMultiplierAndRShift, lib/Support/MathUtils.cpp:538-562 */
+int64_t orc_apply_multiplier_and_rshift(int64_t v, int64_t multiplier,
+                                        int64_t rshift, int qmode,
+                                        int round_mode, int is_cv18xx) {
+  switch (qmode) {
+  case ORC_RQ_MULTIPLIER_SHIFT:
+    if (is_cv18xx) {
+      /* (float)v * multiplier: the int64 multiplier is converted to float */
+      float f = ((float)v * (float)multiplier) / (float)(1 << rshift);
+      return orc_to_int_f32(f, round_mode);
+    }
+    return orc_right_shift_round(v * multiplier, (int)rshift, round_mode);
+  case ORC_RQ_ONLY_SHIFT:
+    return orc_right_shift_round(v, (int)rshift, round_mode);
+  case ORC_RQ_QDM:
+  case ORC_RQ_TFLITE:
+  case ORC_RQ_TFLITE_LSHIFT:
+    if (is_cv18xx)
+      rshift = -rshift;
+    return orc_multiply_by_quantized_multiplier((int32_t)v, (int32_t)multiplier,
+                                                (int32_t)rshift, round_mode);
+  default:
+    return 0;
+  }
+}
+
+/* saturate<T>(v, IntegerType), lib/Support/MathUtils.cpp:849-872, with the
+ * default rounding ROUNDING_HALF_AWAY_FROM_ZERO of MathUtils.h:305-307 */
+static int64_t clamp_bits(int64_t v, int bits, int is_unsigned) {
+  int64_t max, min;
+  if (is_unsigned) {
+    max = bits >= 63 ? INT64_MAX : (int64_t)((1ull << bits) - 1);
+    min = 0;
+  } else {
+    max = (int64_t)((1ull << (bits - 1)) - 1);
+    min = -max - 1;
+  }
+  return v > max ? max : (v < min ? min : v);
+}
+int64_t orc_saturate_i64(int64_t v, int bits, int is_unsigned) {
+  return clamp_bits(v, bits, is_unsigned);
+}
+int64_t orc_saturate_f32(float v, int bits, int is_unsigned) {
+  return clamp_bits(orc_to_int_f32(v, ORC_ROUNDING_HALF_AWAY_FROM_ZERO), bits,
+                    is_unsigned);
+}
+
+/* ======================================================================== */
+/* f32 <-> bf16 / f16                                                        */
+/* ======================================================================== */
+static inline uint32_t f2u(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return u;
+}
+static inline float u2f(uint32_t u) {
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+/* bm_f32_to_bf16 = fp32_to_bf16_all(src, ROUNDING_HALF_TO_EVEN),
+ * lib/Support/Float16.cpp:603-646,716-720 (normals :606-625 via
+ * RightShiftRound of the whole bit pattern, then fp32_to_bf16 :521-548 of an
+ * already representable value; denormals :550-601). */
+static uint16_t bm_f32_to_bf16(float src) {
+  uint32_t bits = f2u(src);
+  uint32_t exp = (bits >> 23) & 0xff;
+  uint32_t frac = bits & 0x7fffff;
+  uint32_t sign = bits >> 31;
+  if (exp > 0 && exp < 255) {
+    int64_t r = orc_right_shift_round((int64_t)bits, 16,
+                                      ORC_ROUNDING_HALF_TO_EVEN);
+    uint32_t rounded = (uint32_t)((r << 16) & 0xFFFFFFFF);
+    /* fp32_to_bf16 on a value whose low 16 bits are zero */
+    uint32_t rexp = (rounded >> 23) & 0xff;
+    if (rexp == 255) /* rounded up to infinity: keep inf (frac is 0) */
+      return (uint16_t)(rounded >> 16);
+    if (rexp == 0)
+      return (uint16_t)(sign << 15);
+    return (uint16_t)(rounded >> 16);
+  }
+  if (exp == 255)
+    return frac != 0 ? 0x7fff : (uint16_t)(sign ? 0xff80 : 0x7f80);
+  if (frac == 0)
+    return (uint16_t)(sign << 15);
+  /* fp32 denormal, fp32_to_bf16_denorm with HALF_TO_EVEN (:550-601):
+   * only 0x007f8000..0x007fffff rounds up to the smallest bf16 normal */
+  if (((frac >> 16) & 0x7f) == 0x7f && (frac & 0x8000))
+    return (uint16_t)((sign << 15) | 0x80);
+  return (uint16_t)(sign << 15);
+}
+
+/* cvi_f32_to_bf16(src, is_tpu=true), lib/Support/Float16.cpp:725-761 */
+static uint16_t cvi_f32_to_bf16(float src) {
+  uint32_t u = f2u(src);
+  uint32_t lsb = (u >> 16) & 1;
+  u += 0x7fff + lsb;
+  uint16_t h = (uint16_t)(u >> 16);
+  return ((h & 0x7f80) == 0x7f80) ? 0x7f7f : h;
+}
+
+/* f32_to_bf16, lib/Support/Float16.cpp:769-774 */
+uint16_t orc_f32_to_bf16(float src, int is_cv18xx) {
+  return is_cv18xx ? cvi_f32_to_bf16(src) : bm_f32_to_bf16(src);
+}
+/* bf16_to_f32, lib/Support/Float16.cpp:788-792 */
+float orc_bf16_to_f32(uint16_t src) { return u2f((uint32_t)src << 16); }
+/* BF16(float), lib/Support/Float16.cpp:824-827 */
+float orc_BF16(float src, int is_cv18xx) {
+  return orc_bf16_to_f32(orc_f32_to_bf16(src, is_cv18xx));
+}
+
+/* exact f32 -> f16 of a value known to be representable or to overflow
+ * (stands in for fp16_ieee_from_fp32_value, lib/Support/Float16.cpp:256-283,
+ * on inputs whose low 13 mantissa bits are zero) */
+static uint16_t f16_from_rounded(uint32_t bits) {
+  uint32_t sign = (bits >> 16) & 0x8000;
+  int32_t e = (int32_t)((bits >> 23) & 0xff) - 127 + 15;
+  uint32_t m = (bits >> 13) & 0x3ff;
+  if (e >= 31)
+    return (uint16_t)(sign | 0x7c00);
+  return (uint16_t)(sign | ((uint32_t)e << 10) | m);
+}
+
+/* f32_to_f16 = fp32_to_fp16_all(src, ROUNDING_HALF_TO_EVEN),
+ * lib/Support/Float16.cpp:664-714,763-767 */
+uint16_t orc_f32_to_f16(float src) {
+  uint32_t bits = f2u(src);
+  uint32_t exp = (bits >> 23) & 0xff;
+  uint32_t frac = bits & 0x7fffff;
+  uint32_t sign = bits >> 31;
+  if (exp > 112 && exp < 255) {
+    int64_t r = orc_right_shift_round((int64_t)bits, 13,
+                                      ORC_ROUNDING_HALF_TO_EVEN);
+    uint32_t rounded = (uint32_t)((r << 13) & 0xFFFFFFFF);
+    if (((rounded >> 23) & 0xff) == 255)
+      return (uint16_t)((sign << 15) | 0x7c00);
+    return f16_from_rounded(rounded);
+  }
+  if (exp > 0 && exp <= 112) {
+    /* result is an f16 subnormal (or rounds up to the smallest normal) */
+    int32_t mant = (int32_t)(frac + (1u << 23));
+    mant = sign ? -mant : mant;
+    int rshift_num = (113 - (int)exp) + 13;
+    mant = (int32_t)orc_right_shift_round((int64_t)mant, rshift_num,
+                                          ORC_ROUNDING_HALF_TO_EVEN);
+    mant = sign ? -mant : mant;
+    return (uint16_t)(((uint32_t)mant & 0x7fff) | (sign << 15));
+  }
+  if (exp == 255)
+    return frac != 0 ? 0x7fff : (uint16_t)(sign ? 0xfc00 : 0x7c00);
+  /* zero and fp32 denormals: far below the f16 subnormal range */
+  return (uint16_t)(sign << 15);
+}
+
+/* f16_to_f32, lib/Support/Float16.cpp:776-786 (NaN -> 0xFFC00000) */
+float orc_f16_to_f32(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000) << 16;
+  uint32_t e = (h >> 10) & 0x1f;
+  uint32_t m = h & 0x3ff;
+  if (e == 31 && m != 0)
+    return u2f(0xFFC00000u);
+  if (e == 31)
+    return u2f(sign | 0x7f800000u);
+  if (e == 0) {
+    float v = (float)m * 0x1.0p-24f;
+    return sign ? -v : v;
+  }
+  return u2f(sign | ((e + 112) << 23) | (m << 13));
+}
+/* F16(float), lib/Support/Float16.cpp:808-811 */
+float orc_F16(float src) { return orc_f16_to_f32(orc_f32_to_f16(src)); }
+
+static inline float round_out(float v, int out_dtype, int is_cv18xx) {
+  if (out_dtype == ORC_OUT_BF16)
+    return orc_BF16(v, is_cv18xx);
+  if (out_dtype == ORC_OUT_F16)
+    return orc_F16(v);
+  return v;
+}
+
+/* ---- array forms -------------------------------------------------------- */
+void orc_right_shift_round_array(const int64_t *src, const int32_t *shift,
+                                 int round_mode, int64_t *dst, int64_t n) {
+  for (int64_t i = 0; i < n; i++)
+    dst[i] = orc_right_shift_round(src[i], shift[i], round_mode);
+}
+void orc_mbqm_array(const int32_t *x, const int32_t *mult, const int32_t *shift,
+                    int round_mode, int32_t *dst, int64_t n) {
+  for (int64_t i = 0; i < n; i++)
+    dst[i] = orc_multiply_by_quantized_multiplier(x[i], mult[i], shift[i],
+                                                  round_mode);
+}
+void orc_f32_to_bf16_array(const float *src, uint16_t *dst, int64_t n,
+                           int is_cv18xx) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; i++)
+    dst[i] = orc_f32_to_bf16(src[i], is_cv18xx);
+}
+void orc_f32_to_f16_array(const float *src, uint16_t *dst, int64_t n) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; i++)
+    dst[i] = orc_f32_to_f16(src[i]);
+}
+void orc_f16_to_f32_array(const uint16_t *src, float *dst, int64_t n) {
+  for (int64_t i = 0; i < n; i++)
+    dst[i] = orc_f16_to_f32(src[i]);
+}
+void orc_to_int_f32_array(const float *src, int round_mode, int64_t *dst,
+                          int64_t n) {
+  for (int64_t i = 0; i < n; i++)
+    dst[i] = orc_to_int_f32(src[i], round_mode);
+}
+
+/* ======================================================================== */
+/* f32 GEMM                                                                  */
+/* ======================================================================== */
+/* The reference's GEMM is oneDNN's f32 matmul (lib/Support/Dnnl/MatMul.cpp:
+ * 150-164,223-227); its summation order is unspecified.  Three stand-ins: */
+
+void orc_sgemm_f32(const float *A, const float *B, const float *bias, float *Y,
+                   int64_t M, int64_t K, int64_t N) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; m++) {
+    float *y = Y + m * N;
+    for (int64_t n = 0; n < N; n++)
+      y[n] = bias ? bias[n] : 0.0f;
+    for (int64_t k = 0; k < K; k++) {
+      float a = A[m * K + k];
+      const float *b = B + k * N;
+      for (int64_t n = 0; n < N; n++)
+        y[n] += a * b[n];
+    }
+  }
+}
+
+void orc_sgemm_f64acc(const float *A, const float *B, const float *bias,
+                      float *Y, int64_t M, int64_t K, int64_t N) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; m++) {
+    double *acc = (double *)malloc(sizeof(double) * (size_t)N);
+    for (int64_t n = 0; n < N; n++)
+      acc[n] = 0.0;
+    for (int64_t k = 0; k < K; k++) {
+      double a = A[m * K + k];
+      const float *b = B + k * N;
+      for (int64_t n = 0; n < N; n++)
+        acc[n] += a * (double)b[n];
+    }
+    for (int64_t n = 0; n < N; n++)
+      Y[m * N + n] = (float)(acc[n] + (bias ? (double)bias[n] : 0.0));
+    free(acc);
+  }
+}
+
+int orc_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* Blocked, threaded over column panels so that skinny (M<=16) problems still
+ * use every core; the inner loop vectorises along n.  This one function may
+ * contract a*b+c into FMA (it is only ever a timing baseline). */
+__attribute__((optimize("fp-contract=fast"))) void orc_sgemm_fast(const float *A, const float *B, const float *bias,
+                    float *Y, int64_t M, int64_t K, int64_t N) {
+  const int64_t NB = 256, KB = 256, MB = 8;
+  int64_t n_panels = (N + NB - 1) / NB;
+  int64_t m_panels = (M + MB - 1) / MB;
+#pragma omp parallel for collapse(2) schedule(dynamic)
+  for (int64_t mp = 0; mp < m_panels; mp++) {
+    for (int64_t np = 0; np < n_panels; np++) {
+      int64_t m0 = mp * MB, m1 = m0 + MB > M ? M : m0 + MB;
+      int64_t n0 = np * NB, n1 = n0 + NB > N ? N : n0 + NB;
+      float acc[8][256];
+      for (int64_t m = m0; m < m1; m++)
+        for (int64_t n = n0; n < n1; n++)
+          acc[m - m0][n - n0] = bias ? bias[n] : 0.0f;
+      for (int64_t k0 = 0; k0 < K; k0 += KB) {
+        int64_t k1 = k0 + KB > K ? K : k0 + KB;
+        for (int64_t k = k0; k < k1; k++) {
+          const float *b = B + k * N + n0;
+          for (int64_t m = m0; m < m1; m++) {
+            float a = A[m * K + k];
+            float *c = acc[m - m0];
+            for (int64_t n = 0; n < n1 - n0; n++)
+              c[n] += a * b[n];
+          }
+        }
+      }
+      for (int64_t m = m0; m < m1; m++)
+        for (int64_t n = n0; n < n1; n++)
+          Y[m * N + n] = acc[m - m0][n - n0];
+    }
+  }
+}
+
+static void run_gemm(int kind, const float *A, const float *B,
+                     const float *bias, float *Y, int64_t M, int64_t K,
+                     int64_t N) {
+  if (kind == 1)
+    orc_sgemm_f64acc(A, B, bias, Y, M, K, N);
+  else if (kind == 2)
+    orc_sgemm_fast(A, B, bias, Y, M, K, N);
+  else
+    orc_sgemm_f32(A, B, bias, Y, M, K, N);
+}
+
+/* tensor_hw_transpose, include/tpu_mlir/Support/MathUtils.h:198-212 with
+ * N*C == 1: dst[w*H + h] = src[h*W + w] */
+void orc_hw_transpose(float *dst, const float *src, int64_t H, int64_t W) {
+  for (int64_t w = 0; w < W; w++)
+    for (int64_t h = 0; h < H; h++)
+      dst[w * H + h] = src[h * W + w];
+}
+
+/* ======================================================================== */
+/* tpu.A16MatMul                                                             */
+/* ======================================================================== */
+
+/* lib/Dialect/Tpu/Interfaces/Common/A16MatMul.cpp:172-198 (4-bit) and
+ * :209-231 (8-bit).  Element i of the row-major stored matrix takes nibble
+ * (i & 1) of byte i/2: low nibble first.  Group index is i / q_group_size
+ * over the flat index; per-row parameters when q_group_size == 0. */
+void orc_a16_dequant(const float *weight, const float *scale, const float *zp,
+                     float *new_weight, int64_t rows, int64_t cols,
+                     int weight_bits, int q_group_size, int out_dtype,
+                     int is_cv18xx) {
+  int64_t total = rows * cols;
+  if (weight_bits == 4) {
+    for (int64_t i = 0; i < total; i += 2) {
+      int64_t qi = q_group_size ? i / q_group_size : i / cols;
+      float zp_i = zp[qi], scale_i = scale[qi];
+      int byte = (int)weight[i / 2];
+      new_weight[i] = ((float)(byte & 0x0F) - zp_i) * scale_i;
+      /* the odd element reuses the even element's group, as the reference's
+       * loop increments i without recomputing quant_idx (:190-197) */
+      new_weight[i + 1] = ((float)(byte >> 4) - zp_i) * scale_i;
+    }
+  } else {
+    for (int64_t i = 0; i < total; i++) {
+      int64_t qi = q_group_size ? i / q_group_size : i / cols;
+      float w = (weight[i] - zp[qi]) * scale[qi];
+      new_weight[i] = round_out(w, out_dtype, is_cv18xx); /* :227-231 */
+    }
+  }
+}
+
+int orc_a16matmul(const orc_a16mm_attr *a, const float *const *inputs,
+                  float *output, float *y_preround) {
+  if (!a || !inputs || !inputs[0] || !inputs[1] || !inputs[2] || !inputs[3])
+    return 1;
+  if (a->weight_bits != 4 && a->weight_bits != 8)
+    return 1;
+  int64_t M = a->M, K = a->K, N = a->N;
+  /* stored matrix: [N,K] when w_transpose, else [K,N] */
+  int64_t rows = a->w_transpose ? N : K, cols = a->w_transpose ? K : N;
+  float *w = (float *)malloc(sizeof(float) * (size_t)(rows * cols));
+  float *wt = NULL;
+  if (!w)
+    return 1;
+  orc_a16_dequant(inputs[1], inputs[2], inputs[3], w, rows, cols,
+                  a->weight_bits, a->q_group_size, a->out_dtype, a->is_cv18xx);
+  const float *B = w;
+  if (a->w_transpose) {
+    /* MatMul::run, lib/Support/Dnnl/MatMul.cpp:170-179: [N,K] -> [K,N] */
+    wt = (float *)malloc(sizeof(float) * (size_t)(rows * cols));
+    if (!wt) {
+      free(w);
+      return 1;
+    }
+    orc_hw_transpose(wt, w, N, K);
+    B = wt;
+  }
+  run_gemm(a->gemm_kind, inputs[0], B, inputs[4], output, M, K, N);
+  if (y_preround)
+    memcpy(y_preround, output, sizeof(float) * (size_t)(M * N));
+  /* output rounding, A16MatMul.cpp:240-245 */
+  for (int64_t i = 0; i < M * N; i++)
+    output[i] = round_out(output[i], a->out_dtype, a->is_cv18xx);
+  free(w);
+  free(wt);
+  return 0;
+}
+
+/* ======================================================================== */
+/* tpu.MatMul (quantised)                                                    */
+/* ======================================================================== */
+
+void orc_igemm_i64(const int8_t *A, const int8_t *B, const int32_t *bias,
+                   int64_t *Y, int64_t M, int64_t K, int64_t N,
+                   int right_transpose, int64_t input_zp, int64_t right_zp) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; m++)
+    for (int64_t n = 0; n < N; n++) {
+      int64_t s = bias ? bias[n] : 0;
+      for (int64_t k = 0; k < K; k++) {
+        int64_t b = right_transpose ? B[n * K + k] : B[k * N + n];
+        s += ((int64_t)A[m * K + k] - input_zp) * (b - right_zp);
+      }
+      Y[m * N + n] = s;
+    }
+}
+
+static int64_t arr_at(const int64_t *v, int n, int64_t i, int64_t dflt) {
+  /* module::getI64Array(attr, num, default): a one-element attribute is
+   * broadcast (lib/Support/Module.cpp:570-578) */
+  if (!v || n <= 0)
+    return dflt;
+  return n == 1 ? v[0] : v[i < n ? i : n - 1];
+}
+
+int orc_matmul_int8(const orc_i8mm_attr *a, const float *const *inputs,
+                    float *output, float *acc_out) {
+  if (!a || !inputs || !inputs[0] || !inputs[1])
+    return 1;
+  int64_t M = a->M, K = a->K, N = a->N;
+  /* MatMul::run, lib/Support/Dnnl/MatMul.cpp:167-201 */
+  float *right = (float *)malloc(sizeof(float) * (size_t)(K * N));
+  float *left = NULL;
+  if (!right)
+    return 1;
+  if (a->right_transpose)
+    orc_hw_transpose(right, inputs[1], N, K);
+  else
+    memcpy(right, inputs[1], sizeof(float) * (size_t)(K * N));
+  if (a->right_zp != 0) /* tensor_sub_zp, MathUtils.cpp:744-750 */
+    for (int64_t i = 0; i < K * N; i++)
+      right[i] = right[i] - (float)a->right_zp;
+  const float *A = inputs[0];
+  if (a->input_zp != 0) {
+    left = (float *)malloc(sizeof(float) * (size_t)(M * K));
+    for (int64_t i = 0; i < M * K; i++)
+      left[i] = inputs[0][i] - (float)a->input_zp;
+    A = left;
+  }
+  run_gemm(a->gemm_kind, A, right, inputs[2], output, M, K, N);
+  free(right);
+  free(left);
+  /* post_relu, lib/Support/Dnnl/DnnlUtils.cpp:15-25 */
+  if (a->do_relu)
+    for (int64_t i = 0; i < M * N; i++) {
+      float v = output[i] > 0.0f ? output[i] : 0.0f;
+      if (a->relu_limit > 0.0 && v > (float)a->relu_limit)
+        v = (float)a->relu_limit;
+      output[i] = v;
+    }
+  if (acc_out)
+    memcpy(acc_out, output, sizeof(float) * (size_t)(M * N));
+  if (a->out_kind == 1)
+    return 0; /* int32 storage: no epilogue (MatMul.cpp:605-607,636) */
+
+  int64_t num = M * N;
+  if (a->is_cv18xx) {
+    /* MatMul.cpp:638-664, batch == 1 */
+    int64_t mult = arr_at(a->multipliers, a->n_multipliers, 0, 1);
+    int64_t rs = arr_at(a->rshifts, a->n_rshifts, 0, 0);
+    for (int64_t j = 0; j < num; j++) {
+      int64_t v = orc_apply_multiplier_and_rshift(
+          (int64_t)output[j], mult, rs, a->quant_mode,
+          ORC_ROUNDING_HALF_AWAY_FROM_ZERO, 1);
+      output[j] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+    }
+    return 0;
+  }
+  /* MatMul.cpp:665-727 */
+  int64_t rshift0 = arr_at(a->rshifts, a->n_rshifts, 0, 0);
+  int64_t mult0 = arr_at(a->multipliers, a->n_multipliers, 0, 1);
+  if (a->quant_mode == ORC_RQ_TFLITE_LSHIFT || a->quant_mode == ORC_RQ_TFLITE) {
+    for (int64_t i = 0; i < num; i++) {
+      int64_t v = (int64_t)orc_multiply_by_quantized_multiplier(
+                      (int32_t)output[i], (int32_t)mult0, -(int32_t)rshift0,
+                      ORC_ROUNDING_HALF_AWAY_FROM_ZERO) +
+                  a->out_zp;
+      output[i] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+    }
+  } else if (a->quant_mode == ORC_RQ_MULTIPLIER_SHIFT) {
+    if (a->fuse_rq) {
+      if (!inputs[3])
+        return 1;
+      for (int64_t i = 0; i < num; i++) {
+        int64_t v = orc_apply_multiplier_and_rshift(
+                        (int64_t)output[i], (int64_t)inputs[3][i % N], rshift0,
+                        ORC_RQ_MULTIPLIER_SHIFT, ORC_ROUNDING_HALF_UP, 0) +
+                    a->out_zp;
+        output[i] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+      }
+    } else {
+      for (int64_t i = 0; i < num; i++) {
+        int64_t v = orc_apply_multiplier_and_rshift(
+                        (int64_t)output[i], mult0, rshift0,
+                        ORC_RQ_MULTIPLIER_SHIFT, ORC_ROUNDING_HALF_UP, 0) +
+                    a->out_zp;
+        output[i] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+      }
+    }
+  } else {
+    return 1;
+  }
+  return 0;
+}
+
+/* ======================================================================== */
+/* tpu.RequantIntAxis / tpu.RequantInt                                       */
+/* ======================================================================== */
+
+static void rq_triple(const orc_rq_axis_attr *a, const float *quant, int64_t c,
+                      int64_t *multi, int64_t *shift, int64_t *zp) {
+  if (a->is_bm1684x) {
+    /* RequantIntAxis.cpp:47-49 */
+    *multi = (int64_t)quant[c * 3];
+    *shift = (int64_t)quant[c * 3 + 1];
+    *zp = (int64_t)quant[c * 3 + 2];
+  } else {
+    /* RequantIntAxis.cpp:50-55: shift in the low byte, zp in the high half */
+    *multi = (int64_t)quant[c * 2];
+    uint32_t tmp = (uint32_t)quant[c * 2 + 1];
+    *shift = (int64_t)((signed char)(tmp & 0xff));
+    *zp = (int64_t)(short)((tmp & 0xffff0000u) >> 16);
+  }
+}
+
+/* lib/Dialect/Tpu/Interfaces/Common/RequantIntAxis.cpp:17-121 */
+int orc_requant_int_axis(const orc_rq_axis_attr *a, const float *input,
+                         const float *quant, float *output) {
+  if (!a || !input || !quant || !output || a->rank < 2)
+    return 1;
+  const int64_t *shape = a->shape;
+  int rank = a->rank;
+  int64_t inner = 1, outer = 1;
+  for (int i = 2; i < rank; i++)
+    inner *= shape[i];
+  for (int i = 0; i < rank - 1; i++)
+    outer *= shape[i];
+  int64_t zp_x = a->input_zp;
+  int mode = a->quant_mode;
+  if (mode == ORC_RQ_TFLITE_LSHIFT || mode == ORC_RQ_TFLITE) {
+    for (int64_t c = 0; c < shape[1]; c++) {
+      int64_t multi, shift_val, zero_point;
+      rq_triple(a, quant, c, &multi, &shift_val, &zero_point);
+      for (int64_t n = 0; n < shape[0]; n++)
+        for (int64_t i = 0; i < inner; i++) {
+          int64_t off = (n * shape[1] + c) * inner + i;
+          int v = (int)(zero_point + orc_multiply_by_quantized_multiplier(
+                                         (int32_t)input[off], (int32_t)multi,
+                                         (int32_t)shift_val, a->round_mode));
+          output[off] =
+              (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+        }
+    }
+  } else if (mode == ORC_RQ_MULTIPLIER_SHIFT) {
+    if (a->fuse_rq_axis) {
+      int64_t W = shape[rank - 1];
+      for (int64_t w = 0; w < W; w++) {
+        int64_t multi, shift_val, zero_point;
+        rq_triple(a, quant, w, &multi, &shift_val, &zero_point);
+        for (int64_t i = 0; i < outer; i++) {
+          int64_t off = i * W + w;
+          /* (float - int64) is evaluated in float, then converted */
+          int64_t x = (int64_t)(input[off] - (float)zp_x);
+          int v = (int)(zero_point +
+                        orc_apply_multiplier_and_rshift(
+                            x, multi, shift_val, ORC_RQ_MULTIPLIER_SHIFT,
+                            a->round_mode, a->is_cv18xx));
+          output[off] =
+              (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+        }
+      }
+    } else {
+      for (int64_t c = 0; c < shape[1]; c++) {
+        int64_t multi, shift_val, zero_point;
+        rq_triple(a, quant, c, &multi, &shift_val, &zero_point);
+        int64_t rshift_val = -shift_val; /* :97,102 */
+        for (int64_t n = 0; n < shape[0]; n++)
+          for (int64_t i = 0; i < inner; i++) {
+            int64_t off = (n * shape[1] + c) * inner + i;
+            int64_t x = (int64_t)(input[off] - (float)zp_x);
+            int v = (int)(zero_point +
+                          orc_apply_multiplier_and_rshift(
+                              x, multi, rshift_val, ORC_RQ_MULTIPLIER_SHIFT,
+                              a->round_mode, a->is_cv18xx));
+            output[off] =
+                (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+          }
+      }
+    }
+  } else {
+    return 1;
+  }
+  return 0;
+}
+
+/* lib/Dialect/Tpu/Interfaces/Common/RequantInt.cpp:17-72 */
+int orc_requant_int(const orc_rq_attr *a, const float *input, float *output) {
+  if (!a || !input || !output)
+    return 1;
+  if (a->rank == 1)
+    return 0; /* :36-38: rank-1 tensors are left untouched */
+  int64_t num = 1;
+  for (int i = 0; i < a->rank; i++)
+    num *= a->shape[i];
+  int64_t shift_val = -a->rshift;
+  if (a->quant_mode == ORC_RQ_TFLITE_LSHIFT || a->quant_mode == ORC_RQ_TFLITE) {
+    for (int64_t i = 0; i < num; i++) {
+      int64_t v = a->out_zp + orc_multiply_by_quantized_multiplier(
+                                  (int32_t)input[i], (int32_t)a->multiplier,
+                                  (int32_t)shift_val, a->round_mode);
+      output[i] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+    }
+  } else if (a->quant_mode == ORC_RQ_MULTIPLIER_SHIFT) {
+    for (int64_t i = 0; i < num; i++) {
+      int64_t x = (int64_t)(input[i] - (float)a->input_zp);
+      int64_t v = a->out_zp + orc_apply_multiplier_and_rshift(
+                                  x, a->multiplier, -shift_val,
+                                  ORC_RQ_MULTIPLIER_SHIFT, a->round_mode,
+                                  a->is_cv18xx);
+      output[i] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+    }
+  } else {
+    return 1;
+  }
+  return 0;
+}

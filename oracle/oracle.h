@@ -1,0 +1,199 @@
+/*
+ * CPU oracle for the quantized-matmul inference path of sophgo/tpu-mlir's
+ * reference interpreter (tpu.A16MatMul, INT8 tpu.MatMul + requant,
+ * tpu.RequantIntAxis, tpu.RequantInt).
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  It exists to check the HIP
+ * path and to be timed as the CPU baseline.  Only tests/, the smoke check and
+ * the benchmark's cpu_baseline leg may load it; nothing in the product library
+ * links, includes or calls it.
+ *
+ * Every function is a plain-C restatement of scalar reference code and cites
+ * the file:line (under the reference tree) that it follows.  The reference's
+ * own build (MLIR/LLVM + oneDNN + TableGen) is not available, so there is no
+ * compiled reference to compare against; instead each function is pinned by
+ * closed forms, brute force and library routines in tests/test_oracle_*.py.
+ *
+ * Pin status (what fixes each function independently of this file's text):
+ *   orc_right_shift_round        exact rational closed forms, brute force
+ *   orc_multiply_by_quantized_multiplier   Python big-int restatement of the
+ *                                published TFLite single-rounding form
+ *   orc_apply_multiplier_and_rshift, orc_to_int, orc_saturate   closed forms
+ *   orc_f32_to_bf16 (bm)         torch RNE float32->bfloat16 on all normals,
+ *                                special-case table for nan/inf/denormals
+ *   orc_f32_to_bf16 (cvi)        add-0x7fff+lsb closed form, inf->0x7f7f
+ *   orc_f32_to_f16               numpy float16 RNE incl. subnormals
+ *   orc_a16_dequant              one-hot activations recover nibble order,
+ *                                group indexing and scale layout
+ *   orc_sgemm_*                  float64 reference with the standard bound
+ *   f32 summation ORDER of the reference's oneDNN sgemm: parity unpinned
+ *                                (third-party, unspecified; affects last-ulp
+ *                                bf16 rounding only)
+ */
+#ifndef TPU_MLIR_AMD_ORACLE_H
+#define TPU_MLIR_AMD_ORACLE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* RoundingMode, include/tpu_mlir/Support/MathUtils.h:29-41 */
+enum {
+  ORC_ROUNDING_HALF_AWAY_FROM_ZERO = 0,
+  ORC_ROUNDING_HALF_UP = 1,
+  ORC_ROUNDING_HALF_DOWN = 2,
+  ORC_ROUNDING_HALF_TO_EVEN = 3,
+  ORC_ROUNDING_HALF_TO_ODD = 4,
+  ORC_ROUNDING_HALF_TOWARDS_ZERO = 5,
+  ORC_ROUNDING_TOWARDS_ZERO = 6,
+  ORC_ROUNDING_AWAY_FROM_ZERO = 7,
+  ORC_ROUNDING_UP = 8,
+  ORC_ROUNDING_DOWN = 9
+};
+
+/* tpu::RequantMode, include/tpu_mlir/Dialect/Tpu/IR/TpuOps.td:160-172 */
+enum {
+  ORC_RQ_TFLITE_LSHIFT = 0,
+  ORC_RQ_TFLITE = 1,
+  ORC_RQ_MULTIPLIER_SHIFT = 2,
+  ORC_RQ_ONLY_SHIFT = 3,
+  ORC_RQ_QDM = 4,
+  ORC_RQ_ONLY_SCALE = 5
+};
+
+/* output storage types the path rounds to */
+enum { ORC_OUT_BF16 = 0, ORC_OUT_F16 = 1, ORC_OUT_F32 = 2 };
+
+/* ---- scalar helpers ---------------------------------------------------- */
+int64_t orc_right_shift_round(int64_t src, int shift_num, int round_mode);
+int32_t orc_multiply_by_quantized_multiplier(int32_t x, int32_t multiplier,
+                                             int shift, int round_mode);
+int64_t orc_apply_multiplier_and_rshift(int64_t v, int64_t multiplier,
+                                        int64_t rshift, int qmode,
+                                        int round_mode, int is_cv18xx);
+int64_t orc_to_int_f32(float v, int round_mode);
+int64_t orc_to_int_f64(double v, int round_mode);
+/* saturate<T>(v, IntegerType{bits, unsigned}) with the default rounding */
+int64_t orc_saturate_i64(int64_t v, int bits, int is_unsigned);
+int64_t orc_saturate_f32(float v, int bits, int is_unsigned);
+
+uint16_t orc_f32_to_bf16(float src, int is_cv18xx);
+float orc_bf16_to_f32(uint16_t src);
+float orc_BF16(float src, int is_cv18xx);
+uint16_t orc_f32_to_f16(float src);
+float orc_f16_to_f32(uint16_t src);
+float orc_F16(float src);
+
+/* array forms used by the Python tests (one call per array, not per element) */
+void orc_right_shift_round_array(const int64_t *src, const int32_t *shift,
+                                 int round_mode, int64_t *dst, int64_t n);
+void orc_mbqm_array(const int32_t *x, const int32_t *mult, const int32_t *shift,
+                    int round_mode, int32_t *dst, int64_t n);
+void orc_f32_to_bf16_array(const float *src, uint16_t *dst, int64_t n,
+                           int is_cv18xx);
+void orc_f32_to_f16_array(const float *src, uint16_t *dst, int64_t n);
+void orc_f16_to_f32_array(const uint16_t *src, float *dst, int64_t n);
+void orc_to_int_f32_array(const float *src, int round_mode, int64_t *dst,
+                          int64_t n);
+
+/* ---- f32 GEMM  Y[M,N] = A[M,K] * B[K,N] (+ bias[N]) -------------------- */
+/* sequential-k float accumulation (one defined order) */
+void orc_sgemm_f32(const float *A, const float *B, const float *bias, float *Y,
+                   int64_t M, int64_t K, int64_t N);
+/* double accumulation of the exact f32 products, rounded once to f32 */
+void orc_sgemm_f64acc(const float *A, const float *B, const float *bias,
+                      float *Y, int64_t M, int64_t K, int64_t N);
+/* blocked OpenMP sgemm used only when timing the CPU baseline */
+void orc_sgemm_fast(const float *A, const float *B, const float *bias,
+                    float *Y, int64_t M, int64_t K, int64_t N);
+int orc_num_threads(void);
+
+/* [H,W] -> [W,H], include/tpu_mlir/Support/MathUtils.h:198-212 */
+void orc_hw_transpose(float *dst, const float *src, int64_t H, int64_t W);
+
+/* ---- tpu.A16MatMul ------------------------------------------------------ */
+/* Weight dequantisation of the static path,
+ * lib/Dialect/Tpu/Interfaces/Common/A16MatMul.cpp:172-231.
+ * rows x cols is the stored logical matrix ([N,K] when w_transpose).
+ * weight is f32-valued: packed bytes 0..255 (4-bit, rows*cols/2 entries) or
+ * one value per element (8-bit).  The 8-bit branch rounds the dequantised
+ * weight to the output dtype, the 4-bit branch does not. */
+void orc_a16_dequant(const float *weight, const float *scale, const float *zp,
+                     float *new_weight, int64_t rows, int64_t cols,
+                     int weight_bits, int q_group_size, int out_dtype,
+                     int is_cv18xx);
+
+/* gemm_kind: 0 = orc_sgemm_f32, 1 = orc_sgemm_f64acc, 2 = orc_sgemm_fast */
+typedef struct {
+  int64_t M, K, N;
+  int weight_bits;   /* 4 or 8 */
+  int w_transpose;   /* 1: weight stored [N, K(/2)] */
+  int q_group_size;  /* 0: per stored row */
+  int out_dtype;     /* ORC_OUT_BF16 / ORC_OUT_F16 */
+  int is_cv18xx;
+  int gemm_kind;
+} orc_a16mm_attr;
+
+/* inputs[0..4] = input, weight, scale, zp, bias(NULL ok); all f32-valued.
+ * y_preround (may be NULL) receives the f32 result before output rounding.
+ * Returns 0 on success. */
+int orc_a16matmul(const orc_a16mm_attr *attr, const float *const *inputs,
+                  float *output, float *y_preround);
+
+/* ---- tpu.MatMul, quantised (case [M,K]x[K,N] or [M,K]x[N,K]^T) ---------- */
+typedef struct {
+  int64_t M, K, N;
+  int right_transpose;
+  int64_t input_zp, right_zp;
+  int do_relu;
+  double relu_limit;
+  int is_cv18xx;
+  int quant_mode;          /* ORC_RQ_* */
+  int fuse_rq;             /* BM168x: per-channel multiplier from inputs[3] */
+  const int64_t *multipliers; int n_multipliers;
+  const int64_t *rshifts;     int n_rshifts;
+  int64_t out_zp;
+  int out_kind;            /* 0: uniform-quantised integer, 1: raw int32 */
+  int out_bits, out_unsigned;
+  int gemm_kind;
+} orc_i8mm_attr;
+
+/* inputs[0..3] = input, right, bias(NULL ok), multi(NULL ok); f32-valued.
+ * acc (may be NULL) receives the f32 accumulators before requantisation. */
+int orc_matmul_int8(const orc_i8mm_attr *attr, const float *const *inputs,
+                    float *output, float *acc);
+
+/* exact-integer GEMM used to cross-check the f32 accumulation domain */
+void orc_igemm_i64(const int8_t *A, const int8_t *B, const int32_t *bias,
+                   int64_t *Y, int64_t M, int64_t K, int64_t N,
+                   int right_transpose, int64_t input_zp, int64_t right_zp);
+
+/* ---- tpu.RequantIntAxis / tpu.RequantInt -------------------------------- */
+typedef struct {
+  int64_t shape[8]; int rank;
+  int quant_mode, round_mode;
+  int fuse_rq_axis;
+  int is_bm1684x;          /* quant tensor [..,3] vs packed [..,2] */
+  int is_cv18xx;
+  int64_t input_zp;        /* zero point of a uniform-quantised input */
+  int out_bits, out_unsigned;
+} orc_rq_axis_attr;
+int orc_requant_int_axis(const orc_rq_axis_attr *attr, const float *input,
+                         const float *quant, float *output);
+
+typedef struct {
+  int64_t shape[8]; int rank;
+  int quant_mode, round_mode;
+  int64_t multiplier, rshift;
+  int is_cv18xx;
+  int64_t input_zp, out_zp;
+  int out_bits, out_unsigned;
+} orc_rq_attr;
+int orc_requant_int(const orc_rq_attr *attr, const float *input, float *output);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

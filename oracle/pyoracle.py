@@ -1,0 +1,266 @@
+"""ctypes binding of the CPU oracle (oracle/liboracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke check and by the
+benchmark's cpu_baseline leg.  The product package never imports this module.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+# RoundingMode / RequantMode values (oracle.h)
+HALF_AWAY_FROM_ZERO, HALF_UP, HALF_DOWN, HALF_TO_EVEN = 0, 1, 2, 3
+HALF_TO_ODD, HALF_TOWARDS_ZERO, TOWARDS_ZERO, AWAY_FROM_ZERO, UP, DOWN = 4, 5, 6, 7, 8, 9
+RQ_TFLITE_LSHIFT, RQ_TFLITE, RQ_MULTIPLIER_SHIFT, RQ_ONLY_SHIFT, RQ_QDM, RQ_ONLY_SCALE = range(6)
+OUT_BF16, OUT_F16, OUT_F32 = 0, 1, 2
+GEMM_F32, GEMM_F64ACC, GEMM_FAST = 0, 1, 2
+
+
+def build(force=False):
+    """Compile liboracle.so with the Makefile beside this file."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(["make", "-C", _HERE, "liboracle.so"], check=True,
+                   stdout=subprocess.DEVNULL)
+
+
+class A16Attr(C.Structure):
+    _fields_ = [("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64),
+                ("weight_bits", C.c_int), ("w_transpose", C.c_int),
+                ("q_group_size", C.c_int), ("out_dtype", C.c_int),
+                ("is_cv18xx", C.c_int), ("gemm_kind", C.c_int)]
+
+
+class I8Attr(C.Structure):
+    _fields_ = [("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64),
+                ("right_transpose", C.c_int),
+                ("input_zp", C.c_int64), ("right_zp", C.c_int64),
+                ("do_relu", C.c_int), ("relu_limit", C.c_double),
+                ("is_cv18xx", C.c_int), ("quant_mode", C.c_int),
+                ("fuse_rq", C.c_int),
+                ("multipliers", C.POINTER(C.c_int64)), ("n_multipliers", C.c_int),
+                ("rshifts", C.POINTER(C.c_int64)), ("n_rshifts", C.c_int),
+                ("out_zp", C.c_int64), ("out_kind", C.c_int),
+                ("out_bits", C.c_int), ("out_unsigned", C.c_int),
+                ("gemm_kind", C.c_int)]
+
+
+class RqAxisAttr(C.Structure):
+    _fields_ = [("shape", C.c_int64 * 8), ("rank", C.c_int),
+                ("quant_mode", C.c_int), ("round_mode", C.c_int),
+                ("fuse_rq_axis", C.c_int), ("is_bm1684x", C.c_int),
+                ("is_cv18xx", C.c_int), ("input_zp", C.c_int64),
+                ("out_bits", C.c_int), ("out_unsigned", C.c_int)]
+
+
+class RqAttr(C.Structure):
+    _fields_ = [("shape", C.c_int64 * 8), ("rank", C.c_int),
+                ("quant_mode", C.c_int), ("round_mode", C.c_int),
+                ("multiplier", C.c_int64), ("rshift", C.c_int64),
+                ("is_cv18xx", C.c_int),
+                ("input_zp", C.c_int64), ("out_zp", C.c_int64),
+                ("out_bits", C.c_int), ("out_unsigned", C.c_int)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = C.CDLL(_LIB_PATH)
+        L.orc_right_shift_round.restype = C.c_int64
+        L.orc_right_shift_round.argtypes = [C.c_int64, C.c_int, C.c_int]
+        L.orc_multiply_by_quantized_multiplier.restype = C.c_int32
+        L.orc_multiply_by_quantized_multiplier.argtypes = [C.c_int32, C.c_int32, C.c_int, C.c_int]
+        L.orc_apply_multiplier_and_rshift.restype = C.c_int64
+        L.orc_apply_multiplier_and_rshift.argtypes = [C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int]
+        L.orc_to_int_f32.restype = C.c_int64
+        L.orc_to_int_f32.argtypes = [C.c_float, C.c_int]
+        L.orc_to_int_f64.restype = C.c_int64
+        L.orc_to_int_f64.argtypes = [C.c_double, C.c_int]
+        L.orc_saturate_i64.restype = C.c_int64
+        L.orc_saturate_i64.argtypes = [C.c_int64, C.c_int, C.c_int]
+        L.orc_saturate_f32.restype = C.c_int64
+        L.orc_saturate_f32.argtypes = [C.c_float, C.c_int, C.c_int]
+        L.orc_f32_to_bf16.restype = C.c_uint16
+        L.orc_f32_to_bf16.argtypes = [C.c_float, C.c_int]
+        L.orc_f32_to_f16.restype = C.c_uint16
+        L.orc_f32_to_f16.argtypes = [C.c_float]
+        L.orc_num_threads.restype = C.c_int
+        for name in ("orc_a16matmul", "orc_matmul_int8", "orc_requant_int_axis", "orc_requant_int"):
+            getattr(L, name).restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def _p(a, ty):
+    return a.ctypes.data_as(C.POINTER(ty))
+
+
+def _f32(a):
+    return None if a is None else np.ascontiguousarray(a, dtype=np.float32)
+
+
+def right_shift_round(src, shift, mode):
+    src = np.ascontiguousarray(src, dtype=np.int64)
+    shift = np.ascontiguousarray(np.broadcast_to(np.asarray(shift, dtype=np.int32), src.shape))
+    dst = np.empty_like(src)
+    lib().orc_right_shift_round_array(_p(src, C.c_int64), _p(shift, C.c_int32), C.c_int(mode),
+                                      _p(dst, C.c_int64), C.c_int64(src.size))
+    return dst
+
+
+def mbqm(x, mult, shift, mode):
+    x = np.ascontiguousarray(x, dtype=np.int32)
+    mult = np.ascontiguousarray(np.broadcast_to(np.asarray(mult, dtype=np.int32), x.shape))
+    shift = np.ascontiguousarray(np.broadcast_to(np.asarray(shift, dtype=np.int32), x.shape))
+    dst = np.empty_like(x)
+    lib().orc_mbqm_array(_p(x, C.c_int32), _p(mult, C.c_int32), _p(shift, C.c_int32), C.c_int(mode),
+                         _p(dst, C.c_int32), C.c_int64(x.size))
+    return dst
+
+
+def f32_to_bf16(x, cv18xx=False):
+    x = _f32(x)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().orc_f32_to_bf16_array(_p(x, C.c_float), _p(out, C.c_uint16), C.c_int64(x.size), C.c_int(int(cv18xx)))
+    return out
+
+
+def bf16_to_f32(h):
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    return (h.astype(np.uint32) << 16).view(np.float32)
+
+
+def BF16(x, cv18xx=False):
+    return bf16_to_f32(f32_to_bf16(x, cv18xx))
+
+
+def f32_to_f16(x):
+    x = _f32(x)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().orc_f32_to_f16_array(_p(x, C.c_float), _p(out, C.c_uint16), C.c_int64(x.size))
+    return out
+
+
+def f16_to_f32(h):
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    out = np.empty(h.shape, dtype=np.float32)
+    lib().orc_f16_to_f32_array(_p(h, C.c_uint16), _p(out, C.c_float), C.c_int64(h.size))
+    return out
+
+
+def F16(x):
+    return f16_to_f32(f32_to_f16(x))
+
+
+def to_int_f32(x, mode):
+    x = _f32(x)
+    out = np.empty(x.shape, dtype=np.int64)
+    lib().orc_to_int_f32_array(_p(x, C.c_float), C.c_int(mode), _p(out, C.c_int64), C.c_int64(x.size))
+    return out
+
+
+def sgemm(A, B, bias=None, kind=GEMM_F32):
+    A, B, bias = _f32(A), _f32(B), _f32(bias)
+    M, K = A.shape
+    N = B.shape[1]
+    Y = np.empty((M, N), dtype=np.float32)
+    fn = {GEMM_F32: lib().orc_sgemm_f32, GEMM_F64ACC: lib().orc_sgemm_f64acc,
+          GEMM_FAST: lib().orc_sgemm_fast}[kind]
+    fn(_p(A, C.c_float), _p(B, C.c_float), None if bias is None else _p(bias, C.c_float),
+       _p(Y, C.c_float), C.c_int64(M), C.c_int64(K), C.c_int64(N))
+    return Y
+
+
+def a16_dequant(weight, scale, zp, rows, cols, weight_bits, q_group_size, out_dtype=OUT_BF16, cv18xx=False):
+    weight, scale, zp = _f32(weight), _f32(scale), _f32(zp)
+    out = np.empty((rows, cols), dtype=np.float32)
+    lib().orc_a16_dequant(_p(weight, C.c_float), _p(scale, C.c_float), _p(zp, C.c_float), _p(out, C.c_float),
+                          C.c_int64(rows), C.c_int64(cols), C.c_int(weight_bits), C.c_int(q_group_size),
+                          C.c_int(out_dtype), C.c_int(int(cv18xx)))
+    return out
+
+
+def a16matmul(x, weight, scale, zp, bias, *, M, K, N, weight_bits, q_group_size, w_transpose=True,
+              out_dtype=OUT_BF16, cv18xx=False, gemm_kind=GEMM_F64ACC):
+    """tpu.A16MatMul on f32-valued operands; returns (output, pre-rounding f32)."""
+    ins = [_f32(x), _f32(weight), _f32(scale), _f32(zp), _f32(bias)]
+    attr = A16Attr(M, K, N, weight_bits, int(w_transpose), q_group_size, out_dtype, int(cv18xx), gemm_kind)
+    arr = (C.POINTER(C.c_float) * 5)(*[None if a is None else _p(a, C.c_float) for a in ins])
+    out = np.empty((M, N), dtype=np.float32)
+    pre = np.empty((M, N), dtype=np.float32)
+    rc = lib().orc_a16matmul(C.byref(attr), arr, _p(out, C.c_float), _p(pre, C.c_float))
+    if rc != 0:
+        raise RuntimeError("orc_a16matmul failed")
+    return out, pre
+
+
+def matmul_int8(x, right, bias, multi, *, M, K, N, right_transpose=False, input_zp=0, right_zp=0,
+                do_relu=False, relu_limit=-1.0, cv18xx=False, quant_mode=RQ_MULTIPLIER_SHIFT, fuse_rq=False,
+                multipliers=(1,), rshifts=(0,), out_zp=0, out_kind=0, out_bits=8, out_unsigned=False,
+                gemm_kind=GEMM_F32):
+    """Quantised tpu.MatMul on f32-valued operands; returns (output, f32 accumulators)."""
+    ins = [_f32(x), _f32(right), _f32(bias), _f32(multi)]
+    mult = np.ascontiguousarray(multipliers, dtype=np.int64)
+    rs = np.ascontiguousarray(rshifts, dtype=np.int64)
+    attr = I8Attr(M, K, N, int(right_transpose), input_zp, right_zp, int(do_relu), relu_limit, int(cv18xx),
+                  quant_mode, int(fuse_rq), _p(mult, C.c_int64), mult.size, _p(rs, C.c_int64), rs.size,
+                  out_zp, out_kind, out_bits, int(out_unsigned), gemm_kind)
+    arr = (C.POINTER(C.c_float) * 4)(*[None if a is None else _p(a, C.c_float) for a in ins])
+    out = np.empty((M, N), dtype=np.float32)
+    acc = np.empty((M, N), dtype=np.float32)
+    rc = lib().orc_matmul_int8(C.byref(attr), arr, _p(out, C.c_float), _p(acc, C.c_float))
+    if rc != 0:
+        raise RuntimeError("orc_matmul_int8 failed")
+    return out, acc
+
+
+def igemm_i64(A, B, bias, *, right_transpose=False, input_zp=0, right_zp=0):
+    A = np.ascontiguousarray(A, dtype=np.int8)
+    B = np.ascontiguousarray(B, dtype=np.int8)
+    M, K = A.shape
+    N = B.shape[0] if right_transpose else B.shape[1]
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+    Y = np.empty((M, N), dtype=np.int64)
+    lib().orc_igemm_i64(_p(A, C.c_int8), _p(B, C.c_int8), None if b is None else _p(b, C.c_int32),
+                        _p(Y, C.c_int64), C.c_int64(M), C.c_int64(K), C.c_int64(N), C.c_int(int(right_transpose)),
+                        C.c_int64(input_zp), C.c_int64(right_zp))
+    return Y
+
+
+def requant_int_axis(x, quant, *, quant_mode, round_mode=HALF_AWAY_FROM_ZERO, fuse_rq_axis=False,
+                     is_bm1684x=True, cv18xx=False, input_zp=0, out_bits=8, out_unsigned=False):
+    x, quant = _f32(x), _f32(quant)
+    shape = (C.c_int64 * 8)(*(list(x.shape) + [1] * (8 - x.ndim)))
+    attr = RqAxisAttr(shape, x.ndim, quant_mode, round_mode, int(fuse_rq_axis), int(is_bm1684x), int(cv18xx),
+                      input_zp, out_bits, int(out_unsigned))
+    out = np.empty_like(x)
+    rc = lib().orc_requant_int_axis(C.byref(attr), _p(x, C.c_float), _p(quant, C.c_float), _p(out, C.c_float))
+    if rc != 0:
+        raise RuntimeError("orc_requant_int_axis failed")
+    return out
+
+
+def requant_int(x, *, quant_mode, multiplier, rshift, round_mode=HALF_AWAY_FROM_ZERO, cv18xx=False,
+                input_zp=0, out_zp=0, out_bits=8, out_unsigned=False):
+    x = _f32(x)
+    shape = (C.c_int64 * 8)(*(list(x.shape) + [1] * (8 - x.ndim)))
+    attr = RqAttr(shape, x.ndim, quant_mode, round_mode, multiplier, rshift, int(cv18xx), input_zp, out_zp,
+                  out_bits, int(out_unsigned))
+    out = x.copy()
+    rc = lib().orc_requant_int(C.byref(attr), _p(x, C.c_float), _p(out, C.c_float))
+    if rc != 0:
+        raise RuntimeError("orc_requant_int failed")
+    return out
+
+
+def num_threads():
+    return lib().orc_num_threads()
