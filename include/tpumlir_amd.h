@@ -1,0 +1,219 @@
+/*
+ * C ABI of the MI355X (gfx950) backend for the reference interpreter's
+ * quantized-matmul ops.  Plain pointers and sizes only; every entry point
+ * returns MI_SUCCESS (0) where the reference returns success() and a non-zero
+ * code where it returns failure() (the caller then keeps its CPU path).
+ *
+ * Two levels:
+ *  1. Operator level -- the surface the interpreter binds.  One
+ *     init/inference/deinit trio per op, taking the op's attributes as a plain
+ *     struct (there is no MLIR here to read them from) and a mirror of
+ *     InferenceParameter.  Operands follow the interpreter's convention: every
+ *     tensor is a host float array holding numel values, whatever its storage
+ *     type (packed nibble bytes arrive as floats 0..255, bf16 values widened).
+ *  2. Device level -- launches on device pointers and a HIP stream, with
+ *     weights already resident in HBM in the kernels' own layout.  This is
+ *     what a device-resident interpreter and the benchmarks use.
+ *
+ * Paths are relative to the reference tree.
+ */
+#ifndef TPUMLIR_AMD_H
+#define TPUMLIR_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status codes --------------------------------------------------------- */
+#define MI_SUCCESS 0        /* success() */
+#define MI_UNSUPPORTED 1    /* failure(): attribute combination not handled on the GPU */
+#define MI_BAD_ARGUMENT 2   /* failure(): null operand, bad shape, K not a multiple of the group */
+#define MI_HIP_ERROR 3      /* failure(): the HIP runtime reported an error (see mi_last_error) */
+
+/* ---- enums: numeric values equal the reference's ---------------------------- */
+/* RoundingMode, include/tpu_mlir/Support/MathUtils.h:29-41 */
+enum {
+  MI_ROUND_HALF_AWAY_FROM_ZERO = 0,
+  MI_ROUND_HALF_UP = 1,
+  MI_ROUND_HALF_DOWN = 2,
+  MI_ROUND_HALF_TO_EVEN = 3,
+  MI_ROUND_TOWARDS_ZERO = 6,
+  MI_ROUND_UP = 8,
+  MI_ROUND_DOWN = 9
+};
+/* tpu::RequantMode, include/tpu_mlir/Dialect/Tpu/IR/TpuOps.td:160-172 */
+enum {
+  MI_RQ_TFLITE_LSHIFT = 0,
+  MI_RQ_TFLITE = 1,
+  MI_RQ_MULTIPLIER_SHIFT = 2,
+  MI_RQ_ONLY_SHIFT = 3,
+  MI_RQ_QDM = 4
+};
+/* storage types */
+enum { MI_DT_BF16 = 0, MI_DT_F16 = 1, MI_DT_I8 = 2, MI_DT_U8 = 3, MI_DT_I16 = 4, MI_DT_U16 = 5, MI_DT_I32 = 6 };
+/* chip family: selects the bf16 rounding flavour and the CV18xx requant branches
+ * (module::isCV18xx(), lib/Support/Float16.cpp:769-774, lib/Support/MathUtils.cpp:538-562) */
+enum { MI_CHIP_BM168X = 0, MI_CHIP_CV18XX = 1 };
+
+/* ---- library ---------------------------------------------------------------- */
+const char *mi_version(void);
+/* text of the last error raised on the calling thread ("" if none) */
+const char *mi_last_error(void);
+/* number of visible GPUs; 0 when there is none (no HIP context is created) */
+int mi_device_count(void);
+
+/* Mirror of tpu_mlir::InferenceParameter (include/tpu_mlir/Interfaces/InferenceInterface.h:15-19):
+ * inputs/outputs in MLIR operand order, a None operand is a null pointer, handle is owned by the op
+ * between init and deinit. */
+typedef struct mi_infer_param {
+  float **inputs;
+  int n_inputs;
+  float **outputs;
+  int n_outputs;
+  void *handle;
+} mi_infer_param;
+
+/* ============================================================================ */
+/* tpu.A16MatMul  (lib/Dialect/Tpu/Interfaces/Common/A16MatMul.cpp:16-249)       */
+/* ============================================================================ */
+typedef struct mi_a16mm_attr {
+  int64_t M;            /* product of the input's leading dims (A16MatMul.cpp:31-35); may change per call */
+  int64_t K, N;         /* input [M,K], output [M,N]; weight holds N output channels */
+  int weight_bits;      /* getWeightBits(): 4 or 8 */
+  int w_transpose;      /* getWTranspose(): 1 = weight stored [N,K] (4-bit: [N,K/2] bytes) */
+  int q_group_size;     /* getQGroupSize() or module::getQuantGroupSize(); 0 = per output channel */
+  int out_dtype;        /* MI_DT_BF16, or MI_DT_F16 when module::isF16Modes() */
+  int chip;             /* MI_CHIP_* */
+  int dynamic_quant;    /* module::isDynamicQuantize(): not handled, returns MI_UNSUPPORTED */
+} mi_a16mm_attr;
+
+/* Replaces tpu::A16MatMulOp::init (A16MatMul.cpp:16-18).  inputs = {input, weight, scale, zp, bias|NULL}.
+ * Repacks weight/scale/zp/bias once into the kernels' layout, keeps them in HBM, stores the handle. */
+int mi_a16mm_init(const mi_a16mm_attr *attr, mi_infer_param *p);
+/* Replaces tpu::A16MatMulOp::inference (A16MatMul.cpp:22-249, static path :171-246).
+ * Reads inputs[0] (f32-valued bf16/f16), writes outputs[0] already rounded to out_dtype. */
+int mi_a16mm_inference(const mi_a16mm_attr *attr, mi_infer_param *p);
+/* Replaces tpu::A16MatMulOp::deinit (A16MatMul.cpp:20). */
+void mi_a16mm_deinit(mi_infer_param *p);
+
+/* ---- device level ---- */
+typedef struct mi_a16_weight mi_a16_weight; /* packed, HBM-resident weight set */
+
+typedef struct mi_a16_weight_desc {
+  int64_t K, N;
+  int weight_bits;     /* 4: weight is uint8 [N,K/2], even k in the low nibble; 8: [N,K] */
+  int weight_signed;   /* 8-bit only: bytes are int8 */
+  int q_group_size;    /* 0 = per channel */
+  int dtype;           /* MI_DT_BF16 / MI_DT_F16: type of activations, scales and outputs */
+  int chip;
+} mi_a16_weight_desc;
+
+/* Builds the packed weight set from HOST arrays in the reference's layout:
+ * weight bytes as above, scale = bf16/f16 bit patterns [N,G], zp = uint8 [N,G] (G = K/g or 1),
+ * bias = float [N] or NULL.  Blocks until the copy and the on-GPU repack are done. */
+int mi_a16_weight_create(mi_a16_weight **out, const mi_a16_weight_desc *desc, const void *weight,
+                         const uint16_t *scale, const uint8_t *zp, const float *bias);
+void mi_a16_weight_destroy(mi_a16_weight *w);
+/* HBM bytes held by the packed set */
+size_t mi_a16_weight_bytes(const mi_a16_weight *w);
+
+/* y[M,N] = round(x[M,K] * dequant(W)^T + bias).  d_x/d_y are DEVICE pointers to bf16/f16 bit patterns;
+ * d_y_f32 (optional DEVICE pointer, may be NULL) receives the fp32 result before output rounding.
+ * Asynchronous on `stream` (a hipStream_t, NULL = default stream). */
+int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
+                    void *stream);
+
+/* ============================================================================ */
+/* tpu.MatMul, quantized  (lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:387-733) */
+/* ============================================================================ */
+typedef struct mi_i8mm_attr {
+  int64_t M, K, N;        /* parseParam() "case 1/2/4/6": batch == 1 (MatMul.cpp:17-135) */
+  int right_transpose;    /* right stored [N,K] */
+  int64_t input_zp, right_zp;
+  int do_relu;
+  double relu_limit;
+  int chip;
+  int quant_mode;         /* MI_RQ_* */
+  int round_mode;         /* the op's round_mode attribute; the CPU interpreter ignores it for this op
+                             (MatMul.cpp:660,703,713), so the operator-level entry points do too */
+  int fuse_rq;            /* per-channel multiplier taken from inputs[3] (MatMul.cpp:709-716) */
+  const int64_t *multipliers; int n_multipliers;   /* getMultipliers() */
+  const int64_t *rshifts;     int n_rshifts;       /* getRshifts() */
+  int64_t out_zp;         /* zero point of the uniform-quantized output type */
+  int out_dtype;          /* MI_DT_I8/U8/I16/U16, or MI_DT_I32 for an un-requantized int32 result */
+  int right_is_weight;    /* module::isWeight(getRight()): right (and bias, multi) are cached in HBM at init */
+} mi_i8mm_attr;
+
+/* Replace tpu::MatMulOp::{init,inference,deinit} (MatMul.cpp:387-396, :440-733, :431-438).
+ * inputs = {input, right, bias|NULL, multi|NULL, buffer|NULL}. */
+int mi_i8mm_init(const mi_i8mm_attr *attr, mi_infer_param *p);
+int mi_i8mm_inference(const mi_i8mm_attr *attr, mi_infer_param *p);
+void mi_i8mm_deinit(mi_infer_param *p);
+
+/* ---- device level ---- */
+/* int32 -> narrow integer requantization applied per output channel n:
+ *   MI_RQ_MULTIPLIER_SHIFT: v = RightShiftRound(acc * mult[n], shift[n], round_mode)      (MathUtils.cpp:541-546)
+ *                           (CV18xx: evaluated in float32 and rounded, MathUtils.cpp:542-543)
+ *   MI_RQ_TFLITE / _LSHIFT / QDM: v = MultiplyByQuantizedMultiplier(acc, mult[n], -shift[n], round_mode)
+ *                           i.e. shift[n] is a RIGHT shift when positive                   (MathUtils.cpp:523-536)
+ *   MI_RQ_ONLY_SHIFT:       v = RightShiftRound(acc, shift[n], round_mode)
+ *   out = saturate(v + zp[n], out_dtype)                                                    (MathUtils.cpp:849-872)
+ * d_multiplier/d_shift/d_zp are DEVICE int32 arrays of length n_channels, or NULL to use the scalar. */
+typedef struct mi_requant_desc {
+  int quant_mode;
+  int round_mode;
+  int chip;
+  int out_dtype;
+  const int32_t *d_multiplier; int32_t multiplier;
+  const int32_t *d_shift;      int32_t shift;
+  const int32_t *d_zp;         int32_t zp;
+} mi_requant_desc;
+
+/* acc[M,N] = (A - input_zp)[M,K] * (B - right_zp) + bias[N], relu, then requant -> d_out.
+ * d_a int8 [M,K]; d_b int8 [N,K] when right_transpose else [K,N]; d_bias int32 [N] or NULL.
+ * a_unsigned / b_unsigned: the bytes are uint8.  rq == NULL: d_out receives the int32 accumulators.
+ * d_acc (optional) also receives the int32 accumulators after relu. */
+int mi_i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned, int right_transpose,
+                   const int32_t *d_bias, int64_t M, int64_t K, int64_t N, int64_t input_zp, int64_t right_zp,
+                   int do_relu, int64_t relu_limit, const mi_requant_desc *rq, void *d_out, int32_t *d_acc,
+                   void *stream);
+
+/* ============================================================================ */
+/* tpu.RequantIntAxis / tpu.RequantInt                                            */
+/* (lib/Dialect/Tpu/Interfaces/Common/RequantIntAxis.cpp:17-121, RequantInt.cpp:17-72) */
+/* ============================================================================ */
+typedef struct mi_rq_axis_attr {
+  int64_t shape[8]; int rank;   /* output shape */
+  int quant_mode, round_mode;
+  int fuse_rq_axis;             /* requant along the last dim, shift used as stored */
+  int quant_triples;            /* 1: quant operand is (multiplier, shift, zp) per channel (module::isBM1684X());
+                                   0: (multiplier, packed shift|zp) pairs */
+  int chip;
+  int64_t input_zp;
+  int out_dtype;
+} mi_rq_axis_attr;
+/* inputs = {input (f32-valued int32), quant}; no state: init/deinit are no-ops in the reference */
+int mi_requant_int_axis_inference(const mi_rq_axis_attr *attr, mi_infer_param *p);
+
+typedef struct mi_rq_attr {
+  int64_t shape[8]; int rank;
+  int quant_mode, round_mode;
+  int64_t multiplier, rshift;   /* getMultiplier(), getRshift() */
+  int chip;
+  int64_t input_zp, out_zp;
+  int out_dtype;
+} mi_rq_attr;
+int mi_requant_int_inference(const mi_rq_attr *attr, mi_infer_param *p);
+
+/* device level: d_in int32 [outer, channels, inner] -> d_out (out_dtype), channel = the axis the
+ * per-channel arrays of rq index; input_zp is subtracted first. */
+int mi_requant_launch(const int32_t *d_in, void *d_out, int64_t outer, int64_t channels, int64_t inner,
+                      int64_t input_zp, const mi_requant_desc *rq, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TPUMLIR_AMD_H */

@@ -1,0 +1,90 @@
+"""CPU-side checks of the C ABI library: it loads, exports every declared symbol, and rejects bad
+arguments without touching a GPU."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from helpers import pkg, ROOT
+
+M = pkg()
+clib = pkg("clib")
+
+
+def test_library_exports_every_declared_symbol():
+    L = clib.lib()
+    header = open(os.path.join(ROOT, "include", "tpumlir_amd.h")).read()
+    declared = set(re.findall(r"\b(mi_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(clib.EXPORTS)
+    for name in declared:
+        assert hasattr(L, name), name
+    assert "gfx950" in M.version()
+
+
+def test_argument_errors_need_no_gpu():
+    L = clib.lib()
+    assert L.mi_a16mm_init(None, None) == clib.MI_BAD_ARGUMENT
+    assert "null" in M.last_error()
+    # dynamic activation quantisation, w_transpose == false, odd bit widths: failure() -> caller keeps CPU path
+    w = np.zeros((4, 64), np.float32)
+    s = np.ones((4, 1), np.float32)
+    z = np.zeros((4, 1), np.float32)
+    for kw, code in ((dict(dynamic_quant=True), clib.MI_UNSUPPORTED),
+                     (dict(w_transpose=False), clib.MI_UNSUPPORTED),
+                     (dict(weight_bits=3), clib.MI_UNSUPPORTED),
+                     (dict(q_group_size=48), clib.MI_BAD_ARGUMENT),      # K % g != 0
+                     (dict(q_group_size=16), clib.MI_UNSUPPORTED)):      # group size the kernels do not handle
+        args = dict(K=128, N=4, weight_bits=4, q_group_size=0)
+        args.update(kw)
+        op = M.A16MatMul(**args)
+        with pytest.raises(M.BackendError) as e:
+            op.init(w, s, z)
+        assert e.value.code == code, kw
+    # None scale / zp are rejected (the reference would dereference them)
+    op = M.A16MatMul(K=128, N=4, weight_bits=4, q_group_size=0)
+    with pytest.raises(M.BackendError) as e:
+        op.init(w, None, z)
+    assert e.value.code == clib.MI_BAD_ARGUMENT
+    # inference before init
+    with pytest.raises(M.BackendError):
+        op.inference(np.zeros((1, 128), np.float32))
+    # non-integer packed weight / scale that is not a bf16 number
+    op = M.A16MatMul(K=128, N=4, weight_bits=4, q_group_size=0)
+    with pytest.raises(M.BackendError) as e:
+        op.init(w + 0.5, s, z)
+    assert e.value.code == clib.MI_UNSUPPORTED
+    with pytest.raises(M.BackendError) as e:
+        op.init(w, s * np.float32(1.0001), z)
+    assert e.value.code == clib.MI_UNSUPPORTED
+
+
+def test_int8_and_requant_argument_errors():
+    L = clib.lib()
+    assert L.mi_i8mm_init(None, None) == clib.MI_BAD_ARGUMENT
+    assert L.mi_requant_launch(None, None, 1, 1, 1, 0, None, None) == clib.MI_BAD_ARGUMENT
+    assert L.mi_i8mm_launch(None, 0, None, 0, 0, None, 1, 1, 1, 0, 0, 0, -1, None, None, None, None) == \
+        clib.MI_BAD_ARGUMENT
+    op = M.MatMulInt8(K=8, N=8, quant_mode=clib.RQ_ONLY_SHIFT)  # BM168x branch has no OnlyShift
+    with pytest.raises(M.BackendError) as e:
+        op.init(np.zeros((2, 8), np.float32), np.zeros((8, 8), np.float32))
+    assert e.value.code == clib.MI_UNSUPPORTED
+    with pytest.raises(M.BackendError) as e:
+        M.requant_int_axis(np.zeros((2, 3), np.float32), np.zeros((3, 3), np.float32), quant_mode=clib.RQ_QDM)
+    assert e.value.code == clib.MI_UNSUPPORTED
+    # rank-1 RequantInt is a no-op in the reference
+    v = np.array([5.0, -7.0], np.float32)
+    assert np.array_equal(M.requant_int(v, quant_mode=clib.RQ_MULTIPLIER_SHIFT, multiplier=1, rshift=1), v)
+
+
+def test_compare_metrics():
+    cmp = pkg("compare")
+    a = np.array([1.0, 2.0, 3.0, 4.0])
+    assert cmp.cosine_similarity(a, a) == pytest.approx(1.0)
+    assert cmp.euclidean_similarity(a, a) == pytest.approx(1.0)
+    assert cmp.sqnr(a, a) == float("inf")
+    b = a + np.array([0.1, -0.1, 0.1, -0.1])
+    assert cmp.euclidean_similarity(a, b) == pytest.approx(1 - np.linalg.norm(a - b) / (np.linalg.norm((a + b) / 2) + 1e-7))
+    assert cmp.sqnr(a, b) == pytest.approx(10 * np.log10(np.var(a) / np.var(a - b)))
+    assert cmp.cosine_similarity(np.zeros(3), a[:3]) == 0.0

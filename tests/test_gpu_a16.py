@@ -1,0 +1,174 @@
+"""GPU parity of tpu.A16MatMul (W4A16 / W8A16) against the CPU oracle, through the C ABI.
+
+Tolerances (bf16/f16 paths): the fp32 result before output rounding must agree with the oracle's
+double-accumulated result to max-abs <= 2e-5 * RMS(output) (the north-star bound is 1e-2 * RMS; the
+reference's own fp32 summation order is unspecified).  After rounding, outputs may differ only where
+the fp32 values straddle a rounding boundary: at most one 16-bit ulp, on fewer than 0.5 % of elements.
+"""
+import numpy as np
+import pytest
+
+from helpers import pkg, f32_valued_a16
+
+pytestmark = pytest.mark.gpu
+
+M_ = pkg()
+S = pkg("synth")
+clib = pkg("clib")
+cmp = pkg("compare")
+
+
+def _torch():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+def _ulp_distance_bf16(a_bits, b_bits):
+    def key(u):
+        u = u.astype(np.int32)
+        return np.where(u & 0x8000, -(u & 0x7FFF), u & 0x7FFF)
+    return np.abs(key(a_bits) - key(b_bits))
+
+
+def _run_device(cfg, dtype=clib.DT_BF16):
+    torch = _torch()
+    tdt = torch.bfloat16 if dtype == clib.DT_BF16 else torch.float16
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"],
+                     None if cfg.get("bias") is None else S.bf16_to_f32(cfg["bias"]),
+                     K=cfg["K"], N=cfg["N"], weight_bits=cfg["bits"], q_group_size=cfg["g"], dtype=dtype)
+    x = torch.from_numpy(cfg["x"].view(np.int16)).cuda().view(tdt)
+    y32 = torch.empty((cfg["M"], cfg["N"]), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_launch(w, x, y_f32=y32)
+    torch.cuda.synchronize()
+    out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    pre = y32.cpu().numpy()
+    w.destroy()
+    return out, pre
+
+
+def _check_against_oracle(orc, cfg, out_bits, pre):
+    x, w, s, z, b = f32_valued_a16(cfg)
+    want, want_pre = orc.a16matmul(x, w, s, z, b, M=cfg["M"], K=cfg["K"], N=cfg["N"], weight_bits=cfg["bits"],
+                                   q_group_size=cfg["g"], gemm_kind=orc.GEMM_F64ACC)
+    err = cmp.max_abs_over_rms(pre, want_pre)
+    assert err <= 2e-5, "fp32 pre-round max-abs/RMS %.3g" % err
+    want_bits = orc.f32_to_bf16(want)
+    ulp = _ulp_distance_bf16(out_bits, want_bits)
+    assert ulp.max() <= 1
+    assert (ulp != 0).mean() < 5e-3
+    # the output must be exactly the reference rounding of the kernel's own fp32 value
+    assert np.array_equal(out_bits, orc.f32_to_bf16(pre))
+    return err
+
+
+W4_CASES = [  # (M, K, N, g)
+    (1, 2048, 6144, 64), (4, 2048, 6144, 64), (16, 2048, 6144, 64),   # Qwen-like decode projection
+    (1, 4096, 4096, 128), (8, 4096, 4096, 128),                        # Llama-7B q_proj at decode
+    (1, 4096, 11008, 128), (1, 11008, 4096, 128),                      # gate/up and down projections
+    (3, 512, 48, 32), (2, 1024, 100, 256), (5, 384, 33, 0),            # other group sizes, ragged N
+    (1, 200, 16, 0), (7, 136, 20, 0),                                  # K not a multiple of the tile
+    (40, 512, 64, 128),                                                # M > 16: several row blocks of x
+]
+
+
+@pytest.mark.parametrize("M,K,N,g", W4_CASES)
+def test_w4a16_device_level(orc, M, K, N, g):
+    cfg = S.w4a16(M, K, N, g, seed=M + K + N, bias=(N % 3 == 0))
+    out, pre = _run_device(cfg)
+    _check_against_oracle(orc, cfg, out, pre)
+
+
+W8_CASES = [  # (M, K, N, g, signed)
+    (1, 4096, 11008, 0, True), (32, 4096, 1024, 0, True),   # per-channel symmetric MLP up-projection
+    (4, 1024, 96, 128, False), (2, 512, 40, 32, False), (3, 256, 24, 64, False),
+    (1, 200, 17, 0, True),
+]
+
+
+@pytest.mark.parametrize("M,K,N,g,signed", W8_CASES)
+def test_w8a16_device_level(orc, M, K, N, g, signed):
+    cfg = S.w8a16(M, K, N, g, seed=M + K, signed=signed, bias=(N % 2 == 0))
+    out, pre = _run_device(cfg)
+    _check_against_oracle(orc, cfg, out, pre)
+
+
+def test_operator_level_matches_oracle(orc):
+    # the interpreter's calling convention: float-expanded operands, init once, inference twice, deinit
+    cfg = S.w4a16(4, 1024, 256, 128, seed=11, bias=True)
+    x, w, s, z, b = f32_valued_a16(cfg)
+    op = M_.A16MatMul(K=1024, N=256, weight_bits=4, q_group_size=128).init(w, s, z, b)
+    for m in (4, 1):
+        y = op.inference(x[:m])
+        want, _ = orc.a16matmul(x[:m], w, s, z, b, M=m, K=1024, N=256, weight_bits=4, q_group_size=128)
+        ulp = _ulp_distance_bf16(orc.f32_to_bf16(y), orc.f32_to_bf16(want))
+        assert ulp.max() <= 1 and (ulp != 0).mean() < 5e-3
+        assert np.array_equal(orc.BF16(y), y)  # outputs are bf16 numbers
+        assert cmp.cosine_similarity(y, want) > 0.9999 and cmp.euclidean_similarity(y, want) > 0.9999
+    op.deinit()
+    # W8, f16 mode
+    cfg = S.w8a16(3, 512, 64, 0, seed=12)
+    x = orc.F16(S.bf16_to_f32(cfg["x"]))
+    scale = orc.F16(S.bf16_to_f32(cfg["scale"]))
+    w = cfg["weight"].astype(np.float32)
+    z = cfg["zp"].astype(np.float32)
+    op = M_.A16MatMul(K=512, N=64, weight_bits=8, q_group_size=0, out_dtype=clib.DT_F16).init(w, scale, z)
+    y = op.inference(x)
+    want, want_pre = orc.a16matmul(x, w, scale, z, None, M=3, K=512, N=64, weight_bits=8, q_group_size=0,
+                                   out_dtype=orc.OUT_F16)
+    assert np.array_equal(orc.F16(y), y)
+    assert np.max(np.abs(y - want)) <= 2.0 ** -10 * np.max(np.abs(want))
+    assert (y != want).mean() < 5e-3
+    op.deinit()
+
+
+def test_full_size_exact_properties():
+    """Size-independent exact checks at the Llama-7B gate/up shape (N=11008, K=4096, g=128)."""
+    torch = _torch()
+    M, K, N, g = 16, 4096, 11008, 128
+    cfg = S.w4a16(M, K, N, g, seed=99, bias=True)
+    # one-hot activation rows: y[m, n] = bf16((q[n,k_m] - zp) * scale + bias[n]) has a single product term, so
+    # no summation order is involved and the result must be bit exact
+    ks = np.array([0, 1, 7, 8, 127, 128, 129, 2047, 2048, 4095, 1000, 3333, 31, 32, 33, 64])
+    xf = np.zeros((M, K), np.float32)
+    xf[np.arange(M), ks] = 1.0
+    cfg["x"] = S.bf16_round(xf)
+    out, pre = _run_device(cfg)
+    s = S.bf16_to_f32(cfg["scale"])
+    q = cfg["q"].astype(np.float32)
+    zp = cfg["zp"].astype(np.float32)
+    bias = S.bf16_to_f32(cfg["bias"])
+    want = ((q[:, ks] - zp[:, ks // g]) * s[:, ks // g]).T.astype(np.float32) + bias[None, :]
+    assert np.array_equal(pre, want.astype(np.float32))
+    assert np.array_equal(out, S.bf16_round(want))
+    # linearity in the activations: f(2x) == 2 f(x) exactly (powers of two commute with every rounding)
+    cfg3 = S.w4a16(2, K, N, g, seed=97)
+    o1, p1 = _run_device(cfg3)
+    cfg3["x"] = S.bf16_round(2.0 * S.bf16_to_f32(cfg3["x"]))
+    o2, p2 = _run_device(cfg3)
+    assert np.array_equal(p2, 2.0 * p1)
+    rms = float(np.sqrt(np.mean(p1.astype(np.float64) ** 2)))
+    # all-zero-point weights: every product vanishes and the output is the bias.  The kernel evaluates each group
+    # as scale * (sum a*(OFFSET+q) - (OFFSET+zp) * sum a), so the cancellation is exact only up to fp32 rounding
+    # of the two sums: bound the residue by the same 2e-5 * RMS of an ordinary output
+    cfg2 = S.w4a16(4, K, N, g, seed=98, bias=True)
+    cfg2["q"][:] = np.repeat(cfg2["zp"], g, axis=1)
+    cfg2["weight"] = S.pack_nibbles(cfg2["q"])
+    out2, pre2 = _run_device(cfg2)
+    assert np.max(np.abs(pre2 - S.bf16_to_f32(cfg2["bias"])[None, :])) <= 2e-5 * rms
+
+
+def test_f16_mode_device_level(orc):
+    torch = _torch()
+    M, K, N, g = 4, 1024, 128, 128
+    cfg = S.w4a16(M, K, N, g, seed=5)
+    xf = orc.F16(S.bf16_to_f32(cfg["x"]))
+    sf = orc.F16(S.bf16_to_f32(cfg["scale"]))
+    cfg16 = dict(cfg)
+    cfg16["x"] = orc.f32_to_f16(xf)
+    cfg16["scale"] = orc.f32_to_f16(sf)
+    out, pre = _run_device(cfg16, dtype=clib.DT_F16)
+    want, want_pre = orc.a16matmul(xf, cfg["weight"].astype(np.float32), sf, cfg["zp"].astype(np.float32), None,
+                                   M=M, K=K, N=N, weight_bits=4, q_group_size=g, out_dtype=orc.OUT_F16)
+    assert cmp.max_abs_over_rms(pre, want_pre) <= 2e-5
+    assert np.array_equal(out, orc.f32_to_f16(pre))

@@ -115,7 +115,7 @@ def test_requant_int_axis(rmode):
                 for v in x[:, c].reshape(-1)]
         assert out[:, c].reshape(-1).astype(np.int64).tolist() == want
     # MultiplierShift, axis 1: stored shift is negated into a right shift (RequantIntAxis.cpp:93-118)
-    multi2 = rng.integers(1, 30000, size=C)
+    multi2 = rng.integers(1, 500, size=C)  # keep |x*m >> s| inside int32 (the reference narrows to int)
     quant2 = np.stack([multi2, shift, zp], axis=1).astype(np.float32).reshape(1, C, 1, 3)
     out = O.requant_int_axis(x, quant2, quant_mode=O.RQ_MULTIPLIER_SHIFT, round_mode=rmode)
     for c in range(C):
@@ -124,7 +124,7 @@ def test_requant_int_axis(rmode):
         assert out[:, c].reshape(-1).astype(np.int64).tolist() == want
     # fused-axis form: last dimension, shift used as stored (positive = right shift) (:68-91)
     W = shape[-1]
-    multi3 = rng.integers(1, 30000, size=W)
+    multi3 = rng.integers(1, 500, size=W)
     shift3 = rng.integers(1, 12, size=W)
     zp3 = rng.integers(-10, 10, size=W)
     quant3 = np.stack([multi3, shift3, zp3], axis=1).astype(np.float32)

@@ -1,0 +1,133 @@
+"""ctypes binding of libtpumlir_amd.so (the C ABI declared in include/tpumlir_amd.h)."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "lib", "libtpumlir_amd.so")
+
+MI_SUCCESS, MI_UNSUPPORTED, MI_BAD_ARGUMENT, MI_HIP_ERROR = 0, 1, 2, 3
+ROUND_HALF_AWAY_FROM_ZERO, ROUND_HALF_UP, ROUND_HALF_DOWN, ROUND_HALF_TO_EVEN = 0, 1, 2, 3
+ROUND_TOWARDS_ZERO, ROUND_UP, ROUND_DOWN = 6, 8, 9
+RQ_TFLITE_LSHIFT, RQ_TFLITE, RQ_MULTIPLIER_SHIFT, RQ_ONLY_SHIFT, RQ_QDM = 0, 1, 2, 3, 4
+DT_BF16, DT_F16, DT_I8, DT_U8, DT_I16, DT_U16, DT_I32 = range(7)
+CHIP_BM168X, CHIP_CV18XX = 0, 1
+
+# every symbol include/tpumlir_amd.h declares
+EXPORTS = [
+    "mi_version", "mi_last_error", "mi_device_count",
+    "mi_a16mm_init", "mi_a16mm_inference", "mi_a16mm_deinit",
+    "mi_a16_weight_create", "mi_a16_weight_destroy", "mi_a16_weight_bytes", "mi_a16mm_launch",
+    "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
+    "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
+]
+
+
+class BackendError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("tpumlir_amd error %d: %s" % (code, msg))
+        self.code = code
+
+
+class InferParam(C.Structure):
+    _fields_ = [("inputs", C.POINTER(C.POINTER(C.c_float))), ("n_inputs", C.c_int),
+                ("outputs", C.POINTER(C.POINTER(C.c_float))), ("n_outputs", C.c_int),
+                ("handle", C.c_void_p)]
+
+
+class A16Attr(C.Structure):
+    _fields_ = [("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64), ("weight_bits", C.c_int),
+                ("w_transpose", C.c_int), ("q_group_size", C.c_int), ("out_dtype", C.c_int), ("chip", C.c_int),
+                ("dynamic_quant", C.c_int)]
+
+
+class A16WeightDesc(C.Structure):
+    _fields_ = [("K", C.c_int64), ("N", C.c_int64), ("weight_bits", C.c_int), ("weight_signed", C.c_int),
+                ("q_group_size", C.c_int), ("dtype", C.c_int), ("chip", C.c_int)]
+
+
+class I8Attr(C.Structure):
+    _fields_ = [("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64), ("right_transpose", C.c_int),
+                ("input_zp", C.c_int64), ("right_zp", C.c_int64), ("do_relu", C.c_int), ("relu_limit", C.c_double),
+                ("chip", C.c_int), ("quant_mode", C.c_int), ("round_mode", C.c_int), ("fuse_rq", C.c_int),
+                ("multipliers", C.POINTER(C.c_int64)), ("n_multipliers", C.c_int),
+                ("rshifts", C.POINTER(C.c_int64)), ("n_rshifts", C.c_int),
+                ("out_zp", C.c_int64), ("out_dtype", C.c_int), ("right_is_weight", C.c_int)]
+
+
+class RequantDescC(C.Structure):
+    _fields_ = [("quant_mode", C.c_int), ("round_mode", C.c_int), ("chip", C.c_int), ("out_dtype", C.c_int),
+                ("d_multiplier", C.c_void_p), ("multiplier", C.c_int32),
+                ("d_shift", C.c_void_p), ("shift", C.c_int32),
+                ("d_zp", C.c_void_p), ("zp", C.c_int32)]
+
+
+class RqAxisAttr(C.Structure):
+    _fields_ = [("shape", C.c_int64 * 8), ("rank", C.c_int), ("quant_mode", C.c_int), ("round_mode", C.c_int),
+                ("fuse_rq_axis", C.c_int), ("quant_triples", C.c_int), ("chip", C.c_int), ("input_zp", C.c_int64),
+                ("out_dtype", C.c_int)]
+
+
+class RqAttr(C.Structure):
+    _fields_ = [("shape", C.c_int64 * 8), ("rank", C.c_int), ("quant_mode", C.c_int), ("round_mode", C.c_int),
+                ("multiplier", C.c_int64), ("rshift", C.c_int64), ("chip", C.c_int), ("input_zp", C.c_int64),
+                ("out_zp", C.c_int64), ("out_dtype", C.c_int)]
+
+
+_lib = None
+
+
+def library_path():
+    return _LIB_PATH
+
+
+def lib():
+    """Loads the built library.  Never builds and never falls back: a missing library is an error."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise BackendError(MI_HIP_ERROR, "%s is missing: build it with `python tpu-mlir_amd/build.py`" % _LIB_PATH)
+        L = C.CDLL(_LIB_PATH)
+        L.mi_version.restype = C.c_char_p
+        L.mi_last_error.restype = C.c_char_p
+        L.mi_device_count.restype = C.c_int
+        L.mi_a16_weight_bytes.restype = C.c_size_t
+        L.mi_a16_weight_bytes.argtypes = [C.c_void_p]
+        L.mi_a16_weight_create.argtypes = [C.POINTER(C.c_void_p), C.POINTER(A16WeightDesc), C.c_void_p, C.c_void_p,
+                                           C.c_void_p, C.c_void_p]
+        L.mi_a16_weight_destroy.argtypes = [C.c_void_p]
+        L.mi_a16_weight_destroy.restype = None
+        L.mi_a16mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi_a16mm_init.argtypes = [C.POINTER(A16Attr), C.POINTER(InferParam)]
+        L.mi_a16mm_inference.argtypes = [C.POINTER(A16Attr), C.POINTER(InferParam)]
+        L.mi_a16mm_deinit.argtypes = [C.POINTER(InferParam)]
+        L.mi_a16mm_deinit.restype = None
+        L.mi_i8mm_init.argtypes = [C.POINTER(I8Attr), C.POINTER(InferParam)]
+        L.mi_i8mm_inference.argtypes = [C.POINTER(I8Attr), C.POINTER(InferParam)]
+        L.mi_i8mm_deinit.argtypes = [C.POINTER(InferParam)]
+        L.mi_i8mm_deinit.restype = None
+        L.mi_i8mm_launch.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int64,
+                                     C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int64,
+                                     C.POINTER(RequantDescC), C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi_requant_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
+                                        C.POINTER(RequantDescC), C.c_void_p]
+        L.mi_requant_int_axis_inference.argtypes = [C.POINTER(RqAxisAttr), C.POINTER(InferParam)]
+        L.mi_requant_int_inference.argtypes = [C.POINTER(RqAttr), C.POINTER(InferParam)]
+        _lib = L
+    return _lib
+
+
+def version():
+    return lib().mi_version().decode()
+
+
+def last_error():
+    return lib().mi_last_error().decode()
+
+
+def device_count():
+    return lib().mi_device_count()
+
+
+def check(rc):
+    if rc != MI_SUCCESS:
+        raise BackendError(rc, last_error())

@@ -1,0 +1,706 @@
+// C ABI of libtpumlir_amd.so: operator-level entry points (float-expanded host operands, as the reference
+// interpreter hands them over) and device-level launches.  See include/tpumlir_amd.h for the contract.
+#include <math.h>
+#include <string.h>
+
+#include <algorithm>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "internal.h"
+
+namespace mi {
+
+static thread_local std::string g_last_error;
+
+void set_error(const std::string &msg) { g_last_error = msg; }
+
+int hip_fail(hipError_t e, const char *what, const char *file, int line) {
+  g_last_error = std::string("HIP error ") + hipGetErrorName(e) + " (" + hipGetErrorString(e) + ") in " + what +
+                 " at " + file + ":" + std::to_string(line);
+  (void)hipGetLastError();  // clear the sticky error so that the next call reports its own
+  return MI_HIP_ERROR;
+}
+
+static inline uint32_t fbits(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return u;
+}
+static inline float bits_f(uint32_t u) {
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+// host-side f32 <-> 16-bit conversions used only to stage interpreter tensors (values that already are
+// bf16/f16 numbers convert exactly; anything else is rounded to nearest even)
+static inline uint16_t h_f32_to_bf16(float f) {
+  uint32_t u = fbits(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u)
+    return 0x7fff;
+  return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+static inline float h_bf16_to_f32(uint16_t h) { return bits_f((uint32_t)h << 16); }
+static inline uint16_t h_f32_to_f16(float f) {
+  _Float16 h = (_Float16)f;
+  uint16_t b;
+  memcpy(&b, &h, 2);
+  return (f != f) ? (uint16_t)0x7fff : b;
+}
+static inline float h_f16_to_f32(uint16_t b) {
+  _Float16 h;
+  memcpy(&h, &b, 2);
+  return (float)h;
+}
+
+// pinned host staging buffer that only grows
+struct Pinned {
+  void *ptr = nullptr;
+  size_t cap = 0;
+  int reserve(size_t bytes) {
+    if (bytes <= cap)
+      return MI_SUCCESS;
+    if (ptr)
+      (void)hipHostFree(ptr);
+    ptr = nullptr;
+    cap = 0;
+    MI_HIP(hipHostMalloc(&ptr, bytes, hipHostMallocDefault));
+    cap = bytes;
+    return MI_SUCCESS;
+  }
+  ~Pinned() {
+    if (ptr)
+      (void)hipHostFree(ptr);
+  }
+};
+
+struct DevBuf {
+  void *ptr = nullptr;
+  size_t cap = 0;
+  int reserve(size_t bytes) {
+    if (bytes <= cap)
+      return MI_SUCCESS;
+    if (ptr)
+      (void)hipFree(ptr);
+    ptr = nullptr;
+    cap = 0;
+    MI_HIP(hipMalloc(&ptr, bytes));
+    cap = bytes;
+    return MI_SUCCESS;
+  }
+  ~DevBuf() {
+    if (ptr)
+      (void)hipFree(ptr);
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// tpu.A16MatMul operator state
+// ---------------------------------------------------------------------------------------------
+struct A16Handle {
+  uint32_t magic = 0xA16A16u;
+  mi_a16_weight *w = nullptr;
+  Pinned h_x, h_y;
+  DevBuf d_x, d_y;
+  hipStream_t stream = nullptr;
+  ~A16Handle() {
+    if (w) {
+      a16_free(w);
+      delete w;
+    }
+    if (stream)
+      (void)hipStreamDestroy(stream);
+  }
+};
+
+static bool group_size_supported(int bits, int g, int64_t K) {
+  if (g == 0)
+    return true;
+  if (g < 0 || K % g != 0)
+    return false;
+  if (bits == 4)
+    return g == 32 || g == 64 || (g % W4_TILE_K) == 0;
+  return g == 32 || (g % W8_TILE_K) == 0;
+}
+
+}  // namespace mi
+
+using namespace mi;
+
+extern "C" {
+
+const char *mi_version(void) { return "tpumlir_amd 0.1 (gfx950)"; }
+const char *mi_last_error(void) { return g_last_error.c_str(); }
+
+int mi_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n;
+}
+
+// ---------------------------------------------------------------------------------------------
+// device level: A16 weights
+// ---------------------------------------------------------------------------------------------
+int mi_a16_weight_create(mi_a16_weight **out, const mi_a16_weight_desc *d, const void *weight,
+                         const uint16_t *scale, const uint8_t *zp, const float *bias) {
+  MI_REQUIRE(out && d && weight && scale && zp, MI_BAD_ARGUMENT, "mi_a16_weight_create: null argument");
+  *out = nullptr;
+  MI_REQUIRE(d->weight_bits == 4 || d->weight_bits == 8, MI_UNSUPPORTED,
+             "mi_a16_weight_create: weight_bits must be 4 or 8");
+  MI_REQUIRE(d->dtype == MI_DT_BF16 || d->dtype == MI_DT_F16, MI_UNSUPPORTED,
+             "mi_a16_weight_create: dtype must be bf16 or f16");
+  MI_REQUIRE(d->K > 0 && d->N > 0, MI_BAD_ARGUMENT, "mi_a16_weight_create: bad shape");
+  MI_REQUIRE(d->K % 8 == 0, MI_UNSUPPORTED, "mi_a16_weight_create: K must be a multiple of 8");
+  MI_REQUIRE(d->q_group_size == 0 || (d->q_group_size > 0 && d->K % d->q_group_size == 0), MI_BAD_ARGUMENT,
+             "mi_a16_weight_create: K is not a multiple of q_group_size");
+  MI_REQUIRE(group_size_supported(d->weight_bits, d->q_group_size, d->K), MI_UNSUPPORTED,
+             "mi_a16_weight_create: group size not handled (4-bit: 32, 64 or a multiple of 128; 8-bit: 32 or a "
+             "multiple of 64)");
+  MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_a16_weight_create: no GPU visible");
+  mi_a16_weight *w = new (std::nothrow) mi_a16_weight();
+  MI_REQUIRE(w, MI_HIP_ERROR, "mi_a16_weight_create: out of host memory");
+  w->K = d->K;
+  w->N = d->N;
+  w->bits = d->weight_bits;
+  w->g = d->q_group_size;
+  w->G = d->q_group_size ? (int)(d->K / d->q_group_size) : 1;
+  w->dtype = d->dtype;
+  w->chip = d->chip;
+  int rc = a16_pack(w, weight, d->weight_signed, scale, zp, bias);
+  if (rc != MI_SUCCESS) {
+    delete w;
+    return rc;
+  }
+  *out = w;
+  return MI_SUCCESS;
+}
+
+void mi_a16_weight_destroy(mi_a16_weight *w) {
+  if (!w)
+    return;
+  a16_free(w);
+  delete w;
+}
+
+size_t mi_a16_weight_bytes(const mi_a16_weight *w) { return w ? w->bytes : 0; }
+
+int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
+                    void *stream) {
+  return a16_launch(w, d_x, M, d_y, d_y_f32, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// operator level: tpu.A16MatMul
+// ---------------------------------------------------------------------------------------------
+int mi_a16mm_init(const mi_a16mm_attr *attr, mi_infer_param *p) {
+  MI_REQUIRE(attr && p, MI_BAD_ARGUMENT, "mi_a16mm_init: null argument");
+  p->handle = nullptr;
+  MI_REQUIRE(p->inputs && p->n_inputs >= 4, MI_BAD_ARGUMENT, "mi_a16mm_init: expects input, weight, scale, zp[, bias]");
+  MI_REQUIRE(!attr->dynamic_quant, MI_UNSUPPORTED, "mi_a16mm_init: dynamic activation quantization is not handled");
+  MI_REQUIRE(attr->w_transpose, MI_UNSUPPORTED, "mi_a16mm_init: only w_transpose weights ([N,K]) are handled");
+  MI_REQUIRE(attr->weight_bits == 4 || attr->weight_bits == 8, MI_UNSUPPORTED, "mi_a16mm_init: weight_bits");
+  MI_REQUIRE(attr->out_dtype == MI_DT_BF16 || attr->out_dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_a16mm_init: out_dtype");
+  const float *weight = p->inputs[1], *scale = p->inputs[2], *zp = p->inputs[3];
+  const float *bias = p->n_inputs > 4 ? p->inputs[4] : nullptr;
+  MI_REQUIRE(weight && scale && zp, MI_BAD_ARGUMENT, "mi_a16mm_init: weight, scale and zp must not be None");
+  const int64_t K = attr->K, N = attr->N;
+  MI_REQUIRE(K > 0 && N > 0, MI_BAD_ARGUMENT, "mi_a16mm_init: bad shape");
+  const int g = attr->q_group_size;
+  MI_REQUIRE(g == 0 || (g > 0 && K % g == 0), MI_BAD_ARGUMENT, "mi_a16mm_init: K is not a multiple of q_group_size");
+  MI_REQUIRE(K % 8 == 0 && group_size_supported(attr->weight_bits, g, K), MI_UNSUPPORTED,
+             "mi_a16mm_init: shape / group size not handled");
+  const int64_t G = g ? K / g : 1;
+
+  // float-expanded operands -> native storage
+  const int64_t nw = attr->weight_bits == 4 ? N * (K / 2) : N * K;
+  std::vector<uint8_t> wbytes((size_t)nw);
+  bool neg = false;
+  for (int64_t i = 0; i < nw; ++i) {
+    float v = weight[i];
+    MI_REQUIRE(v == truncf(v) && v >= -128.f && v <= 255.f, MI_UNSUPPORTED, "mi_a16mm_init: weight is not 8-bit integer valued");
+    neg |= v < 0.f;
+    wbytes[(size_t)i] = (uint8_t)(int)v;
+  }
+  MI_REQUIRE(!(neg && attr->weight_bits == 4), MI_UNSUPPORTED, "mi_a16mm_init: negative packed byte");
+  if (neg)
+    for (int64_t i = 0; i < nw; ++i)
+      MI_REQUIRE(weight[i] <= 127.f, MI_UNSUPPORTED, "mi_a16mm_init: weight mixes int8 and uint8 ranges");
+  std::vector<uint16_t> sbits((size_t)(N * G));
+  std::vector<uint8_t> zbytes((size_t)(N * G));
+  for (int64_t i = 0; i < N * G; ++i) {
+    float s = scale[i];
+    uint16_t b = attr->out_dtype == MI_DT_F16 ? h_f32_to_f16(s) : h_f32_to_bf16(s);
+    float back = attr->out_dtype == MI_DT_F16 ? h_f16_to_f32(b) : h_bf16_to_f32(b);
+    MI_REQUIRE(back == s, MI_UNSUPPORTED, "mi_a16mm_init: scale is not representable in the 16-bit activation type");
+    sbits[(size_t)i] = b;
+    float z = zp[i];
+    MI_REQUIRE(z == truncf(z) && z >= 0.f && z <= 255.f, MI_UNSUPPORTED, "mi_a16mm_init: zero point is not a u8 value");
+    zbytes[(size_t)i] = (uint8_t)(int)z;
+  }
+  mi_a16_weight_desc d;
+  d.K = K;
+  d.N = N;
+  d.weight_bits = attr->weight_bits;
+  d.weight_signed = neg ? 1 : 0;
+  d.q_group_size = g;
+  d.dtype = attr->out_dtype;
+  d.chip = attr->chip;
+  A16Handle *h = new (std::nothrow) A16Handle();
+  MI_REQUIRE(h, MI_HIP_ERROR, "mi_a16mm_init: out of host memory");
+  int rc = mi_a16_weight_create(&h->w, &d, wbytes.data(), sbits.data(), zbytes.data(), bias);
+  if (rc == MI_SUCCESS) {
+    hipError_t e = hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking);
+    if (e != hipSuccess)
+      rc = hip_fail(e, "hipStreamCreateWithFlags", __FILE__, __LINE__);
+  }
+  if (rc != MI_SUCCESS) {
+    delete h;
+    return rc;
+  }
+  p->handle = h;
+  return MI_SUCCESS;
+}
+
+int mi_a16mm_inference(const mi_a16mm_attr *attr, mi_infer_param *p) {
+  MI_REQUIRE(attr && p, MI_BAD_ARGUMENT, "mi_a16mm_inference: null argument");
+  MI_REQUIRE(p->handle, MI_BAD_ARGUMENT, "mi_a16mm_inference: init has not been called");
+  A16Handle *h = (A16Handle *)p->handle;
+  MI_REQUIRE(h->magic == 0xA16A16u, MI_BAD_ARGUMENT, "mi_a16mm_inference: handle does not belong to an A16MatMul");
+  MI_REQUIRE(p->inputs && p->n_inputs >= 1 && p->inputs[0] && p->outputs && p->n_outputs >= 1 && p->outputs[0],
+             MI_BAD_ARGUMENT, "mi_a16mm_inference: null input or output");
+  MI_REQUIRE(attr->K == h->w->K && attr->N == h->w->N, MI_BAD_ARGUMENT, "mi_a16mm_inference: K/N differ from init");
+  const int64_t M = attr->M, K = attr->K, N = attr->N;
+  MI_REQUIRE(M >= 0, MI_BAD_ARGUMENT, "mi_a16mm_inference: negative M");
+  if (M == 0)
+    return MI_SUCCESS;
+  int rc;
+  if ((rc = h->h_x.reserve((size_t)M * K * 2)) || (rc = h->h_y.reserve((size_t)M * N * 2)) ||
+      (rc = h->d_x.reserve((size_t)M * K * 2)) || (rc = h->d_y.reserve((size_t)M * N * 2)))
+    return rc;
+  const float *x = p->inputs[0];
+  uint16_t *hx = (uint16_t *)h->h_x.ptr;
+  const bool f16 = h->w->dtype == MI_DT_F16;
+  for (int64_t i = 0; i < M * K; ++i)
+    hx[i] = f16 ? h_f32_to_f16(x[i]) : h_f32_to_bf16(x[i]);
+  MI_HIP(hipMemcpyAsync(h->d_x.ptr, hx, (size_t)M * K * 2, hipMemcpyHostToDevice, h->stream));
+  rc = a16_launch(h->w, (const uint16_t *)h->d_x.ptr, M, (uint16_t *)h->d_y.ptr, nullptr, h->stream);
+  if (rc != MI_SUCCESS)
+    return rc;
+  MI_HIP(hipMemcpyAsync(h->h_y.ptr, h->d_y.ptr, (size_t)M * N * 2, hipMemcpyDeviceToHost, h->stream));
+  MI_HIP(hipStreamSynchronize(h->stream));
+  const uint16_t *hy = (const uint16_t *)h->h_y.ptr;
+  float *y = p->outputs[0];
+  for (int64_t i = 0; i < M * N; ++i)
+    y[i] = f16 ? h_f16_to_f32(hy[i]) : h_bf16_to_f32(hy[i]);
+  return MI_SUCCESS;
+}
+
+void mi_a16mm_deinit(mi_infer_param *p) {
+  if (!p || !p->handle)
+    return;
+  A16Handle *h = (A16Handle *)p->handle;
+  if (h->magic == 0xA16A16u)
+    delete h;
+  p->handle = nullptr;
+}
+
+// ---------------------------------------------------------------------------------------------
+// device level: int8 matmul / requant
+// ---------------------------------------------------------------------------------------------
+int mi_i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned, int right_transpose,
+                   const int32_t *d_bias, int64_t M, int64_t K, int64_t N, int64_t input_zp, int64_t right_zp,
+                   int do_relu, int64_t relu_limit, const mi_requant_desc *rq, void *d_out, int32_t *d_acc,
+                   void *stream) {
+  return i8mm_launch(d_a, a_unsigned, d_b, b_unsigned, right_transpose, d_bias, M, K, N, input_zp, right_zp, do_relu,
+                     relu_limit, rq, d_out, d_acc, (hipStream_t)stream);
+}
+
+int mi_requant_launch(const int32_t *d_in, void *d_out, int64_t outer, int64_t channels, int64_t inner,
+                      int64_t input_zp, const mi_requant_desc *rq, void *stream) {
+  return requant_launch(d_in, d_out, outer, channels, inner, input_zp, rq, (hipStream_t)stream);
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------------------------
+// operator level: tpu.MatMul (quantized)
+// ---------------------------------------------------------------------------------------------
+namespace mi {
+
+struct I8Handle {
+  uint32_t magic = 0x18181818u;
+  int64_t K = 0, N = 0;
+  bool right_cached = false;
+  int right_unsigned = 0;
+  DevBuf d_a, d_b, d_bias, d_multi, d_out;
+  Pinned h_a, h_b, h_out;
+  bool has_bias = false, has_multi = false;
+  hipStream_t stream = nullptr;
+  ~I8Handle() {
+    if (stream)
+      (void)hipStreamDestroy(stream);
+  }
+};
+
+static int out_elem_size(int dt) {
+  switch (dt) {
+  case MI_DT_I8:
+  case MI_DT_U8:
+    return 1;
+  case MI_DT_I16:
+  case MI_DT_U16:
+    return 2;
+  default:
+    return 4;
+  }
+}
+
+// float-expanded 8-bit integers -> bytes; reports whether they are int8 or uint8 valued
+static int floats_to_bytes(const float *src, int64_t n, uint8_t *dst, int *is_unsigned, const char *who) {
+  float lo = 0.f, hi = 0.f;
+  for (int64_t i = 0; i < n; ++i) {
+    float v = src[i];
+    lo = v < lo ? v : lo;
+    hi = v > hi ? v : hi;
+    dst[i] = (uint8_t)(int)v;
+  }
+  MI_REQUIRE(lo >= -128.f && hi <= 255.f && !(lo < 0.f && hi > 127.f), MI_UNSUPPORTED,
+             std::string(who) + ": operand does not fit an 8-bit integer type");
+  *is_unsigned = hi > 127.f;
+  return MI_SUCCESS;
+}
+
+static int floats_to_i32_dev(const float *src, int64_t n, DevBuf &buf, hipStream_t st) {
+  std::vector<int32_t> tmp((size_t)n);
+  for (int64_t i = 0; i < n; ++i)
+    tmp[(size_t)i] = (int32_t)(int64_t)src[i];
+  int rc = buf.reserve((size_t)n * 4);
+  if (rc)
+    return rc;
+  MI_HIP(hipMemcpyAsync(buf.ptr, tmp.data(), (size_t)n * 4, hipMemcpyHostToDevice, st));
+  MI_HIP(hipStreamSynchronize(st));
+  return MI_SUCCESS;
+}
+
+static int upload_right(I8Handle *h, const mi_i8mm_attr *attr, const float *right) {
+  const int64_t n = attr->K * attr->N;
+  int rc = h->h_b.reserve((size_t)n);
+  if (rc)
+    return rc;
+  if ((rc = floats_to_bytes(right, n, (uint8_t *)h->h_b.ptr, &h->right_unsigned, "mi_i8mm")))
+    return rc;
+  if ((rc = h->d_b.reserve((size_t)n)))
+    return rc;
+  MI_HIP(hipMemcpyAsync(h->d_b.ptr, h->h_b.ptr, (size_t)n, hipMemcpyHostToDevice, h->stream));
+  return MI_SUCCESS;
+}
+
+static int check_i8_attr(const mi_i8mm_attr *a, const char *who) {
+  MI_REQUIRE(a->M >= 0 && a->K > 0 && a->N > 0, MI_BAD_ARGUMENT, std::string(who) + ": bad shape");
+  const int o = a->out_dtype;
+  MI_REQUIRE(o == MI_DT_I8 || o == MI_DT_U8 || o == MI_DT_I16 || o == MI_DT_U16 || o == MI_DT_I32, MI_UNSUPPORTED,
+             std::string(who) + ": output type not handled");
+  if (o != MI_DT_I32) {
+    const int q = a->quant_mode;
+    if (a->chip == MI_CHIP_CV18XX)
+      MI_REQUIRE(q == MI_RQ_MULTIPLIER_SHIFT || q == MI_RQ_ONLY_SHIFT || q == MI_RQ_QDM || q == MI_RQ_TFLITE ||
+                     q == MI_RQ_TFLITE_LSHIFT,
+                 MI_UNSUPPORTED, std::string(who) + ": requant mode not handled");
+    else
+      MI_REQUIRE(q == MI_RQ_MULTIPLIER_SHIFT || q == MI_RQ_TFLITE || q == MI_RQ_TFLITE_LSHIFT, MI_UNSUPPORTED,
+                 std::string(who) + ": requant mode not handled");
+    MI_REQUIRE(a->multipliers && a->n_multipliers >= 1 && a->rshifts && a->n_rshifts >= 1, MI_BAD_ARGUMENT,
+               std::string(who) + ": multipliers / rshifts missing");
+  }
+  return MI_SUCCESS;
+}
+
+}  // namespace mi
+
+extern "C" {
+
+int mi_i8mm_init(const mi_i8mm_attr *attr, mi_infer_param *p) {
+  MI_REQUIRE(attr && p, MI_BAD_ARGUMENT, "mi_i8mm_init: null argument");
+  p->handle = nullptr;
+  MI_REQUIRE(p->inputs && p->n_inputs >= 2 && p->inputs[0] && p->inputs[1], MI_BAD_ARGUMENT,
+             "mi_i8mm_init: input and right must not be None");
+  int rc = check_i8_attr(attr, "mi_i8mm_init");
+  if (rc)
+    return rc;
+  MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_i8mm_init: no GPU visible");
+  I8Handle *h = new (std::nothrow) I8Handle();
+  MI_REQUIRE(h, MI_HIP_ERROR, "mi_i8mm_init: out of host memory");
+  h->K = attr->K;
+  h->N = attr->N;
+  hipError_t e = hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    delete h;
+    return hip_fail(e, "hipStreamCreateWithFlags", __FILE__, __LINE__);
+  }
+  const float *bias = p->n_inputs > 2 ? p->inputs[2] : nullptr;
+  const float *multi = p->n_inputs > 3 ? p->inputs[3] : nullptr;
+  if (attr->right_is_weight) {
+    rc = upload_right(h, attr, p->inputs[1]);
+    h->right_cached = rc == MI_SUCCESS;
+  }
+  if (rc == MI_SUCCESS && bias) {
+    rc = floats_to_i32_dev(bias, attr->N, h->d_bias, h->stream);
+    h->has_bias = rc == MI_SUCCESS;
+  }
+  if (rc == MI_SUCCESS && multi && attr->fuse_rq) {
+    rc = floats_to_i32_dev(multi, attr->N, h->d_multi, h->stream);
+    h->has_multi = rc == MI_SUCCESS;
+  }
+  if (rc == MI_SUCCESS) {
+    e = hipStreamSynchronize(h->stream);
+    if (e != hipSuccess)
+      rc = hip_fail(e, "hipStreamSynchronize", __FILE__, __LINE__);
+  }
+  if (rc != MI_SUCCESS) {
+    delete h;
+    return rc;
+  }
+  p->handle = h;
+  return MI_SUCCESS;
+}
+
+int mi_i8mm_inference(const mi_i8mm_attr *attr, mi_infer_param *p) {
+  MI_REQUIRE(attr && p, MI_BAD_ARGUMENT, "mi_i8mm_inference: null argument");
+  if (!p->handle) {  // the reference initialises lazily (MatMul.cpp:441-443)
+    int rc0 = mi_i8mm_init(attr, p);
+    if (rc0)
+      return rc0;
+  }
+  I8Handle *h = (I8Handle *)p->handle;
+  MI_REQUIRE(h->magic == 0x18181818u, MI_BAD_ARGUMENT, "mi_i8mm_inference: handle does not belong to a MatMul");
+  MI_REQUIRE(p->inputs && p->n_inputs >= 2 && p->inputs[0] && p->inputs[1] && p->outputs && p->n_outputs >= 1 &&
+                 p->outputs[0],
+             MI_BAD_ARGUMENT, "mi_i8mm_inference: null input or output");
+  int rc = check_i8_attr(attr, "mi_i8mm_inference");
+  if (rc)
+    return rc;
+  MI_REQUIRE(attr->K == h->K && attr->N == h->N, MI_BAD_ARGUMENT, "mi_i8mm_inference: K/N differ from init");
+  const int64_t M = attr->M, K = attr->K, N = attr->N;
+  if (M == 0)
+    return MI_SUCCESS;
+  const int osz = out_elem_size(attr->out_dtype);
+  if ((rc = h->h_a.reserve((size_t)M * K)) || (rc = h->d_a.reserve((size_t)M * K)) ||
+      (rc = h->h_out.reserve((size_t)M * N * osz)) || (rc = h->d_out.reserve((size_t)M * N * osz)))
+    return rc;
+  int a_unsigned = 0;
+  if ((rc = floats_to_bytes(p->inputs[0], M * K, (uint8_t *)h->h_a.ptr, &a_unsigned, "mi_i8mm_inference")))
+    return rc;
+  MI_HIP(hipMemcpyAsync(h->d_a.ptr, h->h_a.ptr, (size_t)M * K, hipMemcpyHostToDevice, h->stream));
+  if (!h->right_cached && (rc = upload_right(h, attr, p->inputs[1])))
+    return rc;
+  const float *bias = p->n_inputs > 2 ? p->inputs[2] : nullptr;
+  const float *multi = p->n_inputs > 3 ? p->inputs[3] : nullptr;
+  if (bias && !h->has_bias) {
+    if ((rc = floats_to_i32_dev(bias, N, h->d_bias, h->stream)))
+      return rc;
+    h->has_bias = attr->right_is_weight;  // weights' bias is constant; otherwise re-upload each call
+  }
+  mi_requant_desc rq;
+  memset(&rq, 0, sizeof(rq));
+  const mi_requant_desc *rqp = nullptr;
+  if (attr->out_dtype != MI_DT_I32) {
+    rqp = &rq;
+    rq.chip = attr->chip;
+    rq.out_dtype = attr->out_dtype;
+    rq.quant_mode = attr->quant_mode;
+    rq.multiplier = (int32_t)attr->multipliers[0];
+    rq.shift = (int32_t)attr->rshifts[0];
+    if (attr->chip == MI_CHIP_CV18XX) {
+      // MatMul.cpp:638-664: per-batch (here: one) multiplier/rshift, half away from zero, no zero point
+      rq.round_mode = MI_ROUND_HALF_AWAY_FROM_ZERO;
+      rq.zp = 0;
+    } else if (attr->quant_mode == MI_RQ_MULTIPLIER_SHIFT) {
+      // MatMul.cpp:708-726: default rounding of applyMultiplierAndRShift is half up (MathUtils.h:178-181)
+      rq.round_mode = MI_ROUND_HALF_UP;
+      rq.zp = (int32_t)attr->out_zp;
+      if (attr->fuse_rq) {
+        MI_REQUIRE(multi, MI_BAD_ARGUMENT, "mi_i8mm_inference: fuse_rq needs the multi operand");
+        if (!h->has_multi) {
+          if ((rc = floats_to_i32_dev(multi, N, h->d_multi, h->stream)))
+            return rc;
+          h->has_multi = attr->right_is_weight;
+        }
+        rq.d_multiplier = (const int32_t *)h->d_multi.ptr;
+      }
+    } else {
+      // MatMul.cpp:696-707: MultiplyByQuantizedMultiplier(acc, mult, -rshift), half away from zero
+      rq.round_mode = MI_ROUND_HALF_AWAY_FROM_ZERO;
+      rq.zp = (int32_t)attr->out_zp;
+    }
+  }
+  const int64_t relu_limit = attr->relu_limit > 0.0 ? (int64_t)floor(attr->relu_limit) : -1;
+  rc = i8mm_launch(h->d_a.ptr, a_unsigned, h->d_b.ptr, h->right_unsigned, attr->right_transpose,
+                   bias ? (const int32_t *)h->d_bias.ptr : nullptr, M, K, N, attr->input_zp, attr->right_zp,
+                   attr->do_relu, relu_limit, rqp, h->d_out.ptr, nullptr, h->stream);
+  if (rc)
+    return rc;
+  MI_HIP(hipMemcpyAsync(h->h_out.ptr, h->d_out.ptr, (size_t)M * N * osz, hipMemcpyDeviceToHost, h->stream));
+  MI_HIP(hipStreamSynchronize(h->stream));
+  float *y = p->outputs[0];
+  const void *ho = h->h_out.ptr;
+  switch (attr->out_dtype) {
+  case MI_DT_I8:
+    for (int64_t i = 0; i < M * N; ++i) y[i] = (float)((const int8_t *)ho)[i];
+    break;
+  case MI_DT_U8:
+    for (int64_t i = 0; i < M * N; ++i) y[i] = (float)((const uint8_t *)ho)[i];
+    break;
+  case MI_DT_I16:
+    for (int64_t i = 0; i < M * N; ++i) y[i] = (float)((const int16_t *)ho)[i];
+    break;
+  case MI_DT_U16:
+    for (int64_t i = 0; i < M * N; ++i) y[i] = (float)((const uint16_t *)ho)[i];
+    break;
+  default:
+    for (int64_t i = 0; i < M * N; ++i) y[i] = (float)((const int32_t *)ho)[i];
+    break;
+  }
+  return MI_SUCCESS;
+}
+
+void mi_i8mm_deinit(mi_infer_param *p) {
+  if (!p || !p->handle)
+    return;
+  I8Handle *h = (I8Handle *)p->handle;
+  if (h->magic == 0x18181818u)
+    delete h;
+  p->handle = nullptr;
+}
+
+// ---------------------------------------------------------------------------------------------
+// operator level: tpu.RequantIntAxis / tpu.RequantInt
+// ---------------------------------------------------------------------------------------------
+static int run_requant_host(const float *in, float *out, int64_t outer, int64_t channels, int64_t inner,
+                            int64_t input_zp, mi_requant_desc rq, const std::vector<int32_t> *mult,
+                            const std::vector<int32_t> *shift, const std::vector<int32_t> *zp) {
+  MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "requant: no GPU visible");
+  const int64_t total = outer * channels * inner;
+  const int osz = out_elem_size(rq.out_dtype);
+  std::vector<int32_t> hin((size_t)total);
+  for (int64_t i = 0; i < total; ++i)
+    hin[(size_t)i] = (int32_t)(int64_t)in[i];
+  DevBuf d_in, d_out, d_m, d_s, d_z;
+  int rc;
+  if ((rc = d_in.reserve((size_t)total * 4)) || (rc = d_out.reserve((size_t)total * osz)))
+    return rc;
+  MI_HIP(hipMemcpy(d_in.ptr, hin.data(), (size_t)total * 4, hipMemcpyHostToDevice));
+  if (mult) {
+    if ((rc = d_m.reserve(mult->size() * 4)) || (rc = d_s.reserve(shift->size() * 4)) ||
+        (rc = d_z.reserve(zp->size() * 4)))
+      return rc;
+    MI_HIP(hipMemcpy(d_m.ptr, mult->data(), mult->size() * 4, hipMemcpyHostToDevice));
+    MI_HIP(hipMemcpy(d_s.ptr, shift->data(), shift->size() * 4, hipMemcpyHostToDevice));
+    MI_HIP(hipMemcpy(d_z.ptr, zp->data(), zp->size() * 4, hipMemcpyHostToDevice));
+    rq.d_multiplier = (const int32_t *)d_m.ptr;
+    rq.d_shift = (const int32_t *)d_s.ptr;
+    rq.d_zp = (const int32_t *)d_z.ptr;
+  }
+  if ((rc = requant_launch((const int32_t *)d_in.ptr, d_out.ptr, outer, channels, inner, input_zp, &rq, nullptr)))
+    return rc;
+  std::vector<uint8_t> hout((size_t)total * osz);
+  MI_HIP(hipMemcpy(hout.data(), d_out.ptr, hout.size(), hipMemcpyDeviceToHost));
+  for (int64_t i = 0; i < total; ++i) {
+    switch (rq.out_dtype) {
+    case MI_DT_I8: out[i] = (float)((const int8_t *)hout.data())[i]; break;
+    case MI_DT_U8: out[i] = (float)((const uint8_t *)hout.data())[i]; break;
+    case MI_DT_I16: out[i] = (float)((const int16_t *)hout.data())[i]; break;
+    case MI_DT_U16: out[i] = (float)((const uint16_t *)hout.data())[i]; break;
+    default: out[i] = (float)((const int32_t *)hout.data())[i]; break;
+    }
+  }
+  return MI_SUCCESS;
+}
+
+int mi_requant_int_axis_inference(const mi_rq_axis_attr *a, mi_infer_param *p) {
+  MI_REQUIRE(a && p && p->inputs && p->n_inputs >= 2 && p->inputs[0] && p->inputs[1] && p->outputs &&
+                 p->n_outputs >= 1 && p->outputs[0],
+             MI_BAD_ARGUMENT, "mi_requant_int_axis_inference: null argument");
+  MI_REQUIRE(a->rank >= 2 && a->rank <= 8, MI_BAD_ARGUMENT, "mi_requant_int_axis_inference: bad rank");
+  const int q = a->quant_mode;
+  MI_REQUIRE(q == MI_RQ_TFLITE || q == MI_RQ_TFLITE_LSHIFT || q == MI_RQ_MULTIPLIER_SHIFT, MI_UNSUPPORTED,
+             "mi_requant_int_axis_inference: requant mode not handled");
+  const bool tflite = q != MI_RQ_MULTIPLIER_SHIFT;
+  const bool last_axis = !tflite && a->fuse_rq_axis;
+  int64_t outer, channels, inner;
+  if (last_axis) {  // RequantIntAxis.cpp:68-91
+    channels = a->shape[a->rank - 1];
+    inner = 1;
+    outer = 1;
+    for (int i = 0; i < a->rank - 1; ++i)
+      outer *= a->shape[i];
+  } else {  // :41-66, :93-118: channel = dim 1
+    outer = a->shape[0];
+    channels = a->shape[1];
+    inner = 1;
+    for (int i = 2; i < a->rank; ++i)
+      inner *= a->shape[i];
+  }
+  const float *quant = p->inputs[1];
+  std::vector<int32_t> mult((size_t)channels), shift((size_t)channels), zp((size_t)channels);
+  for (int64_t c = 0; c < channels; ++c) {
+    int64_t m, s, z;
+    if (a->quant_triples) {
+      m = (int64_t)quant[c * 3];
+      s = (int64_t)quant[c * 3 + 1];
+      z = (int64_t)quant[c * 3 + 2];
+    } else {  // :50-55: shift in the low byte, zero point in the high half-word
+      m = (int64_t)quant[c * 2];
+      uint32_t tmp = (uint32_t)quant[c * 2 + 1];
+      s = (int64_t)((signed char)(tmp & 0xff));
+      z = (int64_t)(short)((tmp & 0xffff0000u) >> 16);
+    }
+    // device convention: positive = right shift.  The TFLite branch hands the stored shift to
+    // MultiplyByQuantizedMultiplier (negative = right); the axis-1 MultiplierShift branch negates the stored
+    // value into a right shift; the fused-axis branch uses it as a right shift directly.
+    int64_t rs = (tflite || !last_axis) ? -s : s;
+    mult[(size_t)c] = (int32_t)m;
+    shift[(size_t)c] = (int32_t)rs;
+    zp[(size_t)c] = (int32_t)z;
+  }
+  mi_requant_desc rq;
+  memset(&rq, 0, sizeof(rq));
+  rq.quant_mode = q;
+  rq.round_mode = a->round_mode;
+  rq.chip = a->chip;
+  rq.out_dtype = a->out_dtype;
+  return run_requant_host(p->inputs[0], p->outputs[0], outer, channels, inner, tflite ? 0 : a->input_zp, rq, &mult,
+                          &shift, &zp);
+}
+
+int mi_requant_int_inference(const mi_rq_attr *a, mi_infer_param *p) {
+  MI_REQUIRE(a && p && p->inputs && p->n_inputs >= 1 && p->inputs[0] && p->outputs && p->n_outputs >= 1 &&
+                 p->outputs[0],
+             MI_BAD_ARGUMENT, "mi_requant_int_inference: null argument");
+  MI_REQUIRE(a->rank >= 1 && a->rank <= 8, MI_BAD_ARGUMENT, "mi_requant_int_inference: bad rank");
+  if (a->rank == 1)
+    return MI_SUCCESS;  // RequantInt.cpp:36-38
+  const int q = a->quant_mode;
+  MI_REQUIRE(q == MI_RQ_TFLITE || q == MI_RQ_TFLITE_LSHIFT || q == MI_RQ_MULTIPLIER_SHIFT, MI_UNSUPPORTED,
+             "mi_requant_int_inference: requant mode not handled");
+  int64_t total = 1;
+  for (int i = 0; i < a->rank; ++i)
+    total *= a->shape[i];
+  mi_requant_desc rq;
+  memset(&rq, 0, sizeof(rq));
+  rq.quant_mode = q;
+  rq.round_mode = a->round_mode;
+  rq.chip = a->chip;
+  rq.out_dtype = a->out_dtype;
+  rq.multiplier = (int32_t)a->multiplier;
+  rq.shift = (int32_t)a->rshift;  // both branches shift right by getRshift() (RequantInt.cpp:31,47,62)
+  rq.zp = (int32_t)a->out_zp;
+  return run_requant_host(p->inputs[0], p->outputs[0], 1, 1, total, q == MI_RQ_MULTIPLIER_SHIFT ? a->input_zp : 0, rq,
+                          nullptr, nullptr, nullptr);
+}
+
+}  // extern "C"

@@ -1,0 +1,208 @@
+// Device-side scalar arithmetic shared by the kernels: output rounding to bf16/f16 and the
+// integer requantization rules of the reference interpreter.  Citations are file:line in the
+// reference tree; the arithmetic is written for 64-wide gfx950 waves (branch-light, 32-bit where
+// the value range allows).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/tpumlir_amd.h"
+
+namespace mi {
+
+__device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+__device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+// f32 -> bf16, BM168x flavour (lib/Support/Float16.cpp:603-646,716-720): round to nearest even on
+// normals, NaN -> 0x7fff, infinities kept, zero / fp32 denormals -> signed zero except
+// 0x007f8000..0x007fffff which becomes the smallest normal (:550-601).
+__device__ __forceinline__ uint16_t f32_to_bf16_bm(float f) {
+  uint32_t u = f2u(f);
+  uint32_t exp = (u >> 23) & 0xffu;
+  uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  if (exp == 255u)
+    r = (u & 0x7fffffu) ? 0x7fffu : (u >> 16);
+  else if (exp == 0u)
+    r = ((u >> 16) & 0x8000u) | (((u & 0x7fffffu) >= 0x7f8000u) ? 0x80u : 0u);
+  return (uint16_t)r;
+}
+
+// f32 -> bf16, CV18xx flavour (lib/Support/Float16.cpp:725-761): add 0x7fff + lsb, truncate, and map
+// every all-ones exponent result to 0x7f7f.
+__device__ __forceinline__ uint16_t f32_to_bf16_cvi(float f) {
+  uint32_t u = f2u(f);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  uint32_t h = u >> 16;
+  return (uint16_t)(((h & 0x7f80u) == 0x7f80u) ? 0x7f7fu : h);
+}
+
+// f32 -> f16 (lib/Support/Float16.cpp:664-714,763-767): round to nearest even including the
+// subnormal range, overflow to infinity, NaN -> 0x7fff.
+__device__ __forceinline__ uint16_t f32_to_f16_ref(float f) {
+  if (f != f)
+    return 0x7fffu;
+  _Float16 h = (_Float16)f;  // v_cvt_f16_f32: RNE, subnormals honoured
+  return __builtin_bit_cast(uint16_t, h);
+}
+
+template <int DT, int CHIP>
+__device__ __forceinline__ uint16_t round_out16(float f) {
+  if constexpr (DT == MI_DT_F16)
+    return f32_to_f16_ref(f);
+  else if constexpr (CHIP == MI_CHIP_CV18XX)
+    return f32_to_bf16_cvi(f);
+  else
+    return f32_to_bf16_bm(f);
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+
+// RightShiftRound<int64_t> (lib/Support/MathUtils.cpp:474-514)
+__device__ __forceinline__ int64_t right_shift_round(int64_t src, int shift, int mode) {
+  if (shift == 0)
+    return src;
+  if (shift > 63)
+    shift = 63;
+  if (shift < 0)
+    return (int64_t)((uint64_t)src << (-shift));
+  int64_t val = src >> shift;
+  int64_t mant = src & (int64_t)((1ull << shift) - 1ull);
+  int64_t half = (int64_t)(1ull << (shift - 1));
+  int64_t inc = 0;
+  switch (mode) {
+  case MI_ROUND_HALF_TO_EVEN:
+    inc = (mant > half) | ((mant == half) & (val & 1));
+    break;
+  case MI_ROUND_HALF_AWAY_FROM_ZERO:
+    inc = (src >= 0) ? (mant >= half) : (mant > half);
+    break;
+  case MI_ROUND_TOWARDS_ZERO:
+    inc = (src < 0) & (mant != 0);
+    break;
+  case MI_ROUND_UP:
+    inc = (mant != 0);
+    break;
+  case MI_ROUND_HALF_UP:
+    inc = (mant >= half);
+    break;
+  case MI_ROUND_HALF_DOWN:
+    inc = (mant > half);
+    break;
+  default:  // MI_ROUND_DOWN and unlisted modes: floor
+    break;
+  }
+  return val + inc;
+}
+
+// MultiplyByQuantizedMultiplier (lib/Support/MathUtils.cpp:523-536)
+__device__ __forceinline__ int32_t multiply_by_quantized_multiplier(int32_t x, int32_t multiplier, int shift,
+                                                                    int mode) {
+  int64_t value = shift > 0 ? (int64_t)(int32_t)((uint32_t)x << shift) : (int64_t)x;
+  value = (value * (int64_t)multiplier + (1ll << 30)) >> 31;  // RightShiftRound(., 31, HALF_UP)
+  value = value > 2147483647ll ? 2147483647ll : (value < -2147483648ll ? -2147483648ll : value);
+  if (shift < 0)
+    value = right_shift_round(value, -shift, mode);
+  return (int32_t)value;
+}
+
+// to_int<float> (lib/Support/MathUtils.cpp:179-213)
+__device__ __forceinline__ int64_t to_int_f32(float v, int mode) {
+  switch (mode) {
+  case MI_ROUND_HALF_AWAY_FROM_ZERO:
+    return (int64_t)roundf(v);
+  case MI_ROUND_UP:
+    return (int64_t)ceilf(v);
+  case MI_ROUND_DOWN:
+    return (int64_t)floorf(v);
+  case MI_ROUND_HALF_UP:
+    return (int64_t)floor((double)v + 0.5);
+  case MI_ROUND_HALF_DOWN:
+    return (int64_t)ceil((double)v - 0.5);
+  case MI_ROUND_TOWARDS_ZERO:
+    return (int64_t)v;
+  case MI_ROUND_HALF_TO_EVEN: {
+    float a = fabsf(v);
+    float ip = truncf(a);
+    float fr = a - ip;
+    int64_t r = (int64_t)ip;
+    if (fr > 0.5f || (fr == 0.5f && (r & 1)))
+      r += 1;
+    return v < 0 ? -r : r;
+  }
+  default:
+    return (int64_t)roundf(v);
+  }
+}
+
+// applyMultiplierAndRShift (lib/Support/MathUtils.cpp:538-562).  `shift` follows the reference's
+// argument: for the QDM family on BM168x a negative value is a right shift; on CV18xx it is negated first.
+__device__ __forceinline__ int64_t apply_multiplier_and_rshift(int64_t v, int64_t multiplier, int64_t rshift,
+                                                               int qmode, int rmode, int chip) {
+  switch (qmode) {
+  case MI_RQ_MULTIPLIER_SHIFT:
+    if (chip == MI_CHIP_CV18XX)
+      return to_int_f32(((float)v * (float)multiplier) / (float)(1 << (int)rshift), rmode);
+    return right_shift_round(v * multiplier, (int)rshift, rmode);
+  case MI_RQ_ONLY_SHIFT:
+    return right_shift_round(v, (int)rshift, rmode);
+  case MI_RQ_QDM:
+  case MI_RQ_TFLITE:
+  case MI_RQ_TFLITE_LSHIFT:
+    if (chip == MI_CHIP_CV18XX)
+      rshift = -rshift;
+    return (int64_t)multiply_by_quantized_multiplier((int32_t)v, (int32_t)multiplier, (int)rshift, rmode);
+  default:
+    return 0;
+  }
+}
+
+// saturate<int64_t>(v, IntegerType) (lib/Support/MathUtils.cpp:849-872)
+__device__ __forceinline__ int64_t saturate_to(int64_t v, int out_dtype) {
+  int64_t lo, hi;
+  switch (out_dtype) {
+  case MI_DT_I8: lo = -128; hi = 127; break;
+  case MI_DT_U8: lo = 0; hi = 255; break;
+  case MI_DT_I16: lo = -32768; hi = 32767; break;
+  case MI_DT_U16: lo = 0; hi = 65535; break;
+  default: lo = -2147483648ll; hi = 2147483647ll; break;
+  }
+  return v < lo ? lo : (v > hi ? hi : v);
+}
+
+// Device-side view of mi_requant_desc, passed by value to kernels.
+struct RequantParams {
+  const int32_t *mult;
+  const int32_t *shift;
+  const int32_t *zp;
+  int32_t mult_s, shift_s, zp_s;
+  int qmode, rmode, chip, out_dtype;
+};
+
+// int32 accumulator of channel n -> saturated output value.  The descriptor's shift is a RIGHT shift
+// when positive for every mode (the device-level convention), so the QDM family passes -shift on.
+__device__ __forceinline__ int32_t requant_one(int32_t acc, int64_t n, const RequantParams &rq) {
+  int64_t m = rq.mult ? rq.mult[n] : rq.mult_s;
+  int64_t s = rq.shift ? rq.shift[n] : rq.shift_s;
+  int64_t z = rq.zp ? rq.zp[n] : rq.zp_s;
+  int64_t v;
+  if (rq.qmode == MI_RQ_MULTIPLIER_SHIFT || rq.qmode == MI_RQ_ONLY_SHIFT)
+    v = apply_multiplier_and_rshift(acc, m, s, rq.qmode, rq.rmode, rq.chip);
+  else
+    v = (int64_t)multiply_by_quantized_multiplier(acc, (int32_t)m, (int)-s, rq.rmode);
+  return (int32_t)saturate_to(v + z, rq.out_dtype);
+}
+
+__device__ __forceinline__ void store_out(void *out, int64_t idx, int32_t v, int out_dtype) {
+  switch (out_dtype) {
+  case MI_DT_I8: ((int8_t *)out)[idx] = (int8_t)v; break;
+  case MI_DT_U8: ((uint8_t *)out)[idx] = (uint8_t)v; break;
+  case MI_DT_I16: ((int16_t *)out)[idx] = (int16_t)v; break;
+  case MI_DT_U16: ((uint16_t *)out)[idx] = (uint16_t)v; break;
+  default: ((int32_t *)out)[idx] = v; break;
+  }
+}
+
+}  // namespace mi

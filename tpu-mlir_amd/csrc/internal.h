@@ -1,0 +1,75 @@
+// Internal declarations shared by the translation units of libtpumlir_amd.so (not part of the C ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "../../include/tpumlir_amd.h"
+
+namespace mi {
+
+void set_error(const std::string &msg);
+int hip_fail(hipError_t e, const char *what, const char *file, int line);
+
+#define MI_HIP(expr)                                                        \
+  do {                                                                      \
+    hipError_t _e = (expr);                                                 \
+    if (_e != hipSuccess)                                                   \
+      return ::mi::hip_fail(_e, #expr, __FILE__, __LINE__);                 \
+  } while (0)
+
+#define MI_REQUIRE(cond, code, msg)                                         \
+  do {                                                                      \
+    if (!(cond)) {                                                          \
+      ::mi::set_error(msg);                                                 \
+      return (code);                                                        \
+    }                                                                       \
+  } while (0)
+
+// K extent of one weight tile, in elements.  A tile is 16 output channels x TILE_K weights laid out so that
+// a wave reads it with one fully coalesced 16-byte-per-lane load (1 KiB).
+constexpr int W4_TILE_K = 128;  // 16 rows x 128 nibbles  = 1024 B
+constexpr int W8_TILE_K = 64;   // 16 rows x 64 bytes     = 1024 B
+constexpr int ROW_BLOCK = 16;   // output channels per tile = one MFMA 16x16 column block
+
+}  // namespace mi
+
+// Packed, HBM-resident weight set of one A16MatMul (the opaque type of the C ABI).
+struct mi_a16_weight {
+  int64_t K = 0, N = 0;
+  int bits = 0;        // 4 / 8
+  int g = 0;           // group size as given (0 = per channel)
+  int G = 1;           // groups per row
+  int dtype = MI_DT_BF16;
+  int chip = MI_CHIP_BM168X;
+  int64_t row_blocks = 0;  // ceil(N / 16)
+  int64_t k_tiles = 0;     // ceil(K / TILE_K)
+  // [row_blocks][k_tiles][64 lanes][16 B]
+  void *qweight = nullptr;
+  // [row_blocks][G][16] scale bit patterns (bf16/f16)
+  uint16_t *scale_t = nullptr;
+  // 4-bit: [row_blocks][G][16] zero points (u8).  8-bit: unused.
+  uint8_t *zp_t = nullptr;
+  // 8-bit: [row_blocks][G][16] float, -(zp + bias_of_unsigned_storage) * scale (exact in f32)
+  float *nzs_t = nullptr;
+  float *bias = nullptr;  // [N] or null
+  size_t bytes = 0;
+};
+
+namespace mi {
+int a16_pack(mi_a16_weight *w, const void *h_weight, int weight_signed, const uint16_t *h_scale,
+             const uint8_t *h_zp, const float *h_bias);
+void a16_free(mi_a16_weight *w);
+int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
+               hipStream_t stream);
+
+struct RequantParams;
+int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned, int right_transpose,
+                const int32_t *d_bias, int64_t M, int64_t K, int64_t N, int64_t input_zp, int64_t right_zp,
+                int do_relu, int64_t relu_limit, const mi_requant_desc *rq, void *d_out, int32_t *d_acc,
+                hipStream_t stream);
+int requant_launch(const int32_t *d_in, void *d_out, int64_t outer, int64_t channels, int64_t inner,
+                   int64_t input_zp, const mi_requant_desc *rq, hipStream_t stream);
+}  // namespace mi

@@ -1,0 +1,290 @@
+"""Python mirrors of the backend's two levels.
+
+Operator level (numpy float32 "f32-valued" operands, exactly what the reference interpreter hands to
+`InferenceInterface::init/inference/deinit`): `A16MatMul`, `MatMulInt8`, `requant_int_axis`, `requant_int`.
+
+Device level (torch CUDA tensors used only as device memory + the current HIP stream): `A16Weight`,
+`a16mm_launch`, `i8mm_launch`, `requant_launch`.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import clib
+from .clib import (A16Attr, A16WeightDesc, I8Attr, InferParam, RequantDescC, RqAttr, RqAxisAttr, check,
+                   CHIP_BM168X, DT_BF16, DT_F16, DT_I8, DT_I32, DT_U8, DT_I16, DT_U16,
+                   RQ_MULTIPLIER_SHIFT, ROUND_HALF_AWAY_FROM_ZERO)
+
+_FP = C.POINTER(C.c_float)
+
+
+def _f32(a):
+    return None if a is None else np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _fptr(a):
+    return C.cast(None, _FP) if a is None else a.ctypes.data_as(_FP)
+
+
+class _Param:
+    """Owns the pointer arrays of one mi_infer_param."""
+
+    def __init__(self, inputs, outputs):
+        self.keep = [inputs, outputs]
+        self.in_arr = (_FP * len(inputs))(*[_fptr(a) for a in inputs])
+        self.out_arr = (_FP * len(outputs))(*[_fptr(a) for a in outputs])
+        self.c = InferParam(self.in_arr, len(inputs), self.out_arr, len(outputs), None)
+
+
+# --------------------------------------------------------------------------------------------------
+# operator level
+# --------------------------------------------------------------------------------------------------
+class A16MatMul:
+    """tpu.A16MatMul with the interpreter's calling convention: init once, inference per invoke, deinit."""
+
+    def __init__(self, K, N, weight_bits, q_group_size, w_transpose=True, out_dtype=DT_BF16, chip=CHIP_BM168X,
+                 dynamic_quant=False):
+        self.attr = A16Attr(0, K, N, weight_bits, int(w_transpose), q_group_size, out_dtype, chip, int(dynamic_quant))
+        self.param = None
+
+    def init(self, weight, scale, zp, bias=None):
+        ins = [None, _f32(weight), _f32(scale), _f32(zp), _f32(bias)]
+        self.param = _Param(ins, [None])
+        check(clib.lib().mi_a16mm_init(C.byref(self.attr), C.byref(self.param.c)))
+        return self
+
+    def inference(self, x):
+        if self.param is None:
+            raise clib.BackendError(clib.MI_BAD_ARGUMENT, "A16MatMul.inference before init")
+        x = _f32(x)
+        M = int(np.prod(x.shape[:-1])) if x.ndim > 1 else 1
+        self.attr.M = M
+        y = np.empty(tuple(x.shape[:-1]) + (self.attr.N,), dtype=np.float32)
+        handle = self.param.c.handle
+        ins = list(self.param.keep[0])
+        ins[0] = x
+        p = _Param(ins, [y])
+        p.c.handle = handle
+        check(clib.lib().mi_a16mm_inference(C.byref(self.attr), C.byref(p.c)))
+        return y
+
+    def deinit(self):
+        if self.param is not None:
+            clib.lib().mi_a16mm_deinit(C.byref(self.param.c))
+            self.param = None
+
+    def __del__(self):
+        try:
+            self.deinit()
+        except Exception:
+            pass
+
+
+class MatMulInt8:
+    """Quantized tpu.MatMul (init / inference / deinit)."""
+
+    def __init__(self, K, N, *, right_transpose=False, input_zp=0, right_zp=0, do_relu=False, relu_limit=-1.0,
+                 chip=CHIP_BM168X, quant_mode=RQ_MULTIPLIER_SHIFT, round_mode=ROUND_HALF_AWAY_FROM_ZERO,
+                 fuse_rq=False, multipliers=(1,), rshifts=(0,), out_zp=0, out_dtype=DT_I8, right_is_weight=True):
+        self._mult = np.ascontiguousarray(multipliers, dtype=np.int64)
+        self._rs = np.ascontiguousarray(rshifts, dtype=np.int64)
+        self.attr = I8Attr(0, K, N, int(right_transpose), input_zp, right_zp, int(do_relu), relu_limit, chip,
+                           quant_mode, round_mode, int(fuse_rq),
+                           self._mult.ctypes.data_as(C.POINTER(C.c_int64)), self._mult.size,
+                           self._rs.ctypes.data_as(C.POINTER(C.c_int64)), self._rs.size,
+                           out_zp, out_dtype, int(right_is_weight))
+        self.param = None
+
+    def init(self, x, right, bias=None, multi=None):
+        ins = [_f32(x), _f32(right), _f32(bias), _f32(multi), None]
+        self.attr.M = ins[0].shape[0] if ins[0] is not None and ins[0].ndim == 2 else 0
+        self.param = _Param(ins, [None])
+        check(clib.lib().mi_i8mm_init(C.byref(self.attr), C.byref(self.param.c)))
+        return self
+
+    def inference(self, x, right=None, bias=None, multi=None):
+        x = _f32(x)
+        keep = self.param.keep[0] if self.param is not None else [None] * 5
+        ins = [x, _f32(right) if right is not None else keep[1], _f32(bias) if bias is not None else keep[2],
+               _f32(multi) if multi is not None else keep[3], None]
+        M = int(np.prod(x.shape[:-1]))
+        self.attr.M = M
+        y = np.empty(tuple(x.shape[:-1]) + (self.attr.N,), dtype=np.float32)
+        p = _Param(ins, [y])
+        p.c.handle = self.param.c.handle if self.param is not None else None
+        check(clib.lib().mi_i8mm_inference(C.byref(self.attr), C.byref(p.c)))
+        if self.param is None:  # lazily initialised by the library: keep the handle for deinit
+            self.param = p
+        else:
+            self.param.c.handle = p.c.handle
+        return y
+
+    def deinit(self):
+        if self.param is not None:
+            clib.lib().mi_i8mm_deinit(C.byref(self.param.c))
+            self.param = None
+
+    def __del__(self):
+        try:
+            self.deinit()
+        except Exception:
+            pass
+
+
+def _shape8(shape):
+    return (C.c_int64 * 8)(*(list(shape) + [1] * (8 - len(shape))))
+
+
+def requant_int_axis(x, quant, *, quant_mode, round_mode=ROUND_HALF_AWAY_FROM_ZERO, fuse_rq_axis=False,
+                     quant_triples=True, chip=CHIP_BM168X, input_zp=0, out_dtype=DT_I8):
+    """tpu.RequantIntAxis.inference on f32-valued operands."""
+    x, quant = _f32(x), _f32(quant)
+    attr = RqAxisAttr(_shape8(x.shape), x.ndim, quant_mode, round_mode, int(fuse_rq_axis), int(quant_triples), chip,
+                      input_zp, out_dtype)
+    y = np.empty_like(x)
+    p = _Param([x, quant], [y])
+    check(clib.lib().mi_requant_int_axis_inference(C.byref(attr), C.byref(p.c)))
+    return y
+
+
+def requant_int(x, *, quant_mode, multiplier, rshift, round_mode=ROUND_HALF_AWAY_FROM_ZERO, chip=CHIP_BM168X,
+                input_zp=0, out_zp=0, out_dtype=DT_I8):
+    """tpu.RequantInt.inference on an f32-valued operand."""
+    x = _f32(x)
+    attr = RqAttr(_shape8(x.shape), x.ndim, quant_mode, round_mode, multiplier, rshift, chip, input_zp, out_zp,
+                  out_dtype)
+    y = x.copy()
+    p = _Param([x], [y])
+    check(clib.lib().mi_requant_int_inference(C.byref(attr), C.byref(p.c)))
+    return y
+
+
+# --------------------------------------------------------------------------------------------------
+# device level
+# --------------------------------------------------------------------------------------------------
+def _stream_ptr(stream):
+    import torch
+    s = torch.cuda.current_stream() if stream is None else stream
+    return C.c_void_p(s.cuda_stream)
+
+
+def _dptr(t):
+    return C.c_void_p(0 if t is None else t.data_ptr())
+
+
+class A16Weight:
+    """HBM-resident packed weights of one A16MatMul, built from native-dtype numpy arrays in the
+    reference layout (uint8 [N,K/2] nibble pairs or int8/uint8 [N,K]; 16-bit scale bit patterns and
+    uint8 zero points [N,G]; float32 bias [N])."""
+
+    def __init__(self, weight, scale_bits, zp, bias=None, *, K, N, weight_bits, q_group_size, dtype=DT_BF16,
+                 chip=CHIP_BM168X):
+        weight = np.ascontiguousarray(weight)
+        signed = weight.dtype == np.int8
+        scale_bits = np.ascontiguousarray(scale_bits, dtype=np.uint16)
+        zp = np.ascontiguousarray(zp, dtype=np.uint8)
+        bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+        desc = A16WeightDesc(K, N, weight_bits, int(signed), q_group_size, dtype, chip)
+        self.handle = C.c_void_p()
+        self.K, self.N, self.dtype = K, N, dtype
+        check(clib.lib().mi_a16_weight_create(C.byref(self.handle), C.byref(desc), weight.ctypes.data,
+                                              scale_bits.ctypes.data, zp.ctypes.data,
+                                              None if bias is None else bias.ctypes.data))
+
+    @property
+    def nbytes(self):
+        return clib.lib().mi_a16_weight_bytes(self.handle)
+
+    def destroy(self):
+        if self.handle:
+            clib.lib().mi_a16_weight_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+def a16mm_launch(w, x, y=None, y_f32=None, stream=None):
+    """y[M,N] = round16(x[M,K] @ dequant(W)^T + bias) on the current stream.  x, y: torch CUDA tensors of the
+    weight set's 16-bit type; y_f32 (optional float32 CUDA tensor) receives the fp32 result before rounding."""
+    import torch
+    tdt = torch.float16 if w.dtype == DT_F16 else torch.bfloat16
+    if not (x.is_cuda and x.dtype == tdt and x.is_contiguous() and x.shape[-1] == w.K):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_launch: x must be a contiguous CUDA tensor [.., K]")
+    M = x.numel() // w.K
+    if y is None:
+        y = torch.empty(tuple(x.shape[:-1]) + (w.N,), dtype=tdt, device=x.device)
+    if not (y.is_cuda and y.dtype == tdt and y.is_contiguous() and y.numel() == M * w.N):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_launch: bad output tensor")
+    if y_f32 is not None and not (y_f32.is_cuda and y_f32.dtype == torch.float32 and y_f32.is_contiguous()
+                                  and y_f32.numel() == M * w.N):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_launch: bad y_f32 tensor")
+    check(clib.lib().mi_a16mm_launch(w.handle, _dptr(x), M, _dptr(y), _dptr(y_f32), _stream_ptr(stream)))
+    return y
+
+
+class RequantDesc:
+    """Per-channel (torch int32 CUDA tensors) or scalar requantization parameters; shift > 0 shifts right."""
+
+    def __init__(self, quant_mode, round_mode, out_dtype=DT_I8, chip=CHIP_BM168X, multiplier=1, shift=0, zp=0):
+        self.tensors = []
+        self.c = RequantDescC(quant_mode, round_mode, chip, out_dtype, None, 1, None, 0, None, 0)
+        for name, v in (("multiplier", multiplier), ("shift", shift), ("zp", zp)):
+            if hasattr(v, "data_ptr"):
+                import torch
+                if not (v.is_cuda and v.dtype == torch.int32 and v.is_contiguous()):
+                    raise clib.BackendError(clib.MI_BAD_ARGUMENT, "RequantDesc: per-channel arrays must be int32 CUDA")
+                self.tensors.append(v)
+                setattr(self.c, "d_" + name, v.data_ptr())
+            else:
+                setattr(self.c, name, int(v))
+
+
+_OUT_TORCH = {DT_I8: "int8", DT_U8: "uint8", DT_I16: "int16", DT_I32: "int32"}
+
+
+def _out_tensor(out_dtype, shape, device):
+    import torch
+    if out_dtype == DT_U16:
+        return torch.empty(shape, dtype=torch.int16, device=device)  # bit pattern holder
+    return torch.empty(shape, dtype=getattr(torch, _OUT_TORCH[out_dtype]), device=device)
+
+
+def i8mm_launch(a, b, bias=None, *, right_transpose=False, input_zp=0, right_zp=0, do_relu=False, relu_limit=-1,
+                rq=None, out=None, acc=None, stream=None):
+    """INT8 matmul + requant on device tensors.  a [M,K], b [K,N] (or [N,K] when right_transpose): torch int8 /
+    uint8 CUDA tensors; bias int32 [N]; rq a RequantDesc or None (int32 result)."""
+    import torch
+    M, K = a.shape
+    N = b.shape[0] if right_transpose else b.shape[1]
+    if (b.shape[1] if right_transpose else b.shape[0]) != K:
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "i8mm_launch: inner dimensions differ")
+    for t in (a, b):
+        if not (t.is_cuda and t.is_contiguous() and t.dtype in (torch.int8, torch.uint8)):
+            raise clib.BackendError(clib.MI_BAD_ARGUMENT, "i8mm_launch: operands must be contiguous 8-bit CUDA tensors")
+    if bias is not None and not (bias.is_cuda and bias.dtype == torch.int32 and bias.numel() == N):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "i8mm_launch: bias must be int32 [N] on the GPU")
+    if out is None:
+        out = _out_tensor(rq.c.out_dtype if rq is not None else DT_I32, (M, N), a.device)
+    if acc is not None and not (acc.is_cuda and acc.dtype == torch.int32 and acc.numel() == M * N):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "i8mm_launch: acc must be int32 [M,N] on the GPU")
+    check(clib.lib().mi_i8mm_launch(_dptr(a), int(a.dtype == torch.uint8), _dptr(b), int(b.dtype == torch.uint8),
+                                    int(right_transpose), _dptr(bias), M, K, N, input_zp, right_zp, int(do_relu),
+                                    int(relu_limit), None if rq is None else C.byref(rq.c), _dptr(out), _dptr(acc),
+                                    _stream_ptr(stream)))
+    return out
+
+
+def requant_launch(x, rq, *, outer, channels, inner, input_zp=0, out=None, stream=None):
+    """Standalone requantization of an int32 CUDA tensor viewed as [outer, channels, inner]."""
+    import torch
+    if not (x.is_cuda and x.dtype == torch.int32 and x.is_contiguous() and x.numel() == outer * channels * inner):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "requant_launch: x must be int32 CUDA [outer*channels*inner]")
+    if out is None:
+        out = _out_tensor(rq.c.out_dtype, tuple(x.shape), x.device)
+    check(clib.lib().mi_requant_launch(_dptr(x), _dptr(out), outer, channels, inner, input_zp, C.byref(rq.c),
+                                       _stream_ptr(stream)))
+    return out
