@@ -55,7 +55,10 @@ def _check_against_oracle(orc, cfg, out_bits, pre):
     assert err <= 2e-5, "fp32 pre-round max-abs/RMS %.3g" % err
     want_bits = orc.f32_to_bf16(want)
     ulp = _ulp_distance_bf16(out_bits, want_bits)
-    assert ulp.max() <= 1
+    # one ulp at most; next to zero (where an ulp is far smaller than the fp32 agreement) the absolute bound rules
+    rms = float(np.sqrt(np.mean(want_pre.astype(np.float64) ** 2)))
+    near_zero = np.abs(S.bf16_to_f32(out_bits) - S.bf16_to_f32(want_bits)) <= 4e-5 * rms
+    assert np.all((ulp <= 1) | near_zero)
     assert (ulp != 0).mean() < 5e-3
     # the output must be exactly the reference rounding of the kernel's own fp32 value
     assert np.array_equal(out_bits, orc.f32_to_bf16(pre))
@@ -102,7 +105,7 @@ def test_operator_level_matches_oracle(orc):
         y = op.inference(x[:m])
         want, _ = orc.a16matmul(x[:m], w, s, z, b, M=m, K=1024, N=256, weight_bits=4, q_group_size=128)
         ulp = _ulp_distance_bf16(orc.f32_to_bf16(y), orc.f32_to_bf16(want))
-        assert ulp.max() <= 1 and (ulp != 0).mean() < 5e-3
+        assert np.all((ulp <= 1) | (np.abs(y - want) <= 1e-4)) and (ulp != 0).mean() < 5e-3
         assert np.array_equal(orc.BF16(y), y)  # outputs are bf16 numbers
         assert cmp.cosine_similarity(y, want) > 0.9999 and cmp.euclidean_similarity(y, want) > 0.9999
     op.deinit()

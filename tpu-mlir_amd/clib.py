@@ -86,6 +86,13 @@ def lib():
     if _lib is None:
         if not os.path.exists(_LIB_PATH):
             raise BackendError(MI_HIP_ERROR, "%s is missing: build it with `python tpu-mlir_amd/build.py`" % _LIB_PATH)
+        # One HIP runtime per process: PyTorch ships its own libamdhip64 and the device-level wrappers share
+        # torch's streams and allocations, so when torch is installed it is imported first and the library
+        # binds to the runtime torch loaded.  (A C++ host without torch uses the system runtime.)
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = C.CDLL(_LIB_PATH)
         L.mi_version.restype = C.c_char_p
         L.mi_last_error.restype = C.c_char_p

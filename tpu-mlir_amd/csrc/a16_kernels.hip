@@ -12,8 +12,8 @@
 //   scale_t  [row_block][G][16]  bf16/f16 bit patterns,   zp_t [row_block][G][16] u8 (4-bit),
 //   nzs_t    [row_block][G][16]  float -(zp')*scale (8-bit)
 //
-// Arithmetic (4-bit): a nibble q is turned into the 16-bit float OFFSET+q by OR-ing it into the mantissa of
-// OFFSET (128 for bf16, 1024 for f16); this is exact.  One MFMA accumulates P = sum_k a_k (OFFSET + q_k) over a
+// Arithmetic (4-bit): a nibble q is turned into the 16-bit float OFFSET+q (OFFSET = 16) by shifting it onto the top
+// mantissa bits of 16.0 and OR-ing; this is exact.  One MFMA accumulates P = sum_k a_k (OFFSET + q_k) over a
 // quantization group and a second one S = sum_k a_k; the group then contributes
 //     scale * (P - (OFFSET + zp) * S)  =  sum_k a_k * (q_k - zp) * scale
 // to the fp32 accumulator.  The reference forms (q - zp) * scale per weight in fp32 and sums in fp32
@@ -38,8 +38,11 @@ struct Half16;
 template <>
 struct Half16<MI_DT_BF16> {
   using vec8 = bf16x8;
-  static constexpr uint32_t MAGIC2 = 0x43004300u;  // two bf16 128.0: mantissa ulp is 1 in [128, 256)
-  static constexpr float OFFSET = 128.0f;
+  // two bf16 16.0: the mantissa ulp is 1/8 in [16, 32), so a nibble at mantissa bits 3..6 adds q exactly
+  static constexpr uint32_t NIB_MAGIC2 = 0x41804180u;
+  static constexpr uint32_t NIB_MASK2 = 0x00780078u;
+  static constexpr int LSHIFT = 3;
+  static constexpr float OFFSET = 16.0f;
   static constexpr uint32_t ONE2 = 0x3F803F80u;
   static __device__ __forceinline__ f32x4 mfma(vec8 a, vec8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
@@ -55,8 +58,11 @@ struct Half16<MI_DT_BF16> {
 template <>
 struct Half16<MI_DT_F16> {
   using vec8 = f16x8;
-  static constexpr uint32_t MAGIC2 = 0x64006400u;  // two f16 1024.0: mantissa ulp is 1 in [1024, 2048)
-  static constexpr float OFFSET = 1024.0f;
+  // two f16 16.0: the mantissa ulp is 1/64 in [16, 32), so a nibble at mantissa bits 6..9 adds q exactly
+  static constexpr uint32_t NIB_MAGIC2 = 0x4C004C00u;
+  static constexpr uint32_t NIB_MASK2 = 0x03C003C0u;
+  static constexpr int LSHIFT = 6;
+  static constexpr float OFFSET = 16.0f;
   static constexpr uint32_t ONE2 = 0x3C003C00u;
   static __device__ __forceinline__ f32x4 mfma(vec8 a, vec8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
@@ -365,10 +371,13 @@ __global__ __launch_bounds__(WAVES * 64) void a16w4_skinny_kernel(SkinnyArgs a) 
         for (int j = 0; j < 4; ++j) {
           const uint32_t d = w[j];
           u32x4 b;
-          b[0] = (d & 0x000F000Fu) | H::MAGIC2;
-          b[1] = ((d >> 4) & 0x000F000Fu) | H::MAGIC2;
-          b[2] = ((d >> 8) & 0x000F000Fu) | H::MAGIC2;
-          b[3] = ((d >> 12) & 0x000F000Fu) | H::MAGIC2;
+#pragma unroll
+          for (int pr = 0; pr < 4; ++pr) {
+            // pair pr sits at bits [4pr, 4pr+4) and [16+4pr, 20+4pr): move it onto the mantissa field
+            const uint32_t sh = (4 * pr >= H::LSHIFT) ? (d >> (4 * pr >= H::LSHIFT ? 4 * pr - H::LSHIFT : 0))
+                                                      : (d << (4 * pr >= H::LSHIFT ? 0 : H::LSHIFT - 4 * pr));
+            b[pr] = (sh & H::NIB_MASK2) | H::NIB_MAGIC2;
+          }
           const vec8 bfrag = __builtin_bit_cast(vec8, b);
           const vec8 afrag = __builtin_bit_cast(vec8, xs[j]);
           P = H::mfma(afrag, bfrag, P);
