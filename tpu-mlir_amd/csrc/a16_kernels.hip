@@ -9,18 +9,22 @@
 //            pair (k+2p, k+2p+1) in the two halves of a register.
 //     8-bit: bytes [8j, 8j+8) of the lane hold k = tile*64 + 32*j + 8*(l>>4) + [0..8), stored unsigned
 //            (int8 weights are biased by 128; the bias is folded into nzs_t).
-//   scale_t  [row_block][G][16]  bf16/f16 bit patterns,   zp_t [row_block][G][16] u8 (4-bit),
-//   nzs_t    [row_block][G][16]  float -(zp')*scale (8-bit)
+//   4-bit: sz_t [row_block][G][16] u32 = scale bit pattern << 16 | zero point (one load per group)
+//   8-bit: scale_t [row_block][G][16] bf16/f16 bit patterns, nzs_t [row_block][G][16] float -(zp')*scale
 //
 // Arithmetic (4-bit): a nibble q is turned into the 16-bit float OFFSET+q (OFFSET = 16) by shifting it onto the top
-// mantissa bits of 16.0 and OR-ing; this is exact.  One MFMA accumulates P = sum_k a_k (OFFSET + q_k) over a
-// quantization group and a second one S = sum_k a_k; the group then contributes
+// mantissa bits of 16.0 and OR-ing; this is exact.  The MFMA accumulates P = sum_k a_k (OFFSET + q_k) over a
+// quantization group; with S = sum_k a_k over the same group (summed once per workgroup while the activations are
+// staged into LDS, or by a second MFMA against a vector of ones when they are not) the group contributes
 //     scale * (P - (OFFSET + zp) * S)  =  sum_k a_k * (q_k - zp) * scale
 // to the fp32 accumulator.  The reference forms (q - zp) * scale per weight in fp32 and sums in fp32
 // (lib/Dialect/Tpu/Interfaces/Common/A16MatMul.cpp:189-198); both are fp32 evaluations of the same real number.
 // Arithmetic (8-bit): the reference rounds the dequantized weight to bf16/f16 before the GEMM (:227-231);
 // fma(q', scale, nzs) is the correctly rounded fp32 (q - zp) * scale because zp' * scale is exact in fp32, and the
 // hardware conversion rounds it to nearest even, so the MFMA sees the reference's weight bit for bit.
+#include <stdio.h>
+#include <stdlib.h>
+
 #include "device_math.cuh"
 #include "internal.h"
 
@@ -123,10 +127,10 @@ __global__ void pack_w8_kernel(const uint8_t *__restrict__ src, uint8_t *__restr
   dst[idx] = v;
 }
 
-// scale [N,G] -> scale_t [rb][G][16];  zp [N,G] -> zp_t (4-bit) or nzs_t (8-bit)
+// scale [N,G], zp [N,G] -> [rb][G][16] tables: 4-bit sz_t = scale bits << 16 | zp; 8-bit scale_t and nzs_t
 template <int DT>
 __global__ void pack_qparams_kernel(const uint16_t *__restrict__ scale, const uint8_t *__restrict__ zp,
-                                    uint16_t *__restrict__ scale_t, uint8_t *__restrict__ zp_t,
+                                    uint16_t *__restrict__ scale_t, uint32_t *__restrict__ sz_t,
                                     float *__restrict__ nzs_t, int64_t N, int G, int64_t total, int zp_bias) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total)
@@ -142,9 +146,10 @@ __global__ void pack_qparams_kernel(const uint16_t *__restrict__ scale, const ui
     s = scale[n * G + gi];
     z = zp[n * G + gi];
   }
-  scale_t[idx] = s;
-  if (zp_t)
-    zp_t[idx] = z;
+  if (scale_t)
+    scale_t[idx] = s;
+  if (sz_t)
+    sz_t[idx] = ((uint32_t)s << 16) | z;
   if (nzs_t)
     nzs_t[idx] = -(float)((int)z + zp_bias) * Half16<DT>::to_f32(s);
 }
@@ -154,12 +159,12 @@ void a16_free(mi_a16_weight *w) {
     return;
   (void)hipFree(w->qweight);
   (void)hipFree(w->scale_t);
-  (void)hipFree(w->zp_t);
+  (void)hipFree(w->sz_t);
   (void)hipFree(w->nzs_t);
   (void)hipFree(w->bias);
   w->qweight = nullptr;
   w->scale_t = nullptr;
-  w->zp_t = nullptr;
+  w->sz_t = nullptr;
   w->nzs_t = nullptr;
   w->bias = nullptr;
 }
@@ -199,12 +204,13 @@ int a16_pack(mi_a16_weight *w, const void *h_weight, int weight_signed, const ui
   PACK_HIP(hipMemcpy(d_scale, h_scale, nq * 2, hipMemcpyHostToDevice));
   PACK_HIP(hipMemcpy(d_zp, h_zp, nq, hipMemcpyHostToDevice));
   PACK_HIP(hipMalloc(&w->qweight, packed_bytes));
-  PACK_HIP(hipMalloc((void **)&w->scale_t, qp * 2));
-  if (w->bits == 4)
-    PACK_HIP(hipMalloc((void **)&w->zp_t, qp));
-  else
+  if (w->bits == 4) {
+    PACK_HIP(hipMalloc((void **)&w->sz_t, qp * 4));
+  } else {
+    PACK_HIP(hipMalloc((void **)&w->scale_t, qp * 2));
     PACK_HIP(hipMalloc((void **)&w->nzs_t, qp * 4));
-  w->bytes = packed_bytes + qp * 2 + (w->bits == 4 ? qp : qp * 4);
+  }
+  w->bytes = packed_bytes + (w->bits == 4 ? qp * 4 : qp * 6);
   if (h_bias) {
     PACK_HIP(hipMalloc((void **)&w->bias, (size_t)N * 4));
     PACK_HIP(hipMemcpy(w->bias, h_bias, (size_t)N * 4, hipMemcpyHostToDevice));
@@ -227,10 +233,10 @@ int a16_pack(mi_a16_weight *w, const void *h_weight, int weight_signed, const ui
     dim3 grid((unsigned)((total + threads - 1) / threads));
     int zp_bias = (w->bits == 8 && weight_signed) ? 128 : 0;
     if (w->dtype == MI_DT_F16)
-      pack_qparams_kernel<MI_DT_F16><<<grid, dim3(threads)>>>(d_scale, d_zp, w->scale_t, w->zp_t, w->nzs_t, N,
+      pack_qparams_kernel<MI_DT_F16><<<grid, dim3(threads)>>>(d_scale, d_zp, w->scale_t, w->sz_t, w->nzs_t, N,
                                                               w->G, total, zp_bias);
     else
-      pack_qparams_kernel<MI_DT_BF16><<<grid, dim3(threads)>>>(d_scale, d_zp, w->scale_t, w->zp_t, w->nzs_t, N,
+      pack_qparams_kernel<MI_DT_BF16><<<grid, dim3(threads)>>>(d_scale, d_zp, w->scale_t, w->sz_t, w->nzs_t, N,
                                                                w->G, total, zp_bias);
   }
   PACK_HIP(hipGetLastError());
@@ -241,13 +247,21 @@ int a16_pack(mi_a16_weight *w, const void *h_weight, int weight_signed, const ui
 }
 
 // ------------------------------------------------------------------------------------------------
-// skinny kernel: up to 16 activation rows per workgroup, one 16-channel row block per workgroup,
-// K split over the workgroup's waves and reduced through LDS.
+// skinny kernel: up to 16 activation rows per workgroup (one MFMA 16x16 block of outputs per row block).
+// A workgroup owns R consecutive 16-channel row blocks over the whole K; its WAVES waves take the K tiles
+// round-robin and their partial sums are reduced through LDS.  A wave works in rounds of TPW tiles: it issues the
+// loads of all TPW tiles (indices clamped, never predicated, so the load count is static and the compiler simply
+// counts them down), then consumes them in order.  TPW is chosen so that one round covers the wave's share of K
+// whenever possible: every byte the wave will read is then in flight at once.
+//
+// XLDS = true (M * K small enough): the activations are staged once per workgroup into LDS, zero filled past K,
+// and the per-group activation sums S are formed during staging; the registers then hold weights only.
+// XLDS = false: activation fragments are loaded per tile from global memory (L2) and S comes from a second MFMA.
 // ------------------------------------------------------------------------------------------------
 struct SkinnyArgs {
   const u32x4 *qw;
+  const uint32_t *sz_t;
   const uint16_t *scale_t;
-  const uint8_t *zp_t;
   const float *nzs_t;
   const float *bias;
   const uint16_t *x;
@@ -255,24 +269,33 @@ struct SkinnyArgs {
   float *y32;
   int M;
   int64_t K, N;
-  int k_tiles;
+  int row_blocks;
+  int k_tiles;          // tiles stored per row block (the last one may be partial)
+  int full_tiles;       // tiles that lie completely inside K
   int G;
-  int tiles_per_group;  // 4-bit, GPT == 1: tiles that share one group (g / 128; k_tiles when per channel)
-  int group_k;          // 8-bit: group size in elements (K when per channel)
+  int tiles_per_group;  // GPT == 1: tiles that share one group (g / TILE_K; k_tiles when per channel)
   int chip;
 };
 
-template <int DT>
-__device__ __forceinline__ void store_result(const SkinnyArgs &a, float (*red)[4][64], int waves, int lane,
-                                             int rb, int m0) {
-  const int col = lane & 15, kq = lane >> 4;
-  const int64_t n = (int64_t)rb * ROW_BLOCK + col;
+template <int DT, int WAVES, int R>
+__device__ __forceinline__ void reduce_and_store(const SkinnyArgs &a, float (*red)[R][4][64], const f32x4 (&acc)[R],
+                                                 int wave, int lane, int rb0, int m0) {
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      red[wave][r][i][lane] = acc[r][i];
+  __syncthreads();
+  // R * 4 * 64 partial sums to finish: spread them over the workgroup's waves
+  const int col = lane & 15, kq = lane >> 4;
+  for (int item = wave; item < R * 4; item += WAVES) {
+    const int r = item >> 2, i = item & 3;
     float v = 0.0f;
-    for (int w = 0; w < waves; ++w)
-      v += red[w][r][lane];
-    const int m = m0 + 4 * kq + r;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w)
+      v += red[w][r][i][lane];
+    const int64_t n = (int64_t)(rb0 + r) * ROW_BLOCK + col;
+    const int m = m0 + 4 * kq + i;
     if (m < a.M && n < a.N) {
       if (a.bias)
         v += a.bias[n];
@@ -284,256 +307,461 @@ __device__ __forceinline__ void store_result(const SkinnyArgs &a, float (*red)[4
   }
 }
 
-template <int DT, int GPT, int WAVES, int PF>
-__global__ __launch_bounds__(WAVES * 64) void a16w4_skinny_kernel(SkinnyArgs a) {
+// (a & mask) | magic in one VALU instruction.  The compiler splits this into v_and + v_or when both constants
+// are literals (VOP3 takes no literal on gfx9), so the operands are pinned: mask in an SGPR, magic in a VGPR.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(magic));
+  return r;
+}
+
+template <int DT>
+__device__ __forceinline__ typename Half16<DT>::vec8 unpack_nibbles(uint32_t d, uint32_t magic) {
+  using H = Half16<DT>;
+  u32x4 b;
+#pragma unroll
+  for (int pr = 0; pr < 4; ++pr) {
+    // pair pr sits at bits [4pr, 4pr+4) and [16+4pr, 20+4pr): move it onto the mantissa field
+    const uint32_t sh = (4 * pr >= H::LSHIFT) ? (d >> (4 * pr >= H::LSHIFT ? 4 * pr - H::LSHIFT : 0))
+                                              : (d << (4 * pr >= H::LSHIFT ? 0 : H::LSHIFT - 4 * pr));
+    b[pr] = and_or(sh, H::NIB_MASK2, magic);
+  }
+  return __builtin_bit_cast(typename H::vec8, b);
+}
+
+template <int DT>
+__device__ __forceinline__ typename Half16<DT>::vec8 dequant_bytes(uint32_t d0, uint32_t d1, float s, float z) {
+  using H = Half16<DT>;
+  u32x4 b;
+  b[0] = H::pack2(fmaf((float)(d0 & 0xffu), s, z), fmaf((float)((d0 >> 8) & 0xffu), s, z));
+  b[1] = H::pack2(fmaf((float)((d0 >> 16) & 0xffu), s, z), fmaf((float)(d0 >> 24), s, z));
+  b[2] = H::pack2(fmaf((float)(d1 & 0xffu), s, z), fmaf((float)((d1 >> 8) & 0xffu), s, z));
+  b[3] = H::pack2(fmaf((float)((d1 >> 16) & 0xffu), s, z), fmaf((float)(d1 >> 24), s, z));
+  return __builtin_bit_cast(typename H::vec8, b);
+}
+
+// LDS carve-up of the skinny kernel: red | S (XLDS, 4-bit) | x rows (XLDS)
+__host__ __device__ constexpr size_t skinny_red_bytes(int waves, int r) { return (size_t)waves * r * 1024; }
+
+#ifdef MI_DBG_TIMING
+__device__ unsigned long long mi_dbg_buf[8 * 4096];
+#define MI_STAMP(slot)                                                                       \
+  do {                                                                                       \
+    if (threadIdx.x == 0 && blockIdx.x < 4096)                                               \
+      mi_dbg_buf[blockIdx.x * 8 + (slot)] = __builtin_readcyclecounter();                    \
+  } while (0)
+#else
+#define MI_STAMP(slot)
+#endif
+
+template <int BITS, int DT, int GPT, int WAVES, int TPW, int R, bool XLDS>
+__global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
+  MI_STAMP(0);
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
-  __shared__ float red[WAVES][4][64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int rb = blockIdx.x, m0 = blockIdx.y * 16;
+  constexpr int TILE_K = BITS == 4 ? W4_TILE_K : W8_TILE_K;
+  constexpr int KSTEPS = TILE_K / 32;             // MFMA k-steps per tile: 4 (4-bit) or 2 (8-bit)
+  constexpr int KSTEPS_PER_UNIT = KSTEPS / GPT;   // k-steps that share one set of group parameters
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  float(*red)[R][4][64] = reinterpret_cast<float(*)[R][4][64]>(smem);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps the tile loops scalar
+  const int rb0 = blockIdx.x * R, m0 = blockIdx.y * 16;
   const int col = lane & 15, kq = lane >> 4;
-  const bool m_ok = (m0 + col) < a.M;
-  const uint16_t *xrow = a.x + (int64_t)(m_ok ? m0 + col : 0) * a.K + kq * 8;
-  const u32x4 *wq = a.qw + (int64_t)rb * a.k_tiles * 64 + lane;
-  const uint16_t *sc = a.scale_t + (int64_t)rb * a.G * 16 + col;
-  const uint8_t *zp = a.zp_t + (int64_t)rb * a.G * 16 + col;
-  constexpr int KSTEPS_PER_GROUP = 4 / GPT;
+  const int rows = (a.M - m0) < 16 ? (a.M - m0) : 16;
+  const int row_ld = col < rows ? col : rows - 1;  // rows past M re-read the last row; their outputs are never stored
+  const int kpad = a.k_tiles * TILE_K;
+  const int n_units = a.k_tiles * GPT;
+  float *s_lds = reinterpret_cast<float *>(smem + skinny_red_bytes(WAVES, R));     // [n_units][16]
+  uint8_t *xs = smem + skinny_red_bytes(WAVES, R) + (BITS == 4 ? (size_t)n_units * 64 : 0);
+  const int xstride = kpad * 2 + 64;  // bytes; +64 puts consecutive rows 16 banks apart
 
-  u32x4 wbuf[PF];
-  u32x4 xbuf[PF][4];
-  uint16_t sbuf[PF][GPT];
-  uint8_t zbuf[PF][GPT];
-
-  auto load_tile = [&](u32x4 &w, u32x4 (&xs)[4], uint16_t (&ss)[GPT], uint8_t (&zs)[GPT], int kt) {
-    w = wq[(int64_t)kt * 64];
+  const u32x4 *wq[R];
+  const uint32_t *szp[R];
+  const uint16_t *scp[R];
+  const float *nzp[R];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int64_t k0 = (int64_t)kt * W4_TILE_K + 32 * j;
-      u32x4 v = {0, 0, 0, 0};
-      if (m_ok && (k0 + kq * 8) < a.K)
-        v = *(const u32x4 *)(xrow + k0);
-      xs[j] = v;
+  for (int r = 0; r < R; ++r) {
+    int rb = (rb0 + r) < a.row_blocks ? (rb0 + r) : (a.row_blocks - 1);  // clamped, discarded at the store
+#ifdef MI_DBG_SAMETILE
+    rb = rb & 3;
+#endif
+    wq[r] = a.qw + (int64_t)rb * a.k_tiles * 64 + lane;
+    if constexpr (BITS == 4) {
+      szp[r] = a.sz_t + (int64_t)rb * a.G * 16 + col;
+    } else {
+      scp[r] = a.scale_t + (int64_t)rb * a.G * 16 + col;
+      nzp[r] = a.nzs_t + (int64_t)rb * a.G * 16 + col;
     }
+  }
+  const uint16_t *xrow = a.x + (int64_t)(m0 + row_ld) * a.K + kq * 8;
+
+  struct Tile {
+    u32x4 w[R];
+    uint32_t sz[R][GPT];  // 4-bit: scale << 16 | zp;  8-bit: scale bits
+    float nz[R][GPT];     // 8-bit only
+    u32x4 x[XLDS ? 1 : KSTEPS];
+  };
+
+  auto unit_group = [&](int kt, int u) {
+    int gi;
+    // tiles_per_group is 1 for the common group size == tile size; the division only runs for larger groups
+    if constexpr (GPT == 1)
+      gi = a.tiles_per_group == 1 ? kt : kt / a.tiles_per_group;
+    else
+      gi = kt * GPT + u;
+    return gi < a.G ? gi : a.G - 1;
+  };
+
+  auto load_tile = [&](Tile &t, int kt) {
+#ifdef MI_DBG_SAMETILE
+    kt = kt & 1;
+#endif
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      t.w[r] = wq[r][(int64_t)kt * 64];
 #pragma unroll
     for (int u = 0; u < GPT; ++u) {
-      int gi = GPT == 1 ? kt / a.tiles_per_group : kt * GPT + u;
-      gi = gi < a.G ? gi : a.G - 1;
-      ss[u] = sc[gi * 16];
-      zs[u] = zp[gi * 16];
+      const int gi = unit_group(kt, u);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if constexpr (BITS == 4) {
+          t.sz[r][u] = szp[r][gi * 16];
+        } else {
+          t.sz[r][u] = scp[r][gi * 16];
+          t.nz[r][u] = nzp[r][gi * 16];
+        }
+      }
+    }
+    if constexpr (!XLDS) {
+#pragma unroll
+      for (int j = 0; j < KSTEPS; ++j) {
+        // only tiles inside K are loaded here; the partial last tile goes through load_tail_x
+        t.x[j] = *(const u32x4 *)(xrow + (int64_t)kt * TILE_K + 32 * j);
+      }
     }
   };
 
+  f32x4 acc[R];
 #pragma unroll
-  for (int p = 0; p < PF; ++p) {
-    const int kt = wave + p * WAVES;
-    if (kt < a.k_tiles) {
-      load_tile(wbuf[p], xbuf[p], sbuf[p], zbuf[p], kt);
-    } else {
-      wbuf[p] = u32x4{0, 0, 0, 0};
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        xbuf[p][j] = u32x4{0, 0, 0, 0};
-#pragma unroll
-      for (int u = 0; u < GPT; ++u) {
-        sbuf[p][u] = 0;
-        zbuf[p][u] = 0;
-      }
-    }
-  }
-
+  for (int r = 0; r < R; ++r)
+    acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
   const u32x4 ones_bits = {H::ONE2, H::ONE2, H::ONE2, H::ONE2};
   const vec8 ones = __builtin_bit_cast(vec8, ones_bits);
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  uint32_t nib_magic = H::NIB_MAGIC2;
+  asm volatile("" : "+v"(nib_magic));  // keep it in a VGPR (see and_or)
 
-  for (int kt0 = wave; kt0 < a.k_tiles; kt0 += PF * WAVES) {
+  auto compute_tile = [&](const Tile &t, int kt) {
+#ifdef MI_DBG_NOCOMPUTE
+    acc[0][0] += __builtin_bit_cast(float, t.w[0][0] ^ t.w[0][1] ^ t.w[0][2] ^ t.w[0][3] ^ t.sz[0][0]);
+    return;
+#endif
+    u32x4 xf[KSTEPS];
 #pragma unroll
-    for (int p = 0; p < PF; ++p) {
-      const int kt = kt0 + p * WAVES;
-      if (kt < a.k_tiles) {
-        const u32x4 w = wbuf[p];
-        u32x4 xs[4];
-        uint16_t ss[GPT];
-        uint8_t zs[GPT];
+    for (int j = 0; j < KSTEPS; ++j) {
+      if constexpr (XLDS)
+        xf[j] = *(const u32x4 *)(xs + row_ld * xstride + kq * 16 + (kt * TILE_K + 32 * j) * 2);
+      else
+        xf[j] = t.x[j];
+    }
+    if constexpr (BITS == 4) {
+      f32x4 P[R], S = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          xs[j] = xbuf[p][j];
+      for (int r = 0; r < R; ++r)
+        P[r] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int u = 0; u < GPT; ++u) {
-          ss[u] = sbuf[p][u];
-          zs[u] = zbuf[p][u];
-        }
-        const int ktn = kt + PF * WAVES;
-        if (ktn < a.k_tiles)
-          load_tile(wbuf[p], xbuf[p], sbuf[p], zbuf[p], ktn);
-
-        f32x4 P = {0.f, 0.f, 0.f, 0.f}, S = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const uint32_t d = w[j];
-          u32x4 b;
-#pragma unroll
-          for (int pr = 0; pr < 4; ++pr) {
-            // pair pr sits at bits [4pr, 4pr+4) and [16+4pr, 20+4pr): move it onto the mantissa field
-            const uint32_t sh = (4 * pr >= H::LSHIFT) ? (d >> (4 * pr >= H::LSHIFT ? 4 * pr - H::LSHIFT : 0))
-                                                      : (d << (4 * pr >= H::LSHIFT ? 0 : H::LSHIFT - 4 * pr));
-            b[pr] = (sh & H::NIB_MASK2) | H::NIB_MAGIC2;
-          }
-          const vec8 bfrag = __builtin_bit_cast(vec8, b);
-          const vec8 afrag = __builtin_bit_cast(vec8, xs[j]);
-          P = H::mfma(afrag, bfrag, P);
+      for (int j = 0; j < KSTEPS; ++j) {
+        const vec8 afrag = __builtin_bit_cast(vec8, xf[j]);
+        if constexpr (!XLDS)
           S = H::mfma(afrag, ones, S);
-          if ((j + 1) % KSTEPS_PER_GROUP == 0) {
-            const int u = j / KSTEPS_PER_GROUP;
-            const float s = H::to_f32(ss[u]);
-            const float c = H::OFFSET + (float)zs[u];
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-              acc[r] = fmaf(s, fmaf(-c, S[r], P[r]), acc[r]);
-            P = f32x4{0.f, 0.f, 0.f, 0.f};
-            S = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int r = 0; r < R; ++r)
+          P[r] = H::mfma(afrag, unpack_nibbles<DT>(t.w[r][j], nib_magic), P[r]);
+        if ((j + 1) % KSTEPS_PER_UNIT == 0) {
+          const int u = j / KSTEPS_PER_UNIT;
+          if constexpr (XLDS)
+            S = *(const f32x4 *)(s_lds + (kt * GPT + u) * 16 + kq * 4);
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            const float s = H::to_f32((uint16_t)(t.sz[r][u] >> 16));
+            const float c = H::OFFSET + (float)(t.sz[r][u] & 0xffu);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              acc[r][i] = fmaf(s, fmaf(-c, S[i], P[r][i]), acc[r][i]);
+            P[r] = f32x4{0.f, 0.f, 0.f, 0.f};
           }
+          S = f32x4{0.f, 0.f, 0.f, 0.f};
         }
       }
-    }
-  }
-
+    } else {
 #pragma unroll
-  for (int r = 0; r < 4; ++r)
-    red[wave][r][lane] = acc[r];
-  __syncthreads();
-  if (wave == 0)
-    store_result<DT>(a, red, WAVES, lane, rb, m0);
-}
-
-template <int DT, int GPT, int WAVES, int PF>
-__global__ __launch_bounds__(WAVES * 64) void a16w8_skinny_kernel(SkinnyArgs a) {
-  using H = Half16<DT>;
-  using vec8 = typename H::vec8;
-  __shared__ float red[WAVES][4][64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int rb = blockIdx.x, m0 = blockIdx.y * 16;
-  const int col = lane & 15, kq = lane >> 4;
-  const bool m_ok = (m0 + col) < a.M;
-  const uint16_t *xrow = a.x + (int64_t)(m_ok ? m0 + col : 0) * a.K + kq * 8;
-  const u32x4 *wq = a.qw + (int64_t)rb * a.k_tiles * 64 + lane;
-  const uint16_t *sc = a.scale_t + (int64_t)rb * a.G * 16 + col;
-  const float *nzs = a.nzs_t + (int64_t)rb * a.G * 16 + col;
-
-  u32x4 wbuf[PF];
-  u32x4 xbuf[PF][2];
-  uint16_t sbuf[PF][GPT];
-  float zbuf[PF][GPT];
-
-  auto load_tile = [&](u32x4 &w, u32x4 (&xs)[2], uint16_t (&ss)[GPT], float (&zs)[GPT], int kt) {
-    w = wq[(int64_t)kt * 64];
+      for (int j = 0; j < KSTEPS; ++j) {
+        const int u = GPT == 1 ? 0 : j;
+        const vec8 afrag = __builtin_bit_cast(vec8, xf[j]);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int64_t k0 = (int64_t)kt * W8_TILE_K + 32 * j;
-      u32x4 v = {0, 0, 0, 0};
-      if (m_ok && (k0 + kq * 8) < a.K)
-        v = *(const u32x4 *)(xrow + k0);
-      xs[j] = v;
-    }
-#pragma unroll
-    for (int u = 0; u < GPT; ++u) {
-      int gi = (int)(((int64_t)kt * W8_TILE_K + (GPT == 1 ? 0 : 32 * u)) / a.group_k);
-      gi = gi < a.G ? gi : a.G - 1;
-      ss[u] = sc[gi * 16];
-      zs[u] = nzs[gi * 16];
+        for (int r = 0; r < R; ++r)
+          acc[r] = H::mfma(afrag,
+                           dequant_bytes<DT>(t.w[r][2 * j], t.w[r][2 * j + 1], H::to_f32((uint16_t)t.sz[r][u]),
+                                             t.nz[r][u]),
+                           acc[r]);
+      }
     }
   };
 
+  // tiles this wave owns: kt = wave + i * WAVES.  With the activations in LDS the (zero padded) partial last tile
+  // is an ordinary tile; otherwise only full tiles are taken here and the tail is handled separately below.
+  const int n_tiles = XLDS ? a.k_tiles : a.full_tiles;
+  const int n_my = wave < n_tiles ? (n_tiles - wave + WAVES - 1) / WAVES : 0;
+  const int last = n_tiles > 0 ? n_tiles - 1 : 0;
+
+  Tile buf_a[TPW];
+  auto issue_round = [&](Tile (&buf)[TPW], int i0) {
 #pragma unroll
-  for (int p = 0; p < PF; ++p) {
-    const int kt = wave + p * WAVES;
-    if (kt < a.k_tiles) {
-      load_tile(wbuf[p], xbuf[p], sbuf[p], zbuf[p], kt);
-    } else {
-      wbuf[p] = u32x4{0, 0, 0, 0};
-      xbuf[p][0] = u32x4{0, 0, 0, 0};
-      xbuf[p][1] = u32x4{0, 0, 0, 0};
+    for (int p = 0; p < TPW; ++p) {
+      const int kt = wave + (i0 + p) * WAVES;
+      load_tile(buf[p], kt < n_tiles ? kt : last);
+    }
+  };
+  auto consume_round = [&](const Tile (&buf)[TPW], int i0) {
+#pragma unroll
+    for (int p = 0; p < TPW; ++p)
+      if (i0 + p < n_my)
+        compute_tile(buf[p], wave + (i0 + p) * WAVES);
+  };
+
+#ifndef MI_DBG_NOSTAGE
+  if constexpr (XLDS) {
+    // Stage the activation rows (16-byte chunks, zero past K) and form the per-unit sums S.  The first batch of
+    // activation loads is issued BEFORE the weight loads and written to LDS after them: loads return in order, so
+    // waiting for the activations then leaves every weight load in flight.
+    constexpr int UNIT_CHUNKS = TILE_K / GPT / 8;  // 16-byte chunks per unit: 16, 8 or 4
+    constexpr int NT = WAVES * 64;
+    constexpr int XB = WAVES >= 16 ? 2 : 4;        // chunks per thread in the first batch
+    const int chunks_per_row = kpad / 8;
+    const int total = rows * chunks_per_row;
+    auto chunk_load = [&](int c, int &row, int &kc, bool &ok) {
+      ok = c < total;
+      const int cc = ok ? c : 0;
+      row = rows == 1 ? 0 : cc / chunks_per_row;
+      kc = cc - row * chunks_per_row;
+      const bool in_k = kc * 8 < a.K;
+      u32x4 v = *(const u32x4 *)(a.x + (int64_t)(m0 + row) * a.K + (in_k ? kc * 8 : 0));  // always in bounds
+      if (!in_k)
+        v = u32x4{0, 0, 0, 0};
+      return v;
+    };
+    auto chunk_store = [&](const u32x4 &v, int row, int kc, bool ok) {
+      if (ok)
+        *(u32x4 *)(xs + row * xstride + kc * 16) = v;
+      if constexpr (BITS == 4) {
+        float part = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          part += H::to_f32((uint16_t)(v[i] & 0xffffu)) + H::to_f32((uint16_t)(v[i] >> 16));
+#pragma unroll
+        for (int off = 1; off < UNIT_CHUNKS; off <<= 1)
+          part += __shfl_xor(part, off, 64);
+        if (ok && (kc % UNIT_CHUNKS) == 0)
+          s_lds[(kc / UNIT_CHUNKS) * 16 + row] = part;
+      }
+    };
+    u32x4 v[XB];
+    int row[XB], kc[XB];
+    bool ok[XB];
+#pragma unroll
+    for (int b = 0; b < XB; ++b)
+      if (b * NT < total)  // workgroup-uniform
+        v[b] = chunk_load(b * NT + tid, row[b], kc[b], ok[b]);
+    if (n_tiles > 0)
+      issue_round(buf_a, 0);
+    MI_STAMP(1);
+#pragma unroll
+    for (int b = 0; b < XB; ++b)
+      if (b * NT < total)
+        chunk_store(v[b], row[b], kc[b], ok[b]);
+    for (int c0 = XB * NT; c0 < total; c0 += NT) {  // large M * K only: these wait behind the weight loads
+      int r1, k1;
+      bool o1;
+      const u32x4 v1 = chunk_load(c0 + tid, r1, k1, o1);
+      chunk_store(v1, r1, k1, o1);
+    }
+    __syncthreads();
+    MI_STAMP(2);
+  } else
+#endif
+  {
+    if (n_tiles > 0)
+      issue_round(buf_a, 0);
+  }
+  // TPW is normally chosen so that one round covers the wave's share of K; larger K takes further rounds, each
+  // self-contained (issue, then consume) so that the load counters stay static
+  if (n_my > 0)
+    consume_round(buf_a, 0);
+  for (int i0 = TPW; i0 < n_my; i0 += TPW) {
+    issue_round(buf_a, i0);
+    consume_round(buf_a, i0);
+  }
+  MI_STAMP(3);
+  if constexpr (!XLDS) {
+    if (a.full_tiles < a.k_tiles && wave == (a.full_tiles % WAVES)) {
+      // partial last tile (K not a multiple of the tile): activations past K must read as zero
+      Tile t;
+      const int kt = a.full_tiles;
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        t.w[r] = wq[r][(int64_t)kt * 64];
 #pragma unroll
       for (int u = 0; u < GPT; ++u) {
-        sbuf[p][u] = 0;
-        zbuf[p][u] = 0.f;
-      }
-    }
-  }
-
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int kt0 = wave; kt0 < a.k_tiles; kt0 += PF * WAVES) {
+        const int gi = unit_group(kt, u);
 #pragma unroll
-    for (int p = 0; p < PF; ++p) {
-      const int kt = kt0 + p * WAVES;
-      if (kt < a.k_tiles) {
-        const u32x4 w = wbuf[p];
-        u32x4 xs[2] = {xbuf[p][0], xbuf[p][1]};
-        uint16_t ss[GPT];
-        float zs[GPT];
-#pragma unroll
-        for (int u = 0; u < GPT; ++u) {
-          ss[u] = sbuf[p][u];
-          zs[u] = zbuf[p][u];
-        }
-        const int ktn = kt + PF * WAVES;
-        if (ktn < a.k_tiles)
-          load_tile(wbuf[p], xbuf[p], sbuf[p], zbuf[p], ktn);
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int u = GPT == 1 ? 0 : j;
-          const float s = H::to_f32(ss[u]);
-          const float z = zs[u];
-          const uint32_t d0 = w[2 * j], d1 = w[2 * j + 1];
-          u32x4 b;
-          b[0] = H::pack2(fmaf((float)(d0 & 0xffu), s, z), fmaf((float)((d0 >> 8) & 0xffu), s, z));
-          b[1] = H::pack2(fmaf((float)((d0 >> 16) & 0xffu), s, z), fmaf((float)(d0 >> 24), s, z));
-          b[2] = H::pack2(fmaf((float)(d1 & 0xffu), s, z), fmaf((float)((d1 >> 8) & 0xffu), s, z));
-          b[3] = H::pack2(fmaf((float)((d1 >> 16) & 0xffu), s, z), fmaf((float)(d1 >> 24), s, z));
-          acc = H::mfma(__builtin_bit_cast(vec8, xs[j]), __builtin_bit_cast(vec8, b), acc);
+        for (int r = 0; r < R; ++r) {
+          if constexpr (BITS == 4) {
+            t.sz[r][u] = szp[r][gi * 16];
+          } else {
+            t.sz[r][u] = scp[r][gi * 16];
+            t.nz[r][u] = nzp[r][gi * 16];
+          }
         }
       }
+#pragma unroll
+      for (int j = 0; j < KSTEPS; ++j) {
+        const int64_t k0 = (int64_t)kt * TILE_K + 32 * j + kq * 8;
+        u32x4 v = {0, 0, 0, 0};
+        if (k0 < a.K)
+          v = *(const u32x4 *)(xrow + (int64_t)kt * TILE_K + 32 * j);
+        t.x[j] = v;
+      }
+      compute_tile(t, kt);
     }
   }
-
-#pragma unroll
-  for (int r = 0; r < 4; ++r)
-    red[wave][r][lane] = acc[r];
-  __syncthreads();
-  if (wave == 0)
-    store_result<DT>(a, red, WAVES, lane, rb, m0);
+  reduce_and_store<DT, WAVES, R>(a, red, acc, wave, lane, rb0, m0);
+  MI_STAMP(4);
+#ifdef MI_DBG_TIMING
+  if (threadIdx.x == 0 && blockIdx.x < 4096) {
+    unsigned hwid;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+    unsigned xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    mi_dbg_buf[blockIdx.x * 8 + 5] = hwid;
+    mi_dbg_buf[blockIdx.x * 8 + 6] = xcc;
+  }
+#endif
 }
+
+#ifdef MI_DBG_TIMING
+extern "C" int mi_dbg_dump(unsigned long long *host, size_t n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mi_dbg_buf), n * sizeof(unsigned long long));
+}
+#endif
 
 // ------------------------------------------------------------------------------------------------
 // host-side dispatch
 // ------------------------------------------------------------------------------------------------
-template <int DT, int GPT>
-static void launch_w4(const SkinnyArgs &a, int waves, dim3 grid, hipStream_t st) {
-  if (waves >= 16)
-    a16w4_skinny_kernel<DT, GPT, 16, 2><<<grid, dim3(1024), 0, st>>>(a);
-  else if (waves >= 8)
-    a16w4_skinny_kernel<DT, GPT, 8, 4><<<grid, dim3(512), 0, st>>>(a);
-  else
-    a16w4_skinny_kernel<DT, GPT, 4, 4><<<grid, dim3(256), 0, st>>>(a);
+struct SkinnyPlan {
+  int waves, tpw, r;
+};
+
+// development hook: MI_A16_PLAN="waves,tpw,r" overrides the heuristic
+static bool plan_override(SkinnyPlan &p) {
+  const char *e = getenv("MI_A16_PLAN");
+  if (!e)
+    return false;
+  return sscanf(e, "%d,%d,%d", &p.waves, &p.tpw, &p.r) == 3;
 }
 
-template <int DT, int GPT>
-static void launch_w8(const SkinnyArgs &a, int waves, dim3 grid, hipStream_t st) {
-  if (waves >= 16)
-    a16w8_skinny_kernel<DT, GPT, 16, 2><<<grid, dim3(1024), 0, st>>>(a);
-  else if (waves >= 8)
-    a16w8_skinny_kernel<DT, GPT, 8, 4><<<grid, dim3(512), 0, st>>>(a);
-  else
-    a16w8_skinny_kernel<DT, GPT, 4, 4><<<grid, dim3(256), 0, st>>>(a);
+static size_t skinny_x_bytes(int rows, int64_t k_tiles, int tile_k) {
+  return (size_t)rows * ((size_t)k_tiles * tile_k * 2 + 64);
+}
+constexpr size_t XLDS_MAX_BYTES = 96 * 1024;  // activation rows staged in LDS up to this size
+
+// K is split over the waves of a workgroup so that one round of TPW tiles covers a wave's share whenever
+// TPW <= 8 allows it (K <= 16384 for 4-bit weights with 16 waves).
+static SkinnyPlan pick_plan(int64_t row_blocks, int64_t m_blocks, int64_t k_tiles, bool xlds) {
+  SkinnyPlan p;
+  if (plan_override(p))
+    return p;
+  p.r = 1;
+  const int cap = xlds ? 8 : 4;
+  const int64_t wgs = row_blocks * m_blocks;
+  // 8 waves per workgroup unless the chip would be short of waves or the share per wave would exceed the cap
+  p.waves = 8;
+  if ((k_tiles + 7) / 8 > cap)
+    p.waves = 16;
+  (void)wgs;
+  const int64_t share = (k_tiles + p.waves - 1) / p.waves;
+  static const int steps_x[] = {1, 2, 3, 4, 6, 8};
+  static const int steps_g[] = {2, 4};
+  p.tpw = cap;
+  if (xlds) {
+    for (int t : steps_x)
+      if (share <= t) {
+        p.tpw = t;
+        break;
+      }
+  } else {
+    for (int t : steps_g)
+      if (share <= t) {
+        p.tpw = t;
+        break;
+      }
+  }
+  return p;
 }
 
-// K is split over `waves` waves of a workgroup: enough waves to put >= ~2048 of them on the chip (256 CUs x 8)
-// while leaving each at least two tiles.
-static int pick_waves(int64_t row_blocks, int64_t m_blocks, int64_t k_tiles) {
-  int64_t wgs = row_blocks * m_blocks;
-  int waves = 4;
-  while (waves < 16 && wgs * waves < 2048 && k_tiles >= 4 * waves)
-    waves *= 2;
-  return waves;
+template <int BITS, int DT, int GPT, int W, int T, int R_, bool XLDS>
+static void launch_instance(const SkinnyArgs &a, int64_t m_blocks, size_t lds_bytes, hipStream_t st) {
+  auto kfn = a16_skinny_kernel<BITS, DT, GPT, W, T, R_, XLDS>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    attr_set = true;
+  }
+  dim3 grid((unsigned)((a.row_blocks + R_ - 1) / R_), (unsigned)m_blocks);
+  kfn<<<grid, dim3(W * 64), lds_bytes, st>>>(a);
+}
+
+#define MI_SKINNY_CASE(W, T, R_)                                                    \
+  if (plan.waves == W && plan.tpw == T && plan.r == R_) {                           \
+    launch_instance<BITS, DT, GPT, W, T, R_, XLDS>(a, m_blocks, lds_bytes, st);     \
+    return true;                                                                    \
+  }
+
+template <int BITS, int DT, int GPT, bool XLDS>
+static bool launch_skinny(const SkinnyArgs &a, const SkinnyPlan &plan, int64_t m_blocks, size_t x_bytes,
+                          hipStream_t st) {
+  const size_t lds_bytes = skinny_red_bytes(plan.waves, plan.r) +
+                           (XLDS ? x_bytes + (BITS == 4 ? (size_t)a.k_tiles * GPT * 64 : 0) : 0);
+  MI_SKINNY_CASE(8, 2, 1)
+  MI_SKINNY_CASE(8, 4, 1)
+  MI_SKINNY_CASE(16, 2, 1)
+  MI_SKINNY_CASE(16, 4, 1)
+  if constexpr (XLDS) {
+    MI_SKINNY_CASE(8, 1, 1)
+    MI_SKINNY_CASE(8, 3, 1)
+    MI_SKINNY_CASE(8, 6, 1)
+    MI_SKINNY_CASE(8, 8, 1)
+    MI_SKINNY_CASE(16, 1, 1)
+    MI_SKINNY_CASE(16, 3, 1)
+    MI_SKINNY_CASE(16, 6, 1)
+    MI_SKINNY_CASE(16, 8, 1)
+  }
+#ifdef MI_TUNE
+  MI_SKINNY_CASE(4, 4, 1)
+  MI_SKINNY_CASE(4, 8, 1)
+  MI_SKINNY_CASE(8, 2, 2)
+  MI_SKINNY_CASE(16, 2, 2)
+  MI_SKINNY_CASE(8, 4, 2)
+  MI_SKINNY_CASE(16, 4, 2)
+  MI_SKINNY_CASE(16, 3, 2)
+#endif
+  return false;
+}
+
+template <int BITS, int DT, int GPT>
+static bool launch_skinny_x(const SkinnyArgs &a, const SkinnyPlan &plan, int64_t m_blocks, bool xlds, size_t x_bytes,
+                            hipStream_t st) {
+  return xlds ? launch_skinny<BITS, DT, GPT, true>(a, plan, m_blocks, x_bytes, st)
+              : launch_skinny<BITS, DT, GPT, false>(a, plan, m_blocks, x_bytes, st);
 }
 
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
@@ -543,10 +771,11 @@ int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t 
   MI_REQUIRE(M >= 0 && M < (1 << 20), MI_BAD_ARGUMENT, "mi_a16mm_launch: M out of range");
   if (M == 0)
     return MI_SUCCESS;
+  const int tile_k = w->bits == 4 ? W4_TILE_K : W8_TILE_K;
   SkinnyArgs a;
   a.qw = (const u32x4 *)w->qweight;
+  a.sz_t = w->sz_t;
   a.scale_t = w->scale_t;
-  a.zp_t = w->zp_t;
   a.nzs_t = w->nzs_t;
   a.bias = w->bias;
   a.x = d_x;
@@ -555,15 +784,18 @@ int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t 
   a.M = (int)M;
   a.K = w->K;
   a.N = w->N;
+  a.row_blocks = (int)w->row_blocks;
   a.k_tiles = (int)w->k_tiles;
+  a.full_tiles = (int)(w->K / tile_k);
   a.G = w->G;
   a.chip = w->chip;
   a.tiles_per_group = 1;
-  a.group_k = (int)w->K;
   const int64_t m_blocks = (M + 15) / 16;
-  dim3 grid((unsigned)w->row_blocks, (unsigned)m_blocks);
-  const int waves = pick_waves(w->row_blocks, m_blocks, w->k_tiles);
+  const size_t x_bytes = skinny_x_bytes((int)(M < 16 ? M : 16), w->k_tiles, tile_k);
+  const bool xlds = x_bytes <= XLDS_MAX_BYTES && !getenv("MI_A16_NO_XLDS");
+  const SkinnyPlan plan = pick_plan(w->row_blocks, m_blocks, w->k_tiles, xlds);
   const bool f16 = w->dtype == MI_DT_F16;
+  bool ok;
   if (w->bits == 4) {
     int gpt = 1;
     if (w->g == 0)
@@ -573,23 +805,30 @@ int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t 
     else
       gpt = W4_TILE_K / w->g;
     if (gpt == 1)
-      f16 ? launch_w4<MI_DT_F16, 1>(a, waves, grid, stream) : launch_w4<MI_DT_BF16, 1>(a, waves, grid, stream);
+      ok = f16 ? launch_skinny_x<4, MI_DT_F16, 1>(a, plan, m_blocks, xlds, x_bytes, stream)
+               : launch_skinny_x<4, MI_DT_BF16, 1>(a, plan, m_blocks, xlds, x_bytes, stream);
     else if (gpt == 2)
-      f16 ? launch_w4<MI_DT_F16, 2>(a, waves, grid, stream) : launch_w4<MI_DT_BF16, 2>(a, waves, grid, stream);
+      ok = f16 ? launch_skinny_x<4, MI_DT_F16, 2>(a, plan, m_blocks, xlds, x_bytes, stream)
+               : launch_skinny_x<4, MI_DT_BF16, 2>(a, plan, m_blocks, xlds, x_bytes, stream);
     else
-      f16 ? launch_w4<MI_DT_F16, 4>(a, waves, grid, stream) : launch_w4<MI_DT_BF16, 4>(a, waves, grid, stream);
+      ok = f16 ? launch_skinny_x<4, MI_DT_F16, 4>(a, plan, m_blocks, xlds, x_bytes, stream)
+               : launch_skinny_x<4, MI_DT_BF16, 4>(a, plan, m_blocks, xlds, x_bytes, stream);
   } else {
     int gpt = 1;
-    if (w->g != 0) {
-      a.group_k = w->g;
-      if (w->g < W8_TILE_K)
-        gpt = 2;
-    }
-    if (gpt == 1)
-      f16 ? launch_w8<MI_DT_F16, 1>(a, waves, grid, stream) : launch_w8<MI_DT_BF16, 1>(a, waves, grid, stream);
+    if (w->g == 0)
+      a.tiles_per_group = (int)w->k_tiles;
+    else if (w->g >= W8_TILE_K)
+      a.tiles_per_group = w->g / W8_TILE_K;
     else
-      f16 ? launch_w8<MI_DT_F16, 2>(a, waves, grid, stream) : launch_w8<MI_DT_BF16, 2>(a, waves, grid, stream);
+      gpt = W8_TILE_K / w->g;
+    if (gpt == 1)
+      ok = f16 ? launch_skinny_x<8, MI_DT_F16, 1>(a, plan, m_blocks, xlds, x_bytes, stream)
+               : launch_skinny_x<8, MI_DT_BF16, 1>(a, plan, m_blocks, xlds, x_bytes, stream);
+    else
+      ok = f16 ? launch_skinny_x<8, MI_DT_F16, 2>(a, plan, m_blocks, xlds, x_bytes, stream)
+               : launch_skinny_x<8, MI_DT_BF16, 2>(a, plan, m_blocks, xlds, x_bytes, stream);
   }
+  MI_REQUIRE(ok, MI_UNSUPPORTED, "mi_a16mm_launch: no kernel instance for the requested plan");
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;
 }

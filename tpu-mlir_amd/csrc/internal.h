@@ -48,10 +48,10 @@ struct mi_a16_weight {
   int64_t k_tiles = 0;     // ceil(K / TILE_K)
   // [row_blocks][k_tiles][64 lanes][16 B]
   void *qweight = nullptr;
-  // [row_blocks][G][16] scale bit patterns (bf16/f16)
+  // 4-bit: [row_blocks][G][16] u32 = scale bit pattern (bf16/f16) << 16 | zero point
+  uint32_t *sz_t = nullptr;
+  // 8-bit: [row_blocks][G][16] scale bit patterns
   uint16_t *scale_t = nullptr;
-  // 4-bit: [row_blocks][G][16] zero points (u8).  8-bit: unused.
-  uint8_t *zp_t = nullptr;
   // 8-bit: [row_blocks][G][16] float, -(zp + bias_of_unsigned_storage) * scale (exact in f32)
   float *nzs_t = nullptr;
   float *bias = nullptr;  // [N] or null
