@@ -6,6 +6,8 @@
 // that domain int32 accumulation is bit-identical.  Zero points are folded algebraically:
 //   sum (a - izp)(b - rzp) = sum a*b - izp * colsum_b[n] - rzp * rowsum_a[m] + K * izp * rzp
 // and uint8 operands are re-biased to int8 (x ^ 0x80, zero point - 128) while they are staged into LDS.
+#include <stdlib.h>
+
 #include "device_math.cuh"
 #include "internal.h"
 
@@ -225,6 +227,247 @@ __global__ __launch_bounds__(256) void i8_gemm_kernel(I8Args a) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Large-tile kernel: 256x256 outputs per workgroup, 4 waves (2x2), each wave 128x128 as 4x4 MFMA 32x32x32 blocks
+// (256 int32 accumulators per lane).  K advances 64 bytes per stage through a 4-stage LDS ring (32 KiB per stage)
+// that is filled by direct-to-LDS 16-byte loads: no staging registers and no LDS store instructions.  The 16-byte
+// chunks of a row are XOR-swizzled with (row >> 2) & 3 so that the fragment reads (32 consecutive rows, one
+// chunk) hit distinct banks.  Requires K % 64 == 0; rows past M/N are clamped (their results are never stored).
+// Workgroups are renumbered so that the 32 (or so) workgroups that land on one XCD cover a compact block of
+// output tiles and share their A/B panels through that XCD's L2.
+// ------------------------------------------------------------------------------------------------
+constexpr int LM = 256, LN = 256, LK = 64, LSTAGES = 4;
+constexpr int LSTAGE_BYTES = (LM + LN) * LK;  // 32 KiB
+enum { EPI_INT32 = 0, EPI_Q31_HALF_AWAY = 1, EPI_GENERIC = 2 };
+
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+__device__ __forceinline__ void wait_vmcnt_16() { __builtin_amdgcn_s_waitcnt(0x4F70); }  // vmcnt(16) only
+__device__ __forceinline__ void wait_vmcnt_8() { __builtin_amdgcn_s_waitcnt(0x0F78); }   // vmcnt(8) only
+__device__ __forceinline__ void wait_vmcnt_0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+template <int EPI>
+__global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int tiles_m, int tiles_n, int per_xcd) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // workgroup -> tile: hardware deals workgroups round-robin over the 8 XCDs; give each XCD a contiguous range of
+  // the tile order, and order tiles in groups of 4 tile-rows (column-major inside a group)
+  const int bid = blockIdx.x;
+  const int L = (bid & 7) * per_xcd + (bid >> 3);
+  if (L >= tiles_m * tiles_n)
+    return;
+  constexpr int GM = 4;
+  const int group = L / (GM * tiles_n);
+  const int gm = (tiles_m - group * GM) < GM ? (tiles_m - group * GM) : GM;
+  const int in_group = L - group * GM * tiles_n;
+  const int tm = group * GM + in_group % gm, tn = in_group / gm;
+  const int64_t m_base = (int64_t)tm * LM, n_base = (int64_t)tn * LN;
+
+  // direct-to-LDS load plan: per stage and operand 1024 chunks of 16 B; instruction i of wave w fills slots
+  // [(i*4+w)*64, +64); slot s holds row s/4, position s%4, i.e. logical chunk (s%4) ^ ((row>>2)&3)
+  const uint8_t *ga[4], *gb[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int slot = (i * 4 + wave) * 64 + lane;
+    const int row = slot >> 2, pos = slot & 3;
+    const int chunk = pos ^ ((row >> 2) & 3);
+    int64_t ra = m_base + row, rb = n_base + row;
+    ra = ra < a.M ? ra : a.M - 1;
+    rb = rb < a.N ? rb : a.N - 1;
+    ga[i] = a.A + ra * a.K + chunk * 16;
+    gb[i] = a.B + rb * a.K + chunk * 16;
+  }
+  const int kt_total = (int)(a.K / LK);
+  auto issue_stage = [&](int kt, int buf) {
+    const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 1) * LK;  // past the end: harmless re-load
+    uint8_t *sa = lds + buf * LSTAGE_BYTES, *sb = sa + LM * LK;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      __builtin_amdgcn_global_load_lds((gptr_t)(ga[i] + koff), (lptr_t)(sa + (i * 4 + wave) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(gb[i] + koff), (lptr_t)(sb + (i * 4 + wave) * 1024), 16, 0, 0);
+    }
+  };
+
+  i32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[i][j][r] = 0;
+
+  // fragment addressing: lane reads row (lane & 31) of a 32-row block, logical chunk ks*2 + (lane >> 5)
+  const int frow = lane & 31, fhalf = lane >> 5;
+  int a_off[4], b_off[4];  // byte offsets of the row inside a stage (without the chunk position)
+  int a_sw[4], b_sw[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ra = wm * 128 + i * 32 + frow, rb = wn * 128 + i * 32 + frow;
+    a_off[i] = ra * LK;
+    b_off[i] = LM * LK + rb * LK;
+    a_sw[i] = (ra >> 2) & 3;
+    b_sw[i] = (rb >> 2) & 3;
+  }
+
+  auto read_frags = [&](i32x4 (&fa)[4], i32x4 (&fb)[4], const uint8_t *st, int ks) {
+    const int c = ks * 2 + fhalf;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      fa[i] = *(const i32x4 *)(st + a_off[i] + ((c ^ a_sw[i]) << 4));
+      fb[i] = *(const i32x4 *)(st + b_off[i] + ((c ^ b_sw[i]) << 4));
+    }
+  };
+  auto mma = [&](const i32x4 (&fa)[4], const i32x4 (&fb)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+  };
+
+  // Software pipeline.  Stage s lives in ring buffer s & 3 and is requested three stages ahead.  The barrier sits
+  // in the MIDDLE of an iteration: the fragments of the second k-step are already on their way when a wave
+  // arrives, and the first fragments of the next stage are requested right after it, so every batch of 16 MFMAs
+  // runs with the next batch's LDS reads in flight.
+#pragma unroll
+  for (int s = 0; s < LSTAGES - 1; ++s)
+    issue_stage(s, s);
+  i32x4 fa0[4], fb0[4], fa1[4], fb1[4];
+  wait_vmcnt_16();  // stage 0 landed (stages 1 and 2 may still be in flight)
+  __builtin_amdgcn_s_barrier();
+  read_frags(fa0, fb0, lds, 0);
+  for (int kt = 0; kt < kt_total; ++kt) {
+    const uint8_t *st = lds + (kt & (LSTAGES - 1)) * LSTAGE_BYTES;
+    read_frags(fa1, fb1, st, 1);
+    __builtin_amdgcn_sched_barrier(0);  // keep the LDS reads ahead of the MFMA batch they overlap with
+    mma(fa0, fb0);
+    __builtin_amdgcn_sched_barrier(0);
+    wait_vmcnt_8();  // this thread's part of stage kt+1 landed (stage kt+2 may still be in flight)
+    // after the barrier everybody's part has, and everybody is done with the buffer of stage kt-1.  A bare
+    // s_barrier: __syncthreads() carries a fence that would drain every outstanding load (vmcnt(0)).
+    __builtin_amdgcn_s_barrier();
+    issue_stage(kt + LSTAGES - 1, (kt + LSTAGES - 1) & (LSTAGES - 1));
+    read_frags(fa0, fb0, lds + ((kt + 1) & (LSTAGES - 1)) * LSTAGE_BYTES, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(fa1, fb1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  wait_vmcnt_0();  // drain the re-loads issued past the end before the workgroup may exit
+
+  // Epilogue.  Register r of lane l in block (i, j) is row 8*(r/4) + 4*(l/32) + (r%4), column l%32 -- a layout
+  // that would store 32-byte row fragments.  Each wave instead passes one 32 x 128 strip at a time through its own
+  // LDS region (row stride 132 dwords) and re-reads it so that a lane owns 16 consecutive columns of a row: the
+  // per-column requant parameters are then loaded once per lane and the int8 result leaves as 16-byte stores.
+  __syncthreads();  // every wave is done with the stage buffers
+  int32_t *strip = reinterpret_cast<int32_t *>(lds) + wave * (32 * 132);
+  const int cc = lane & 7, rsub = lane >> 3;  // column chunk (16 columns) and row within a group of 8 rows
+  const int64_t n0 = n_base + wn * 128 + cc * 16;
+  const bool vec_ok = (a.N % 16) == 0 && n0 + 16 <= a.N;
+  int32_t p_bias[16], p_mult[16], p_shift[16], p_zp[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int64_t n = (n0 + e) < a.N ? (n0 + e) : (a.N - 1);
+    p_bias[e] = a.bias ? a.bias[n] : 0;
+    if constexpr (EPI == EPI_Q31_HALF_AWAY) {
+      p_mult[e] = a.rq.mult ? a.rq.mult[n] : a.rq.mult_s;
+      p_shift[e] = a.rq.shift ? a.rq.shift[n] : a.rq.shift_s;
+      p_zp[e] = a.rq.zp ? a.rq.zp[n] : a.rq.zp_s;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        strip[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * 132 + j * 32 + (lane & 31)] = acc[i][j][r];
+    // same-wave LDS traffic is ordered; the compiler waits on lgkmcnt before the reads below
+    for (int it = 0; it < 4; ++it) {
+      const int row = it * 8 + rsub;
+      const int64_t m = m_base + wm * 128 + i * 32 + row;
+      int32_t v[16];
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const i32x4 t = *(const i32x4 *)(strip + row * 132 + cc * 16 + q4 * 4);
+        v[q4 * 4 + 0] = t[0];
+        v[q4 * 4 + 1] = t[1];
+        v[q4 * 4 + 2] = t[2];
+        v[q4 * 4 + 3] = t[3];
+      }
+      if (m >= a.M || n0 >= a.N)
+        continue;
+      const int32_t rt = a.row_term ? a.row_term[m] : 0;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        int32_t x = v[e] + p_bias[e] + rt;
+        if (a.do_relu) {
+          x = x > 0 ? x : 0;
+          if (a.relu_limit > 0 && x > a.relu_limit)
+            x = (int32_t)a.relu_limit;
+        }
+        v[e] = x;
+      }
+      const int64_t o = m * a.N + n0;
+      if (a.acc_out) {
+        if (vec_ok) {
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4)
+            *(i32x4 *)(a.acc_out + o + q4 * 4) = i32x4{v[q4 * 4], v[q4 * 4 + 1], v[q4 * 4 + 2], v[q4 * 4 + 3]};
+        } else {
+          for (int e = 0; e < 16; ++e)
+            if (n0 + e < a.N)
+              a.acc_out[o + e] = v[e];
+        }
+      }
+      if constexpr (EPI == EPI_INT32) {
+        if (a.out) {
+          int32_t *out = (int32_t *)a.out;
+          if (vec_ok) {
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4)
+              *(i32x4 *)(out + o + q4 * 4) = i32x4{v[q4 * 4], v[q4 * 4 + 1], v[q4 * 4 + 2], v[q4 * 4 + 3]};
+          } else {
+            for (int e = 0; e < 16; ++e)
+              if (n0 + e < a.N)
+                out[o + e] = v[e];
+          }
+        }
+      } else if constexpr (EPI == EPI_Q31_HALF_AWAY) {
+        // MultiplyByQuantizedMultiplier(x, mult, -shift, HALF_AWAY) with shift in [1, 31], in 32-bit steps:
+        // t = (x*mult + 2^30) >> 31 fits int32 for |x|, mult < 2^31, so the reference's clamp never fires, and
+        // half-away rounding of t >> shift is (t + half + (t >> 31)) >> shift.
+        uint32_t packed[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int64_t p = (int64_t)v[e] * (int64_t)p_mult[e] + (1ll << 30);
+          const int32_t t = (int32_t)(p >> 31);
+          int32_t q = (t + (1 << (p_shift[e] - 1)) + (t >> 31)) >> p_shift[e];
+          q += p_zp[e];
+          q = q < -128 ? -128 : (q > 127 ? 127 : q);
+          packed[e >> 2] |= (uint32_t)(q & 0xff) << (8 * (e & 3));
+        }
+        int8_t *out = (int8_t *)a.out;
+        if (vec_ok) {
+          *(u32x4 *)(out + o) = u32x4{packed[0], packed[1], packed[2], packed[3]};
+        } else {
+          for (int e = 0; e < 16; ++e)
+            if (n0 + e < a.N)
+              out[o + e] = (int8_t)((packed[e >> 2] >> (8 * (e & 3))) & 0xff);
+        }
+      } else {
+        for (int e = 0; e < 16; ++e)
+          if (n0 + e < a.N)
+            store_out(a.out, o + e, requant_one(v[e], n0 + e, a.rq), a.rq.out_dtype);
+      }
+    }
+  }
+}
+
 static RequantParams make_rq(const mi_requant_desc *rq) {
   RequantParams p;
   p.mult = rq->d_multiplier;
@@ -319,8 +562,44 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
     a.rq = make_rq(rq);
   else
     a.rq = RequantParams{nullptr, nullptr, nullptr, 1, 0, 0, MI_RQ_MULTIPLIER_SHIFT, 0, 0, MI_DT_I32};
-  dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
-  i8_gemm_kernel<<<grid, dim3(256), 0, stream>>>(a);
+  const bool large = (K % LK) == 0 && M >= 128 && N >= 128 && !getenv("MI_I8_SMALL_TILE");
+  if (large) {
+    const int tiles_m = (int)((M + LM - 1) / LM), tiles_n = (int)((N + LN - 1) / LN);
+    const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+    const size_t lds_bytes = (size_t)LSTAGES * LSTAGE_BYTES;
+    int epi = EPI_INT32;
+    if (rq) {
+      const bool q31 = rq->quant_mode == MI_RQ_QDM || rq->quant_mode == MI_RQ_TFLITE ||
+                       rq->quant_mode == MI_RQ_TFLITE_LSHIFT;
+      // the 32-bit fast path needs a right shift in [1, 31] on every channel; per-channel shifts are the
+      // caller's device array, so it is only taken for a scalar shift or when the caller vouches via the desc
+      epi = (q31 && rq->round_mode == MI_ROUND_HALF_AWAY_FROM_ZERO && rq->out_dtype == MI_DT_I8 &&
+             (rq->d_shift || (rq->shift >= 1 && rq->shift <= 31)))
+                ? EPI_Q31_HALF_AWAY
+                : EPI_GENERIC;
+    }
+    dim3 grid((unsigned)(per_xcd * 8));
+#define MI_LARGE(E)                                                                                         \
+  {                                                                                                         \
+    static bool attr_set = false;                                                                           \
+    if (!attr_set) {                                                                                        \
+      (void)hipFuncSetAttribute((const void *)i8_gemm_large_kernel<E>,                                      \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                    \
+      attr_set = true;                                                                                      \
+    }                                                                                                       \
+    i8_gemm_large_kernel<E><<<grid, dim3(256), lds_bytes, stream>>>(a, tiles_m, tiles_n, per_xcd);          \
+  }
+    if (epi == EPI_INT32)
+      MI_LARGE(EPI_INT32)
+    else if (epi == EPI_Q31_HALF_AWAY)
+      MI_LARGE(EPI_Q31_HALF_AWAY)
+    else
+      MI_LARGE(EPI_GENERIC)
+#undef MI_LARGE
+  } else {
+    dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
+    i8_gemm_kernel<<<grid, dim3(256), 0, stream>>>(a);
+  }
   MI_HIP(hipGetLastError());
   if (bt)
     MI_HIP(hipFreeAsync(bt, stream));
