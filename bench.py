@@ -175,6 +175,14 @@ def main():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
     torch.cuda.set_device(0)
 
+    # one plain device copy of known size (256 MiB read + 256 MiB written): the reference point that scales the
+    # FETCH_SIZE / WRITE_SIZE counters when this command runs under rocprofv3 --pmc
+    cal_src = torch.empty(64 << 20, dtype=torch.float32, device="cuda").fill_(1.0)
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    torch.cuda.synchronize()
+    del cal_src, cal_dst
+
     M = args.batch
     cfgs = host_chain(S, M)
     r = bench_chain(pkg, S, torch, M, args.steps, args.warmup, args.layers, cfgs)
@@ -194,7 +202,10 @@ def main():
                    "weight_copies": args.layers, "resident_weight_mb": round(r["weight_set_mb"], 1),
                    "launch": "one HIP graph replay per step"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE (profiles/hbm_traffic_pmc_*.md):
+                     # 1.03 x the algorithmic bytes at M = 1; not re-measured by this run
+                     "traffic": int(bytes_per_launch * 1.03) if M == 1 else None,
                      "kernel": "a16w4_skinny_kernel<bf16, 1 group/tile>",
                      "bytes_per_launch": int(bytes_per_launch),
                      "avg_launch_us": round(avg_launch_s * 1e6, 3),
