@@ -236,19 +236,34 @@ __global__ __launch_bounds__(256) void i8_gemm_kernel(I8Args a) {
 // Workgroups are renumbered so that the 32 (or so) workgroups that land on one XCD cover a compact block of
 // output tiles and share their A/B panels through that XCD's L2.
 // ------------------------------------------------------------------------------------------------
-constexpr int LM = 256, LN = 256, LK = 64, LSTAGES = 4;
-constexpr int LSTAGE_BYTES = (LM + LN) * LK;  // 32 KiB
+constexpr int LM = 256, LN = 256;
 enum { EPI_INT32 = 0, EPI_Q31_HALF_AWAY = 1, EPI_GENERIC = 2 };
 
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
-__device__ __forceinline__ void wait_vmcnt_16() { __builtin_amdgcn_s_waitcnt(0x4F70); }  // vmcnt(16) only
-__device__ __forceinline__ void wait_vmcnt_8() { __builtin_amdgcn_s_waitcnt(0x0F78); }   // vmcnt(8) only
-__device__ __forceinline__ void wait_vmcnt_0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// s_waitcnt immediates (gfx9 encoding): wait for vmcnt <= n only / for lgkmcnt == 0 only
+constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
+constexpr int WAITCNT_LGKM0 = 0xC07F;
 
-template <int EPI>
+#ifndef MI_I8_DBG
+#define MI_I8_DBG 0  // development switches: 1 no global loads, 2 no fragment reads, 4 no MFMA
+#endif
+#ifdef MI_I8_TIMING
+__device__ unsigned long long mi_i8_dbg[64 * 4 * 4];
+extern "C" int mi_i8_dbg_dump(unsigned long long *host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mi_i8_dbg), sizeof(mi_i8_dbg));
+}
+#endif
+
+// LK_ = bytes of K per stage (64 or 128), NST = stages in the LDS ring (NST * 512 * LK_ bytes)
+template <int EPI, int LK_, int NST>
 __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int tiles_m, int tiles_n, int per_xcd) {
+  constexpr int CH = LK_ / 16;                // 16-byte chunks per row
+  constexpr int KS = LK_ / 32;                // MFMA k-steps per stage
+  constexpr int LOADS = LM * CH / 256;        // direct-to-LDS instructions per operand, stage and wave
+  constexpr int LPS = 2 * LOADS;              // loads per thread and stage
+  constexpr int STAGE_BYTES = (LM + LN) * LK_;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -267,28 +282,41 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
   const int tm = group * GM + in_group % gm, tn = in_group / gm;
   const int64_t m_base = (int64_t)tm * LM, n_base = (int64_t)tn * LN;
 
-  // direct-to-LDS load plan: per stage and operand 1024 chunks of 16 B; instruction i of wave w fills slots
-  // [(i*4+w)*64, +64); slot s holds row s/4, position s%4, i.e. logical chunk (s%4) ^ ((row>>2)&3)
-  const uint8_t *ga[4], *gb[4];
+  // Row swizzle: the 16-byte chunk c of row r is stored at position c ^ sw(r) so that 16 consecutive rows reading
+  // the same logical chunk touch 16 different 16-byte bank groups.
+  auto sw = [](int row) { return LK_ == 64 ? ((row >> 2) & 3) : ((row >> 1) & 7); };
+
+  // direct-to-LDS load plan: instruction i of wave w fills slots [(i*4+w)*64, +64) of an operand's stage;
+  // slot s is row s / CH, position s % CH
+  const uint8_t *ga[LOADS], *gb[LOADS];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < LOADS; ++i) {
     const int slot = (i * 4 + wave) * 64 + lane;
-    const int row = slot >> 2, pos = slot & 3;
-    const int chunk = pos ^ ((row >> 2) & 3);
+    const int row = slot / CH, pos = slot % CH;
+    const int chunk = pos ^ sw(row);
     int64_t ra = m_base + row, rb = n_base + row;
-    ra = ra < a.M ? ra : a.M - 1;
+    ra = ra < a.M ? ra : a.M - 1;  // rows past the matrix re-read the last row; their results are never stored
     rb = rb < a.N ? rb : a.N - 1;
     ga[i] = a.A + ra * a.K + chunk * 16;
     gb[i] = a.B + rb * a.K + chunk * 16;
   }
-  const int kt_total = (int)(a.K / LK);
-  auto issue_stage = [&](int kt, int buf) {
-    const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 1) * LK;  // past the end: harmless re-load
-    uint8_t *sa = lds + buf * LSTAGE_BYTES, *sb = sa + LM * LK;
+  const int kt_total = (int)(a.K / LK_);
+  // A stage is requested in KS parts (one per MFMA batch) so that its direct-to-LDS instructions are spread over a
+  // whole stage's worth of MFMAs instead of queueing up behind one batch.
+  constexpr int PART = LOADS / KS;
+  static_assert(PART * KS == LOADS, "loads per operand must split evenly over the k-steps");
+  auto issue_part = [&](int kt, int part) {
+    const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 1) * LK_;  // past the end: harmless re-load
+    uint8_t *sa = lds + (kt % NST) * STAGE_BYTES, *sb = sa + LM * LK_;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = part * PART; i < (part + 1) * PART; ++i) {
+#if defined(MI_I8_DBG) && (MI_I8_DBG & 64)  // every load re-reads the same 2 KiB: vector-cache hits
+      __builtin_amdgcn_global_load_lds((gptr_t)(ga[0]), (lptr_t)(sa + (i * 4 + wave) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(gb[0]), (lptr_t)(sb + (i * 4 + wave) * 1024), 16, 0, 0);
+#else
       __builtin_amdgcn_global_load_lds((gptr_t)(ga[i] + koff), (lptr_t)(sa + (i * 4 + wave) * 1024), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((gptr_t)(gb[i] + koff), (lptr_t)(sb + (i * 4 + wave) * 1024), 16, 0, 0);
+#endif
     }
   };
 
@@ -308,13 +336,14 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int ra = wm * 128 + i * 32 + frow, rb = wn * 128 + i * 32 + frow;
-    a_off[i] = ra * LK;
-    b_off[i] = LM * LK + rb * LK;
-    a_sw[i] = (ra >> 2) & 3;
-    b_sw[i] = (rb >> 2) & 3;
+    a_off[i] = ra * LK_;
+    b_off[i] = LM * LK_ + rb * LK_;
+    a_sw[i] = sw(ra);
+    b_sw[i] = sw(rb);
   }
 
-  auto read_frags = [&](i32x4 (&fa)[4], i32x4 (&fb)[4], const uint8_t *st, int ks) {
+  auto read_frags = [&](i32x4 (&fa)[4], i32x4 (&fb)[4], int kt, int ks) {
+    const uint8_t *st = lds + (kt % NST) * STAGE_BYTES;
     const int c = ks * 2 + fhalf;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -322,52 +351,135 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
       fb[i] = *(const i32x4 *)(st + b_off[i] + ((c ^ b_sw[i]) << 4));
     }
   };
-  auto mma = [&](const i32x4 (&fa)[4], const i32x4 (&fb)[4]) {
+  // One batch: the 16 MFMAs of k-step `cur` with, pinned between them in this order, the 8 fragment reads of the
+  // next k-step (in the order the next batch consumes them) and one part of a future stage's loads.  The explicit
+  // scheduling barriers keep the compiler from clumping the memory instructions at the head of the batch, where
+  // they would hold up MFMA issue.
+  auto batch = [&](const i32x4 (&ca)[4], const i32x4 (&cb)[4], i32x4 (&na)[4], i32x4 (&nb)[4], int rkt, int rks,
+                   int lkt, int lpart) {
+    const uint8_t *st = lds + (rkt % NST) * STAGE_BYTES;
+    const int c = rks * 2 + fhalf;
+    const int64_t koff = (int64_t)(lkt < kt_total ? lkt : kt_total - 1) * LK_;  // past the end: harmless re-load
+    uint8_t *sa = lds + (lkt % NST) * STAGE_BYTES, *sb = sa + LM * LK_;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int t = 0; t < 16; ++t) {
+      const int i = t >> 2, j = t & 3;
+#if !(MI_I8_DBG & 4)
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ca[i], cb[j], acc[i][j], 0, 0, 0);
+#endif
+#if !(MI_I8_DBG & 2)
+      if (t == 0)
+        na[0] = *(const i32x4 *)(st + a_off[0] + ((c ^ a_sw[0]) << 4));
+      else if (t <= 4)
+        nb[t - 1] = *(const i32x4 *)(st + b_off[t - 1] + ((c ^ b_sw[t - 1]) << 4));
+      else if (t <= 7)
+        na[t - 4] = *(const i32x4 *)(st + a_off[t - 4] + ((c ^ a_sw[t - 4]) << 4));
+#endif
+#if !(MI_I8_DBG & 1)
+      if (t >= 8) {
+        constexpr int SLOTS = 8, N_LD = 2 * PART;  // loads of this part, spread over the last 8 MFMAs
+        const int q0 = (t - 8) * N_LD / SLOTS, q1 = (t - 7) * N_LD / SLOTS;
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        for (int q = q0; q < q1; ++q) {
+          const int li = lpart * PART + (q >> 1);
+          if (q & 1)
+            __builtin_amdgcn_global_load_lds((gptr_t)(gb[li] + koff), (lptr_t)(sb + (li * 4 + wave) * 1024), 16, 0,
+                                             0);
+          else
+            __builtin_amdgcn_global_load_lds((gptr_t)(ga[li] + koff), (lptr_t)(sa + (li * 4 + wave) * 1024), 16, 0,
+                                             0);
+        }
+      }
+#endif
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
 
-  // Software pipeline.  Stage s lives in ring buffer s & 3 and is requested three stages ahead.  The barrier sits
-  // in the MIDDLE of an iteration: the fragments of the second k-step are already on their way when a wave
-  // arrives, and the first fragments of the next stage are requested right after it, so every batch of 16 MFMAs
-  // runs with the next batch's LDS reads in flight.
+  // Software pipeline.  Stage s lives in ring buffer s % NST.  Each batch of 16 MFMAs (one k-step) runs with the
+  // next batch's fragment reads in flight (two fragment register sets alternate) and with one part of a future
+  // stage's loads slotted between its MFMAs.  The one barrier per stage sits before the LAST batch of stage kt: by
+  // then every wave has received that stage's last fragments (lgkmcnt(0)) and its own share of stage kt+1 (vmcnt),
+  // so after the barrier buffer kt % NST is free and stage kt+1 is complete.  Stage kt+NST is then requested in
+  // parts: part 0 in this last batch, parts 1.. in the first KS-1 batches of stage kt+1; it is needed NST-2 full
+  // stages after its last part went out.  A bare s_barrier is used: __syncthreads() carries a fence that would
+  // drain every outstanding load (vmcnt(0)).
+  static_assert(NST >= 3, "the spread-out stage requests need two stages of slack");
 #pragma unroll
-  for (int s = 0; s < LSTAGES - 1; ++s)
-    issue_stage(s, s);
-  i32x4 fa0[4], fb0[4], fa1[4], fb1[4];
-  wait_vmcnt_16();  // stage 0 landed (stages 1 and 2 may still be in flight)
+  for (int s = 0; s < NST - 1; ++s)
+#pragma unroll
+    for (int part = 0; part < KS; ++part)
+      issue_part(s, part);
+  issue_part(NST - 1, 0);
+  i32x4 fa[2][4], fb[2][4];
+#ifdef MI_I8_TIMING
+  unsigned long long t_lgkm = 0, t_vm = 0, t_bar = 0;
+  const unsigned long long t_begin = __builtin_readcyclecounter();
+#endif
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm((NST - 2) * LPS + 2 * PART));  // stage 0 landed
   __builtin_amdgcn_s_barrier();
-  read_frags(fa0, fb0, lds, 0);
+  read_frags(fa[0], fb[0], 0, 0);
   for (int kt = 0; kt < kt_total; ++kt) {
-    const uint8_t *st = lds + (kt & (LSTAGES - 1)) * LSTAGE_BYTES;
-    read_frags(fa1, fb1, st, 1);
-    __builtin_amdgcn_sched_barrier(0);  // keep the LDS reads ahead of the MFMA batch they overlap with
-    mma(fa0, fb0);
-    __builtin_amdgcn_sched_barrier(0);
-    wait_vmcnt_8();  // this thread's part of stage kt+1 landed (stage kt+2 may still be in flight)
-    // after the barrier everybody's part has, and everybody is done with the buffer of stage kt-1.  A bare
-    // s_barrier: __syncthreads() carries a fence that would drain every outstanding load (vmcnt(0)).
-    __builtin_amdgcn_s_barrier();
-    issue_stage(kt + LSTAGES - 1, (kt + LSTAGES - 1) & (LSTAGES - 1));
-    read_frags(fa0, fb0, lds + ((kt + 1) & (LSTAGES - 1)) * LSTAGE_BYTES, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(fa1, fb1);
-    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 1 < KS) {
+        batch(fa[ks & 1], fb[ks & 1], fa[(ks + 1) & 1], fb[(ks + 1) & 1], kt, ks + 1, kt + NST - 1, ks + 1);
+      } else {
+#ifdef MI_I8_TIMING
+        const unsigned long long tw0 = __builtin_readcyclecounter();
+#endif
+        __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);
+#ifdef MI_I8_TIMING
+        const unsigned long long tw1 = __builtin_readcyclecounter();
+#endif
+#if !(MI_I8_DBG & 1)
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm((NST - 2) * LPS));  // this thread's share of stage kt+1 landed
+#endif
+#ifdef MI_I8_TIMING
+        const unsigned long long tw2 = __builtin_readcyclecounter();
+#endif
+        __builtin_amdgcn_s_barrier();
+#ifdef MI_I8_TIMING
+        const unsigned long long tw3 = __builtin_readcyclecounter();
+        t_lgkm += tw1 - tw0;
+        t_vm += tw2 - tw1;
+        t_bar += tw3 - tw2;
+#endif
+        batch(fa[ks & 1], fb[ks & 1], fa[(ks + 1) & 1], fb[(ks + 1) & 1], kt + 1, 0, kt + NST, 0);
+      }
+    }
   }
-  wait_vmcnt_0();  // drain the re-loads issued past the end before the workgroup may exit
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // drain the re-loads issued past the end before the workgroup may exit
+#ifdef MI_I8_TIMING
+  if (lane == 0 && blockIdx.x < 64) {
+    const unsigned long long t_end = __builtin_readcyclecounter();
+    unsigned long long *d = mi_i8_dbg + (blockIdx.x * 4 + wave) * 4;
+    d[0] = t_end - t_begin;
+    d[1] = t_lgkm;
+    d[2] = t_vm;
+    d[3] = t_bar;
+  }
+#endif
 
   // Epilogue.  Register r of lane l in block (i, j) is row 8*(r/4) + 4*(l/32) + (r%4), column l%32 -- a layout
   // that would store 32-byte row fragments.  Each wave instead passes one 32 x 128 strip at a time through its own
   // LDS region (row stride 132 dwords) and re-reads it so that a lane owns 16 consecutive columns of a row: the
   // per-column requant parameters are then loaded once per lane and the int8 result leaves as 16-byte stores.
   __syncthreads();  // every wave is done with the stage buffers
+#if defined(MI_I8_DBG) && (MI_I8_DBG & 8)
+  {
+    if (acc[0][0][0] == 0x7fffffff)
+      ((int32_t *)a.out)[0] = acc[1][1][1] + acc[2][2][2] + acc[3][3][3];
+    return;
+  }
+#endif
   int32_t *strip = reinterpret_cast<int32_t *>(lds) + wave * (32 * 132);
   const int cc = lane & 7, rsub = lane >> 3;  // column chunk (16 columns) and row within a group of 8 rows
   const int64_t n0 = n_base + wn * 128 + cc * 16;
   const bool vec_ok = (a.N % 16) == 0 && n0 + 16 <= a.N;
+  // relu (and its optional upper limit) as one clamp; without relu the bounds are the int32 range
+  const int32_t relu_lo = a.do_relu ? 0 : INT32_MIN;
+  const int32_t relu_hi =
+      (a.do_relu && a.relu_limit > 0 && a.relu_limit < INT32_MAX) ? (int32_t)a.relu_limit : INT32_MAX;
   int32_t p_bias[16], p_mult[16], p_shift[16], p_zp[16];
 #pragma unroll
   for (int e = 0; e < 16; ++e) {
@@ -404,13 +516,8 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
       const int32_t rt = a.row_term ? a.row_term[m] : 0;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        int32_t x = v[e] + p_bias[e] + rt;
-        if (a.do_relu) {
-          x = x > 0 ? x : 0;
-          if (a.relu_limit > 0 && x > a.relu_limit)
-            x = (int32_t)a.relu_limit;
-        }
-        v[e] = x;
+        const int32_t x = v[e] + p_bias[e] + rt;
+        v[e] = x < relu_lo ? relu_lo : (x > relu_hi ? relu_hi : x);  // one v_med3_i32
       }
       const int64_t o = m * a.N + n0;
       if (a.acc_out) {
@@ -562,11 +669,13 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
     a.rq = make_rq(rq);
   else
     a.rq = RequantParams{nullptr, nullptr, nullptr, 1, 0, 0, MI_RQ_MULTIPLIER_SHIFT, 0, 0, MI_DT_I32};
-  const bool large = (K % LK) == 0 && M >= 128 && N >= 128 && !getenv("MI_I8_SMALL_TILE");
+  const bool large = (K % 128) == 0 && M >= 128 && N >= 128 && !getenv("MI_I8_SMALL_TILE");
   if (large) {
     const int tiles_m = (int)((M + LM - 1) / LM), tiles_n = (int)((N + LN - 1) / LN);
     const int per_xcd = (tiles_m * tiles_n + 7) / 8;
-    const size_t lds_bytes = (size_t)LSTAGES * LSTAGE_BYTES;
+    const char *ring_env = getenv("MI_I8_RING");  // development switch: stages in the LDS ring (3, 4 or 5)
+    const int ring = ring_env ? atoi(ring_env) : 4;
+    const size_t lds_bytes = (size_t)(ring == 5 ? 5 : ring == 3 ? 3 : 4) * 32 * 1024;
     int epi = EPI_INT32;
     if (rq) {
       const bool q31 = rq->quant_mode == MI_RQ_QDM || rq->quant_mode == MI_RQ_TFLITE ||
@@ -579,15 +688,24 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
                 : EPI_GENERIC;
     }
     dim3 grid((unsigned)(per_xcd * 8));
-#define MI_LARGE(E)                                                                                         \
+#define MI_LARGE_I(E, LK_, NST)                                                                             \
   {                                                                                                         \
     static bool attr_set = false;                                                                           \
     if (!attr_set) {                                                                                        \
-      (void)hipFuncSetAttribute((const void *)i8_gemm_large_kernel<E>,                                      \
+      (void)hipFuncSetAttribute((const void *)i8_gemm_large_kernel<E, LK_, NST>,                            \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                    \
       attr_set = true;                                                                                      \
     }                                                                                                       \
-    i8_gemm_large_kernel<E><<<grid, dim3(256), lds_bytes, stream>>>(a, tiles_m, tiles_n, per_xcd);          \
+    i8_gemm_large_kernel<E, LK_, NST><<<grid, dim3(256), lds_bytes, stream>>>(a, tiles_m, tiles_n, per_xcd);\
+  }
+#define MI_LARGE(E)         \
+  {                         \
+    if (ring == 5)          \
+      MI_LARGE_I(E, 64, 5)  \
+    else if (ring == 3)     \
+      MI_LARGE_I(E, 64, 3)  \
+    else                    \
+      MI_LARGE_I(E, 64, 4)  \
   }
     if (epi == EPI_INT32)
       MI_LARGE(EPI_INT32)
@@ -595,6 +713,7 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
       MI_LARGE(EPI_Q31_HALF_AWAY)
     else
       MI_LARGE(EPI_GENERIC)
+#undef MI_LARGE_I
 #undef MI_LARGE
   } else {
     dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
