@@ -104,6 +104,48 @@ def test_zero_points_unsigned_operands_relu_and_int16(orc):
     want = (a.astype(np.int64) - 3) @ (bu.astype(np.int64).T - 128)
     assert np.array_equal(out.cpu().numpy().astype(np.int64), want)
 
+@pytest.mark.parametrize("rt", [True, False])
+def test_large_tile_path_unsigned_zero_points_relu_ragged_edges(orc, rt):
+    """Shapes that take the 256x256 direct-to-LDS kernel (M, N >= 128, K % 128 == 0) with everything the small
+    cases cover: unsigned operands, both zero points, bias, relu with a limit, a ragged last tile in M and N,
+    per-channel Q31 requant with per-channel output zero points, and the int32 side output."""
+    torch = _torch()
+    rng = np.random.default_rng(11)
+    M, K, N = 300, 384, 272
+    a = rng.integers(0, 256, size=(M, K)).astype(np.uint8)
+    b = rng.integers(0, 256, size=(N, K) if rt else (K, N)).astype(np.uint8)
+    bias = rng.integers(-20000, 20000, size=N).astype(np.int32)
+    izp, rzp = 121, 133
+    bm = (b.T if rt else b).astype(np.int64)
+    acc_want = (a.astype(np.int64) - izp) @ (bm - rzp) + bias
+    # int32 result
+    out = M_.i8mm_launch(_dev(a), _dev(b), _dev(bias), right_transpose=rt, input_zp=izp, right_zp=rzp)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().astype(np.int64), acc_want)
+    # relu with limit + per-channel Q31 requant (the 32-bit fast epilogue) + int32 side output
+    mult = rng.integers(1 << 30, (1 << 31) - 1, size=N).astype(np.int32)
+    shift = rng.integers(6, 12, size=N).astype(np.int32)
+    zp = rng.integers(-20, 20, size=N).astype(np.int32)
+    rq = M_.RequantDesc(clib.RQ_QDM, clib.ROUND_HALF_AWAY_FROM_ZERO, out_dtype=clib.DT_I8, multiplier=_dev(mult),
+                        shift=_dev(shift), zp=_dev(zp))
+    acc = torch.empty((M, N), dtype=torch.int32, device="cuda")
+    out = M_.i8mm_launch(_dev(a), _dev(b), _dev(bias), right_transpose=rt, input_zp=izp, right_zp=rzp, do_relu=True,
+                         relu_limit=150000, rq=rq, acc=acc)
+    torch.cuda.synchronize()
+    relu = np.clip(acc_want, 0, 150000)
+    assert np.array_equal(acc.cpu().numpy().astype(np.int64), relu)
+    v = orc.mbqm(relu, np.broadcast_to(mult.astype(np.int64), relu.shape), np.broadcast_to(-shift.astype(np.int64), relu.shape),
+                 orc.HALF_AWAY_FROM_ZERO)
+    want = _sat(v + zp[None, :], clib.DT_I8)
+    assert np.array_equal(out.cpu().numpy().astype(np.int64), want)
+    # no relu, scalar multiplier-shift to uint8 (generic epilogue)
+    rq2 = M_.RequantDesc(clib.RQ_MULTIPLIER_SHIFT, clib.ROUND_HALF_UP, out_dtype=clib.DT_U8, multiplier=77, shift=15,
+                         zp=100)
+    out = M_.i8mm_launch(_dev(a), _dev(b), _dev(bias), right_transpose=rt, input_zp=izp, right_zp=rzp, rq=rq2)
+    torch.cuda.synchronize()
+    want = _sat(orc.right_shift_round(acc_want * 77, 15, orc.HALF_UP) + 100, clib.DT_U8)
+    assert np.array_equal(out.cpu().numpy().astype(np.int64), want)
+
 
 def test_operator_level_against_oracle(orc):
     c = S.int8_matmul(48, 256, 64, seed=4, qdm=False)

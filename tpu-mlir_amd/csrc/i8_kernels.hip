@@ -38,6 +38,22 @@ __global__ void transpose_bytes_kernel(const uint8_t *__restrict__ src, uint8_t 
   }
 }
 
+// dst = src ^ 0x80 per byte: an unsigned operand u becomes the signed value u - 128 the matrix cores take
+__global__ void flip_bytes_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t n) {
+  const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 16;
+  if (i + 16 <= n) {
+    u32x4 v = *(const u32x4 *)(src + i);
+    v[0] ^= 0x80808080u;
+    v[1] ^= 0x80808080u;
+    v[2] ^= 0x80808080u;
+    v[3] ^= 0x80808080u;
+    *(u32x4 *)(dst + i) = v;
+  } else {
+    for (int64_t j = i; j < n; ++j)
+      dst[j] = src[j] ^ 0x80;
+  }
+}
+
 // sums[r] = sum_k (signed or unsigned) x[r, k]; one wave per row
 __global__ void row_sums_kernel(const uint8_t *__restrict__ x, int is_unsigned, int32_t *__restrict__ sums,
                                 int64_t rows, int64_t K) {
@@ -250,11 +266,26 @@ constexpr int WAITCNT_LGKM0 = 0xC07F;
 #define MI_I8_DBG 0  // development switches: 1 no global loads, 2 no fragment reads, 4 no MFMA
 #endif
 #ifdef MI_I8_TIMING
-__device__ unsigned long long mi_i8_dbg[64 * 4 * 4];
+__device__ unsigned long long mi_i8_dbg[64 * 4 * 4 + 64 * 8];
 extern "C" int mi_i8_dbg_dump(unsigned long long *host) {
   return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mi_i8_dbg), sizeof(mi_i8_dbg));
 }
 #endif
+
+__device__ __forceinline__ int32_t med3_i32(int32_t x, int32_t lo, int32_t hi) {
+  int32_t r;
+  asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(lo), "v"(hi));
+  return r;
+}
+// four int32 -> four bytes, each saturated to [0, 255] (byte u of the result is value u)
+__device__ __forceinline__ uint32_t sat_pack_u8(int32_t q0, int32_t q1, int32_t q2, int32_t q3) {
+  uint32_t p01, p23, b01, b23;
+  asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(q0), "v"(q1));
+  asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(q2), "v"(q3));
+  asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
+  asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
+  return (b01 & 0xffffu) | (b23 << 16);
+}
 
 // LK_ = bytes of K per stage (64 or 128), NST = stages in the LDS ring (NST * 512 * LK_ bytes)
 template <int EPI, int LK_, int NST>
@@ -268,6 +299,9 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
+#ifdef MI_I8_TIMING
+  const unsigned long long r_entry = __builtin_amdgcn_s_memrealtime();
+#endif
 
   // workgroup -> tile: hardware deals workgroups round-robin over the 8 XCDs; give each XCD a contiguous range of
   // the tile order, and order tiles in groups of 4 tile-rows (column-major inside a group)
@@ -328,6 +362,19 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         acc[i][j][r] = 0;
+  // The accumulators start from the per-column bias instead of zero, so the epilogue has no bias to add.  Lane l of block (i, j) holds column 32 j + l % 32, rows 8 (r/4) + 4 (l/32) + r % 4.
+  if (a.bias) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t n = n_base + wn * 128 + j * 32 + (lane & 31);
+      const int32_t b = a.bias[n < a.N ? n : a.N - 1];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          acc[i][j][r] = b;
+    }
+  }
 
   // fragment addressing: lane reads row (lane & 31) of a 32-row block, logical chunk ks*2 + (lane >> 5)
   const int frow = lane & 31, fhalf = lane >> 5;
@@ -412,8 +459,9 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
   issue_part(NST - 1, 0);
   i32x4 fa[2][4], fb[2][4];
 #ifdef MI_I8_TIMING
-  unsigned long long t_lgkm = 0, t_vm = 0, t_bar = 0;
+  unsigned long long t_lgkm = 0, t_vm = 0, t_bar = 0, t_lgkm2 = 0;
   const unsigned long long t_begin = __builtin_readcyclecounter();
+  const unsigned long long r_begin = __builtin_amdgcn_s_memrealtime();
 #endif
   __builtin_amdgcn_s_waitcnt(waitcnt_vm((NST - 2) * LPS + 2 * PART));  // stage 0 landed
   __builtin_amdgcn_s_barrier();
@@ -422,6 +470,11 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + 1 < KS) {
+#ifdef MI_I8_TIMING
+        const unsigned long long tv0 = __builtin_readcyclecounter();
+        __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);
+        t_lgkm2 += __builtin_readcyclecounter() - tv0;
+#endif
         batch(fa[ks & 1], fb[ks & 1], fa[(ks + 1) & 1], fb[(ks + 1) & 1], kt, ks + 1, kt + NST - 1, ks + 1);
       } else {
 #ifdef MI_I8_TIMING
@@ -454,6 +507,12 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
     const unsigned long long t_end = __builtin_readcyclecounter();
     unsigned long long *d = mi_i8_dbg + (blockIdx.x * 4 + wave) * 4;
     d[0] = t_end - t_begin;
+    if (wave == 0) {  // 10 ns units
+      mi_i8_dbg[1024 + blockIdx.x * 8 + 0] = r_entry;
+      mi_i8_dbg[1024 + blockIdx.x * 8 + 4] = t_lgkm2;
+      mi_i8_dbg[1024 + blockIdx.x * 8 + 1] = r_begin - r_entry;                        // prologue
+      mi_i8_dbg[1024 + blockIdx.x * 8 + 2] = __builtin_amdgcn_s_memrealtime() - r_begin;  // main loop
+    }
     d[1] = t_lgkm;
     d[2] = t_vm;
     d[3] = t_bar;
@@ -476,19 +535,17 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
   const int cc = lane & 7, rsub = lane >> 3;  // column chunk (16 columns) and row within a group of 8 rows
   const int64_t n0 = n_base + wn * 128 + cc * 16;
   const bool vec_ok = (a.N % 16) == 0 && n0 + 16 <= a.N;
-  // relu (and its optional upper limit) as one clamp; without relu the bounds are the int32 range
-  const int32_t relu_lo = a.do_relu ? 0 : INT32_MIN;
-  const int32_t relu_hi =
-      (a.do_relu && a.relu_limit > 0 && a.relu_limit < INT32_MAX) ? (int32_t)a.relu_limit : INT32_MAX;
-  int32_t p_bias[16], p_mult[16], p_shift[16], p_zp[16];
+  // relu (and its optional upper limit) is one clamp, applied only when asked for
+  const int32_t relu_hi = (a.relu_limit > 0 && a.relu_limit < INT32_MAX) ? (int32_t)a.relu_limit : INT32_MAX;
+  int32_t p_mult[16], p_half[16], p_shift[16], p_zp[16];
+  if constexpr (EPI == EPI_Q31_HALF_AWAY) {
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int64_t n = (n0 + e) < a.N ? (n0 + e) : (a.N - 1);
-    p_bias[e] = a.bias ? a.bias[n] : 0;
-    if constexpr (EPI == EPI_Q31_HALF_AWAY) {
+    for (int e = 0; e < 16; ++e) {
+      const int64_t n = (n0 + e) < a.N ? (n0 + e) : (a.N - 1);
       p_mult[e] = a.rq.mult ? a.rq.mult[n] : a.rq.mult_s;
       p_shift[e] = a.rq.shift ? a.rq.shift[n] : a.rq.shift_s;
-      p_zp[e] = a.rq.zp ? a.rq.zp[n] : a.rq.zp_s;
+      p_half[e] = 1 << (p_shift[e] - 1);
+      p_zp[e] = (a.rq.zp ? a.rq.zp[n] : a.rq.zp_s) + 128;  // +128: saturate as unsigned, flip the sign bits after
     }
   }
 #pragma unroll
@@ -499,7 +556,8 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
       for (int r = 0; r < 16; ++r)
         strip[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * 132 + j * 32 + (lane & 31)] = acc[i][j][r];
     // same-wave LDS traffic is ordered; the compiler waits on lgkmcnt before the reads below
-    for (int it = 0; it < 4; ++it) {
+#pragma unroll 1
+    for (int it = 0; it < 4; ++it) {  // kept rolled: unrolling it spills registers
       const int row = it * 8 + rsub;
       const int64_t m = m_base + wm * 128 + i * 32 + row;
       int32_t v[16];
@@ -511,16 +569,20 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
         v[q4 * 4 + 2] = t[2];
         v[q4 * 4 + 3] = t[3];
       }
-      if (m >= a.M || n0 >= a.N)
-        continue;
-      const int32_t rt = a.row_term ? a.row_term[m] : 0;
+      if (a.row_term) {  // per-row term of a nonzero right zero point
+        const int32_t rt = a.row_term[m < a.M ? m : a.M - 1];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int32_t x = v[e] + p_bias[e] + rt;
-        v[e] = x < relu_lo ? relu_lo : (x > relu_hi ? relu_hi : x);  // one v_med3_i32
+        for (int e = 0; e < 16; ++e)
+          v[e] += rt;
       }
+      if (a.do_relu) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          v[e] = med3_i32(v[e], 0, relu_hi);
+      }
+      const bool live = m < a.M && n0 < a.N;
       const int64_t o = m * a.N + n0;
-      if (a.acc_out) {
+      if (a.acc_out && live) {
         if (vec_ok) {
 #pragma unroll
           for (int q4 = 0; q4 < 4; ++q4)
@@ -532,7 +594,7 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
         }
       }
       if constexpr (EPI == EPI_INT32) {
-        if (a.out) {
+        if (a.out && live) {
           int32_t *out = (int32_t *)a.out;
           if (vec_ok) {
 #pragma unroll
@@ -547,32 +609,44 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
       } else if constexpr (EPI == EPI_Q31_HALF_AWAY) {
         // MultiplyByQuantizedMultiplier(x, mult, -shift, HALF_AWAY) with shift in [1, 31], in 32-bit steps:
         // t = (x*mult + 2^30) >> 31 fits int32 for |x|, mult < 2^31, so the reference's clamp never fires, and
-        // half-away rounding of t >> shift is (t + half + (t >> 31)) >> shift.
-        uint32_t packed[4] = {0, 0, 0, 0};
+        // half-away rounding of t >> shift is (t + half + (t >> 31)) >> shift.  The int8 saturation is done as
+        // an unsigned one on q + 128 (two saturating pack instructions per four values), undone by flipping the
+        // sign bits of the packed bytes.
+        uint32_t packed[4];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int64_t p = (int64_t)v[e] * (int64_t)p_mult[e] + (1ll << 30);
-          const int32_t t = (int32_t)(p >> 31);
-          int32_t q = (t + (1 << (p_shift[e] - 1)) + (t >> 31)) >> p_shift[e];
-          q += p_zp[e];
-          q = q < -128 ? -128 : (q > 127 ? 127 : q);
-          packed[e >> 2] |= (uint32_t)(q & 0xff) << (8 * (e & 3));
+        for (int q4 = 0; q4 < 4; ++q4) {
+          int32_t q[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int e = q4 * 4 + u;
+            const int64_t p = (int64_t)v[e] * (int64_t)p_mult[e] + (1ll << 30);
+            const int32_t t = (int32_t)(p >> 31);
+            q[u] = ((t + p_half[e] + (t >> 31)) >> p_shift[e]) + p_zp[e];
+          }
+          packed[q4] = sat_pack_u8(q[0], q[1], q[2], q[3]) ^ 0x80808080u;
         }
-        int8_t *out = (int8_t *)a.out;
-        if (vec_ok) {
-          *(u32x4 *)(out + o) = u32x4{packed[0], packed[1], packed[2], packed[3]};
-        } else {
-          for (int e = 0; e < 16; ++e)
-            if (n0 + e < a.N)
-              out[o + e] = (int8_t)((packed[e >> 2] >> (8 * (e & 3))) & 0xff);
+        if (live) {
+          int8_t *out = (int8_t *)a.out;
+          if (vec_ok) {
+            *(u32x4 *)(out + o) = u32x4{packed[0], packed[1], packed[2], packed[3]};
+          } else {
+            for (int e = 0; e < 16; ++e)
+              if (n0 + e < a.N)
+                out[o + e] = (int8_t)((packed[e >> 2] >> (8 * (e & 3))) & 0xff);
+          }
         }
       } else {
-        for (int e = 0; e < 16; ++e)
-          if (n0 + e < a.N)
-            store_out(a.out, o + e, requant_one(v[e], n0 + e, a.rq), a.rq.out_dtype);
+        if (live)
+          for (int e = 0; e < 16; ++e)
+            if (n0 + e < a.N)
+              store_out(a.out, o + e, requant_one(v[e], n0 + e, a.rq), a.rq.out_dtype);
       }
     }
   }
+#ifdef MI_I8_TIMING
+  if (lane == 0 && blockIdx.x < 64 && wave == 0)
+    mi_i8_dbg[1024 + blockIdx.x * 8 + 3] = __builtin_amdgcn_s_memrealtime() - r_entry;  // whole kernel
+#endif
 }
 
 static RequantParams make_rq(const mi_requant_desc *rq) {
@@ -670,7 +744,20 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
   else
     a.rq = RequantParams{nullptr, nullptr, nullptr, 1, 0, 0, MI_RQ_MULTIPLIER_SHIFT, 0, 0, MI_DT_I32};
   const bool large = (K % 128) == 0 && M >= 128 && N >= 128 && !getenv("MI_I8_SMALL_TILE");
+  uint8_t *a_signed = nullptr, *b_signed = nullptr;
   if (large) {
+    // the direct-to-LDS loads of the large-tile kernel cannot flip sign bits on the way: unsigned operands are
+    // rewritten once (after the zero-point sums above, which read the original bytes)
+    if (a_unsigned) {
+      MI_HIP(hipMallocAsync((void **)&a_signed, (size_t)M * K, stream));
+      flip_bytes_kernel<<<dim3((unsigned)((M * K / 16 + 256) / 256)), dim3(256), 0, stream>>>(a.A, a_signed, M * K);
+      a.A = a_signed;
+    }
+    if (b_unsigned) {
+      MI_HIP(hipMallocAsync((void **)&b_signed, (size_t)N * K, stream));
+      flip_bytes_kernel<<<dim3((unsigned)((N * K / 16 + 256) / 256)), dim3(256), 0, stream>>>(a.B, b_signed, N * K);
+      a.B = b_signed;
+    }
     const int tiles_m = (int)((M + LM - 1) / LM), tiles_n = (int)((N + LN - 1) / LN);
     const int per_xcd = (tiles_m * tiles_n + 7) / 8;
     const char *ring_env = getenv("MI_I8_RING");  // development switch: stages in the LDS ring (3, 4 or 5)
@@ -720,6 +807,10 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
     i8_gemm_kernel<<<grid, dim3(256), 0, stream>>>(a);
   }
   MI_HIP(hipGetLastError());
+  if (a_signed)
+    MI_HIP(hipFreeAsync(a_signed, stream));
+  if (b_signed)
+    MI_HIP(hipFreeAsync(b_signed, stream));
   if (bt)
     MI_HIP(hipFreeAsync(bt, stream));
   if (colsum)
