@@ -263,7 +263,13 @@ constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; 
 constexpr int WAITCNT_LGKM0 = 0xC07F;
 
 #ifndef MI_I8_DBG
-#define MI_I8_DBG 0  // development switches: 1 no global loads, 2 no fragment reads, 4 no MFMA
+#define MI_I8_DBG 0  // development switches (results become wrong): 1 no global loads, 2 no fragment reads, 4 no MFMA,
+                     // 8 no barrier, 16 no wait for the loads
+#endif
+#if defined(MI_I8_TIMING) && MI_I8_TIMING >= 2
+#define MI_I8_STAMP(v) const unsigned long long v = __builtin_readcyclecounter()
+#else
+#define MI_I8_STAMP(v)
 #endif
 #ifdef MI_I8_TIMING
 __device__ unsigned long long mi_i8_dbg[64 * 4 * 4 + 64 * 8];
@@ -470,29 +476,20 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + 1 < KS) {
-#ifdef MI_I8_TIMING
-        const unsigned long long tv0 = __builtin_readcyclecounter();
-        __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);
-        t_lgkm2 += __builtin_readcyclecounter() - tv0;
-#endif
         batch(fa[ks & 1], fb[ks & 1], fa[(ks + 1) & 1], fb[(ks + 1) & 1], kt, ks + 1, kt + NST - 1, ks + 1);
       } else {
-#ifdef MI_I8_TIMING
-        const unsigned long long tw0 = __builtin_readcyclecounter();
-#endif
+        MI_I8_STAMP(tw0);
         __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);
-#ifdef MI_I8_TIMING
-        const unsigned long long tw1 = __builtin_readcyclecounter();
-#endif
-#if !(MI_I8_DBG & 1)
+        MI_I8_STAMP(tw1);
+#if !(MI_I8_DBG & 1) && !(MI_I8_DBG & 16)
         __builtin_amdgcn_s_waitcnt(waitcnt_vm((NST - 2) * LPS));  // this thread's share of stage kt+1 landed
 #endif
-#ifdef MI_I8_TIMING
-        const unsigned long long tw2 = __builtin_readcyclecounter();
-#endif
+        MI_I8_STAMP(tw2);
+#if !(MI_I8_DBG & 8)
         __builtin_amdgcn_s_barrier();
-#ifdef MI_I8_TIMING
-        const unsigned long long tw3 = __builtin_readcyclecounter();
+#endif
+        MI_I8_STAMP(tw3);
+#if defined(MI_I8_TIMING) && MI_I8_TIMING >= 2
         t_lgkm += tw1 - tw0;
         t_vm += tw2 - tw1;
         t_bar += tw3 - tw2;
@@ -524,13 +521,6 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
   // LDS region (row stride 132 dwords) and re-reads it so that a lane owns 16 consecutive columns of a row: the
   // per-column requant parameters are then loaded once per lane and the int8 result leaves as 16-byte stores.
   __syncthreads();  // every wave is done with the stage buffers
-#if defined(MI_I8_DBG) && (MI_I8_DBG & 8)
-  {
-    if (acc[0][0][0] == 0x7fffffff)
-      ((int32_t *)a.out)[0] = acc[1][1][1] + acc[2][2][2] + acc[3][3][3];
-    return;
-  }
-#endif
   int32_t *strip = reinterpret_cast<int32_t *>(lds) + wave * (32 * 132);
   const int cc = lane & 7, rsub = lane >> 3;  // column chunk (16 columns) and row within a group of 8 rows
   const int64_t n0 = n_base + wn * 128 + cc * 16;
