@@ -58,23 +58,38 @@ def build_chain(pkg, S, torch, M, n_layers, cfgs):
     return layers, acts, outs
 
 
-def run_chain(pkg, mats, acts, outs):
-    for name, K, N, w in mats:
-        pkg.a16mm_launch(w, acts[K], outs[name])
+# sibling projections that read the same activations go out as one grouped launch
+CHAIN_GROUPS = [("q_proj", "k_proj", "v_proj"), ("o_proj",), ("gate_proj", "up_proj"), ("down_proj",)]
 
 
-def bench_chain(pkg, S, torch, M, steps, warmup, n_layers, cfgs):
+def run_chain(pkg, mats, acts, outs, grouped=True):
+    """One pass over the seven matmuls; returns the number of kernel launches."""
+    if not grouped:
+        for name, K, N, w in mats:
+            pkg.a16mm_launch(w, acts[K], outs[name])
+        return len(mats)
+    by_name = {name: (K, w) for name, K, N, w in mats}
+    for grp in CHAIN_GROUPS:
+        K = by_name[grp[0]][0]
+        if len(grp) == 1:
+            pkg.a16mm_launch(by_name[grp[0]][1], acts[K], outs[grp[0]])
+        else:
+            pkg.a16mm_launch_group([by_name[n][1] for n in grp], acts[K], [outs[n] for n in grp])
+    return len(CHAIN_GROUPS)
+
+
+def bench_chain(pkg, S, torch, M, steps, warmup, n_layers, cfgs, grouped=True):
     layers, acts, outs = build_chain(pkg, S, torch, M, n_layers, cfgs)
     stream = torch.cuda.Stream()
     graphs = []
     with torch.cuda.stream(stream):
         for mats in layers:  # eager pass first: loads the code objects before capture
-            run_chain(pkg, mats, acts, outs)
+            launches = run_chain(pkg, mats, acts, outs, grouped)
         stream.synchronize()
         for mats in layers:
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=stream):
-                run_chain(pkg, mats, acts, outs)
+                run_chain(pkg, mats, acts, outs, grouped)
             graphs.append(g)
         for i in range(warmup):
             graphs[i % n_layers].replay()
@@ -92,7 +107,6 @@ def bench_chain(pkg, S, torch, M, steps, warmup, n_layers, cfgs):
     wall_s = t1 - t0
     gpu_s = ev0.elapsed_time(ev1) * 1e-3
     chain_bytes = sum(S.w4_gemv_bytes(M, K, N, 128) for _, K, N in S.LLAMA7B_CHAIN)
-    launches = len(S.LLAMA7B_CHAIN)
     res = {
         "wall_s": wall_s, "gpu_s": gpu_s, "chain_bytes": chain_bytes, "launches_per_step": launches,
         "weight_set_mb": sum(w.nbytes for m in layers for *_, w in m) / 1e6,
@@ -162,6 +176,8 @@ def main():
     ap.add_argument("--layers", type=int, default=4, help="distinct weight copies rotated through (4 x 101 MB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-int8", action="store_true")
+    ap.add_argument("--no-group", action="store_true",
+                    help="one launch per matmul (7) instead of grouping q/k/v and gate/up (4 launches)")
     ap.add_argument("--int8-size", type=int, default=4096)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -185,7 +201,7 @@ def main():
 
     M = args.batch
     cfgs = host_chain(S, M)
-    r = bench_chain(pkg, S, torch, M, args.steps, args.warmup, args.layers, cfgs)
+    r = bench_chain(pkg, S, torch, M, args.steps, args.warmup, args.layers, cfgs, grouped=not args.no_group)
     value = r["chain_bytes"] * args.steps / r["wall_s"] / 1e9
     n_launch = args.steps * r["launches_per_step"]
     avg_launch_s = r["gpu_s"] / n_launch
@@ -200,7 +216,8 @@ def main():
                                "down 4096x11008)" % M,
                    "bytes_per_step": r["chain_bytes"], "launches_per_step": r["launches_per_step"],
                    "weight_copies": args.layers, "resident_weight_mb": round(r["weight_set_mb"], 1),
-                   "launch": "one HIP graph replay per step"},
+                   "launch": "one HIP graph replay per step; q/k/v and gate/up each as one grouped launch"
+                             if not args.no_group else "one HIP graph replay per step; one launch per matmul"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE (profiles/hbm_traffic_pmc_*.md):

@@ -126,6 +126,15 @@ size_t mi_a16_weight_bytes(const mi_a16_weight *w);
 int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                     void *stream);
 
+/* The same for n (1..4) weight sets that read the SAME activations, in one kernel launch: y_i = x * dequant(W_i)^T.
+ * These are the sibling linears the reference's LLM export emits on one input -- q/k/v on the normed hidden state
+ * (python/llm/LlmConverter.py:1797-1812), gate/up in the MLP -- each of which the interpreter runs as its own
+ * A16MatMulOp::inference (A16MatMul.cpp:150-273).  Results are identical to n calls of mi_a16mm_launch.  The sets
+ * must agree in K, weight_bits, q_group_size, dtype and chip; N may differ.  d_y[i] / d_y_f32[i] as above
+ * (d_y_f32 itself may be NULL, as may any of its entries). */
+int mi_a16mm_launch_group(const mi_a16_weight *const *w, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_y,
+                          float *const *d_y_f32, void *stream);
+
 /* ============================================================================ */
 /* tpu.MatMul, quantized  (lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:387-733) */
 /* ============================================================================ */

@@ -175,3 +175,39 @@ def test_f16_mode_device_level(orc):
                                    M=M, K=K, N=N, weight_bits=4, q_group_size=g, out_dtype=orc.OUT_F16)
     assert cmp.max_abs_over_rms(pre, want_pre) <= 2e-5
     assert np.array_equal(out, orc.f32_to_f16(pre))
+
+
+@pytest.mark.parametrize("bits,M", [(4, 1), (4, 5), (8, 3), (4, 40)])
+def test_grouped_launch_equals_separate_launches(bits, M):
+    """Sibling weight sets on one input (q/k/v, gate/up) in one launch: bit-identical to one launch per set,
+    including ragged N, optional bias, the fp32 side output, and a group that does not fill the segment table."""
+    torch = _torch()
+    K = 512
+    Ns = (160, 40, 100) if bits == 4 else (64, 200)
+    cfgs = []
+    for i, N in enumerate(Ns):
+        c = S.w4a16(M, K, N, 128, seed=20 + i, bias=(i != 1)) if bits == 4 else \
+            S.w8a16(M, K, N, 0, seed=20 + i, bias=(i == 0))
+        cfgs.append(c)
+    x = torch.from_numpy(cfgs[0]["x"].view(np.int16)).cuda().view(torch.bfloat16)
+    ws = [M_.A16Weight(c["weight"], c["scale"], c["zp"], None if c.get("bias") is None else S.bf16_to_f32(c["bias"]),
+                       K=K, N=c["N"], weight_bits=bits, q_group_size=c["g"]) for c in cfgs]
+    f32s = [torch.empty((M, c["N"]), dtype=torch.float32, device="cuda") for c in cfgs]
+    f32s[1] = None  # an absent fp32 side output in the middle of the group
+    ys = M_.a16mm_launch_group(ws, x, ys_f32=f32s)
+    torch.cuda.synchronize()
+    for w, c, y, f in zip(ws, cfgs, ys, f32s):
+        f1 = torch.empty((M, c["N"]), dtype=torch.float32, device="cuda")
+        y1 = M_.a16mm_launch(w, x, y_f32=f1)
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16), y1.view(torch.int16))
+        if f is not None:
+            assert torch.equal(f.view(torch.int32), f1.view(torch.int32))
+    # sets that disagree in K are refused
+    other = S.w4a16(M, 256, 32, 128, seed=9) if bits == 4 else S.w8a16(M, 256, 32, 0, seed=9)
+    wo = M_.A16Weight(other["weight"], other["scale"], other["zp"], None, K=256, N=32, weight_bits=bits,
+                      q_group_size=other["g"])
+    with pytest.raises(clib.BackendError):
+        M_.a16mm_launch_group([ws[0], wo], x)
+    for w in ws + [wo]:
+        w.destroy()

@@ -17,6 +17,7 @@ EXPORTS = [
     "mi_version", "mi_last_error", "mi_device_count",
     "mi_a16mm_init", "mi_a16mm_inference", "mi_a16mm_deinit",
     "mi_a16_weight_create", "mi_a16_weight_destroy", "mi_a16_weight_bytes", "mi_a16mm_launch",
+    "mi_a16mm_launch_group",
     "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
     "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
 ]
@@ -104,6 +105,8 @@ def lib():
         L.mi_a16_weight_destroy.argtypes = [C.c_void_p]
         L.mi_a16_weight_destroy.restype = None
         L.mi_a16mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi_a16mm_launch_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int64,
+                                            C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_void_p]
         L.mi_a16mm_init.argtypes = [C.POINTER(A16Attr), C.POINTER(InferParam)]
         L.mi_a16mm_inference.argtypes = [C.POINTER(A16Attr), C.POINTER(InferParam)]
         L.mi_a16mm_deinit.argtypes = [C.POINTER(InferParam)]

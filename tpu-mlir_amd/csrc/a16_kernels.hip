@@ -258,18 +258,28 @@ int a16_pack(mi_a16_weight *w, const void *h_weight, int weight_signed, const ui
 // and the per-group activation sums S are formed during staging; the registers then hold weights only.
 // XLDS = false: activation fragments are loaded per tile from global memory (L2) and S comes from a second MFMA.
 // ------------------------------------------------------------------------------------------------
-struct SkinnyArgs {
+// One launch covers up to MAX_SEG weight sets that consume the same activations (sibling projections such as
+// q/k/v or gate/up): their row blocks are laid end to end on the grid, and a workgroup finds its weight set by
+// comparing its row-block index with the segment starts.
+constexpr int MAX_SEG = 4;
+struct SkinnySeg {
   const u32x4 *qw;
   const uint32_t *sz_t;
   const uint16_t *scale_t;
   const float *nzs_t;
   const float *bias;
-  const uint16_t *x;
   uint16_t *y;
   float *y32;
+  int64_t N;
+  int rb_begin;  // first row block of this weight set on the grid
+};
+struct SkinnyArgs {
+  SkinnySeg seg[MAX_SEG];
+  int n_seg;
+  const uint16_t *x;
   int M;
-  int64_t K, N;
-  int row_blocks;
+  int64_t K;
+  int row_blocks;       // of all segments together
   int k_tiles;          // tiles stored per row block (the last one may be partial)
   int full_tiles;       // tiles that lie completely inside K
   int G;
@@ -277,9 +287,28 @@ struct SkinnyArgs {
   int chip;
 };
 
+// Where a row block lives: its weight set and its index inside it.
+struct RowBlockRef {
+  int seg, rb;
+  bool live;  // false: past the end of the grid (loads are clamped, nothing is stored)
+};
+__device__ __forceinline__ RowBlockRef locate_row_block(const SkinnyArgs &a, int rbg) {
+  RowBlockRef r;
+  r.live = rbg < a.row_blocks;
+  const int c = r.live ? rbg : a.row_blocks - 1;
+  r.seg = 0;
+#pragma unroll
+  for (int q = 1; q < MAX_SEG; ++q)
+    if (q < a.n_seg && c >= a.seg[q].rb_begin)
+      r.seg = q;
+  r.rb = c - a.seg[r.seg].rb_begin;
+  return r;
+}
+
 template <int DT, int WAVES, int R>
 __device__ __forceinline__ void reduce_and_store(const SkinnyArgs &a, float (*red)[R][4][64], const f32x4 (&acc)[R],
-                                                 int wave, int lane, int rb0, int m0) {
+                                                 int wave, int lane, const RowBlockRef (&ref)[R],
+                                                 const float (&bias_v)[R], int m0) {
 #pragma unroll
   for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -288,21 +317,23 @@ __device__ __forceinline__ void reduce_and_store(const SkinnyArgs &a, float (*re
   __syncthreads();
   // R * 4 * 64 partial sums to finish: spread them over the workgroup's waves
   const int col = lane & 15, kq = lane >> 4;
-  for (int item = wave; item < R * 4; item += WAVES) {
-    const int r = item >> 2, i = item & 3;
-    float v = 0.0f;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w)
-      v += red[w][r][i][lane];
-    const int64_t n = (int64_t)(rb0 + r) * ROW_BLOCK + col;
-    const int m = m0 + 4 * kq + i;
-    if (m < a.M && n < a.N) {
-      if (a.bias)
-        v += a.bias[n];
-      const int64_t o = (int64_t)m * a.N + n;
-      if (a.y32)
-        a.y32[o] = v;
-      a.y[o] = (a.chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+  for (int r = 0; r < R; ++r) {
+    const SkinnySeg &sg = a.seg[ref[r].seg];
+    for (int i = wave; i < 4; i += WAVES) {
+      float v = 0.0f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w)
+        v += red[w][r][i][lane];
+      const int64_t n = (int64_t)ref[r].rb * ROW_BLOCK + col;
+      const int m = m0 + 4 * kq + i;
+      if (ref[r].live && m < a.M && n < sg.N) {
+        v += bias_v[r];
+        const int64_t o = (int64_t)m * sg.N + n;
+        if (sg.y32)
+          sg.y32[o] = v;
+        sg.y[o] = (a.chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+      }
     }
   }
 }
@@ -380,19 +411,25 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
   const uint32_t *szp[R];
   const uint16_t *scp[R];
   const float *nzp[R];
+  RowBlockRef ref[R];
+  float bias_v[R];  // this lane's output channel; requested now so that it has arrived by the time of the store
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    int rb = (rb0 + r) < a.row_blocks ? (rb0 + r) : (a.row_blocks - 1);  // clamped, discarded at the store
+    ref[r] = locate_row_block(a, rb0 + r);
+    const SkinnySeg &sg = a.seg[ref[r].seg];
+    int rb = ref[r].rb;
 #ifdef MI_DBG_SAMETILE
     rb = rb & 3;
 #endif
-    wq[r] = a.qw + (int64_t)rb * a.k_tiles * 64 + lane;
+    wq[r] = sg.qw + (int64_t)rb * a.k_tiles * 64 + lane;
     if constexpr (BITS == 4) {
-      szp[r] = a.sz_t + (int64_t)rb * a.G * 16 + col;
+      szp[r] = sg.sz_t + (int64_t)rb * a.G * 16 + col;
     } else {
-      scp[r] = a.scale_t + (int64_t)rb * a.G * 16 + col;
-      nzp[r] = a.nzs_t + (int64_t)rb * a.G * 16 + col;
+      scp[r] = sg.scale_t + (int64_t)rb * a.G * 16 + col;
+      nzp[r] = sg.nzs_t + (int64_t)rb * a.G * 16 + col;
     }
+    const int64_t n = (int64_t)rb * ROW_BLOCK + col;
+    bias_v[r] = (sg.bias && n < sg.N) ? sg.bias[n] : 0.0f;
   }
   const uint16_t *xrow = a.x + (int64_t)(m0 + row_ld) * a.K + kq * 8;
 
@@ -634,7 +671,7 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
       compute_tile(t, kt);
     }
   }
-  reduce_and_store<DT, WAVES, R>(a, red, acc, wave, lane, rb0, m0);
+  reduce_and_store<DT, WAVES, R>(a, red, acc, wave, lane, ref, bias_v, m0);
   MI_STAMP(4);
 #ifdef MI_DBG_TIMING
   if (threadIdx.x == 0 && blockIdx.x < 4096) {
@@ -766,25 +803,48 @@ static bool launch_skinny_x(const SkinnyArgs &a, const SkinnyPlan &plan, int64_t
 
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                hipStream_t stream) {
-  MI_REQUIRE(w && w->qweight, MI_BAD_ARGUMENT, "mi_a16mm_launch: weight set is empty");
-  MI_REQUIRE(d_x && d_y, MI_BAD_ARGUMENT, "mi_a16mm_launch: null activation or output pointer");
+  return a16_launch_group(&w, 1, d_x, M, &d_y, d_y_f32 ? &d_y_f32 : nullptr, stream);
+}
+
+int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
+                     float *const *d_y32s, hipStream_t stream) {
+  MI_REQUIRE(ws && n >= 1 && n <= MAX_SEG, MI_BAD_ARGUMENT,
+             "mi_a16mm_launch_group: between 1 and " + std::to_string(MAX_SEG) + " weight sets per launch");
+  MI_REQUIRE(d_x && d_ys, MI_BAD_ARGUMENT, "mi_a16mm_launch: null activation or output pointer");
   MI_REQUIRE(M >= 0 && M < (1 << 20), MI_BAD_ARGUMENT, "mi_a16mm_launch: M out of range");
+  const mi_a16_weight *w = ws[0];
+  int64_t total_rb = 0;
+  SkinnyArgs a;
+  for (int i = 0; i < MAX_SEG; ++i) {
+    const int q = i < n ? i : 0;  // unused slots repeat the first set; the kernel never selects them
+    MI_REQUIRE(ws[q] && ws[q]->qweight, MI_BAD_ARGUMENT, "mi_a16mm_launch: weight set is empty");
+    MI_REQUIRE(d_ys[q], MI_BAD_ARGUMENT, "mi_a16mm_launch: null output pointer");
+    const mi_a16_weight *v = ws[q];
+    MI_REQUIRE(v->K == w->K && v->bits == w->bits && v->g == w->g && v->dtype == w->dtype && v->chip == w->chip,
+               MI_BAD_ARGUMENT,
+               "mi_a16mm_launch_group: the weight sets must agree in K, bit width, group size, data type and chip");
+    SkinnySeg &sg = a.seg[i];
+    sg.qw = (const u32x4 *)v->qweight;
+    sg.sz_t = v->sz_t;
+    sg.scale_t = v->scale_t;
+    sg.nzs_t = v->nzs_t;
+    sg.bias = v->bias;
+    sg.y = d_ys[q];
+    sg.y32 = d_y32s ? d_y32s[q] : nullptr;
+    sg.N = v->N;
+    sg.rb_begin = (int)total_rb;
+    if (i < n)
+      total_rb += v->row_blocks;
+  }
+  MI_REQUIRE(total_rb < (1ll << 31), MI_BAD_ARGUMENT, "mi_a16mm_launch: too many output channels for one launch");
   if (M == 0)
     return MI_SUCCESS;
   const int tile_k = w->bits == 4 ? W4_TILE_K : W8_TILE_K;
-  SkinnyArgs a;
-  a.qw = (const u32x4 *)w->qweight;
-  a.sz_t = w->sz_t;
-  a.scale_t = w->scale_t;
-  a.nzs_t = w->nzs_t;
-  a.bias = w->bias;
+  a.n_seg = n;
   a.x = d_x;
-  a.y = d_y;
-  a.y32 = d_y_f32;
   a.M = (int)M;
   a.K = w->K;
-  a.N = w->N;
-  a.row_blocks = (int)w->row_blocks;
+  a.row_blocks = (int)total_rb;
   a.k_tiles = (int)w->k_tiles;
   a.full_tiles = (int)(w->K / tile_k);
   a.G = w->G;
@@ -793,7 +853,7 @@ int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t 
   const int64_t m_blocks = (M + 15) / 16;
   const size_t x_bytes = skinny_x_bytes((int)(M < 16 ? M : 16), w->k_tiles, tile_k);
   const bool xlds = x_bytes <= XLDS_MAX_BYTES && !getenv("MI_A16_NO_XLDS");
-  const SkinnyPlan plan = pick_plan(w->row_blocks, m_blocks, w->k_tiles, xlds);
+  const SkinnyPlan plan = pick_plan(total_rb, m_blocks, w->k_tiles, xlds);
   const bool f16 = w->dtype == MI_DT_F16;
   bool ok;
   if (w->bits == 4) {

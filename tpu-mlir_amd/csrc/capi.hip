@@ -194,6 +194,11 @@ int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
   return a16_launch(w, d_x, M, d_y, d_y_f32, (hipStream_t)stream);
 }
 
+int mi_a16mm_launch_group(const mi_a16_weight *const *w, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_y,
+                          float *const *d_y_f32, void *stream) {
+  return a16_launch_group(w, n, d_x, M, d_y, d_y_f32, (hipStream_t)stream);
+}
+
 // ---------------------------------------------------------------------------------------------
 // operator level: tpu.A16MatMul
 // ---------------------------------------------------------------------------------------------

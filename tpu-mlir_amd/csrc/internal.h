@@ -64,6 +64,8 @@ int a16_pack(mi_a16_weight *w, const void *h_weight, int weight_signed, const ui
 void a16_free(mi_a16_weight *w);
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                hipStream_t stream);
+int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
+                     float *const *d_y32s, hipStream_t stream);
 
 struct RequantParams;
 int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned, int right_transpose,

@@ -226,6 +226,37 @@ def a16mm_launch(w, x, y=None, y_f32=None, stream=None):
     return y
 
 
+def a16mm_launch_group(ws, x, ys=None, ys_f32=None, stream=None):
+    """Several weight sets that read the same activations (q/k/v, gate/up) in ONE kernel launch; the results equal
+    those of one a16mm_launch per set.  ws: A16Weight list (same K, bits, group size, dtype); returns the outputs."""
+    import torch
+    w0 = ws[0]
+    tdt = torch.float16 if w0.dtype == DT_F16 else torch.bfloat16
+    if not (x.is_cuda and x.dtype == tdt and x.is_contiguous() and x.shape[-1] == w0.K):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_launch_group: x must be a contiguous CUDA tensor [.., K]")
+    M = x.numel() // w0.K
+    if ys is None:
+        ys = [torch.empty(tuple(x.shape[:-1]) + (w.N,), dtype=tdt, device=x.device) for w in ws]
+    if len(ys) != len(ws) or (ys_f32 is not None and len(ys_f32) != len(ws)):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_launch_group: one output per weight set")
+    for w, y in zip(ws, ys):
+        if not (y.is_cuda and y.dtype == tdt and y.is_contiguous() and y.numel() == M * w.N):
+            raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_launch_group: bad output tensor")
+    n = len(ws)
+    Arr = C.c_void_p * n
+    wh = Arr(*[w.handle.value if isinstance(w.handle, C.c_void_p) else w.handle for w in ws])
+    yp = Arr(*[y.data_ptr() for y in ys])
+    fp = None
+    if ys_f32 is not None:
+        for w, f in zip(ws, ys_f32):
+            if f is not None and not (f.is_cuda and f.dtype == torch.float32 and f.is_contiguous()
+                                      and f.numel() == M * w.N):
+                raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_launch_group: bad y_f32 tensor")
+        fp = Arr(*[None if f is None else f.data_ptr() for f in ys_f32])
+    check(clib.lib().mi_a16mm_launch_group(wh, n, _dptr(x), M, yp, fp, _stream_ptr(stream)))
+    return ys
+
+
 class RequantDesc:
     """Per-channel (torch int32 CUDA tensors) or scalar requantization parameters; shift > 0 shifts right."""
 
