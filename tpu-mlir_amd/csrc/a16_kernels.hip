@@ -287,21 +287,40 @@ struct SkinnyArgs {
   int chip;
 };
 
-// Where a row block lives: its weight set and its index inside it.
+// Where a row block lives: its weight set (copied out of the argument block) and its index inside it.  Every
+// segment's fields are requested from the kernel-argument block up front and the right one is then SELECTED, instead
+// of indexing the table with the segment number: an indexed read could only be requested after the segment is
+// known, a second trip to memory in front of the first weight request.
 struct RowBlockRef {
-  int seg, rb;
+  SkinnySeg sg;
+  int rb;
   bool live;  // false: past the end of the grid (loads are clamped, nothing is stored)
 };
+template <class T>
+__device__ __forceinline__ T pick4(int s, T v0, T v1, T v2, T v3) {
+  return s == 3 ? v3 : (s == 2 ? v2 : (s == 1 ? v1 : v0));
+}
 __device__ __forceinline__ RowBlockRef locate_row_block(const SkinnyArgs &a, int rbg) {
   RowBlockRef r;
   r.live = rbg < a.row_blocks;
   const int c = r.live ? rbg : a.row_blocks - 1;
-  r.seg = 0;
+  int s = 0;
 #pragma unroll
   for (int q = 1; q < MAX_SEG; ++q)
     if (q < a.n_seg && c >= a.seg[q].rb_begin)
-      r.seg = q;
-  r.rb = c - a.seg[r.seg].rb_begin;
+      s = q;
+#define MI_PICK(f) r.sg.f = pick4(s, a.seg[0].f, a.seg[1].f, a.seg[2].f, a.seg[3].f)
+  MI_PICK(qw);
+  MI_PICK(sz_t);
+  MI_PICK(scale_t);
+  MI_PICK(nzs_t);
+  MI_PICK(bias);
+  MI_PICK(y);
+  MI_PICK(y32);
+  MI_PICK(N);
+  MI_PICK(rb_begin);
+#undef MI_PICK
+  r.rb = c - r.sg.rb_begin;
   return r;
 }
 
@@ -319,7 +338,7 @@ __device__ __forceinline__ void reduce_and_store(const SkinnyArgs &a, float (*re
   const int col = lane & 15, kq = lane >> 4;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const SkinnySeg &sg = a.seg[ref[r].seg];
+    const SkinnySeg &sg = ref[r].sg;
     for (int i = wave; i < 4; i += WAVES) {
       float v = 0.0f;
 #pragma unroll
@@ -416,7 +435,7 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     ref[r] = locate_row_block(a, rb0 + r);
-    const SkinnySeg &sg = a.seg[ref[r].seg];
+    const SkinnySeg &sg = ref[r].sg;
     int rb = ref[r].rb;
 #ifdef MI_DBG_SAMETILE
     rb = rb & 3;
@@ -576,18 +595,19 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
     constexpr int XB = WAVES >= 16 ? 2 : 4;        // chunks per thread in the first batch
     const int chunks_per_row = kpad / 8;
     const int total = rows * chunks_per_row;
+    // the load only requests the data; anything that needs the VALUE (zeroing the padding past K included) waits
+    // until chunk_store, so that nothing stalls between this request and the weight requests that follow it
     auto chunk_load = [&](int c, int &row, int &kc, bool &ok) {
       ok = c < total;
       const int cc = ok ? c : 0;
       row = rows == 1 ? 0 : cc / chunks_per_row;
       kc = cc - row * chunks_per_row;
       const bool in_k = kc * 8 < a.K;
-      u32x4 v = *(const u32x4 *)(a.x + (int64_t)(m0 + row) * a.K + (in_k ? kc * 8 : 0));  // always in bounds
-      if (!in_k)
-        v = u32x4{0, 0, 0, 0};
-      return v;
+      return *(const u32x4 *)(a.x + (int64_t)(m0 + row) * a.K + (in_k ? kc * 8 : 0));  // always in bounds
     };
-    auto chunk_store = [&](const u32x4 &v, int row, int kc, bool ok) {
+    auto chunk_store = [&](u32x4 v, int row, int kc, bool ok) {
+      if (kc * 8 >= a.K)
+        v = u32x4{0, 0, 0, 0};
       if (ok)
         *(u32x4 *)(xs + row * xstride + kc * 16) = v;
       if constexpr (BITS == 4) {
@@ -606,11 +626,9 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
     int row[XB], kc[XB];
     bool ok[XB];
 #pragma unroll
-    for (int b = 0; b < XB; ++b)
-      if (b * NT < total)  // workgroup-uniform
-        v[b] = chunk_load(b * NT + tid, row[b], kc[b], ok[b]);
-    if (n_tiles > 0)
-      issue_round(buf_a, 0);
+    for (int b = 0; b < XB; ++b)  // unconditional (slots past the end re-read chunk 0): keeps the load count static
+      v[b] = chunk_load(b * NT + tid, row[b], kc[b], ok[b]);
+    issue_round(buf_a, 0);  // unconditional (k_tiles >= 1): a branch here would hide the load count from the waits below
     MI_STAMP(1);
 #pragma unroll
     for (int b = 0; b < XB; ++b)
