@@ -75,6 +75,46 @@ W4_CASES = [  # (M, K, N, g)
 ]
 
 
+PREFILL_CASES = [  # (bits, M, K, N, g, signed): M > 16 takes the tiled MFMA GEMM when K % 128 == 0
+    (4, 100, 1024, 300, 128, False), (4, 130, 512, 272, 64, False), (4, 70, 256, 40, 32, False),
+    (4, 33, 1024, 64, 256, False), (4, 64, 384, 48, 0, False), (4, 17, 128, 16, 128, False),
+    (8, 50, 512, 96, 128, False), (8, 40, 256, 40, 32, False), (8, 36, 512, 130, 64, False),
+    (8, 45, 384, 70, 0, True),
+    (4, 40, 200, 48, 0, False),  # K % 128 != 0: stays on the skinny kernel
+]
+
+
+@pytest.mark.parametrize("tile", ["128", "256"])
+@pytest.mark.parametrize("bits,M,K,N,g,signed", PREFILL_CASES)
+def test_prefill_gemm_device_level(orc, monkeypatch, bits, M, K, N, g, signed, tile):
+    monkeypatch.setenv("MI_A16_GEMM_TILE", tile)  # both block shapes of the tiled kernel
+    if bits == 4:
+        cfg = S.w4a16(M, K, N, g, seed=M + K + N, bias=(N % 3 == 0))
+    else:
+        cfg = S.w8a16(M, K, N, g, seed=M + K, signed=signed, bias=(N % 2 == 0))
+    out, pre = _run_device(cfg)
+    _check_against_oracle(orc, cfg, out, pre)
+
+
+def test_prefill_gemm_full_width_and_f16_mode(orc):
+    cfg = S.w4a16(192, 1024, 1024, 128, seed=77, bias=True)
+    out, pre = _run_device(cfg)
+    _check_against_oracle(orc, cfg, out, pre)
+    # f16 activations / scales / outputs through the tiled kernel
+    M, K, N, g = 48, 512, 96, 64
+    cfg = S.w4a16(M, K, N, g, seed=6)
+    xf = orc.F16(S.bf16_to_f32(cfg["x"]))
+    sf = orc.F16(S.bf16_to_f32(cfg["scale"]))
+    cfg16 = dict(cfg)
+    cfg16["x"] = orc.f32_to_f16(xf)
+    cfg16["scale"] = orc.f32_to_f16(sf)
+    out, pre = _run_device(cfg16, dtype=clib.DT_F16)
+    want, want_pre = orc.a16matmul(xf, cfg["weight"].astype(np.float32), sf, cfg["zp"].astype(np.float32), None,
+                                   M=M, K=K, N=N, weight_bits=4, q_group_size=g, out_dtype=orc.OUT_F16)
+    assert cmp.max_abs_over_rms(pre, want_pre) <= 2e-5
+    assert np.array_equal(out, orc.f32_to_f16(pre))
+
+
 @pytest.mark.parametrize("M,K,N,g", W4_CASES)
 def test_w4a16_device_level(orc, M, K, N, g):
     cfg = S.w4a16(M, K, N, g, seed=M + K + N, bias=(N % 3 == 0))

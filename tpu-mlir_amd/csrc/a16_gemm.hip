@@ -1,0 +1,361 @@
+// W4A16 / W8A16 matmul for gfx950, many activation rows (prefill): a tiled MFMA GEMM that reads the same packed
+// weights as the skinny kernel.
+//
+// A workgroup (8 waves, two per SIMD) owns a GM x GN block of outputs.  Its activation rows stream through a ring of
+// LDS stages (128 columns of K each) with direct-to-LDS loads; weights never touch LDS: the packed layout hands each
+// lane exactly the MFMA B fragment of its output channel and k-quarter, so a wave loads the tiles of its own columns
+// straight into registers one stage ahead and dequantizes them there.
+//
+// Arithmetic is that of the skinny kernel (see a16_kernels.hip), per quantization group:
+//   4-bit: P = sum_k a_k (16 + q_k) by MFMA, S = sum_k a_k by one more MFMA against ones, then
+//          acc += scale * (P - (16 + zp) * S) in fp32.
+//   8-bit: the weight is rounded to the 16-bit type exactly as the reference does, and the MFMA accumulates directly.
+#include "a16_common.cuh"
+#include "internal.h"
+
+namespace mi {
+
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+constexpr int GEMM_KS = 128;     // K per LDS stage (one 4-bit weight tile, two 8-bit tiles)
+constexpr int GEMM_NST = 3;      // LDS ring depth
+constexpr int GEMM_WAVES = 8;
+constexpr int waitcnt_vm_only(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
+
+struct GemmArgs {
+  const u32x4 *qw;
+  const uint32_t *sz_t;
+  const uint16_t *scale_t;
+  const float *nzs_t;
+  const float *bias;
+  const uint16_t *x;
+  uint16_t *y;
+  float *y32;
+  int M;
+  int64_t K, N;
+  int row_blocks, k_tiles, G;
+  int tiles_per_group;  // GPT == 1: weight tiles that share one group (g / TILE_K; k_tiles when per channel)
+  int chip;
+  int tiles_m, tiles_n, per_xcd;
+};
+
+// WM x WN waves, each TM x TN MFMA tiles of 16 x 16:  GM = WM * TM * 16 rows, GN = WN * TN * 16 columns.
+template <int BITS, int DT, int GPT, int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a) {
+  static_assert(WM * WN == GEMM_WAVES, "eight waves per workgroup");
+  using H = Half16<DT>;
+  using vec8 = typename H::vec8;
+  constexpr int GM = WM * TM * 16, GN = WN * TN * 16;
+  constexpr int TILE_K = BITS == 4 ? W4_TILE_K : W8_TILE_K;
+  constexpr int WT = GEMM_KS / TILE_K;                 // weight tiles per stage: 1 (4-bit) or 2 (8-bit)
+  constexpr int KSTEPS = GEMM_KS / 32;                 // MFMA k-steps per stage
+  constexpr int UNITS = BITS == 4 ? GPT : WT * GPT;    // quantization groups per stage
+  constexpr int KSTEPS_PER_UNIT = KSTEPS / UNITS;
+  constexpr int STAGE_BYTES = GM * GEMM_KS * 2;
+  constexpr int XL = STAGE_BYTES / 16 / (GEMM_WAVES * 64);  // direct-to-LDS instructions per thread and stage
+  static_assert(KSTEPS_PER_UNIT >= 1, "at most one group per MFMA k-step");
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int col = lane & 15, kq = lane >> 4;
+
+  // workgroup -> output block: the hardware deals workgroups round-robin over the 8 XCDs; each XCD gets a contiguous
+  // run of the block order (column-major inside groups of 4 block-rows) so that its L2 sees few distinct panels
+  const int bid = blockIdx.x;
+  const int L = (bid & 7) * a.per_xcd + (bid >> 3);
+  if (L >= a.tiles_m * a.tiles_n)
+    return;
+  constexpr int GRP = 4;
+  const int group = L / (GRP * a.tiles_n);
+  const int gm = (a.tiles_m - group * GRP) < GRP ? (a.tiles_m - group * GRP) : GRP;
+  const int in_group = L - group * GRP * a.tiles_n;
+  const int tm = group * GRP + in_group % gm, tn = in_group / gm;
+  const int64_t m_base = (int64_t)tm * GM, n_base = (int64_t)tn * GN;
+
+  // ---- activations: direct-to-LDS plan.  A stage is GM rows x 16 chunks of 16 bytes; chunk c of row r is stored at
+  // position c ^ (r & 15) so that the 16 rows of an MFMA fragment read 16 different bank groups.
+  const uint16_t *gx[XL];
+#pragma unroll
+  for (int i = 0; i < XL; ++i) {
+    const int slot = (i * GEMM_WAVES + wave) * 64 + lane;
+    const int row = slot >> 4, pos = slot & 15;
+    const int chunk = pos ^ (row & 15);
+    int64_t m = m_base + row;
+    m = m < a.M ? m : a.M - 1;  // rows past M re-read the last row; their results are never stored
+    gx[i] = a.x + m * a.K + chunk * 8;
+  }
+  const int kt_total = (int)(a.K / GEMM_KS);
+  auto issue_x = [&](int kt) {
+    const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 1) * GEMM_KS;  // past the end: harmless re-load
+    uint8_t *st = lds + (kt % GEMM_NST) * STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < XL; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t)(gx[i] + koff), (lptr_t)(st + (i * GEMM_WAVES + wave) * 1024), 16, 0, 0);
+  };
+  int a_off[TM];  // byte offset of this lane's fragment row inside a stage
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+    a_off[i] = (wm * TM * 16 + i * 16 + col) * (GEMM_KS * 2);
+
+  // ---- weights: registers, one stage ahead
+  struct WStage {
+    u32x4 w[TN][WT];
+    uint32_t sz[TN][UNITS];  // 4-bit: scale << 16 | zp;  8-bit: scale bits
+    float nz[TN][UNITS];     // 8-bit only
+  };
+  const u32x4 *wq[TN];
+  const uint32_t *szp[TN];
+  const uint16_t *scp[TN];
+  const float *nzp[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    int64_t rb = n_base / 16 + (wn * TN + j);
+    rb = rb < a.row_blocks ? rb : a.row_blocks - 1;  // clamped, discarded at the store
+    wq[j] = a.qw + rb * a.k_tiles * 64 + lane;
+    if constexpr (BITS == 4) {
+      szp[j] = a.sz_t + rb * a.G * 16 + col;
+    } else {
+      scp[j] = a.scale_t + rb * a.G * 16 + col;
+      nzp[j] = a.nzs_t + rb * a.G * 16 + col;
+    }
+  }
+  auto unit_group = [&](int tile, int u) {
+    int gi;
+    if constexpr (GPT == 1)
+      gi = a.tiles_per_group == 1 ? tile : tile / a.tiles_per_group;
+    else
+      gi = tile * GPT + u;
+    return gi < a.G ? gi : a.G - 1;
+  };
+  auto load_w = [&](WStage &s, int kt) {
+    const int ktc = kt < kt_total ? kt : kt_total - 1;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int t = 0; t < WT; ++t) {
+        const int tile = ktc * WT + t;
+        s.w[j][t] = wq[j][(int64_t)tile * 64];
+#pragma unroll
+        for (int u = 0; u < GPT; ++u) {
+          const int gi = unit_group(tile, u);
+          if constexpr (BITS == 4) {
+            s.sz[j][t * GPT + u] = szp[j][gi * 16];
+          } else {
+            s.sz[j][t * GPT + u] = scp[j][gi * 16];
+            s.nz[j][t * GPT + u] = nzp[j][gi * 16];
+          }
+        }
+      }
+    }
+  };
+  constexpr int W_LOADS = TN * WT * (1 + GPT * (BITS == 4 ? 1 : 2));  // vector-memory instructions of one load_w
+
+  f32x4 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  const u32x4 ones_bits = {H::ONE2, H::ONE2, H::ONE2, H::ONE2};
+  const vec8 ones = __builtin_bit_cast(vec8, ones_bits);
+  uint32_t nib_magic = H::NIB_MAGIC2;
+  asm volatile("" : "+v"(nib_magic));  // keep it in a VGPR (see and_or)
+
+  auto compute_stage = [&](const WStage &s, int kt) {
+    const uint8_t *st = lds + (kt % GEMM_NST) * STAGE_BYTES;
+    f32x4 P[TM][TN], S[TM];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const bool first = (ks % KSTEPS_PER_UNIT) == 0;
+      vec8 af[TM];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int row15 = col;  // (wm*TM*16 + i*16 + col) & 15
+        const u32x4 v = *(const u32x4 *)(st + a_off[i] + (((ks * 4 + kq) ^ row15) << 4));
+        af[i] = __builtin_bit_cast(vec8, v);
+      }
+      if constexpr (BITS == 4) {
+        vec8 bf[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          bf[j] = unpack_nibbles<DT>(s.w[j][0][ks], nib_magic);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          S[i] = H::mfma(af[i], ones, first ? zero4 : S[i]);
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            P[i][j] = H::mfma(af[i], bf[j], first ? zero4 : P[i][j]);
+        }
+        if ((ks + 1) % KSTEPS_PER_UNIT == 0) {
+          const int u = ks / KSTEPS_PER_UNIT;
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            const float sc = H::to_f32((uint16_t)(s.sz[j][u] >> 16));
+            const float c = H::OFFSET + (float)(s.sz[j][u] & 0xffu);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+                acc[i][j][r] = fmaf(sc, fmaf(-c, S[i][r], P[i][j][r]), acc[i][j][r]);
+          }
+        }
+      } else {
+        // 8-bit tile t covers k-steps 2t, 2t+1: bytes [8(ks&1)*2 .. ) of the lane's 16
+        const int t = ks >> 1, h = ks & 1;
+        const int u = t * GPT + (GPT == 1 ? 0 : h);
+        vec8 bf[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          bf[j] = dequant_bytes<DT>(s.w[j][t][2 * h], s.w[j][t][2 * h + 1], H::to_f32((uint16_t)s.sz[j][u]), s.nz[j][u]);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = H::mfma(af[i], bf[j], acc[i][j]);
+      }
+    }
+  };
+
+  // ---- pipeline.  At the top of stage kt a wave has outstanding, in issue order: ..., x(kt) [requested two stages
+  // ago], W(kt) then x(kt+1) [requested one stage ago].  Waiting until only the XL requests of x(kt+1) remain means
+  // x(kt) and W(kt) have landed; the barrier then also says every wave is done reading stage kt-1, whose buffer
+  // takes x(kt+2).
+  WStage wa, wb;
+  issue_x(0);
+  load_w(wa, 0);
+  issue_x(1);
+  auto stage = [&](WStage &cur, WStage &nxt, int kt) {
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_only(XL));
+    __builtin_amdgcn_s_barrier();
+    load_w(nxt, kt + 1);
+    issue_x(kt + 2);
+    compute_stage(cur, kt);
+  };
+  int kt = 0;
+  for (; kt + 1 < kt_total; kt += 2) {
+    stage(wa, wb, kt);
+    stage(wb, wa, kt + 1);
+  }
+  if (kt < kt_total)
+    stage(wa, wb, kt);
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_only(0));  // drain the re-loads issued past the end
+  (void)W_LOADS;
+
+  // ---- epilogue: lane holds column (l & 15), rows 4 (l >> 4) + r of each 16 x 16 tile
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int64_t n = n_base + (wn * TN + j) * 16 + col;
+    const bool n_ok = n < a.N;
+    const float b = (a.bias && n_ok) ? a.bias[n] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int64_t m = m_base + (wm * TM + i) * 16 + 4 * kq + r;
+        if (n_ok && m < a.M) {
+          const float v = acc[i][j][r] + b;
+          const int64_t o = m * a.N + n;
+          if (a.y32)
+            a.y32[o] = v;
+          a.y[o] = (a.chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+        }
+      }
+  }
+}
+
+template <int BITS, int DT, int GPT, int WM, int WN, int TM, int TN>
+static void launch_gemm_instance(GemmArgs &a, hipStream_t st) {
+  constexpr int GM = WM * TM * 16, GN = WN * TN * 16;
+  a.tiles_m = (int)((a.M + GM - 1) / GM);
+  a.tiles_n = (int)((a.N + GN - 1) / GN);
+  a.per_xcd = (a.tiles_m * a.tiles_n + 7) / 8;
+  auto kfn = a16_gemm_kernel<BITS, DT, GPT, WM, WN, TM, TN>;
+  const size_t lds_bytes = (size_t)GEMM_NST * GM * GEMM_KS * 2;
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    attr_set = true;
+  }
+  kfn<<<dim3((unsigned)(a.per_xcd * 8)), dim3(GEMM_WAVES * 64), lds_bytes, st>>>(a);
+}
+
+template <int BITS, int DT, int GPT>
+static void launch_gemm_shape(GemmArgs &a, hipStream_t st) {
+  // 128 x 256 blocks when they fill the chip, else 128 x 128
+  const int64_t big = ((a.M + 127) / 128) * ((a.N + 255) / 256);
+  const char *e = getenv("MI_A16_GEMM_TILE");  // development switch: "256" / "128"
+  const bool wide = e ? atoi(e) == 256 : big >= 192;
+  if (wide)
+    launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 4>(a, st);
+  else
+    launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 2>(a, st);
+}
+
+bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M) {
+  if (getenv("MI_A16_NO_GEMM"))
+    return false;
+  const int tile_k = w->bits == 4 ? W4_TILE_K : W8_TILE_K;
+  const int g = w->g;
+  // whole LDS stages, at most one group per MFMA k-step, groups that do not straddle a weight tile
+  const bool group_ok = g == 0 || (g >= tile_k && g % tile_k == 0) || (g < tile_k && tile_k % g == 0 && g >= 32);
+  return M > 16 && (w->K % GEMM_KS) == 0 && group_ok;
+}
+
+int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
+                    hipStream_t stream) {
+  GemmArgs a;
+  a.qw = (const u32x4 *)w->qweight;
+  a.sz_t = w->sz_t;
+  a.scale_t = w->scale_t;
+  a.nzs_t = w->nzs_t;
+  a.bias = w->bias;
+  a.x = d_x;
+  a.y = d_y;
+  a.y32 = d_y32;
+  a.M = (int)M;
+  a.K = w->K;
+  a.N = w->N;
+  a.row_blocks = (int)w->row_blocks;
+  a.k_tiles = (int)w->k_tiles;
+  a.G = w->G;
+  a.chip = w->chip;
+  a.tiles_per_group = 1;
+  const int tile_k = w->bits == 4 ? W4_TILE_K : W8_TILE_K;
+  int gpt = 1;
+  if (w->g == 0)
+    a.tiles_per_group = (int)w->k_tiles;
+  else if (w->g >= tile_k)
+    a.tiles_per_group = w->g / tile_k;
+  else
+    gpt = tile_k / w->g;
+  const bool f16 = w->dtype == MI_DT_F16;
+#define MI_GEMM(BITS_, GPT_)                                      \
+  {                                                               \
+    if (f16)                                                      \
+      launch_gemm_shape<BITS_, MI_DT_F16, GPT_>(a, stream);       \
+    else                                                          \
+      launch_gemm_shape<BITS_, MI_DT_BF16, GPT_>(a, stream);      \
+  }
+  if (w->bits == 4) {
+    if (gpt == 1)
+      MI_GEMM(4, 1)
+    else if (gpt == 2)
+      MI_GEMM(4, 2)
+    else
+      MI_GEMM(4, 4)
+  } else {
+    if (gpt == 1)
+      MI_GEMM(8, 1)
+    else
+      MI_GEMM(8, 2)
+  }
+#undef MI_GEMM
+  MI_HIP(hipGetLastError());
+  return MI_SUCCESS;
+}
+
+}  // namespace mi

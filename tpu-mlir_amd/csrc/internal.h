@@ -64,6 +64,10 @@ int a16_pack(mi_a16_weight *w, const void *h_weight, int weight_signed, const ui
 void a16_free(mi_a16_weight *w);
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                hipStream_t stream);
+// tiled MFMA GEMM for many activation rows (prefill)
+bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M);
+int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
+                    hipStream_t stream);
 int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
                      float *const *d_y32s, hipStream_t stream);
 
