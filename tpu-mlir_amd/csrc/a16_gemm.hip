@@ -2,9 +2,10 @@
 // weights as the skinny kernel.
 //
 // A workgroup (8 waves, two per SIMD) owns a GM x GN block of outputs.  Its activation rows stream through a ring of
-// LDS stages (128 columns of K each) with direct-to-LDS loads; weights never touch LDS: the packed layout hands each
-// lane exactly the MFMA B fragment of its output channel and k-quarter, so a wave loads the tiles of its own columns
-// straight into registers one stage ahead and dequantizes them there.
+// LDS stages (128 columns of K each) filled by direct-to-LDS loads.  The packed weight layout hands each lane exactly
+// the MFMA B fragment of its output channel and k-quarter, so weights need no rearranging: 4-bit tiles (and their
+// scale|zero-point words) ride the same LDS ring, which keeps two stages of them in flight without costing
+// registers; 8-bit tiles are loaded straight into registers one stage ahead.  Dequantization happens in registers.
 //
 // Arithmetic is that of the skinny kernel (see a16_kernels.hip), per quantization group:
 //   4-bit: P = sum_k a_k (16 + q_k) by MFMA, S = sum_k a_k by one more MFMA against ones, then
@@ -22,6 +23,16 @@ constexpr int GEMM_KS = 128;     // K per LDS stage (one 4-bit weight tile, two 
 constexpr int GEMM_NST = 3;      // LDS ring depth
 constexpr int GEMM_WAVES = 8;
 constexpr int waitcnt_vm_only(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
+
+#ifdef MI_GEMM_TIMING
+__device__ unsigned long long mi_gemm_dbg[64 * 8];
+extern "C" int mi_gemm_dbg_dump(unsigned long long *host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mi_gemm_dbg), sizeof(mi_gemm_dbg));
+}
+#define MI_GT(v) const unsigned long long v = __builtin_readcyclecounter()
+#else
+#define MI_GT(v)
+#endif
 
 struct GemmArgs {
   const u32x4 *qw;
@@ -52,8 +63,16 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
   constexpr int KSTEPS = GEMM_KS / 32;                 // MFMA k-steps per stage
   constexpr int UNITS = BITS == 4 ? GPT : WT * GPT;    // quantization groups per stage
   constexpr int KSTEPS_PER_UNIT = KSTEPS / UNITS;
-  constexpr int STAGE_BYTES = GM * GEMM_KS * 2;
-  constexpr int XL = STAGE_BYTES / 16 / (GEMM_WAVES * 64);  // direct-to-LDS instructions per thread and stage
+  constexpr bool WLDS = BITS == 4;                     // weights and group parameters through the LDS ring
+  constexpr int X_BYTES = GM * GEMM_KS * 2;
+  constexpr int W_BYTES = WLDS ? (GN / 16) * 1024 : 0;         // one 1 KiB tile per 16 output channels
+  constexpr int SZ_BYTES = WLDS ? GEMM_WAVES * GPT * 256 : 0;  // per wave and group: 64 scale|zp words
+  constexpr int STAGE_BYTES = X_BYTES + W_BYTES + SZ_BYTES;
+  constexpr int XL = X_BYTES / 16 / (GEMM_WAVES * 64);  // activation direct-to-LDS instructions per thread and stage
+  constexpr int WL = W_BYTES / 1024 / GEMM_WAVES;        // weight tiles each wave requests per stage
+  constexpr int LPS = XL + WL + (WLDS ? GPT : 0);        // direct-to-LDS instructions per thread and stage
+  static_assert(!WLDS || (GN / 16) % GEMM_WAVES == 0, "weight tiles split evenly over the waves");
+  static_assert(GEMM_NST * STAGE_BYTES <= 160 * 1024, "LDS ring exceeds 160 KiB");
   static_assert(KSTEPS_PER_UNIT >= 1, "at most one group per MFMA k-step");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
@@ -88,12 +107,44 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
     gx[i] = a.x + m * a.K + chunk * 8;
   }
   const int kt_total = (int)(a.K / GEMM_KS);
+  // this wave's share of the weight tiles of the block, and the scale|zp words of its own columns (lane l fetches
+  // channel l & 15 of its row block (l >> 4) % TN)
+  int64_t w_tile_rb[WL > 0 ? WL : 1];
+  int64_t sz_rb = 0;
+  if constexpr (WLDS) {
+#pragma unroll
+    for (int i = 0; i < WL; ++i) {
+      int64_t rb = n_base / 16 + (i * GEMM_WAVES + wave);
+      w_tile_rb[i] = rb < a.row_blocks ? rb : a.row_blocks - 1;  // clamped, discarded at the store
+    }
+    sz_rb = n_base / 16 + wn * TN + (kq & (TN - 1));
+    sz_rb = sz_rb < a.row_blocks ? sz_rb : a.row_blocks - 1;
+  }
+  auto unit_group = [&](int tile, int u) {
+    int gi;
+    if constexpr (GPT == 1)
+      gi = a.tiles_per_group == 1 ? tile : tile / a.tiles_per_group;
+    else
+      gi = tile * GPT + u;
+    return gi < a.G ? gi : a.G - 1;
+  };
   auto issue_x = [&](int kt) {
-    const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 1) * GEMM_KS;  // past the end: harmless re-load
+    const int ktc = kt < kt_total ? kt : kt_total - 1;  // past the end: harmless re-load
+    const int64_t koff = (int64_t)ktc * GEMM_KS;
     uint8_t *st = lds + (kt % GEMM_NST) * STAGE_BYTES;
 #pragma unroll
     for (int i = 0; i < XL; ++i)
       __builtin_amdgcn_global_load_lds((gptr_t)(gx[i] + koff), (lptr_t)(st + (i * GEMM_WAVES + wave) * 1024), 16, 0, 0);
+    if constexpr (WLDS) {
+#pragma unroll
+      for (int i = 0; i < WL; ++i)
+        __builtin_amdgcn_global_load_lds((gptr_t)(a.qw + (w_tile_rb[i] * a.k_tiles + ktc) * 64 + lane),
+                                         (lptr_t)(st + X_BYTES + (i * GEMM_WAVES + wave) * 1024), 16, 0, 0);
+#pragma unroll
+      for (int u = 0; u < GPT; ++u)
+        __builtin_amdgcn_global_load_lds((gptr_t)(a.sz_t + (sz_rb * a.G + unit_group(ktc, u)) * 16 + col),
+                                         (lptr_t)(st + X_BYTES + W_BYTES + (wave * GPT + u) * 256), 4, 0, 0);
+    }
   };
   int a_off[TM];  // byte offset of this lane's fragment row inside a stage
 #pragma unroll
@@ -107,30 +158,19 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
     float nz[TN][UNITS];     // 8-bit only
   };
   const u32x4 *wq[TN];
-  const uint32_t *szp[TN];
   const uint16_t *scp[TN];
   const float *nzp[TN];
+  if constexpr (!WLDS) {
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    int64_t rb = n_base / 16 + (wn * TN + j);
-    rb = rb < a.row_blocks ? rb : a.row_blocks - 1;  // clamped, discarded at the store
-    wq[j] = a.qw + rb * a.k_tiles * 64 + lane;
-    if constexpr (BITS == 4) {
-      szp[j] = a.sz_t + rb * a.G * 16 + col;
-    } else {
+    for (int j = 0; j < TN; ++j) {
+      int64_t rb = n_base / 16 + (wn * TN + j);
+      rb = rb < a.row_blocks ? rb : a.row_blocks - 1;  // clamped, discarded at the store
+      wq[j] = a.qw + rb * a.k_tiles * 64 + lane;
       scp[j] = a.scale_t + rb * a.G * 16 + col;
       nzp[j] = a.nzs_t + rb * a.G * 16 + col;
     }
   }
-  auto unit_group = [&](int tile, int u) {
-    int gi;
-    if constexpr (GPT == 1)
-      gi = a.tiles_per_group == 1 ? tile : tile / a.tiles_per_group;
-    else
-      gi = tile * GPT + u;
-    return gi < a.G ? gi : a.G - 1;
-  };
-  auto load_w = [&](WStage &s, int kt) {
+  auto load_w = [&](WStage &s, int kt) {  // 8-bit: global -> registers, issued one stage ahead
     const int ktc = kt < kt_total ? kt : kt_total - 1;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
@@ -141,17 +181,22 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
 #pragma unroll
         for (int u = 0; u < GPT; ++u) {
           const int gi = unit_group(tile, u);
-          if constexpr (BITS == 4) {
-            s.sz[j][t * GPT + u] = szp[j][gi * 16];
-          } else {
-            s.sz[j][t * GPT + u] = scp[j][gi * 16];
-            s.nz[j][t * GPT + u] = nzp[j][gi * 16];
-          }
+          s.sz[j][t * GPT + u] = scp[j][gi * 16];
+          s.nz[j][t * GPT + u] = nzp[j][gi * 16];
         }
       }
     }
   };
-  constexpr int W_LOADS = TN * WT * (1 + GPT * (BITS == 4 ? 1 : 2));  // vector-memory instructions of one load_w
+  auto read_w = [&](WStage &s, int kt) {  // 4-bit: this wave's tiles and words out of the landed LDS stage
+    const uint8_t *st = lds + (kt % GEMM_NST) * STAGE_BYTES + X_BYTES;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      s.w[j][0] = *(const u32x4 *)(st + (wn * TN + j) * 1024 + lane * 16);
+#pragma unroll
+      for (int u = 0; u < GPT; ++u)
+        s.sz[j][u] = *(const uint32_t *)(st + W_BYTES + (wave * GPT + u) * 256 + (j * 16 + col) * 4);
+    }
+  };
 
   f32x4 acc[TM][TN];
 #pragma unroll
@@ -220,20 +265,42 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
     }
   };
 
-  // ---- pipeline.  At the top of stage kt a wave has outstanding, in issue order: ..., x(kt) [requested two stages
-  // ago], W(kt) then x(kt+1) [requested one stage ago].  Waiting until only the XL requests of x(kt+1) remain means
-  // x(kt) and W(kt) have landed; the barrier then also says every wave is done reading stage kt-1, whose buffer
-  // takes x(kt+2).
+  // ---- pipeline.  Stage kt+NST-1 is requested at the top of stage kt, right after the barrier that says every wave
+  // is done with stage kt-1 (whose buffer it takes).  Before that barrier a wave waits for its own share of stage
+  // kt: requests complete in order, so "at most (NST-2) stages' worth outstanding" means stage kt has landed.
+  // 8-bit weights additionally travel global -> registers one stage ahead, between the two.
   WStage wa, wb;
-  issue_x(0);
-  load_w(wa, 0);
-  issue_x(1);
+#pragma unroll
+  for (int s0 = 0; s0 < GEMM_NST - 1; ++s0) {
+    if (!WLDS && s0 == 1)
+      load_w(wa, 0);  // issue order: x(0), W(0), x(1)
+    issue_x(s0);
+  }
+#ifdef MI_GEMM_TIMING
+  unsigned long long t_wait = 0, t_bar = 0, t_issue = 0, t_comp = 0;
+  const unsigned long long t_begin = __builtin_readcyclecounter();
+#endif
   auto stage = [&](WStage &cur, WStage &nxt, int kt) {
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm_only(XL));
+    MI_GT(g0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_only((GEMM_NST - 2) * LPS));
+    MI_GT(g1);
     __builtin_amdgcn_s_barrier();
-    load_w(nxt, kt + 1);
-    issue_x(kt + 2);
+    MI_GT(g2);
+    if constexpr (WLDS)
+      read_w(cur, kt);
+    else
+      load_w(nxt, kt + 1);
+    issue_x(kt + GEMM_NST - 1);
+    MI_GT(g3);
     compute_stage(cur, kt);
+#ifdef MI_GEMM_TIMING
+    __builtin_amdgcn_sched_barrier(0);
+    const unsigned long long g4 = __builtin_readcyclecounter();
+    t_wait += g1 - g0;
+    t_bar += g2 - g1;
+    t_issue += g3 - g2;
+    t_comp += g4 - g3;
+#endif
   };
   int kt = 0;
   for (; kt + 1 < kt_total; kt += 2) {
@@ -243,7 +310,16 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
   if (kt < kt_total)
     stage(wa, wb, kt);
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_only(0));  // drain the re-loads issued past the end
-  (void)W_LOADS;
+#ifdef MI_GEMM_TIMING
+  if (lane == 0 && blockIdx.x < 64 && wave == 0) {
+    unsigned long long *d = mi_gemm_dbg + blockIdx.x * 8;
+    d[0] = __builtin_readcyclecounter() - t_begin;
+    d[1] = t_wait;
+    d[2] = t_bar;
+    d[3] = t_issue;
+    d[4] = t_comp;
+  }
+#endif
 
   // ---- epilogue: lane holds column (l & 15), rows 4 (l >> 4) + r of each 16 x 16 tile
 #pragma unroll
@@ -274,7 +350,7 @@ static void launch_gemm_instance(GemmArgs &a, hipStream_t st) {
   a.tiles_n = (int)((a.N + GN - 1) / GN);
   a.per_xcd = (a.tiles_m * a.tiles_n + 7) / 8;
   auto kfn = a16_gemm_kernel<BITS, DT, GPT, WM, WN, TM, TN>;
-  const size_t lds_bytes = (size_t)GEMM_NST * GM * GEMM_KS * 2;
+  const size_t lds_bytes = (size_t)GEMM_NST * (GM * GEMM_KS * 2 + (BITS == 4 ? (GN / 16) * 1024 + GEMM_WAVES * GPT * 256 : 0));
   static bool attr_set = false;
   if (!attr_set) {
     (void)hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -288,11 +364,16 @@ static void launch_gemm_shape(GemmArgs &a, hipStream_t st) {
   // 128 x 256 blocks when they fill the chip, else 128 x 128
   const int64_t big = ((a.M + 127) / 128) * ((a.N + 255) / 256);
   const char *e = getenv("MI_A16_GEMM_TILE");  // development switch: "256" / "128"
-  const bool wide = e ? atoi(e) == 256 : big >= 192;
-  if (wide)
-    launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 4>(a, st);
-  else
-    launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 2>(a, st);
+  constexpr bool fits = !(BITS == 4 && GPT == 4);  // 32-wide groups: a 256-column block's scale|zp words overflow LDS
+  const bool wide = fits && (e ? atoi(e) == 256 : big >= 192);
+  if constexpr (fits) {
+    if (wide) {
+      launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 4>(a, st);
+      return;
+    }
+  }
+  (void)wide;
+  launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 2>(a, st);
 }
 
 bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M) {
