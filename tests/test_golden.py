@@ -1,0 +1,170 @@
+"""The committed fixtures of tests/golden/ (made by tests/golden/make_fixtures.py).
+
+CPU part: the oracle against the known-answer files (computed from the published definitions with exact
+integer/rational arithmetic, independent of the oracle) and against its own frozen operator cases.
+GPU part (marked gpu): the HIP path, through the C ABI, against the same operator cases.  Bars: integer work
+bit-exact; bf16 outputs equal to the reference rounding of an fp32 result that agrees with the fixture's
+double-accumulated fp32 to max-abs <= 2e-5 * RMS.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from helpers import pkg, f32_valued_a16
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+S = pkg("synth")
+A16_CASES = ["w4_g64_bias", "w4_g128_ragged", "w4_per_channel", "w8_per_channel", "w8_g32_unsigned", "w4_prefill"]
+
+
+def _load(name):
+    return np.load(os.path.join(GOLD, name), allow_pickle=False)
+
+
+def _a16_cfg(d):
+    M, K, N, g, bits = [int(v) for v in d["meta"]]
+    return {"x": d["x"], "weight": d["weight"], "scale": d["scale"], "zp": d["zp"],
+            "bias": d["bias"] if d["bias"].size else None, "M": M, "K": K, "N": N, "g": g, "bits": bits}
+
+
+# ----------------------------------------------------------------------------------------------- CPU
+def test_oracle_right_shift_round_known_answers(orc):
+    d = _load("kat_right_shift_round.npz")
+    for mode in np.unique(d["mode"]):
+        m = d["mode"] == mode
+        got = orc.right_shift_round(d["x"][m], d["shift"][m].astype(np.int32), int(mode))
+        assert np.array_equal(got, d["want"][m]), "mode %d" % mode
+    # enum values RightShiftRound has no branch for (MathUtils.cpp:475-514: half-to-odd, half-towards-zero,
+    # away-from-zero) leave the arithmetic shift, i.e. floor
+    m = d["mode"] == orc.DOWN
+    for other in (orc.HALF_TO_ODD, orc.HALF_TOWARDS_ZERO, orc.AWAY_FROM_ZERO):
+        assert np.array_equal(orc.right_shift_round(d["x"][m], d["shift"][m].astype(np.int32), other), d["want"][m])
+
+
+def test_oracle_mbqm_known_answers(orc):
+    d = _load("kat_mbqm.npz")
+    for mode in np.unique(d["mode"]):
+        m = d["mode"] == mode
+        got = orc.mbqm(d["x"][m], d["mult"][m], d["shift"][m], int(mode))
+        assert np.array_equal(got.astype(np.int64), d["want"][m]), "mode %d" % mode
+
+
+def test_oracle_float16_known_answers(orc):
+    d = _load("kat_float16.npz")
+    assert np.array_equal(orc.f32_to_bf16(d["f32_bits"].view(np.float32)), d["bf16"])
+    assert np.array_equal(orc.f32_to_f16(d["f16_in_bits"].view(np.float32)), d["f16"])
+    assert np.array_equal(orc.f32_to_bf16(d["special_f32_bits"].view(np.float32)), d["special_bf16_bm"])
+
+
+@pytest.mark.parametrize("name", A16_CASES)
+def test_oracle_reproduces_a16_cases(orc, name):
+    d = _load("case_a16_%s.npz" % name)
+    cfg = _a16_cfg(d)
+    x, w, s, z, b = f32_valued_a16(cfg)
+    out, pre = orc.a16matmul(x, w, s, z, b, M=cfg["M"], K=cfg["K"], N=cfg["N"], weight_bits=cfg["bits"],
+                             q_group_size=cfg["g"], gemm_kind=orc.GEMM_F64ACC)
+    assert np.array_equal(orc.f32_to_bf16(out), d["want_bf16"])
+    assert np.array_equal(pre, d["want_pre"])
+
+
+I8_RUNS = {
+    "r1_fused_per_channel": dict(per_channel=True, kw=dict(quant_mode="MULTIPLIER_SHIFT", fuse_rq=True,
+                                                           rshifts=[22] * 40, out_zp=3)),
+    "r2_scalar_relu_u8": dict(kw=dict(multipliers=[3500], rshifts=[20], do_relu=True, out_unsigned=True)),
+    "r3_tflite": dict(kw=dict(quant_mode="TFLITE", multipliers=[(1 << 30) + 424242], rshifts=[9], out_zp=-5)),
+    "r4_cv18xx_qdm": dict(kw=dict(cv18xx=True, quant_mode="QDM", multipliers=[(1 << 30) + 424242], rshifts=[8])),
+    "r5_cv18xx_mshift": dict(kw=dict(cv18xx=True, quant_mode="MULTIPLIER_SHIFT", multipliers=[77], rshifts=[13])),
+    "r6_int32_zero_points": dict(kw=dict(input_zp=5, right_zp=-3, out_kind=1)),
+}
+
+
+@pytest.mark.parametrize("name", sorted(I8_RUNS))
+def test_oracle_reproduces_int8_cases(orc, name):
+    d = _load("case_i8_matmul.npz")
+    r = I8_RUNS[name]
+    kw = dict(r["kw"])
+    if "quant_mode" in kw:
+        kw["quant_mode"] = getattr(orc, "RQ_" + kw["quant_mode"])
+    multi = d["mult"].astype(np.float32) if r.get("per_channel") else None
+    want, _ = orc.matmul_int8(d["a"].astype(np.float32), d["b"].astype(np.float32), d["bias"].astype(np.float32),
+                              multi, M=24, K=192, N=40, **kw)
+    assert np.array_equal(want.astype(np.int32), d["want_" + name])
+
+
+def test_oracle_reproduces_requant_cases(orc):
+    d = _load("case_requant.npz")
+    got = orc.requant_int_axis(d["x"], d["quant"], quant_mode=orc.RQ_TFLITE, round_mode=orc.HALF_AWAY_FROM_ZERO)
+    assert np.array_equal(got.astype(np.int32), d["want_axis"])
+    got = orc.requant_int(d["x"], multiplier=91, rshift=11, quant_mode=orc.RQ_MULTIPLIER_SHIFT, round_mode=orc.HALF_UP)
+    assert np.array_equal(got.astype(np.int32), d["want_int"])
+
+
+# ----------------------------------------------------------------------------------------------- GPU
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", A16_CASES)
+def test_gpu_a16_against_fixture(name, monkeypatch):
+    import torch
+    M_ = pkg()
+    cmp = pkg("compare")
+    monkeypatch.setenv("MI_A16_GEMM_MIN_M", "17")  # w4_prefill (M = 40) goes through the tiled kernel
+    d = _load("case_a16_%s.npz" % name)
+    cfg = _a16_cfg(d)
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"],
+                     None if cfg["bias"] is None else S.bf16_to_f32(cfg["bias"]),
+                     K=cfg["K"], N=cfg["N"], weight_bits=cfg["bits"], q_group_size=cfg["g"])
+    x = torch.from_numpy(cfg["x"].view(np.int16)).cuda().view(torch.bfloat16)
+    y32 = torch.empty((cfg["M"], cfg["N"]), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_launch(w, x, y_f32=y32)
+    torch.cuda.synchronize()
+    pre = y32.cpu().numpy()
+    out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    w.destroy()
+    assert cmp.max_abs_over_rms(pre, d["want_pre"]) <= 2e-5
+    # outputs: equal to the fixture except where the two fp32 results straddle a bf16 rounding boundary
+    rms = float(np.sqrt(np.mean(d["want_pre"].astype(np.float64) ** 2)))
+    diff = np.abs(S.bf16_to_f32(out) - S.bf16_to_f32(d["want_bf16"]))
+    ulp = np.abs(S.bf16_to_f32(d["want_bf16"])) * 2.0 ** -7
+    assert np.all((diff <= ulp) | (diff <= 4e-5 * rms))
+    assert np.mean(out != d["want_bf16"]) < 0.005
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(I8_RUNS))
+def test_gpu_int8_against_fixture(name):
+    M_ = pkg()
+    clib = pkg("clib")
+    d = _load("case_i8_matmul.npz")
+    r = I8_RUNS[name]
+    kw = dict(r["kw"])
+    a, b, bias = d["a"].astype(np.float32), d["b"].astype(np.float32), d["bias"].astype(np.float32)
+    args = dict(K=192, N=40)
+    if "quant_mode" in kw:
+        args["quant_mode"] = getattr(clib, "RQ_" + kw.pop("quant_mode"))
+    if kw.pop("cv18xx", False):
+        args["chip"] = clib.CHIP_CV18XX
+    if kw.pop("out_unsigned", False):
+        args["out_dtype"] = clib.DT_U8
+    if kw.pop("out_kind", 0) == 1:
+        args["out_dtype"] = clib.DT_I32
+    args.update(kw)
+    op = M_.MatMulInt8(**args)
+    if r.get("per_channel"):
+        op.init(a, b, bias, d["mult"].astype(np.float32))
+    else:
+        op.init(a, b, bias)
+    got = op.inference(a)
+    op.deinit()
+    assert np.array_equal(got.astype(np.int32), d["want_" + name])
+
+
+@pytest.mark.gpu
+def test_gpu_requant_against_fixture():
+    M_ = pkg()
+    clib = pkg("clib")
+    d = _load("case_requant.npz")
+    got = M_.requant_int_axis(d["x"], d["quant"], quant_mode=clib.RQ_TFLITE, round_mode=clib.ROUND_HALF_AWAY_FROM_ZERO)
+    assert np.array_equal(got.astype(np.int32), d["want_axis"])
+    got = M_.requant_int(d["x"], multiplier=91, rshift=11, quant_mode=clib.RQ_MULTIPLIER_SHIFT,
+                         round_mode=clib.ROUND_HALF_UP)
+    assert np.array_equal(got.astype(np.int32), d["want_int"])

@@ -88,6 +88,7 @@ PREFILL_CASES = [  # (bits, M, K, N, g, signed): M > 16 takes the tiled MFMA GEM
 @pytest.mark.parametrize("bits,M,K,N,g,signed", PREFILL_CASES)
 def test_prefill_gemm_device_level(orc, monkeypatch, bits, M, K, N, g, signed, tile):
     monkeypatch.setenv("MI_A16_GEMM_TILE", tile)  # both block shapes of the tiled kernel
+    monkeypatch.setenv("MI_A16_GEMM_MIN_M", "17")  # ... from the smallest M it accepts (default: 160 rows and up)
     if bits == 4:
         cfg = S.w4a16(M, K, N, g, seed=M + K + N, bias=(N % 3 == 0))
     else:
@@ -96,7 +97,8 @@ def test_prefill_gemm_device_level(orc, monkeypatch, bits, M, K, N, g, signed, t
     _check_against_oracle(orc, cfg, out, pre)
 
 
-def test_prefill_gemm_full_width_and_f16_mode(orc):
+def test_prefill_gemm_full_width_and_f16_mode(orc, monkeypatch):
+    monkeypatch.setenv("MI_A16_GEMM_MIN_M", "17")
     cfg = S.w4a16(192, 1024, 1024, 128, seed=77, bias=True)
     out, pre = _run_device(cfg)
     _check_against_oracle(orc, cfg, out, pre)

@@ -383,7 +383,10 @@ bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M) {
   const int g = w->g;
   // whole LDS stages, at most one group per MFMA k-step, groups that do not straddle a weight tile
   const bool group_ok = g == 0 || (g >= tile_k && g % tile_k == 0) || (g < tile_k && tile_k % g == 0 && g >= 32);
-  return M > 16 && (w->K % GEMM_KS) == 0 && group_ok;
+  // below about 160 rows the skinny kernel (one pass over the weights per 16 rows) is still faster
+  const char *e = getenv("MI_A16_GEMM_MIN_M");  // development / test switch
+  const int64_t min_m = e ? atoll(e) : 160;
+  return M >= min_m && M > 16 && (w->K % GEMM_KS) == 0 && group_ok;
 }
 
 int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
