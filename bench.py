@@ -117,14 +117,15 @@ def bench_chain(pkg, S, torch, M, steps, warmup, n_layers, cfgs, grouped=True):
     return res
 
 
-def bench_int8(pkg, S, torch, clib, n, steps, warmup):
-    """INT8 requant GEMM, M = N = K = n, per-channel Q31 multiplier + right shift, int8 output."""
-    c = S.int8_matmul(n, n, n, seed=7, right_transpose=True)
+def bench_int8(pkg, S, torch, clib, n, steps, warmup, M=None):
+    """INT8 requant GEMM, N = K = n and M rows (default n), per-channel Q31 multiplier + right shift, int8 output."""
+    M = n if M is None else M
+    c = S.int8_matmul(M, n, n, seed=7, right_transpose=True)
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
     a, b, bias = dev(c["a"]), dev(c["b"]), dev(c["bias"])
     rq = pkg.RequantDesc(clib.RQ_QDM, clib.ROUND_HALF_AWAY_FROM_ZERO, out_dtype=clib.DT_I8,
                          multiplier=dev(c["mult"]), shift=dev(c["shift"]))
-    out = torch.empty((n, n), dtype=torch.int8, device="cuda")
+    out = torch.empty((M, n), dtype=torch.int8, device="cuda")
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         for _ in range(warmup):
@@ -137,10 +138,93 @@ def bench_int8(pkg, S, torch, clib, n, steps, warmup):
         ev1.record(stream)
         stream.synchronize()
     sec = ev0.elapsed_time(ev1) * 1e-3 / steps
-    tops = 2.0 * n * n * n / sec / 1e12
-    return {"workload": "int8_requant_gemm_M%d_N%d_K%d_qdm_per_channel" % (n, n, n), "tops": round(tops, 2),
+    tops = 2.0 * M * n * n / sec / 1e12
+    return {"workload": "int8_requant_gemm_M%d_N%d_K%d_qdm_per_channel" % (M, n, n), "tops": round(tops, 2),
             "us_per_launch": round(sec * 1e6, 2), "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4),
             "dtype": "int8*int8->int32->int8"}
+
+
+def _time_launches(torch, fn, steps, warmup=5):
+    """Average device time of fn() (which enqueues on the current stream), by HIP events, in seconds."""
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(warmup):
+            fn()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        stream.synchronize()
+        ev0.record(stream)
+        for _ in range(steps):
+            fn()
+        ev1.record(stream)
+        stream.synchronize()
+    return ev0.elapsed_time(ev1) * 1e-3 / steps
+
+
+def bench_single_matmuls(pkg, S, torch, steps=60):
+    """Per-matmul figures of the secondary configurations: decode GEMVs (HBM GB/s of algorithmic bytes) and
+    prefill GEMMs (TFLOP/s).  Each case rotates over enough weight copies to stay out of the 256 MB cache when the
+    weights are small enough for that to matter."""
+    out = []
+
+    def one(tag, bits, M, K, N, g, copies):
+        cfg = S.w4a16(1, K, N, g, seed=31) if bits == 4 else S.w8a16(1, K, N, g, seed=31)
+        ws = [pkg.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=K, N=N, weight_bits=bits, q_group_size=g)
+              for _ in range(copies)]
+        x = _dev_bf16(torch, S.bf16_round(np.random.default_rng(5).standard_normal((M, K), dtype=np.float32)))
+        y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+        g_ = torch.cuda.CUDAGraph()
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            for w in ws:
+                pkg.a16mm_launch(w, x, y)
+            stream.synchronize()
+            with torch.cuda.graph(g_, stream=stream):
+                for w in ws:
+                    pkg.a16mm_launch(w, x, y)
+        sec = _time_launches(torch, g_.replay, max(3, steps // copies)) / copies
+        nbytes = S.w4_gemv_bytes(M, K, N, g) if bits == 4 else S.w8_gemv_bytes(M, K, N, g)
+        rec = {"case": tag, "bits": bits, "M": M, "K": K, "N": N, "g": g, "us": round(sec * 1e6, 2)}
+        if M <= 32:
+            rec["GBps"] = round(nbytes / sec / 1e9, 1)
+            rec["frac_hbm_peak"] = round(nbytes / sec / 1e9 / HBM_PEAK_GBS, 4)
+        else:
+            rec["TFLOPs"] = round(2.0 * M * N * K / sec / 1e12, 1)
+            rec["frac_bf16_peak"] = round(2.0 * M * N * K / sec / 1e12 / BF16_PEAK_TFLOPS, 4)
+        out.append(rec)
+        for w in ws:
+            w.destroy()
+
+    # decode GEMVs at K = 4096 (weights from HBM: 32 x 8.8 MB / 12 x 23.6 MB exceed the cache)
+    one("w4_g128_q_proj", 4, 1, 4096, 4096, 128, 32)
+    one("w4_g128_gate_proj", 4, 1, 4096, 11008, 128, 12)
+    one("w4_g128_down_proj", 4, 1, 11008, 4096, 128, 12)
+    one("w4_g128_lm_head", 4, 1, 4096, 32000, 128, 5)
+    for M in (1, 4, 16):
+        one("w4_g64_2048x6144", 4, M, 2048, 6144, 64, 40)
+    for M in (1, 32):
+        one("w8_pc_11008x4096", 8, M, 4096, 11008, 0, 6)
+    # prefill
+    for M in (128, 1024, 2048):
+        one("w4_g128_prefill_4096x4096", 4, M, 4096, 4096, 128, 2)
+    one("w8_pc_prefill_11008x4096", 8, 512, 4096, 11008, 0, 2)
+    return out
+
+
+def bench_operator_boundary(pkg, S, steps=20):
+    """The same q_proj GEMV through the reference's operator interface (float32-expanded host tensors in and out,
+    like InferenceParameter): includes the host<->device copies and conversions, so it is NOT a roofline figure."""
+    K = N = 4096
+    cfg = S.w4a16(1, K, N, 128, seed=41)
+    x, w, s, z, _ = S.f32_valued_a16(cfg)
+    op = pkg.A16MatMul(K=K, N=N, weight_bits=4, q_group_size=128).init(w, s, z, None)
+    op.inference(x)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        op.inference(x)
+    sec = (time.perf_counter() - t0) / steps
+    op.deinit()
+    return {"case": "A16MatMul.inference, float32 host tensors, M=1 4096x4096", "us_per_call": round(sec * 1e6, 1),
+            "GBps_algorithmic": round(S.w4_gemv_bytes(1, K, N, 128) / sec / 1e9, 1)}
 
 
 def cpu_baseline_chain(S, M, cfgs, budget_s=20.0):
@@ -179,6 +263,8 @@ def main():
     ap.add_argument("--no-group", action="store_true",
                     help="one launch per matmul (7) instead of grouping q/k/v and gate/up (4 launches)")
     ap.add_argument("--int8-size", type=int, default=4096)
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the secondary figures (other M, single matmuls, prefill, cache-resident chain)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; every GPU box of this run has one. Use --gpus 1.")
@@ -232,6 +318,22 @@ def main():
     if not args.no_int8:
         line["int8_requant_gemm"] = bench_int8(pkg, S, torch, clib, args.int8_size, max(5, args.steps // 10),
                                                max(2, args.warmup // 10))
+    if not args.no_extras:
+        ex = {}
+        # the same chain with one weight copy (101 MB: resident in the 256 MB cache after the first pass)
+        r1 = bench_chain(pkg, S, torch, M, max(20, args.steps // 2), 5, 1, cfgs, grouped=not args.no_group)
+        ex["chain_cache_resident_GBps"] = round(r1["chain_bytes"] / (r1["gpu_s"] / max(20, args.steps // 2)) / 1e9, 1)
+        # one launch per matmul, for comparison with the grouped default
+        r7 = bench_chain(pkg, S, torch, M, max(20, args.steps // 2), 5, args.layers, cfgs, grouped=False)
+        ex["chain_7_launches_GBps"] = round(r7["chain_bytes"] / (r7["gpu_s"] / max(20, args.steps // 2)) / 1e9, 1)
+        for m in (8, 32):
+            cm = host_chain(S, m)
+            rm = bench_chain(pkg, S, torch, m, 40, 5, args.layers, cm, grouped=not args.no_group)
+            ex["chain_M%d_GBps" % m] = round(rm["chain_bytes"] / (rm["gpu_s"] / 40) / 1e9, 1)
+        ex["single_matmuls"] = bench_single_matmuls(pkg, S, torch)
+        ex["int8_256x1024x1024"] = bench_int8(pkg, S, torch, clib, 1024, 40, 5, M=256)
+        ex["operator_boundary"] = bench_operator_boundary(pkg, S)
+        line["extras"] = ex
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_chain(S, M, cfgs)
     print(json.dumps(line), flush=True)

@@ -17,12 +17,5 @@ def pkg(sub=None):
 
 
 def f32_valued_a16(cfg):
-    """Expand native-dtype synthetic operands to the interpreter's f32-valued convention
-    (every tensor a float array; packed bytes 0..255, bf16 values widened)."""
-    S = pkg("synth")
-    x = S.bf16_to_f32(cfg["x"])
-    w = cfg["weight"].astype(np.float32)
-    scale = S.bf16_to_f32(cfg["scale"])
-    zp = cfg["zp"].astype(np.float32)
-    bias = None if cfg.get("bias") is None else S.bf16_to_f32(cfg["bias"])
-    return x, w, scale, zp, bias
+    """Native-dtype synthetic operands expanded to the interpreter's f32-valued convention."""
+    return pkg("synth").f32_valued_a16(cfg)

@@ -25,6 +25,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "a16_common.cuh"
 #include "internal.h"
 
@@ -238,39 +240,23 @@ struct SkinnyArgs {
   int chip;
 };
 
-// Where a row block lives: its weight set (copied out of the argument block) and its index inside it.  Every
-// segment's fields are requested from the kernel-argument block up front and the right one is then SELECTED, instead
-// of indexing the table with the segment number: an indexed read could only be requested after the segment is
-// known, a second trip to memory in front of the first weight request.
+// Where a row block lives: its weight set and its index inside it.  The segment number comes from three scalar
+// compares against the segment starts (unused slots start at INT_MAX), without branches; the segment's fields are
+// then read from the kernel-argument block, which the scalar cache already holds.
 struct RowBlockRef {
   SkinnySeg sg;
   int rb;
   bool live;  // false: past the end of the grid (loads are clamped, nothing is stored)
 };
-template <class T>
-__device__ __forceinline__ T pick4(int s, T v0, T v1, T v2, T v3) {
-  return s == 3 ? v3 : (s == 2 ? v2 : (s == 1 ? v1 : v0));
-}
-__device__ __forceinline__ RowBlockRef locate_row_block(const SkinnyArgs &a, int rbg) {
+__device__ __forceinline__ RowBlockRef locate_row_block(const SkinnyArgs &a, int rbg, int row_blocks, int b1, int b2,
+                                                        int b3) {
   RowBlockRef r;
-  r.live = rbg < a.row_blocks;
-  const int c = r.live ? rbg : a.row_blocks - 1;
-  int s = 0;
-#pragma unroll
-  for (int q = 1; q < MAX_SEG; ++q)
-    if (q < a.n_seg && c >= a.seg[q].rb_begin)
-      s = q;
-#define MI_PICK(f) r.sg.f = pick4(s, a.seg[0].f, a.seg[1].f, a.seg[2].f, a.seg[3].f)
-  MI_PICK(qw);
-  MI_PICK(sz_t);
-  MI_PICK(scale_t);
-  MI_PICK(nzs_t);
-  MI_PICK(bias);
-  MI_PICK(y);
-  MI_PICK(y32);
-  MI_PICK(N);
-  MI_PICK(rb_begin);
-#undef MI_PICK
+  r.live = rbg < row_blocks;
+  const int c = r.live ? rbg : row_blocks - 1;
+  const int s = (c >= b1) + (c >= b2) + (c >= b3);
+  r.sg = a.seg[s];
+  asm volatile("" ::"s"(r.sg.qw), "s"(r.sg.sz_t), "s"(r.sg.scale_t), "s"(r.sg.nzs_t), "s"(r.sg.bias), "s"(r.sg.y),
+               "s"(r.sg.y32), "s"(r.sg.N), "s"(r.sg.rb_begin));  // one batch, as above
   r.rb = c - r.sg.rb_begin;
   return r;
 }
@@ -325,6 +311,24 @@ __device__ unsigned long long mi_dbg_buf[8 * 4096];
 template <int BITS, int DT, int GPT, int WAVES, int TPW, int R, bool XLDS>
 __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
   MI_STAMP(0);
+#ifdef MI_DBG_TIMING
+  {
+    int m_ = a.M;  // the first value read from the kernel-argument block
+    asm volatile("" ::"s"(m_));
+    MI_STAMP(7);
+  }
+#endif
+  // Every scalar the prologue needs leaves the kernel-argument block in ONE batch of scalar loads (the empty asm pins
+  // them all here): read one by one where they are used, each costs its own round trip to the scalar cache, and a
+  // dozen of those in a row would stand in front of the first weight request.
+  struct {
+    const uint16_t *x;
+    int64_t K;
+    int M, row_blocks, k_tiles, full_tiles, G, tiles_per_group, b1, b2, b3;
+  } h = {a.x, a.K, a.M, a.row_blocks, a.k_tiles, a.full_tiles, a.G, a.tiles_per_group,
+         a.seg[1].rb_begin, a.seg[2].rb_begin, a.seg[3].rb_begin};
+  asm volatile("" ::"s"(h.x), "s"(h.K), "s"(h.M), "s"(h.row_blocks), "s"(h.k_tiles), "s"(h.full_tiles), "s"(h.G),
+               "s"(h.tiles_per_group), "s"(h.b1), "s"(h.b2), "s"(h.b3));
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
   constexpr int TILE_K = BITS == 4 ? W4_TILE_K : W8_TILE_K;
@@ -336,39 +340,44 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps the tile loops scalar
   const int rb0 = blockIdx.x * R, m0 = blockIdx.y * 16;
   const int col = lane & 15, kq = lane >> 4;
-  const int rows = (a.M - m0) < 16 ? (a.M - m0) : 16;
+  const int rows = (h.M - m0) < 16 ? (h.M - m0) : 16;
   const int row_ld = col < rows ? col : rows - 1;  // rows past M re-read the last row; their outputs are never stored
-  const int kpad = a.k_tiles * TILE_K;
-  const int n_units = a.k_tiles * GPT;
+  const int kpad = h.k_tiles * TILE_K;
+  const int n_units = h.k_tiles * GPT;
   float *s_lds = reinterpret_cast<float *>(smem + skinny_red_bytes(WAVES, R));     // [n_units][16]
   uint8_t *xs = smem + skinny_red_bytes(WAVES, R) + (BITS == 4 ? (size_t)n_units * 64 : 0);
   const int xstride = kpad * 2 + 64;  // bytes; +64 puts consecutive rows 16 banks apart
 
-  const u32x4 *wq[R];
-  const uint32_t *szp[R];
-  const uint16_t *scp[R];
-  const float *nzp[R];
+  // Addresses are kept as a wave-uniform 64-bit base (scalar registers) plus a small per-lane byte offset, so that
+  // the loads below cost one vector instruction each and the address arithmetic stays on the scalar unit.
+  const uint8_t *wq[R];   // base of the row block's tiles; lane offset lane * 16
+  const uint8_t *szp[R];  // base of the row block's group words; lane offset col * 4 (4-bit) / col * 2, col * 4 (8-bit)
+  const uint8_t *scp[R];
+  const uint8_t *nzp[R];
   RowBlockRef ref[R];
   float bias_v[R];  // this lane's output channel; requested now so that it has arrived by the time of the store
+  const uint32_t lane16 = (uint32_t)lane * 16u, col4 = (uint32_t)col * 4u, col2 = (uint32_t)col * 2u;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    ref[r] = locate_row_block(a, rb0 + r);
+    ref[r] = locate_row_block(a, rb0 + r, h.row_blocks, h.b1, h.b2, h.b3);
     const SkinnySeg &sg = ref[r].sg;
     int rb = ref[r].rb;
 #ifdef MI_DBG_SAMETILE
     rb = rb & 3;
 #endif
-    wq[r] = sg.qw + (int64_t)rb * a.k_tiles * 64 + lane;
+    wq[r] = (const uint8_t *)sg.qw + (int64_t)rb * h.k_tiles * 1024;
     if constexpr (BITS == 4) {
-      szp[r] = sg.sz_t + (int64_t)rb * a.G * 16 + col;
+      szp[r] = (const uint8_t *)sg.sz_t + (int64_t)rb * h.G * 64;
     } else {
-      scp[r] = sg.scale_t + (int64_t)rb * a.G * 16 + col;
-      nzp[r] = sg.nzs_t + (int64_t)rb * a.G * 16 + col;
+      scp[r] = (const uint8_t *)sg.scale_t + (int64_t)rb * h.G * 32;
+      nzp[r] = (const uint8_t *)sg.nzs_t + (int64_t)rb * h.G * 64;
     }
     const int64_t n = (int64_t)rb * ROW_BLOCK + col;
-    bias_v[r] = (sg.bias && n < sg.N) ? sg.bias[n] : 0.0f;
+    bias_v[r] = 0.0f;
+    if (sg.bias)
+      bias_v[r] = sg.bias[n < sg.N ? n : sg.N - 1];
   }
-  const uint16_t *xrow = a.x + (int64_t)(m0 + row_ld) * a.K + kq * 8;
+  const uint16_t *xrow = h.x + (int64_t)(m0 + row_ld) * h.K + kq * 8;
 
   struct Tile {
     u32x4 w[R];
@@ -381,10 +390,10 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
     int gi;
     // tiles_per_group is 1 for the common group size == tile size; the division only runs for larger groups
     if constexpr (GPT == 1)
-      gi = a.tiles_per_group == 1 ? kt : kt / a.tiles_per_group;
+      gi = h.tiles_per_group == 1 ? kt : kt / h.tiles_per_group;
     else
       gi = kt * GPT + u;
-    return gi < a.G ? gi : a.G - 1;
+    return gi < h.G ? gi : h.G - 1;
   };
 
   auto load_tile = [&](Tile &t, int kt) {
@@ -393,17 +402,17 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
 #endif
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      t.w[r] = wq[r][(int64_t)kt * 64];
+      t.w[r] = *(const u32x4 *)(wq[r] + (int64_t)kt * 1024 + lane16);
 #pragma unroll
     for (int u = 0; u < GPT; ++u) {
       const int gi = unit_group(kt, u);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         if constexpr (BITS == 4) {
-          t.sz[r][u] = szp[r][gi * 16];
+          t.sz[r][u] = *(const uint32_t *)(szp[r] + gi * 64 + col4);
         } else {
-          t.sz[r][u] = scp[r][gi * 16];
-          t.nz[r][u] = nzp[r][gi * 16];
+          t.sz[r][u] = *(const uint16_t *)(scp[r] + gi * 32 + col2);
+          t.nz[r][u] = *(const float *)(nzp[r] + gi * 64 + col4);
         }
       }
     }
@@ -484,7 +493,7 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
 
   // tiles this wave owns: kt = wave + i * WAVES.  With the activations in LDS the (zero padded) partial last tile
   // is an ordinary tile; otherwise only full tiles are taken here and the tail is handled separately below.
-  const int n_tiles = XLDS ? a.k_tiles : a.full_tiles;
+  const int n_tiles = XLDS ? h.k_tiles : h.full_tiles;
   const int n_my = wave < n_tiles ? (n_tiles - wave + WAVES - 1) / WAVES : 0;
   const int last = n_tiles > 0 ? n_tiles - 1 : 0;
 
@@ -515,16 +524,18 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
     const int total = rows * chunks_per_row;
     // the load only requests the data; anything that needs the VALUE (zeroing the padding past K included) waits
     // until chunk_store, so that nothing stalls between this request and the weight requests that follow it
+    const uint8_t *xbase = (const uint8_t *)(h.x + (int64_t)m0 * h.K);  // wave-uniform; rows * K * 2 < 4 GiB
     auto chunk_load = [&](int c, int &row, int &kc, bool &ok) {
       ok = c < total;
       const int cc = ok ? c : 0;
       row = rows == 1 ? 0 : cc / chunks_per_row;
       kc = cc - row * chunks_per_row;
-      const bool in_k = kc * 8 < a.K;
-      return *(const u32x4 *)(a.x + (int64_t)(m0 + row) * a.K + (in_k ? kc * 8 : 0));  // always in bounds
+      const bool in_k = kc * 8 < h.K;
+      const uint32_t off = ((uint32_t)row * (uint32_t)h.K + (in_k ? (uint32_t)kc * 8u : 0u)) * 2u;  // always in bounds
+      return *(const u32x4 *)(xbase + off);
     };
     auto chunk_store = [&](u32x4 v, int row, int kc, bool ok) {
-      if (kc * 8 >= a.K)
+      if (kc * 8 >= h.K)
         v = u32x4{0, 0, 0, 0};
       if (ok)
         *(u32x4 *)(xs + row * xstride + kc * 16) = v;
@@ -540,18 +551,29 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
           s_lds[(kc / UNIT_CHUNKS) * 16 + row] = part;
       }
     };
-    u32x4 v[XB];
-    int row[XB], kc[XB];
-    bool ok[XB];
+    // The first batch holds exactly the chunk slots this shape needs (1, 2 or XB_MAX per thread): every slot costs
+    // address arithmetic in front of the weight requests, and at M = 1 one slot usually covers the whole row.  Each
+    // case is its own straight-line code (requests, weight requests, stores), so the load counts stay static.
+    auto first_batch = [&](auto xb_tag) {
+      constexpr int XBN = decltype(xb_tag)::value;
+      u32x4 v[XBN];
+      int row[XBN], kc[XBN];
+      bool ok[XBN];
 #pragma unroll
-    for (int b = 0; b < XB; ++b)  // unconditional (slots past the end re-read chunk 0): keeps the load count static
-      v[b] = chunk_load(b * NT + tid, row[b], kc[b], ok[b]);
-    issue_round(buf_a, 0);  // unconditional (k_tiles >= 1): a branch here would hide the load count from the waits below
-    MI_STAMP(1);
+      for (int b = 0; b < XBN; ++b)  // unconditional (a slot past the end re-reads chunk 0)
+        v[b] = chunk_load(b * NT + tid, row[b], kc[b], ok[b]);
+      issue_round(buf_a, 0);  // unconditional (k_tiles >= 1): a branch would hide the load count from the waits
+      MI_STAMP(1);
 #pragma unroll
-    for (int b = 0; b < XB; ++b)
-      if (b * NT < total)
+      for (int b = 0; b < XBN; ++b)
         chunk_store(v[b], row[b], kc[b], ok[b]);
+    };
+    if (total <= NT)
+      first_batch(std::integral_constant<int, 1>{});
+    else if (total <= 2 * NT || XB == 2)
+      first_batch(std::integral_constant<int, 2>{});
+    else
+      first_batch(std::integral_constant<int, XB>{});
     for (int c0 = XB * NT; c0 < total; c0 += NT) {  // large M * K only: these wait behind the weight loads
       int r1, k1;
       bool o1;
@@ -576,23 +598,23 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
   }
   MI_STAMP(3);
   if constexpr (!XLDS) {
-    if (a.full_tiles < a.k_tiles && wave == (a.full_tiles % WAVES)) {
+    if (h.full_tiles < h.k_tiles && wave == (h.full_tiles % WAVES)) {
       // partial last tile (K not a multiple of the tile): activations past K must read as zero
       Tile t;
-      const int kt = a.full_tiles;
+      const int kt = h.full_tiles;
 #pragma unroll
       for (int r = 0; r < R; ++r)
-        t.w[r] = wq[r][(int64_t)kt * 64];
+        t.w[r] = *(const u32x4 *)(wq[r] + (int64_t)kt * 1024 + lane16);
 #pragma unroll
       for (int u = 0; u < GPT; ++u) {
         const int gi = unit_group(kt, u);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           if constexpr (BITS == 4) {
-            t.sz[r][u] = szp[r][gi * 16];
+            t.sz[r][u] = *(const uint32_t *)(szp[r] + gi * 64 + col4);
           } else {
-            t.sz[r][u] = scp[r][gi * 16];
-            t.nz[r][u] = nzp[r][gi * 16];
+            t.sz[r][u] = *(const uint16_t *)(scp[r] + gi * 32 + col2);
+            t.nz[r][u] = *(const float *)(nzp[r] + gi * 64 + col4);
           }
         }
       }
@@ -600,7 +622,7 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
       for (int j = 0; j < KSTEPS; ++j) {
         const int64_t k0 = (int64_t)kt * TILE_K + 32 * j + kq * 8;
         u32x4 v = {0, 0, 0, 0};
-        if (k0 < a.K)
+        if (k0 < h.K)
           v = *(const u32x4 *)(xrow + (int64_t)kt * TILE_K + 32 * j);
         t.x[j] = v;
       }
@@ -768,7 +790,7 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
     sg.y = d_ys[q];
     sg.y32 = d_y32s ? d_y32s[q] : nullptr;
     sg.N = v->N;
-    sg.rb_begin = (int)total_rb;
+    sg.rb_begin = i < n ? (int)total_rb : INT32_MAX;  // unused slots are never selected
     if (i < n)
       total_rb += v->row_blocks;
   }

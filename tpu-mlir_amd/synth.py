@@ -89,6 +89,17 @@ def int8_matmul(M, K, N, seed=0, right_transpose=False, qdm=True):
             "right_transpose": right_transpose}
 
 
+def f32_valued_a16(cfg):
+    """Expands native-dtype operands to the interpreter's convention: every tensor a float32 array (packed weight
+    bytes as 0..255, bf16 values widened), as ModuleInterpreter hands them to A16MatMulOp::inference."""
+    x = bf16_to_f32(cfg["x"])
+    w = cfg["weight"].astype(np.float32)
+    scale = bf16_to_f32(cfg["scale"])
+    zp = cfg["zp"].astype(np.float32)
+    bias = None if cfg.get("bias") is None else bf16_to_f32(cfg["bias"])
+    return x, w, scale, zp, bias
+
+
 # Llama-7B decoder block projections, (name, K, N): hidden 4096, MLP 11008
 LLAMA7B_CHAIN = [("q_proj", 4096, 4096), ("k_proj", 4096, 4096), ("v_proj", 4096, 4096),
                  ("o_proj", 4096, 4096), ("gate_proj", 4096, 11008), ("up_proj", 4096, 11008),
