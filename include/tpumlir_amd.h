@@ -222,6 +222,26 @@ int mi_requant_int_inference(const mi_rq_attr *attr, mi_infer_param *p);
 int mi_requant_launch(const int32_t *d_in, void *d_out, int64_t outer, int64_t channels, int64_t inner,
                       int64_t input_zp, const mi_requant_desc *rq, void *stream);
 
+/* ============================================================================ */
+/* tpu.Cast  (lib/Dialect/Tpu/Interfaces/Common/Cast.cpp:35-200; requant()/dequant() of     */
+/* lib/Support/CastUtils.cpp:15-46).  BM168x branches; CV18xx and fp8 casts: MI_UNSUPPORTED. */
+/* ============================================================================ */
+enum { MI_ST_F32 = 0, MI_ST_BF16, MI_ST_F16, MI_ST_I8, MI_ST_U8, MI_ST_I16, MI_ST_U16, MI_ST_I32, MI_ST_U32 };
+typedef struct mi_cast_attr {
+  int64_t num_elem;           /* module::getNumElements(getOutput()) */
+  int in_type, out_type;      /* MI_ST_*: module::getStorageType() of input / output */
+  int in_quant, out_quant;    /* module::isUniformQuantized() of input / output */
+  double scale;               /* of the quantized side: qtype.getScale() */
+  int64_t zero_point;         /* qtype.getZeroPoint() */
+  int expressed;              /* MI_ST_F32 / BF16 / F16: qtype.getExpressedType() */
+  int round_mode;             /* round_mode_convert(getRoundMode()) */
+  int chip;
+} mi_cast_attr;
+/* inputs = {input}, float-expanded as everywhere in the interpreter; stateless (init/deinit are no-ops, :35-36) */
+int mi_cast_inference(const mi_cast_attr *attr, mi_infer_param *p);
+/* device level: d_in / d_out hold the NATIVE storage types (bf16/f16 bit patterns, int8 ...); asynchronous */
+int mi_cast_launch(const mi_cast_attr *attr, const void *d_in, void *d_out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -763,3 +763,66 @@ int orc_requant_int(const orc_rq_attr *a, const float *input, float *output) {
   }
   return 0;
 }
+
+/* ---------------------------------------------------------------------------
+ * tpu.Cast, lib/Dialect/Tpu/Interfaces/Common/Cast.cpp:38-200 (the branches a
+ * BM168x module reaches; CV18xx and fp8 are left out and return -1), with
+ * requant()/dequant() of lib/Support/CastUtils.cpp:15-46.
+ * ------------------------------------------------------------------------- */
+static int st_is_float(int t) { return t == ORC_ST_F32 || t == ORC_ST_BF16 || t == ORC_ST_F16; }
+
+/* requant(data, qtype), CastUtils.cpp:15-31: std::round is half away from zero;
+ * 1.0 / scale is formed in double and narrowed to float */
+static float cast_requant(float data, const orc_cast_attr *a) {
+  const float inv = (float)(1.0 / a->scale);
+  if (a->expressed == ORC_ST_F16)
+    return roundf(orc_F16(data * orc_F16(inv))) + (float)a->zero_point;
+  if (a->expressed == ORC_ST_BF16)
+    return roundf(orc_BF16(data * orc_BF16(inv, 0), 0)) + (float)a->zero_point;
+  return roundf(data * inv) + (float)a->zero_point;
+}
+
+static int st_bits(int t) {
+  switch (t) {
+  case ORC_ST_I8: case ORC_ST_U8: return 8;
+  case ORC_ST_I16: case ORC_ST_U16: return 16;
+  default: return 32;
+  }
+}
+static int st_unsigned(int t) { return t == ORC_ST_U8 || t == ORC_ST_U16 || t == ORC_ST_U32; }
+
+int orc_cast(const orc_cast_attr *a, const float *in, float *out, int64_t n) {
+  const int fin = st_is_float(a->in_type), fout = st_is_float(a->out_type);
+  if (a->in_type == ORC_ST_F32 && a->out_type == ORC_ST_F16) {          /* Cast.cpp:55-56 */
+    for (int64_t i = 0; i < n; ++i) out[i] = orc_F16(in[i]);
+  } else if (a->in_type == ORC_ST_F32 && a->out_type == ORC_ST_BF16) {  /* :57-58 */
+    for (int64_t i = 0; i < n; ++i) out[i] = orc_BF16(in[i], 0);
+  } else if (a->out_quant && fin) {                                     /* :77-95 */
+    for (int64_t i = 0; i < n; ++i) {
+      const float x = a->in_type == ORC_ST_BF16 ? orc_BF16(in[i], 0) : in[i];
+      const float v = cast_requant(x, a);
+      /* saturate<float>(v, type, mode), MathUtils.cpp:849-872: to_int then clamp to the integer type */
+      out[i] = (float)orc_saturate_i64(orc_to_int_f32(v, a->round_mode), st_bits(a->out_type),
+                                       st_unsigned(a->out_type));
+    }
+  } else if (a->in_quant && fout) {                                     /* :96-121 */
+    const float zp = (float)a->zero_point;
+    for (int64_t i = 0; i < n; ++i) {
+      if (a->out_type == ORC_ST_F16)
+        out[i] = orc_F16(orc_F16((float)a->scale) * orc_F16(in[i] - zp));
+      else if (a->out_type == ORC_ST_BF16)
+        out[i] = orc_BF16(orc_BF16((float)a->scale, 0) * orc_BF16(in[i] - zp, 0), 0);
+      else
+        out[i] = (float)a->scale * (in[i] - zp);
+    }
+  } else if (fin && (a->out_type == ORC_ST_I32 || a->out_type == ORC_ST_U32)) {  /* :145-151: no clamp */
+    for (int64_t i = 0; i < n; ++i) out[i] = (float)orc_to_int_f32(in[i], a->round_mode);
+  } else if (fin && !fout) {                                            /* :152-171 */
+    for (int64_t i = 0; i < n; ++i)
+      out[i] = (float)orc_saturate_i64(orc_to_int_f32(in[i], a->round_mode), st_bits(a->out_type),
+                                       st_unsigned(a->out_type));
+  } else {                                                              /* :172-174 */
+    memcpy(out, in, (size_t)n * sizeof(float));
+  }
+  return 0;
+}

@@ -23,6 +23,7 @@
  *                                special-case table for nan/inf/denormals
  *   orc_f32_to_bf16 (cvi)        add-0x7fff+lsb closed form, inf->0x7f7f
  *   orc_f32_to_f16               numpy float16 RNE incl. subnormals
+ *   orc_cast                     numpy closed forms per branch (tests/test_oracle_cast.py)
  *   orc_a16_dequant              one-hot activations recover nibble order,
  *                                group indexing and scale layout
  *   orc_sgemm_*                  float64 reference with the standard bound
@@ -192,6 +193,20 @@ typedef struct {
   int out_bits, out_unsigned;
 } orc_rq_attr;
 int orc_requant_int(const orc_rq_attr *attr, const float *input, float *output);
+
+/* ---- tpu.Cast (BM168x branches) ------------------------------------------ */
+/* storage types of the tensor on either side; every element is still handed over as a float (f32-valued) */
+enum { ORC_ST_F32 = 0, ORC_ST_BF16, ORC_ST_F16, ORC_ST_I8, ORC_ST_U8, ORC_ST_I16, ORC_ST_U16, ORC_ST_I32, ORC_ST_U32 };
+typedef struct {
+  int in_type, out_type;      /* ORC_ST_* */
+  int in_quant, out_quant;    /* the side is a uniform-quantised type */
+  double scale;               /* of the quantised side */
+  int64_t zero_point;
+  int expressed;              /* expressed type of the quantised side: ORC_ST_F32 / BF16 / F16 */
+  int round_mode;
+} orc_cast_attr;
+/* returns 0, or -1 for a branch this restatement leaves out (CV18xx, fp8) */
+int orc_cast(const orc_cast_attr *attr, const float *input, float *output, int64_t n);
 
 #ifdef __cplusplus
 }

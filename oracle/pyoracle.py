@@ -18,6 +18,7 @@ HALF_TO_ODD, HALF_TOWARDS_ZERO, TOWARDS_ZERO, AWAY_FROM_ZERO, UP, DOWN = 4, 5, 6
 RQ_TFLITE_LSHIFT, RQ_TFLITE, RQ_MULTIPLIER_SHIFT, RQ_ONLY_SHIFT, RQ_QDM, RQ_ONLY_SCALE = range(6)
 OUT_BF16, OUT_F16, OUT_F32 = 0, 1, 2
 GEMM_F32, GEMM_F64ACC, GEMM_FAST = 0, 1, 2
+ST_F32, ST_BF16, ST_F16, ST_I8, ST_U8, ST_I16, ST_U16, ST_I32, ST_U32 = range(9)
 
 
 def build(force=False):
@@ -64,6 +65,11 @@ class RqAttr(C.Structure):
                 ("is_cv18xx", C.c_int),
                 ("input_zp", C.c_int64), ("out_zp", C.c_int64),
                 ("out_bits", C.c_int), ("out_unsigned", C.c_int)]
+
+
+class CastAttr(C.Structure):
+    _fields_ = [("in_type", C.c_int), ("out_type", C.c_int), ("in_quant", C.c_int), ("out_quant", C.c_int),
+                ("scale", C.c_double), ("zero_point", C.c_int64), ("expressed", C.c_int), ("round_mode", C.c_int)]
 
 
 _lib = None
@@ -259,6 +265,19 @@ def requant_int(x, *, quant_mode, multiplier, rshift, round_mode=HALF_AWAY_FROM_
     rc = lib().orc_requant_int(C.byref(attr), _p(x, C.c_float), _p(out, C.c_float))
     if rc != 0:
         raise RuntimeError("orc_requant_int failed")
+    return out
+
+
+def cast(x, *, in_type, out_type, in_quant=False, out_quant=False, scale=1.0, zero_point=0, expressed=ST_F32,
+         round_mode=HALF_AWAY_FROM_ZERO):
+    """tpu.Cast on f32-valued data (BM168x branches)."""
+    x = _f32(x)
+    attr = CastAttr(in_type, out_type, int(in_quant), int(out_quant), float(scale), int(zero_point), expressed,
+                    round_mode)
+    out = np.empty_like(x)
+    rc = lib().orc_cast(C.byref(attr), _p(x, C.c_float), _p(out, C.c_float), C.c_int64(x.size))
+    if rc != 0:
+        raise RuntimeError("orc_cast: branch not restated")
     return out
 
 

@@ -1,0 +1,84 @@
+"""GPU parity of tpu.Cast against the CPU oracle, through the C ABI: bit-exact on every branch."""
+import numpy as np
+import pytest
+
+from helpers import pkg
+
+pytestmark = pytest.mark.gpu
+
+M_ = pkg()
+S = pkg("synth")
+clib = pkg("clib")
+
+
+def _values(seed, n=6000, spread=40.0):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal(n) * spread).astype(np.float32)
+    ties = rng.integers(-300, 300, size=300).astype(np.float32) + 0.5
+    return np.concatenate([x, ties, np.float32([0.0, -0.0, 127.49, 127.5, -128.5, -128.51, 3e4, -3e4])])
+
+
+CASES = [  # in, out, in_quant, out_quant, scale, zp, expressed
+    ("F32", "F16", False, False, 1.0, 0, "F32"), ("F32", "BF16", False, False, 1.0, 0, "F32"),
+    ("F32", "I8", False, True, 0.0371, 3, "F32"), ("F32", "U8", False, True, 0.11, 128, "F32"),
+    ("BF16", "I8", False, True, 0.17, -7, "BF16"), ("F16", "I8", False, True, 0.17, -7, "F16"),
+    ("F32", "I16", False, True, 0.002, 0, "F32"),
+    ("I8", "F32", True, False, 0.0123, 5, "F32"), ("I8", "BF16", True, False, 0.0123, 5, "BF16"),
+    ("U8", "F16", True, False, 0.031, 120, "F16"),
+    ("F32", "I32", False, False, 1.0, 0, "F32"), ("F32", "I8", False, False, 1.0, 0, "F32"),
+    ("F32", "U16", False, False, 1.0, 0, "F32"), ("F32", "F32", False, False, 1.0, 0, "F32"),
+]
+
+
+def _inputs(in_name, orc):
+    x = _values(hash(in_name) % 1000)
+    if in_name == "BF16":
+        return S.bf16_to_f32(S.bf16_round(x))
+    if in_name == "F16":
+        return orc.F16(x)
+    if in_name == "I8":
+        return np.clip(np.round(x), -128, 127).astype(np.float32)
+    if in_name == "U8":
+        return np.clip(np.round(x) + 128, 0, 255).astype(np.float32)
+    return x
+
+
+@pytest.mark.parametrize("rmode", ["HALF_AWAY_FROM_ZERO", "HALF_TO_EVEN", "DOWN", "HALF_UP", "TOWARDS_ZERO"])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "%s-%s%s" % (c[0], c[1], "q" if c[2] or c[3] else ""))
+def test_operator_level_against_oracle(orc, case, rmode):
+    i, o, iq, oq, scale, zp, ex = case
+    x = _inputs(i, orc)
+    kw = dict(in_type=getattr(clib, "ST_" + i), out_type=getattr(clib, "ST_" + o), in_quant=iq, out_quant=oq,
+              scale=scale, zero_point=zp, expressed=getattr(clib, "ST_" + ex))
+    got = M_.cast(x, round_mode=getattr(clib, "ROUND_" + rmode), **kw)
+    okw = dict(kw, in_type=getattr(orc, "ST_" + i), out_type=getattr(orc, "ST_" + o),
+               expressed=getattr(orc, "ST_" + ex))
+    want = orc.cast(x, round_mode=getattr(orc, rmode), **okw)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_device_level_native_storage(orc):
+    """bf16 activations -> int8 (quantize) -> bf16 (dequantize) on device tensors, in native storage."""
+    import torch
+    x = S.bf16_round(_values(9, n=100000, spread=3.0))
+    xd = torch.from_numpy(x.view(np.int16)).cuda().view(torch.bfloat16)
+    q = M_.cast_launch(xd, in_type=clib.ST_BF16, out_type=clib.ST_I8, out_quant=True, scale=0.05, zero_point=2,
+                       expressed=clib.ST_BF16)
+    y = M_.cast_launch(q, in_type=clib.ST_I8, out_type=clib.ST_BF16, in_quant=True, scale=0.05, zero_point=2,
+                       expressed=clib.ST_BF16)
+    torch.cuda.synchronize()
+    xf = S.bf16_to_f32(x)
+    want_q = orc.cast(xf, in_type=orc.ST_BF16, out_type=orc.ST_I8, out_quant=True, scale=0.05, zero_point=2,
+                      expressed=orc.ST_BF16)
+    assert np.array_equal(q.cpu().numpy().astype(np.float32), want_q)
+    want_y = orc.cast(want_q, in_type=orc.ST_I8, out_type=orc.ST_BF16, in_quant=True, scale=0.05, zero_point=2,
+                      expressed=orc.ST_BF16)
+    assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), orc.f32_to_bf16(want_y))
+
+
+def test_unsupported_branches_fail_loudly():
+    x = np.zeros(8, dtype=np.float32)
+    with pytest.raises(clib.BackendError):
+        M_.cast(x, in_type=clib.ST_F32, out_type=clib.ST_I8, out_quant=True, scale=0.1, chip=clib.CHIP_CV18XX)
+    with pytest.raises(clib.BackendError):
+        M_.cast(x, in_type=clib.ST_F32, out_type=clib.ST_I8, out_quant=True, scale=0.0)

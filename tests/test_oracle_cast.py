@@ -1,0 +1,89 @@
+"""Pins oracle.orc_cast (tpu.Cast, lib/Dialect/Tpu/Interfaces/Common/Cast.cpp:38-200) with independent numpy
+formulas per branch: library float16/bfloat16 rounding, half-away-from-zero via floor(|x| + 0.5), explicit clamps."""
+import numpy as np
+import pytest
+
+from helpers import pkg
+
+S = pkg("synth")
+
+
+def _half_away(x):
+    x = np.asarray(x, dtype=np.float32)
+    return (np.sign(x) * np.floor(np.abs(x).astype(np.float64) + 0.5)).astype(np.float32)
+
+
+def _bf16(x):
+    return S.bf16_to_f32(S.bf16_round(np.asarray(x, dtype=np.float32)))
+
+
+def _f16(x):
+    return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
+
+
+def _values(seed, n=4000, spread=40.0):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal(n) * spread).astype(np.float32)
+    ties = (rng.integers(-300, 300, size=200).astype(np.float32) + 0.5)  # exact .5 ties
+    return np.concatenate([x, ties, np.float32([0.0, -0.0, 127.49, 127.5, -128.5, -128.51, 1e9, -1e9])])
+
+
+def test_float_narrowing(orc):
+    x = _values(1, spread=3.0)
+    xs = x[np.abs(x) < 6e4]
+    assert np.array_equal(orc.cast(xs, in_type=orc.ST_F32, out_type=orc.ST_F16), _f16(xs))
+    assert np.array_equal(orc.cast(x, in_type=orc.ST_F32, out_type=orc.ST_BF16), _bf16(x))
+
+
+@pytest.mark.parametrize("out_type,lo,hi", [("ST_I8", -128, 127), ("ST_U8", 0, 255), ("ST_I16", -32768, 32767)])
+def test_quantize_expressed_f32(orc, out_type, lo, hi):
+    x = _values(2)
+    scale, zp = 0.0371, 3
+    inv = np.float32(1.0 / scale)
+    want = np.clip(_half_away(_half_away(x * inv) + np.float32(zp)), lo, hi)
+    got = orc.cast(x, in_type=orc.ST_F32, out_type=getattr(orc, out_type), out_quant=True, scale=scale, zero_point=zp)
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+def test_quantize_expressed_bf16_and_f16(orc):
+    x = _bf16(_values(3))
+    scale, zp = 0.125 * 1.37, -7
+    inv = np.float32(1.0 / scale)
+    want = np.clip(_half_away(_half_away(_bf16(x * _bf16(inv))) + np.float32(zp)), -128, 127)
+    got = orc.cast(x, in_type=orc.ST_BF16, out_type=orc.ST_I8, out_quant=True, scale=scale, zero_point=zp,
+                   expressed=orc.ST_BF16)
+    assert np.array_equal(got, want.astype(np.float32))
+    xh = _values(4, spread=10.0)
+    xh = _f16(xh[np.abs(xh) < 6e4])  # inside the half range
+    want = np.clip(_half_away(_half_away(_f16(xh * _f16(inv))) + np.float32(zp)), -128, 127)
+    got = orc.cast(xh, in_type=orc.ST_F16, out_type=orc.ST_I8, out_quant=True, scale=scale, zero_point=zp,
+                   expressed=orc.ST_F16)
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+def test_dequantize(orc):
+    q = np.arange(-128, 128, dtype=np.float32)
+    scale, zp = 0.0123, 5
+    d = q - np.float32(zp)
+    assert np.array_equal(orc.cast(q, in_type=orc.ST_I8, out_type=orc.ST_F32, in_quant=True, scale=scale, zero_point=zp),
+                          np.float32(scale) * d)
+    assert np.array_equal(orc.cast(q, in_type=orc.ST_I8, out_type=orc.ST_BF16, in_quant=True, scale=scale,
+                                   zero_point=zp, expressed=orc.ST_BF16), _bf16(_bf16(np.float32(scale)) * _bf16(d)))
+    assert np.array_equal(orc.cast(q, in_type=orc.ST_I8, out_type=orc.ST_F16, in_quant=True, scale=scale,
+                                   zero_point=zp, expressed=orc.ST_F16), _f16(_f16(np.float32(scale)) * _f16(d)))
+
+
+def test_float_to_plain_integers_and_rounding_modes(orc):
+    x = _values(5)
+    assert np.array_equal(orc.cast(x, in_type=orc.ST_F32, out_type=orc.ST_I8), np.clip(_half_away(x), -128, 127))
+    assert np.array_equal(orc.cast(x, in_type=orc.ST_F32, out_type=orc.ST_U16), np.clip(_half_away(x), 0, 65535))
+    # int32: rounded, not clamped (Cast.cpp:145-151)
+    small = x[np.abs(x) < 1e6]
+    assert np.array_equal(orc.cast(small, in_type=orc.ST_F32, out_type=orc.ST_I32), _half_away(small))
+    assert np.array_equal(orc.cast(small, in_type=orc.ST_F32, out_type=orc.ST_I32, round_mode=orc.DOWN), np.floor(small))
+    assert np.array_equal(orc.cast(small, in_type=orc.ST_F32, out_type=orc.ST_I32, round_mode=orc.TOWARDS_ZERO),
+                          np.trunc(small))
+    even = np.round(small.astype(np.float64)).astype(np.float32)  # numpy rounds half to even
+    assert np.array_equal(orc.cast(small, in_type=orc.ST_F32, out_type=orc.ST_I32, round_mode=orc.HALF_TO_EVEN), even)
+    # anything else is a copy (:172-174)
+    assert np.array_equal(orc.cast(x, in_type=orc.ST_F32, out_type=orc.ST_F32), x)

@@ -11,6 +11,7 @@ ROUND_TOWARDS_ZERO, ROUND_UP, ROUND_DOWN = 6, 8, 9
 RQ_TFLITE_LSHIFT, RQ_TFLITE, RQ_MULTIPLIER_SHIFT, RQ_ONLY_SHIFT, RQ_QDM = 0, 1, 2, 3, 4
 DT_BF16, DT_F16, DT_I8, DT_U8, DT_I16, DT_U16, DT_I32 = range(7)
 CHIP_BM168X, CHIP_CV18XX = 0, 1
+ST_F32, ST_BF16, ST_F16, ST_I8, ST_U8, ST_I16, ST_U16, ST_I32, ST_U32 = range(9)
 
 # every symbol include/tpumlir_amd.h declares
 EXPORTS = [
@@ -20,6 +21,7 @@ EXPORTS = [
     "mi_a16mm_launch_group",
     "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
     "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
+    "mi_cast_inference", "mi_cast_launch",
 ]
 
 
@@ -74,6 +76,12 @@ class RqAttr(C.Structure):
                 ("out_zp", C.c_int64), ("out_dtype", C.c_int)]
 
 
+class CastAttr(C.Structure):
+    _fields_ = [("num_elem", C.c_int64), ("in_type", C.c_int), ("out_type", C.c_int), ("in_quant", C.c_int),
+                ("out_quant", C.c_int), ("scale", C.c_double), ("zero_point", C.c_int64), ("expressed", C.c_int),
+                ("round_mode", C.c_int), ("chip", C.c_int)]
+
+
 _lib = None
 
 
@@ -107,6 +115,8 @@ def lib():
         L.mi_a16mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_launch_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int64,
                                             C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_void_p]
+        L.mi_cast_inference.argtypes = [C.POINTER(CastAttr), C.POINTER(InferParam)]
+        L.mi_cast_launch.argtypes = [C.POINTER(CastAttr), C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_init.argtypes = [C.POINTER(A16Attr), C.POINTER(InferParam)]
         L.mi_a16mm_inference.argtypes = [C.POINTER(A16Attr), C.POINTER(InferParam)]
         L.mi_a16mm_deinit.argtypes = [C.POINTER(InferParam)]

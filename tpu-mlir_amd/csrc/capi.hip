@@ -708,4 +708,75 @@ int mi_requant_int_inference(const mi_rq_attr *a, mi_infer_param *p) {
                           nullptr, nullptr, nullptr);
 }
 
+// ---------------------------------------------------------------------------------------------
+// tpu.Cast
+// ---------------------------------------------------------------------------------------------
+static bool st_float(int t) { return t == MI_ST_F32 || t == MI_ST_BF16 || t == MI_ST_F16; }
+
+// the scalars the reference forms once per call: (float)(1.0 / scale) narrowed to the expressed type
+// (CastUtils.cpp:18-27) and the scale narrowed to the output type of a dequantizing cast (Cast.cpp:107-117)
+static int cast_scalars(const mi_cast_attr *a, float *inv_scale, float *scale) {
+  MI_REQUIRE(a, MI_BAD_ARGUMENT, "mi_cast: null attribute");
+  MI_REQUIRE(a->in_type >= MI_ST_F32 && a->in_type <= MI_ST_U32 && a->out_type >= MI_ST_F32 &&
+                 a->out_type <= MI_ST_U32,
+             MI_UNSUPPORTED, "mi_cast: storage type not handled (fp8 casts run on the CPU path)");
+  MI_REQUIRE(a->chip == MI_CHIP_BM168X, MI_UNSUPPORTED, "mi_cast: the CV18xx bf16 table arithmetic is not built");
+  MI_REQUIRE(a->num_elem >= 0, MI_BAD_ARGUMENT, "mi_cast: negative element count");
+  *inv_scale = 1.0f;
+  *scale = (float)a->scale;
+  const bool quantizing = a->out_quant && st_float(a->in_type);
+  const bool dequantizing = !quantizing && a->in_quant && st_float(a->out_type);
+  if (quantizing || dequantizing)
+    MI_REQUIRE(a->scale != 0.0 && a->scale == a->scale, MI_BAD_ARGUMENT, "mi_cast: scale must be a nonzero number");
+  if (quantizing) {
+    MI_REQUIRE(a->expressed == MI_ST_F32 || a->expressed == MI_ST_BF16 || a->expressed == MI_ST_F16,
+               MI_UNSUPPORTED, "mi_cast: expressed type not handled");
+    float inv = (float)(1.0 / a->scale);
+    if (a->expressed == MI_ST_F16)
+      inv = h_f16_to_f32(h_f32_to_f16(inv));
+    else if (a->expressed == MI_ST_BF16)
+      inv = h_bf16_to_f32(h_f32_to_bf16(inv));
+    *inv_scale = inv;
+  }
+  if (dequantizing) {
+    if (a->out_type == MI_ST_F16)
+      *scale = h_f16_to_f32(h_f32_to_f16((float)a->scale));
+    else if (a->out_type == MI_ST_BF16)
+      *scale = h_bf16_to_f32(h_f32_to_bf16((float)a->scale));
+  }
+  return MI_SUCCESS;
+}
+
+int mi_cast_launch(const mi_cast_attr *a, const void *d_in, void *d_out, void *stream) {
+  float inv, sc;
+  int rc = cast_scalars(a, &inv, &sc);
+  if (rc)
+    return rc;
+  MI_REQUIRE(a->num_elem == 0 || (d_in && d_out), MI_BAD_ARGUMENT, "mi_cast_launch: null operand");
+  return cast_launch(a, d_in, d_out, a->num_elem, inv, sc, false, (hipStream_t)stream);
+}
+
+int mi_cast_inference(const mi_cast_attr *a, mi_infer_param *p) {
+  MI_REQUIRE(a && p && p->inputs && p->n_inputs >= 1 && p->inputs[0] && p->outputs && p->n_outputs >= 1 &&
+                 p->outputs[0],
+             MI_BAD_ARGUMENT, "mi_cast_inference: null argument");
+  float inv, sc;
+  int rc = cast_scalars(a, &inv, &sc);
+  if (rc)
+    return rc;
+  MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_cast_inference: no GPU visible");
+  const int64_t n = a->num_elem;
+  // the interpreter's tensors are float arrays whatever the storage type: both sides travel as f32 here and the
+  // kernel applies the op's arithmetic between them
+  DevBuf d_in, d_out;
+  if ((rc = d_in.reserve((size_t)n * 4 + 4)) || (rc = d_out.reserve((size_t)n * 4 + 4)))
+    return rc;
+  MI_HIP(hipMemcpy(d_in.ptr, p->inputs[0], (size_t)n * 4, hipMemcpyHostToDevice));
+  rc = cast_launch(a, d_in.ptr, d_out.ptr, n, inv, sc, true, nullptr);
+  if (rc)
+    return rc;
+  MI_HIP(hipMemcpy(p->outputs[0], d_out.ptr, (size_t)n * 4, hipMemcpyDeviceToHost));
+  return MI_SUCCESS;
+}
+
 }  // extern "C"

@@ -108,32 +108,42 @@ __device__ __forceinline__ int32_t multiply_by_quantized_multiplier(int32_t x, i
   return (int32_t)value;
 }
 
+// float/double -> int64 as the reference's host does it: the x86-64 conversion instruction returns INT64_MIN for NaN
+// and for anything outside the int64 range (the GPU's own conversion saturates and maps NaN to 0), and the clamp that
+// follows in the reference then turns that into the type's minimum.
+__device__ __forceinline__ int64_t cvt_i64_host(float v) {
+  return (fabsf(v) < 9.2233720368547758e18f) ? (int64_t)v : INT64_MIN;
+}
+__device__ __forceinline__ int64_t cvt_i64_host(double v) {
+  return (fabs(v) < 9.2233720368547758e18) ? (int64_t)v : INT64_MIN;
+}
+
 // to_int<float> (lib/Support/MathUtils.cpp:179-213)
 __device__ __forceinline__ int64_t to_int_f32(float v, int mode) {
   switch (mode) {
   case MI_ROUND_HALF_AWAY_FROM_ZERO:
-    return (int64_t)roundf(v);
+    return cvt_i64_host(roundf(v));
   case MI_ROUND_UP:
-    return (int64_t)ceilf(v);
+    return cvt_i64_host(ceilf(v));
   case MI_ROUND_DOWN:
-    return (int64_t)floorf(v);
+    return cvt_i64_host(floorf(v));
   case MI_ROUND_HALF_UP:
-    return (int64_t)floor((double)v + 0.5);
+    return cvt_i64_host(floor((double)v + 0.5));
   case MI_ROUND_HALF_DOWN:
-    return (int64_t)ceil((double)v - 0.5);
+    return cvt_i64_host(ceil((double)v - 0.5));
   case MI_ROUND_TOWARDS_ZERO:
-    return (int64_t)v;
+    return cvt_i64_host(v);
   case MI_ROUND_HALF_TO_EVEN: {
     float a = fabsf(v);
     float ip = truncf(a);
     float fr = a - ip;
-    int64_t r = (int64_t)ip;
+    int64_t r = cvt_i64_host(ip);
     if (fr > 0.5f || (fr == 0.5f && (r & 1)))
       r += 1;
     return v < 0 ? -r : r;
   }
   default:
-    return (int64_t)roundf(v);
+    return cvt_i64_host(roundf(v));
   }
 }
 

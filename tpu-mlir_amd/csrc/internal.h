@@ -71,6 +71,9 @@ int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
 int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
                      float *const *d_y32s, hipStream_t stream);
 
+int cast_launch(const mi_cast_attr *c, const void *d_in, void *d_out, int64_t n, float inv_scale, float scale,
+                bool f32_io, hipStream_t stream);
+
 struct RequantParams;
 int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned, int right_transpose,
                 const int32_t *d_bias, int64_t M, int64_t K, int64_t N, int64_t input_zp, int64_t right_zp,

@@ -159,6 +159,18 @@ def requant_int(x, *, quant_mode, multiplier, rshift, round_mode=ROUND_HALF_AWAY
     return y
 
 
+def cast(x, *, in_type, out_type, in_quant=False, out_quant=False, scale=1.0, zero_point=0, expressed=None,
+         round_mode=ROUND_HALF_AWAY_FROM_ZERO, chip=CHIP_BM168X):
+    """tpu.Cast.inference on an f32-valued operand (storage types are clib.ST_*)."""
+    x = _f32(x)
+    attr = clib.CastAttr(x.size, in_type, out_type, int(in_quant), int(out_quant), float(scale), int(zero_point),
+                         clib.ST_F32 if expressed is None else expressed, round_mode, chip)
+    y = np.empty_like(x)
+    p = _Param([x], [y])
+    check(clib.lib().mi_cast_inference(C.byref(attr), C.byref(p.c)))
+    return y
+
+
 # --------------------------------------------------------------------------------------------------
 # device level
 # --------------------------------------------------------------------------------------------------
@@ -255,6 +267,28 @@ def a16mm_launch_group(ws, x, ys=None, ys_f32=None, stream=None):
         fp = Arr(*[None if f is None else f.data_ptr() for f in ys_f32])
     check(clib.lib().mi_a16mm_launch_group(wh, n, _dptr(x), M, yp, fp, _stream_ptr(stream)))
     return ys
+
+
+_ST_TORCH = {clib.ST_F32: "float32", clib.ST_BF16: "bfloat16", clib.ST_F16: "float16", clib.ST_I8: "int8",
+             clib.ST_U8: "uint8", clib.ST_I16: "int16", clib.ST_U16: "int16", clib.ST_I32: "int32", clib.ST_U32: "int32"}
+
+
+def cast_launch(x, *, in_type, out_type, in_quant=False, out_quant=False, scale=1.0, zero_point=0, expressed=None,
+                round_mode=ROUND_HALF_AWAY_FROM_ZERO, out=None, stream=None):
+    """tpu.Cast between NATIVE storage types on device tensors (uint16 / uint32 bit patterns travel in
+    int16 / int32 tensors)."""
+    import torch
+    if not (x.is_cuda and x.is_contiguous() and x.dtype == getattr(torch, _ST_TORCH[in_type])):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "cast_launch: input tensor does not match in_type")
+    if out is None:
+        out = torch.empty(x.shape, dtype=getattr(torch, _ST_TORCH[out_type]), device=x.device)
+    if not (out.is_cuda and out.is_contiguous() and out.numel() == x.numel()
+            and out.dtype == getattr(torch, _ST_TORCH[out_type])):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "cast_launch: output tensor does not match out_type")
+    attr = clib.CastAttr(x.numel(), in_type, out_type, int(in_quant), int(out_quant), float(scale), int(zero_point),
+                         clib.ST_F32 if expressed is None else expressed, round_mode, CHIP_BM168X)
+    check(clib.lib().mi_cast_launch(C.byref(attr), _dptr(x), _dptr(out), _stream_ptr(stream)))
+    return out
 
 
 class RequantDesc:
