@@ -242,6 +242,46 @@ int mi_cast_inference(const mi_cast_attr *attr, mi_infer_param *p);
 /* device level: d_in / d_out hold the NATIVE storage types (bf16/f16 bit patterns, int8 ...); asynchronous */
 int mi_cast_launch(const mi_cast_attr *attr, const void *d_in, void *d_out, void *stream);
 
+/* ============================================================================ */
+/* Device-resident mini-interpreter: the ops above run back to back on one stream, activations stay in HBM in  */
+/* their native storage types.  Counterpart of the reference's GPU interpreter class py_cuda                  */
+/* (bindings/pymlir/pycuda.cpp: gpu_load :17-49, set_tensor :399-436, gpu_invoke :438-669,                     */
+/* cuda_to_host / get_tensor :289-397,954-966), with tensors and ops added by the caller instead of parsed     */
+/* from MLIR.                                                                                                 */
+/* ============================================================================ */
+typedef struct mi_module mi_module;
+int mi_module_create(mi_module **out);
+void mi_module_destroy(mi_module *m);
+/* an activation (input, intermediate or output): allocated once in HBM (py_cuda::cuda_malloc :271-278) */
+int mi_module_add_tensor(mi_module *m, const char *name, int storage_type /* MI_ST_* */, int64_t num_elem);
+/* tpu.A16MatMul: host arrays as for mi_a16_weight_create; M = numel(input) / K.  Consecutive A16MatMuls that
+ * read the same tensor with compatible weight sets are issued as one grouped launch. */
+int mi_module_add_a16matmul(mi_module *m, const char *input, const char *output, const mi_a16_weight_desc *desc,
+                            const void *weight, const uint16_t *scale, const uint8_t *zp, const float *bias);
+typedef struct mi_module_i8_desc {
+  int64_t K, N;
+  const void *right;        /* HOST int8/uint8 weight, [K,N] or (right_transpose) [N,K] */
+  int right_transpose, right_unsigned;
+  const int32_t *bias;      /* HOST [N] or NULL */
+  int64_t input_zp, right_zp;
+  int do_relu;
+  int64_t relu_limit;
+  int has_requant;          /* 0: int32 output */
+  mi_requant_desc rq;       /* its d_* per-channel arrays are HOST pointers here (copied to the device) */
+} mi_module_i8_desc;
+/* quantized tpu.MatMul (+ fused requant): input int8/uint8 [M,K] */
+int mi_module_add_matmul_int8(mi_module *m, const char *input, const char *output, const mi_module_i8_desc *desc);
+/* tpu.Cast between two tensors of the module */
+int mi_module_add_cast(mi_module *m, const char *input, const char *output, const mi_cast_attr *attr);
+/* float data in (converted on the device to the tensor's storage), as py_cuda::set_tensor */
+int mi_module_set_tensor(mi_module *m, const char *name, const float *data, int64_t num_elem);
+/* runs every op in the order added and waits for the stream; from the second call on the launches are replayed
+ * from a HIP graph when every op is a plain kernel launch */
+int mi_module_invoke(mi_module *m);
+int mi_module_uses_graph(const mi_module *m);
+/* float data out (expanded on the device), as py_cuda::get_tensor */
+int mi_module_get_tensor(mi_module *m, const char *name, float *out, int64_t num_elem);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,110 @@
+"""The device-resident op list (mi_module_*) against the CPU oracle run op by op: float32 arrays in through
+set_tensor, every op on the GPU with activations in native storage, float32 arrays out through get_tensor."""
+import numpy as np
+import pytest
+
+from helpers import pkg, f32_valued_a16
+
+pytestmark = pytest.mark.gpu
+
+M_ = pkg()
+S = pkg("synth")
+clib = pkg("clib")
+cmp = pkg("compare")
+
+
+def test_w4a16_block_with_grouped_siblings(orc):
+    """f32 input -> Cast to bf16 -> q/k/v projections (siblings: one grouped launch) -> o projection on q."""
+    M, K = 3, 512
+    cq = S.w4a16(M, K, 256, 128, seed=301, bias=True)
+    ck = S.w4a16(M, K, 64, 128, seed=302)
+    cv = S.w4a16(M, K, 64, 128, seed=303)
+    co = S.w4a16(M, 256, 512, 128, seed=304)
+    x32 = (np.random.default_rng(1).standard_normal((M, K)) * 0.7).astype(np.float32)
+
+    m = M_.Module()
+    m.add_tensor("x", clib.ST_F32, (M, K)).add_tensor("xb", clib.ST_BF16, (M, K))
+    m.add_tensor("q", clib.ST_BF16, (M, 256)).add_tensor("k", clib.ST_BF16, (M, 64)).add_tensor("v", clib.ST_BF16, (M, 64))
+    m.add_tensor("o", clib.ST_BF16, (M, 512))
+    m.add_cast("x", "xb", in_type=clib.ST_F32, out_type=clib.ST_BF16)
+    for name, c in (("q", cq), ("k", ck), ("v", cv)):
+        m.add_a16matmul("xb", name, c["weight"], c["scale"], c["zp"],
+                        None if c["bias"] is None else S.bf16_to_f32(c["bias"]), K=K, N=c["N"], weight_bits=4,
+                        q_group_size=128)
+    m.add_a16matmul("q", "o", co["weight"], co["scale"], co["zp"], None, K=256, N=512, weight_bits=4, q_group_size=128)
+
+    def reference(x):
+        xb = orc.cast(x, in_type=orc.ST_F32, out_type=orc.ST_BF16)
+        outs = {}
+        for name, c in (("q", cq), ("k", ck), ("v", cv)):
+            _, w, s, z, b = f32_valued_a16(c)
+            outs[name], _ = orc.a16matmul(xb, w, s, z, b, M=M, K=K, N=c["N"], weight_bits=4, q_group_size=128,
+                                          gemm_kind=orc.GEMM_F64ACC)
+        return xb, outs
+
+    for rep in range(3):  # the first call runs eagerly, the later ones replay the captured graph
+        x = x32 * (1.0 + rep)
+        m.set_tensor("x", x)
+        m.invoke()
+        xb, outs = reference(x)
+        assert np.array_equal(m.get_tensor("xb"), xb)
+        got = {n: m.get_tensor(n) for n in ("q", "k", "v", "o")}
+        for n in ("q", "k", "v"):
+            rms = float(np.sqrt(np.mean(outs[n].astype(np.float64) ** 2)))
+            assert np.max(np.abs(got[n] - outs[n])) <= 2.0 ** -7 * np.max(np.abs(outs[n])) + 1e-6, n
+            assert cmp.max_abs_over_rms(got[n], outs[n]) <= 1e-2, n  # the north-star bound on bf16 outputs
+            assert rms > 0
+        # o is computed from the DEVICE's q (bf16 values): feed exactly those to the oracle
+        _, w, s, z, b = f32_valued_a16(co)
+        want_o, _ = orc.a16matmul(got["q"], w, s, z, None, M=M, K=256, N=512, weight_bits=4, q_group_size=128,
+                                  gemm_kind=orc.GEMM_F64ACC)
+        assert cmp.max_abs_over_rms(got["o"], want_o) <= 1e-2
+        assert np.mean(got["o"] != want_o) < 0.01  # at most a last-place difference on a few elements
+    assert m.uses_graph()
+    m.destroy()
+
+
+def test_int8_pipeline_bit_exact(orc):
+    """f32 activations -> quantize (Cast) -> INT8 MatMul with per-channel Q31 requant -> dequantize (Cast)."""
+    M, K, N = 20, 256, 96
+    c = S.int8_matmul(M, K, N, seed=311, qdm=True)
+    x = (np.random.default_rng(2).standard_normal((M, K)) * 1.5).astype(np.float32)
+    in_scale, in_zp, out_scale, out_zp = 0.021, 0, 0.37, 4
+    m = M_.Module()
+    m.add_tensor("x", clib.ST_F32, (M, K)).add_tensor("xq", clib.ST_I8, (M, K))
+    m.add_tensor("yq", clib.ST_I8, (M, N)).add_tensor("y", clib.ST_F32, (M, N))
+    m.add_cast("x", "xq", in_type=clib.ST_F32, out_type=clib.ST_I8, out_quant=True, scale=in_scale, zero_point=in_zp)
+    zps = np.full(N, out_zp, dtype=np.int32)
+    m.add_matmul_int8("xq", "yq", c["b"], c["bias"], K=K, N=N, quant_mode=clib.RQ_QDM, multiplier=c["mult"],
+                      shift=c["shift"], zp=zps)
+    m.add_cast("yq", "y", in_type=clib.ST_I8, out_type=clib.ST_F32, in_quant=True, scale=out_scale, zero_point=out_zp)
+    for rep in range(2):
+        xr = x * (1 + 0.5 * rep)
+        m.set_tensor("x", xr)
+        m.invoke()
+        xq = orc.cast(xr, in_type=orc.ST_F32, out_type=orc.ST_I8, out_quant=True, scale=in_scale, zero_point=in_zp)
+        assert np.array_equal(m.get_tensor("xq"), xq)
+        acc = xq.astype(np.int64) @ c["b"].astype(np.int64) + c["bias"].astype(np.int64)
+        v = orc.mbqm(acc, np.broadcast_to(c["mult"].astype(np.int64), acc.shape),
+                     np.broadcast_to(-c["shift"].astype(np.int64), acc.shape), orc.HALF_AWAY_FROM_ZERO)
+        yq = np.clip(v.astype(np.int64) + out_zp, -128, 127).astype(np.float32)
+        assert np.array_equal(m.get_tensor("yq"), yq)
+        y = orc.cast(yq, in_type=orc.ST_I8, out_type=orc.ST_F32, in_quant=True, scale=out_scale, zero_point=out_zp)
+        assert np.array_equal(m.get_tensor("y"), y)
+    assert m.uses_graph()
+    m.destroy()
+
+
+def test_argument_errors():
+    m = M_.Module()
+    m.add_tensor("a", clib.ST_BF16, (2, 128))
+    with pytest.raises(clib.BackendError):
+        m.add_tensor("a", clib.ST_BF16, (2, 128))  # duplicate name
+    with pytest.raises(clib.BackendError):
+        m.add_cast("a", "missing", in_type=clib.ST_BF16, out_type=clib.ST_F32)
+    m.add_tensor("b", clib.ST_F32, (2, 64))
+    with pytest.raises(clib.BackendError):
+        m.add_cast("a", "b", in_type=clib.ST_BF16, out_type=clib.ST_F32)  # sizes differ
+    with pytest.raises(clib.BackendError):
+        m.set_tensor("a", np.zeros(5, dtype=np.float32))
+    m.destroy()

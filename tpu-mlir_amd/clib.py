@@ -22,6 +22,9 @@ EXPORTS = [
     "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
     "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
     "mi_cast_inference", "mi_cast_launch",
+    "mi_module_create", "mi_module_destroy", "mi_module_add_tensor", "mi_module_add_a16matmul",
+    "mi_module_add_matmul_int8", "mi_module_add_cast", "mi_module_set_tensor", "mi_module_invoke",
+    "mi_module_uses_graph", "mi_module_get_tensor",
 ]
 
 
@@ -76,6 +79,12 @@ class RqAttr(C.Structure):
                 ("out_zp", C.c_int64), ("out_dtype", C.c_int)]
 
 
+class ModuleI8Desc(C.Structure):
+    _fields_ = [("K", C.c_int64), ("N", C.c_int64), ("right", C.c_void_p), ("right_transpose", C.c_int),
+                ("right_unsigned", C.c_int), ("bias", C.c_void_p), ("input_zp", C.c_int64), ("right_zp", C.c_int64),
+                ("do_relu", C.c_int), ("relu_limit", C.c_int64), ("has_requant", C.c_int), ("rq", RequantDescC)]
+
+
 class CastAttr(C.Structure):
     _fields_ = [("num_elem", C.c_int64), ("in_type", C.c_int), ("out_type", C.c_int), ("in_quant", C.c_int),
                 ("out_quant", C.c_int), ("scale", C.c_double), ("zero_point", C.c_int64), ("expressed", C.c_int),
@@ -115,6 +124,18 @@ def lib():
         L.mi_a16mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_launch_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int64,
                                             C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_void_p]
+        L.mi_module_create.argtypes = [C.POINTER(C.c_void_p)]
+        L.mi_module_destroy.argtypes = [C.c_void_p]
+        L.mi_module_destroy.restype = None
+        L.mi_module_add_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_int64]
+        L.mi_module_add_a16matmul.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(A16WeightDesc), C.c_void_p,
+                                              C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi_module_add_matmul_int8.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(ModuleI8Desc)]
+        L.mi_module_add_cast.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(CastAttr)]
+        L.mi_module_set_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int64]
+        L.mi_module_invoke.argtypes = [C.c_void_p]
+        L.mi_module_uses_graph.argtypes = [C.c_void_p]
+        L.mi_module_get_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int64]
         L.mi_cast_inference.argtypes = [C.POINTER(CastAttr), C.POINTER(InferParam)]
         L.mi_cast_launch.argtypes = [C.POINTER(CastAttr), C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_init.argtypes = [C.POINTER(A16Attr), C.POINTER(InferParam)]

@@ -715,7 +715,9 @@ static bool st_float(int t) { return t == MI_ST_F32 || t == MI_ST_BF16 || t == M
 
 // the scalars the reference forms once per call: (float)(1.0 / scale) narrowed to the expressed type
 // (CastUtils.cpp:18-27) and the scale narrowed to the output type of a dequantizing cast (Cast.cpp:107-117)
-static int cast_scalars(const mi_cast_attr *a, float *inv_scale, float *scale) {
+}  // extern "C"
+namespace mi {
+int cast_scalars(const mi_cast_attr *a, float *inv_scale, float *scale) {
   MI_REQUIRE(a, MI_BAD_ARGUMENT, "mi_cast: null attribute");
   MI_REQUIRE(a->in_type >= MI_ST_F32 && a->in_type <= MI_ST_U32 && a->out_type >= MI_ST_F32 &&
                  a->out_type <= MI_ST_U32,
@@ -746,6 +748,8 @@ static int cast_scalars(const mi_cast_attr *a, float *inv_scale, float *scale) {
   }
   return MI_SUCCESS;
 }
+}  // namespace mi
+extern "C" {
 
 int mi_cast_launch(const mi_cast_attr *a, const void *d_in, void *d_out, void *stream) {
   float inv, sc;

@@ -74,6 +74,9 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
 int cast_launch(const mi_cast_attr *c, const void *d_in, void *d_out, int64_t n, float inv_scale, float scale,
                 bool f32_io, hipStream_t stream);
 
+// validates a cast attribute and forms the scalars the reference computes once per call
+int cast_scalars(const mi_cast_attr *a, float *inv_scale, float *scale);
+
 struct RequantParams;
 int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned, int right_transpose,
                 const int32_t *d_bias, int64_t M, int64_t K, int64_t N, int64_t input_zp, int64_t right_zp,

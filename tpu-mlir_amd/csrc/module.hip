@@ -1,0 +1,425 @@
+// Device-resident mini-interpreter: a list of the ops this library implements, run back to back on one stream with
+// every activation staying in HBM in its native storage type.  It is the shape of the reference's GPU interpreter
+// (bindings/pymlir/pycuda.cpp: gpu_load :17-49 uploads native-dtype weights once, set_tensor :399-436 converts the
+// float input on the device, gpu_invoke :438-669 walks the ops, cuda_to_host/get_tensor :289-397,954-966 expand the
+// result to float), without the MLIR parsing in front of it: the caller adds tensors and ops programmatically.
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "internal.h"
+
+namespace {
+
+using namespace mi;
+
+int st_bytes(int t) {
+  return (t == MI_ST_F32 || t == MI_ST_I32 || t == MI_ST_U32) ? 4 : ((t == MI_ST_I8 || t == MI_ST_U8) ? 1 : 2);
+}
+
+struct DevMem {
+  void *ptr = nullptr;
+  int alloc(size_t bytes) {
+    MI_HIP(hipMalloc(&ptr, bytes ? bytes : 4));
+    return MI_SUCCESS;
+  }
+  ~DevMem() {
+    if (ptr)
+      (void)hipFree(ptr);
+  }
+  DevMem() = default;
+  DevMem(const DevMem &) = delete;
+  DevMem &operator=(const DevMem &) = delete;
+};
+
+struct Tensor {
+  std::string name;
+  int st = MI_ST_F32;
+  int64_t n = 0;
+  std::unique_ptr<DevMem> mem;
+};
+
+enum OpKind { OP_A16, OP_I8, OP_CAST, OP_REQUANT };
+
+struct Op {
+  OpKind kind;
+  int in = -1, out = -1;
+  // A16MatMul
+  mi_a16_weight *w = nullptr;
+  int64_t M = 0;
+  // quantized MatMul
+  std::unique_ptr<DevMem> right, bias, mult, shift, zp;
+  int64_t K = 0, N = 0;
+  int a_unsigned = 0, b_unsigned = 0;
+  int64_t input_zp = 0, right_zp = 0;
+  int do_relu = 0;
+  int64_t relu_limit = -1;
+  bool has_rq = false;
+  mi_requant_desc rq{};
+  // Cast
+  mi_cast_attr cast{};
+  float inv_scale = 1.0f, scale = 1.0f;
+  // standalone requant
+  int64_t outer = 1, channels = 1, inner = 1;
+  bool capturable = true;
+};
+
+}  // namespace
+
+struct mi_module {
+  std::vector<Tensor> tensors;
+  std::map<std::string, int> index;
+  std::vector<Op> ops;
+  hipStream_t stream = nullptr;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  bool graph_tried = false;
+  DevMem staging;  // float staging for set_tensor / get_tensor
+  size_t staging_bytes = 0;
+  ~mi_module() {
+    if (exec)
+      (void)hipGraphExecDestroy(exec);
+    if (graph)
+      (void)hipGraphDestroy(graph);
+    for (auto &o : ops)
+      if (o.w)
+        mi_a16_weight_destroy(o.w);
+    if (stream)
+      (void)hipStreamDestroy(stream);
+  }
+};
+
+namespace {
+
+int find(mi_module *m, const char *name, int *idx) {
+  MI_REQUIRE(m && name, MI_BAD_ARGUMENT, "mi_module: null argument");
+  auto it = m->index.find(name);
+  MI_REQUIRE(it != m->index.end(), MI_BAD_ARGUMENT, std::string("mi_module: no tensor named '") + name + "'");
+  *idx = it->second;
+  return MI_SUCCESS;
+}
+
+int upload(std::unique_ptr<DevMem> &dst, const void *src, size_t bytes) {
+  dst.reset(new DevMem());
+  int rc = dst->alloc(bytes);
+  if (rc)
+    return rc;
+  MI_HIP(hipMemcpy(dst->ptr, src, bytes, hipMemcpyHostToDevice));
+  return MI_SUCCESS;
+}
+
+int need_staging(mi_module *m, size_t bytes) {
+  if (bytes <= m->staging_bytes)
+    return MI_SUCCESS;
+  if (m->staging.ptr)
+    (void)hipFree(m->staging.ptr);
+  m->staging.ptr = nullptr;
+  m->staging_bytes = 0;
+  int rc = m->staging.alloc(bytes);
+  if (rc)
+    return rc;
+  m->staging_bytes = bytes;
+  return MI_SUCCESS;
+}
+
+void drop_graph(mi_module *m) {
+  if (m->exec)
+    (void)hipGraphExecDestroy(m->exec);
+  if (m->graph)
+    (void)hipGraphDestroy(m->graph);
+  m->exec = nullptr;
+  m->graph = nullptr;
+  m->graph_tried = false;
+}
+
+// plain storage conversion (the interpreter's float view <-> native storage): a Cast with no quantization on either
+// side; values are already representable in the target type, so nothing is rounded or clamped
+mi_cast_attr plain_cast(int in_t, int out_t, int64_t n) {
+  mi_cast_attr c{};
+  c.num_elem = n;
+  c.in_type = in_t;
+  c.out_type = out_t;
+  c.scale = 1.0;
+  c.expressed = MI_ST_F32;
+  c.round_mode = MI_ROUND_HALF_AWAY_FROM_ZERO;
+  c.chip = MI_CHIP_BM168X;
+  return c;
+}
+
+// Enqueues every op on the module's stream.  Consecutive A16MatMuls that read the same tensor with compatible
+// weight sets (the q/k/v and gate/up siblings) go out as one grouped launch.
+int enqueue_all(mi_module *m) {
+  const size_t n_ops = m->ops.size();
+  for (size_t i = 0; i < n_ops;) {
+    Op &o = m->ops[i];
+    Tensor &tin = m->tensors[o.in], &tout = m->tensors[o.out];
+    int rc = MI_SUCCESS;
+    size_t step = 1;
+    switch (o.kind) {
+    case OP_A16: {
+      const mi_a16_weight *ws[4];
+      uint16_t *ys[4];
+      int g = 0;
+      while (g < 4 && i + g < n_ops) {
+        const Op &c = m->ops[i + g];
+        if (c.kind != OP_A16 || c.in != o.in || c.M != o.M || c.w->K != o.w->K || c.w->bits != o.w->bits ||
+            c.w->g != o.w->g || c.w->dtype != o.w->dtype || c.w->chip != o.w->chip)
+          break;
+        ws[g] = c.w;
+        ys[g] = (uint16_t *)m->tensors[c.out].mem->ptr;
+        ++g;
+      }
+      rc = a16_launch_group(ws, g, (const uint16_t *)tin.mem->ptr, o.M, ys, nullptr, m->stream);
+      step = (size_t)g;
+      break;
+    }
+    case OP_I8:
+      rc = i8mm_launch(tin.mem->ptr, o.a_unsigned, o.right->ptr, o.b_unsigned, /*right_transpose=*/1,
+                       o.bias ? (const int32_t *)o.bias->ptr : nullptr, o.M, o.K, o.N, o.input_zp, o.right_zp,
+                       o.do_relu, o.relu_limit, o.has_rq ? &o.rq : nullptr, tout.mem->ptr, nullptr, m->stream);
+      break;
+    case OP_CAST:
+      rc = cast_launch(&o.cast, tin.mem->ptr, tout.mem->ptr, o.cast.num_elem, o.inv_scale, o.scale, false, m->stream);
+      break;
+    case OP_REQUANT:
+      rc = requant_launch((const int32_t *)tin.mem->ptr, tout.mem->ptr, o.outer, o.channels, o.inner, o.input_zp,
+                          &o.rq, m->stream);
+      break;
+    }
+    if (rc)
+      return rc;
+    i += step;
+  }
+  return MI_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_module_create(mi_module **out) {
+  MI_REQUIRE(out, MI_BAD_ARGUMENT, "mi_module_create: null argument");
+  MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_module_create: no GPU visible");
+  std::unique_ptr<mi_module> m(new mi_module());
+  MI_HIP(hipStreamCreate(&m->stream));
+  *out = m.release();
+  return MI_SUCCESS;
+}
+
+void mi_module_destroy(mi_module *m) { delete m; }
+
+int mi_module_add_tensor(mi_module *m, const char *name, int storage_type, int64_t num_elem) {
+  MI_REQUIRE(m && name, MI_BAD_ARGUMENT, "mi_module_add_tensor: null argument");
+  MI_REQUIRE(storage_type >= MI_ST_F32 && storage_type <= MI_ST_U32 && num_elem > 0, MI_BAD_ARGUMENT,
+             "mi_module_add_tensor: bad storage type or size");
+  MI_REQUIRE(!m->index.count(name), MI_BAD_ARGUMENT, std::string("mi_module_add_tensor: duplicate tensor '") + name + "'");
+  Tensor t;
+  t.name = name;
+  t.st = storage_type;
+  t.n = num_elem;
+  t.mem.reset(new DevMem());
+  int rc = t.mem->alloc((size_t)num_elem * st_bytes(storage_type));
+  if (rc)
+    return rc;
+  m->index[name] = (int)m->tensors.size();
+  m->tensors.push_back(std::move(t));
+  return MI_SUCCESS;
+}
+
+int mi_module_add_a16matmul(mi_module *m, const char *input, const char *output, const mi_a16_weight_desc *desc,
+                            const void *weight, const uint16_t *scale, const uint8_t *zp, const float *bias) {
+  int in, out, rc;
+  if ((rc = find(m, input, &in)) || (rc = find(m, output, &out)))
+    return rc;
+  MI_REQUIRE(desc, MI_BAD_ARGUMENT, "mi_module_add_a16matmul: null descriptor");
+  const int st = desc->dtype == MI_DT_F16 ? MI_ST_F16 : MI_ST_BF16;
+  const Tensor &ti = m->tensors[in], &to = m->tensors[out];
+  MI_REQUIRE(ti.st == st && to.st == st, MI_BAD_ARGUMENT,
+             "mi_module_add_a16matmul: input and output must be stored in the weight set's 16-bit type");
+  MI_REQUIRE(desc->K > 0 && ti.n % desc->K == 0, MI_BAD_ARGUMENT, "mi_module_add_a16matmul: input size is not M * K");
+  const int64_t M = ti.n / desc->K;
+  MI_REQUIRE(to.n == M * desc->N, MI_BAD_ARGUMENT, "mi_module_add_a16matmul: output size is not M * N");
+  Op o;
+  o.kind = OP_A16;
+  o.in = in;
+  o.out = out;
+  o.M = M;
+  rc = mi_a16_weight_create(&o.w, desc, weight, scale, zp, bias);
+  if (rc)
+    return rc;
+  m->ops.push_back(std::move(o));
+  drop_graph(m);
+  return MI_SUCCESS;
+}
+
+int mi_module_add_matmul_int8(mi_module *m, const char *input, const char *output, const mi_module_i8_desc *d) {
+  int in, out, rc;
+  if ((rc = find(m, input, &in)) || (rc = find(m, output, &out)))
+    return rc;
+  MI_REQUIRE(d && d->right, MI_BAD_ARGUMENT, "mi_module_add_matmul_int8: null descriptor or weight");
+  const Tensor &ti = m->tensors[in], &to = m->tensors[out];
+  MI_REQUIRE(ti.st == MI_ST_I8 || ti.st == MI_ST_U8, MI_BAD_ARGUMENT, "mi_module_add_matmul_int8: input must be 8-bit");
+  MI_REQUIRE(d->K > 0 && d->N > 0 && ti.n % d->K == 0, MI_BAD_ARGUMENT, "mi_module_add_matmul_int8: input size is not M * K");
+  const int64_t M = ti.n / d->K;
+  MI_REQUIRE(to.n == M * d->N, MI_BAD_ARGUMENT, "mi_module_add_matmul_int8: output size is not M * N");
+  Op o;
+  o.kind = OP_I8;
+  o.in = in;
+  o.out = out;
+  o.M = M;
+  o.K = d->K;
+  o.N = d->N;
+  o.a_unsigned = ti.st == MI_ST_U8;
+  o.b_unsigned = d->right_unsigned;
+  o.input_zp = d->input_zp;
+  o.right_zp = d->right_zp;
+  o.do_relu = d->do_relu;
+  o.relu_limit = d->relu_limit;
+  // the weight is kept [N, K] (transposed once here when it comes as [K, N])
+  std::vector<uint8_t> nk;
+  const uint8_t *src = (const uint8_t *)d->right;
+  if (!d->right_transpose) {
+    nk.resize((size_t)d->K * d->N);
+    for (int64_t k = 0; k < d->K; ++k)
+      for (int64_t n = 0; n < d->N; ++n)
+        nk[(size_t)n * d->K + k] = src[(size_t)k * d->N + n];
+    src = nk.data();
+  }
+  if ((rc = upload(o.right, src, (size_t)d->K * d->N)))
+    return rc;
+  if (d->bias && (rc = upload(o.bias, d->bias, (size_t)d->N * 4)))
+    return rc;
+  o.has_rq = d->has_requant != 0;
+  if (o.has_rq) {
+    o.rq = d->rq;
+    const int want = o.rq.out_dtype == MI_DT_I8 ? MI_ST_I8 : o.rq.out_dtype == MI_DT_U8 ? MI_ST_U8
+                   : o.rq.out_dtype == MI_DT_I16 ? MI_ST_I16 : o.rq.out_dtype == MI_DT_U16 ? MI_ST_U16 : MI_ST_I32;
+    MI_REQUIRE(to.st == want, MI_BAD_ARGUMENT, "mi_module_add_matmul_int8: output storage differs from the requant type");
+    // per-channel arrays arrive as HOST pointers in this descriptor and move to the device here
+    if (d->rq.d_multiplier) {
+      if ((rc = upload(o.mult, d->rq.d_multiplier, (size_t)d->N * 4)))
+        return rc;
+      o.rq.d_multiplier = (const int32_t *)o.mult->ptr;
+    }
+    if (d->rq.d_shift) {
+      if ((rc = upload(o.shift, d->rq.d_shift, (size_t)d->N * 4)))
+        return rc;
+      o.rq.d_shift = (const int32_t *)o.shift->ptr;
+    }
+    if (d->rq.d_zp) {
+      if ((rc = upload(o.zp, d->rq.d_zp, (size_t)d->N * 4)))
+        return rc;
+      o.rq.d_zp = (const int32_t *)o.zp->ptr;
+    }
+  } else {
+    MI_REQUIRE(to.st == MI_ST_I32, MI_BAD_ARGUMENT, "mi_module_add_matmul_int8: an un-requantized output is int32");
+  }
+  // zero points and unsigned operands make the launch allocate scratch: such ops stay out of a captured graph
+  o.capturable = !o.a_unsigned && !o.b_unsigned && o.input_zp == 0 && o.right_zp == 0;
+  m->ops.push_back(std::move(o));
+  drop_graph(m);
+  return MI_SUCCESS;
+}
+
+int mi_module_add_cast(mi_module *m, const char *input, const char *output, const mi_cast_attr *attr) {
+  int in, out, rc;
+  if ((rc = find(m, input, &in)) || (rc = find(m, output, &out)))
+    return rc;
+  MI_REQUIRE(attr, MI_BAD_ARGUMENT, "mi_module_add_cast: null attribute");
+  const Tensor &ti = m->tensors[in], &to = m->tensors[out];
+  MI_REQUIRE(ti.st == attr->in_type && to.st == attr->out_type && ti.n == to.n, MI_BAD_ARGUMENT,
+             "mi_module_add_cast: tensors do not match the cast's types or sizes");
+  Op o;
+  o.kind = OP_CAST;
+  o.in = in;
+  o.out = out;
+  o.cast = *attr;
+  o.cast.num_elem = ti.n;
+  // validates the attribute and forms the per-call scalars exactly as mi_cast_launch does
+  rc = cast_scalars(&o.cast, &o.inv_scale, &o.scale);
+  if (rc)
+    return rc;
+  m->ops.push_back(std::move(o));
+  drop_graph(m);
+  return MI_SUCCESS;
+}
+
+int mi_module_set_tensor(mi_module *m, const char *name, const float *data, int64_t num_elem) {
+  int idx, rc;
+  if ((rc = find(m, name, &idx)))
+    return rc;
+  Tensor &t = m->tensors[idx];
+  MI_REQUIRE(data && num_elem == t.n, MI_BAD_ARGUMENT, "mi_module_set_tensor: data size is not the tensor's");
+  if (t.st == MI_ST_F32) {
+    MI_HIP(hipMemcpyAsync(t.mem->ptr, data, (size_t)t.n * 4, hipMemcpyHostToDevice, m->stream));
+    MI_HIP(hipStreamSynchronize(m->stream));
+    return MI_SUCCESS;
+  }
+  if ((rc = need_staging(m, (size_t)t.n * 4)))
+    return rc;
+  MI_HIP(hipMemcpyAsync(m->staging.ptr, data, (size_t)t.n * 4, hipMemcpyHostToDevice, m->stream));
+  mi_cast_attr c = plain_cast(MI_ST_F32, t.st, t.n);
+  if ((rc = cast_launch(&c, m->staging.ptr, t.mem->ptr, t.n, 1.0f, 1.0f, false, m->stream)))
+    return rc;
+  MI_HIP(hipStreamSynchronize(m->stream));
+  return MI_SUCCESS;
+}
+
+int mi_module_invoke(mi_module *m) {
+  MI_REQUIRE(m, MI_BAD_ARGUMENT, "mi_module_invoke: null module");
+  if (m->exec) {
+    MI_HIP(hipGraphLaunch(m->exec, m->stream));
+    MI_HIP(hipStreamSynchronize(m->stream));
+    return MI_SUCCESS;
+  }
+  int rc = enqueue_all(m);
+  if (rc)
+    return rc;
+  MI_HIP(hipStreamSynchronize(m->stream));
+  // after the first (eager) pass: record the same launches into a graph when every op is a plain kernel launch
+  if (!m->graph_tried) {
+    m->graph_tried = true;
+    bool ok = !m->ops.empty();
+    for (const auto &o : m->ops)
+      ok = ok && o.capturable;
+    if (ok && hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal) == hipSuccess) {
+      rc = enqueue_all(m);
+      hipGraph_t g = nullptr;
+      hipError_t e = hipStreamEndCapture(m->stream, &g);
+      if (rc == MI_SUCCESS && e == hipSuccess && g && hipGraphInstantiate(&m->exec, g, nullptr, nullptr, 0) == hipSuccess) {
+        m->graph = g;
+      } else {
+        if (g)
+          (void)hipGraphDestroy(g);
+        m->exec = nullptr;
+        (void)hipGetLastError();
+      }
+    }
+  }
+  return MI_SUCCESS;
+}
+
+int mi_module_get_tensor(mi_module *m, const char *name, float *out, int64_t num_elem) {
+  int idx, rc;
+  if ((rc = find(m, name, &idx)))
+    return rc;
+  Tensor &t = m->tensors[idx];
+  MI_REQUIRE(out && num_elem == t.n, MI_BAD_ARGUMENT, "mi_module_get_tensor: buffer size is not the tensor's");
+  const void *src = t.mem->ptr;
+  if (t.st != MI_ST_F32) {
+    if ((rc = need_staging(m, (size_t)t.n * 4)))
+      return rc;
+    mi_cast_attr c = plain_cast(t.st, MI_ST_F32, t.n);
+    if ((rc = cast_launch(&c, t.mem->ptr, m->staging.ptr, t.n, 1.0f, 1.0f, false, m->stream)))
+      return rc;
+    src = m->staging.ptr;
+  }
+  MI_HIP(hipMemcpyAsync(out, src, (size_t)t.n * 4, hipMemcpyDeviceToHost, m->stream));
+  MI_HIP(hipStreamSynchronize(m->stream));
+  return MI_SUCCESS;
+}
+
+int mi_module_uses_graph(const mi_module *m) { return m && m->exec ? 1 : 0; }
+
+}  // extern "C"

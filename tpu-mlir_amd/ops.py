@@ -353,3 +353,87 @@ def requant_launch(x, rq, *, outer, channels, inner, input_zp=0, out=None, strea
     check(clib.lib().mi_requant_launch(_dptr(x), _dptr(out), outer, channels, inner, input_zp, C.byref(rq.c),
                                        _stream_ptr(stream)))
     return out
+
+
+class Module:
+    """Device-resident op list with the calling convention of the reference's interpreter classes
+    (pymlir.module / pymlir.cuda: set_tensor, invoke, get_tensor on float32 numpy arrays); activations stay in HBM
+    in their native storage between the ops."""
+
+    def __init__(self):
+        self.handle = C.c_void_p()
+        self.shapes = {}
+        check(clib.lib().mi_module_create(C.byref(self.handle)))
+
+    def add_tensor(self, name, storage_type, shape):
+        n = int(np.prod(shape))
+        check(clib.lib().mi_module_add_tensor(self.handle, name.encode(), storage_type, n))
+        self.shapes[name] = tuple(shape)
+        return self
+
+    def add_a16matmul(self, input, output, weight, scale_bits, zp, bias=None, *, K, N, weight_bits, q_group_size,
+                      dtype=DT_BF16, chip=CHIP_BM168X):
+        weight = np.ascontiguousarray(weight)
+        scale_bits = np.ascontiguousarray(scale_bits, dtype=np.uint16)
+        zp = np.ascontiguousarray(zp, dtype=np.uint8)
+        bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+        desc = A16WeightDesc(K, N, weight_bits, int(weight.dtype == np.int8), q_group_size, dtype, chip)
+        check(clib.lib().mi_module_add_a16matmul(self.handle, input.encode(), output.encode(), C.byref(desc),
+                                                 weight.ctypes.data, scale_bits.ctypes.data, zp.ctypes.data,
+                                                 None if bias is None else bias.ctypes.data))
+        return self
+
+    def add_matmul_int8(self, input, output, right, bias=None, *, K, N, right_transpose=False, input_zp=0, right_zp=0,
+                        do_relu=False, relu_limit=-1, quant_mode=None, round_mode=ROUND_HALF_AWAY_FROM_ZERO,
+                        out_dtype=DT_I8, chip=CHIP_BM168X, multiplier=1, shift=0, zp=0):
+        """multiplier / shift / zp: scalars or int32 numpy arrays [N] (per channel); shift > 0 shifts right.
+        quant_mode None leaves the int32 accumulators as the output."""
+        right = np.ascontiguousarray(right)
+        bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+        keep = []
+        rq = RequantDescC(quant_mode or 0, round_mode, chip, out_dtype, None, 1, None, 0, None, 0)
+        for name, v in (("multiplier", multiplier), ("shift", shift), ("zp", zp)):
+            if isinstance(v, np.ndarray):
+                a = np.ascontiguousarray(v, dtype=np.int32)
+                keep.append(a)
+                setattr(rq, "d_" + name, a.ctypes.data)
+            else:
+                setattr(rq, name, int(v))
+        d = clib.ModuleI8Desc(K, N, right.ctypes.data, int(right_transpose), int(right.dtype == np.uint8),
+                              None if bias is None else bias.ctypes.data, input_zp, right_zp, int(do_relu),
+                              int(relu_limit), int(quant_mode is not None), rq)
+        check(clib.lib().mi_module_add_matmul_int8(self.handle, input.encode(), output.encode(), C.byref(d)))
+        return self
+
+    def add_cast(self, input, output, *, in_type, out_type, in_quant=False, out_quant=False, scale=1.0, zero_point=0,
+                 expressed=None, round_mode=ROUND_HALF_AWAY_FROM_ZERO):
+        attr = clib.CastAttr(0, in_type, out_type, int(in_quant), int(out_quant), float(scale), int(zero_point),
+                             clib.ST_F32 if expressed is None else expressed, round_mode, CHIP_BM168X)
+        check(clib.lib().mi_module_add_cast(self.handle, input.encode(), output.encode(), C.byref(attr)))
+        return self
+
+    def set_tensor(self, name, data):
+        data = _f32(data)
+        check(clib.lib().mi_module_set_tensor(self.handle, name.encode(), data.ctypes.data, data.size))
+
+    def invoke(self):
+        check(clib.lib().mi_module_invoke(self.handle))
+
+    def uses_graph(self):
+        return bool(clib.lib().mi_module_uses_graph(self.handle))
+
+    def get_tensor(self, name):
+        out = np.empty(self.shapes[name], dtype=np.float32)
+        check(clib.lib().mi_module_get_tensor(self.handle, name.encode(), out.ctypes.data, out.size))
+        return out
+
+    def destroy(self):
+        if self.handle:
+            clib.lib().mi_module_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
