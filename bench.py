@@ -227,6 +227,42 @@ def bench_operator_boundary(pkg, S, steps=20):
             "GBps_algorithmic": round(S.w4_gemv_bytes(1, K, N, 128) / sec / 1e9, 1)}
 
 
+def bench_module_block(pkg, S, clib, cfgs, steps=50):
+    """The decode block as a device-resident op list (float32 in through set_tensor, Cast to bf16, the seven
+    matmuls chained q/k/v <- x, o <- q, gate/up <- o, down <- gate, float32 out through get_tensor): wall time of
+    invoke() alone (graph replay + stream sync) and of the whole set_tensor/invoke/get_tensor round trip."""
+    by = {name: cfg for cfg, (name, K, N) in zip(cfgs, S.LLAMA7B_CHAIN)}
+    m = pkg.Module()
+    m.add_tensor("x", clib.ST_F32, (1, 4096)).add_tensor("xb", clib.ST_BF16, (1, 4096))
+    for name, K, N in S.LLAMA7B_CHAIN:
+        m.add_tensor(name, clib.ST_BF16, (1, N))
+    m.add_cast("x", "xb", in_type=clib.ST_F32, out_type=clib.ST_BF16)
+    src = {"q_proj": "xb", "k_proj": "xb", "v_proj": "xb", "o_proj": "q_proj", "gate_proj": "o_proj",
+           "up_proj": "o_proj", "down_proj": "gate_proj"}
+    for name, K, N in S.LLAMA7B_CHAIN:
+        c = by[name]
+        m.add_a16matmul(src[name], name, c["weight"], c["scale"], c["zp"], None, K=K, N=N, weight_bits=4,
+                        q_group_size=128)
+    x = np.random.default_rng(3).standard_normal((1, 4096)).astype(np.float32)
+    m.set_tensor("x", x)
+    for _ in range(5):
+        m.invoke()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        m.invoke()
+    t_inv = (time.perf_counter() - t0) / steps
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        m.set_tensor("x", x)
+        m.invoke()
+        m.get_tensor("down_proj")
+    t_all = (time.perf_counter() - t0) / steps
+    graph = m.uses_graph()
+    m.destroy()
+    return {"case": "llama7b decode block as mi_module (cast + 7 A16MatMul, one weight copy)",
+            "invoke_us": round(t_inv * 1e6, 1), "set_invoke_get_us": round(t_all * 1e6, 1), "graph_replay": graph}
+
+
 def cpu_baseline_chain(S, M, cfgs, budget_s=20.0):
     """The restated reference algorithm (oracle) on the host cores: per call dequantize [N,K] to f32,
     transpose to [K,N], f32 GEMM, round to bf16 -- what A16MatMul.cpp:172-245 + Dnnl/MatMul.cpp:167-227 do."""
@@ -333,6 +369,7 @@ def main():
         ex["single_matmuls"] = bench_single_matmuls(pkg, S, torch)
         ex["int8_256x1024x1024"] = bench_int8(pkg, S, torch, clib, 1024, 40, 5, M=256)
         ex["operator_boundary"] = bench_operator_boundary(pkg, S)
+        ex["device_resident_block"] = bench_module_block(pkg, S, clib, cfgs)
         line["extras"] = ex
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_chain(S, M, cfgs)
