@@ -237,6 +237,7 @@ struct SkinnyArgs {
   int full_tiles;       // tiles that lie completely inside K
   int G;
   int tiles_per_group;  // GPT == 1: tiles that share one group (g / TILE_K; k_tiles when per channel)
+  int group_shift;      // log2(tiles_per_group) when that is a power of two, 31 when one group spans K, else -1
   int chip;
 };
 
@@ -324,11 +325,11 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
   struct {
     const uint16_t *x;
     int64_t K;
-    int M, row_blocks, k_tiles, full_tiles, G, tiles_per_group, b1, b2, b3;
-  } h = {a.x, a.K, a.M, a.row_blocks, a.k_tiles, a.full_tiles, a.G, a.tiles_per_group,
+    int M, row_blocks, k_tiles, full_tiles, G, tiles_per_group, group_shift, b1, b2, b3;
+  } h = {a.x, a.K, a.M, a.row_blocks, a.k_tiles, a.full_tiles, a.G, a.tiles_per_group, a.group_shift,
          a.seg[1].rb_begin, a.seg[2].rb_begin, a.seg[3].rb_begin};
   asm volatile("" ::"s"(h.x), "s"(h.K), "s"(h.M), "s"(h.row_blocks), "s"(h.k_tiles), "s"(h.full_tiles), "s"(h.G),
-               "s"(h.tiles_per_group), "s"(h.b1), "s"(h.b2), "s"(h.b3));
+               "s"(h.tiles_per_group), "s"(h.group_shift), "s"(h.b1), "s"(h.b2), "s"(h.b3));
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
   constexpr int TILE_K = BITS == 4 ? W4_TILE_K : W8_TILE_K;
@@ -388,31 +389,35 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
 
   auto unit_group = [&](int kt, int u) {
     int gi;
-    // tiles_per_group is 1 for the common group size == tile size; the division only runs for larger groups
+    // one shift for the usual group sizes (a tile, a power-of-two number of tiles, or all of K); the division only
+    // runs for the odd multiples of the tile size
     if constexpr (GPT == 1)
-      gi = h.tiles_per_group == 1 ? kt : kt / h.tiles_per_group;
+      gi = h.group_shift >= 0 ? (kt >> h.group_shift) : kt / h.tiles_per_group;
     else
       gi = kt * GPT + u;
     return gi < h.G ? gi : h.G - 1;
   };
 
+  // byte offsets inside a row block fit 32 bits (k_tiles * 1 KiB): scalar tile offset + per-lane offset, one vector
+  // add per request, against the row block's 64-bit base in scalar registers
   auto load_tile = [&](Tile &t, int kt) {
 #ifdef MI_DBG_SAMETILE
     kt = kt & 1;
 #endif
+    const uint32_t woff = (uint32_t)kt * 1024u + lane16;
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      t.w[r] = *(const u32x4 *)(wq[r] + (int64_t)kt * 1024 + lane16);
+      t.w[r] = *(const u32x4 *)(wq[r] + woff);
 #pragma unroll
     for (int u = 0; u < GPT; ++u) {
-      const int gi = unit_group(kt, u);
+      const uint32_t gi = (uint32_t)unit_group(kt, u);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         if constexpr (BITS == 4) {
-          t.sz[r][u] = *(const uint32_t *)(szp[r] + gi * 64 + col4);
+          t.sz[r][u] = *(const uint32_t *)(szp[r] + (gi * 64u + col4));
         } else {
-          t.sz[r][u] = *(const uint16_t *)(scp[r] + gi * 32 + col2);
-          t.nz[r][u] = *(const float *)(nzp[r] + gi * 64 + col4);
+          t.sz[r][u] = *(const uint16_t *)(scp[r] + (gi * 32u + col2));
+          t.nz[r][u] = *(const float *)(nzp[r] + (gi * 64u + col4));
         }
       }
     }
@@ -604,17 +609,17 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
       const int kt = h.full_tiles;
 #pragma unroll
       for (int r = 0; r < R; ++r)
-        t.w[r] = *(const u32x4 *)(wq[r] + (int64_t)kt * 1024 + lane16);
+        t.w[r] = *(const u32x4 *)(wq[r] + ((uint32_t)kt * 1024u + lane16));
 #pragma unroll
       for (int u = 0; u < GPT; ++u) {
-        const int gi = unit_group(kt, u);
+        const uint32_t gi = (uint32_t)unit_group(kt, u);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           if constexpr (BITS == 4) {
-            t.sz[r][u] = *(const uint32_t *)(szp[r] + gi * 64 + col4);
+            t.sz[r][u] = *(const uint32_t *)(szp[r] + (gi * 64u + col4));
           } else {
-            t.sz[r][u] = *(const uint16_t *)(scp[r] + gi * 32 + col2);
-            t.nz[r][u] = *(const float *)(nzp[r] + gi * 64 + col4);
+            t.sz[r][u] = *(const uint16_t *)(scp[r] + (gi * 32u + col2));
+            t.nz[r][u] = *(const float *)(nzp[r] + (gi * 64u + col4));
           }
         }
       }
@@ -759,6 +764,20 @@ static bool launch_skinny_x(const SkinnyArgs &a, const SkinnyPlan &plan, int64_t
               : launch_skinny<BITS, DT, GPT, false>(a, plan, m_blocks, x_bytes, st);
 }
 
+// log2 of the tiles one group spans when that is a power of two; 31 (index 0 for every tile) when a single group spans
+// all of K; -1 when the kernel has to divide
+static int group_shift_of(int tiles_per_group, int k_tiles) {
+  if (tiles_per_group >= k_tiles)
+    return 31;
+  if ((tiles_per_group & (tiles_per_group - 1)) == 0) {
+    int s = 0;
+    while ((1 << s) < tiles_per_group)
+      ++s;
+    return s;
+  }
+  return -1;
+}
+
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                hipStream_t stream) {
   return a16_launch_group(&w, 1, d_x, M, &d_y, d_y_f32 ? &d_y_f32 : nullptr, stream);
@@ -816,6 +835,7 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
   a.G = w->G;
   a.chip = w->chip;
   a.tiles_per_group = 1;
+  a.group_shift = 0;
   const int64_t m_blocks = (M + 15) / 16;
   const size_t x_bytes = skinny_x_bytes((int)(M < 16 ? M : 16), w->k_tiles, tile_k);
   const bool xlds = x_bytes <= XLDS_MAX_BYTES && !getenv("MI_A16_NO_XLDS");
@@ -830,6 +850,7 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
       a.tiles_per_group = w->g / W4_TILE_K;
     else
       gpt = W4_TILE_K / w->g;
+    a.group_shift = group_shift_of(a.tiles_per_group, (int)w->k_tiles);
     if (gpt == 1)
       ok = f16 ? launch_skinny_x<4, MI_DT_F16, 1>(a, plan, m_blocks, xlds, x_bytes, stream)
                : launch_skinny_x<4, MI_DT_BF16, 1>(a, plan, m_blocks, xlds, x_bytes, stream);
@@ -847,6 +868,7 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
       a.tiles_per_group = w->g / W8_TILE_K;
     else
       gpt = W8_TILE_K / w->g;
+    a.group_shift = group_shift_of(a.tiles_per_group, (int)w->k_tiles);
     if (gpt == 1)
       ok = f16 ? launch_skinny_x<8, MI_DT_F16, 1>(a, plan, m_blocks, xlds, x_bytes, stream)
                : launch_skinny_x<8, MI_DT_BF16, 1>(a, plan, m_blocks, xlds, x_bytes, stream);
