@@ -343,8 +343,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE (profiles/hbm_traffic_pmc_*.md):
-                     # 1.03 x the algorithmic bytes at M = 1; not re-measured by this run
-                     "traffic": int(bytes_per_launch * 1.03) if M == 1 else None,
+                     # 1.022 x the algorithmic bytes at M = 1 with grouped launches; not re-measured by this run
+                     "traffic": int(bytes_per_launch * 1.022) if (M == 1 and not args.no_group) else None,
                      "kernel": "a16w4_skinny_kernel<bf16, 1 group/tile>",
                      "bytes_per_launch": int(bytes_per_launch),
                      "avg_launch_us": round(avg_launch_s * 1e6, 3),
