@@ -120,6 +120,37 @@ void mi_a16_weight_destroy(mi_a16_weight *w);
 /* HBM bytes held by the packed set */
 size_t mi_a16_weight_bytes(const mi_a16_weight *w);
 
+/* The packed set as one relocatable blob (header + the tile-ordered arrays exactly as they sit in HBM): the
+ * on-disk, gfx950-ordered weight format.  Counterpart of the reference's chip-specific weight reorder
+ * (lib/Dialect/Tpu/Transforms/WeightReorder/BM1684X/A16MatMul.cpp:61-319), which likewise stores the weight in
+ * the order its kernel reads it.  import uploads a blob without repacking. */
+size_t mi_a16_weight_export_size(const mi_a16_weight *w);
+int mi_a16_weight_export(const mi_a16_weight *w, void *blob, size_t capacity);
+int mi_a16_weight_import(mi_a16_weight **out, const void *blob, size_t size);
+
+/* ---- weight producers (the compile-time side of tpu.A16MatMul), computed on the GPU, host arrays in and out ---- */
+typedef struct mi_a16_quant_desc {
+  int64_t K, N;
+  int weight_bits;   /* 4 / 8 */
+  int q_group_size;  /* 0 per channel, > 0 groups along K, -1 one group per row */
+  int symmetric;     /* module::isQuantSymmetric(); ignored per channel */
+  int dtype;         /* MI_DT_BF16 / MI_DT_F16: type the scales are stored in */
+} mi_a16_quant_desc;
+/* A16MatMulAdjust (lib/Dialect/Tpu/Canonicalize/A16MatMul.cpp:270-429; computePerChannelParam :22-48,
+ * computePerGroupParam :78-115, weightQuantization :147-216; static quantization, uint8 zero points).
+ * w_kn: the f32 weight [K, N] of the top-level matmul.  Out, in the layout mi_a16_weight_create takes:
+ * weight [N, K/2] (4-bit) or [N, K]; scale16 [N, G] bit patterns; scale_f32 [N, G] (may be NULL); zp [N, G];
+ * *sign = !(min(w) > 0); *weight_signed = the 8-bit bytes are int8 (per channel and sign). */
+int mi_a16_quantize(const mi_a16_quant_desc *desc, const float *w_kn, void *weight, uint16_t *scale16,
+                    float *scale_f32, uint8_t *zp, int *sign, int *weight_signed);
+/* GPTQ / AWQ checkpoint tensors -> the same layout (python/llm/LlmConverter.py:320-389 unpack_weights and the
+ * transposes at :1454-1475).  qweight: GPTQ int32 [K*bits/32, N], AWQ int32 [K, N*bits/32]; qzeros int32
+ * [G, N*bits/32] (GPTQ stores zero - 1).  AWQ is 4-bit only.  The scales of such checkpoints are [G, N] 16-bit
+ * values and only need transposing, which is left to the caller. */
+enum { MI_PACK_GPTQ = 0, MI_PACK_AWQ = 1 };
+int mi_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qzeros, int64_t K, int64_t N, int64_t G,
+                  uint8_t *weight, uint8_t *zp);
+
 /* y[M,N] = round(x[M,K] * dequant(W)^T + bias).  d_x/d_y are DEVICE pointers to bf16/f16 bit patterns;
  * d_y_f32 (optional DEVICE pointer, may be NULL) receives the fp32 result before output rounding.
  * Asynchronous on `stream` (a hipStream_t, NULL = default stream). */

@@ -826,3 +826,153 @@ int orc_cast(const orc_cast_attr *a, const float *in, float *out, int64_t n) {
   }
   return 0;
 }
+
+/* ---- weight producers ---------------------------------------------------------------------- */
+/* findMinMax / findMaxabs: lib/Support/MathUtils.cpp:80-109 */
+static void orc_min_max(const float *p, int64_t n, float *mn, float *mx) {
+  float lo = p[0], hi = p[0];
+  for (int64_t i = 0; i < n; ++i) {
+    lo = p[i] < lo ? p[i] : lo;
+    hi = p[i] > hi ? p[i] : hi;
+  }
+  *mn = lo;
+  *mx = hi;
+}
+static float orc_max_abs(const float *p, int64_t n) {
+  float m = 0.0f;
+  for (int64_t i = 0; i < n; ++i)
+    m = fabsf(p[i]) > m ? fabsf(p[i]) : m;
+  return m;
+}
+/* to_uint4 / to_uint8 / to_int8: MathUtils.h:325-352 (to_int with HALF_AWAY, then clamp) */
+static int64_t orc_clamp_code(float v, int64_t lo, int64_t hi) {
+  int64_t i = orc_to_int_f32(v, ORC_ROUNDING_HALF_AWAY_FROM_ZERO);
+  return i > hi ? hi : i < lo ? lo : i;
+}
+static int orc_clampi(int v, int lo, int hi) { return v < lo ? lo : v > hi ? hi : v; }
+
+int orc_a16_quantize(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16,
+                     uint8_t *q, float *scale_f32, uint16_t *scale16, uint8_t *zp, int *sign_out,
+                     int *weight_signed_out) {
+  if ((bits != 4 && bits != 8) || K <= 0 || N <= 0 || (bits == 4 && (K & 1)))
+    return -1;
+  /* :312-321 transpose to [row = N, col = K] */
+  const int64_t row = N, col = K;
+  float *w = (float *)malloc(sizeof(float) * (size_t)(row * col));
+  if (!w)
+    return -1;
+  for (int64_t k = 0; k < K; ++k)
+    for (int64_t n = 0; n < N; ++n)
+      w[n * K + k] = w_kn[k * N + n];
+  /* :323-326 */
+  float gmin, gmax;
+  orc_min_max(w, row * col, &gmin, &gmax);
+  const int sign = !(gmin > 0);
+  int64_t gs = g;
+  if (gs == -1)
+    gs = col; /* :362-363 */
+  if (gs != 0 && (gs < 0 || col % gs != 0)) {
+    free(w);
+    return -1;
+  }
+  const int sym = gs != 0 ? symmetric : 0; /* :335 */
+  const int64_t G = gs ? col / gs : 1;
+  const int max_int = bits == 4 ? 15 : 255;
+  for (int64_t i = 0; i < row * G; ++i)
+    zp[i] = sym ? (bits == 4 ? 8 : 128) : 0; /* :340-345 */
+  if (!gs) {
+    /* computePerChannelParam :22-48 */
+    for (int64_t c = 0; c < row; ++c) {
+      const float *p = w + c * col;
+      if (bits != 4) {
+        const float w_max = orc_max_abs(p, col);
+        const int pow_value = sign ? bits - 1 : bits;
+        scale_f32[c] = (float)(w_max / (pow(2, pow_value) - 1));
+      } else {
+        float mn, mx;
+        orc_min_max(p, col, &mn, &mx);
+        const float d = mx - mn;
+        scale_f32[c] = (d > 1e-5f ? d : 1e-5f) / max_int;
+        zp[c] = (uint8_t)orc_clampi(-(int)roundf(mn / scale_f32[c]), 0, max_int);
+      }
+    }
+  } else {
+    /* computePerGroupParam :78-115 (not dynamic-quant) */
+    for (int64_t i = 0; i < row * G; ++i) {
+      const float *p = w + i * gs;
+      float mn, mx;
+      orc_min_max(p, gs, &mn, &mx);
+      const float abs_max = orc_max_abs(p, gs);
+      if (sym) {
+        scale_f32[i] = 2 * fabsf(abs_max) / max_int;
+      } else {
+        const float d = mx - mn;
+        scale_f32[i] = (d > 1e-5f ? d : 1e-5f) / (max_int - 0);
+        zp[i] = (uint8_t)orc_clampi(-(int)roundf(mn / scale_f32[i]), 0, max_int);
+      }
+    }
+  }
+  /* weightQuantization :147-216 */
+  const int as_int8 = !gs && sign && bits == 8; /* :413-416 */
+  for (int64_t c = 0; c < row; ++c)
+    for (int64_t i = 0; i < col; ++i) {
+      const int64_t qi = gs ? (c * col + i) / gs : c;
+      const float t = roundf(w[c * col + i] / scale_f32[qi]) + (float)zp[qi];
+      if (bits == 8) {
+        if (as_int8)
+          q[c * col + i] = (uint8_t)(int8_t)orc_clamp_code(t, -128, 127);
+        else
+          q[c * col + i] = (uint8_t)orc_clamp_code(t, 0, 255);
+      } else {
+        const uint8_t code = (uint8_t)orc_clamp_code(t, 0, 15);
+        uint8_t *dst = q + (c * col) / 2 + i / 2;
+        if (i % 2)
+          *dst |= (uint8_t)(code << 4);
+        else
+          *dst = code;
+      }
+    }
+  /* :385-392 clone_f16 / clone_bf16 of the f32 scale */
+  for (int64_t i = 0; i < row * G; ++i)
+    scale16[i] = f16 ? orc_f32_to_f16(scale_f32[i]) : orc_f32_to_bf16(scale_f32[i], 0);
+  *sign_out = sign;
+  *weight_signed_out = as_int8;
+  free(w);
+  return 0;
+}
+
+int orc_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qzeros, int64_t K, int64_t N, int64_t G,
+                   uint8_t *q, uint8_t *zp) {
+  if ((bits != 4 && bits != 8) || (mode != ORC_PACK_GPTQ && mode != ORC_PACK_AWQ))
+    return -1;
+  const int ratio = 32 / bits;                 /* LlmConverter.py:322 */
+  const uint32_t mask = bits == 4 ? 0xF : 0xFF;
+  static const int awq_order[8] = {0, 4, 1, 5, 2, 6, 3, 7}; /* :349 */
+  if (K % ratio || N % ratio || (bits == 4 && (K & 1)) || (mode == ORC_PACK_AWQ && bits != 4))
+    return -1;
+  for (int64_t k = 0; k < K; ++k)
+    for (int64_t n = 0; n < N; ++n) {
+      uint32_t v;
+      if (mode == ORC_PACK_GPTQ) /* :336-339: row k of the unpacked weight sits in word k / ratio, slot k % ratio */
+        v = ((uint32_t)qweight[(k / ratio) * N + n] >> (bits * (k % ratio))) & mask;
+      else /* :350-352: column n sits in word n / ratio, slot order_map[n % ratio] */
+        v = ((uint32_t)qweight[k * (N / ratio) + n / ratio] >> (bits * awq_order[n % ratio])) & mask;
+      /* :340-346 pack pairs of k, then :1470 transpose to [N, K/2] */
+      if (bits == 8)
+        q[n * K + k] = (uint8_t)v;
+      else if (k % 2 == 0)
+        q[n * (K / 2) + k / 2] = (uint8_t)v;
+      else
+        q[n * (K / 2) + k / 2] |= (uint8_t)(v << 4);
+    }
+  for (int64_t gi = 0; gi < G; ++gi)
+    for (int64_t n = 0; n < N; ++n) {
+      /* :365-367: the zero points use the same slot order as the mode's weights */
+      const int slot = mode == ORC_PACK_GPTQ ? (int)(n % ratio) : awq_order[n % ratio];
+      uint32_t z = ((uint32_t)qzeros[gi * (N / ratio) + n / ratio] >> (bits * slot)) & mask;
+      if (mode == ORC_PACK_GPTQ)
+        z = (uint8_t)(z + 1); /* :386-387, numpy uint8 arithmetic wraps */
+      zp[n * G + gi] = (uint8_t)z;
+    }
+  return 0;
+}

@@ -24,6 +24,11 @@
  *   orc_f32_to_bf16 (cvi)        add-0x7fff+lsb closed form, inf->0x7f7f
  *   orc_f32_to_f16               numpy float16 RNE incl. subnormals
  *   orc_cast                     numpy closed forms per branch (tests/test_oracle_cast.py)
+ *   orc_a16_quantize             on-grid weights are recovered exactly, |w - dequant(q)| <= scale/2 inside the
+ *                                clamp range, closed-form scale/zp, nibble order via the A16MatMul dequantizer
+ *                                (tests/test_oracle_packers.py)
+ *   orc_llm_unpack               inverse of independently written GPTQ / AWQ packers, AutoAWQ's published pack
+ *                                order (tests/test_oracle_packers.py)
  *   orc_a16_dequant              one-hot activations recover nibble order,
  *                                group indexing and scale layout
  *   orc_sgemm_*                  float64 reference with the standard bound
@@ -207,6 +212,23 @@ typedef struct {
 } orc_cast_attr;
 /* returns 0, or -1 for a branch this restatement leaves out (CV18xx, fp8) */
 int orc_cast(const orc_cast_attr *attr, const float *input, float *output, int64_t n);
+
+/* ---- weight producers (compile-time side of tpu.A16MatMul) ------------------- */
+/* A16MatMulAdjust, lib/Dialect/Tpu/Canonicalize/A16MatMul.cpp:270-429, static uint8-zero-point variant:
+ * w_kn is the f32 weight [K, N] of the top-level matmul; the result is the [N, K] ("w_transpose") operand set:
+ * q [N, K/2] (4-bit, low nibble = even k) or [N, K] (8-bit; int8 values when *weight_signed), scale [N, G] as f32 and
+ * as the 16-bit pattern the WeightOp clone stores, zp [N, G].  g: 0 per channel, > 0 groups along K, -1 one group
+ * per row.  Returns 0, or -1 for arguments the reference asserts on. */
+int orc_a16_quantize(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16,
+                     uint8_t *q, float *scale_f32, uint16_t *scale16, uint8_t *zp, int *sign, int *weight_signed);
+
+/* GPTQ / AWQ checkpoints -> the [N, K/2] + [N, G] layout, python/llm/LlmConverter.py:320-389 (unpack_weights) and
+ * :1454-1475 (the transposes).  qweight: GPTQ int32 [K*bits/32, N] (packed along K), AWQ int32 [K, N*bits/32]
+ * (packed along N in the order 0,4,1,5,2,6,3,7).  qzeros int32 [G, N*bits/32]; GPTQ stores zero - 1.
+ * Out: q [N, K/2] (4-bit) or [N, K]; zp [N, G]. */
+enum { ORC_PACK_GPTQ = 0, ORC_PACK_AWQ = 1 };
+int orc_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qzeros, int64_t K, int64_t N, int64_t G,
+                   uint8_t *q, uint8_t *zp);
 
 #ifdef __cplusplus
 }

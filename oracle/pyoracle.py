@@ -281,5 +281,49 @@ def cast(x, *, in_type, out_type, in_quant=False, out_quant=False, scale=1.0, ze
     return out
 
 
+PACK_GPTQ, PACK_AWQ = 0, 1
+
+
+def a16_quantize(w_kn, *, bits, g, symmetric=False, f16=False):
+    """A16MatMulAdjust on the f32 weight [K, N] of a top-level matmul.
+
+    Returns dict(weight [N, K/2] or [N, K] uint8 (int8 bit patterns when weight_signed), scale_f32 [N, G],
+    scale16 [N, G] bit patterns, zp [N, G] uint8, sign, weight_signed).
+    """
+    w = np.ascontiguousarray(w_kn, dtype=np.float32)
+    K, N = w.shape
+    gs = K if g == -1 else g
+    G = K // gs if gs else 1
+    q = np.zeros((N, K // 2 if bits == 4 else K), dtype=np.uint8)
+    sf = np.zeros((N, G), dtype=np.float32)
+    s16 = np.zeros((N, G), dtype=np.uint16)
+    zp = np.zeros((N, G), dtype=np.uint8)
+    sign, wsigned = C.c_int(0), C.c_int(0)
+    L = lib()
+    L.orc_a16_quantize.restype = C.c_int
+    rc = L.orc_a16_quantize(_p(w, C.c_float), C.c_int64(K), C.c_int64(N), C.c_int(bits), C.c_int(g),
+                            C.c_int(int(symmetric)), C.c_int(int(f16)), _p(q, C.c_uint8), _p(sf, C.c_float),
+                            _p(s16, C.c_uint16), _p(zp, C.c_uint8), C.byref(sign), C.byref(wsigned))
+    if rc != 0:
+        raise RuntimeError("orc_a16_quantize: bad arguments")
+    return dict(weight=q, scale_f32=sf, scale16=s16, zp=zp, sign=bool(sign.value), weight_signed=bool(wsigned.value))
+
+
+def llm_unpack(mode, bits, qweight, qzeros, K, N):
+    """GPTQ / AWQ int32 checkpoint tensors -> (weight [N, K/2] or [N, K] uint8, zp [N, G] uint8)."""
+    qweight = np.ascontiguousarray(qweight, dtype=np.int32)
+    qzeros = np.ascontiguousarray(qzeros, dtype=np.int32)
+    G = qzeros.shape[0]
+    q = np.zeros((N, K // 2 if bits == 4 else K), dtype=np.uint8)
+    zp = np.zeros((N, G), dtype=np.uint8)
+    L = lib()
+    L.orc_llm_unpack.restype = C.c_int
+    rc = L.orc_llm_unpack(C.c_int(mode), C.c_int(bits), _p(qweight, C.c_int32), _p(qzeros, C.c_int32), C.c_int64(K),
+                          C.c_int64(N), C.c_int64(G), _p(q, C.c_uint8), _p(zp, C.c_uint8))
+    if rc != 0:
+        raise RuntimeError("orc_llm_unpack: bad arguments")
+    return q, zp
+
+
 def num_threads():
     return lib().orc_num_threads()

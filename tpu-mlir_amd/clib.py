@@ -19,6 +19,7 @@ EXPORTS = [
     "mi_a16mm_init", "mi_a16mm_inference", "mi_a16mm_deinit",
     "mi_a16_weight_create", "mi_a16_weight_destroy", "mi_a16_weight_bytes", "mi_a16mm_launch",
     "mi_a16mm_launch_group",
+    "mi_a16_weight_export_size", "mi_a16_weight_export", "mi_a16_weight_import", "mi_a16_quantize", "mi_llm_unpack",
     "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
     "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
     "mi_cast_inference", "mi_cast_launch",
@@ -49,6 +50,11 @@ class A16Attr(C.Structure):
 class A16WeightDesc(C.Structure):
     _fields_ = [("K", C.c_int64), ("N", C.c_int64), ("weight_bits", C.c_int), ("weight_signed", C.c_int),
                 ("q_group_size", C.c_int), ("dtype", C.c_int), ("chip", C.c_int)]
+
+
+class A16QuantDesc(C.Structure):
+    _fields_ = [("K", C.c_int64), ("N", C.c_int64), ("weight_bits", C.c_int), ("q_group_size", C.c_int),
+                ("symmetric", C.c_int), ("dtype", C.c_int)]
 
 
 class I8Attr(C.Structure):
@@ -120,6 +126,14 @@ def lib():
         L.mi_a16_weight_create.argtypes = [C.POINTER(C.c_void_p), C.POINTER(A16WeightDesc), C.c_void_p, C.c_void_p,
                                            C.c_void_p, C.c_void_p]
         L.mi_a16_weight_destroy.argtypes = [C.c_void_p]
+        L.mi_a16_weight_export_size.restype = C.c_size_t
+        L.mi_a16_weight_export_size.argtypes = [C.c_void_p]
+        L.mi_a16_weight_export.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        L.mi_a16_weight_import.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_size_t]
+        L.mi_a16_quantize.argtypes = [C.POINTER(A16QuantDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                      C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        L.mi_llm_unpack.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
+                                    C.c_void_p, C.c_void_p]
         L.mi_a16_weight_destroy.restype = None
         L.mi_a16mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_launch_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int64,

@@ -189,6 +189,152 @@ void mi_a16_weight_destroy(mi_a16_weight *w) {
 
 size_t mi_a16_weight_bytes(const mi_a16_weight *w) { return w ? w->bytes : 0; }
 
+// ---- packed weight set <-> blob ---------------------------------------------------------------------------------
+namespace {
+struct BlobHeader {
+  char magic[8];  // "MIA16W1\0"
+  int64_t K, N, row_blocks, k_tiles;
+  int32_t bits, g, G, dtype, chip, has_bias;
+  uint64_t packed_bytes, qparam_entries;  // qparam_entries = row_blocks * G * 16
+};
+const char kBlobMagic[8] = {'M', 'I', 'A', '1', '6', 'W', '1', 0};
+size_t blob_payload(const BlobHeader &h) {
+  return (size_t)h.packed_bytes + (size_t)h.qparam_entries * (h.bits == 4 ? 4 : 6) + (h.has_bias ? (size_t)h.N * 4 : 0);
+}
+BlobHeader blob_header_of(const mi_a16_weight *w) {
+  BlobHeader h;
+  memset(&h, 0, sizeof(h));
+  memcpy(h.magic, kBlobMagic, 8);
+  h.K = w->K;
+  h.N = w->N;
+  h.row_blocks = w->row_blocks;
+  h.k_tiles = w->k_tiles;
+  h.bits = w->bits;
+  h.g = w->g;
+  h.G = w->G;
+  h.dtype = w->dtype;
+  h.chip = w->chip;
+  h.has_bias = w->bias != nullptr;
+  h.packed_bytes = (uint64_t)w->row_blocks * w->k_tiles * 1024;
+  h.qparam_entries = (uint64_t)w->row_blocks * w->G * 16;
+  return h;
+}
+}  // namespace
+
+size_t mi_a16_weight_export_size(const mi_a16_weight *w) {
+  if (!w)
+    return 0;
+  const BlobHeader h = blob_header_of(w);
+  return sizeof(BlobHeader) + blob_payload(h);
+}
+
+int mi_a16_weight_export(const mi_a16_weight *w, void *blob, size_t capacity) {
+  MI_REQUIRE(w && blob, MI_BAD_ARGUMENT, "mi_a16_weight_export: null argument");
+  const BlobHeader h = blob_header_of(w);
+  MI_REQUIRE(capacity >= sizeof(BlobHeader) + blob_payload(h), MI_BAD_ARGUMENT,
+             "mi_a16_weight_export: buffer smaller than mi_a16_weight_export_size()");
+  uint8_t *p = (uint8_t *)blob;
+  memcpy(p, &h, sizeof(h));
+  p += sizeof(h);
+  MI_HIP(hipMemcpy(p, w->qweight, h.packed_bytes, hipMemcpyDeviceToHost));
+  p += h.packed_bytes;
+  if (w->bits == 4) {
+    MI_HIP(hipMemcpy(p, w->sz_t, h.qparam_entries * 4, hipMemcpyDeviceToHost));
+    p += h.qparam_entries * 4;
+  } else {
+    MI_HIP(hipMemcpy(p, w->scale_t, h.qparam_entries * 2, hipMemcpyDeviceToHost));
+    p += h.qparam_entries * 2;
+    MI_HIP(hipMemcpy(p, w->nzs_t, h.qparam_entries * 4, hipMemcpyDeviceToHost));
+    p += h.qparam_entries * 4;
+  }
+  if (h.has_bias)
+    MI_HIP(hipMemcpy(p, w->bias, (size_t)h.N * 4, hipMemcpyDeviceToHost));
+  return MI_SUCCESS;
+}
+
+int mi_a16_weight_import(mi_a16_weight **out, const void *blob, size_t size) {
+  MI_REQUIRE(out && blob, MI_BAD_ARGUMENT, "mi_a16_weight_import: null argument");
+  *out = nullptr;
+  MI_REQUIRE(size >= sizeof(BlobHeader), MI_BAD_ARGUMENT, "mi_a16_weight_import: truncated blob");
+  BlobHeader h;
+  memcpy(&h, blob, sizeof(h));
+  MI_REQUIRE(memcmp(h.magic, kBlobMagic, 8) == 0, MI_BAD_ARGUMENT, "mi_a16_weight_import: not a packed A16 weight blob");
+  MI_REQUIRE((h.bits == 4 || h.bits == 8) && h.K > 0 && h.N > 0 && h.G >= 1 &&
+                 (h.dtype == MI_DT_BF16 || h.dtype == MI_DT_F16),
+             MI_BAD_ARGUMENT, "mi_a16_weight_import: bad header");
+  const int tile_k = h.bits == 4 ? mi::W4_TILE_K : mi::W8_TILE_K;
+  MI_REQUIRE(h.row_blocks == (h.N + 15) / 16 && h.k_tiles == (h.K + tile_k - 1) / tile_k &&
+                 h.packed_bytes == (uint64_t)h.row_blocks * h.k_tiles * 1024 &&
+                 h.qparam_entries == (uint64_t)h.row_blocks * h.G * 16 && (h.g == 0 ? h.G == 1 : (int64_t)h.g * h.G == h.K),
+             MI_BAD_ARGUMENT, "mi_a16_weight_import: header fields disagree with each other");
+  MI_REQUIRE(group_size_supported(h.bits, h.g, h.K), MI_UNSUPPORTED, "mi_a16_weight_import: group size not handled");
+  MI_REQUIRE(size == sizeof(BlobHeader) + blob_payload(h), MI_BAD_ARGUMENT, "mi_a16_weight_import: size mismatch");
+  MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_a16_weight_import: no GPU visible");
+  mi_a16_weight *w = new (std::nothrow) mi_a16_weight();
+  MI_REQUIRE(w, MI_HIP_ERROR, "mi_a16_weight_import: out of host memory");
+  w->K = h.K;
+  w->N = h.N;
+  w->bits = h.bits;
+  w->g = h.g;
+  w->G = h.G;
+  w->dtype = h.dtype;
+  w->chip = h.chip;
+  w->row_blocks = h.row_blocks;
+  w->k_tiles = h.k_tiles;
+  const uint8_t *p = (const uint8_t *)blob + sizeof(h);
+  auto upload = [&](void **dst, size_t bytes) -> int {
+    MI_HIP(hipMalloc(dst, bytes));
+    MI_HIP(hipMemcpy(*dst, p, bytes, hipMemcpyHostToDevice));
+    p += bytes;
+    w->bytes += bytes;
+    return MI_SUCCESS;
+  };
+  int rc = upload(&w->qweight, h.packed_bytes);
+  if (rc == MI_SUCCESS && h.bits == 4)
+    rc = upload((void **)&w->sz_t, h.qparam_entries * 4);
+  if (rc == MI_SUCCESS && h.bits == 8)
+    rc = upload((void **)&w->scale_t, h.qparam_entries * 2);
+  if (rc == MI_SUCCESS && h.bits == 8)
+    rc = upload((void **)&w->nzs_t, h.qparam_entries * 4);
+  if (rc == MI_SUCCESS && h.has_bias)
+    rc = upload((void **)&w->bias, (size_t)h.N * 4);
+  if (rc != MI_SUCCESS) {
+    a16_free(w);
+    delete w;
+    return rc;
+  }
+  *out = w;
+  return MI_SUCCESS;
+}
+
+// ---- weight producers ----------------------------------------------------------------------------------------
+int mi_a16_quantize(const mi_a16_quant_desc *d, const float *w_kn, void *weight, uint16_t *scale16, float *scale_f32,
+                    uint8_t *zp, int *sign, int *weight_signed) {
+  MI_REQUIRE(d && w_kn && weight && scale16 && zp, MI_BAD_ARGUMENT, "mi_a16_quantize: null argument");
+  MI_REQUIRE(d->weight_bits == 4 || d->weight_bits == 8, MI_UNSUPPORTED, "mi_a16_quantize: weight_bits must be 4 or 8");
+  MI_REQUIRE(d->dtype == MI_DT_BF16 || d->dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_a16_quantize: dtype must be bf16 or f16");
+  MI_REQUIRE(d->K > 0 && d->N > 0 && (d->weight_bits == 8 || d->K % 2 == 0), MI_BAD_ARGUMENT, "mi_a16_quantize: bad shape");
+  const int64_t gs = d->q_group_size == -1 ? d->K : d->q_group_size;
+  MI_REQUIRE(gs >= 0 && (gs == 0 || d->K % gs == 0), MI_BAD_ARGUMENT, "mi_a16_quantize: K is not a multiple of q_group_size");
+  MI_REQUIRE(gs == 0 || d->K / gs <= 65535, MI_UNSUPPORTED, "mi_a16_quantize: more than 65535 groups per row");
+  MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_a16_quantize: no GPU visible");
+  return a16_quantize(d, w_kn, weight, scale16, scale_f32, zp, sign, weight_signed);
+}
+
+int mi_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qzeros, int64_t K, int64_t N, int64_t G,
+                  uint8_t *weight, uint8_t *zp) {
+  MI_REQUIRE(qweight && qzeros && weight && zp, MI_BAD_ARGUMENT, "mi_llm_unpack: null argument");
+  MI_REQUIRE(mode == MI_PACK_GPTQ || mode == MI_PACK_AWQ, MI_BAD_ARGUMENT, "mi_llm_unpack: mode");
+  MI_REQUIRE(bits == 4 || (bits == 8 && mode == MI_PACK_GPTQ), MI_UNSUPPORTED,
+             "mi_llm_unpack: 4-bit, or 8-bit GPTQ");
+  const int ratio = 32 / bits;
+  MI_REQUIRE(K > 0 && N > 0 && G > 0 && K % ratio == 0 && N % ratio == 0 && K % 2 == 0, MI_BAD_ARGUMENT,
+             "mi_llm_unpack: K and N must be multiples of the values per int32");
+  MI_REQUIRE(G <= 65535 && K <= 65535 * 2, MI_UNSUPPORTED, "mi_llm_unpack: shape too large");
+  MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_llm_unpack: no GPU visible");
+  return llm_unpack(mode, bits, qweight, qzeros, K, N, G, weight, zp);
+}
+
 int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                     void *stream) {
   return a16_launch(w, d_x, M, d_y, d_y_f32, (hipStream_t)stream);

@@ -71,6 +71,12 @@ int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
 int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
                      float *const *d_y32s, hipStream_t stream);
 
+// weight producers (quant_kernels.hip); arguments are validated by the callers
+int a16_quantize(const mi_a16_quant_desc *d, const float *h_w_kn, void *h_weight, uint16_t *h_scale16,
+                 float *h_scale_f32, uint8_t *h_zp, int *sign_out, int *weight_signed_out);
+int llm_unpack(int mode, int bits, const int32_t *h_qweight, const int32_t *h_qzeros, int64_t K, int64_t N, int64_t G,
+               uint8_t *h_weight, uint8_t *h_zp);
+
 int cast_launch(const mi_cast_attr *c, const void *d_in, void *d_out, int64_t n, float inv_scale, float scale,
                 bool f32_io, hipStream_t stream);
 

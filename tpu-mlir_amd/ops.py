@@ -207,6 +207,25 @@ class A16Weight:
     def nbytes(self):
         return clib.lib().mi_a16_weight_bytes(self.handle)
 
+    def export_blob(self):
+        """The packed set as bytes (header + tile-ordered arrays as they sit in HBM)."""
+        n = clib.lib().mi_a16_weight_export_size(self.handle)
+        buf = np.empty(n, dtype=np.uint8)
+        check(clib.lib().mi_a16_weight_export(self.handle, buf.ctypes.data, n))
+        return buf
+
+    @classmethod
+    def from_blob(cls, blob):
+        """Uploads a blob written by export_blob(); no repacking."""
+        blob = np.ascontiguousarray(np.frombuffer(blob, dtype=np.uint8))
+        self = cls.__new__(cls)
+        self.handle = C.c_void_p()
+        check(clib.lib().mi_a16_weight_import(C.byref(self.handle), blob.ctypes.data, blob.size))
+        hdr = np.frombuffer(blob[8:40].tobytes(), dtype=np.int64)
+        self.K, self.N = int(hdr[0]), int(hdr[1])
+        self.dtype = int(np.frombuffer(blob[52:56].tobytes(), dtype=np.int32)[0])
+        return self
+
     def destroy(self):
         if self.handle:
             clib.lib().mi_a16_weight_destroy(self.handle)
@@ -217,6 +236,53 @@ class A16Weight:
             self.destroy()
         except Exception:
             pass
+
+
+PACK_GPTQ, PACK_AWQ = 0, 1
+
+
+def a16_quantize(w_kn, *, weight_bits, q_group_size, symmetric=False, dtype=DT_BF16):
+    """A16MatMulAdjust on the GPU: f32 weight [K, N] of a top-level matmul -> the operand set of tpu.A16MatMul.
+
+    Returns dict(weight uint8/int8 [N, K/2] or [N, K], scale_bits uint16 [N, G], scale_f32 [N, G], zp uint8 [N, G],
+    sign, weight_signed); weight/scale_bits/zp are what A16Weight takes.
+    """
+    w = np.ascontiguousarray(w_kn, dtype=np.float32)
+    if w.ndim != 2:
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16_quantize: weight must be [K, N]")
+    K, N = w.shape
+    gs = K if q_group_size == -1 else q_group_size
+    if gs < 0 or (gs and K % gs):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16_quantize: K is not a multiple of q_group_size")
+    G = K // gs if gs else 1
+    q = np.zeros((N, K // 2 if weight_bits == 4 else K), dtype=np.uint8)
+    s16 = np.zeros((N, G), dtype=np.uint16)
+    sf = np.zeros((N, G), dtype=np.float32)
+    zp = np.zeros((N, G), dtype=np.uint8)
+    sign, wsigned = C.c_int(0), C.c_int(0)
+    desc = clib.A16QuantDesc(K, N, weight_bits, q_group_size, int(symmetric), dtype)
+    check(clib.lib().mi_a16_quantize(C.byref(desc), w.ctypes.data, q.ctypes.data, s16.ctypes.data, sf.ctypes.data,
+                                     zp.ctypes.data, C.byref(sign), C.byref(wsigned)))
+    if wsigned.value:
+        q = q.view(np.int8)
+    return dict(weight=q, scale_bits=s16, scale_f32=sf, zp=zp, sign=bool(sign.value),
+                weight_signed=bool(wsigned.value))
+
+
+def llm_unpack(mode, bits, qweight, qzeros, *, K, N):
+    """GPTQ / AWQ int32 checkpoint tensors -> (weight uint8 [N, K/2] or [N, K], zp uint8 [N, G]) on the GPU."""
+    qweight = np.ascontiguousarray(qweight, dtype=np.int32)
+    qzeros = np.ascontiguousarray(qzeros, dtype=np.int32)
+    ratio = 32 // bits
+    want = (K // ratio, N) if mode == PACK_GPTQ else (K, N // ratio)
+    if qweight.shape != want or qzeros.ndim != 2 or qzeros.shape[1] != N // ratio:
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "llm_unpack: tensor shapes do not match K, N and the mode")
+    G = qzeros.shape[0]
+    q = np.zeros((N, K // 2 if bits == 4 else K), dtype=np.uint8)
+    zp = np.zeros((N, G), dtype=np.uint8)
+    check(clib.lib().mi_llm_unpack(mode, bits, qweight.ctypes.data, qzeros.ctypes.data, K, N, G, q.ctypes.data,
+                                   zp.ctypes.data))
+    return q, zp
 
 
 def a16mm_launch(w, x, y=None, y_f32=None, stream=None):
