@@ -11,6 +11,11 @@
 //   4-bit: P = sum_k a_k (16 + q_k) by MFMA, S = sum_k a_k by one more MFMA against ones, then
 //          acc += scale * (P - (16 + zp) * S) in fp32.
 //   8-bit: the weight is rounded to the 16-bit type exactly as the reference does, and the MFMA accumulates directly.
+#include <algorithm>
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "a16_common.cuh"
 #include "internal.h"
 
@@ -49,6 +54,10 @@ struct GemmArgs {
   int tiles_per_group;  // GPT == 1: weight tiles that share one group (g / TILE_K; k_tiles when per channel)
   int chip;
   int tiles_m, tiles_n, per_xcd;
+  // split K: each output block is computed by k_splits workgroups over kt_per_split stages each, which add their
+  // fp32 partial sums into acc [M, N] (zero on entry); bias and rounding happen in a16_gemm_finish_kernel
+  int k_splits, kt_per_split;
+  float *acc;
 };
 
 // WM x WN waves, each TM x TN MFMA tiles of 16 x 16:  GM = WM * TM * 16 rows, GN = WN * TN * 16 columns.
@@ -84,9 +93,11 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
   // workgroup -> output block: the hardware deals workgroups round-robin over the 8 XCDs; each XCD gets a contiguous
   // run of the block order (column-major inside groups of 4 block-rows) so that its L2 sees few distinct panels
   const int bid = blockIdx.x;
-  const int L = (bid & 7) * a.per_xcd + (bid >> 3);
-  if (L >= a.tiles_m * a.tiles_n)
+  const int Ls = (bid & 7) * a.per_xcd + (bid >> 3);
+  if (Ls >= a.tiles_m * a.tiles_n * a.k_splits)
     return;
+  const int L = a.k_splits == 1 ? Ls : Ls / a.k_splits;
+  const int split = Ls - L * a.k_splits;
   constexpr int GRP = 4;
   const int group = L / (GRP * a.tiles_n);
   const int gm = (a.tiles_m - group * GRP) < GRP ? (a.tiles_m - group * GRP) : GRP;
@@ -106,7 +117,10 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
     m = m < a.M ? m : a.M - 1;  // rows past M re-read the last row; their results are never stored
     gx[i] = a.x + m * a.K + chunk * 8;
   }
-  const int kt_total = (int)(a.K / GEMM_KS);
+  // this workgroup's stages: [kt0, kt0 + kt_total) of the K / GEMM_KS stages of the whole product
+  const int kt_all = (int)(a.K / GEMM_KS);
+  const int kt0 = split * a.kt_per_split;
+  const int kt_total = (kt_all - kt0) < a.kt_per_split ? (kt_all - kt0) : a.kt_per_split;
   // this wave's share of the weight tiles of the block, and the scale|zp words of its own columns (lane l fetches
   // channel l & 15 of its row block (l >> 4) % TN)
   int64_t w_tile_rb[WL > 0 ? WL : 1];
@@ -129,7 +143,7 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
     return gi < a.G ? gi : a.G - 1;
   };
   auto issue_x = [&](int kt) {
-    const int ktc = kt < kt_total ? kt : kt_total - 1;  // past the end: harmless re-load
+    const int ktc = kt0 + (kt < kt_total ? kt : kt_total - 1);  // past the end: harmless re-load
     const int64_t koff = (int64_t)ktc * GEMM_KS;
     uint8_t *st = lds + (kt % GEMM_NST) * STAGE_BYTES;
 #pragma unroll
@@ -171,7 +185,7 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
     }
   }
   auto load_w = [&](WStage &s, int kt) {  // 8-bit: global -> registers, issued one stage ahead
-    const int ktc = kt < kt_total ? kt : kt_total - 1;
+    const int ktc = kt0 + (kt < kt_total ? kt : kt_total - 1);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
 #pragma unroll
@@ -332,7 +346,9 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int64_t m = m_base + (wm * TM + i) * 16 + 4 * kq + r;
-        if (n_ok && m < a.M) {
+        if (n_ok && m < a.M && a.acc) {
+          atomicAdd(a.acc + m * a.N + n, acc[i][j][r]);  // bias and rounding: a16_gemm_finish_kernel
+        } else if (n_ok && m < a.M) {
           const float v = acc[i][j][r] + b;
           const int64_t o = m * a.N + n;
           if (a.y32)
@@ -343,12 +359,91 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
   }
 }
 
+// Second half of a split-K product: y = round16(acc + bias) (and the fp32 value, if asked for), and acc goes back to
+// zero so that the next product on this stream finds it clean.
+template <int DT>
+__global__ void a16_gemm_finish_kernel(float *__restrict__ acc, const float *__restrict__ bias, uint16_t *__restrict__ y,
+                                       float *__restrict__ y32, int64_t total, int64_t N, int chip) {
+  const int64_t i4 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i4 >= total)
+    return;
+  const f32x4 v4 = *(const f32x4 *)(acc + i4);  // N % 4 == 0 (checked by the host): a group of 4 stays in one row
+  *(f32x4 *)(acc + i4) = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int64_t n = i4 % N;
+  uint16_t h[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float v = v4[e] + (bias ? bias[n + e] : 0.0f);
+    if (y32)
+      y32[i4 + e] = v;
+    h[e] = (chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+  }
+  *(u32x2 *)(y + i4) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+}
+
+// fp32 partial-sum buffers of split-K products, one per (device, stream): a product leaves its buffer zeroed, products
+// on one stream are ordered, and products on different streams never share a buffer.  A buffer only grows; it is
+// allocated (and cleared) on first use, i.e. never inside a captured graph whose first run was eager.
+namespace {
+struct SplitBuf {
+  float *ptr = nullptr;
+  size_t elems = 0;
+};
+std::mutex g_split_mutex;
+std::map<std::pair<int, hipStream_t>, SplitBuf> g_split_bufs;
+
+int split_buffer(hipStream_t st, size_t elems, float **out) {
+  int dev = 0;
+  MI_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_split_mutex);
+  SplitBuf &b = g_split_bufs[{dev, st}];
+  if (b.elems < elems) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(st, &cs);
+    MI_REQUIRE(cs == hipStreamCaptureStatusNone, MI_HIP_ERROR,
+               "a16 split-K product: its partial-sum buffer must exist before the stream is captured (run the same "
+               "shape once eagerly first)");
+    if (b.ptr) {
+      MI_HIP(hipStreamSynchronize(st));
+      MI_HIP(hipFree(b.ptr));
+      b.ptr = nullptr;
+      b.elems = 0;
+    }
+    MI_HIP(hipMalloc((void **)&b.ptr, elems * sizeof(float)));
+    MI_HIP(hipMemset(b.ptr, 0, elems * sizeof(float)));
+    b.elems = elems;
+  }
+  *out = b.ptr;
+  return MI_SUCCESS;
+}
+}  // namespace
+
 template <int BITS, int DT, int GPT, int WM, int WN, int TM, int TN>
-static void launch_gemm_instance(GemmArgs &a, hipStream_t st) {
+static int launch_gemm_instance(GemmArgs &a, hipStream_t st) {
   constexpr int GM = WM * TM * 16, GN = WN * TN * 16;
   a.tiles_m = (int)((a.M + GM - 1) / GM);
   a.tiles_n = (int)((a.N + GN - 1) / GN);
-  a.per_xcd = (a.tiles_m * a.tiles_n + 7) / 8;
+  // split K when the output blocks alone leave most of the 256 CUs idle: enough workgroups for one per CU, at least
+  // four stages each
+  const int tiles = a.tiles_m * a.tiles_n;
+  const int kt_all = (int)(a.K / GEMM_KS);
+  int splits = 1;
+  const char *e = getenv("MI_A16_GEMM_SPLITS");  // development switch
+  if (e)
+    splits = atoi(e);
+  else if (tiles < 160 && (a.N % 4) == 0)
+    splits = std::min(std::max(256 / tiles, 1), std::max(kt_all / 4, 1));
+  splits = std::max(1, std::min(splits, kt_all));
+  a.kt_per_split = (kt_all + splits - 1) / splits;
+  a.k_splits = (kt_all + a.kt_per_split - 1) / a.kt_per_split;  // no empty split
+  a.acc = nullptr;
+  if (a.k_splits > 1) {
+    MI_REQUIRE((a.N % 4) == 0, MI_BAD_ARGUMENT, "a16 split-K product: N must be a multiple of 4");
+    int rc = split_buffer(st, (size_t)a.M * a.N, &a.acc);
+    if (rc != MI_SUCCESS)
+      return rc;
+  }
+  a.per_xcd = (tiles * a.k_splits + 7) / 8;
   auto kfn = a16_gemm_kernel<BITS, DT, GPT, WM, WN, TM, TN>;
   const size_t lds_bytes = (size_t)GEMM_NST * (GM * GEMM_KS * 2 + (BITS == 4 ? (GN / 16) * 1024 + GEMM_WAVES * GPT * 256 : 0));
   static bool attr_set = false;
@@ -357,23 +452,34 @@ static void launch_gemm_instance(GemmArgs &a, hipStream_t st) {
     attr_set = true;
   }
   kfn<<<dim3((unsigned)(a.per_xcd * 8)), dim3(GEMM_WAVES * 64), lds_bytes, st>>>(a);
+  if (a.k_splits > 1) {
+    const int64_t total = (int64_t)a.M * a.N;
+    a16_gemm_finish_kernel<DT><<<dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, st>>>(a.acc, a.bias, a.y, a.y32,
+                                                                                             total, a.N, a.chip);
+  }
+  return MI_SUCCESS;
 }
 
 template <int BITS, int DT, int GPT>
-static void launch_gemm_shape(GemmArgs &a, hipStream_t st) {
+static int launch_gemm_shape(GemmArgs &a, hipStream_t st) {
   // 128 x 256 blocks when they fill the chip, else 128 x 128
   const int64_t big = ((a.M + 127) / 128) * ((a.N + 255) / 256);
   const char *e = getenv("MI_A16_GEMM_TILE");  // development switch: "256" / "128"
   constexpr bool fits = !(BITS == 4 && GPT == 4);  // 32-wide groups: a 256-column block's scale|zp words overflow LDS
   const bool wide = fits && (e ? atoi(e) == 256 : big >= 192);
   if constexpr (fits) {
-    if (wide) {
-      launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 4>(a, st);
-      return;
-    }
+    if (wide)
+      return launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 4>(a, st);
   }
   (void)wide;
-  launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 2>(a, st);
+  // few rows: shorter blocks waste fewer MFMAs on rows that do not exist
+  const char *r = getenv("MI_A16_GEMM_ROWS");  // development switch: "32" / "64" / "128"
+  const int rows = r ? atoi(r) : (a.M <= 32 ? 32 : a.M <= 640 ? 64 : 128);  // measured: 64-row blocks win up to there
+  if (rows == 32)
+    return launch_gemm_instance<BITS, DT, GPT, 2, 4, 1, 2>(a, st);
+  if (rows == 64)
+    return launch_gemm_instance<BITS, DT, GPT, 2, 4, 2, 2>(a, st);
+  return launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 2>(a, st);
 }
 
 bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M) {
@@ -383,9 +489,9 @@ bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M) {
   const int g = w->g;
   // whole LDS stages, at most one group per MFMA k-step, groups that do not straddle a weight tile
   const bool group_ok = g == 0 || (g >= tile_k && g % tile_k == 0) || (g < tile_k && tile_k % g == 0 && g >= 32);
-  // below about 160 rows the skinny kernel (one pass over the weights per 16 rows) is still faster
+  // up to 16 rows the skinny kernel makes one pass over the weights; beyond that it would make one per 16 rows
   const char *e = getenv("MI_A16_GEMM_MIN_M");  // development / test switch
-  const int64_t min_m = e ? atoll(e) : 160;
+  const int64_t min_m = e ? atoll(e) : 17;
   return M >= min_m && M > 16 && (w->K % GEMM_KS) == 0 && group_ok;
 }
 
@@ -417,12 +523,13 @@ int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
   else
     gpt = tile_k / w->g;
   const bool f16 = w->dtype == MI_DT_F16;
+  int rc = MI_SUCCESS;
 #define MI_GEMM(BITS_, GPT_)                                      \
   {                                                               \
     if (f16)                                                      \
-      launch_gemm_shape<BITS_, MI_DT_F16, GPT_>(a, stream);       \
+      rc = launch_gemm_shape<BITS_, MI_DT_F16, GPT_>(a, stream);  \
     else                                                          \
-      launch_gemm_shape<BITS_, MI_DT_BF16, GPT_>(a, stream);      \
+      rc = launch_gemm_shape<BITS_, MI_DT_BF16, GPT_>(a, stream); \
   }
   if (w->bits == 4) {
     if (gpt == 1)
@@ -438,6 +545,8 @@ int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
       MI_GEMM(8, 2)
   }
 #undef MI_GEMM
+  if (rc != MI_SUCCESS)
+    return rc;
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;
 }
