@@ -97,6 +97,16 @@ def test_prefill_gemm_device_level(orc, monkeypatch, bits, M, K, N, g, signed, t
     _check_against_oracle(orc, cfg, out, pre)
 
 
+@pytest.mark.parametrize("bits,M,K,N,g", [(4, 8, 1024, 272, 128), (4, 16, 512, 130, 64), (4, 2, 2048, 128, 0),
+                                         (8, 5, 512, 96, 128), (8, 13, 1024, 200, 0)])
+def test_tiled_kernel_sixteen_row_blocks(orc, monkeypatch, bits, M, K, N, g):
+    """At most 16 rows through the tiled kernel (what large matrices take from 8 rows on)."""
+    monkeypatch.setenv("MI_A16_GEMM_MIN_M", "2")
+    cfg = S.w4a16(M, K, N, g, seed=M + N, bias=(N % 8 == 0)) if bits == 4 else S.w8a16(M, K, N, g, seed=M + N)
+    out, pre = _run_device(cfg)
+    _check_against_oracle(orc, cfg, out, pre)
+
+
 @pytest.mark.parametrize("bits,M,K,N,g", [(4, 64, 4096, 256, 128), (4, 130, 2048, 512, 64), (8, 48, 2048, 384, 128)])
 def test_prefill_gemm_split_k(orc, monkeypatch, bits, M, K, N, g):
     """Few output blocks, long K: the product is split along K over several workgroups (fp32 atomics + a finishing

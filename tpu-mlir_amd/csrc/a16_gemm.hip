@@ -73,7 +73,10 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
   constexpr int UNITS = BITS == 4 ? GPT : WT * GPT;    // quantization groups per stage
   constexpr int KSTEPS_PER_UNIT = KSTEPS / UNITS;
   constexpr bool WLDS = BITS == 4;                     // weights and group parameters through the LDS ring
-  constexpr int X_BYTES = GM * GEMM_KS * 2;
+  // activation rows per stage: at least 32, so that every thread has one 16-byte request (a 16-row block re-reads its
+  // rows; fragments only ever read the first GM)
+  constexpr int XROWS = GM < 32 ? 32 : GM;
+  constexpr int X_BYTES = XROWS * GEMM_KS * 2;
   constexpr int W_BYTES = WLDS ? (GN / 16) * 1024 : 0;         // one 1 KiB tile per 16 output channels
   constexpr int SZ_BYTES = WLDS ? GEMM_WAVES * GPT * 256 : 0;  // per wave and group: 64 scale|zp words
   constexpr int STAGE_BYTES = X_BYTES + W_BYTES + SZ_BYTES;
@@ -445,7 +448,8 @@ static int launch_gemm_instance(GemmArgs &a, hipStream_t st) {
   }
   a.per_xcd = (tiles * a.k_splits + 7) / 8;
   auto kfn = a16_gemm_kernel<BITS, DT, GPT, WM, WN, TM, TN>;
-  const size_t lds_bytes = (size_t)GEMM_NST * (GM * GEMM_KS * 2 + (BITS == 4 ? (GN / 16) * 1024 + GEMM_WAVES * GPT * 256 : 0));
+  const size_t lds_bytes =
+      (size_t)GEMM_NST * ((GM < 32 ? 32 : GM) * GEMM_KS * 2 + (BITS == 4 ? (GN / 16) * 1024 + GEMM_WAVES * GPT * 256 : 0));
   static bool attr_set = false;
   if (!attr_set) {
     (void)hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -474,7 +478,9 @@ static int launch_gemm_shape(GemmArgs &a, hipStream_t st) {
   (void)wide;
   // few rows: shorter blocks waste fewer MFMAs on rows that do not exist
   const char *r = getenv("MI_A16_GEMM_ROWS");  // development switch: "32" / "64" / "128"
-  const int rows = r ? atoi(r) : (a.M <= 32 ? 32 : a.M <= 640 ? 64 : 128);  // measured: 64-row blocks win up to there
+  const int rows = r ? atoi(r) : (a.M <= 16 ? 16 : a.M <= 32 ? 32 : a.M <= 640 ? 64 : 128);  // measured: 64-row blocks win up to there
+  if (rows == 16)
+    return launch_gemm_instance<BITS, DT, GPT, 1, 8, 1, 1>(a, st);
   if (rows == 32)
     return launch_gemm_instance<BITS, DT, GPT, 2, 4, 1, 2>(a, st);
   if (rows == 64)
@@ -489,10 +495,17 @@ bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M) {
   const int g = w->g;
   // whole LDS stages, at most one group per MFMA k-step, groups that do not straddle a weight tile
   const bool group_ok = g == 0 || (g >= tile_k && g % tile_k == 0) || (g < tile_k && tile_k % g == 0 && g >= 32);
-  // up to 16 rows the skinny kernel makes one pass over the weights; beyond that it would make one per 16 rows
+  // Up to 16 rows the skinny kernel makes one pass over the weights; beyond that it would make one per 16 rows.  From
+  // 8 rows on, large matrices are already better off here (measured with weights streaming from HBM: 11008 x 4096 at
+  // M = 8: 13.0 us against 14.8; 4096 x 4096: 8.1 against 7.5), because a workgroup of the skinny kernel stages all of
+  // x in LDS and runs at low occupancy once x has several rows.
   const char *e = getenv("MI_A16_GEMM_MIN_M");  // development / test switch
-  const int64_t min_m = e ? atoll(e) : 17;
-  return M >= min_m && M > 16 && (w->K % GEMM_KS) == 0 && group_ok;
+  bool rows_ok;
+  if (e)
+    rows_ok = M >= atoll(e) && M > 1;
+  else
+    rows_ok = M >= 17 || (M >= 8 && w->N * w->K >= (int64_t(1) << 25));
+  return rows_ok && (w->K % GEMM_KS) == 0 && group_ok;
 }
 
 int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
