@@ -210,6 +210,30 @@ def bench_single_matmuls(pkg, S, torch, steps=60):
     return out
 
 
+def bench_dynamic_quant(pkg, S, torch, steps=40):
+    """tpu.A16MatMul with dynamic integer activation quantization (activation quantizer + integer product per call),
+    weights rotating through HBM; eager launches (the call allocates its code buffers on the stream)."""
+    out = []
+    for M, K, N, copies in ((1, 4096, 4096, 32), (16, 4096, 4096, 32), (1, 4096, 11008, 12), (128, 4096, 4096, 32)):
+        cfg = S.w4a16(1, K, N, 128, seed=33)
+        ws = [pkg.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=K, N=N, weight_bits=4, q_group_size=128)
+              for _ in range(copies)]
+        x = _dev_bf16(torch, S.bf16_round(np.random.default_rng(6).standard_normal((M, K), dtype=np.float32)))
+        y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+
+        def run():
+            for w in ws:
+                pkg.a16mm_dq_launch(w, x, y)
+
+        sec = _time_launches(torch, run, max(3, steps // copies), warmup=2) / copies
+        nbytes = S.w4_gemv_bytes(M, K, N, 128)
+        out.append({"case": "w4_g128_dynamic_int", "M": M, "K": K, "N": N, "us": round(sec * 1e6, 2),
+                    "GBps": round(nbytes / sec / 1e9, 1)})
+        for w in ws:
+            w.destroy()
+    return out
+
+
 def bench_operator_boundary(pkg, S, steps=20):
     """The same q_proj GEMV through the reference's operator interface (float32-expanded host tensors in and out,
     like InferenceParameter): includes the host<->device copies and conversions, so it is NOT a roofline figure."""
@@ -367,6 +391,7 @@ def main():
             rm = bench_chain(pkg, S, torch, m, 40, 5, args.layers, cm, grouped=not args.no_group)
             ex["chain_M%d_GBps" % m] = round(rm["chain_bytes"] / (rm["gpu_s"] / 40) / 1e9, 1)
         ex["single_matmuls"] = bench_single_matmuls(pkg, S, torch)
+        ex["dynamic_quant"] = bench_dynamic_quant(pkg, S, torch)
         ex["int8_256x1024x1024"] = bench_int8(pkg, S, torch, clib, 1024, 40, 5, M=256)
         ex["operator_boundary"] = bench_operator_boundary(pkg, S)
         ex["device_resident_block"] = bench_module_block(pkg, S, clib, cfgs)

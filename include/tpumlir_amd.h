@@ -79,6 +79,10 @@ typedef struct mi_infer_param {
 /* ============================================================================ */
 /* tpu.A16MatMul  (lib/Dialect/Tpu/Interfaces/Common/A16MatMul.cpp:16-249)       */
 /* ============================================================================ */
+/* dynamic activation quantization of tpu.A16MatMul (A16MatMul.cpp:40-170): MI_DQ_INT covers dq_type "INT4" and
+ * "INT8", whose arithmetic differs only through the weight width (imax = 2^(weight_bits-1) - 1, :53-54) */
+enum { MI_DQ_NONE = 0, MI_DQ_INT = 1, MI_DQ_F8E4M3 = 2, MI_DQ_F4 = 3 };
+
 typedef struct mi_a16mm_attr {
   int64_t M;            /* product of the input's leading dims (A16MatMul.cpp:31-35); may change per call */
   int64_t K, N;         /* input [M,K], output [M,N]; weight holds N output channels */
@@ -87,7 +91,8 @@ typedef struct mi_a16mm_attr {
   int q_group_size;     /* getQGroupSize() or module::getQuantGroupSize(); 0 = per output channel */
   int out_dtype;        /* MI_DT_BF16, or MI_DT_F16 when module::isF16Modes() */
   int chip;             /* MI_CHIP_* */
-  int dynamic_quant;    /* module::isDynamicQuantize(): not handled, returns MI_UNSUPPORTED */
+  int dynamic_quant;    /* MI_DQ_*: module::isDynamicQuantize() and getDqType().  MI_DQ_INT with 4-bit weights,
+                         * K % 128 == 0 and groups of 64 or k*128 is handled; anything else is MI_UNSUPPORTED */
 } mi_a16mm_attr;
 
 /* Replaces tpu::A16MatMulOp::init (A16MatMul.cpp:16-18).  inputs = {input, weight, scale, zp, bias|NULL}.
@@ -163,6 +168,11 @@ int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
  * A16MatMulOp::inference (A16MatMul.cpp:150-273).  Results are identical to n calls of mi_a16mm_launch.  The sets
  * must agree in K, weight_bits, q_group_size, dtype and chip; N may differ.  d_y[i] / d_y_f32[i] as above
  * (d_y_f32 itself may be NULL, as may any of its entries). */
+/* The dynamic-quantization flavour of the same product (A16MatMul.cpp:40-170, integer dq types, 4-bit weights):
+ * activations are quantized per row and group to [-7, 7], the group products are integer MFMA sums, and the groups
+ * are added in the reference's order -- results are bit-identical to the reference's. */
+int mi_a16mm_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
+                       void *stream);
 int mi_a16mm_launch_group(const mi_a16_weight *const *w, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_y,
                           float *const *d_y_f32, void *stream);
 

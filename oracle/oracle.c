@@ -525,6 +525,86 @@ int orc_a16matmul(const orc_a16mm_attr *a, const float *const *inputs,
   return 0;
 }
 
+/* A16MatMul.cpp:40-170 (module::isDynamicQuantize()), dq_type INT4 / INT8, w_transpose */
+int orc_a16matmul_dynamic(const orc_a16mm_attr *a, const float *const *inputs, float *output, float *y_preround) {
+  if (!a || !inputs || !inputs[0] || !inputs[1] || !inputs[2] || !inputs[3])
+    return 1;
+  if ((a->weight_bits != 4 && a->weight_bits != 8) || !a->w_transpose)
+    return 1;
+  const int64_t M = a->M, K = a->K, N = a->N;
+  int64_t g = a->q_group_size;
+  if (!g)
+    return 1; /* :42-43 */
+  if (g == -1)
+    g = K; /* :47-49 with w_transpose (the row length of the [N, K] weight) */
+  const float imax = (float)((1 << (a->weight_bits - 1)) - 1); /* :53-54 */
+  const float *x = inputs[0], *weight = inputs[1], *scale = inputs[2], *zp = inputs[3], *bias = inputs[4];
+  const int64_t group_num = (K + g - 1) / g;
+  /* :63-91 integer weight minus zero point, [N, K] */
+  float *nw = (float *)malloc(sizeof(float) * (size_t)(N * K));
+  float *act = (float *)malloc(sizeof(float) * (size_t)(M * g));
+  float *amax = (float *)malloc(sizeof(float) * (size_t)M);
+  if (!nw || !act || !amax) {
+    free(nw);
+    free(act);
+    free(amax);
+    return 1;
+  }
+  for (int64_t i = 0; i < N * K; i++) {
+    const float z = zp[i / g];
+    if (a->weight_bits == 4) {
+      const int b = (int)weight[i / 2];
+      nw[i] = (float)((i & 1) ? (b >> 4) : (b & 0x0F)) - z;
+    } else {
+      nw[i] = (float)(int)weight[i] - z;
+    }
+  }
+  for (int64_t i = 0; i < M * N; i++)
+    output[i] = 0.0f; /* the interpreter hands over a zeroed buffer; the op only ever adds to it */
+  int inexact = 0;
+  for (int64_t gi = 0; gi < group_num; gi++) {
+    /* :98-108 */
+    for (int64_t row = 0; row < M; row++) {
+      amax[row] = (float)1e-8;
+      for (int64_t col = 0; col < g; col++)
+        if (gi * g + col < K) {
+          const float v = fabsf(x[row * K + gi * g + col]);
+          amax[row] = amax[row] > v ? amax[row] : v;
+        }
+    }
+    /* :109-132 */
+    for (int64_t row = 0; row < M; row++)
+      for (int64_t col = 0; col < g; col++)
+        act[row * g + col] = (gi * g + col < K) ? roundf(x[row * K + gi * g + col] / amax[row] * imax) : 0.0f;
+    /* :133-160: group product (integer-valued operands), then the rescaled accumulation in row-major order */
+    for (int64_t row = 0; row < M; row++)
+      for (int64_t col = 0; col < N; col++) {
+        int64_t s = 0, peak = 0;
+        for (int64_t k = 0; k < g && gi * g + k < K; k++) {
+          s += (int64_t)act[row * g + k] * (int64_t)nw[col * K + gi * g + k];
+          const int64_t m = s < 0 ? -s : s;
+          peak = m > peak ? m : peak;
+        }
+        if (peak >= (1 << 24))
+          inexact = 1;
+        float *o = output + row * N + col;
+        *o += (float)s * (amax[row] / imax) * scale[col * group_num + gi];
+        if (gi == 0 && bias)
+          *o += bias[col];
+      }
+  }
+  free(nw);
+  free(act);
+  free(amax);
+  if (inexact)
+    return 2;
+  if (y_preround)
+    memcpy(y_preround, output, sizeof(float) * (size_t)(M * N));
+  for (int64_t i = 0; i < M * N; i++)
+    output[i] = round_out(output[i], a->out_dtype, a->is_cv18xx); /* :161-166 */
+  return 0;
+}
+
 /* ======================================================================== */
 /* tpu.MatMul (quantised)                                                    */
 /* ======================================================================== */

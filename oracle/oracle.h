@@ -24,6 +24,8 @@
  *   orc_f32_to_bf16 (cvi)        add-0x7fff+lsb closed form, inf->0x7f7f
  *   orc_f32_to_f16               numpy float16 RNE incl. subnormals
  *   orc_cast                     numpy closed forms per branch (tests/test_oracle_cast.py)
+ *   orc_a16matmul_dynamic        lossless-activation cases against orc_a16matmul, exact power-of-two row
+ *                                scaling, half-step error bound, group order (tests/test_oracle_dynamic.py)
  *   orc_a16_quantize             on-grid weights are recovered exactly, |w - dequant(q)| <= scale/2 inside the
  *                                clamp range, closed-form scale/zp, nibble order via the A16MatMul dequantizer
  *                                (tests/test_oracle_packers.py)
@@ -212,6 +214,15 @@ typedef struct {
 } orc_cast_attr;
 /* returns 0, or -1 for a branch this restatement leaves out (CV18xx, fp8) */
 int orc_cast(const orc_cast_attr *attr, const float *input, float *output, int64_t n);
+
+/* ---- tpu.A16MatMul with dynamic activation quantization (INT4 / INT8) -------- */
+/* lib/Dialect/Tpu/Interfaces/Common/A16MatMul.cpp:40-170, w_transpose weights, dq_type "INT4" (4-bit weights,
+ * imax 7) or "INT8" (8-bit weights, imax 127): per row and per group of K the activation is scaled by its own
+ * abs-max to integers in [-imax, imax]; the group products are integer sums (exact in the reference's f32 sgemm
+ * while they stay below 2^24 -- this restatement returns 2 instead of a result when they do not), rescaled and
+ * added group by group in fp32, bias after the first group.  inputs as for orc_a16matmul; the 8-bit weight is
+ * read as the reference reads it, `int(weight[i])`.  Returns 0, 1 (bad arguments), 2 (outside the exact domain). */
+int orc_a16matmul_dynamic(const orc_a16mm_attr *a, const float *const *inputs, float *output, float *y_preround);
 
 /* ---- weight producers (compile-time side of tpu.A16MatMul) ------------------- */
 /* A16MatMulAdjust, lib/Dialect/Tpu/Canonicalize/A16MatMul.cpp:270-429, static uint8-zero-point variant:

@@ -209,6 +209,23 @@ def a16matmul(x, weight, scale, zp, bias, *, M, K, N, weight_bits, q_group_size,
     return out, pre
 
 
+def a16matmul_dynamic(x, weight, scale, zp, bias, *, M, K, N, weight_bits, q_group_size, out_dtype=OUT_BF16):
+    """tpu.A16MatMul with dynamic INT4 / INT8 activation quantization; returns (output, pre-rounding f32)."""
+    ins = [_f32(x), _f32(weight), _f32(scale), _f32(zp), _f32(bias)]
+    attr = A16Attr(M, K, N, weight_bits, 1, q_group_size, out_dtype, 0, GEMM_F64ACC)
+    arr = (C.POINTER(C.c_float) * 5)(*[None if a is None else _p(a, C.c_float) for a in ins])
+    out = np.empty((M, N), dtype=np.float32)
+    pre = np.empty((M, N), dtype=np.float32)
+    L = lib()
+    L.orc_a16matmul_dynamic.restype = C.c_int
+    rc = L.orc_a16matmul_dynamic(C.byref(attr), arr, _p(out, C.c_float), _p(pre, C.c_float))
+    if rc == 2:
+        raise ValueError("orc_a16matmul_dynamic: group sums leave the range the reference's f32 product is exact in")
+    if rc != 0:
+        raise RuntimeError("orc_a16matmul_dynamic failed")
+    return out, pre
+
+
 def matmul_int8(x, right, bias, multi, *, M, K, N, right_transpose=False, input_zp=0, right_zp=0,
                 do_relu=False, relu_limit=-1.0, cv18xx=False, quant_mode=RQ_MULTIPLIER_SHIFT, fuse_rq=False,
                 multipliers=(1,), rshifts=(0,), out_zp=0, out_kind=0, out_bits=8, out_unsigned=False,

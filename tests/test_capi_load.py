@@ -31,7 +31,9 @@ def test_argument_errors_need_no_gpu():
     w = np.zeros((4, 64), np.float32)
     s = np.ones((4, 1), np.float32)
     z = np.zeros((4, 1), np.float32)
-    for kw, code in ((dict(dynamic_quant=True), clib.MI_UNSUPPORTED),
+    for kw, code in ((dict(dynamic_quant=clib.DQ_F8E4M3, q_group_size=64), clib.MI_UNSUPPORTED),
+                     (dict(dynamic_quant=clib.DQ_INT), clib.MI_BAD_ARGUMENT),        # no group size
+                     (dict(dynamic_quant=clib.DQ_INT, q_group_size=32), clib.MI_UNSUPPORTED),
                      (dict(w_transpose=False), clib.MI_UNSUPPORTED),
                      (dict(weight_bits=3), clib.MI_UNSUPPORTED),
                      (dict(q_group_size=48), clib.MI_BAD_ARGUMENT),      # K % g != 0

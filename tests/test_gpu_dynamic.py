@@ -1,0 +1,85 @@
+"""GPU parity of tpu.A16MatMul with dynamic integer activation quantization (A16MatMul.cpp:40-170) against the CPU
+oracle, through the C ABI.  The reference fixes every operation and its order on this path, so the bar is
+bit-exact: the fp32 value before output rounding and the 16-bit output."""
+import numpy as np
+import pytest
+
+from helpers import pkg, f32_valued_a16
+
+pytestmark = pytest.mark.gpu
+
+M_ = pkg()
+S = pkg("synth")
+clib = pkg("clib")
+
+
+def _device(cfg, dtype=clib.DT_BF16):
+    import torch
+    tdt = torch.bfloat16 if dtype == clib.DT_BF16 else torch.float16
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"],
+                     None if cfg.get("bias") is None else S.bf16_to_f32(cfg["bias"]),
+                     K=cfg["K"], N=cfg["N"], weight_bits=4, q_group_size=cfg["g"], dtype=dtype)
+    x = torch.from_numpy(cfg["x"].view(np.int16)).cuda().view(tdt)
+    y32 = torch.empty((cfg["M"], cfg["N"]), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_dq_launch(w, x, y_f32=y32)
+    torch.cuda.synchronize()
+    out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    pre = y32.cpu().numpy()
+    w.destroy()
+    return out, pre
+
+
+CASES = [  # (M, K, N, g, bias)
+    (1, 512, 48, 64, False), (5, 1024, 100, 128, True), (16, 4096, 64, 128, False), (33, 2048, 40, 256, True),
+    (3, 256, 16, 64, True), (2, 1024, 24, 1024, False), (1, 4096, 4096, 128, False), (8, 11008, 128, 128, True),
+    (20, 17408, 32, 128, False),  # 136 groups: more than one LDS chunk of terms
+]
+
+
+@pytest.mark.parametrize("M,K,N,g,bias", CASES)
+def test_dynamic_int_device_level(orc, M, K, N, g, bias):
+    cfg = S.w4a16(M, K, N, g, seed=M + K + N, bias=bias)
+    out, pre = _device(cfg)
+    x, w, s, z, b = f32_valued_a16(cfg)
+    want, want_pre = orc.a16matmul_dynamic(x, w, s, z, b, M=M, K=K, N=N, weight_bits=4, q_group_size=g)
+    assert np.array_equal(pre.view(np.uint32), want_pre.view(np.uint32))
+    assert np.array_equal(out, orc.f32_to_bf16(want))
+
+
+def test_dynamic_int_zero_rows_and_large_values(orc):
+    M, K, N, g = 6, 512, 32, 128
+    cfg = S.w4a16(M, K, N, g, seed=9)
+    xf = S.bf16_to_f32(cfg["x"]).copy()
+    xf[1] = 0.0                      # amax falls back to 1e-8
+    xf[2, :128] = 0.0                # one empty group
+    xf[3] *= 1e20                    # huge but finite
+    xf[4] *= 1e-30                   # tiny
+    cfg = dict(cfg)
+    cfg["x"] = S.bf16_round(xf.astype(np.float32))
+    out, pre = _device(cfg)
+    x, w, s, z, b = f32_valued_a16(cfg)
+    want, want_pre = orc.a16matmul_dynamic(x, w, s, z, b, M=M, K=K, N=N, weight_bits=4, q_group_size=g)
+    assert np.array_equal(pre.view(np.uint32), want_pre.view(np.uint32))
+    assert np.array_equal(out, orc.f32_to_bf16(want))
+
+
+def test_dynamic_int_operator_level(orc):
+    M, K, N, g = 4, 1024, 80, 128
+    cfg = S.w4a16(M, K, N, g, seed=21, bias=True)
+    x, w, s, z, b = f32_valued_a16(cfg)
+    op = M_.A16MatMul(K=K, N=N, weight_bits=4, q_group_size=g, dynamic_quant=clib.DQ_INT).init(w, s, z, b)
+    y = op.inference(x)
+    op.deinit()
+    want, _ = orc.a16matmul_dynamic(x, w, s, z, b, M=M, K=K, N=N, weight_bits=4, q_group_size=g)
+    assert np.array_equal(y, want)
+
+
+def test_dynamic_int_rejects_what_it_does_not_handle():
+    cfg = S.w4a16(1, 256, 16, 32, seed=1)
+    import torch
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=256, N=16, weight_bits=4, q_group_size=32)
+    x = torch.zeros((1, 256), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(clib.BackendError) as e:
+        M_.a16mm_dq_launch(w, x)
+    assert e.value.code == clib.MI_UNSUPPORTED
+    w.destroy()

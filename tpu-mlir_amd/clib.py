@@ -18,7 +18,7 @@ EXPORTS = [
     "mi_version", "mi_last_error", "mi_device_count",
     "mi_a16mm_init", "mi_a16mm_inference", "mi_a16mm_deinit",
     "mi_a16_weight_create", "mi_a16_weight_destroy", "mi_a16_weight_bytes", "mi_a16mm_launch",
-    "mi_a16mm_launch_group",
+    "mi_a16mm_launch_group", "mi_a16mm_dq_launch",
     "mi_a16_weight_export_size", "mi_a16_weight_export", "mi_a16_weight_import", "mi_a16_quantize", "mi_llm_unpack",
     "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
     "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
@@ -39,6 +39,9 @@ class InferParam(C.Structure):
     _fields_ = [("inputs", C.POINTER(C.POINTER(C.c_float))), ("n_inputs", C.c_int),
                 ("outputs", C.POINTER(C.POINTER(C.c_float))), ("n_outputs", C.c_int),
                 ("handle", C.c_void_p)]
+
+
+DQ_NONE, DQ_INT, DQ_F8E4M3, DQ_F4 = 0, 1, 2, 3
 
 
 class A16Attr(C.Structure):
@@ -136,6 +139,7 @@ def lib():
                                     C.c_void_p, C.c_void_p]
         L.mi_a16_weight_destroy.restype = None
         L.mi_a16mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi_a16mm_dq_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_launch_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int64,
                                             C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_void_p]
         L.mi_module_create.argtypes = [C.POINTER(C.c_void_p)]

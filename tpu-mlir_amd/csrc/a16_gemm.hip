@@ -12,9 +12,6 @@
 //          acc += scale * (P - (16 + zp) * S) in fp32.
 //   8-bit: the weight is rounded to the 16-bit type exactly as the reference does, and the MFMA accumulates directly.
 #include <algorithm>
-#include <map>
-#include <mutex>
-#include <utility>
 
 #include "a16_common.cuh"
 #include "internal.h"
@@ -384,43 +381,6 @@ __global__ void a16_gemm_finish_kernel(float *__restrict__ acc, const float *__r
   *(u32x2 *)(y + i4) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
 }
 
-// fp32 partial-sum buffers of split-K products, one per (device, stream): a product leaves its buffer zeroed, products
-// on one stream are ordered, and products on different streams never share a buffer.  A buffer only grows; it is
-// allocated (and cleared) on first use, i.e. never inside a captured graph whose first run was eager.
-namespace {
-struct SplitBuf {
-  float *ptr = nullptr;
-  size_t elems = 0;
-};
-std::mutex g_split_mutex;
-std::map<std::pair<int, hipStream_t>, SplitBuf> g_split_bufs;
-
-int split_buffer(hipStream_t st, size_t elems, float **out) {
-  int dev = 0;
-  MI_HIP(hipGetDevice(&dev));
-  std::lock_guard<std::mutex> lock(g_split_mutex);
-  SplitBuf &b = g_split_bufs[{dev, st}];
-  if (b.elems < elems) {
-    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-    (void)hipStreamIsCapturing(st, &cs);
-    MI_REQUIRE(cs == hipStreamCaptureStatusNone, MI_HIP_ERROR,
-               "a16 split-K product: its partial-sum buffer must exist before the stream is captured (run the same "
-               "shape once eagerly first)");
-    if (b.ptr) {
-      MI_HIP(hipStreamSynchronize(st));
-      MI_HIP(hipFree(b.ptr));
-      b.ptr = nullptr;
-      b.elems = 0;
-    }
-    MI_HIP(hipMalloc((void **)&b.ptr, elems * sizeof(float)));
-    MI_HIP(hipMemset(b.ptr, 0, elems * sizeof(float)));
-    b.elems = elems;
-  }
-  *out = b.ptr;
-  return MI_SUCCESS;
-}
-}  // namespace
-
 template <int BITS, int DT, int GPT, int WM, int WN, int TM, int TN>
 static int launch_gemm_instance(GemmArgs &a, hipStream_t st) {
   constexpr int GM = WM * TM * 16, GN = WN * TN * 16;
@@ -442,7 +402,9 @@ static int launch_gemm_instance(GemmArgs &a, hipStream_t st) {
   a.acc = nullptr;
   if (a.k_splits > 1) {
     MI_REQUIRE((a.N % 4) == 0, MI_BAD_ARGUMENT, "a16 split-K product: N must be a multiple of 4");
-    int rc = split_buffer(st, (size_t)a.M * a.N, &a.acc);
+    // fp32 partial sums: the stream's own buffer, zero whenever no product is in flight (the finishing pass clears
+    // what it reads)
+    int rc = stream_workspace(st, WS_SPLIT_K, (size_t)a.M * a.N * sizeof(float), true, (void **)&a.acc);
     if (rc != MI_SUCCESS)
       return rc;
   }

@@ -340,6 +340,11 @@ int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
   return a16_launch(w, d_x, M, d_y, d_y_f32, (hipStream_t)stream);
 }
 
+int mi_a16mm_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
+                       void *stream) {
+  return a16_dq_launch(w, d_x, M, d_y, d_y_f32, (hipStream_t)stream);
+}
+
 int mi_a16mm_launch_group(const mi_a16_weight *const *w, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_y,
                           float *const *d_y_f32, void *stream) {
   return a16_launch_group(w, n, d_x, M, d_y, d_y_f32, (hipStream_t)stream);
@@ -352,7 +357,16 @@ int mi_a16mm_init(const mi_a16mm_attr *attr, mi_infer_param *p) {
   MI_REQUIRE(attr && p, MI_BAD_ARGUMENT, "mi_a16mm_init: null argument");
   p->handle = nullptr;
   MI_REQUIRE(p->inputs && p->n_inputs >= 4, MI_BAD_ARGUMENT, "mi_a16mm_init: expects input, weight, scale, zp[, bias]");
-  MI_REQUIRE(!attr->dynamic_quant, MI_UNSUPPORTED, "mi_a16mm_init: dynamic activation quantization is not handled");
+  MI_REQUIRE(attr->dynamic_quant == MI_DQ_NONE || attr->dynamic_quant == MI_DQ_INT, MI_UNSUPPORTED,
+             "mi_a16mm_init: only the integer dynamic-quantization types are handled");
+  if (attr->dynamic_quant == MI_DQ_INT) {
+    MI_REQUIRE(attr->q_group_size != 0, MI_BAD_ARGUMENT,
+               "mi_a16mm_init: dynamic quantization needs a group size (A16MatMul.cpp:42-43)");
+    MI_REQUIRE(attr->weight_bits == 4 && attr->q_group_size > 0 && attr->K % 128 == 0 &&
+                   (attr->q_group_size == 64 || attr->q_group_size % 128 == 0),
+               MI_UNSUPPORTED,
+               "mi_a16mm_init: dynamic quantization is handled for 4-bit weights, K % 128 == 0, groups of 64 or k*128");
+  }
   MI_REQUIRE(attr->w_transpose, MI_UNSUPPORTED, "mi_a16mm_init: only w_transpose weights ([N,K]) are handled");
   MI_REQUIRE(attr->weight_bits == 4 || attr->weight_bits == 8, MI_UNSUPPORTED, "mi_a16mm_init: weight_bits");
   MI_REQUIRE(attr->out_dtype == MI_DT_BF16 || attr->out_dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_a16mm_init: out_dtype");
@@ -439,7 +453,10 @@ int mi_a16mm_inference(const mi_a16mm_attr *attr, mi_infer_param *p) {
   for (int64_t i = 0; i < M * K; ++i)
     hx[i] = f16 ? h_f32_to_f16(x[i]) : h_f32_to_bf16(x[i]);
   MI_HIP(hipMemcpyAsync(h->d_x.ptr, hx, (size_t)M * K * 2, hipMemcpyHostToDevice, h->stream));
-  rc = a16_launch(h->w, (const uint16_t *)h->d_x.ptr, M, (uint16_t *)h->d_y.ptr, nullptr, h->stream);
+  if (attr->dynamic_quant == MI_DQ_INT)
+    rc = a16_dq_launch(h->w, (const uint16_t *)h->d_x.ptr, M, (uint16_t *)h->d_y.ptr, nullptr, h->stream);
+  else
+    rc = a16_launch(h->w, (const uint16_t *)h->d_x.ptr, M, (uint16_t *)h->d_y.ptr, nullptr, h->stream);
   if (rc != MI_SUCCESS)
     return rc;
   MI_HIP(hipMemcpyAsync(h->h_y.ptr, h->d_y.ptr, (size_t)M * N * 2, hipMemcpyDeviceToHost, h->stream));

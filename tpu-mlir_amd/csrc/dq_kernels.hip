@@ -1,0 +1,264 @@
+// tpu.A16MatMul with dynamic activation quantization, integer flavour (dq_type "INT4" / "INT8"), 4-bit weights:
+// lib/Dialect/Tpu/Interfaces/Common/A16MatMul.cpp:40-170.
+//
+// Per activation row and per quantization group along K the reference scales the activations by their own abs-max to
+// integers in [-imax, imax] (imax = 7 for 4-bit weights), multiplies them with the integer weights (q - zp) group by
+// group, and adds   isum * (amax / imax) * scale[n][g]   into the output in group order, the bias after the first
+// group.  Every piece of that is deterministic, so this path is bit-exact:
+//
+//   dq_act_kernel    one wave per (row, group): abs-max, the integer codes, their sum.  The codes are written straight
+//                    into the A-fragment order of v_mfma_i32_16x16x64_i8 that mirrors the packed weight tiles, so the
+//                    product kernel loads both operands with one coalesced 16-byte read per lane and never shuffles.
+//   dq_gemm_kernel   a workgroup owns 16 rows x 16 output channels; its waves take quantization groups round-robin,
+//                    each group an integer MFMA sum (nibbles 0..15 as int8, the zero point applied as zp * sum(codes)),
+//                    then the two fp32 multiplies of the reference; the per-group terms wait in LDS until 256 threads
+//                    add them up in group order.  Parallel over groups, sequential where the reference is.
+//
+// The packed weight set is the one the static kernels read (a16_kernels.hip).
+#include "a16_common.cuh"
+#include "internal.h"
+
+#pragma clang fp contract(off)
+
+namespace mi {
+
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+
+constexpr int DQ_WAVES = 8;
+constexpr int DQ_CHUNK = 128;  // groups whose terms fit the LDS buffer at once (1 KiB each)
+
+// position of element e (0..7) of a packed dword inside the 8 operand bytes it unpacks to: the low-nibble bytes of
+// the dword are elements 0,4,1,5 and the high-nibble bytes elements 2,6,3,7 (see unpack below)
+__device__ __forceinline__ int dq_slot(int e) { return ((e & 1) << 1) | ((e & 2) << 1) | (e >> 2); }
+
+// ---- activations -> integer codes in fragment order
+// aq: [m_blocks][k_tiles][2][64 lanes][16 B]; as_t / asum_t: [m_blocks][G][16 rows]
+template <int DT>
+__global__ __launch_bounds__(256) void dq_act_kernel(const uint16_t *__restrict__ x, int64_t M, int64_t K, int g, int G,
+                                                      float imax, int64_t k_tiles, uint8_t *__restrict__ aq,
+                                                      float *__restrict__ as_t, int32_t *__restrict__ asum_t,
+                                                      int64_t rows_padded) {
+  using H = Half16<DT>;
+  const int lane = threadIdx.x & 63;
+  const int64_t wid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (wid >= rows_padded * G)
+    return;
+  const int64_t m = wid / G;
+  const int gi = (int)(wid - m * G);
+  const bool live = m < M;
+  // A16MatMul.cpp:98-108: amax starts at 1e-8
+  float amax = (float)1e-8;
+  if (live)
+    for (int k = lane; k < g; k += 64) {
+      const float v = fabsf(H::to_f32(x[m * K + (int64_t)gi * g + k]));
+      amax = amax > v ? amax : v;
+    }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float other = __shfl_xor(amax, o, 64);
+    amax = amax > other ? amax : other;
+  }
+  // :109-120: round(x / amax * imax), half away from zero
+  int sum = 0;
+  const int64_t mb = m >> 4;
+  const int row = (int)(m & 15);
+  for (int k = lane; k < g; k += 64) {
+    const int64_t kk = (int64_t)gi * g + k;
+    int code = 0;
+    if (live)
+      code = (int)roundf(H::to_f32(x[m * K + kk]) / amax * imax);
+    sum += code;
+    const int64_t kt = kk >> 7;
+    const int in_tile = (int)(kk & 127);
+    const int j = in_tile >> 5, kq = (in_tile >> 3) & 3, e = in_tile & 7;
+    const int64_t at = ((((mb * k_tiles + kt) * 2 + (j >> 1)) * 64) + kq * 16 + row) * 16 + (j & 1) * 8 + dq_slot(e);
+    aq[at] = (uint8_t)(int8_t)code;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1)
+    sum += __shfl_xor(sum, o, 64);
+  if (lane == 0) {
+    const int64_t at = (mb * G + gi) * 16 + row;
+    as_t[at] = live ? amax / imax : 0.0f;  // :143-145 (cur_group_act_max[row] / imax)
+    asum_t[at] = sum;
+  }
+}
+
+struct DqArgs {
+  const u32x4 *qw;
+  const uint32_t *sz_t;
+  const float *bias;
+  const u32x4 *aq;
+  const float *as_t;
+  const int32_t *asum_t;
+  uint16_t *y;
+  float *y32;
+  int64_t M, N;
+  int64_t k_tiles;
+  int G;
+  int unit_tiles;   // weight tiles per unit of work: g / 128 when g >= 128, else 1 (the unit then holds two groups)
+  int unit_groups;  // groups per unit: 1, or 2 when g == 64
+  int chip;
+};
+
+// nibbles of a packed dword as bytes: low nibbles (elements 0,4,1,5), high nibbles (elements 2,6,3,7)
+__device__ __forceinline__ void unpack_bytes(uint32_t d, int &lo, int &hi) {
+  lo = (int)(d & 0x0F0F0F0Fu);
+  hi = (int)((d >> 4) & 0x0F0F0F0Fu);
+}
+
+template <int DT>
+__global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
+  using H = Half16<DT>;
+  extern __shared__ __attribute__((aligned(16))) float terms[];  // [groups of the chunk][16 rows][16 columns]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, kq = lane >> 4;
+  const int64_t rb = blockIdx.x, mb = blockIdx.y;
+  const u32x4 *wq = a.qw + rb * a.k_tiles * 64 + lane;
+  const u32x4 *aq = a.aq + mb * a.k_tiles * 128 + lane;
+  const uint32_t *sz = a.sz_t + rb * a.G * 16 + col;
+  const float *as_p = a.as_t + mb * a.G * 16 + 4 * kq;
+  const int32_t *asum_p = a.asum_t + mb * a.G * 16 + 4 * kq;
+
+  // the ordered sum: thread t < 256 owns output (row t >> 4, column t & 15)
+  float out = 0.0f;
+  const int64_t n_out = rb * 16 + (tid & 15), m_out = mb * 16 + (tid >> 4);
+  const bool owns = tid < 256 && n_out < a.N && m_out < a.M;
+  const float bias = (owns && a.bias) ? a.bias[n_out] : 0.0f;
+
+  const int units = (a.G + a.unit_groups - 1) / a.unit_groups;
+  const int chunk_units = DQ_CHUNK / a.unit_groups;
+  for (int u0 = 0; u0 < units; u0 += chunk_units) {
+    const int u1 = (u0 + chunk_units) < units ? (u0 + chunk_units) : units;
+    for (int u = u0 + wave; u < u1; u += DQ_WAVES) {
+      i32x4 acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+      for (int t = 0; t < a.unit_tiles; ++t) {
+        const int64_t kt = (int64_t)u * a.unit_tiles + t;
+        const u32x4 w = wq[kt * 64];
+        const u32x4 a0 = aq[kt * 128], a1 = aq[kt * 128 + 64];
+        int lo[4], hi[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          unpack_bytes(w[j], lo[j], hi[j]);
+        const i32x4 b0 = {lo[0], hi[0], lo[1], hi[1]}, b1 = {lo[2], hi[2], lo[3], hi[3]};
+        // k 0..63 of the tile, then k 64..127; with 64-wide groups these are two groups
+        acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0), b0, acc[0], 0, 0, 0);
+        if (a.unit_groups == 2)
+          acc[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1), b1, acc[1], 0, 0, 0);
+        else
+          acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1), b1, acc[0], 0, 0, 0);
+      }
+      for (int h = 0; h < a.unit_groups; ++h) {
+        const int gi = u * a.unit_groups + h;
+        if (gi >= a.G)
+          break;
+        const uint32_t szw = sz[(int64_t)gi * 16];
+        const float sc = H::to_f32((uint16_t)(szw >> 16));
+        const int zp = (int)(szw & 0xffu);
+        const f32x4 as4 = *(const f32x4 *)(as_p + (int64_t)gi * 16);
+        const i32x4 sum4 = *(const i32x4 *)(asum_p + (int64_t)gi * 16);
+        float *dst = terms + (size_t)(gi - u0 * a.unit_groups) * 256;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int isum = acc[h][r] - zp * sum4[r];     // sum_k code_k (q_k - zp): exact
+          float t = (float)isum;                          // below 2^24 (checked on the host): exact
+          t = t * as4[r];                                 // A16MatMul.cpp:153-156, left to right
+          t = t * sc;
+          dst[(4 * kq + r) * 16 + col] = t;
+        }
+      }
+    }
+    __syncthreads();
+    if (owns) {
+      const int g0 = u0 * a.unit_groups;
+      const int g1 = (u1 * a.unit_groups) < a.G ? (u1 * a.unit_groups) : a.G;
+      for (int gi = g0; gi < g1; ++gi) {
+        out = out + terms[(size_t)(gi - g0) * 256 + tid];
+        if (gi == 0 && a.bias)
+          out = out + bias;  // :157-159
+      }
+    }
+    __syncthreads();
+  }
+  if (owns) {
+    const int64_t o = m_out * a.N + n_out;
+    if (a.y32)
+      a.y32[o] = out;
+    a.y[o] = (a.chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(out) : round_out16<DT, MI_CHIP_BM168X>(out);
+  }
+}
+
+int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
+                  hipStream_t stream) {
+  MI_REQUIRE(w && w->qweight && d_x && d_y, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: null argument");
+  MI_REQUIRE(M >= 0 && M < (1 << 20), MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: M out of range");
+  MI_REQUIRE(w->bits == 4, MI_UNSUPPORTED, "mi_a16mm_dq_launch: only 4-bit weights are handled");
+  MI_REQUIRE(w->g != 0, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: dynamic quantization needs a group size (A16MatMul.cpp:42)");
+  const int g = w->g;
+  MI_REQUIRE((w->K % 128) == 0 && (g == 64 || g % 128 == 0), MI_UNSUPPORTED,
+             "mi_a16mm_dq_launch: K must be a multiple of 128 and the group size 64 or a multiple of 128");
+  MI_REQUIRE((int64_t)g * 7 * 15 < (1 << 24), MI_UNSUPPORTED,
+             "mi_a16mm_dq_launch: group too long for the integer sums to stay exact in the reference's f32 product");
+  if (M == 0)
+    return MI_SUCCESS;
+  const int64_t m_blocks = (M + 15) / 16, rows_padded = m_blocks * 16;
+  const int G = w->G;
+  // codes, scales and code sums of this call: the stream's scratch buffer
+  const size_t aq_bytes = ((size_t)rows_padded * w->K + 255) & ~(size_t)255, qp_bytes = (size_t)rows_padded * G * 4;
+  uint8_t *aq = nullptr;
+  int rc = stream_workspace(stream, WS_DYNAMIC_QUANT, aq_bytes + 2 * qp_bytes, false, (void **)&aq);
+  if (rc != MI_SUCCESS)
+    return rc;
+  float *as_t = (float *)(aq + aq_bytes);
+  int32_t *asum_t = (int32_t *)(aq + aq_bytes + qp_bytes);
+  const float imax = 7.0f;  // (1 << (weight_bits - 1)) - 1, A16MatMul.cpp:53-54
+  const int64_t waves = rows_padded * G;
+  const bool f16 = w->dtype == MI_DT_F16;
+  if (f16)
+    dq_act_kernel<MI_DT_F16><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(
+        d_x, M, w->K, g, G, imax, w->k_tiles, aq, as_t, asum_t, rows_padded);
+  else
+    dq_act_kernel<MI_DT_BF16><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(
+        d_x, M, w->K, g, G, imax, w->k_tiles, aq, as_t, asum_t, rows_padded);
+  DqArgs a;
+  a.qw = (const u32x4 *)w->qweight;
+  a.sz_t = w->sz_t;
+  a.bias = w->bias;
+  a.aq = (const u32x4 *)aq;
+  a.as_t = as_t;
+  a.asum_t = asum_t;
+  a.y = d_y;
+  a.y32 = d_y32;
+  a.M = M;
+  a.N = w->N;
+  a.k_tiles = w->k_tiles;
+  a.G = G;
+  a.unit_tiles = g >= 128 ? g / 128 : 1;
+  a.unit_groups = g == 64 ? 2 : 1;
+  a.chip = w->chip;
+  const int chunk_groups = G < DQ_CHUNK ? G : DQ_CHUNK;
+  const size_t lds_bytes = (size_t)(chunk_groups + 1) * 1024;
+  dim3 grid((unsigned)w->row_blocks, (unsigned)m_blocks);
+  if (f16) {
+    static bool attr_set = false;
+    if (!attr_set) {
+      (void)hipFuncSetAttribute((const void *)dq_gemm_kernel<MI_DT_F16>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024);
+      attr_set = true;
+    }
+    dq_gemm_kernel<MI_DT_F16><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);
+  } else {
+    static bool attr_set = false;
+    if (!attr_set) {
+      (void)hipFuncSetAttribute((const void *)dq_gemm_kernel<MI_DT_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024);
+      attr_set = true;
+    }
+    dq_gemm_kernel<MI_DT_BF16><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);
+  }
+  MI_HIP(hipGetLastError());
+  return MI_SUCCESS;
+}
+
+}  // namespace mi

@@ -71,6 +71,15 @@ int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
 int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
                      float *const *d_y32s, hipStream_t stream);
 
+// library-owned scratch, one buffer per (device, stream, purpose) (workspace.hip).  zeroed: cleared when allocated;
+// the user of such a buffer leaves it zero.
+enum { WS_SPLIT_K = 0, WS_DYNAMIC_QUANT = 1 };
+int stream_workspace(hipStream_t st, int purpose, size_t bytes, bool zeroed, void **out);
+
+// dynamic activation quantization, integer flavour (dq_kernels.hip)
+int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
+                  hipStream_t stream);
+
 // weight producers (quant_kernels.hip); arguments are validated by the callers
 int a16_quantize(const mi_a16_quant_desc *d, const float *h_w_kn, void *h_weight, uint16_t *h_scale16,
                  float *h_scale_f32, uint8_t *h_zp, int *sign_out, int *weight_signed_out);

@@ -285,6 +285,24 @@ def llm_unpack(mode, bits, qweight, qzeros, *, K, N):
     return q, zp
 
 
+def a16mm_dq_launch(w, x, y=None, y_f32=None, stream=None):
+    """As a16mm_launch, with the reference's dynamic integer activation quantization (4-bit weights)."""
+    import torch
+    tdt = torch.float16 if w.dtype == DT_F16 else torch.bfloat16
+    if not (x.is_cuda and x.dtype == tdt and x.is_contiguous() and x.shape[-1] == w.K):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_dq_launch: x must be a contiguous CUDA tensor [.., K]")
+    M = x.numel() // w.K
+    if y is None:
+        y = torch.empty(tuple(x.shape[:-1]) + (w.N,), dtype=tdt, device=x.device)
+    if not (y.is_cuda and y.dtype == tdt and y.is_contiguous() and y.numel() == M * w.N):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_dq_launch: bad output tensor")
+    if y_f32 is not None and not (y_f32.is_cuda and y_f32.dtype == torch.float32 and y_f32.is_contiguous()
+                                  and y_f32.numel() == M * w.N):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_dq_launch: bad y_f32 tensor")
+    check(clib.lib().mi_a16mm_dq_launch(w.handle, _dptr(x), M, _dptr(y), _dptr(y_f32), _stream_ptr(stream)))
+    return y
+
+
 def a16mm_launch(w, x, y=None, y_f32=None, stream=None):
     """y[M,N] = round16(x[M,K] @ dequant(W)^T + bias) on the current stream.  x, y: torch CUDA tensors of the
     weight set's 16-bit type; y_f32 (optional float32 CUDA tensor) receives the fp32 result before rounding."""
