@@ -193,10 +193,15 @@ struct RequantParams {
 
 // int32 accumulator of channel n -> saturated output value.  The descriptor's shift is a RIGHT shift
 // when positive for every mode (the device-level convention), so the QDM family passes -shift on.
+__device__ __forceinline__ int32_t requant_with(int32_t acc, int64_t m, int64_t s, int64_t z, const RequantParams &rq);
 __device__ __forceinline__ int32_t requant_one(int32_t acc, int64_t n, const RequantParams &rq) {
   int64_t m = rq.mult ? rq.mult[n] : rq.mult_s;
   int64_t s = rq.shift ? rq.shift[n] : rq.shift_s;
   int64_t z = rq.zp ? rq.zp[n] : rq.zp_s;
+  return requant_with(acc, m, s, z, rq);
+}
+// the same with the channel's multiplier, shift and zero point already in hand
+__device__ __forceinline__ int32_t requant_with(int32_t acc, int64_t m, int64_t s, int64_t z, const RequantParams &rq) {
   int64_t v;
   if (rq.qmode == MI_RQ_MULTIPLIER_SHIFT || rq.qmode == MI_RQ_ONLY_SHIFT)
     v = apply_multiplier_and_rshift(acc, m, s, rq.qmode, rq.rmode, rq.chip);

@@ -116,6 +116,7 @@ struct I8Args {
   int do_relu;
   int64_t relu_limit;
   int has_rq;
+  int q31_half_away;  // the requantization is the Q31 multiplier / right shift in [1, 31] / half away / int8 case
   RequantParams rq;
 };
 
@@ -209,35 +210,35 @@ __global__ __launch_bounds__(256) void i8_gemm_kernel(I8Args a) {
     }
   }
 
-  // epilogue: 32x32 block layout -- register r of lane l is row 8*(r/4) + 4*(l/32) + (r%4), column l%32
+  // epilogue: 32x32 block layout -- register r of lane l is row 8*(r/4) + 4*(l/32) + (r%4), column l%32.  The loops
+  // carry no early exits so that they unroll completely and the accumulators stay in registers.
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int64_t n = n_base + wn * 64 + j * 32 + (lane & 31);
-    if (n >= a.N)
-      continue;
-    const int32_t bias_n = a.bias ? a.bias[n] : 0;
+    const bool n_ok = n < a.N;
+    const int32_t bias_n = (a.bias && n_ok) ? a.bias[n] : 0;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int64_t m = m_base + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (m >= a.M)
-          continue;
-        int32_t v = acc[i][j][r] + bias_n;
-        if (a.row_term)
-          v += a.row_term[m];
-        if (a.do_relu) {
-          v = v > 0 ? v : 0;
-          if (a.relu_limit > 0 && v > a.relu_limit)
-            v = (int32_t)a.relu_limit;
+        if (n_ok && m < a.M) {
+          int32_t v = acc[i][j][r] + bias_n;
+          if (a.row_term)
+            v += a.row_term[m];
+          if (a.do_relu) {
+            v = v > 0 ? v : 0;
+            if (a.relu_limit > 0 && v > a.relu_limit)
+              v = (int32_t)a.relu_limit;
+          }
+          const int64_t o = m * a.N + n;
+          if (a.acc_out)
+            a.acc_out[o] = v;
+          if (a.has_rq)
+            store_out(a.out, o, requant_one(v, n, a.rq), a.rq.out_dtype);
+          else if (a.out)
+            ((int32_t *)a.out)[o] = v;
         }
-        const int64_t o = m * a.N + n;
-        if (a.acc_out)
-          a.acc_out[o] = v;
-        if (a.has_rq)
-          store_out(a.out, o, requant_one(v, n, a.rq), a.rq.out_dtype);
-        else if (a.out)
-          ((int32_t *)a.out)[o] = v;
       }
     }
   }
@@ -271,12 +272,6 @@ constexpr int WAITCNT_LGKM0 = 0xC07F;
 #else
 #define MI_I8_STAMP(v)
 #endif
-#ifdef MI_I8_TIMING
-__device__ unsigned long long mi_i8_dbg[64 * 4 * 4 + 64 * 8];
-extern "C" int mi_i8_dbg_dump(unsigned long long *host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mi_i8_dbg), sizeof(mi_i8_dbg));
-}
-#endif
 
 __device__ __forceinline__ int32_t med3_i32(int32_t x, int32_t lo, int32_t hi) {
   int32_t r;
@@ -291,6 +286,274 @@ __device__ __forceinline__ uint32_t sat_pack_u8(int32_t q0, int32_t q1, int32_t 
   asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
   asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
   return (b01 & 0xffffu) | (b23 << 16);
+}
+
+#ifdef MI_I8_TIMING
+__device__ unsigned long long mi_i8_dbg[64 * 4 * 4 + 64 * 8];
+extern "C" int mi_i8_dbg_dump(unsigned long long *host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mi_i8_dbg), sizeof(mi_i8_dbg));
+}
+#endif
+
+// ------------------------------------------------------------------------------------------------
+// Mid-size kernel: 128x128 outputs per workgroup (4 waves, each 64x64 as 2x2 MFMA 32x32x32 blocks), K advancing 64
+// bytes per stage through a 4-stage LDS ring filled by direct-to-LDS loads -- the large kernel's data path at a
+// quarter of its tile, for shapes that would leave most CUs without a 256x256 tile.  Three stages of loads are in
+// flight while one is computed, so a short K loop costs about one memory latency, not one per step.
+// Requires K % 64 == 0; rows past M/N are clamped on the way in and masked on the way out.
+// ------------------------------------------------------------------------------------------------
+constexpr int MID_M = 128, MID_N = 128, MID_K = 64;
+constexpr int MID_STAGE = (MID_M + MID_N) * MID_K;  // 16 KiB
+constexpr int MID_STRIDE = 68;                      // dwords per row of an epilogue strip (64 + 4: 16-byte aligned rows)
+constexpr int mid_lds_bytes(int nst) { return nst * MID_STAGE > 4 * 64 * MID_STRIDE * 4 ? nst * MID_STAGE : 4 * 64 * MID_STRIDE * 4; }
+
+// MID_NST = stages in the LDS ring: 4 (two workgroups per CU) when there are more tiles than CUs, 8 when every
+// workgroup has a CU to itself -- a short grid is bound by the bytes it keeps in flight.
+template <int MID_NST>
+__global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m, int tiles_n, int per_xcd) {
+  constexpr int LOADS = MID_M * (MID_K / 16) / 256;  // direct-to-LDS instructions per operand, stage and thread: 2
+  constexpr int LPS = 2 * LOADS;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+#ifdef MI_I8_TIMING
+  const unsigned long long t_entry = __builtin_amdgcn_s_memrealtime();
+#endif
+  const int bid = blockIdx.x;
+  const int L = (bid & 7) * per_xcd + (bid >> 3);  // each XCD gets a contiguous run of the tile order
+  if (L >= tiles_m * tiles_n)
+    return;
+  constexpr int GM = 4;
+  const int group = L / (GM * tiles_n);
+  const int gm = (tiles_m - group * GM) < GM ? (tiles_m - group * GM) : GM;
+  const int in_group = L - group * GM * tiles_n;
+  const int tm = group * GM + in_group % gm, tn = in_group / gm;
+  const int64_t m_base = (int64_t)tm * MID_M, n_base = (int64_t)tn * MID_N;
+
+  // the 16-byte chunk c of row r is stored at position c ^ ((r >> 2) & 3): the 32 rows of a fragment read hit
+  // distinct bank groups
+  const uint8_t *ga[LOADS], *gb[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int slot = (i * 4 + wave) * 64 + lane;
+    const int row = slot >> 2, pos = slot & 3;
+    const int chunk = pos ^ ((row >> 2) & 3);
+    int64_t ra = m_base + row, rb = n_base + row;
+    ra = ra < a.M ? ra : a.M - 1;  // re-read the last row; never stored
+    rb = rb < a.N ? rb : a.N - 1;
+    ga[i] = a.A + ra * a.K + chunk * 16;
+    gb[i] = a.B + rb * a.K + chunk * 16;
+  }
+  const int kt_total = (int)(a.K / MID_K);
+  auto issue = [&](int kt) {
+    const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 1) * MID_K;  // past the end: harmless re-load
+    uint8_t *sa = lds + (kt % MID_NST) * MID_STAGE, *sb = sa + MID_M * MID_K;
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      __builtin_amdgcn_global_load_lds((gptr_t)(ga[i] + koff), (lptr_t)(sa + (i * 4 + wave) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(gb[i] + koff), (lptr_t)(sb + (i * 4 + wave) * 1024), 16, 0, 0);
+    }
+  };
+
+  i32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[i][j][r] = 0;
+
+  const int frow = lane & 31, kh = lane >> 5;
+  int a_off[2], b_off[2], f_sw[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int ra = wm * 64 + i * 32 + frow, rb = wn * 64 + i * 32 + frow;
+    a_off[i] = ra * MID_K;
+    b_off[i] = MID_M * MID_K + rb * MID_K;
+    f_sw[i] = (frow >> 2) & 3;  // (row >> 2) & 3 with row = 32-aligned base + frow
+  }
+
+  // epilogue parameters of this lane's 16 output columns, requested ahead of every stage request (requests complete
+  // in order and the waits in the K loop count them) so that their latency hides behind the K loop; nothing uses
+  // them before the epilogue
+  const int cc = lane & 3, rsub = lane >> 2;  // 16-column chunk, row within a group of 16 rows
+  const int64_t n0 = n_base + wn * 64 + cc * 16;
+  const bool vec_ok = (a.N % 16) == 0 && n0 + 16 <= a.N;
+  const int32_t relu_hi = (a.relu_limit > 0 && a.relu_limit < INT32_MAX) ? (int32_t)a.relu_limit : INT32_MAX;
+  int32_t p_bias[16], p_mult[16], p_shift[16], p_zp[16];
+  // one array -> 16 registers: four 16-byte loads when the lane's columns are whole and aligned (the arrays are
+  // device allocations and n0 is a multiple of 16), else element by element with the index clamped
+  auto load16 = [&](const int32_t *src, int32_t dflt, int32_t (&dst)[16]) {
+    if (!src) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        dst[e] = dflt;
+    } else if (vec_ok) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const i32x4 t = *(const i32x4 *)(src + n0 + q4 * 4);
+        dst[q4 * 4 + 0] = t[0];
+        dst[q4 * 4 + 1] = t[1];
+        dst[q4 * 4 + 2] = t[2];
+        dst[q4 * 4 + 3] = t[3];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        dst[e] = src[(n0 + e) < a.N ? (n0 + e) : (a.N - 1)];
+    }
+  };
+  load16(a.bias, 0, p_bias);
+  if (a.q31_half_away) {
+    load16(a.rq.mult, a.rq.mult_s, p_mult);
+    load16(a.rq.shift, a.rq.shift_s, p_shift);
+    load16(a.rq.zp, a.rq.zp_s, p_zp);
+  }
+#pragma unroll
+  for (int s0 = 0; s0 < MID_NST - 1; ++s0)
+    issue(s0);
+#ifdef MI_I8_TIMING
+  const unsigned long long t_loop = __builtin_amdgcn_s_memrealtime();
+#endif
+  for (int kt = 0; kt < kt_total; ++kt) {
+    // requests complete in order: at most (NST - 2) stages' worth outstanding means stage kt has landed
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((MID_NST - 2) * LPS));
+    __builtin_amdgcn_s_barrier();  // everyone's share of stage kt is in LDS; everyone is done with stage kt - 1
+    issue(kt + MID_NST - 1);
+    const uint8_t *st = lds + (kt % MID_NST) * MID_STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      i32x4 fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        fa[i] = *(const i32x4 *)(st + a_off[i] + (((ks * 2 + kh) ^ f_sw[i]) << 4));
+        fb[i] = *(const i32x4 *)(st + b_off[i] + (((ks * 2 + kh) ^ f_sw[i]) << 4));
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // drain the re-loads issued past the end
+#ifdef MI_I8_TIMING
+  const unsigned long long t_epi = __builtin_amdgcn_s_memrealtime();
+#endif
+
+  // epilogue.  The accumulators (register r of lane l = row 8*(r/4) + 4*(l/32) + (r%4), column l%32 of a 32x32
+  // block) pass through a per-wave 64 x 64 strip in LDS so that a lane owns 16 consecutive columns of a row: per-column
+  // parameters are loaded once per lane, and int8 results leave as 16-byte stores.
+  __builtin_amdgcn_s_barrier();  // every wave is done reading the ring
+  int32_t *strip = (int32_t *)lds + wave * (64 * MID_STRIDE);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        strip[(i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * MID_STRIDE + j * 32 + (lane & 31)] = acc[i][j][r];
+  // a wave only reads what it wrote: no barrier, the LDS counter orders it
+  int32_t p_half[16];
+  if (a.q31_half_away) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      p_half[e] = 1 << (p_shift[e] - 1);
+      p_zp[e] += 128;  // saturate as unsigned, flip the sign bits after
+    }
+  }
+#pragma unroll 1
+  for (int it = 0; it < 4; ++it) {
+    const int row = it * 16 + rsub;
+    const int64_t m = m_base + wm * 64 + row;
+    int32_t v[16];
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const i32x4 t = *(const i32x4 *)(strip + row * MID_STRIDE + cc * 16 + q4 * 4);
+      v[q4 * 4 + 0] = t[0] + p_bias[q4 * 4 + 0];
+      v[q4 * 4 + 1] = t[1] + p_bias[q4 * 4 + 1];
+      v[q4 * 4 + 2] = t[2] + p_bias[q4 * 4 + 2];
+      v[q4 * 4 + 3] = t[3] + p_bias[q4 * 4 + 3];
+    }
+    if (a.row_term) {  // per-row term of a nonzero right zero point
+      const int32_t rt = a.row_term[m < a.M ? m : a.M - 1];
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        v[e] += rt;
+    }
+    if (a.do_relu) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        v[e] = med3_i32(v[e], 0, relu_hi);
+    }
+    const bool live = m < a.M && n0 < a.N;
+    const int64_t o = m * a.N + n0;
+    if (a.acc_out && live) {
+      if (vec_ok) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)
+          *(i32x4 *)(a.acc_out + o + q4 * 4) = i32x4{v[q4 * 4], v[q4 * 4 + 1], v[q4 * 4 + 2], v[q4 * 4 + 3]};
+      } else {
+        for (int e = 0; e < 16; ++e)
+          if (n0 + e < a.N)
+            a.acc_out[o + e] = v[e];
+      }
+    }
+    if (a.q31_half_away) {
+      // MultiplyByQuantizedMultiplier(x, mult, -shift, HALF_AWAY) with shift in [1, 31], in 32-bit steps, saturated
+      // as unsigned on q + 128 and flipped back (see the large kernel's epilogue)
+      uint32_t packed[4];
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        int32_t q[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int e = q4 * 4 + u;
+          const int64_t p = (int64_t)v[e] * (int64_t)p_mult[e] + (1ll << 30);
+          const int32_t t = (int32_t)(p >> 31);
+          q[u] = ((t + p_half[e] + (t >> 31)) >> p_shift[e]) + p_zp[e];
+        }
+        packed[q4] = sat_pack_u8(q[0], q[1], q[2], q[3]) ^ 0x80808080u;
+      }
+      if (live) {
+        int8_t *out = (int8_t *)a.out;
+        if (vec_ok) {
+          *(u32x4 *)(out + o) = u32x4{packed[0], packed[1], packed[2], packed[3]};
+        } else {
+          for (int e = 0; e < 16; ++e)
+            if (n0 + e < a.N)
+              out[o + e] = (int8_t)((packed[e >> 2] >> (8 * (e & 3))) & 0xff);
+        }
+      }
+    } else if (a.has_rq) {
+      if (live)
+        for (int e = 0; e < 16; ++e)
+          if (n0 + e < a.N)
+            store_out(a.out, o + e, requant_one(v[e], n0 + e, a.rq), a.rq.out_dtype);
+    } else if (a.out && live) {
+      int32_t *out = (int32_t *)a.out;
+      if (vec_ok) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)
+          *(i32x4 *)(out + o + q4 * 4) = i32x4{v[q4 * 4], v[q4 * 4 + 1], v[q4 * 4 + 2], v[q4 * 4 + 3]};
+      } else {
+        for (int e = 0; e < 16; ++e)
+          if (n0 + e < a.N)
+            out[o + e] = v[e];
+      }
+    }
+  }
+#ifdef MI_I8_TIMING
+  if (lane == 0 && wave == 0 && blockIdx.x < 64) {
+    unsigned long long *d = mi_i8_dbg + 1024 + blockIdx.x * 8;
+    d[0] = t_entry;
+    d[1] = t_loop - t_entry;
+    d[2] = t_epi - t_loop;
+    d[3] = __builtin_amdgcn_s_memrealtime() - t_entry;
+  }
+#endif
 }
 
 // LK_ = bytes of K per stage (64 or 128), NST = stages in the LDS ring (NST * 512 * LK_ bytes)
@@ -729,15 +992,34 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
   a.do_relu = do_relu;
   a.relu_limit = relu_limit;
   a.has_rq = rq != nullptr;
+  int epi = EPI_INT32;
+  if (rq) {
+    const bool q31 = rq->quant_mode == MI_RQ_QDM || rq->quant_mode == MI_RQ_TFLITE ||
+                     rq->quant_mode == MI_RQ_TFLITE_LSHIFT;
+    // the 32-bit fast path needs a right shift in [1, 31] on every channel; per-channel shifts are the
+    // caller's device array, so it is only taken for a scalar shift or when the caller vouches via the desc
+    epi = (q31 && rq->round_mode == MI_ROUND_HALF_AWAY_FROM_ZERO && rq->out_dtype == MI_DT_I8 &&
+           (rq->d_shift || (rq->shift >= 1 && rq->shift <= 31)))
+              ? EPI_Q31_HALF_AWAY
+              : EPI_GENERIC;
+  }
+  a.q31_half_away = epi == EPI_Q31_HALF_AWAY;
   if (rq)
     a.rq = make_rq(rq);
   else
     a.rq = RequantParams{nullptr, nullptr, nullptr, 1, 0, 0, MI_RQ_MULTIPLIER_SHIFT, 0, 0, MI_DT_I32};
-  const bool large = (K % 128) == 0 && M >= 128 && N >= 128 && !getenv("MI_I8_SMALL_TILE");
+  // 256x256 tiles when there are enough of them to occupy the chip, else 128x128 tiles on the same data path; the
+  // register-staged kernel takes what is left (K % 64 != 0)
+  const int64_t tiles_large = ((M + LM - 1) / LM) * ((N + LN - 1) / LN);
+  const char *tile_env = getenv("MI_I8_TILE");  // development switch: "256" / "128" / "0" (register-staged)
+  const bool large_ok = (K % 128) == 0 && M >= 128 && N >= 128, mid_ok = (K % 64) == 0;
+  const int tile_pick = tile_env ? atoi(tile_env) : (large_ok && tiles_large >= 144 ? 256 : 128);  // measured crossover
+  const bool large = large_ok && tile_pick == 256;
+  const bool mid = !large && mid_ok && tile_pick != 0;
   uint8_t *a_signed = nullptr, *b_signed = nullptr;
-  if (large) {
-    // the direct-to-LDS loads of the large-tile kernel cannot flip sign bits on the way: unsigned operands are
-    // rewritten once (after the zero-point sums above, which read the original bytes)
+  if (large || mid) {
+    // direct-to-LDS loads cannot flip sign bits on the way: unsigned operands are rewritten once (after the
+    // zero-point sums above, which read the original bytes)
     if (a_unsigned) {
       MI_HIP(hipMallocAsync((void **)&a_signed, (size_t)M * K, stream));
       flip_bytes_kernel<<<dim3((unsigned)((M * K / 16 + 256) / 256)), dim3(256), 0, stream>>>(a.A, a_signed, M * K);
@@ -748,22 +1030,32 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
       flip_bytes_kernel<<<dim3((unsigned)((N * K / 16 + 256) / 256)), dim3(256), 0, stream>>>(a.B, b_signed, N * K);
       a.B = b_signed;
     }
+  }
+  if (mid) {
+    const int tiles_m = (int)((M + MID_M - 1) / MID_M), tiles_n = (int)((N + MID_N - 1) / MID_N);
+    const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+    static bool attr_set = false;
+    if (!attr_set) {
+      (void)hipFuncSetAttribute((const void *)i8_gemm_mid_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024);
+      (void)hipFuncSetAttribute((const void *)i8_gemm_mid_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024);
+      attr_set = true;
+    }
+    const char *ring_env = getenv("MI_I8_MID_RING");  // development switch: 4 / 8
+    const int ring = ring_env ? atoi(ring_env) : (tiles_m * tiles_n <= 256 ? 8 : 4);
+    if (ring == 8)
+      i8_gemm_mid_kernel<8><<<dim3((unsigned)(per_xcd * 8)), dim3(256), mid_lds_bytes(8), stream>>>(a, tiles_m, tiles_n,
+                                                                                                   per_xcd);
+    else
+      i8_gemm_mid_kernel<4><<<dim3((unsigned)(per_xcd * 8)), dim3(256), mid_lds_bytes(4), stream>>>(a, tiles_m, tiles_n,
+                                                                                                   per_xcd);
+  } else if (large) {
     const int tiles_m = (int)((M + LM - 1) / LM), tiles_n = (int)((N + LN - 1) / LN);
     const int per_xcd = (tiles_m * tiles_n + 7) / 8;
     const char *ring_env = getenv("MI_I8_RING");  // development switch: stages in the LDS ring (3, 4 or 5)
     const int ring = ring_env ? atoi(ring_env) : 4;
     const size_t lds_bytes = (size_t)(ring == 5 ? 5 : ring == 3 ? 3 : 4) * 32 * 1024;
-    int epi = EPI_INT32;
-    if (rq) {
-      const bool q31 = rq->quant_mode == MI_RQ_QDM || rq->quant_mode == MI_RQ_TFLITE ||
-                       rq->quant_mode == MI_RQ_TFLITE_LSHIFT;
-      // the 32-bit fast path needs a right shift in [1, 31] on every channel; per-channel shifts are the
-      // caller's device array, so it is only taken for a scalar shift or when the caller vouches via the desc
-      epi = (q31 && rq->round_mode == MI_ROUND_HALF_AWAY_FROM_ZERO && rq->out_dtype == MI_DT_I8 &&
-             (rq->d_shift || (rq->shift >= 1 && rq->shift <= 31)))
-                ? EPI_Q31_HALF_AWAY
-                : EPI_GENERIC;
-    }
     dim3 grid((unsigned)(per_xcd * 8));
 #define MI_LARGE_I(E, LK_, NST)                                                                             \
   {                                                                                                         \
