@@ -91,8 +91,9 @@ typedef struct mi_a16mm_attr {
   int q_group_size;     /* getQGroupSize() or module::getQuantGroupSize(); 0 = per output channel */
   int out_dtype;        /* MI_DT_BF16, or MI_DT_F16 when module::isF16Modes() */
   int chip;             /* MI_CHIP_* */
-  int dynamic_quant;    /* MI_DQ_*: module::isDynamicQuantize() and getDqType().  MI_DQ_INT with 4-bit weights,
-                         * K % 128 == 0 and groups of 64 or k*128 is handled; anything else is MI_UNSUPPORTED */
+  int dynamic_quant;    /* MI_DQ_*: module::isDynamicQuantize() and getDqType().  MI_DQ_INT with K % 128 == 0 and
+                         * groups of 64 or k*128 (8-bit weights: up to 512) is handled; anything else is
+                         * MI_UNSUPPORTED */
 } mi_a16mm_attr;
 
 /* Replaces tpu::A16MatMulOp::init (A16MatMul.cpp:16-18).  inputs = {input, weight, scale, zp, bias|NULL}.
@@ -168,8 +169,8 @@ int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
  * A16MatMulOp::inference (A16MatMul.cpp:150-273).  Results are identical to n calls of mi_a16mm_launch.  The sets
  * must agree in K, weight_bits, q_group_size, dtype and chip; N may differ.  d_y[i] / d_y_f32[i] as above
  * (d_y_f32 itself may be NULL, as may any of its entries). */
-/* The dynamic-quantization flavour of the same product (A16MatMul.cpp:40-170, integer dq types, 4-bit weights):
- * activations are quantized per row and group to [-7, 7], the group products are integer MFMA sums, and the groups
+/* The dynamic-quantization flavour of the same product (A16MatMul.cpp:40-170, integer dq types): activations are
+ * quantized per row and group to [-7, 7] (4-bit weights) or [-127, 127] (8-bit), the group products are integer MFMA sums, and the groups
  * are added in the reference's order -- results are bit-identical to the reference's. */
 int mi_a16mm_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                        void *stream);

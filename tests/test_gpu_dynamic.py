@@ -18,7 +18,7 @@ def _device(cfg, dtype=clib.DT_BF16):
     tdt = torch.bfloat16 if dtype == clib.DT_BF16 else torch.float16
     w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"],
                      None if cfg.get("bias") is None else S.bf16_to_f32(cfg["bias"]),
-                     K=cfg["K"], N=cfg["N"], weight_bits=4, q_group_size=cfg["g"], dtype=dtype)
+                     K=cfg["K"], N=cfg["N"], weight_bits=cfg["bits"], q_group_size=cfg["g"], dtype=dtype)
     x = torch.from_numpy(cfg["x"].view(np.int16)).cuda().view(tdt)
     y32 = torch.empty((cfg["M"], cfg["N"]), dtype=torch.float32, device="cuda")
     y = M_.a16mm_dq_launch(w, x, y_f32=y32)
@@ -42,6 +42,26 @@ def test_dynamic_int_device_level(orc, M, K, N, g, bias):
     out, pre = _device(cfg)
     x, w, s, z, b = f32_valued_a16(cfg)
     want, want_pre = orc.a16matmul_dynamic(x, w, s, z, b, M=M, K=K, N=N, weight_bits=4, q_group_size=g)
+    assert np.array_equal(pre.view(np.uint32), want_pre.view(np.uint32))
+    assert np.array_equal(out, orc.f32_to_bf16(want))
+
+
+W8_CASES = [  # (M, K, N, g, bias): 8-bit weights, imax 127
+    (1, 512, 48, 64, False), (5, 1024, 100, 128, True), (16, 2048, 64, 256, False), (33, 1024, 40, 512, True),
+    (1, 4096, 1024, 128, False),
+]
+
+
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("M,K,N,g,bias", W8_CASES)
+def test_dynamic_int_w8_device_level(orc, M, K, N, g, bias, signed):
+    """uint8 weights with arbitrary zero points (what the quantizer writes for grouped weights) and int8 weights."""
+    cfg = S.w8a16(M, K, N, g, seed=M + K + N, bias=bias, signed=signed)
+    if not signed:
+        cfg["zp"] = np.random.default_rng(M + N).integers(0, 256, size=cfg["zp"].shape).astype(np.uint8)
+    out, pre = _device(cfg)
+    x, w, s, z, b = f32_valued_a16(cfg)
+    want, want_pre = orc.a16matmul_dynamic(x, w, s, z, b, M=M, K=K, N=N, weight_bits=8, q_group_size=g)
     assert np.array_equal(pre.view(np.uint32), want_pre.view(np.uint32))
     assert np.array_equal(out, orc.f32_to_bf16(want))
 
@@ -75,11 +95,13 @@ def test_dynamic_int_operator_level(orc):
 
 
 def test_dynamic_int_rejects_what_it_does_not_handle():
-    cfg = S.w4a16(1, 256, 16, 32, seed=1)
     import torch
-    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=256, N=16, weight_bits=4, q_group_size=32)
-    x = torch.zeros((1, 256), dtype=torch.bfloat16, device="cuda")
-    with pytest.raises(clib.BackendError) as e:
-        M_.a16mm_dq_launch(w, x)
-    assert e.value.code == clib.MI_UNSUPPORTED
-    w.destroy()
+    for cfg, bits in ((S.w4a16(1, 256, 16, 32, seed=1), 4),        # 32-wide groups
+                      (S.w8a16(1, 1024, 16, 1024, seed=1), 8)):    # 8-bit group too long to stay exact
+        w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=cfg["K"], N=16, weight_bits=bits,
+                         q_group_size=cfg["g"])
+        x = torch.zeros((1, cfg["K"]), dtype=torch.bfloat16, device="cuda")
+        with pytest.raises(clib.BackendError) as e:
+            M_.a16mm_dq_launch(w, x)
+        assert e.value.code == clib.MI_UNSUPPORTED
+        w.destroy()

@@ -362,10 +362,12 @@ int mi_a16mm_init(const mi_a16mm_attr *attr, mi_infer_param *p) {
   if (attr->dynamic_quant == MI_DQ_INT) {
     MI_REQUIRE(attr->q_group_size != 0, MI_BAD_ARGUMENT,
                "mi_a16mm_init: dynamic quantization needs a group size (A16MatMul.cpp:42-43)");
-    MI_REQUIRE(attr->weight_bits == 4 && attr->q_group_size > 0 && attr->K % 128 == 0 &&
-                   (attr->q_group_size == 64 || attr->q_group_size % 128 == 0),
+    MI_REQUIRE(attr->q_group_size > 0 && attr->K % 128 == 0 &&
+                   (attr->q_group_size == 64 || attr->q_group_size % 128 == 0) &&
+                   (attr->weight_bits == 4 || attr->q_group_size <= 512),
                MI_UNSUPPORTED,
-               "mi_a16mm_init: dynamic quantization is handled for 4-bit weights, K % 128 == 0, groups of 64 or k*128");
+               "mi_a16mm_init: dynamic quantization is handled for K % 128 == 0 and groups of 64 or k*128 (8-bit "
+               "weights: up to 512, where the reference's f32 group product stops being exact)");
   }
   MI_REQUIRE(attr->w_transpose, MI_UNSUPPORTED, "mi_a16mm_init: only w_transpose weights ([N,K]) are handled");
   MI_REQUIRE(attr->weight_bits == 4 || attr->weight_bits == 8, MI_UNSUPPORTED, "mi_a16mm_init: weight_bits");

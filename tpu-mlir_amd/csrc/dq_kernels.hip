@@ -1,8 +1,8 @@
-// tpu.A16MatMul with dynamic activation quantization, integer flavour (dq_type "INT4" / "INT8"), 4-bit weights:
+// tpu.A16MatMul with dynamic activation quantization, integer flavour (dq_type "INT4" / "INT8"), 4- and 8-bit weights:
 // lib/Dialect/Tpu/Interfaces/Common/A16MatMul.cpp:40-170.
 //
 // Per activation row and per quantization group along K the reference scales the activations by their own abs-max to
-// integers in [-imax, imax] (imax = 7 for 4-bit weights), multiplies them with the integer weights (q - zp) group by
+// integers in [-imax, imax] (imax = 7 for 4-bit weights, 127 for 8-bit), multiplies them with the integer weights (q - zp) group by
 // group, and adds   isum * (amax / imax) * scale[n][g]   into the output in group order, the bias after the first
 // group.  Every piece of that is deterministic, so this path is bit-exact:
 //
@@ -14,7 +14,10 @@
 //                    then the two fp32 multiplies of the reference; the per-group terms wait in LDS until 256 threads
 //                    add them up in group order.  Parallel over groups, sequential where the reference is.
 //
-// The packed weight set is the one the static kernels read (a16_kernels.hip).
+// The packed weight set is the one the static kernels read (a16_kernels.hip).  8-bit tiles hold unsigned bytes (int8
+// weights were flipped by 0x80 when packed) and, instead of an integer zero point, the exact float -(zp') * scale with
+// zp' the zero point in that unsigned domain: zp' = -nzs / scale comes back exactly, and the MFMA runs on the bytes
+// flipped to signed, so  sum_k code_k (w_k - zp) = mfma - (zp' - 128) * sum(codes).
 #include "a16_common.cuh"
 #include "internal.h"
 
@@ -32,8 +35,9 @@ constexpr int DQ_CHUNK = 128;  // groups whose terms fit the LDS buffer at once 
 __device__ __forceinline__ int dq_slot(int e) { return ((e & 1) << 1) | ((e & 2) << 1) | (e >> 2); }
 
 // ---- activations -> integer codes in fragment order
-// aq: [m_blocks][k_tiles][2][64 lanes][16 B]; as_t / asum_t: [m_blocks][G][16 rows]
-template <int DT>
+// aq, 4-bit: [m_blocks][k_tiles of 128][2][64 lanes][16 B]; 8-bit: [m_blocks][k_tiles of 64][64 lanes][16 B] with byte
+// 8 h + e of lane (row, kq) = k 32 h + 8 kq + e of the tile.  as_t / asum_t: [m_blocks][G][16 rows]
+template <int DT, int BITS>
 __global__ __launch_bounds__(256) void dq_act_kernel(const uint16_t *__restrict__ x, int64_t M, int64_t K, int g, int G,
                                                       float imax, int64_t k_tiles, uint8_t *__restrict__ aq,
                                                       float *__restrict__ as_t, int32_t *__restrict__ asum_t,
@@ -68,10 +72,18 @@ __global__ __launch_bounds__(256) void dq_act_kernel(const uint16_t *__restrict_
     if (live)
       code = (int)roundf(H::to_f32(x[m * K + kk]) / amax * imax);
     sum += code;
-    const int64_t kt = kk >> 7;
-    const int in_tile = (int)(kk & 127);
-    const int j = in_tile >> 5, kq = (in_tile >> 3) & 3, e = in_tile & 7;
-    const int64_t at = ((((mb * k_tiles + kt) * 2 + (j >> 1)) * 64) + kq * 16 + row) * 16 + (j & 1) * 8 + dq_slot(e);
+    int64_t at;
+    if constexpr (BITS == 4) {
+      const int64_t kt = kk >> 7;
+      const int in_tile = (int)(kk & 127);
+      const int j = in_tile >> 5, kq = (in_tile >> 3) & 3, e = in_tile & 7;
+      at = ((((mb * k_tiles + kt) * 2 + (j >> 1)) * 64) + kq * 16 + row) * 16 + (j & 1) * 8 + dq_slot(e);
+    } else {
+      const int64_t kt = kk >> 6;
+      const int in_tile = (int)(kk & 63);
+      const int h = in_tile >> 5, kq = (in_tile >> 3) & 3, e = in_tile & 7;
+      at = (((mb * k_tiles + kt) * 64) + kq * 16 + row) * 16 + h * 8 + e;
+    }
     aq[at] = (uint8_t)(int8_t)code;
   }
 #pragma unroll
@@ -86,7 +98,9 @@ __global__ __launch_bounds__(256) void dq_act_kernel(const uint16_t *__restrict_
 
 struct DqArgs {
   const u32x4 *qw;
-  const uint32_t *sz_t;
+  const uint32_t *sz_t;      // 4-bit
+  const uint16_t *scale_t;   // 8-bit
+  const float *nzs_t;        // 8-bit
   const float *bias;
   const u32x4 *aq;
   const float *as_t;
@@ -96,8 +110,9 @@ struct DqArgs {
   int64_t M, N;
   int64_t k_tiles;
   int G;
-  int unit_tiles;   // weight tiles per unit of work: g / 128 when g >= 128, else 1 (the unit then holds two groups)
-  int unit_groups;  // groups per unit: 1, or 2 when g == 64
+  int unit_tiles;   // weight tiles per unit of work.  4-bit: g / 128 when g >= 128, else 1 (the unit then holds two
+                    // groups); 8-bit: g / 64
+  int unit_groups;  // groups per unit: 1, or 2 for 4-bit weights with g == 64
   int chip;
 };
 
@@ -107,7 +122,7 @@ __device__ __forceinline__ void unpack_bytes(uint32_t d, int &lo, int &hi) {
   hi = (int)((d >> 4) & 0x0F0F0F0Fu);
 }
 
-template <int DT>
+template <int DT, int BITS>
 __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
   using H = Half16<DT>;
   extern __shared__ __attribute__((aligned(16))) float terms[];  // [groups of the chunk][16 rows][16 columns]
@@ -116,8 +131,8 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
   const int col = lane & 15, kq = lane >> 4;
   const int64_t rb = blockIdx.x, mb = blockIdx.y;
   const u32x4 *wq = a.qw + rb * a.k_tiles * 64 + lane;
-  const u32x4 *aq = a.aq + mb * a.k_tiles * 128 + lane;
-  const uint32_t *sz = a.sz_t + rb * a.G * 16 + col;
+  const u32x4 *aq = a.aq + mb * a.k_tiles * (BITS == 4 ? 128 : 64) + lane;
+  const int64_t qp = rb * a.G * 16 + col;  // this lane's channel in the [row block][group][16] parameter tables
   const float *as_p = a.as_t + mb * a.G * 16 + 4 * kq;
   const int32_t *asum_p = a.asum_t + mb * a.G * 16 + 4 * kq;
 
@@ -136,26 +151,41 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
       for (int t = 0; t < a.unit_tiles; ++t) {
         const int64_t kt = (int64_t)u * a.unit_tiles + t;
         const u32x4 w = wq[kt * 64];
-        const u32x4 a0 = aq[kt * 128], a1 = aq[kt * 128 + 64];
-        int lo[4], hi[4];
+        if constexpr (BITS == 8) {
+          const u32x4 a0 = aq[kt * 64];
+          const u32x4 ws = {w[0] ^ 0x80808080u, w[1] ^ 0x80808080u, w[2] ^ 0x80808080u, w[3] ^ 0x80808080u};
+          acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0), __builtin_bit_cast(i32x4, ws),
+                                                         acc[0], 0, 0, 0);
+        } else {
+          const u32x4 a0 = aq[kt * 128], a1 = aq[kt * 128 + 64];
+          int lo[4], hi[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          unpack_bytes(w[j], lo[j], hi[j]);
-        const i32x4 b0 = {lo[0], hi[0], lo[1], hi[1]}, b1 = {lo[2], hi[2], lo[3], hi[3]};
-        // k 0..63 of the tile, then k 64..127; with 64-wide groups these are two groups
-        acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0), b0, acc[0], 0, 0, 0);
-        if (a.unit_groups == 2)
-          acc[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1), b1, acc[1], 0, 0, 0);
-        else
-          acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1), b1, acc[0], 0, 0, 0);
+          for (int j = 0; j < 4; ++j)
+            unpack_bytes(w[j], lo[j], hi[j]);
+          const i32x4 b0 = {lo[0], hi[0], lo[1], hi[1]}, b1 = {lo[2], hi[2], lo[3], hi[3]};
+          // k 0..63 of the tile, then k 64..127; with 64-wide groups these are two groups
+          acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0), b0, acc[0], 0, 0, 0);
+          if (a.unit_groups == 2)
+            acc[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1), b1, acc[1], 0, 0, 0);
+          else
+            acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1), b1, acc[0], 0, 0, 0);
+        }
       }
       for (int h = 0; h < a.unit_groups; ++h) {
         const int gi = u * a.unit_groups + h;
         if (gi >= a.G)
           break;
-        const uint32_t szw = sz[(int64_t)gi * 16];
-        const float sc = H::to_f32((uint16_t)(szw >> 16));
-        const int zp = (int)(szw & 0xffu);
+        float sc;
+        int zp;  // what multiplies sum(codes)
+        if constexpr (BITS == 4) {
+          const uint32_t szw = a.sz_t[qp + (int64_t)gi * 16];
+          sc = H::to_f32((uint16_t)(szw >> 16));
+          zp = (int)(szw & 0xffu);
+        } else {
+          sc = H::to_f32(a.scale_t[qp + (int64_t)gi * 16]);
+          const float nzs = a.nzs_t[qp + (int64_t)gi * 16];
+          zp = (sc != 0.0f ? (int)rintf(-nzs / sc) : 128) - 128;  // exact: nzs is -(zp') * scale without rounding
+        }
         const f32x4 as4 = *(const f32x4 *)(as_p + (int64_t)gi * 16);
         const i32x4 sum4 = *(const i32x4 *)(asum_p + (int64_t)gi * 16);
         float *dst = terms + (size_t)(gi - u0 * a.unit_groups) * 256;
@@ -193,12 +223,15 @@ int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16
                   hipStream_t stream) {
   MI_REQUIRE(w && w->qweight && d_x && d_y, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: null argument");
   MI_REQUIRE(M >= 0 && M < (1 << 20), MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: M out of range");
-  MI_REQUIRE(w->bits == 4, MI_UNSUPPORTED, "mi_a16mm_dq_launch: only 4-bit weights are handled");
   MI_REQUIRE(w->g != 0, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: dynamic quantization needs a group size (A16MatMul.cpp:42)");
   const int g = w->g;
+  const int bits = w->bits;
   MI_REQUIRE((w->K % 128) == 0 && (g == 64 || g % 128 == 0), MI_UNSUPPORTED,
              "mi_a16mm_dq_launch: K must be a multiple of 128 and the group size 64 or a multiple of 128");
-  MI_REQUIRE((int64_t)g * 7 * 15 < (1 << 24), MI_UNSUPPORTED,
+  // (1 << (weight_bits - 1)) - 1, A16MatMul.cpp:53-54; the reference's f32 group product is exact only while the
+  // integer sums stay below 2^24
+  const float imax = bits == 4 ? 7.0f : 127.0f;
+  MI_REQUIRE((int64_t)g * (bits == 4 ? 7 * 15 : 127 * 255) < (1 << 24), MI_UNSUPPORTED,
              "mi_a16mm_dq_launch: group too long for the integer sums to stay exact in the reference's f32 product");
   if (M == 0)
     return MI_SUCCESS;
@@ -212,18 +245,28 @@ int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16
     return rc;
   float *as_t = (float *)(aq + aq_bytes);
   int32_t *asum_t = (int32_t *)(aq + aq_bytes + qp_bytes);
-  const float imax = 7.0f;  // (1 << (weight_bits - 1)) - 1, A16MatMul.cpp:53-54
   const int64_t waves = rows_padded * G;
   const bool f16 = w->dtype == MI_DT_F16;
-  if (f16)
-    dq_act_kernel<MI_DT_F16><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(
-        d_x, M, w->K, g, G, imax, w->k_tiles, aq, as_t, asum_t, rows_padded);
-  else
-    dq_act_kernel<MI_DT_BF16><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(
-        d_x, M, w->K, g, G, imax, w->k_tiles, aq, as_t, asum_t, rows_padded);
+#define MI_DQ_ACT(DT_, BITS_)                                                                      \
+  dq_act_kernel<DT_, BITS_><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(          \
+      d_x, M, w->K, g, G, imax, w->k_tiles, aq, as_t, asum_t, rows_padded)
+  if (bits == 4) {
+    if (f16)
+      MI_DQ_ACT(MI_DT_F16, 4);
+    else
+      MI_DQ_ACT(MI_DT_BF16, 4);
+  } else {
+    if (f16)
+      MI_DQ_ACT(MI_DT_F16, 8);
+    else
+      MI_DQ_ACT(MI_DT_BF16, 8);
+  }
+#undef MI_DQ_ACT
   DqArgs a;
   a.qw = (const u32x4 *)w->qweight;
   a.sz_t = w->sz_t;
+  a.scale_t = w->scale_t;
+  a.nzs_t = w->nzs_t;
   a.bias = w->bias;
   a.aq = (const u32x4 *)aq;
   a.as_t = as_t;
@@ -234,29 +277,34 @@ int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16
   a.N = w->N;
   a.k_tiles = w->k_tiles;
   a.G = G;
-  a.unit_tiles = g >= 128 ? g / 128 : 1;
-  a.unit_groups = g == 64 ? 2 : 1;
+  a.unit_tiles = bits == 4 ? (g >= 128 ? g / 128 : 1) : g / 64;
+  a.unit_groups = (bits == 4 && g == 64) ? 2 : 1;
   a.chip = w->chip;
   const int chunk_groups = G < DQ_CHUNK ? G : DQ_CHUNK;
   const size_t lds_bytes = (size_t)(chunk_groups + 1) * 1024;
   dim3 grid((unsigned)w->row_blocks, (unsigned)m_blocks);
-  if (f16) {
-    static bool attr_set = false;
-    if (!attr_set) {
-      (void)hipFuncSetAttribute((const void *)dq_gemm_kernel<MI_DT_F16>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024);
-      attr_set = true;
-    }
-    dq_gemm_kernel<MI_DT_F16><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);
-  } else {
-    static bool attr_set = false;
-    if (!attr_set) {
-      (void)hipFuncSetAttribute((const void *)dq_gemm_kernel<MI_DT_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024);
-      attr_set = true;
-    }
-    dq_gemm_kernel<MI_DT_BF16><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);
+#define MI_DQ_GEMM(DT_, BITS_)                                                                                   \
+  {                                                                                                             \
+    static bool attr_set = false;                                                                               \
+    if (!attr_set) {                                                                                            \
+      (void)hipFuncSetAttribute((const void *)dq_gemm_kernel<DT_, BITS_>,                                       \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                        \
+      attr_set = true;                                                                                          \
+    }                                                                                                           \
+    dq_gemm_kernel<DT_, BITS_><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);                            \
   }
+  if (bits == 4) {
+    if (f16)
+      MI_DQ_GEMM(MI_DT_F16, 4)
+    else
+      MI_DQ_GEMM(MI_DT_BF16, 4)
+  } else {
+    if (f16)
+      MI_DQ_GEMM(MI_DT_F16, 8)
+    else
+      MI_DQ_GEMM(MI_DT_BF16, 8)
+  }
+#undef MI_DQ_GEMM
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;
 }

@@ -1,7 +1,9 @@
 // Device scratch buffers owned by the library, one per (device, stream, purpose).  Work on one stream is ordered, so
 // consecutive calls can share a buffer; calls on different streams never do.  A buffer only grows; growing it
 // synchronizes the stream, frees the old buffer and allocates a new one, which cannot happen while the stream is
-// being captured into a graph: run a shape once eagerly before capturing it.
+// being captured into a graph: run a shape once eagerly before capturing it.  A graph captured on a stream holds the
+// address of that stream's buffer: a later, larger call on the same stream replaces the buffer and with it invalidates
+// such a graph (capture the largest shape last, or keep graphs and larger eager calls on different streams).
 #include <map>
 #include <mutex>
 #include <tuple>
