@@ -80,6 +80,41 @@ def test_int8_and_requant_argument_errors():
     assert np.array_equal(M.requant_int(v, quant_mode=clib.RQ_MULTIPLIER_SHIFT, multiplier=1, rshift=1), v)
 
 
+def test_weight_producer_and_blob_argument_errors():
+    """Argument checks of the weight producers, the packed-blob import and the dynamic-quantization launch happen on
+    the host, before anything touches a GPU."""
+    L = clib.lib()
+    assert L.mi_a16_quantize(None, None, None, None, None, None, None, None) == clib.MI_BAD_ARGUMENT
+    assert L.mi_llm_unpack(0, 4, None, None, 8, 8, 1, None, None) == clib.MI_BAD_ARGUMENT
+    assert L.mi_a16mm_dq_launch(None, None, 1, None, None, None) == clib.MI_BAD_ARGUMENT
+    w = np.zeros((64, 8), np.float32)
+    with pytest.raises(M.BackendError) as e:
+        M.a16_quantize(w, weight_bits=3, q_group_size=0)
+    assert e.value.code == clib.MI_UNSUPPORTED
+    with pytest.raises(M.BackendError) as e:
+        M.a16_quantize(w, weight_bits=4, q_group_size=48)   # 64 % 48 != 0
+    assert e.value.code == clib.MI_BAD_ARGUMENT
+    with pytest.raises(M.BackendError) as e:
+        M.a16_quantize(np.zeros((63, 8), np.float32), weight_bits=4, q_group_size=0)  # odd K cannot pack nibbles
+    assert e.value.code == clib.MI_BAD_ARGUMENT
+    with pytest.raises(M.BackendError) as e:
+        M.llm_unpack(M.PACK_AWQ, 8, np.zeros((64, 2), np.int32), np.zeros((1, 2), np.int32), K=64, N=8)
+    assert e.value.code == clib.MI_UNSUPPORTED                # AWQ is 4-bit only
+    with pytest.raises(M.BackendError) as e:
+        M.llm_unpack(M.PACK_GPTQ, 4, np.zeros((8, 16), np.int32), np.zeros((1, 3), np.int32), K=64, N=16)
+    assert e.value.code == clib.MI_BAD_ARGUMENT               # qzeros does not match N
+    # blobs: magic, truncated header, inconsistent header -- all refused before a device is needed
+    hdr = np.zeros(80, np.uint8)
+    for blob in (hdr, hdr[:10]):
+        with pytest.raises(M.BackendError) as e:
+            M.A16Weight.from_blob(blob.tobytes())
+        assert e.value.code == clib.MI_BAD_ARGUMENT
+    hdr[:8] = np.frombuffer(b"MIA16W1\0", np.uint8)
+    with pytest.raises(M.BackendError) as e:
+        M.A16Weight.from_blob(hdr.tobytes())                  # right magic, all-zero fields
+    assert e.value.code == clib.MI_BAD_ARGUMENT
+
+
 def test_compare_metrics():
     cmp = pkg("compare")
     a = np.array([1.0, 2.0, 3.0, 4.0])
