@@ -81,7 +81,9 @@ typedef struct mi_infer_param {
 /* ============================================================================ */
 /* dynamic activation quantization of tpu.A16MatMul (A16MatMul.cpp:40-170): MI_DQ_INT covers dq_type "INT4" and
  * "INT8", whose arithmetic differs only through the weight width (imax = 2^(weight_bits-1) - 1, :53-54) */
-enum { MI_DQ_NONE = 0, MI_DQ_INT = 1, MI_DQ_F8E4M3 = 2, MI_DQ_F4 = 3 };
+enum { MI_DQ_NONE = 0, MI_DQ_INT = 1, MI_DQ_F8E4M3 = 2, MI_DQ_F4 = 3,
+       /* tpu.MatMul takes imax from the type name (MatMul.cpp:449-453): */
+       MI_DQ_INT8 = 4 /* imax 127 */, MI_DQ_INT4 = 5 /* imax 7 */ };
 
 typedef struct mi_a16mm_attr {
   int64_t M;            /* product of the input's leading dims (A16MatMul.cpp:31-35); may change per call */
@@ -133,6 +135,27 @@ size_t mi_a16_weight_bytes(const mi_a16_weight *w);
 size_t mi_a16_weight_export_size(const mi_a16_weight *w);
 int mi_a16_weight_export(const mi_a16_weight *w, void *blob, size_t capacity);
 int mi_a16_weight_import(mi_a16_weight **out, const void *blob, size_t size);
+
+/* ---- tpu.MatMul with both operands quantized dynamically -------------------------------------------------- */
+/* The module::isDynamicQuantize() branch of tpu::MatMulOp::inference for a non-weight right operand
+ * (lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:447-597), integer dq types, batch 1: per group of K every left row
+ * and every right column is scaled by its own abs-max to [-imax, imax], the group products are integer MFMA sums,
+ * rescaled and added in group order.  No bias, no relu (the reference applies none on this branch).  Results are
+ * bit-identical to the reference's while its f32 group product is exact (group * imax^2 < 2^24), which is checked.
+ * K and the group size must be multiples of 64. */
+typedef struct mi_matmul_dq_attr {
+  int64_t M, K, N;
+  int right_transpose;  /* right operand stored [N, K] instead of [K, N] */
+  int q_group_size;     /* getQGroupSize() or module::getQuantGroupSize(); -1 = K */
+  int dq_type;          /* MI_DQ_INT8 / MI_DQ_INT4 */
+  int out_dtype;        /* MI_DT_BF16, or MI_DT_F16 when module::isF16Modes() */
+} mi_matmul_dq_attr;
+/* inputs = {left [M,K], right}, outputs = {[M,N]}, all f32-valued */
+int mi_matmul_dq_inference(const mi_matmul_dq_attr *attr, mi_infer_param *p);
+/* device level: 16-bit operands and output in HBM, optional fp32 result before rounding */
+int mi_matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
+                        int64_t N, int q_group_size, int dq_type, int dtype, uint16_t *d_y, float *d_y_f32,
+                        void *stream);
 
 /* ---- weight producers (the compile-time side of tpu.A16MatMul), computed on the GPU, host arrays in and out ---- */
 typedef struct mi_a16_quant_desc {

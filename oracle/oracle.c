@@ -605,6 +605,85 @@ int orc_a16matmul_dynamic(const orc_a16mm_attr *a, const float *const *inputs, f
   return 0;
 }
 
+/* MatMul.cpp:447-597, INT8 / INT4, batch 1 */
+int orc_matmul_dynamic(const float *left, const float *right, int64_t M, int64_t K, int64_t N, int right_transpose,
+                       int q_group_size, int imax_i, int out_dtype, float *output, float *y_preround) {
+  if (!left || !right || !output || M <= 0 || K <= 0 || N <= 0 || (imax_i != 127 && imax_i != 7))
+    return 1;
+  int64_t g = q_group_size;
+  if (g == -1)
+    g = K; /* :465-466 */
+  if (g <= 0)
+    return 1;
+  const float imax = (float)imax_i;
+  const int64_t group_num = (K + g - 1) / g; /* :467 */
+  float *ql = (float *)malloc(sizeof(float) * (size_t)(M * g));
+  float *qr = (float *)malloc(sizeof(float) * (size_t)(N * g));
+  float *lmax = (float *)malloc(sizeof(float) * (size_t)M);
+  float *rmax = (float *)malloc(sizeof(float) * (size_t)N);
+  if (!ql || !qr || !lmax || !rmax) {
+    free(ql);
+    free(qr);
+    free(lmax);
+    free(rmax);
+    return 1;
+  }
+  for (int64_t i = 0; i < M * N; i++)
+    output[i] = 0.0f;
+  int inexact = 0;
+  for (int64_t gi = 0; gi < group_num; gi++) {
+    /* :478-505 abs-max per left row and per right column, floor 1e-8 */
+    for (int64_t row = 0; row < M; row++) {
+      lmax[row] = (float)1e-8;
+      for (int64_t col = 0; col < g && gi * g + col < K; col++) {
+        const float v = fabsf(left[row * K + gi * g + col]);
+        lmax[row] = lmax[row] > v ? lmax[row] : v;
+      }
+    }
+    for (int64_t n = 0; n < N; n++) {
+      rmax[n] = (float)1e-8;
+      for (int64_t col = 0; col < g && gi * g + col < K; col++) {
+        const int64_t k = gi * g + col;
+        const float v = fabsf(right_transpose ? right[n * K + k] : right[k * N + n]);
+        rmax[n] = rmax[n] > v ? rmax[n] : v;
+      }
+    }
+    /* :507-566 codes */
+    for (int64_t row = 0; row < M; row++)
+      for (int64_t col = 0; col < g; col++)
+        ql[row * g + col] = (gi * g + col < K) ? roundf(left[row * K + gi * g + col] / lmax[row] * imax) : 0.0f;
+    for (int64_t n = 0; n < N; n++)
+      for (int64_t col = 0; col < g; col++) {
+        const int64_t k = gi * g + col;
+        qr[n * g + col] = (k < K) ? roundf((right_transpose ? right[n * K + k] : right[k * N + n]) / rmax[n] * imax) : 0.0f;
+      }
+    /* :567-583 group product and rescaled accumulation */
+    for (int64_t row = 0; row < M; row++)
+      for (int64_t n = 0; n < N; n++) {
+        int64_t s = 0, peak = 0;
+        for (int64_t k = 0; k < g; k++) {
+          s += (int64_t)ql[row * g + k] * (int64_t)qr[n * g + k];
+          const int64_t m = s < 0 ? -s : s;
+          peak = m > peak ? m : peak;
+        }
+        if (peak >= (1 << 24))
+          inexact = 1;
+        output[row * N + n] += (float)s * (lmax[row] / imax) * (rmax[n] / imax);
+      }
+  }
+  free(ql);
+  free(qr);
+  free(lmax);
+  free(rmax);
+  if (inexact)
+    return 2;
+  if (y_preround)
+    memcpy(y_preround, output, sizeof(float) * (size_t)(M * N));
+  for (int64_t i = 0; i < M * N; i++)
+    output[i] = round_out(output[i], out_dtype, 0); /* :585-590 */
+  return 0;
+}
+
 /* ======================================================================== */
 /* tpu.MatMul (quantised)                                                    */
 /* ======================================================================== */

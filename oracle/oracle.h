@@ -26,6 +26,7 @@
  *   orc_cast                     numpy closed forms per branch (tests/test_oracle_cast.py)
  *   orc_a16matmul_dynamic        lossless-activation cases against orc_a16matmul, exact power-of-two row
  *                                scaling, half-step error bound, group order (tests/test_oracle_dynamic.py)
+ *   orc_matmul_dynamic           the same four properties, on both operands (tests/test_oracle_dynamic.py)
  *   orc_a16_quantize             on-grid weights are recovered exactly, |w - dequant(q)| <= scale/2 inside the
  *                                clamp range, closed-form scale/zp, nibble order via the A16MatMul dequantizer
  *                                (tests/test_oracle_packers.py)
@@ -223,6 +224,14 @@ int orc_cast(const orc_cast_attr *attr, const float *input, float *output, int64
  * added group by group in fp32, bias after the first group.  inputs as for orc_a16matmul; the 8-bit weight is
  * read as the reference reads it, `int(weight[i])`.  Returns 0, 1 (bad arguments), 2 (outside the exact domain). */
 int orc_a16matmul_dynamic(const orc_a16mm_attr *a, const float *const *inputs, float *output, float *y_preround);
+
+/* tpu.MatMul with both operands quantized dynamically (lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:447-597, dq_type
+ * "INT8": imax 127, "INT4": imax 7; batch 1): left [M, K], right [K, N] or [N, K] when right_transpose, both
+ * f32-valued; per group of K every left row and every right column is scaled by its own abs-max.  The branch adds no
+ * bias and applies no relu; the output is rounded to out_dtype.  Returns 0, 1 (bad arguments), 2 (group sums reach
+ * 2^24, where the reference's f32 product stops being exact). */
+int orc_matmul_dynamic(const float *left, const float *right, int64_t M, int64_t K, int64_t N, int right_transpose,
+                       int q_group_size, int imax, int out_dtype, float *output, float *y_preround);
 
 /* ---- weight producers (compile-time side of tpu.A16MatMul) ------------------- */
 /* A16MatMulAdjust, lib/Dialect/Tpu/Canonicalize/A16MatMul.cpp:270-429, static uint8-zero-point variant:

@@ -226,6 +226,25 @@ def a16matmul_dynamic(x, weight, scale, zp, bias, *, M, K, N, weight_bits, q_gro
     return out, pre
 
 
+def matmul_dynamic(left, right, *, right_transpose=False, q_group_size, imax=127, out_dtype=OUT_BF16):
+    """tpu.MatMul with both operands quantized dynamically (INT8: imax 127, INT4: imax 7); returns (output, pre)."""
+    left, right = _f32(left), _f32(right)
+    M, K = left.shape
+    N = right.shape[0] if right_transpose else right.shape[1]
+    out = np.empty((M, N), dtype=np.float32)
+    pre = np.empty((M, N), dtype=np.float32)
+    L = lib()
+    L.orc_matmul_dynamic.restype = C.c_int
+    rc = L.orc_matmul_dynamic(_p(left, C.c_float), _p(right, C.c_float), C.c_int64(M), C.c_int64(K), C.c_int64(N),
+                              C.c_int(int(right_transpose)), C.c_int(q_group_size), C.c_int(imax), C.c_int(out_dtype),
+                              _p(out, C.c_float), _p(pre, C.c_float))
+    if rc == 2:
+        raise ValueError("orc_matmul_dynamic: group sums leave the range the reference's f32 product is exact in")
+    if rc != 0:
+        raise RuntimeError("orc_matmul_dynamic failed")
+    return out, pre
+
+
 def matmul_int8(x, right, bias, multi, *, M, K, N, right_transpose=False, input_zp=0, right_zp=0,
                 do_relu=False, relu_limit=-1.0, cv18xx=False, quant_mode=RQ_MULTIPLIER_SHIFT, fuse_rq=False,
                 multipliers=(1,), rshifts=(0,), out_zp=0, out_kind=0, out_bits=8, out_unsigned=False,

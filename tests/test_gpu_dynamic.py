@@ -105,3 +105,47 @@ def test_dynamic_int_rejects_what_it_does_not_handle():
             M_.a16mm_dq_launch(w, x)
         assert e.value.code == clib.MI_UNSUPPORTED
         w.destroy()
+
+
+# ---- tpu.MatMul with both operands quantized (MatMul.cpp:447-597) ------------------------------------------------
+MM_CASES = [  # (M, K, N, g, right_transpose, dq_type)
+    (1, 128, 16, 64, True, "DQ_INT8"), (5, 512, 100, 128, False, "DQ_INT8"), (37, 1024, 70, 256, True, "DQ_INT8"),
+    (16, 256, 48, -1, False, "DQ_INT8"), (20, 2048, 33, 64, False, "DQ_INT4"), (128, 128, 128, 128, True, "DQ_INT4"),
+    (3, 8704, 24, 64, True, "DQ_INT8"),  # 136 groups: more than one LDS chunk of terms
+]
+
+
+@pytest.mark.parametrize("M,K,N,g,rt,dq", MM_CASES)
+def test_matmul_dynamic_device_level(orc, M, K, N, g, rt, dq):
+    import torch
+    rng = np.random.default_rng(M + K + N)
+    lb = S.bf16_round((rng.standard_normal((M, K)) * rng.uniform(0.2, 3.0, size=(M, 1))).astype(np.float32))
+    rb = S.bf16_round(rng.standard_normal((N, K) if rt else (K, N)).astype(np.float32))
+    left = torch.from_numpy(lb.view(np.int16)).cuda().view(torch.bfloat16)
+    right = torch.from_numpy(rb.view(np.int16)).cuda().view(torch.bfloat16)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.matmul_dq_launch(left, right, right_transpose=rt, q_group_size=g, dq_type=getattr(clib, dq), y_f32=y32)
+    torch.cuda.synchronize()
+    want, want_pre = orc.matmul_dynamic(S.bf16_to_f32(lb), S.bf16_to_f32(rb), right_transpose=rt, q_group_size=g,
+                                        imax=127 if dq == "DQ_INT8" else 7)
+    assert np.array_equal(y32.cpu().numpy().view(np.uint32), want_pre.view(np.uint32))
+    assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), orc.f32_to_bf16(want))
+
+
+def test_matmul_dynamic_operator_level_and_rejections(orc):
+    rng = np.random.default_rng(77)
+    M, K, N, g = 6, 256, 40, 64
+    left = S.bf16_to_f32(S.bf16_round(rng.standard_normal((M, K)).astype(np.float32)))
+    right = S.bf16_to_f32(S.bf16_round(rng.standard_normal((K, N)).astype(np.float32)))
+    y = M_.matmul_dq(left, right, q_group_size=g)
+    want, _ = orc.matmul_dynamic(left, right, q_group_size=g)
+    assert np.array_equal(y, want)
+    with pytest.raises(clib.BackendError) as e:
+        M_.matmul_dq(left, right, q_group_size=g, dq_type=clib.DQ_F8E4M3)
+    assert e.value.code == clib.MI_UNSUPPORTED
+    with pytest.raises(clib.BackendError) as e:
+        M_.matmul_dq(left, right, q_group_size=48)
+    assert e.value.code == clib.MI_UNSUPPORTED
+    with pytest.raises(clib.BackendError) as e:  # 2048 x 127^2 >= 2^24: outside the reference's exact range
+        M_.matmul_dq(np.zeros((1, 2048), np.float32), np.zeros((2048, 4), np.float32), q_group_size=2048)
+    assert e.value.code == clib.MI_UNSUPPORTED

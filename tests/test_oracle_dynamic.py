@@ -120,3 +120,77 @@ def test_outside_exact_domain_is_reported(orc):
     with pytest.raises(ValueError):
         orc.a16matmul_dynamic(x, wf, np.ones((N, 1), np.float32), np.zeros((N, 1), np.float32), None, M=1, K=K, N=N,
                               weight_bits=8, q_group_size=g)
+
+
+# ---- tpu.MatMul with both operands quantized (MatMul.cpp:447-597) ------------------------------------------------
+def _on_grid(rng, rows, K, g, imax):
+    """[rows, K] values = integer codes x a power of two per (row, group), every (row, group) reaching imax."""
+    ints = rng.integers(-imax, imax + 1, size=(rows, K // g, g))
+    ints[:, :, 0] = imax
+    c = np.float32(2.0) ** rng.integers(-5, 3, size=(rows, K // g, 1)).astype(np.float32)
+    return (ints * c).reshape(rows, K).astype(np.float32)
+
+
+@pytest.mark.parametrize("imax,rt", [(127, True), (127, False), (7, True)])
+def test_matmul_dynamic_lossless_operands_give_the_exact_product(orc, imax, rt):
+    rng = np.random.default_rng(imax + rt)
+    M, K, N, g = 5, 256, 12, 64
+    left, right_nk = _on_grid(rng, M, K, g, imax), _on_grid(rng, N, K, g, imax)
+    right = right_nk if rt else np.ascontiguousarray(right_nk.T)
+    _, pre = orc.matmul_dynamic(left, right, right_transpose=rt, q_group_size=g, imax=imax)
+    exact = left.astype(np.float64) @ right_nk.astype(np.float64).T
+    mag = np.abs(left).astype(np.float64) @ np.abs(right_nk).astype(np.float64).T
+    assert np.all(np.abs(pre - exact) <= mag * 2.0 ** -21)
+
+
+def test_matmul_dynamic_power_of_two_scaling_of_rows_and_columns(orc):
+    rng = np.random.default_rng(8)
+    M, K, N, g = 4, 128, 6, 64
+    left = S.bf16_to_f32(S.bf16_round(rng.standard_normal((M, K)).astype(np.float32)))
+    right = S.bf16_to_f32(S.bf16_round(rng.standard_normal((K, N)).astype(np.float32)))
+    _, pre = orc.matmul_dynamic(left, right, q_group_size=g)
+    fl = np.float32([0.5, 1, 4, 32])[:, None]
+    fr = np.float32([2, 1, 0.25, 8, 16, 0.125])[None, :]
+    _, pre2 = orc.matmul_dynamic(left * fl, right * fr, q_group_size=g)
+    assert np.array_equal(pre2, pre * fl * fr)
+
+
+def test_matmul_dynamic_half_step_bound(orc):
+    rng = np.random.default_rng(9)
+    M, K, N, g, imax = 6, 256, 10, 128, 127
+    left = S.bf16_to_f32(S.bf16_round(rng.standard_normal((M, K)).astype(np.float32)))
+    right = S.bf16_to_f32(S.bf16_round(rng.standard_normal((N, K)).astype(np.float32)))
+    _, pre = orc.matmul_dynamic(left, right, right_transpose=True, q_group_size=g, imax=imax)
+    exact = left.astype(np.float64) @ right.astype(np.float64).T
+    G = K // g
+    lm = np.abs(left).reshape(M, G, g).max(axis=2).astype(np.float64)
+    rm = np.abs(right).reshape(N, G, g).max(axis=2).astype(np.float64)
+    la = np.abs(left).reshape(M, G, g).sum(axis=2)
+    ra = np.abs(right).reshape(N, G, g).sum(axis=2)
+    dl, dr = lm / (2 * imax), rm / (2 * imax)
+    # |sum (a + da)(b + db) - sum a b| <= da sum|b| + db sum|a| + g da db, per group
+    bound = np.einsum("mg,ng->mn", dl, ra) + np.einsum("mg,ng->mn", la, dr) + g * np.einsum("mg,ng->mn", dl, dr)
+    err = np.abs(pre - exact)
+    assert np.all(err <= bound * 1.001 + 1e-6)
+    assert err.max() > 1e-4
+
+
+def test_matmul_dynamic_single_group_closed_form(orc):
+    rng = np.random.default_rng(12)
+    M, K, N, g, imax = 3, 192, 5, 64, np.float32(127)
+    left = np.zeros((M, K), np.float32)
+    right = np.zeros((K, N), np.float32)
+    ls = S.bf16_to_f32(S.bf16_round(rng.standard_normal((M, g)).astype(np.float32)))
+    rs = S.bf16_to_f32(S.bf16_round(rng.standard_normal((g, N)).astype(np.float32)))
+    left[:, g:2 * g], right[g:2 * g, :] = ls, rs
+    _, pre = orc.matmul_dynamic(left, right, q_group_size=g, imax=127)
+
+    def codes(v, mx):
+        r = (v / mx * imax).astype(np.float32)
+        return (np.sign(r) * np.floor(np.abs(r).astype(np.float64) + 0.5)).astype(np.int64)
+    lmax = np.maximum(np.abs(ls).max(axis=1), np.float32(1e-8)).astype(np.float32)
+    rmax = np.maximum(np.abs(rs).max(axis=0), np.float32(1e-8)).astype(np.float32)
+    isum = codes(ls, lmax[:, None]) @ codes(rs, rmax[None, :])
+    t = (isum.astype(np.float32) * (lmax / imax)[:, None]).astype(np.float32)
+    want = (t * (rmax / imax)[None, :]).astype(np.float32)
+    assert np.array_equal(pre, want)

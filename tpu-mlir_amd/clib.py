@@ -18,7 +18,7 @@ EXPORTS = [
     "mi_version", "mi_last_error", "mi_device_count",
     "mi_a16mm_init", "mi_a16mm_inference", "mi_a16mm_deinit",
     "mi_a16_weight_create", "mi_a16_weight_destroy", "mi_a16_weight_bytes", "mi_a16mm_launch",
-    "mi_a16mm_launch_group", "mi_a16mm_dq_launch",
+    "mi_a16mm_launch_group", "mi_a16mm_dq_launch", "mi_matmul_dq_launch", "mi_matmul_dq_inference",
     "mi_a16_weight_export_size", "mi_a16_weight_export", "mi_a16_weight_import", "mi_a16_quantize", "mi_llm_unpack",
     "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
     "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
@@ -41,7 +41,7 @@ class InferParam(C.Structure):
                 ("handle", C.c_void_p)]
 
 
-DQ_NONE, DQ_INT, DQ_F8E4M3, DQ_F4 = 0, 1, 2, 3
+DQ_NONE, DQ_INT, DQ_F8E4M3, DQ_F4, DQ_INT8, DQ_INT4 = 0, 1, 2, 3, 4, 5
 
 
 class A16Attr(C.Structure):
@@ -53,6 +53,11 @@ class A16Attr(C.Structure):
 class A16WeightDesc(C.Structure):
     _fields_ = [("K", C.c_int64), ("N", C.c_int64), ("weight_bits", C.c_int), ("weight_signed", C.c_int),
                 ("q_group_size", C.c_int), ("dtype", C.c_int), ("chip", C.c_int)]
+
+
+class MatMulDqAttr(C.Structure):
+    _fields_ = [("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64), ("right_transpose", C.c_int),
+                ("q_group_size", C.c_int), ("dq_type", C.c_int), ("out_dtype", C.c_int)]
 
 
 class A16QuantDesc(C.Structure):
@@ -139,6 +144,8 @@ def lib():
                                     C.c_void_p, C.c_void_p]
         L.mi_a16_weight_destroy.restype = None
         L.mi_a16mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi_matmul_dq_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int,
+                                          C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_dq_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_launch_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int64,
                                             C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_void_p]

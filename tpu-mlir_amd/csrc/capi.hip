@@ -948,4 +948,55 @@ int mi_cast_inference(const mi_cast_attr *a, mi_infer_param *p) {
   return MI_SUCCESS;
 }
 
+// ---- tpu.MatMul, both operands quantized dynamically (MatMul.cpp:447-597) -------------------------------------
+int mi_matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
+                        int64_t N, int q_group_size, int dq_type, int dtype, uint16_t *d_y, float *d_y_f32,
+                        void *stream) {
+  MI_REQUIRE(dq_type == MI_DQ_INT8 || dq_type == MI_DQ_INT4, MI_UNSUPPORTED,
+             "mi_matmul_dq_launch: only the INT8 / INT4 dynamic-quantization types are handled");
+  return matmul_dq_launch(d_left, d_right, right_transpose, M, K, N, q_group_size, dq_type == MI_DQ_INT8 ? 127 : 7,
+                          dtype, d_y, d_y_f32, (hipStream_t)stream);
+}
+
+int mi_matmul_dq_inference(const mi_matmul_dq_attr *a, mi_infer_param *p) {
+  MI_REQUIRE(a && p && p->inputs && p->n_inputs >= 2 && p->inputs[0] && p->inputs[1] && p->outputs &&
+                 p->n_outputs >= 1 && p->outputs[0],
+             MI_BAD_ARGUMENT, "mi_matmul_dq_inference: null argument");
+  MI_REQUIRE(a->M >= 0 && a->K > 0 && a->N > 0, MI_BAD_ARGUMENT, "mi_matmul_dq_inference: bad shape");
+  MI_REQUIRE(a->dq_type == MI_DQ_INT8 || a->dq_type == MI_DQ_INT4, MI_UNSUPPORTED,
+             "mi_matmul_dq_inference: only the INT8 / INT4 dynamic-quantization types are handled");
+  MI_REQUIRE(a->out_dtype == MI_DT_BF16 || a->out_dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_matmul_dq_inference: out_dtype");
+  const int64_t g = a->q_group_size == -1 ? a->K : a->q_group_size;
+  MI_REQUIRE(g > 0, MI_BAD_ARGUMENT, "mi_matmul_dq_inference: dynamic quantization needs a group size");
+  MI_REQUIRE((a->K % 64) == 0 && (g % 64) == 0 && (a->K % g) == 0, MI_UNSUPPORTED,
+             "mi_matmul_dq_inference: K and the group size must be multiples of 64");
+  if (a->M == 0)
+    return MI_SUCCESS;
+  MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_matmul_dq_inference: no GPU visible");
+  const bool f16 = a->out_dtype == MI_DT_F16;
+  const size_t nl = (size_t)a->M * a->K, nr = (size_t)a->K * a->N, no = (size_t)a->M * a->N;
+  // the operands are activations in the 16-bit type (f32-valued on the host side)
+  std::vector<uint16_t> hl(nl), hr(nr), ho(no);
+  for (size_t i = 0; i < nl; ++i)
+    hl[i] = f16 ? h_f32_to_f16(p->inputs[0][i]) : h_f32_to_bf16(p->inputs[0][i]);
+  for (size_t i = 0; i < nr; ++i)
+    hr[i] = f16 ? h_f32_to_f16(p->inputs[1][i]) : h_f32_to_bf16(p->inputs[1][i]);
+  DevBuf dl, dr, dy;
+  int rc;
+  if ((rc = dl.reserve(nl * 2)) || (rc = dr.reserve(nr * 2)) || (rc = dy.reserve(no * 2)))
+    return rc;
+  MI_HIP(hipMemcpy(dl.ptr, hl.data(), nl * 2, hipMemcpyHostToDevice));
+  MI_HIP(hipMemcpy(dr.ptr, hr.data(), nr * 2, hipMemcpyHostToDevice));
+  rc = matmul_dq_launch((const uint16_t *)dl.ptr, (const uint16_t *)dr.ptr, a->right_transpose, a->M, a->K, a->N,
+                        a->q_group_size, a->dq_type == MI_DQ_INT8 ? 127 : 7, a->out_dtype, (uint16_t *)dy.ptr, nullptr,
+                        nullptr);
+  if (rc)
+    return rc;
+  MI_HIP(hipDeviceSynchronize());
+  MI_HIP(hipMemcpy(ho.data(), dy.ptr, no * 2, hipMemcpyDeviceToHost));
+  for (size_t i = 0; i < no; ++i)
+    p->outputs[0][i] = f16 ? h_f16_to_f32(ho[i]) : h_bf16_to_f32(ho[i]);
+  return MI_SUCCESS;
+}
+
 }  // extern "C"

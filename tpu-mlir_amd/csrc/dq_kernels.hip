@@ -219,6 +219,164 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
   }
 }
 
+// ---- tpu.MatMul with both operands quantized dynamically (lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:447-597,
+// integer dq types, batch 1).  Both operands go through dq_act_kernel (a [K, N] right operand is transposed first), and
+// the product kernel is the one above with a second fragment stream in place of the weight tiles and the right
+// column's amax / imax in place of the weight scale.  The reference adds no bias and applies no relu on this branch.
+__global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t *__restrict__ src, uint16_t *__restrict__ dst,
+                                                           int64_t rows, int64_t cols) {
+  __shared__ uint16_t tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  const int64_t c0 = (int64_t)blockIdx.x * 32, r0 = (int64_t)blockIdx.y * 32;
+  for (int i = ty; i < 32; i += 8)
+    if (r0 + i < rows && c0 + tx < cols)
+      tile[i][tx] = src[(r0 + i) * cols + c0 + tx];
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8)
+    if (c0 + i < cols && r0 + tx < rows)
+      dst[(c0 + i) * rows + r0 + tx] = tile[tx][i];
+}
+
+struct Dq2Args {
+  const u32x4 *aq_l, *aq_r;   // [m_blocks][k_tiles of 64][64 lanes][16 B], [n_blocks][...]
+  const float *as_l, *as_r;   // [m_blocks][G][16], [n_blocks][G][16]: amax / imax
+  uint16_t *y;
+  float *y32;
+  int64_t M, N;
+  int64_t k_tiles;
+  int G, unit_tiles;  // tiles of 64 per group
+};
+
+template <int DT>
+__global__ __launch_bounds__(DQ_WAVES * 64) void dq2_gemm_kernel(Dq2Args a) {
+  extern __shared__ __attribute__((aligned(16))) float terms[];  // [groups of the chunk][16 rows][16 columns]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, kq = lane >> 4;
+  const int64_t nb = blockIdx.x, mb = blockIdx.y;
+  const u32x4 *al = a.aq_l + mb * a.k_tiles * 64 + lane;
+  const u32x4 *ar = a.aq_r + nb * a.k_tiles * 64 + lane;
+  const float *asl = a.as_l + mb * a.G * 16 + 4 * kq;
+  const float *asr = a.as_r + nb * a.G * 16 + col;
+  float out = 0.0f;
+  const int64_t n_out = nb * 16 + (tid & 15), m_out = mb * 16 + (tid >> 4);
+  const bool owns = tid < 256 && n_out < a.N && m_out < a.M;
+  for (int g0 = 0; g0 < a.G; g0 += DQ_CHUNK) {
+    const int g1 = (g0 + DQ_CHUNK) < a.G ? (g0 + DQ_CHUNK) : a.G;
+    for (int gi = g0 + wave; gi < g1; gi += DQ_WAVES) {
+      i32x4 acc = {0, 0, 0, 0};
+      for (int t = 0; t < a.unit_tiles; ++t) {
+        const int64_t kt = (int64_t)gi * a.unit_tiles + t;
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, al[kt * 64]),
+                                                    __builtin_bit_cast(i32x4, ar[kt * 64]), acc, 0, 0, 0);
+      }
+      const f32x4 l4 = *(const f32x4 *)(asl + (int64_t)gi * 16);
+      const float r1 = asr[(int64_t)gi * 16];
+      float *dst = terms + (size_t)(gi - g0) * 256;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float t = (float)acc[r];  // below 2^24 (checked on the host): exact
+        t = t * l4[r];            // MatMul.cpp:577-581, left to right
+        t = t * r1;
+        dst[(4 * kq + r) * 16 + col] = t;
+      }
+    }
+    __syncthreads();
+    if (owns)
+      for (int gi = g0; gi < g1; ++gi)
+        out = out + terms[(size_t)(gi - g0) * 256 + tid];
+    __syncthreads();
+  }
+  if (owns) {
+    const int64_t o = m_out * a.N + n_out;
+    if (a.y32)
+      a.y32[o] = out;
+    a.y[o] = round_out16<DT, MI_CHIP_BM168X>(out);
+  }
+}
+
+int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
+                     int64_t N, int q_group_size, int imax_i, int dtype, uint16_t *d_y, float *d_y32,
+                     hipStream_t stream) {
+  MI_REQUIRE(d_left && d_right && d_y, MI_BAD_ARGUMENT, "mi_matmul_dq_launch: null argument");
+  MI_REQUIRE(M >= 0 && M < (1 << 20) && N > 0 && N < (1 << 20) && K > 0, MI_BAD_ARGUMENT,
+             "mi_matmul_dq_launch: bad shape");
+  MI_REQUIRE(imax_i == 127 || imax_i == 7, MI_UNSUPPORTED, "mi_matmul_dq_launch: integer dq types only (imax 127 / 7)");
+  MI_REQUIRE(dtype == MI_DT_BF16 || dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_matmul_dq_launch: dtype");
+  const int64_t g = q_group_size == -1 ? K : q_group_size;  // MatMul.cpp:465-466
+  MI_REQUIRE(g > 0, MI_BAD_ARGUMENT, "mi_matmul_dq_launch: dynamic quantization needs a group size");
+  MI_REQUIRE((K % 64) == 0 && (g % 64) == 0 && (K % g) == 0, MI_UNSUPPORTED,
+             "mi_matmul_dq_launch: K and the group size must be multiples of 64, K a multiple of the group size");
+  MI_REQUIRE(g * imax_i * imax_i < (1 << 24), MI_UNSUPPORTED,
+             "mi_matmul_dq_launch: group too long for the integer sums to stay exact in the reference's f32 product");
+  if (M == 0)
+    return MI_SUCCESS;
+  const int G = (int)(K / g);
+  const int64_t k_tiles = K / 64;
+  const int64_t m_blocks = (M + 15) / 16, n_blocks = (N + 15) / 16;
+  const size_t al_bytes = (size_t)m_blocks * 16 * K, ar_bytes = (size_t)n_blocks * 16 * K;
+  const size_t sl_bytes = (size_t)m_blocks * 16 * G * 4, sr_bytes = (size_t)n_blocks * 16 * G * 4;
+  const size_t tr_bytes = right_transpose ? 0 : (((size_t)N * K * 2 + 255) & ~(size_t)255);
+  uint8_t *ws = nullptr;
+  int rc = stream_workspace(stream, WS_DYNAMIC_QUANT, tr_bytes + al_bytes + ar_bytes + 2 * (sl_bytes + sr_bytes), false,
+                            (void **)&ws);
+  if (rc != MI_SUCCESS)
+    return rc;
+  uint16_t *rt = (uint16_t *)ws;
+  uint8_t *aq_l = ws + tr_bytes, *aq_r = aq_l + al_bytes;
+  float *as_l = (float *)(aq_r + ar_bytes), *as_r = as_l + sl_bytes / 4;
+  int32_t *sum_l = (int32_t *)(as_r + sr_bytes / 4), *sum_r = sum_l + sl_bytes / 4;  // written, not read
+  const uint16_t *right_nk = d_right;
+  if (!right_transpose) {
+    transpose16_kernel<<<dim3((unsigned)((N + 31) / 32), (unsigned)((K + 31) / 32)), dim3(256), 0, stream>>>(d_right, rt,
+                                                                                                        K, N);
+    right_nk = rt;
+  }
+  const float imax = (float)imax_i;
+  const bool f16 = dtype == MI_DT_F16;
+  const int64_t wl = m_blocks * 16 * G, wr = n_blocks * 16 * G;
+  if (f16) {
+    dq_act_kernel<MI_DT_F16, 8><<<dim3((unsigned)((wl + 3) / 4)), dim3(256), 0, stream>>>(
+        d_left, M, K, (int)g, G, imax, k_tiles, aq_l, as_l, sum_l, m_blocks * 16);
+    dq_act_kernel<MI_DT_F16, 8><<<dim3((unsigned)((wr + 3) / 4)), dim3(256), 0, stream>>>(
+        right_nk, N, K, (int)g, G, imax, k_tiles, aq_r, as_r, sum_r, n_blocks * 16);
+  } else {
+    dq_act_kernel<MI_DT_BF16, 8><<<dim3((unsigned)((wl + 3) / 4)), dim3(256), 0, stream>>>(
+        d_left, M, K, (int)g, G, imax, k_tiles, aq_l, as_l, sum_l, m_blocks * 16);
+    dq_act_kernel<MI_DT_BF16, 8><<<dim3((unsigned)((wr + 3) / 4)), dim3(256), 0, stream>>>(
+        right_nk, N, K, (int)g, G, imax, k_tiles, aq_r, as_r, sum_r, n_blocks * 16);
+  }
+  Dq2Args a;
+  a.aq_l = (const u32x4 *)aq_l;
+  a.aq_r = (const u32x4 *)aq_r;
+  a.as_l = as_l;
+  a.as_r = as_r;
+  a.y = d_y;
+  a.y32 = d_y32;
+  a.M = M;
+  a.N = N;
+  a.k_tiles = k_tiles;
+  a.G = G;
+  a.unit_tiles = (int)(g / 64);
+  const int chunk_groups = G < DQ_CHUNK ? G : DQ_CHUNK;
+  const size_t lds_bytes = (size_t)(chunk_groups + 1) * 1024;
+  dim3 grid((unsigned)n_blocks, (unsigned)m_blocks);
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void *)dq2_gemm_kernel<MI_DT_F16>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              160 * 1024);
+    (void)hipFuncSetAttribute((const void *)dq2_gemm_kernel<MI_DT_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              160 * 1024);
+    attr_set = true;
+  }
+  if (f16)
+    dq2_gemm_kernel<MI_DT_F16><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);
+  else
+    dq2_gemm_kernel<MI_DT_BF16><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);
+  MI_HIP(hipGetLastError());
+  return MI_SUCCESS;
+}
+
 int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                   hipStream_t stream) {
   MI_REQUIRE(w && w->qweight && d_x && d_y, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: null argument");

@@ -80,6 +80,10 @@ int stream_workspace(hipStream_t st, int purpose, size_t bytes, bool zeroed, voi
 int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                   hipStream_t stream);
 
+int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
+                     int64_t N, int q_group_size, int imax, int dtype, uint16_t *d_y, float *d_y32,
+                     hipStream_t stream);
+
 // weight producers (quant_kernels.hip); arguments are validated by the callers
 int a16_quantize(const mi_a16_quant_desc *d, const float *h_w_kn, void *h_weight, uint16_t *h_scale16,
                  float *h_scale_f32, uint8_t *h_zp, int *sign_out, int *weight_signed_out);

@@ -285,6 +285,39 @@ def llm_unpack(mode, bits, qweight, qzeros, *, K, N):
     return q, zp
 
 
+def matmul_dq(left, right, *, right_transpose=False, q_group_size, dq_type=clib.DQ_INT8, out_dtype=DT_BF16):
+    """tpu.MatMul with both operands quantized dynamically, interpreter convention (float32 numpy in and out)."""
+    left, right = _f32(left), _f32(right)
+    M, K = left.shape
+    N = right.shape[0] if right_transpose else right.shape[1]
+    attr = clib.MatMulDqAttr(M, K, N, int(right_transpose), q_group_size, dq_type, out_dtype)
+    y = np.empty((M, N), dtype=np.float32)
+    p = _Param([left, right], [y])
+    check(clib.lib().mi_matmul_dq_inference(C.byref(attr), C.byref(p.c)))
+    return y
+
+
+def matmul_dq_launch(left, right, *, right_transpose=False, q_group_size, dq_type=clib.DQ_INT8, y=None, y_f32=None,
+                     stream=None):
+    """Device level: left [M, K], right [K, N] ([N, K] when right_transpose) as bf16 / f16 CUDA tensors."""
+    import torch
+    if not (left.is_cuda and right.is_cuda and left.dtype == right.dtype and left.is_contiguous()
+            and right.is_contiguous() and left.dtype in (torch.bfloat16, torch.float16) and left.dim() == 2
+            and right.dim() == 2):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "matmul_dq_launch: operands must be contiguous 2-D CUDA tensors "
+                                "of one 16-bit float type")
+    M, K = left.shape
+    N = right.shape[0] if right_transpose else right.shape[1]
+    if (right.shape[1] if right_transpose else right.shape[0]) != K:
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "matmul_dq_launch: inner dimensions differ")
+    if y is None:
+        y = torch.empty((M, N), dtype=left.dtype, device=left.device)
+    dt = DT_F16 if left.dtype == torch.float16 else DT_BF16
+    check(clib.lib().mi_matmul_dq_launch(_dptr(left), _dptr(right), int(right_transpose), M, K, N, q_group_size,
+                                         dq_type, dt, _dptr(y), _dptr(y_f32), _stream_ptr(stream)))
+    return y
+
+
 def a16mm_dq_launch(w, x, y=None, y_f32=None, stream=None):
     """As a16mm_launch, with the reference's dynamic integer activation quantization (4-bit weights)."""
     import torch
