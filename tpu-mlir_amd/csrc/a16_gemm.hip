@@ -457,16 +457,21 @@ bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M) {
   const int g = w->g;
   // whole LDS stages, at most one group per MFMA k-step, groups that do not straddle a weight tile
   const bool group_ok = g == 0 || (g >= tile_k && g % tile_k == 0) || (g < tile_k && tile_k % g == 0 && g >= 32);
-  // Up to 16 rows the skinny kernel makes one pass over the weights; beyond that it would make one per 16 rows.  From
-  // 8 rows on, large matrices are already better off here (measured with weights streaming from HBM: 11008 x 4096 at
-  // M = 8: 13.0 us against 14.8; 4096 x 4096: 8.1 against 7.5), because a workgroup of the skinny kernel stages all of
-  // x in LDS and runs at low occupancy once x has several rows.
+  // Up to 16 rows the skinny kernel makes one pass over the weights; beyond that it would make one per 16 rows.  Below
+  // that its time grows with the number of rows (every workgroup reads all of x) while this kernel's hardly does, so
+  // large matrices cross over earlier.  Measured with weights streaming from HBM, skinny / tiled in us:
+  //   4096 x 4096    M = 8: 5.8 / 8.1    M = 16:  7.1 /  8.9      -> skinny up to 16 rows
+  //   11008 x 4096   M = 8: 11.3 / 13.0  M = 12: 12.9 / 13.4   M = 16: 14.9 / 13.5
+  //   4096 x 11008   M = 6: 12.2 / 11.4  M = 8: 13.9 / 12.2    (long K: few, long workgroups in the skinny kernel)
+  //   32000 x 4096   M = 6: 22.6 / 22.9  M = 8: 25.1 / 22.2
   const char *e = getenv("MI_A16_GEMM_MIN_M");  // development / test switch
+  const int64_t nk = w->N * w->K;
   bool rows_ok;
   if (e)
     rows_ok = M >= atoll(e) && M > 1;
   else
-    rows_ok = M >= 17 || (M >= 8 && w->N * w->K >= (int64_t(1) << 25));
+    rows_ok = M >= 17 || (M >= 13 && nk >= (int64_t(1) << 25)) || (M >= 8 && nk >= (int64_t(1) << 26)) ||
+              (M >= 6 && w->K >= 8192 && nk >= (int64_t(1) << 25));
   return rows_ok && (w->K % GEMM_KS) == 0 && group_ok;
 }
 
