@@ -788,7 +788,7 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
   MI_REQUIRE(ws && n >= 1 && n <= MAX_SEG, MI_BAD_ARGUMENT,
              "mi_a16mm_launch_group: between 1 and " + std::to_string(MAX_SEG) + " weight sets per launch");
   MI_REQUIRE(d_x && d_ys, MI_BAD_ARGUMENT, "mi_a16mm_launch: null activation or output pointer");
-  MI_REQUIRE(M >= 0 && M < (1 << 20), MI_BAD_ARGUMENT, "mi_a16mm_launch: M out of range");
+  MI_REQUIRE(M >= 0 && M <= 65535 * 16, MI_BAD_ARGUMENT, "mi_a16mm_launch: M out of range");
   const mi_a16_weight *w = ws[0];
   int64_t total_rb = 0;
   SkinnyArgs a;

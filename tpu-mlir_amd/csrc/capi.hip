@@ -330,7 +330,7 @@ int mi_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qze
   const int ratio = 32 / bits;
   MI_REQUIRE(K > 0 && N > 0 && G > 0 && K % ratio == 0 && N % ratio == 0 && K % 2 == 0, MI_BAD_ARGUMENT,
              "mi_llm_unpack: K and N must be multiples of the values per int32");
-  MI_REQUIRE(G <= 65535 && K <= 65535 * 2, MI_UNSUPPORTED, "mi_llm_unpack: shape too large");
+  MI_REQUIRE(G <= 65535 && (bits == 4 ? K / 2 : K) <= 65535, MI_UNSUPPORTED, "mi_llm_unpack: shape too large");
   MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_llm_unpack: no GPU visible");
   return llm_unpack(mode, bits, qweight, qzeros, K, N, G, weight, zp);
 }
