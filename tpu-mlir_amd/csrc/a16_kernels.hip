@@ -787,15 +787,16 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
                      float *const *d_y32s, hipStream_t stream) {
   MI_REQUIRE(ws && n >= 1 && n <= MAX_SEG, MI_BAD_ARGUMENT,
              "mi_a16mm_launch_group: between 1 and " + std::to_string(MAX_SEG) + " weight sets per launch");
-  MI_REQUIRE(d_x && d_ys, MI_BAD_ARGUMENT, "mi_a16mm_launch: null activation or output pointer");
   MI_REQUIRE(M >= 0 && M <= 65535 * 16, MI_BAD_ARGUMENT, "mi_a16mm_launch: M out of range");
+  // no rows: nothing to read or write (an empty tensor's data pointer may well be null)
+  MI_REQUIRE(M == 0 || (d_x && d_ys), MI_BAD_ARGUMENT, "mi_a16mm_launch: null activation or output pointer");
   const mi_a16_weight *w = ws[0];
   int64_t total_rb = 0;
   SkinnyArgs a;
   for (int i = 0; i < MAX_SEG; ++i) {
     const int q = i < n ? i : 0;  // unused slots repeat the first set; the kernel never selects them
     MI_REQUIRE(ws[q] && ws[q]->qweight, MI_BAD_ARGUMENT, "mi_a16mm_launch: weight set is empty");
-    MI_REQUIRE(d_ys[q], MI_BAD_ARGUMENT, "mi_a16mm_launch: null output pointer");
+    MI_REQUIRE(M == 0 || d_ys[q], MI_BAD_ARGUMENT, "mi_a16mm_launch: null output pointer");
     const mi_a16_weight *v = ws[q];
     MI_REQUIRE(v->K == w->K && v->bits == w->bits && v->g == w->g && v->dtype == w->dtype && v->chip == w->chip,
                MI_BAD_ARGUMENT,

@@ -298,9 +298,9 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq2_gemm_kernel(Dq2Args a) {
 int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
                      int64_t N, int q_group_size, int imax_i, int dtype, uint16_t *d_y, float *d_y32,
                      hipStream_t stream) {
-  MI_REQUIRE(d_left && d_right && d_y, MI_BAD_ARGUMENT, "mi_matmul_dq_launch: null argument");
   MI_REQUIRE(M >= 0 && M <= 65535 * 16 && N > 0 && N <= 65535 * 16 && K > 0, MI_BAD_ARGUMENT,
              "mi_matmul_dq_launch: bad shape");
+  MI_REQUIRE(M == 0 || (d_left && d_right && d_y), MI_BAD_ARGUMENT, "mi_matmul_dq_launch: null argument");
   MI_REQUIRE(imax_i == 127 || imax_i == 7, MI_UNSUPPORTED, "mi_matmul_dq_launch: integer dq types only (imax 127 / 7)");
   MI_REQUIRE(dtype == MI_DT_BF16 || dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_matmul_dq_launch: dtype");
   const int64_t g = q_group_size == -1 ? K : q_group_size;  // MatMul.cpp:465-466
@@ -379,8 +379,8 @@ int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_
 
 int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                   hipStream_t stream) {
-  MI_REQUIRE(w && w->qweight && d_x && d_y, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: null argument");
   MI_REQUIRE(M >= 0 && M <= 65535 * 16, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: M out of range");
+  MI_REQUIRE(w && w->qweight && (M == 0 || (d_x && d_y)), MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: null argument");
   MI_REQUIRE(w->g != 0, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: dynamic quantization needs a group size (A16MatMul.cpp:42)");
   const int g = w->g;
   const int bits = w->bits;

@@ -932,14 +932,15 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
                 const int32_t *d_bias, int64_t M, int64_t K, int64_t N, int64_t input_zp, int64_t right_zp,
                 int do_relu, int64_t relu_limit, const mi_requant_desc *rq, void *d_out, int32_t *d_acc,
                 hipStream_t stream) {
-  MI_REQUIRE(d_a && d_b && (d_out || d_acc), MI_BAD_ARGUMENT, "mi_i8mm_launch: null operand");
   MI_REQUIRE(M >= 0 && K > 0 && N > 0 && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), MI_BAD_ARGUMENT,
              "mi_i8mm_launch: bad shape");
+  // no rows: nothing to read or write (an empty tensor's data pointer may well be null)
+  MI_REQUIRE(M == 0 || (d_a && d_b && (d_out || d_acc)), MI_BAD_ARGUMENT, "mi_i8mm_launch: null operand");
   if (rq) {
     int rc = check_rq(rq, "mi_i8mm_launch");
     if (rc)
       return rc;
-    MI_REQUIRE(d_out, MI_BAD_ARGUMENT, "mi_i8mm_launch: requant needs an output pointer");
+    MI_REQUIRE(M == 0 || d_out, MI_BAD_ARGUMENT, "mi_i8mm_launch: requant needs an output pointer");
   }
   if (M == 0)
     return MI_SUCCESS;
