@@ -185,12 +185,56 @@ def case_i8():
                         want_int=want_int.astype(np.int32))
 
 
+def case_producers_and_dynamic():
+    """Weight producers and the dynamic-quantization matmuls: every output here is integer / bit-pattern work or a
+    fully ordered fp32 computation, so the GPU has to reproduce the files bit for bit."""
+    rng = np.random.default_rng(301)
+    # quantizer: 4-bit grouped asymmetric, 4-bit per channel, 8-bit grouped symmetric, 8-bit per channel (signed)
+    w = (rng.standard_normal((256, 40)) * 0.05).astype(np.float32)
+    out = {"w_kn": w}
+    for tag, kw in (("w4_g64", dict(bits=4, g=64)), ("w4_pc", dict(bits=4, g=0)),
+                    ("w8_g128_sym", dict(bits=8, g=128, symmetric=True)), ("w8_pc", dict(bits=8, g=0))):
+        r = O.a16_quantize(w, **kw)
+        out["q_" + tag] = r["weight"]
+        out["scale16_" + tag] = r["scale16"]
+        out["zp_" + tag] = r["zp"]
+        out["flags_" + tag] = np.array([r["sign"], r["weight_signed"]], dtype=np.int32)
+    np.savez_compressed(os.path.join(HERE, "case_quantizer.npz"), **out)
+    # GPTQ / AWQ unpack of random words
+    K, N, G = 128, 48, 2
+    qw_g = rng.integers(-2 ** 31, 2 ** 31, size=(K // 8, N), dtype=np.int64).astype(np.int32)
+    qw_a = rng.integers(-2 ** 31, 2 ** 31, size=(K, N // 8), dtype=np.int64).astype(np.int32)
+    qz = rng.integers(-2 ** 31, 2 ** 31, size=(G, N // 8), dtype=np.int64).astype(np.int32)
+    gq, gz = O.llm_unpack(O.PACK_GPTQ, 4, qw_g, qz, K, N)
+    aq, az = O.llm_unpack(O.PACK_AWQ, 4, qw_a, qz, K, N)
+    np.savez_compressed(os.path.join(HERE, "case_llm_unpack.npz"), qweight_gptq=qw_g, qweight_awq=qw_a, qzeros=qz,
+                        gptq_weight=gq, gptq_zp=gz, awq_weight=aq, awq_zp=az)
+    # dynamic integer quantization: A16MatMul (4- and 8-bit weights) and MatMul with two activations
+    out = {}
+    for tag, cfg in (("w4", S.w4a16(5, 512, 40, 128, seed=302, bias=True)),
+                     ("w8", S.w8a16(3, 256, 24, 64, seed=303, signed=False))):
+        x, wf, sc, z, b = f32_valued_a16(cfg)
+        y, pre = O.a16matmul_dynamic(x, wf, sc, z, b, M=cfg["M"], K=cfg["K"], N=cfg["N"], weight_bits=cfg["bits"],
+                                     q_group_size=cfg["g"])
+        out.update({tag + "_x": cfg["x"], tag + "_weight": cfg["weight"], tag + "_scale": cfg["scale"],
+                    tag + "_zp": cfg["zp"],
+                    tag + "_bias": np.zeros(0, np.uint16) if cfg.get("bias") is None else cfg["bias"],
+                    tag + "_meta": np.array([cfg["M"], cfg["K"], cfg["N"], cfg["g"], cfg["bits"]], dtype=np.int64),
+                    tag + "_want_bf16": O.f32_to_bf16(y), tag + "_want_pre": pre})
+    left = S.bf16_round(rng.standard_normal((7, 256)).astype(np.float32))
+    right = S.bf16_round(rng.standard_normal((256, 20)).astype(np.float32))
+    y, pre = O.matmul_dynamic(S.bf16_to_f32(left), S.bf16_to_f32(right), q_group_size=64, imax=127)
+    out.update(mm_left=left, mm_right=right, mm_want_bf16=O.f32_to_bf16(y), mm_want_pre=pre)
+    np.savez_compressed(os.path.join(HERE, "case_dynamic.npz"), **out)
+
+
 if __name__ == "__main__":
     kat_right_shift_round()
     kat_mbqm()
     kat_float16()
     case_a16()
     case_i8()
+    case_producers_and_dynamic()
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print("%-40s %7d bytes" % (f, os.path.getsize(os.path.join(HERE, f))))

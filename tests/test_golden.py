@@ -100,7 +100,73 @@ def test_oracle_reproduces_requant_cases(orc):
     assert np.array_equal(got.astype(np.int32), d["want_int"])
 
 
+QUANT_TAGS = {"w4_g64": dict(bits=4, g=64), "w4_pc": dict(bits=4, g=0), "w8_g128_sym": dict(bits=8, g=128, symmetric=True),
+              "w8_pc": dict(bits=8, g=0)}
+
+
+def test_oracle_reproduces_producer_and_dynamic_cases(orc):
+    d = _load("case_quantizer.npz")
+    for tag, kw in QUANT_TAGS.items():
+        r = orc.a16_quantize(d["w_kn"], **kw)
+        assert np.array_equal(r["weight"], d["q_" + tag]) and np.array_equal(r["scale16"], d["scale16_" + tag])
+        assert np.array_equal(r["zp"], d["zp_" + tag])
+        assert [int(r["sign"]), int(r["weight_signed"])] == d["flags_" + tag].tolist()
+    u = _load("case_llm_unpack.npz")
+    K, N = u["qweight_awq"].shape[0], u["qweight_gptq"].shape[1]
+    q, z = orc.llm_unpack(orc.PACK_GPTQ, 4, u["qweight_gptq"], u["qzeros"], K, N)
+    assert np.array_equal(q, u["gptq_weight"]) and np.array_equal(z, u["gptq_zp"])
+    q, z = orc.llm_unpack(orc.PACK_AWQ, 4, u["qweight_awq"], u["qzeros"], K, N)
+    assert np.array_equal(q, u["awq_weight"]) and np.array_equal(z, u["awq_zp"])
+    y = _load("case_dynamic.npz")
+    for tag in ("w4", "w8"):
+        cfg = _a16_cfg({k[len(tag) + 1:]: y[k] for k in y.files if k.startswith(tag + "_")})
+        x, wf, sc, zp, b = f32_valued_a16(cfg)
+        out, pre = orc.a16matmul_dynamic(x, wf, sc, zp, b, M=cfg["M"], K=cfg["K"], N=cfg["N"],
+                                         weight_bits=cfg["bits"], q_group_size=cfg["g"])
+        assert np.array_equal(pre, y[tag + "_want_pre"]) and np.array_equal(orc.f32_to_bf16(out), y[tag + "_want_bf16"])
+    out, pre = orc.matmul_dynamic(S.bf16_to_f32(y["mm_left"]), S.bf16_to_f32(y["mm_right"]), q_group_size=64, imax=127)
+    assert np.array_equal(pre, y["mm_want_pre"])
+
+
 # ----------------------------------------------------------------------------------------------- GPU
+@pytest.mark.gpu
+def test_gpu_producers_and_dynamic_against_fixtures():
+    """Bit-exact, with nothing but numpy on the expected side."""
+    import torch
+    M_ = pkg()
+    clib = pkg("clib")
+    d = _load("case_quantizer.npz")
+    for tag, kw in QUANT_TAGS.items():
+        r = M_.a16_quantize(d["w_kn"], weight_bits=kw["bits"], q_group_size=kw["g"], symmetric=kw.get("symmetric", False))
+        assert np.array_equal(r["weight"].view(np.uint8), d["q_" + tag]), tag
+        assert np.array_equal(r["scale_bits"], d["scale16_" + tag]) and np.array_equal(r["zp"], d["zp_" + tag]), tag
+        assert [int(r["sign"]), int(r["weight_signed"])] == d["flags_" + tag].tolist()
+    u = _load("case_llm_unpack.npz")
+    K, N = u["qweight_awq"].shape[0], u["qweight_gptq"].shape[1]
+    q, z = M_.llm_unpack(M_.PACK_GPTQ, 4, u["qweight_gptq"], u["qzeros"], K=K, N=N)
+    assert np.array_equal(q, u["gptq_weight"]) and np.array_equal(z, u["gptq_zp"])
+    q, z = M_.llm_unpack(M_.PACK_AWQ, 4, u["qweight_awq"], u["qzeros"], K=K, N=N)
+    assert np.array_equal(q, u["awq_weight"]) and np.array_equal(z, u["awq_zp"])
+    y = _load("case_dynamic.npz")
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda().view(torch.bfloat16)
+    for tag in ("w4", "w8"):
+        cfg = _a16_cfg({k[len(tag) + 1:]: y[k] for k in y.files if k.startswith(tag + "_")})
+        w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"],
+                         None if cfg["bias"] is None else S.bf16_to_f32(cfg["bias"]),
+                         K=cfg["K"], N=cfg["N"], weight_bits=cfg["bits"], q_group_size=cfg["g"])
+        y32 = torch.empty((cfg["M"], cfg["N"]), dtype=torch.float32, device="cuda")
+        out = M_.a16mm_dq_launch(w, dev(cfg["x"]), y_f32=y32)
+        torch.cuda.synchronize()
+        assert np.array_equal(y32.cpu().numpy().view(np.uint32), y[tag + "_want_pre"].view(np.uint32)), tag
+        assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), y[tag + "_want_bf16"]), tag
+        w.destroy()
+    y32 = torch.empty(y["mm_want_pre"].shape, dtype=torch.float32, device="cuda")
+    out = M_.matmul_dq_launch(dev(y["mm_left"]), dev(y["mm_right"]), q_group_size=64, dq_type=clib.DQ_INT8, y_f32=y32)
+    torch.cuda.synchronize()
+    assert np.array_equal(y32.cpu().numpy().view(np.uint32), y["mm_want_pre"].view(np.uint32))
+    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), y["mm_want_bf16"])
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", A16_CASES)
 def test_gpu_a16_against_fixture(name, monkeypatch):
