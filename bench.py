@@ -231,6 +231,30 @@ def bench_dynamic_quant(pkg, S, torch, steps=40):
                     "GBps": round(nbytes / sec / 1e9, 1)})
         for w in ws:
             w.destroy()
+    # the float code types: E2M1 codes in 4-bit and E4M3 codes in 8-bit weights (weights: random codes, scales as above)
+    K = N = 4096
+    for case, bits, dq, cfg in (("w4_g128_dynamic_f4", 4, "DQ_F4", S.w4a16(1, K, N, 128, seed=34)),
+                                ("w8_g128_dynamic_f8e4m3", 8, "DQ_F8E4M3", S.w8a16(1, K, N, 128, seed=35, signed=False))):
+        if bits == 8:
+            cfg["weight"] = cfg["weight"] & np.uint8(0x77)  # finite E4M3 codes
+        cfg["zp"] = np.zeros_like(cfg["zp"])
+        copies = 16
+        ws = [pkg.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=K, N=N, weight_bits=bits, q_group_size=128)
+              for _ in range(copies)]
+        for M in (1, 16):
+            x = _dev_bf16(torch, S.bf16_round(np.random.default_rng(6).standard_normal((M, K), dtype=np.float32)))
+            y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+
+            def run():
+                for w in ws:
+                    pkg.a16mm_dq_launch(w, x, y, dq_type=getattr(pkg, dq))
+
+            sec = _time_launches(torch, run, max(3, steps // copies), warmup=2) / copies
+            nbytes = S.w4_gemv_bytes(M, K, N, 128) + (N * K // 2 if bits == 8 else 0)
+            out.append({"case": case, "M": M, "K": K, "N": N, "us": round(sec * 1e6, 2),
+                        "GBps": round(nbytes / sec / 1e9, 1)})
+        for w in ws:
+            w.destroy()
     return out
 
 

@@ -93,9 +93,9 @@ typedef struct mi_a16mm_attr {
   int q_group_size;     /* getQGroupSize() or module::getQuantGroupSize(); 0 = per output channel */
   int out_dtype;        /* MI_DT_BF16, or MI_DT_F16 when module::isF16Modes() */
   int chip;             /* MI_CHIP_* */
-  int dynamic_quant;    /* MI_DQ_*: module::isDynamicQuantize() and getDqType().  MI_DQ_INT with K % 128 == 0 and
-                         * groups of 64 or k*128 (8-bit weights: up to 512) is handled; anything else is
-                         * MI_UNSUPPORTED */
+  int dynamic_quant;    /* MI_DQ_*: module::isDynamicQuantize() and getDqType().  MI_DQ_INT, MI_DQ_F8E4M3 (8-bit
+                         * weights) and MI_DQ_F4 (4-bit weights) with K % 128 == 0 and groups of 64 or k*128 (integer
+                         * codes in 8-bit weights: up to 512) are handled; anything else is MI_UNSUPPORTED */
 } mi_a16mm_attr;
 
 /* Replaces tpu::A16MatMulOp::init (A16MatMul.cpp:16-18).  inputs = {input, weight, scale, zp, bias|NULL}.
@@ -138,16 +138,17 @@ int mi_a16_weight_import(mi_a16_weight **out, const void *blob, size_t size);
 
 /* ---- tpu.MatMul with both operands quantized dynamically -------------------------------------------------- */
 /* The module::isDynamicQuantize() branch of tpu::MatMulOp::inference for a non-weight right operand
- * (lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:447-597), integer dq types, batch 1: per group of K every left row
- * and every right column is scaled by its own abs-max to [-imax, imax], the group products are integer MFMA sums,
- * rescaled and added in group order.  No bias, no relu (the reference applies none on this branch).  Results are
- * bit-identical to the reference's while its f32 group product is exact (group * imax^2 < 2^24), which is checked.
- * K and the group size must be multiples of 64. */
+ * (lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:447-597), batch 1: per group of K every left row and every right
+ * column is scaled by its own abs-max to [-imax, imax] and rounded to the code type, the group products are matrix-core
+ * sums, rescaled and added in group order.  No bias, no relu (the reference applies none on this branch).  Integer
+ * types and F4: results are bit-identical to the reference's while its f32 group product is exact (group * imax^2
+ * < 2^24 in code units), which is checked.  F8E4M3: exact products, fp32 group sums -- agreement to the fp32 rounding
+ * of a group sum, whose order the reference leaves to its matmul library.  K and the group size must be multiples of 64. */
 typedef struct mi_matmul_dq_attr {
   int64_t M, K, N;
   int right_transpose;  /* right operand stored [N, K] instead of [K, N] */
   int q_group_size;     /* getQGroupSize() or module::getQuantGroupSize(); -1 = K */
-  int dq_type;          /* MI_DQ_INT8 / MI_DQ_INT4 */
+  int dq_type;          /* MI_DQ_INT8 / MI_DQ_INT4 / MI_DQ_F8E4M3 (imax 448) / MI_DQ_F4 (imax 6), MatMul.cpp:449-462 */
   int out_dtype;        /* MI_DT_BF16, or MI_DT_F16 when module::isF16Modes() */
 } mi_matmul_dq_attr;
 /* inputs = {left [M,K], right}, outputs = {[M,N]}, all f32-valued */
@@ -164,6 +165,10 @@ typedef struct mi_a16_quant_desc {
   int q_group_size;  /* 0 per channel, > 0 groups along K, -1 one group per row */
   int symmetric;     /* module::isQuantSymmetric(); ignored per channel */
   int dtype;         /* MI_DT_BF16 / MI_DT_F16: type the scales are stored in */
+  int dq_type;       /* MI_DQ_NONE / MI_DQ_INT: integer codes.  Under module::isDynamicQuantize() with groups,
+                      * MI_DQ_F8E4M3 (8-bit) and MI_DQ_F4 (4-bit) store float codes: scale = |absmax| / 448 or / 6,
+                      * zp = 0, code = f32_to_f8e4m3(w / scale, saturating) or f32_to_f4e2m1(w / scale)
+                      * (Canonicalize/A16MatMul.cpp:96-106, :179-209) */
 } mi_a16_quant_desc;
 /* A16MatMulAdjust (lib/Dialect/Tpu/Canonicalize/A16MatMul.cpp:270-429; computePerChannelParam :22-48,
  * computePerGroupParam :78-115, weightQuantization :147-216; static quantization, uint8 zero points).
@@ -197,6 +202,15 @@ int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
  * are added in the reference's order -- results are bit-identical to the reference's. */
 int mi_a16mm_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                        void *stream);
+/* The same branch for any dq_type it names (A16MatMul.cpp:51-61).  MI_DQ_INT is mi_a16mm_dq_launch.  MI_DQ_F8E4M3:
+ * the 8-bit weight bytes are E4M3 codes (f8e4m3_to_f32, lib/Support/Float8.cpp:140-191), activations are divided by
+ * amax / 448 and rounded to E4M3 (F8E4M3(src, step, true), Float8.cpp:259-261); group products are fp32 sums of the
+ * exact products (bf16 matrix instructions on the widened codes), so results agree with the reference's f32 matmul to
+ * fp32 rounding of a group sum -- its summation order is the matmul library's.  MI_DQ_F4: the 4-bit weight nibbles are E2M1 codes (lib/Support/Float4.cpp:7-24), activations
+ * are divided by amax / 6 and rounded to E2M1 (ties to the smaller magnitude); every product is a multiple of 1/4, the
+ * sums are exact, results are bit-identical.  Same shape limits as mi_a16mm_dq_launch. */
+int mi_a16mm_dq_type_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int64_t M, uint16_t *d_y,
+                            float *d_y_f32, void *stream);
 int mi_a16mm_launch_group(const mi_a16_weight *const *w, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_y,
                           float *const *d_y_f32, void *stream);
 

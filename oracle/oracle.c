@@ -526,7 +526,119 @@ int orc_a16matmul(const orc_a16mm_attr *a, const float *const *inputs,
 }
 
 /* A16MatMul.cpp:40-170 (module::isDynamicQuantize()), dq_type INT4 / INT8, w_transpose */
+/* ---- 8- and 4-bit floats of the dynamic-quantization flavours "F8E4M3" and "F4" ----------------------------- */
+/* shift right with round-half-to-even, on a value that may be negative (lib/Support/Float8.cpp:7-44, the
+ * ROUNDING_HALF_TO_EVEN arm; shifts above 63 act as 63) */
+static long long f8_shift_rne(long long src, int shift) {
+  if (shift == 0)
+    return src;
+  if (shift > 63)
+    shift = 63;
+  const long long val = src >> shift;
+  const long long rem = src & (long long)((1ull << shift) - 1);
+  const long long half = (long long)(1ull << (shift - 1));
+  if (rem == half)
+    return val + (val & 1);
+  return rem > half ? val + 1 : val;
+}
+
+/* lib/Support/Float8.cpp:46-131 with the E4M3 constants (bias 7, 4 significand bits, MAXNORM 0x7e, no infinities,
+ * 0x7f = NaN) and ROUNDING_HALF_TO_EVEN, which is how f32_to_f8e4m3 (:133-136) calls it */
+uint8_t orc_f32_to_f8e4m3(float src, int saturate) {
+  uint32_t bits;
+  memcpy(&bits, &src, 4);
+  const uint32_t sign = bits >> 31, exp = (bits >> 23) & 0xff, frac = bits & 0x7fffff;
+  uint8_t res = 0;
+  if (exp > 127 - 7 && exp < 0xff) { /* :74-96 f8 normals: round the f32 pattern to 3 fraction bits */
+    uint32_t tmp = (uint32_t)f8_shift_rne((long long)bits, 20);
+    tmp <<= 20;
+    const uint32_t e = ((tmp >> 23) & 0xff) - 127 + 7;
+    const uint32_t f = (tmp >> 20) & 0x7;
+    if (e > 0xf || (e == 0xf && f == 0x7))
+      res = saturate ? 0x7e : 0x7f;
+    else
+      res = (uint8_t)((e << 3) | f);
+  } else if (exp > 0 && exp <= 127 - 7) { /* :97-106 f8 subnormals and zero: units of 2^-9 */
+    int32_t mant = (int32_t)(frac + (1u << 23));
+    mant = sign ? -mant : mant;
+    const int shift = (127 - 7 + 1) - (int)exp + 20;
+    mant = (int32_t)f8_shift_rne(mant, shift);
+    mant = sign ? -mant : mant;
+    res = (uint8_t)(mant & 0x7f);
+  } else if (exp == 0xff && frac != 0) { /* :107-116 */
+    res = 0x7f;
+  } else if (exp == 0xff) { /* :117-124 */
+    res = saturate ? 0x7e : 0x7f;
+  } /* f32 zero and subnormals: 0 */
+  return (uint8_t)(res | (sign << 7));
+}
+
+/* lib/Support/Float8.cpp:140-186 with the E4M3 constants */
+float orc_f8e4m3_to_f32(uint8_t src) {
+  const uint32_t sign = (src >> 7) & 1;
+  uint32_t exponent = (src >> 3) & 0xf;
+  uint32_t mantissa = (uint32_t)(src & 0x7) << 20;
+  if ((src & 0x7f) == 0x7f) {
+    exponent = 0xff;
+    mantissa = 0x7fffff | (sign << 23);
+  } else if (exponent == 0) {
+    if (mantissa != 0) { /* normalize the subnormal */
+      uint32_t msb;
+      exponent = 127 - 6;
+      do {
+        msb = mantissa & 0x400000;
+        mantissa <<= 1;
+        exponent--;
+      } while (msb == 0);
+      mantissa &= 0x7fffff;
+    }
+  } else {
+    exponent += 127 - 7;
+  }
+  const uint32_t bits = (sign << 31) | (exponent << 23) | mantissa;
+  float out;
+  memcpy(&out, &bits, 4);
+  return out;
+}
+
+/* lib/Support/Float4.cpp:7-24: the sixteen E2M1 values; the first nearest one in table order wins, so ties go to the
+ * smaller magnitude, a negative input nearest to zero gives +0, and NaN / infinities give code 0 */
+static const float ORC_F4_TABLE[16] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f,
+                                       -0.0f, -0.5f, -1.0f, -1.5f, -2.0f, -3.0f, -4.0f, -6.0f};
+uint8_t orc_f32_to_f4e2m1(float src) {
+  uint8_t nearest = 0;
+  float best = fabsf(src - ORC_F4_TABLE[0]);
+  for (uint8_t i = 1; i < 16; i++) {
+    const float d = fabsf(src - ORC_F4_TABLE[i]);
+    if (d < best) {
+      best = d;
+      nearest = i;
+    }
+  }
+  return nearest;
+}
+float orc_f4e2m1_to_f32(uint8_t code) { return ORC_F4_TABLE[code & 15]; }
+
+/* array forms for the tests */
+void orc_f32_to_f8e4m3_n(const float *src, int64_t n, int saturate, uint8_t *dst) {
+  for (int64_t i = 0; i < n; i++)
+    dst[i] = orc_f32_to_f8e4m3(src[i], saturate);
+}
+void orc_f8e4m3_to_f32_n(const uint8_t *src, int64_t n, float *dst) {
+  for (int64_t i = 0; i < n; i++)
+    dst[i] = orc_f8e4m3_to_f32(src[i]);
+}
+void orc_f32_to_f4e2m1_n(const float *src, int64_t n, uint8_t *dst) {
+  for (int64_t i = 0; i < n; i++)
+    dst[i] = orc_f32_to_f4e2m1(src[i]);
+}
+
 int orc_a16matmul_dynamic(const orc_a16mm_attr *a, const float *const *inputs, float *output, float *y_preround) {
+  return orc_a16matmul_dynamic_dq(a, ORC_DQ_INT, inputs, output, y_preround);
+}
+
+int orc_a16matmul_dynamic_dq(const orc_a16mm_attr *a, int dq_type, const float *const *inputs, float *output,
+                             float *y_preround) {
   if (!a || !inputs || !inputs[0] || !inputs[1] || !inputs[2] || !inputs[3])
     return 1;
   if ((a->weight_bits != 4 && a->weight_bits != 8) || !a->w_transpose)
@@ -537,7 +649,16 @@ int orc_a16matmul_dynamic(const orc_a16mm_attr *a, const float *const *inputs, f
     return 1; /* :42-43 */
   if (g == -1)
     g = K; /* :47-49 with w_transpose (the row length of the [N, K] weight) */
-  const float imax = (float)((1 << (a->weight_bits - 1)) - 1); /* :53-54 */
+  /* :51-61; the weight loops :63-91 decode F4 only from 4-bit and F8E4M3 only from 8-bit storage */
+  float imax;
+  if (dq_type == ORC_DQ_INT)
+    imax = (float)((1 << (a->weight_bits - 1)) - 1);
+  else if (dq_type == ORC_DQ_F8E4M3 && a->weight_bits == 8)
+    imax = 448.0f; /* get_f8e4m3_max(), Float8.cpp:251 */
+  else if (dq_type == ORC_DQ_F4 && a->weight_bits == 4)
+    imax = 6.0f; /* get_f4e2m1_max(), Float4.cpp:26 */
+  else
+    return 1;
   const float *x = inputs[0], *weight = inputs[1], *scale = inputs[2], *zp = inputs[3], *bias = inputs[4];
   const int64_t group_num = (K + g - 1) / g;
   /* :63-91 integer weight minus zero point, [N, K] */
@@ -554,7 +675,10 @@ int orc_a16matmul_dynamic(const orc_a16mm_attr *a, const float *const *inputs, f
     const float z = zp[i / g];
     if (a->weight_bits == 4) {
       const int b = (int)weight[i / 2];
-      nw[i] = (float)((i & 1) ? (b >> 4) : (b & 0x0F)) - z;
+      const int code = (i & 1) ? (b >> 4) : (b & 0x0F);
+      nw[i] = (dq_type == ORC_DQ_F4 ? orc_f4e2m1_to_f32((uint8_t)code) : (float)code) - z;
+    } else if (dq_type == ORC_DQ_F8E4M3) {
+      nw[i] = orc_f8e4m3_to_f32((uint8_t)weight[i]) - z;
     } else {
       nw[i] = (float)(int)weight[i] - z;
     }
@@ -574,21 +698,54 @@ int orc_a16matmul_dynamic(const orc_a16mm_attr *a, const float *const *inputs, f
     }
     /* :109-132 */
     for (int64_t row = 0; row < M; row++)
-      for (int64_t col = 0; col < g; col++)
-        act[row * g + col] = (gi * g + col < K) ? roundf(x[row * K + gi * g + col] / amax[row] * imax) : 0.0f;
-    /* :133-160: group product (integer-valued operands), then the rescaled accumulation in row-major order */
+      for (int64_t col = 0; col < g; col++) {
+        float q = 0.0f;
+        if (gi * g + col < K) {
+          const float v = x[row * K + gi * g + col];
+          if (dq_type == ORC_DQ_INT) {
+            q = roundf(v / amax[row] * imax);
+          } else if (dq_type == ORC_DQ_F8E4M3) {
+            /* F8E4M3(src, double step, true), Float8.cpp:259-261: the quotient is formed in double, then narrowed */
+            const double step = (double)(amax[row] / imax);
+            q = orc_f8e4m3_to_f32(orc_f32_to_f8e4m3((float)((double)v / step), 1));
+          } else {
+            /* F4E2M1(src, float step), Float4.cpp:28-30 */
+            const float step = amax[row] / imax;
+            q = orc_f4e2m1_to_f32(orc_f32_to_f4e2m1(v / step));
+          }
+        }
+        act[row * g + col] = q;
+      }
+    /* :133-160: group product, then the rescaled accumulation in row-major order.  Integer codes: the product is an
+     * integer sum, exact in the reference's f32 matmul while it stays below 2^24.  F4: every product is a multiple of
+     * 1/4 no larger than 36 (times the zero-point shift), exact the same way.  F8E4M3: the f32 product depends on the
+     * matmul library's summation order, which the reference does not fix; the sum is formed in double here and
+     * rounded once, and comparisons with it carry a tolerance. */
     for (int64_t row = 0; row < M; row++)
       for (int64_t col = 0; col < N; col++) {
-        int64_t s = 0, peak = 0;
-        for (int64_t k = 0; k < g && gi * g + k < K; k++) {
-          s += (int64_t)act[row * g + k] * (int64_t)nw[col * K + gi * g + k];
-          const int64_t m = s < 0 ? -s : s;
-          peak = m > peak ? m : peak;
+        float prod;
+        if (dq_type == ORC_DQ_INT) {
+          int64_t s = 0, peak = 0;
+          for (int64_t k = 0; k < g && gi * g + k < K; k++) {
+            s += (int64_t)act[row * g + k] * (int64_t)nw[col * K + gi * g + k];
+            const int64_t m = s < 0 ? -s : s;
+            peak = m > peak ? m : peak;
+          }
+          if (peak >= (1 << 24))
+            inexact = 1;
+          prod = (float)s;
+        } else {
+          double s = 0.0, peak = 0.0;
+          for (int64_t k = 0; k < g && gi * g + k < K; k++) {
+            s += (double)act[row * g + k] * (double)nw[col * K + gi * g + k];
+            peak = fabs(s) > peak ? fabs(s) : peak;
+          }
+          if (dq_type == ORC_DQ_F4 && peak * 4.0 >= (double)(1 << 24))
+            inexact = 1;
+          prod = (float)s;
         }
-        if (peak >= (1 << 24))
-          inexact = 1;
         float *o = output + row * N + col;
-        *o += (float)s * (amax[row] / imax) * scale[col * group_num + gi];
+        *o += prod * (amax[row] / imax) * scale[col * group_num + gi];
         if (gi == 0 && bias)
           *o += bias[col];
       }
@@ -608,7 +765,33 @@ int orc_a16matmul_dynamic(const orc_a16mm_attr *a, const float *const *inputs, f
 /* MatMul.cpp:447-597, INT8 / INT4, batch 1 */
 int orc_matmul_dynamic(const float *left, const float *right, int64_t M, int64_t K, int64_t N, int right_transpose,
                        int q_group_size, int imax_i, int out_dtype, float *output, float *y_preround) {
-  if (!left || !right || !output || M <= 0 || K <= 0 || N <= 0 || (imax_i != 127 && imax_i != 7))
+  return orc_matmul_dynamic_dq(left, right, M, K, N, right_transpose, q_group_size, ORC_DQ_INT, imax_i, out_dtype,
+                               output, y_preround);
+}
+
+/* one operand element -> its code value, MatMul.cpp:507-566 (the same three rules as A16MatMul.cpp:109-132) */
+static float dq_code(float v, float amax, float imax, int dq_type) {
+  if (dq_type == ORC_DQ_INT)
+    return roundf(v / amax * imax);
+  if (dq_type == ORC_DQ_F8E4M3) {
+    const double step = (double)(amax / imax);
+    return orc_f8e4m3_to_f32(orc_f32_to_f8e4m3((float)((double)v / step), 1));
+  }
+  return orc_f4e2m1_to_f32(orc_f32_to_f4e2m1(v / (amax / imax)));
+}
+
+int orc_matmul_dynamic_dq(const float *left, const float *right, int64_t M, int64_t K, int64_t N, int right_transpose,
+                          int q_group_size, int dq_type, int imax_i, int out_dtype, float *output,
+                          float *y_preround) {
+  if (!left || !right || !output || M <= 0 || K <= 0 || N <= 0)
+    return 1;
+  if (dq_type == ORC_DQ_INT && imax_i != 127 && imax_i != 7)
+    return 1;
+  if (dq_type == ORC_DQ_F8E4M3)
+    imax_i = 448; /* :454-455 */
+  else if (dq_type == ORC_DQ_F4)
+    imax_i = 6; /* :458-459 */
+  else if (dq_type != ORC_DQ_INT)
     return 1;
   int64_t g = q_group_size;
   if (g == -1)
@@ -651,24 +834,37 @@ int orc_matmul_dynamic(const float *left, const float *right, int64_t M, int64_t
     /* :507-566 codes */
     for (int64_t row = 0; row < M; row++)
       for (int64_t col = 0; col < g; col++)
-        ql[row * g + col] = (gi * g + col < K) ? roundf(left[row * K + gi * g + col] / lmax[row] * imax) : 0.0f;
+        ql[row * g + col] = (gi * g + col < K) ? dq_code(left[row * K + gi * g + col], lmax[row], imax, dq_type) : 0.0f;
     for (int64_t n = 0; n < N; n++)
       for (int64_t col = 0; col < g; col++) {
         const int64_t k = gi * g + col;
-        qr[n * g + col] = (k < K) ? roundf((right_transpose ? right[n * K + k] : right[k * N + n]) / rmax[n] * imax) : 0.0f;
+        qr[n * g + col] = (k < K) ? dq_code(right_transpose ? right[n * K + k] : right[k * N + n], rmax[n], imax, dq_type) : 0.0f;
       }
     /* :567-583 group product and rescaled accumulation */
     for (int64_t row = 0; row < M; row++)
       for (int64_t n = 0; n < N; n++) {
-        int64_t s = 0, peak = 0;
-        for (int64_t k = 0; k < g; k++) {
-          s += (int64_t)ql[row * g + k] * (int64_t)qr[n * g + k];
-          const int64_t m = s < 0 ? -s : s;
-          peak = m > peak ? m : peak;
+        float prod;
+        if (dq_type == ORC_DQ_INT) {
+          int64_t s = 0, peak = 0;
+          for (int64_t k = 0; k < g; k++) {
+            s += (int64_t)ql[row * g + k] * (int64_t)qr[n * g + k];
+            const int64_t m = s < 0 ? -s : s;
+            peak = m > peak ? m : peak;
+          }
+          if (peak >= (1 << 24))
+            inexact = 1;
+          prod = (float)s;
+        } else { /* F4: quarter units, exact; F8E4M3: summed in double, rounded once (the reference's order is open) */
+          double s = 0.0, peak = 0.0;
+          for (int64_t k = 0; k < g; k++) {
+            s += (double)ql[row * g + k] * (double)qr[n * g + k];
+            peak = fabs(s) > peak ? fabs(s) : peak;
+          }
+          if (dq_type == ORC_DQ_F4 && peak * 4.0 >= (double)(1 << 24))
+            inexact = 1;
+          prod = (float)s;
         }
-        if (peak >= (1 << 24))
-          inexact = 1;
-        output[row * N + n] += (float)s * (lmax[row] / imax) * (rmax[n] / imax);
+        output[row * N + n] += prod * (lmax[row] / imax) * (rmax[n] / imax);
       }
   }
   free(ql);
@@ -1013,7 +1209,18 @@ static int orc_clampi(int v, int lo, int hi) { return v < lo ? lo : v > hi ? hi 
 int orc_a16_quantize(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16,
                      uint8_t *q, float *scale_f32, uint16_t *scale16, uint8_t *zp, int *sign_out,
                      int *weight_signed_out) {
+  return orc_a16_quantize_dq(w_kn, K, N, bits, g, symmetric, f16, ORC_DQ_INT, q, scale_f32, scale16, zp, sign_out,
+                             weight_signed_out);
+}
+
+int orc_a16_quantize_dq(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16, int dq_type,
+                        uint8_t *q, float *scale_f32, uint16_t *scale16, uint8_t *zp, int *sign_out,
+                        int *weight_signed_out) {
   if ((bits != 4 && bits != 8) || K <= 0 || N <= 0 || (bits == 4 && (K & 1)))
+    return -1;
+  /* the float code types exist only on the per-group path (computePerGroupParam :78-115 takes dq_type,
+   * computePerChannelParam does not), F8E4M3 in 8-bit and F4 in 4-bit storage (:183-209) */
+  if (dq_type != ORC_DQ_INT && (g == 0 || (dq_type == ORC_DQ_F8E4M3 && bits != 8) || (dq_type == ORC_DQ_F4 && bits != 4)))
     return -1;
   /* :312-321 transpose to [row = N, col = K] */
   const int64_t row = N, col = K;
@@ -1062,7 +1269,13 @@ int orc_a16_quantize(const float *w_kn, int64_t K, int64_t N, int bits, int g, i
       float mn, mx;
       orc_min_max(p, gs, &mn, &mx);
       const float abs_max = orc_max_abs(p, gs);
-      if (sym) {
+      if (dq_type == ORC_DQ_F8E4M3) { /* :98-100 */
+        scale_f32[i] = fabsf(abs_max) / 448.0f;
+        zp[i] = 0;
+      } else if (dq_type == ORC_DQ_F4) { /* :104-106 */
+        scale_f32[i] = fabsf(abs_max) / 6.0f;
+        zp[i] = 0;
+      } else if (sym) {
         scale_f32[i] = 2 * fabsf(abs_max) / max_int;
       } else {
         const float d = mx - mn;
@@ -1076,8 +1289,20 @@ int orc_a16_quantize(const float *w_kn, int64_t K, int64_t N, int bits, int g, i
   for (int64_t c = 0; c < row; ++c)
     for (int64_t i = 0; i < col; ++i) {
       const int64_t qi = gs ? (c * col + i) / gs : c;
-      const float t = roundf(w[c * col + i] / scale_f32[qi]) + (float)zp[qi];
-      if (bits == 8) {
+      float t = w[c * col + i] / scale_f32[qi];
+      if (dq_type == ORC_DQ_INT) /* :181-182: the float code types keep the quotient unrounded */
+        t = roundf(t);
+      t += (float)zp[qi];
+      if (dq_type == ORC_DQ_F8E4M3) { /* :185-186 */
+        q[c * col + i] = orc_f32_to_f8e4m3(t, 1);
+      } else if (dq_type == ORC_DQ_F4) { /* :194-200 */
+        const uint8_t code = orc_f32_to_f4e2m1(t);
+        uint8_t *dst = q + (c * col) / 2 + i / 2;
+        if (i % 2)
+          *dst |= (uint8_t)(code << 4);
+        else
+          *dst = code;
+      } else if (bits == 8) {
         if (as_int8)
           q[c * col + i] = (uint8_t)(int8_t)orc_clamp_code(t, -128, 127);
         else

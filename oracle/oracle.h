@@ -27,6 +27,14 @@
  *   orc_a16matmul_dynamic        lossless-activation cases against orc_a16matmul, exact power-of-two row
  *                                scaling, half-step error bound, group order (tests/test_oracle_dynamic.py)
  *   orc_matmul_dynamic           the same four properties, on both operands (tests/test_oracle_dynamic.py)
+ *   orc_f32_to_f8e4m3 / orc_f8e4m3_to_f32   torch.float8_e4m3fn on all codes, all bf16 patterns and random f32 inside
+ *                                +-448, every tie and its neighbours, saturation / subnormal table
+ *   orc_f32_to_f4e2m1 / orc_f4e2m1_to_f32   e2m1 closed form, float64 brute-force nearest with first-minimum ties
+ *   orc_a16matmul_dynamic_dq, orc_matmul_dynamic_dq (F8E4M3 / F4)   on-grid operands against a float64 product of
+ *                                independently decoded operands; half-spacing bound.  F8E4M3 group sums are
+ *                                order-dependent in the reference: pinned to fp32 rounding of a group sum, not bit
+ *                                for bit (tests/test_oracle_float_codes.py)
+ *   orc_a16_quantize_dq          closed-form scale, zp = 0, on-grid recovery, half-spacing bound
  *   orc_a16_quantize             on-grid weights are recovered exactly, |w - dequant(q)| <= scale/2 inside the
  *                                clamp range, closed-form scale/zp, nibble order via the A16MatMul dequantizer
  *                                (tests/test_oracle_packers.py)
@@ -224,6 +232,22 @@ int orc_cast(const orc_cast_attr *attr, const float *input, float *output, int64
  * added group by group in fp32, bias after the first group.  inputs as for orc_a16matmul; the 8-bit weight is
  * read as the reference reads it, `int(weight[i])`.  Returns 0, 1 (bad arguments), 2 (outside the exact domain). */
 int orc_a16matmul_dynamic(const orc_a16mm_attr *a, const float *const *inputs, float *output, float *y_preround);
+/* The same operator for any dq_type of :51-61.  ORC_DQ_F8E4M3 (8-bit weights holding E4M3 codes; activations rounded to
+ * E4M3 after division by amax / 448) and ORC_DQ_F4 (4-bit weights holding E2M1 codes; activations rounded to E2M1
+ * after division by amax / 6).  F4 is exact like the integer types; for F8E4M3 the group products are summed in double
+ * and rounded once, where the reference's f32 matmul rounds in an order its library chooses. */
+enum { ORC_DQ_INT = 0, ORC_DQ_F8E4M3 = 1, ORC_DQ_F4 = 2 };
+int orc_a16matmul_dynamic_dq(const orc_a16mm_attr *a, int dq_type, const float *const *inputs, float *output,
+                             float *y_preround);
+/* lib/Support/Float8.cpp:46-136 (round half to even; saturate: overflow and infinities give +-448, else NaN 0x7f),
+ * :140-191, and lib/Support/Float4.cpp:7-24 */
+uint8_t orc_f32_to_f8e4m3(float src, int saturate);
+float orc_f8e4m3_to_f32(uint8_t code);
+uint8_t orc_f32_to_f4e2m1(float src);
+float orc_f4e2m1_to_f32(uint8_t code);
+void orc_f32_to_f8e4m3_n(const float *src, int64_t n, int saturate, uint8_t *dst);
+void orc_f8e4m3_to_f32_n(const uint8_t *src, int64_t n, float *dst);
+void orc_f32_to_f4e2m1_n(const float *src, int64_t n, uint8_t *dst);
 
 /* tpu.MatMul with both operands quantized dynamically (lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:447-597, dq_type
  * "INT8": imax 127, "INT4": imax 7; batch 1): left [M, K], right [K, N] or [N, K] when right_transpose, both
@@ -232,6 +256,10 @@ int orc_a16matmul_dynamic(const orc_a16mm_attr *a, const float *const *inputs, f
  * 2^24, where the reference's f32 product stops being exact). */
 int orc_matmul_dynamic(const float *left, const float *right, int64_t M, int64_t K, int64_t N, int right_transpose,
                        int q_group_size, int imax, int out_dtype, float *output, float *y_preround);
+/* The same branch for dq_type "F8E4M3" (imax 448) and "F4" (imax 6), MatMul.cpp:454-459 and :519-563; ORC_DQ_INT takes
+ * imax as above.  F4 is exact; F8E4M3 group sums are formed in double and rounded once. */
+int orc_matmul_dynamic_dq(const float *left, const float *right, int64_t M, int64_t K, int64_t N, int right_transpose,
+                          int q_group_size, int dq_type, int imax, int out_dtype, float *output, float *y_preround);
 
 /* ---- weight producers (compile-time side of tpu.A16MatMul) ------------------- */
 /* A16MatMulAdjust, lib/Dialect/Tpu/Canonicalize/A16MatMul.cpp:270-429, static uint8-zero-point variant:
@@ -241,6 +269,11 @@ int orc_matmul_dynamic(const float *left, const float *right, int64_t M, int64_t
  * per row.  Returns 0, or -1 for arguments the reference asserts on. */
 int orc_a16_quantize(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16,
                      uint8_t *q, float *scale_f32, uint16_t *scale16, uint8_t *zp, int *sign, int *weight_signed);
+/* The same pass under module::isDynamicQuantize() with dq_type "F8E4M3" (8-bit) or "F4" (4-bit), groups only:
+ * scale = |absmax| / 448 or / 6, zp = 0 (:96-106), codes = f32_to_f8e4m3(w / scale, saturating) or f32_to_f4e2m1(w / scale)
+ * without integer rounding (:179-209).  ORC_DQ_INT is orc_a16_quantize. */
+int orc_a16_quantize_dq(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16, int dq_type,
+                        uint8_t *q, float *scale_f32, uint16_t *scale16, uint8_t *zp, int *sign, int *weight_signed);
 
 /* GPTQ / AWQ checkpoints -> the [N, K/2] + [N, G] layout, python/llm/LlmConverter.py:320-389 (unpack_weights) and
  * :1454-1475 (the transposes).  qweight: GPTQ int32 [K*bits/32, N] (packed along K), AWQ int32 [K, N*bits/32]

@@ -209,16 +209,53 @@ def a16matmul(x, weight, scale, zp, bias, *, M, K, N, weight_bits, q_group_size,
     return out, pre
 
 
-def a16matmul_dynamic(x, weight, scale, zp, bias, *, M, K, N, weight_bits, q_group_size, out_dtype=OUT_BF16):
-    """tpu.A16MatMul with dynamic INT4 / INT8 activation quantization; returns (output, pre-rounding f32)."""
+DQ_INT, DQ_F8E4M3, DQ_F4 = 0, 1, 2
+
+
+def f32_to_f8e4m3(x, saturate=True):
+    """E4M3 codes (uint8) of an f32 array, round half to even."""
+    x = _f32(x)
+    out = np.empty(x.shape, dtype=np.uint8)
+    L = lib()
+    L.orc_f32_to_f8e4m3_n.restype = None
+    L.orc_f32_to_f8e4m3_n(_p(x, C.c_float), C.c_int64(x.size), C.c_int(int(saturate)), _p(out, C.c_uint8))
+    return out
+
+
+def f8e4m3_to_f32(codes):
+    codes = np.ascontiguousarray(codes, dtype=np.uint8)
+    out = np.empty(codes.shape, dtype=np.float32)
+    L = lib()
+    L.orc_f8e4m3_to_f32_n.restype = None
+    L.orc_f8e4m3_to_f32_n(_p(codes, C.c_uint8), C.c_int64(codes.size), _p(out, C.c_float))
+    return out
+
+
+F4_VALUES = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0],
+                     dtype=np.float32)
+
+
+def f32_to_f4e2m1(x):
+    """E2M1 codes (uint8, 0..15) of an f32 array."""
+    x = _f32(x)
+    out = np.empty(x.shape, dtype=np.uint8)
+    L = lib()
+    L.orc_f32_to_f4e2m1_n.restype = None
+    L.orc_f32_to_f4e2m1_n(_p(x, C.c_float), C.c_int64(x.size), _p(out, C.c_uint8))
+    return out
+
+
+def a16matmul_dynamic(x, weight, scale, zp, bias, *, M, K, N, weight_bits, q_group_size, out_dtype=OUT_BF16,
+                      dq_type=DQ_INT):
+    """tpu.A16MatMul with dynamic activation quantization (INT4 / INT8, F8E4M3, F4); returns (output, pre-rounding f32)."""
     ins = [_f32(x), _f32(weight), _f32(scale), _f32(zp), _f32(bias)]
     attr = A16Attr(M, K, N, weight_bits, 1, q_group_size, out_dtype, 0, GEMM_F64ACC)
     arr = (C.POINTER(C.c_float) * 5)(*[None if a is None else _p(a, C.c_float) for a in ins])
     out = np.empty((M, N), dtype=np.float32)
     pre = np.empty((M, N), dtype=np.float32)
     L = lib()
-    L.orc_a16matmul_dynamic.restype = C.c_int
-    rc = L.orc_a16matmul_dynamic(C.byref(attr), arr, _p(out, C.c_float), _p(pre, C.c_float))
+    L.orc_a16matmul_dynamic_dq.restype = C.c_int
+    rc = L.orc_a16matmul_dynamic_dq(C.byref(attr), C.c_int(dq_type), arr, _p(out, C.c_float), _p(pre, C.c_float))
     if rc == 2:
         raise ValueError("orc_a16matmul_dynamic: group sums leave the range the reference's f32 product is exact in")
     if rc != 0:
@@ -226,17 +263,18 @@ def a16matmul_dynamic(x, weight, scale, zp, bias, *, M, K, N, weight_bits, q_gro
     return out, pre
 
 
-def matmul_dynamic(left, right, *, right_transpose=False, q_group_size, imax=127, out_dtype=OUT_BF16):
-    """tpu.MatMul with both operands quantized dynamically (INT8: imax 127, INT4: imax 7); returns (output, pre)."""
+def matmul_dynamic(left, right, *, right_transpose=False, q_group_size, imax=127, out_dtype=OUT_BF16, dq_type=DQ_INT):
+    """tpu.MatMul with both operands quantized dynamically (INT8: imax 127, INT4: imax 7, or dq_type DQ_F8E4M3 /
+    DQ_F4); returns (output, pre)."""
     left, right = _f32(left), _f32(right)
     M, K = left.shape
     N = right.shape[0] if right_transpose else right.shape[1]
     out = np.empty((M, N), dtype=np.float32)
     pre = np.empty((M, N), dtype=np.float32)
     L = lib()
-    L.orc_matmul_dynamic.restype = C.c_int
-    rc = L.orc_matmul_dynamic(_p(left, C.c_float), _p(right, C.c_float), C.c_int64(M), C.c_int64(K), C.c_int64(N),
-                              C.c_int(int(right_transpose)), C.c_int(q_group_size), C.c_int(imax), C.c_int(out_dtype),
+    L.orc_matmul_dynamic_dq.restype = C.c_int
+    rc = L.orc_matmul_dynamic_dq(_p(left, C.c_float), _p(right, C.c_float), C.c_int64(M), C.c_int64(K), C.c_int64(N),
+                              C.c_int(int(right_transpose)), C.c_int(q_group_size), C.c_int(dq_type), C.c_int(imax), C.c_int(out_dtype),
                               _p(out, C.c_float), _p(pre, C.c_float))
     if rc == 2:
         raise ValueError("orc_matmul_dynamic: group sums leave the range the reference's f32 product is exact in")
@@ -320,7 +358,7 @@ def cast(x, *, in_type, out_type, in_quant=False, out_quant=False, scale=1.0, ze
 PACK_GPTQ, PACK_AWQ = 0, 1
 
 
-def a16_quantize(w_kn, *, bits, g, symmetric=False, f16=False):
+def a16_quantize(w_kn, *, bits, g, symmetric=False, f16=False, dq_type=DQ_INT):
     """A16MatMulAdjust on the f32 weight [K, N] of a top-level matmul.
 
     Returns dict(weight [N, K/2] or [N, K] uint8 (int8 bit patterns when weight_signed), scale_f32 [N, G],
@@ -336,9 +374,9 @@ def a16_quantize(w_kn, *, bits, g, symmetric=False, f16=False):
     zp = np.zeros((N, G), dtype=np.uint8)
     sign, wsigned = C.c_int(0), C.c_int(0)
     L = lib()
-    L.orc_a16_quantize.restype = C.c_int
-    rc = L.orc_a16_quantize(_p(w, C.c_float), C.c_int64(K), C.c_int64(N), C.c_int(bits), C.c_int(g),
-                            C.c_int(int(symmetric)), C.c_int(int(f16)), _p(q, C.c_uint8), _p(sf, C.c_float),
+    L.orc_a16_quantize_dq.restype = C.c_int
+    rc = L.orc_a16_quantize_dq(_p(w, C.c_float), C.c_int64(K), C.c_int64(N), C.c_int(bits), C.c_int(g),
+                            C.c_int(int(symmetric)), C.c_int(int(f16)), C.c_int(dq_type), _p(q, C.c_uint8), _p(sf, C.c_float),
                             _p(s16, C.c_uint16), _p(zp, C.c_uint8), C.byref(sign), C.byref(wsigned))
     if rc != 0:
         raise RuntimeError("orc_a16_quantize: bad arguments")

@@ -228,6 +228,57 @@ def case_producers_and_dynamic():
     np.savez_compressed(os.path.join(HERE, "case_dynamic.npz"), **out)
 
 
+def case_float_codes():
+    """dq_type "F8E4M3" / "F4": conversion tables, the float-code weight producer, and the dynamic matmuls.  F4 and the
+    small-integer F8 case are exact (bit for bit on the GPU); the random F8 case carries fp32 summation error."""
+    rng = np.random.default_rng(401)
+    codes = np.arange(256, dtype=np.uint8)
+    lo = O.f8e4m3_to_f32(codes[:0x7e])
+    mid = ((lo.astype(np.float64) + O.f8e4m3_to_f32(codes[1:0x7f])) / 2).astype(np.float32)
+    xs = np.concatenate([mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(np.inf)),
+                         np.array([448, 464, 465, 1e9, np.inf, 2.0 ** -10, 2.0 ** -11, 1e-45, 0], np.float32),
+                         (rng.standard_normal(2000) * 2.0 ** rng.integers(-12, 9, size=2000)).astype(np.float32)])
+    xs = np.concatenate([xs, -xs])
+    x4 = np.concatenate([np.arange(-32, 33) * 0.25, rng.uniform(-8, 8, 500),
+                         np.array([1e6, 2.0 ** 26, 1e30, np.inf])]).astype(np.float32)
+    out = dict(f8_decode=O.f8e4m3_to_f32(codes), f8_in=xs, f8_codes_sat=O.f32_to_f8e4m3(xs, True),
+               f8_codes_nosat=O.f32_to_f8e4m3(xs, False), f4_in=x4, f4_codes=O.f32_to_f4e2m1(x4))
+    w = (rng.standard_normal((256, 40)) * 0.05).astype(np.float32)
+    w[:64, 5] = 0.0   # an all-zero group: scale 0
+    out["w_kn"] = w
+    for tag, kw in (("f8_g64", dict(bits=8, g=64, dq_type=O.DQ_F8E4M3)), ("f4_g128", dict(bits=4, g=128, dq_type=O.DQ_F4))):
+        r = O.a16_quantize(w, **kw)
+        out["q_" + tag] = r["weight"]
+        out["scale16_" + tag] = r["scale16"]
+    # dynamic F4: random nibbles read as E2M1 codes, zero points 0 / random
+    for tag, zps in (("f4", False), ("f4zp", True)):
+        cfg = S.w4a16(5, 512, 40, 128, seed=402, bias=True)
+        if not zps:
+            cfg["zp"] = np.zeros_like(cfg["zp"])
+        x, wf, sc, z, b = f32_valued_a16(cfg)
+        y, pre = O.a16matmul_dynamic(x, wf, sc, z, b, M=5, K=512, N=40, weight_bits=4, q_group_size=128, dq_type=O.DQ_F4)
+        out.update({tag + "_x": cfg["x"], tag + "_weight": cfg["weight"], tag + "_scale": cfg["scale"],
+                    tag + "_zp": cfg["zp"], tag + "_bias": cfg["bias"], tag + "_want_bf16": O.f32_to_bf16(y),
+                    tag + "_want_pre": pre})
+    # dynamic F8E4M3: (a) small integers with 448 * 2^e per group -- exact; (b) random codes -- tolerance
+    M, K, N, g = 4, 256, 24, 64
+    scale = S.bf16_round((np.abs(rng.standard_normal((N, K // g))) * 0.01 + 1e-3).astype(np.float32))
+    ints = rng.integers(-15, 16, size=(M, K // g, g)).astype(np.float32)
+    ints[:, :, 7] = 448.0
+    xa = S.bf16_round((ints * np.float32(2.0) ** rng.integers(-6, 3, size=(M, K // g, 1)).astype(np.float32)).reshape(M, K))
+    wa = O.f32_to_f8e4m3(rng.integers(-15, 16, size=(N, K)).astype(np.float32))
+    xb = S.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    wb = rng.integers(0, 256, size=(N, K)).astype(np.uint8)
+    wb[(wb & 0x7f) == 0x7f] = 0x3a
+    for tag, xx, ww in (("f8exact", xa, wa), ("f8rand", xb, wb)):
+        y, pre = O.a16matmul_dynamic(S.bf16_to_f32(xx), ww.astype(np.float32), S.bf16_to_f32(scale),
+                                     np.zeros((N, K // g), np.float32), None, M=M, K=K, N=N, weight_bits=8,
+                                     q_group_size=g, dq_type=O.DQ_F8E4M3)
+        out.update({tag + "_x": xx, tag + "_weight": ww, tag + "_want_bf16": O.f32_to_bf16(y), tag + "_want_pre": pre})
+    out["f8_scale"] = scale
+    np.savez_compressed(os.path.join(HERE, "case_float_codes.npz"), **out)
+
+
 if __name__ == "__main__":
     kat_right_shift_round()
     kat_mbqm()
@@ -235,6 +286,7 @@ if __name__ == "__main__":
     case_a16()
     case_i8()
     case_producers_and_dynamic()
+    case_float_codes()
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print("%-40s %7d bytes" % (f, os.path.getsize(os.path.join(HERE, f))))

@@ -87,6 +87,11 @@ def test_weight_producer_and_blob_argument_errors():
     assert L.mi_a16_quantize(None, None, None, None, None, None, None, None) == clib.MI_BAD_ARGUMENT
     assert L.mi_llm_unpack(0, 4, None, None, 8, 8, 1, None, None) == clib.MI_BAD_ARGUMENT
     assert L.mi_a16mm_dq_launch(None, None, 1, None, None, None) == clib.MI_BAD_ARGUMENT
+    assert L.mi_a16mm_dq_type_launch(None, clib.DQ_F8E4M3, None, 1, None, None, None) == clib.MI_BAD_ARGUMENT
+    for bits, g, dq in ((8, 0, clib.DQ_F8E4M3), (4, 64, clib.DQ_F8E4M3), (8, 64, clib.DQ_F4)):
+        with pytest.raises(M.BackendError) as e:   # float codes: groups only, E4M3 in 8-bit and E2M1 in 4-bit storage
+            M.a16_quantize(np.zeros((64, 8), np.float32), weight_bits=bits, q_group_size=g, dq_type=dq)
+        assert e.value.code == clib.MI_UNSUPPORTED
     w = np.zeros((64, 8), np.float32)
     with pytest.raises(M.BackendError) as e:
         M.a16_quantize(w, weight_bits=3, q_group_size=0)

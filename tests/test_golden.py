@@ -128,6 +128,73 @@ def test_oracle_reproduces_producer_and_dynamic_cases(orc):
     assert np.array_equal(pre, y["mm_want_pre"])
 
 
+def test_oracle_reproduces_float_code_cases(orc):
+    d = _load("case_float_codes.npz")
+    dec = orc.f8e4m3_to_f32(np.arange(256, dtype=np.uint8))
+    assert np.array_equal(dec.view(np.uint32) & 0x7fffffff, d["f8_decode"].view(np.uint32) & 0x7fffffff)
+    assert np.array_equal(orc.f32_to_f8e4m3(d["f8_in"], True), d["f8_codes_sat"])
+    assert np.array_equal(orc.f32_to_f8e4m3(d["f8_in"], False), d["f8_codes_nosat"])
+    assert np.array_equal(orc.f32_to_f4e2m1(d["f4_in"]), d["f4_codes"])
+    for tag, kw in FLOAT_QUANT_TAGS.items():
+        r = orc.a16_quantize(d["w_kn"], bits=kw["bits"], g=kw["g"], dq_type=getattr(orc, kw["dq"]))
+        assert np.array_equal(r["weight"], d["q_" + tag]) and np.array_equal(r["scale16"], d["scale16_" + tag])
+        assert not r["zp"].any()
+    for tag in ("f4", "f4zp"):
+        out, pre = orc.a16matmul_dynamic(S.bf16_to_f32(d[tag + "_x"]), d[tag + "_weight"].astype(np.float32),
+                                         S.bf16_to_f32(d[tag + "_scale"]), d[tag + "_zp"].astype(np.float32),
+                                         S.bf16_to_f32(d[tag + "_bias"]), M=5, K=512, N=40, weight_bits=4,
+                                         q_group_size=128, dq_type=orc.DQ_F4)
+        assert np.array_equal(pre, d[tag + "_want_pre"]) and np.array_equal(orc.f32_to_bf16(out), d[tag + "_want_bf16"])
+    for tag in ("f8exact", "f8rand"):
+        out, pre = orc.a16matmul_dynamic(S.bf16_to_f32(d[tag + "_x"]), d[tag + "_weight"].astype(np.float32),
+                                         S.bf16_to_f32(d["f8_scale"]), np.zeros(d["f8_scale"].shape, np.float32), None,
+                                         M=4, K=256, N=24, weight_bits=8, q_group_size=64, dq_type=orc.DQ_F8E4M3)
+        assert np.array_equal(pre, d[tag + "_want_pre"]) and np.array_equal(orc.f32_to_bf16(out), d[tag + "_want_bf16"])
+
+
+FLOAT_QUANT_TAGS = {"f8_g64": dict(bits=8, g=64, dq="DQ_F8E4M3"), "f4_g128": dict(bits=4, g=128, dq="DQ_F4")}
+
+
+@pytest.mark.gpu
+def test_gpu_float_codes_against_fixture():
+    """Producer codes, F4 and the small-integer F8 matmul bit for bit; the random F8 matmul to 2^-20 of the sum of
+    absolute terms (its group sums are fp32 sums in an order the reference leaves open)."""
+    import torch
+    M_ = pkg()
+    clib = pkg("clib")
+    d = _load("case_float_codes.npz")
+    for tag, kw in FLOAT_QUANT_TAGS.items():
+        r = M_.a16_quantize(d["w_kn"], weight_bits=kw["bits"], q_group_size=kw["g"], dq_type=getattr(clib, kw["dq"]))
+        assert np.array_equal(r["weight"].view(np.uint8), d["q_" + tag]), tag
+        assert np.array_equal(r["scale_bits"], d["scale16_" + tag]) and not r["zp"].any(), tag
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda().view(torch.bfloat16)
+
+    def run(x, weight, scale, zp, bias, bits, g, dq):
+        M, K = x.shape
+        N = weight.shape[0]
+        w = M_.A16Weight(weight, scale, zp, bias, K=K, N=N, weight_bits=bits, q_group_size=g)
+        y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        out = M_.a16mm_dq_launch(w, dev(x), y_f32=y32, dq_type=dq)
+        torch.cuda.synchronize()
+        w.destroy()
+        return out.view(torch.int16).cpu().numpy().view(np.uint16), y32.cpu().numpy()
+
+    for tag in ("f4", "f4zp"):
+        out, pre = run(d[tag + "_x"], d[tag + "_weight"], d[tag + "_scale"], d[tag + "_zp"],
+                       S.bf16_to_f32(d[tag + "_bias"]), 4, 128, clib.DQ_F4)
+        assert np.array_equal(pre.view(np.uint32), d[tag + "_want_pre"].view(np.uint32)), tag
+        assert np.array_equal(out, d[tag + "_want_bf16"]), tag
+    zp = np.zeros(d["f8_scale"].shape, np.uint8)
+    out, pre = run(d["f8exact_x"], d["f8exact_weight"], d["f8_scale"], zp, None, 8, 64, clib.DQ_F8E4M3)
+    assert np.array_equal(pre.view(np.uint32), d["f8exact_want_pre"].view(np.uint32))
+    assert np.array_equal(out, d["f8exact_want_bf16"])
+    out, pre = run(d["f8rand_x"], d["f8rand_weight"], d["f8_scale"], zp, None, 8, 64, clib.DQ_F8E4M3)
+    wv = np.abs(d["f8_decode"][d["f8rand_weight"]].astype(np.float64)).reshape(24, 4, 64)
+    deq = (wv * S.bf16_to_f32(d["f8_scale"]).astype(np.float64)[:, :, None]).reshape(24, 256)
+    mag = np.abs(S.bf16_to_f32(d["f8rand_x"]).astype(np.float64)) * 1.07 @ deq.T
+    assert np.all(np.abs(pre.astype(np.float64) - d["f8rand_want_pre"]) <= mag * 2.0 ** -20)
+
+
 # ----------------------------------------------------------------------------------------------- GPU
 @pytest.mark.gpu
 def test_gpu_producers_and_dynamic_against_fixtures():

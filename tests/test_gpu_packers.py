@@ -140,3 +140,64 @@ def test_packed_blob_round_trip(bits, g, signed, bias):
         M_.A16Weight.from_blob(bad.tobytes())
     w1.destroy()
     w2.destroy()
+
+
+FLOAT_CODE_CASES = [  # (dq, bits, K, N, g, kind)
+    ("DQ_F8E4M3", 8, 512, 96, 128, "normal"), ("DQ_F8E4M3", 8, 256, 40, 64, "normal"), ("DQ_F8E4M3", 8, 256, 24, 128, "flat"),
+    ("DQ_F8E4M3", 8, 256, 24, -1, "positive"),
+    ("DQ_F4", 4, 1024, 300, 128, "normal"), ("DQ_F4", 4, 512, 70, 64, "normal"), ("DQ_F4", 4, 256, 24, 128, "flat"),
+    ("DQ_F4", 4, 256, 48, 32, "positive"),
+]
+
+
+@pytest.mark.parametrize("dq,bits,K,N,g,kind", FLOAT_CODE_CASES)
+def test_float_code_quantizer_matches_oracle_bit_for_bit(orc, dq, bits, K, N, g, kind):
+    """dq_type "F8E4M3" / "F4": scale = absmax / 448 or / 6, zero point 0, unrounded quotient -> E4M3 / E2M1 code.
+    The "flat" weights hold all-zero groups (scale 0: the reference's 0 / 0 goes to NaN code 0x7f, or E2M1 code 0)."""
+    w = _weights(bits * 1000 + K + N + 1, K, N, kind)
+    want = orc.a16_quantize(w, bits=bits, g=g, symmetric=True, dq_type=getattr(orc, dq))
+    got = M_.a16_quantize(w, weight_bits=bits, q_group_size=g, symmetric=True, dq_type=getattr(clib, dq))
+    assert got["sign"] == want["sign"] and not got["weight_signed"] and not want["weight_signed"]
+    assert np.array_equal(got["scale_f32"].view(np.uint32), want["scale_f32"].view(np.uint32))
+    assert np.array_equal(got["scale_bits"], want["scale16"])
+    assert not got["zp"].any() and not want["zp"].any()
+    assert np.array_equal(got["weight"].view(np.uint8), want["weight"])
+
+
+def test_float_code_quantizer_rejects_per_channel_and_wrong_width():
+    w = _weights(1, 128, 8)
+    for bits, g, dq in ((8, 0, clib.DQ_F8E4M3), (4, 0, clib.DQ_F4), (4, 64, clib.DQ_F8E4M3), (8, 64, clib.DQ_F4)):
+        with pytest.raises(clib.BackendError) as e:
+            M_.a16_quantize(w, weight_bits=bits, q_group_size=g, dq_type=dq)
+        assert e.value.code == clib.MI_UNSUPPORTED
+
+
+@pytest.mark.parametrize("dq,bits", [("DQ_F8E4M3", 8), ("DQ_F4", 4)])
+def test_float_code_quantize_pack_run(orc, dq, bits):
+    """f32 weight -> float-code quantizer -> packed set -> dynamic matmul of the same type, against the oracle chain."""
+    import torch
+    rng = np.random.default_rng(bits)
+    M, K, N, g = 5, 512, 64, 128
+    w = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    xb = S.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    r = M_.a16_quantize(w, weight_bits=bits, q_group_size=g, dq_type=getattr(clib, dq))
+    ws = M_.A16Weight(r["weight"], r["scale_bits"], r["zp"], None, K=K, N=N, weight_bits=bits, q_group_size=g)
+    x = torch.from_numpy(xb.view(np.int16)).cuda().view(torch.bfloat16)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    M_.a16mm_dq_launch(ws, x, y_f32=y32, dq_type=getattr(clib, dq))
+    torch.cuda.synchronize()
+    ws.destroy()
+    o = orc.a16_quantize(w, bits=bits, g=g, dq_type=getattr(orc, dq))
+    _, want_pre = orc.a16matmul_dynamic(S.bf16_to_f32(xb), o["weight"].astype(np.float32), S.bf16_to_f32(o["scale16"]),
+                                        o["zp"].astype(np.float32), None, M=M, K=K, N=N, weight_bits=bits,
+                                        q_group_size=g, dq_type=getattr(orc, dq))
+    got = y32.cpu().numpy()
+    if bits == 4:
+        assert np.array_equal(got.view(np.uint32), want_pre.view(np.uint32))
+    else:
+        mag = np.abs(S.bf16_to_f32(xb).astype(np.float64)) @ np.abs(w.astype(np.float64)) * 1.2
+        assert np.all(np.abs(got - want_pre) <= mag * 2.0 ** -20)
+    # and the quantized product is close to the unquantized one
+    exact = S.bf16_to_f32(xb).astype(np.float64) @ w.astype(np.float64)
+    rel = np.linalg.norm(got - exact) / np.linalg.norm(exact)
+    assert rel < (0.06 if bits == 8 else 0.25)

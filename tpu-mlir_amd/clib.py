@@ -18,7 +18,8 @@ EXPORTS = [
     "mi_version", "mi_last_error", "mi_device_count",
     "mi_a16mm_init", "mi_a16mm_inference", "mi_a16mm_deinit",
     "mi_a16_weight_create", "mi_a16_weight_destroy", "mi_a16_weight_bytes", "mi_a16mm_launch",
-    "mi_a16mm_launch_group", "mi_a16mm_dq_launch", "mi_matmul_dq_launch", "mi_matmul_dq_inference",
+    "mi_a16mm_launch_group", "mi_a16mm_dq_launch", "mi_a16mm_dq_type_launch", "mi_matmul_dq_launch",
+    "mi_matmul_dq_inference",
     "mi_a16_weight_export_size", "mi_a16_weight_export", "mi_a16_weight_import", "mi_a16_quantize", "mi_llm_unpack",
     "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
     "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
@@ -62,7 +63,7 @@ class MatMulDqAttr(C.Structure):
 
 class A16QuantDesc(C.Structure):
     _fields_ = [("K", C.c_int64), ("N", C.c_int64), ("weight_bits", C.c_int), ("q_group_size", C.c_int),
-                ("symmetric", C.c_int), ("dtype", C.c_int)]
+                ("symmetric", C.c_int), ("dtype", C.c_int), ("dq_type", C.c_int)]
 
 
 class I8Attr(C.Structure):
@@ -147,6 +148,8 @@ def lib():
         L.mi_matmul_dq_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int,
                                           C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_dq_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi_a16mm_dq_type_launch.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
+                                              C.c_void_p]
         L.mi_a16mm_launch_group.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_int64,
                                             C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_void_p]
         L.mi_module_create.argtypes = [C.POINTER(C.c_void_p)]

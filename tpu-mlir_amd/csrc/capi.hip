@@ -317,6 +317,10 @@ int mi_a16_quantize(const mi_a16_quant_desc *d, const float *w_kn, void *weight,
   const int64_t gs = d->q_group_size == -1 ? d->K : d->q_group_size;
   MI_REQUIRE(gs >= 0 && (gs == 0 || d->K % gs == 0), MI_BAD_ARGUMENT, "mi_a16_quantize: K is not a multiple of q_group_size");
   MI_REQUIRE(gs == 0 || d->K / gs <= 65535, MI_UNSUPPORTED, "mi_a16_quantize: more than 65535 groups per row");
+  MI_REQUIRE(d->dq_type == MI_DQ_NONE || d->dq_type == MI_DQ_INT ||
+                 (gs != 0 && ((d->dq_type == MI_DQ_F8E4M3 && d->weight_bits == 8) ||
+                              (d->dq_type == MI_DQ_F4 && d->weight_bits == 4))),
+             MI_UNSUPPORTED, "mi_a16_quantize: float code types need groups, F8E4M3 8-bit and F4 4-bit weights");
   MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_a16_quantize: no GPU visible");
   return a16_quantize(d, w_kn, weight, scale16, scale_f32, zp, sign, weight_signed);
 }
@@ -342,7 +346,12 @@ int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
 
 int mi_a16mm_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                        void *stream) {
-  return a16_dq_launch(w, d_x, M, d_y, d_y_f32, (hipStream_t)stream);
+  return a16_dq_launch(w, MI_DQ_INT, d_x, M, d_y, d_y_f32, (hipStream_t)stream);
+}
+
+int mi_a16mm_dq_type_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int64_t M, uint16_t *d_y,
+                            float *d_y_f32, void *stream) {
+  return a16_dq_launch(w, dq_type, d_x, M, d_y, d_y_f32, (hipStream_t)stream);
 }
 
 int mi_a16mm_launch_group(const mi_a16_weight *const *w, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_y,
@@ -357,17 +366,21 @@ int mi_a16mm_init(const mi_a16mm_attr *attr, mi_infer_param *p) {
   MI_REQUIRE(attr && p, MI_BAD_ARGUMENT, "mi_a16mm_init: null argument");
   p->handle = nullptr;
   MI_REQUIRE(p->inputs && p->n_inputs >= 4, MI_BAD_ARGUMENT, "mi_a16mm_init: expects input, weight, scale, zp[, bias]");
-  MI_REQUIRE(attr->dynamic_quant == MI_DQ_NONE || attr->dynamic_quant == MI_DQ_INT, MI_UNSUPPORTED,
-             "mi_a16mm_init: only the integer dynamic-quantization types are handled");
-  if (attr->dynamic_quant == MI_DQ_INT) {
+  const int dq = attr->dynamic_quant;
+  MI_REQUIRE(dq == MI_DQ_NONE || dq == MI_DQ_INT || dq == MI_DQ_F8E4M3 || dq == MI_DQ_F4, MI_UNSUPPORTED,
+             "mi_a16mm_init: dynamic_quant must be MI_DQ_NONE, MI_DQ_INT, MI_DQ_F8E4M3 or MI_DQ_F4");
+  if (dq != MI_DQ_NONE) {
     MI_REQUIRE(attr->q_group_size != 0, MI_BAD_ARGUMENT,
                "mi_a16mm_init: dynamic quantization needs a group size (A16MatMul.cpp:42-43)");
+    // A16MatMul.cpp:63-91 decodes F4 codes only from 4-bit and F8E4M3 codes only from 8-bit weights
+    MI_REQUIRE((dq != MI_DQ_F8E4M3 || attr->weight_bits == 8) && (dq != MI_DQ_F4 || attr->weight_bits == 4),
+               MI_UNSUPPORTED, "mi_a16mm_init: F8E4M3 needs 8-bit and F4 needs 4-bit weights");
     MI_REQUIRE(attr->q_group_size > 0 && attr->K % 128 == 0 &&
                    (attr->q_group_size == 64 || attr->q_group_size % 128 == 0) &&
-                   (attr->weight_bits == 4 || attr->q_group_size <= 512),
+                   (dq != MI_DQ_INT || attr->weight_bits == 4 || attr->q_group_size <= 512),
                MI_UNSUPPORTED,
-               "mi_a16mm_init: dynamic quantization is handled for K % 128 == 0 and groups of 64 or k*128 (8-bit "
-               "weights: up to 512, where the reference's f32 group product stops being exact)");
+               "mi_a16mm_init: dynamic quantization is handled for K % 128 == 0 and groups of 64 or k*128 (integer "
+               "codes with 8-bit weights: up to 512, where the reference's f32 group product stops being exact)");
   }
   MI_REQUIRE(attr->w_transpose, MI_UNSUPPORTED, "mi_a16mm_init: only w_transpose weights ([N,K]) are handled");
   MI_REQUIRE(attr->weight_bits == 4 || attr->weight_bits == 8, MI_UNSUPPORTED, "mi_a16mm_init: weight_bits");
@@ -455,8 +468,9 @@ int mi_a16mm_inference(const mi_a16mm_attr *attr, mi_infer_param *p) {
   for (int64_t i = 0; i < M * K; ++i)
     hx[i] = f16 ? h_f32_to_f16(x[i]) : h_f32_to_bf16(x[i]);
   MI_HIP(hipMemcpyAsync(h->d_x.ptr, hx, (size_t)M * K * 2, hipMemcpyHostToDevice, h->stream));
-  if (attr->dynamic_quant == MI_DQ_INT)
-    rc = a16_dq_launch(h->w, (const uint16_t *)h->d_x.ptr, M, (uint16_t *)h->d_y.ptr, nullptr, h->stream);
+  if (attr->dynamic_quant != MI_DQ_NONE)
+    rc = a16_dq_launch(h->w, attr->dynamic_quant, (const uint16_t *)h->d_x.ptr, M, (uint16_t *)h->d_y.ptr, nullptr,
+                       h->stream);
   else
     rc = a16_launch(h->w, (const uint16_t *)h->d_x.ptr, M, (uint16_t *)h->d_y.ptr, nullptr, h->stream);
   if (rc != MI_SUCCESS)
@@ -952,10 +966,8 @@ int mi_cast_inference(const mi_cast_attr *a, mi_infer_param *p) {
 int mi_matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
                         int64_t N, int q_group_size, int dq_type, int dtype, uint16_t *d_y, float *d_y_f32,
                         void *stream) {
-  MI_REQUIRE(dq_type == MI_DQ_INT8 || dq_type == MI_DQ_INT4, MI_UNSUPPORTED,
-             "mi_matmul_dq_launch: only the INT8 / INT4 dynamic-quantization types are handled");
-  return matmul_dq_launch(d_left, d_right, right_transpose, M, K, N, q_group_size, dq_type == MI_DQ_INT8 ? 127 : 7,
-                          dtype, d_y, d_y_f32, (hipStream_t)stream);
+  return matmul_dq_launch(d_left, d_right, right_transpose, M, K, N, q_group_size, dq_type, dtype, d_y, d_y_f32,
+                          (hipStream_t)stream);
 }
 
 int mi_matmul_dq_inference(const mi_matmul_dq_attr *a, mi_infer_param *p) {
@@ -963,8 +975,8 @@ int mi_matmul_dq_inference(const mi_matmul_dq_attr *a, mi_infer_param *p) {
                  p->n_outputs >= 1 && p->outputs[0],
              MI_BAD_ARGUMENT, "mi_matmul_dq_inference: null argument");
   MI_REQUIRE(a->M >= 0 && a->K > 0 && a->N > 0, MI_BAD_ARGUMENT, "mi_matmul_dq_inference: bad shape");
-  MI_REQUIRE(a->dq_type == MI_DQ_INT8 || a->dq_type == MI_DQ_INT4, MI_UNSUPPORTED,
-             "mi_matmul_dq_inference: only the INT8 / INT4 dynamic-quantization types are handled");
+  MI_REQUIRE(a->dq_type == MI_DQ_INT8 || a->dq_type == MI_DQ_INT4 || a->dq_type == MI_DQ_F8E4M3 || a->dq_type == MI_DQ_F4,
+             MI_UNSUPPORTED, "mi_matmul_dq_inference: dq_type must be MI_DQ_INT8, MI_DQ_INT4, MI_DQ_F8E4M3 or MI_DQ_F4");
   MI_REQUIRE(a->out_dtype == MI_DT_BF16 || a->out_dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_matmul_dq_inference: out_dtype");
   const int64_t g = a->q_group_size == -1 ? a->K : a->q_group_size;
   MI_REQUIRE(g > 0, MI_BAD_ARGUMENT, "mi_matmul_dq_inference: dynamic quantization needs a group size");
@@ -988,8 +1000,7 @@ int mi_matmul_dq_inference(const mi_matmul_dq_attr *a, mi_infer_param *p) {
   MI_HIP(hipMemcpy(dl.ptr, hl.data(), nl * 2, hipMemcpyHostToDevice));
   MI_HIP(hipMemcpy(dr.ptr, hr.data(), nr * 2, hipMemcpyHostToDevice));
   rc = matmul_dq_launch((const uint16_t *)dl.ptr, (const uint16_t *)dr.ptr, a->right_transpose, a->M, a->K, a->N,
-                        a->q_group_size, a->dq_type == MI_DQ_INT8 ? 127 : 7, a->out_dtype, (uint16_t *)dy.ptr, nullptr,
-                        nullptr);
+                        a->q_group_size, a->dq_type, a->out_dtype, (uint16_t *)dy.ptr, nullptr, nullptr);
   if (rc)
     return rc;
   MI_HIP(hipDeviceSynchronize());

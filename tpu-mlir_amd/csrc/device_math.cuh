@@ -220,4 +220,56 @@ __device__ __forceinline__ void store_out(void *out, int64_t idx, int32_t v, int
   }
 }
 
+// ---- the 8- and 4-bit float codes of dynamic quantization (dq_type "F8E4M3", "F4")
+// f32 -> E4M3 code, round half to even, saturating to +-448, NaN -> 0x7f (f32_to_f8e4m3(src, true),
+// lib/Support/Float8.cpp:46-136).  Normals: add half an E4M3 ulp minus one plus the keep-bit, truncate, rebias the
+// exponent by 127 - 7.  Below 2^-6 the code is the value in units of 2^-9, which rintf gives directly (8 = the
+// smallest normal); f32 subnormals and zero give 0.
+__device__ __forceinline__ uint32_t f8e4m3_from_f32(float v) {
+  const uint32_t b = __float_as_uint(v);
+  const uint32_t a = b & 0x7fffffffu;
+  uint32_t r;
+  if (a > 0x7f800000u) {
+    r = 0x7f;
+  } else if (a >= 0x43e80000u) {  // 464 and above, infinity included: past the midpoint to the next code -> MAXNORM
+    r = 0x7e;                     // (464 itself is a tie that goes to the even code 0x7e)
+  } else if (a >= 0x3c800000u) {  // 2^-6
+    r = ((a + 0x7ffffu + ((a >> 20) & 1u)) >> 20) - (120u << 3);
+  } else if (a >= 0x00800000u) {
+    r = (uint32_t)rintf(__uint_as_float(a) * 512.0f);
+  } else {
+    r = 0;
+  }
+  return r | ((b >> 24) & 0x80u);
+}
+
+// E4M3 code -> f32 (f8e4m3_to_f32, Float8.cpp:140-191); 0x7f / 0xff are NaN
+__device__ __forceinline__ float f8e4m3_to_f32(uint32_t c) {
+  const uint32_t m = c & 0x7fu;
+  float mag = m >= 8 ? __uint_as_float((m << 20) + (120u << 23)) : (float)m * (1.0f / 512.0f);
+  if (m == 0x7f)
+    mag = __uint_as_float(0x7fffffffu);
+  return (c & 0x80u) ? -mag : mag;
+}
+
+// f32 -> E2M1 code (bit 3 = sign; magnitudes {0, .5, 1, 1.5, 2, 3, 4, 6}): f32_to_f4e2m1, lib/Support/Float4.cpp:7-22,
+// evaluated as written -- the first table entry with the strictly smallest fp32 |src - value| wins.  Ties therefore go
+// to the smaller magnitude, a negative input nearest to zero gives +0, and NaN, infinities and inputs too large for
+// the subtraction to change them give code 0.
+__device__ __forceinline__ uint32_t f4e2m1_from_f32(float v) {
+  uint32_t nearest = 0;
+  float best = fabsf(v - 0.0f);
+#pragma unroll
+  for (uint32_t i = 1; i < 16; ++i) {
+    const uint32_t m = i & 7u;
+    const float mag = m < 4 ? 0.5f * (float)m : (m == 4 ? 2.0f : (m == 5 ? 3.0f : (m == 6 ? 4.0f : 6.0f)));
+    const float d = fabsf(v - ((i & 8u) ? -mag : mag));
+    if (d < best) {
+      best = d;
+      nearest = i;
+    }
+  }
+  return nearest;
+}
+
 }  // namespace mi

@@ -1,5 +1,5 @@
-// tpu.A16MatMul with dynamic activation quantization, integer flavour (dq_type "INT4" / "INT8"), 4- and 8-bit weights:
-// lib/Dialect/Tpu/Interfaces/Common/A16MatMul.cpp:40-170.
+// tpu.A16MatMul with dynamic activation quantization, lib/Dialect/Tpu/Interfaces/Common/A16MatMul.cpp:40-170: the
+// integer types (dq_type "INT4" / "INT8", 4- and 8-bit weights) described first, the float code types at the end.
 //
 // Per activation row and per quantization group along K the reference scales the activations by their own abs-max to
 // integers in [-imax, imax] (imax = 7 for 4-bit weights, 127 for 8-bit), multiplies them with the integer weights (q - zp) group by
@@ -18,14 +18,42 @@
 // weights were flipped by 0x80 when packed) and, instead of an integer zero point, the exact float -(zp') * scale with
 // zp' the zero point in that unsigned domain: zp' = -nzs / scale comes back exactly, and the MFMA runs on the bytes
 // flipped to signed, so  sum_k code_k (w_k - zp) = mfma - (zp' - 128) * sum(codes).
+//
+// dq_type "F4" (4-bit weights hold E2M1 codes) and "F8E4M3" (8-bit weights hold E4M3 codes) run through the same two
+// kernels.  Activations are divided by amax / 6 or amax / 448 and rounded to the format; what is stored is the E4M3 byte
+// of that value (every E2M1 value is an E4M3 value), in the same fragment order.
+//   F4      nibbles -> E4M3 bytes with one byte permute per four, products on v_mfma_f32_16x16x32_fp8_fp8.  Every
+//           product is a multiple of 1/4 and the sums stay far below 2^24, so the result is exact in any order and the
+//           flavour is bit-exact like the integer ones.
+//   F8E4M3  both operands widened to bf16 (exact) and multiplied on v_mfma_f32_16x16x32_bf16: the reference's group
+//           product is an f32 matmul whose summation order its library chooses, so parity is to fp32 rounding of the
+//           group sums; the fp8 instruction itself loses about 2^-14 of a sum to operand alignment and is not used.
 #include "a16_common.cuh"
 #include "internal.h"
+
+#include <type_traits>
 
 #pragma clang fp contract(off)
 
 namespace mi {
 
 typedef __attribute__((ext_vector_type(4))) int i32x4;
+
+// dq_type families: integer codes (INT4 / INT8), E4M3 codes in 8-bit storage (F8E4M3), E2M1 codes in 4-bit storage (F4)
+constexpr int FLAV_INT = 0, FLAV_F8 = 1, FLAV_F4 = 2;
+
+// E2M1 magnitude codes are {0, .5, 1, 1.5, 2, 3, 4, 6}; as E4M3 bytes:
+constexpr uint32_t F4_AS_F8_LO = 0x3C383000u;  // 0, 0.5, 1, 1.5
+constexpr uint32_t F4_AS_F8_HI = 0x4C484440u;  // 2, 3, 4, 6
+__device__ __forceinline__ uint32_t f4_code_as_f8(uint32_t c) {
+  const uint32_t m = c & 7u;
+  const uint32_t tbl = m < 4 ? F4_AS_F8_LO : F4_AS_F8_HI;
+  return ((tbl >> (8 * (m & 3u))) & 0xffu) | ((c & 8u) << 4);
+}
+// four nibbles held one per byte (0..15 each) -> four E4M3 bytes
+__device__ __forceinline__ uint32_t f4x4_as_f8(uint32_t nib) {
+  return __builtin_amdgcn_perm(F4_AS_F8_HI, F4_AS_F8_LO, nib & 0x07070707u) | ((nib & 0x08080808u) << 4);
+}
 
 constexpr int DQ_WAVES = 8;
 constexpr int DQ_CHUNK = 128;  // groups whose terms fit the LDS buffer at once (1 KiB each)
@@ -37,7 +65,7 @@ __device__ __forceinline__ int dq_slot(int e) { return ((e & 1) << 1) | ((e & 2)
 // ---- activations -> integer codes in fragment order
 // aq, 4-bit: [m_blocks][k_tiles of 128][2][64 lanes][16 B]; 8-bit: [m_blocks][k_tiles of 64][64 lanes][16 B] with byte
 // 8 h + e of lane (row, kq) = k 32 h + 8 kq + e of the tile.  as_t / asum_t: [m_blocks][G][16 rows]
-template <int DT, int BITS>
+template <int DT, int BITS, int FLAV>
 __global__ __launch_bounds__(256) void dq_act_kernel(const uint16_t *__restrict__ x, int64_t M, int64_t K, int g, int G,
                                                       float imax, int64_t k_tiles, uint8_t *__restrict__ aq,
                                                       float *__restrict__ as_t, int32_t *__restrict__ asum_t,
@@ -62,16 +90,31 @@ __global__ __launch_bounds__(256) void dq_act_kernel(const uint16_t *__restrict_
     const float other = __shfl_xor(amax, o, 64);
     amax = amax > other ? amax : other;
   }
-  // :109-120: round(x / amax * imax), half away from zero
+  // :109-132: integer types round(x / amax * imax), half away from zero; the float types round x / (amax / imax) to
+  // their own grid, and the MFMA operand is that grid value's E4M3 byte (every E2M1 value is an E4M3 value)
   int sum = 0;
+  float fsum = 0.0f;
+  const float step = amax / imax;
   const int64_t mb = m >> 4;
   const int row = (int)(m & 15);
   for (int k = lane; k < g; k += 64) {
     const int64_t kk = (int64_t)gi * g + k;
     int code = 0;
-    if (live)
-      code = (int)roundf(H::to_f32(x[m * K + kk]) / amax * imax);
-    sum += code;
+    if (live) {
+      const float v = H::to_f32(x[m * K + kk]);
+      if constexpr (FLAV == FLAV_INT) {
+        code = (int)roundf(v / amax * imax);
+        sum += code;
+      } else if constexpr (FLAV == FLAV_F8) {
+        // F8E4M3(src, double step, true): the double quotient narrowed to f32 equals the f32 quotient (a quotient of
+        // two f32 values never lies close enough to an f32 rounding boundary for the double rounding to matter)
+        code = (int)f8e4m3_from_f32(__fdiv_rn(v, step));
+        fsum += f8e4m3_to_f32((uint32_t)code);
+      } else {
+        code = (int)f4_code_as_f8(f4e2m1_from_f32(__fdiv_rn(v, step)));
+        fsum += f8e4m3_to_f32((uint32_t)code);
+      }
+    }
     int64_t at;
     if constexpr (BITS == 4) {
       const int64_t kt = kk >> 7;
@@ -87,12 +130,14 @@ __global__ __launch_bounds__(256) void dq_act_kernel(const uint16_t *__restrict_
     aq[at] = (uint8_t)(int8_t)code;
   }
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1)
+  for (int o = 32; o > 0; o >>= 1) {
     sum += __shfl_xor(sum, o, 64);
+    fsum += __shfl_xor(fsum, o, 64);
+  }
   if (lane == 0) {
     const int64_t at = (mb * G + gi) * 16 + row;
-    as_t[at] = live ? amax / imax : 0.0f;  // :143-145 (cur_group_act_max[row] / imax)
-    asum_t[at] = sum;
+    as_t[at] = live ? step : 0.0f;  // :143-145 (cur_group_act_max[row] / imax)
+    asum_t[at] = FLAV == FLAV_INT ? sum : __float_as_int(fsum);  // what a nonzero weight zero point multiplies
   }
 }
 
@@ -122,8 +167,27 @@ __device__ __forceinline__ void unpack_bytes(uint32_t d, int &lo, int &hi) {
   hi = (int)((d >> 4) & 0x0F0F0F0Fu);
 }
 
-template <int DT, int BITS>
+__device__ __forceinline__ long pack64(uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); }
+
+// eight E4M3 bytes -> eight bf16 values (exact: 4 significant bits into 8).  The fp8 matrix instructions align their
+// products to the largest one and drop low bits (about 2^-14 of the group sum here); the bf16 instruction fed with the
+// same values adds the exact products with fp32 rounding, which is what the reference's f32 matmul does.
+__device__ __forceinline__ bf16x8 f8x8_as_bf16(uint32_t lo, uint32_t hi) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2;
+  const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, true);
+  const f32x2 p2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, false), p3 = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, true);
+  const u32x4 r = {__builtin_amdgcn_perm(__float_as_uint(p0[1]), __float_as_uint(p0[0]), 0x07060302u),
+                   __builtin_amdgcn_perm(__float_as_uint(p1[1]), __float_as_uint(p1[0]), 0x07060302u),
+                   __builtin_amdgcn_perm(__float_as_uint(p2[1]), __float_as_uint(p2[0]), 0x07060302u),
+                   __builtin_amdgcn_perm(__float_as_uint(p3[1]), __float_as_uint(p3[0]), 0x07060302u)};
+  return __builtin_bit_cast(bf16x8, r);
+}
+
+template <int DT, int BITS, int FLAV>
 __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
+  static_assert(FLAV == FLAV_INT || (FLAV == FLAV_F8 && BITS == 8) || (FLAV == FLAV_F4 && BITS == 4), "storage width");
+  // group sums: int32 for integer codes, fp32 for the float codes (32 k per matrix instruction)
+  using acc_t = typename std::conditional<FLAV == FLAV_INT, i32x4, f32x4>::type;
   using H = Half16<DT>;
   extern __shared__ __attribute__((aligned(16))) float terms[];  // [groups of the chunk][16 rows][16 columns]
   const int tid = threadIdx.x, lane = tid & 63;
@@ -147,11 +211,34 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
   for (int u0 = 0; u0 < units; u0 += chunk_units) {
     const int u1 = (u0 + chunk_units) < units ? (u0 + chunk_units) : units;
     for (int u = u0 + wave; u < u1; u += DQ_WAVES) {
-      i32x4 acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+      acc_t acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
       for (int t = 0; t < a.unit_tiles; ++t) {
         const int64_t kt = (int64_t)u * a.unit_tiles + t;
         const u32x4 w = wq[kt * 64];
-        if constexpr (BITS == 8) {
+        if constexpr (FLAV == FLAV_F8) {
+          // bytes [0, 8) of both operands are k 8 kq .. + 8 of the tile's first 32, bytes [8, 16) of its second 32
+          const u32x4 a0 = aq[kt * 64];
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(a0[0], a0[1]), f8x8_as_bf16(w[0], w[1]), acc[0], 0,
+                                                           0, 0);
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(a0[2], a0[3]), f8x8_as_bf16(w[2], w[3]), acc[0], 0,
+                                                           0, 0);
+        } else if constexpr (FLAV == FLAV_F4) {
+          const u32x4 a0 = aq[kt * 128], a1 = aq[kt * 128 + 64];
+          uint32_t lo[4], hi[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            lo[j] = f4x4_as_f8(w[j] & 0x0F0F0F0Fu);
+            hi[j] = f4x4_as_f8((w[j] >> 4) & 0x0F0F0F0Fu);
+          }
+          // dword j of the lane is k 32 j + 8 kq .. + 8; the activation bytes were written in the same slot order
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(a0[0], a0[1]), pack64(lo[0], hi[0]), acc[0], 0, 0, 0);
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(a0[2], a0[3]), pack64(lo[1], hi[1]), acc[0], 0, 0, 0);
+          const int second = a.unit_groups == 2 ? 1 : 0;  // with 64-wide groups k 64..127 is the next group
+          acc[second] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(a1[0], a1[1]), pack64(lo[2], hi[2]),
+                                                                   acc[second], 0, 0, 0);
+          acc[second] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(a1[2], a1[3]), pack64(lo[3], hi[3]),
+                                                                   acc[second], 0, 0, 0);
+        } else if constexpr (BITS == 8) {
           const u32x4 a0 = aq[kt * 64];
           const u32x4 ws = {w[0] ^ 0x80808080u, w[1] ^ 0x80808080u, w[2] ^ 0x80808080u, w[3] ^ 0x80808080u};
           acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0), __builtin_bit_cast(i32x4, ws),
@@ -184,15 +271,26 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
         } else {
           sc = H::to_f32(a.scale_t[qp + (int64_t)gi * 16]);
           const float nzs = a.nzs_t[qp + (int64_t)gi * 16];
-          zp = (sc != 0.0f ? (int)rintf(-nzs / sc) : 128) - 128;  // exact: nzs is -(zp') * scale without rounding
+          if constexpr (FLAV == FLAV_INT)
+            zp = (sc != 0.0f ? (int)rintf(-nzs / sc) : 128) - 128;  // exact: nzs is -(zp') * scale without rounding
+          else
+            zp = sc != 0.0f ? (int)rintf(-nzs / sc) : 0;  // E4M3 codes are stored as they are
         }
         const f32x4 as4 = *(const f32x4 *)(as_p + (int64_t)gi * 16);
         const i32x4 sum4 = *(const i32x4 *)(asum_p + (int64_t)gi * 16);
         float *dst = terms + (size_t)(gi - u0 * a.unit_groups) * 256;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int isum = acc[h][r] - zp * sum4[r];     // sum_k code_k (q_k - zp): exact
-          float t = (float)isum;                          // below 2^24 (checked on the host): exact
+          float t;
+          if constexpr (FLAV == FLAV_INT) {
+            const int isum = acc[h][r] - zp * sum4[r];   // sum_k code_k (q_k - zp): exact
+            t = (float)isum;                              // below 2^24 (checked on the host): exact
+          } else {
+            // sum_k a_k (w_k - zp) = sum_k a_k w_k - zp sum_k a_k; the producer of these weights sets zp = 0
+            // (Canonicalize/A16MatMul.cpp:98-106).  E2M1 operands keep every term a multiple of 1/4 far below 2^24,
+            // so that flavour is exact; E4M3 sums round in the matrix core's order.
+            t = zp != 0 ? acc[h][r] - (float)zp * __int_as_float(sum4[r]) : acc[h][r];
+          }
           t = t * as4[r];                                 // A16MatMul.cpp:153-156, left to right
           t = t * sc;
           dst[(4 * kq + r) * 16 + col] = t;
@@ -247,8 +345,9 @@ struct Dq2Args {
   int G, unit_tiles;  // tiles of 64 per group
 };
 
-template <int DT>
+template <int DT, int FLAV>
 __global__ __launch_bounds__(DQ_WAVES * 64) void dq2_gemm_kernel(Dq2Args a) {
+  using acc_t = typename std::conditional<FLAV == FLAV_INT, i32x4, f32x4>::type;
   extern __shared__ __attribute__((aligned(16))) float terms[];  // [groups of the chunk][16 rows][16 columns]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -264,18 +363,27 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq2_gemm_kernel(Dq2Args a) {
   for (int g0 = 0; g0 < a.G; g0 += DQ_CHUNK) {
     const int g1 = (g0 + DQ_CHUNK) < a.G ? (g0 + DQ_CHUNK) : a.G;
     for (int gi = g0 + wave; gi < g1; gi += DQ_WAVES) {
-      i32x4 acc = {0, 0, 0, 0};
+      acc_t acc = {0, 0, 0, 0};
       for (int t = 0; t < a.unit_tiles; ++t) {
         const int64_t kt = (int64_t)gi * a.unit_tiles + t;
-        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, al[kt * 64]),
-                                                    __builtin_bit_cast(i32x4, ar[kt * 64]), acc, 0, 0, 0);
+        const u32x4 l = al[kt * 64], r = ar[kt * 64];
+        if constexpr (FLAV == FLAV_INT) {
+          acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, l), __builtin_bit_cast(i32x4, r), acc, 0, 0,
+                                                      0);
+        } else if constexpr (FLAV == FLAV_F4) {  // E2M1 values as E4M3 bytes: exact sums on the fp8 instruction
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(l[0], l[1]), pack64(r[0], r[1]), acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(l[2], l[3]), pack64(r[2], r[3]), acc, 0, 0, 0);
+        } else {                                 // E4M3: exact products, fp32 sums (see f8x8_as_bf16)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(l[0], l[1]), f8x8_as_bf16(r[0], r[1]), acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(l[2], l[3]), f8x8_as_bf16(r[2], r[3]), acc, 0, 0, 0);
+        }
       }
       const f32x4 l4 = *(const f32x4 *)(asl + (int64_t)gi * 16);
       const float r1 = asr[(int64_t)gi * 16];
       float *dst = terms + (size_t)(gi - g0) * 256;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        float t = (float)acc[r];  // below 2^24 (checked on the host): exact
+        float t = (float)acc[r];  // integer codes: below 2^24 (checked on the host), exact
         t = t * l4[r];            // MatMul.cpp:577-581, left to right
         t = t * r1;
         dst[(4 * kq + r) * 16 + col] = t;
@@ -296,19 +404,29 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq2_gemm_kernel(Dq2Args a) {
 }
 
 int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
-                     int64_t N, int q_group_size, int imax_i, int dtype, uint16_t *d_y, float *d_y32,
+                     int64_t N, int q_group_size, int dq_type, int dtype, uint16_t *d_y, float *d_y32,
                      hipStream_t stream) {
   MI_REQUIRE(M >= 0 && M <= 65535 * 16 && N > 0 && N <= 65535 * 16 && K > 0, MI_BAD_ARGUMENT,
              "mi_matmul_dq_launch: bad shape");
   MI_REQUIRE(M == 0 || (d_left && d_right && d_y), MI_BAD_ARGUMENT, "mi_matmul_dq_launch: null argument");
-  MI_REQUIRE(imax_i == 127 || imax_i == 7, MI_UNSUPPORTED, "mi_matmul_dq_launch: integer dq types only (imax 127 / 7)");
+  // MatMul.cpp:449-462: imax by type name
+  float imax;
+  int64_t peak;  // largest |product| in the units that must stay below 2^24 for the reference's f32 sums to be exact
+  switch (dq_type) {
+  case MI_DQ_INT8: imax = 127.0f; peak = 127 * 127; break;
+  case MI_DQ_INT4: imax = 7.0f; peak = 7 * 7; break;
+  case MI_DQ_F4: imax = 6.0f; peak = 6 * 6 * 4; break;
+  case MI_DQ_F8E4M3: imax = 448.0f; peak = 0; break;  // rounded by the reference as well
+  default:
+    MI_REQUIRE(false, MI_UNSUPPORTED, "mi_matmul_dq_launch: dq_type must be MI_DQ_INT8, MI_DQ_INT4, MI_DQ_F8E4M3 or MI_DQ_F4");
+  }
   MI_REQUIRE(dtype == MI_DT_BF16 || dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_matmul_dq_launch: dtype");
   const int64_t g = q_group_size == -1 ? K : q_group_size;  // MatMul.cpp:465-466
   MI_REQUIRE(g > 0, MI_BAD_ARGUMENT, "mi_matmul_dq_launch: dynamic quantization needs a group size");
   MI_REQUIRE((K % 64) == 0 && (g % 64) == 0 && (K % g) == 0, MI_UNSUPPORTED,
              "mi_matmul_dq_launch: K and the group size must be multiples of 64, K a multiple of the group size");
-  MI_REQUIRE(g * imax_i * imax_i < (1 << 24), MI_UNSUPPORTED,
-             "mi_matmul_dq_launch: group too long for the integer sums to stay exact in the reference's f32 product");
+  MI_REQUIRE(g * peak < (1 << 24), MI_UNSUPPORTED,
+             "mi_matmul_dq_launch: group too long for the group sums to stay exact in the reference's f32 product");
   if (M == 0)
     return MI_SUCCESS;
   const int G = (int)(K / g);
@@ -332,20 +450,8 @@ int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_
                                                                                                         K, N);
     right_nk = rt;
   }
-  const float imax = (float)imax_i;
   const bool f16 = dtype == MI_DT_F16;
   const int64_t wl = m_blocks * 16 * G, wr = n_blocks * 16 * G;
-  if (f16) {
-    dq_act_kernel<MI_DT_F16, 8><<<dim3((unsigned)((wl + 3) / 4)), dim3(256), 0, stream>>>(
-        d_left, M, K, (int)g, G, imax, k_tiles, aq_l, as_l, sum_l, m_blocks * 16);
-    dq_act_kernel<MI_DT_F16, 8><<<dim3((unsigned)((wr + 3) / 4)), dim3(256), 0, stream>>>(
-        right_nk, N, K, (int)g, G, imax, k_tiles, aq_r, as_r, sum_r, n_blocks * 16);
-  } else {
-    dq_act_kernel<MI_DT_BF16, 8><<<dim3((unsigned)((wl + 3) / 4)), dim3(256), 0, stream>>>(
-        d_left, M, K, (int)g, G, imax, k_tiles, aq_l, as_l, sum_l, m_blocks * 16);
-    dq_act_kernel<MI_DT_BF16, 8><<<dim3((unsigned)((wr + 3) / 4)), dim3(256), 0, stream>>>(
-        right_nk, N, K, (int)g, G, imax, k_tiles, aq_r, as_r, sum_r, n_blocks * 16);
-  }
   Dq2Args a;
   a.aq_l = (const u32x4 *)aq_l;
   a.aq_r = (const u32x4 *)aq_r;
@@ -361,36 +467,71 @@ int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_
   const int chunk_groups = G < DQ_CHUNK ? G : DQ_CHUNK;
   const size_t lds_bytes = (size_t)(chunk_groups + 1) * 1024;
   dim3 grid((unsigned)n_blocks, (unsigned)m_blocks);
-  static bool attr_set = false;
-  if (!attr_set) {
-    (void)hipFuncSetAttribute((const void *)dq2_gemm_kernel<MI_DT_F16>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              160 * 1024);
-    (void)hipFuncSetAttribute((const void *)dq2_gemm_kernel<MI_DT_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              160 * 1024);
-    attr_set = true;
+  // both operands in the 8-bit fragment layout, whatever the code type
+#define MI_DQ2_RUN(DT_, FLAV_)                                                                                  \
+  {                                                                                                             \
+    dq_act_kernel<DT_, 8, FLAV_><<<dim3((unsigned)((wl + 3) / 4)), dim3(256), 0, stream>>>(                     \
+        d_left, M, K, (int)g, G, imax, k_tiles, aq_l, as_l, sum_l, m_blocks * 16);                              \
+    dq_act_kernel<DT_, 8, FLAV_><<<dim3((unsigned)((wr + 3) / 4)), dim3(256), 0, stream>>>(                     \
+        right_nk, N, K, (int)g, G, imax, k_tiles, aq_r, as_r, sum_r, n_blocks * 16);                            \
+    static bool attr_set = false;                                                                               \
+    if (!attr_set) {                                                                                            \
+      (void)hipFuncSetAttribute((const void *)dq2_gemm_kernel<DT_, FLAV_>,                                      \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                        \
+      attr_set = true;                                                                                          \
+    }                                                                                                           \
+    dq2_gemm_kernel<DT_, FLAV_><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);                           \
   }
-  if (f16)
-    dq2_gemm_kernel<MI_DT_F16><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);
-  else
-    dq2_gemm_kernel<MI_DT_BF16><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);
+  if (dq_type == MI_DQ_F8E4M3) {
+    if (f16)
+      MI_DQ2_RUN(MI_DT_F16, FLAV_F8)
+    else
+      MI_DQ2_RUN(MI_DT_BF16, FLAV_F8)
+  } else if (dq_type == MI_DQ_F4) {
+    if (f16)
+      MI_DQ2_RUN(MI_DT_F16, FLAV_F4)
+    else
+      MI_DQ2_RUN(MI_DT_BF16, FLAV_F4)
+  } else {
+    if (f16)
+      MI_DQ2_RUN(MI_DT_F16, FLAV_INT)
+    else
+      MI_DQ2_RUN(MI_DT_BF16, FLAV_INT)
+  }
+#undef MI_DQ2_RUN
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;
 }
 
-int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
+int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                   hipStream_t stream) {
   MI_REQUIRE(M >= 0 && M <= 65535 * 16, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: M out of range");
   MI_REQUIRE(w && w->qweight && (M == 0 || (d_x && d_y)), MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: null argument");
   MI_REQUIRE(w->g != 0, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: dynamic quantization needs a group size (A16MatMul.cpp:42)");
   const int g = w->g;
   const int bits = w->bits;
+  // A16MatMul.cpp:51-91: F8E4M3 codes are read from 8-bit, F4 codes from 4-bit weights
+  MI_REQUIRE(dq_type == MI_DQ_INT || (dq_type == MI_DQ_F8E4M3 && bits == 8) || (dq_type == MI_DQ_F4 && bits == 4),
+             MI_UNSUPPORTED, "mi_a16mm_dq_launch: dq_type must be MI_DQ_INT, MI_DQ_F8E4M3 (8-bit weights) or MI_DQ_F4 (4-bit)");
   MI_REQUIRE((w->K % 128) == 0 && (g == 64 || g % 128 == 0), MI_UNSUPPORTED,
              "mi_a16mm_dq_launch: K must be a multiple of 128 and the group size 64 or a multiple of 128");
-  // (1 << (weight_bits - 1)) - 1, A16MatMul.cpp:53-54; the reference's f32 group product is exact only while the
-  // integer sums stay below 2^24
-  const float imax = bits == 4 ? 7.0f : 127.0f;
-  MI_REQUIRE((int64_t)g * (bits == 4 ? 7 * 15 : 127 * 255) < (1 << 24), MI_UNSUPPORTED,
-             "mi_a16mm_dq_launch: group too long for the integer sums to stay exact in the reference's f32 product");
+  // imax: (1 << (weight_bits - 1)) - 1, get_f8e4m3_max() or get_f4e2m1_max(), A16MatMul.cpp:51-61.  The reference's f32
+  // group product is exact only while the sums of integer codes stay below 2^24; E2M1 products are quarter units up
+  // to 36 (15 with a zero point), E4M3 sums are rounded by the reference as well
+  float imax;
+  int64_t peak;
+  if (dq_type == MI_DQ_F8E4M3) {
+    imax = 448.0f;
+    peak = 0;
+  } else if (dq_type == MI_DQ_F4) {
+    imax = 6.0f;
+    peak = 6 * (6 + 15) * 4;
+  } else {
+    imax = bits == 4 ? 7.0f : 127.0f;
+    peak = bits == 4 ? 7 * 15 : 127 * 255;
+  }
+  MI_REQUIRE((int64_t)g * peak < (1 << 24), MI_UNSUPPORTED,
+             "mi_a16mm_dq_launch: group too long for the group sums to stay exact in the reference's f32 product");
   if (M == 0)
     return MI_SUCCESS;
   const int64_t m_blocks = (M + 15) / 16, rows_padded = m_blocks * 16;
@@ -405,21 +546,6 @@ int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16
   int32_t *asum_t = (int32_t *)(aq + aq_bytes + qp_bytes);
   const int64_t waves = rows_padded * G;
   const bool f16 = w->dtype == MI_DT_F16;
-#define MI_DQ_ACT(DT_, BITS_)                                                                      \
-  dq_act_kernel<DT_, BITS_><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(          \
-      d_x, M, w->K, g, G, imax, w->k_tiles, aq, as_t, asum_t, rows_padded)
-  if (bits == 4) {
-    if (f16)
-      MI_DQ_ACT(MI_DT_F16, 4);
-    else
-      MI_DQ_ACT(MI_DT_BF16, 4);
-  } else {
-    if (f16)
-      MI_DQ_ACT(MI_DT_F16, 8);
-    else
-      MI_DQ_ACT(MI_DT_BF16, 8);
-  }
-#undef MI_DQ_ACT
   DqArgs a;
   a.qw = (const u32x4 *)w->qweight;
   a.sz_t = w->sz_t;
@@ -441,28 +567,40 @@ int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16
   const int chunk_groups = G < DQ_CHUNK ? G : DQ_CHUNK;
   const size_t lds_bytes = (size_t)(chunk_groups + 1) * 1024;
   dim3 grid((unsigned)w->row_blocks, (unsigned)m_blocks);
-#define MI_DQ_GEMM(DT_, BITS_)                                                                                   \
+#define MI_DQ_RUN(DT_, BITS_, FLAV_)                                                                             \
   {                                                                                                             \
+    dq_act_kernel<DT_, BITS_, FLAV_><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(              \
+        d_x, M, w->K, g, G, imax, w->k_tiles, aq, as_t, asum_t, rows_padded);                                   \
     static bool attr_set = false;                                                                               \
     if (!attr_set) {                                                                                            \
-      (void)hipFuncSetAttribute((const void *)dq_gemm_kernel<DT_, BITS_>,                                       \
+      (void)hipFuncSetAttribute((const void *)dq_gemm_kernel<DT_, BITS_, FLAV_>,                                \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                        \
       attr_set = true;                                                                                          \
     }                                                                                                           \
-    dq_gemm_kernel<DT_, BITS_><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);                            \
+    dq_gemm_kernel<DT_, BITS_, FLAV_><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);                     \
   }
-  if (bits == 4) {
+  if (dq_type == MI_DQ_F8E4M3) {
     if (f16)
-      MI_DQ_GEMM(MI_DT_F16, 4)
+      MI_DQ_RUN(MI_DT_F16, 8, FLAV_F8)
     else
-      MI_DQ_GEMM(MI_DT_BF16, 4)
+      MI_DQ_RUN(MI_DT_BF16, 8, FLAV_F8)
+  } else if (dq_type == MI_DQ_F4) {
+    if (f16)
+      MI_DQ_RUN(MI_DT_F16, 4, FLAV_F4)
+    else
+      MI_DQ_RUN(MI_DT_BF16, 4, FLAV_F4)
+  } else if (bits == 4) {
+    if (f16)
+      MI_DQ_RUN(MI_DT_F16, 4, FLAV_INT)
+    else
+      MI_DQ_RUN(MI_DT_BF16, 4, FLAV_INT)
   } else {
     if (f16)
-      MI_DQ_GEMM(MI_DT_F16, 8)
+      MI_DQ_RUN(MI_DT_F16, 8, FLAV_INT)
     else
-      MI_DQ_GEMM(MI_DT_BF16, 8)
+      MI_DQ_RUN(MI_DT_BF16, 8, FLAV_INT)
   }
-#undef MI_DQ_GEMM
+#undef MI_DQ_RUN
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;
 }

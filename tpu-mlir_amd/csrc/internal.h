@@ -76,12 +76,12 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
 enum { WS_SPLIT_K = 0, WS_DYNAMIC_QUANT = 1 };
 int stream_workspace(hipStream_t st, int purpose, size_t bytes, bool zeroed, void **out);
 
-// dynamic activation quantization, integer flavour (dq_kernels.hip)
-int a16_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
+// dynamic activation quantization (dq_kernels.hip); dq_type: MI_DQ_INT, MI_DQ_F8E4M3 (8-bit weights), MI_DQ_F4 (4-bit)
+int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                   hipStream_t stream);
 
 int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
-                     int64_t N, int q_group_size, int imax, int dtype, uint16_t *d_y, float *d_y32,
+                     int64_t N, int q_group_size, int dq_type, int dtype, uint16_t *d_y, float *d_y32,
                      hipStream_t stream);
 
 // weight producers (quant_kernels.hip); arguments are validated by the callers

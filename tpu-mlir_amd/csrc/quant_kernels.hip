@@ -65,8 +65,9 @@ __global__ void quant_sign_kernel(const float *__restrict__ mn, int64_t count, i
 //                                max_int = 15 / 255
 __global__ void quant_params_kernel(const float *__restrict__ mn, const float *__restrict__ mx,
                                     const float *__restrict__ amax, int64_t count, int bits, int grouped, int sym,
-                                    int f16, const int *__restrict__ sign_p, float *__restrict__ scale_out,
-                                    uint16_t *__restrict__ scale16_out, uint8_t *__restrict__ zp_out) {
+                                    int f16, int dq_type, const int *__restrict__ sign_p,
+                                    float *__restrict__ scale_out, uint16_t *__restrict__ scale16_out,
+                                    uint8_t *__restrict__ zp_out) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= count)
     return;
@@ -77,6 +78,9 @@ __global__ void quant_params_kernel(const float *__restrict__ mn, const float *_
   if (!grouped && bits != 4) {
     const int pow_value = sign ? bits - 1 : bits;
     scale = (float)((double)amax[i] / (double)((1 << pow_value) - 1));
+  } else if (grouped && (dq_type == MI_DQ_F8E4M3 || dq_type == MI_DQ_F4)) {
+    scale = fabsf(amax[i]) / (dq_type == MI_DQ_F4 ? 6.0f : 448.0f);  // :96-106, get_f4e2m1_max() / get_f8e4m3_max()
+    zp = 0;
   } else if (grouped && sym) {
     scale = 2 * fabsf(amax[i]) / max_int;
   } else {
@@ -93,7 +97,7 @@ __global__ void quant_params_kernel(const float *__restrict__ mn, const float *_
 // ---- pass 3: quantize + transpose + pack (weightQuantization :147-216).  A workgroup owns a 64 (k) x 64 (n) tile.
 constexpr int QT = 64;
 __global__ __launch_bounds__(256) void quant_pack_kernel(const float *__restrict__ w_kn, int64_t K, int64_t N,
-                                                          int64_t gs, int64_t G, int bits, int as_int8,
+                                                          int64_t gs, int64_t G, int bits, int as_int8, int dq_type,
                                                           const float *__restrict__ scale,
                                                           const uint8_t *__restrict__ zp, uint8_t *__restrict__ q) {
   __shared__ uint8_t tile[QT][QT + 4];  // [k][n]
@@ -104,9 +108,21 @@ __global__ __launch_bounds__(256) void quant_pack_kernel(const float *__restrict
     uint8_t code = 0;
     if (k < K && n < N) {
       const int64_t qi = gs ? n * G + k / gs : n;
-      const float t = roundf(w_kn[k * N + n] / scale[qi]) + (float)zp[qi];
+      float t = w_kn[k * N + n] / scale[qi];
+      if (dq_type != MI_DQ_F8E4M3 && dq_type != MI_DQ_F4)
+        t = roundf(t);  // :181-182: the float code types keep the quotient
+      t += (float)zp[qi];
       const int64_t v = to_int_f32(t, MI_ROUND_HALF_AWAY_FROM_ZERO);  // to_uint4 / to_uint8 / to_int8
-      if (bits == 4)
+      if (dq_type == MI_DQ_F8E4M3) {
+        code = (uint8_t)f8e4m3_from_f32(t);  // :185-186, saturating
+        // an all-zero group has scale 0 and the quotient 0 / 0: the NaN an x86 host generates there carries the sign
+        // bit, which the conversion copies into the code
+        if (t != t && scale[qi] == scale[qi] && w_kn[k * N + n] == w_kn[k * N + n])
+          code = 0xff;
+      }
+      else if (dq_type == MI_DQ_F4)
+        code = (uint8_t)f4e2m1_from_f32(t);  // :194-200
+      else if (bits == 4)
         code = (uint8_t)(v > 15 ? 15 : (v < 0 ? 0 : v));
       else if (as_int8)
         code = (uint8_t)(int8_t)(v > 127 ? 127 : (v < -128 ? -128 : v));
@@ -235,12 +251,12 @@ int a16_quantize(const mi_a16_quant_desc *d, const float *h_w_kn, void *h_weight
                                                                                     d_am);
   quant_sign_kernel<<<dim3(1), dim3(256)>>>(d_mn, count, d_sign);
   quant_params_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256)>>>(
-      d_mn, d_mx, d_am, count, bits, gs != 0, sym, d->dtype == MI_DT_F16, d_sign, d_scale, d_s16, d_zp);
+      d_mn, d_mx, d_am, count, bits, gs != 0, sym, d->dtype == MI_DT_F16, d->dq_type, d_sign, d_scale, d_s16, d_zp);
   int sign = 0;
   MI_HIP(hipMemcpy(&sign, d_sign, 4, hipMemcpyDeviceToHost));
   const int as_int8 = !gs && sign && bits == 8;  // :413-416
   quant_pack_kernel<<<dim3((unsigned)((N + QT - 1) / QT), (unsigned)((K + QT - 1) / QT)), dim3(256)>>>(
-      d_w, K, N, gs, G, bits, as_int8, d_scale, d_zp, d_q);
+      d_w, K, N, gs, G, bits, as_int8, d->dq_type, d_scale, d_zp, d_q);
   MI_HIP(hipGetLastError());
   MI_HIP(hipMemcpy(h_weight, d_q, qbytes, hipMemcpyDeviceToHost));
   MI_HIP(hipMemcpy(h_scale16, d_s16, (size_t)count * 2, hipMemcpyDeviceToHost));

@@ -241,11 +241,12 @@ class A16Weight:
 PACK_GPTQ, PACK_AWQ = 0, 1
 
 
-def a16_quantize(w_kn, *, weight_bits, q_group_size, symmetric=False, dtype=DT_BF16):
+def a16_quantize(w_kn, *, weight_bits, q_group_size, symmetric=False, dtype=DT_BF16, dq_type=clib.DQ_NONE):
     """A16MatMulAdjust on the GPU: f32 weight [K, N] of a top-level matmul -> the operand set of tpu.A16MatMul.
 
     Returns dict(weight uint8/int8 [N, K/2] or [N, K], scale_bits uint16 [N, G], scale_f32 [N, G], zp uint8 [N, G],
-    sign, weight_signed); weight/scale_bits/zp are what A16Weight takes.
+    sign, weight_signed); weight/scale_bits/zp are what A16Weight takes.  dq_type DQ_F8E4M3 (8-bit) / DQ_F4 (4-bit)
+    store the float codes of the matching dynamic-quantization types instead of integers (groups only).
     """
     w = np.ascontiguousarray(w_kn, dtype=np.float32)
     if w.ndim != 2:
@@ -260,7 +261,7 @@ def a16_quantize(w_kn, *, weight_bits, q_group_size, symmetric=False, dtype=DT_B
     sf = np.zeros((N, G), dtype=np.float32)
     zp = np.zeros((N, G), dtype=np.uint8)
     sign, wsigned = C.c_int(0), C.c_int(0)
-    desc = clib.A16QuantDesc(K, N, weight_bits, q_group_size, int(symmetric), dtype)
+    desc = clib.A16QuantDesc(K, N, weight_bits, q_group_size, int(symmetric), dtype, int(dq_type))
     check(clib.lib().mi_a16_quantize(C.byref(desc), w.ctypes.data, q.ctypes.data, s16.ctypes.data, sf.ctypes.data,
                                      zp.ctypes.data, C.byref(sign), C.byref(wsigned)))
     if wsigned.value:
@@ -318,8 +319,9 @@ def matmul_dq_launch(left, right, *, right_transpose=False, q_group_size, dq_typ
     return y
 
 
-def a16mm_dq_launch(w, x, y=None, y_f32=None, stream=None):
-    """As a16mm_launch, with the reference's dynamic integer activation quantization (4-bit weights)."""
+def a16mm_dq_launch(w, x, y=None, y_f32=None, stream=None, dq_type=clib.DQ_INT):
+    """As a16mm_launch, with the reference's dynamic activation quantization: dq_type DQ_INT (integer codes, 4- or 8-bit
+    weights), DQ_F8E4M3 (8-bit weights holding E4M3 codes) or DQ_F4 (4-bit weights holding E2M1 codes)."""
     import torch
     tdt = torch.float16 if w.dtype == DT_F16 else torch.bfloat16
     if not (x.is_cuda and x.dtype == tdt and x.is_contiguous() and x.shape[-1] == w.K):
@@ -332,7 +334,8 @@ def a16mm_dq_launch(w, x, y=None, y_f32=None, stream=None):
     if y_f32 is not None and not (y_f32.is_cuda and y_f32.dtype == torch.float32 and y_f32.is_contiguous()
                                   and y_f32.numel() == M * w.N):
         raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_dq_launch: bad y_f32 tensor")
-    check(clib.lib().mi_a16mm_dq_launch(w.handle, _dptr(x), M, _dptr(y), _dptr(y_f32), _stream_ptr(stream)))
+    check(clib.lib().mi_a16mm_dq_type_launch(w.handle, int(dq_type), _dptr(x), M, _dptr(y), _dptr(y_f32),
+                                             _stream_ptr(stream)))
     return y
 
 
