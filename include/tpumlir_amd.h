@@ -184,6 +184,11 @@ int mi_a16_quantize(const mi_a16_quant_desc *desc, const float *w_kn, void *weig
 enum { MI_PACK_GPTQ = 0, MI_PACK_AWQ = 1 };
 int mi_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qzeros, int64_t K, int64_t N, int64_t G,
                   uint8_t *weight, uint8_t *zp);
+/* A16MatMulToGroup (lib/Dialect/Tpu/Canonicalize/A16MatMul.cpp:432-499): the rewrite of a per-channel op
+ * (q_group_size <= 0, 16-bit scales, u8 zero points) into the grouped form -- every scale and zero point repeated
+ * K / 128 times ([N, s] -> [N, s * K / 128]); the caller then sets q_group_size = 128.  Same math, same results. */
+int mi_a16_to_group(const uint16_t *scale, int64_t scale_num, const uint8_t *zp, int64_t zp_num, int64_t K,
+                    uint16_t *scale_out, uint8_t *zp_out);
 
 /* y[M,N] = round(x[M,K] * dequant(W)^T + bias).  d_x/d_y are DEVICE pointers to bf16/f16 bit patterns;
  * d_y_f32 (optional DEVICE pointer, may be NULL) receives the fp32 result before output rounding.

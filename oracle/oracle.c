@@ -1325,6 +1325,22 @@ int orc_a16_quantize_dq(const float *w_kn, int64_t K, int64_t N, int bits, int g
   return 0;
 }
 
+/* A16MatMulToGroup, lib/Dialect/Tpu/Canonicalize/A16MatMul.cpp:432-499 (:460-475: tile = K / 128, every entry
+ * repeated tile times) */
+int orc_a16_to_group(const uint16_t *scale, int64_t scale_num, const uint8_t *zp, int64_t zp_num, int64_t K,
+                     uint16_t *scale_out, uint8_t *zp_out) {
+  const int64_t tile = K / 128;
+  if (!scale || !zp || !scale_out || !zp_out || tile <= 0 || K % 128)
+    return -1;
+  for (int64_t i = 0; i < scale_num; ++i)
+    for (int64_t j = 0; j < tile; ++j)
+      scale_out[i * tile + j] = scale[i];
+  for (int64_t i = 0; i < zp_num; ++i)
+    for (int64_t j = 0; j < tile; ++j)
+      zp_out[i * tile + j] = zp[i];
+  return 0;
+}
+
 int orc_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qzeros, int64_t K, int64_t N, int64_t G,
                    uint8_t *q, uint8_t *zp) {
   if ((bits != 4 && bits != 8) || (mode != ORC_PACK_GPTQ && mode != ORC_PACK_AWQ))

@@ -38,6 +38,8 @@
  *   orc_a16_quantize             on-grid weights are recovered exactly, |w - dequant(q)| <= scale/2 inside the
  *                                clamp range, closed-form scale/zp, nibble order via the A16MatMul dequantizer
  *                                (tests/test_oracle_packers.py)
+ *   orc_a16_to_group             numpy.repeat; the per-channel and the regrouped operand sets give identical
+ *                                orc_a16matmul results (tests/test_oracle_packers.py)
  *   orc_llm_unpack               inverse of independently written GPTQ / AWQ packers, AutoAWQ's published pack
  *                                order (tests/test_oracle_packers.py)
  *   orc_a16_dequant              one-hot activations recover nibble order,
@@ -282,6 +284,9 @@ int orc_a16_quantize_dq(const float *w_kn, int64_t K, int64_t N, int bits, int g
 enum { ORC_PACK_GPTQ = 0, ORC_PACK_AWQ = 1 };
 int orc_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qzeros, int64_t K, int64_t N, int64_t G,
                    uint8_t *q, uint8_t *zp);
+/* A16MatMulToGroup (Canonicalize/A16MatMul.cpp:432-499): per-channel scale / zp entries repeated K / 128 times. */
+int orc_a16_to_group(const uint16_t *scale, int64_t scale_num, const uint8_t *zp, int64_t zp_num, int64_t K,
+                     uint16_t *scale_out, uint8_t *zp_out);
 
 #ifdef __cplusplus
 }

@@ -383,6 +383,22 @@ def a16_quantize(w_kn, *, bits, g, symmetric=False, f16=False, dq_type=DQ_INT):
     return dict(weight=q, scale_f32=sf, scale16=s16, zp=zp, sign=bool(sign.value), weight_signed=bool(wsigned.value))
 
 
+def a16_to_group(scale16, zp, K):
+    """A16MatMulToGroup on scale bit patterns [N, s] and zero points [N, s]."""
+    scale16 = np.ascontiguousarray(scale16, dtype=np.uint16)
+    zp = np.ascontiguousarray(zp, dtype=np.uint8)
+    tile = K // 128
+    so = np.zeros((scale16.shape[0], scale16.shape[1] * tile), dtype=np.uint16)
+    zo = np.zeros((zp.shape[0], zp.shape[1] * tile), dtype=np.uint8)
+    L = lib()
+    L.orc_a16_to_group.restype = C.c_int
+    rc = L.orc_a16_to_group(_p(scale16, C.c_uint16), C.c_int64(scale16.size), _p(zp, C.c_uint8), C.c_int64(zp.size),
+                            C.c_int64(K), _p(so, C.c_uint16), _p(zo, C.c_uint8))
+    if rc != 0:
+        raise RuntimeError("orc_a16_to_group: bad arguments")
+    return so, zo
+
+
 def llm_unpack(mode, bits, qweight, qzeros, K, N):
     """GPTQ / AWQ int32 checkpoint tensors -> (weight [N, K/2] or [N, K] uint8, zp [N, G] uint8)."""
     qweight = np.ascontiguousarray(qweight, dtype=np.int32)

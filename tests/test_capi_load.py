@@ -86,6 +86,9 @@ def test_weight_producer_and_blob_argument_errors():
     L = clib.lib()
     assert L.mi_a16_quantize(None, None, None, None, None, None, None, None) == clib.MI_BAD_ARGUMENT
     assert L.mi_llm_unpack(0, 4, None, None, 8, 8, 1, None, None) == clib.MI_BAD_ARGUMENT
+    assert L.mi_a16_to_group(None, 1, None, 1, 128, None, None) == clib.MI_BAD_ARGUMENT
+    so, zo = M.a16_to_group(np.array([[7], [9]], np.uint16), np.array([[1], [2]], np.uint8), K=256)  # host only
+    assert so.tolist() == [[7, 7], [9, 9]] and zo.tolist() == [[1, 1], [2, 2]]
     assert L.mi_a16mm_dq_launch(None, None, 1, None, None, None) == clib.MI_BAD_ARGUMENT
     assert L.mi_a16mm_dq_type_launch(None, clib.DQ_F8E4M3, None, 1, None, None, None) == clib.MI_BAD_ARGUMENT
     for bits, g, dq in ((8, 0, clib.DQ_F8E4M3), (4, 64, clib.DQ_F8E4M3), (8, 64, clib.DQ_F4)):

@@ -201,3 +201,32 @@ def test_float_code_quantize_pack_run(orc, dq, bits):
     exact = S.bf16_to_f32(xb).astype(np.float64) @ w.astype(np.float64)
     rel = np.linalg.norm(got - exact) / np.linalg.norm(exact)
     assert rel < (0.06 if bits == 8 else 0.25)
+
+
+def test_to_group_and_run(orc):
+    """A16MatMulToGroup through the C ABI: the repeated parameters equal the oracle's, and the regrouped set (g = 128)
+    multiplies to the same result as the per-channel set, within the fp32 agreement of the two kernels' summation."""
+    import torch
+    cmp = pkg("compare")
+    rng = np.random.default_rng(3)
+    M, K, N = 4, 512, 96
+    w = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    xb = S.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    x = torch.from_numpy(xb.view(np.int16)).cuda().view(torch.bfloat16)
+    for bits in (4, 8):
+        r = M_.a16_quantize(w, weight_bits=bits, q_group_size=0)
+        so, zo = M_.a16_to_group(r["scale_bits"], r["zp"], K=K)
+        wso, wzo = orc.a16_to_group(r["scale_bits"], r["zp"], K)
+        assert np.array_equal(so, wso) and np.array_equal(zo, wzo) and so.shape == (N, K // 128)
+        pre = []
+        for sc, zp, g in ((r["scale_bits"], r["zp"], 0), (so, zo, 128)):
+            ws = M_.A16Weight(r["weight"], sc, zp, None, K=K, N=N, weight_bits=bits, q_group_size=g)
+            y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+            M_.a16mm_launch(ws, x, y_f32=y32)
+            torch.cuda.synchronize()
+            ws.destroy()
+            pre.append(y32.cpu().numpy())
+        assert cmp.max_abs_over_rms(pre[0], pre[1]) <= 2e-5
+    with pytest.raises(clib.BackendError) as e:
+        M_.a16_to_group(r["scale_bits"], r["zp"], K=200)
+    assert e.value.code == clib.MI_UNSUPPORTED

@@ -193,3 +193,25 @@ def test_awq_unpack_inverts_packer(orc):
     q, zp = orc.llm_unpack(orc.PACK_AWQ, 4, qw, qz, K, N)
     assert np.array_equal(_unpack4(q), codes.T)
     assert np.array_equal(zp, zeros.T)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_to_group_repeats_and_keeps_the_product(orc, bits):
+    """A16MatMulToGroup: entries repeated K / 128 times; the per-channel operand set and the regrouped one (run with
+    q_group_size 128) must give the same matmul result, bit for bit, in the (separately pinned) oracle matmul."""
+    rng = np.random.default_rng(bits)
+    K, N, M = 384, 20, 3
+    w = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    r = orc.a16_quantize(w, bits=bits, g=0)
+    so, zo = orc.a16_to_group(r["scale16"], r["zp"], K)
+    assert so.shape == (N, 3) and zo.shape == (N, 3)
+    assert np.array_equal(so, np.repeat(r["scale16"], 3, axis=1)) and np.array_equal(zo, np.repeat(r["zp"], 3, axis=1))
+    x = S.bf16_to_f32(S.bf16_round(rng.standard_normal((M, K)).astype(np.float32)))
+    wf = (r["weight"].view(np.int8) if r["weight_signed"] else r["weight"]).astype(np.float32)
+    a, _ = orc.a16matmul(x, wf, S.bf16_to_f32(r["scale16"]), r["zp"].astype(np.float32), None, M=M, K=K, N=N,
+                         weight_bits=bits, q_group_size=0)
+    b, _ = orc.a16matmul(x, wf, S.bf16_to_f32(so), zo.astype(np.float32), None, M=M, K=K, N=N, weight_bits=bits,
+                         q_group_size=128)
+    assert np.array_equal(a, b)
+    with pytest.raises(RuntimeError):
+        orc.a16_to_group(r["scale16"], r["zp"], 200)

@@ -10,4 +10,4 @@ from .clib import (MI_SUCCESS, MI_UNSUPPORTED, MI_BAD_ARGUMENT, MI_HIP_ERROR, Ba
                    device_count, last_error, library_path, version)
 from .ops import (A16MatMul, A16Weight, MatMulInt8, Module, RequantDesc, a16mm_launch,  # noqa: F401
                   a16mm_launch_group, i8mm_launch, cast, cast_launch, requant_int, requant_int_axis, requant_launch,
-                  a16_quantize, llm_unpack, a16mm_dq_launch, matmul_dq, matmul_dq_launch, PACK_GPTQ, PACK_AWQ)
+                  a16_quantize, a16_to_group, llm_unpack, a16mm_dq_launch, matmul_dq, matmul_dq_launch, PACK_GPTQ, PACK_AWQ)

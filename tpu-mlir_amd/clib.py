@@ -21,6 +21,7 @@ EXPORTS = [
     "mi_a16mm_launch_group", "mi_a16mm_dq_launch", "mi_a16mm_dq_type_launch", "mi_matmul_dq_launch",
     "mi_matmul_dq_inference",
     "mi_a16_weight_export_size", "mi_a16_weight_export", "mi_a16_weight_import", "mi_a16_quantize", "mi_llm_unpack",
+    "mi_a16_to_group",
     "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
     "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
     "mi_cast_inference", "mi_cast_launch",
@@ -141,6 +142,7 @@ def lib():
         L.mi_a16_weight_import.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_size_t]
         L.mi_a16_quantize.argtypes = [C.POINTER(A16QuantDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        L.mi_a16_to_group.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
         L.mi_llm_unpack.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
                                     C.c_void_p, C.c_void_p]
         L.mi_a16_weight_destroy.restype = None

@@ -339,6 +339,23 @@ int mi_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qze
   return llm_unpack(mode, bits, qweight, qzeros, K, N, G, weight, zp);
 }
 
+// A16MatMulToGroup (Canonicalize/A16MatMul.cpp:432-499): per-channel parameters repeated K / 128 times along a new
+// group axis, after which the op carries q_group_size 128.  Tiny host arrays: no kernel.
+int mi_a16_to_group(const uint16_t *scale, int64_t scale_num, const uint8_t *zp, int64_t zp_num, int64_t K,
+                    uint16_t *scale_out, uint8_t *zp_out) {
+  MI_REQUIRE(scale && zp && scale_out && zp_out && scale_num > 0 && zp_num > 0, MI_BAD_ARGUMENT,
+             "mi_a16_to_group: null argument");
+  MI_REQUIRE(K >= 128 && K % 128 == 0, MI_UNSUPPORTED, "mi_a16_to_group: K must be a multiple of 128");
+  const int64_t tile = K / 128;  // :460-461
+  for (int64_t i = 0; i < scale_num; ++i)
+    for (int64_t j = 0; j < tile; ++j)
+      scale_out[i * tile + j] = scale[i];
+  for (int64_t i = 0; i < zp_num; ++i)
+    for (int64_t j = 0; j < tile; ++j)
+      zp_out[i * tile + j] = zp[i];
+  return MI_SUCCESS;
+}
+
 int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                     void *stream) {
   return a16_launch(w, d_x, M, d_y, d_y_f32, (hipStream_t)stream);

@@ -270,6 +270,21 @@ def a16_quantize(w_kn, *, weight_bits, q_group_size, symmetric=False, dtype=DT_B
                 weight_signed=bool(wsigned.value))
 
 
+def a16_to_group(scale_bits, zp, *, K):
+    """A16MatMulToGroup: per-channel scale bit patterns [N, s] / zero points [N, s] -> [N, s * K / 128]; the op then
+    runs with q_group_size = 128."""
+    scale_bits = np.ascontiguousarray(scale_bits, dtype=np.uint16)
+    zp = np.ascontiguousarray(zp, dtype=np.uint8)
+    if scale_bits.ndim != 2 or zp.ndim != 2:
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16_to_group: scale and zp must be 2-D")
+    tile = max(K // 128, 0)
+    so = np.zeros((scale_bits.shape[0], scale_bits.shape[1] * tile), dtype=np.uint16)
+    zo = np.zeros((zp.shape[0], zp.shape[1] * tile), dtype=np.uint8)
+    check(clib.lib().mi_a16_to_group(scale_bits.ctypes.data, scale_bits.size, zp.ctypes.data, zp.size, K,
+                                     so.ctypes.data, zo.ctypes.data))
+    return so, zo
+
+
 def llm_unpack(mode, bits, qweight, qzeros, *, K, N):
     """GPTQ / AWQ int32 checkpoint tensors -> (weight uint8 [N, K/2] or [N, K], zp uint8 [N, G]) on the GPU."""
     qweight = np.ascontiguousarray(qweight, dtype=np.int32)
