@@ -258,6 +258,28 @@ def bench_dynamic_quant(pkg, S, torch, steps=40):
     return out
 
 
+def bench_f8_matmul(pkg, torch, clib, steps=20):
+    """tpu.MatMul on E4M3 codes with per-channel F8 output requantization (codes out), random finite codes."""
+    out = []
+    rng = np.random.default_rng(12)
+    for M, K, N in ((4096, 4096, 4096), (256, 1024, 1024)):
+        a = torch.from_numpy((rng.integers(0, 256, size=(M, K)).astype(np.uint8) & np.uint8(0xD7))).cuda()
+        b = torch.from_numpy((rng.integers(0, 256, size=(N, K)).astype(np.uint8) & np.uint8(0xD7))).cuda()
+        bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).cuda()
+        scales = torch.from_numpy(rng.uniform(0.5, 2.0, size=N) * 0.01).cuda()
+
+        y = torch.empty((M, N), dtype=torch.uint8, device="cuda")
+
+        def run():
+            pkg.f8mm_launch(a, b, bias, right_transpose=True, out_scales=scales, out=y)
+
+        sec = _time_launches(torch, run, steps, warmup=3)
+        tf = 2.0 * M * N * K / sec / 1e12
+        out.append({"case": "f8e4m3_matmul_requant_M%d_N%d_K%d" % (M, N, K), "us": round(sec * 1e6, 2),
+                    "TFLOPs": round(tf, 1), "frac_fp8_peak": round(tf / 5000.0, 4)})
+    return out
+
+
 def bench_operator_boundary(pkg, S, steps=20):
     """The same q_proj GEMV through the reference's operator interface (float32-expanded host tensors in and out,
     like InferenceParameter): includes the host<->device copies and conversions, so it is NOT a roofline figure."""
@@ -417,6 +439,7 @@ def main():
         ex["single_matmuls"] = bench_single_matmuls(pkg, S, torch)
         ex["dynamic_quant"] = bench_dynamic_quant(pkg, S, torch)
         ex["int8_256x1024x1024"] = bench_int8(pkg, S, torch, clib, 1024, 40, 5, M=256)
+        ex["f8_matmul"] = bench_f8_matmul(pkg, torch, clib)
         ex["operator_boundary"] = bench_operator_boundary(pkg, S)
         ex["device_resident_block"] = bench_module_block(pkg, S, clib, cfgs)
         line["extras"] = ex

@@ -158,6 +158,33 @@ int mi_matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int rig
                         int64_t N, int q_group_size, int dq_type, int dtype, uint16_t *d_y, float *d_y_f32,
                         void *stream);
 
+/* ---- tpu.MatMul on F8E4M3 operands with the F8 output requantization ------------------------------------------- */
+/* The plain product of tpu::MatMulOp::inference (lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:598-604: f32 matmul,
+ * bias, relu / relu_limit) on operands that hold E4M3 values, followed by :608-629: output = F8E4M3(v, 1 / scale, true)
+ * with one scale (getOutScales() of size 1: the step is narrowed to float first, as F8E4M3(src, dst, num, float step,
+ * satu) of lib/Support/Float8.cpp:267-272 does) or one per output channel (the double 1.0 / scale).  batch 1.
+ * The products are formed on the fp8 matrix cores: exact products, fp32 sums that carry about 2^-13 relative error
+ * (the reference's f32 matmul leaves its summation order to the library as well), so a small fraction of outputs
+ * -- about one in a thousand -- lands on the neighbouring E4M3 code. */
+enum { MI_F8_OUT_CODES = 0 /* uint8 E4M3 codes */, MI_F8_OUT_F32 = 1 /* the E4M3 values as f32 */,
+       MI_F8_OUT_BF16 = 2, MI_F8_OUT_F16 = 3 /* the same values in a 16-bit type (exact) */ };
+typedef struct mi_f8mm_attr {
+  int64_t M, K, N;        /* parseParam(): batch == 1 */
+  int right_transpose;    /* right stored [N, K] */
+  int do_relu;
+  double relu_limit;
+  const double *out_scales; /* getOutScales() */
+  int n_out_scales;       /* 1 or N */
+} mi_f8mm_attr;
+/* inputs = {left [M,K], right, bias [N] | NULL}: f32 arrays holding E4M3 values (anything else: MI_UNSUPPORTED);
+ * outputs[0] [M,N] receives the requantized E4M3 values as f32. */
+int mi_f8mm_inference(const mi_f8mm_attr *attr, mi_infer_param *p);
+/* device level: E4M3 codes in HBM; d_out_scales: per-channel scales [N] (doubles, device) or NULL for out_scale;
+ * d_acc_f32 (may be NULL) receives the fp32 value before requantization. */
+int mi_f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, const float *d_bias, int64_t M,
+                   int64_t K, int64_t N, int do_relu, double relu_limit, double out_scale, const double *d_out_scales,
+                   int out_kind, void *d_out, float *d_acc_f32, void *stream);
+
 /* ---- weight producers (the compile-time side of tpu.A16MatMul), computed on the GPU, host arrays in and out ---- */
 typedef struct mi_a16_quant_desc {
   int64_t K, N;

@@ -899,6 +899,48 @@ void orc_igemm_i64(const int8_t *A, const int8_t *B, const int32_t *bias,
     }
 }
 
+/* tpu.MatMul with F8E4M3 operands: the plain f32 product of lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:598-604
+ * (bias and relu inside MatMul::run) followed by the F8 output requantization of :608-629.  One scale: the array form
+ * F8E4M3(src, dst, num, float step, true) (Float8.cpp:267-272) narrows 1 / scale to float before the scalar routine
+ * widens it again; per channel: the scalar form with the double 1.0 / scale (:622-627).  The output holds the E4M3
+ * values themselves.  The f32 product is summed in double here (the reference's order is its matmul library's). */
+int orc_matmul_f8(const float *left, const float *right, const float *bias, int64_t M, int64_t K, int64_t N,
+                  int right_transpose, int do_relu, double relu_limit, const double *scales, int n_scales,
+                  float *output, float *acc_out) {
+  if (!left || !right || !output || !scales || M <= 0 || K <= 0 || N <= 0 || (n_scales != 1 && n_scales != N))
+    return 1;
+  float *r_kn = (float *)malloc(sizeof(float) * (size_t)(K * N));
+  if (!r_kn)
+    return 1;
+  if (right_transpose)
+    orc_hw_transpose(r_kn, right, N, K);
+  else
+    memcpy(r_kn, right, sizeof(float) * (size_t)(K * N));
+  orc_sgemm_f64acc(left, r_kn, bias, output, M, K, N);
+  free(r_kn);
+  if (do_relu) /* post_relu, lib/Support/Dnnl/DnnlUtils.cpp:15-25 */
+    for (int64_t i = 0; i < M * N; i++) {
+      float v = output[i] > 0.0f ? output[i] : 0.0f;
+      if (relu_limit > 0.0 && v > (float)relu_limit)
+        v = (float)relu_limit;
+      output[i] = v;
+    }
+  if (acc_out)
+    memcpy(acc_out, output, sizeof(float) * (size_t)(M * N));
+  if (n_scales == 1) {
+    const float step_f = (float)(1 / scales[0]); /* :613-615 and the float parameter of the array form */
+    const double step = (double)step_f;
+    for (int64_t i = 0; i < M * N; i++)
+      output[i] = orc_f8e4m3_to_f32(orc_f32_to_f8e4m3((float)((double)output[i] / step), 1));
+  } else {
+    for (int64_t i = 0; i < M * N; i++) {
+      const double step = 1.0 / scales[i % N];
+      output[i] = orc_f8e4m3_to_f32(orc_f32_to_f8e4m3((float)((double)output[i] / step), 1));
+    }
+  }
+  return 0;
+}
+
 static int64_t arr_at(const int64_t *v, int n, int64_t i, int64_t dflt) {
   /* module::getI64Array(attr, num, default): a one-element attribute is
    * broadcast (lib/Support/Module.cpp:570-578) */

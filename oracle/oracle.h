@@ -34,6 +34,9 @@
  *                                independently decoded operands; half-spacing bound.  F8E4M3 group sums are
  *                                order-dependent in the reference: pinned to fp32 rounding of a group sum, not bit
  *                                for bit (tests/test_oracle_float_codes.py)
+ *   orc_matmul_f8                float64 product of torch-decoded operands; the requantization against torch's
+ *                                float8 cast of the same quotient; per-channel vs one-scale step (float-narrowed)
+ *                                on a case built to tell them apart (tests/test_oracle_float_codes.py)
  *   orc_a16_quantize_dq          closed-form scale, zp = 0, on-grid recovery, half-spacing bound
  *   orc_a16_quantize             on-grid weights are recovered exactly, |w - dequant(q)| <= scale/2 inside the
  *                                clamp range, closed-form scale/zp, nibble order via the A16MatMul dequantizer
@@ -183,6 +186,13 @@ typedef struct {
  * acc (may be NULL) receives the f32 accumulators before requantisation. */
 int orc_matmul_int8(const orc_i8mm_attr *attr, const float *const *inputs,
                     float *output, float *acc);
+
+/* tpu.MatMul on F8E4M3 operands with the F8 output requantization (MatMul.cpp:598-629): left [M, K], right [K, N]
+ * or [N, K], both holding E4M3 values as f32; output = E4M3 values of relu(left x right + bias) / (1 / scale), one scale
+ * or one per output channel.  acc_out (may be NULL) receives the f32 value before requantization.  Returns 0 / 1. */
+int orc_matmul_f8(const float *left, const float *right, const float *bias, int64_t M, int64_t K, int64_t N,
+                  int right_transpose, int do_relu, double relu_limit, const double *scales, int n_scales,
+                  float *output, float *acc_out);
 
 /* exact-integer GEMM used to cross-check the f32 accumulation domain */
 void orc_igemm_i64(const int8_t *A, const int8_t *B, const int32_t *bias,

@@ -358,6 +358,26 @@ def cast(x, *, in_type, out_type, in_quant=False, out_quant=False, scale=1.0, ze
 PACK_GPTQ, PACK_AWQ = 0, 1
 
 
+def matmul_f8(left, right, bias=None, *, right_transpose=False, do_relu=False, relu_limit=-1.0, scales=(1.0,)):
+    """tpu.MatMul on E4M3-valued operands with F8 output requantization; returns (E4M3 values, f32 before requant)."""
+    left, right = _f32(left), _f32(right)
+    M, K = left.shape
+    N = right.shape[0] if right_transpose else right.shape[1]
+    sc = np.ascontiguousarray(scales, dtype=np.float64).reshape(-1)
+    out = np.empty((M, N), dtype=np.float32)
+    acc = np.empty((M, N), dtype=np.float32)
+    b = _f32(bias)
+    L = lib()
+    L.orc_matmul_f8.restype = C.c_int
+    rc = L.orc_matmul_f8(_p(left, C.c_float), _p(right, C.c_float), None if b is None else _p(b, C.c_float),
+                         C.c_int64(M), C.c_int64(K), C.c_int64(N), C.c_int(int(right_transpose)), C.c_int(int(do_relu)),
+                         C.c_double(relu_limit), _p(sc, C.c_double), C.c_int(sc.size), _p(out, C.c_float),
+                         _p(acc, C.c_float))
+    if rc != 0:
+        raise RuntimeError("orc_matmul_f8: bad arguments")
+    return out, acc
+
+
 def a16_quantize(w_kn, *, bits, g, symmetric=False, f16=False, dq_type=DQ_INT):
     """A16MatMulAdjust on the f32 weight [K, N] of a top-level matmul.
 

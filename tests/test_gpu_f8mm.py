@@ -1,0 +1,182 @@
+"""GPU parity of tpu.MatMul on F8E4M3 operands with the F8 output requantization (MatMul.cpp:598-629) against the CPU
+oracle, through the C ABI.
+
+The products are exact on the fp8 matrix cores; their fp32 sums are not the reference's (whose order is its matmul
+library's) and carry the alignment error of the fp8 pipeline.  Bars, written out in the tests: the fp32 value before
+requantization within 2^-11 of the sum of absolute terms; the E4M3 output equal to the oracle's on at least 99 % of the
+elements and never more than one code away (next to zero, where codes are denser than that agreement: within it).  Where every partial sum is exact (small integers) everything must match
+bit for bit, and so must the requantization of the kernel's own fp32 value everywhere.
+"""
+import numpy as np
+import pytest
+
+from helpers import pkg
+
+pytestmark = pytest.mark.gpu
+
+M_ = pkg()
+S = pkg("synth")
+clib = pkg("clib")
+
+
+def _codes(rng, shape, top=0x7e):
+    c = rng.integers(0, 256, size=shape).astype(np.uint8)
+    mag = c & 0x7f
+    mag = np.minimum(mag, top).astype(np.uint8)
+    return ((c & 0x80) | mag).astype(np.uint8)
+
+
+def _run(a_codes, b_codes, bias, rt, relu, limit, scale, scales, out_kind=None):
+    import torch
+    out_kind = clib.F8_OUT_CODES if out_kind is None else out_kind
+    M, N = a_codes.shape[0], (b_codes.shape[0] if rt else b_codes.shape[1])
+    acc = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.f8mm_launch(torch.from_numpy(a_codes).cuda(), torch.from_numpy(b_codes).cuda(),
+                       None if bias is None else torch.from_numpy(bias).cuda(), right_transpose=rt, do_relu=relu,
+                       relu_limit=limit, out_scale=scale,
+                       out_scales=None if scales is None else torch.from_numpy(scales).cuda(), out_kind=out_kind,
+                       acc_f32=acc)
+    torch.cuda.synchronize()
+    return y.cpu(), acc.cpu().numpy()
+
+
+def _code_distance(a, b):
+    def key(c):
+        c = c.astype(np.int32)
+        return np.where(c & 0x80, -(c & 0x7f), c & 0x7f)
+    return np.abs(key(a) - key(b))
+
+
+CASES = [  # (M, K, N, right_transpose, relu, per_channel, bias)
+    (1, 64, 16, True, False, False, False), (5, 512, 100, False, False, False, True),
+    (130, 1024, 200, True, True, False, True), (64, 200, 48, False, False, True, False),   # K % 64 != 0
+    (256, 4096, 256, True, False, True, True), (33, 72, 130, True, True, True, True),      # K % 16 != 0
+]
+
+
+@pytest.mark.parametrize("M,K,N,rt,relu,per_channel,bias", CASES)
+def test_f8_matmul_device_level(orc, M, K, N, rt, relu, per_channel, bias):
+    rng = np.random.default_rng(M + K + N)
+    a = _codes(rng, (M, K), top=0x58)                       # magnitudes up to 16: sums stay far from fp32 overflow
+    b = _codes(rng, (N, K) if rt else (K, N), top=0x58)
+    bv = (rng.standard_normal(N) * 50).astype(np.float32) if bias else None
+    af, bf = orc.f8e4m3_to_f32(a), orc.f8e4m3_to_f32(b)
+    b_kn = bf.T if rt else bf
+    mag = np.abs(af.astype(np.float64)) @ np.abs(b_kn.astype(np.float64))
+    rms = float(np.sqrt(np.mean((af.astype(np.float64) @ b_kn) ** 2))) + 1e-9
+    scales = (rng.uniform(0.5, 2.0, size=N) * 100.0 / rms) if per_channel else None
+    scale = 100.0 / rms
+    limit = 2.0 * rms if relu else -1.0
+    y, acc = _run(a, b, bv, rt, relu, limit, scale, scales)
+    want, want_acc = orc.matmul_f8(af, bf, bv, right_transpose=rt, do_relu=relu, relu_limit=limit,
+                                   scales=scales if per_channel else [scale])
+    assert np.all(np.abs(acc.astype(np.float64) - want_acc) <= mag * 2.0 ** -11 + 1e-6)
+    got = y.numpy()
+    want_codes = orc.f32_to_f8e4m3(want)
+    dist = _code_distance(got, want_codes)
+    # one code at most -- except next to zero, where the codes lie closer together than the fp32 agreement itself
+    step = (1.0 / scales[None, :]) if per_channel else np.float64(np.float32(1.0 / scale))
+    near_zero = np.abs(orc.f8e4m3_to_f32(got).astype(np.float64) - want) <= (mag * 2.0 ** -11 + 1e-6) / step
+    assert np.all((dist <= 1) | near_zero)
+    assert (dist == 0).mean() >= 0.99
+    # the requantization itself is exact arithmetic: apply the oracle's to the kernel's own fp32 value
+    if per_channel:
+        q = (acc.astype(np.float64) / (1.0 / scales[None, :])).astype(np.float32)
+    else:
+        q = (acc.astype(np.float64) / np.float64(np.float32(1.0 / scale))).astype(np.float32)
+    assert np.array_equal(got, orc.f32_to_f8e4m3(q))
+
+
+def test_f8_matmul_exact_domain_and_output_kinds(orc):
+    """Integer-valued operands up to 15: every partial sum is an integer below 2^24, so the fp32 value and every output
+    form (codes, f32, bf16, f16) must equal the oracle's bit for bit."""
+    import torch
+    rng = np.random.default_rng(4)
+    M, K, N = 70, 384, 90
+    af = rng.integers(-15, 16, size=(M, K)).astype(np.float32)
+    bf = rng.integers(-15, 16, size=(K, N)).astype(np.float32)
+    bias = rng.integers(-100, 101, size=N).astype(np.float32)
+    a, b = orc.f32_to_f8e4m3(af), orc.f32_to_f8e4m3(bf)
+    scale = 0.02
+    want, want_acc = orc.matmul_f8(af, bf, bias, scales=[scale])
+    y, acc = _run(a, b, bias, False, False, -1.0, scale, None)
+    assert np.array_equal(acc.view(np.uint32), want_acc.view(np.uint32))
+    assert np.array_equal(y.numpy(), orc.f32_to_f8e4m3(want))
+    y32, _ = _run(a, b, bias, False, False, -1.0, scale, None, out_kind=clib.F8_OUT_F32)
+    assert np.array_equal(y32.numpy(), want)
+    yb, _ = _run(a, b, bias, False, False, -1.0, scale, None, out_kind=clib.F8_OUT_BF16)
+    assert np.array_equal(yb.float().numpy(), want)
+    yh, _ = _run(a, b, bias, False, False, -1.0, scale, None, out_kind=clib.F8_OUT_F16)
+    assert np.array_equal(yh.float().numpy(), want)
+    assert np.unique(y.numpy()).size > 30
+
+
+def test_f8_matmul_saturation_ties_and_step_narrowing(orc):
+    """A zero product plus a bias reads the requantization back on its own: values on and next to every E4M3 rounding
+    boundary, far beyond 448 (saturation), and the one-scale / per-channel difference in the step."""
+    codes = np.arange(0, 0x7e, dtype=np.uint8)              # subnormal codes included
+    mid = (orc.f8e4m3_to_f32(codes).astype(np.float64) + orc.f8e4m3_to_f32(codes + 1)) / 2
+    scale = 3.0
+    cand = np.concatenate([np.float32(mid / scale), np.float32(mid * np.float64(np.float32(1.0 / scale)))])
+    cand = np.concatenate([cand, np.nextafter(cand, np.float32(0)), np.nextafter(cand, np.float32(1e9)),
+                           np.array([1e4, 3e38, 149.3, 154.6, 154.7, 1e-6, 0.0], np.float32)])
+    cand = np.concatenate([cand, -cand]).astype(np.float32)
+    N = cand.size
+    for K in (64, 48):                                      # the ring kernel and the register-staged one
+        a = np.zeros((3, K), np.uint8)
+        b = np.zeros((K, N), np.uint8)
+        af, bf = orc.f8e4m3_to_f32(a), orc.f8e4m3_to_f32(b)
+        for scales in (None, np.full(N, scale)):
+            y, acc = _run(a, b, cand, False, False, -1.0, scale, scales)
+            want, _ = orc.matmul_f8(af, bf, cand, scales=[scale] if scales is None else scales)
+            assert np.array_equal(acc, np.tile(cand, (3, 1)))
+            assert np.array_equal(y.numpy(), orc.f32_to_f8e4m3(want))
+    one, _ = orc.matmul_f8(af, bf, cand, scales=[scale])
+    per, _ = orc.matmul_f8(af, bf, cand, scales=np.full(N, scale))
+    assert np.any(one != per)                               # the case really tells the two step rules apart
+
+
+def test_f8_matmul_operator_level_and_rejections(orc):
+    rng = np.random.default_rng(8)
+    M, K, N = 6, 128, 40
+    af = rng.integers(-15, 16, size=(M, K)).astype(np.float32)
+    bf = rng.integers(-15, 16, size=(N, K)).astype(np.float32) * 0.25
+    bias = rng.integers(-100, 101, size=N).astype(np.float32)
+    scales = rng.uniform(0.01, 0.05, size=N)
+    y = M_.matmul_f8(af, bf, bias, right_transpose=True, do_relu=True, relu_limit=200.0, out_scales=scales)
+    want, _ = orc.matmul_f8(af, bf, bias, right_transpose=True, do_relu=True, relu_limit=200.0, scales=scales)
+    assert np.array_equal(y, want)
+    y = M_.matmul_f8(af, np.ascontiguousarray(bf.T), None, out_scales=[0.02])
+    want, _ = orc.matmul_f8(af, np.ascontiguousarray(bf.T), None, scales=[0.02])
+    assert np.array_equal(y, want)
+    bad = af.copy()
+    bad[0, 0] = 0.3                                          # not an E4M3 value
+    with pytest.raises(clib.BackendError) as e:
+        M_.matmul_f8(bad, bf, None, right_transpose=True, out_scales=[1.0])
+    assert e.value.code == clib.MI_UNSUPPORTED
+    with pytest.raises(clib.BackendError) as e:
+        M_.matmul_f8(af, bf, None, right_transpose=True, out_scales=[1.0, 2.0])
+    assert e.value.code == clib.MI_BAD_ARGUMENT
+    with pytest.raises(clib.BackendError) as e:
+        M_.matmul_f8(af, bf, None, right_transpose=True, out_scales=[0.0])
+    assert e.value.code == clib.MI_BAD_ARGUMENT
+
+
+def test_f8_matmul_full_size_linearity():
+    """4096^3 is beyond the oracle's reach in test time: doubling every left code's exponent (x 2, exact in E4M3) must
+    double the fp32 result exactly, and zeroing the right operand must give the bias."""
+    import torch
+    rng = np.random.default_rng(0)
+    M = N = K = 4096
+    a = _codes(rng, (M, K), top=0x4f)
+    b = _codes(rng, (N, K), top=0x4f)
+    a2 = (a + np.uint8(8)).astype(np.uint8)                  # exponent + 1 (zero and subnormal codes excluded below)
+    keep = (a & 0x78) != 0
+    a = np.where(keep, a, 0x38).astype(np.uint8)
+    a2 = np.where(keep, a2, 0x40).astype(np.uint8)
+    _, acc1 = _run(a, b, None, True, False, -1.0, 1e-4, None)
+    _, acc2 = _run(a2, b, None, True, False, -1.0, 1e-4, None)
+    assert np.array_equal(acc2, acc1 * np.float32(2.0))
+    bias = rng.standard_normal(N).astype(np.float32)
+    _, acc0 = _run(a, np.zeros_like(b), bias, True, False, -1.0, 1.0, None)
+    assert np.array_equal(acc0, np.tile(bias, (M, 1)))

@@ -288,3 +288,67 @@ def test_two_operand_matmul_on_grid(orc, dq, fmax):
             exact = left.astype(np.float64) @ right_nk.T.astype(np.float64)
             bound = np.abs(left.astype(np.float64)) @ np.abs(right_nk.T.astype(np.float64)) * 2.0 ** -21
             assert np.all(np.abs(pre - exact) <= bound)
+
+
+def _f8_grid():
+    return _torch_decode(np.array([c for c in range(256) if (c & 0x7f) != 0x7f], dtype=np.uint8))
+
+
+@pytest.mark.parametrize("rt,relu,per_channel", [(False, False, False), (True, True, False), (False, True, True),
+                                                 (True, False, True)])
+def test_f8_matmul_product_and_requantization(orc, rt, relu, per_channel):
+    """orc_matmul_f8: the fp32 value before requantization against a float64 product (both operand layouts, bias,
+    relu with a limit), and the requantization stage against torch's float8 cast of the same quotient."""
+    rng = np.random.default_rng(rt * 4 + relu * 2 + per_channel)
+    M, K, N = 9, 160, 24
+    grid = _f8_grid()
+    grid = grid[np.abs(grid) <= 8]
+    a = rng.choice(grid, size=(M, K)).astype(np.float32)
+    b_kn = rng.choice(grid, size=(K, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32) * 10
+    scales = rng.uniform(0.05, 0.3, size=N) if per_channel else np.array([0.11])
+    limit = 60.0 if relu else -1.0
+    out, acc = orc.matmul_f8(a, np.ascontiguousarray(b_kn.T) if rt else b_kn, bias, right_transpose=rt, do_relu=relu,
+                             relu_limit=limit, scales=scales)
+    want = a.astype(np.float64) @ b_kn.astype(np.float64) + bias
+    if relu:
+        want = np.clip(want, 0.0, limit)
+    assert np.all(np.abs(acc - want) <= np.abs(want) * 2.0 ** -22 + 1e-30)
+    if relu:
+        assert acc.min() == 0.0 and acc.max() == limit
+    if per_channel:
+        step = 1.0 / scales[None, :]
+    else:
+        step = np.float64(np.float32(1.0 / scales[0]))
+    q = (acc.astype(np.float64) / step).astype(np.float32)
+    q = np.clip(q, -448.0, 448.0)                                  # saturating
+    assert np.array_equal(out, torch.from_numpy(q).to(torch.float8_e4m3fn).float().numpy())
+    assert np.unique(out).size > 20                                # a real spread of codes, not all saturated
+
+
+def test_f8_matmul_one_scale_step_is_narrowed_to_float(orc):
+    """With one scale the reference passes 1 / scale through a float parameter; per channel it keeps the double.  With
+    a zero product the value is the bias, which the test places next to E4M3 rounding boundaries until the two
+    quotients fall on different sides."""
+    codes = np.arange(8, 0x7e, dtype=np.uint8)
+    mid = (orc.f8e4m3_to_f32(codes).astype(np.float64) + orc.f8e4m3_to_f32(codes + 1)) / 2
+    found = 0
+    for scale in (3.0, 7.0, 0.3, 1.7, 11.0):
+        step_d = 1.0 / scale
+        step_f = np.float64(np.float32(1.0 / scale))
+        cand = np.concatenate([np.float32(mid * step_d), np.float32(mid * step_f)])
+        cand = np.concatenate([cand, np.nextafter(cand, np.float32(0)), np.nextafter(cand, np.float32(1e9))])
+        qd = (cand.astype(np.float64) / step_d).astype(np.float32)
+        qf = (cand.astype(np.float64) / step_f).astype(np.float32)
+        cd, cf = orc.f32_to_f8e4m3(qd), orc.f32_to_f8e4m3(qf)
+        for v, d, f in zip(cand[cd != cf][:4], cd[cd != cf][:4], cf[cd != cf][:4]):
+            found += 1
+            a = np.zeros((1, 1), np.float32)
+            b = np.ones((1, 2), np.float32)                        # N = 2 so that two scales mean "per channel"
+            bias = np.array([v, v], np.float32)
+            one, _ = orc.matmul_f8(a, b, bias, scales=[scale])
+            per, _ = orc.matmul_f8(a, b, bias, scales=[scale, scale])
+            assert one[0, 0] == orc.f8e4m3_to_f32(np.array([f], np.uint8))[0]
+            assert per[0, 0] == orc.f8e4m3_to_f32(np.array([d], np.uint8))[0]
+            assert one[0, 0] != per[0, 0]
+    assert found > 0

@@ -19,7 +19,7 @@ EXPORTS = [
     "mi_a16mm_init", "mi_a16mm_inference", "mi_a16mm_deinit",
     "mi_a16_weight_create", "mi_a16_weight_destroy", "mi_a16_weight_bytes", "mi_a16mm_launch",
     "mi_a16mm_launch_group", "mi_a16mm_dq_launch", "mi_a16mm_dq_type_launch", "mi_matmul_dq_launch",
-    "mi_matmul_dq_inference",
+    "mi_matmul_dq_inference", "mi_f8mm_inference", "mi_f8mm_launch",
     "mi_a16_weight_export_size", "mi_a16_weight_export", "mi_a16_weight_import", "mi_a16_quantize", "mi_llm_unpack",
     "mi_a16_to_group",
     "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
@@ -60,6 +60,15 @@ class A16WeightDesc(C.Structure):
 class MatMulDqAttr(C.Structure):
     _fields_ = [("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64), ("right_transpose", C.c_int),
                 ("q_group_size", C.c_int), ("dq_type", C.c_int), ("out_dtype", C.c_int)]
+
+
+class F8MMAttr(C.Structure):
+    _fields_ = [("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64), ("right_transpose", C.c_int),
+                ("do_relu", C.c_int), ("relu_limit", C.c_double), ("out_scales", C.POINTER(C.c_double)),
+                ("n_out_scales", C.c_int)]
+
+
+F8_OUT_CODES, F8_OUT_F32, F8_OUT_BF16, F8_OUT_F16 = 0, 1, 2, 3
 
 
 class A16QuantDesc(C.Structure):
@@ -142,6 +151,8 @@ def lib():
         L.mi_a16_weight_import.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_size_t]
         L.mi_a16_quantize.argtypes = [C.POINTER(A16QuantDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        L.mi_f8mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int,
+                                     C.c_double, C.c_double, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16_to_group.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
         L.mi_llm_unpack.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
                                     C.c_void_p, C.c_void_p]

@@ -979,6 +979,92 @@ int mi_cast_inference(const mi_cast_attr *a, mi_infer_param *p) {
   return MI_SUCCESS;
 }
 
+// ---- tpu.MatMul on F8E4M3 operands with F8 output requantization (MatMul.cpp:598-629) --------------------------
+int mi_f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, const float *d_bias, int64_t M,
+                   int64_t K, int64_t N, int do_relu, double relu_limit, double out_scale, const double *d_out_scales,
+                   int out_kind, void *d_out, float *d_acc_f32, void *stream) {
+  return f8mm_launch(d_a, d_b, right_transpose, d_bias, M, K, N, do_relu, relu_limit, out_scale, d_out_scales, out_kind,
+                     d_out, d_acc_f32, (hipStream_t)stream);
+}
+
+// f32 -> the E4M3 code of exactly that value, or -1 (host side of the operator entry: the interpreter hands over
+// f32 arrays that hold E4M3 values)
+static int f8_code_of(float v) {
+  uint32_t b;
+  memcpy(&b, &v, 4);
+  const uint32_t sign = (b >> 24) & 0x80u, a = b & 0x7fffffffu;
+  if (a == 0)
+    return (int)sign;
+  const int e = (int)(a >> 23) - 127;  // unbiased
+  const uint32_t frac = a & 0x7fffffu;
+  if (e >= -6 && e <= 8) {             // E4M3 normals: 3 fraction bits
+    if (frac & 0xfffffu)
+      return -1;
+    const uint32_t code = ((uint32_t)(e + 7) << 3) | (frac >> 20);
+    return code >= 0x7f ? -1 : (int)(code | sign);
+  }
+  if (e >= -9 && e < -6) {             // subnormals: multiples of 2^-9 below 2^-6
+    const uint32_t mant = (frac | 0x800000u);  // 1.f at bit 23, value = mant * 2^(e - 23)
+    const int shift = 23 - (e + 9);            // units of 2^-9
+    if (mant & ((1u << shift) - 1))
+      return -1;
+    return (int)((mant >> shift) | sign);
+  }
+  return -1;
+}
+
+int mi_f8mm_inference(const mi_f8mm_attr *a, mi_infer_param *p) {
+  MI_REQUIRE(a && p && p->inputs && p->n_inputs >= 2 && p->inputs[0] && p->inputs[1] && p->outputs &&
+                 p->n_outputs >= 1 && p->outputs[0],
+             MI_BAD_ARGUMENT, "mi_f8mm_inference: null argument");
+  MI_REQUIRE(a->M >= 0 && a->K > 0 && a->N > 0, MI_BAD_ARGUMENT, "mi_f8mm_inference: bad shape");
+  MI_REQUIRE(a->out_scales && (a->n_out_scales == 1 || a->n_out_scales == a->N), MI_BAD_ARGUMENT,
+             "mi_f8mm_inference: out_scales must hold one scale or one per output channel");
+  for (int i = 0; i < a->n_out_scales; ++i)
+    MI_REQUIRE(a->out_scales[i] == a->out_scales[i] && a->out_scales[i] != 0.0, MI_BAD_ARGUMENT,
+               "mi_f8mm_inference: output scales must be nonzero numbers");
+  if (a->M == 0)
+    return MI_SUCCESS;
+  MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_f8mm_inference: no GPU visible");
+  const size_t nl = (size_t)a->M * a->K, nr = (size_t)a->K * a->N, no = (size_t)a->M * a->N;
+  std::vector<uint8_t> hl(nl), hr(nr);
+  for (size_t i = 0; i < nl; ++i) {
+    const int c = f8_code_of(p->inputs[0][i]);
+    MI_REQUIRE(c >= 0, MI_UNSUPPORTED, "mi_f8mm_inference: left operand holds a value that is not an E4M3 number");
+    hl[i] = (uint8_t)c;
+  }
+  for (size_t i = 0; i < nr; ++i) {
+    const int c = f8_code_of(p->inputs[1][i]);
+    MI_REQUIRE(c >= 0, MI_UNSUPPORTED, "mi_f8mm_inference: right operand holds a value that is not an E4M3 number");
+    hr[i] = (uint8_t)c;
+  }
+  const float *bias = p->n_inputs > 2 ? p->inputs[2] : nullptr;
+  DevBuf dl, dr, db, ds, dy;
+  int rc;
+  if ((rc = dl.reserve(nl)) || (rc = dr.reserve(nr)) || (rc = dy.reserve(no * 4)))
+    return rc;
+  MI_HIP(hipMemcpy(dl.ptr, hl.data(), nl, hipMemcpyHostToDevice));
+  MI_HIP(hipMemcpy(dr.ptr, hr.data(), nr, hipMemcpyHostToDevice));
+  if (bias) {
+    if ((rc = db.reserve((size_t)a->N * 4)))
+      return rc;
+    MI_HIP(hipMemcpy(db.ptr, bias, (size_t)a->N * 4, hipMemcpyHostToDevice));
+  }
+  if (a->n_out_scales != 1) {
+    if ((rc = ds.reserve((size_t)a->N * 8)))
+      return rc;
+    MI_HIP(hipMemcpy(ds.ptr, a->out_scales, (size_t)a->N * 8, hipMemcpyHostToDevice));
+  }
+  rc = f8mm_launch((const uint8_t *)dl.ptr, (const uint8_t *)dr.ptr, a->right_transpose, bias ? (const float *)db.ptr : nullptr,
+                   a->M, a->K, a->N, a->do_relu, a->relu_limit, a->out_scales[0],
+                   a->n_out_scales != 1 ? (const double *)ds.ptr : nullptr, MI_F8_OUT_F32, dy.ptr, nullptr, nullptr);
+  if (rc)
+    return rc;
+  MI_HIP(hipDeviceSynchronize());
+  MI_HIP(hipMemcpy(p->outputs[0], dy.ptr, no * 4, hipMemcpyDeviceToHost));
+  return MI_SUCCESS;
+}
+
 // ---- tpu.MatMul, both operands quantized dynamically (MatMul.cpp:447-597) -------------------------------------
 int mi_matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
                         int64_t N, int q_group_size, int dq_type, int dtype, uint16_t *d_y, float *d_y_f32,

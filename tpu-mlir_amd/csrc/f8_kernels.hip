@@ -1,0 +1,468 @@
+// tpu.MatMul on F8E4M3 operands with the F8 output requantization, for gfx950:
+//   acc[m,n] = sum_k A[m,k] * B[n,k] + bias[n]          (E4M3 codes in, fp32 out of v_mfma_f32_32x32x64_f8f6f4)
+//   v        = relu / clip
+//   out      = E4M3( v / step ),  step = 1 / scale (one scale: narrowed to fp32 first, as the reference's array routine
+//              does; per channel: the double)                lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:598-629
+//
+// 128 x 128 outputs per workgroup, 4 waves (2 x 2), each wave 64 x 64 as 2 x 2 blocks of 32 x 32.  K advances 64 bytes per
+// stage; one matrix instruction consumes a whole stage of a block (64 k: lane l holds two 16-byte pieces of row l % 32
+// for both operands -- the contraction order inside an instruction is free as long as both sides agree).
+//   f8_gemm_ring_kernel   K % 64 == 0: a ring of LDS stages filled by direct-to-LDS loads (no staging registers, several
+//                         stages of requests in flight), 16-byte chunks XOR-swizzled against bank conflicts, workgroups
+//                         renumbered so that each XCD's L2 sees a compact block of tiles.
+//   f8_gemm_kernel        any K: operands staged through registers into two padded LDS stages.
+//
+// The fp8 matrix pipeline aligns the products of one instruction to the largest and drops low bits, so a long sum
+// carries a relative error of about 2^-13 where an fp32 FMA chain has 2^-24; after the E4M3 rounding (2^-4 steps) that
+// moves a result across a rounding boundary about once in a thousand outputs.  The reference's own fp32 matmul fixes
+// no summation order either; tests bound the fp32 value and count the differing codes.
+#include "device_math.cuh"
+#include "internal.h"
+
+namespace mi {
+
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int F8_BM = 128, F8_BN = 128, F8_BK = 64;
+constexpr int F8_LDS_ROW = 80;
+
+struct F8Args {
+  const uint8_t *A;     // [M, K] E4M3 codes
+  const uint8_t *B;     // [N, K] E4M3 codes
+  const float *bias;    // [N] or null
+  void *out;
+  float *acc_out;       // fp32 value before requantization, or null
+  int64_t M, K, N;
+  int do_relu;
+  float relu_limit;
+  int out_kind;         // MI_F8_OUT_*
+  double step;          // one scale: (double)(float)(1 / scale)
+  const double *scales; // per channel [N], or null
+};
+
+__device__ __forceinline__ u32x4 f8_load_chunk(const uint8_t *base, int64_t row, int64_t rows, int64_t k, int64_t K,
+                                               bool vec_ok) {
+  u32x4 v = {0, 0, 0, 0};  // code 0 = +0: rows and columns past the matrix add nothing
+  if (row < rows && k < K) {
+    const uint8_t *p = base + row * K + k;
+    if (vec_ok && k + 16 <= K) {
+      v = *(const u32x4 *)p;
+    } else {
+      uint8_t tmp[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        tmp[i] = (k + i < K) ? p[i] : (uint8_t)0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        v[i] = (uint32_t)tmp[4 * i] | ((uint32_t)tmp[4 * i + 1] << 8) | ((uint32_t)tmp[4 * i + 2] << 16) |
+               ((uint32_t)tmp[4 * i + 3] << 24);
+    }
+  }
+  return v;
+}
+
+__device__ __forceinline__ void f8_epilogue(const F8Args &a, const f32x16 (&acc)[2][2], int64_t m0, int64_t n0, int lane);
+
+__global__ __launch_bounds__(256) void f8_gemm_kernel(F8Args a) {
+  __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][F8_BM * F8_LDS_ROW];
+  __shared__ __attribute__((aligned(16))) uint8_t lds_b[2][F8_BN * F8_LDS_ROW];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t m_base = (int64_t)blockIdx.y * F8_BM, n_base = (int64_t)blockIdx.x * F8_BN;
+  const bool vec_ok = (a.K % 16) == 0;
+
+  // staging: 128 rows x 4 chunks of 16 B per operand tile = 512 chunks, two per thread
+  const int c_row0 = tid >> 2, c_col = tid & 3;  // rows c_row0 and c_row0 + 64
+  u32x4 ra[2], rb[2];
+  auto gload = [&](int64_t k0) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      ra[h] = f8_load_chunk(a.A, m_base + c_row0 + 64 * h, a.M, k0 + 16 * c_col, a.K, vec_ok);
+      rb[h] = f8_load_chunk(a.B, n_base + c_row0 + 64 * h, a.N, k0 + 16 * c_col, a.K, vec_ok);
+    }
+  };
+  auto lstore = [&](int stage) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      *(u32x4 *)&lds_a[stage][(c_row0 + 64 * h) * F8_LDS_ROW + 16 * c_col] = ra[h];
+      *(u32x4 *)&lds_b[stage][(c_row0 + 64 * h) * F8_LDS_ROW + 16 * c_col] = rb[h];
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[i][j][r] = 0.0f;
+
+  const int64_t k_iters = (a.K + F8_BK - 1) / F8_BK;
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  const int frow = lane & 31, fk = (lane >> 5) * 32;
+  for (int64_t it = 0; it < k_iters; ++it) {
+    const int stage = (int)(it & 1);
+    if (it + 1 < k_iters)
+      gload((it + 1) * F8_BK);
+    i32x8 fa[2], fb[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint8_t *pa = &lds_a[stage][(wm * 64 + i * 32 + frow) * F8_LDS_ROW + fk];
+      const uint8_t *pb = &lds_b[stage][(wn * 64 + i * 32 + frow) * F8_LDS_ROW + fk];
+      const u32x4 a0 = *(const u32x4 *)pa, a1 = *(const u32x4 *)(pa + 16);
+      const u32x4 b0 = *(const u32x4 *)pb, b1 = *(const u32x4 *)(pb + 16);
+      fa[i] = i32x8{(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
+      fb[i] = i32x8{(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)  // formats 0 / 0 = E4M3 x E4M3, no block scales
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+    if (it + 1 < k_iters) {
+      lstore(stage ^ 1);
+      __syncthreads();
+    }
+  }
+
+  f8_epilogue(a, acc, m_base + wm * 64, n_base + wn * 64, lane);
+}
+
+// epilogue of a wave's 64 x 64 block: register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of its
+// 32 x 32 block (i, j)
+__device__ __forceinline__ void f8_epilogue(const F8Args &a, const f32x16 (&acc)[2][2], int64_t m0, int64_t n0, int lane) {
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int64_t n = n0 + j * 32 + (lane & 31);
+    const bool n_ok = n < a.N;
+    const float bias_n = (a.bias && n_ok) ? a.bias[n] : 0.0f;
+    const double step = (a.scales && n_ok) ? 1.0 / a.scales[n] : a.step;
+    const double inv_step = 1.0 / step;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t m = m0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (n_ok && m < a.M) {
+          float v = acc[i][j][r] + bias_n;
+          if (a.do_relu) {  // post_relu, lib/Support/Dnnl/DnnlUtils.cpp:15-25
+            v = v > 0.0f ? v : 0.0f;
+            if (a.relu_limit > 0.0f && v > a.relu_limit)
+              v = a.relu_limit;
+          }
+          const int64_t o = m * a.N + n;
+          if (a.acc_out)
+            a.acc_out[o] = v;
+          // F8E4M3(v, step, true): the quotient in double, narrowed to fp32, rounded to E4M3 (Float8.cpp:259-261).
+          // v * (1 / step) is within two double ulps of that quotient, so the narrowing can come out differently
+          // only when the 29 bits it drops sit next to the halfway pattern; only then is the division carried out.
+          double qd = (double)v * inv_step;
+          const int32_t low = (int32_t)((uint32_t)__double_as_longlong(qd) & 0x1fffffffu);
+          if (low >= 0x10000000 - 4 && low <= 0x10000000 + 4)
+            qd = (double)v / step;
+          const uint32_t code = f8e4m3_from_f32((float)qd);
+          if (a.out_kind == MI_F8_OUT_CODES)
+            ((uint8_t *)a.out)[o] = (uint8_t)code;
+          else if (a.out_kind == MI_F8_OUT_F32)
+            ((float *)a.out)[o] = f8e4m3_to_f32(code);
+          else if (a.out_kind == MI_F8_OUT_BF16)  // exact: E4M3 values fit both 16-bit types
+            ((uint16_t *)a.out)[o] = (uint16_t)(__float_as_uint(f8e4m3_to_f32(code)) >> 16);
+          else
+            ((uint16_t *)a.out)[o] = __builtin_bit_cast(uint16_t, (_Float16)f8e4m3_to_f32(code));
+        }
+      }
+    }
+  }
+}
+
+// E4M3 code of q, round half to even, saturating, NaN -> 0x7f | sign: the hardware conversion on a value clamped to
+// +-448 (it rounds to nearest even, subnormals included), which equals f8e4m3_from_f32 on every input
+__device__ __forceinline__ uint32_t f8_pair_codes(float q0, float q1) {
+  const float c0 = __builtin_fminf(__builtin_fmaxf(q0, -448.0f), 448.0f);  // NaN -> a number; patched below
+  const float c1 = __builtin_fminf(__builtin_fmaxf(q1, -448.0f), 448.0f);
+  uint32_t r = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c0, c1, 0, false) & 0xffffu;
+  if (q0 != q0)
+    r = (r & 0xff00u) | 0x7fu | ((__float_as_uint(q0) >> 24) & 0x80u);
+  if (q1 != q1)
+    r = (r & 0x00ffu) | ((0x7fu | ((__float_as_uint(q1) >> 24) & 0x80u)) << 8);
+  return r;
+}
+
+constexpr int F8_STRIDE = 68;  // dwords per row of an epilogue strip (64 + 4: 16-byte aligned rows, staggered banks)
+
+// Epilogue of a wave's 64 x 64 block through its own strip of LDS: the accumulators (register r of lane l = row
+// 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of block (i, j)) are laid out row-major so that a lane owns 16
+// consecutive columns of a row -- per-column parameters are fetched once per lane, results leave as 16-byte stores.
+__device__ __forceinline__ void f8_strip_epilogue(const F8Args &a, const f32x16 (&acc)[2][2], float *strip, int64_t m0,
+                                                  int64_t nb, int lane) {
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        strip[(i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * F8_STRIDE + j * 32 + (lane & 31)] = acc[i][j][r];
+  // a wave only reads what it wrote: no barrier, the LDS counter orders it
+  const int cc = lane & 3, rsub = lane >> 2;  // 16-column chunk, row within a group of 16 rows
+  const int64_t n0 = nb + cc * 16;
+  const bool vec_ok = (a.N % 16) == 0 && n0 + 16 <= a.N;
+  float bias[16];
+  double inv[16];  // 1 / step per column
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int64_t n = (n0 + e) < a.N ? (n0 + e) : (a.N - 1);
+    bias[e] = a.bias ? a.bias[n] : 0.0f;
+    inv[e] = 1.0 / (a.scales ? 1.0 / a.scales[n] : a.step);
+  }
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const int row = p * 16 + rsub;
+    const int64_t m = m0 + row;
+    float v[16];
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const f32x4 t = *(const f32x4 *)(strip + row * F8_STRIDE + cc * 16 + q4 * 4);
+      v[q4 * 4 + 0] = t[0];
+      v[q4 * 4 + 1] = t[1];
+      v[q4 * 4 + 2] = t[2];
+      v[q4 * 4 + 3] = t[3];
+    }
+    float q[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      v[e] += bias[e];
+      if (a.do_relu) {  // post_relu, lib/Support/Dnnl/DnnlUtils.cpp:15-25
+        v[e] = v[e] > 0.0f ? v[e] : 0.0f;
+        if (a.relu_limit > 0.0f && v[e] > a.relu_limit)
+          v[e] = a.relu_limit;
+      }
+      // F8E4M3(v, step, true) = E4M3((float)((double)v / step)), Float8.cpp:259-261.  v * (1 / step) is within two
+      // double ulps of that quotient, so the narrowing can come out differently only when the 29 bits it drops sit
+      // next to the halfway pattern; only then is the division carried out.
+      double qd = (double)v[e] * inv[e];
+      const int32_t low = (int32_t)((uint32_t)__double_as_longlong(qd) & 0x1fffffffu);
+      if (low >= 0x10000000 - 4 && low <= 0x10000000 + 4) {
+        const int64_t n = (n0 + e) < a.N ? (n0 + e) : (a.N - 1);
+        qd = (double)v[e] / (a.scales ? 1.0 / a.scales[n] : a.step);
+      }
+      q[e] = (float)qd;
+    }
+    if (m >= a.M)
+      continue;
+    uint32_t c2[8];  // two codes each
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      c2[e] = f8_pair_codes(q[2 * e], q[2 * e + 1]);
+    const int64_t o = m * a.N + n0;
+    if (vec_ok) {
+      if (a.acc_out) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)
+          *(f32x4 *)(a.acc_out + o + q4 * 4) = f32x4{v[q4 * 4], v[q4 * 4 + 1], v[q4 * 4 + 2], v[q4 * 4 + 3]};
+      }
+      if (a.out_kind == MI_F8_OUT_CODES) {
+        *(u32x4 *)((uint8_t *)a.out + o) = u32x4{c2[0] | (c2[1] << 16), c2[2] | (c2[3] << 16), c2[4] | (c2[5] << 16),
+                                                 c2[6] | (c2[7] << 16)};
+        continue;
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      if (n0 + e >= a.N)
+        continue;
+      if (a.acc_out && !vec_ok)
+        a.acc_out[o + e] = v[e];
+      const uint32_t code = (c2[e >> 1] >> (8 * (e & 1))) & 0xffu;
+      if (a.out_kind == MI_F8_OUT_CODES)
+        ((uint8_t *)a.out)[o + e] = (uint8_t)code;
+      else if (a.out_kind == MI_F8_OUT_F32)
+        ((float *)a.out)[o + e] = f8e4m3_to_f32(code);
+      else if (a.out_kind == MI_F8_OUT_BF16)  // exact: E4M3 values fit both 16-bit types
+        ((uint16_t *)a.out)[o + e] = (uint16_t)(__float_as_uint(f8e4m3_to_f32(code)) >> 16);
+      else
+        ((uint16_t *)a.out)[o + e] = __builtin_bit_cast(uint16_t, (_Float16)f8e4m3_to_f32(code));
+    }
+  }
+}
+
+typedef const __attribute__((address_space(1))) void *f8_gptr_t;
+typedef __attribute__((address_space(3))) void *f8_lptr_t;
+constexpr int F8_STAGE = (F8_BM + F8_BN) * F8_BK;  // 16 KiB
+constexpr int f8_waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }  // s_waitcnt vmcnt(n) only
+// the ring, or the four epilogue strips that reuse its memory, whichever is larger
+constexpr int f8_ring_lds_bytes(int nst) { return nst * F8_STAGE > 4 * 64 * F8_STRIDE * 4 ? nst * F8_STAGE : 4 * 64 * F8_STRIDE * 4; }
+
+// NST = stages in the LDS ring: 4 (two workgroups per CU) when there are more tiles than CUs, 8 when every workgroup
+// has a CU to itself
+template <int NST>
+__global__ __launch_bounds__(256) void f8_gemm_ring_kernel(F8Args a, int tiles_m, int tiles_n, int per_xcd) {
+  constexpr int LOADS = F8_BM * (F8_BK / 16) / 256;  // direct-to-LDS instructions per operand, stage and thread: 2
+  constexpr int LPS = 2 * LOADS;
+  extern __shared__ __attribute__((aligned(16))) uint8_t f8_lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int bid = blockIdx.x;
+  const int L = (bid & 7) * per_xcd + (bid >> 3);  // each XCD gets a contiguous run of the tile order
+  if (L >= tiles_m * tiles_n)
+    return;
+  constexpr int GM = 4;  // tiles are ordered in groups of 4 tile rows, column-major inside a group
+  const int group = L / (GM * tiles_n);
+  const int gm = (tiles_m - group * GM) < GM ? (tiles_m - group * GM) : GM;
+  const int in_group = L - group * GM * tiles_n;
+  const int tm = group * GM + in_group % gm, tn = in_group / gm;
+  const int64_t m_base = (int64_t)tm * F8_BM, n_base = (int64_t)tn * F8_BN;
+
+  // the 16-byte chunk c of row r is stored at position c ^ ((r >> 2) & 3): the 32 rows of a fragment read hit distinct
+  // bank groups
+  const uint8_t *ga[LOADS], *gb[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int slot = (i * 4 + wave) * 64 + lane;
+    const int row = slot >> 2, pos = slot & 3;
+    const int chunk = pos ^ ((row >> 2) & 3);
+    int64_t ra = m_base + row, rb = n_base + row;
+    ra = ra < a.M ? ra : a.M - 1;  // rows past the matrix re-read the last one; their results are never stored
+    rb = rb < a.N ? rb : a.N - 1;
+    ga[i] = a.A + ra * a.K + chunk * 16;
+    gb[i] = a.B + rb * a.K + chunk * 16;
+  }
+  const int kt_total = (int)(a.K / F8_BK);
+  auto issue = [&](int kt) {
+    const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 1) * F8_BK;  // past the end: harmless re-load
+    uint8_t *sa = f8_lds + (kt % NST) * F8_STAGE, *sb = sa + F8_BM * F8_BK;
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      __builtin_amdgcn_global_load_lds((f8_gptr_t)(ga[i] + koff), (f8_lptr_t)(sa + (i * 4 + wave) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((f8_gptr_t)(gb[i] + koff), (f8_lptr_t)(sb + (i * 4 + wave) * 1024), 16, 0, 0);
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[i][j][r] = 0.0f;
+
+  const int frow = lane & 31, kh = lane >> 5;
+  int a_off[2], b_off[2];
+  const int f_sw = (frow >> 2) & 3;  // (row >> 2) & 3 with row = 32-aligned base + frow
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    a_off[i] = (wm * 64 + i * 32 + frow) * F8_BK;
+    b_off[i] = F8_BM * F8_BK + (wn * 64 + i * 32 + frow) * F8_BK;
+  }
+#pragma unroll
+  for (int s0 = 0; s0 < NST - 1; ++s0)
+    issue(s0);
+  for (int kt = 0; kt < kt_total; ++kt) {
+    // requests complete in order: at most (NST - 2) stages' worth outstanding means stage kt has landed
+    __builtin_amdgcn_s_waitcnt(f8_waitcnt_vm((NST - 2) * LPS));
+    __builtin_amdgcn_s_barrier();  // everyone's share of stage kt is in LDS; everyone is done with stage kt - 1
+    issue(kt + NST - 1);
+    const uint8_t *st = f8_lds + (kt % NST) * F8_STAGE;
+    // lane (row, kh) takes chunks kh and 2 + kh of its row for both operands
+    i32x8 fa[2], fb[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const u32x4 a0 = *(const u32x4 *)(st + a_off[i] + ((kh ^ f_sw) << 4));
+      const u32x4 a1 = *(const u32x4 *)(st + a_off[i] + (((2 + kh) ^ f_sw) << 4));
+      const u32x4 b0 = *(const u32x4 *)(st + b_off[i] + ((kh ^ f_sw) << 4));
+      const u32x4 b1 = *(const u32x4 *)(st + b_off[i] + (((2 + kh) ^ f_sw) << 4));
+      fa[i] = i32x8{(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
+      fb[i] = i32x8{(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+  }
+  __builtin_amdgcn_s_waitcnt(f8_waitcnt_vm(0));  // drain the re-loads issued past the end
+  __builtin_amdgcn_s_barrier();                  // every wave is done reading the ring
+  f8_strip_epilogue(a, acc, (float *)f8_lds + wave * (64 * F8_STRIDE), m_base + wm * 64, n_base + wn * 64, lane);
+}
+
+__global__ void f8_transpose_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t K, int64_t N) {
+  // [K, N] -> [N, K], 32 x 32 tiles through LDS
+  __shared__ uint8_t tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  const int64_t n0 = (int64_t)blockIdx.x * 32, k0 = (int64_t)blockIdx.y * 32;
+  for (int i = ty; i < 32; i += 8)
+    if (k0 + i < K && n0 + tx < N)
+      tile[i][tx] = src[(k0 + i) * N + n0 + tx];
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8)
+    if (n0 + i < N && k0 + tx < K)
+      dst[(n0 + i) * K + k0 + tx] = tile[tx][i];
+}
+
+int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, const float *d_bias, int64_t M, int64_t K,
+                int64_t N, int do_relu, double relu_limit, double out_scale, const double *d_out_scales, int out_kind,
+                void *d_out, float *d_acc, hipStream_t stream) {
+  MI_REQUIRE(M >= 0 && K > 0 && N > 0, MI_BAD_ARGUMENT, "mi_f8mm_launch: bad shape");
+  MI_REQUIRE(M == 0 || (d_a && d_b && d_out), MI_BAD_ARGUMENT, "mi_f8mm_launch: null argument");
+  MI_REQUIRE(out_kind >= MI_F8_OUT_CODES && out_kind <= MI_F8_OUT_F16, MI_BAD_ARGUMENT, "mi_f8mm_launch: out_kind");
+  MI_REQUIRE(d_out_scales || (out_scale == out_scale && out_scale != 0.0), MI_BAD_ARGUMENT,
+             "mi_f8mm_launch: the output scale must be a nonzero number");
+  MI_REQUIRE((M + F8_BM - 1) / F8_BM <= 65535, MI_UNSUPPORTED, "mi_f8mm_launch: M too large for one launch");
+  if (M == 0)
+    return MI_SUCCESS;
+  const uint8_t *b_nk = d_b;
+  if (!right_transpose) {  // [K, N] -> [N, K] into the stream's scratch buffer
+    uint8_t *t = nullptr;
+    int rc = stream_workspace(stream, WS_F8_TRANSPOSE, (size_t)N * K, false, (void **)&t);
+    if (rc != MI_SUCCESS)
+      return rc;
+    f8_transpose_kernel<<<dim3((unsigned)((N + 31) / 32), (unsigned)((K + 31) / 32)), dim3(256), 0, stream>>>(d_b, t, K, N);
+    b_nk = t;
+  }
+  F8Args a;
+  a.A = d_a;
+  a.B = b_nk;
+  a.bias = d_bias;
+  a.out = d_out;
+  a.acc_out = d_acc;
+  a.M = M;
+  a.K = K;
+  a.N = N;
+  a.do_relu = do_relu;
+  a.relu_limit = (float)relu_limit;
+  a.out_kind = out_kind;
+  a.step = (double)(float)(1 / out_scale);  // MatMul.cpp:613-615 into the float parameter of Float8.cpp:267
+  a.scales = d_out_scales;
+  const int64_t tiles_m = (M + F8_BM - 1) / F8_BM, tiles_n = (N + F8_BN - 1) / F8_BN;
+  if ((K % F8_BK) == 0 && tiles_m * tiles_n < (int64_t(1) << 30)) {
+    const int tiles = (int)(tiles_m * tiles_n), per_xcd = (tiles + 7) / 8;
+    static bool attr_set = false;
+    if (!attr_set) {
+      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                f8_ring_lds_bytes(8));
+      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                f8_ring_lds_bytes(4));
+      attr_set = true;
+    }
+    if (tiles <= 256)
+      f8_gemm_ring_kernel<8><<<dim3((unsigned)(per_xcd * 8)), dim3(256), f8_ring_lds_bytes(8), stream>>>(
+          a, (int)tiles_m, (int)tiles_n, per_xcd);
+    else
+      f8_gemm_ring_kernel<4><<<dim3((unsigned)(per_xcd * 8)), dim3(256), f8_ring_lds_bytes(4), stream>>>(
+          a, (int)tiles_m, (int)tiles_n, per_xcd);
+  } else {
+    dim3 grid((unsigned)tiles_n, (unsigned)tiles_m);
+    f8_gemm_kernel<<<grid, dim3(256), 0, stream>>>(a);
+  }
+  MI_HIP(hipGetLastError());
+  return MI_SUCCESS;
+}
+
+}  // namespace mi

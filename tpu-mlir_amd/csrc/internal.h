@@ -73,12 +73,17 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
 
 // library-owned scratch, one buffer per (device, stream, purpose) (workspace.hip).  zeroed: cleared when allocated;
 // the user of such a buffer leaves it zero.
-enum { WS_SPLIT_K = 0, WS_DYNAMIC_QUANT = 1 };
+enum { WS_SPLIT_K = 0, WS_DYNAMIC_QUANT = 1, WS_F8_TRANSPOSE = 2 };
 int stream_workspace(hipStream_t st, int purpose, size_t bytes, bool zeroed, void **out);
 
 // dynamic activation quantization (dq_kernels.hip); dq_type: MI_DQ_INT, MI_DQ_F8E4M3 (8-bit weights), MI_DQ_F4 (4-bit)
 int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                   hipStream_t stream);
+
+// tpu.MatMul on F8E4M3 codes with the F8 output requantization (f8_kernels.hip)
+int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, const float *d_bias, int64_t M, int64_t K,
+                int64_t N, int do_relu, double relu_limit, double out_scale, const double *d_out_scales, int out_kind,
+                void *d_out, float *d_acc, hipStream_t stream);
 
 int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
                      int64_t N, int q_group_size, int dq_type, int dtype, uint16_t *d_y, float *d_y32,

@@ -334,6 +334,54 @@ def matmul_dq_launch(left, right, *, right_transpose=False, q_group_size, dq_typ
     return y
 
 
+def matmul_f8(left, right, bias=None, *, right_transpose=False, do_relu=False, relu_limit=-1.0, out_scales=(1.0,)):
+    """tpu.MatMul on operands holding E4M3 values with the F8 output requantization, interpreter convention (float32
+    numpy in and out; the output holds E4M3 values).  out_scales: one scale or one per output channel."""
+    left, right = _f32(left), _f32(right)
+    M, K = left.shape
+    N = right.shape[0] if right_transpose else right.shape[1]
+    sc = np.ascontiguousarray(out_scales, dtype=np.float64).reshape(-1)
+    attr = clib.F8MMAttr(M, K, N, int(right_transpose), int(do_relu), float(relu_limit),
+                         sc.ctypes.data_as(C.POINTER(C.c_double)), sc.size)
+    y = np.empty((M, N), dtype=np.float32)
+    ins = [left, right] + ([] if bias is None else [_f32(bias)])
+    p = _Param(ins, [y])
+    check(clib.lib().mi_f8mm_inference(C.byref(attr), C.byref(p.c)))
+    return y
+
+
+def f8mm_launch(a_codes, b_codes, bias=None, *, right_transpose=False, do_relu=False, relu_limit=-1.0, out_scale=1.0,
+                out_scales=None, out_kind=clib.F8_OUT_CODES, acc_f32=None, out=None, stream=None):
+    """Device level: a_codes [M, K], b_codes [K, N] ([N, K] when right_transpose) uint8 CUDA tensors of E4M3 codes; bias
+    float32 [N]; out_scales float64 [N] CUDA tensor for per-channel requantization.  Returns the output tensor (uint8
+    codes, or the values as float32 / bfloat16 / float16 by out_kind)."""
+    import torch
+    if not (a_codes.is_cuda and b_codes.is_cuda and a_codes.dtype == torch.uint8 and b_codes.dtype == torch.uint8
+            and a_codes.is_contiguous() and b_codes.is_contiguous() and a_codes.dim() == 2 and b_codes.dim() == 2):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "f8mm_launch: operands must be contiguous 2-D uint8 CUDA tensors")
+    M, K = a_codes.shape
+    N = b_codes.shape[0] if right_transpose else b_codes.shape[1]
+    if (b_codes.shape[1] if right_transpose else b_codes.shape[0]) != K:
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "f8mm_launch: inner dimensions differ")
+    if bias is not None and not (bias.is_cuda and bias.dtype == torch.float32 and bias.numel() == N):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "f8mm_launch: bias must be a float32 CUDA tensor [N]")
+    if out_scales is not None and not (out_scales.is_cuda and out_scales.dtype == torch.float64
+                                       and out_scales.numel() == N and out_scales.is_contiguous()):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "f8mm_launch: out_scales must be a float64 CUDA tensor [N]")
+    if acc_f32 is not None and not (acc_f32.is_cuda and acc_f32.dtype == torch.float32 and acc_f32.numel() == M * N
+                                    and acc_f32.is_contiguous()):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "f8mm_launch: acc_f32 must be a float32 CUDA tensor [M, N]")
+    tdt = {clib.F8_OUT_CODES: torch.uint8, clib.F8_OUT_F32: torch.float32, clib.F8_OUT_BF16: torch.bfloat16,
+           clib.F8_OUT_F16: torch.float16}[out_kind]
+    y = torch.empty((M, N), dtype=tdt, device=a_codes.device) if out is None else out
+    if not (y.is_cuda and y.dtype == tdt and y.is_contiguous() and y.numel() == M * N):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "f8mm_launch: bad output tensor")
+    check(clib.lib().mi_f8mm_launch(_dptr(a_codes), _dptr(b_codes), int(right_transpose), _dptr(bias), M, K, N,
+                                    int(do_relu), float(relu_limit), float(out_scale), _dptr(out_scales), out_kind,
+                                    _dptr(y), _dptr(acc_f32), _stream_ptr(stream)))
+    return y
+
+
 def a16mm_dq_launch(w, x, y=None, y_f32=None, stream=None, dq_type=clib.DQ_INT):
     """As a16mm_launch, with the reference's dynamic activation quantization: dq_type DQ_INT (integer codes, 4- or 8-bit
     weights), DQ_F8E4M3 (8-bit weights holding E4M3 codes) or DQ_F4 (4-bit weights holding E2M1 codes)."""
