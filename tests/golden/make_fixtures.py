@@ -276,6 +276,16 @@ def case_float_codes():
                                      q_group_size=g, dq_type=O.DQ_F8E4M3)
         out.update({tag + "_x": xx, tag + "_weight": ww, tag + "_want_bf16": O.f32_to_bf16(y), tag + "_want_pre": pre})
     out["f8_scale"] = scale
+    # tpu.MatMul on E4M3 operands with F8 output requantization: small integers (every sum exact), per-channel scales,
+    # bias, relu with a limit, right operand [N, K]
+    M, K, N = 40, 192, 72
+    la = rng.integers(-15, 16, size=(M, K)).astype(np.float32)
+    rb = rng.integers(-15, 16, size=(N, K)).astype(np.float32) * 0.5
+    bias = rng.integers(-200, 201, size=N).astype(np.float32)
+    mm_scales = rng.uniform(0.01, 0.05, size=N)
+    y, acc = O.matmul_f8(la, rb, bias, right_transpose=True, do_relu=True, relu_limit=900.0, scales=mm_scales)
+    out.update(f8mm_left=O.f32_to_f8e4m3(la), f8mm_right=O.f32_to_f8e4m3(rb), f8mm_bias=bias, f8mm_scales=mm_scales,
+               f8mm_want_codes=O.f32_to_f8e4m3(y), f8mm_want_acc=acc)
     np.savez_compressed(os.path.join(HERE, "case_float_codes.npz"), **out)
 
 

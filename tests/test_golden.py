@@ -152,6 +152,11 @@ def test_oracle_reproduces_float_code_cases(orc):
         assert np.array_equal(pre, d[tag + "_want_pre"]) and np.array_equal(orc.f32_to_bf16(out), d[tag + "_want_bf16"])
 
 
+    y, acc = orc.matmul_f8(orc.f8e4m3_to_f32(d["f8mm_left"]), orc.f8e4m3_to_f32(d["f8mm_right"]), d["f8mm_bias"],
+                           right_transpose=True, do_relu=True, relu_limit=900.0, scales=d["f8mm_scales"])
+    assert np.array_equal(orc.f32_to_f8e4m3(y), d["f8mm_want_codes"]) and np.array_equal(acc, d["f8mm_want_acc"])
+
+
 FLOAT_QUANT_TAGS = {"f8_g64": dict(bits=8, g=64, dq="DQ_F8E4M3"), "f4_g128": dict(bits=4, g=128, dq="DQ_F4")}
 
 
@@ -188,6 +193,13 @@ def test_gpu_float_codes_against_fixture():
     out, pre = run(d["f8exact_x"], d["f8exact_weight"], d["f8_scale"], zp, None, 8, 64, clib.DQ_F8E4M3)
     assert np.array_equal(pre.view(np.uint32), d["f8exact_want_pre"].view(np.uint32))
     assert np.array_equal(out, d["f8exact_want_bf16"])
+    acc = torch.empty(d["f8mm_want_acc"].shape, dtype=torch.float32, device="cuda")
+    y = M_.f8mm_launch(torch.from_numpy(d["f8mm_left"]).cuda(), torch.from_numpy(d["f8mm_right"]).cuda(),
+                       torch.from_numpy(d["f8mm_bias"]).cuda(), right_transpose=True, do_relu=True, relu_limit=900.0,
+                       out_scales=torch.from_numpy(d["f8mm_scales"]).cuda(), acc_f32=acc)
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy().view(np.uint32), d["f8mm_want_acc"].view(np.uint32))
+    assert np.array_equal(y.cpu().numpy(), d["f8mm_want_codes"])
     out, pre = run(d["f8rand_x"], d["f8rand_weight"], d["f8_scale"], zp, None, 8, 64, clib.DQ_F8E4M3)
     wv = np.abs(d["f8_decode"][d["f8rand_weight"]].astype(np.float64)).reshape(24, 4, 64)
     deq = (wv * S.bf16_to_f32(d["f8_scale"]).astype(np.float64)[:, :, None]).reshape(24, 256)
