@@ -226,7 +226,9 @@ int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
 /* The same for n (1..4) weight sets that read the SAME activations, in one kernel launch: y_i = x * dequant(W_i)^T.
  * These are the sibling linears the reference's LLM export emits on one input -- q/k/v on the normed hidden state
  * (python/llm/LlmConverter.py:1797-1812), gate/up in the MLP -- each of which the interpreter runs as its own
- * A16MatMulOp::inference (A16MatMul.cpp:150-273).  Results are identical to n calls of mi_a16mm_launch.  The sets
+ * A16MatMulOp::inference (A16MatMul.cpp:150-273).  Results are identical to n calls of mi_a16mm_launch (with more
+ * than 16 rows and a K long enough to be split over workgroups, identical up to the order of the fp32 partial sums,
+ * as between two calls of mi_a16mm_launch itself; such launches cover three sets at a time).  The sets
  * must agree in K, weight_bits, q_group_size, dtype and chip; N may differ.  d_y[i] / d_y_f32[i] as above
  * (d_y_f32 itself may be NULL, as may any of its entries). */
 /* The dynamic-quantization flavour of the same product (A16MatMul.cpp:40-170, integer dq types): activations are

@@ -284,3 +284,27 @@ def test_grouped_launch_equals_separate_launches(bits, M):
         M_.a16mm_launch_group([ws[0], wo], x)
     for w in ws + [wo]:
         w.destroy()
+
+
+@pytest.mark.parametrize("bits,M,K,Ns,g", [(4, 32, 4096, (256, 128, 64), 128), (4, 100, 2048, (512, 384), 64),
+                                          (8, 48, 2048, (128, 256, 128), 0), (4, 24, 1024, (48, 20, 36, 64), 128)])
+def test_grouped_launch_through_the_tiled_kernel(orc, bits, M, K, Ns, g):
+    """Sibling weight sets with more than 16 rows: one tiled launch (and one finishing pass when K is split) covers up
+    to three sets; every output is checked against the oracle, twice in a row (the second call finds the partial-sum
+    buffer the first one left behind).  Four sets take two launches."""
+    torch = _torch()
+    cfgs = [S.w4a16(M, K, N, g, seed=40 + i, bias=(i != 1)) if bits == 4 else S.w8a16(M, K, N, g, seed=40 + i, bias=(i == 0))
+            for i, N in enumerate(Ns)]
+    for c in cfgs:
+        c["x"] = cfgs[0]["x"]
+    x = torch.from_numpy(cfgs[0]["x"].view(np.int16)).cuda().view(torch.bfloat16)
+    ws = [M_.A16Weight(c["weight"], c["scale"], c["zp"], None if c.get("bias") is None else S.bf16_to_f32(c["bias"]),
+                       K=K, N=c["N"], weight_bits=bits, q_group_size=c["g"]) for c in cfgs]
+    for _ in range(2):
+        f32s = [torch.empty((M, c["N"]), dtype=torch.float32, device="cuda") for c in cfgs]
+        ys = M_.a16mm_launch_group(ws, x, ys_f32=f32s)
+        torch.cuda.synchronize()
+        for c, y, f in zip(cfgs, ys, f32s):
+            _check_against_oracle(orc, c, y.view(torch.int16).cpu().numpy().view(np.uint16), f.cpu().numpy())
+    for w in ws:
+        w.destroy()

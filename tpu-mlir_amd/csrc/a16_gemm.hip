@@ -12,6 +12,8 @@
 //          acc += scale * (P - (16 + zp) * S) in fp32.
 //   8-bit: the weight is rounded to the 16-bit type exactly as the reference does, and the MFMA accumulates directly.
 #include <algorithm>
+#include <climits>
+#include <cstdint>
 
 #include "a16_common.cuh"
 #include "internal.h"
@@ -36,21 +38,35 @@ extern "C" int mi_gemm_dbg_dump(unsigned long long *host) {
 #define MI_GT(v)
 #endif
 
-struct GemmArgs {
+// One weight set of a launch.  Sibling sets on one input (q/k/v, gate/up: same K, width, group size and type) share a
+// launch: their output blocks are numbered one set after the other.
+constexpr int GEMM_MAX_SEG = 3;
+struct GemmSeg {
   const u32x4 *qw;
   const uint32_t *sz_t;
   const uint16_t *scale_t;
   const float *nzs_t;
   const float *bias;
-  const uint16_t *x;
   uint16_t *y;
   float *y32;
+  int64_t N;
+  int row_blocks;
+  int tiles_n;        // output blocks across N
+  int tile_begin;     // first output block of this set in the launch's numbering (INT32_MAX: unused slot)
+  int64_t acc_begin;  // first element of this set's [M, N] partial sums in the split-K buffer
+};
+
+struct GemmArgs {
+  GemmSeg seg[GEMM_MAX_SEG];
+  int n_seg;
+  int tiles_total;  // output blocks of all sets
+  const uint16_t *x;
   int M;
-  int64_t K, N;
-  int row_blocks, k_tiles, G;
+  int64_t K;
+  int k_tiles, G;
   int tiles_per_group;  // GPT == 1: weight tiles that share one group (g / TILE_K; k_tiles when per channel)
   int chip;
-  int tiles_m, tiles_n, per_xcd;
+  int tiles_m, per_xcd;
   // split K: each output block is computed by k_splits workgroups over kt_per_split stages each, which add their
   // fp32 partial sums into acc [M, N] (zero on entry); bias and rounding happen in a16_gemm_finish_kernel
   int k_splits, kt_per_split;
@@ -94,14 +110,22 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
   // run of the block order (column-major inside groups of 4 block-rows) so that its L2 sees few distinct panels
   const int bid = blockIdx.x;
   const int Ls = (bid & 7) * a.per_xcd + (bid >> 3);
-  if (Ls >= a.tiles_m * a.tiles_n * a.k_splits)
+  if (Ls >= a.tiles_total * a.k_splits)
     return;
-  const int L = a.k_splits == 1 ? Ls : Ls / a.k_splits;
-  const int split = Ls - L * a.k_splits;
+  const int Lg = a.k_splits == 1 ? Ls : Ls / a.k_splits;
+  const int split = Ls - Lg * a.k_splits;
+  // which weight set: wave-uniform, so everything taken from it lives in scalar registers
+  const int si = (Lg >= a.seg[1].tile_begin ? 1 : 0) + (Lg >= a.seg[2].tile_begin ? 1 : 0);
+  GemmSeg sg = a.seg[0];  // selected, not indexed: a runtime index would move the argument block to scratch memory
+  if (si == 1)
+    sg = a.seg[1];
+  else if (si == 2)
+    sg = a.seg[2];
+  const int L = Lg - sg.tile_begin;
   constexpr int GRP = 4;
-  const int group = L / (GRP * a.tiles_n);
+  const int group = L / (GRP * sg.tiles_n);
   const int gm = (a.tiles_m - group * GRP) < GRP ? (a.tiles_m - group * GRP) : GRP;
-  const int in_group = L - group * GRP * a.tiles_n;
+  const int in_group = L - group * GRP * sg.tiles_n;
   const int tm = group * GRP + in_group % gm, tn = in_group / gm;
   const int64_t m_base = (int64_t)tm * GM, n_base = (int64_t)tn * GN;
 
@@ -129,10 +153,10 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
 #pragma unroll
     for (int i = 0; i < WL; ++i) {
       int64_t rb = n_base / 16 + (i * GEMM_WAVES + wave);
-      w_tile_rb[i] = rb < a.row_blocks ? rb : a.row_blocks - 1;  // clamped, discarded at the store
+      w_tile_rb[i] = rb < sg.row_blocks ? rb : sg.row_blocks - 1;  // clamped, discarded at the store
     }
     sz_rb = n_base / 16 + wn * TN + (kq & (TN - 1));
-    sz_rb = sz_rb < a.row_blocks ? sz_rb : a.row_blocks - 1;
+    sz_rb = sz_rb < sg.row_blocks ? sz_rb : sg.row_blocks - 1;
   }
   auto unit_group = [&](int tile, int u) {
     int gi;
@@ -152,11 +176,11 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
     if constexpr (WLDS) {
 #pragma unroll
       for (int i = 0; i < WL; ++i)
-        __builtin_amdgcn_global_load_lds((gptr_t)(a.qw + (w_tile_rb[i] * a.k_tiles + ktc) * 64 + lane),
+        __builtin_amdgcn_global_load_lds((gptr_t)(sg.qw + (w_tile_rb[i] * a.k_tiles + ktc) * 64 + lane),
                                          (lptr_t)(st + X_BYTES + (i * GEMM_WAVES + wave) * 1024), 16, 0, 0);
 #pragma unroll
       for (int u = 0; u < GPT; ++u)
-        __builtin_amdgcn_global_load_lds((gptr_t)(a.sz_t + (sz_rb * a.G + unit_group(ktc, u)) * 16 + col),
+        __builtin_amdgcn_global_load_lds((gptr_t)(sg.sz_t + (sz_rb * a.G + unit_group(ktc, u)) * 16 + col),
                                          (lptr_t)(st + X_BYTES + W_BYTES + (wave * GPT + u) * 256), 4, 0, 0);
     }
   };
@@ -178,10 +202,10 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       int64_t rb = n_base / 16 + (wn * TN + j);
-      rb = rb < a.row_blocks ? rb : a.row_blocks - 1;  // clamped, discarded at the store
-      wq[j] = a.qw + rb * a.k_tiles * 64 + lane;
-      scp[j] = a.scale_t + rb * a.G * 16 + col;
-      nzp[j] = a.nzs_t + rb * a.G * 16 + col;
+      rb = rb < sg.row_blocks ? rb : sg.row_blocks - 1;  // clamped, discarded at the store
+      wq[j] = sg.qw + rb * a.k_tiles * 64 + lane;
+      scp[j] = sg.scale_t + rb * a.G * 16 + col;
+      nzp[j] = sg.nzs_t + rb * a.G * 16 + col;
     }
   }
   auto load_w = [&](WStage &s, int kt) {  // 8-bit: global -> registers, issued one stage ahead
@@ -339,76 +363,109 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int64_t n = n_base + (wn * TN + j) * 16 + col;
-    const bool n_ok = n < a.N;
-    const float b = (a.bias && n_ok) ? a.bias[n] : 0.0f;
+    const bool n_ok = n < sg.N;
+    const float b = (sg.bias && n_ok) ? sg.bias[n] : 0.0f;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int64_t m = m_base + (wm * TM + i) * 16 + 4 * kq + r;
         if (n_ok && m < a.M && a.acc) {
-          atomicAdd(a.acc + m * a.N + n, acc[i][j][r]);  // bias and rounding: a16_gemm_finish_kernel
+          atomicAdd(a.acc + sg.acc_begin + m * sg.N + n, acc[i][j][r]);  // bias and rounding: a16_gemm_finish_kernel
         } else if (n_ok && m < a.M) {
           const float v = acc[i][j][r] + b;
-          const int64_t o = m * a.N + n;
-          if (a.y32)
-            a.y32[o] = v;
-          a.y[o] = (a.chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+          const int64_t o = m * sg.N + n;
+          if (sg.y32)
+            sg.y32[o] = v;
+          sg.y[o] = (a.chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
         }
       }
   }
 }
 
 // Second half of a split-K product: y = round16(acc + bias) (and the fp32 value, if asked for), and acc goes back to
-// zero so that the next product on this stream finds it clean.
+// zero so that the next product on this stream finds it clean.  One launch covers every weight set of the product.
+struct FinishArgs {
+  float *acc;
+  const float *bias[GEMM_MAX_SEG];
+  uint16_t *y[GEMM_MAX_SEG];
+  float *y32[GEMM_MAX_SEG];
+  int64_t N[GEMM_MAX_SEG];
+  int64_t begin[GEMM_MAX_SEG];  // first element of the set in acc (INT64_MAX: unused slot)
+  int64_t total;
+  int chip;
+};
+
 template <int DT>
-__global__ void a16_gemm_finish_kernel(float *__restrict__ acc, const float *__restrict__ bias, uint16_t *__restrict__ y,
-                                       float *__restrict__ y32, int64_t total, int64_t N, int chip) {
+__global__ void a16_gemm_finish_kernel(FinishArgs f) {
   const int64_t i4 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
-  if (i4 >= total)
+  if (i4 >= f.total)
     return;
-  const f32x4 v4 = *(const f32x4 *)(acc + i4);  // N % 4 == 0 (checked by the host): a group of 4 stays in one row
-  *(f32x4 *)(acc + i4) = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int64_t n = i4 % N;
+  const f32x4 v4 = *(const f32x4 *)(f.acc + i4);  // every N % 4 == 0 (checked by the host): a group of 4 stays in one row
+  *(f32x4 *)(f.acc + i4) = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int si = (i4 >= f.begin[1] ? 1 : 0) + (i4 >= f.begin[2] ? 1 : 0);
+  // selected, not indexed: a runtime index would move the argument arrays to scratch memory
+  const float *bias = si == 0 ? f.bias[0] : si == 1 ? f.bias[1] : f.bias[2];
+  uint16_t *y = si == 0 ? f.y[0] : si == 1 ? f.y[1] : f.y[2];
+  float *y32 = si == 0 ? f.y32[0] : si == 1 ? f.y32[1] : f.y32[2];
+  const int64_t N = si == 0 ? f.N[0] : si == 1 ? f.N[1] : f.N[2];
+  const int64_t o = i4 - (si == 0 ? f.begin[0] : si == 1 ? f.begin[1] : f.begin[2]);
+  const int64_t n = o % N;
   uint16_t h[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const float v = v4[e] + (bias ? bias[n + e] : 0.0f);
     if (y32)
-      y32[i4 + e] = v;
-    h[e] = (chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+      y32[o + e] = v;
+    h[e] = (f.chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
   }
-  *(u32x2 *)(y + i4) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+  *(u32x2 *)(y + o) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
 }
 
 template <int BITS, int DT, int GPT, int WM, int WN, int TM, int TN>
 static int launch_gemm_instance(GemmArgs &a, hipStream_t st) {
   constexpr int GM = WM * TM * 16, GN = WN * TN * 16;
   a.tiles_m = (int)((a.M + GM - 1) / GM);
-  a.tiles_n = (int)((a.N + GN - 1) / GN);
+  int64_t tiles = 0, acc_elems = 0;
+  bool n4 = true;
+  for (int i = 0; i < GEMM_MAX_SEG; ++i) {
+    GemmSeg &sg = a.seg[i];
+    if (i >= a.n_seg) {
+      sg = a.seg[0];
+      sg.tile_begin = INT32_MAX;  // never selected
+      continue;
+    }
+    sg.tiles_n = (int)((sg.N + GN - 1) / GN);
+    sg.tile_begin = (int)tiles;
+    sg.acc_begin = acc_elems;
+    tiles += (int64_t)a.tiles_m * sg.tiles_n;
+    acc_elems += (int64_t)a.M * sg.N;
+    n4 = n4 && (sg.N % 4) == 0;
+  }
+  MI_REQUIRE(tiles < (int64_t(1) << 24), MI_BAD_ARGUMENT, "a16 tiled product: too many output blocks for one launch");
+  a.tiles_total = (int)tiles;
   // split K when the output blocks alone leave most of the 256 CUs idle: enough workgroups for one per CU, at least
   // four stages each
-  const int tiles = a.tiles_m * a.tiles_n;
   const int kt_all = (int)(a.K / GEMM_KS);
   int splits = 1;
   const char *e = getenv("MI_A16_GEMM_SPLITS");  // development switch
   if (e)
     splits = atoi(e);
-  else if (tiles < 160 && (a.N % 4) == 0)
-    splits = std::min(std::max(256 / tiles, 1), std::max(kt_all / 4, 1));
+  else if (tiles < 160 && n4)
+    splits = std::min(std::max(256 / (int)tiles, 1), std::max(kt_all / 4, 1));
   splits = std::max(1, std::min(splits, kt_all));
   a.kt_per_split = (kt_all + splits - 1) / splits;
   a.k_splits = (kt_all + a.kt_per_split - 1) / a.kt_per_split;  // no empty split
   a.acc = nullptr;
   if (a.k_splits > 1) {
-    MI_REQUIRE((a.N % 4) == 0, MI_BAD_ARGUMENT, "a16 split-K product: N must be a multiple of 4");
+    MI_REQUIRE(n4, MI_BAD_ARGUMENT, "a16 split-K product: N must be a multiple of 4");
     // fp32 partial sums: the stream's own buffer, zero whenever no product is in flight (the finishing pass clears
     // what it reads)
-    int rc = stream_workspace(st, WS_SPLIT_K, (size_t)a.M * a.N * sizeof(float), true, (void **)&a.acc);
+    int rc = stream_workspace(st, WS_SPLIT_K, (size_t)acc_elems * sizeof(float), true, (void **)&a.acc);
     if (rc != MI_SUCCESS)
       return rc;
   }
-  a.per_xcd = (tiles * a.k_splits + 7) / 8;
+  a.per_xcd = (a.tiles_total * a.k_splits + 7) / 8;
   auto kfn = a16_gemm_kernel<BITS, DT, GPT, WM, WN, TM, TN>;
   const size_t lds_bytes =
       (size_t)GEMM_NST * ((GM < 32 ? 32 : GM) * GEMM_KS * 2 + (BITS == 4 ? (GN / 16) * 1024 + GEMM_WAVES * GPT * 256 : 0));
@@ -419,9 +476,19 @@ static int launch_gemm_instance(GemmArgs &a, hipStream_t st) {
   }
   kfn<<<dim3((unsigned)(a.per_xcd * 8)), dim3(GEMM_WAVES * 64), lds_bytes, st>>>(a);
   if (a.k_splits > 1) {
-    const int64_t total = (int64_t)a.M * a.N;
-    a16_gemm_finish_kernel<DT><<<dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, st>>>(a.acc, a.bias, a.y, a.y32,
-                                                                                             total, a.N, a.chip);
+    FinishArgs f;
+    f.acc = a.acc;
+    for (int i = 0; i < GEMM_MAX_SEG; ++i) {
+      const GemmSeg &sg = a.seg[i];
+      f.bias[i] = sg.bias;
+      f.y[i] = sg.y;
+      f.y32[i] = sg.y32;
+      f.N[i] = sg.N;
+      f.begin[i] = i < a.n_seg ? sg.acc_begin : INT64_MAX;
+    }
+    f.total = acc_elems;
+    f.chip = a.chip;
+    a16_gemm_finish_kernel<DT><<<dim3((unsigned)((acc_elems / 4 + 255) / 256)), dim3(256), 0, st>>>(f);
   }
   return MI_SUCCESS;
 }
@@ -429,7 +496,9 @@ static int launch_gemm_instance(GemmArgs &a, hipStream_t st) {
 template <int BITS, int DT, int GPT>
 static int launch_gemm_shape(GemmArgs &a, hipStream_t st) {
   // 128 x 256 blocks when they fill the chip, else 128 x 128
-  const int64_t big = ((a.M + 127) / 128) * ((a.N + 255) / 256);
+  int64_t big = 0;
+  for (int i = 0; i < a.n_seg; ++i)
+    big += ((a.M + 127) / 128) * ((a.seg[i].N + 255) / 256);
   const char *e = getenv("MI_A16_GEMM_TILE");  // development switch: "256" / "128"
   constexpr bool fits = !(BITS == 4 && GPT == 4);  // 32-wide groups: a 256-column block's scale|zp words overflow LDS
   const bool wide = fits && (e ? atoi(e) == 256 : big >= 192);
@@ -477,19 +546,35 @@ bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M) {
 
 int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                     hipStream_t stream) {
+  return a16_gemm_launch_group(&w, 1, d_x, M, &d_y, d_y32 ? &d_y32 : nullptr, stream);
+}
+
+// ws[0..n): sibling weight sets on one input -- same K, width, group size, type and chip (checked by the caller)
+int a16_gemm_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
+                          float *const *d_y32s, hipStream_t stream) {
+  MI_REQUIRE(n >= 1 && n <= GEMM_MAX_SEG, MI_BAD_ARGUMENT, "a16 tiled product: one to three weight sets per launch");
+  const mi_a16_weight *w = ws[0];
   GemmArgs a;
-  a.qw = (const u32x4 *)w->qweight;
-  a.sz_t = w->sz_t;
-  a.scale_t = w->scale_t;
-  a.nzs_t = w->nzs_t;
-  a.bias = w->bias;
+  a.n_seg = n;
+  for (int i = 0; i < n; ++i) {
+    const mi_a16_weight *v = ws[i];
+    GemmSeg &sg = a.seg[i];
+    sg.qw = (const u32x4 *)v->qweight;
+    sg.sz_t = v->sz_t;
+    sg.scale_t = v->scale_t;
+    sg.nzs_t = v->nzs_t;
+    sg.bias = v->bias;
+    sg.y = d_ys[i];
+    sg.y32 = d_y32s ? d_y32s[i] : nullptr;
+    sg.N = v->N;
+    sg.row_blocks = (int)v->row_blocks;
+    sg.tiles_n = 0;
+    sg.tile_begin = 0;
+    sg.acc_begin = 0;
+  }
   a.x = d_x;
-  a.y = d_y;
-  a.y32 = d_y32;
   a.M = (int)M;
   a.K = w->K;
-  a.N = w->N;
-  a.row_blocks = (int)w->row_blocks;
   a.k_tiles = (int)w->k_tiles;
   a.G = w->G;
   a.chip = w->chip;

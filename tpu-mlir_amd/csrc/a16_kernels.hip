@@ -817,9 +817,10 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
   MI_REQUIRE(total_rb < (1ll << 31), MI_BAD_ARGUMENT, "mi_a16mm_launch: too many output channels for one launch");
   if (M == 0)
     return MI_SUCCESS;
-  if (a16_gemm_applicable(w, M)) {  // many rows: the tiled MFMA GEMM, one launch per weight set
-    for (int i = 0; i < n; ++i) {
-      const int rc = a16_gemm_launch(ws[i], d_x, M, d_ys[i], d_y32s ? d_y32s[i] : nullptr, stream);
+  if (a16_gemm_applicable(w, M)) {  // many rows: the tiled MFMA GEMM, up to three sibling sets per launch
+    for (int i = 0; i < n; i += 3) {
+      const int cnt = (n - i) < 3 ? (n - i) : 3;
+      const int rc = a16_gemm_launch_group(ws + i, cnt, d_x, M, d_ys + i, d_y32s ? d_y32s + i : nullptr, stream);
       if (rc != MI_SUCCESS)
         return rc;
     }

@@ -68,6 +68,9 @@ int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t 
 bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M);
 int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                     hipStream_t stream);
+// up to three sibling weight sets (same K, width, group size, type, chip) on one input in one launch
+int a16_gemm_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
+                          float *const *d_y32s, hipStream_t stream);
 int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
                      float *const *d_y32s, hipStream_t stream);
 
