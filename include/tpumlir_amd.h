@@ -371,6 +371,11 @@ int mi_module_add_tensor(mi_module *m, const char *name, int storage_type /* MI_
  * read the same tensor with compatible weight sets are issued as one grouped launch. */
 int mi_module_add_a16matmul(mi_module *m, const char *input, const char *output, const mi_a16_weight_desc *desc,
                             const void *weight, const uint16_t *scale, const uint8_t *zp, const float *bias);
+/* the same op under module::isDynamicQuantize() (A16MatMul.cpp:40-170): dq_type MI_DQ_INT / MI_DQ_F8E4M3 / MI_DQ_F4 as
+ * for mi_a16mm_dq_type_launch; shapes the dynamic kernels do not handle are refused here (MI_UNSUPPORTED) */
+int mi_module_add_a16matmul_dq(mi_module *m, const char *input, const char *output, const mi_a16_weight_desc *desc,
+                               int dq_type, const void *weight, const uint16_t *scale, const uint8_t *zp,
+                               const float *bias);
 typedef struct mi_module_i8_desc {
   int64_t K, N;
   const void *right;        /* HOST int8/uint8 weight, [K,N] or (right_transpose) [N,K] */

@@ -108,3 +108,44 @@ def test_argument_errors():
     with pytest.raises(clib.BackendError):
         m.set_tensor("a", np.zeros(5, dtype=np.float32))
     m.destroy()
+
+
+@pytest.mark.parametrize("dq,bits", [("DQ_INT", 4), ("DQ_INT", 8), ("DQ_F4", 4)])
+def test_dynamic_quant_a16matmul_in_a_module(orc, dq, bits):
+    """Cast f32 -> bf16, then A16MatMul with dynamic activation quantization, then a second one on its output, all
+    device-resident; the integer and F4 code types are exact, so every tensor must equal the oracle's bit for bit --
+    on the eager first invoke and on the graph replays after it."""
+    M, K, N, g = 5, 512, 256, 128
+    c1 = S.w4a16(M, K, N, g, seed=311, bias=True) if bits == 4 else S.w8a16(M, K, N, g, seed=311, bias=True, signed=False)
+    c2 = S.w4a16(M, N, 128, g, seed=312) if bits == 4 else S.w8a16(M, N, 128, g, seed=312, signed=False)
+    if dq == "DQ_F4":
+        c1["zp"], c2["zp"] = np.zeros_like(c1["zp"]), np.zeros_like(c2["zp"])
+    m = M_.Module()
+    m.add_tensor("x", clib.ST_F32, (M, K)).add_tensor("xb", clib.ST_BF16, (M, K))
+    m.add_tensor("h", clib.ST_BF16, (M, N)).add_tensor("y", clib.ST_BF16, (M, 128))
+    m.add_cast("x", "xb", in_type=clib.ST_F32, out_type=clib.ST_BF16)
+    m.add_a16matmul("xb", "h", c1["weight"], c1["scale"], c1["zp"], S.bf16_to_f32(c1["bias"]), K=K, N=N,
+                    weight_bits=bits, q_group_size=g, dq_type=getattr(clib, dq))
+    m.add_a16matmul("h", "y", c2["weight"], c2["scale"], c2["zp"], None, K=N, N=128, weight_bits=bits, q_group_size=g,
+                    dq_type=getattr(clib, dq))
+    x32 = (np.random.default_rng(2).standard_normal((M, K)) * 0.7).astype(np.float32)
+    odq = getattr(orc, dq)
+    for rep in range(3):
+        x = x32 * (1.0 + rep)
+        m.set_tensor("x", x)
+        m.invoke()
+        xb = orc.cast(x, in_type=orc.ST_F32, out_type=orc.ST_BF16)
+        _, w, s, z, b = f32_valued_a16(c1)
+        h, _ = orc.a16matmul_dynamic(xb, w, s, z, b, M=M, K=K, N=N, weight_bits=bits, q_group_size=g, dq_type=odq)
+        _, w, s, z, _ = f32_valued_a16(c2)
+        y, _ = orc.a16matmul_dynamic(h, w, s, z, None, M=M, K=N, N=128, weight_bits=bits, q_group_size=g, dq_type=odq)
+        assert np.array_equal(m.get_tensor("h"), h), rep
+        assert np.array_equal(m.get_tensor("y"), y), rep
+    # shapes the dynamic kernels do not handle are refused when the op is added
+    bad = S.w4a16(M, 256, 16, 32, seed=1)
+    m2 = M_.Module()
+    m2.add_tensor("a", clib.ST_BF16, (M, 256)).add_tensor("b", clib.ST_BF16, (M, 16))
+    with pytest.raises(clib.BackendError) as e:
+        m2.add_a16matmul("a", "b", bad["weight"], bad["scale"], bad["zp"], None, K=256, N=16, weight_bits=4,
+                         q_group_size=32, dq_type=clib.DQ_INT)
+    assert e.value.code == clib.MI_UNSUPPORTED

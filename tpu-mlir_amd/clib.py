@@ -25,7 +25,7 @@ EXPORTS = [
     "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
     "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
     "mi_cast_inference", "mi_cast_launch",
-    "mi_module_create", "mi_module_destroy", "mi_module_add_tensor", "mi_module_add_a16matmul",
+    "mi_module_create", "mi_module_destroy", "mi_module_add_tensor", "mi_module_add_a16matmul", "mi_module_add_a16matmul_dq",
     "mi_module_add_matmul_int8", "mi_module_add_cast", "mi_module_set_tensor", "mi_module_invoke",
     "mi_module_uses_graph", "mi_module_get_tensor",
 ]
@@ -171,6 +171,8 @@ def lib():
         L.mi_module_add_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_int64]
         L.mi_module_add_a16matmul.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(A16WeightDesc), C.c_void_p,
                                               C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi_module_add_a16matmul_dq.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(A16WeightDesc), C.c_int,
+                                                 C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_module_add_matmul_int8.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(ModuleI8Desc)]
         L.mi_module_add_cast.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(CastAttr)]
         L.mi_module_set_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int64]

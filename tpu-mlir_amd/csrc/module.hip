@@ -48,6 +48,7 @@ struct Op {
   // A16MatMul
   mi_a16_weight *w = nullptr;
   int64_t M = 0;
+  int dq_type = MI_DQ_NONE;  // dynamic activation quantization of this A16MatMul
   // quantized MatMul
   std::unique_ptr<DevMem> right, bias, mult, shift, zp;
   int64_t K = 0, N = 0;
@@ -158,12 +159,17 @@ int enqueue_all(mi_module *m) {
     size_t step = 1;
     switch (o.kind) {
     case OP_A16: {
+      if (o.dq_type != MI_DQ_NONE) {  // dynamic activation quantization: its own pair of kernels, one op per launch
+        rc = a16_dq_launch(o.w, o.dq_type, (const uint16_t *)tin.mem->ptr, o.M, (uint16_t *)tout.mem->ptr, nullptr,
+                           m->stream);
+        break;
+      }
       const mi_a16_weight *ws[4];
       uint16_t *ys[4];
       int g = 0;
       while (g < 4 && i + g < n_ops) {
         const Op &c = m->ops[i + g];
-        if (c.kind != OP_A16 || c.in != o.in || c.M != o.M || c.w->K != o.w->K || c.w->bits != o.w->bits ||
+        if (c.kind != OP_A16 || c.dq_type != MI_DQ_NONE || c.in != o.in || c.M != o.M || c.w->K != o.w->K || c.w->bits != o.w->bits ||
             c.w->g != o.w->g || c.w->dtype != o.w->dtype || c.w->chip != o.w->chip)
           break;
         ws[g] = c.w;
@@ -229,7 +235,15 @@ int mi_module_add_tensor(mi_module *m, const char *name, int storage_type, int64
 
 int mi_module_add_a16matmul(mi_module *m, const char *input, const char *output, const mi_a16_weight_desc *desc,
                             const void *weight, const uint16_t *scale, const uint8_t *zp, const float *bias) {
+  return mi_module_add_a16matmul_dq(m, input, output, desc, MI_DQ_NONE, weight, scale, zp, bias);
+}
+
+int mi_module_add_a16matmul_dq(mi_module *m, const char *input, const char *output, const mi_a16_weight_desc *desc,
+                               int dq_type, const void *weight, const uint16_t *scale, const uint8_t *zp,
+                               const float *bias) {
   int in, out, rc;
+  MI_REQUIRE(dq_type == MI_DQ_NONE || dq_type == MI_DQ_INT || dq_type == MI_DQ_F8E4M3 || dq_type == MI_DQ_F4,
+             MI_UNSUPPORTED, "mi_module_add_a16matmul_dq: dq_type must be MI_DQ_NONE, MI_DQ_INT, MI_DQ_F8E4M3 or MI_DQ_F4");
   if ((rc = find(m, input, &in)) || (rc = find(m, output, &out)))
     return rc;
   MI_REQUIRE(desc, MI_BAD_ARGUMENT, "mi_module_add_a16matmul: null descriptor");
@@ -245,9 +259,19 @@ int mi_module_add_a16matmul(mi_module *m, const char *input, const char *output,
   o.in = in;
   o.out = out;
   o.M = M;
+  o.dq_type = dq_type;
   rc = mi_a16_weight_create(&o.w, desc, weight, scale, zp, bias);
   if (rc)
     return rc;
+  if (dq_type != MI_DQ_NONE) {
+    // the shapes and code types the dynamic kernels handle are checked now, not at the first invoke: a launch with
+    // no rows runs every check and nothing else
+    rc = a16_dq_launch(o.w, dq_type, nullptr, 0, nullptr, nullptr, m->stream);
+    if (rc) {
+      mi_a16_weight_destroy(o.w);
+      return rc;
+    }
+  }
   m->ops.push_back(std::move(o));
   drop_graph(m);
   return MI_SUCCESS;

@@ -555,15 +555,15 @@ class Module:
         return self
 
     def add_a16matmul(self, input, output, weight, scale_bits, zp, bias=None, *, K, N, weight_bits, q_group_size,
-                      dtype=DT_BF16, chip=CHIP_BM168X):
+                      dtype=DT_BF16, chip=CHIP_BM168X, dq_type=clib.DQ_NONE):
         weight = np.ascontiguousarray(weight)
         scale_bits = np.ascontiguousarray(scale_bits, dtype=np.uint16)
         zp = np.ascontiguousarray(zp, dtype=np.uint8)
         bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
         desc = A16WeightDesc(K, N, weight_bits, int(weight.dtype == np.int8), q_group_size, dtype, chip)
-        check(clib.lib().mi_module_add_a16matmul(self.handle, input.encode(), output.encode(), C.byref(desc),
-                                                 weight.ctypes.data, scale_bits.ctypes.data, zp.ctypes.data,
-                                                 None if bias is None else bias.ctypes.data))
+        check(clib.lib().mi_module_add_a16matmul_dq(self.handle, input.encode(), output.encode(), C.byref(desc),
+                                                    int(dq_type), weight.ctypes.data, scale_bits.ctypes.data,
+                                                    zp.ctypes.data, None if bias is None else bias.ctypes.data))
         return self
 
     def add_matmul_int8(self, input, output, right, bias=None, *, K, N, right_transpose=False, input_zp=0, right_zp=0,
