@@ -51,11 +51,14 @@ CASES = [  # (M, K, N, right_transpose, relu, per_channel, bias)
     (1, 64, 16, True, False, False, False), (5, 512, 100, False, False, False, True),
     (130, 1024, 200, True, True, False, True), (64, 200, 48, False, False, True, False),   # K % 64 != 0
     (256, 4096, 256, True, False, True, True), (33, 72, 130, True, True, True, True),      # K % 16 != 0
+    (300, 320, 520, False, True, False, True),                                             # ragged 256-tiles
 ]
 
 
+@pytest.mark.parametrize("tile", ["128", "256"])
 @pytest.mark.parametrize("M,K,N,rt,relu,per_channel,bias", CASES)
-def test_f8_matmul_device_level(orc, M, K, N, rt, relu, per_channel, bias):
+def test_f8_matmul_device_level(orc, monkeypatch, M, K, N, rt, relu, per_channel, bias, tile):
+    monkeypatch.setenv("MI_F8_TILE", tile)  # both tile shapes of the ring kernels (K % 64 != 0 takes neither)
     rng = np.random.default_rng(M + K + N)
     a = _codes(rng, (M, K), top=0x58)                       # magnitudes up to 16: sums stay far from fp32 overflow
     b = _codes(rng, (N, K) if rt else (K, N), top=0x58)

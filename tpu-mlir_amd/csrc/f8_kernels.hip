@@ -16,6 +16,8 @@
 // carries a relative error of about 2^-13 where an fp32 FMA chain has 2^-24; after the E4M3 rounding (2^-4 steps) that
 // moves a result across a rounding boundary about once in a thousand outputs.  The reference's own fp32 matmul fixes
 // no summation order either; tests bound the fp32 value and count the differing codes.
+#include <cstdlib>
+
 #include "device_math.cuh"
 #include "internal.h"
 
@@ -40,6 +42,7 @@ struct F8Args {
   float relu_limit;
   int out_kind;         // MI_F8_OUT_*
   double step;          // one scale: (double)(float)(1 / scale)
+  float inv_step;       // one scale: fl32(1 / step)
   const double *scales; // per channel [N], or null
 };
 
@@ -181,17 +184,33 @@ __device__ __forceinline__ void f8_epilogue(const F8Args &a, const f32x16 (&acc)
   }
 }
 
-// E4M3 code of q, round half to even, saturating, NaN -> 0x7f | sign: the hardware conversion on a value clamped to
-// +-448 (it rounds to nearest even, subnormals included), which equals f8e4m3_from_f32 on every input
-__device__ __forceinline__ uint32_t f8_pair_codes(float q0, float q1) {
-  const float c0 = __builtin_fminf(__builtin_fmaxf(q0, -448.0f), 448.0f);  // NaN -> a number; patched below
-  const float c1 = __builtin_fminf(__builtin_fmaxf(q1, -448.0f), 448.0f);
-  uint32_t r = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c0, c1, 0, false) & 0xffffu;
-  if (q0 != q0)
-    r = (r & 0xff00u) | 0x7fu | ((__float_as_uint(q0) >> 24) & 0x80u);
-  if (q1 != q1)
-    r = (r & 0x00ffu) | ((0x7fu | ((__float_as_uint(q1) >> 24) & 0x80u)) << 8);
-  return r;
+// The reference's requantization is E4M3((float)((double)v / step)), Float8.cpp:259-261.  With inv an fp32 number within
+// 2^-23 of 1 / step (per channel: the scale itself rounded to fp32, since step = 1 / scale; one scale: fl32(1 / step)
+// from the host), q0 = v * inv is within 3.01 fp32 ulps of the real quotient v / step and the reference's fp32 quotient
+// within 0.51, so the two can only round to different E4M3 codes when a rounding boundary lies within 4 ulps of q0.
+// The test: q0 shrunk and grown
+// by 2^-20 (8 ulps or more) must convert to the same code; conversion is monotonic, so then every value in between
+// does, the reference's included.  Otherwise (about 6 outputs in 10^5) the division is carried out as written.  The
+// hardware conversion (v_cvt_pk_fp8_f32: round to nearest even, subnormals included) runs on values clamped to
+// +-448, which is the reference's saturation; NaN goes down the slow path.
+// the requantization as the reference writes it; out of line, so that the many unrolled call sites of the fast path
+// do not each carry a copy of two double divisions and the software conversion
+__device__ __attribute__((noinline)) uint32_t f8_requant_exact(float v, double step) {
+  return f8e4m3_from_f32((float)((double)v / step));
+}
+
+__device__ __forceinline__ uint32_t f8_requant_pair(const F8Args &a, float v0, float v1, float inv0, float inv1,
+                                                    int64_t n0, int64_t n1) {
+  const float q0 = __builtin_fminf(__builtin_fmaxf(v0 * inv0, -448.0f), 448.0f);
+  const float q1 = __builtin_fminf(__builtin_fmaxf(v1 * inv1, -448.0f), 448.0f);
+  constexpr float DN = 1.0f - 0x1p-20f, UP = 1.0f + 0x1p-20f;
+  const uint32_t mid = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q0, q1, 0, false) & 0xffffu;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q0 * DN, q1 * DN, 0, false) & 0xffffu;
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q0 * UP, q1 * UP, 0, false) & 0xffffu;
+  if (lo == hi && v0 == v0 && v1 == v1)
+    return mid;
+  const double step0 = a.scales ? 1.0 / a.scales[n0] : a.step, step1 = a.scales ? 1.0 / a.scales[n1] : a.step;
+  return f8_requant_exact(v0, step0) | (f8_requant_exact(v1, step1) << 8);
 }
 
 constexpr int F8_STRIDE = 68;  // dwords per row of an epilogue strip (64 + 4: 16-byte aligned rows, staggered banks)
@@ -212,14 +231,14 @@ __device__ __forceinline__ void f8_strip_epilogue(const F8Args &a, const f32x16 
   const int cc = lane & 3, rsub = lane >> 2;  // 16-column chunk, row within a group of 16 rows
   const int64_t n0 = nb + cc * 16;
   const bool vec_ok = (a.N % 16) == 0 && n0 + 16 <= a.N;
-  float bias[16];
-  double inv[16];  // 1 / step per column
+  float bias[16], inv[16];  // per column: bias, fl32(1 / step)
 #pragma unroll
   for (int e = 0; e < 16; ++e) {
     const int64_t n = (n0 + e) < a.N ? (n0 + e) : (a.N - 1);
     bias[e] = a.bias ? a.bias[n] : 0.0f;
-    inv[e] = 1.0 / (a.scales ? 1.0 / a.scales[n] : a.step);
+    inv[e] = a.scales ? (float)a.scales[n] : a.inv_step;
   }
+  const float relu_hi = (a.do_relu && a.relu_limit > 0.0f) ? a.relu_limit : __builtin_inff();
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     const int row = p * 16 + rsub;
@@ -233,32 +252,23 @@ __device__ __forceinline__ void f8_strip_epilogue(const F8Args &a, const f32x16 
       v[q4 * 4 + 2] = t[2];
       v[q4 * 4 + 3] = t[3];
     }
-    float q[16];
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       v[e] += bias[e];
-      if (a.do_relu) {  // post_relu, lib/Support/Dnnl/DnnlUtils.cpp:15-25
+      if (a.do_relu) {  // post_relu, lib/Support/Dnnl/DnnlUtils.cpp:15-25 (its comparison sends a NaN to 0 as well)
         v[e] = v[e] > 0.0f ? v[e] : 0.0f;
-        if (a.relu_limit > 0.0f && v[e] > a.relu_limit)
-          v[e] = a.relu_limit;
+        v[e] = v[e] > relu_hi ? relu_hi : v[e];
       }
-      // F8E4M3(v, step, true) = E4M3((float)((double)v / step)), Float8.cpp:259-261.  v * (1 / step) is within two
-      // double ulps of that quotient, so the narrowing can come out differently only when the 29 bits it drops sit
-      // next to the halfway pattern; only then is the division carried out.
-      double qd = (double)v[e] * inv[e];
-      const int32_t low = (int32_t)((uint32_t)__double_as_longlong(qd) & 0x1fffffffu);
-      if (low >= 0x10000000 - 4 && low <= 0x10000000 + 4) {
-        const int64_t n = (n0 + e) < a.N ? (n0 + e) : (a.N - 1);
-        qd = (double)v[e] / (a.scales ? 1.0 / a.scales[n] : a.step);
-      }
-      q[e] = (float)qd;
     }
     if (m >= a.M)
       continue;
     uint32_t c2[8];  // two codes each
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
-      c2[e] = f8_pair_codes(q[2 * e], q[2 * e + 1]);
+    for (int e = 0; e < 8; ++e) {
+      const int64_t n_a = (n0 + 2 * e) < a.N ? (n0 + 2 * e) : (a.N - 1);
+      const int64_t n_b = (n0 + 2 * e + 1) < a.N ? (n0 + 2 * e + 1) : (a.N - 1);
+      c2[e] = f8_requant_pair(a, v[2 * e], v[2 * e + 1], inv[2 * e], inv[2 * e + 1], n_a, n_b);
+    }
     const int64_t o = m * a.N + n0;
     if (vec_ok) {
       if (a.acc_out) {
@@ -392,6 +402,150 @@ __global__ __launch_bounds__(256) void f8_gemm_ring_kernel(F8Args a, int tiles_m
   f8_strip_epilogue(a, acc, (float *)f8_lds + wave * (64 * F8_STRIDE), m_base + wm * 64, n_base + wn * 64, lane);
 }
 
+// ---- 256 x 256 outputs per workgroup, 4 waves (2 x 2), each wave 128 x 128 as 4 x 4 blocks of 32 x 32 (256 fp32
+// accumulators per lane).  K advances 64 bytes per stage through a 4-stage LDS ring (32 KiB per stage) filled by
+// direct-to-LDS loads.  One stage = one batch of 16 matrix instructions per wave; the fragment reads of the next stage
+// and the requests of a later one are pinned between them so that they issue in the matrix pipeline's shadow.  One
+// barrier per stage: by then every wave holds the fragments of stage kt in registers (its LDS buffer is free for stage
+// kt + NST) and has received its own share of stage kt + 1.
+constexpr int F8L_M = 256, F8L_N = 256;
+constexpr int F8L_STAGE = (F8L_M + F8L_N) * F8_BK;  // 32 KiB
+constexpr int F8L_NST = 4;
+constexpr int F8_WAITCNT_LGKM0 = 0xC07F;
+
+__global__ __launch_bounds__(256, 1) void f8_gemm_large_kernel(F8Args a, int tiles_m, int tiles_n, int per_xcd) {
+  constexpr int NST = F8L_NST;
+  constexpr int LOADS = F8L_M * (F8_BK / 16) / 256;  // direct-to-LDS instructions per operand, stage and thread: 4
+  constexpr int LPS = 2 * LOADS;
+  extern __shared__ __attribute__((aligned(16))) uint8_t f8_lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int bid = blockIdx.x;
+  const int L = (bid & 7) * per_xcd + (bid >> 3);  // each XCD gets a contiguous run of the tile order
+  if (L >= tiles_m * tiles_n)
+    return;
+  constexpr int GM = 4;
+  const int group = L / (GM * tiles_n);
+  const int gm = (tiles_m - group * GM) < GM ? (tiles_m - group * GM) : GM;
+  const int in_group = L - group * GM * tiles_n;
+  const int tm = group * GM + in_group % gm, tn = in_group / gm;
+  const int64_t m_base = (int64_t)tm * F8L_M, n_base = (int64_t)tn * F8L_N;
+
+  const uint8_t *ga[LOADS], *gb[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int slot = (i * 4 + wave) * 64 + lane;
+    const int row = slot >> 2, pos = slot & 3;
+    const int chunk = pos ^ ((row >> 2) & 3);
+    int64_t ra = m_base + row, rb = n_base + row;
+    ra = ra < a.M ? ra : a.M - 1;  // rows past the matrix re-read the last one; their results are never stored
+    rb = rb < a.N ? rb : a.N - 1;
+    ga[i] = a.A + ra * a.K + chunk * 16;
+    gb[i] = a.B + rb * a.K + chunk * 16;
+  }
+  const int kt_total = (int)(a.K / F8_BK);
+  // request q (0 .. LPS-1) of stage kt: even q operand A, odd q operand B
+  auto issue_one = [&](int kt, int q) {
+    const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 1) * F8_BK;  // past the end: harmless re-load
+    uint8_t *sa = f8_lds + (kt % NST) * F8L_STAGE, *sb = sa + F8L_M * F8_BK;
+    const int li = q >> 1;
+    if (q & 1)
+      __builtin_amdgcn_global_load_lds((f8_gptr_t)(gb[li] + koff), (f8_lptr_t)(sb + (li * 4 + wave) * 1024), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds((f8_gptr_t)(ga[li] + koff), (f8_lptr_t)(sa + (li * 4 + wave) * 1024), 16, 0, 0);
+  };
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[i][j][r] = 0.0f;
+
+  const int frow = lane & 31, kh = lane >> 5;
+  const int f_sw = (frow >> 2) & 3;
+  const int c0 = (kh ^ f_sw) << 4, c1 = ((2 + kh) ^ f_sw) << 4;  // this lane's two chunks of a row, swizzled
+  int a_off[4], b_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    a_off[i] = (wm * 128 + i * 32 + frow) * F8_BK;
+    b_off[i] = F8L_M * F8_BK + (wn * 128 + i * 32 + frow) * F8_BK;
+  }
+  auto read_frag = [&](i32x8 &f, const uint8_t *st, int off) {
+    const u32x4 lo = *(const u32x4 *)(st + off + c0), hi = *(const u32x4 *)(st + off + c1);
+    f = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+  };
+
+  // one stage: wait, barrier, then 16 matrix instructions on the fragments of stage kt with the 8 fragment reads of
+  // stage kt + 1 and the 8 requests of stage kt + NST pinned between them
+  auto stage = [&](const i32x8 (&ca)[4], const i32x8 (&cb)[4], i32x8 (&na)[4], i32x8 (&nb)[4], int kt) {
+    __builtin_amdgcn_s_waitcnt(F8_WAITCNT_LGKM0);                // the fragments of stage kt are in registers
+    __builtin_amdgcn_s_waitcnt(f8_waitcnt_vm((NST - 2) * LPS));  // this thread's share of stage kt + 1 has landed
+    __builtin_amdgcn_s_barrier();
+    const uint8_t *st = f8_lds + ((kt + 1) % NST) * F8L_STAGE;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      const int i = t >> 2, j = t & 3;
+      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ca[i], cb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+      if (t < 4)
+        read_frag(na[t], st, a_off[t]);
+      else if (t < 8)
+        read_frag(nb[t - 4], st, b_off[t - 4]);
+      else
+        issue_one(kt + NST, t - 8);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+#pragma unroll
+  for (int s0 = 0; s0 < NST; ++s0)
+#pragma unroll
+    for (int q = 0; q < LPS; ++q)
+      issue_one(s0, q);
+  i32x8 fa[2][4], fb[2][4];
+  __builtin_amdgcn_s_waitcnt(f8_waitcnt_vm((NST - 1) * LPS));  // stage 0 landed
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    read_frag(fa[0][i], f8_lds, a_off[i]);
+    read_frag(fb[0][i], f8_lds, b_off[i]);
+  }
+  int kt = 0;
+  for (; kt + 1 < kt_total; kt += 2) {
+    stage(fa[0], fb[0], fa[1], fb[1], kt);
+    stage(fa[1], fb[1], fa[0], fb[0], kt + 1);
+  }
+  if (kt < kt_total)
+    stage(fa[0], fb[0], fa[1], fb[1], kt);
+  __builtin_amdgcn_s_waitcnt(f8_waitcnt_vm(0));  // drain the re-loads issued past the end
+  __builtin_amdgcn_s_waitcnt(F8_WAITCNT_LGKM0);
+  __builtin_amdgcn_s_barrier();                  // every wave is done with the ring
+
+  // four 64 x 64 quadrants, written out one by one: inside a loop the accumulator indices would stop being
+  // compile-time constants and the accumulators would move to scratch memory
+  float *strip = (float *)f8_lds + wave * (64 * F8_STRIDE);
+  const int64_t mw = m_base + wm * 128, nw = n_base + wn * 128;
+  {
+    const f32x16 sub[2][2] = {{acc[0][0], acc[0][1]}, {acc[1][0], acc[1][1]}};
+    f8_strip_epilogue(a, sub, strip, mw, nw, lane);
+  }
+  {
+    const f32x16 sub[2][2] = {{acc[0][2], acc[0][3]}, {acc[1][2], acc[1][3]}};
+    f8_strip_epilogue(a, sub, strip, mw, nw + 64, lane);
+  }
+  {
+    const f32x16 sub[2][2] = {{acc[2][0], acc[2][1]}, {acc[3][0], acc[3][1]}};
+    f8_strip_epilogue(a, sub, strip, mw + 64, nw, lane);
+  }
+  {
+    const f32x16 sub[2][2] = {{acc[2][2], acc[2][3]}, {acc[3][2], acc[3][3]}};
+    f8_strip_epilogue(a, sub, strip, mw + 64, nw + 64, lane);
+  }
+}
+
 __global__ void f8_transpose_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t K, int64_t N) {
   // [K, N] -> [N, K], 32 x 32 tiles through LDS
   __shared__ uint8_t tile[32][33];
@@ -439,6 +593,7 @@ int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, con
   a.relu_limit = (float)relu_limit;
   a.out_kind = out_kind;
   a.step = (double)(float)(1 / out_scale);  // MatMul.cpp:613-615 into the float parameter of Float8.cpp:267
+  a.inv_step = (float)(1.0 / a.step);
   a.scales = d_out_scales;
   const int64_t tiles_m = (M + F8_BM - 1) / F8_BM, tiles_n = (N + F8_BN - 1) / F8_BN;
   if ((K % F8_BK) == 0 && tiles_m * tiles_n < (int64_t(1) << 30)) {
@@ -451,7 +606,20 @@ int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, con
                                 f8_ring_lds_bytes(4));
       attr_set = true;
     }
-    if (tiles <= 256)
+    const int64_t tl_m = (M + F8L_M - 1) / F8L_M, tl_n = (N + F8L_N - 1) / F8L_N;
+    const char *e = getenv("MI_F8_TILE");  // development switch: "256" / "128"
+    const bool large = e ? atoi(e) == 256 : tl_m * tl_n >= 144;  // the INT8 kernels' measured crossover
+    if (large) {
+      static bool attr_large = false;
+      if (!attr_large) {
+        (void)hipFuncSetAttribute((const void *)f8_gemm_large_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F8L_NST * F8L_STAGE);
+        attr_large = true;
+      }
+      const int tl = (int)(tl_m * tl_n), pl = (tl + 7) / 8;
+      f8_gemm_large_kernel<<<dim3((unsigned)(pl * 8)), dim3(256), F8L_NST * F8L_STAGE, stream>>>(a, (int)tl_m, (int)tl_n,
+                                                                                              pl);
+    } else if (tiles <= 256)
       f8_gemm_ring_kernel<8><<<dim3((unsigned)(per_xcd * 8)), dim3(256), f8_ring_lds_bytes(8), stream>>>(
           a, (int)tiles_m, (int)tiles_n, per_xcd);
     else
