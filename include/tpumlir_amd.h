@@ -94,7 +94,7 @@ typedef struct mi_a16mm_attr {
   int out_dtype;        /* MI_DT_BF16, or MI_DT_F16 when module::isF16Modes() */
   int chip;             /* MI_CHIP_* */
   int dynamic_quant;    /* MI_DQ_*: module::isDynamicQuantize() and getDqType().  MI_DQ_INT, MI_DQ_F8E4M3 (8-bit
-                         * weights) and MI_DQ_F4 (4-bit weights) with K % 128 == 0 and groups of 64 or k*128 (integer
+                         * weights) and MI_DQ_F4 (4-bit weights) with K % 128 == 0 and groups of 32, 64 or k*128 (integer
                          * codes in 8-bit weights: up to 512) are handled; anything else is MI_UNSUPPORTED */
 } mi_a16mm_attr;
 
@@ -143,7 +143,7 @@ int mi_a16_weight_import(mi_a16_weight **out, const void *blob, size_t size);
  * sums, rescaled and added in group order.  No bias, no relu (the reference applies none on this branch).  Integer
  * types and F4: results are bit-identical to the reference's while its f32 group product is exact (group * imax^2
  * < 2^24 in code units), which is checked.  F8E4M3: exact products, fp32 group sums -- agreement to the fp32 rounding
- * of a group sum, whose order the reference leaves to its matmul library.  K and the group size must be multiples of 64. */
+ * of a group sum, whose order the reference leaves to its matmul library.  K must be a multiple of 64, the group size 32 or a multiple of 64. */
 typedef struct mi_matmul_dq_attr {
   int64_t M, K, N;
   int right_transpose;  /* right operand stored [N, K] instead of [K, N] */

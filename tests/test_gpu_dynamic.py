@@ -33,6 +33,7 @@ CASES = [  # (M, K, N, g, bias)
     (1, 512, 48, 64, False), (5, 1024, 100, 128, True), (16, 4096, 64, 128, False), (33, 2048, 40, 256, True),
     (3, 256, 16, 64, True), (2, 1024, 24, 1024, False), (1, 4096, 4096, 128, False), (8, 11008, 128, 128, True),
     (20, 17408, 32, 128, False),  # 136 groups: more than one LDS chunk of terms
+    (3, 256, 16, 32, True), (17, 4608, 48, 32, False),  # 32-wide groups (144 of them: more than one chunk)
 ]
 
 
@@ -48,7 +49,7 @@ def test_dynamic_int_device_level(orc, M, K, N, g, bias):
 
 W8_CASES = [  # (M, K, N, g, bias): 8-bit weights, imax 127
     (1, 512, 48, 64, False), (5, 1024, 100, 128, True), (16, 2048, 64, 256, False), (33, 1024, 40, 512, True),
-    (1, 4096, 1024, 128, False),
+    (1, 4096, 1024, 128, False), (5, 512, 40, 32, True),
 ]
 
 
@@ -96,7 +97,7 @@ def test_dynamic_int_operator_level(orc):
 
 def test_dynamic_int_rejects_what_it_does_not_handle():
     import torch
-    for cfg, bits in ((S.w4a16(1, 256, 16, 32, seed=1), 4),        # 32-wide groups
+    for cfg, bits in ((S.w4a16(1, 192, 16, 64, seed=1), 4),        # K is not a multiple of 128
                       (S.w8a16(1, 1024, 16, 1024, seed=1), 8)):    # 8-bit group too long to stay exact
         w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=cfg["K"], N=16, weight_bits=bits,
                          q_group_size=cfg["g"])
@@ -112,6 +113,7 @@ MM_CASES = [  # (M, K, N, g, right_transpose, dq_type)
     (1, 128, 16, 64, True, "DQ_INT8"), (5, 512, 100, 128, False, "DQ_INT8"), (37, 1024, 70, 256, True, "DQ_INT8"),
     (16, 256, 48, -1, False, "DQ_INT8"), (20, 2048, 33, 64, False, "DQ_INT4"), (128, 128, 128, 128, True, "DQ_INT4"),
     (3, 8704, 24, 64, True, "DQ_INT8"),  # 136 groups: more than one LDS chunk of terms
+    (5, 256, 20, 32, True, "DQ_INT8"), (9, 4224, 40, 32, False, "DQ_INT4"),  # 32-wide groups
 ]
 
 
@@ -180,7 +182,7 @@ def _device_typed(cfg, dq_type):
 F4_CASES = [  # (M, K, N, g, bias, zero points)
     (1, 512, 48, 64, False, False), (5, 1024, 100, 128, True, False), (16, 4096, 64, 128, False, True),
     (33, 2048, 40, 256, True, True), (3, 256, 16, 64, True, True), (1, 4096, 4096, 128, False, False),
-    (20, 17408, 32, 128, False, False),
+    (20, 17408, 32, 128, False, False), (4, 512, 32, 32, True, True), (1, 256, 16, 32, False, False),
 ]
 
 
@@ -224,7 +226,7 @@ def test_dynamic_f4_ties_zero_rows_and_extremes(orc):
 
 
 F8_CASES = [(1, 512, 48, 64, False), (5, 1024, 100, 128, True), (16, 2048, 64, 256, False), (33, 1024, 40, 512, True),
-            (1, 4096, 1024, 128, False), (4, 2048, 24, 2048, False)]
+            (1, 4096, 1024, 128, False), (4, 2048, 24, 2048, False), (4, 512, 24, 32, True)]
 
 
 @pytest.mark.parametrize("M,K,N,g,bias", F8_CASES)
@@ -349,7 +351,7 @@ MM_FLOAT_CASES = [  # (M, K, N, g, right_transpose, dq_type)
     (1, 128, 16, 64, True, "DQ_F4"), (5, 512, 100, 128, False, "DQ_F4"), (37, 1024, 70, 256, True, "DQ_F4"),
     (3, 8704, 24, 64, True, "DQ_F4"),
     (1, 128, 16, 64, True, "DQ_F8E4M3"), (5, 512, 100, 128, False, "DQ_F8E4M3"), (37, 1024, 70, 256, True, "DQ_F8E4M3"),
-    (16, 256, 48, -1, False, "DQ_F8E4M3"),
+    (16, 256, 48, -1, False, "DQ_F8E4M3"), (5, 256, 20, 32, True, "DQ_F4"), (5, 256, 20, 32, False, "DQ_F8E4M3"),
 ]
 
 

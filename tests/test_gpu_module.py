@@ -142,10 +142,10 @@ def test_dynamic_quant_a16matmul_in_a_module(orc, dq, bits):
         assert np.array_equal(m.get_tensor("h"), h), rep
         assert np.array_equal(m.get_tensor("y"), y), rep
     # shapes the dynamic kernels do not handle are refused when the op is added
-    bad = S.w4a16(M, 256, 16, 32, seed=1)
+    bad = S.w4a16(M, 192, 16, 64, seed=1)  # K is not a multiple of 128
     m2 = M_.Module()
-    m2.add_tensor("a", clib.ST_BF16, (M, 256)).add_tensor("b", clib.ST_BF16, (M, 16))
+    m2.add_tensor("a", clib.ST_BF16, (M, 192)).add_tensor("b", clib.ST_BF16, (M, 16))
     with pytest.raises(clib.BackendError) as e:
-        m2.add_a16matmul("a", "b", bad["weight"], bad["scale"], bad["zp"], None, K=256, N=16, weight_bits=4,
-                         q_group_size=32, dq_type=clib.DQ_INT)
+        m2.add_a16matmul("a", "b", bad["weight"], bad["scale"], bad["zp"], None, K=192, N=16, weight_bits=4,
+                         q_group_size=64, dq_type=clib.DQ_INT)
     assert e.value.code == clib.MI_UNSUPPORTED

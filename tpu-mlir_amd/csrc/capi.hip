@@ -393,10 +393,10 @@ int mi_a16mm_init(const mi_a16mm_attr *attr, mi_infer_param *p) {
     MI_REQUIRE((dq != MI_DQ_F8E4M3 || attr->weight_bits == 8) && (dq != MI_DQ_F4 || attr->weight_bits == 4),
                MI_UNSUPPORTED, "mi_a16mm_init: F8E4M3 needs 8-bit and F4 needs 4-bit weights");
     MI_REQUIRE(attr->q_group_size > 0 && attr->K % 128 == 0 &&
-                   (attr->q_group_size == 64 || attr->q_group_size % 128 == 0) &&
+                   (attr->q_group_size == 32 || attr->q_group_size == 64 || attr->q_group_size % 128 == 0) &&
                    (dq != MI_DQ_INT || attr->weight_bits == 4 || attr->q_group_size <= 512),
                MI_UNSUPPORTED,
-               "mi_a16mm_init: dynamic quantization is handled for K % 128 == 0 and groups of 64 or k*128 (integer "
+               "mi_a16mm_init: dynamic quantization is handled for K % 128 == 0 and groups of 32, 64 or k*128 (integer "
                "codes with 8-bit weights: up to 512, where the reference's f32 group product stops being exact)");
   }
   MI_REQUIRE(attr->w_transpose, MI_UNSUPPORTED, "mi_a16mm_init: only w_transpose weights ([N,K]) are handled");
@@ -1083,8 +1083,8 @@ int mi_matmul_dq_inference(const mi_matmul_dq_attr *a, mi_infer_param *p) {
   MI_REQUIRE(a->out_dtype == MI_DT_BF16 || a->out_dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_matmul_dq_inference: out_dtype");
   const int64_t g = a->q_group_size == -1 ? a->K : a->q_group_size;
   MI_REQUIRE(g > 0, MI_BAD_ARGUMENT, "mi_matmul_dq_inference: dynamic quantization needs a group size");
-  MI_REQUIRE((a->K % 64) == 0 && (g % 64) == 0 && (a->K % g) == 0, MI_UNSUPPORTED,
-             "mi_matmul_dq_inference: K and the group size must be multiples of 64");
+  MI_REQUIRE((a->K % 64) == 0 && (g == 32 || (g % 64) == 0) && (a->K % g) == 0, MI_UNSUPPORTED,
+             "mi_matmul_dq_inference: K must be a multiple of 64 and the group size 32 or a multiple of 64");
   if (a->M == 0)
     return MI_SUCCESS;
   MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_matmul_dq_inference: no GPU visible");

@@ -157,7 +157,7 @@ struct DqArgs {
   int G;
   int unit_tiles;   // weight tiles per unit of work.  4-bit: g / 128 when g >= 128, else 1 (the unit then holds two
                     // groups); 8-bit: g / 64
-  int unit_groups;  // groups per unit: 1, or 2 for 4-bit weights with g == 64
+  int unit_groups;  // groups per unit: 1; 4-bit weights: 2 with g == 64, 4 with g == 32; 8-bit weights: 2 with g == 32
   int chip;
 };
 
@@ -181,6 +181,19 @@ __device__ __forceinline__ bf16x8 f8x8_as_bf16(uint32_t lo, uint32_t hi) {
                    __builtin_amdgcn_perm(__float_as_uint(p2[1]), __float_as_uint(p2[0]), 0x07060302u),
                    __builtin_amdgcn_perm(__float_as_uint(p3[1]), __float_as_uint(p3[0]), 0x07060302u)};
   return __builtin_bit_cast(bf16x8, r);
+}
+
+// acc[which] += A x B on the fp8 instruction, which wave-uniform but not a compile-time constant: every accumulator
+// is named, so none of them is indexed
+__device__ __forceinline__ void acc_f4_add(f32x4 (&acc)[4], int which, long av, long bv) {
+  if (which == 0)
+    acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(av, bv, acc[0], 0, 0, 0);
+  else if (which == 1)
+    acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(av, bv, acc[1], 0, 0, 0);
+  else if (which == 2)
+    acc[2] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(av, bv, acc[2], 0, 0, 0);
+  else
+    acc[3] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(av, bv, acc[3], 0, 0, 0);
 }
 
 template <int DT, int BITS, int FLAV>
@@ -211,7 +224,7 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
   for (int u0 = 0; u0 < units; u0 += chunk_units) {
     const int u1 = (u0 + chunk_units) < units ? (u0 + chunk_units) : units;
     for (int u = u0 + wave; u < u1; u += DQ_WAVES) {
-      acc_t acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+      acc_t acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};  // one per group of the unit
       for (int t = 0; t < a.unit_tiles; ++t) {
         const int64_t kt = (int64_t)u * a.unit_tiles + t;
         const u32x4 w = wq[kt * 64];
@@ -220,8 +233,12 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
           const u32x4 a0 = aq[kt * 64];
           acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(a0[0], a0[1]), f8x8_as_bf16(w[0], w[1]), acc[0], 0,
                                                            0, 0);
-          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(a0[2], a0[3]), f8x8_as_bf16(w[2], w[3]), acc[0], 0,
-                                                           0, 0);
+          if (a.unit_groups == 2)  // 32-wide groups: the tile's second 32 k are the next group
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(a0[2], a0[3]), f8x8_as_bf16(w[2], w[3]), acc[1],
+                                                             0, 0, 0);
+          else
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(a0[2], a0[3]), f8x8_as_bf16(w[2], w[3]), acc[0],
+                                                             0, 0, 0);
         } else if constexpr (FLAV == FLAV_F4) {
           const u32x4 a0 = aq[kt * 128], a1 = aq[kt * 128 + 64];
           uint32_t lo[4], hi[4];
@@ -231,18 +248,24 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
             hi[j] = f4x4_as_f8((w[j] >> 4) & 0x0F0F0F0Fu);
           }
           // dword j of the lane is k 32 j + 8 kq .. + 8; the activation bytes were written in the same slot order
+          // the four 32-wide blocks of the tile go to the accumulator of their group: one group (g >= 128), two
+          // (g = 64) or four (g = 32) per tile
+          const int s1 = a.unit_groups == 4 ? 1 : 0, s2 = a.unit_groups == 4 ? 2 : a.unit_groups == 2 ? 1 : 0;
+          const int s3 = a.unit_groups == 4 ? 3 : s2;
           acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(a0[0], a0[1]), pack64(lo[0], hi[0]), acc[0], 0, 0, 0);
-          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(a0[2], a0[3]), pack64(lo[1], hi[1]), acc[0], 0, 0, 0);
-          const int second = a.unit_groups == 2 ? 1 : 0;  // with 64-wide groups k 64..127 is the next group
-          acc[second] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(a1[0], a1[1]), pack64(lo[2], hi[2]),
-                                                                   acc[second], 0, 0, 0);
-          acc[second] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(a1[2], a1[3]), pack64(lo[3], hi[3]),
-                                                                   acc[second], 0, 0, 0);
+          acc_f4_add(acc, s1, pack64(a0[2], a0[3]), pack64(lo[1], hi[1]));
+          acc_f4_add(acc, s2, pack64(a1[0], a1[1]), pack64(lo[2], hi[2]));
+          acc_f4_add(acc, s3, pack64(a1[2], a1[3]), pack64(lo[3], hi[3]));
         } else if constexpr (BITS == 8) {
           const u32x4 a0 = aq[kt * 64];
           const u32x4 ws = {w[0] ^ 0x80808080u, w[1] ^ 0x80808080u, w[2] ^ 0x80808080u, w[3] ^ 0x80808080u};
-          acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0), __builtin_bit_cast(i32x4, ws),
-                                                         acc[0], 0, 0, 0);
+          if (a.unit_groups == 2) {  // 32-wide groups: two K = 32 instructions, one per half of the tile
+            acc[0] = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(a0[0], a0[1]), pack64(ws[0], ws[1]), acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(a0[2], a0[3]), pack64(ws[2], ws[3]), acc[1], 0, 0, 0);
+          } else {
+            acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0), __builtin_bit_cast(i32x4, ws),
+                                                           acc[0], 0, 0, 0);
+          }
         } else {
           const u32x4 a0 = aq[kt * 128], a1 = aq[kt * 128 + 64];
           int lo[4], hi[4];
@@ -251,17 +274,25 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
             unpack_bytes(w[j], lo[j], hi[j]);
           const i32x4 b0 = {lo[0], hi[0], lo[1], hi[1]}, b1 = {lo[2], hi[2], lo[3], hi[3]};
           // k 0..63 of the tile, then k 64..127; with 64-wide groups these are two groups
-          acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0), b0, acc[0], 0, 0, 0);
-          if (a.unit_groups == 2)
-            acc[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1), b1, acc[1], 0, 0, 0);
-          else
-            acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1), b1, acc[0], 0, 0, 0);
+          if (a.unit_groups == 4) {  // 32-wide groups: four K = 32 instructions, one per 32-wide block of the tile
+            acc[0] = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(a0[0], a0[1]), pack64(lo[0], hi[0]), acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(a0[2], a0[3]), pack64(lo[1], hi[1]), acc[1], 0, 0, 0);
+            acc[2] = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(a1[0], a1[1]), pack64(lo[2], hi[2]), acc[2], 0, 0, 0);
+            acc[3] = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(a1[2], a1[3]), pack64(lo[3], hi[3]), acc[3], 0, 0, 0);
+          } else {
+            acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0), b0, acc[0], 0, 0, 0);
+            if (a.unit_groups == 2)
+              acc[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1), b1, acc[1], 0, 0, 0);
+            else
+              acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1), b1, acc[0], 0, 0, 0);
+          }
         }
       }
-      for (int h = 0; h < a.unit_groups; ++h) {
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {  // unrolled: the accumulator index stays a compile-time constant
         const int gi = u * a.unit_groups + h;
-        if (gi >= a.G)
-          break;
+        if (h >= a.unit_groups || gi >= a.G)
+          continue;
         float sc;
         int zp;  // what multiplies sum(codes)
         if constexpr (BITS == 4) {
@@ -342,7 +373,8 @@ struct Dq2Args {
   float *y32;
   int64_t M, N;
   int64_t k_tiles;
-  int G, unit_tiles;  // tiles of 64 per group
+  int G, unit_tiles;  // tiles of 64 per unit of work
+  int unit_groups;    // groups per unit: 1, or 2 with 32-wide groups
 };
 
 template <int DT, int FLAV>
@@ -360,33 +392,56 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq2_gemm_kernel(Dq2Args a) {
   float out = 0.0f;
   const int64_t n_out = nb * 16 + (tid & 15), m_out = mb * 16 + (tid >> 4);
   const bool owns = tid < 256 && n_out < a.N && m_out < a.M;
-  for (int g0 = 0; g0 < a.G; g0 += DQ_CHUNK) {
-    const int g1 = (g0 + DQ_CHUNK) < a.G ? (g0 + DQ_CHUNK) : a.G;
-    for (int gi = g0 + wave; gi < g1; gi += DQ_WAVES) {
-      acc_t acc = {0, 0, 0, 0};
+  const int units = (a.G + a.unit_groups - 1) / a.unit_groups;
+  const int chunk_units = DQ_CHUNK / a.unit_groups;
+  for (int u0 = 0; u0 < units; u0 += chunk_units) {
+    const int u1 = (u0 + chunk_units) < units ? (u0 + chunk_units) : units;
+    const int g0 = u0 * a.unit_groups, g1 = (u1 * a.unit_groups) < a.G ? (u1 * a.unit_groups) : a.G;
+    for (int u = u0 + wave; u < u1; u += DQ_WAVES) {
+      acc_t acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
       for (int t = 0; t < a.unit_tiles; ++t) {
-        const int64_t kt = (int64_t)gi * a.unit_tiles + t;
+        const int64_t kt = (int64_t)u * a.unit_tiles + t;
         const u32x4 l = al[kt * 64], r = ar[kt * 64];
         if constexpr (FLAV == FLAV_INT) {
-          acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, l), __builtin_bit_cast(i32x4, r), acc, 0, 0,
-                                                      0);
+          if (a.unit_groups == 2) {  // 32-wide groups: one K = 32 instruction per half of the tile
+            acc[0] = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(l[0], l[1]), pack64(r[0], r[1]), acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(l[2], l[3]), pack64(r[2], r[3]), acc[1], 0, 0, 0);
+          } else {
+            acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, l), __builtin_bit_cast(i32x4, r),
+                                                           acc[0], 0, 0, 0);
+          }
         } else if constexpr (FLAV == FLAV_F4) {  // E2M1 values as E4M3 bytes: exact sums on the fp8 instruction
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(l[0], l[1]), pack64(r[0], r[1]), acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(l[2], l[3]), pack64(r[2], r[3]), acc, 0, 0, 0);
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(l[0], l[1]), pack64(r[0], r[1]), acc[0], 0, 0, 0);
+          if (a.unit_groups == 2)
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(l[2], l[3]), pack64(r[2], r[3]), acc[1], 0, 0, 0);
+          else
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(pack64(l[2], l[3]), pack64(r[2], r[3]), acc[0], 0, 0, 0);
         } else {                                 // E4M3: exact products, fp32 sums (see f8x8_as_bf16)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(l[0], l[1]), f8x8_as_bf16(r[0], r[1]), acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(l[2], l[3]), f8x8_as_bf16(r[2], r[3]), acc, 0, 0, 0);
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(l[0], l[1]), f8x8_as_bf16(r[0], r[1]), acc[0], 0,
+                                                           0, 0);
+          if (a.unit_groups == 2)
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(l[2], l[3]), f8x8_as_bf16(r[2], r[3]), acc[1],
+                                                             0, 0, 0);
+          else
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f8x8_as_bf16(l[2], l[3]), f8x8_as_bf16(r[2], r[3]), acc[0],
+                                                             0, 0, 0);
         }
       }
-      const f32x4 l4 = *(const f32x4 *)(asl + (int64_t)gi * 16);
-      const float r1 = asr[(int64_t)gi * 16];
-      float *dst = terms + (size_t)(gi - g0) * 256;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float t = (float)acc[r];  // integer codes: below 2^24 (checked on the host), exact
-        t = t * l4[r];            // MatMul.cpp:577-581, left to right
-        t = t * r1;
-        dst[(4 * kq + r) * 16 + col] = t;
+      for (int h = 0; h < 2; ++h) {
+        const int gi = u * a.unit_groups + h;
+        if (h >= a.unit_groups || gi >= a.G)
+          continue;
+        const f32x4 l4 = *(const f32x4 *)(asl + (int64_t)gi * 16);
+        const float r1 = asr[(int64_t)gi * 16];
+        float *dst = terms + (size_t)(gi - g0) * 256;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float t = (float)acc[h][r];  // integer codes: below 2^24 (checked on the host), exact
+          t = t * l4[r];               // MatMul.cpp:577-581, left to right
+          t = t * r1;
+          dst[(4 * kq + r) * 16 + col] = t;
+        }
       }
     }
     __syncthreads();
@@ -423,8 +478,9 @@ int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_
   MI_REQUIRE(dtype == MI_DT_BF16 || dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_matmul_dq_launch: dtype");
   const int64_t g = q_group_size == -1 ? K : q_group_size;  // MatMul.cpp:465-466
   MI_REQUIRE(g > 0, MI_BAD_ARGUMENT, "mi_matmul_dq_launch: dynamic quantization needs a group size");
-  MI_REQUIRE((K % 64) == 0 && (g % 64) == 0 && (K % g) == 0, MI_UNSUPPORTED,
-             "mi_matmul_dq_launch: K and the group size must be multiples of 64, K a multiple of the group size");
+  MI_REQUIRE((K % 64) == 0 && (g == 32 || (g % 64) == 0) && (K % g) == 0, MI_UNSUPPORTED,
+             "mi_matmul_dq_launch: K must be a multiple of 64, the group size 32 or a multiple of 64, K a multiple of "
+             "the group size");
   MI_REQUIRE(g * peak < (1 << 24), MI_UNSUPPORTED,
              "mi_matmul_dq_launch: group too long for the group sums to stay exact in the reference's f32 product");
   if (M == 0)
@@ -463,7 +519,8 @@ int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_
   a.N = N;
   a.k_tiles = k_tiles;
   a.G = G;
-  a.unit_tiles = (int)(g / 64);
+  a.unit_tiles = g >= 64 ? (int)(g / 64) : 1;
+  a.unit_groups = g == 32 ? 2 : 1;
   const int chunk_groups = G < DQ_CHUNK ? G : DQ_CHUNK;
   const size_t lds_bytes = (size_t)(chunk_groups + 1) * 1024;
   dim3 grid((unsigned)n_blocks, (unsigned)m_blocks);
@@ -513,8 +570,8 @@ int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int6
   // A16MatMul.cpp:51-91: F8E4M3 codes are read from 8-bit, F4 codes from 4-bit weights
   MI_REQUIRE(dq_type == MI_DQ_INT || (dq_type == MI_DQ_F8E4M3 && bits == 8) || (dq_type == MI_DQ_F4 && bits == 4),
              MI_UNSUPPORTED, "mi_a16mm_dq_launch: dq_type must be MI_DQ_INT, MI_DQ_F8E4M3 (8-bit weights) or MI_DQ_F4 (4-bit)");
-  MI_REQUIRE((w->K % 128) == 0 && (g == 64 || g % 128 == 0), MI_UNSUPPORTED,
-             "mi_a16mm_dq_launch: K must be a multiple of 128 and the group size 64 or a multiple of 128");
+  MI_REQUIRE((w->K % 128) == 0 && (g == 32 || g == 64 || g % 128 == 0), MI_UNSUPPORTED,
+             "mi_a16mm_dq_launch: K must be a multiple of 128 and the group size 32, 64 or a multiple of 128");
   // imax: (1 << (weight_bits - 1)) - 1, get_f8e4m3_max() or get_f4e2m1_max(), A16MatMul.cpp:51-61.  The reference's f32
   // group product is exact only while the sums of integer codes stay below 2^24; E2M1 products are quarter units up
   // to 36 (15 with a zero point), E4M3 sums are rounded by the reference as well
@@ -561,8 +618,8 @@ int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int6
   a.N = w->N;
   a.k_tiles = w->k_tiles;
   a.G = G;
-  a.unit_tiles = bits == 4 ? (g >= 128 ? g / 128 : 1) : g / 64;
-  a.unit_groups = (bits == 4 && g == 64) ? 2 : 1;
+  a.unit_tiles = bits == 4 ? (g >= 128 ? g / 128 : 1) : (g >= 64 ? g / 64 : 1);
+  a.unit_groups = bits == 4 ? (g == 32 ? 4 : g == 64 ? 2 : 1) : (g == 32 ? 2 : 1);
   a.chip = w->chip;
   const int chunk_groups = G < DQ_CHUNK ? G : DQ_CHUNK;
   const size_t lds_bytes = (size_t)(chunk_groups + 1) * 1024;

@@ -40,8 +40,8 @@ int stream_workspace(hipStream_t st, int purpose, size_t bytes, bool zeroed, voi
     }
     const size_t want = (bytes + 255) & ~(size_t)255;
     MI_HIP(hipMalloc(&b.ptr, want));
-    if (zeroed)
-      MI_HIP(hipMemset(b.ptr, 0, want));
+    if (zeroed)  // on the user's stream (which is not being captured here): ordered before whatever it runs next
+      MI_HIP(hipMemsetAsync(b.ptr, 0, want, st));
     b.bytes = want;
   }
   *out = b.ptr;
