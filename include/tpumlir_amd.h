@@ -168,22 +168,32 @@ int mi_matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int rig
  * -- about one in a thousand -- lands on the neighbouring E4M3 code. */
 enum { MI_F8_OUT_CODES = 0 /* uint8 E4M3 codes */, MI_F8_OUT_F32 = 1 /* the E4M3 values as f32 */,
        MI_F8_OUT_BF16 = 2, MI_F8_OUT_F16 = 3 /* the same values in a 16-bit type (exact) */ };
+/* Operand type.  MI_F8_E5M2: the operands hold E5M2 values and the output follows the arms of MatMul.cpp:630-635 --
+ * F8E5M2(v, 1.0, true) for an E5M2 result (lib/Support/Float8.cpp:134-138,263-265: round half to even, overflow to
+ * the infinity 0x7c, no saturation whatever the flag says), F16(v) / BF16(v) for a 16-bit result; no scales. */
+enum { MI_F8_E4M3 = 0, MI_F8_E5M2 = 1 };
 typedef struct mi_f8mm_attr {
   int64_t M, K, N;        /* parseParam(): batch == 1 */
   int right_transpose;    /* right stored [N, K] */
   int do_relu;
   double relu_limit;
-  const double *out_scales; /* getOutScales() */
+  const double *out_scales; /* getOutScales(); not read for MI_F8_E5M2 */
   int n_out_scales;       /* 1 or N */
+  int f8_type;            /* MI_F8_E4M3 / MI_F8_E5M2: the storage type of the operands and of the output */
 } mi_f8mm_attr;
-/* inputs = {left [M,K], right, bias [N] | NULL}: f32 arrays holding E4M3 values (anything else: MI_UNSUPPORTED);
- * outputs[0] [M,N] receives the requantized E4M3 values as f32. */
+/* inputs = {left [M,K], right, bias [N] | NULL}: f32 arrays holding E4M3 (E5M2) values (anything else:
+ * MI_UNSUPPORTED); outputs[0] [M,N] receives the requantized E4M3 (E5M2) values as f32. */
 int mi_f8mm_inference(const mi_f8mm_attr *attr, mi_infer_param *p);
 /* device level: E4M3 codes in HBM; d_out_scales: per-channel scales [N] (doubles, device) or NULL for out_scale;
  * d_acc_f32 (may be NULL) receives the fp32 value before requantization. */
 int mi_f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, const float *d_bias, int64_t M,
                    int64_t K, int64_t N, int do_relu, double relu_limit, double out_scale, const double *d_out_scales,
                    int out_kind, void *d_out, float *d_acc_f32, void *stream);
+/* the same on E5M2 codes: out_kind MI_F8_OUT_CODES (E5M2 codes), MI_F8_OUT_F32 (their values), MI_F8_OUT_BF16 /
+ * MI_F8_OUT_F16 (the BF16() / F16() rounding of the fp32 value, MatMul.cpp:632-635) */
+int mi_f8mm_e5m2_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, const float *d_bias, int64_t M,
+                        int64_t K, int64_t N, int do_relu, double relu_limit, int out_kind, void *d_out,
+                        float *d_acc_f32, void *stream);
 
 /* ---- weight producers (the compile-time side of tpu.A16MatMul), computed on the GPU, host arrays in and out ---- */
 typedef struct mi_a16_quant_desc {

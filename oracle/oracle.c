@@ -601,6 +601,75 @@ float orc_f8e4m3_to_f32(uint8_t src) {
   return out;
 }
 
+/* lib/Support/Float8.cpp:46-131 with the E5M2 constants (bias 15, 3 significand bits, infinities at 0x7c) as
+ * f32_to_f8e5m2 (:134-138) calls it: ROUNDING_HALF_TO_EVEN and saturate forced to false whatever the caller asks, so
+ * anything that rounds to 2^16 or beyond, and the infinities, become 0x7c */
+uint8_t orc_f32_to_f8e5m2(float src) {
+  uint32_t bits;
+  memcpy(&bits, &src, 4);
+  const uint32_t sign = bits >> 31, exp = (bits >> 23) & 0xff, frac = bits & 0x7fffff;
+  uint8_t res = 0;
+  if (exp > 127 - 15 && exp < 0xff) { /* :74-96 */
+    uint32_t tmp = (uint32_t)f8_shift_rne((long long)bits, 21);
+    tmp <<= 21;
+    const uint32_t e = ((tmp >> 23) & 0xff) - 127 + 15;
+    const uint32_t f = (tmp >> 21) & 0x3;
+    if (e >= 0x1f)
+      res = 0x7c;
+    else
+      res = (uint8_t)((e << 2) | f);
+  } else if (exp > 0 && exp <= 127 - 15) { /* :97-106: units of 2^-16 */
+    int32_t mant = (int32_t)(frac + (1u << 23));
+    mant = sign ? -mant : mant;
+    const int shift = (127 - 15 + 1) - (int)exp + 21;
+    mant = (int32_t)f8_shift_rne(mant, shift);
+    mant = sign ? -mant : mant;
+    res = (uint8_t)(mant & 0x7f);
+  } else if (exp == 0xff && frac != 0) { /* :107-113: 0x7e | the top two fraction bits of 0x7fffffff */
+    res = 0x7f;
+  } else if (exp == 0xff) { /* :117-124 */
+    res = 0x7c;
+  }
+  return (uint8_t)(res | (sign << 7));
+}
+
+/* lib/Support/Float8.cpp:140-186 with the E5M2 constants */
+float orc_f8e5m2_to_f32(uint8_t src) {
+  const uint32_t sign = (src >> 7) & 1;
+  uint32_t exponent = (src >> 2) & 0x1f;
+  uint32_t mantissa = (uint32_t)(src & 0x3) << 21;
+  if (exponent == 0x1f) {
+    exponent = 0xff;
+    if (mantissa != 0)
+      mantissa = 0x7fffff | (sign << 23);
+  } else if (exponent == 0) {
+    if (mantissa != 0) {
+      uint32_t msb;
+      exponent = 127 - 14;
+      do {
+        msb = mantissa & 0x400000;
+        mantissa <<= 1;
+        exponent--;
+      } while (msb == 0);
+      mantissa &= 0x7fffff;
+    }
+  } else {
+    exponent += 127 - 15;
+  }
+  const uint32_t bits = (sign << 31) | (exponent << 23) | mantissa;
+  float out;
+  memcpy(&out, &bits, 4);
+  return out;
+}
+void orc_f32_to_f8e5m2_n(const float *src, int64_t n, uint8_t *dst) {
+  for (int64_t i = 0; i < n; i++)
+    dst[i] = orc_f32_to_f8e5m2(src[i]);
+}
+void orc_f8e5m2_to_f32_n(const uint8_t *src, int64_t n, float *dst) {
+  for (int64_t i = 0; i < n; i++)
+    dst[i] = orc_f8e5m2_to_f32(src[i]);
+}
+
 /* lib/Support/Float4.cpp:7-24: the sixteen E2M1 values; the first nearest one in table order wins, so ties go to the
  * smaller magnitude, a negative input nearest to zero gives +0, and NaN / infinities give code 0 */
 static const float ORC_F4_TABLE[16] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f,
@@ -937,6 +1006,41 @@ int orc_matmul_f8(const float *left, const float *right, const float *bias, int6
       const double step = 1.0 / scales[i % N];
       output[i] = orc_f8e4m3_to_f32(orc_f32_to_f8e4m3((float)((double)output[i] / step), 1));
     }
+  }
+  return 0;
+}
+
+/* tpu.MatMul with F8E5M2 operands: the same f32 product, then the output arm that the storage type selects
+ * (MatMul.cpp:630-635): ORC_F8E5M2_OUT_E5M2 = F8E5M2(v, 1.0, true) (the division by the step 1.0 changes nothing),
+ * ORC_F8E5M2_OUT_F16 = F16(v), ORC_F8E5M2_OUT_BF16 = BF16(v).  The output holds the rounded values. */
+int orc_matmul_f8e5m2(const float *left, const float *right, const float *bias, int64_t M, int64_t K, int64_t N,
+                      int right_transpose, int do_relu, double relu_limit, int out_arm, float *output,
+                      float *acc_out) {
+  if (!left || !right || !output || M <= 0 || K <= 0 || N <= 0 || out_arm < 0 || out_arm > 2)
+    return 1;
+  float *r_kn = (float *)malloc(sizeof(float) * (size_t)(K * N));
+  if (!r_kn)
+    return 1;
+  if (right_transpose)
+    orc_hw_transpose(r_kn, right, N, K);
+  else
+    memcpy(r_kn, right, sizeof(float) * (size_t)(K * N));
+  orc_sgemm_f64acc(left, r_kn, bias, output, M, K, N);
+  free(r_kn);
+  if (do_relu)
+    for (int64_t i = 0; i < M * N; i++) {
+      float v = output[i] > 0.0f ? output[i] : 0.0f;
+      if (relu_limit > 0.0 && v > (float)relu_limit)
+        v = (float)relu_limit;
+      output[i] = v;
+    }
+  if (acc_out)
+    memcpy(acc_out, output, sizeof(float) * (size_t)(M * N));
+  for (int64_t i = 0; i < M * N; i++) {
+    if (out_arm == ORC_F8E5M2_OUT_E5M2)
+      output[i] = orc_f8e5m2_to_f32(orc_f32_to_f8e5m2((float)((double)output[i] / 1.0)));
+    else
+      output[i] = round_out(output[i], out_arm == ORC_F8E5M2_OUT_F16 ? ORC_OUT_F16 : ORC_OUT_BF16, 0);
   }
   return 0;
 }

@@ -37,6 +37,10 @@
  *   orc_matmul_f8                float64 product of torch-decoded operands; the requantization against torch's
  *                                float8 cast of the same quotient; per-channel vs one-scale step (float-narrowed)
  *                                on a case built to tell them apart (tests/test_oracle_float_codes.py)
+ *   orc_f32_to_f8e5m2 / orc_f8e5m2_to_f32   torch.float8_e5m2 and numpy float16 (an E5M2 code is the top byte of an
+ *                                IEEE half) on all codes, all bf16 patterns, every tie and its neighbours, overflow
+ *                                to infinity at 61440 (tests/test_oracle_float_codes.py)
+ *   orc_matmul_f8e5m2            float64 product of numpy-decoded operands, rounded by torch / numpy casts
  *   orc_a16_quantize_dq          closed-form scale, zp = 0, on-grid recovery, half-spacing bound
  *   orc_a16_quantize             on-grid weights are recovered exactly, |w - dequant(q)| <= scale/2 inside the
  *                                clamp range, closed-form scale/zp, nibble order via the A16MatMul dequantizer
@@ -194,6 +198,13 @@ int orc_matmul_f8(const float *left, const float *right, const float *bias, int6
                   int right_transpose, int do_relu, double relu_limit, const double *scales, int n_scales,
                   float *output, float *acc_out);
 
+/* tpu.MatMul on F8E5M2 operands (the same product) with the output arm its storage type selects, MatMul.cpp:630-635:
+ * F8E5M2(v, 1.0, true), F16(v) or BF16(v). */
+enum { ORC_F8E5M2_OUT_E5M2 = 0, ORC_F8E5M2_OUT_F16 = 1, ORC_F8E5M2_OUT_BF16 = 2 };
+int orc_matmul_f8e5m2(const float *left, const float *right, const float *bias, int64_t M, int64_t K, int64_t N,
+                      int right_transpose, int do_relu, double relu_limit, int out_arm, float *output,
+                      float *acc_out);
+
 /* exact-integer GEMM used to cross-check the f32 accumulation domain */
 void orc_igemm_i64(const int8_t *A, const int8_t *B, const int32_t *bias,
                    int64_t *Y, int64_t M, int64_t K, int64_t N,
@@ -260,6 +271,11 @@ float orc_f4e2m1_to_f32(uint8_t code);
 void orc_f32_to_f8e4m3_n(const float *src, int64_t n, int saturate, uint8_t *dst);
 void orc_f8e4m3_to_f32_n(const uint8_t *src, int64_t n, float *dst);
 void orc_f32_to_f4e2m1_n(const float *src, int64_t n, uint8_t *dst);
+/* lib/Support/Float8.cpp:134-138 (never saturates: overflow gives the infinity 0x7c) and :193-196 */
+uint8_t orc_f32_to_f8e5m2(float src);
+float orc_f8e5m2_to_f32(uint8_t code);
+void orc_f32_to_f8e5m2_n(const float *src, int64_t n, uint8_t *dst);
+void orc_f8e5m2_to_f32_n(const uint8_t *src, int64_t n, float *dst);
 
 /* tpu.MatMul with both operands quantized dynamically (lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:447-597, dq_type
  * "INT8": imax 127, "INT4": imax 7; batch 1): left [M, K], right [K, N] or [N, K] when right_transpose, both

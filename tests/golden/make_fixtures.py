@@ -286,6 +286,24 @@ def case_float_codes():
     y, acc = O.matmul_f8(la, rb, bias, right_transpose=True, do_relu=True, relu_limit=900.0, scales=mm_scales)
     out.update(f8mm_left=O.f32_to_f8e4m3(la), f8mm_right=O.f32_to_f8e4m3(rb), f8mm_bias=bias, f8mm_scales=mm_scales,
                f8mm_want_codes=O.f32_to_f8e4m3(y), f8mm_want_acc=acc)
+    # E5M2: the conversion on a spread of values (ties, subnormals, overflow to infinity), the decode table, and a
+    # small-integer product with the E5M2 / F16 / BF16 output arms of MatMul.cpp:630-635.  Appended after everything
+    # else so that the generator's stream for the entries above stays what it was.
+    x5 = np.concatenate([(rng.standard_normal(300) * 2.0 ** rng.integers(-18, 17, size=300)).astype(np.float32),
+                         np.array([0.0, -0.0, 2.0 ** -17, 3 * 2.0 ** -17, 2.0 ** -16, 1.25, 1.125, 1.375, 57344.0,
+                                   61439.9, 61440.0, -61440.0, 1e9, np.inf, -np.inf], np.float32)])
+    out.update(e5m2_src=x5, e5m2_codes=O.f32_to_f8e5m2(x5), e5m2_decode=O.f8e5m2_to_f32(np.arange(256, dtype=np.uint8)))
+    vals = np.array([0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16], np.float32)
+    M, K, N = 24, 128, 40
+    la = (rng.choice(vals, size=(M, K)) * rng.choice(np.array([-1, 1], np.float32), size=(M, K))).astype(np.float32)
+    rb = (rng.choice(vals, size=(N, K)) * rng.choice(np.array([-1, 1], np.float32), size=(N, K)) * 0.25).astype(np.float32)
+    bias = rng.integers(-200, 201, size=N).astype(np.float32)
+    y5, acc5 = O.matmul_f8e5m2(la, rb, bias, right_transpose=True, do_relu=True, relu_limit=3000.0)
+    yh, _ = O.matmul_f8e5m2(la, rb, bias, right_transpose=True, do_relu=True, relu_limit=3000.0, out_arm=O.F8E5M2_OUT_F16)
+    yb, _ = O.matmul_f8e5m2(la, rb, bias, right_transpose=True, do_relu=True, relu_limit=3000.0, out_arm=O.F8E5M2_OUT_BF16)
+    out.update(e5m2mm_left=O.f32_to_f8e5m2(la), e5m2mm_right=O.f32_to_f8e5m2(rb), e5m2mm_bias=bias,
+               e5m2mm_want_codes=O.f32_to_f8e5m2(y5), e5m2mm_want_acc=acc5, e5m2mm_want_f16=O.f32_to_f16(yh),
+               e5m2mm_want_bf16=O.f32_to_bf16(yb))
     np.savez_compressed(os.path.join(HERE, "case_float_codes.npz"), **out)
 
 

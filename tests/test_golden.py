@@ -155,6 +155,16 @@ def test_oracle_reproduces_float_code_cases(orc):
     y, acc = orc.matmul_f8(orc.f8e4m3_to_f32(d["f8mm_left"]), orc.f8e4m3_to_f32(d["f8mm_right"]), d["f8mm_bias"],
                            right_transpose=True, do_relu=True, relu_limit=900.0, scales=d["f8mm_scales"])
     assert np.array_equal(orc.f32_to_f8e4m3(y), d["f8mm_want_codes"]) and np.array_equal(acc, d["f8mm_want_acc"])
+    assert np.array_equal(orc.f32_to_f8e5m2(d["e5m2_src"]), d["e5m2_codes"])
+    assert np.array_equal(orc.f8e5m2_to_f32(np.arange(256, dtype=np.uint8)).view(np.uint32), d["e5m2_decode"].view(np.uint32))
+    la, rb = orc.f8e5m2_to_f32(d["e5m2mm_left"]), orc.f8e5m2_to_f32(d["e5m2mm_right"])
+    kw = dict(right_transpose=True, do_relu=True, relu_limit=3000.0)
+    y, acc = orc.matmul_f8e5m2(la, rb, d["e5m2mm_bias"], **kw)
+    assert np.array_equal(orc.f32_to_f8e5m2(y), d["e5m2mm_want_codes"]) and np.array_equal(acc, d["e5m2mm_want_acc"])
+    y, _ = orc.matmul_f8e5m2(la, rb, d["e5m2mm_bias"], out_arm=orc.F8E5M2_OUT_F16, **kw)
+    assert np.array_equal(orc.f32_to_f16(y), d["e5m2mm_want_f16"])
+    y, _ = orc.matmul_f8e5m2(la, rb, d["e5m2mm_bias"], out_arm=orc.F8E5M2_OUT_BF16, **kw)
+    assert np.array_equal(orc.f32_to_bf16(y), d["e5m2mm_want_bf16"])
 
 
 FLOAT_QUANT_TAGS = {"f8_g64": dict(bits=8, g=64, dq="DQ_F8E4M3"), "f4_g128": dict(bits=4, g=128, dq="DQ_F4")}
@@ -200,6 +210,16 @@ def test_gpu_float_codes_against_fixture():
     torch.cuda.synchronize()
     assert np.array_equal(acc.cpu().numpy().view(np.uint32), d["f8mm_want_acc"].view(np.uint32))
     assert np.array_equal(y.cpu().numpy(), d["f8mm_want_codes"])
+    for kind, key, tdt in ((clib.F8_OUT_CODES, "e5m2mm_want_codes", None), (clib.F8_OUT_F16, "e5m2mm_want_f16", torch.int16),
+                           (clib.F8_OUT_BF16, "e5m2mm_want_bf16", torch.int16)):
+        acc = torch.empty(d["e5m2mm_want_acc"].shape, dtype=torch.float32, device="cuda")
+        y = M_.f8mm_launch(torch.from_numpy(d["e5m2mm_left"]).cuda(), torch.from_numpy(d["e5m2mm_right"]).cuda(),
+                           torch.from_numpy(d["e5m2mm_bias"]).cuda(), right_transpose=True, do_relu=True,
+                           relu_limit=3000.0, out_kind=kind, acc_f32=acc, f8_type=clib.F8_E5M2)
+        torch.cuda.synchronize()
+        assert np.array_equal(acc.cpu().numpy().view(np.uint32), d["e5m2mm_want_acc"].view(np.uint32))
+        got = y.cpu() if tdt is None else y.view(tdt).cpu()
+        assert np.array_equal(got.numpy().view(d[key].dtype), d[key]), key
     out, pre = run(d["f8rand_x"], d["f8rand_weight"], d["f8_scale"], zp, None, 8, 64, clib.DQ_F8E4M3)
     wv = np.abs(d["f8_decode"][d["f8rand_weight"]].astype(np.float64)).reshape(24, 4, 64)
     deq = (wv * S.bf16_to_f32(d["f8_scale"]).astype(np.float64)[:, :, None]).reshape(24, 256)

@@ -183,3 +183,130 @@ def test_f8_matmul_full_size_linearity():
     bias = rng.standard_normal(N).astype(np.float32)
     _, acc0 = _run(a, np.zeros_like(b), bias, True, False, -1.0, 1.0, None)
     assert np.array_equal(acc0, np.tile(bias, (M, 1)))
+
+
+# ---- E5M2 operands and the output arms of MatMul.cpp:630-635 ----------------------------------------------------
+def _e5m2_codes(rng, shape, top=0x58):
+    c = rng.integers(0, 256, size=shape).astype(np.uint8)
+    return ((c & 0x80) | np.minimum(c & 0x7f, top)).astype(np.uint8)     # 0x58 = 128: finite, sums far from overflow
+
+
+def _run_e5m2(a, b, bias, rt, relu, limit, out_kind):
+    return _run_typed(a, b, bias, rt, relu, limit, out_kind, clib.F8_E5M2)
+
+
+def _run_typed(a, b, bias, rt, relu, limit, out_kind, f8_type):
+    import torch
+    M, N = a.shape[0], (b.shape[0] if rt else b.shape[1])
+    acc = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.f8mm_launch(torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(),
+                       None if bias is None else torch.from_numpy(bias).cuda(), right_transpose=rt, do_relu=relu,
+                       relu_limit=limit, out_kind=out_kind, acc_f32=acc, f8_type=f8_type)
+    torch.cuda.synchronize()
+    return y.cpu(), acc.cpu().numpy()
+
+
+E5M2_CASES = [  # (M, K, N, right_transpose, relu, bias)
+    (1, 64, 16, True, False, False), (5, 512, 100, False, False, True), (130, 1024, 200, True, True, True),
+    (64, 200, 48, False, False, False), (33, 72, 130, True, True, True), (300, 320, 520, False, True, True),
+]
+
+
+@pytest.mark.parametrize("tile", ["128", "256"])
+@pytest.mark.parametrize("M,K,N,rt,relu,bias", E5M2_CASES)
+def test_e5m2_matmul_device_level(orc, monkeypatch, M, K, N, rt, relu, bias, tile):
+    monkeypatch.setenv("MI_F8_TILE", tile)
+    rng = np.random.default_rng(M + K + N + 1)
+    a = _e5m2_codes(rng, (M, K))
+    b = _e5m2_codes(rng, (N, K) if rt else (K, N))
+    bv = (rng.standard_normal(N) * 500).astype(np.float32) if bias else None
+    af, bf = orc.f8e5m2_to_f32(a), orc.f8e5m2_to_f32(b)
+    b_kn = bf.T if rt else bf
+    mag = np.abs(af.astype(np.float64)) @ np.abs(b_kn.astype(np.float64))
+    rms = float(np.sqrt(np.mean((af.astype(np.float64) @ b_kn) ** 2))) + 1e-9
+    limit = 2.0 * rms if relu else -1.0
+    want, want_acc = orc.matmul_f8e5m2(af, bf, bv, right_transpose=rt, do_relu=relu, relu_limit=limit)
+    y, acc = _run_e5m2(a, b, bv, rt, relu, limit, clib.F8_OUT_CODES)
+    assert np.all(np.abs(acc.astype(np.float64) - want_acc) <= mag * 2.0 ** -11 + 1e-6)
+    got = y.numpy()
+    # the output arm is exact arithmetic on the kernel's own fp32 value
+    assert np.array_equal(got, orc.f32_to_f8e5m2(acc))
+    # against the oracle's codes: the fp32 values agree to ~2^-13, the codes are 2^-3 apart, so nearly all are equal
+    dist = _code_distance(got, orc.f32_to_f8e5m2(want))
+    with np.errstate(invalid="ignore"):                      # sums past 61440 are infinite on both sides
+        near_zero = np.abs(orc.f8e5m2_to_f32(got).astype(np.float64) - want) <= mag * 2.0 ** -11 + 1e-6
+    assert np.all((dist <= 1) | near_zero)
+    assert (dist == 0).mean() >= 0.99
+    y32, acc32 = _run_e5m2(a, b, bv, rt, relu, limit, clib.F8_OUT_F32)
+    assert np.array_equal(acc32, acc)
+    assert np.array_equal(y32.numpy(), orc.f8e5m2_to_f32(got))
+    # 16-bit outputs: BF16() / F16() of the fp32 value (MatMul.cpp:632-635), through the oracle's own roundings
+    yb, _ = _run_e5m2(a, b, bv, rt, relu, limit, clib.F8_OUT_BF16)
+    assert np.array_equal(yb.view(dtype=__import__("torch").int16).numpy().view(np.uint16), orc.f32_to_bf16(acc))
+    yh, _ = _run_e5m2(a, b, bv, rt, relu, limit, clib.F8_OUT_F16)
+    assert np.array_equal(yh.view(dtype=__import__("torch").int16).numpy().view(np.uint16), orc.f32_to_f16(acc))
+
+
+def test_e5m2_matmul_exact_domain(orc):
+    """Small integer operands (E5M2 holds 0..8, 10, 12, 14, 16 exactly): every partial sum is an integer below 2^24, so
+    the fp32 value and every output form equal the oracle's bit for bit."""
+    rng = np.random.default_rng(14)
+    M, K, N = 70, 384, 90
+    vals = np.array([0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16], np.float32)
+    af = rng.choice(vals, size=(M, K)) * rng.choice(np.array([-1, 1], np.float32), size=(M, K))
+    bf = rng.choice(vals, size=(K, N)) * rng.choice(np.array([-1, 1], np.float32), size=(K, N))
+    bias = rng.integers(-100, 101, size=N).astype(np.float32)
+    a, b = orc.f32_to_f8e5m2(af), orc.f32_to_f8e5m2(bf)
+    assert np.array_equal(orc.f8e5m2_to_f32(a), af + np.float32(0))
+    for arm, kind in ((0, clib.F8_OUT_F32), (1, clib.F8_OUT_F16), (2, clib.F8_OUT_BF16)):
+        want, want_acc = orc.matmul_f8e5m2(af, bf, bias, out_arm=arm)
+        y, acc = _run_e5m2(a, b, bias, False, False, -1.0, kind)
+        assert np.array_equal(acc.view(np.uint32), want_acc.view(np.uint32))
+        assert np.array_equal(y.float().numpy(), want)
+    codes, _ = _run_e5m2(a, b, bias, False, False, -1.0, clib.F8_OUT_CODES)
+    want, _ = orc.matmul_f8e5m2(af, bf, bias)
+    assert np.array_equal(codes.numpy(), orc.f32_to_f8e5m2(want))
+    assert np.unique(codes.numpy()).size > 30
+
+
+def test_e5m2_output_rounding_boundaries(orc):
+    """A zero product plus a bias reads the output conversion back on its own: every E5M2 rounding boundary and its
+    neighbours, the subnormal range, overflow (to infinity: the routine never saturates), infinities and NaN."""
+    codes = np.arange(0, 0x7b, dtype=np.uint8)
+    mid = ((orc.f8e5m2_to_f32(codes).astype(np.float64) + orc.f8e5m2_to_f32(codes + 1)) / 2).astype(np.float32)
+    cand = np.concatenate([mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(1e9)),
+                           np.array([57344.0, 61439.0, 61440.0, 65536.0, 3e38, np.inf, 1e-8, 2.0 ** -17, 0.0, 1e-45],
+                                    np.float32)])
+    cand = np.concatenate([cand, -cand, np.array([np.nan], np.float32)]).astype(np.float32)
+    N = cand.size
+    for K in (64, 48):
+        a = np.zeros((3, K), np.uint8)
+        b = np.zeros((K, N), np.uint8)
+        y, acc = _run_e5m2(a, b, cand, False, False, -1.0, clib.F8_OUT_CODES)
+        assert np.array_equal(acc, np.tile(cand, (3, 1)), equal_nan=True)   # (0 + -0 is +0: values, not patterns)
+        assert np.array_equal(y.numpy(), orc.f32_to_f8e5m2(acc))
+        y32, _ = _run_e5m2(a, b, cand, False, False, -1.0, clib.F8_OUT_F32)
+        want = orc.f8e5m2_to_f32(orc.f32_to_f8e5m2(acc))
+        assert np.array_equal(np.isnan(y32.numpy()), np.isnan(want))
+        ok = ~np.isnan(want)
+        assert np.array_equal(y32.numpy()[ok].view(np.uint32), want[ok].view(np.uint32))
+    assert 0x7c in y.numpy() and 0xfc in y.numpy() and 0x7f in y.numpy()
+
+
+def test_e5m2_matmul_operator_level_and_rejections(orc):
+    rng = np.random.default_rng(18)
+    M, K, N = 6, 128, 40
+    af = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
+    bf = rng.integers(-8, 9, size=(N, K)).astype(np.float32) * 0.25
+    bias = rng.integers(-100, 101, size=N).astype(np.float32)
+    y = M_.matmul_f8(af, bf, bias, right_transpose=True, do_relu=True, relu_limit=200.0, f8_type=clib.F8_E5M2)
+    want, _ = orc.matmul_f8e5m2(af, bf, bias, right_transpose=True, do_relu=True, relu_limit=200.0)
+    assert np.array_equal(y, want)
+    bad = af.copy()
+    bad[0, 0] = 9.0                                          # E5M2 has 8 and 10, not 9
+    with pytest.raises(clib.BackendError) as e:
+        M_.matmul_f8(bad, bf, None, right_transpose=True, f8_type=clib.F8_E5M2)
+    assert e.value.code == clib.MI_UNSUPPORTED
+    with pytest.raises(clib.BackendError) as e:
+        M_.matmul_f8(af, bf, None, right_transpose=True, f8_type=7)
+    assert e.value.code == clib.MI_BAD_ARGUMENT

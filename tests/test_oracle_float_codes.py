@@ -352,3 +352,103 @@ def test_f8_matmul_one_scale_step_is_narrowed_to_float(orc):
             assert per[0, 0] == orc.f8e4m3_to_f32(np.array([d], np.uint8))[0]
             assert one[0, 0] != per[0, 0]
     assert found > 0
+
+
+# ---- E5M2 (lib/Support/Float8.cpp with is_e5m2: the MatMul output arm MatMul.cpp:630-631) -----------------------
+def _half_decode(codes):
+    """An E5M2 code is the top byte of an IEEE half."""
+    return (np.ascontiguousarray(codes, dtype=np.uint8).astype(np.uint16) << 8).view(np.float16).astype(np.float32)
+
+
+def test_e5m2_decode_all_codes(orc):
+    codes = np.arange(256, dtype=np.uint8)
+    got = orc.f8e5m2_to_f32(codes)
+    want = _half_decode(codes)
+    tw = torch.from_numpy(codes).view(torch.float8_e5m2).float().numpy()
+    nan = ((codes >> 2) & 31 == 31) & ((codes & 3) != 0)
+    assert np.array_equal(np.isnan(got), nan) and np.array_equal(np.isnan(want), nan) and np.array_equal(np.isnan(tw), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    assert np.array_equal(got[~nan].view(np.uint32), tw[~nan].view(np.uint32))
+    assert got[0x7b] == 57344.0 and got[0x01] == 2.0 ** -16 and got[0x04] == 2.0 ** -14 and np.isinf(got[0x7c])
+    assert np.signbit(got[0x80]) and got[0x80] == 0.0
+
+
+def test_e5m2_encode_against_torch_and_numpy_half(orc):
+    bf = (np.arange(65536, dtype=np.uint32) << 16).view(np.float32)
+    rng = np.random.default_rng(2)
+    rnd = np.concatenate([
+        rng.standard_normal(200000).astype(np.float32) * 1000,
+        (rng.standard_normal(100000) * 2.0 ** rng.integers(-20, 17, size=100000)).astype(np.float32),
+        rng.integers(0, 1 << 32, size=200000, dtype=np.uint64).astype(np.uint32).view(np.float32)])
+    x = np.concatenate([bf, rnd])
+    x = x[~np.isnan(x)]
+    got = orc.f32_to_f8e5m2(x)
+    want = torch.from_numpy(x).to(torch.float8_e5m2).view(torch.uint8).numpy()  # RNE, overflow to infinity
+    assert np.array_equal(got, want)
+    # values that are already halves: the code is the half's top byte rounded to even on the dropped byte
+    h = np.arange(65536, dtype=np.uint16)
+    hv = h.view(np.float16).astype(np.float32)
+    keep = ~np.isnan(hv)
+    low, top = (h & 0xff).astype(np.int32), (h >> 8).astype(np.int32)
+    up = (low > 0x80) | ((low == 0x80) & (top & 1 == 1))
+    want_h = (top + up).astype(np.uint8)                     # a carry walks into the exponent, up to infinity
+    assert np.array_equal(orc.f32_to_f8e5m2(hv[keep]), want_h[keep])
+
+
+def test_e5m2_encode_ties_overflow_and_specials(orc):
+    codes = np.arange(0, 0x7b, dtype=np.uint8)
+    lo = orc.f8e5m2_to_f32(codes).astype(np.float64)
+    hi = orc.f8e5m2_to_f32(codes + 1).astype(np.float64)
+    mid = ((lo + hi) / 2).astype(np.float32)
+    assert np.array_equal(mid.astype(np.float64), (lo + hi) / 2)
+    even = np.where(codes % 2 == 0, codes, codes + 1).astype(np.uint8)
+    assert np.array_equal(orc.f32_to_f8e5m2(mid), even)
+    assert np.array_equal(orc.f32_to_f8e5m2(-mid), even | 0x80)
+    assert np.array_equal(orc.f32_to_f8e5m2(np.nextafter(mid, np.float32(0))), codes)
+    assert np.array_equal(orc.f32_to_f8e5m2(np.nextafter(mid, np.float32(np.inf))), codes + 1)
+    f = np.float32
+    # the routine never saturates (Float8.cpp:134-138): the tie at 61440 goes to the even neighbour, which is infinity
+    x = np.array([57344.0, 61439.99, 61440.0, 65536.0, 3e38, np.inf, -61440.0, -np.inf, 0.0, -0.0, 1e-45, -1e-45,
+                  2.0 ** -17, np.nextafter(f(2.0 ** -17), f(1)), 3 * 2.0 ** -17, 2.0 ** -16], dtype=f)
+    want = np.array([0x7b, 0x7b, 0x7c, 0x7c, 0x7c, 0x7c, 0xfc, 0xfc, 0x00, 0x80, 0x00, 0x80,
+                     0x00, 0x01, 0x02, 0x01], dtype=np.uint8)
+    assert np.array_equal(orc.f32_to_f8e5m2(x), want)
+    nan = np.array([np.nan, -np.nan], dtype=f)
+    nan_bits = nan.view(np.uint32)
+    want_nan = np.where(nan_bits >> 31 == 1, 0xff, 0x7f).astype(np.uint8)
+    assert np.array_equal(orc.f32_to_f8e5m2(nan), want_nan)
+    allc = np.array([c for c in range(256) if not ((c >> 2) & 31 == 31 and c & 3)], dtype=np.uint8)
+    assert np.array_equal(orc.f32_to_f8e5m2(orc.f8e5m2_to_f32(allc)), allc)
+
+
+def test_matmul_f8e5m2_against_float64_and_library_roundings(orc):
+    rng = np.random.default_rng(5)
+    M, K, N = 7, 96, 11
+    a = rng.integers(0, 256, size=(M, K)).astype(np.uint8)
+    b = rng.integers(0, 256, size=(N, K)).astype(np.uint8)
+    a = np.where((a & 0x7f) >= 0x58, a & 0x83 | 0x30, a).astype(np.uint8)    # magnitudes below 64: finite, no overflow
+    b = np.where((b & 0x7f) >= 0x58, b & 0x83 | 0x30, b).astype(np.uint8)
+    af, bf = _half_decode(a), _half_decode(b)
+    bias = (rng.standard_normal(N) * 30).astype(np.float32)
+    exact = af.astype(np.float64) @ bf.astype(np.float64).T + bias
+    mag = np.abs(af.astype(np.float64)) @ np.abs(bf.astype(np.float64)).T + np.abs(bias)
+    for relu, limit in ((False, -1.0), (True, 500.0)):
+        want32 = exact.copy()
+        if relu:
+            want32 = np.minimum(np.maximum(want32, 0.0), limit)
+        for arm, cast in ((0, lambda v: torch.from_numpy(v).to(torch.float8_e5m2).float().numpy()),
+                          (1, lambda v: v.astype(np.float16).astype(np.float32)),
+                          (2, lambda v: torch.from_numpy(v).to(torch.bfloat16).float().numpy())):
+            out, acc = orc.matmul_f8e5m2(af, bf, bias, right_transpose=True, do_relu=relu, relu_limit=limit, out_arm=arm)
+            assert np.all(np.abs(acc.astype(np.float64) - want32) <= mag * 2.0 ** -23)
+            assert np.array_equal(out, cast(acc))               # the arm is the library's cast of the f32 value
+    # [K, N] right operand, no bias: same product
+    o1, _ = orc.matmul_f8e5m2(af, np.ascontiguousarray(bf.T), None)
+    o2, _ = orc.matmul_f8e5m2(af, bf, None, right_transpose=True)
+    assert np.array_equal(o1, o2)
+    # small integers: everything exact, codes by hand: 3 * 5 * K_used
+    one = np.zeros((1, 8), np.float32)
+    one[0, :3] = 3.0
+    col = np.full((8, 1), 5.0, np.float32)
+    out, acc = orc.matmul_f8e5m2(one, col, np.array([0.5], np.float32))
+    assert acc[0, 0] == 45.5 and out[0, 0] == 48.0           # 45.5 between 40 and 48 (spacing 8): nearer to 48

@@ -19,7 +19,7 @@ EXPORTS = [
     "mi_a16mm_init", "mi_a16mm_inference", "mi_a16mm_deinit",
     "mi_a16_weight_create", "mi_a16_weight_destroy", "mi_a16_weight_bytes", "mi_a16mm_launch",
     "mi_a16mm_launch_group", "mi_a16mm_dq_launch", "mi_a16mm_dq_type_launch", "mi_matmul_dq_launch",
-    "mi_matmul_dq_inference", "mi_f8mm_inference", "mi_f8mm_launch",
+    "mi_matmul_dq_inference", "mi_f8mm_inference", "mi_f8mm_launch", "mi_f8mm_e5m2_launch",
     "mi_a16_weight_export_size", "mi_a16_weight_export", "mi_a16_weight_import", "mi_a16_quantize", "mi_llm_unpack",
     "mi_a16_to_group",
     "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
@@ -65,10 +65,11 @@ class MatMulDqAttr(C.Structure):
 class F8MMAttr(C.Structure):
     _fields_ = [("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64), ("right_transpose", C.c_int),
                 ("do_relu", C.c_int), ("relu_limit", C.c_double), ("out_scales", C.POINTER(C.c_double)),
-                ("n_out_scales", C.c_int)]
+                ("n_out_scales", C.c_int), ("f8_type", C.c_int)]
 
 
 F8_OUT_CODES, F8_OUT_F32, F8_OUT_BF16, F8_OUT_F16 = 0, 1, 2, 3
+F8_E4M3, F8_E5M2 = 0, 1
 
 
 class A16QuantDesc(C.Structure):
@@ -153,6 +154,8 @@ def lib():
                                       C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         L.mi_f8mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int,
                                      C.c_double, C.c_double, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi_f8mm_e5m2_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
+                                          C.c_int, C.c_double, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16_to_group.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
         L.mi_llm_unpack.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
                                     C.c_void_p, C.c_void_p]

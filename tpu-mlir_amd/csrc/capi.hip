@@ -987,6 +987,37 @@ int mi_f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, 
                      d_out, d_acc_f32, (hipStream_t)stream);
 }
 
+int mi_f8mm_e5m2_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, const float *d_bias, int64_t M,
+                        int64_t K, int64_t N, int do_relu, double relu_limit, int out_kind, void *d_out,
+                        float *d_acc_f32, void *stream) {
+  return f8mm_launch(d_a, d_b, right_transpose, d_bias, M, K, N, do_relu, relu_limit, 1.0, nullptr, out_kind, d_out,
+                     d_acc_f32, (hipStream_t)stream, MI_F8_E5M2);
+}
+
+// f32 -> the E5M2 code of exactly that value (finite values only), or -1: an E5M2 value is a half whose low byte is 0
+static int f8e5m2_code_of(float v) {
+  uint32_t b;
+  memcpy(&b, &v, 4);
+  const uint32_t sign = (b >> 24) & 0x80u, a = b & 0x7fffffffu;
+  if (a == 0)
+    return (int)sign;
+  const int e = (int)(a >> 23) - 127;
+  const uint32_t frac = a & 0x7fffffu;
+  if (e >= -14 && e <= 15) {           // normals: 2 fraction bits
+    if (frac & 0x1fffffu)
+      return -1;
+    return (int)((((uint32_t)(e + 15) << 2) | (frac >> 21)) | sign);
+  }
+  if (e >= -16 && e < -14) {           // subnormals: multiples of 2^-16 below 2^-14
+    const uint32_t mant = frac | 0x800000u;
+    const int shift = 23 - (e + 16);
+    if (mant & ((1u << shift) - 1))
+      return -1;
+    return (int)((mant >> shift) | sign);
+  }
+  return -1;
+}
+
 // f32 -> the E4M3 code of exactly that value, or -1 (host side of the operator entry: the interpreter hands over
 // f32 arrays that hold E4M3 values)
 static int f8_code_of(float v) {
@@ -1018,9 +1049,11 @@ int mi_f8mm_inference(const mi_f8mm_attr *a, mi_infer_param *p) {
                  p->n_outputs >= 1 && p->outputs[0],
              MI_BAD_ARGUMENT, "mi_f8mm_inference: null argument");
   MI_REQUIRE(a->M >= 0 && a->K > 0 && a->N > 0, MI_BAD_ARGUMENT, "mi_f8mm_inference: bad shape");
-  MI_REQUIRE(a->out_scales && (a->n_out_scales == 1 || a->n_out_scales == a->N), MI_BAD_ARGUMENT,
+  MI_REQUIRE(a->f8_type == MI_F8_E4M3 || a->f8_type == MI_F8_E5M2, MI_BAD_ARGUMENT, "mi_f8mm_inference: f8_type");
+  const bool e5m2 = a->f8_type == MI_F8_E5M2;
+  MI_REQUIRE(e5m2 || (a->out_scales && (a->n_out_scales == 1 || a->n_out_scales == a->N)), MI_BAD_ARGUMENT,
              "mi_f8mm_inference: out_scales must hold one scale or one per output channel");
-  for (int i = 0; i < a->n_out_scales; ++i)
+  for (int i = 0; !e5m2 && i < a->n_out_scales; ++i)
     MI_REQUIRE(a->out_scales[i] == a->out_scales[i] && a->out_scales[i] != 0.0, MI_BAD_ARGUMENT,
                "mi_f8mm_inference: output scales must be nonzero numbers");
   if (a->M == 0)
@@ -1029,13 +1062,13 @@ int mi_f8mm_inference(const mi_f8mm_attr *a, mi_infer_param *p) {
   const size_t nl = (size_t)a->M * a->K, nr = (size_t)a->K * a->N, no = (size_t)a->M * a->N;
   std::vector<uint8_t> hl(nl), hr(nr);
   for (size_t i = 0; i < nl; ++i) {
-    const int c = f8_code_of(p->inputs[0][i]);
-    MI_REQUIRE(c >= 0, MI_UNSUPPORTED, "mi_f8mm_inference: left operand holds a value that is not an E4M3 number");
+    const int c = e5m2 ? f8e5m2_code_of(p->inputs[0][i]) : f8_code_of(p->inputs[0][i]);
+    MI_REQUIRE(c >= 0, MI_UNSUPPORTED, "mi_f8mm_inference: left operand holds a value that is not a finite number of its 8-bit type");
     hl[i] = (uint8_t)c;
   }
   for (size_t i = 0; i < nr; ++i) {
-    const int c = f8_code_of(p->inputs[1][i]);
-    MI_REQUIRE(c >= 0, MI_UNSUPPORTED, "mi_f8mm_inference: right operand holds a value that is not an E4M3 number");
+    const int c = e5m2 ? f8e5m2_code_of(p->inputs[1][i]) : f8_code_of(p->inputs[1][i]);
+    MI_REQUIRE(c >= 0, MI_UNSUPPORTED, "mi_f8mm_inference: right operand holds a value that is not a finite number of its 8-bit type");
     hr[i] = (uint8_t)c;
   }
   const float *bias = p->n_inputs > 2 ? p->inputs[2] : nullptr;
@@ -1050,14 +1083,15 @@ int mi_f8mm_inference(const mi_f8mm_attr *a, mi_infer_param *p) {
       return rc;
     MI_HIP(hipMemcpy(db.ptr, bias, (size_t)a->N * 4, hipMemcpyHostToDevice));
   }
-  if (a->n_out_scales != 1) {
+  if (!e5m2 && a->n_out_scales != 1) {
     if ((rc = ds.reserve((size_t)a->N * 8)))
       return rc;
     MI_HIP(hipMemcpy(ds.ptr, a->out_scales, (size_t)a->N * 8, hipMemcpyHostToDevice));
   }
   rc = f8mm_launch((const uint8_t *)dl.ptr, (const uint8_t *)dr.ptr, a->right_transpose, bias ? (const float *)db.ptr : nullptr,
-                   a->M, a->K, a->N, a->do_relu, a->relu_limit, a->out_scales[0],
-                   a->n_out_scales != 1 ? (const double *)ds.ptr : nullptr, MI_F8_OUT_F32, dy.ptr, nullptr, nullptr);
+                   a->M, a->K, a->N, a->do_relu, a->relu_limit, e5m2 ? 1.0 : a->out_scales[0],
+                   !e5m2 && a->n_out_scales != 1 ? (const double *)ds.ptr : nullptr, MI_F8_OUT_F32, dy.ptr, nullptr,
+                   nullptr, a->f8_type);
   if (rc)
     return rc;
   MI_HIP(hipDeviceSynchronize());

@@ -252,6 +252,33 @@ __device__ __forceinline__ float f8e4m3_to_f32(uint32_t c) {
   return (c & 0x80u) ? -mag : mag;
 }
 
+// f32 -> E5M2 code as f32_to_f8e5m2 calls the conversion (lib/Support/Float8.cpp:134-138: round half to even, never
+// saturating): what rounds to 2^16 or beyond, and the infinities, give 0x7c; NaN 0x7f; below 2^-14 the code is the
+// value in units of 2^-16 (4 = the smallest normal); f32 subnormals and zero give 0.
+__device__ __forceinline__ uint32_t f8e5m2_from_f32(float v) {
+  const uint32_t b = __float_as_uint(v);
+  const uint32_t a = b & 0x7fffffffu;
+  uint32_t r;
+  if (a > 0x7f800000u) {
+    r = 0x7f;
+  } else if (a >= 0x38800000u) {  // 2^-14
+    r = ((a + 0xfffffu + ((a >> 21) & 1u)) >> 21) - (112u << 2);
+    r = r > 0x7cu ? 0x7cu : r;
+  } else if (a >= 0x00800000u) {
+    r = (uint32_t)rintf(__uint_as_float(a) * 65536.0f);
+  } else {
+    r = 0;
+  }
+  return r | ((b >> 24) & 0x80u);
+}
+
+// E5M2 code -> f32 (f8e5m2_to_f32, Float8.cpp:140-196): the code is the top byte of an IEEE half
+__device__ __forceinline__ float f8e5m2_to_f32(uint32_t c) {
+  if ((c & 0x7fu) > 0x7cu)
+    return __uint_as_float(0x7fffffffu | ((c & 0x80u) << 24));
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)(c << 8));
+}
+
 // f32 -> E2M1 code (bit 3 = sign; magnitudes {0, .5, 1, 1.5, 2, 3, 4, 6}): f32_to_f4e2m1, lib/Support/Float4.cpp:7-22,
 // evaluated as written -- the first table entry with the strictly smallest fp32 |src - value| wins.  Ties therefore go
 // to the smaller magnitude, a negative input nearest to zero gives +0, and NaN, infinities and inputs too large for

@@ -67,8 +67,26 @@ __device__ __forceinline__ u32x4 f8_load_chunk(const uint8_t *base, int64_t row,
   return v;
 }
 
+// operand format of v_mfma_f32_32x32x64_f8f6f4 (its cbsz / blgp fields): 0 = E4M3, 1 = E5M2
+constexpr int F8_FMT_E4M3 = 0, F8_FMT_E5M2 = 1;
+
+// The output arms of a product of E5M2 operands (MatMul.cpp:630-635): F8E5M2(v, 1.0, true) for an E5M2 result (as
+// codes or as the values in f32), F16(v) / BF16(v) for a 16-bit result.
+__device__ __forceinline__ void f8_store_e5m2(const F8Args &a, int64_t o, float v) {
+  if (a.out_kind == MI_F8_OUT_CODES)
+    ((uint8_t *)a.out)[o] = (uint8_t)f8e5m2_from_f32(v);
+  else if (a.out_kind == MI_F8_OUT_F32)
+    ((float *)a.out)[o] = f8e5m2_to_f32(f8e5m2_from_f32(v));
+  else if (a.out_kind == MI_F8_OUT_BF16)
+    ((uint16_t *)a.out)[o] = f32_to_bf16_bm(v);
+  else
+    ((uint16_t *)a.out)[o] = f32_to_f16_ref(v);
+}
+
+template <int FMT>
 __device__ __forceinline__ void f8_epilogue(const F8Args &a, const f32x16 (&acc)[2][2], int64_t m0, int64_t n0, int lane);
 
+template <int FMT>
 __global__ __launch_bounds__(256) void f8_gemm_kernel(F8Args a) {
   __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][F8_BM * F8_LDS_ROW];
   __shared__ __attribute__((aligned(16))) uint8_t lds_b[2][F8_BN * F8_LDS_ROW];
@@ -127,18 +145,19 @@ __global__ __launch_bounds__(256) void f8_gemm_kernel(F8Args a) {
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j)  // formats 0 / 0 = E4M3 x E4M3, no block scales
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], FMT, FMT, 0, 0, 0, 0);
     if (it + 1 < k_iters) {
       lstore(stage ^ 1);
       __syncthreads();
     }
   }
 
-  f8_epilogue(a, acc, m_base + wm * 64, n_base + wn * 64, lane);
+  f8_epilogue<FMT>(a, acc, m_base + wm * 64, n_base + wn * 64, lane);
 }
 
 // epilogue of a wave's 64 x 64 block: register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of its
 // 32 x 32 block (i, j)
+template <int FMT>
 __device__ __forceinline__ void f8_epilogue(const F8Args &a, const f32x16 (&acc)[2][2], int64_t m0, int64_t n0, int lane) {
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
@@ -162,6 +181,10 @@ __device__ __forceinline__ void f8_epilogue(const F8Args &a, const f32x16 (&acc)
           const int64_t o = m * a.N + n;
           if (a.acc_out)
             a.acc_out[o] = v;
+          if constexpr (FMT == F8_FMT_E5M2) {
+            f8_store_e5m2(a, o, v);
+            continue;
+          }
           // F8E4M3(v, step, true): the quotient in double, narrowed to fp32, rounded to E4M3 (Float8.cpp:259-261).
           // v * (1 / step) is within two double ulps of that quotient, so the narrowing can come out differently
           // only when the 29 bits it drops sit next to the halfway pattern; only then is the division carried out.
@@ -218,6 +241,7 @@ constexpr int F8_STRIDE = 68;  // dwords per row of an epilogue strip (64 + 4: 1
 // Epilogue of a wave's 64 x 64 block through its own strip of LDS: the accumulators (register r of lane l = row
 // 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of block (i, j)) are laid out row-major so that a lane owns 16
 // consecutive columns of a row -- per-column parameters are fetched once per lane, results leave as 16-byte stores.
+template <int FMT>
 __device__ __forceinline__ void f8_strip_epilogue(const F8Args &a, const f32x16 (&acc)[2][2], float *strip, int64_t m0,
                                                   int64_t nb, int lane) {
 #pragma unroll
@@ -262,6 +286,32 @@ __device__ __forceinline__ void f8_strip_epilogue(const F8Args &a, const f32x16 
     }
     if (m >= a.M)
       continue;
+    const int64_t o = m * a.N + n0;
+    if constexpr (FMT == F8_FMT_E5M2) {
+      if (vec_ok && a.acc_out) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)
+          *(f32x4 *)(a.acc_out + o + q4 * 4) = f32x4{v[q4 * 4], v[q4 * 4 + 1], v[q4 * 4 + 2], v[q4 * 4 + 3]};
+      }
+      if (vec_ok && a.out_kind == MI_F8_OUT_CODES) {
+        uint32_t w[4];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)
+          w[q4] = f8e5m2_from_f32(v[q4 * 4]) | (f8e5m2_from_f32(v[q4 * 4 + 1]) << 8) |
+                  (f8e5m2_from_f32(v[q4 * 4 + 2]) << 16) | (f8e5m2_from_f32(v[q4 * 4 + 3]) << 24);
+        *(u32x4 *)((uint8_t *)a.out + o) = u32x4{w[0], w[1], w[2], w[3]};
+        continue;
+      }
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        if (n0 + e >= a.N)
+          continue;
+        if (a.acc_out && !vec_ok)
+          a.acc_out[o + e] = v[e];
+        f8_store_e5m2(a, o + e, v[e]);
+      }
+      continue;
+    }
     uint32_t c2[8];  // two codes each
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -269,7 +319,6 @@ __device__ __forceinline__ void f8_strip_epilogue(const F8Args &a, const f32x16 
       const int64_t n_b = (n0 + 2 * e + 1) < a.N ? (n0 + 2 * e + 1) : (a.N - 1);
       c2[e] = f8_requant_pair(a, v[2 * e], v[2 * e + 1], inv[2 * e], inv[2 * e + 1], n_a, n_b);
     }
-    const int64_t o = m * a.N + n0;
     if (vec_ok) {
       if (a.acc_out) {
 #pragma unroll
@@ -310,7 +359,7 @@ constexpr int f8_ring_lds_bytes(int nst) { return nst * F8_STAGE > 4 * 64 * F8_S
 
 // NST = stages in the LDS ring: 4 (two workgroups per CU) when there are more tiles than CUs, 8 when every workgroup
 // has a CU to itself
-template <int NST>
+template <int NST, int FMT>
 __global__ __launch_bounds__(256) void f8_gemm_ring_kernel(F8Args a, int tiles_m, int tiles_n, int per_xcd) {
   constexpr int LOADS = F8_BM * (F8_BK / 16) / 256;  // direct-to-LDS instructions per operand, stage and thread: 2
   constexpr int LPS = 2 * LOADS;
@@ -395,11 +444,11 @@ __global__ __launch_bounds__(256) void f8_gemm_ring_kernel(F8Args a, int tiles_m
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], FMT, FMT, 0, 0, 0, 0);
   }
   __builtin_amdgcn_s_waitcnt(f8_waitcnt_vm(0));  // drain the re-loads issued past the end
   __builtin_amdgcn_s_barrier();                  // every wave is done reading the ring
-  f8_strip_epilogue(a, acc, (float *)f8_lds + wave * (64 * F8_STRIDE), m_base + wm * 64, n_base + wn * 64, lane);
+  f8_strip_epilogue<FMT>(a, acc, (float *)f8_lds + wave * (64 * F8_STRIDE), m_base + wm * 64, n_base + wn * 64, lane);
 }
 
 // ---- 256 x 256 outputs per workgroup, 4 waves (2 x 2), each wave 128 x 128 as 4 x 4 blocks of 32 x 32 (256 fp32
@@ -413,6 +462,7 @@ constexpr int F8L_STAGE = (F8L_M + F8L_N) * F8_BK;  // 32 KiB
 constexpr int F8L_NST = 4;
 constexpr int F8_WAITCNT_LGKM0 = 0xC07F;
 
+template <int FMT>
 __global__ __launch_bounds__(256, 1) void f8_gemm_large_kernel(F8Args a, int tiles_m, int tiles_n, int per_xcd) {
   constexpr int NST = F8L_NST;
   constexpr int LOADS = F8L_M * (F8_BK / 16) / 256;  // direct-to-LDS instructions per operand, stage and thread: 4
@@ -489,7 +539,7 @@ __global__ __launch_bounds__(256, 1) void f8_gemm_large_kernel(F8Args a, int til
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
       const int i = t >> 2, j = t & 3;
-      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ca[i], cb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ca[i], cb[j], acc[i][j], FMT, FMT, 0, 0, 0, 0);
       if (t < 4)
         read_frag(na[t], st, a_off[t]);
       else if (t < 8)
@@ -530,19 +580,19 @@ __global__ __launch_bounds__(256, 1) void f8_gemm_large_kernel(F8Args a, int til
   const int64_t mw = m_base + wm * 128, nw = n_base + wn * 128;
   {
     const f32x16 sub[2][2] = {{acc[0][0], acc[0][1]}, {acc[1][0], acc[1][1]}};
-    f8_strip_epilogue(a, sub, strip, mw, nw, lane);
+    f8_strip_epilogue<FMT>(a, sub, strip, mw, nw, lane);
   }
   {
     const f32x16 sub[2][2] = {{acc[0][2], acc[0][3]}, {acc[1][2], acc[1][3]}};
-    f8_strip_epilogue(a, sub, strip, mw, nw + 64, lane);
+    f8_strip_epilogue<FMT>(a, sub, strip, mw, nw + 64, lane);
   }
   {
     const f32x16 sub[2][2] = {{acc[2][0], acc[2][1]}, {acc[3][0], acc[3][1]}};
-    f8_strip_epilogue(a, sub, strip, mw + 64, nw, lane);
+    f8_strip_epilogue<FMT>(a, sub, strip, mw + 64, nw, lane);
   }
   {
     const f32x16 sub[2][2] = {{acc[2][2], acc[2][3]}, {acc[3][2], acc[3][3]}};
-    f8_strip_epilogue(a, sub, strip, mw + 64, nw + 64, lane);
+    f8_strip_epilogue<FMT>(a, sub, strip, mw + 64, nw + 64, lane);
   }
 }
 
@@ -562,7 +612,12 @@ __global__ void f8_transpose_kernel(const uint8_t *__restrict__ src, uint8_t *__
 
 int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, const float *d_bias, int64_t M, int64_t K,
                 int64_t N, int do_relu, double relu_limit, double out_scale, const double *d_out_scales, int out_kind,
-                void *d_out, float *d_acc, hipStream_t stream) {
+                void *d_out, float *d_acc, hipStream_t stream, int f8_type) {
+  MI_REQUIRE(f8_type == MI_F8_E4M3 || f8_type == MI_F8_E5M2, MI_BAD_ARGUMENT, "mi_f8mm_launch: f8_type");
+  if (f8_type == MI_F8_E5M2) {  // MatMul.cpp:630-635: no scales on these arms
+    d_out_scales = nullptr;
+    out_scale = 1.0;
+  }
   MI_REQUIRE(M >= 0 && K > 0 && N > 0, MI_BAD_ARGUMENT, "mi_f8mm_launch: bad shape");
   MI_REQUIRE(M == 0 || (d_a && d_b && d_out), MI_BAD_ARGUMENT, "mi_f8mm_launch: null argument");
   MI_REQUIRE(out_kind >= MI_F8_OUT_CODES && out_kind <= MI_F8_OUT_F16, MI_BAD_ARGUMENT, "mi_f8mm_launch: out_kind");
@@ -595,15 +650,20 @@ int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, con
   a.step = (double)(float)(1 / out_scale);  // MatMul.cpp:613-615 into the float parameter of Float8.cpp:267
   a.inv_step = (float)(1.0 / a.step);
   a.scales = d_out_scales;
+  const bool e5m2 = f8_type == MI_F8_E5M2;
   const int64_t tiles_m = (M + F8_BM - 1) / F8_BM, tiles_n = (N + F8_BN - 1) / F8_BN;
   if ((K % F8_BK) == 0 && tiles_m * tiles_n < (int64_t(1) << 30)) {
     const int tiles = (int)(tiles_m * tiles_n), per_xcd = (tiles + 7) / 8;
     static bool attr_set = false;
     if (!attr_set) {
-      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                f8_ring_lds_bytes(8));
-      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                f8_ring_lds_bytes(4));
+      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<8, F8_FMT_E4M3>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, f8_ring_lds_bytes(8));
+      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<4, F8_FMT_E4M3>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, f8_ring_lds_bytes(4));
+      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<8, F8_FMT_E5M2>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, f8_ring_lds_bytes(8));
+      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<4, F8_FMT_E5M2>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, f8_ring_lds_bytes(4));
       attr_set = true;
     }
     const int64_t tl_m = (M + F8L_M - 1) / F8L_M, tl_n = (N + F8L_N - 1) / F8L_N;
@@ -612,22 +672,39 @@ int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, con
     if (large) {
       static bool attr_large = false;
       if (!attr_large) {
-        (void)hipFuncSetAttribute((const void *)f8_gemm_large_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  F8L_NST * F8L_STAGE);
+        (void)hipFuncSetAttribute((const void *)f8_gemm_large_kernel<F8_FMT_E4M3>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, F8L_NST * F8L_STAGE);
+        (void)hipFuncSetAttribute((const void *)f8_gemm_large_kernel<F8_FMT_E5M2>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, F8L_NST * F8L_STAGE);
         attr_large = true;
       }
       const int tl = (int)(tl_m * tl_n), pl = (tl + 7) / 8;
-      f8_gemm_large_kernel<<<dim3((unsigned)(pl * 8)), dim3(256), F8L_NST * F8L_STAGE, stream>>>(a, (int)tl_m, (int)tl_n,
-                                                                                              pl);
-    } else if (tiles <= 256)
-      f8_gemm_ring_kernel<8><<<dim3((unsigned)(per_xcd * 8)), dim3(256), f8_ring_lds_bytes(8), stream>>>(
-          a, (int)tiles_m, (int)tiles_n, per_xcd);
-    else
-      f8_gemm_ring_kernel<4><<<dim3((unsigned)(per_xcd * 8)), dim3(256), f8_ring_lds_bytes(4), stream>>>(
-          a, (int)tiles_m, (int)tiles_n, per_xcd);
+      const dim3 grid((unsigned)(pl * 8));
+      if (e5m2)
+        f8_gemm_large_kernel<F8_FMT_E5M2><<<grid, dim3(256), F8L_NST * F8L_STAGE, stream>>>(a, (int)tl_m, (int)tl_n, pl);
+      else
+        f8_gemm_large_kernel<F8_FMT_E4M3><<<grid, dim3(256), F8L_NST * F8L_STAGE, stream>>>(a, (int)tl_m, (int)tl_n, pl);
+    } else {
+      const dim3 grid((unsigned)(per_xcd * 8));
+      const int tm = (int)tiles_m, tn = (int)tiles_n;
+      if (tiles <= 256) {
+        if (e5m2)
+          f8_gemm_ring_kernel<8, F8_FMT_E5M2><<<grid, dim3(256), f8_ring_lds_bytes(8), stream>>>(a, tm, tn, per_xcd);
+        else
+          f8_gemm_ring_kernel<8, F8_FMT_E4M3><<<grid, dim3(256), f8_ring_lds_bytes(8), stream>>>(a, tm, tn, per_xcd);
+      } else {
+        if (e5m2)
+          f8_gemm_ring_kernel<4, F8_FMT_E5M2><<<grid, dim3(256), f8_ring_lds_bytes(4), stream>>>(a, tm, tn, per_xcd);
+        else
+          f8_gemm_ring_kernel<4, F8_FMT_E4M3><<<grid, dim3(256), f8_ring_lds_bytes(4), stream>>>(a, tm, tn, per_xcd);
+      }
+    }
   } else {
     dim3 grid((unsigned)tiles_n, (unsigned)tiles_m);
-    f8_gemm_kernel<<<grid, dim3(256), 0, stream>>>(a);
+    if (e5m2)
+      f8_gemm_kernel<F8_FMT_E5M2><<<grid, dim3(256), 0, stream>>>(a);
+    else
+      f8_gemm_kernel<F8_FMT_E4M3><<<grid, dim3(256), 0, stream>>>(a);
   }
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;

@@ -86,7 +86,7 @@ int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int6
 // tpu.MatMul on F8E4M3 codes with the F8 output requantization (f8_kernels.hip)
 int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, const float *d_bias, int64_t M, int64_t K,
                 int64_t N, int do_relu, double relu_limit, double out_scale, const double *d_out_scales, int out_kind,
-                void *d_out, float *d_acc, hipStream_t stream);
+                void *d_out, float *d_acc, hipStream_t stream, int f8_type = MI_F8_E4M3);
 
 int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
                      int64_t N, int q_group_size, int dq_type, int dtype, uint16_t *d_y, float *d_y32,

@@ -334,15 +334,17 @@ def matmul_dq_launch(left, right, *, right_transpose=False, q_group_size, dq_typ
     return y
 
 
-def matmul_f8(left, right, bias=None, *, right_transpose=False, do_relu=False, relu_limit=-1.0, out_scales=(1.0,)):
+def matmul_f8(left, right, bias=None, *, right_transpose=False, do_relu=False, relu_limit=-1.0, out_scales=(1.0,),
+              f8_type=clib.F8_E4M3):
     """tpu.MatMul on operands holding E4M3 values with the F8 output requantization, interpreter convention (float32
-    numpy in and out; the output holds E4M3 values).  out_scales: one scale or one per output channel."""
+    numpy in and out; the output holds E4M3 values).  out_scales: one scale or one per output channel.
+    f8_type=F8_E5M2: operands and output hold E5M2 values; no scales."""
     left, right = _f32(left), _f32(right)
     M, K = left.shape
     N = right.shape[0] if right_transpose else right.shape[1]
     sc = np.ascontiguousarray(out_scales, dtype=np.float64).reshape(-1)
     attr = clib.F8MMAttr(M, K, N, int(right_transpose), int(do_relu), float(relu_limit),
-                         sc.ctypes.data_as(C.POINTER(C.c_double)), sc.size)
+                         sc.ctypes.data_as(C.POINTER(C.c_double)), sc.size, int(f8_type))
     y = np.empty((M, N), dtype=np.float32)
     ins = [left, right] + ([] if bias is None else [_f32(bias)])
     p = _Param(ins, [y])
@@ -351,10 +353,11 @@ def matmul_f8(left, right, bias=None, *, right_transpose=False, do_relu=False, r
 
 
 def f8mm_launch(a_codes, b_codes, bias=None, *, right_transpose=False, do_relu=False, relu_limit=-1.0, out_scale=1.0,
-                out_scales=None, out_kind=clib.F8_OUT_CODES, acc_f32=None, out=None, stream=None):
+                out_scales=None, out_kind=clib.F8_OUT_CODES, acc_f32=None, out=None, stream=None, f8_type=clib.F8_E4M3):
     """Device level: a_codes [M, K], b_codes [K, N] ([N, K] when right_transpose) uint8 CUDA tensors of E4M3 codes; bias
     float32 [N]; out_scales float64 [N] CUDA tensor for per-channel requantization.  Returns the output tensor (uint8
-    codes, or the values as float32 / bfloat16 / float16 by out_kind)."""
+    codes, or the values as float32 / bfloat16 / float16 by out_kind).  f8_type=F8_E5M2: E5M2 codes in, no scales, the
+    16-bit kinds are the plain roundings of the fp32 value."""
     import torch
     if not (a_codes.is_cuda and b_codes.is_cuda and a_codes.dtype == torch.uint8 and b_codes.dtype == torch.uint8
             and a_codes.is_contiguous() and b_codes.is_contiguous() and a_codes.dim() == 2 and b_codes.dim() == 2):
@@ -376,6 +379,11 @@ def f8mm_launch(a_codes, b_codes, bias=None, *, right_transpose=False, do_relu=F
     y = torch.empty((M, N), dtype=tdt, device=a_codes.device) if out is None else out
     if not (y.is_cuda and y.dtype == tdt and y.is_contiguous() and y.numel() == M * N):
         raise clib.BackendError(clib.MI_BAD_ARGUMENT, "f8mm_launch: bad output tensor")
+    if f8_type == clib.F8_E5M2:
+        check(clib.lib().mi_f8mm_e5m2_launch(_dptr(a_codes), _dptr(b_codes), int(right_transpose), _dptr(bias), M, K, N,
+                                             int(do_relu), float(relu_limit), out_kind, _dptr(y), _dptr(acc_f32),
+                                             _stream_ptr(stream)))
+        return y
     check(clib.lib().mi_f8mm_launch(_dptr(a_codes), _dptr(b_codes), int(right_transpose), _dptr(bias), M, K, N,
                                     int(do_relu), float(relu_limit), float(out_scale), _dptr(out_scales), out_kind,
                                     _dptr(y), _dptr(acc_f32), _stream_ptr(stream)))
