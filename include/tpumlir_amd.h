@@ -206,6 +206,11 @@ typedef struct mi_a16_quant_desc {
                       * MI_DQ_F8E4M3 (8-bit) and MI_DQ_F4 (4-bit) store float codes: scale = |absmax| / 448 or / 6,
                       * zp = 0, code = f32_to_f8e4m3(w / scale, saturating) or f32_to_f4e2m1(w / scale)
                       * (Canonicalize/A16MatMul.cpp:96-106, :179-209) */
+  int zp_float;      /* 1: the float-zero-point overloads that module::isSG2380() and use_dq2 (:287-295) select
+                      * (computePerChannelParam :50-77, computePerGroupParam :119-141, weightQuantization :218-268):
+                      * the same scales and zero points, zp written as [N, G] 16-bit patterns of dtype (:397-404, the
+                      * zp argument then points to uint16_t), and per channel code = round((w + zp) / scale).
+                      * Integer codes only. */
 } mi_a16_quant_desc;
 /* A16MatMulAdjust (lib/Dialect/Tpu/Canonicalize/A16MatMul.cpp:270-429; computePerChannelParam :22-48,
  * computePerGroupParam :78-115, weightQuantization :147-216; static quantization, uint8 zero points).

@@ -1359,9 +1359,41 @@ int orc_a16_quantize(const float *w_kn, int64_t K, int64_t N, int bits, int g, i
                              weight_signed_out);
 }
 
+static int a16_quantize_impl(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16,
+                             int dq_type, int zp_float, uint8_t *q, float *scale_f32, uint16_t *scale16, uint8_t *zp,
+                             int *sign_out, int *weight_signed_out);
+
 int orc_a16_quantize_dq(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16, int dq_type,
                         uint8_t *q, float *scale_f32, uint16_t *scale16, uint8_t *zp, int *sign_out,
                         int *weight_signed_out) {
+  return a16_quantize_impl(w_kn, K, N, bits, g, symmetric, f16, dq_type, 0, q, scale_f32, scale16, zp, sign_out,
+                           weight_signed_out);
+}
+
+/* The float-zero-point overloads that SG2380 (and CV184X / SGTPUV8 with 4-bit weights in groups of a multiple of 32,
+ * use_dq2 :287-295) select: computePerChannelParam :50-77 and computePerGroupParam :119-141 produce the same numbers
+ * with the zero point held as a float, which :397-404 then stores in the activation's 16-bit type; weightQuantization
+ * :218-268 is the same for groups and writes round((w + zp) / scale) per channel (:230-231). */
+int orc_a16_quantize_fzp(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16, uint8_t *q,
+                         float *scale_f32, uint16_t *scale16, uint16_t *zp16, int *sign_out, int *weight_signed_out) {
+  if (K <= 0 || N <= 0 || g < -1)
+    return -1;
+  const int64_t gs = g == -1 ? K : g;
+  const int64_t count = N * (gs ? K / gs : 1);
+  uint8_t *zp = (uint8_t *)malloc((size_t)(count > 0 ? count : 1));
+  if (!zp)
+    return -1;
+  const int rc = a16_quantize_impl(w_kn, K, N, bits, g, symmetric, f16, ORC_DQ_INT, 1, q, scale_f32, scale16, zp,
+                                   sign_out, weight_signed_out);
+  for (int64_t i = 0; rc == 0 && i < count; ++i)
+    zp16[i] = f16 ? orc_f32_to_f16((float)zp[i]) : orc_f32_to_bf16((float)zp[i], 0);
+  free(zp);
+  return rc;
+}
+
+static int a16_quantize_impl(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16,
+                             int dq_type, int zp_float, uint8_t *q, float *scale_f32, uint16_t *scale16, uint8_t *zp,
+                             int *sign_out, int *weight_signed_out) {
   if ((bits != 4 && bits != 8) || K <= 0 || N <= 0 || (bits == 4 && (K & 1)))
     return -1;
   /* the float code types exist only on the per-group path (computePerGroupParam :78-115 takes dq_type,
@@ -1439,6 +1471,8 @@ int orc_a16_quantize_dq(const float *w_kn, int64_t K, int64_t N, int bits, int g
       if (dq_type == ORC_DQ_INT) /* :181-182: the float code types keep the quotient unrounded */
         t = roundf(t);
       t += (float)zp[qi];
+      if (zp_float && !gs) /* :230-231, the per-channel arm of the float-zero-point overload */
+        t = roundf((w[c * col + i] + (float)zp[qi]) / scale_f32[qi]);
       if (dq_type == ORC_DQ_F8E4M3) { /* :185-186 */
         q[c * col + i] = orc_f32_to_f8e4m3(t, 1);
       } else if (dq_type == ORC_DQ_F4) { /* :194-200 */

@@ -41,6 +41,9 @@
  *                                IEEE half) on all codes, all bf16 patterns, every tie and its neighbours, overflow
  *                                to infinity at 61440 (tests/test_oracle_float_codes.py)
  *   orc_matmul_f8e5m2            float64 product of numpy-decoded operands, rounded by torch / numpy casts
+ *   orc_a16_quantize_fzp         equal to orc_a16_quantize in groups (zero points as exact 16-bit floats); per channel
+ *                                a numpy closed form of round((w + zp) / scale) on a case where it differs from
+ *                                round(w / scale) + zp (tests/test_oracle_packers.py)
  *   orc_a16_quantize_dq          closed-form scale, zp = 0, on-grid recovery, half-spacing bound
  *   orc_a16_quantize             on-grid weights are recovered exactly, |w - dequant(q)| <= scale/2 inside the
  *                                clamp range, closed-form scale/zp, nibble order via the A16MatMul dequantizer
@@ -302,6 +305,11 @@ int orc_a16_quantize(const float *w_kn, int64_t K, int64_t N, int bits, int g, i
  * without integer rounding (:179-209).  ORC_DQ_INT is orc_a16_quantize. */
 int orc_a16_quantize_dq(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16, int dq_type,
                         uint8_t *q, float *scale_f32, uint16_t *scale16, uint8_t *zp, int *sign, int *weight_signed);
+/* The float-zero-point overloads (SG2380; use_dq2 on CV184X / SGTPUV8, :287-295): same scales and zero points, the
+ * zero point stored in the 16-bit activation type (:397-404); per channel the code is round((w + zp) / scale)
+ * (:230-231), in groups round(w / scale) + zp as before (:250-252). */
+int orc_a16_quantize_fzp(const float *w_kn, int64_t K, int64_t N, int bits, int g, int symmetric, int f16, uint8_t *q,
+                         float *scale_f32, uint16_t *scale16, uint16_t *zp16, int *sign, int *weight_signed);
 
 /* GPTQ / AWQ checkpoints -> the [N, K/2] + [N, G] layout, python/llm/LlmConverter.py:320-389 (unpack_weights) and
  * :1454-1475 (the transposes).  qweight: GPTQ int32 [K*bits/32, N] (packed along K), AWQ int32 [K, N*bits/32]

@@ -420,11 +420,12 @@ def matmul_f8e5m2(left, right, bias=None, *, right_transpose=False, do_relu=Fals
     return out, acc
 
 
-def a16_quantize(w_kn, *, bits, g, symmetric=False, f16=False, dq_type=DQ_INT):
+def a16_quantize(w_kn, *, bits, g, symmetric=False, f16=False, dq_type=DQ_INT, zp_float=False):
     """A16MatMulAdjust on the f32 weight [K, N] of a top-level matmul.
 
     Returns dict(weight [N, K/2] or [N, K] uint8 (int8 bit patterns when weight_signed), scale_f32 [N, G],
-    scale16 [N, G] bit patterns, zp [N, G] uint8, sign, weight_signed).
+    scale16 [N, G] bit patterns, zp [N, G] uint8, sign, weight_signed).  zp_float: the float-zero-point overloads
+    (SG2380 / use_dq2); zp then holds [N, G] uint16 bit patterns of the activation type.
     """
     w = np.ascontiguousarray(w_kn, dtype=np.float32)
     K, N = w.shape
@@ -436,6 +437,17 @@ def a16_quantize(w_kn, *, bits, g, symmetric=False, f16=False, dq_type=DQ_INT):
     zp = np.zeros((N, G), dtype=np.uint8)
     sign, wsigned = C.c_int(0), C.c_int(0)
     L = lib()
+    if zp_float:
+        if dq_type != DQ_INT:
+            raise RuntimeError("orc_a16_quantize_fzp: integer codes only")
+        zp = np.zeros((N, G), dtype=np.uint16)
+        L.orc_a16_quantize_fzp.restype = C.c_int
+        rc = L.orc_a16_quantize_fzp(_p(w, C.c_float), C.c_int64(K), C.c_int64(N), C.c_int(bits), C.c_int(g),
+                                    C.c_int(int(symmetric)), C.c_int(int(f16)), _p(q, C.c_uint8), _p(sf, C.c_float),
+                                    _p(s16, C.c_uint16), _p(zp, C.c_uint16), C.byref(sign), C.byref(wsigned))
+        if rc != 0:
+            raise RuntimeError("orc_a16_quantize_fzp: bad arguments")
+        return dict(weight=q, scale_f32=sf, scale16=s16, zp=zp, sign=bool(sign.value), weight_signed=bool(wsigned.value))
     L.orc_a16_quantize_dq.restype = C.c_int
     rc = L.orc_a16_quantize_dq(_p(w, C.c_float), C.c_int64(K), C.c_int64(N), C.c_int(bits), C.c_int(g),
                             C.c_int(int(symmetric)), C.c_int(int(f16)), C.c_int(dq_type), _p(q, C.c_uint8), _p(sf, C.c_float),

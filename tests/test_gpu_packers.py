@@ -230,3 +230,33 @@ def test_to_group_and_run(orc):
     with pytest.raises(clib.BackendError) as e:
         M_.a16_to_group(r["scale_bits"], r["zp"], K=200)
     assert e.value.code == clib.MI_UNSUPPORTED
+
+
+FLOAT_ZP_CASES = [  # (bits, K, N, g, symmetric, dtype is f16, kind)
+    (4, 512, 70, 64, False, False, "normal"), (4, 256, 48, 32, True, False, "normal"), (4, 384, 33, 0, False, False, "normal"),
+    (4, 200, 17, 0, False, True, "normal"), (8, 512, 96, 128, False, True, "normal"), (8, 384, 70, 0, False, False, "normal"),
+    (4, 256, 24, 128, False, False, "flat"), (4, 256, 24, 0, False, False, "flat"), (8, 256, 40, 64, True, False, "normal"),
+]
+
+
+@pytest.mark.parametrize("bits,K,N,g,sym,f16,kind", FLOAT_ZP_CASES)
+def test_float_zero_point_quantizer_matches_oracle_bit_for_bit(orc, bits, K, N, g, sym, f16, kind):
+    """The SG2380 / use_dq2 overloads: zero points as 16-bit float patterns, per-channel codes round((w + zp) / scale)."""
+    w = _weights(bits * 77 + K + N, K, N, kind)
+    want = orc.a16_quantize(w, bits=bits, g=g, symmetric=sym, f16=f16, zp_float=True)
+    got = M_.a16_quantize(w, weight_bits=bits, q_group_size=g, symmetric=sym, dtype=clib.DT_F16 if f16 else clib.DT_BF16,
+                          zp_float=True)
+    assert got["sign"] == want["sign"] and got["weight_signed"] == want["weight_signed"]
+    assert np.array_equal(got["scale_bits"], want["scale16"])
+    assert got["zp"].dtype == np.uint16 and np.array_equal(got["zp"], want["zp"])
+    assert np.array_equal(got["weight"].view(np.uint8), want["weight"])
+    if bits == 4 and g == 0:  # the arm that differs from the integer-zero-point overload really is exercised
+        plain = M_.a16_quantize(w, weight_bits=bits, q_group_size=g, symmetric=sym)
+        assert not np.array_equal(plain["weight"], got["weight"])
+
+
+def test_float_zero_point_rejects_float_codes():
+    w = _weights(3, 256, 16)
+    with pytest.raises(clib.BackendError) as e:
+        M_.a16_quantize(w, weight_bits=8, q_group_size=64, dq_type=clib.DQ_F8E4M3, zp_float=True)
+    assert e.value.code == clib.MI_UNSUPPORTED

@@ -215,3 +215,43 @@ def test_to_group_repeats_and_keeps_the_product(orc, bits):
     assert np.array_equal(a, b)
     with pytest.raises(RuntimeError):
         orc.a16_to_group(r["scale16"], r["zp"], 200)
+
+
+# ---- float-zero-point overloads (SG2380 / use_dq2, Canonicalize/A16MatMul.cpp:50-77, :119-141, :218-268) ---------
+@pytest.mark.parametrize("bits,g,sym,f16", [(4, 32, False, False), (4, 128, True, False), (8, 64, False, True),
+                                            (8, 0, False, False), (4, -1, False, True)])
+def test_float_zp_equals_integer_zp_where_the_overloads_agree(orc, bits, g, sym, f16):
+    """In groups (and per channel with 8-bit weights, whose zero point is 0) both overloads compute the same numbers;
+    only the zero point's storage differs: the integer as an exact 16-bit float."""
+    rng = np.random.default_rng(40 + bits + g)
+    w = (rng.standard_normal((256, 20)) * 0.05).astype(np.float32)
+    a = orc.a16_quantize(w, bits=bits, g=g, symmetric=sym, f16=f16)
+    b = orc.a16_quantize(w, bits=bits, g=g, symmetric=sym, f16=f16, zp_float=True)
+    assert np.array_equal(a["weight"], b["weight"]) and np.array_equal(a["scale16"], b["scale16"])
+    assert a["sign"] == b["sign"] and a["weight_signed"] == b["weight_signed"]
+    as_float = b["zp"].view(np.float16).astype(np.float32) if f16 else S.bf16_to_f32(b["zp"])
+    assert np.array_equal(as_float, a["zp"].astype(np.float32))
+    assert b["zp"].dtype == np.uint16
+
+
+def test_float_zp_per_channel_w4_adds_before_dividing(orc):
+    """Per channel with 4-bit weights the overload writes round((w + zp) / scale) (:230-231).  Closed form on numbers
+    where every step is exact: scale 2^-4 (min -0.5, max 0.4375 = 15 steps), so zp = 8 and
+    code = round_half_away(16 w + 128) clamped to 0..15 -- 15 for every w above -7, which no other reading of the
+    line produces; the integer-zp overload gives round(16 w) + 8 on the same weights."""
+    K, N = 32, 3
+    steps = np.arange(-8, 8, dtype=np.float32)                  # -8 .. 7 in units of 2^-4: both extremes present
+    w_nk = np.stack([np.tile(steps, 2), np.tile(steps[::-1], 2), np.tile(steps, 2)]) * np.float32(2.0 ** -4)
+    w_nk[2] *= np.float32(2.0 ** -10)                           # a row with a tiny scale: (w + zp) / scale is huge
+    w = np.ascontiguousarray(w_nk.T)
+    r = orc.a16_quantize(w, bits=4, g=0, zp_float=True)
+    base = orc.a16_quantize(w, bits=4, g=0)
+    assert np.array_equal(S.bf16_to_f32(r["zp"]), base["zp"].astype(np.float32)) and np.all(base["zp"] == 8)
+    assert np.array_equal(r["scale16"], base["scale16"])
+    sc = base["scale_f32"][:, 0].astype(np.float64)
+    t = (w_nk.astype(np.float64) + 8.0) / sc[:, None]           # exact: every operand is a small dyadic number
+    code = np.clip(np.sign(t) * np.floor(np.abs(t) + 0.5), 0, 15).astype(np.uint8)
+    assert np.array_equal(_unpack4(r["weight"]), code)
+    assert np.all(code[0] == 15) and np.all(code[2] == 15)      # 16 w + 128 >= 120: always clamped
+    assert np.array_equal(_unpack4(base["weight"])[0], (np.tile(steps, 2) + 8).astype(np.uint8))
+    assert not np.array_equal(r["weight"], base["weight"])

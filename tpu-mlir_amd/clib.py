@@ -74,7 +74,7 @@ F8_E4M3, F8_E5M2 = 0, 1
 
 class A16QuantDesc(C.Structure):
     _fields_ = [("K", C.c_int64), ("N", C.c_int64), ("weight_bits", C.c_int), ("q_group_size", C.c_int),
-                ("symmetric", C.c_int), ("dtype", C.c_int), ("dq_type", C.c_int)]
+                ("symmetric", C.c_int), ("dtype", C.c_int), ("dq_type", C.c_int), ("zp_float", C.c_int)]
 
 
 class I8Attr(C.Structure):

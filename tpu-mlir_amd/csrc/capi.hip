@@ -321,6 +321,8 @@ int mi_a16_quantize(const mi_a16_quant_desc *d, const float *w_kn, void *weight,
                  (gs != 0 && ((d->dq_type == MI_DQ_F8E4M3 && d->weight_bits == 8) ||
                               (d->dq_type == MI_DQ_F4 && d->weight_bits == 4))),
              MI_UNSUPPORTED, "mi_a16_quantize: float code types need groups, F8E4M3 8-bit and F4 4-bit weights");
+  MI_REQUIRE(!d->zp_float || d->dq_type == MI_DQ_NONE || d->dq_type == MI_DQ_INT, MI_UNSUPPORTED,
+             "mi_a16_quantize: float zero points go with integer codes only");
   MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_a16_quantize: no GPU visible");
   return a16_quantize(d, w_kn, weight, scale16, scale_f32, zp, sign, weight_signed);
 }

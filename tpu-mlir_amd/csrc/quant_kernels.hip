@@ -98,7 +98,7 @@ __global__ void quant_params_kernel(const float *__restrict__ mn, const float *_
 constexpr int QT = 64;
 __global__ __launch_bounds__(256) void quant_pack_kernel(const float *__restrict__ w_kn, int64_t K, int64_t N,
                                                           int64_t gs, int64_t G, int bits, int as_int8, int dq_type,
-                                                          const float *__restrict__ scale,
+                                                          int zp_float, const float *__restrict__ scale,
                                                           const uint8_t *__restrict__ zp, uint8_t *__restrict__ q) {
   __shared__ uint8_t tile[QT][QT + 4];  // [k][n]
   const int64_t n0 = (int64_t)blockIdx.x * QT, k0 = (int64_t)blockIdx.y * QT;
@@ -112,6 +112,8 @@ __global__ __launch_bounds__(256) void quant_pack_kernel(const float *__restrict
       if (dq_type != MI_DQ_F8E4M3 && dq_type != MI_DQ_F4)
         t = roundf(t);  // :181-182: the float code types keep the quotient
       t += (float)zp[qi];
+      if (zp_float && !gs)  // :230-231: the per-channel arm of the float-zero-point overload adds before dividing
+        t = roundf((w_kn[k * N + n] + (float)zp[qi]) / scale[qi]);
       const int64_t v = to_int_f32(t, MI_ROUND_HALF_AWAY_FROM_ZERO);  // to_uint4 / to_uint8 / to_int8
       if (dq_type == MI_DQ_F8E4M3) {
         code = (uint8_t)f8e4m3_from_f32(t);  // :185-186, saturating
@@ -256,13 +258,31 @@ int a16_quantize(const mi_a16_quant_desc *d, const float *h_w_kn, void *h_weight
   MI_HIP(hipMemcpy(&sign, d_sign, 4, hipMemcpyDeviceToHost));
   const int as_int8 = !gs && sign && bits == 8;  // :413-416
   quant_pack_kernel<<<dim3((unsigned)((N + QT - 1) / QT), (unsigned)((K + QT - 1) / QT)), dim3(256)>>>(
-      d_w, K, N, gs, G, bits, as_int8, d->dq_type, d_scale, d_zp, d_q);
+      d_w, K, N, gs, G, bits, as_int8, d->dq_type, d->zp_float, d_scale, d_zp, d_q);
   MI_HIP(hipGetLastError());
   MI_HIP(hipMemcpy(h_weight, d_q, qbytes, hipMemcpyDeviceToHost));
   MI_HIP(hipMemcpy(h_scale16, d_s16, (size_t)count * 2, hipMemcpyDeviceToHost));
   if (h_scale_f32)
     MI_HIP(hipMemcpy(h_scale_f32, d_scale, (size_t)count * 4, hipMemcpyDeviceToHost));
-  MI_HIP(hipMemcpy(h_zp, d_zp, (size_t)count, hipMemcpyDeviceToHost));
+  if (d->zp_float) {  // :397-404: the zero points (integers up to 255: exact in both types) in the activation's type
+    std::vector<uint8_t> z((size_t)count);
+    MI_HIP(hipMemcpy(z.data(), d_zp, (size_t)count, hipMemcpyDeviceToHost));
+    uint16_t *z16 = (uint16_t *)h_zp;
+    for (int64_t i = 0; i < count; ++i) {
+      const uint32_t v = z[(size_t)i];
+      int e = 0;
+      while ((v >> e) > 1)
+        ++e;
+      if (v == 0)
+        z16[i] = 0;
+      else if (d->dtype == MI_DT_F16)
+        z16[i] = (uint16_t)(((uint32_t)(e + 15) << 10) | ((v << (10 - e)) & 0x3ffu));
+      else
+        z16[i] = (uint16_t)(((uint32_t)(e + 127) << 7) | ((v << 7 >> e) & 0x7fu));
+    }
+  } else {
+    MI_HIP(hipMemcpy(h_zp, d_zp, (size_t)count, hipMemcpyDeviceToHost));
+  }
   if (sign_out)
     *sign_out = sign;
   if (weight_signed_out)

@@ -241,12 +241,14 @@ class A16Weight:
 PACK_GPTQ, PACK_AWQ = 0, 1
 
 
-def a16_quantize(w_kn, *, weight_bits, q_group_size, symmetric=False, dtype=DT_BF16, dq_type=clib.DQ_NONE):
+def a16_quantize(w_kn, *, weight_bits, q_group_size, symmetric=False, dtype=DT_BF16, dq_type=clib.DQ_NONE,
+                 zp_float=False):
     """A16MatMulAdjust on the GPU: f32 weight [K, N] of a top-level matmul -> the operand set of tpu.A16MatMul.
 
     Returns dict(weight uint8/int8 [N, K/2] or [N, K], scale_bits uint16 [N, G], scale_f32 [N, G], zp uint8 [N, G],
     sign, weight_signed); weight/scale_bits/zp are what A16Weight takes.  dq_type DQ_F8E4M3 (8-bit) / DQ_F4 (4-bit)
     store the float codes of the matching dynamic-quantization types instead of integers (groups only).
+    zp_float: the float-zero-point overloads (SG2380 / use_dq2): zp comes back as uint16 bit patterns of dtype.
     """
     w = np.ascontiguousarray(w_kn, dtype=np.float32)
     if w.ndim != 2:
@@ -259,9 +261,9 @@ def a16_quantize(w_kn, *, weight_bits, q_group_size, symmetric=False, dtype=DT_B
     q = np.zeros((N, K // 2 if weight_bits == 4 else K), dtype=np.uint8)
     s16 = np.zeros((N, G), dtype=np.uint16)
     sf = np.zeros((N, G), dtype=np.float32)
-    zp = np.zeros((N, G), dtype=np.uint8)
+    zp = np.zeros((N, G), dtype=np.uint16 if zp_float else np.uint8)
     sign, wsigned = C.c_int(0), C.c_int(0)
-    desc = clib.A16QuantDesc(K, N, weight_bits, q_group_size, int(symmetric), dtype, int(dq_type))
+    desc = clib.A16QuantDesc(K, N, weight_bits, q_group_size, int(symmetric), dtype, int(dq_type), int(bool(zp_float)))
     check(clib.lib().mi_a16_quantize(C.byref(desc), w.ctypes.data, q.ctypes.data, s16.ctypes.data, sf.ctypes.data,
                                      zp.ctypes.data, C.byref(sign), C.byref(wsigned)))
     if wsigned.value:
