@@ -404,6 +404,18 @@ typedef struct mi_module_i8_desc {
 } mi_module_i8_desc;
 /* quantized tpu.MatMul (+ fused requant): input int8/uint8 [M,K] */
 int mi_module_add_matmul_int8(mi_module *m, const char *input, const char *output, const mi_module_i8_desc *desc);
+/* tpu.RequantIntAxis / tpu.RequantInt between two tensors of the module: int32 [outer, channels, inner] -> the narrow
+ * integer type of rq.out_dtype, as mi_requant_launch; rq.d_* per-channel arrays are HOST pointers here */
+typedef struct mi_module_rq_desc {
+  int64_t outer, channels, inner;
+  int64_t input_zp;
+  mi_requant_desc rq;
+} mi_module_rq_desc;
+int mi_module_add_requant(mi_module *m, const char *input, const char *output, const mi_module_rq_desc *desc);
+/* tpu.MatMul of two activations under module::isDynamicQuantize() (MatMul.cpp:447-597), as mi_matmul_dq_launch:
+ * left [M, K], right [K, N] ([N, K] when right_transpose), output [M, N], all of one 16-bit float type */
+int mi_module_add_matmul_dq(mi_module *m, const char *left, const char *right, const char *output, int64_t K,
+                            int64_t N, int right_transpose, int q_group_size, int dq_type);
 /* tpu.Cast between two tensors of the module */
 int mi_module_add_cast(mi_module *m, const char *input, const char *output, const mi_cast_attr *attr);
 /* float data in (converted on the device to the tensor's storage), as py_cuda::set_tensor */

@@ -95,6 +95,77 @@ def test_int8_pipeline_bit_exact(orc):
     m.destroy()
 
 
+def test_int8_matmul_with_a_standalone_requant_op(orc):
+    """The unfused form of the same pipeline: INT8 MatMul leaving int32, then tpu.RequantIntAxis as its own op (per
+    channel Q31 multipliers, half away from zero), then a per-tensor tpu.RequantInt (MultiplierShift, half up) of the
+    same accumulators into a second tensor -- both must equal the fused result / the oracle bit for bit."""
+    M, K, N = 20, 256, 96
+    c = S.int8_matmul(M, K, N, seed=312, qdm=True)
+    rng = np.random.default_rng(5)
+    xq = rng.integers(-128, 128, size=(M, K)).astype(np.float32)
+    zps = np.full(N, 3, dtype=np.int32)
+    m = M_.Module()
+    m.add_tensor("xq", clib.ST_I8, (M, K)).add_tensor("acc", clib.ST_I32, (M, N))
+    m.add_tensor("yq", clib.ST_I8, (M, N)).add_tensor("yfused", clib.ST_I8, (M, N)).add_tensor("y16", clib.ST_I16, (M, N))
+    m.add_matmul_int8("xq", "acc", c["b"], c["bias"], K=K, N=N)
+    m.add_requant("acc", "yq", outer=M, channels=N, quant_mode=clib.RQ_QDM, multiplier=c["mult"], shift=c["shift"], zp=zps)
+    m.add_requant("acc", "y16", channels=1, inner=M * N, quant_mode=clib.RQ_MULTIPLIER_SHIFT,
+                  round_mode=clib.ROUND_HALF_UP, out_dtype=clib.DT_I16, multiplier=5, shift=9, zp=-2)
+    m.add_matmul_int8("xq", "yfused", c["b"], c["bias"], K=K, N=N, quant_mode=clib.RQ_QDM, multiplier=c["mult"],
+                      shift=c["shift"], zp=zps)
+    for rep in range(3):
+        x = np.roll(xq, rep, axis=0)
+        m.set_tensor("xq", x)
+        m.invoke()
+        acc = x.astype(np.int64) @ c["b"].astype(np.int64) + c["bias"].astype(np.int64)
+        assert np.array_equal(m.get_tensor("acc"), acc.astype(np.float32))
+        v = orc.mbqm(acc, np.broadcast_to(c["mult"].astype(np.int64), acc.shape),
+                     np.broadcast_to(-c["shift"].astype(np.int64), acc.shape), orc.HALF_AWAY_FROM_ZERO)
+        yq = np.clip(v.astype(np.int64) + 3, -128, 127).astype(np.float32)
+        assert np.array_equal(m.get_tensor("yq"), yq)
+        assert np.array_equal(m.get_tensor("yfused"), yq)
+        y16 = np.clip(np.floor((acc * 5 + 256) / 512.0).astype(np.int64) - 2, -32768, 32767).astype(np.float32)
+        assert np.array_equal(m.get_tensor("y16"), y16)
+    assert m.uses_graph()
+    with pytest.raises(clib.BackendError):   # the input of a requant is an int32 tensor
+        m.add_requant("xq", "yq", channels=N, outer=M, quant_mode=clib.RQ_QDM)
+    with pytest.raises(clib.BackendError):   # output storage must be the requant's type
+        m.add_requant("acc", "yq", channels=N, outer=M, quant_mode=clib.RQ_QDM, out_dtype=clib.DT_I16)
+    m.destroy()
+
+
+@pytest.mark.parametrize("dq,imax,rt", [("DQ_INT8", 127, True), ("DQ_INT4", 7, False)])
+def test_two_activation_matmul_with_dynamic_quantization_in_a_module(orc, dq, imax, rt):
+    """Two f32 inputs cast to bf16, then tpu.MatMul with both operands quantized per group on the fly (the form an
+    attention score product takes under module::isDynamicQuantize()); integer codes: bit for bit, eager and replayed."""
+    M, K, N, g = 9, 256, 40, 64
+    rng = np.random.default_rng(21)
+    m = M_.Module()
+    rshape = (N, K) if rt else (K, N)
+    m.add_tensor("a32", clib.ST_F32, (M, K)).add_tensor("b32", clib.ST_F32, rshape)
+    m.add_tensor("a", clib.ST_BF16, (M, K)).add_tensor("b", clib.ST_BF16, rshape).add_tensor("y", clib.ST_BF16, (M, N))
+    m.add_cast("a32", "a", in_type=clib.ST_F32, out_type=clib.ST_BF16)
+    m.add_cast("b32", "b", in_type=clib.ST_F32, out_type=clib.ST_BF16)
+    m.add_matmul_dq("a", "b", "y", K=K, N=N, right_transpose=rt, q_group_size=g, dq_type=getattr(clib, dq))
+    for rep in range(3):
+        a32 = (rng.standard_normal((M, K)) * (1 + rep)).astype(np.float32)
+        b32 = rng.standard_normal(rshape).astype(np.float32)
+        m.set_tensor("a32", a32)
+        m.set_tensor("b32", b32)
+        m.invoke()
+        a, b = S.bf16_to_f32(orc.f32_to_bf16(a32)), S.bf16_to_f32(orc.f32_to_bf16(b32))
+        want, _ = orc.matmul_dynamic(a, b, right_transpose=rt, q_group_size=g, imax=imax)
+        assert np.array_equal(orc.f32_to_bf16(m.get_tensor("y")), orc.f32_to_bf16(want))
+    assert m.uses_graph()
+    with pytest.raises(clib.BackendError) as e:
+        m.add_matmul_dq("a", "b", "y", K=K, N=N, right_transpose=rt, q_group_size=48, dq_type=getattr(clib, dq))
+    assert e.value.code == clib.MI_UNSUPPORTED
+    with pytest.raises(clib.BackendError) as e:
+        m.add_matmul_dq("a", "b", "a32", K=K, N=N, right_transpose=rt, q_group_size=g, dq_type=getattr(clib, dq))
+    assert e.value.code == clib.MI_BAD_ARGUMENT
+    m.destroy()
+
+
 def test_argument_errors():
     m = M_.Module()
     m.add_tensor("a", clib.ST_BF16, (2, 128))

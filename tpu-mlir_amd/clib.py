@@ -26,7 +26,7 @@ EXPORTS = [
     "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
     "mi_cast_inference", "mi_cast_launch",
     "mi_module_create", "mi_module_destroy", "mi_module_add_tensor", "mi_module_add_a16matmul", "mi_module_add_a16matmul_dq",
-    "mi_module_add_matmul_int8", "mi_module_add_cast", "mi_module_set_tensor", "mi_module_invoke",
+    "mi_module_add_matmul_int8", "mi_module_add_requant", "mi_module_add_matmul_dq", "mi_module_add_cast", "mi_module_set_tensor", "mi_module_invoke",
     "mi_module_uses_graph", "mi_module_get_tensor",
 ]
 
@@ -111,6 +111,11 @@ class ModuleI8Desc(C.Structure):
                 ("do_relu", C.c_int), ("relu_limit", C.c_int64), ("has_requant", C.c_int), ("rq", RequantDescC)]
 
 
+class ModuleRqDesc(C.Structure):
+    _fields_ = [("outer", C.c_int64), ("channels", C.c_int64), ("inner", C.c_int64), ("input_zp", C.c_int64),
+                ("rq", RequantDescC)]
+
+
 class CastAttr(C.Structure):
     _fields_ = [("num_elem", C.c_int64), ("in_type", C.c_int), ("out_type", C.c_int), ("in_quant", C.c_int),
                 ("out_quant", C.c_int), ("scale", C.c_double), ("zero_point", C.c_int64), ("expressed", C.c_int),
@@ -178,6 +183,9 @@ def lib():
                                                  C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_module_add_matmul_int8.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(ModuleI8Desc)]
         L.mi_module_add_cast.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(CastAttr)]
+        L.mi_module_add_matmul_dq.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_char_p, C.c_int64, C.c_int64,
+                                              C.c_int, C.c_int, C.c_int]
+        L.mi_module_add_requant.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(ModuleRqDesc)]
         L.mi_module_set_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int64]
         L.mi_module_invoke.argtypes = [C.c_void_p]
         L.mi_module_uses_graph.argtypes = [C.c_void_p]

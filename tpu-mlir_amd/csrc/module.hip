@@ -40,7 +40,7 @@ struct Tensor {
   std::unique_ptr<DevMem> mem;
 };
 
-enum OpKind { OP_A16, OP_I8, OP_CAST, OP_REQUANT };
+enum OpKind { OP_A16, OP_I8, OP_CAST, OP_REQUANT, OP_MATMUL_DQ };
 
 struct Op {
   OpKind kind;
@@ -63,6 +63,8 @@ struct Op {
   float inv_scale = 1.0f, scale = 1.0f;
   // standalone requant
   int64_t outer = 1, channels = 1, inner = 1;
+  // MatMul of two activations with dynamic quantization of both
+  int in2 = -1, right_transpose = 0, q_group_size = 0, dtype = MI_DT_BF16;
   bool capturable = true;
 };
 
@@ -191,6 +193,11 @@ int enqueue_all(mi_module *m) {
     case OP_REQUANT:
       rc = requant_launch((const int32_t *)tin.mem->ptr, tout.mem->ptr, o.outer, o.channels, o.inner, o.input_zp,
                           &o.rq, m->stream);
+      break;
+    case OP_MATMUL_DQ:
+      rc = matmul_dq_launch((const uint16_t *)tin.mem->ptr, (const uint16_t *)m->tensors[o.in2].mem->ptr,
+                            o.right_transpose, o.M, o.K, o.N, o.q_group_size, o.dq_type, o.dtype,
+                            (uint16_t *)tout.mem->ptr, nullptr, m->stream);
       break;
     }
     if (rc)
@@ -341,6 +348,85 @@ int mi_module_add_matmul_int8(mi_module *m, const char *input, const char *outpu
   }
   // zero points and unsigned operands make the launch allocate scratch: such ops stay out of a captured graph
   o.capturable = !o.a_unsigned && !o.b_unsigned && o.input_zp == 0 && o.right_zp == 0;
+  m->ops.push_back(std::move(o));
+  drop_graph(m);
+  return MI_SUCCESS;
+}
+
+int mi_module_add_requant(mi_module *m, const char *input, const char *output, const mi_module_rq_desc *d) {
+  int in, out, rc;
+  if ((rc = find(m, input, &in)) || (rc = find(m, output, &out)))
+    return rc;
+  MI_REQUIRE(d, MI_BAD_ARGUMENT, "mi_module_add_requant: null descriptor");
+  const Tensor &ti = m->tensors[in], &to = m->tensors[out];
+  MI_REQUIRE(ti.st == MI_ST_I32, MI_BAD_ARGUMENT, "mi_module_add_requant: the input must be an int32 tensor");
+  MI_REQUIRE(d->outer > 0 && d->channels > 0 && d->inner > 0 && ti.n == d->outer * d->channels * d->inner && to.n == ti.n,
+             MI_BAD_ARGUMENT, "mi_module_add_requant: tensor sizes are not outer * channels * inner");
+  const int want = d->rq.out_dtype == MI_DT_I8 ? MI_ST_I8 : d->rq.out_dtype == MI_DT_U8 ? MI_ST_U8
+                 : d->rq.out_dtype == MI_DT_I16 ? MI_ST_I16 : d->rq.out_dtype == MI_DT_U16 ? MI_ST_U16 : -1;
+  MI_REQUIRE(want >= 0 && to.st == want, MI_BAD_ARGUMENT,
+             "mi_module_add_requant: output storage differs from the requant type");
+  Op o;
+  o.kind = OP_REQUANT;
+  o.in = in;
+  o.out = out;
+  o.outer = d->outer;
+  o.channels = d->channels;
+  o.inner = d->inner;
+  o.input_zp = d->input_zp;
+  o.rq = d->rq;
+  // per-channel arrays arrive as HOST pointers in this descriptor and move to the device here
+  if (d->rq.d_multiplier) {
+    if ((rc = upload(o.mult, d->rq.d_multiplier, (size_t)d->channels * 4)))
+      return rc;
+    o.rq.d_multiplier = (const int32_t *)o.mult->ptr;
+  }
+  if (d->rq.d_shift) {
+    if ((rc = upload(o.shift, d->rq.d_shift, (size_t)d->channels * 4)))
+      return rc;
+    o.rq.d_shift = (const int32_t *)o.shift->ptr;
+  }
+  if (d->rq.d_zp) {
+    if ((rc = upload(o.zp, d->rq.d_zp, (size_t)d->channels * 4)))
+      return rc;
+    o.rq.d_zp = (const int32_t *)o.zp->ptr;
+  }
+  // modes, rounding and chip are checked by the launch itself: a launch over no elements validates them here
+  rc = requant_launch((const int32_t *)ti.mem->ptr, to.mem->ptr, 0, d->channels, d->inner, d->input_zp, &o.rq, m->stream);
+  if (rc)
+    return rc;
+  m->ops.push_back(std::move(o));
+  drop_graph(m);
+  return MI_SUCCESS;
+}
+
+int mi_module_add_matmul_dq(mi_module *m, const char *left, const char *right, const char *output, int64_t K,
+                            int64_t N, int right_transpose, int q_group_size, int dq_type) {
+  int in, in2, out, rc;
+  if ((rc = find(m, left, &in)) || (rc = find(m, right, &in2)) || (rc = find(m, output, &out)))
+    return rc;
+  const Tensor &tl = m->tensors[in], &tr = m->tensors[in2], &to = m->tensors[out];
+  MI_REQUIRE((tl.st == MI_ST_BF16 || tl.st == MI_ST_F16) && tr.st == tl.st && to.st == tl.st, MI_BAD_ARGUMENT,
+             "mi_module_add_matmul_dq: the three tensors must share one 16-bit float type");
+  MI_REQUIRE(K > 0 && N > 0 && tl.n % K == 0 && tr.n == K * N && to.n == tl.n / K * N, MI_BAD_ARGUMENT,
+             "mi_module_add_matmul_dq: tensor sizes are not M * K, K * N and M * N");
+  Op o;
+  o.kind = OP_MATMUL_DQ;
+  o.in = in;
+  o.in2 = in2;
+  o.out = out;
+  o.M = tl.n / K;
+  o.K = K;
+  o.N = N;
+  o.right_transpose = right_transpose != 0;
+  o.q_group_size = q_group_size;
+  o.dq_type = dq_type;
+  o.dtype = tl.st == MI_ST_F16 ? MI_DT_F16 : MI_DT_BF16;
+  // the launch checks type, group size and exactness limits: over no rows it does only that
+  rc = matmul_dq_launch((const uint16_t *)tl.mem->ptr, (const uint16_t *)tr.mem->ptr, o.right_transpose, 0, K, N,
+                        q_group_size, dq_type, o.dtype, (uint16_t *)to.mem->ptr, nullptr, m->stream);
+  if (rc)
+    return rc;
   m->ops.push_back(std::move(o));
   drop_graph(m);
   return MI_SUCCESS;

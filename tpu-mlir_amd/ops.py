@@ -598,6 +598,30 @@ class Module:
         check(clib.lib().mi_module_add_matmul_int8(self.handle, input.encode(), output.encode(), C.byref(d)))
         return self
 
+    def add_requant(self, input, output, *, outer=1, channels, inner=1, input_zp=0, quant_mode,
+                    round_mode=ROUND_HALF_AWAY_FROM_ZERO, out_dtype=DT_I8, chip=CHIP_BM168X, multiplier=1, shift=0, zp=0):
+        """tpu.RequantIntAxis / tpu.RequantInt on an int32 tensor [outer, channels, inner]; multiplier / shift / zp:
+        scalars or int32 numpy arrays [channels]; shift > 0 shifts right."""
+        keep = []
+        rq = RequantDescC(quant_mode, round_mode, chip, out_dtype, None, 1, None, 0, None, 0)
+        for name, v in (("multiplier", multiplier), ("shift", shift), ("zp", zp)):
+            if isinstance(v, np.ndarray):
+                a = np.ascontiguousarray(v, dtype=np.int32)
+                keep.append(a)
+                setattr(rq, "d_" + name, a.ctypes.data)
+            else:
+                setattr(rq, name, int(v))
+        d = clib.ModuleRqDesc(outer, channels, inner, input_zp, rq)
+        check(clib.lib().mi_module_add_requant(self.handle, input.encode(), output.encode(), C.byref(d)))
+        return self
+
+    def add_matmul_dq(self, left, right, output, *, K, N, right_transpose=False, q_group_size, dq_type=clib.DQ_INT8):
+        """tpu.MatMul of two activation tensors with both quantized dynamically per group (DQ_INT8 / DQ_INT4 /
+        DQ_F8E4M3 / DQ_F4)."""
+        check(clib.lib().mi_module_add_matmul_dq(self.handle, left.encode(), right.encode(), output.encode(), K, N,
+                                                 int(right_transpose), q_group_size, dq_type))
+        return self
+
     def add_cast(self, input, output, *, in_type, out_type, in_quant=False, out_quant=False, scale=1.0, zero_point=0,
                  expressed=None, round_mode=ROUND_HALF_AWAY_FROM_ZERO):
         attr = clib.CastAttr(0, in_type, out_type, int(in_quant), int(out_quant), float(scale), int(zero_point),
