@@ -117,8 +117,10 @@ def bench_chain(pkg, S, torch, M, steps, warmup, n_layers, cfgs, grouped=True):
     return res
 
 
-def bench_int8(pkg, S, torch, clib, n, steps, warmup, M=None):
-    """INT8 requant GEMM, N = K = n and M rows (default n), per-channel Q31 multiplier + right shift, int8 output."""
+def bench_int8(pkg, S, torch, clib, n, steps, warmup, M=None, graph=False):
+    """INT8 requant GEMM, N = K = n and M rows (default n), per-channel Q31 multiplier + right shift, int8 output.
+    graph: replay the launches from a HIP graph -- for launches of a few microseconds, which issued one by one from
+    Python would be timed by the host's call rate."""
     M = n if M is None else M
     c = S.int8_matmul(M, n, n, seed=7, right_transpose=True)
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
@@ -126,18 +128,17 @@ def bench_int8(pkg, S, torch, clib, n, steps, warmup, M=None):
     rq = pkg.RequantDesc(clib.RQ_QDM, clib.ROUND_HALF_AWAY_FROM_ZERO, out_dtype=clib.DT_I8,
                          multiplier=dev(c["mult"]), shift=dev(c["shift"]))
     out = torch.empty((M, n), dtype=torch.int8, device="cuda")
-    stream = torch.cuda.Stream()
-    with torch.cuda.stream(stream):
-        for _ in range(warmup):
-            pkg.i8mm_launch(a, b, bias, right_transpose=True, rq=rq, out=out)
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        stream.synchronize()
-        ev0.record(stream)
-        for _ in range(steps):
-            pkg.i8mm_launch(a, b, bias, right_transpose=True, rq=rq, out=out)
-        ev1.record(stream)
-        stream.synchronize()
-    sec = ev0.elapsed_time(ev1) * 1e-3 / steps
+    def run():
+        pkg.i8mm_launch(a, b, bias, right_transpose=True, rq=rq, out=out)
+
+    def run10():
+        for _ in range(10):
+            run()
+
+    if graph:
+        sec = _time_graph(torch, run10, max(3, steps // 10)) / 10
+    else:
+        sec = _time_launches(torch, run, steps, warmup=warmup)
     tops = 2.0 * M * n * n / sec / 1e12
     return {"workload": "int8_requant_gemm_M%d_N%d_K%d_qdm_per_channel" % (M, n, n), "tops": round(tops, 2),
             "us_per_launch": round(sec * 1e6, 2), "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4),
@@ -158,6 +159,20 @@ def _time_launches(torch, fn, steps, warmup=5):
         ev1.record(stream)
         stream.synchronize()
     return ev0.elapsed_time(ev1) * 1e-3 / steps
+
+
+def _time_graph(torch, fn, replays, warmup=2):
+    """Average device time of one fn() when fn's launches are replayed from a HIP graph (fn runs eagerly first, so
+    that whatever it allocates on its stream exists before the capture): a launch of a few microseconds issued from
+    Python would otherwise be timed by the host's call rate."""
+    stream = torch.cuda.Stream()
+    g_ = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        fn()
+        stream.synchronize()
+        with torch.cuda.graph(g_, stream=stream):
+            fn()
+    return _time_launches(torch, g_.replay, replays, warmup=warmup)
 
 
 def bench_single_matmuls(pkg, S, torch, steps=60):
@@ -212,7 +227,7 @@ def bench_single_matmuls(pkg, S, torch, steps=60):
 
 def bench_dynamic_quant(pkg, S, torch, steps=40):
     """tpu.A16MatMul with dynamic integer activation quantization (activation quantizer + integer product per call),
-    weights rotating through HBM; eager launches (the call allocates its code buffers on the stream)."""
+    weights rotating through HBM; launches replayed from a HIP graph."""
     out = []
     for M, K, N, copies in ((1, 4096, 4096, 32), (16, 4096, 4096, 32), (1, 4096, 11008, 12), (128, 4096, 4096, 32)):
         cfg = S.w4a16(1, K, N, 128, seed=33)
@@ -225,7 +240,7 @@ def bench_dynamic_quant(pkg, S, torch, steps=40):
             for w in ws:
                 pkg.a16mm_dq_launch(w, x, y)
 
-        sec = _time_launches(torch, run, max(3, steps // copies), warmup=2) / copies
+        sec = _time_graph(torch, run, max(3, steps // copies)) / copies
         nbytes = S.w4_gemv_bytes(M, K, N, 128)
         out.append({"case": "w4_g128_dynamic_int", "M": M, "K": K, "N": N, "us": round(sec * 1e6, 2),
                     "GBps": round(nbytes / sec / 1e9, 1)})
@@ -249,7 +264,7 @@ def bench_dynamic_quant(pkg, S, torch, steps=40):
                 for w in ws:
                     pkg.a16mm_dq_launch(w, x, y, dq_type=getattr(pkg, dq))
 
-            sec = _time_launches(torch, run, max(3, steps // copies), warmup=2) / copies
+            sec = _time_graph(torch, run, max(3, steps // copies)) / copies
             nbytes = S.w4_gemv_bytes(M, K, N, 128) + (N * K // 2 if bits == 8 else 0)
             out.append({"case": case, "M": M, "K": K, "N": N, "us": round(sec * 1e6, 2),
                         "GBps": round(nbytes / sec / 1e9, 1)})
@@ -273,7 +288,12 @@ def bench_f8_matmul(pkg, torch, clib, steps=20):
         def run():
             pkg.f8mm_launch(a, b, bias, right_transpose=True, out_scales=scales, out=y)
 
-        sec = _time_launches(torch, run, steps, warmup=3)
+        def run10():
+            for _ in range(10):
+                run()
+
+        # the small shape from a graph: issued one by one from Python it would be timed by the host's call rate
+        sec = _time_launches(torch, run, steps, warmup=3) if M >= 2048 else _time_graph(torch, run10, 4) / 10
         tf = 2.0 * M * N * K / sec / 1e12
         out.append({"case": "f8e4m3_matmul_requant_M%d_N%d_K%d" % (M, N, K), "us": round(sec * 1e6, 2),
                     "TFLOPs": round(tf, 1), "frac_fp8_peak": round(tf / 5000.0, 4)})
@@ -453,7 +473,7 @@ def main():
             ex["chain_M%d_GBps" % m] = round(rm["chain_bytes"] / (rm["gpu_s"] / 40) / 1e9, 1)
         ex["single_matmuls"] = bench_single_matmuls(pkg, S, torch)
         ex["dynamic_quant"] = bench_dynamic_quant(pkg, S, torch)
-        ex["int8_256x1024x1024"] = bench_int8(pkg, S, torch, clib, 1024, 40, 5, M=256)
+        ex["int8_256x1024x1024"] = bench_int8(pkg, S, torch, clib, 1024, 40, 5, M=256, graph=True)
         ex["f8_matmul"] = bench_f8_matmul(pkg, torch, clib)
         ex["operator_boundary"] = bench_operator_boundary(pkg, S)
         ex["device_resident_block"] = bench_module_block(pkg, S, clib, cfgs)

@@ -303,15 +303,28 @@ extern "C" int mi_i8_dbg_dump(unsigned long long *host) {
 // Requires K % 64 == 0; rows past M/N are clamped on the way in and masked on the way out.
 // ------------------------------------------------------------------------------------------------
 constexpr int MID_M = 128, MID_N = 128, MID_K = 64;
-constexpr int MID_STAGE = (MID_M + MID_N) * MID_K;  // 16 KiB
-constexpr int MID_STRIDE = 68;                      // dwords per row of an epilogue strip (64 + 4: 16-byte aligned rows)
-constexpr int mid_lds_bytes(int nst) { return nst * MID_STAGE > 4 * 64 * MID_STRIDE * 4 ? nst * MID_STAGE : 4 * 64 * MID_STRIDE * 4; }
+// bt = tile edge: 128, or 64 (4 waves x one 32x32 block) for grids that would leave most CUs without a 128-tile --
+// there the whole of a short K fits a 16-stage ring, so the K loop costs one memory latency, and a lane's share of
+// the epilogue is 16 outputs instead of 64
+constexpr int mid_stage_bytes(int bt) { return 2 * bt * MID_K; }  // 16 KiB / 8 KiB
+constexpr int mid_stride(int bt) { return bt / 2 + 4; }  // dwords per row of an epilogue strip (16-byte aligned rows)
+constexpr int mid_lds_bytes(int nst, int bt = 128) {
+  return nst * mid_stage_bytes(bt) > 4 * (bt / 2) * mid_stride(bt) * 4 ? nst * mid_stage_bytes(bt)
+                                                                         : 4 * (bt / 2) * mid_stride(bt) * 4;
+}
 
 // MID_NST = stages in the LDS ring: 4 (two workgroups per CU) when there are more tiles than CUs, 8 when every
 // workgroup has a CU to itself -- a short grid is bound by the bytes it keeps in flight.
-template <int MID_NST>
+template <int MID_NST, int BT = 128>
 __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m, int tiles_n, int per_xcd) {
-  constexpr int LOADS = MID_M * (MID_K / 16) / 256;  // direct-to-LDS instructions per operand, stage and thread: 2
+  constexpr int WT = BT / 2;                       // a wave's square of outputs: 64 or 32
+  constexpr int NB = WT / 32;                      // 32x32 MFMA blocks per side of it
+  constexpr int MID_STAGE = mid_stage_bytes(BT);
+  constexpr int MID_STRIDE = mid_stride(BT);
+  constexpr int CPR = WT / 16;                     // epilogue: 16-column chunks per strip row (4 or 2) ...
+  constexpr int RPP = 64 / CPR;                    // ... rows covered by one pass of the wave (16 or 32) ...
+  constexpr int PASSES = WT / RPP;                 // ... passes (4 or 1)
+  constexpr int LOADS = BT * (MID_K / 16) / 256;   // direct-to-LDS instructions per operand, stage and thread: 2 or 1
   constexpr int LPS = 2 * LOADS;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -329,7 +342,7 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
   const int gm = (tiles_m - group * GM) < GM ? (tiles_m - group * GM) : GM;
   const int in_group = L - group * GM * tiles_n;
   const int tm = group * GM + in_group % gm, tn = in_group / gm;
-  const int64_t m_base = (int64_t)tm * MID_M, n_base = (int64_t)tn * MID_N;
+  const int64_t m_base = (int64_t)tm * BT, n_base = (int64_t)tn * BT;
 
   // the 16-byte chunk c of row r is stored at position c ^ ((r >> 2) & 3): the 32 rows of a fragment read hit
   // distinct bank groups
@@ -348,7 +361,7 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
   const int kt_total = (int)(a.K / MID_K);
   auto issue = [&](int kt) {
     const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 1) * MID_K;  // past the end: harmless re-load
-    uint8_t *sa = lds + (kt % MID_NST) * MID_STAGE, *sb = sa + MID_M * MID_K;
+    uint8_t *sa = lds + (kt % MID_NST) * MID_STAGE, *sb = sa + BT * MID_K;
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       __builtin_amdgcn_global_load_lds((gptr_t)(ga[i] + koff), (lptr_t)(sa + (i * 4 + wave) * 1024), 16, 0, 0);
@@ -356,30 +369,30 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
     }
   };
 
-  i32x16 acc[2][2];
+  i32x16 acc[NB][NB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NB; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         acc[i][j][r] = 0;
 
   const int frow = lane & 31, kh = lane >> 5;
-  int a_off[2], b_off[2], f_sw[2];
+  int a_off[NB], b_off[NB], f_sw[NB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int ra = wm * 64 + i * 32 + frow, rb = wn * 64 + i * 32 + frow;
+  for (int i = 0; i < NB; ++i) {
+    const int ra = wm * WT + i * 32 + frow, rb = wn * WT + i * 32 + frow;
     a_off[i] = ra * MID_K;
-    b_off[i] = MID_M * MID_K + rb * MID_K;
+    b_off[i] = BT * MID_K + rb * MID_K;
     f_sw[i] = (frow >> 2) & 3;  // (row >> 2) & 3 with row = 32-aligned base + frow
   }
 
   // epilogue parameters of this lane's 16 output columns, requested ahead of every stage request (requests complete
   // in order and the waits in the K loop count them) so that their latency hides behind the K loop; nothing uses
   // them before the epilogue
-  const int cc = lane & 3, rsub = lane >> 2;  // 16-column chunk, row within a group of 16 rows
-  const int64_t n0 = n_base + wn * 64 + cc * 16;
+  const int cc = lane % CPR, rsub = lane / CPR;  // 16-column chunk, row within a group of RPP rows
+  const int64_t n0 = n_base + wn * WT + cc * 16;
   const bool vec_ok = (a.N % 16) == 0 && n0 + 16 <= a.N;
   const int32_t relu_hi = (a.relu_limit > 0 && a.relu_limit < INT32_MAX) ? (int32_t)a.relu_limit : INT32_MAX;
   int32_t p_bias[16], p_mult[16], p_shift[16], p_zp[16];
@@ -425,16 +438,16 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
     const uint8_t *st = lds + (kt % MID_NST) * MID_STAGE;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      i32x4 fa[2], fb[2];
+      i32x4 fa[NB], fb[NB];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < NB; ++i) {
         fa[i] = *(const i32x4 *)(st + a_off[i] + (((ks * 2 + kh) ^ f_sw[i]) << 4));
         fb[i] = *(const i32x4 *)(st + b_off[i] + (((ks * 2 + kh) ^ f_sw[i]) << 4));
       }
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < NB; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NB; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
     }
   }
@@ -447,11 +460,11 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
   // block) pass through a per-wave 64 x 64 strip in LDS so that a lane owns 16 consecutive columns of a row: per-column
   // parameters are loaded once per lane, and int8 results leave as 16-byte stores.
   __builtin_amdgcn_s_barrier();  // every wave is done reading the ring
-  int32_t *strip = (int32_t *)lds + wave * (64 * MID_STRIDE);
+  int32_t *strip = (int32_t *)lds + wave * (WT * MID_STRIDE);
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NB; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         strip[(i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * MID_STRIDE + j * 32 + (lane & 31)] = acc[i][j][r];
@@ -465,9 +478,9 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
     }
   }
 #pragma unroll 1
-  for (int it = 0; it < 4; ++it) {
-    const int row = it * 16 + rsub;
-    const int64_t m = m_base + wm * 64 + row;
+  for (int it = 0; it < PASSES; ++it) {
+    const int row = it * RPP + rsub;
+    const int64_t m = m_base + wm * WT + row;
     int32_t v[16];
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4) {
@@ -1033,19 +1046,27 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
     }
   }
   if (mid) {
-    const int tiles_m = (int)((M + MID_M - 1) / MID_M), tiles_n = (int)((N + MID_N - 1) / MID_N);
-    const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+    int tiles_m = (int)((M + MID_M - 1) / MID_M), tiles_n = (int)((N + MID_N - 1) / MID_N);
+    int per_xcd = (tiles_m * tiles_n + 7) / 8;
     static bool attr_set = false;
     if (!attr_set) {
       (void)hipFuncSetAttribute((const void *)i8_gemm_mid_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 160 * 1024);
       (void)hipFuncSetAttribute((const void *)i8_gemm_mid_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 160 * 1024);
+      (void)hipFuncSetAttribute((const void *)i8_gemm_mid_kernel<16, 64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024);
       attr_set = true;
     }
-    const char *ring_env = getenv("MI_I8_MID_RING");  // development switch: 4 / 8
-    const int ring = ring_env ? atoi(ring_env) : (tiles_m * tiles_n <= 256 ? 8 : 4);
-    if (ring == 8)
+    const char *ring_env = getenv("MI_I8_MID_RING");  // development switch: 4 / 8 / 16 (the 64-tile variant)
+    const int ring = ring_env ? atoi(ring_env) : (tiles_m * tiles_n < 64 ? 16 : tiles_m * tiles_n <= 256 ? 8 : 4);
+    if (ring == 16) {  // fewer 128-tiles than a quarter of the CUs: 64-tiles, all of a short K in flight at once
+      tiles_m = (int)((M + 63) / 64);
+      tiles_n = (int)((N + 63) / 64);
+      per_xcd = (tiles_m * tiles_n + 7) / 8;
+      i8_gemm_mid_kernel<16, 64><<<dim3((unsigned)(per_xcd * 8)), dim3(256), mid_lds_bytes(16, 64), stream>>>(
+          a, tiles_m, tiles_n, per_xcd);
+    } else if (ring == 8)
       i8_gemm_mid_kernel<8><<<dim3((unsigned)(per_xcd * 8)), dim3(256), mid_lds_bytes(8), stream>>>(a, tiles_m, tiles_n,
                                                                                                    per_xcd);
     else
