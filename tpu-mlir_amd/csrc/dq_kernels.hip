@@ -196,8 +196,9 @@ __device__ __forceinline__ void acc_f4_add(f32x4 (&acc)[4], int which, long av, 
     acc[3] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(av, bv, acc[3], 0, 0, 0);
 }
 
+// Launched with DQ_WAVES waves, or twice that when the grid leaves a CU no second workgroup to hide latency with.
 template <int DT, int BITS, int FLAV>
-__global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
+__global__ __launch_bounds__(2 * DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
   static_assert(FLAV == FLAV_INT || (FLAV == FLAV_F8 && BITS == 8) || (FLAV == FLAV_F4 && BITS == 4), "storage width");
   // group sums: int32 for integer codes, fp32 for the float codes (32 k per matrix instruction)
   using acc_t = typename std::conditional<FLAV == FLAV_INT, i32x4, f32x4>::type;
@@ -205,6 +206,7 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
   extern __shared__ __attribute__((aligned(16))) float terms[];  // [groups of the chunk][16 rows][16 columns]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n_waves = (int)(blockDim.x >> 6);
   const int col = lane & 15, kq = lane >> 4;
   const int64_t rb = blockIdx.x, mb = blockIdx.y;
   const u32x4 *wq = a.qw + rb * a.k_tiles * 64 + lane;
@@ -223,7 +225,7 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq_gemm_kernel(DqArgs a) {
   const int chunk_units = DQ_CHUNK / a.unit_groups;
   for (int u0 = 0; u0 < units; u0 += chunk_units) {
     const int u1 = (u0 + chunk_units) < units ? (u0 + chunk_units) : units;
-    for (int u = u0 + wave; u < u1; u += DQ_WAVES) {
+    for (int u = u0 + wave; u < u1; u += n_waves) {
       acc_t acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};  // one per group of the unit
       for (int t = 0; t < a.unit_tiles; ++t) {
         const int64_t kt = (int64_t)u * a.unit_tiles + t;
@@ -624,6 +626,8 @@ int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int6
   const int chunk_groups = G < DQ_CHUNK ? G : DQ_CHUNK;
   const size_t lds_bytes = (size_t)(chunk_groups + 1) * 1024;
   dim3 grid((unsigned)w->row_blocks, (unsigned)m_blocks);
+  const char *we = getenv("MI_DQ_WAVES");  // development switch: 8 / 16
+  const int gemm_waves = we ? atoi(we) : ((int64_t)w->row_blocks * m_blocks <= 256 ? 2 * DQ_WAVES : DQ_WAVES);
 #define MI_DQ_RUN(DT_, BITS_, FLAV_)                                                                             \
   {                                                                                                             \
     dq_act_kernel<DT_, BITS_, FLAV_><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(              \
@@ -634,7 +638,7 @@ int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int6
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                        \
       attr_set = true;                                                                                          \
     }                                                                                                           \
-    dq_gemm_kernel<DT_, BITS_, FLAV_><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);                     \
+    dq_gemm_kernel<DT_, BITS_, FLAV_><<<grid, dim3(gemm_waves * 64), lds_bytes, stream>>>(a);                   \
   }
   if (dq_type == MI_DQ_F8E4M3) {
     if (f16)
