@@ -303,9 +303,9 @@ extern "C" int mi_i8_dbg_dump(unsigned long long *host) {
 // Requires K % 64 == 0; rows past M/N are clamped on the way in and masked on the way out.
 // ------------------------------------------------------------------------------------------------
 constexpr int MID_M = 128, MID_N = 128, MID_K = 64;
-// bt = tile edge: 128, or 64 (4 waves x one 32x32 block) for grids that would leave most CUs without a 128-tile --
-// there the whole of a short K fits a 16-stage ring, so the K loop costs one memory latency, and a lane's share of
-// the epilogue is 16 outputs instead of 64
+// bt = tile edge: 128, or 64 (4 waves x one 32x32 block) for grids that would leave half the CUs without a 128-tile:
+// four times the workgroups, four of them per CU hiding each other's waits, and a lane's share of the epilogue is 16
+// outputs instead of 64
 constexpr int mid_stage_bytes(int bt) { return 2 * bt * MID_K; }  // 16 KiB / 8 KiB
 constexpr int mid_stride(int bt) { return bt / 2 + 4; }  // dwords per row of an epilogue strip (16-byte aligned rows)
 constexpr int mid_lds_bytes(int nst, int bt = 128) {
@@ -1054,17 +1054,20 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
                                 160 * 1024);
       (void)hipFuncSetAttribute((const void *)i8_gemm_mid_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 160 * 1024);
-      (void)hipFuncSetAttribute((const void *)i8_gemm_mid_kernel<16, 64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+      (void)hipFuncSetAttribute((const void *)i8_gemm_mid_kernel<4, 64>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 160 * 1024);
       attr_set = true;
     }
-    const char *ring_env = getenv("MI_I8_MID_RING");  // development switch: 4 / 8 / 16 (the 64-tile variant)
-    const int ring = ring_env ? atoi(ring_env) : (tiles_m * tiles_n < 64 ? 16 : tiles_m * tiles_n <= 256 ? 8 : 4);
-    if (ring == 16) {  // fewer 128-tiles than a quarter of the CUs: 64-tiles, all of a short K in flight at once
+    // up to 128 tiles of 128 x 128 (half the CUs): 64 x 64 tiles with a 4-stage ring, four workgroups per CU hiding
+    // each other's waits (measured against the 128-tile forms: 5.8 vs 10.2 us at 256 x 1024 x 1024, 6.2 vs 10.5 at
+    // 1024^3, 11.2 vs 15.4 at 1024 x 2048 x 2048; from 160 tiles on the 128-tile forms win)
+    const char *ring_env = getenv("MI_I8_MID_RING");  // development switch: 4 / 8 (128-tiles), 64 (64-tiles)
+    const int ring = ring_env ? atoi(ring_env) : (tiles_m * tiles_n <= 128 ? 64 : tiles_m * tiles_n <= 256 ? 8 : 4);
+    if (ring == 64) {
       tiles_m = (int)((M + 63) / 64);
       tiles_n = (int)((N + 63) / 64);
       per_xcd = (tiles_m * tiles_n + 7) / 8;
-      i8_gemm_mid_kernel<16, 64><<<dim3((unsigned)(per_xcd * 8)), dim3(256), mid_lds_bytes(16, 64), stream>>>(
+      i8_gemm_mid_kernel<4, 64><<<dim3((unsigned)(per_xcd * 8)), dim3(256), mid_lds_bytes(4, 64), stream>>>(
           a, tiles_m, tiles_n, per_xcd);
     } else if (ring == 8)
       i8_gemm_mid_kernel<8><<<dim3((unsigned)(per_xcd * 8)), dim3(256), mid_lds_bytes(8), stream>>>(a, tiles_m, tiles_n,
