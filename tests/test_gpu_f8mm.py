@@ -55,7 +55,7 @@ CASES = [  # (M, K, N, right_transpose, relu, per_channel, bias)
 ]
 
 
-@pytest.mark.parametrize("tile", ["128", "256"])
+@pytest.mark.parametrize("tile", ["64", "128", "256"])
 @pytest.mark.parametrize("M,K,N,rt,relu,per_channel,bias", CASES)
 def test_f8_matmul_device_level(orc, monkeypatch, M, K, N, rt, relu, per_channel, bias, tile):
     monkeypatch.setenv("MI_F8_TILE", tile)  # both tile shapes of the ring kernels (K % 64 != 0 takes neither)
@@ -212,7 +212,7 @@ E5M2_CASES = [  # (M, K, N, right_transpose, relu, bias)
 ]
 
 
-@pytest.mark.parametrize("tile", ["128", "256"])
+@pytest.mark.parametrize("tile", ["64", "128", "256"])
 @pytest.mark.parametrize("M,K,N,rt,relu,bias", E5M2_CASES)
 def test_e5m2_matmul_device_level(orc, monkeypatch, M, K, N, rt, relu, bias, tile):
     monkeypatch.setenv("MI_F8_TILE", tile)

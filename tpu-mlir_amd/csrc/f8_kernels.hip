@@ -241,18 +241,21 @@ constexpr int F8_STRIDE = 68;  // dwords per row of an epilogue strip (64 + 4: 1
 // Epilogue of a wave's 64 x 64 block through its own strip of LDS: the accumulators (register r of lane l = row
 // 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of block (i, j)) are laid out row-major so that a lane owns 16
 // consecutive columns of a row -- per-column parameters are fetched once per lane, results leave as 16-byte stores.
-template <int FMT>
-__device__ __forceinline__ void f8_strip_epilogue(const F8Args &a, const f32x16 (&acc)[2][2], float *strip, int64_t m0,
-                                                  int64_t nb, int lane) {
+// WT = edge of the wave's square of outputs (64: 2 x 2 blocks, 32: one block); the strip has WT + 4 dwords per row
+template <int FMT, int WT = 64>
+__device__ __forceinline__ void f8_strip_epilogue(const F8Args &a, const f32x16 (&acc)[WT / 32][WT / 32], float *strip,
+                                                  int64_t m0, int64_t nb, int lane) {
+  constexpr int NB = WT / 32, F8_STRIDE = WT + 4;
+  constexpr int CPR = WT / 16, RPP = 64 / CPR, PASSES = WT / RPP;  // 16-column chunks per row, rows per pass, passes
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NB; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         strip[(i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * F8_STRIDE + j * 32 + (lane & 31)] = acc[i][j][r];
   // a wave only reads what it wrote: no barrier, the LDS counter orders it
-  const int cc = lane & 3, rsub = lane >> 2;  // 16-column chunk, row within a group of 16 rows
+  const int cc = lane % CPR, rsub = lane / CPR;  // 16-column chunk, row within a group of RPP rows
   const int64_t n0 = nb + cc * 16;
   const bool vec_ok = (a.N % 16) == 0 && n0 + 16 <= a.N;
   float bias[16], inv[16];  // per column: bias, fl32(1 / step)
@@ -264,8 +267,8 @@ __device__ __forceinline__ void f8_strip_epilogue(const F8Args &a, const f32x16 
   }
   const float relu_hi = (a.do_relu && a.relu_limit > 0.0f) ? a.relu_limit : __builtin_inff();
 #pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    const int row = p * 16 + rsub;
+  for (int p = 0; p < PASSES; ++p) {
+    const int row = p * RPP + rsub;
     const int64_t m = m0 + row;
     float v[16];
 #pragma unroll
@@ -352,16 +355,23 @@ __device__ __forceinline__ void f8_strip_epilogue(const F8Args &a, const f32x16 
 
 typedef const __attribute__((address_space(1))) void *f8_gptr_t;
 typedef __attribute__((address_space(3))) void *f8_lptr_t;
-constexpr int F8_STAGE = (F8_BM + F8_BN) * F8_BK;  // 16 KiB
+constexpr int f8_stage_bytes(int bt) { return 2 * bt * F8_BK; }  // 16 KiB (128-tiles) / 8 KiB (64-tiles)
 constexpr int f8_waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }  // s_waitcnt vmcnt(n) only
 // the ring, or the four epilogue strips that reuse its memory, whichever is larger
-constexpr int f8_ring_lds_bytes(int nst) { return nst * F8_STAGE > 4 * 64 * F8_STRIDE * 4 ? nst * F8_STAGE : 4 * 64 * F8_STRIDE * 4; }
+constexpr int f8_ring_lds_bytes(int nst, int bt = 128) {
+  return nst * f8_stage_bytes(bt) > 4 * (bt / 2) * (bt / 2 + 4) * 4 ? nst * f8_stage_bytes(bt)
+                                                                      : 4 * (bt / 2) * (bt / 2 + 4) * 4;
+}
 
 // NST = stages in the LDS ring: 4 (two workgroups per CU) when there are more tiles than CUs, 8 when every workgroup
 // has a CU to itself
-template <int NST, int FMT>
+// BT = tile edge: 128 (a wave 64 x 64), or 64 (a wave one 32 x 32 block) for grids of up to 128 tiles of 128 x 128:
+// four times the workgroups, several per CU hiding each other's waits (the INT8 kernel's measured crossover)
+template <int NST, int FMT, int BT = 128>
 __global__ __launch_bounds__(256) void f8_gemm_ring_kernel(F8Args a, int tiles_m, int tiles_n, int per_xcd) {
-  constexpr int LOADS = F8_BM * (F8_BK / 16) / 256;  // direct-to-LDS instructions per operand, stage and thread: 2
+  constexpr int WT = BT / 2, NB = WT / 32;
+  constexpr int F8_STAGE = f8_stage_bytes(BT);
+  constexpr int LOADS = BT * (F8_BK / 16) / 256;  // direct-to-LDS instructions per operand, stage and thread: 2 or 1
   constexpr int LPS = 2 * LOADS;
   extern __shared__ __attribute__((aligned(16))) uint8_t f8_lds[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -376,7 +386,7 @@ __global__ __launch_bounds__(256) void f8_gemm_ring_kernel(F8Args a, int tiles_m
   const int gm = (tiles_m - group * GM) < GM ? (tiles_m - group * GM) : GM;
   const int in_group = L - group * GM * tiles_n;
   const int tm = group * GM + in_group % gm, tn = in_group / gm;
-  const int64_t m_base = (int64_t)tm * F8_BM, n_base = (int64_t)tn * F8_BN;
+  const int64_t m_base = (int64_t)tm * BT, n_base = (int64_t)tn * BT;
 
   // the 16-byte chunk c of row r is stored at position c ^ ((r >> 2) & 3): the 32 rows of a fragment read hit distinct
   // bank groups
@@ -395,7 +405,7 @@ __global__ __launch_bounds__(256) void f8_gemm_ring_kernel(F8Args a, int tiles_m
   const int kt_total = (int)(a.K / F8_BK);
   auto issue = [&](int kt) {
     const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 1) * F8_BK;  // past the end: harmless re-load
-    uint8_t *sa = f8_lds + (kt % NST) * F8_STAGE, *sb = sa + F8_BM * F8_BK;
+    uint8_t *sa = f8_lds + (kt % NST) * F8_STAGE, *sb = sa + BT * F8_BK;
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       __builtin_amdgcn_global_load_lds((f8_gptr_t)(ga[i] + koff), (f8_lptr_t)(sa + (i * 4 + wave) * 1024), 16, 0, 0);
@@ -403,22 +413,22 @@ __global__ __launch_bounds__(256) void f8_gemm_ring_kernel(F8Args a, int tiles_m
     }
   };
 
-  f32x16 acc[2][2];
+  f32x16 acc[NB][NB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NB; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         acc[i][j][r] = 0.0f;
 
   const int frow = lane & 31, kh = lane >> 5;
-  int a_off[2], b_off[2];
+  int a_off[NB], b_off[NB];
   const int f_sw = (frow >> 2) & 3;  // (row >> 2) & 3 with row = 32-aligned base + frow
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    a_off[i] = (wm * 64 + i * 32 + frow) * F8_BK;
-    b_off[i] = F8_BM * F8_BK + (wn * 64 + i * 32 + frow) * F8_BK;
+  for (int i = 0; i < NB; ++i) {
+    a_off[i] = (wm * WT + i * 32 + frow) * F8_BK;
+    b_off[i] = BT * F8_BK + (wn * WT + i * 32 + frow) * F8_BK;
   }
 #pragma unroll
   for (int s0 = 0; s0 < NST - 1; ++s0)
@@ -430,9 +440,9 @@ __global__ __launch_bounds__(256) void f8_gemm_ring_kernel(F8Args a, int tiles_m
     issue(kt + NST - 1);
     const uint8_t *st = f8_lds + (kt % NST) * F8_STAGE;
     // lane (row, kh) takes chunks kh and 2 + kh of its row for both operands
-    i32x8 fa[2], fb[2];
+    i32x8 fa[NB], fb[NB];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NB; ++i) {
       const u32x4 a0 = *(const u32x4 *)(st + a_off[i] + ((kh ^ f_sw) << 4));
       const u32x4 a1 = *(const u32x4 *)(st + a_off[i] + (((2 + kh) ^ f_sw) << 4));
       const u32x4 b0 = *(const u32x4 *)(st + b_off[i] + ((kh ^ f_sw) << 4));
@@ -441,14 +451,14 @@ __global__ __launch_bounds__(256) void f8_gemm_ring_kernel(F8Args a, int tiles_m
       fb[i] = i32x8{(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NB; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < NB; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], FMT, FMT, 0, 0, 0, 0);
   }
   __builtin_amdgcn_s_waitcnt(f8_waitcnt_vm(0));  // drain the re-loads issued past the end
   __builtin_amdgcn_s_barrier();                  // every wave is done reading the ring
-  f8_strip_epilogue<FMT>(a, acc, (float *)f8_lds + wave * (64 * F8_STRIDE), m_base + wm * 64, n_base + wn * 64, lane);
+  f8_strip_epilogue<FMT, WT>(a, acc, (float *)f8_lds + wave * (WT * (WT + 4)), m_base + wm * WT, n_base + wn * WT, lane);
 }
 
 // ---- 256 x 256 outputs per workgroup, 4 waves (2 x 2), each wave 128 x 128 as 4 x 4 blocks of 32 x 32 (256 fp32
@@ -667,9 +677,20 @@ int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, con
       attr_set = true;
     }
     const int64_t tl_m = (M + F8L_M - 1) / F8L_M, tl_n = (N + F8L_N - 1) / F8L_N;
-    const char *e = getenv("MI_F8_TILE");  // development switch: "256" / "128"
+    const char *e = getenv("MI_F8_TILE");  // development switch: "256" / "128" / "64"
     const bool large = e ? atoi(e) == 256 : tl_m * tl_n >= 144;  // the INT8 kernels' measured crossover
-    if (large) {
+    const bool small = e ? atoi(e) == 64 : tiles <= 128;         // likewise
+    if (small && !large) {
+      const int64_t ts_m = (M + 63) / 64, ts_n = (N + 63) / 64;
+      const int ts = (int)(ts_m * ts_n), ps = (ts + 7) / 8;
+      const dim3 grid((unsigned)(ps * 8));
+      if (e5m2)
+        f8_gemm_ring_kernel<4, F8_FMT_E5M2, 64><<<grid, dim3(256), f8_ring_lds_bytes(4, 64), stream>>>(a, (int)ts_m,
+                                                                                                      (int)ts_n, ps);
+      else
+        f8_gemm_ring_kernel<4, F8_FMT_E4M3, 64><<<grid, dim3(256), f8_ring_lds_bytes(4, 64), stream>>>(a, (int)ts_m,
+                                                                                                      (int)ts_n, ps);
+    } else if (large) {
       static bool attr_large = false;
       if (!attr_large) {
         (void)hipFuncSetAttribute((const void *)f8_gemm_large_kernel<F8_FMT_E4M3>,
