@@ -352,9 +352,11 @@ int mi_requant_launch(const int32_t *d_in, void *d_out, int64_t outer, int64_t c
 
 /* ============================================================================ */
 /* tpu.Cast  (lib/Dialect/Tpu/Interfaces/Common/Cast.cpp:35-200; requant()/dequant() of     */
-/* lib/Support/CastUtils.cpp:15-46).  BM168x branches; CV18xx and fp8 casts: MI_UNSUPPORTED. */
+/* lib/Support/CastUtils.cpp:15-46).  BM168x branches incl. F32/F16 <-> F8 (:59-73); CV18xx: MI_UNSUPPORTED.    */
 /* ============================================================================ */
-enum { MI_ST_F32 = 0, MI_ST_BF16, MI_ST_F16, MI_ST_I8, MI_ST_U8, MI_ST_I16, MI_ST_U16, MI_ST_I32, MI_ST_U32 };
+enum { MI_ST_F32 = 0, MI_ST_BF16, MI_ST_F16, MI_ST_I8, MI_ST_U8, MI_ST_I16, MI_ST_U16, MI_ST_I32, MI_ST_U32,
+       MI_ST_F8E4M3, MI_ST_F8E5M2 /* one byte; tpu.Cast from / to F32 and F16 only (Cast.cpp:59-73); not a storage
+                                     type of mi_module tensors */ };
 typedef struct mi_cast_attr {
   int64_t num_elem;           /* module::getNumElements(getOutput()) */
   int in_type, out_type;      /* MI_ST_*: module::getStorageType() of input / output */

@@ -1267,7 +1267,7 @@ int orc_requant_int(const orc_rq_attr *a, const float *input, float *output) {
 
 /* ---------------------------------------------------------------------------
  * tpu.Cast, lib/Dialect/Tpu/Interfaces/Common/Cast.cpp:38-200 (the branches a
- * BM168x module reaches; CV18xx and fp8 are left out and return -1), with
+ * BM168x module reaches; CV18xx is left out and returns -1; 8-bit floats cast from / to F32 and F16 only), with
  * requant()/dequant() of lib/Support/CastUtils.cpp:15-46.
  * ------------------------------------------------------------------------- */
 static int st_is_float(int t) { return t == ORC_ST_F32 || t == ORC_ST_BF16 || t == ORC_ST_F16; }
@@ -1298,6 +1298,17 @@ int orc_cast(const orc_cast_attr *a, const float *in, float *out, int64_t n) {
     for (int64_t i = 0; i < n; ++i) out[i] = orc_F16(in[i]);
   } else if (a->in_type == ORC_ST_F32 && a->out_type == ORC_ST_BF16) {  /* :57-58 */
     for (int64_t i = 0; i < n; ++i) out[i] = orc_BF16(in[i], 0);
+  } else if ((a->in_type == ORC_ST_F32 || a->in_type == ORC_ST_F16) && a->out_type == ORC_ST_F8E4M3) { /* :59-60 */
+    for (int64_t i = 0; i < n; ++i) /* F8E4M3(src, dst, n, 1.0f, true): the quotient by the step 1.0 is the value */
+      out[i] = orc_f8e4m3_to_f32(orc_f32_to_f8e4m3((float)((double)in[i] / 1.0), 1));
+  } else if ((a->in_type == ORC_ST_F32 || a->in_type == ORC_ST_F16) && a->out_type == ORC_ST_F8E5M2) { /* :61-62 */
+    for (int64_t i = 0; i < n; ++i)
+      out[i] = orc_f8e5m2_to_f32(orc_f32_to_f8e5m2((float)((double)in[i] / 1.0)));
+  } else if ((a->in_type == ORC_ST_F8E4M3 || a->in_type == ORC_ST_F8E5M2) &&
+             (a->out_type == ORC_ST_F32 || a->out_type == ORC_ST_F16)) { /* :63-73: the values as they are */
+    memcpy(out, in, (size_t)n * sizeof(float));
+  } else if (a->in_type >= ORC_ST_F8E4M3 || a->out_type >= ORC_ST_F8E4M3) {
+    return 1; /* other combinations with an 8-bit float are not restated */
   } else if (a->out_quant && fin) {                                     /* :77-95 */
     for (int64_t i = 0; i < n; ++i) {
       const float x = a->in_type == ORC_ST_BF16 ? orc_BF16(in[i], 0) : in[i];

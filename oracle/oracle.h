@@ -238,7 +238,8 @@ int orc_requant_int(const orc_rq_attr *attr, const float *input, float *output);
 
 /* ---- tpu.Cast (BM168x branches) ------------------------------------------ */
 /* storage types of the tensor on either side; every element is still handed over as a float (f32-valued) */
-enum { ORC_ST_F32 = 0, ORC_ST_BF16, ORC_ST_F16, ORC_ST_I8, ORC_ST_U8, ORC_ST_I16, ORC_ST_U16, ORC_ST_I32, ORC_ST_U32 };
+enum { ORC_ST_F32 = 0, ORC_ST_BF16, ORC_ST_F16, ORC_ST_I8, ORC_ST_U8, ORC_ST_I16, ORC_ST_U16, ORC_ST_I32, ORC_ST_U32,
+       ORC_ST_F8E4M3, ORC_ST_F8E5M2 /* Cast.cpp:59-73: from / to F32 and F16 only */ };
 typedef struct {
   int in_type, out_type;      /* ORC_ST_* */
   int in_quant, out_quant;    /* the side is a uniform-quantised type */

@@ -18,7 +18,7 @@ HALF_TO_ODD, HALF_TOWARDS_ZERO, TOWARDS_ZERO, AWAY_FROM_ZERO, UP, DOWN = 4, 5, 6
 RQ_TFLITE_LSHIFT, RQ_TFLITE, RQ_MULTIPLIER_SHIFT, RQ_ONLY_SHIFT, RQ_QDM, RQ_ONLY_SCALE = range(6)
 OUT_BF16, OUT_F16, OUT_F32 = 0, 1, 2
 GEMM_F32, GEMM_F64ACC, GEMM_FAST = 0, 1, 2
-ST_F32, ST_BF16, ST_F16, ST_I8, ST_U8, ST_I16, ST_U16, ST_I32, ST_U32 = range(9)
+ST_F32, ST_BF16, ST_F16, ST_I8, ST_U8, ST_I16, ST_U16, ST_I32, ST_U32, ST_F8E4M3, ST_F8E5M2 = range(11)
 
 
 def build(force=False):

@@ -27,6 +27,9 @@ CASES = [  # in, out, in_quant, out_quant, scale, zp, expressed
     ("U8", "F16", True, False, 0.031, 120, "F16"),
     ("F32", "I32", False, False, 1.0, 0, "F32"), ("F32", "I8", False, False, 1.0, 0, "F32"),
     ("F32", "U16", False, False, 1.0, 0, "F32"), ("F32", "F32", False, False, 1.0, 0, "F32"),
+    ("F32", "F8E4M3", False, False, 1.0, 0, "F32"), ("F16", "F8E4M3", False, False, 1.0, 0, "F32"),
+    ("F32", "F8E5M2", False, False, 1.0, 0, "F32"), ("F16", "F8E5M2", False, False, 1.0, 0, "F32"),
+    ("F8E4M3", "F32", False, False, 1.0, 0, "F32"), ("F8E5M2", "F16", False, False, 1.0, 0, "F32"),
 ]
 
 
@@ -40,6 +43,10 @@ def _inputs(in_name, orc):
         return np.clip(np.round(x), -128, 127).astype(np.float32)
     if in_name == "U8":
         return np.clip(np.round(x) + 128, 0, 255).astype(np.float32)
+    if in_name == "F8E4M3":
+        return orc.f8e4m3_to_f32(orc.f32_to_f8e4m3(x, True))
+    if in_name == "F8E5M2":
+        return orc.f8e5m2_to_f32(orc.f32_to_f8e5m2(x))
     return x
 
 
@@ -76,8 +83,32 @@ def test_device_level_native_storage(orc):
     assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), orc.f32_to_bf16(want_y))
 
 
+def test_device_level_8bit_float_codes(orc):
+    """f32 / f16 device tensors -> one-byte E4M3 / E5M2 codes -> f32 / f16, against the oracle's code converters."""
+    import torch
+    x = np.concatenate([_values(21, n=50000, spread=60.0), _values(22, n=20000, spread=0.05),
+                        np.float32([17, 19, -21, 440, 447.9, 448, 464, 1e4, -1e4])])
+    xd = torch.from_numpy(x).cuda()
+    for st, enc, dec in ((clib.ST_F8E4M3, lambda v: orc.f32_to_f8e4m3(v, True), orc.f8e4m3_to_f32),
+                         (clib.ST_F8E5M2, orc.f32_to_f8e5m2, orc.f8e5m2_to_f32)):
+        codes = M_.cast_launch(xd, in_type=clib.ST_F32, out_type=st)
+        codes_h = M_.cast_launch(xd.half(), in_type=clib.ST_F16, out_type=st)
+        back = M_.cast_launch(codes, in_type=st, out_type=clib.ST_F32)
+        back_h = M_.cast_launch(codes, in_type=st, out_type=clib.ST_F16)
+        torch.cuda.synchronize()
+        want = enc(x)
+        assert codes.dtype == torch.uint8 and np.array_equal(codes.cpu().numpy(), want)
+        assert np.array_equal(codes_h.cpu().numpy(), enc(orc.F16(x)))
+        assert np.array_equal(back.cpu().numpy().view(np.uint32), dec(want).view(np.uint32))
+        assert np.array_equal(back_h.float().cpu().numpy().view(np.uint32), dec(want).view(np.uint32))
+
+
 def test_unsupported_branches_fail_loudly():
     x = np.zeros(8, dtype=np.float32)
+    with pytest.raises(clib.BackendError):  # an 8-bit float casts from and to F32 / F16 only
+        M_.cast(x, in_type=clib.ST_BF16, out_type=clib.ST_F8E4M3)
+    with pytest.raises(clib.BackendError):
+        M_.cast(x, in_type=clib.ST_F8E5M2, out_type=clib.ST_I8)
     with pytest.raises(clib.BackendError):
         M_.cast(x, in_type=clib.ST_F32, out_type=clib.ST_I8, out_quant=True, scale=0.1, chip=clib.CHIP_CV18XX)
     with pytest.raises(clib.BackendError):

@@ -87,3 +87,48 @@ def test_float_to_plain_integers_and_rounding_modes(orc):
     assert np.array_equal(orc.cast(small, in_type=orc.ST_F32, out_type=orc.ST_I32, round_mode=orc.HALF_TO_EVEN), even)
     # anything else is a copy (:172-174)
     assert np.array_equal(orc.cast(x, in_type=orc.ST_F32, out_type=orc.ST_F32), x)
+
+
+def _nearest_on_grid(x, positive, max_value):
+    """Brute-force round-to-nearest (ties to the even code) onto an ascending table of non-negative grid values,
+    magnitudes beyond the table's end clamped to it."""
+    pos = positive.astype(np.float64)
+    ax = np.minimum(np.abs(x).astype(np.float64), max_value)
+    idx = np.clip(np.searchsorted(pos, ax), 1, len(pos) - 1)
+    lo, hi = pos[idx - 1], pos[idx]
+    dl, dh = ax - lo, hi - ax
+    pick_hi = (dh < dl) | ((dh == dl) & (idx % 2 == 0))
+    return np.copysign(np.where(pick_hi, hi, lo), x).astype(np.float32)
+
+
+def _f8_values(seed, limit):
+    rng = np.random.default_rng(seed)
+    x = np.concatenate([_values(seed), (rng.standard_normal(2000) * 0.05).astype(np.float32),
+                        (rng.standard_normal(2000) * 3000).astype(np.float32),
+                        np.float32([17, 19, 21, -17, 23, 0.0, -0.0, 440, 447.9, 448, 464, 1e4, -1e4, 36, 44, -52])])
+    return np.clip(x, -limit, limit)
+
+
+@pytest.mark.parametrize("in_type", ["ST_F32", "ST_F16"])
+def test_cast_to_8bit_floats_is_nearest_grid_value(orc, in_type):
+    """Cast.cpp:59-62 against a brute-force nearest-value search over the decoded code tables: E4M3 saturates at
+    448, E5M2 is checked inside its finite range (its conversion does not saturate)."""
+    e4 = orc.f8e4m3_to_f32(np.arange(0x7f, dtype=np.uint8))   # 0x7f is NaN
+    e5 = orc.f8e5m2_to_f32(np.arange(0x7c, dtype=np.uint8))   # 0x7c.. are inf / NaN
+    assert e4[-1] == 448.0 and e5[-1] == 57344.0 and np.all(np.diff(e4) > 0) and np.all(np.diff(e5) > 0)
+    for out_type, table, limit in (("ST_F8E4M3", e4, 3e4), ("ST_F8E5M2", e5, 57344.0)):
+        x = _f8_values(5, limit)
+        if in_type == "ST_F16":
+            x = orc.F16(x)
+        got = orc.cast(x, in_type=getattr(orc, in_type), out_type=getattr(orc, out_type))
+        want = _nearest_on_grid(x, table, float(table[-1]))
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_cast_from_8bit_floats_keeps_values(orc):
+    """Cast.cpp:63-73: the interpreter hands grid values over unchanged."""
+    v = orc.f8e4m3_to_f32(np.arange(0x7f, dtype=np.uint8))
+    for o in (orc.ST_F32, orc.ST_F16):
+        assert np.array_equal(orc.cast(v, in_type=orc.ST_F8E4M3, out_type=o), v)
+    with pytest.raises(RuntimeError):
+        orc.cast(v, in_type=orc.ST_F8E4M3, out_type=orc.ST_I8)

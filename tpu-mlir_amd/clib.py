@@ -11,7 +11,7 @@ ROUND_TOWARDS_ZERO, ROUND_UP, ROUND_DOWN = 6, 8, 9
 RQ_TFLITE_LSHIFT, RQ_TFLITE, RQ_MULTIPLIER_SHIFT, RQ_ONLY_SHIFT, RQ_QDM = 0, 1, 2, 3, 4
 DT_BF16, DT_F16, DT_I8, DT_U8, DT_I16, DT_U16, DT_I32 = range(7)
 CHIP_BM168X, CHIP_CV18XX = 0, 1
-ST_F32, ST_BF16, ST_F16, ST_I8, ST_U8, ST_I16, ST_U16, ST_I32, ST_U32 = range(9)
+ST_F32, ST_BF16, ST_F16, ST_I8, ST_U8, ST_I16, ST_U16, ST_I32, ST_U32, ST_F8E4M3, ST_F8E5M2 = range(11)
 
 # every symbol include/tpumlir_amd.h declares
 EXPORTS = [

@@ -917,9 +917,17 @@ static bool st_float(int t) { return t == MI_ST_F32 || t == MI_ST_BF16 || t == M
 namespace mi {
 int cast_scalars(const mi_cast_attr *a, float *inv_scale, float *scale) {
   MI_REQUIRE(a, MI_BAD_ARGUMENT, "mi_cast: null attribute");
-  MI_REQUIRE(a->in_type >= MI_ST_F32 && a->in_type <= MI_ST_U32 && a->out_type >= MI_ST_F32 &&
-                 a->out_type <= MI_ST_U32,
-             MI_UNSUPPORTED, "mi_cast: storage type not handled (fp8 casts run on the CPU path)");
+  MI_REQUIRE(a->in_type >= MI_ST_F32 && a->in_type <= MI_ST_F8E5M2 && a->out_type >= MI_ST_F32 &&
+                 a->out_type <= MI_ST_F8E5M2,
+             MI_UNSUPPORTED, "mi_cast: storage type not handled");
+  {  // 8-bit floats: from and to F32 / F16 only, never quantized (Cast.cpp:59-73)
+    const bool f8_in = a->in_type >= MI_ST_F8E4M3, f8_out = a->out_type >= MI_ST_F8E4M3;
+    const bool wide_in = a->in_type == MI_ST_F32 || a->in_type == MI_ST_F16;
+    const bool wide_out = a->out_type == MI_ST_F32 || a->out_type == MI_ST_F16;
+    MI_REQUIRE((!f8_in && !f8_out) || (f8_out && wide_in && !a->in_quant && !a->out_quant) ||
+                   (f8_in && wide_out && !a->in_quant && !a->out_quant),
+               MI_UNSUPPORTED, "mi_cast: an 8-bit float casts from and to F32 / F16 only");
+  }
   MI_REQUIRE(a->chip == MI_CHIP_BM168X, MI_UNSUPPORTED, "mi_cast: the CV18xx bf16 table arithmetic is not built");
   MI_REQUIRE(a->num_elem >= 0, MI_BAD_ARGUMENT, "mi_cast: negative element count");
   *inv_scale = 1.0f;

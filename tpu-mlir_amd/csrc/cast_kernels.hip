@@ -19,7 +19,9 @@ struct CastArgs {
 };
 
 __device__ __forceinline__ int st_size(int t) {
-  return (t == MI_ST_F32 || t == MI_ST_I32 || t == MI_ST_U32) ? 4 : ((t == MI_ST_I8 || t == MI_ST_U8) ? 1 : 2);
+  return (t == MI_ST_F32 || t == MI_ST_I32 || t == MI_ST_U32)
+             ? 4
+             : ((t == MI_ST_I8 || t == MI_ST_U8 || t == MI_ST_F8E4M3 || t == MI_ST_F8E5M2) ? 1 : 2);
 }
 
 // the value the interpreter would hold in its float tensor for element i
@@ -33,6 +35,8 @@ __device__ __forceinline__ float load_as_float(const void *p, int64_t i, int t) 
   case MI_ST_I16: return (float)((const int16_t *)p)[i];
   case MI_ST_U16: return (float)((const uint16_t *)p)[i];
   case MI_ST_I32: return (float)((const int32_t *)p)[i];
+  case MI_ST_F8E4M3: return f8e4m3_to_f32(((const uint8_t *)p)[i]);
+  case MI_ST_F8E5M2: return f8e5m2_to_f32(((const uint8_t *)p)[i]);
   default: return (float)((const uint32_t *)p)[i];
   }
 }
@@ -48,6 +52,8 @@ __device__ __forceinline__ void store_from_float(void *p, int64_t i, int t, floa
   case MI_ST_I16: ((int16_t *)p)[i] = (int16_t)(int32_t)v; break;
   case MI_ST_U16: ((uint16_t *)p)[i] = (uint16_t)(int32_t)v; break;
   case MI_ST_I32: ((int32_t *)p)[i] = (int32_t)(int64_t)v; break;
+  case MI_ST_F8E4M3: ((uint8_t *)p)[i] = (uint8_t)f8e4m3_from_f32(v); break;  // v is already on the grid
+  case MI_ST_F8E5M2: ((uint8_t *)p)[i] = (uint8_t)f8e5m2_from_f32(v); break;
   default: ((uint32_t *)p)[i] = (uint32_t)(int64_t)v; break;
   }
 }
@@ -75,6 +81,14 @@ __device__ __forceinline__ float cast_one(float x, const CastArgs &a) {
     return F16r(x);
   if (a.in_type == MI_ST_F32 && a.out_type == MI_ST_BF16)
     return BF16r(x);
+  // Cast.cpp:59-73: F8E4M3(x, 1.0, true) (saturating), F8E5M2(x, 1.0, true) (whose conversion never saturates,
+  // Float8.cpp:134-138); the other direction hands the values over as they are
+  if (a.out_type == MI_ST_F8E4M3)
+    return f8e4m3_to_f32(f8e4m3_from_f32(x));
+  if (a.out_type == MI_ST_F8E5M2)
+    return f8e5m2_to_f32(f8e5m2_from_f32(x));
+  if (a.in_type == MI_ST_F8E4M3 || a.in_type == MI_ST_F8E5M2)
+    return x;
   if (a.out_quant && fin) {
     if (a.in_type == MI_ST_BF16)
       x = BF16r(x);

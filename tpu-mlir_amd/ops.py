@@ -463,7 +463,8 @@ def a16mm_launch_group(ws, x, ys=None, ys_f32=None, stream=None):
 
 
 _ST_TORCH = {clib.ST_F32: "float32", clib.ST_BF16: "bfloat16", clib.ST_F16: "float16", clib.ST_I8: "int8",
-             clib.ST_U8: "uint8", clib.ST_I16: "int16", clib.ST_U16: "int16", clib.ST_I32: "int32", clib.ST_U32: "int32"}
+             clib.ST_U8: "uint8", clib.ST_I16: "int16", clib.ST_U16: "int16", clib.ST_I32: "int32", clib.ST_U32: "int32",
+             clib.ST_F8E4M3: "uint8", clib.ST_F8E5M2: "uint8"}  # 8-bit floats travel as their codes
 
 
 def cast_launch(x, *, in_type, out_type, in_quant=False, out_quant=False, scale=1.0, zero_point=0, expressed=None,
