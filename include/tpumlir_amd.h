@@ -307,6 +307,11 @@ typedef struct mi_requant_desc {
   const int32_t *d_multiplier; int32_t multiplier;
   const int32_t *d_shift;      int32_t shift;
   const int32_t *d_zp;         int32_t zp;
+  int per_channel_q31_checked; /* 1: the caller has checked that every d_shift[n] lies in [1, 31] and no
+                                * d_multiplier[n] is INT32_MIN.  Allows the 32-bit epilogue for the Q31 modes with
+                                * per-channel arrays (round half away from zero, int8 output); 0 keeps such arrays
+                                * on the general 64-bit path.  Scalars are checked by the library itself.  Results
+                                * are identical either way. */
 } mi_requant_desc;
 
 /* acc[M,N] = (A - input_zp)[M,K] * (B - right_zp) + bias[N], relu, then requant -> d_out.

@@ -268,11 +268,11 @@ def test_gpu_producers_and_dynamic_against_fixtures():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", A16_CASES)
-def test_gpu_a16_against_fixture(name, monkeypatch):
+def test_gpu_a16_against_fixture(name, plan):
     import torch
     M_ = pkg()
     cmp = pkg("compare")
-    monkeypatch.setenv("MI_A16_GEMM_MIN_M", "17")  # w4_prefill (M = 40) goes through the tiled kernel
+    plan(a16_gemm_min_m=17)  # w4_prefill (M = 40) goes through the tiled kernel
     d = _load("case_a16_%s.npz" % name)
     cfg = _a16_cfg(d)
     w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"],

@@ -86,9 +86,9 @@ PREFILL_CASES = [  # (bits, M, K, N, g, signed): M > 16 takes the tiled MFMA GEM
 
 @pytest.mark.parametrize("tile", ["128", "256"])
 @pytest.mark.parametrize("bits,M,K,N,g,signed", PREFILL_CASES)
-def test_prefill_gemm_device_level(orc, monkeypatch, bits, M, K, N, g, signed, tile):
-    monkeypatch.setenv("MI_A16_GEMM_TILE", tile)  # both block shapes of the tiled kernel
-    monkeypatch.setenv("MI_A16_GEMM_MIN_M", "17")  # ... from the smallest M it accepts (also the default)
+def test_prefill_gemm_device_level(orc, plan, bits, M, K, N, g, signed, tile):
+    # both block shapes of the tiled kernel, from the smallest M it accepts (also the default)
+    plan(a16_gemm_tile=int(tile), a16_gemm_min_m=17)
     if bits == 4:
         cfg = S.w4a16(M, K, N, g, seed=M + K + N, bias=(N % 3 == 0))
     else:
@@ -99,27 +99,27 @@ def test_prefill_gemm_device_level(orc, monkeypatch, bits, M, K, N, g, signed, t
 
 @pytest.mark.parametrize("bits,M,K,N,g", [(4, 8, 1024, 272, 128), (4, 16, 512, 130, 64), (4, 2, 2048, 128, 0),
                                          (8, 5, 512, 96, 128), (8, 13, 1024, 200, 0)])
-def test_tiled_kernel_sixteen_row_blocks(orc, monkeypatch, bits, M, K, N, g):
+def test_tiled_kernel_sixteen_row_blocks(orc, plan, bits, M, K, N, g):
     """At most 16 rows through the tiled kernel (what large matrices take from 8 rows on)."""
-    monkeypatch.setenv("MI_A16_GEMM_MIN_M", "2")
+    plan(a16_gemm_min_m=2)
     cfg = S.w4a16(M, K, N, g, seed=M + N, bias=(N % 8 == 0)) if bits == 4 else S.w8a16(M, K, N, g, seed=M + N)
     out, pre = _run_device(cfg)
     _check_against_oracle(orc, cfg, out, pre)
 
 
 @pytest.mark.parametrize("bits,M,K,N,g", [(4, 64, 4096, 256, 128), (4, 130, 2048, 512, 64), (8, 48, 2048, 384, 128)])
-def test_prefill_gemm_split_k(orc, monkeypatch, bits, M, K, N, g):
+def test_prefill_gemm_split_k(orc, plan, bits, M, K, N, g):
     """Few output blocks, long K: the product is split along K over several workgroups (fp32 atomics + a finishing
     pass); twice in a row, the second call finding the partial-sum buffer the first one left behind."""
-    monkeypatch.setenv("MI_A16_GEMM_MIN_M", "17")
+    plan(a16_gemm_min_m=17)
     cfg = S.w4a16(M, K, N, g, seed=M + N, bias=True) if bits == 4 else S.w8a16(M, K, N, g, seed=M + N, bias=True)
     for _ in range(2):
         out, pre = _run_device(cfg)
         _check_against_oracle(orc, cfg, out, pre)
 
 
-def test_prefill_gemm_full_width_and_f16_mode(orc, monkeypatch):
-    monkeypatch.setenv("MI_A16_GEMM_MIN_M", "17")
+def test_prefill_gemm_full_width_and_f16_mode(orc, plan):
+    plan(a16_gemm_min_m=17)
     cfg = S.w4a16(192, 1024, 1024, 128, seed=77, bias=True)
     out, pre = _run_device(cfg)
     _check_against_oracle(orc, cfg, out, pre)
@@ -146,10 +146,10 @@ def test_w4a16_device_level(orc, M, K, N, g):
 
 
 @pytest.mark.parametrize("bits,M,K,N,g", [(4, 40, 512, 64, 128), (4, 33, 1024, 100, 64), (8, 32, 4096, 1024, 0)])
-def test_skinny_kernel_with_several_row_blocks(orc, monkeypatch, bits, M, K, N, g):
+def test_skinny_kernel_with_several_row_blocks(orc, plan, bits, M, K, N, g):
     """More than 16 rows normally go to the tiled kernel; the skinny kernel still has to handle them (it is what runs
     when K is not a multiple of 128), one pass over the weights per 16 rows."""
-    monkeypatch.setenv("MI_A16_NO_GEMM", "1")
+    plan(a16_no_gemm=1)
     cfg = S.w4a16(M, K, N, g, seed=M + K) if bits == 4 else S.w8a16(M, K, N, g, seed=M + K, signed=True)
     out, pre = _run_device(cfg)
     _check_against_oracle(orc, cfg, out, pre)

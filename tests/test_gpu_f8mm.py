@@ -57,8 +57,8 @@ CASES = [  # (M, K, N, right_transpose, relu, per_channel, bias)
 
 @pytest.mark.parametrize("tile", ["64", "128", "256"])
 @pytest.mark.parametrize("M,K,N,rt,relu,per_channel,bias", CASES)
-def test_f8_matmul_device_level(orc, monkeypatch, M, K, N, rt, relu, per_channel, bias, tile):
-    monkeypatch.setenv("MI_F8_TILE", tile)  # both tile shapes of the ring kernels (K % 64 != 0 takes neither)
+def test_f8_matmul_device_level(orc, plan, M, K, N, rt, relu, per_channel, bias, tile):
+    plan(f8_tile=int(tile))  # both tile shapes of the ring kernels (K % 64 != 0 takes neither)
     rng = np.random.default_rng(M + K + N)
     a = _codes(rng, (M, K), top=0x58)                       # magnitudes up to 16: sums stay far from fp32 overflow
     b = _codes(rng, (N, K) if rt else (K, N), top=0x58)
@@ -214,8 +214,8 @@ E5M2_CASES = [  # (M, K, N, right_transpose, relu, bias)
 
 @pytest.mark.parametrize("tile", ["64", "128", "256"])
 @pytest.mark.parametrize("M,K,N,rt,relu,bias", E5M2_CASES)
-def test_e5m2_matmul_device_level(orc, monkeypatch, M, K, N, rt, relu, bias, tile):
-    monkeypatch.setenv("MI_F8_TILE", tile)
+def test_e5m2_matmul_device_level(orc, plan, M, K, N, rt, relu, bias, tile):
+    plan(f8_tile=int(tile))
     rng = np.random.default_rng(M + K + N + 1)
     a = _e5m2_codes(rng, (M, K))
     b = _e5m2_codes(rng, (N, K) if rt else (K, N))

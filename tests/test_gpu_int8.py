@@ -104,17 +104,15 @@ def test_zero_points_unsigned_operands_relu_and_int16(orc):
     want = (a.astype(np.int64) - 3) @ (bu.astype(np.int64).T - 128)
     assert np.array_equal(out.cpu().numpy().astype(np.int64), want)
 
-@pytest.mark.parametrize("tile", ["256", "128/8", "128/4", "128/64", "0"])
+@pytest.mark.parametrize("tile", ["256", "128/8", "128/4", "128/64", "-1"])
 @pytest.mark.parametrize("rt", [True, False])
-def test_large_tile_path_unsigned_zero_points_relu_ragged_edges(orc, monkeypatch, rt, tile):
+def test_large_tile_path_unsigned_zero_points_relu_ragged_edges(orc, plan, rt, tile):
     """Each of the GEMM kernels (256x256 direct-to-LDS tiles; 128x128 tiles with a ring of 8 or 4 stages and the
     64x64-tile form of the same kernel; register-staged 128x128) on a shape all of them accept (M, N >= 128,
     K % 128 == 0), with everything the small cases cover: unsigned operands, both zero points, bias, relu with a
     limit, a ragged last tile in M and N, per-channel Q31 requant with per-channel output zero points, and the int32
     side output."""
-    monkeypatch.setenv("MI_I8_TILE", tile.split("/")[0])
-    if "/" in tile:
-        monkeypatch.setenv("MI_I8_MID_RING", tile.split("/")[1])
+    plan(i8_tile=int(tile.split("/")[0]), i8_mid_ring=int(tile.split("/")[1]) if "/" in tile else 0)
     torch = _torch()
     rng = np.random.default_rng(11)
     M, K, N = 300, 384, 272

@@ -90,7 +90,7 @@ class RequantDescC(C.Structure):
     _fields_ = [("quant_mode", C.c_int), ("round_mode", C.c_int), ("chip", C.c_int), ("out_dtype", C.c_int),
                 ("d_multiplier", C.c_void_p), ("multiplier", C.c_int32),
                 ("d_shift", C.c_void_p), ("shift", C.c_int32),
-                ("d_zp", C.c_void_p), ("zp", C.c_int32)]
+                ("d_zp", C.c_void_p), ("zp", C.c_int32), ("per_channel_q31_checked", C.c_int)]
 
 
 class RqAxisAttr(C.Structure):

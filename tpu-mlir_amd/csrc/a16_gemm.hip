@@ -28,15 +28,6 @@ constexpr int GEMM_NST = 3;      // LDS ring depth
 constexpr int GEMM_WAVES = 8;
 constexpr int waitcnt_vm_only(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
 
-#ifdef MI_GEMM_TIMING
-__device__ unsigned long long mi_gemm_dbg[64 * 8];
-extern "C" int mi_gemm_dbg_dump(unsigned long long *host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mi_gemm_dbg), sizeof(mi_gemm_dbg));
-}
-#define MI_GT(v) const unsigned long long v = __builtin_readcyclecounter()
-#else
-#define MI_GT(v)
-#endif
 
 // One weight set of a launch.  Sibling sets on one input (q/k/v, gate/up: same K, width, group size and type) share a
 // launch: their output blocks are numbered one set after the other.
@@ -67,10 +58,13 @@ struct GemmArgs {
   int tiles_per_group;  // GPT == 1: weight tiles that share one group (g / TILE_K; k_tiles when per channel)
   int chip;
   int tiles_m, per_xcd;
-  // split K: each output block is computed by k_splits workgroups over kt_per_split stages each, which add their
-  // fp32 partial sums into acc [M, N] (zero on entry); bias and rounding happen in a16_gemm_finish_kernel
+  // split K: each output block is computed by k_splits workgroups over kt_per_split stages each; workgroup `split`
+  // stores its fp32 partial sums into its own slab, slab + split * slab_stride, laid out like the outputs ([M, N] per
+  // weight set, one set after the other).  a16_gemm_finish_kernel adds the slabs in split order, so the result does
+  // not depend on which workgroup finishes first; bias and rounding happen there.
   int k_splits, kt_per_split;
-  float *acc;
+  float *slab;
+  int64_t slab_stride;
 };
 
 // WM x WN waves, each TM x TN MFMA tiles of 16 x 16:  GM = WM * TM * 16 rows, GN = WN * TN * 16 columns.
@@ -314,31 +308,15 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
       load_w(wa, 0);  // issue order: x(0), W(0), x(1)
     issue_x(s0);
   }
-#ifdef MI_GEMM_TIMING
-  unsigned long long t_wait = 0, t_bar = 0, t_issue = 0, t_comp = 0;
-  const unsigned long long t_begin = __builtin_readcyclecounter();
-#endif
   auto stage = [&](WStage &cur, WStage &nxt, int kt) {
-    MI_GT(g0);
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_only((GEMM_NST - 2) * LPS));
-    MI_GT(g1);
     __builtin_amdgcn_s_barrier();
-    MI_GT(g2);
     if constexpr (WLDS)
       read_w(cur, kt);
     else
       load_w(nxt, kt + 1);
     issue_x(kt + GEMM_NST - 1);
-    MI_GT(g3);
     compute_stage(cur, kt);
-#ifdef MI_GEMM_TIMING
-    __builtin_amdgcn_sched_barrier(0);
-    const unsigned long long g4 = __builtin_readcyclecounter();
-    t_wait += g1 - g0;
-    t_bar += g2 - g1;
-    t_issue += g3 - g2;
-    t_comp += g4 - g3;
-#endif
   };
   int kt = 0;
   for (; kt + 1 < kt_total; kt += 2) {
@@ -348,16 +326,6 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
   if (kt < kt_total)
     stage(wa, wb, kt);
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_only(0));  // drain the re-loads issued past the end
-#ifdef MI_GEMM_TIMING
-  if (lane == 0 && blockIdx.x < 64 && wave == 0) {
-    unsigned long long *d = mi_gemm_dbg + blockIdx.x * 8;
-    d[0] = __builtin_readcyclecounter() - t_begin;
-    d[1] = t_wait;
-    d[2] = t_bar;
-    d[3] = t_issue;
-    d[4] = t_comp;
-  }
-#endif
 
   // ---- epilogue: lane holds column (l & 15), rows 4 (l >> 4) + r of each 16 x 16 tile
 #pragma unroll
@@ -370,8 +338,8 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int64_t m = m_base + (wm * TM + i) * 16 + 4 * kq + r;
-        if (n_ok && m < a.M && a.acc) {
-          atomicAdd(a.acc + sg.acc_begin + m * sg.N + n, acc[i][j][r]);  // bias and rounding: a16_gemm_finish_kernel
+        if (n_ok && m < a.M && a.slab) {
+          a.slab[split * a.slab_stride + sg.acc_begin + m * sg.N + n] = acc[i][j][r];  // summed by the finishing pass
         } else if (n_ok && m < a.M) {
           const float v = acc[i][j][r] + b;
           const int64_t o = m * sg.N + n;
@@ -383,10 +351,12 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
   }
 }
 
-// Second half of a split-K product: y = round16(acc + bias) (and the fp32 value, if asked for), and acc goes back to
-// zero so that the next product on this stream finds it clean.  One launch covers every weight set of the product.
+// Second half of a split-K product: y = round16(slab 0 + slab 1 + ... + bias), added in that order (and the fp32
+// value, if asked for).  One launch covers every weight set of the product.
 struct FinishArgs {
-  float *acc;
+  const float *slab;
+  int64_t slab_stride;
+  int k_splits;
   const float *bias[GEMM_MAX_SEG];
   uint16_t *y[GEMM_MAX_SEG];
   float *y32[GEMM_MAX_SEG];
@@ -401,8 +371,15 @@ __global__ void a16_gemm_finish_kernel(FinishArgs f) {
   const int64_t i4 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (i4 >= f.total)
     return;
-  const f32x4 v4 = *(const f32x4 *)(f.acc + i4);  // every N % 4 == 0 (checked by the host): a group of 4 stays in one row
-  *(f32x4 *)(f.acc + i4) = f32x4{0.f, 0.f, 0.f, 0.f};
+  // every N % 4 == 0 (checked by the host): a group of 4 stays in one row
+  f32x4 v4 = *(const f32x4 *)(f.slab + i4);
+  for (int sp = 1; sp < f.k_splits; ++sp) {
+    const f32x4 t = *(const f32x4 *)(f.slab + sp * f.slab_stride + i4);
+    v4[0] += t[0];
+    v4[1] += t[1];
+    v4[2] += t[2];
+    v4[3] += t[3];
+  }
   const int si = (i4 >= f.begin[1] ? 1 : 0) + (i4 >= f.begin[2] ? 1 : 0);
   // selected, not indexed: a runtime index would move the argument arrays to scratch memory
   const float *bias = si == 0 ? f.bias[0] : si == 1 ? f.bias[1] : f.bias[2];
@@ -423,7 +400,7 @@ __global__ void a16_gemm_finish_kernel(FinishArgs f) {
 }
 
 template <int BITS, int DT, int GPT, int WM, int WN, int TM, int TN>
-static int launch_gemm_instance(GemmArgs &a, hipStream_t st) {
+static int launch_gemm_instance(GemmArgs &a, hipStream_t st, const A16Scratch *fixed) {
   constexpr int GM = WM * TM * 16, GN = WN * TN * 16;
   a.tiles_m = (int)((a.M + GM - 1) / GM);
   int64_t tiles = 0, acc_elems = 0;
@@ -448,36 +425,43 @@ static int launch_gemm_instance(GemmArgs &a, hipStream_t st) {
   // four stages each
   const int kt_all = (int)(a.K / GEMM_KS);
   int splits = 1;
-  const char *e = getenv("MI_A16_GEMM_SPLITS");  // development switch
-  if (e)
-    splits = atoi(e);
+  if (plan().a16_gemm_splits > 0)
+    splits = plan().a16_gemm_splits;
   else if (tiles < 160 && n4)
     splits = std::min(std::max(256 / (int)tiles, 1), std::max(kt_all / 4, 1));
   splits = std::max(1, std::min(splits, kt_all));
   a.kt_per_split = (kt_all + splits - 1) / splits;
   a.k_splits = (kt_all + a.kt_per_split - 1) / a.kt_per_split;  // no empty split
-  a.acc = nullptr;
+  a.slab = nullptr;
+  a.slab_stride = (acc_elems + 3) & ~(int64_t)3;  // slabs stay 16-byte aligned
   if (a.k_splits > 1) {
     MI_REQUIRE(n4, MI_BAD_ARGUMENT, "a16 split-K product: N must be a multiple of 4");
-    // fp32 partial sums: the stream's own buffer, zero whenever no product is in flight (the finishing pass clears
-    // what it reads)
-    int rc = stream_workspace(st, WS_SPLIT_K, (size_t)acc_elems * sizeof(float), true, (void **)&a.acc);
-    if (rc != MI_SUCCESS)
-      return rc;
+    // fp32 partial sums, one slab per split: the caller's fixed scratch, or the stream's own buffer.  Every element a
+    // finishing pass reads was written by this launch, so the buffer needs no clearing.
+    const size_t need = (size_t)a.k_splits * a.slab_stride * sizeof(float);
+    if (fixed) {
+      MI_REQUIRE(need <= fixed->bytes, MI_BAD_ARGUMENT,
+                 "this product needs " + std::to_string(need) + " bytes of split-K scratch, more than the " +
+                     std::to_string(fixed->bytes) + " bytes of the library's fixed scratch area: use mi_a16mm_launch");
+      a.slab = (float *)fixed->ptr;
+    } else {
+      int rc = stream_workspace(st, WS_SPLIT_K, need, (void **)&a.slab);
+      if (rc != MI_SUCCESS)
+        return rc;
+    }
   }
   a.per_xcd = (a.tiles_total * a.k_splits + 7) / 8;
   auto kfn = a16_gemm_kernel<BITS, DT, GPT, WM, WN, TM, TN>;
   const size_t lds_bytes =
       (size_t)GEMM_NST * ((GM < 32 ? 32 : GM) * GEMM_KS * 2 + (BITS == 4 ? (GN / 16) * 1024 + GEMM_WAVES * GPT * 256 : 0));
-  static bool attr_set = false;
-  if (!attr_set) {
-    (void)hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    attr_set = true;
-  }
+  static LdsLimitOnce lds_limit;
+  lds_limit.ensure((const void *)kfn, 160 * 1024);
   kfn<<<dim3((unsigned)(a.per_xcd * 8)), dim3(GEMM_WAVES * 64), lds_bytes, st>>>(a);
   if (a.k_splits > 1) {
     FinishArgs f;
-    f.acc = a.acc;
+    f.slab = a.slab;
+    f.slab_stride = a.slab_stride;
+    f.k_splits = a.k_splits;
     for (int i = 0; i < GEMM_MAX_SEG; ++i) {
       const GemmSeg &sg = a.seg[i];
       f.bias[i] = sg.bias;
@@ -494,33 +478,32 @@ static int launch_gemm_instance(GemmArgs &a, hipStream_t st) {
 }
 
 template <int BITS, int DT, int GPT>
-static int launch_gemm_shape(GemmArgs &a, hipStream_t st) {
+static int launch_gemm_shape(GemmArgs &a, hipStream_t st, const A16Scratch *fixed) {
   // 128 x 256 blocks when they fill the chip, else 128 x 128
   int64_t big = 0;
   for (int i = 0; i < a.n_seg; ++i)
     big += ((a.M + 127) / 128) * ((a.seg[i].N + 255) / 256);
-  const char *e = getenv("MI_A16_GEMM_TILE");  // development switch: "256" / "128"
+  const int tile = plan().a16_gemm_tile;
   constexpr bool fits = !(BITS == 4 && GPT == 4);  // 32-wide groups: a 256-column block's scale|zp words overflow LDS
-  const bool wide = fits && (e ? atoi(e) == 256 : big >= 192);
+  const bool wide = fits && (tile ? tile == 256 : big >= 192);
   if constexpr (fits) {
     if (wide)
-      return launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 4>(a, st);
+      return launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 4>(a, st, fixed);
   }
   (void)wide;
   // few rows: shorter blocks waste fewer MFMAs on rows that do not exist
-  const char *r = getenv("MI_A16_GEMM_ROWS");  // development switch: "32" / "64" / "128"
-  const int rows = r ? atoi(r) : (a.M <= 16 ? 16 : a.M <= 32 ? 32 : a.M <= 640 ? 64 : 128);  // measured: 64-row blocks win up to there
+  const int rows = plan().a16_gemm_rows ? plan().a16_gemm_rows : (a.M <= 16 ? 16 : a.M <= 32 ? 32 : a.M <= 640 ? 64 : 128);  // measured: 64-row blocks win up to there
   if (rows == 16)
-    return launch_gemm_instance<BITS, DT, GPT, 1, 8, 1, 1>(a, st);
+    return launch_gemm_instance<BITS, DT, GPT, 1, 8, 1, 1>(a, st, fixed);
   if (rows == 32)
-    return launch_gemm_instance<BITS, DT, GPT, 2, 4, 1, 2>(a, st);
+    return launch_gemm_instance<BITS, DT, GPT, 2, 4, 1, 2>(a, st, fixed);
   if (rows == 64)
-    return launch_gemm_instance<BITS, DT, GPT, 2, 4, 2, 2>(a, st);
-  return launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 2>(a, st);
+    return launch_gemm_instance<BITS, DT, GPT, 2, 4, 2, 2>(a, st, fixed);
+  return launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 2>(a, st, fixed);
 }
 
 bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M) {
-  if (getenv("MI_A16_NO_GEMM"))
+  if (plan().a16_no_gemm)
     return false;
   const int tile_k = w->bits == 4 ? W4_TILE_K : W8_TILE_K;
   const int g = w->g;
@@ -533,25 +516,20 @@ bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M) {
   //   11008 x 4096   M = 8: 11.3 / 13.0  M = 12: 12.9 / 13.4   M = 16: 14.9 / 13.5
   //   4096 x 11008   M = 6: 12.2 / 11.4  M = 8: 13.9 / 12.2    (long K: few, long workgroups in the skinny kernel)
   //   32000 x 4096   M = 6: 22.6 / 22.9  M = 8: 25.1 / 22.2
-  const char *e = getenv("MI_A16_GEMM_MIN_M");  // development / test switch
   const int64_t nk = w->N * w->K;
   bool rows_ok;
-  if (e)
-    rows_ok = M >= atoll(e) && M > 1;
+  if (plan().a16_gemm_min_m > 0)
+    rows_ok = M >= plan().a16_gemm_min_m && M > 1;
   else
     rows_ok = M >= 17 || (M >= 13 && nk >= (int64_t(1) << 25)) || (M >= 8 && nk >= (int64_t(1) << 26)) ||
               (M >= 6 && w->K >= 8192 && nk >= (int64_t(1) << 25));
   return rows_ok && (w->K % GEMM_KS) == 0 && group_ok;
 }
 
-int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
-                    hipStream_t stream) {
-  return a16_gemm_launch_group(&w, 1, d_x, M, &d_y, d_y32 ? &d_y32 : nullptr, stream);
-}
 
 // ws[0..n): sibling weight sets on one input -- same K, width, group size, type and chip (checked by the caller)
 int a16_gemm_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
-                          float *const *d_y32s, hipStream_t stream) {
+                          float *const *d_y32s, hipStream_t stream, const A16Scratch *fixed) {
   MI_REQUIRE(n >= 1 && n <= GEMM_MAX_SEG, MI_BAD_ARGUMENT, "a16 tiled product: one to three weight sets per launch");
   const mi_a16_weight *w = ws[0];
   GemmArgs a;
@@ -589,12 +567,12 @@ int a16_gemm_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t 
     gpt = tile_k / w->g;
   const bool f16 = w->dtype == MI_DT_F16;
   int rc = MI_SUCCESS;
-#define MI_GEMM(BITS_, GPT_)                                      \
-  {                                                               \
-    if (f16)                                                      \
-      rc = launch_gemm_shape<BITS_, MI_DT_F16, GPT_>(a, stream);  \
-    else                                                          \
-      rc = launch_gemm_shape<BITS_, MI_DT_BF16, GPT_>(a, stream); \
+#define MI_GEMM(BITS_, GPT_)                                             \
+  {                                                                      \
+    if (f16)                                                             \
+      rc = launch_gemm_shape<BITS_, MI_DT_F16, GPT_>(a, stream, fixed);  \
+    else                                                                 \
+      rc = launch_gemm_shape<BITS_, MI_DT_BF16, GPT_>(a, stream, fixed); \
   }
   if (w->bits == 4) {
     if (gpt == 1)
@@ -617,3 +595,4 @@ int a16_gemm_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t 
 }
 
 }  // namespace mi
+

@@ -298,27 +298,9 @@ __device__ __forceinline__ void reduce_and_store(const SkinnyArgs &a, float (*re
 // LDS carve-up of the skinny kernel: red | S (XLDS, 4-bit) | x rows (XLDS)
 __host__ __device__ constexpr size_t skinny_red_bytes(int waves, int r) { return (size_t)waves * r * 1024; }
 
-#ifdef MI_DBG_TIMING
-__device__ unsigned long long mi_dbg_buf[8 * 4096];
-#define MI_STAMP(slot)                                                                       \
-  do {                                                                                       \
-    if (threadIdx.x == 0 && blockIdx.x < 4096)                                               \
-      mi_dbg_buf[blockIdx.x * 8 + (slot)] = __builtin_readcyclecounter();                    \
-  } while (0)
-#else
-#define MI_STAMP(slot)
-#endif
 
 template <int BITS, int DT, int GPT, int WAVES, int TPW, int R, bool XLDS>
 __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
-  MI_STAMP(0);
-#ifdef MI_DBG_TIMING
-  {
-    int m_ = a.M;  // the first value read from the kernel-argument block
-    asm volatile("" ::"s"(m_));
-    MI_STAMP(7);
-  }
-#endif
   // Every scalar the prologue needs leaves the kernel-argument block in ONE batch of scalar loads (the empty asm pins
   // them all here): read one by one where they are used, each costs its own round trip to the scalar cache, and a
   // dozen of those in a row would stand in front of the first weight request.
@@ -363,9 +345,6 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
     ref[r] = locate_row_block(a, rb0 + r, h.row_blocks, h.b1, h.b2, h.b3);
     const SkinnySeg &sg = ref[r].sg;
     int rb = ref[r].rb;
-#ifdef MI_DBG_SAMETILE
-    rb = rb & 3;
-#endif
     wq[r] = (const uint8_t *)sg.qw + (int64_t)rb * h.k_tiles * 1024;
     if constexpr (BITS == 4) {
       szp[r] = (const uint8_t *)sg.sz_t + (int64_t)rb * h.G * 64;
@@ -401,9 +380,6 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
   // byte offsets inside a row block fit 32 bits (k_tiles * 1 KiB): scalar tile offset + per-lane offset, one vector
   // add per request, against the row block's 64-bit base in scalar registers
   auto load_tile = [&](Tile &t, int kt) {
-#ifdef MI_DBG_SAMETILE
-    kt = kt & 1;
-#endif
     const uint32_t woff = (uint32_t)kt * 1024u + lane16;
 #pragma unroll
     for (int r = 0; r < R; ++r)
@@ -440,10 +416,6 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
   asm volatile("" : "+v"(nib_magic));  // keep it in a VGPR (see and_or)
 
   auto compute_tile = [&](const Tile &t, int kt) {
-#ifdef MI_DBG_NOCOMPUTE
-    acc[0][0] += __builtin_bit_cast(float, t.w[0][0] ^ t.w[0][1] ^ t.w[0][2] ^ t.w[0][3] ^ t.sz[0][0]);
-    return;
-#endif
     u32x4 xf[KSTEPS];
 #pragma unroll
     for (int j = 0; j < KSTEPS; ++j) {
@@ -517,7 +489,6 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
         compute_tile(buf[p], wave + (i0 + p) * WAVES);
   };
 
-#ifndef MI_DBG_NOSTAGE
   if constexpr (XLDS) {
     // Stage the activation rows (16-byte chunks, zero past K) and form the per-unit sums S.  The first batch of
     // activation loads is issued BEFORE the weight loads and written to LDS after them: loads return in order, so
@@ -568,7 +539,6 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
       for (int b = 0; b < XBN; ++b)  // unconditional (a slot past the end re-reads chunk 0)
         v[b] = chunk_load(b * NT + tid, row[b], kc[b], ok[b]);
       issue_round(buf_a, 0);  // unconditional (k_tiles >= 1): a branch would hide the load count from the waits
-      MI_STAMP(1);
 #pragma unroll
       for (int b = 0; b < XBN; ++b)
         chunk_store(v[b], row[b], kc[b], ok[b]);
@@ -586,9 +556,7 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
       chunk_store(v1, r1, k1, o1);
     }
     __syncthreads();
-    MI_STAMP(2);
   } else
-#endif
   {
     if (n_tiles > 0)
       issue_round(buf_a, 0);
@@ -601,7 +569,6 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
     issue_round(buf_a, i0);
     consume_round(buf_a, i0);
   }
-  MI_STAMP(3);
   if constexpr (!XLDS) {
     if (h.full_tiles < h.k_tiles && wave == (h.full_tiles % WAVES)) {
       // partial last tile (K not a multiple of the tile): activations past K must read as zero
@@ -635,24 +602,8 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
     }
   }
   reduce_and_store<DT, WAVES, R>(a, red, acc, wave, lane, ref, bias_v, m0);
-  MI_STAMP(4);
-#ifdef MI_DBG_TIMING
-  if (threadIdx.x == 0 && blockIdx.x < 4096) {
-    unsigned hwid;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-    unsigned xcc;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-    mi_dbg_buf[blockIdx.x * 8 + 5] = hwid;
-    mi_dbg_buf[blockIdx.x * 8 + 6] = xcc;
-  }
-#endif
 }
 
-#ifdef MI_DBG_TIMING
-extern "C" int mi_dbg_dump(unsigned long long *host, size_t n) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mi_dbg_buf), n * sizeof(unsigned long long));
-}
-#endif
 
 // ------------------------------------------------------------------------------------------------
 // host-side dispatch
@@ -661,12 +612,14 @@ struct SkinnyPlan {
   int waves, tpw, r;
 };
 
-// development hook: MI_A16_PLAN="waves,tpw,r" overrides the heuristic
 static bool plan_override(SkinnyPlan &p) {
-  const char *e = getenv("MI_A16_PLAN");
-  if (!e)
+  const mi_internal_plan &o = plan();
+  if (!o.a16_waves)
     return false;
-  return sscanf(e, "%d,%d,%d", &p.waves, &p.tpw, &p.r) == 3;
+  p.waves = o.a16_waves;
+  p.tpw = o.a16_tpw;
+  p.r = o.a16_rows;
+  return true;
 }
 
 static size_t skinny_x_bytes(int rows, int64_t k_tiles, int tile_k) {
@@ -711,11 +664,8 @@ static SkinnyPlan pick_plan(int64_t row_blocks, int64_t m_blocks, int64_t k_tile
 template <int BITS, int DT, int GPT, int W, int T, int R_, bool XLDS>
 static void launch_instance(const SkinnyArgs &a, int64_t m_blocks, size_t lds_bytes, hipStream_t st) {
   auto kfn = a16_skinny_kernel<BITS, DT, GPT, W, T, R_, XLDS>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    (void)hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    attr_set = true;
-  }
+  static LdsLimitOnce lds_limit;
+  lds_limit.ensure((const void *)kfn, 160 * 1024);
   dim3 grid((unsigned)((a.row_blocks + R_ - 1) / R_), (unsigned)m_blocks);
   kfn<<<grid, dim3(W * 64), lds_bytes, st>>>(a);
 }
@@ -745,15 +695,6 @@ static bool launch_skinny(const SkinnyArgs &a, const SkinnyPlan &plan, int64_t m
     MI_SKINNY_CASE(16, 6, 1)
     MI_SKINNY_CASE(16, 8, 1)
   }
-#ifdef MI_TUNE
-  MI_SKINNY_CASE(4, 4, 1)
-  MI_SKINNY_CASE(4, 8, 1)
-  MI_SKINNY_CASE(8, 2, 2)
-  MI_SKINNY_CASE(16, 2, 2)
-  MI_SKINNY_CASE(8, 4, 2)
-  MI_SKINNY_CASE(16, 4, 2)
-  MI_SKINNY_CASE(16, 3, 2)
-#endif
   return false;
 }
 
@@ -784,7 +725,7 @@ int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t 
 }
 
 int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
-                     float *const *d_y32s, hipStream_t stream) {
+                     float *const *d_y32s, hipStream_t stream, const A16Scratch *fixed) {
   MI_REQUIRE(ws && n >= 1 && n <= MAX_SEG, MI_BAD_ARGUMENT,
              "mi_a16mm_launch_group: between 1 and " + std::to_string(MAX_SEG) + " weight sets per launch");
   MI_REQUIRE(M >= 0 && M <= 65535 * 16, MI_BAD_ARGUMENT, "mi_a16mm_launch: M out of range");
@@ -820,7 +761,8 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
   if (a16_gemm_applicable(w, M)) {  // many rows: the tiled MFMA GEMM, up to three sibling sets per launch
     for (int i = 0; i < n; i += 3) {
       const int cnt = (n - i) < 3 ? (n - i) : 3;
-      const int rc = a16_gemm_launch_group(ws + i, cnt, d_x, M, d_ys + i, d_y32s ? d_y32s + i : nullptr, stream);
+      // (with a fixed scratch area, consecutive launches of one call reuse it: they are ordered on the stream)
+      const int rc = a16_gemm_launch_group(ws + i, cnt, d_x, M, d_ys + i, d_y32s ? d_y32s + i : nullptr, stream, fixed);
       if (rc != MI_SUCCESS)
         return rc;
     }
@@ -842,8 +784,8 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
   const size_t x_bytes = skinny_x_bytes((int)(M < 16 ? M : 16), w->k_tiles, tile_k);
   // Activation rows staged in LDS pay off for up to three rows; from four on the staging costs more occupancy than
   // the reuse returns and the fragments come straight from L2 (measured, 11008 x 4096 at M = 8: 14.7 -> 11.1 us)
-  const char *xe = getenv("MI_A16_XLDS");  // development switch: "0" / "1"
-  const bool xlds = x_bytes <= XLDS_MAX_BYTES && (xe ? atoi(xe) != 0 : M <= 3) && !getenv("MI_A16_NO_XLDS");
+  const int xo = plan().a16_xlds;
+  const bool xlds = x_bytes <= XLDS_MAX_BYTES && (xo ? xo == 1 : M <= 3);
   const SkinnyPlan plan = pick_plan(total_rb, m_blocks, w->k_tiles, xlds);
   const bool f16 = w->dtype == MI_DT_F16;
   bool ok;

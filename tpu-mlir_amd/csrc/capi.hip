@@ -13,6 +13,9 @@
 namespace mi {
 
 static thread_local std::string g_last_error;
+static mi_internal_plan g_plan = {};
+
+const mi_internal_plan &plan() { return g_plan; }
 
 void set_error(const std::string &msg) { g_last_error = msg; }
 
@@ -110,8 +113,10 @@ struct A16Handle {
       a16_free(w);
       delete w;
     }
-    if (stream)
+    if (stream) {
+      release_stream_workspaces(stream);
       (void)hipStreamDestroy(stream);
+    }
   }
 };
 
@@ -130,6 +135,8 @@ static bool group_size_supported(int bits, int g, int64_t K) {
 using namespace mi;
 
 extern "C" {
+
+void mi_internal_set_plan(const mi_internal_plan *p) { g_plan = p ? *p : mi_internal_plan{}; }
 
 const char *mi_version(void) { return "tpumlir_amd 0.1 (gfx950)"; }
 const char *mi_last_error(void) { return g_last_error.c_str(); }
@@ -545,8 +552,10 @@ struct I8Handle {
   bool has_bias = false, has_multi = false;
   hipStream_t stream = nullptr;
   ~I8Handle() {
-    if (stream)
+    if (stream) {
+      release_stream_workspaces(stream);
       (void)hipStreamDestroy(stream);
+    }
   }
 };
 
@@ -566,14 +575,17 @@ static int out_elem_size(int dt) {
 // float-expanded 8-bit integers -> bytes; reports whether they are int8 or uint8 valued
 static int floats_to_bytes(const float *src, int64_t n, uint8_t *dst, int *is_unsigned, const char *who) {
   float lo = 0.f, hi = 0.f;
+  bool whole = true;  // integer valued and inside [-128, 255] (false for NaN and infinities as well)
   for (int64_t i = 0; i < n; ++i) {
-    float v = src[i];
+    const float v = src[i];
+    whole &= (v >= -128.f) & (v <= 255.f) & (v == truncf(v));
     lo = v < lo ? v : lo;
     hi = v > hi ? v : hi;
-    dst[i] = (uint8_t)(int)v;
   }
-  MI_REQUIRE(lo >= -128.f && hi <= 255.f && !(lo < 0.f && hi > 127.f), MI_UNSUPPORTED,
-             std::string(who) + ": operand does not fit an 8-bit integer type");
+  MI_REQUIRE(whole && !(lo < 0.f && hi > 127.f), MI_UNSUPPORTED,
+             std::string(who) + ": operand does not hold the values of one 8-bit integer type");
+  for (int64_t i = 0; i < n; ++i)
+    dst[i] = (uint8_t)(int)src[i];
   *is_unsigned = hi > 127.f;
   return MI_SUCCESS;
 }
@@ -653,11 +665,11 @@ int mi_i8mm_init(const mi_i8mm_attr *attr, mi_infer_param *p) {
   }
   if (rc == MI_SUCCESS && bias) {
     rc = floats_to_i32_dev(bias, attr->N, h->d_bias, h->stream);
-    h->has_bias = rc == MI_SUCCESS;
+    h->has_bias = rc == MI_SUCCESS && attr->right_is_weight;  // constant only beside a weight; else re-read per call
   }
   if (rc == MI_SUCCESS && multi && attr->fuse_rq) {
     rc = floats_to_i32_dev(multi, attr->N, h->d_multi, h->stream);
-    h->has_multi = rc == MI_SUCCESS;
+    h->has_multi = rc == MI_SUCCESS && attr->right_is_weight;
   }
   if (rc == MI_SUCCESS) {
     e = hipStreamSynchronize(h->stream);

@@ -494,7 +494,7 @@ int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_
   const size_t sl_bytes = (size_t)m_blocks * 16 * G * 4, sr_bytes = (size_t)n_blocks * 16 * G * 4;
   const size_t tr_bytes = right_transpose ? 0 : (((size_t)N * K * 2 + 255) & ~(size_t)255);
   uint8_t *ws = nullptr;
-  int rc = stream_workspace(stream, WS_DYNAMIC_QUANT, tr_bytes + al_bytes + ar_bytes + 2 * (sl_bytes + sr_bytes), false,
+  int rc = stream_workspace(stream, WS_DYNAMIC_QUANT, tr_bytes + al_bytes + ar_bytes + 2 * (sl_bytes + sr_bytes),
                             (void **)&ws);
   if (rc != MI_SUCCESS)
     return rc;
@@ -533,12 +533,8 @@ int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_
         d_left, M, K, (int)g, G, imax, k_tiles, aq_l, as_l, sum_l, m_blocks * 16);                              \
     dq_act_kernel<DT_, 8, FLAV_><<<dim3((unsigned)((wr + 3) / 4)), dim3(256), 0, stream>>>(                     \
         right_nk, N, K, (int)g, G, imax, k_tiles, aq_r, as_r, sum_r, n_blocks * 16);                            \
-    static bool attr_set = false;                                                                               \
-    if (!attr_set) {                                                                                            \
-      (void)hipFuncSetAttribute((const void *)dq2_gemm_kernel<DT_, FLAV_>,                                      \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                        \
-      attr_set = true;                                                                                          \
-    }                                                                                                           \
+    static LdsLimitOnce lds_limit;                                                                              \
+    lds_limit.ensure((const void *)dq2_gemm_kernel<DT_, FLAV_>, 160 * 1024);                                    \
     dq2_gemm_kernel<DT_, FLAV_><<<grid, dim3(DQ_WAVES * 64), lds_bytes, stream>>>(a);                           \
   }
   if (dq_type == MI_DQ_F8E4M3) {
@@ -598,7 +594,7 @@ int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int6
   // codes, scales and code sums of this call: the stream's scratch buffer
   const size_t aq_bytes = ((size_t)rows_padded * w->K + 255) & ~(size_t)255, qp_bytes = (size_t)rows_padded * G * 4;
   uint8_t *aq = nullptr;
-  int rc = stream_workspace(stream, WS_DYNAMIC_QUANT, aq_bytes + 2 * qp_bytes, false, (void **)&aq);
+  int rc = stream_workspace(stream, WS_DYNAMIC_QUANT, aq_bytes + 2 * qp_bytes, (void **)&aq);
   if (rc != MI_SUCCESS)
     return rc;
   float *as_t = (float *)(aq + aq_bytes);
@@ -626,18 +622,14 @@ int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int6
   const int chunk_groups = G < DQ_CHUNK ? G : DQ_CHUNK;
   const size_t lds_bytes = (size_t)(chunk_groups + 1) * 1024;
   dim3 grid((unsigned)w->row_blocks, (unsigned)m_blocks);
-  const char *we = getenv("MI_DQ_WAVES");  // development switch: 8 / 16
-  const int gemm_waves = we ? atoi(we) : ((int64_t)w->row_blocks * m_blocks <= 256 ? 2 * DQ_WAVES : DQ_WAVES);
+  const int wo = plan().dq_waves;
+  const int gemm_waves = (wo == DQ_WAVES || wo == 2 * DQ_WAVES) ? wo : ((int64_t)w->row_blocks * m_blocks <= 256 ? 2 * DQ_WAVES : DQ_WAVES);
 #define MI_DQ_RUN(DT_, BITS_, FLAV_)                                                                             \
   {                                                                                                             \
     dq_act_kernel<DT_, BITS_, FLAV_><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(              \
         d_x, M, w->K, g, G, imax, w->k_tiles, aq, as_t, asum_t, rows_padded);                                   \
-    static bool attr_set = false;                                                                               \
-    if (!attr_set) {                                                                                            \
-      (void)hipFuncSetAttribute((const void *)dq_gemm_kernel<DT_, BITS_, FLAV_>,                                \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                        \
-      attr_set = true;                                                                                          \
-    }                                                                                                           \
+    static LdsLimitOnce lds_limit;                                                                              \
+    lds_limit.ensure((const void *)dq_gemm_kernel<DT_, BITS_, FLAV_>, 160 * 1024);                              \
     dq_gemm_kernel<DT_, BITS_, FLAV_><<<grid, dim3(gemm_waves * 64), lds_bytes, stream>>>(a);                   \
   }
   if (dq_type == MI_DQ_F8E4M3) {

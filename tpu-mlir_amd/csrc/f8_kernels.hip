@@ -639,7 +639,7 @@ int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, con
   const uint8_t *b_nk = d_b;
   if (!right_transpose) {  // [K, N] -> [N, K] into the stream's scratch buffer
     uint8_t *t = nullptr;
-    int rc = stream_workspace(stream, WS_F8_TRANSPOSE, (size_t)N * K, false, (void **)&t);
+    int rc = stream_workspace(stream, WS_F8_TRANSPOSE, (size_t)N * K, (void **)&t);
     if (rc != MI_SUCCESS)
       return rc;
     f8_transpose_kernel<<<dim3((unsigned)((N + 31) / 32), (unsigned)((K + 31) / 32)), dim3(256), 0, stream>>>(d_b, t, K, N);
@@ -664,22 +664,15 @@ int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, con
   const int64_t tiles_m = (M + F8_BM - 1) / F8_BM, tiles_n = (N + F8_BN - 1) / F8_BN;
   if ((K % F8_BK) == 0 && tiles_m * tiles_n < (int64_t(1) << 30)) {
     const int tiles = (int)(tiles_m * tiles_n), per_xcd = (tiles + 7) / 8;
-    static bool attr_set = false;
-    if (!attr_set) {
-      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<8, F8_FMT_E4M3>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, f8_ring_lds_bytes(8));
-      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<4, F8_FMT_E4M3>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, f8_ring_lds_bytes(4));
-      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<8, F8_FMT_E5M2>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, f8_ring_lds_bytes(8));
-      (void)hipFuncSetAttribute((const void *)f8_gemm_ring_kernel<4, F8_FMT_E5M2>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, f8_ring_lds_bytes(4));
-      attr_set = true;
-    }
+    static LdsLimitOnce lim8a, lim4a, lim8b, lim4b;
+    lim8a.ensure((const void *)f8_gemm_ring_kernel<8, F8_FMT_E4M3>, f8_ring_lds_bytes(8));
+    lim4a.ensure((const void *)f8_gemm_ring_kernel<4, F8_FMT_E4M3>, f8_ring_lds_bytes(4));
+    lim8b.ensure((const void *)f8_gemm_ring_kernel<8, F8_FMT_E5M2>, f8_ring_lds_bytes(8));
+    lim4b.ensure((const void *)f8_gemm_ring_kernel<4, F8_FMT_E5M2>, f8_ring_lds_bytes(4));
     const int64_t tl_m = (M + F8L_M - 1) / F8L_M, tl_n = (N + F8L_N - 1) / F8L_N;
-    const char *e = getenv("MI_F8_TILE");  // development switch: "256" / "128" / "64"
-    const bool large = e ? atoi(e) == 256 : tl_m * tl_n >= 144;  // the INT8 kernels' measured crossover
-    const bool small = e ? atoi(e) == 64 : tiles <= 128;         // likewise
+    const int e = plan().f8_tile;
+    const bool large = e ? e == 256 : tl_m * tl_n >= 144;  // the INT8 kernels' measured crossover
+    const bool small = e ? e == 64 : tiles <= 128;         // likewise
     if (small && !large) {
       const int64_t ts_m = (M + 63) / 64, ts_n = (N + 63) / 64;
       const int ts = (int)(ts_m * ts_n), ps = (ts + 7) / 8;
@@ -691,14 +684,9 @@ int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, con
         f8_gemm_ring_kernel<4, F8_FMT_E4M3, 64><<<grid, dim3(256), f8_ring_lds_bytes(4, 64), stream>>>(a, (int)ts_m,
                                                                                                       (int)ts_n, ps);
     } else if (large) {
-      static bool attr_large = false;
-      if (!attr_large) {
-        (void)hipFuncSetAttribute((const void *)f8_gemm_large_kernel<F8_FMT_E4M3>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, F8L_NST * F8L_STAGE);
-        (void)hipFuncSetAttribute((const void *)f8_gemm_large_kernel<F8_FMT_E5M2>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, F8L_NST * F8L_STAGE);
-        attr_large = true;
-      }
+      static LdsLimitOnce lim_a, lim_b;
+      lim_a.ensure((const void *)f8_gemm_large_kernel<F8_FMT_E4M3>, F8L_NST * F8L_STAGE);
+      lim_b.ensure((const void *)f8_gemm_large_kernel<F8_FMT_E5M2>, F8L_NST * F8L_STAGE);
       const int tl = (int)(tl_m * tl_n), pl = (tl + 7) / 8;
       const dim3 grid((unsigned)(pl * 8));
       if (e5m2)

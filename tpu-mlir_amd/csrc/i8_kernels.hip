@@ -263,15 +263,6 @@ typedef __attribute__((address_space(3))) void *lptr_t;
 constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
 constexpr int WAITCNT_LGKM0 = 0xC07F;
 
-#ifndef MI_I8_DBG
-#define MI_I8_DBG 0  // development switches (results become wrong): 1 no global loads, 2 no fragment reads, 4 no MFMA,
-                     // 8 no barrier, 16 no wait for the loads
-#endif
-#if defined(MI_I8_TIMING) && MI_I8_TIMING >= 2
-#define MI_I8_STAMP(v) const unsigned long long v = __builtin_readcyclecounter()
-#else
-#define MI_I8_STAMP(v)
-#endif
 
 __device__ __forceinline__ int32_t med3_i32(int32_t x, int32_t lo, int32_t hi) {
   int32_t r;
@@ -288,12 +279,15 @@ __device__ __forceinline__ uint32_t sat_pack_u8(int32_t q0, int32_t q1, int32_t 
   return (b01 & 0xffffu) | (b23 << 16);
 }
 
-#ifdef MI_I8_TIMING
-__device__ unsigned long long mi_i8_dbg[64 * 4 * 4 + 64 * 8];
-extern "C" int mi_i8_dbg_dump(unsigned long long *host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mi_i8_dbg), sizeof(mi_i8_dbg));
+// round-half-away-from-zero of t / 2^s for s in [1, 31], exact for every int32 t.  The sum t + 2^(s-1) - (t < 0) needs
+// 33 bits when t is close to INT32_MAX: it is formed modulo 2^32, its high word (0 for t >= 0, the sign of the sum for
+// t < 0, where the sum fits 32 bits) is rebuilt from the signs, and the 64-bit right shift takes both.
+__device__ __forceinline__ int32_t rshift_half_away_32(int32_t t, int32_t half, int32_t s) {
+  const uint32_t u = (uint32_t)t + (uint32_t)half + (uint32_t)(t >> 31);
+  const uint32_t hi = (uint32_t)((int32_t)((uint32_t)t & u) >> 31);
+  return (int32_t)__builtin_amdgcn_alignbit(hi, u, (uint32_t)s);
 }
-#endif
+
 
 // ------------------------------------------------------------------------------------------------
 // Mid-size kernel: 128x128 outputs per workgroup (4 waves, each 64x64 as 2x2 MFMA 32x32x32 blocks), K advancing 64
@@ -330,9 +324,6 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-#ifdef MI_I8_TIMING
-  const unsigned long long t_entry = __builtin_amdgcn_s_memrealtime();
-#endif
   const int bid = blockIdx.x;
   const int L = (bid & 7) * per_xcd + (bid >> 3);  // each XCD gets a contiguous run of the tile order
   if (L >= tiles_m * tiles_n)
@@ -427,9 +418,6 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
 #pragma unroll
   for (int s0 = 0; s0 < MID_NST - 1; ++s0)
     issue(s0);
-#ifdef MI_I8_TIMING
-  const unsigned long long t_loop = __builtin_amdgcn_s_memrealtime();
-#endif
   for (int kt = 0; kt < kt_total; ++kt) {
     // requests complete in order: at most (NST - 2) stages' worth outstanding means stage kt has landed
     __builtin_amdgcn_s_waitcnt(waitcnt_vm((MID_NST - 2) * LPS));
@@ -452,9 +440,6 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
     }
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // drain the re-loads issued past the end
-#ifdef MI_I8_TIMING
-  const unsigned long long t_epi = __builtin_amdgcn_s_memrealtime();
-#endif
 
   // epilogue.  The accumulators (register r of lane l = row 8*(r/4) + 4*(l/32) + (r%4), column l%32 of a 32x32
   // block) pass through a per-wave 64 x 64 strip in LDS so that a lane owns 16 consecutive columns of a row: per-column
@@ -526,7 +511,7 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
           const int e = q4 * 4 + u;
           const int64_t p = (int64_t)v[e] * (int64_t)p_mult[e] + (1ll << 30);
           const int32_t t = (int32_t)(p >> 31);
-          q[u] = ((t + p_half[e] + (t >> 31)) >> p_shift[e]) + p_zp[e];
+          q[u] = rshift_half_away_32(t, p_half[e], p_shift[e]) + p_zp[e];
         }
         packed[q4] = sat_pack_u8(q[0], q[1], q[2], q[3]) ^ 0x80808080u;
       }
@@ -558,15 +543,6 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
       }
     }
   }
-#ifdef MI_I8_TIMING
-  if (lane == 0 && wave == 0 && blockIdx.x < 64) {
-    unsigned long long *d = mi_i8_dbg + 1024 + blockIdx.x * 8;
-    d[0] = t_entry;
-    d[1] = t_loop - t_entry;
-    d[2] = t_epi - t_loop;
-    d[3] = __builtin_amdgcn_s_memrealtime() - t_entry;
-  }
-#endif
 }
 
 // LK_ = bytes of K per stage (64 or 128), NST = stages in the LDS ring (NST * 512 * LK_ bytes)
@@ -581,9 +557,6 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-#ifdef MI_I8_TIMING
-  const unsigned long long r_entry = __builtin_amdgcn_s_memrealtime();
-#endif
 
   // workgroup -> tile: hardware deals workgroups round-robin over the 8 XCDs; give each XCD a contiguous range of
   // the tile order, and order tiles in groups of 4 tile-rows (column-major inside a group)
@@ -626,13 +599,8 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
     uint8_t *sa = lds + (kt % NST) * STAGE_BYTES, *sb = sa + LM * LK_;
 #pragma unroll
     for (int i = part * PART; i < (part + 1) * PART; ++i) {
-#if defined(MI_I8_DBG) && (MI_I8_DBG & 64)  // every load re-reads the same 2 KiB: vector-cache hits
-      __builtin_amdgcn_global_load_lds((gptr_t)(ga[0]), (lptr_t)(sa + (i * 4 + wave) * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_t)(gb[0]), (lptr_t)(sb + (i * 4 + wave) * 1024), 16, 0, 0);
-#else
       __builtin_amdgcn_global_load_lds((gptr_t)(ga[i] + koff), (lptr_t)(sa + (i * 4 + wave) * 1024), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((gptr_t)(gb[i] + koff), (lptr_t)(sb + (i * 4 + wave) * 1024), 16, 0, 0);
-#endif
     }
   };
 
@@ -693,18 +661,13 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
       const int i = t >> 2, j = t & 3;
-#if !(MI_I8_DBG & 4)
       acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ca[i], cb[j], acc[i][j], 0, 0, 0);
-#endif
-#if !(MI_I8_DBG & 2)
       if (t == 0)
         na[0] = *(const i32x4 *)(st + a_off[0] + ((c ^ a_sw[0]) << 4));
       else if (t <= 4)
         nb[t - 1] = *(const i32x4 *)(st + b_off[t - 1] + ((c ^ b_sw[t - 1]) << 4));
       else if (t <= 7)
         na[t - 4] = *(const i32x4 *)(st + a_off[t - 4] + ((c ^ a_sw[t - 4]) << 4));
-#endif
-#if !(MI_I8_DBG & 1)
       if (t >= 8) {
         constexpr int SLOTS = 8, N_LD = 2 * PART;  // loads of this part, spread over the last 8 MFMAs
         const int q0 = (t - 8) * N_LD / SLOTS, q1 = (t - 7) * N_LD / SLOTS;
@@ -719,7 +682,6 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
                                              0);
         }
       }
-#endif
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -740,11 +702,6 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
       issue_part(s, part);
   issue_part(NST - 1, 0);
   i32x4 fa[2][4], fb[2][4];
-#ifdef MI_I8_TIMING
-  unsigned long long t_lgkm = 0, t_vm = 0, t_bar = 0, t_lgkm2 = 0;
-  const unsigned long long t_begin = __builtin_readcyclecounter();
-  const unsigned long long r_begin = __builtin_amdgcn_s_memrealtime();
-#endif
   __builtin_amdgcn_s_waitcnt(waitcnt_vm((NST - 2) * LPS + 2 * PART));  // stage 0 landed
   __builtin_amdgcn_s_barrier();
   read_frags(fa[0], fb[0], 0, 0);
@@ -754,43 +711,14 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
       if (ks + 1 < KS) {
         batch(fa[ks & 1], fb[ks & 1], fa[(ks + 1) & 1], fb[(ks + 1) & 1], kt, ks + 1, kt + NST - 1, ks + 1);
       } else {
-        MI_I8_STAMP(tw0);
         __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);
-        MI_I8_STAMP(tw1);
-#if !(MI_I8_DBG & 1) && !(MI_I8_DBG & 16)
         __builtin_amdgcn_s_waitcnt(waitcnt_vm((NST - 2) * LPS));  // this thread's share of stage kt+1 landed
-#endif
-        MI_I8_STAMP(tw2);
-#if !(MI_I8_DBG & 8)
         __builtin_amdgcn_s_barrier();
-#endif
-        MI_I8_STAMP(tw3);
-#if defined(MI_I8_TIMING) && MI_I8_TIMING >= 2
-        t_lgkm += tw1 - tw0;
-        t_vm += tw2 - tw1;
-        t_bar += tw3 - tw2;
-#endif
         batch(fa[ks & 1], fb[ks & 1], fa[(ks + 1) & 1], fb[(ks + 1) & 1], kt + 1, 0, kt + NST, 0);
       }
     }
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // drain the re-loads issued past the end before the workgroup may exit
-#ifdef MI_I8_TIMING
-  if (lane == 0 && blockIdx.x < 64) {
-    const unsigned long long t_end = __builtin_readcyclecounter();
-    unsigned long long *d = mi_i8_dbg + (blockIdx.x * 4 + wave) * 4;
-    d[0] = t_end - t_begin;
-    if (wave == 0) {  // 10 ns units
-      mi_i8_dbg[1024 + blockIdx.x * 8 + 0] = r_entry;
-      mi_i8_dbg[1024 + blockIdx.x * 8 + 4] = t_lgkm2;
-      mi_i8_dbg[1024 + blockIdx.x * 8 + 1] = r_begin - r_entry;                        // prologue
-      mi_i8_dbg[1024 + blockIdx.x * 8 + 2] = __builtin_amdgcn_s_memrealtime() - r_begin;  // main loop
-    }
-    d[1] = t_lgkm;
-    d[2] = t_vm;
-    d[3] = t_bar;
-  }
-#endif
 
   // Epilogue.  Register r of lane l in block (i, j) is row 8*(r/4) + 4*(l/32) + (r%4), column l%32 -- a layout
   // that would store 32-byte row fragments.  Each wave instead passes one 32 x 128 strip at a time through its own
@@ -874,8 +802,8 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
         }
       } else if constexpr (EPI == EPI_Q31_HALF_AWAY) {
         // MultiplyByQuantizedMultiplier(x, mult, -shift, HALF_AWAY) with shift in [1, 31], in 32-bit steps:
-        // t = (x*mult + 2^30) >> 31 fits int32 for |x|, mult < 2^31, so the reference's clamp never fires, and
-        // half-away rounding of t >> shift is (t + half + (t >> 31)) >> shift.  The int8 saturation is done as
+        // t = (x*mult + 2^30) >> 31 fits int32 unless x = mult = INT32_MIN (excluded by the host), so the reference's
+        // clamp never fires; then the half-away rounding of t >> shift.  The int8 saturation is done as
         // an unsigned one on q + 128 (two saturating pack instructions per four values), undone by flipping the
         // sign bits of the packed bytes.
         uint32_t packed[4];
@@ -887,7 +815,7 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
             const int e = q4 * 4 + u;
             const int64_t p = (int64_t)v[e] * (int64_t)p_mult[e] + (1ll << 30);
             const int32_t t = (int32_t)(p >> 31);
-            q[u] = ((t + p_half[e] + (t >> 31)) >> p_shift[e]) + p_zp[e];
+            q[u] = rshift_half_away_32(t, p_half[e], p_shift[e]) + p_zp[e];
           }
           packed[q4] = sat_pack_u8(q[0], q[1], q[2], q[3]) ^ 0x80808080u;
         }
@@ -909,10 +837,6 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
       }
     }
   }
-#ifdef MI_I8_TIMING
-  if (lane == 0 && blockIdx.x < 64 && wave == 0)
-    mi_i8_dbg[1024 + blockIdx.x * 8 + 3] = __builtin_amdgcn_s_memrealtime() - r_entry;  // whole kernel
-#endif
 }
 
 static RequantParams make_rq(const mi_requant_desc *rq) {
@@ -1010,10 +934,12 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
   if (rq) {
     const bool q31 = rq->quant_mode == MI_RQ_QDM || rq->quant_mode == MI_RQ_TFLITE ||
                      rq->quant_mode == MI_RQ_TFLITE_LSHIFT;
-    // the 32-bit fast path needs a right shift in [1, 31] on every channel; per-channel shifts are the
-    // caller's device array, so it is only taken for a scalar shift or when the caller vouches via the desc
-    epi = (q31 && rq->round_mode == MI_ROUND_HALF_AWAY_FROM_ZERO && rq->out_dtype == MI_DT_I8 &&
-           (rq->d_shift || (rq->shift >= 1 && rq->shift <= 31)))
+    // the 32-bit epilogue needs a right shift in [1, 31] and a multiplier other than INT32_MIN on every channel.
+    // Scalars are checked here; per-channel values live in the caller's device arrays, which the host cannot read
+    // without a synchronization, so such arrays take it only when the caller vouches for them in the descriptor.
+    const bool shift_ok = rq->d_shift ? rq->per_channel_q31_checked != 0 : (rq->shift >= 1 && rq->shift <= 31);
+    const bool mult_ok = rq->d_multiplier ? rq->per_channel_q31_checked != 0 : rq->multiplier != INT32_MIN;
+    epi = (q31 && rq->round_mode == MI_ROUND_HALF_AWAY_FROM_ZERO && rq->out_dtype == MI_DT_I8 && shift_ok && mult_ok)
               ? EPI_Q31_HALF_AWAY
               : EPI_GENERIC;
   }
@@ -1025,11 +951,10 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
   // 256x256 tiles when there are enough of them to occupy the chip, else 128x128 tiles on the same data path; the
   // register-staged kernel takes what is left (K % 64 != 0)
   const int64_t tiles_large = ((M + LM - 1) / LM) * ((N + LN - 1) / LN);
-  const char *tile_env = getenv("MI_I8_TILE");  // development switch: "256" / "128" / "0" (register-staged)
   const bool large_ok = (K % 128) == 0 && M >= 128 && N >= 128, mid_ok = (K % 64) == 0;
-  const int tile_pick = tile_env ? atoi(tile_env) : (large_ok && tiles_large >= 144 ? 256 : 128);  // measured crossover
+  const int tile_pick = plan().i8_tile ? plan().i8_tile : (large_ok && tiles_large >= 144 ? 256 : 128);  // measured crossover
   const bool large = large_ok && tile_pick == 256;
-  const bool mid = !large && mid_ok && tile_pick != 0;
+  const bool mid = !large && mid_ok && tile_pick > 0;
   uint8_t *a_signed = nullptr, *b_signed = nullptr;
   if (large || mid) {
     // direct-to-LDS loads cannot flip sign bits on the way: unsigned operands are rewritten once (after the
@@ -1048,21 +973,14 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
   if (mid) {
     int tiles_m = (int)((M + MID_M - 1) / MID_M), tiles_n = (int)((N + MID_N - 1) / MID_N);
     int per_xcd = (tiles_m * tiles_n + 7) / 8;
-    static bool attr_set = false;
-    if (!attr_set) {
-      (void)hipFuncSetAttribute((const void *)i8_gemm_mid_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024);
-      (void)hipFuncSetAttribute((const void *)i8_gemm_mid_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024);
-      (void)hipFuncSetAttribute((const void *)i8_gemm_mid_kernel<4, 64>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024);
-      attr_set = true;
-    }
+    static LdsLimitOnce lim4, lim8, lim64;
+    lim4.ensure((const void *)i8_gemm_mid_kernel<4>, 160 * 1024);
+    lim8.ensure((const void *)i8_gemm_mid_kernel<8>, 160 * 1024);
+    lim64.ensure((const void *)i8_gemm_mid_kernel<4, 64>, 160 * 1024);
     // up to 128 tiles of 128 x 128 (half the CUs): 64 x 64 tiles with a 4-stage ring, four workgroups per CU hiding
     // each other's waits (measured against the 128-tile forms: 5.8 vs 10.2 us at 256 x 1024 x 1024, 6.2 vs 10.5 at
     // 1024^3, 11.2 vs 15.4 at 1024 x 2048 x 2048; from 160 tiles on the 128-tile forms win)
-    const char *ring_env = getenv("MI_I8_MID_RING");  // development switch: 4 / 8 (128-tiles), 64 (64-tiles)
-    const int ring = ring_env ? atoi(ring_env) : (tiles_m * tiles_n <= 128 ? 64 : tiles_m * tiles_n <= 256 ? 8 : 4);
+    const int ring = plan().i8_mid_ring ? plan().i8_mid_ring : (tiles_m * tiles_n <= 128 ? 64 : tiles_m * tiles_n <= 256 ? 8 : 4);
     if (ring == 64) {
       tiles_m = (int)((M + 63) / 64);
       tiles_n = (int)((N + 63) / 64);
@@ -1078,18 +996,13 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
   } else if (large) {
     const int tiles_m = (int)((M + LM - 1) / LM), tiles_n = (int)((N + LN - 1) / LN);
     const int per_xcd = (tiles_m * tiles_n + 7) / 8;
-    const char *ring_env = getenv("MI_I8_RING");  // development switch: stages in the LDS ring (3, 4 or 5)
-    const int ring = ring_env ? atoi(ring_env) : 4;
+    const int ring = plan().i8_ring ? plan().i8_ring : 4;
     const size_t lds_bytes = (size_t)(ring == 5 ? 5 : ring == 3 ? 3 : 4) * 32 * 1024;
     dim3 grid((unsigned)(per_xcd * 8));
 #define MI_LARGE_I(E, LK_, NST)                                                                             \
   {                                                                                                         \
-    static bool attr_set = false;                                                                           \
-    if (!attr_set) {                                                                                        \
-      (void)hipFuncSetAttribute((const void *)i8_gemm_large_kernel<E, LK_, NST>,                            \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                    \
-      attr_set = true;                                                                                      \
-    }                                                                                                       \
+    static LdsLimitOnce lds_limit;                                                                          \
+    lds_limit.ensure((const void *)i8_gemm_large_kernel<E, LK_, NST>, 160 * 1024);                          \
     i8_gemm_large_kernel<E, LK_, NST><<<grid, dim3(256), lds_bytes, stream>>>(a, tiles_m, tiles_n, per_xcd);\
   }
 #define MI_LARGE(E)         \

@@ -8,7 +8,45 @@
 
 #include "../../include/tpumlir_amd.h"
 
+// Kernel-selection overrides for the test-suite and for tuning runs: one process-wide record that the launch paths
+// consult in place of their heuristics wherever a field is non-zero.  Not part of the C ABI (the public header does
+// not declare it): the tests bind mi_internal_set_plan by name.  Not thread safe; set it while nothing is launching.
+extern "C" {
+typedef struct mi_internal_plan {
+  int a16_waves, a16_tpw, a16_rows;  // skinny kernel instance (waves per workgroup, tiles per wave and round, row blocks)
+  int a16_xlds;                      // 1: stage the activations in LDS, 2: read them from L2
+  int a16_no_gemm;                   // 1: never take the tiled kernel
+  int a16_gemm_min_m;                // > 0: tiled kernel from this many rows on (M > 1)
+  int a16_gemm_splits;               // > 0: number of K splits of the tiled kernel
+  int a16_gemm_tile;                 // 128 / 256: columns per output block
+  int a16_gemm_rows;                 // 16 / 32 / 64 / 128: rows per output block
+  int i8_tile;                       // 256 / 128 / -1 (register-staged kernel)
+  int i8_mid_ring;                   // 4 / 8 (128-tiles), 64 (64-tiles)
+  int i8_ring;                       // 3 / 4 / 5: LDS ring stages of the large kernel
+  int dq_waves;                      // 8 / 16
+  int f8_tile;                       // 256 / 128 / 64
+} mi_internal_plan;
+void mi_internal_set_plan(const mi_internal_plan *p);  // null: back to the heuristics
+}
+
 namespace mi {
+
+const mi_internal_plan &plan();
+
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per kernel and device: the attribute belongs to the device's
+// copy of the function.  One static instance per kernel instantiation.
+struct LdsLimitOnce {
+  uint64_t done = 0;  // bit d: set on device d (devices past 63 set it on every launch)
+  void ensure(const void *fn, int bytes) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const uint64_t bit = dev < 64 ? (uint64_t)1 << dev : 0;
+    if (__atomic_load_n(&done, __ATOMIC_ACQUIRE) & bit)
+      return;
+    (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    __atomic_fetch_or(&done, bit, __ATOMIC_RELEASE);
+  }
+};
 
 void set_error(const std::string &msg);
 int hip_fail(hipError_t e, const char *what, const char *file, int line);
@@ -64,20 +102,25 @@ int a16_pack(mi_a16_weight *w, const void *h_weight, int weight_signed, const ui
 void a16_free(mi_a16_weight *w);
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                hipStream_t stream);
+// a caller-provided scratch area that a launch must make do with (instead of the stream's growable buffer)
+struct A16Scratch {
+  void *ptr;
+  size_t bytes;
+};
 // tiled MFMA GEMM for many activation rows (prefill)
 bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M);
-int a16_gemm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
-                    hipStream_t stream);
 // up to three sibling weight sets (same K, width, group size, type, chip) on one input in one launch
 int a16_gemm_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
-                          float *const *d_y32s, hipStream_t stream);
+                          float *const *d_y32s, hipStream_t stream, const A16Scratch *fixed = nullptr);
 int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
-                     float *const *d_y32s, hipStream_t stream);
+                     float *const *d_y32s, hipStream_t stream, const A16Scratch *fixed = nullptr);
 
-// library-owned scratch, one buffer per (device, stream, purpose) (workspace.hip).  zeroed: cleared when allocated;
-// the user of such a buffer leaves it zero.
+// library-owned scratch, one buffer per (device, stream, purpose) (workspace.hip); contents are whatever the last
+// user left
 enum { WS_SPLIT_K = 0, WS_DYNAMIC_QUANT = 1, WS_F8_TRANSPOSE = 2 };
-int stream_workspace(hipStream_t st, int purpose, size_t bytes, bool zeroed, void **out);
+int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out);
+// frees every buffer of a stream (current and retired); for owners of private streams, right before hipStreamDestroy
+void release_stream_workspaces(hipStream_t st);
 
 // dynamic activation quantization (dq_kernels.hip); dq_type: MI_DQ_INT, MI_DQ_F8E4M3 (8-bit weights), MI_DQ_F4 (4-bit)
 int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,

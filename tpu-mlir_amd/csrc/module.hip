@@ -88,8 +88,10 @@ struct mi_module {
     for (auto &o : ops)
       if (o.w)
         mi_a16_weight_destroy(o.w);
-    if (stream)
+    if (stream) {
+      mi::release_stream_workspaces(stream);  // after the graph that may name them
       (void)hipStreamDestroy(stream);
+    }
   }
 };
 
@@ -254,6 +256,7 @@ int mi_module_add_a16matmul_dq(mi_module *m, const char *input, const char *outp
   if ((rc = find(m, input, &in)) || (rc = find(m, output, &out)))
     return rc;
   MI_REQUIRE(desc, MI_BAD_ARGUMENT, "mi_module_add_a16matmul: null descriptor");
+  MI_REQUIRE(in != out, MI_BAD_ARGUMENT, "mi_module_add_a16matmul: a matmul cannot write the tensor it reads");
   const int st = desc->dtype == MI_DT_F16 ? MI_ST_F16 : MI_ST_BF16;
   const Tensor &ti = m->tensors[in], &to = m->tensors[out];
   MI_REQUIRE(ti.st == st && to.st == st, MI_BAD_ARGUMENT,
@@ -289,6 +292,7 @@ int mi_module_add_matmul_int8(mi_module *m, const char *input, const char *outpu
   if ((rc = find(m, input, &in)) || (rc = find(m, output, &out)))
     return rc;
   MI_REQUIRE(d && d->right, MI_BAD_ARGUMENT, "mi_module_add_matmul_int8: null descriptor or weight");
+  MI_REQUIRE(in != out, MI_BAD_ARGUMENT, "mi_module_add_matmul_int8: a matmul cannot write the tensor it reads");
   const Tensor &ti = m->tensors[in], &to = m->tensors[out];
   MI_REQUIRE(ti.st == MI_ST_I8 || ti.st == MI_ST_U8, MI_BAD_ARGUMENT, "mi_module_add_matmul_int8: input must be 8-bit");
   MI_REQUIRE(d->K > 0 && d->N > 0 && ti.n % d->K == 0, MI_BAD_ARGUMENT, "mi_module_add_matmul_int8: input size is not M * K");
@@ -327,7 +331,15 @@ int mi_module_add_matmul_int8(mi_module *m, const char *input, const char *outpu
     const int want = o.rq.out_dtype == MI_DT_I8 ? MI_ST_I8 : o.rq.out_dtype == MI_DT_U8 ? MI_ST_U8
                    : o.rq.out_dtype == MI_DT_I16 ? MI_ST_I16 : o.rq.out_dtype == MI_DT_U16 ? MI_ST_U16 : MI_ST_I32;
     MI_REQUIRE(to.st == want, MI_BAD_ARGUMENT, "mi_module_add_matmul_int8: output storage differs from the requant type");
-    // per-channel arrays arrive as HOST pointers in this descriptor and move to the device here
+    // per-channel arrays arrive as HOST pointers in this descriptor and move to the device here; being host arrays
+    // they can be range-checked for the 32-bit epilogue on the spot
+    o.rq.per_channel_q31_checked = 1;
+    for (int64_t n = 0; n < d->N; ++n) {
+      if (d->rq.d_shift && (d->rq.d_shift[n] < 1 || d->rq.d_shift[n] > 31))
+        o.rq.per_channel_q31_checked = 0;
+      if (d->rq.d_multiplier && d->rq.d_multiplier[n] == INT32_MIN)
+        o.rq.per_channel_q31_checked = 0;
+    }
     if (d->rq.d_multiplier) {
       if ((rc = upload(o.mult, d->rq.d_multiplier, (size_t)d->N * 4)))
         return rc;
@@ -406,6 +418,7 @@ int mi_module_add_matmul_dq(mi_module *m, const char *left, const char *right, c
   if ((rc = find(m, left, &in)) || (rc = find(m, right, &in2)) || (rc = find(m, output, &out)))
     return rc;
   const Tensor &tl = m->tensors[in], &tr = m->tensors[in2], &to = m->tensors[out];
+  MI_REQUIRE(out != in && out != in2, MI_BAD_ARGUMENT, "mi_module_add_matmul_dq: a matmul cannot write a tensor it reads");
   MI_REQUIRE((tl.st == MI_ST_BF16 || tl.st == MI_ST_F16) && tr.st == tl.st && to.st == tl.st, MI_BAD_ARGUMENT,
              "mi_module_add_matmul_dq: the three tensors must share one 16-bit float type");
   MI_REQUIRE(K > 0 && N > 0 && tl.n % K == 0 && tr.n == K * N && to.n == tl.n / K * N, MI_BAD_ARGUMENT,

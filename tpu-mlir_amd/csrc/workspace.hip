@@ -1,12 +1,16 @@
 // Device scratch buffers owned by the library, one per (device, stream, purpose).  Work on one stream is ordered, so
-// consecutive calls can share a buffer; calls on different streams never do.  A buffer only grows; growing it
-// synchronizes the stream, frees the old buffer and allocates a new one, which cannot happen while the stream is
-// being captured into a graph: run a shape once eagerly before capturing it.  A graph captured on a stream holds the
-// address of that stream's buffer: a later, larger call on the same stream replaces the buffer and with it invalidates
-// such a graph (capture the largest shape last, or keep graphs and larger eager calls on different streams).
+// consecutive calls can share a buffer; calls on different streams never do.
+//
+// A buffer only grows, and growing never frees: a HIP graph captured on the stream holds the old buffer's address, and
+// replaying that graph must keep working.  The old buffer is therefore retired, not freed; retired buffers stay
+// allocated (and valid for such graphs) until release_stream_workspaces() is called for the stream -- by the owner of
+// a private stream (an operator handle, a module) right before it destroys the stream, after destroying its graphs.
+// Buffers of caller-owned streams live until the process ends.  Growing allocates, which cannot happen while the
+// stream is being captured into a graph: run a shape once eagerly before capturing it.
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <vector>
 
 #include "internal.h"
 
@@ -16,12 +20,13 @@ namespace {
 struct Buf {
   void *ptr = nullptr;
   size_t bytes = 0;
+  std::vector<void *> retired;  // smaller predecessors that a captured graph may still name
 };
 std::mutex g_mutex;
 std::map<std::tuple<int, hipStream_t, int>, Buf> g_bufs;
 }  // namespace
 
-int stream_workspace(hipStream_t st, int purpose, size_t bytes, bool zeroed, void **out) {
+int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out) {
   int dev = 0;
   MI_HIP(hipGetDevice(&dev));
   std::lock_guard<std::mutex> lock(g_mutex);
@@ -32,20 +37,35 @@ int stream_workspace(hipStream_t st, int purpose, size_t bytes, bool zeroed, voi
     MI_REQUIRE(cs == hipStreamCaptureStatusNone, MI_HIP_ERROR,
                "a scratch buffer has to grow while its stream is being captured: run the same shape once eagerly "
                "before capturing it");
-    if (b.ptr) {
-      MI_HIP(hipStreamSynchronize(st));
-      MI_HIP(hipFree(b.ptr));
-      b.ptr = nullptr;
-      b.bytes = 0;
-    }
     const size_t want = (bytes + 255) & ~(size_t)255;
-    MI_HIP(hipMalloc(&b.ptr, want));
-    if (zeroed)  // on the user's stream (which is not being captured here): ordered before whatever it runs next
-      MI_HIP(hipMemsetAsync(b.ptr, 0, want, st));
+    void *fresh = nullptr;
+    MI_HIP(hipMalloc(&fresh, want));
+    if (b.ptr)
+      b.retired.push_back(b.ptr);
+    b.ptr = fresh;
     b.bytes = want;
   }
   *out = b.ptr;
   return MI_SUCCESS;
+}
+
+void release_stream_workspaces(hipStream_t st) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess)
+    return;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  for (auto it = g_bufs.begin(); it != g_bufs.end();) {
+    if (std::get<0>(it->first) == dev && std::get<1>(it->first) == st) {
+      (void)hipStreamSynchronize(st);
+      for (void *p : it->second.retired)
+        (void)hipFree(p);
+      if (it->second.ptr)
+        (void)hipFree(it->second.ptr);
+      it = g_bufs.erase(it);
+    } else {
+      ++it;
+    }
+  }
 }
 
 }  // namespace mi

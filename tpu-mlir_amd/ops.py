@@ -500,6 +500,14 @@ class RequantDesc:
                 setattr(self.c, "d_" + name, v.data_ptr())
             else:
                 setattr(self.c, name, int(v))
+        # the library cannot look into device arrays without a synchronization; look once, here, so that the Q31
+        # modes may take the 32-bit epilogue (see mi_requant_desc.per_channel_q31_checked)
+        ok = True
+        if hasattr(shift, "data_ptr"):
+            ok = ok and bool(((shift >= 1) & (shift <= 31)).all().item())
+        if hasattr(multiplier, "data_ptr"):
+            ok = ok and bool((multiplier != -2 ** 31).all().item())
+        self.c.per_channel_q31_checked = int(ok)
 
 
 _OUT_TORCH = {DT_I8: "int8", DT_U8: "uint8", DT_I16: "int16", DT_I32: "int32"}
