@@ -238,6 +238,18 @@ int mi_a16_to_group(const uint16_t *scale, int64_t scale_num, const uint8_t *zp,
 int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                     void *stream);
 
+/* mi_a16mm_launch for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid it).  No counterpart in the reference.  Same arguments, same kernels, bit-identical results;
+ * it calls no hipMalloc / hipFree or allocating library routine.  The only scratch memory the product needs -- the
+ * fp32 partial-sum slabs of a K-split tiled launch (more than 16 rows, few output blocks) -- lives in a 16 MiB device
+ * array inside the library (one copy per GPU, held until the process ends) instead of the stream's growable buffer.
+ * A product whose slabs need more (k_splits * M * N * 4 bytes; e.g. M = 128, N = 4096 with 4 splits is 8 MiB) is
+ * refused with MI_BAD_ARGUMENT and a message that says so.  The slabs need no clearing (every element read is written
+ * by the same launch), but every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race -- serialize them. */
+int mi_a16mm_launch_noalloc(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
+                            void *stream);
+
 /* The same for n (1..4) weight sets that read the SAME activations, in one kernel launch: y_i = x * dequant(W_i)^T.
  * These are the sibling linears the reference's LLM export emits on one input -- q/k/v on the normed hidden state
  * (python/llm/LlmConverter.py:1797-1812), gate/up in the MLP -- each of which the interpreter runs as its own

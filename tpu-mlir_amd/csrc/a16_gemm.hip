@@ -596,3 +596,31 @@ int a16_gemm_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t 
 
 }  // namespace mi
 
+// ------------------------------------------------------------------------------------------------
+// A launch that allocates nothing: mi_a16mm_launch with the split-K slabs in a fixed device array.
+// ------------------------------------------------------------------------------------------------
+namespace {
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)16 << 20;
+constexpr int NOALLOC_MAX_DEVICES = 64;
+// Each GPU the library runs on holds its own copy of this array, at its own address, until the process ends.  In
+// host code the name below is only a handle for hipGetSymbolAddress, never a device address.
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+void *g_scratch_ptr[NOALLOC_MAX_DEVICES];  // per device: address of that device's copy, once looked up
+}  // namespace
+
+extern "C" int mi_a16mm_launch_noalloc(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y,
+                                       float *d_y_f32, void *stream) {
+  using namespace mi;
+  MI_REQUIRE(w, MI_BAD_ARGUMENT, "mi_a16mm_launch_noalloc: null weight set");
+  int dev = 0;
+  MI_HIP(hipGetDevice(&dev));
+  MI_REQUIRE(dev >= 0 && dev < NOALLOC_MAX_DEVICES, MI_UNSUPPORTED, "mi_a16mm_launch_noalloc: device index past 63");
+  void *ptr = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (!ptr) {  // first call on this device (which is current): look its copy of the array up, once
+    MI_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    MI_REQUIRE(ptr, MI_HIP_ERROR, "mi_a16mm_launch_noalloc: the scratch array has no address on this device");
+    __atomic_store_n(&g_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
+  }
+  const A16Scratch fixed = {ptr, NOALLOC_SCRATCH_BYTES};
+  return a16_launch_group(&w, 1, d_x, M, &d_y, d_y_f32 ? &d_y_f32 : nullptr, (hipStream_t)stream, &fixed);
+}
