@@ -175,6 +175,29 @@ def _time_graph(torch, fn, replays, warmup=2):
     return _time_launches(torch, g_.replay, replays, warmup=warmup)
 
 
+def bench_read_ceiling(pkg, torch, sizes, steps=60, pool_mb=1024):
+    """What a single launch that only READS n bytes from HBM costs on this machine (mi_bench_read_launch: one 16-byte
+    load per lane, every load of a wave requested up front), timed exactly as the GEMVs are: launches replayed from
+    a HIP graph, each on a different region of a pool larger than the 256 MB cache.  The best of 2 / 4 / 8 chunks per
+    wave is kept.  Returns {n_bytes: {"us": .., "GBps": ..}}."""
+    pool = torch.empty(pool_mb << 20, dtype=torch.uint8, device="cuda").fill_(1)
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    out = {}
+    for nbytes in sizes:
+        stride = (nbytes + 4095) & ~4095
+        copies = max(2, min(64, (pool_mb << 20) // stride))
+        best = None
+        for cpw in (2, 4, 8):
+            def run():
+                for c in range(copies):
+                    pkg.bench_read_launch(pool[c * stride:], nbytes, sink, chunks_per_wave=cpw)
+            sec = _time_graph(torch, run, max(3, steps // copies)) / copies
+            best = sec if best is None else min(best, sec)
+        out[int(nbytes)] = {"us": round(best * 1e6, 2), "GBps": round(nbytes / best / 1e9, 1)}
+    del pool
+    return out
+
+
 def bench_single_matmuls(pkg, S, torch, steps=60):
     """Per-matmul figures of the secondary configurations: decode GEMVs (HBM GB/s of algorithmic bytes) and
     prefill GEMMs (TFLOP/s).  Each case rotates over enough weight copies to stay out of the 256 MB cache when the

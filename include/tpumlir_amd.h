@@ -446,6 +446,15 @@ int mi_module_uses_graph(const mi_module *m);
 /* float data out (expanded on the device), as py_cuda::get_tensor */
 int mi_module_get_tensor(mi_module *m, const char *name, float *out, int64_t num_elem);
 
+/* ============================================================================ */
+/* Measurement aid (no counterpart in the reference)                             */
+/* ============================================================================ */
+/* Streams `bytes` (rounded down to whole KiB chunks) from d_src with one 16-byte load per lane, every wave requesting
+ * chunks_per_wave (2, 4 or 8) chunks before it consumes any, and writes nothing (d_sink: 4 writable bytes, never
+ * written for ordinary data).  The launch time of this kernel is the ceiling for any single launch that has to move
+ * the same bytes from HBM; the benchmark reports the decode kernels against it. */
+int mi_bench_read_launch(const void *d_src, size_t bytes, int chunks_per_wave, void *d_sink, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -12,4 +12,4 @@ from .clib import (MI_SUCCESS, MI_UNSUPPORTED, MI_BAD_ARGUMENT, MI_HIP_ERROR, Ba
 from .ops import (A16MatMul, A16Weight, MatMulInt8, Module, RequantDesc, a16mm_launch,  # noqa: F401
                   a16mm_launch_group, i8mm_launch, cast, cast_launch, requant_int, requant_int_axis, requant_launch,
                   a16_quantize, a16_to_group, llm_unpack, a16mm_dq_launch, matmul_dq, matmul_dq_launch, matmul_f8,
-                  f8mm_launch, PACK_GPTQ, PACK_AWQ)
+                  f8mm_launch, bench_read_launch, PACK_GPTQ, PACK_AWQ)

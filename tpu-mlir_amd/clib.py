@@ -29,6 +29,7 @@ EXPORTS = [
     "mi_module_create", "mi_module_destroy", "mi_module_add_tensor", "mi_module_add_a16matmul", "mi_module_add_a16matmul_dq",
     "mi_module_add_matmul_int8", "mi_module_add_requant", "mi_module_add_matmul_dq", "mi_module_add_cast", "mi_module_set_tensor", "mi_module_invoke",
     "mi_module_uses_graph", "mi_module_get_tensor",
+    "mi_bench_read_launch",
 ]
 
 
@@ -209,6 +210,7 @@ def lib():
                                         C.POINTER(RequantDescC), C.c_void_p]
         L.mi_requant_int_axis_inference.argtypes = [C.POINTER(RqAxisAttr), C.POINTER(InferParam)]
         L.mi_requant_int_inference.argtypes = [C.POINTER(RqAttr), C.POINTER(InferParam)]
+        L.mi_bench_read_launch.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_void_p]
         _lib = L
     return _lib
 

@@ -1,0 +1,421 @@
+// W4A16 / W8A16 matmul for gfx950, decode (at most four activation rows): the kernel behind the GEMV numbers.
+//
+// Same packed weights, same arithmetic and the same results as the skinny kernel of a16_kernels.hip; what differs is
+// everything around the arithmetic.  At decode sizes a launch lives for a few microseconds, and a workgroup's fixed
+// costs -- what stands between kernel entry and its first weight request, and between the last byte's arrival and the
+// store -- are as long as the memory stream itself.  So:
+//   * A workgroup owns one 16-channel row block over the whole K; its waves take the K tiles round-robin and each wave
+//     requests ALL its tiles in one go (static count, indices clamped, never predicated).
+//   * The kernel arguments are one flat record.  Sibling weight sets (q/k/v, gate/up) are told apart by three scalar
+//     compares against the sets' first row blocks; the host has pre-subtracted each set's offset from its pointers,
+//     so every address is `pointer of the set + global row block * stride` with no per-set index arithmetic.
+//   * A wave loads ITS slice of the activation rows (one 16-byte request per lane and row for the usual shapes),
+//     parks it in its own corner of LDS, forms the per-group activation sums with cross-lane (DPP) adds, and reads the
+//     MFMA A fragments back, all by itself (no workgroup barrier): a wave starts multiplying as soon as ITS data
+//     has arrived.
+//   * Tiles are multiplied two at a time -- two independent MFMA chains -- with the LDS reads of both issued before
+//     the wave waits for the weights: with two waves per SIMD there is little else to hide latencies behind.
+//   * Only lanes 0..15 hold live output rows (rows 0..3 of the 16 x 16 MFMA block): they alone take part in the
+//     cross-wave sum: one 16-byte LDS write per lane, the kernel's one barrier, and wave 0 adds the partial sums in
+//     wave order and stores the 64 outputs (their addresses were settled in the prologue).
+// Arithmetic (see a16_kernels.hip): 4-bit  acc += scale * (sum a (16 + q) - (16 + zp) * sum a)  per group, in fp32;
+// 8-bit  weights rounded to the 16-bit type exactly as the reference does, accumulated directly.
+#include <climits>
+
+#include "a16_common.cuh"
+#include "internal.h"
+
+namespace mi {
+
+// v + (v of the lane a DPP control names): the cross-lane adds of the activation sums
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+constexpr int DEC_MAX_SEG = 4;
+constexpr int DEC_MAX_ROWS = 4;
+
+struct DecodeArgs {
+  const uint8_t *x;                 // activations [M, K], 16-bit
+  int M, k_tiles;                   // k_tiles = K / TILE_K (K is a whole number of tiles here)
+  int G, group_shift;               // GPT == 1: group of tile kt = kt >> group_shift (31: one group spans K)
+  int x_row_bytes, chip;
+  int rb_begin[DEC_MAX_SEG];        // first row block of each weight set on the grid (unused slots: INT_MAX)
+  // per weight set, each pre-offset by the host so that it is indexed by the GLOBAL row block / channel number
+  const uint8_t *qw[DEC_MAX_SEG];   // - rb_begin * k_tiles * 1024
+  const uint8_t *sz[DEC_MAX_SEG];   // 4-bit: scale|zp words, - rb_begin * G * 64;  8-bit: scale bits, - rb_begin * G * 32
+  const uint8_t *nz[DEC_MAX_SEG];   // 8-bit: -zp' * scale floats, - rb_begin * G * 64
+  const float *bias[DEC_MAX_SEG];   // - rb_begin * 16, or null
+  uint16_t *y[DEC_MAX_SEG];         // - rb_begin * 16
+  float *y32[DEC_MAX_SEG];          // - rb_begin * 16, or null
+  int n_end[DEC_MAX_SEG];           // rb_begin * 16 + N: first global channel number past the set
+  int n_cols[DEC_MAX_SEG];          // N of the set (row stride of its outputs)
+};
+
+template <int BITS, int DT, int GPT, int WAVES, int TPW, int MR>
+__global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
+  using H = Half16<DT>;
+  using vec8 = typename H::vec8;
+  constexpr int TILE_K = BITS == 4 ? W4_TILE_K : W8_TILE_K;
+  constexpr int KSTEPS = TILE_K / 32;
+  constexpr int KSTEPS_PER_UNIT = KSTEPS / GPT;
+  constexpr int CPT = TILE_K / 8;                // 16-byte activation chunks per tile: 16 / 8
+  constexpr int XCHUNKS = TPW * CPT;             // chunks of one row in this wave's slice
+  constexpr int XL = (XCHUNKS + 63) / 64;        // requests per lane and row
+  constexpr int XROW = XL * 64 * 16;             // bytes of LDS per row (padded to whole requests)
+  constexpr int UNIT_CHUNKS = CPT / GPT;         // chunks per quantization group inside a tile
+  constexpr int UNITS = TPW * GPT;
+  constexpr int S_BYTES = BITS == 4 ? UNITS * 16 : 0;  // per unit: the sums of rows 0..3
+  constexpr int WAVE_LDS = MR * XROW + S_BYTES;
+  constexpr int RED_BYTES = WAVES * 256;         // partial sums of the final reduction
+  static_assert(TPW % 2 == 0, "tiles are taken two at a time");
+  static_assert(KSTEPS_PER_UNIT >= 1 && UNIT_CHUNKS >= 1, "at most one group per MFMA k-step");
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rb = blockIdx.x;
+  const int col = lane & 15, kq = lane >> 4;
+
+  // ---- which weight set: everything scalar, selected (not indexed: an index would go back to memory)
+  const int s1 = rb >= a.rb_begin[1], s2 = rb >= a.rb_begin[2], s3 = rb >= a.rb_begin[3];
+#define MI_SEL(f) (s3 ? a.f[3] : s2 ? a.f[2] : s1 ? a.f[1] : a.f[0])
+  const uint8_t *qw = MI_SEL(qw) + (int64_t)rb * a.k_tiles * 1024;
+  const int k_tiles = a.k_tiles;
+  const uint32_t lane16 = (uint32_t)lane * 16u;
+
+  // ---- requests.  First this wave's slice of the activation rows (cache hits for all but the first workgroups; it
+  // is needed first), then every weight tile with its group parameters, then the bias.
+  u32x4 xv[MR][XL];
+#pragma unroll
+  for (int ld = 0; ld < XL; ++ld) {
+    const int q = ld * 64 + lane;
+    int p = q / CPT;
+    p = p < TPW ? p : TPW - 1;  // lanes past the slice repeat its last tile (their LDS slots are padding)
+    int kt = wave + p * WAVES;
+    kt = kt < k_tiles ? kt : k_tiles - 1;
+    const uint32_t off = (uint32_t)(kt * TILE_K + (q % CPT) * 8) * 2u;
+#pragma unroll
+    for (int r = 0; r < MR; ++r) {
+      const int row = r < a.M ? r : a.M - 1;
+      xv[r][ld] = *(const u32x4 *)(a.x + ((uint32_t)row * (uint32_t)a.x_row_bytes + off));
+    }
+  }
+  u32x4 w[TPW];
+  uint32_t szv[TPW][GPT];
+  float nzv[TPW][GPT];
+  const uint8_t *szp = MI_SEL(sz) + (int64_t)rb * a.G * (BITS == 4 ? 64 : 32);
+  const uint8_t *nzp = nullptr;
+  if constexpr (BITS == 8)
+    nzp = MI_SEL(nz) + (int64_t)rb * a.G * 64;
+#pragma unroll
+  for (int p = 0; p < TPW; ++p) {
+    int kt = wave + p * WAVES;
+    kt = kt < k_tiles ? kt : k_tiles - 1;  // past the end: a harmless re-load, never multiplied
+    w[p] = *(const u32x4 *)(qw + ((uint32_t)kt * 1024u + lane16));
+#pragma unroll
+    for (int u = 0; u < GPT; ++u) {
+      uint32_t gi = GPT == 1 ? (uint32_t)(kt >> a.group_shift) : (uint32_t)(kt * GPT + u);
+      if constexpr (BITS == 4) {
+        szv[p][u] = *(const uint32_t *)(szp + (gi * 64u + (uint32_t)col * 4u));
+      } else {
+        szv[p][u] = *(const uint16_t *)(szp + (gi * 32u + (uint32_t)col * 2u));
+        nzv[p][u] = *(const float *)(nzp + (gi * 64u + (uint32_t)col * 4u));
+      }
+    }
+  }
+  const float *biasp = MI_SEL(bias);
+  const int n_end = MI_SEL(n_end);
+  const int n = rb * 16 + col;                       // global channel number
+  const int nc = n < n_end ? n : n_end - 1;
+  float bias_v = 0.0f;
+  if (biasp)
+    bias_v = biasp[nc];
+
+  // output addressing, settled now (scalar selects and one 64-bit multiply) so that nothing but the sum stands
+  // between the last partial result and the store
+  const int n_cols = MI_SEL(n_cols);
+  float *const y32 = MI_SEL(y32);
+  uint16_t *const y = MI_SEL(y);
+  asm volatile("" ::"s"(n_cols), "s"(y32), "s"(y));  // fetched with the first batch of scalar loads, not at the end
+  const int64_t o = (int64_t)kq * n_cols + n;
+
+  // ---- this wave's activations: LDS slice, group sums, fragments
+  uint8_t *xs = smem + RED_BYTES + wave * WAVE_LDS;          // [MR][XROW]
+  float *s_lds = reinterpret_cast<float *>(xs + MR * XROW);  // [UNITS][4]
+#pragma unroll
+  for (int r = 0; r < MR; ++r)
+#pragma unroll
+    for (int ld = 0; ld < XL; ++ld) {
+      const int q = ld * 64 + lane;
+      *(u32x4 *)(xs + r * XROW + q * 16) = xv[r][ld];
+      if constexpr (BITS == 4) {
+        float part = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          part += H::to_f32((uint16_t)(xv[r][ld][i] & 0xffffu)) + H::to_f32((uint16_t)(xv[r][ld][i] >> 16));
+        // sum over the UNIT_CHUNKS (16, 8 or 4) neighbouring lanes of the group: butterfly inside a row of 16 lanes
+        part += dpp_f32<0xB1>(part);      // quad_perm [1,0,3,2]
+        part += dpp_f32<0x4E>(part);      // quad_perm [2,3,0,1]
+        if constexpr (UNIT_CHUNKS >= 8)
+          part += dpp_f32<0x141>(part);   // row_half_mirror: the other quad of the half row
+        if constexpr (UNIT_CHUNKS >= 16)
+          part += dpp_f32<0x140>(part);   // row_mirror: the other half row
+        if ((q % UNIT_CHUNKS) == 0 && q < XCHUNKS)
+          s_lds[(q / UNIT_CHUNKS) * 4 + r] = part;
+      }
+    }
+  // The fragments below are other lanes' chunks of this wave's own slice: order the wave's LDS writes before its
+  // reads (no other wave touches the slice, so no workgroup barrier)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  const int row_ld = col < a.M ? col : a.M - 1;  // output rows past M repeat the last row; they are never stored
+  const int row_x = row_ld < MR ? row_ld : MR - 1;
+  const uint8_t *xfp = xs + row_x * XROW + kq * 16;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  uint32_t nib_magic = H::NIB_MAGIC2;
+  asm volatile("" : "+v"(nib_magic));  // keep it in a VGPR (see and_or)
+
+  // Tiles are taken two at a time: the A fragments and activation sums of both are read from LDS before the wave
+  // waits for the weights, and the two tiles' MFMA chains are independent, so one chain's latency hides behind the
+  // other's unpacking.
+  auto fold4 = [&](const f32x4 &P, int unit, uint32_t szw, bool live) {
+    const float sc = H::to_f32((uint16_t)(szw >> 16));
+    const float c = H::OFFSET + (float)(szw & 0xffu);
+    if constexpr (MR == 1) {  // one live row: register 0
+      const float S0 = s_lds[unit * 4];
+      const float t = fmaf(-c, S0, P[0]);
+      acc[0] = fmaf(sc, live ? t : 0.0f, acc[0]);
+    } else {
+      const f32x4 S = *(const f32x4 *)(s_lds + unit * 4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float t = fmaf(-c, S[i], P[i]);
+        acc[i] = fmaf(sc, live ? t : 0.0f, acc[i]);
+      }
+    }
+  };
+#pragma unroll
+  for (int pb = 0; pb < TPW; pb += 2) {
+    constexpr int NB = 2;
+    u32x4 xf[NB][KSTEPS];
+    bool live[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      live[b] = wave + (pb + b) * WAVES < k_tiles;  // wave-uniform; a dead tile is a re-load whose product is dropped
+#pragma unroll
+      for (int j = 0; j < KSTEPS; ++j)
+        xf[b][j] = *(const u32x4 *)(xfp + ((pb + b) * CPT + 4 * j) * 16);
+    }
+    if constexpr (BITS == 4) {
+      f32x4 P[NB];
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+        P[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < KSTEPS; ++j) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+          P[b] = H::mfma(__builtin_bit_cast(vec8, xf[b][j]), unpack_nibbles<DT>(w[pb + b][j], nib_magic), P[b]);
+        if ((j + 1) % KSTEPS_PER_UNIT == 0) {
+          const int u = j / KSTEPS_PER_UNIT;
+#pragma unroll
+          for (int b = 0; b < NB; ++b) {
+            // With one live row only register 0 of P is read below.  The whole tuple is named as read here: otherwise
+            // the three dead registers are handed to the next fragment's unpacking while the matrix unit has yet to
+            // write them (observed: fragments overwritten by late MFMA results).
+            asm volatile("" ::"v"(P[b]));
+            fold4(P[b], (pb + b) * GPT + u, szv[pb + b][u], live[b]);
+            P[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        if (live[b]) {
+#pragma unroll
+          for (int j = 0; j < KSTEPS; ++j) {
+            const int u = GPT == 1 ? 0 : j;
+            acc = H::mfma(__builtin_bit_cast(vec8, xf[b][j]),
+                          dequant_bytes<DT>(w[pb + b][2 * j], w[pb + b][2 * j + 1],
+                                            H::to_f32((uint16_t)szv[pb + b][u]), nzv[pb + b][u]),
+                          acc);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- cross-wave sum.  Rows 0..3 of the block live in lanes 0..15 (register i = row i): 256 bytes per wave, one
+  // barrier (the only one of the kernel), and wave 0 adds the WAVES partial sums in wave order and stores.  (Letting
+  // the wave that arrives last do this, behind an LDS ticket instead of the barrier, was measured: the barrier that
+  // then has to publish the cleared ticket costs more than it saves, 8.2 against 6.8 us at K = 11008.)
+  f32x4 *red = reinterpret_cast<f32x4 *>(smem);  // [WAVES][16]
+  if (kq == 0)
+    red[wave * 16 + col] = acc;
+  __syncthreads();
+  if (wave == 0) {
+    // lane (col, kq) finishes row kq of channel col
+    const float *redf = reinterpret_cast<const float *>(smem);
+    float v = 0.0f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv)
+      v += redf[(wv * 16 + col) * 4 + kq];
+    if (kq < a.M && n < n_end) {
+      v += bias_v;
+      if (y32)
+        y32[o] = v;
+      y[o] = (a.chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+    }
+  }
+#undef MI_SEL
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+constexpr size_t DEC_MAX_LDS = 40 * 1024;  // keeps four workgroups on a CU
+
+static size_t decode_lds_bytes(int bits, int gpt, int waves, int tpw, int mr) {
+  const int cpt = (bits == 4 ? W4_TILE_K : W8_TILE_K) / 8;
+  const int xl = (tpw * cpt + 63) / 64;
+  const size_t wave_lds = (size_t)mr * xl * 64 * 16 + (bits == 4 ? (size_t)tpw * gpt * 16 : 0);
+  return (size_t)waves * 256 + (size_t)waves * wave_lds;
+}
+
+struct DecodePlan {
+  int waves, tpw, mr, gpt;
+  bool ok;
+};
+
+static DecodePlan decode_plan(const mi_a16_weight *w, int64_t M) {
+  DecodePlan p = {8, 0, 0, 1, false};
+  const int tile_k = w->bits == 4 ? W4_TILE_K : W8_TILE_K;
+  if (M < 1 || M > DEC_MAX_ROWS || (w->K % tile_k) != 0)
+    return p;
+  if (w->g != 0 && w->g < tile_k)
+    p.gpt = tile_k / w->g;
+  else if (w->g != 0) {
+    const int tpg = w->g / tile_k;  // whole tiles per group: the kernel shifts, so it has to be a power of two
+    if ((tpg & (tpg - 1)) != 0 && tpg < w->k_tiles)
+      return p;
+  }
+  const int64_t kt = w->k_tiles;
+  p.waves = (kt + 7) / 8 > 8 ? 16 : 8;
+  const int64_t share = (kt + p.waves - 1) / p.waves;
+  static const int steps[] = {2, 4, 6, 8};
+  for (int t : steps)
+    if (share <= t) {
+      p.tpw = t;
+      break;
+    }
+  if (!p.tpw)
+    return p;  // K too long for one round of requests
+  if (p.waves == 16 && p.tpw < 6)
+    p.tpw = 6;  // the instantiated set
+  p.mr = M == 1 ? 1 : 4;
+  p.ok = decode_lds_bytes(w->bits, p.gpt, p.waves, p.tpw, p.mr) <= DEC_MAX_LDS;
+  return p;
+}
+
+template <int BITS, int DT, int GPT, int W, int T, int MR>
+static void launch_decode_instance(const DecodeArgs &a, int row_blocks, size_t lds_bytes, hipStream_t st) {
+  auto kfn = a16_decode_kernel<BITS, DT, GPT, W, T, MR>;  // at most 40 KiB of LDS: inside the default limit
+  kfn<<<dim3((unsigned)row_blocks), dim3(W * 64), lds_bytes, st>>>(a);
+}
+
+template <int BITS, int DT, int GPT>
+static bool launch_decode_shape(const DecodeArgs &a, const DecodePlan &p, int row_blocks, size_t lds, hipStream_t st) {
+#define MI_DEC_CASE(W, T)                                                         \
+  if (p.waves == W && p.tpw == T) {                                               \
+    if (p.mr == 1)                                                                \
+      launch_decode_instance<BITS, DT, GPT, W, T, 1>(a, row_blocks, lds, st);     \
+    else                                                                          \
+      launch_decode_instance<BITS, DT, GPT, W, T, 4>(a, row_blocks, lds, st);     \
+    return true;                                                                  \
+  }
+  MI_DEC_CASE(8, 2)
+  MI_DEC_CASE(8, 4)
+  MI_DEC_CASE(8, 6)
+  MI_DEC_CASE(8, 8)
+  MI_DEC_CASE(16, 6)
+  MI_DEC_CASE(16, 8)
+#undef MI_DEC_CASE
+  return false;
+}
+
+// True when the decode kernel takes the launch (and then it has been issued); false leaves it to the general kernels.
+bool a16_decode_launch(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
+                       float *const *d_y32s, hipStream_t stream) {
+  const mi_a16_weight *w = ws[0];
+  if (n < 1 || n > DEC_MAX_SEG)
+    return false;
+  const DecodePlan p = decode_plan(w, M);
+  if (!p.ok)
+    return false;
+  const int64_t gbytes = w->bits == 4 ? 64 : 32;
+  DecodeArgs a;
+  a.x = (const uint8_t *)d_x;
+  a.M = (int)M;
+  a.k_tiles = (int)w->k_tiles;
+  a.G = w->G;
+  a.chip = w->chip;
+  a.x_row_bytes = (int)(w->K * 2);
+  a.group_shift = 0;
+  if (p.gpt == 1) {
+    const int tile_k = w->bits == 4 ? W4_TILE_K : W8_TILE_K;
+    const int tpg = w->g == 0 ? (int)w->k_tiles : w->g / tile_k;
+    if (tpg >= w->k_tiles)
+      a.group_shift = 31;
+    else
+      while ((1 << a.group_shift) < tpg)
+        ++a.group_shift;
+  }
+  int64_t rb0 = 0;
+  for (int i = 0; i < DEC_MAX_SEG; ++i) {
+    const int q = i < n ? i : 0;  // unused slots repeat the first set; the kernel never selects them
+    const mi_a16_weight *v = ws[q];
+    const int64_t first = i < n ? rb0 : 0;
+    a.rb_begin[i] = i < n ? (int)rb0 : INT_MAX;
+    a.qw[i] = (const uint8_t *)v->qweight - first * v->k_tiles * 1024;
+    a.sz[i] = (v->bits == 4 ? (const uint8_t *)v->sz_t : (const uint8_t *)v->scale_t) - first * v->G * gbytes;
+    a.nz[i] = v->bits == 8 ? (const uint8_t *)v->nzs_t - first * v->G * 64 : nullptr;
+    a.bias[i] = v->bias ? v->bias - first * 16 : nullptr;
+    a.y[i] = d_ys[q] - first * 16;
+    a.y32[i] = (d_y32s && d_y32s[q]) ? d_y32s[q] - first * 16 : nullptr;
+    a.n_end[i] = (int)(first * 16 + v->N);
+    a.n_cols[i] = (int)v->N;
+    if (i < n)
+      rb0 += v->row_blocks;
+  }
+  if (rb0 * 16 >= INT_MAX)
+    return false;
+  const size_t lds = decode_lds_bytes(w->bits, p.gpt, p.waves, p.tpw, p.mr);
+  const bool f16 = w->dtype == MI_DT_F16;
+  bool ok = false;
+#define MI_DEC(BITS_, GPT_)                                                                \
+  ok = f16 ? launch_decode_shape<BITS_, MI_DT_F16, GPT_>(a, p, (int)rb0, lds, stream)      \
+           : launch_decode_shape<BITS_, MI_DT_BF16, GPT_>(a, p, (int)rb0, lds, stream);
+  if (w->bits == 4) {
+    if (p.gpt == 1) {
+      MI_DEC(4, 1)
+    } else if (p.gpt == 2) {
+      MI_DEC(4, 2)
+    } else if (p.gpt == 4) {
+      MI_DEC(4, 4)
+    }
+  } else {
+    if (p.gpt == 1) {
+      MI_DEC(8, 1)
+    } else if (p.gpt == 2) {
+      MI_DEC(8, 2)
+    }
+  }
+#undef MI_DEC
+  return ok;
+}
+
+}  // namespace mi

@@ -768,6 +768,10 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
     }
     return MI_SUCCESS;
   }
+  if (!plan().a16_no_decode && a16_decode_launch(ws, n, d_x, M, d_ys, d_y32s, stream)) {
+    MI_HIP(hipGetLastError());
+    return MI_SUCCESS;
+  }
   const int tile_k = w->bits == 4 ? W4_TILE_K : W8_TILE_K;
   a.n_seg = n;
   a.x = d_x;

@@ -16,6 +16,7 @@ typedef struct mi_internal_plan {
   int a16_waves, a16_tpw, a16_rows;  // skinny kernel instance (waves per workgroup, tiles per wave and round, row blocks)
   int a16_xlds;                      // 1: stage the activations in LDS, 2: read them from L2
   int a16_no_gemm;                   // 1: never take the tiled kernel
+  int a16_no_decode;                 // 1: never take the decode kernel (at most four rows)
   int a16_gemm_min_m;                // > 0: tiled kernel from this many rows on (M > 1)
   int a16_gemm_splits;               // > 0: number of K splits of the tiled kernel
   int a16_gemm_tile;                 // 128 / 256: columns per output block
@@ -107,6 +108,10 @@ struct A16Scratch {
   void *ptr;
   size_t bytes;
 };
+// decode kernel (a16_decode.hip): at most four rows, K a whole number of tiles.  Returns false, having launched
+// nothing, when the shape is not its own; the general kernels then take it.
+bool a16_decode_launch(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
+                       float *const *d_y32s, hipStream_t stream);
 // tiled MFMA GEMM for many activation rows (prefill)
 bool a16_gemm_applicable(const mi_a16_weight *w, int64_t M);
 // up to three sibling weight sets (same K, width, group size, type, chip) on one input in one launch

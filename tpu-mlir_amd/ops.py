@@ -488,6 +488,14 @@ def cast_launch(x, *, in_type, out_type, in_quant=False, out_quant=False, scale=
     return out
 
 
+def bench_read_launch(src, nbytes, sink, chunks_per_wave=4, stream=None):
+    """Measurement aid: streams the first nbytes of the CUDA tensor src from HBM (mi_bench_read_launch)."""
+    if not (src.is_cuda and src.is_contiguous() and src.numel() * src.element_size() >= nbytes):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "bench_read_launch: src must be a contiguous CUDA tensor of nbytes")
+    check(clib.lib().mi_bench_read_launch(_dptr(src), int(nbytes), int(chunks_per_wave), _dptr(sink),
+                                          _stream_ptr(stream)))
+
+
 class RequantDesc:
     """Per-channel (torch int32 CUDA tensors) or scalar requantization parameters; shift > 0 shifts right."""
 
