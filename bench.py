@@ -28,6 +28,7 @@ from __graft_entry__ import load_package  # noqa: E402
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, AMD's published figure
 INT8_PEAK_TOPS = 5000.0      # dense INT8 MFMA
 BF16_PEAK_TFLOPS = 2500.0    # dense bf16 MFMA
+HBM_TRAFFIC_RATIO = 1.022    # measured HBM bytes / algorithmic bytes of the decode chain (see roofline.traffic_source)
 
 
 def _dev_bf16(torch, bits):
@@ -78,28 +79,40 @@ def run_chain(pkg, mats, acts, outs, grouped=True):
     return len(CHAIN_GROUPS)
 
 
-def bench_chain(pkg, S, torch, M, steps, warmup, n_layers, cfgs, grouped=True):
+def bench_chain(pkg, S, torch, M, steps, warmup, n_layers, cfgs, grouped=True, graph_steps=None):
+    """Times exactly `steps` steps (one step = the seven matmuls of one layer).  The launches are replayed from HIP
+    graphs: one graph holds the steps of all n_layers weight copies back to back (as a decoder's graph holds its
+    layers), a second one the steps % n_layers left over, so that a graph launch's own cost is spread over several
+    steps as it is in a real decode step.  graph_steps: steps per graph when that is not n_layers (the weight copies are
+    then used round-robin)."""
     layers, acts, outs = build_chain(pkg, S, torch, M, n_layers, cfgs)
+    per_graph = graph_steps or n_layers
     stream = torch.cuda.Stream()
-    graphs = []
     with torch.cuda.stream(stream):
         for mats in layers:  # eager pass first: loads the code objects before capture
             launches = run_chain(pkg, mats, acts, outs, grouped)
         stream.synchronize()
-        for mats in layers:
+
+        def capture(count):
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=stream):
-                run_chain(pkg, mats, acts, outs, grouped)
-            graphs.append(g)
-        for i in range(warmup):
-            graphs[i % n_layers].replay()
+                for i in range(count):
+                    run_chain(pkg, layers[i % n_layers], acts, outs, grouped)
+            return g
+
+        full = capture(per_graph)
+        rest = capture(steps % per_graph) if steps % per_graph else None
+        for i in range(max(1, warmup // per_graph)):
+            full.replay()
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         stream.synchronize()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         ev0.record(stream)
-        for i in range(steps):
-            graphs[i % n_layers].replay()
+        for i in range(steps // per_graph):
+            full.replay()
+        if rest is not None:
+            rest.replay()
         ev1.record(stream)
         stream.synchronize()
         torch.cuda.synchronize()
@@ -159,6 +172,61 @@ def _time_launches(torch, fn, steps, warmup=5):
         ev1.record(stream)
         stream.synchronize()
     return ev0.elapsed_time(ev1) * 1e-3 / steps
+
+
+def bench_int8_context(pkg, S, torch, clib, n, launches=100):
+    """What bounds the INT8 figure on this machine, measured in the same run: the vendor library's int8 GEMM
+    (torch._int_mm: int32 output, no requantization) on the same random operands, and both kernels on all-zero operands.
+    The matrix cores' clock under load depends on the data (power): the gap between the random and the zero rows is
+    that effect, and no kernel here reaches the nominal 5 POPS (2.4 GHz) on random int8 data."""
+    out = {}
+    dev = lambda x: torch.from_numpy(np.ascontiguousarray(x)).cuda()
+    c = S.int8_matmul(8, 8, n, seed=7)
+    rq = pkg.RequantDesc(clib.RQ_QDM, clib.ROUND_HALF_AWAY_FROM_ZERO, out_dtype=clib.DT_I8,
+                         multiplier=dev(c["mult"]), shift=dev(c["shift"]))
+    bias = torch.zeros(n, dtype=torch.int32, device="cuda")
+    y = torch.empty((n, n), dtype=torch.int8, device="cuda")
+    for label in ("random", "zeros"):
+        if label == "random":
+            a = torch.randint(-128, 128, (n, n), dtype=torch.int8, device="cuda")
+            b = torch.randint(-128, 128, (n, n), dtype=torch.int8, device="cuda")
+        else:
+            a = torch.zeros((n, n), dtype=torch.int8, device="cuda")
+            b = torch.zeros((n, n), dtype=torch.int8, device="cuda")
+        ours = _time_launches(torch, lambda: pkg.i8mm_launch(a, b, bias, right_transpose=True, rq=rq, out=y), launches)
+        rec = {"this_kernel_us": round(ours * 1e6, 2), "this_kernel_tops": round(2.0 * n ** 3 / ours / 1e12, 1)}
+        if hasattr(torch, "_int_mm"):
+            try:
+                ven = _time_launches(torch, lambda: torch._int_mm(a, b.t()), launches)
+                rec["vendor_int_mm_us"] = round(ven * 1e6, 2)
+                rec["vendor_int_mm_tops"] = round(2.0 * n ** 3 / ven / 1e12, 1)
+            except Exception as e:  # the vendor path is a reference point only
+                rec["vendor_int_mm_error"] = str(e)[:80]
+        out[label] = rec
+    out["launches_each"] = launches
+    return out
+
+
+def cpu_baseline_int8(S, budget_s=8.0):
+    """The restated reference algorithm of the quantized tpu.MatMul on the host cores (oracle: int8 operands widened to
+    f32, f32 GEMM, per-channel MultiplyByQuantizedMultiplier in a scalar loop -- MatMul.cpp:598-604, :696-707), on a
+    bounded sample: M = 256 rows of the 4096 x 4096 product per pass."""
+    from oracle import pyoracle as O  # CPU baseline leg only
+    M, K, N = 256, 4096, 4096
+    c = S.int8_matmul(M, K, N, seed=7, right_transpose=True)
+    a, b = c["a"].astype(np.float32), c["b"].astype(np.float32)
+    bias, multi = c["bias"].astype(np.float32), c["mult"].astype(np.float32)
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        O.matmul_int8(a, b, bias, multi, M=M, K=K, N=N, right_transpose=True, quant_mode=O.RQ_TFLITE,
+                      multipliers=[int(c["mult"][0])], rshifts=[int(c["shift"][0])], gemm_kind=O.GEMM_FAST)
+        passes += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or passes >= 20:
+            break
+    return {"value": round(2.0 * M * K * N * passes / el / 1e12, 4), "unit": "TOPS", "cores": O.num_threads(),
+            "kind": "port", "sample": "%d passes of a 256 x 4096 x 4096 slice in %.1f s (f32 GEMM on the host cores, "
+                                      "scalar requantization loop)" % (passes, el)}
 
 
 def _time_graph(torch, fn, replays, warmup=2):
@@ -421,7 +489,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--batch", type=int, default=1, help="activation rows M of the decode chain")
-    ap.add_argument("--layers", type=int, default=4, help="distinct weight copies rotated through (4 x 101 MB)")
+    ap.add_argument("--layers", type=int, default=4, help="distinct weight copies rotated through (4 x 101 MB); one "
+                    "HIP graph replay covers one step on each of them")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-int8", action="store_true")
     ap.add_argument("--no-group", action="store_true",
@@ -457,6 +526,13 @@ def main():
     avg_launch_s = r["gpu_s"] / n_launch
     bytes_per_launch = r["chain_bytes"] / r["launches_per_step"]
     achieved = bytes_per_launch / avg_launch_s / 1e9
+    # The ceiling for a launch of n bytes on this machine: a kernel that only reads n bytes, timed the same way in the
+    # same run.  The four launches of a step move these byte counts (q+k+v, o, gate+up, down):
+    by = {name: S.w4_gemv_bytes(M, K, N, 128) for name, K, N in S.LLAMA7B_CHAIN}
+    launch_bytes = [sum(by[n] for n in grp) for grp in CHAIN_GROUPS] if not args.no_group else list(by.values())
+    ceil = bench_read_ceiling(pkg, torch, sorted(set(launch_bytes + [8 << 20, 512 << 20])))
+    ceil_step_us = sum(ceil[b]["us"] for b in launch_bytes)
+    step_us = r["gpu_s"] / args.steps * 1e6
     line = {
         "metric": "W4A16 decode GEMV HBM GB/s (% peak); INT8 requant GEMM TOPS (% MFMA peak)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -466,26 +542,42 @@ def main():
                                "down 4096x11008)" % M,
                    "bytes_per_step": r["chain_bytes"], "launches_per_step": r["launches_per_step"],
                    "weight_copies": args.layers, "resident_weight_mb": round(r["weight_set_mb"], 1),
-                   "launch": "one HIP graph replay per step; q/k/v and gate/up each as one grouped launch"
-                             if not args.no_group else "one HIP graph replay per step; one launch per matmul"},
+                   "launch": ("one HIP graph replay per %d steps (one per weight copy); " % args.layers) +
+                             ("q/k/v and gate/up each as one grouped launch" if not args.no_group
+                              else "one launch per matmul"),
+                   "timing": "value: host wall clock around the timed region; roofline: HIP events on the launch stream"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE (profiles/hbm_traffic_pmc_*.md):
-                     # 1.022 x the algorithmic bytes at M = 1 with grouped launches; not re-measured by this run
-                     "traffic": int(bytes_per_launch * 1.022) if (M == 1 and not args.no_group) else None,
-                     "kernel": "a16w4_skinny_kernel<bf16, 1 group/tile>",
+                     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of this command
+                     # (profiles/hbm_traffic_pmc_*.md): a ratio to the algorithmic bytes measured once under the
+                     # profiler at M = 1 with grouped launches, applied here; this run does not re-measure it
+                     "traffic": int(bytes_per_launch * HBM_TRAFFIC_RATIO) if (M == 1 and not args.no_group) else None,
+                     "traffic_source": "profiles/hbm_traffic_pmc_decode_chain_and_int8_gemm.md (ratio %.3f)"
+                                       % HBM_TRAFFIC_RATIO,
+                     "kernel": "a16_decode_kernel<4-bit, bf16, 1 group per tile> (both instances: 8 waves x 4 tiles, "
+                               "16 waves x 6 tiles)",
                      "bytes_per_launch": int(bytes_per_launch),
                      "avg_launch_us": round(avg_launch_s * 1e6, 3),
-                     "timing": "HIP events on the launch stream around the whole timed region / launches"},
+                     "timing": "HIP events on the launch stream around the whole timed region / launches",
+                     # the same step made of read-only launches of the same byte counts, measured in this run
+                     "read_only_ceiling_us_per_step": round(ceil_step_us, 2),
+                     "frac_of_measured_ceiling": round(ceil_step_us / step_us, 4)},
         "frac_of_hbm_peak_whole_job": round(value / HBM_PEAK_GBS, 4),
     }
     if not args.no_int8:
-        line["int8_requant_gemm"] = bench_int8(pkg, S, torch, clib, args.int8_size, max(5, args.steps // 10),
-                                               max(2, args.warmup // 10))
+        # at least 100 launches whatever --steps says: short runs flatter a kernel whose clock sags under load
+        line["int8_requant_gemm"] = bench_int8(pkg, S, torch, clib, args.int8_size, max(100, args.steps // 2), 10)
+        line["int8_requant_gemm"]["launches_timed"] = max(100, args.steps // 2)
+        if not args.no_cpu_baseline:
+            line["int8_requant_gemm"]["cpu_baseline"] = cpu_baseline_int8(S)
     if not args.no_extras:
         ex = {}
+        ex["read_ceiling"] = {str(k): v for k, v in ceil.items()}
+        if not args.no_int8:
+            ex["int8_context"] = bench_int8_context(pkg, S, torch, clib, args.int8_size)
         # the same chain with one weight copy (101 MB: resident in the 256 MB cache after the first pass)
-        r1 = bench_chain(pkg, S, torch, M, max(20, args.steps // 2), 5, 1, cfgs, grouped=not args.no_group)
+        r1 = bench_chain(pkg, S, torch, M, max(20, args.steps // 2), 5, 1, cfgs, grouped=not args.no_group,
+                         graph_steps=args.layers)
         ex["chain_cache_resident_GBps"] = round(r1["chain_bytes"] / (r1["gpu_s"] / max(20, args.steps // 2)) / 1e9, 1)
         # one launch per matmul, for comparison with the grouped default
         r7 = bench_chain(pkg, S, torch, M, max(20, args.steps // 2), 5, args.layers, cfgs, grouped=False)
