@@ -364,11 +364,11 @@ def bench_dynamic_quant(pkg, S, torch, steps=40):
     return out
 
 
-def bench_f8_matmul(pkg, torch, clib, steps=20):
+def bench_f8_matmul(pkg, torch, clib, steps=20, shapes=((4096, 4096, 4096), (256, 1024, 1024))):
     """tpu.MatMul on E4M3 codes with per-channel F8 output requantization (codes out), random finite codes."""
     out = []
     rng = np.random.default_rng(12)
-    for M, K, N in ((4096, 4096, 4096), (256, 1024, 1024)):
+    for M, K, N in shapes:
         a = torch.from_numpy((rng.integers(0, 256, size=(M, K)).astype(np.uint8) & np.uint8(0xD7))).cuda()
         b = torch.from_numpy((rng.integers(0, 256, size=(N, K)).astype(np.uint8) & np.uint8(0xD7))).cuda()
         bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).cuda()
@@ -391,20 +391,57 @@ def bench_f8_matmul(pkg, torch, clib, steps=20):
     return out
 
 
-def bench_operator_boundary(pkg, S, steps=20):
+def bench_mfma_kernels(pkg, S, torch, clib, launches=10):
+    """The three MFMA-bound kernels alone, a few eager launches each: the short command the hardware-counter profiles
+    of these kernels are taken with (--only-mfma)."""
+    out = {"int8_4096": bench_int8(pkg, S, torch, clib, 4096, launches, 2)}
+    K = N = 4096
+    cfg = S.w4a16(1, K, N, 128, seed=31)
+    w = pkg.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=K, N=N, weight_bits=4, q_group_size=128)
+    x = _dev_bf16(torch, S.bf16_round(np.random.default_rng(5).standard_normal((2048, K), dtype=np.float32)))
+    y = torch.empty((2048, N), dtype=torch.bfloat16, device="cuda")
+    sec = _time_launches(torch, lambda: pkg.a16mm_launch(w, x, y), launches, warmup=2)
+    out["w4_g128_prefill_M2048_4096x4096"] = {"us": round(sec * 1e6, 2),
+                                              "TFLOPs": round(2.0 * 2048 * N * K / sec / 1e12, 1)}
+    w.destroy()
+    out["f8_matmul"] = bench_f8_matmul(pkg, torch, clib, steps=launches, shapes=((4096, 4096, 4096),))
+    return out
+
+
+def bench_operator_boundary(pkg, S, steps=200):
     """The same q_proj GEMV through the reference's operator interface (float32-expanded host tensors in and out,
-    like InferenceParameter): includes the host<->device copies and conversions, so it is NOT a roofline figure."""
+    like InferenceParameter): includes the host<->device transfers and conversions, so it is NOT a roofline figure.
+    us_per_call times the C entry point with a prepared parameter block, as the interpreter's C++ walk would call it;
+    python_wrapper_us_per_call goes through the numpy front end (which allocates the output and builds the block)."""
+    import ctypes
+    clib = load_package("clib")
     K = N = 4096
     cfg = S.w4a16(1, K, N, 128, seed=41)
     x, w, s, z, _ = S.f32_valued_a16(cfg)
     op = pkg.A16MatMul(K=K, N=N, weight_bits=4, q_group_size=128).init(w, s, z, None)
-    op.inference(x)
+    for _ in range(50):  # an idle GPU answers the first calls slowly
+        op.inference(x)
     t0 = time.perf_counter()
     for _ in range(steps):
         op.inference(x)
+    sec_py = (time.perf_counter() - t0) / steps
+    y = np.empty((1, N), dtype=np.float32)
+    fp = ctypes.POINTER(ctypes.c_float)
+    ins = (fp * 5)(x.ctypes.data_as(fp), w.ctypes.data_as(fp), s.ctypes.data_as(fp), z.ctypes.data_as(fp), None)
+    outs = (fp * 1)(y.ctypes.data_as(fp))
+    prm = clib.InferParam(ins, 5, outs, 1, op.param.c.handle)
+    op.attr.M = 1
+    fn, a_ref, p_ref = clib.lib().mi_a16mm_inference, ctypes.byref(op.attr), ctypes.byref(prm)
+    for _ in range(10):
+        fn(a_ref, p_ref)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        rc = fn(a_ref, p_ref)
     sec = (time.perf_counter() - t0) / steps
+    assert rc == 0 and np.array_equal(y, op.inference(x))
     op.deinit()
     return {"case": "A16MatMul.inference, float32 host tensors, M=1 4096x4096", "us_per_call": round(sec * 1e6, 1),
+            "python_wrapper_us_per_call": round(sec_py * 1e6, 1),
             "GBps_algorithmic": round(S.w4_gemv_bytes(1, K, N, 128) / sec / 1e9, 1)}
 
 
@@ -498,6 +535,9 @@ def main():
     ap.add_argument("--int8-size", type=int, default=4096)
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the secondary figures (other M, single matmuls, prefill, cache-resident chain)")
+    ap.add_argument("--only-mfma", action="store_true",
+                    help="run only the three MFMA-bound kernels (INT8 4096^3, W4A16 prefill M=2048, F8 4096^3), a few "
+                         "launches each, and print their figures: the command for hardware-counter profiles")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; every GPU box of this run has one. Use --gpus 1.")
@@ -517,6 +557,10 @@ def main():
     cal_dst.copy_(cal_src)
     torch.cuda.synchronize()
     del cal_src, cal_dst
+
+    if args.only_mfma:
+        print(json.dumps({"only_mfma": bench_mfma_kernels(pkg, S, torch, clib)}), flush=True)
+        return
 
     M = args.batch
     cfgs = host_chain(S, M)

@@ -102,11 +102,42 @@ struct DevBuf {
 // ---------------------------------------------------------------------------------------------
 // tpu.A16MatMul operator state
 // ---------------------------------------------------------------------------------------------
+// The interpreter's tensors are f32 arrays; the matmul wants 16-bit operands.  These two kernels convert on the device
+// (the same rounding as h_f32_to_bf16 / h_f32_to_f16), so that a call costs no host loop over the elements.  For a
+// small call `in` / `out` are pinned host buffers read and written over the bus by the kernel itself, which saves the
+// two copy commands and their latency.
+__global__ __launch_bounds__(256) void stage_f32_to_16_kernel(const float *in, uint16_t *out, int64_t n, int f16) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const float f = in[i];
+    const uint32_t u = __builtin_bit_cast(uint32_t, f);
+    uint16_t h;
+    if ((u & 0x7fffffffu) > 0x7f800000u)
+      h = 0x7fff;
+    else if (f16)
+      h = __builtin_bit_cast(uint16_t, (_Float16)f);
+    else
+      h = (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+    out[i] = h;
+  }
+}
+__global__ __launch_bounds__(256) void expand_16_to_f32_kernel(const uint16_t *in, float *out, int64_t n, int f16) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const uint16_t h = in[i];
+    out[i] = f16 ? (float)__builtin_bit_cast(_Float16, h) : __builtin_bit_cast(float, (uint32_t)h << 16);
+  }
+}
+static unsigned stage_grid(int64_t n) {
+  int64_t b = (n + 255) / 256;
+  return (unsigned)(b > 4096 ? 4096 : b);
+}
+// calls with at most this many elements on a side go through the pinned buffers
+constexpr int64_t SMALL_CALL_ELEMS = 1 << 16;
+
 struct A16Handle {
   uint32_t magic = 0xA16A16u;
   mi_a16_weight *w = nullptr;
-  Pinned h_x, h_y;
-  DevBuf d_x, d_y;
+  Pinned h_x, h_y;             // small calls: f32 activations in, 16-bit results out, both touched by the kernels directly
+  DevBuf d_x, d_y, d_xf, d_yf; // 16-bit operands of the matmul; f32 staging of large calls
   hipStream_t stream = nullptr;
   ~A16Handle() {
     if (w) {
@@ -484,29 +515,46 @@ int mi_a16mm_inference(const mi_a16mm_attr *attr, mi_infer_param *p) {
   MI_REQUIRE(M >= 0, MI_BAD_ARGUMENT, "mi_a16mm_inference: negative M");
   if (M == 0)
     return MI_SUCCESS;
+  const int64_t nx = M * K, ny = M * N;
+  const bool small_in = nx <= SMALL_CALL_ELEMS, small_out = ny <= SMALL_CALL_ELEMS;
+  const int f16 = h->w->dtype == MI_DT_F16;
   int rc;
-  if ((rc = h->h_x.reserve((size_t)M * K * 2)) || (rc = h->h_y.reserve((size_t)M * N * 2)) ||
-      (rc = h->d_x.reserve((size_t)M * K * 2)) || (rc = h->d_y.reserve((size_t)M * N * 2)))
+  if ((rc = h->d_x.reserve((size_t)nx * 2)))
     return rc;
-  const float *x = p->inputs[0];
-  uint16_t *hx = (uint16_t *)h->h_x.ptr;
-  const bool f16 = h->w->dtype == MI_DT_F16;
-  for (int64_t i = 0; i < M * K; ++i)
-    hx[i] = f16 ? h_f32_to_f16(x[i]) : h_f32_to_bf16(x[i]);
-  MI_HIP(hipMemcpyAsync(h->d_x.ptr, hx, (size_t)M * K * 2, hipMemcpyHostToDevice, h->stream));
+  const float *src;
+  if (small_in) {
+    if ((rc = h->h_x.reserve((size_t)nx * 4)))
+      return rc;
+    memcpy(h->h_x.ptr, p->inputs[0], (size_t)nx * 4);
+    src = (const float *)h->h_x.ptr;
+  } else {
+    if ((rc = h->d_xf.reserve((size_t)nx * 4)))
+      return rc;
+    MI_HIP(hipMemcpyAsync(h->d_xf.ptr, p->inputs[0], (size_t)nx * 4, hipMemcpyHostToDevice, h->stream));
+    src = (const float *)h->d_xf.ptr;
+  }
+  stage_f32_to_16_kernel<<<dim3(stage_grid(nx)), dim3(256), 0, h->stream>>>(src, (uint16_t *)h->d_x.ptr, nx, f16);
+  if ((rc = small_out ? h->h_y.reserve((size_t)ny * 2) : h->d_y.reserve((size_t)ny * 2)))
+    return rc;
+  uint16_t *y16 = (uint16_t *)(small_out ? h->h_y.ptr : h->d_y.ptr);
   if (attr->dynamic_quant != MI_DQ_NONE)
-    rc = a16_dq_launch(h->w, attr->dynamic_quant, (const uint16_t *)h->d_x.ptr, M, (uint16_t *)h->d_y.ptr, nullptr,
-                       h->stream);
+    rc = a16_dq_launch(h->w, attr->dynamic_quant, (const uint16_t *)h->d_x.ptr, M, y16, nullptr, h->stream);
   else
-    rc = a16_launch(h->w, (const uint16_t *)h->d_x.ptr, M, (uint16_t *)h->d_y.ptr, nullptr, h->stream);
+    rc = a16_launch(h->w, (const uint16_t *)h->d_x.ptr, M, y16, nullptr, h->stream);
   if (rc != MI_SUCCESS)
     return rc;
-  MI_HIP(hipMemcpyAsync(h->h_y.ptr, h->d_y.ptr, (size_t)M * N * 2, hipMemcpyDeviceToHost, h->stream));
-  MI_HIP(hipStreamSynchronize(h->stream));
-  const uint16_t *hy = (const uint16_t *)h->h_y.ptr;
   float *y = p->outputs[0];
-  for (int64_t i = 0; i < M * N; ++i)
-    y[i] = f16 ? h_f16_to_f32(hy[i]) : h_bf16_to_f32(hy[i]);
+  if (small_out) {
+    MI_HIP(hipStreamSynchronize(h->stream));
+    for (int64_t i = 0; i < ny; ++i)
+      y[i] = f16 ? h_f16_to_f32(y16[i]) : h_bf16_to_f32(y16[i]);
+  } else {
+    if ((rc = h->d_yf.reserve((size_t)ny * 4)))
+      return rc;
+    expand_16_to_f32_kernel<<<dim3(stage_grid(ny)), dim3(256), 0, h->stream>>>(y16, (float *)h->d_yf.ptr, ny, f16);
+    MI_HIP(hipMemcpyAsync(y, h->d_yf.ptr, (size_t)ny * 4, hipMemcpyDeviceToHost, h->stream));
+    MI_HIP(hipStreamSynchronize(h->stream));
+  }
   return MI_SUCCESS;
 }
 
