@@ -302,6 +302,30 @@ int mi_i8mm_init(const mi_i8mm_attr *attr, mi_infer_param *p);
 int mi_i8mm_inference(const mi_i8mm_attr *attr, mi_infer_param *p);
 void mi_i8mm_deinit(mi_infer_param *p);
 
+/* Operands of any rank.  mi_matmul_parse_param replaces tpu::MatMulOp::parseParam (MatMul.cpp:24-135): the shapes of
+ * input, right and output (as module::getShape gives them) and the op's transpose attributes in; batch, batch_low, M,
+ * K, N out (the six cases of the comment at :17-22: 1-D operands, left batch dims folded into M when the right operand
+ * has none, batched right operands).  Returns MI_BAD_ARGUMENT for shapes the reference asserts on. */
+typedef struct mi_matmul_shapes {
+  int a_dims; int64_t a_shape[8];   /* getInput() */
+  int b_dims; int64_t b_shape[8];   /* getRight() */
+  int o_dims; int64_t o_shape[8];   /* getOutput() */
+  int left_transpose, output_transpose, hdim_is_batch;
+} mi_matmul_shapes;
+typedef struct mi_matmul_param {
+  int64_t batch, batch_low, M, K, N;
+  int right_transpose, left_transpose, output_transpose, hdim_is_batch;
+} mi_matmul_param;
+int mi_matmul_parse_param(const mi_matmul_shapes *shapes, int right_transpose, int chip /* MI_CHIP_* */,
+                          mi_matmul_param *out);
+/* mi_i8mm_inference with M, K, N and the batch taken from the shapes instead of attr (whose M, K, N are ignored):
+ * batch matmuls [batch, M, K] x [batch, K, N] (right stored [batch, N, K] under right_transpose) with one bias[N] and
+ * the requantization of the op (MatMul.cpp:598-729; on CV18xx multipliers[b] / rshifts[b] belong to batch b when one
+ * per batch is given, :638-664).  left_transpose, output_transpose and hdim_is_batch are MI_UNSUPPORTED, and so are
+ * operands that do not hold exactly batch matrices each (the reference's quantized path has no other broadcasting).
+ * p->handle is released by mi_i8mm_deinit. */
+int mi_i8mm_inference_nd(const mi_i8mm_attr *attr, const mi_matmul_shapes *shapes, mi_infer_param *p);
+
 /* ---- device level ---- */
 /* int32 -> narrow integer requantization applied per output channel n:
  *   MI_RQ_MULTIPLIER_SHIFT: v = RightShiftRound(acc * mult[n], shift[n], round_mode)      (MathUtils.cpp:541-546)
@@ -445,6 +469,33 @@ int mi_module_invoke(mi_module *m);
 int mi_module_uses_graph(const mi_module *m);
 /* float data out (expanded on the device), as py_cuda::get_tensor */
 int mi_module_get_tensor(mi_module *m, const char *name, float *out, int64_t num_elem);
+
+/* ============================================================================ */
+/* top.A16MatMul: the f32 twin of tpu.A16MatMul (the "top" stage the reference's   */
+/* differential tests compare the quantized op against)                            */
+/* ============================================================================ */
+typedef struct mi_top_a16mm_attr {
+  int64_t M;            /* product of the output's leading dims (Top/Interfaces/A16MatMul.cpp:61-64); may change per call */
+  int64_t K, N;
+  int weight_bits;      /* 4 or 8 */
+  int q_group_size;     /* < 1: one group per K elements (A16MatMul.cpp:88-91) */
+  int right_transpose;  /* 1 = weight stored [N, K] (4-bit: [N, K/2] bytes); 0 is MI_UNSUPPORTED */
+} mi_top_a16mm_attr;
+/* Replaces top::A16MatMulOp::inference (lib/Dialect/Top/Interfaces/A16MatMul.cpp:82-102), whose init and deinit are
+ * empty (:76-80): inputs = {input, weight, scale, zp, bias|NULL}, all f32 (weight: packed bytes 0..255 as floats);
+ * outputs[0] = input x dequant(weight)^T + bias in f32, nothing rounded.  Weights are dequantized as
+ * MatMul::dequant_weight does (lib/Support/Dnnl/MatMul.cpp:24-41: zero point truncated to int, scale in f32).  The
+ * first call uploads the weight operands and stores a handle in p->handle; later calls assume the same weights. */
+int mi_top_a16mm_inference(const mi_top_a16mm_attr *attr, mi_infer_param *p);
+void mi_top_a16mm_deinit(mi_infer_param *p);
+/* device level: weight = uint8 [N, K * bits / 8], scale / zp = float [N, G] (G = K / group), bias = float [N] or NULL,
+ * all HOST arrays; d_x float [M, K] (16-byte aligned), d_y float [M, N]; asynchronous on stream */
+typedef struct mi_top_a16_weight mi_top_a16_weight;
+int mi_top_a16_weight_create(mi_top_a16_weight **out, int64_t K, int64_t N, int weight_bits, int q_group_size,
+                             int right_transpose, const uint8_t *weight, const float *scale, const float *zp,
+                             const float *bias);
+void mi_top_a16_weight_destroy(mi_top_a16_weight *w);
+int mi_top_a16mm_launch(const mi_top_a16_weight *w, const float *d_x, int64_t M, float *d_y, void *stream);
 
 /* ============================================================================ */
 /* Measurement aid (no counterpart in the reference)                             */

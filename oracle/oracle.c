@@ -1567,3 +1567,184 @@ int orc_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qz
     }
   return 0;
 }
+
+/* ---- top.A16MatMul --------------------------------------------------------------------------------------------- */
+/* lib/Support/Dnnl/MatMul.cpp:24-41 */
+void orc_dequant_weight(float *dq_weight, const float *weight, const float *scale, const float *zp,
+                        int64_t weight_len, int q_group_size, int weight_bits) {
+  const int compress_ratio = 8 / weight_bits;
+  const int mask = weight_bits == 4 ? 0xF : 0xFF;
+  for (int64_t i = 0; i < weight_len; i += compress_ratio) {
+    const int64_t quant_idx = i / q_group_size;
+    const float zp_i = zp[quant_idx];
+    const float scale_i = scale[quant_idx];
+    for (int j = 0; j < compress_ratio; j++)
+      dq_weight[i + j] = (float)((((int)weight[i / compress_ratio] >> (weight_bits * j)) & mask) - (int)zp_i) * scale_i;
+  }
+}
+
+/* lib/Dialect/Top/Interfaces/A16MatMul.cpp:82-102; the matmul is MatMul::setup / run with right_transpose
+ * (lib/Support/Dnnl/MatMul.cpp:91-179), no zero points, no relu */
+int orc_top_a16matmul(const orc_top_a16mm_attr *a, const float *const *inputs, float *output) {
+  if (!a || !inputs || !inputs[0] || !inputs[1] || !inputs[2] || !inputs[3] || !output)
+    return 1;
+  if (a->weight_bits != 4 && a->weight_bits != 8)
+    return 1;
+  const int64_t M = a->M, K = a->K, N = a->N, weight_len = N * K;
+  int g = a->q_group_size;
+  if (g < 1)
+    g = (int)K;
+  float *w = (float *)malloc(sizeof(float) * (size_t)weight_len);
+  float *wt = NULL;
+  if (!w)
+    return 1;
+  orc_dequant_weight(w, inputs[1], inputs[2], inputs[3], weight_len, g, a->weight_bits);
+  const float *B = w;
+  if (a->right_transpose) {
+    wt = (float *)malloc(sizeof(float) * (size_t)weight_len);
+    if (!wt) {
+      free(w);
+      return 1;
+    }
+    orc_hw_transpose(wt, w, N, K);
+    B = wt;
+  }
+  run_gemm(a->gemm_kind, inputs[0], B, inputs[4], output, M, K, N);
+  free(w);
+  free(wt);
+  return 0;
+}
+
+/* ---- tpu.MatMul shapes ----------------------------------------------------------------------------------------- */
+/* lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:24-135 */
+int orc_matmul_parse_param(const int64_t *a_shape, int a_dims, const int64_t *b_shape, int b_dims,
+                           const int64_t *o_shape, int o_dims, int right_transpose, int left_transpose,
+                           int output_transpose, int hdim_is_batch, int chip, orc_matmul_param *p) {
+  int64_t a_s[10], b_s[10], o_s[10];
+  if (!a_shape || !b_shape || !o_shape || !p || a_dims < 1 || b_dims < 1 || o_dims < 0 || a_dims > 8 || b_dims > 8 ||
+      o_dims > 8)
+    return 1;
+  memcpy(a_s, a_shape, sizeof(int64_t) * (size_t)a_dims);
+  memcpy(b_s, b_shape, sizeof(int64_t) * (size_t)b_dims);
+  memcpy(o_s, o_shape, sizeof(int64_t) * (size_t)o_dims);
+  memset(p, 0, sizeof(*p));
+  p->right_transpose = right_transpose;
+  p->left_transpose = left_transpose;
+  p->output_transpose = output_transpose;
+  p->hdim_is_batch = hdim_is_batch;
+  p->batch = 1;
+  p->batch_low = 1;
+  if (b_dims == 1) { /* :44-50 */
+    if (right_transpose)
+      return 1;
+    b_s[b_dims++] = 1;
+    o_s[o_dims++] = 1;
+  }
+  if (a_dims == 1) { /* :51-57 */
+    if (left_transpose)
+      return 1;
+    memmove(a_s + 1, a_s, sizeof(int64_t) * (size_t)a_dims);
+    a_s[0] = 1;
+    memmove(o_s + 1, o_s, sizeof(int64_t) * (size_t)o_dims);
+    o_s[0] = 1;
+    a_dims++;
+    o_dims++;
+  }
+  if (o_dims < 2 || (hdim_is_batch && (a_dims < 3 || b_dims < 3 || o_dims < 3)))
+    return 1;
+  if (right_transpose) { /* :63-79 */
+    if (hdim_is_batch) {
+      p->K = b_s[b_dims - 3];
+      p->N = b_s[b_dims - 1];
+      if (chip == 0) {
+        p->N = b_s[b_dims - 3];
+        p->K = b_s[b_dims - 1];
+      }
+    } else {
+      p->N = b_s[b_dims - 2];
+      p->K = b_s[b_dims - 1];
+    }
+  } else {
+    p->N = b_s[b_dims - 1];
+    p->K = b_s[b_dims - 2];
+  }
+  if (left_transpose) /* :81-90 */
+    p->M = hdim_is_batch ? a_s[a_dims - 3] : a_s[a_dims - 1];
+  else
+    p->M = a_s[a_dims - 2];
+  for (int i = 0; i < o_dims - 2; i++) /* :92-94 */
+    p->batch *= o_s[i];
+  if (hdim_is_batch) { /* :96-104 */
+    p->batch = o_s[0];
+    if (!output_transpose && chip == 1) {
+      p->batch_low = o_s[1];
+    } else {
+      p->batch_low = o_s[2];
+      p->output_transpose = 1;
+    }
+  } else { /* :105-133 */
+    int64_t right_batch = 1;
+    for (int i = 0; i < b_dims - 2; i++)
+      right_batch *= b_s[i];
+    if (right_batch != p->batch && right_batch == 1)
+      p->batch = 1;
+    if (p->batch > 1 || o_dims <= 2) {
+      p->M = output_transpose ? o_s[o_dims - 1] : o_s[o_dims - 2];
+    } else {
+      p->M = 1;
+      for (int i = 0; i < o_dims - 1; i++)
+        p->M *= o_s[i];
+    }
+    int64_t b_temp = 1;
+    for (int i = 1; i < b_dims - 2; i++)
+      b_temp *= b_s[i];
+    if (a_s[0] == b_s[0] && b_temp == 1 && b_dims > 2) {
+      p->batch = b_s[0];
+      int64_t a_temp = 1;
+      for (int i = 1; i < a_dims - 2; i++)
+        a_temp *= a_s[i];
+      p->M = a_s[o_dims - 2 + left_transpose] * a_temp;
+    }
+  }
+  return 0;
+}
+
+int orc_matmul_int8_nd(const orc_i8mm_attr *attr, const int64_t *a_shape, int a_dims, const int64_t *b_shape,
+                       int b_dims, const int64_t *o_shape, int o_dims, int chip, const float *const *inputs,
+                       float *output) {
+  orc_matmul_param p;
+  if (!attr || !inputs || !output)
+    return 1;
+  if (orc_matmul_parse_param(a_shape, a_dims, b_shape, b_dims, o_shape, o_dims, attr->right_transpose, 0, 0, 0, chip, &p))
+    return 1;
+  const int64_t full_batch = p.batch * p.batch_low;
+  /* the operands must hold exactly batch matrices each: the reference's quantized path passes no shapes to
+   * MatMul::setup, so it has no broadcasting beyond what parseParam folded into M */
+  int64_t a_num = 1, b_num = 1;
+  for (int i = 0; i < a_dims; i++)
+    a_num *= a_shape[i];
+  for (int i = 0; i < b_dims; i++)
+    b_num *= b_shape[i];
+  if (a_num != full_batch * p.M * p.K || b_num != full_batch * p.K * p.N)
+    return 1;
+  for (int64_t b = 0; b < full_batch; b++) {
+    orc_i8mm_attr one = *attr;
+    one.M = p.M;
+    one.K = p.K;
+    one.N = p.N;
+    int64_t mult_b, rs_b;
+    if (attr->is_cv18xx && attr->n_multipliers == full_batch && attr->n_rshifts == full_batch && full_batch > 1) {
+      /* MatMul.cpp:645-663: one multiplier / rshift per batch when the right operand is a weight */
+      mult_b = attr->multipliers[b];
+      rs_b = attr->rshifts[b];
+      one.multipliers = &mult_b;
+      one.n_multipliers = 1;
+      one.rshifts = &rs_b;
+      one.n_rshifts = 1;
+    }
+    const float *ins[4] = {inputs[0] + b * p.M * p.K, inputs[1] + b * p.K * p.N, inputs[2], inputs[3]};
+    if (orc_matmul_int8(&one, ins, output + b * p.M * p.N, NULL))
+      return 1;
+  }
+  return 0;
+}

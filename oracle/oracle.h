@@ -52,6 +52,15 @@
  *                                orc_a16matmul results (tests/test_oracle_packers.py)
  *   orc_llm_unpack               inverse of independently written GPTQ / AWQ packers, AutoAWQ's published pack
  *                                order (tests/test_oracle_packers.py)
+ *   orc_dequant_weight, orc_top_a16matmul   hand-computed known answers; equal to orc_a16_dequant (the tpu-dialect
+ *                                restatement of a different reference function) on integer zero points; truncation
+ *                                of fractional zero points; f64 product of independently unpacked operands
+ *                                (tests/test_oracle_top_a16.py)
+ *   orc_matmul_parse_param       the six cases the reference documents above the function (MatMul.cpp:17-22) and
+ *                                numpy.matmul's broadcasting shapes (tests/test_oracle_matmul_nd.py); the
+ *                                hdim_is_batch branch only as far as the layout comment at :58-62 goes: its K / N
+ *                                without right_transpose are PARITY UNPINNED
+ *   orc_matmul_int8_nd           numpy.matmul on int64 per batch + the pinned scalar requantization
  *   orc_a16_dequant              one-hot activations recover nibble order,
  *                                group indexing and scale layout
  *   orc_sgemm_*                  float64 reference with the standard bound
@@ -322,6 +331,42 @@ int orc_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qz
 /* A16MatMulToGroup (Canonicalize/A16MatMul.cpp:432-499): per-channel scale / zp entries repeated K / 128 times. */
 int orc_a16_to_group(const uint16_t *scale, int64_t scale_num, const uint8_t *zp, int64_t zp_num, int64_t K,
                      uint16_t *scale_out, uint8_t *zp_out);
+
+/* ---- top.A16MatMul: the f32 twin of tpu.A16MatMul ------------------------- */
+/* MatMul::dequant_weight, lib/Support/Dnnl/MatMul.cpp:24-41: weight is f32-valued (packed bytes 0..255 for 4 bits,
+ * weight_len / 2 entries; one value per element for 8 bits); quantization groups are runs of q_group_size
+ * consecutive elements of the FLATTENED weight; the zero point is truncated to int; nothing is rounded. */
+void orc_dequant_weight(float *dq_weight, const float *weight, const float *scale, const float *zp,
+                        int64_t weight_len, int q_group_size, int weight_bits);
+typedef struct {
+  int64_t M, K, N;
+  int weight_bits;      /* 4 or 8 */
+  int q_group_size;     /* < 1: one group per K elements (A16MatMul.cpp:88-91) */
+  int right_transpose;  /* 1: weight stored [N, K(/2)] */
+  int gemm_kind;
+} orc_top_a16mm_attr;
+/* top::A16MatMulOp::inference, lib/Dialect/Top/Interfaces/A16MatMul.cpp:82-102: inputs[0..4] = input, weight, scale,
+ * zp, bias (NULL ok); f32 in, f32 out, no rounding anywhere.  Returns 0 on success. */
+int orc_top_a16matmul(const orc_top_a16mm_attr *attr, const float *const *inputs, float *output);
+
+/* ---- tpu.MatMul: shapes -> batch, M, K, N --------------------------------- */
+typedef struct {
+  int64_t batch, batch_low, M, K, N;
+  int right_transpose, left_transpose, output_transpose, hdim_is_batch;
+} orc_matmul_param;
+/* tpu::MatMulOp::parseParam, lib/Dialect/Tpu/Interfaces/Common/MatMul.cpp:24-135 (the six cases its comment lists,
+ * :17-22, are the known answers).  chip: 0 = BM1684X / BM1690 family, 1 = CV18xx, 2 = any other.  Returns 0, or 1 for
+ * shapes the reference asserts on (a 1-D right operand with right_transpose, a 1-D left with left_transpose). */
+int orc_matmul_parse_param(const int64_t *a_shape, int a_dims, const int64_t *b_shape, int b_dims,
+                           const int64_t *o_shape, int o_dims, int right_transpose, int left_transpose,
+                           int output_transpose, int hdim_is_batch, int chip, orc_matmul_param *out);
+/* tpu.MatMul (quantized) on operands of any rank the plain branch of parseParam covers (no hdim_is_batch, no left or
+ * output transpose): batch matmuls [batch, M, K] x [batch, K, N] (right stored [batch, N, K] under right_transpose),
+ * one bias[N] for all, then the requantization of orc_matmul_int8 over the whole output; on CV18xx the multiplier /
+ * rshift of batch b when one per batch is given (MatMul.cpp:638-664).  attr->M/K/N are ignored. */
+int orc_matmul_int8_nd(const orc_i8mm_attr *attr, const int64_t *a_shape, int a_dims, const int64_t *b_shape,
+                       int b_dims, const int64_t *o_shape, int o_dims, int chip, const float *const *inputs,
+                       float *output);
 
 #ifdef __cplusplus
 }

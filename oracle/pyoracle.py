@@ -491,3 +491,84 @@ def llm_unpack(mode, bits, qweight, qzeros, K, N):
 
 def num_threads():
     return lib().orc_num_threads()
+
+
+class TopA16Attr(C.Structure):
+    _fields_ = [("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64), ("weight_bits", C.c_int),
+                ("q_group_size", C.c_int), ("right_transpose", C.c_int), ("gemm_kind", C.c_int)]
+
+
+class MatMulParam(C.Structure):
+    _fields_ = [("batch", C.c_int64), ("batch_low", C.c_int64), ("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64),
+                ("right_transpose", C.c_int), ("left_transpose", C.c_int), ("output_transpose", C.c_int),
+                ("hdim_is_batch", C.c_int)]
+
+
+CHIP_BM1684X, CHIP_CV18XX, CHIP_OTHER = 0, 1, 2
+
+
+def dequant_weight(weight, scale, zp, *, weight_len, q_group_size, weight_bits):
+    """MatMul::dequant_weight of the top dialect: f32-valued packed weight -> f32 weights, flat."""
+    weight, scale, zp = _f32(weight), _f32(scale), _f32(zp)
+    out = np.zeros(weight_len, dtype=np.float32)
+    L = lib()
+    L.orc_dequant_weight.restype = None
+    L.orc_dequant_weight(_p(out, C.c_float), _p(weight, C.c_float), _p(scale, C.c_float), _p(zp, C.c_float),
+                         C.c_int64(weight_len), C.c_int(q_group_size), C.c_int(weight_bits))
+    return out
+
+
+def top_a16matmul(x, weight, scale, zp, bias, *, M, K, N, weight_bits, q_group_size, right_transpose=True,
+                  gemm_kind=GEMM_F64ACC):
+    """top.A16MatMul on f32 operands; returns the f32 output (nothing is rounded)."""
+    ins = [_f32(x), _f32(weight), _f32(scale), _f32(zp), _f32(bias)]
+    attr = TopA16Attr(M, K, N, weight_bits, q_group_size, int(right_transpose), gemm_kind)
+    arr = (C.POINTER(C.c_float) * 5)(*[None if a is None else _p(a, C.c_float) for a in ins])
+    out = np.empty((M, N), dtype=np.float32)
+    L = lib()
+    L.orc_top_a16matmul.restype = C.c_int
+    if L.orc_top_a16matmul(C.byref(attr), arr, _p(out, C.c_float)) != 0:
+        raise RuntimeError("orc_top_a16matmul failed")
+    return out
+
+
+def _shape_arr(shape):
+    return (C.c_int64 * max(1, len(shape)))(*[int(v) for v in shape])
+
+
+def matmul_parse_param(a_shape, b_shape, o_shape, *, right_transpose=False, left_transpose=False,
+                       output_transpose=False, hdim_is_batch=False, chip=CHIP_BM1684X):
+    """tpu::MatMulOp::parseParam: dict with batch, batch_low, M, K, N and the (possibly rewritten) flags."""
+    p = MatMulParam()
+    L = lib()
+    L.orc_matmul_parse_param.restype = C.c_int
+    rc = L.orc_matmul_parse_param(_shape_arr(a_shape), C.c_int(len(a_shape)), _shape_arr(b_shape), C.c_int(len(b_shape)),
+                                  _shape_arr(o_shape), C.c_int(len(o_shape)), C.c_int(int(right_transpose)),
+                                  C.c_int(int(left_transpose)), C.c_int(int(output_transpose)),
+                                  C.c_int(int(hdim_is_batch)), C.c_int(chip), C.byref(p))
+    if rc != 0:
+        raise ValueError("orc_matmul_parse_param: shapes the reference asserts on")
+    return {k: int(getattr(p, k)) for k, _ in MatMulParam._fields_}
+
+
+def matmul_int8_nd(x, right, bias, multi, *, out_shape, right_transpose=False, input_zp=0, right_zp=0, do_relu=False,
+                   relu_limit=-1.0, cv18xx=False, quant_mode=RQ_MULTIPLIER_SHIFT, fuse_rq=False, multipliers=(1,),
+                   rshifts=(0,), out_zp=0, out_kind=0, out_bits=8, out_unsigned=False, gemm_kind=GEMM_F32):
+    """Quantised tpu.MatMul on operands of any rank (plain branch of parseParam); returns the output, shaped out_shape."""
+    x, right = _f32(x), _f32(right)
+    ins = [x, right, _f32(bias), _f32(multi)]
+    mult = np.ascontiguousarray(multipliers, dtype=np.int64)
+    rs = np.ascontiguousarray(rshifts, dtype=np.int64)
+    attr = I8Attr(0, 0, 0, int(right_transpose), input_zp, right_zp, int(do_relu), relu_limit, int(cv18xx),
+                  quant_mode, int(fuse_rq), _p(mult, C.c_int64), mult.size, _p(rs, C.c_int64), rs.size,
+                  out_zp, out_kind, out_bits, int(out_unsigned), gemm_kind)
+    arr = (C.POINTER(C.c_float) * 4)(*[None if a is None else _p(a, C.c_float) for a in ins])
+    out = np.empty(tuple(out_shape), dtype=np.float32)
+    L = lib()
+    L.orc_matmul_int8_nd.restype = C.c_int
+    rc = L.orc_matmul_int8_nd(C.byref(attr), _shape_arr(x.shape), C.c_int(x.ndim), _shape_arr(right.shape),
+                              C.c_int(right.ndim), _shape_arr(out_shape), C.c_int(len(out_shape)),
+                              C.c_int(CHIP_CV18XX if cv18xx else CHIP_BM1684X), arr, _p(out, C.c_float))
+    if rc != 0:
+        raise RuntimeError("orc_matmul_int8_nd failed")
+    return out

@@ -1,0 +1,118 @@
+"""GPU parity of the two ops either side of the hot path's core: top.A16MatMul (the f32 twin, lib/Dialect/Top/
+Interfaces/A16MatMul.cpp:82-102) and tpu.MatMul on operands of any rank (parseParam, lib/Dialect/Tpu/Interfaces/Common/
+MatMul.cpp:24-135), against the oracle."""
+import numpy as np
+import pytest
+
+from helpers import pkg
+
+pytestmark = pytest.mark.gpu
+S = pkg("synth")
+
+
+def _top_operands(bits, M, K, N, g, seed):
+    rng = np.random.default_rng(seed)
+    cfg = S.w4a16(M, K, N, g, seed=seed) if bits == 4 else S.w8a16(M, K, N, g, seed=seed, signed=False)
+    G = K // g if g else 1
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    scale = (np.abs(rng.standard_normal((N, G))) * 0.01 + 1e-4).astype(np.float32)
+    zp = cfg["zp"].astype(np.float32) + np.float32(0.7)          # fractional: (int) truncates it
+    bias = rng.standard_normal(N).astype(np.float32)
+    return cfg, x, scale, zp, bias
+
+
+# fp32 FMA accumulation over K terms against the oracle's float64 accumulation: K * 2^-24 relative to the row's
+# magnitude bounds the difference; 2e-5 of the output RMS leaves a factor of ten at K = 4096
+TOP_TOL = 2e-5
+
+
+@pytest.mark.parametrize("bits,M,K,N,g", [(4, 1, 4096, 4096, 128), (4, 5, 2048, 1000, 64), (4, 3, 512, 48, 0),
+                                          (8, 1, 4096, 1024, 0), (8, 6, 1024, 130, 128)])
+def test_top_a16matmul_operator_against_oracle(orc, bits, M, K, N, g):
+    m = pkg()
+    cfg, x, scale, zp, bias = _top_operands(bits, M, K, N, g, seed=bits + M)
+    w = cfg["weight"].astype(np.float32)
+    ref = orc.top_a16matmul(x, w, scale, zp, bias, M=M, K=K, N=N, weight_bits=bits, q_group_size=g)
+    op = m.TopA16MatMul(K=K, N=N, weight_bits=bits, q_group_size=g)
+    y = op.inference(x, w, scale, zp, bias)
+    y2 = op.inference(x[:1], w, scale, zp, bias)               # second call, fewer rows, cached weights
+    op.deinit()
+    rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+    err = float(np.max(np.abs(y.astype(np.float64) - ref)))
+    print("top.A16MatMul bits=%d M=%d K=%d N=%d g=%d: max-abs/RMS %.2e" % (bits, M, K, N, g, err / rms))
+    assert err <= TOP_TOL * rms
+    assert np.max(np.abs(y2.astype(np.float64) - ref[:1])) <= TOP_TOL * rms
+
+
+def test_top_a16matmul_one_hot_is_exact_and_unrounded(orc):
+    import torch
+    m = pkg()
+    K, N, g = 256, 40, 32
+    cfg, _, _, zp, _ = _top_operands(4, 1, K, N, g, seed=9)
+    scale = np.full((N, K // g), np.float32(1.0) / 3, dtype=np.float32)
+    w = m.TopA16Weight(cfg["weight"], scale, zp, None, K=K, N=N, weight_bits=4, q_group_size=g)
+    x = torch.eye(K, dtype=torch.float32, device="cuda")
+    y = m.top_a16mm_launch(w, x)
+    torch.cuda.synchronize()
+    expect = orc.dequant_weight(cfg["weight"].astype(np.float32), scale, zp, weight_len=N * K, q_group_size=g,
+                                weight_bits=4).reshape(N, K).T
+    assert np.array_equal(y.cpu().numpy(), expect)              # single products: bit-exact
+    w.destroy()
+
+
+def test_top_a16matmul_refuses_what_it_does_not_handle():
+    m = pkg()
+    clib = pkg("clib")
+    cfg, x, scale, zp, bias = _top_operands(4, 1, 64, 8, 0, seed=2)
+    with pytest.raises(clib.BackendError) as e:
+        m.TopA16MatMul(K=64, N=8, weight_bits=4, q_group_size=0, right_transpose=False).inference(
+            x, cfg["weight"].astype(np.float32), scale, zp, bias)
+    assert e.value.code == clib.MI_UNSUPPORTED
+
+
+@pytest.mark.parametrize("a,b,rt", [((3, 64, 128), (3, 128, 96), False), ((2, 2, 33, 64), (2, 2, 40, 64), True),
+                                    ((3, 20, 128), (128, 64), False), ((64,), (64, 48), False)])
+def test_matmul_int8_nd_against_oracle(orc, a, b, rt):
+    m = pkg()
+    clib = pkg("clib")
+    rng = np.random.default_rng(sum(a) * 3 + sum(b))
+    A = rng.integers(-128, 128, size=a).astype(np.float32)
+    B = rng.integers(-128, 128, size=b).astype(np.float32)
+    N = b[-2] if rt else b[-1]
+    bias = rng.integers(-5000, 5000, size=N).astype(np.float32)
+    multi = rng.integers(1000, 10000, size=N).astype(np.float32)
+    op = m.MatMulInt8(K=a[-1], N=N, right_transpose=rt, quant_mode=clib.RQ_MULTIPLIER_SHIFT, fuse_rq=True,
+                      multipliers=(1,), rshifts=(20,), out_zp=-3)
+    y = op.inference_nd(A, B, bias, multi)
+    y_again = op.inference_nd(A, B, bias, multi)                # cached right operand
+    op.deinit()
+    ref = orc.matmul_int8_nd(A, B, bias, multi, out_shape=y.shape, right_transpose=rt,
+                             quant_mode=orc.RQ_MULTIPLIER_SHIFT, fuse_rq=True, multipliers=(1,), rshifts=(20,), out_zp=-3)
+    assert np.array_equal(y, ref) and np.array_equal(y_again, ref)
+
+
+def test_matmul_int8_nd_cv18xx_per_batch_requant(orc):
+    m = pkg()
+    clib = pkg("clib")
+    rng = np.random.default_rng(8)
+    A = rng.integers(-128, 128, size=(3, 16, 64)).astype(np.float32)
+    B = rng.integers(-128, 128, size=(3, 64, 32)).astype(np.float32)
+    mult, rs = (1 << 30, 3 << 29, 5 << 28), (9, 10, 11)
+    op = m.MatMulInt8(K=64, N=32, chip=clib.CHIP_CV18XX, quant_mode=clib.RQ_QDM, multipliers=mult, rshifts=rs)
+    y = op.inference_nd(A, B)
+    op.deinit()
+    ref = orc.matmul_int8_nd(A, B, None, None, out_shape=y.shape, cv18xx=True, quant_mode=orc.RQ_QDM, multipliers=mult,
+                             rshifts=rs)
+    assert np.array_equal(y, ref)
+
+
+def test_matmul_int8_nd_refuses_broadcast_batches_and_transposes():
+    m = pkg()
+    clib = pkg("clib")
+    op = m.MatMulInt8(K=8, N=4, multipliers=(1,), rshifts=(0,))
+    A = np.zeros((3, 2, 5, 8), dtype=np.float32)
+    B = np.zeros((2, 8, 4), dtype=np.float32)                    # right batch 2 against output batch 6
+    with pytest.raises(clib.BackendError) as e:
+        op.inference_nd(A, B)
+    assert e.value.code == clib.MI_UNSUPPORTED
+    op.deinit()

@@ -23,12 +23,15 @@ EXPORTS = [
     "mi_matmul_dq_inference", "mi_f8mm_inference", "mi_f8mm_launch", "mi_f8mm_e5m2_launch",
     "mi_a16_weight_export_size", "mi_a16_weight_export", "mi_a16_weight_import", "mi_a16_quantize", "mi_llm_unpack",
     "mi_a16_to_group",
-    "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch",
+    "mi_i8mm_init", "mi_i8mm_inference", "mi_i8mm_deinit", "mi_i8mm_launch", "mi_matmul_parse_param",
+    "mi_i8mm_inference_nd",
     "mi_requant_int_axis_inference", "mi_requant_int_inference", "mi_requant_launch",
     "mi_cast_inference", "mi_cast_launch",
     "mi_module_create", "mi_module_destroy", "mi_module_add_tensor", "mi_module_add_a16matmul", "mi_module_add_a16matmul_dq",
     "mi_module_add_matmul_int8", "mi_module_add_requant", "mi_module_add_matmul_dq", "mi_module_add_cast", "mi_module_set_tensor", "mi_module_invoke",
     "mi_module_uses_graph", "mi_module_get_tensor",
+    "mi_top_a16mm_inference", "mi_top_a16mm_deinit", "mi_top_a16_weight_create", "mi_top_a16_weight_destroy",
+    "mi_top_a16mm_launch",
     "mi_bench_read_launch",
 ]
 
@@ -52,6 +55,23 @@ class A16Attr(C.Structure):
     _fields_ = [("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64), ("weight_bits", C.c_int),
                 ("w_transpose", C.c_int), ("q_group_size", C.c_int), ("out_dtype", C.c_int), ("chip", C.c_int),
                 ("dynamic_quant", C.c_int)]
+
+
+class TopA16Attr(C.Structure):
+    _fields_ = [("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64), ("weight_bits", C.c_int),
+                ("q_group_size", C.c_int), ("right_transpose", C.c_int)]
+
+
+class MatMulShapes(C.Structure):
+    _fields_ = [("a_dims", C.c_int), ("a_shape", C.c_int64 * 8), ("b_dims", C.c_int), ("b_shape", C.c_int64 * 8),
+                ("o_dims", C.c_int), ("o_shape", C.c_int64 * 8), ("left_transpose", C.c_int),
+                ("output_transpose", C.c_int), ("hdim_is_batch", C.c_int)]
+
+
+class MatMulParam(C.Structure):
+    _fields_ = [("batch", C.c_int64), ("batch_low", C.c_int64), ("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64),
+                ("right_transpose", C.c_int), ("left_transpose", C.c_int), ("output_transpose", C.c_int),
+                ("hdim_is_batch", C.c_int)]
 
 
 class A16WeightDesc(C.Structure):
@@ -169,6 +189,12 @@ def lib():
         L.mi_a16_weight_destroy.restype = None
         L.mi_a16mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_launch_noalloc.argtypes = L.mi_a16mm_launch.argtypes
+        L.mi_top_a16_weight_create.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                               C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi_top_a16_weight_destroy.argtypes = [C.c_void_p]
+        L.mi_top_a16_weight_destroy.restype = None
+        L.mi_top_a16mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
+        L.mi_top_a16mm_deinit.restype = None
         L.mi_matmul_dq_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int,
                                           C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_dq_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]

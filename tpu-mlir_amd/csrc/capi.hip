@@ -831,13 +831,159 @@ int mi_i8mm_inference(const mi_i8mm_attr *attr, mi_infer_param *p) {
   return MI_SUCCESS;
 }
 
+// one operator handle per batch (each caches its own right operand when that is a weight)
+struct I8BatchHandle {
+  uint32_t magic = 0x18B18B18u;
+  std::vector<void *> per_batch;
+};
+
 void mi_i8mm_deinit(mi_infer_param *p) {
   if (!p || !p->handle)
     return;
   I8Handle *h = (I8Handle *)p->handle;
-  if (h->magic == 0x18181818u)
+  if (h->magic == 0x18181818u) {
     delete h;
+  } else if (h->magic == 0x18B18B18u) {
+    I8BatchHandle *bh = (I8BatchHandle *)p->handle;
+    for (void *one : bh->per_batch)
+      if (one && ((I8Handle *)one)->magic == 0x18181818u)
+        delete (I8Handle *)one;
+    delete bh;
+  }
   p->handle = nullptr;
+}
+
+int mi_matmul_parse_param(const mi_matmul_shapes *sh, int right_transpose, int chip, mi_matmul_param *out) {
+  MI_REQUIRE(sh && out, MI_BAD_ARGUMENT, "mi_matmul_parse_param: null argument");
+  MI_REQUIRE(sh->a_dims >= 1 && sh->a_dims <= 8 && sh->b_dims >= 1 && sh->b_dims <= 8 && sh->o_dims >= 0 && sh->o_dims <= 8,
+             MI_BAD_ARGUMENT, "mi_matmul_parse_param: ranks must be 1 .. 8");
+  std::vector<int64_t> a(sh->a_shape, sh->a_shape + sh->a_dims), b(sh->b_shape, sh->b_shape + sh->b_dims),
+      o(sh->o_shape, sh->o_shape + sh->o_dims);
+  mi_matmul_param p;
+  memset(&p, 0, sizeof(p));
+  p.right_transpose = right_transpose;
+  p.left_transpose = sh->left_transpose;
+  p.output_transpose = sh->output_transpose;
+  p.hdim_is_batch = sh->hdim_is_batch;
+  p.batch = p.batch_low = 1;
+  if (b.size() == 1) {  // a vector on the right is a one-column matrix (MatMul.cpp:44-50)
+    MI_REQUIRE(!right_transpose, MI_BAD_ARGUMENT, "mi_matmul_parse_param: 1-D right operand with right_transpose");
+    b.push_back(1);
+    o.push_back(1);
+  }
+  if (a.size() == 1) {  // a vector on the left is a one-row matrix (:51-57)
+    MI_REQUIRE(!sh->left_transpose, MI_BAD_ARGUMENT, "mi_matmul_parse_param: 1-D left operand with left_transpose");
+    a.insert(a.begin(), 1);
+    o.insert(o.begin(), 1);
+  }
+  const size_t ad = a.size(), bd = b.size(), od = o.size();
+  MI_REQUIRE(od >= 2 && (!p.hdim_is_batch || (ad >= 3 && bd >= 3 && od >= 3)), MI_BAD_ARGUMENT,
+             "mi_matmul_parse_param: output rank too small for these operands");
+  const bool bm1684x = chip == MI_CHIP_BM168X;
+  if (right_transpose && p.hdim_is_batch) {  // :63-72
+    p.K = bm1684x ? b[bd - 1] : b[bd - 3];
+    p.N = bm1684x ? b[bd - 3] : b[bd - 1];
+  } else {
+    p.N = right_transpose ? b[bd - 2] : b[bd - 1];
+    p.K = right_transpose ? b[bd - 1] : b[bd - 2];
+  }
+  p.M = sh->left_transpose ? (p.hdim_is_batch ? a[ad - 3] : a[ad - 1]) : a[ad - 2];  // :81-90
+  for (size_t i = 0; i + 2 < od; ++i)
+    p.batch *= o[i];
+  if (p.hdim_is_batch) {  // :96-104
+    p.batch = o[0];
+    if (!sh->output_transpose && chip == MI_CHIP_CV18XX) {
+      p.batch_low = o[1];
+    } else {
+      p.batch_low = o[2];
+      p.output_transpose = 1;
+    }
+  } else {  // :105-133
+    int64_t right_batch = 1;
+    for (size_t i = 0; i + 2 < bd; ++i)
+      right_batch *= b[i];
+    if (right_batch != p.batch && right_batch == 1)
+      p.batch = 1;  // a right operand without batch dims: the left batch dims become rows
+    if (p.batch > 1 || od <= 2) {
+      p.M = sh->output_transpose ? o[od - 1] : o[od - 2];
+    } else {
+      p.M = 1;
+      for (size_t i = 0; i + 1 < od; ++i)
+        p.M *= o[i];
+    }
+    int64_t b_inner = 1;
+    for (size_t i = 1; i + 2 < bd; ++i)
+      b_inner *= b[i];
+    if (a[0] == b[0] && b_inner == 1 && bd > 2) {
+      p.batch = b[0];
+      int64_t a_inner = 1;
+      for (size_t i = 1; i + 2 < ad; ++i)
+        a_inner *= a[i];
+      const size_t idx = od - 2 + (sh->left_transpose ? 1 : 0);
+      MI_REQUIRE(idx < ad, MI_BAD_ARGUMENT, "mi_matmul_parse_param: left rank too small for the output");
+      p.M = a[idx] * a_inner;
+    }
+  }
+  *out = p;
+  return MI_SUCCESS;
+}
+
+int mi_i8mm_inference_nd(const mi_i8mm_attr *attr, const mi_matmul_shapes *shapes, mi_infer_param *p) {
+  MI_REQUIRE(attr && shapes && p, MI_BAD_ARGUMENT, "mi_i8mm_inference_nd: null argument");
+  MI_REQUIRE(!shapes->left_transpose && !shapes->output_transpose && !shapes->hdim_is_batch, MI_UNSUPPORTED,
+             "mi_i8mm_inference_nd: left_transpose, output_transpose and hdim_is_batch are not handled");
+  mi_matmul_param mp;
+  int rc = mi_matmul_parse_param(shapes, attr->right_transpose, attr->chip, &mp);
+  if (rc)
+    return rc;
+  const int64_t batch = mp.batch * mp.batch_low;
+  int64_t a_num = 1, b_num = 1;
+  for (int i = 0; i < shapes->a_dims; ++i)
+    a_num *= shapes->a_shape[i];
+  for (int i = 0; i < shapes->b_dims; ++i)
+    b_num *= shapes->b_shape[i];
+  MI_REQUIRE(a_num == batch * mp.M * mp.K && b_num == batch * mp.K * mp.N, MI_UNSUPPORTED,
+             "mi_i8mm_inference_nd: the operands do not hold exactly one matrix per batch (broadcast batches are not "
+             "handled)");
+  MI_REQUIRE(p->inputs && p->n_inputs >= 2 && p->inputs[0] && p->inputs[1] && p->outputs && p->n_outputs >= 1 &&
+                 p->outputs[0],
+             MI_BAD_ARGUMENT, "mi_i8mm_inference_nd: null input or output");
+  I8BatchHandle *bh = (I8BatchHandle *)p->handle;
+  if (!bh) {
+    bh = new I8BatchHandle;
+    bh->per_batch.assign((size_t)batch, nullptr);
+    p->handle = bh;
+  }
+  MI_REQUIRE(bh->magic == 0x18B18B18u && (int64_t)bh->per_batch.size() == batch, MI_BAD_ARGUMENT,
+             "mi_i8mm_inference_nd: the handle belongs to another op or another batch size");
+  const bool per_batch_q = attr->chip == MI_CHIP_CV18XX && batch > 1 && attr->n_multipliers == batch &&
+                           attr->n_rshifts == batch;
+  for (int64_t b = 0; b < batch; ++b) {
+    mi_i8mm_attr one = *attr;
+    one.M = mp.M;
+    one.K = mp.K;
+    one.N = mp.N;
+    if (per_batch_q) {
+      one.multipliers = attr->multipliers + b;
+      one.n_multipliers = 1;
+      one.rshifts = attr->rshifts + b;
+      one.n_rshifts = 1;
+    }
+    const float *ins[5] = {p->inputs[0] + b * mp.M * mp.K, p->inputs[1] + b * mp.K * mp.N,
+                           p->n_inputs > 2 ? p->inputs[2] : nullptr, p->n_inputs > 3 ? p->inputs[3] : nullptr, nullptr};
+    float *outs[1] = {p->outputs[0] + b * mp.M * mp.N};
+    mi_infer_param sub;
+    sub.inputs = (float **)ins;
+    sub.n_inputs = 5;
+    sub.outputs = outs;
+    sub.n_outputs = 1;
+    sub.handle = bh->per_batch[(size_t)b];
+    rc = mi_i8mm_inference(&one, &sub);
+    bh->per_batch[(size_t)b] = sub.handle;
+    if (rc)
+      return rc;
+  }
+  return MI_SUCCESS;
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -80,6 +80,100 @@ class A16MatMul:
             pass
 
 
+class TopA16MatMul:
+    """top.A16MatMul, the f32 twin of tpu.A16MatMul (f32 in, f32 out, nothing rounded).  The reference's init and
+    deinit are empty; here the first inference uploads the weight operands and deinit frees them."""
+
+    def __init__(self, K, N, weight_bits, q_group_size, right_transpose=True):
+        self.attr = clib.TopA16Attr(0, K, N, weight_bits, q_group_size, int(right_transpose))
+        self.handle = None
+        self._keep = None
+
+    def inference(self, x, weight, scale, zp, bias=None):
+        x = _f32(x)
+        M = int(np.prod(x.shape[:-1])) if x.ndim > 1 else 1
+        self.attr.M = M
+        y = np.empty(tuple(x.shape[:-1]) + (self.attr.N,), dtype=np.float32)
+        p = _Param([x, _f32(weight), _f32(scale), _f32(zp), _f32(bias)], [y])
+        p.c.handle = self.handle
+        check(clib.lib().mi_top_a16mm_inference(C.byref(self.attr), C.byref(p.c)))
+        self.handle = p.c.handle
+        return y
+
+    def deinit(self):
+        if self.handle is not None:
+            p = _Param([None], [None])
+            p.c.handle = self.handle
+            clib.lib().mi_top_a16mm_deinit(C.byref(p.c))
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.deinit()
+        except Exception:
+            pass
+
+
+class TopA16Weight:
+    """Device-resident operands of a top.A16MatMul: uint8 weight [N, K * bits / 8], float32 scale / zp [N, G], bias."""
+
+    def __init__(self, weight, scale, zp, bias=None, *, K, N, weight_bits, q_group_size, right_transpose=True):
+        weight = np.ascontiguousarray(weight, dtype=np.uint8)
+        scale, zp, bias = _f32(scale), _f32(zp), _f32(bias)
+        self.handle = C.c_void_p()
+        self.K, self.N = K, N
+        check(clib.lib().mi_top_a16_weight_create(C.byref(self.handle), K, N, weight_bits, q_group_size,
+                                                  int(right_transpose), weight.ctypes.data, scale.ctypes.data,
+                                                  zp.ctypes.data, None if bias is None else bias.ctypes.data))
+
+    def destroy(self):
+        if self.handle:
+            clib.lib().mi_top_a16_weight_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+def top_a16mm_launch(w, x, y=None, stream=None):
+    """y[M, N] = x[M, K] @ dequant(W)^T + bias in float32 (x, y: float32 CUDA tensors)."""
+    import torch
+    if not (x.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and x.shape[-1] == w.K):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "top_a16mm_launch: x must be a contiguous float32 CUDA tensor [.., K]")
+    M = x.numel() // w.K
+    if y is None:
+        y = torch.empty(tuple(x.shape[:-1]) + (w.N,), dtype=torch.float32, device=x.device)
+    if not (y.is_cuda and y.dtype == torch.float32 and y.is_contiguous() and y.numel() == M * w.N):
+        raise clib.BackendError(clib.MI_BAD_ARGUMENT, "top_a16mm_launch: bad output tensor")
+    check(clib.lib().mi_top_a16mm_launch(w.handle, _dptr(x), M, _dptr(y), _stream_ptr(stream)))
+    return y
+
+
+def _matmul_shapes(a_shape, b_shape, o_shape, left_transpose=False, output_transpose=False, hdim_is_batch=False):
+    sh = clib.MatMulShapes()
+    for name, shape in (("a", a_shape), ("b", b_shape), ("o", o_shape)):
+        if len(shape) > 8:
+            raise clib.BackendError(clib.MI_BAD_ARGUMENT, "matmul shapes: rank above 8")
+        setattr(sh, name + "_dims", len(shape))
+        arr = getattr(sh, name + "_shape")
+        for i, v in enumerate(shape):
+            arr[i] = int(v)
+    sh.left_transpose, sh.output_transpose, sh.hdim_is_batch = int(left_transpose), int(output_transpose), int(hdim_is_batch)
+    return sh
+
+
+def matmul_parse_param(a_shape, b_shape, o_shape, *, right_transpose=False, left_transpose=False,
+                       output_transpose=False, hdim_is_batch=False, chip=CHIP_BM168X):
+    """tpu::MatMulOp::parseParam (mi_matmul_parse_param): dict with batch, batch_low, M, K, N and the flags."""
+    sh = _matmul_shapes(a_shape, b_shape, o_shape, left_transpose, output_transpose, hdim_is_batch)
+    out = clib.MatMulParam()
+    check(clib.lib().mi_matmul_parse_param(C.byref(sh), int(right_transpose), chip, C.byref(out)))
+    return {k: int(getattr(out, k)) for k, _ in clib.MatMulParam._fields_}
+
+
 class MatMulInt8:
     """Quantized tpu.MatMul (init / inference / deinit)."""
 
@@ -119,10 +213,35 @@ class MatMulInt8:
             self.param.c.handle = p.c.handle
         return y
 
+    def inference_nd(self, x, right, bias=None, multi=None):
+        """Operands of any rank (mi_i8mm_inference_nd): numpy.matmul's shapes, with the right operand stored
+        [.., N, K] under right_transpose.  Keeps its own handle (one per batch inside the library)."""
+        x, right = _f32(x), _f32(right)
+        n = right.shape[-2] if self.attr.right_transpose else (right.shape[-1] if right.ndim > 1 else None)
+        if right.ndim == 1:
+            o_shape = tuple(x.shape[:-1])
+        elif right.ndim == 2 or x.ndim == 1:
+            o_shape = tuple(x.shape[:-1]) + (n,) if x.ndim > 1 else tuple(right.shape[:-2]) + (n,)
+        else:
+            o_shape = tuple(np.broadcast_shapes(x.shape[:-2], right.shape[:-2])) + (x.shape[-2], n)
+        sh = _matmul_shapes(x.shape, right.shape, o_shape)
+        y = np.empty(o_shape, dtype=np.float32)
+        p = _Param([x, right, _f32(bias), _f32(multi), None], [y])
+        p.c.handle = getattr(self, "_nd_handle", None)
+        rc = clib.lib().mi_i8mm_inference_nd(C.byref(self.attr), C.byref(sh), C.byref(p.c))
+        self._nd_handle = p.c.handle
+        check(rc)
+        return y
+
     def deinit(self):
         if self.param is not None:
             clib.lib().mi_i8mm_deinit(C.byref(self.param.c))
             self.param = None
+        if getattr(self, "_nd_handle", None) is not None:
+            p = _Param([None], [None])
+            p.c.handle = self._nd_handle
+            clib.lib().mi_i8mm_deinit(C.byref(p.c))
+            self._nd_handle = None
 
     def __del__(self):
         try:
