@@ -467,8 +467,32 @@ int mi_module_set_tensor(mi_module *m, const char *name, const float *data, int6
  * from a HIP graph when every op is a plain kernel launch */
 int mi_module_invoke(mi_module *m);
 int mi_module_uses_graph(const mi_module *m);
-/* float data out (expanded on the device), as py_cuda::get_tensor */
+/* float data out (expanded on the device), as py_cuda::get_tensor / cuda_to_host (pycuda.cpp:289-397): a tensor
+ * declared uniform-quantized by mi_module_set_quant comes back scaled -- 8-bit ((float)q - (float)zp) * (float)scale,
+ * int16 q * scale -- every other tensor as its values. */
 int mi_module_get_tensor(mi_module *m, const char *name, float *out, int64_t num_elem);
+/* the stored values without the scaling (cuda_to_host's for_infer branch, pycuda.cpp:311-323) */
+int mi_module_get_tensor_raw(mi_module *m, const char *name, float *out, int64_t num_elem);
+/* declares an int8 / uint8 / int16 tensor uniform-quantized: module::getUniformQuantizedType's scale and zero point */
+int mi_module_set_quant(mi_module *m, const char *name, double scale, int64_t zero_point);
+/* Activation lifetimes (py_cuda frees an activation after its last consumer, pycuda.cpp:633-660; the host interpreter
+ * packs dead tensors into reused memory, host/ModuleInterpreter.cpp:86-232).  Here the saving is planned once, so that
+ * graph replay keeps working: mi_module_plan_memory, called after the last op is added, moves every intermediate
+ * (written by an op and not marked as an output) into one arena in which tensors whose lifetimes do not overlap share
+ * bytes.  arena_bytes / unplanned_bytes (optional) receive the arena's size and what the same tensors took before.
+ * A tensor that shares bytes cannot be read back afterwards (MI_BAD_ARGUMENT), exactly as an activation the reference
+ * has freed; mark what must stay readable with mi_module_mark_output first.  No tensors or ops can be added after. */
+int mi_module_mark_output(mi_module *m, const char *name);
+int mi_module_plan_memory(mi_module *m, int64_t *arena_bytes, int64_t *unplanned_bytes);
+/* before / after hooks around every op, named by its output tensor (ModuleInterpreter::call_before_hook /
+ * call_after_hook, host/ModuleInterpreter.cpp:1531-1540).  The stream is drained before an after hook runs, so the
+ * hook may call mi_module_get_tensor.  With a hook set, invoke launches op by op instead of replaying its graph. */
+typedef void (*mi_module_hook)(const char *op_name, void *user);
+int mi_module_set_hooks(mi_module *m, mi_module_hook before, mi_module_hook after, void *user);
+/* runs the one op that writes `name` / every op from that one on (ModuleInterpreter::invoke_at / invoke_from,
+ * host/ModuleInterpreter.cpp:1209-1253), hooks included; not available once a memory plan is made */
+int mi_module_invoke_at(mi_module *m, const char *name);
+int mi_module_invoke_from(mi_module *m, const char *name);
 
 /* ============================================================================ */
 /* top.A16MatMul: the f32 twin of tpu.A16MatMul (the "top" stage the reference's   */

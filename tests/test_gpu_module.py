@@ -220,3 +220,112 @@ def test_dynamic_quant_a16matmul_in_a_module(orc, dq, bits):
         m2.add_a16matmul("a", "b", bad["weight"], bad["scale"], bad["zp"], None, K=192, N=16, weight_bits=4,
                          q_group_size=64, dq_type=clib.DQ_INT)
     assert e.value.code == clib.MI_UNSUPPORTED
+
+
+def _decoder_like_module(M=2, K=512, mlp=1024, plan=False, outputs=("down",)):
+    """x -> cast -> q,k,v (grouped) -> o (from q) -> gate,up (grouped, from o) -> down (from gate)."""
+    cfgs = {"q": S.w4a16(M, K, K, 128, seed=401), "k": S.w4a16(M, K, K, 128, seed=402), "v": S.w4a16(M, K, K, 128, seed=403),
+            "o": S.w4a16(M, K, K, 128, seed=404), "gate": S.w4a16(M, K, mlp, 128, seed=405),
+            "up": S.w4a16(M, K, mlp, 128, seed=406), "down": S.w4a16(M, mlp, K, 128, seed=407)}
+    src = {"q": "xb", "k": "xb", "v": "xb", "o": "q", "gate": "o", "up": "o", "down": "gate"}
+    m = M_.Module()
+    m.add_tensor("x", clib.ST_F32, (M, K)).add_tensor("xb", clib.ST_BF16, (M, K))
+    for n, c in cfgs.items():
+        m.add_tensor(n, clib.ST_BF16, (M, c["N"]))
+    m.add_cast("x", "xb", in_type=clib.ST_F32, out_type=clib.ST_BF16)
+    for n, c in cfgs.items():
+        m.add_a16matmul(src[n], n, c["weight"], c["scale"], c["zp"], None, K=c["K"], N=c["N"], weight_bits=4,
+                        q_group_size=128)
+    for n in outputs:
+        m.mark_output(n)
+    sizes = m.plan_memory() if plan else None
+    return m, cfgs, sizes
+
+
+def test_memory_plan_shares_dead_activations_and_keeps_results():
+    """pycuda.cpp:633-660 frees an activation after its last consumer; here the same saving is planned once.  The
+    planned module must give bit-identical outputs (eagerly and from its graph), use less memory, keep marked
+    outputs readable and refuse to read back a tensor whose bytes were reused."""
+    M, K = 2, 512
+    x = np.random.default_rng(5).standard_normal((M, K)).astype(np.float32)
+    plain, _, _ = _decoder_like_module(M, K)
+    planned, _, (arena, before) = _decoder_like_module(M, K, plan=True, outputs=("down", "k"))
+    # intermediates: xb, q, v, o, gate, up (k and down are outputs); xb is dead once q/k/v ran, q once o ran, ...
+    assert 0 < arena < before
+    for rep in range(3):
+        for mod in (plain, planned):
+            mod.set_tensor("x", x * (1 + rep))
+            mod.invoke()
+        assert np.array_equal(plain.get_tensor("down"), planned.get_tensor("down"))
+        assert np.array_equal(plain.get_tensor("k"), planned.get_tensor("k"))
+    assert planned.uses_graph()
+    with pytest.raises(clib.BackendError) as e:
+        planned.get_tensor("xb")
+    assert e.value.code == clib.MI_BAD_ARGUMENT
+    with pytest.raises(clib.BackendError):
+        planned.add_tensor("late", clib.ST_F32, (1, 4))
+    with pytest.raises(clib.BackendError):
+        planned.invoke_at("o")
+    plain.destroy()
+    planned.destroy()
+
+
+def test_hooks_invoke_at_and_invoke_from():
+    """ModuleInterpreter::call_before_hook / call_after_hook around every op, invoke_at, invoke_from
+    (host/ModuleInterpreter.cpp:1209-1253, :1531-1540)."""
+    M, K = 1, 512
+    x = np.random.default_rng(6).standard_normal((M, K)).astype(np.float32)
+    m, _, _ = _decoder_like_module(M, K)
+    m.set_tensor("x", x)
+    m.invoke()
+    want = {n: m.get_tensor(n) for n in ("xb", "q", "k", "v", "o", "gate", "up", "down")}
+    calls, seen = [], {}
+    m.set_hooks(before=lambda n: calls.append(("before", n)),
+                after=lambda n: (calls.append(("after", n)), seen.__setitem__(n, m.get_tensor(n))))
+    m.invoke()
+    order = ["xb", "q", "k", "v", "o", "gate", "up", "down"]
+    assert [n for kind, n in calls if kind == "before"] == order
+    assert [n for kind, n in calls if kind == "after"] == order
+    for n in order:  # an op's before hook comes ahead of its own after hook, and the hook sees the finished tensor
+        assert calls.index(("before", n)) < calls.index(("after", n))
+        assert np.array_equal(seen[n], want[n])
+    # invoke_at: one op; invoke_from: that op and everything after it
+    calls.clear()
+    assert np.array_equal(m.invoke_at("o"), want["o"])
+    assert calls == [("before", "o"), ("after", "o")]
+    calls.clear()
+    m.set_tensor("x", 2 * x)          # changes nothing downstream of q unless q is recomputed
+    m.invoke_from("gate")
+    assert [n for kind, n in calls if kind == "before"] == ["gate", "up", "down"]
+    assert np.array_equal(m.get_tensor("down"), want["down"])
+    m.set_hooks(None, None)
+    m.invoke()                         # now x = 2x reaches every op
+    assert not np.array_equal(m.get_tensor("down"), want["down"])
+    with pytest.raises(clib.BackendError):
+        m.invoke_at("x")               # no op writes the input
+    m.destroy()
+
+
+def test_get_tensor_scales_uniform_quantized_tensors():
+    """py_cuda::cuda_to_host: int8 / uint8 ((float)q - (float)zp) * (float)scale, int16 q * scale; the raw read does
+    not scale (pycuda.cpp:311-343, :370-379)."""
+    m = M_.Module()
+    n = 300
+    m.add_tensor("a", clib.ST_I8, (n,)).add_tensor("b", clib.ST_U8, (n,)).add_tensor("c", clib.ST_I16, (n,))
+    m.add_tensor("plain", clib.ST_I8, (n,))
+    rng = np.random.default_rng(3)
+    a = rng.integers(-128, 128, size=n).astype(np.float32)
+    b = rng.integers(0, 256, size=n).astype(np.float32)
+    c = rng.integers(-32768, 32768, size=n).astype(np.float32)
+    m.set_quant("a", 0.0123, -7).set_quant("b", 0.37, 131).set_quant("c", 1.7e-3, 5)
+    for name, v in (("a", a), ("b", b), ("c", c), ("plain", a)):
+        m.set_tensor(name, v)
+    assert np.array_equal(m.get_tensor("a"), (a - np.float32(-7)) * np.float32(0.0123))
+    assert np.array_equal(m.get_tensor("b"), (b - np.float32(131)) * np.float32(0.37))
+    assert np.array_equal(m.get_tensor("c"), (c.astype(np.float64) * 1.7e-3).astype(np.float32))  # no zero point
+    assert np.array_equal(m.get_tensor("plain"), a)
+    for name, v in (("a", a), ("b", b), ("c", c)):
+        assert np.array_equal(m.get_tensor_raw(name), v)
+    with pytest.raises(clib.BackendError):
+        m.add_tensor("f", clib.ST_F32, (4,)).set_quant("f", 1.0, 0)
+    m.destroy()

@@ -29,11 +29,15 @@ EXPORTS = [
     "mi_cast_inference", "mi_cast_launch",
     "mi_module_create", "mi_module_destroy", "mi_module_add_tensor", "mi_module_add_a16matmul", "mi_module_add_a16matmul_dq",
     "mi_module_add_matmul_int8", "mi_module_add_requant", "mi_module_add_matmul_dq", "mi_module_add_cast", "mi_module_set_tensor", "mi_module_invoke",
-    "mi_module_uses_graph", "mi_module_get_tensor",
+    "mi_module_uses_graph", "mi_module_get_tensor", "mi_module_get_tensor_raw", "mi_module_set_quant",
+    "mi_module_mark_output", "mi_module_plan_memory", "mi_module_set_hooks", "mi_module_invoke_at", "mi_module_invoke_from",
     "mi_top_a16mm_inference", "mi_top_a16mm_deinit", "mi_top_a16_weight_create", "mi_top_a16_weight_destroy",
     "mi_top_a16mm_launch",
     "mi_bench_read_launch",
 ]
+
+
+MODULE_HOOK = C.CFUNCTYPE(None, C.c_char_p, C.c_void_p)
 
 
 class BackendError(RuntimeError):
@@ -219,6 +223,13 @@ def lib():
         L.mi_module_invoke.argtypes = [C.c_void_p]
         L.mi_module_uses_graph.argtypes = [C.c_void_p]
         L.mi_module_get_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int64]
+        L.mi_module_get_tensor_raw.argtypes = L.mi_module_get_tensor.argtypes
+        L.mi_module_set_quant.argtypes = [C.c_void_p, C.c_char_p, C.c_double, C.c_int64]
+        L.mi_module_mark_output.argtypes = [C.c_void_p, C.c_char_p]
+        L.mi_module_plan_memory.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi_module_set_hooks.argtypes = [C.c_void_p, MODULE_HOOK, MODULE_HOOK, C.c_void_p]
+        L.mi_module_invoke_at.argtypes = [C.c_void_p, C.c_char_p]
+        L.mi_module_invoke_from.argtypes = [C.c_void_p, C.c_char_p]
         L.mi_cast_inference.argtypes = [C.POINTER(CastAttr), C.POINTER(InferParam)]
         L.mi_cast_launch.argtypes = [C.POINTER(CastAttr), C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_init.argtypes = [C.POINTER(A16Attr), C.POINTER(InferParam)]

@@ -783,6 +783,41 @@ class Module:
         check(clib.lib().mi_module_get_tensor(self.handle, name.encode(), out.ctypes.data, out.size))
         return out
 
+    def get_tensor_raw(self, name):
+        """The stored values as floats, without the scaling of a uniform-quantized tensor."""
+        out = np.empty(self.shapes[name], dtype=np.float32)
+        check(clib.lib().mi_module_get_tensor_raw(self.handle, name.encode(), out.ctypes.data, out.size))
+        return out
+
+    def set_quant(self, name, scale, zero_point=0):
+        check(clib.lib().mi_module_set_quant(self.handle, name.encode(), C.c_double(scale), C.c_int64(zero_point)))
+        return self
+
+    def mark_output(self, name):
+        check(clib.lib().mi_module_mark_output(self.handle, name.encode()))
+        return self
+
+    def plan_memory(self):
+        """Packs the intermediates into one arena by lifetime; returns (arena bytes, bytes the same tensors took)."""
+        arena, before = C.c_int64(0), C.c_int64(0)
+        check(clib.lib().mi_module_plan_memory(self.handle, C.byref(arena), C.byref(before)))
+        return arena.value, before.value
+
+    def set_hooks(self, before=None, after=None):
+        """before(op_name) / after(op_name) around every op (named by its output tensor); None clears."""
+        self._hooks = (None if before is None else clib.MODULE_HOOK(lambda n, u: before(n.decode())),
+                       None if after is None else clib.MODULE_HOOK(lambda n, u: after(n.decode())))
+        nullf = C.cast(None, clib.MODULE_HOOK)
+        check(clib.lib().mi_module_set_hooks(self.handle, self._hooks[0] or nullf, self._hooks[1] or nullf, None))
+        return self
+
+    def invoke_at(self, name):
+        check(clib.lib().mi_module_invoke_at(self.handle, name.encode()))
+        return self.get_tensor(name)
+
+    def invoke_from(self, name):
+        check(clib.lib().mi_module_invoke_from(self.handle, name.encode()))
+
     def destroy(self):
         if self.handle:
             clib.lib().mi_module_destroy(self.handle)
