@@ -50,7 +50,8 @@ enum {
   MI_RQ_TFLITE = 1,
   MI_RQ_MULTIPLIER_SHIFT = 2,
   MI_RQ_ONLY_SHIFT = 3,
-  MI_RQ_QDM = 4
+  MI_RQ_QDM = 4,
+  MI_RQ_ONLY_SCALE = 5
 };
 /* storage types */
 enum { MI_DT_BF16 = 0, MI_DT_F16 = 1, MI_DT_I8 = 2, MI_DT_U8 = 3, MI_DT_I16 = 4, MI_DT_U16 = 5, MI_DT_I32 = 6 };
@@ -294,6 +295,7 @@ typedef struct mi_i8mm_attr {
   int64_t out_zp;         /* zero point of the uniform-quantized output type */
   int out_dtype;          /* MI_DT_I8/U8/I16/U16, or MI_DT_I32 for an un-requantized int32 result */
   int right_is_weight;    /* module::isWeight(getRight()): right (and bias, multi) are cached in HBM at init */
+  double out_scale;       /* MI_RQ_ONLY_SCALE: getOutScales()[0] (MatMul.cpp:683-685) */
 } mi_i8mm_attr;
 
 /* Replace tpu::MatMulOp::{init,inference,deinit} (MatMul.cpp:387-396, :440-733, :431-438).
@@ -333,6 +335,8 @@ int mi_i8mm_inference_nd(const mi_i8mm_attr *attr, const mi_matmul_shapes *shape
  *   MI_RQ_TFLITE / _LSHIFT / QDM: v = MultiplyByQuantizedMultiplier(acc, mult[n], -shift[n], round_mode)
  *                           i.e. shift[n] is a RIGHT shift when positive                   (MathUtils.cpp:523-536)
  *   MI_RQ_ONLY_SHIFT:       v = RightShiftRound(acc, shift[n], round_mode)
+ *   MI_RQ_ONLY_SCALE:       v = (int32)roundf((float)acc * only_scale), one scale for every channel, half away from
+ *                           zero (tpu.MatMul only, MatMul.cpp:673-695; the per-channel variant asserts there)
  *   out = saturate(v + zp[n], out_dtype)                                                    (MathUtils.cpp:849-872)
  * d_multiplier/d_shift/d_zp are DEVICE int32 arrays of length n_channels, or NULL to use the scalar. */
 typedef struct mi_requant_desc {
@@ -348,6 +352,7 @@ typedef struct mi_requant_desc {
                                 * per-channel arrays (round half away from zero, int8 output); 0 keeps such arrays
                                 * on the general 64-bit path.  Scalars are checked by the library itself.  Results
                                 * are identical either way. */
+  float only_scale;            /* MI_RQ_ONLY_SCALE: (float)getOutScales()[0] */
 } mi_requant_desc;
 
 /* acc[M,N] = (A - input_zp)[M,K] * (B - right_zp) + bias[N], relu, then requant -> d_out.

@@ -1109,7 +1109,16 @@ int orc_matmul_int8(const orc_i8mm_attr *a, const float *const *inputs,
   /* MatMul.cpp:665-727 */
   int64_t rshift0 = arr_at(a->rshifts, a->n_rshifts, 0, 0);
   int64_t mult0 = arr_at(a->multipliers, a->n_multipliers, 0, 1);
-  if (a->quant_mode == ORC_RQ_TFLITE_LSHIFT || a->quant_mode == ORC_RQ_TFLITE) {
+  if (a->quant_mode == ORC_RQ_ONLY_SCALE) {
+    /* MatMul.cpp:673-695; the fused (per-channel) flavour asserts (:674-676) */
+    if (a->fuse_rq)
+      return 1;
+    const float scale = (float)a->out_scale;
+    for (int64_t i = 0; i < num; i++) {
+      float v = output[i] * scale;
+      output[i] = (float)orc_saturate_i64((int64_t)(int32_t)roundf(v) + a->out_zp, a->out_bits, a->out_unsigned);
+    }
+  } else if (a->quant_mode == ORC_RQ_TFLITE_LSHIFT || a->quant_mode == ORC_RQ_TFLITE) {
     for (int64_t i = 0; i < num; i++) {
       int64_t v = (int64_t)orc_multiply_by_quantized_multiplier(
                       (int32_t)output[i], (int32_t)mult0, -(int32_t)rshift0,

@@ -196,6 +196,7 @@ typedef struct {
   int out_kind;            /* 0: uniform-quantised integer, 1: raw int32 */
   int out_bits, out_unsigned;
   int gemm_kind;
+  double out_scale;        /* ORC_RQ_ONLY_SCALE: getOutScales()[0] */
 } orc_i8mm_attr;
 
 /* inputs[0..3] = input, right, bias(NULL ok), multi(NULL ok); f32-valued.

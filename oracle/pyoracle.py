@@ -47,7 +47,7 @@ class I8Attr(C.Structure):
                 ("rshifts", C.POINTER(C.c_int64)), ("n_rshifts", C.c_int),
                 ("out_zp", C.c_int64), ("out_kind", C.c_int),
                 ("out_bits", C.c_int), ("out_unsigned", C.c_int),
-                ("gemm_kind", C.c_int)]
+                ("gemm_kind", C.c_int), ("out_scale", C.c_double)]
 
 
 class RqAxisAttr(C.Structure):
@@ -305,14 +305,14 @@ def matmul_dynamic(left, right, *, right_transpose=False, q_group_size, imax=127
 def matmul_int8(x, right, bias, multi, *, M, K, N, right_transpose=False, input_zp=0, right_zp=0,
                 do_relu=False, relu_limit=-1.0, cv18xx=False, quant_mode=RQ_MULTIPLIER_SHIFT, fuse_rq=False,
                 multipliers=(1,), rshifts=(0,), out_zp=0, out_kind=0, out_bits=8, out_unsigned=False,
-                gemm_kind=GEMM_F32):
+                gemm_kind=GEMM_F32, out_scale=1.0):
     """Quantised tpu.MatMul on f32-valued operands; returns (output, f32 accumulators)."""
     ins = [_f32(x), _f32(right), _f32(bias), _f32(multi)]
     mult = np.ascontiguousarray(multipliers, dtype=np.int64)
     rs = np.ascontiguousarray(rshifts, dtype=np.int64)
     attr = I8Attr(M, K, N, int(right_transpose), input_zp, right_zp, int(do_relu), relu_limit, int(cv18xx),
                   quant_mode, int(fuse_rq), _p(mult, C.c_int64), mult.size, _p(rs, C.c_int64), rs.size,
-                  out_zp, out_kind, out_bits, int(out_unsigned), gemm_kind)
+                  out_zp, out_kind, out_bits, int(out_unsigned), gemm_kind, out_scale)
     arr = (C.POINTER(C.c_float) * 4)(*[None if a is None else _p(a, C.c_float) for a in ins])
     out = np.empty((M, N), dtype=np.float32)
     acc = np.empty((M, N), dtype=np.float32)
@@ -553,7 +553,8 @@ def matmul_parse_param(a_shape, b_shape, o_shape, *, right_transpose=False, left
 
 def matmul_int8_nd(x, right, bias, multi, *, out_shape, right_transpose=False, input_zp=0, right_zp=0, do_relu=False,
                    relu_limit=-1.0, cv18xx=False, quant_mode=RQ_MULTIPLIER_SHIFT, fuse_rq=False, multipliers=(1,),
-                   rshifts=(0,), out_zp=0, out_kind=0, out_bits=8, out_unsigned=False, gemm_kind=GEMM_F32):
+                   rshifts=(0,), out_zp=0, out_kind=0, out_bits=8, out_unsigned=False, gemm_kind=GEMM_F32,
+                   out_scale=1.0):
     """Quantised tpu.MatMul on operands of any rank (plain branch of parseParam); returns the output, shaped out_shape."""
     x, right = _f32(x), _f32(right)
     ins = [x, right, _f32(bias), _f32(multi)]
@@ -561,7 +562,7 @@ def matmul_int8_nd(x, right, bias, multi, *, out_shape, right_transpose=False, i
     rs = np.ascontiguousarray(rshifts, dtype=np.int64)
     attr = I8Attr(0, 0, 0, int(right_transpose), input_zp, right_zp, int(do_relu), relu_limit, int(cv18xx),
                   quant_mode, int(fuse_rq), _p(mult, C.c_int64), mult.size, _p(rs, C.c_int64), rs.size,
-                  out_zp, out_kind, out_bits, int(out_unsigned), gemm_kind)
+                  out_zp, out_kind, out_bits, int(out_unsigned), gemm_kind, out_scale)
     arr = (C.POINTER(C.c_float) * 4)(*[None if a is None else _p(a, C.c_float) for a in ins])
     out = np.empty(tuple(out_shape), dtype=np.float32)
     L = lib()

@@ -189,6 +189,18 @@ def test_operator_level_against_oracle(orc):
                                   multipliers=[mult], rshifts=[rs])
         assert np.array_equal(op.inference(a), want), qm
         op.deinit()
+    # OnlyScale (MatMul.cpp:673-695): one float scale, roundf; the per-channel flavour is refused as the reference's assert
+    for od, uns in ((clib.DT_I8, False), (clib.DT_U8, True)):
+        op = M_.MatMulInt8(K=256, N=64, quant_mode=clib.RQ_ONLY_SCALE, out_scale=3.1e-4, out_zp=7, out_dtype=od)
+        op.init(a, b, bias)
+        want, _ = orc.matmul_int8(a, b, bias, None, M=48, K=256, N=64, quant_mode=orc.RQ_ONLY_SCALE, out_scale=3.1e-4,
+                                  out_zp=7, out_unsigned=uns)
+        assert np.array_equal(op.inference(a), want)
+        assert len(np.unique(want)) > 20
+        op.deinit()
+    with pytest.raises(clib.BackendError) as e:
+        M_.MatMulInt8(K=256, N=64, quant_mode=clib.RQ_ONLY_SCALE, fuse_rq=True, out_scale=1e-3).init(a, b, bias, multi)
+    assert e.value.code == clib.MI_UNSUPPORTED
     # int32 output (un-fused form), right operand is an activation (not cached), lazy init through inference
     op = M_.MatMulInt8(K=256, N=64, out_dtype=clib.DT_I32, right_is_weight=False, input_zp=4, right_zp=-2)
     want, _ = orc.matmul_int8(a, b, bias, None, M=48, K=256, N=64, input_zp=4, right_zp=-2, out_kind=1)

@@ -166,3 +166,31 @@ def test_requant_int_per_tensor():
     # rank-1 tensors pass through untouched (RequantInt.cpp:36-38)
     v = np.array([1000.0, -1000.0], dtype=np.float32)
     assert np.array_equal(O.requant_int(v, quant_mode=O.RQ_MULTIPLIER_SHIFT, multiplier=1, rshift=3), v)
+
+
+def test_only_scale_mode_against_numpy(orc):
+    """RequantMode::OnlyScale (MatMul.cpp:673-695): (int32)roundf(acc * (float)scale) + zp, saturated.  Pinned by a
+    numpy closed form of round-half-away on float32 products, on accumulators built to hit exact .5 ties of both
+    signs, and by the refusal of the per-channel flavour (the reference asserts there)."""
+    M, K, N = 6, 4, 8
+    a = np.zeros((M, K), dtype=np.float32)
+    a[:, 0] = [1, 3, -1, -3, 5, -5]                     # acc = a[:, 0] * b[0, :] = odd numbers times 1
+    b = np.zeros((K, N), dtype=np.float32)
+    b[0, :] = [1, 1, 3, 3, 5, 7, 9, 11]
+    acc = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    out, accf = orc.matmul_int8(a, b, None, None, M=M, K=K, N=N, quant_mode=orc.RQ_ONLY_SCALE, out_scale=0.5, out_zp=3)
+    assert np.array_equal(accf, acc)
+    v = acc * np.float32(0.5)                            # x.5 everywhere: ties
+    want = np.clip(np.sign(v) * np.floor(np.abs(v) + 0.5) + 3, -128, 127)
+    assert np.array_equal(out, want)
+    rng = np.random.default_rng(11)
+    a = rng.integers(-128, 128, size=(16, 64)).astype(np.float32)
+    b = rng.integers(-128, 128, size=(64, 24)).astype(np.float32)
+    out, accf = orc.matmul_int8(a, b, None, None, M=16, K=64, N=24, quant_mode=orc.RQ_ONLY_SCALE, out_scale=0.0037,
+                                out_zp=-5, out_unsigned=True)
+    v = accf * np.float32(0.0037)
+    want = np.clip(np.sign(v) * np.floor(np.abs(v) + np.float32(0.5)) - 5, 0, 255)
+    assert np.array_equal(out, want)
+    with pytest.raises(RuntimeError):
+        orc.matmul_int8(a, b, None, np.ones(24, dtype=np.float32), M=16, K=64, N=24, quant_mode=orc.RQ_ONLY_SCALE,
+                        fuse_rq=True, out_scale=0.5)

@@ -8,7 +8,7 @@ _LIB_PATH = os.path.join(_HERE, "lib", "libtpumlir_amd.so")
 MI_SUCCESS, MI_UNSUPPORTED, MI_BAD_ARGUMENT, MI_HIP_ERROR = 0, 1, 2, 3
 ROUND_HALF_AWAY_FROM_ZERO, ROUND_HALF_UP, ROUND_HALF_DOWN, ROUND_HALF_TO_EVEN = 0, 1, 2, 3
 ROUND_TOWARDS_ZERO, ROUND_UP, ROUND_DOWN = 6, 8, 9
-RQ_TFLITE_LSHIFT, RQ_TFLITE, RQ_MULTIPLIER_SHIFT, RQ_ONLY_SHIFT, RQ_QDM = 0, 1, 2, 3, 4
+RQ_TFLITE_LSHIFT, RQ_TFLITE, RQ_MULTIPLIER_SHIFT, RQ_ONLY_SHIFT, RQ_QDM, RQ_ONLY_SCALE = 0, 1, 2, 3, 4, 5
 DT_BF16, DT_F16, DT_I8, DT_U8, DT_I16, DT_U16, DT_I32 = range(7)
 CHIP_BM168X, CHIP_CV18XX = 0, 1
 ST_F32, ST_BF16, ST_F16, ST_I8, ST_U8, ST_I16, ST_U16, ST_I32, ST_U32, ST_F8E4M3, ST_F8E5M2 = range(11)
@@ -109,14 +109,16 @@ class I8Attr(C.Structure):
                 ("chip", C.c_int), ("quant_mode", C.c_int), ("round_mode", C.c_int), ("fuse_rq", C.c_int),
                 ("multipliers", C.POINTER(C.c_int64)), ("n_multipliers", C.c_int),
                 ("rshifts", C.POINTER(C.c_int64)), ("n_rshifts", C.c_int),
-                ("out_zp", C.c_int64), ("out_dtype", C.c_int), ("right_is_weight", C.c_int)]
+                ("out_zp", C.c_int64), ("out_dtype", C.c_int), ("right_is_weight", C.c_int),
+                ("out_scale", C.c_double)]
 
 
 class RequantDescC(C.Structure):
     _fields_ = [("quant_mode", C.c_int), ("round_mode", C.c_int), ("chip", C.c_int), ("out_dtype", C.c_int),
                 ("d_multiplier", C.c_void_p), ("multiplier", C.c_int32),
                 ("d_shift", C.c_void_p), ("shift", C.c_int32),
-                ("d_zp", C.c_void_p), ("zp", C.c_int32), ("per_channel_q31_checked", C.c_int)]
+                ("d_zp", C.c_void_p), ("zp", C.c_int32), ("per_channel_q31_checked", C.c_int),
+                ("only_scale", C.c_float)]
 
 
 class RqAxisAttr(C.Structure):

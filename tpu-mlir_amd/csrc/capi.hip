@@ -675,8 +675,13 @@ static int check_i8_attr(const mi_i8mm_attr *a, const char *who) {
                      q == MI_RQ_TFLITE_LSHIFT,
                  MI_UNSUPPORTED, std::string(who) + ": requant mode not handled");
     else
-      MI_REQUIRE(q == MI_RQ_MULTIPLIER_SHIFT || q == MI_RQ_TFLITE || q == MI_RQ_TFLITE_LSHIFT, MI_UNSUPPORTED,
-                 std::string(who) + ": requant mode not handled");
+      MI_REQUIRE(q == MI_RQ_MULTIPLIER_SHIFT || q == MI_RQ_TFLITE || q == MI_RQ_TFLITE_LSHIFT || q == MI_RQ_ONLY_SCALE,
+                 MI_UNSUPPORTED, std::string(who) + ": requant mode not handled");
+    // the reference asserts on the per-channel flavour of OnlyScale (MatMul.cpp:674-676)
+    MI_REQUIRE(!(q == MI_RQ_ONLY_SCALE && a->fuse_rq), MI_UNSUPPORTED,
+               std::string(who) + ": OnlyScale with fuse_rq is not supported; use MultiplierShift");
+    if (q == MI_RQ_ONLY_SCALE)
+      return MI_SUCCESS;
     MI_REQUIRE(a->multipliers && a->n_multipliers >= 1 && a->rshifts && a->n_rshifts >= 1, MI_BAD_ARGUMENT,
                std::string(who) + ": multipliers / rshifts missing");
   }
@@ -776,12 +781,17 @@ int mi_i8mm_inference(const mi_i8mm_attr *attr, mi_infer_param *p) {
     rq.chip = attr->chip;
     rq.out_dtype = attr->out_dtype;
     rq.quant_mode = attr->quant_mode;
-    rq.multiplier = (int32_t)attr->multipliers[0];
-    rq.shift = (int32_t)attr->rshifts[0];
+    rq.multiplier = attr->multipliers && attr->n_multipliers > 0 ? (int32_t)attr->multipliers[0] : 1;
+    rq.shift = attr->rshifts && attr->n_rshifts > 0 ? (int32_t)attr->rshifts[0] : 0;
     if (attr->chip == MI_CHIP_CV18XX) {
       // MatMul.cpp:638-664: per-batch (here: one) multiplier/rshift, half away from zero, no zero point
       rq.round_mode = MI_ROUND_HALF_AWAY_FROM_ZERO;
       rq.zp = 0;
+    } else if (attr->quant_mode == MI_RQ_ONLY_SCALE) {
+      // MatMul.cpp:683-691: (int32)roundf(acc * (float)out_scales[0]) + zero point
+      rq.round_mode = MI_ROUND_HALF_AWAY_FROM_ZERO;
+      rq.zp = (int32_t)attr->out_zp;
+      rq.only_scale = (float)attr->out_scale;
     } else if (attr->quant_mode == MI_RQ_MULTIPLIER_SHIFT) {
       // MatMul.cpp:708-726: default rounding of applyMultiplierAndRShift is half up (MathUtils.h:178-181)
       rq.round_mode = MI_ROUND_HALF_UP;

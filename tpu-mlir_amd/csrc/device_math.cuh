@@ -189,6 +189,7 @@ struct RequantParams {
   const int32_t *zp;
   int32_t mult_s, shift_s, zp_s;
   int qmode, rmode, chip, out_dtype;
+  float scale_f;  // MI_RQ_ONLY_SCALE
 };
 
 // int32 accumulator of channel n -> saturated output value.  The descriptor's shift is a RIGHT shift
@@ -203,7 +204,9 @@ __device__ __forceinline__ int32_t requant_one(int32_t acc, int64_t n, const Req
 // the same with the channel's multiplier, shift and zero point already in hand
 __device__ __forceinline__ int32_t requant_with(int32_t acc, int64_t m, int64_t s, int64_t z, const RequantParams &rq) {
   int64_t v;
-  if (rq.qmode == MI_RQ_MULTIPLIER_SHIFT || rq.qmode == MI_RQ_ONLY_SHIFT)
+  if (rq.qmode == MI_RQ_ONLY_SCALE)  // MatMul.cpp:686-691: the float accumulator times the scale, roundf, then zp
+    v = (int64_t)(int32_t)roundf((float)acc * rq.scale_f);
+  else if (rq.qmode == MI_RQ_MULTIPLIER_SHIFT || rq.qmode == MI_RQ_ONLY_SHIFT)
     v = apply_multiplier_and_rshift(acc, m, s, rq.qmode, rq.rmode, rq.chip);
   else
     v = (int64_t)multiply_by_quantized_multiplier(acc, (int32_t)m, (int)-s, rq.rmode);

@@ -851,13 +851,14 @@ static RequantParams make_rq(const mi_requant_desc *rq) {
   p.rmode = rq->round_mode;
   p.chip = rq->chip;
   p.out_dtype = rq->out_dtype;
+  p.scale_f = rq->only_scale;
   return p;
 }
 
 static int check_rq(const mi_requant_desc *rq, const char *who) {
   const int q = rq->quant_mode;
   MI_REQUIRE(q == MI_RQ_TFLITE_LSHIFT || q == MI_RQ_TFLITE || q == MI_RQ_MULTIPLIER_SHIFT || q == MI_RQ_ONLY_SHIFT ||
-                 q == MI_RQ_QDM,
+                 q == MI_RQ_QDM || q == MI_RQ_ONLY_SCALE,
              MI_UNSUPPORTED, std::string(who) + ": unsupported requant mode");
   const int o = rq->out_dtype;
   MI_REQUIRE(o == MI_DT_I8 || o == MI_DT_U8 || o == MI_DT_I16 || o == MI_DT_U16 || o == MI_DT_I32, MI_UNSUPPORTED,
@@ -947,7 +948,7 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
   if (rq)
     a.rq = make_rq(rq);
   else
-    a.rq = RequantParams{nullptr, nullptr, nullptr, 1, 0, 0, MI_RQ_MULTIPLIER_SHIFT, 0, 0, MI_DT_I32};
+    a.rq = RequantParams{nullptr, nullptr, nullptr, 1, 0, 0, MI_RQ_MULTIPLIER_SHIFT, 0, 0, MI_DT_I32, 1.0f};
   // 256x256 tiles when there are enough of them to occupy the chip, else 128x128 tiles on the same data path; the
   // register-staged kernel takes what is left (K % 64 != 0)
   const int64_t tiles_large = ((M + LM - 1) / LM) * ((N + LN - 1) / LN);

@@ -179,14 +179,15 @@ class MatMulInt8:
 
     def __init__(self, K, N, *, right_transpose=False, input_zp=0, right_zp=0, do_relu=False, relu_limit=-1.0,
                  chip=CHIP_BM168X, quant_mode=RQ_MULTIPLIER_SHIFT, round_mode=ROUND_HALF_AWAY_FROM_ZERO,
-                 fuse_rq=False, multipliers=(1,), rshifts=(0,), out_zp=0, out_dtype=DT_I8, right_is_weight=True):
+                 fuse_rq=False, multipliers=(1,), rshifts=(0,), out_zp=0, out_dtype=DT_I8, right_is_weight=True,
+                 out_scale=1.0):
         self._mult = np.ascontiguousarray(multipliers, dtype=np.int64)
         self._rs = np.ascontiguousarray(rshifts, dtype=np.int64)
         self.attr = I8Attr(0, K, N, int(right_transpose), input_zp, right_zp, int(do_relu), relu_limit, chip,
                            quant_mode, round_mode, int(fuse_rq),
                            self._mult.ctypes.data_as(C.POINTER(C.c_int64)), self._mult.size,
                            self._rs.ctypes.data_as(C.POINTER(C.c_int64)), self._rs.size,
-                           out_zp, out_dtype, int(right_is_weight))
+                           out_zp, out_dtype, int(right_is_weight), float(out_scale))
         self.param = None
 
     def init(self, x, right, bias=None, multi=None):
@@ -618,9 +619,11 @@ def bench_read_launch(src, nbytes, sink, chunks_per_wave=4, stream=None):
 class RequantDesc:
     """Per-channel (torch int32 CUDA tensors) or scalar requantization parameters; shift > 0 shifts right."""
 
-    def __init__(self, quant_mode, round_mode, out_dtype=DT_I8, chip=CHIP_BM168X, multiplier=1, shift=0, zp=0):
+    def __init__(self, quant_mode, round_mode, out_dtype=DT_I8, chip=CHIP_BM168X, multiplier=1, shift=0, zp=0,
+                 only_scale=1.0):
         self.tensors = []
         self.c = RequantDescC(quant_mode, round_mode, chip, out_dtype, None, 1, None, 0, None, 0)
+        self.c.only_scale = float(only_scale)
         for name, v in (("multiplier", multiplier), ("shift", shift), ("zp", zp)):
             if hasattr(v, "data_ptr"):
                 import torch
