@@ -398,7 +398,9 @@ int mi_requant_launch(const int32_t *d_in, void *d_out, int64_t outer, int64_t c
 
 /* ============================================================================ */
 /* tpu.Cast  (lib/Dialect/Tpu/Interfaces/Common/Cast.cpp:35-200; requant()/dequant() of     */
-/* lib/Support/CastUtils.cpp:15-46).  BM168x branches incl. F32/F16 <-> F8 (:59-73); CV18xx: MI_UNSUPPORTED.    */
+/* lib/Support/CastUtils.cpp:15-46).  BM168x branches incl. F32/F16 <-> F8 (:59-73).  chip = MI_CHIP_CV18XX: the     */
+/* CV18xx branches (half to even whatever round_mode says :52-53, F32 -> BF16 by truncation :57-58, quantizing and */
+/* dequantizing through the chip's bf16_mul :82-84,:96-98, lib/Support/Float16.cpp:834-962); no 8-bit floats there. */
 /* ============================================================================ */
 enum { MI_ST_F32 = 0, MI_ST_BF16, MI_ST_F16, MI_ST_I8, MI_ST_U8, MI_ST_I16, MI_ST_U16, MI_ST_I32, MI_ST_U32,
        MI_ST_F8E4M3, MI_ST_F8E5M2 /* one byte; tpu.Cast from / to F32 and F16 only (Cast.cpp:59-73); not a storage

@@ -5,6 +5,7 @@
  */
 #include "oracle.h"
 
+#include <float.h>
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
@@ -1283,6 +1284,75 @@ static int st_is_float(int t) { return t == ORC_ST_F32 || t == ORC_ST_BF16 || t 
 
 /* requant(data, qtype), CastUtils.cpp:15-31: std::round is half away from zero;
  * 1.0 / scale is formed in double and narrowed to float */
+/* ---- CV18xx bf16 hardware model, lib/Support/Float16.cpp:834-962 -------------------------------------------- */
+static uint32_t cvi_hex(float v) {
+  uint32_t u;
+  memcpy(&u, &v, 4);
+  return u;
+}
+/* bf16_unnormal_value_fp32, :854-874 */
+static int cvi_unnormal(float *f, int trans_pos) {
+  int unnormal = 0;
+  const uint32_t u = cvi_hex(*f);
+  if ((u & 0x7F800000u) == 0) {
+    *f = 0;
+  } else if ((u & 0x7F800000u) == 0x7F800000u) {
+    *f = FLT_MAX;
+    unnormal = 1;
+  } else if ((u & 0xFF800000u) == 0xFF800000u) {
+    *f = trans_pos ? FLT_MAX : -FLT_MAX;
+    unnormal = 1;
+  } else if (*f == FLT_MAX || *f == -FLT_MAX) {
+    if (trans_pos)
+      *f = FLT_MAX;
+    unnormal = 1;
+  }
+  return unnormal;
+}
+/* check_max_inf_value, :897-905 */
+static int cvi_max_inf(float a) {
+  const uint32_t u = cvi_hex(a);
+  return (u & 0x7F800000u) == 0x7F800000u || (u & 0xFF800000u) == 0xFF800000u || (u & 0x7F7FFFFFu) == 0x7F7FFFFFu ||
+         (u & 0xFF7FFFFFu) == 0xFF7FFFFFu;
+}
+/* bf16_mul, :954-962, with bf16_cal_mac :907-940 (res starts at 0) */
+float orc_cvi_bf16_mul(float a, float b) {
+  int overflow = 0;
+  float res = 0.0f;
+  const int inf_a = cvi_max_inf(a), inf_b = cvi_max_inf(b);
+  if (!inf_a && (cvi_hex(a) & 0x7F800000u) == 0)
+    a = 0;
+  if (!inf_b && (cvi_hex(b) & 0x7F800000u) == 0)
+    b = 0;
+  if (inf_a || inf_b) {
+    res = ((cvi_hex(a) >> 31) ^ (cvi_hex(b) >> 31)) ? FLT_MAX : -FLT_MAX;
+    overflow = 1;
+  } else {
+    float mac = a * b;
+    if ((cvi_hex(mac) & 0x7F800000u) == 0) {
+      mac = 0;
+    } else if (cvi_max_inf(mac) || (cvi_hex(mac) & 0x7F7FFFFFu) == 0x7F7FFFFFu) {
+      res = FLT_MAX;
+      overflow = 1;
+    }
+    if (!overflow)
+      res += mac;
+  }
+  cvi_unnormal(&res, 1);
+  return orc_BF16(res, 1);
+}
+void orc_cvi_bf16_mul_n(const float *lhs, const float *rhs, float *out, int64_t n) {
+  for (int64_t i = 0; i < n; ++i)
+    out[i] = orc_cvi_bf16_mul(lhs[i], rhs[i]);
+}
+/* f32_to_bf16(src, false) on CV18xx, :764-766: the upper half of the pattern */
+static float cvi_bf16_truncate(float v) {
+  uint32_t u = cvi_hex(v) & 0xFFFF0000u;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
 static float cast_requant(float data, const orc_cast_attr *a) {
   const float inv = (float)(1.0 / a->scale);
   if (a->expressed == ORC_ST_F16)
@@ -1301,8 +1371,43 @@ static int st_bits(int t) {
 }
 static int st_unsigned(int t) { return t == ORC_ST_U8 || t == ORC_ST_U16 || t == ORC_ST_U32; }
 
+/* tpu::CastOp::inference under module::isCV18xx(), Cast.cpp:38-176 */
+static int orc_cast_cv18xx(const orc_cast_attr *a, const float *in, float *out, int64_t n) {
+  const int fin = st_is_float(a->in_type), fout = st_is_float(a->out_type);
+  const int rmode = ORC_ROUNDING_HALF_TO_EVEN; /* :52-53 */
+  if (a->in_type >= ORC_ST_F8E4M3 || a->out_type >= ORC_ST_F8E4M3)
+    return 1;
+  if (a->in_type == ORC_ST_F32 && a->out_type == ORC_ST_F16) {
+    for (int64_t i = 0; i < n; ++i) out[i] = orc_F16(in[i]);
+  } else if (a->in_type == ORC_ST_F32 && a->out_type == ORC_ST_BF16) { /* BF16(in, out, n, false): truncation */
+    for (int64_t i = 0; i < n; ++i) out[i] = cvi_bf16_truncate(in[i]);
+  } else if (a->out_quant && fin) { /* :82-84, :94 */
+    const float inv = orc_BF16((float)(1. / a->scale), 1);
+    for (int64_t i = 0; i < n; ++i) {
+      float v = orc_cvi_bf16_mul(cvi_bf16_truncate(in[i]), inv);
+      v += (float)a->zero_point;
+      out[i] = (float)orc_saturate_i64(orc_to_int_f32(v, rmode), st_bits(a->out_type), st_unsigned(a->out_type));
+    }
+  } else if (a->in_quant && fout) { /* cvi_int8_to_bf16 with is_tpu = true, :18-26 */
+    const float scale = orc_BF16((float)a->scale, 1);
+    const int zp = (int)a->zero_point;
+    for (int64_t i = 0; i < n; ++i)
+      out[i] = orc_cvi_bf16_mul(cvi_bf16_truncate(in[i]) - (float)zp, scale);
+  } else if (fin && (a->out_type == ORC_ST_I32 || a->out_type == ORC_ST_U32)) {
+    for (int64_t i = 0; i < n; ++i) out[i] = (float)orc_to_int_f32(in[i], rmode);
+  } else if (fin && !fout) {
+    for (int64_t i = 0; i < n; ++i)
+      out[i] = (float)orc_saturate_i64(orc_to_int_f32(in[i], rmode), st_bits(a->out_type), st_unsigned(a->out_type));
+  } else {
+    memcpy(out, in, (size_t)n * sizeof(float));
+  }
+  return 0;
+}
+
 int orc_cast(const orc_cast_attr *a, const float *in, float *out, int64_t n) {
   const int fin = st_is_float(a->in_type), fout = st_is_float(a->out_type);
+  if (a->is_cv18xx)
+    return orc_cast_cv18xx(a, in, out, n);
   if (a->in_type == ORC_ST_F32 && a->out_type == ORC_ST_F16) {          /* Cast.cpp:55-56 */
     for (int64_t i = 0; i < n; ++i) out[i] = orc_F16(in[i]);
   } else if (a->in_type == ORC_ST_F32 && a->out_type == ORC_ST_BF16) {  /* :57-58 */

@@ -257,8 +257,15 @@ typedef struct {
   int64_t zero_point;
   int expressed;              /* expressed type of the quantised side: ORC_ST_F32 / BF16 / F16 */
   int round_mode;
+  int is_cv18xx;              /* module::isCV18xx(): round half to even whatever round_mode says (Cast.cpp:52-53),
+                               * F32 -> BF16 by truncation (:57-58 with is_tpu = false), the quantizing and
+                               * dequantizing branches through bf16_mul (:82-84, :96-98) */
 } orc_cast_attr;
-/* returns 0, or -1 for a branch this restatement leaves out (CV18xx, fp8) */
+/* bf16_mul of the CV18xx hardware model, lib/Support/Float16.cpp:834-962: denormal operands and products count as zero,
+ * infinities / NaNs / +-FLT_MAX saturate, the product is rounded to bf16 by adding 0x7fff + lsb and truncating */
+float orc_cvi_bf16_mul(float lhs, float rhs);
+void orc_cvi_bf16_mul_n(const float *lhs, const float *rhs, float *out, int64_t n);
+/* returns 0, or 1 for a branch this restatement leaves out (8-bit floats outside F32 / F16) */
 int orc_cast(const orc_cast_attr *attr, const float *input, float *output, int64_t n);
 
 /* ---- tpu.A16MatMul with dynamic activation quantization (INT4 / INT8) -------- */

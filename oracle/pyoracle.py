@@ -69,7 +69,8 @@ class RqAttr(C.Structure):
 
 class CastAttr(C.Structure):
     _fields_ = [("in_type", C.c_int), ("out_type", C.c_int), ("in_quant", C.c_int), ("out_quant", C.c_int),
-                ("scale", C.c_double), ("zero_point", C.c_int64), ("expressed", C.c_int), ("round_mode", C.c_int)]
+                ("scale", C.c_double), ("zero_point", C.c_int64), ("expressed", C.c_int), ("round_mode", C.c_int),
+                ("is_cv18xx", C.c_int)]
 
 
 _lib = None
@@ -361,12 +362,22 @@ def requant_int(x, *, quant_mode, multiplier, rshift, round_mode=HALF_AWAY_FROM_
     return out
 
 
+def cvi_bf16_mul(a, b):
+    """bf16_mul of the CV18xx hardware model, elementwise on float32 arrays."""
+    a, b = _f32(a), _f32(b)
+    out = np.empty_like(a)
+    L = lib()
+    L.orc_cvi_bf16_mul_n.restype = None
+    L.orc_cvi_bf16_mul_n(_p(a, C.c_float), _p(b, C.c_float), _p(out, C.c_float), C.c_int64(a.size))
+    return out
+
+
 def cast(x, *, in_type, out_type, in_quant=False, out_quant=False, scale=1.0, zero_point=0, expressed=ST_F32,
-         round_mode=HALF_AWAY_FROM_ZERO):
-    """tpu.Cast on f32-valued data (BM168x branches)."""
+         round_mode=HALF_AWAY_FROM_ZERO, cv18xx=False):
+    """tpu.Cast on f32-valued data (BM168x branches; cv18xx=True: the CV18xx ones)."""
     x = _f32(x)
     attr = CastAttr(in_type, out_type, int(in_quant), int(out_quant), float(scale), int(zero_point), expressed,
-                    round_mode)
+                    round_mode, int(cv18xx))
     out = np.empty_like(x)
     rc = lib().orc_cast(C.byref(attr), _p(x, C.c_float), _p(out, C.c_float), C.c_int64(x.size))
     if rc != 0:

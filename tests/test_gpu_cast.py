@@ -109,7 +109,35 @@ def test_unsupported_branches_fail_loudly():
         M_.cast(x, in_type=clib.ST_BF16, out_type=clib.ST_F8E4M3)
     with pytest.raises(clib.BackendError):
         M_.cast(x, in_type=clib.ST_F8E5M2, out_type=clib.ST_I8)
-    with pytest.raises(clib.BackendError):
-        M_.cast(x, in_type=clib.ST_F32, out_type=clib.ST_I8, out_quant=True, scale=0.1, chip=clib.CHIP_CV18XX)
+    with pytest.raises(clib.BackendError):  # CV18xx has no 8-bit float branch
+        M_.cast(x, in_type=clib.ST_F32, out_type=clib.ST_F8E4M3, chip=clib.CHIP_CV18XX)
     with pytest.raises(clib.BackendError):
         M_.cast(x, in_type=clib.ST_F32, out_type=clib.ST_I8, out_quant=True, scale=0.0)
+
+
+CV_CASES = [  # in, out, in_quant, out_quant, scale, zp
+    ("F32", "BF16", False, False, 1.0, 0), ("F32", "F16", False, False, 1.0, 0),
+    ("F32", "I8", False, True, 0.0371, 3), ("BF16", "I8", False, True, 0.17, -7), ("F32", "U8", False, True, 0.11, 128),
+    ("I8", "BF16", True, False, 0.0123, 5), ("U8", "F32", True, False, 0.031, 120),
+    ("F32", "I32", False, False, 1.0, 0), ("F32", "I8", False, False, 1.0, 0), ("BF16", "U16", False, False, 1.0, 0),
+]
+
+
+@pytest.mark.parametrize("case", CV_CASES, ids=lambda c: "%s-%s%s" % (c[0], c[1], "q" if c[2] or c[3] else ""))
+def test_cv18xx_branches_against_oracle(orc, case):
+    """Cast.cpp under module::isCV18xx(): half to even whatever the attribute says, F32 -> BF16 by truncation, the
+    quantizing and dequantizing branches through the chip's bf16_mul; special values included."""
+    i, o, iq, oq, scale, zp = case
+    x = _inputs(i, orc)
+    if i in ("F32", "BF16"):
+        special = np.float32([np.inf, -np.inf, np.nan, 1e-40, -1e-40, 3.4028235e38, -3.4028235e38, 1e38, -2.5e38])
+        x = np.concatenate([x, S.bf16_to_f32(S.bf16_round(special)) if i == "BF16" else special])
+    kw = dict(in_type=getattr(clib, "ST_" + i), out_type=getattr(clib, "ST_" + o), in_quant=iq, out_quant=oq, scale=scale,
+              zero_point=zp)
+    got = M_.cast(x, round_mode=clib.ROUND_HALF_UP, chip=clib.CHIP_CV18XX, **kw)   # the attribute is ignored
+    okw = dict(in_type=getattr(orc, "ST_" + i), out_type=getattr(orc, "ST_" + o), in_quant=iq, out_quant=oq, scale=scale,
+               zero_point=zp)
+    want = orc.cast(x, round_mode=orc.HALF_UP, cv18xx=True, **okw)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    if (i, o) == ("F32", "BF16") or (oq and i == "F32"):   # and these branches do differ from the BM168x ones
+        assert not np.array_equal(want.view(np.uint32), orc.cast(x, round_mode=orc.HALF_TO_EVEN, **okw).view(np.uint32))

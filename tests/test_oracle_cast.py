@@ -132,3 +132,69 @@ def test_cast_from_8bit_floats_keeps_values(orc):
         assert np.array_equal(orc.cast(v, in_type=orc.ST_F8E4M3, out_type=o), v)
     with pytest.raises(RuntimeError):
         orc.cast(v, in_type=orc.ST_F8E4M3, out_type=orc.ST_I8)
+
+
+# ---- CV18xx -------------------------------------------------------------------------------------------------------
+def _cvi_round(x):
+    """add 0x7fff + lsb to the pattern, truncate, all-ones exponent -> 0x7f7f (Float16.cpp:725-761), with numpy integers"""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7fff + ((u >> 16) & 1)) & 0xffffffff
+    h = (u >> 16).astype(np.uint32)
+    h = np.where((h & 0x7f80) == 0x7f80, np.uint32(0x7f7f) | (h & 0x8000) * 0, h)
+    return (h << 16).astype(np.uint32).view(np.float32)
+
+
+def test_cvi_bf16_mul_is_the_rounded_float32_product_on_ordinary_values(orc):
+    """bf16_mul (Float16.cpp:907-962) away from its special cases: the float32 product, rounded to bf16 the chip's way.
+    numpy forms the product, an integer closed form does the rounding; neither shares code with the oracle."""
+    rng = np.random.default_rng(0)
+    a = (rng.standard_normal(200000) * 10.0 ** rng.integers(-6, 6, size=200000)).astype(np.float32)
+    b = (rng.standard_normal(200000) * 10.0 ** rng.integers(-6, 6, size=200000)).astype(np.float32)
+    want = _cvi_round(a * b)
+    got = orc.cvi_bf16_mul(a, b)
+    keep = np.abs(a * b) > 1e-30                       # stay clear of the denormal rule
+    assert np.array_equal(got[keep].view(np.uint32), want[keep].view(np.uint32))
+
+
+def test_cvi_bf16_mul_special_values(orc):
+    """Known answers worked out by hand from Float16.cpp:854-962: a denormal operand or product counts as zero; an
+    infinity, a NaN or +-FLT_MAX on either side saturates -- to +FLT_MAX whatever the signs, because the final
+    bf16_unnormal_value_fp32(.., trans_pos = 1) maps -FLT_MAX to +FLT_MAX -- and the chip's rounding then turns FLT_MAX
+    into the pattern 0x7f7f (3.3895e38); an overflowing finite product does the same."""
+    fmax = np.float32(3.4028235e38)
+    sat = np.uint32(0x7f7f0000)
+    cases = [(1e-40, 5.0, 0), (5.0, -1e-40, 0), (1e-20, 1e-20, 0),
+             (np.inf, 2.0, sat), (-np.inf, 2.0, sat), (2.0, -np.inf, sat), (np.nan, 1.0, sat), (fmax, 1.0, sat),
+             (-fmax, 1.0, sat), (1e30, 1e30, sat), (-1e30, 1e30, sat),
+             (1.5, 2.0, np.float32(3.0).view(np.uint32)), (-1.5, 2.0, np.float32(-3.0).view(np.uint32))]
+    a = np.float32([c[0] for c in cases])
+    b = np.float32([c[1] for c in cases])
+    got = orc.cvi_bf16_mul(a, b).view(np.uint32)
+    assert got.tolist() == [int(c[2]) for c in cases]
+
+
+def test_cast_cv18xx_branches_against_closed_forms(orc):
+    x = (np.random.default_rng(1).standard_normal(50000) * 30).astype(np.float32)
+    trunc = (x.view(np.uint32) & np.uint32(0xffff0000)).view(np.float32)
+    # F32 -> BF16 truncates (BF16(.., is_tpu = false), Cast.cpp:57-58 with Float16.cpp:764-766)
+    got = orc.cast(x, in_type=orc.ST_F32, out_type=orc.ST_BF16, cv18xx=True)
+    assert np.array_equal(got.view(np.uint32), trunc.view(np.uint32))
+    # quantizing: bf16_mul(truncate(x), BF16(1 / scale)) + zp, half to even whatever round_mode says
+    scale, zp = 0.0371, 3
+    inv = _cvi_round(np.float32([1.0 / scale]))[0]
+    v = _cvi_round(trunc * inv) + np.float32(zp)
+    want = np.clip(np.rint(v), -128, 127).astype(np.float32)       # numpy rint: half to even
+    got = orc.cast(x, in_type=orc.ST_F32, out_type=orc.ST_I8, out_quant=True, scale=scale, zero_point=zp,
+                   round_mode=orc.HALF_AWAY_FROM_ZERO, cv18xx=True)
+    assert np.array_equal(got, want)
+    # dequantizing: bf16_mul(q - zp, BF16(scale))
+    q = np.random.default_rng(2).integers(-128, 128, size=5000).astype(np.float32)
+    sc = _cvi_round(np.float32([0.0123]))[0]
+    want = _cvi_round((q - np.float32(5)) * sc)
+    got = orc.cast(q, in_type=orc.ST_I8, out_type=orc.ST_BF16, in_quant=True, scale=0.0123, zero_point=5, cv18xx=True)
+    nz = want != 0
+    assert np.array_equal(got[nz].view(np.uint32), want[nz].view(np.uint32)) and np.all(got[~nz] == 0)
+    # float -> integer without quantization: half to even
+    ties = np.float32([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 127.5, -128.5])
+    got = orc.cast(ties, in_type=orc.ST_F32, out_type=orc.ST_I8, round_mode=orc.HALF_UP, cv18xx=True)
+    assert got.tolist() == [0, 2, 2, 0, -2, -2, 127, -128]

@@ -1144,10 +1144,31 @@ int cast_scalars(const mi_cast_attr *a, float *inv_scale, float *scale) {
                    (f8_in && wide_out && !a->in_quant && !a->out_quant),
                MI_UNSUPPORTED, "mi_cast: an 8-bit float casts from and to F32 / F16 only");
   }
-  MI_REQUIRE(a->chip == MI_CHIP_BM168X, MI_UNSUPPORTED, "mi_cast: the CV18xx bf16 table arithmetic is not built");
+  MI_REQUIRE(a->chip == MI_CHIP_BM168X || a->chip == MI_CHIP_CV18XX, MI_BAD_ARGUMENT, "mi_cast: unknown chip");
   MI_REQUIRE(a->num_elem >= 0, MI_BAD_ARGUMENT, "mi_cast: negative element count");
   *inv_scale = 1.0f;
   *scale = (float)a->scale;
+  if (a->chip == MI_CHIP_CV18XX) {
+    // Cast.cpp:82-84, :18-26: BF16(1. / scale) and BF16(scale) with the chip's rounding (add 0x7fff + lsb, truncate,
+    // an all-ones exponent becomes 0x7f7f: Float16.cpp:725-761)
+    MI_REQUIRE(a->in_type < MI_ST_F8E4M3 && a->out_type < MI_ST_F8E4M3, MI_UNSUPPORTED,
+               "mi_cast: 8-bit floats are not handled for CV18xx");
+    auto cvi = [](float f) {
+      uint32_t u = fbits(f);
+      u += 0x7fffu + ((u >> 16) & 1u);
+      uint32_t h = u >> 16;
+      if ((h & 0x7f80u) == 0x7f80u)
+        h = 0x7f7fu;
+      return bits_f(h << 16);
+    };
+    if (a->out_quant && st_float(a->in_type)) {
+      MI_REQUIRE(a->scale != 0.0 && a->scale == a->scale, MI_BAD_ARGUMENT, "mi_cast: scale must be a nonzero number");
+      *inv_scale = cvi((float)(1. / a->scale));
+    } else if (a->in_quant && st_float(a->out_type)) {
+      *scale = cvi((float)a->scale);
+    }
+    return MI_SUCCESS;
+  }
   const bool quantizing = a->out_quant && st_float(a->in_type);
   const bool dequantizing = !quantizing && a->in_quant && st_float(a->out_type);
   if (quantizing || dequantizing)

@@ -16,7 +16,13 @@ struct CastArgs {
   float inv_scale;   // (float)(1.0 / scale), already rounded to the expressed type when that is 16-bit
   float scale;       // (float)scale, already rounded to the output type for a dequantizing cast
   float zero_point;  // (float)zero_point
+  int chip;          // MI_CHIP_CV18XX: the branches of Cast.cpp that go through the chip's bf16 hardware model
 };
+
+// f16_to_f32 as the reference writes it (lib/Support/Float16.cpp:776-786): every NaN code widens to 0xFFC00000
+__device__ __forceinline__ float f16_widen_ref(uint16_t h) {
+  return ((h & 0x7c00u) == 0x7c00u && (h & 0x03ffu) != 0) ? u2f(0xFFC00000u) : f16_bits_to_f32(h);
+}
 
 __device__ __forceinline__ int st_size(int t) {
   return (t == MI_ST_F32 || t == MI_ST_I32 || t == MI_ST_U32)
@@ -29,7 +35,7 @@ __device__ __forceinline__ float load_as_float(const void *p, int64_t i, int t) 
   switch (t) {
   case MI_ST_F32: return ((const float *)p)[i];
   case MI_ST_BF16: return bf16_bits_to_f32(((const uint16_t *)p)[i]);
-  case MI_ST_F16: return f16_bits_to_f32(((const uint16_t *)p)[i]);
+  case MI_ST_F16: return f16_widen_ref(((const uint16_t *)p)[i]);
   case MI_ST_I8: return (float)((const int8_t *)p)[i];
   case MI_ST_U8: return (float)((const uint8_t *)p)[i];
   case MI_ST_I16: return (float)((const int16_t *)p)[i];
@@ -60,7 +66,41 @@ __device__ __forceinline__ void store_from_float(void *p, int64_t i, int t, floa
 
 __device__ __forceinline__ bool st_is_float(int t) { return t == MI_ST_F32 || t == MI_ST_BF16 || t == MI_ST_F16; }
 __device__ __forceinline__ float BF16r(float v) { return bf16_bits_to_f32(f32_to_bf16_bm(v)); }
-__device__ __forceinline__ float F16r(float v) { return f16_bits_to_f32(f32_to_f16_ref(v)); }
+__device__ __forceinline__ float F16r(float v) { return f16_widen_ref(f32_to_f16_ref(v)); }
+
+// ---- CV18xx bf16 hardware model (lib/Support/Float16.cpp:834-962) ----
+__device__ __forceinline__ float CVIr(float v) { return bf16_bits_to_f32(f32_to_bf16_cvi(v)); }
+__device__ __forceinline__ float cvi_truncate(float v) { return u2f(f2u(v) & 0xffff0000u); }  // f32_to_bf16(v, false)
+__device__ __forceinline__ bool cvi_max_inf(float a) {  // check_max_inf_value
+  const uint32_t u = f2u(a);
+  return (u & 0x7F800000u) == 0x7F800000u || (u & 0x7F7FFFFFu) == 0x7F7FFFFFu;
+}
+// bf16_mul: denormal operands and products count as zero; infinities, NaNs and +-FLT_MAX saturate (to +FLT_MAX after
+// the final "unnormal" step, whatever the signs); the product is rounded by adding 0x7fff + lsb and truncating
+__device__ __forceinline__ float cvi_bf16_mul(float a, float b) {
+  const float FMAX = u2f(0x7F7FFFFFu);
+  const bool inf_a = cvi_max_inf(a), inf_b = cvi_max_inf(b);
+  if (!inf_a && (f2u(a) & 0x7F800000u) == 0)
+    a = 0.0f;
+  if (!inf_b && (f2u(b) & 0x7F800000u) == 0)
+    b = 0.0f;
+  float res;
+  if (inf_a || inf_b) {
+    res = FMAX;  // +-FLT_MAX by the signs, then bf16_unnormal_value_fp32(.., 1) makes either one +FLT_MAX
+  } else {
+    float mac = a * b;
+    if ((f2u(mac) & 0x7F800000u) == 0)
+      mac = 0.0f;
+    res = cvi_max_inf(mac) ? FMAX : 0.0f + mac;
+  }
+  // bf16_unnormal_value_fp32(&res, 1): zero exponent -> 0, all-ones exponent or +-FLT_MAX -> +FLT_MAX
+  const uint32_t u = f2u(res);
+  if ((u & 0x7F800000u) == 0)
+    res = 0.0f;
+  else if ((u & 0x7F800000u) == 0x7F800000u || (u & 0x7FFFFFFFu) == 0x7F7FFFFFu)
+    res = FMAX;
+  return CVIr(res);
+}
 
 __device__ __forceinline__ float clamp_to(int64_t v, int t) {
   int64_t lo, hi;
@@ -75,8 +115,31 @@ __device__ __forceinline__ float clamp_to(int64_t v, int t) {
   return (float)(v < lo ? lo : (v > hi ? hi : v));
 }
 
+// tpu::CastOp::inference under module::isCV18xx() (Cast.cpp:38-176): half to even everywhere (:52-53), F32 -> BF16 by
+// truncation (BF16(.., false), :57-58), quantizing through bf16_mul(BF16(x, false), BF16(1 / scale)) + zp (:82-84) and
+// dequantizing through bf16_mul(BF16(q, false) - zp, BF16(scale)) (cvi_int8_to_bf16, :18-26)
+__device__ __forceinline__ float cast_one_cv18xx(float x, const CastArgs &a) {
+  const bool fin = st_is_float(a.in_type), fout = st_is_float(a.out_type);
+  if (a.in_type == MI_ST_F32 && a.out_type == MI_ST_F16)
+    return F16r(x);
+  if (a.in_type == MI_ST_F32 && a.out_type == MI_ST_BF16)
+    return cvi_truncate(x);
+  if (a.out_quant && fin)
+    return clamp_to(to_int_f32(cvi_bf16_mul(cvi_truncate(x), a.inv_scale) + a.zero_point, MI_ROUND_HALF_TO_EVEN),
+                    a.out_type);
+  if (a.in_quant && fout)
+    return cvi_bf16_mul(cvi_truncate(x) - a.zero_point, a.scale);
+  if (fin && (a.out_type == MI_ST_I32 || a.out_type == MI_ST_U32))
+    return (float)to_int_f32(x, MI_ROUND_HALF_TO_EVEN);
+  if (fin && !fout)
+    return clamp_to(to_int_f32(x, MI_ROUND_HALF_TO_EVEN), a.out_type);
+  return x;
+}
+
 __device__ __forceinline__ float cast_one(float x, const CastArgs &a) {
   const bool fin = st_is_float(a.in_type), fout = st_is_float(a.out_type);
+  if (a.chip == MI_CHIP_CV18XX)
+    return cast_one_cv18xx(x, a);
   if (a.in_type == MI_ST_F32 && a.out_type == MI_ST_F16)
     return F16r(x);
   if (a.in_type == MI_ST_F32 && a.out_type == MI_ST_BF16)
@@ -143,6 +206,7 @@ int cast_launch(const mi_cast_attr *c, const void *d_in, void *d_out, int64_t n,
   a.inv_scale = inv_scale;
   a.scale = scale;
   a.zero_point = (float)c->zero_point;
+  a.chip = c->chip;
   int64_t blocks = (n + 256 * 8 - 1) / (256 * 8);
   if (blocks > 256 * 32)
     blocks = 256 * 32;
