@@ -90,7 +90,8 @@ typedef struct mi_a16mm_attr {
   int64_t M;            /* product of the input's leading dims (A16MatMul.cpp:31-35); may change per call */
   int64_t K, N;         /* input [M,K], output [M,N]; weight holds N output channels */
   int weight_bits;      /* getWeightBits(): 4 or 8 */
-  int w_transpose;      /* getWTranspose(): 1 = weight stored [N,K] (4-bit: [N,K/2] bytes) */
+  int w_transpose;      /* getWTranspose(): 1 = weight stored [N,K] (4-bit: [N,K/2] bytes); 0 = stored [K,N/2], 4-bit
+                         * only, scale / zp per stored row or per q_group_size elements along N */
   int q_group_size;     /* getQGroupSize() or module::getQuantGroupSize(); 0 = per output channel */
   int out_dtype;        /* MI_DT_BF16, or MI_DT_F16 when module::isF16Modes() */
   int chip;             /* MI_CHIP_* */
@@ -126,6 +127,13 @@ typedef struct mi_a16_weight_desc {
 int mi_a16_weight_create(mi_a16_weight **out, const mi_a16_weight_desc *desc, const void *weight,
                          const uint16_t *scale, const uint8_t *zp, const float *bias);
 void mi_a16_weight_destroy(mi_a16_weight *w);
+/* The same for w_transpose = false (A16MatMul.cpp:172-208 without the swap at :199-201), 4-bit only: weight = uint8
+ * [K, N/2] as stored (the reduction dimension is the stored row; even n in the low nibble), scale / zp = float
+ * [K, G] with G = N / q_group_size, or [K, 1] for q_group_size = 0 -- per stored row, as the reference indexes them.
+ * The result is used like any other weight set by mi_a16mm_launch (one set per launch; no dynamic quantization, no
+ * export).  A plain fp32 kernel serves it: the converter never emits this form, so it is built for completeness. */
+int mi_a16_weight_create_kn(mi_a16_weight **out, const mi_a16_weight_desc *desc, const uint8_t *weight,
+                            const float *scale, const float *zp, const float *bias);
 /* HBM bytes held by the packed set */
 size_t mi_a16_weight_bytes(const mi_a16_weight *w);
 

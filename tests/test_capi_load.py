@@ -27,14 +27,15 @@ def test_argument_errors_need_no_gpu():
     L = clib.lib()
     assert L.mi_a16mm_init(None, None) == clib.MI_BAD_ARGUMENT
     assert "null" in M.last_error()
-    # dynamic activation quantisation, w_transpose == false, odd bit widths: failure() -> caller keeps CPU path
+    # dynamic activation quantisation, untransposed 8-bit weights, odd bit widths: failure() -> caller keeps CPU path
     w = np.zeros((4, 64), np.float32)
     s = np.ones((4, 1), np.float32)
     z = np.zeros((4, 1), np.float32)
     for kw, code in ((dict(dynamic_quant=clib.DQ_F8E4M3, q_group_size=64), clib.MI_UNSUPPORTED),
                      (dict(dynamic_quant=clib.DQ_INT), clib.MI_BAD_ARGUMENT),        # no group size
                      (dict(dynamic_quant=clib.DQ_INT, q_group_size=32), clib.MI_UNSUPPORTED),
-                     (dict(w_transpose=False), clib.MI_UNSUPPORTED),
+                     (dict(w_transpose=False, weight_bits=8), clib.MI_UNSUPPORTED),   # untransposed: 4-bit only
+                     (dict(w_transpose=False, q_group_size=3), clib.MI_UNSUPPORTED),  # groups run along N there
                      (dict(weight_bits=3), clib.MI_UNSUPPORTED),
                      (dict(q_group_size=48), clib.MI_BAD_ARGUMENT),      # K % g != 0
                      (dict(q_group_size=16), clib.MI_UNSUPPORTED)):      # group size the kernels do not handle

@@ -116,3 +116,36 @@ def test_matmul_int8_nd_refuses_broadcast_batches_and_transposes():
         op.inference_nd(A, B)
     assert e.value.code == clib.MI_UNSUPPORTED
     op.deinit()
+
+
+@pytest.mark.parametrize("M,K,N,g", [(1, 256, 512, 0), (5, 512, 320, 32), (9, 128, 64, 64), (3, 64, 130, 0)])
+def test_untransposed_a16_weights_against_oracle(orc, M, K, N, g):
+    """tpu.A16MatMul with w_transpose = false: weight stored [K, N/2], parameters per stored row or per g elements
+    along N.  fp32 accumulation against the oracle's float64 one: 2e-5 of the output RMS, 16-bit outputs the reference
+    rounding of the kernel's fp32 value."""
+    m = pkg()
+    cmp = pkg("compare")
+    rng = np.random.default_rng(M * 7 + g)
+    q = rng.integers(0, 16, size=(K, N)).astype(np.uint8)
+    packed = (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.float32)
+    G = N // g if g else 1
+    scale = (np.abs(rng.standard_normal((K, G))) * 0.02 + 1e-3).astype(np.float32)
+    zp = rng.integers(0, 16, size=(K, G)).astype(np.float32)
+    x = S.bf16_to_f32(S.bf16_round(rng.standard_normal((M, K)).astype(np.float32)))
+    bias = rng.standard_normal(N).astype(np.float32)
+    want, pre = orc.a16matmul(x, packed, scale, zp, bias, M=M, K=K, N=N, weight_bits=4, q_group_size=g,
+                              w_transpose=False, gemm_kind=orc.GEMM_F64ACC)
+    op = m.A16MatMul(K=K, N=N, weight_bits=4, q_group_size=g, w_transpose=False).init(packed, scale, zp, bias)
+    got = op.inference(x)
+    got1 = op.inference(x[:1])
+    op.deinit()
+    rms = float(np.sqrt(np.mean(pre.astype(np.float64) ** 2)))
+    assert cmp.max_abs_over_rms(got, want) <= max(1e-2, 2.0 ** -7 * float(np.max(np.abs(want))) / rms)
+    assert np.mean(got != want) < 0.01 and np.array_equal(got1, got[:1])
+    # one-hot activations read single dequantized weights back exactly (rounded to bf16 by the op's output rounding)
+    eye = np.eye(K, dtype=np.float32)
+    rep = g if g else N
+    deq = (q.astype(np.float32) - np.repeat(zp, rep, axis=1)) * np.repeat(scale, rep, axis=1)
+    op = m.A16MatMul(K=K, N=N, weight_bits=4, q_group_size=g, w_transpose=False).init(packed, scale, zp, None)
+    assert np.array_equal(op.inference(eye), S.bf16_to_f32(S.bf16_round(deq)))
+    op.deinit()

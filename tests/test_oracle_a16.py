@@ -94,3 +94,26 @@ def test_gemm_standins_against_float64():
     want = (Ai.astype(np.int64) @ Bi.astype(np.int64)).astype(np.float32)
     for kind in (O.GEMM_F32, O.GEMM_F64ACC, O.GEMM_FAST):
         assert np.array_equal(O.sgemm(Ai, Bi, None, kind), want)
+
+
+@pytest.mark.parametrize("g", [0, 8, 32])
+def test_untransposed_weight_against_float64(orc, g):
+    """w_transpose = false (A16MatMul.cpp:172-208 without the swap): weight stored [K, N/2], one scale / zero point per
+    stored row k (g = 0) or per g consecutive elements of the flattened [K, N] matrix, i.e. per (k, n // g).  Unpacked
+    and multiplied here in float64, independently of the oracle's dequantizer."""
+    M, K, N = 5, 48, 64
+    rng = np.random.default_rng(20 + g)
+    q = rng.integers(0, 16, size=(K, N)).astype(np.uint8)
+    packed = (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.float32)            # even n in the low nibble
+    G = N // g if g else 1
+    scale = (np.abs(rng.standard_normal((K, G))) * 0.02 + 1e-3).astype(np.float32)
+    zp = rng.integers(0, 16, size=(K, G)).astype(np.float32)
+    x = S.bf16_to_f32(S.bf16_round(rng.standard_normal((M, K)).astype(np.float32)))
+    bias = rng.standard_normal(N).astype(np.float32)
+    out, pre = orc.a16matmul(x, packed, scale, zp, bias, M=M, K=K, N=N, weight_bits=4, q_group_size=g, w_transpose=False,
+                             gemm_kind=orc.GEMM_F64ACC)
+    rep = g if g else N
+    deq = ((q.astype(np.float32) - np.repeat(zp, rep, axis=1)) * np.repeat(scale, rep, axis=1)).astype(np.float64)
+    ref = x.astype(np.float64) @ deq + bias
+    assert np.max(np.abs(pre - ref)) <= 1e-6 * np.sqrt(np.mean(ref ** 2)) * np.sqrt(K)
+    assert np.array_equal(out, S.bf16_to_f32(S.bf16_round(pre)))

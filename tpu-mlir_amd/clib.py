@@ -17,7 +17,7 @@ ST_F32, ST_BF16, ST_F16, ST_I8, ST_U8, ST_I16, ST_U16, ST_I32, ST_U32, ST_F8E4M3
 EXPORTS = [
     "mi_version", "mi_last_error", "mi_device_count",
     "mi_a16mm_init", "mi_a16mm_inference", "mi_a16mm_deinit",
-    "mi_a16_weight_create", "mi_a16_weight_destroy", "mi_a16_weight_bytes", "mi_a16mm_launch",
+    "mi_a16_weight_create", "mi_a16_weight_create_kn", "mi_a16_weight_destroy", "mi_a16_weight_bytes", "mi_a16mm_launch",
     "mi_a16mm_launch_noalloc",
     "mi_a16mm_launch_group", "mi_a16mm_dq_launch", "mi_a16mm_dq_type_launch", "mi_matmul_dq_launch",
     "mi_matmul_dq_inference", "mi_f8mm_inference", "mi_f8mm_launch", "mi_f8mm_e5m2_launch",
@@ -193,6 +193,7 @@ def lib():
         L.mi_llm_unpack.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
                                     C.c_void_p, C.c_void_p]
         L.mi_a16_weight_destroy.restype = None
+        L.mi_a16_weight_create_kn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_launch_noalloc.argtypes = L.mi_a16mm_launch.argtypes
         L.mi_top_a16_weight_create.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p,

@@ -115,6 +115,11 @@ void a16_free(mi_a16_weight *w) {
   (void)hipFree(w->sz_t);
   (void)hipFree(w->nzs_t);
   (void)hipFree(w->bias);
+  (void)hipFree(w->kn_w);
+  (void)hipFree(w->kn_scale);
+  (void)hipFree(w->kn_zp);
+  w->kn_w = nullptr;
+  w->kn_scale = w->kn_zp = nullptr;
   w->qweight = nullptr;
   w->scale_t = nullptr;
   w->sz_t = nullptr;
@@ -732,6 +737,10 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
   // no rows: nothing to read or write (an empty tensor's data pointer may well be null)
   MI_REQUIRE(M == 0 || (d_x && d_ys), MI_BAD_ARGUMENT, "mi_a16mm_launch: null activation or output pointer");
   const mi_a16_weight *w = ws[0];
+  if (w && w->kn) {  // w_transpose = false: its own kernel, one weight set per launch
+    MI_REQUIRE(n == 1, MI_UNSUPPORTED, "mi_a16mm_launch_group: untransposed weights are launched one set at a time");
+    return a16_kn_launch(w, d_x, M, d_ys ? d_ys[0] : nullptr, d_y32s ? d_y32s[0] : nullptr, stream);
+  }
   int64_t total_rb = 0;
   SkinnyArgs a;
   for (int i = 0; i < MAX_SEG; ++i) {

@@ -274,6 +274,7 @@ int mi_a16_weight_export(const mi_a16_weight *w, void *blob, size_t capacity) {
   uint8_t *p = (uint8_t *)blob;
   memcpy(p, &h, sizeof(h));
   p += sizeof(h);
+  MI_REQUIRE(!w->kn, MI_UNSUPPORTED, "mi_a16_weight_export: an untransposed weight has no packed form");
   MI_HIP(hipMemcpy(p, w->qweight, h.packed_bytes, hipMemcpyDeviceToHost));
   p += h.packed_bytes;
   if (w->bits == 4) {
@@ -439,7 +440,6 @@ int mi_a16mm_init(const mi_a16mm_attr *attr, mi_infer_param *p) {
                "mi_a16mm_init: dynamic quantization is handled for K % 128 == 0 and groups of 32, 64 or k*128 (integer "
                "codes with 8-bit weights: up to 512, where the reference's f32 group product stops being exact)");
   }
-  MI_REQUIRE(attr->w_transpose, MI_UNSUPPORTED, "mi_a16mm_init: only w_transpose weights ([N,K]) are handled");
   MI_REQUIRE(attr->weight_bits == 4 || attr->weight_bits == 8, MI_UNSUPPORTED, "mi_a16mm_init: weight_bits");
   MI_REQUIRE(attr->out_dtype == MI_DT_BF16 || attr->out_dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_a16mm_init: out_dtype");
   const float *weight = p->inputs[1], *scale = p->inputs[2], *zp = p->inputs[3];
@@ -447,6 +447,42 @@ int mi_a16mm_init(const mi_a16mm_attr *attr, mi_infer_param *p) {
   MI_REQUIRE(weight && scale && zp, MI_BAD_ARGUMENT, "mi_a16mm_init: weight, scale and zp must not be None");
   const int64_t K = attr->K, N = attr->N;
   MI_REQUIRE(K > 0 && N > 0, MI_BAD_ARGUMENT, "mi_a16mm_init: bad shape");
+  if (!attr->w_transpose) {
+    // A16MatMul.cpp:172-208 without the swap: weight stored [K, N/2], parameters per stored row k or per run of
+    // q_group_size elements of the flattened [K, N] matrix; floats as the interpreter holds them, used as they are
+    MI_REQUIRE(dq == MI_DQ_NONE, MI_UNSUPPORTED, "mi_a16mm_init: dynamic quantization needs w_transpose weights");
+    MI_REQUIRE(N % 2 == 0, MI_UNSUPPORTED, "mi_a16mm_init: an untransposed 4-bit weight needs an even N");
+    const int64_t nw = K * (N / 2);
+    std::vector<uint8_t> wbytes((size_t)nw);
+    for (int64_t i = 0; i < nw; ++i) {
+      const float v = weight[i];
+      MI_REQUIRE(v == truncf(v) && v >= 0.f && v <= 255.f, MI_UNSUPPORTED,
+                 "mi_a16mm_init: weight is not a packed byte value");
+      wbytes[(size_t)i] = (uint8_t)(int)v;
+    }
+    mi_a16_weight_desc d;
+    d.K = K;
+    d.N = N;
+    d.weight_bits = attr->weight_bits;
+    d.weight_signed = 0;
+    d.q_group_size = attr->q_group_size;
+    d.dtype = attr->out_dtype;
+    d.chip = attr->chip;
+    A16Handle *h = new (std::nothrow) A16Handle();
+    MI_REQUIRE(h, MI_HIP_ERROR, "mi_a16mm_init: out of host memory");
+    int rc = mi_a16_weight_create_kn(&h->w, &d, wbytes.data(), scale, zp, bias);
+    if (rc == MI_SUCCESS) {
+      hipError_t e = hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking);
+      if (e != hipSuccess)
+        rc = hip_fail(e, "hipStreamCreateWithFlags", __FILE__, __LINE__);
+    }
+    if (rc != MI_SUCCESS) {
+      delete h;
+      return rc;
+    }
+    p->handle = h;
+    return MI_SUCCESS;
+  }
   const int g = attr->q_group_size;
   MI_REQUIRE(g == 0 || (g > 0 && K % g == 0), MI_BAD_ARGUMENT, "mi_a16mm_init: K is not a multiple of q_group_size");
   MI_REQUIRE(K % 8 == 0 && group_size_supported(attr->weight_bits, g, K), MI_UNSUPPORTED,

@@ -95,6 +95,11 @@ struct mi_a16_weight {
   float *nzs_t = nullptr;
   float *bias = nullptr;  // [N] or null
   size_t bytes = 0;
+  // w_transpose = false (a16_kn.hip): the weight as stored, [K][N/2] bytes, with float scale / zero point [K][G]
+  // (G = N / g, or 1); none of the tile arrays above exist then
+  bool kn = false;
+  void *kn_w = nullptr;
+  float *kn_scale = nullptr, *kn_zp = nullptr;
 };
 
 namespace mi {
@@ -103,6 +108,7 @@ int a16_pack(mi_a16_weight *w, const void *h_weight, int weight_signed, const ui
 void a16_free(mi_a16_weight *w);
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                hipStream_t stream);
+int a16_kn_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32, hipStream_t st);
 // a caller-provided scratch area that a launch must make do with (instead of the stream's growable buffer)
 struct A16Scratch {
   void *ptr;
