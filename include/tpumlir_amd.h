@@ -331,8 +331,11 @@ int mi_matmul_parse_param(const mi_matmul_shapes *shapes, int right_transpose, i
 /* mi_i8mm_inference with M, K, N and the batch taken from the shapes instead of attr (whose M, K, N are ignored):
  * batch matmuls [batch, M, K] x [batch, K, N] (right stored [batch, N, K] under right_transpose) with one bias[N] and
  * the requantization of the op (MatMul.cpp:598-729; on CV18xx multipliers[b] / rshifts[b] belong to batch b when one
- * per batch is given, :638-664).  left_transpose, output_transpose and hdim_is_batch are MI_UNSUPPORTED, and so are
- * operands that do not hold exactly batch matrices each (the reference's quantized path has no other broadcasting).
+ * per batch is given, :638-664).  left_transpose, output_transpose and hdim_is_batch re-lay operands and output as
+ * MatMul::run does (lib/Support/Dnnl/MatMul.cpp:167-239: per-batch matrix transposes, or the (B0, M, B1, K) x
+ * (B0, K, B1, N) = (B0, M, B1, N) layouts of MatMul.cpp:58-62 under hdim_is_batch); a per-channel multi operand then has
+ * one entry per element of the OUTPUT's last dimension (:666-668).  Operands that do not hold exactly batch matrices
+ * each are MI_UNSUPPORTED (the reference's quantized path has no other broadcasting).
  * p->handle is released by mi_i8mm_deinit. */
 int mi_i8mm_inference_nd(const mi_i8mm_attr *attr, const mi_matmul_shapes *shapes, mi_infer_param *p);
 

@@ -1054,6 +1054,64 @@ static int64_t arr_at(const int64_t *v, int n, int64_t i, int64_t dflt) {
   return n == 1 ? v[0] : v[i < n ? i : n - 1];
 }
 
+/* The requantization of tpu::MatMulOp::inference (MatMul.cpp:636-727) over `num` consecutive outputs whose last
+ * dimension is n_last; mult0 / rs0: the scalar multiplier and rshift in force (on CV18xx those of this batch). */
+static int i8mm_requant_flat(const orc_i8mm_attr *a, const float *multi, float *output, int64_t num, int64_t n_last,
+                             int64_t mult0, int64_t rshift0) {
+  if (a->is_cv18xx) {
+    /* MatMul.cpp:638-664 */
+    for (int64_t j = 0; j < num; j++) {
+      int64_t v = orc_apply_multiplier_and_rshift(
+          (int64_t)output[j], mult0, rshift0, a->quant_mode,
+          ORC_ROUNDING_HALF_AWAY_FROM_ZERO, 1);
+      output[j] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+    }
+    return 0;
+  }
+  /* MatMul.cpp:665-727 */
+  if (a->quant_mode == ORC_RQ_ONLY_SCALE) {
+    /* MatMul.cpp:673-695; the fused (per-channel) flavour asserts (:674-676) */
+    if (a->fuse_rq)
+      return 1;
+    const float scale = (float)a->out_scale;
+    for (int64_t i = 0; i < num; i++) {
+      float v = output[i] * scale;
+      output[i] = (float)orc_saturate_i64((int64_t)(int32_t)roundf(v) + a->out_zp, a->out_bits, a->out_unsigned);
+    }
+  } else if (a->quant_mode == ORC_RQ_TFLITE_LSHIFT || a->quant_mode == ORC_RQ_TFLITE) {
+    for (int64_t i = 0; i < num; i++) {
+      int64_t v = (int64_t)orc_multiply_by_quantized_multiplier(
+                      (int32_t)output[i], (int32_t)mult0, -(int32_t)rshift0,
+                      ORC_ROUNDING_HALF_AWAY_FROM_ZERO) +
+                  a->out_zp;
+      output[i] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+    }
+  } else if (a->quant_mode == ORC_RQ_MULTIPLIER_SHIFT) {
+    if (a->fuse_rq) {
+      if (!multi)
+        return 1;
+      for (int64_t i = 0; i < num; i++) {
+        int64_t v = orc_apply_multiplier_and_rshift(
+                        (int64_t)output[i], (int64_t)multi[i % n_last], rshift0,
+                        ORC_RQ_MULTIPLIER_SHIFT, ORC_ROUNDING_HALF_UP, 0) +
+                    a->out_zp;
+        output[i] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+      }
+    } else {
+      for (int64_t i = 0; i < num; i++) {
+        int64_t v = orc_apply_multiplier_and_rshift(
+                        (int64_t)output[i], mult0, rshift0,
+                        ORC_RQ_MULTIPLIER_SHIFT, ORC_ROUNDING_HALF_UP, 0) +
+                    a->out_zp;
+        output[i] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
+      }
+    }
+  } else {
+    return 1;
+  }
+  return 0;
+}
+
 int orc_matmul_int8(const orc_i8mm_attr *a, const float *const *inputs,
                     float *output, float *acc_out) {
   if (!a || !inputs || !inputs[0] || !inputs[1])
@@ -1094,63 +1152,8 @@ int orc_matmul_int8(const orc_i8mm_attr *a, const float *const *inputs,
   if (a->out_kind == 1)
     return 0; /* int32 storage: no epilogue (MatMul.cpp:605-607,636) */
 
-  int64_t num = M * N;
-  if (a->is_cv18xx) {
-    /* MatMul.cpp:638-664, batch == 1 */
-    int64_t mult = arr_at(a->multipliers, a->n_multipliers, 0, 1);
-    int64_t rs = arr_at(a->rshifts, a->n_rshifts, 0, 0);
-    for (int64_t j = 0; j < num; j++) {
-      int64_t v = orc_apply_multiplier_and_rshift(
-          (int64_t)output[j], mult, rs, a->quant_mode,
-          ORC_ROUNDING_HALF_AWAY_FROM_ZERO, 1);
-      output[j] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
-    }
-    return 0;
-  }
-  /* MatMul.cpp:665-727 */
-  int64_t rshift0 = arr_at(a->rshifts, a->n_rshifts, 0, 0);
-  int64_t mult0 = arr_at(a->multipliers, a->n_multipliers, 0, 1);
-  if (a->quant_mode == ORC_RQ_ONLY_SCALE) {
-    /* MatMul.cpp:673-695; the fused (per-channel) flavour asserts (:674-676) */
-    if (a->fuse_rq)
-      return 1;
-    const float scale = (float)a->out_scale;
-    for (int64_t i = 0; i < num; i++) {
-      float v = output[i] * scale;
-      output[i] = (float)orc_saturate_i64((int64_t)(int32_t)roundf(v) + a->out_zp, a->out_bits, a->out_unsigned);
-    }
-  } else if (a->quant_mode == ORC_RQ_TFLITE_LSHIFT || a->quant_mode == ORC_RQ_TFLITE) {
-    for (int64_t i = 0; i < num; i++) {
-      int64_t v = (int64_t)orc_multiply_by_quantized_multiplier(
-                      (int32_t)output[i], (int32_t)mult0, -(int32_t)rshift0,
-                      ORC_ROUNDING_HALF_AWAY_FROM_ZERO) +
-                  a->out_zp;
-      output[i] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
-    }
-  } else if (a->quant_mode == ORC_RQ_MULTIPLIER_SHIFT) {
-    if (a->fuse_rq) {
-      if (!inputs[3])
-        return 1;
-      for (int64_t i = 0; i < num; i++) {
-        int64_t v = orc_apply_multiplier_and_rshift(
-                        (int64_t)output[i], (int64_t)inputs[3][i % N], rshift0,
-                        ORC_RQ_MULTIPLIER_SHIFT, ORC_ROUNDING_HALF_UP, 0) +
-                    a->out_zp;
-        output[i] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
-      }
-    } else {
-      for (int64_t i = 0; i < num; i++) {
-        int64_t v = orc_apply_multiplier_and_rshift(
-                        (int64_t)output[i], mult0, rshift0,
-                        ORC_RQ_MULTIPLIER_SHIFT, ORC_ROUNDING_HALF_UP, 0) +
-                    a->out_zp;
-        output[i] = (float)orc_saturate_i64(v, a->out_bits, a->out_unsigned);
-      }
-    }
-  } else {
-    return 1;
-  }
-  return 0;
+  return i8mm_requant_flat(a, inputs[3], output, M * N, N, arr_at(a->multipliers, a->n_multipliers, 0, 1),
+                           arr_at(a->rshifts, a->n_rshifts, 0, 0));
 }
 
 /* ======================================================================== */
@@ -1823,42 +1826,110 @@ int orc_matmul_parse_param(const int64_t *a_shape, int a_dims, const int64_t *b_
   return 0;
 }
 
+/* tensor_hw_transpose / tensor_hc_transpose, include/tpu_mlir/Support/MathUtils.h:198-228 */
+static void orc_hw_transpose4(float *dst, const float *src, int64_t N, int64_t C, int64_t H, int64_t W) {
+  for (int64_t nc = 0; nc < N * C; nc++)
+    for (int64_t w = 0; w < W; w++)
+      for (int64_t h = 0; h < H; h++)
+        dst[nc * H * W + w * H + h] = src[nc * H * W + h * W + w];
+}
+static void orc_hc_transpose4(float *dst, const float *src, int64_t N, int64_t C, int64_t H, int64_t W) {
+  for (int64_t n = 0; n < N; n++)
+    for (int64_t h = 0; h < H; h++)
+      for (int64_t c = 0; c < C; c++)
+        for (int64_t w = 0; w < W; w++)
+          dst[w + c * W + h * C * W + n * C * H * W] = src[w + h * W + c * H * W + n * C * H * W];
+}
+
 int orc_matmul_int8_nd(const orc_i8mm_attr *attr, const int64_t *a_shape, int a_dims, const int64_t *b_shape,
-                       int b_dims, const int64_t *o_shape, int o_dims, int chip, const float *const *inputs,
-                       float *output) {
+                       int b_dims, const int64_t *o_shape, int o_dims, int left_transpose, int output_transpose,
+                       int hdim_is_batch, int chip, const float *const *inputs, float *output) {
   orc_matmul_param p;
-  if (!attr || !inputs || !output)
+  if (!attr || !inputs || !inputs[0] || !inputs[1] || !output || o_dims < 1)
     return 1;
-  if (orc_matmul_parse_param(a_shape, a_dims, b_shape, b_dims, o_shape, o_dims, attr->right_transpose, 0, 0, 0, chip, &p))
+  if (orc_matmul_parse_param(a_shape, a_dims, b_shape, b_dims, o_shape, o_dims, attr->right_transpose, left_transpose,
+                             output_transpose, hdim_is_batch, chip, &p))
     return 1;
-  const int64_t full_batch = p.batch * p.batch_low;
+  const int64_t B = p.batch, BL = p.batch_low, FB = B * BL, M = p.M, K = p.K, N = p.N;
   /* the operands must hold exactly batch matrices each: the reference's quantized path passes no shapes to
    * MatMul::setup, so it has no broadcasting beyond what parseParam folded into M */
-  int64_t a_num = 1, b_num = 1;
+  int64_t a_num = 1, b_num = 1, o_num = 1;
   for (int i = 0; i < a_dims; i++)
     a_num *= a_shape[i];
   for (int i = 0; i < b_dims; i++)
     b_num *= b_shape[i];
-  if (a_num != full_batch * p.M * p.K || b_num != full_batch * p.K * p.N)
+  for (int i = 0; i < o_dims; i++)
+    o_num *= o_shape[i];
+  if (a_num != FB * M * K || b_num != FB * K * N || o_num != FB * M * N)
     return 1;
-  for (int64_t b = 0; b < full_batch; b++) {
-    orc_i8mm_attr one = *attr;
-    one.M = p.M;
-    one.K = p.K;
-    one.N = p.N;
-    int64_t mult_b, rs_b;
-    if (attr->is_cv18xx && attr->n_multipliers == full_batch && attr->n_rshifts == full_batch && full_batch > 1) {
-      /* MatMul.cpp:645-663: one multiplier / rshift per batch when the right operand is a weight */
-      mult_b = attr->multipliers[b];
-      rs_b = attr->rshifts[b];
-      one.multipliers = &mult_b;
-      one.n_multipliers = 1;
-      one.rshifts = &rs_b;
-      one.n_rshifts = 1;
-    }
-    const float *ins[4] = {inputs[0] + b * p.M * p.K, inputs[1] + b * p.K * p.N, inputs[2], inputs[3]};
-    if (orc_matmul_int8(&one, ins, output + b * p.M * p.N, NULL))
-      return 1;
+  float *left = (float *)malloc(sizeof(float) * (size_t)(a_num ? a_num : 1));
+  float *right = (float *)malloc(sizeof(float) * (size_t)(b_num ? b_num : 1));
+  float *tmp = (float *)malloc(sizeof(float) * (size_t)(o_num ? o_num : 1));
+  if (!left || !right || !tmp) {
+    free(left);
+    free(right);
+    free(tmp);
+    return 1;
   }
-  return 0;
+  /* MatMul::run, lib/Support/Dnnl/MatMul.cpp:167-201 */
+  if (p.right_transpose) {
+    if (p.hdim_is_batch)
+      orc_hc_transpose4(right, inputs[1], B, K, BL, N);
+    else
+      orc_hw_transpose4(right, inputs[1], 1, B, N, K);
+  } else {
+    memcpy(right, inputs[1], sizeof(float) * (size_t)b_num);
+  }
+  if (p.left_transpose) {
+    if (p.hdim_is_batch)
+      orc_hc_transpose4(left, inputs[0], B, M, BL, K);
+    else
+      orc_hw_transpose4(left, inputs[0], 1, B, K, M);
+  } else {
+    memcpy(left, inputs[0], sizeof(float) * (size_t)a_num);
+  }
+  if (attr->right_zp != 0)
+    for (int64_t i = 0; i < b_num; i++)
+      right[i] = right[i] - (float)attr->right_zp;
+  if (attr->input_zp != 0)
+    for (int64_t i = 0; i < a_num; i++)
+      left[i] = left[i] - (float)attr->input_zp;
+  for (int64_t b = 0; b < FB; b++)
+    run_gemm(attr->gemm_kind, left + b * M * K, right + b * K * N, inputs[2], output + b * M * N, M, K, N);
+  free(left);
+  free(right);
+  /* post_relu, lib/Support/Dnnl/DnnlUtils.cpp:15-25 */
+  if (attr->do_relu)
+    for (int64_t i = 0; i < o_num; i++) {
+      float v = output[i] > 0.0f ? output[i] : 0.0f;
+      if (attr->relu_limit > 0.0 && v > (float)attr->relu_limit)
+        v = (float)attr->relu_limit;
+      output[i] = v;
+    }
+  /* Dnnl/MatMul.cpp:228-238 */
+  if (p.output_transpose) {
+    if (p.hdim_is_batch)
+      orc_hc_transpose4(tmp, output, B, BL, M, N);
+    else
+      orc_hw_transpose4(tmp, output, B, BL, M, N);
+    memcpy(output, tmp, sizeof(float) * (size_t)o_num);
+  }
+  free(tmp);
+  if (attr->out_kind == 1)
+    return 0; /* int32 storage: no epilogue (MatMul.cpp:605-607,636) */
+  if (attr->is_cv18xx) {
+    /* MatMul.cpp:638-664: one multiplier / rshift per batch when the right operand is a weight, else the first */
+    const int per_batch = attr->n_multipliers == FB && attr->n_rshifts == FB && FB > 1;
+    for (int64_t b = 0; b < FB; b++) {
+      const int64_t mult = arr_at(attr->multipliers, attr->n_multipliers, per_batch ? b : 0, 1);
+      const int64_t rs = arr_at(attr->rshifts, attr->n_rshifts, per_batch ? b : 0, 0);
+      if (i8mm_requant_flat(attr, inputs[3], output + b * M * N, M * N, N, mult, rs))
+        return 1;
+    }
+    return 0;
+  }
+  /* MatMul.cpp:666-668: the per-channel operand is indexed by the OUTPUT's last dimension */
+  return i8mm_requant_flat(attr, inputs[3], output, o_num, o_shape[o_dims - 1],
+                           arr_at(attr->multipliers, attr->n_multipliers, 0, 1),
+                           arr_at(attr->rshifts, attr->n_rshifts, 0, 0));
 }

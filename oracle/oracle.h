@@ -58,9 +58,12 @@
  *                                (tests/test_oracle_top_a16.py)
  *   orc_matmul_parse_param       the six cases the reference documents above the function (MatMul.cpp:17-22) and
  *                                numpy.matmul's broadcasting shapes (tests/test_oracle_matmul_nd.py); the
- *                                hdim_is_batch branch only as far as the layout comment at :58-62 goes: its K / N
- *                                without right_transpose are PARITY UNPINNED
- *   orc_matmul_int8_nd           numpy.matmul on int64 per batch + the pinned scalar requantization
+ *                                hdim_is_batch branch on the two layouts the comment at :58-62 documents
+ *   orc_matmul_int8_nd           numpy.matmul on int64 per batch + the pinned scalar requantization; the transposes
+ *                                against numpy.swapaxes, hdim_is_batch against numpy.einsum on the documented
+ *                                layouts (MatMul.cpp:58-62).  BM1684X family with a transposed right operand and
+ *                                K != N (parseParam swaps K and N there, MatMul::run does not): follows the code
+ *                                literally, PARITY UNPINNED
  *   orc_a16_dequant              one-hot activations recover nibble order,
  *                                group indexing and scale layout
  *   orc_sgemm_*                  float64 reference with the standard bound
@@ -368,13 +371,15 @@ typedef struct {
 int orc_matmul_parse_param(const int64_t *a_shape, int a_dims, const int64_t *b_shape, int b_dims,
                            const int64_t *o_shape, int o_dims, int right_transpose, int left_transpose,
                            int output_transpose, int hdim_is_batch, int chip, orc_matmul_param *out);
-/* tpu.MatMul (quantized) on operands of any rank the plain branch of parseParam covers (no hdim_is_batch, no left or
- * output transpose): batch matmuls [batch, M, K] x [batch, K, N] (right stored [batch, N, K] under right_transpose),
- * one bias[N] for all, then the requantization of orc_matmul_int8 over the whole output; on CV18xx the multiplier /
- * rshift of batch b when one per batch is given (MatMul.cpp:638-664).  attr->M/K/N are ignored. */
+/* tpu.MatMul (quantized) on operands of any rank: tpu::MatMulOp::inference (MatMul.cpp:598-729) with MatMul::run's
+ * operand and output transposes (lib/Support/Dnnl/MatMul.cpp:167-239: tensor_hw_transpose per batch, or
+ * tensor_hc_transpose under hdim_is_batch), batch matmuls [batch * batch_low, M, K] x [.., K, N], one bias[N] for
+ * all, then the requantization over the flat output -- per-channel operands indexed by the output's LAST dimension
+ * (:666-668), on CV18xx the multiplier / rshift of batch b when one per batch is given (:638-664).  attr->M/K/N are
+ * ignored.  Operands must hold exactly batch * batch_low matrices (the quantized path never broadcasts). */
 int orc_matmul_int8_nd(const orc_i8mm_attr *attr, const int64_t *a_shape, int a_dims, const int64_t *b_shape,
-                       int b_dims, const int64_t *o_shape, int o_dims, int chip, const float *const *inputs,
-                       float *output);
+                       int b_dims, const int64_t *o_shape, int o_dims, int left_transpose, int output_transpose,
+                       int hdim_is_batch, int chip, const float *const *inputs, float *output);
 
 #ifdef __cplusplus
 }

@@ -565,8 +565,9 @@ def matmul_parse_param(a_shape, b_shape, o_shape, *, right_transpose=False, left
 def matmul_int8_nd(x, right, bias, multi, *, out_shape, right_transpose=False, input_zp=0, right_zp=0, do_relu=False,
                    relu_limit=-1.0, cv18xx=False, quant_mode=RQ_MULTIPLIER_SHIFT, fuse_rq=False, multipliers=(1,),
                    rshifts=(0,), out_zp=0, out_kind=0, out_bits=8, out_unsigned=False, gemm_kind=GEMM_F32,
-                   out_scale=1.0):
-    """Quantised tpu.MatMul on operands of any rank (plain branch of parseParam); returns the output, shaped out_shape."""
+                   out_scale=1.0, left_transpose=False, output_transpose=False, hdim_is_batch=False, chip=None):
+    """Quantised tpu.MatMul on operands of any rank, with MatMul::run's transposes; returns the output, shaped
+    out_shape.  chip: CHIP_* (default: CV18xx when cv18xx, else BM1684X)."""
     x, right = _f32(x), _f32(right)
     ins = [x, right, _f32(bias), _f32(multi)]
     mult = np.ascontiguousarray(multipliers, dtype=np.int64)
@@ -580,7 +581,9 @@ def matmul_int8_nd(x, right, bias, multi, *, out_shape, right_transpose=False, i
     L.orc_matmul_int8_nd.restype = C.c_int
     rc = L.orc_matmul_int8_nd(C.byref(attr), _shape_arr(x.shape), C.c_int(x.ndim), _shape_arr(right.shape),
                               C.c_int(right.ndim), _shape_arr(out_shape), C.c_int(len(out_shape)),
-                              C.c_int(CHIP_CV18XX if cv18xx else CHIP_BM1684X), arr, _p(out, C.c_float))
+                              C.c_int(int(left_transpose)), C.c_int(int(output_transpose)), C.c_int(int(hdim_is_batch)),
+                              C.c_int((CHIP_CV18XX if cv18xx else CHIP_BM1684X) if chip is None else chip), arr,
+                              _p(out, C.c_float))
     if rc != 0:
         raise RuntimeError("orc_matmul_int8_nd failed")
     return out

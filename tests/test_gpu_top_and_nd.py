@@ -106,7 +106,74 @@ def test_matmul_int8_nd_cv18xx_per_batch_requant(orc):
     assert np.array_equal(y, ref)
 
 
-def test_matmul_int8_nd_refuses_broadcast_batches_and_transposes():
+ND_RELAID = [
+    # a_shape, b_shape, o_shape, flags (right, left, output, hdim), chip
+    ((3, 64, 20), (3, 64, 48), (3, 20, 48), (0, 1, 0, 0), "BM168X"),       # left stored [b, K, M]
+    ((3, 20, 64), (3, 48, 64), (3, 48, 20), (1, 0, 1, 0), "BM168X"),       # output stored [b, N, M]
+    ((2, 2, 64, 33), (2, 2, 64, 40), (2, 2, 40, 33), (0, 1, 1, 0), "BM168X"),
+    ((2, 17, 3, 64), (2, 64, 3, 64), (2, 17, 3, 64), (1, 1, 1, 1), "BM168X"),   # (B0,M,B1,K) x (B0,K,B1,N), K == N
+    ((2, 17, 3, 48), (2, 32, 3, 48), (2, 17, 3, 32), (1, 1, 1, 1), "BM168X"),   # K != N: the reference swaps K and N
+    ((2, 3, 17, 64), (2, 64, 3, 40), (2, 3, 17, 40), (1, 0, 0, 1), "CV18XX"),   # (B0,B1,M,K) x (B0,K,B1,N)
+    ((2, 17, 3, 64), (2, 3, 64, 40), (2, 17, 3, 40), (0, 1, 0, 1), "BM168X"),   # right already (B0,B1,K,N)
+]
+
+
+@pytest.mark.parametrize("a,b,o,flags,chip", ND_RELAID)
+@pytest.mark.parametrize("variant", ["per_channel", "scalar_zp_relu", "int32"])
+def test_matmul_int8_nd_transposed_layouts_against_oracle(orc, a, b, o, flags, chip, variant):
+    """left_transpose / output_transpose / hdim_is_batch of tpu.MatMul (MatMul::run's tensor_hw_transpose and
+    tensor_hc_transpose): bit-exact against the oracle, whose layouts are pinned by numpy on the documented cases."""
+    m = pkg()
+    clib = pkg("clib")
+    rt, lt, ot, hd = flags
+    cv = chip == "CV18XX"
+    rng = np.random.default_rng(sum(a) * 5 + sum(b) + len(variant))
+    unsigned = variant == "scalar_zp_relu"
+    A = rng.integers(0 if unsigned else -128, 256 if unsigned else 128, size=a).astype(np.float32)
+    B = rng.integers(-128, 128, size=b).astype(np.float32)
+    p = orc.matmul_parse_param(a, b, o, right_transpose=rt, left_transpose=lt, output_transpose=ot, hdim_is_batch=hd,
+                               chip=orc.CHIP_CV18XX if cv else orc.CHIP_BM1684X)
+    N, fb = p["N"], p["batch"] * p["batch_low"]
+    bias = rng.integers(-5000, 5000, size=N).astype(np.float32)
+    common = dict(right_transpose=bool(rt))
+    okw = dict(left_transpose=bool(lt), output_transpose=bool(ot), hdim_is_batch=bool(hd), cv18xx=cv)
+    multi = None
+    if variant == "int32":
+        dev = dict(out_dtype=clib.DT_I32)
+        ora = dict(out_kind=1)
+    elif cv:
+        mult = tuple(int(v) for v in rng.integers(1 << 29, 1 << 31, size=fb))
+        rs = tuple(int(v) for v in rng.integers(8, 14, size=fb))
+        if variant == "scalar_zp_relu":
+            mult, rs = mult[:1], rs[:1]
+        dev = dict(chip=clib.CHIP_CV18XX, quant_mode=clib.RQ_QDM, multipliers=mult, rshifts=rs)
+        ora = dict(quant_mode=orc.RQ_QDM, multipliers=mult, rshifts=rs)
+    elif variant == "per_channel":
+        multi = rng.integers(1000, 10000, size=o[-1]).astype(np.float32)   # one per element of the output's last dim
+        dev = dict(quant_mode=clib.RQ_MULTIPLIER_SHIFT, fuse_rq=True, multipliers=(1,), rshifts=(20,), out_zp=-3)
+        ora = dict(quant_mode=orc.RQ_MULTIPLIER_SHIFT, fuse_rq=True, multipliers=(1,), rshifts=(20,), out_zp=-3)
+    else:
+        dev = dict(quant_mode=clib.RQ_TFLITE, multipliers=(1518500250,), rshifts=(9,), out_zp=5, input_zp=7, right_zp=-2,
+                   do_relu=True, relu_limit=90000.0, out_dtype=clib.DT_U8)
+        ora = dict(quant_mode=orc.RQ_TFLITE, multipliers=(1518500250,), rshifts=(9,), out_zp=5, input_zp=7, right_zp=-2,
+                   do_relu=True, relu_limit=90000.0, out_unsigned=True)
+    if variant == "scalar_zp_relu" and cv:
+        dev.update(input_zp=0, right_zp=0, do_relu=True)
+        ora.update(do_relu=True)
+    if cv:
+        dev["chip"] = clib.CHIP_CV18XX
+    op = m.MatMulInt8(K=p["K"], N=N, right_is_weight=False, **common, **dev)
+    y = op.inference_nd(A, B, bias, multi, out_shape=o, left_transpose=bool(lt), output_transpose=bool(ot),
+                        hdim_is_batch=bool(hd))
+    y_again = op.inference_nd(A, B, bias, multi, out_shape=o, left_transpose=bool(lt), output_transpose=bool(ot),
+                              hdim_is_batch=bool(hd))
+    op.deinit()
+    ref = orc.matmul_int8_nd(A, B, bias, multi, out_shape=o, **common, **okw, **ora)
+    assert np.array_equal(y, ref) and np.array_equal(y_again, ref)
+    assert len(np.unique(ref)) > 4
+
+
+def test_matmul_int8_nd_refuses_broadcast_batches():
     m = pkg()
     clib = pkg("clib")
     op = m.MatMulInt8(K=8, N=4, multipliers=(1,), rshifts=(0,))

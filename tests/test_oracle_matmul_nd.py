@@ -88,3 +88,56 @@ def test_matmul_int8_nd_cv18xx_per_batch_multipliers(orc):
         assert np.array_equal(out[b], one)
     assert not np.array_equal(out[1], orc.matmul_int8_nd(A[1], B[1], None, None, out_shape=acc[1].shape, cv18xx=True,
                                                         quant_mode=orc.RQ_QDM, multipliers=(mult[0],), rshifts=(rs[0],)))
+
+
+def _half_up(acc, mult, shift, zp):
+    return np.clip(np.floor((acc * mult + (1 << (shift - 1))) / float(1 << shift)).astype(np.int64) + zp, -128, 127)
+
+
+def test_matmul_int8_nd_left_and_output_transpose_against_numpy(orc):
+    """Without hdim_is_batch the flags are per-batch matrix transposes (tensor_hw_transpose): the left operand is stored
+    [batch, K, M], the output [batch, N, M]; a per-channel multiplier follows the output's last dimension."""
+    rng = np.random.default_rng(21)
+    b, M, K, N = 3, 5, 16, 7
+    A = rng.integers(-128, 128, size=(b, M, K)).astype(np.int64)
+    B = rng.integers(-128, 128, size=(b, K, N)).astype(np.int64)
+    bias = rng.integers(-500, 500, size=N).astype(np.int64)
+    acc = np.matmul(A, B) + bias
+    out = orc.matmul_int8_nd(np.swapaxes(A, 1, 2).copy(), B, bias, None, out_shape=(b, M, N), left_transpose=True,
+                             multipliers=(91,), rshifts=(13,), out_zp=-2)
+    assert np.array_equal(out.astype(np.int64), _half_up(acc, 91, 13, -2))
+    out = orc.matmul_int8_nd(A, B, bias, None, out_shape=(b, N, M), output_transpose=True, multipliers=(91,),
+                             rshifts=(13,), out_zp=-2)
+    assert np.array_equal(out.astype(np.int64), _half_up(np.swapaxes(acc, 1, 2), 91, 13, -2))
+    multi = rng.integers(40, 120, size=M).astype(np.int64)  # one per element of the output's last dimension: M here
+    out = orc.matmul_int8_nd(A, B, bias, multi, out_shape=(b, N, M), output_transpose=True, fuse_rq=True, rshifts=(13,))
+    assert np.array_equal(out.astype(np.int64), _half_up(np.swapaxes(acc, 1, 2) * multi, 1, 13, 0))
+
+
+@pytest.mark.parametrize("chip_name,K,N", [("CHIP_OTHER", 16, 6), ("CHIP_BM1684X", 8, 8)])
+def test_matmul_int8_nd_hdim_is_batch_documented_layout(orc, chip_name, K, N):
+    """MatMul.cpp:58-62: (B0, M, B1, K) x (B0, K, B1, N) = (B0, M, B1, N) with all three transposes set.  On the BM1684X
+    family parseParam swaps K and N of a transposed right operand (:66-71) while MatMul::run keeps indexing the buffer
+    as (B0, K, B1, N): the documented layout then holds for K == N only, which is the case checked for that chip."""
+    chip = getattr(orc, chip_name)
+    rng = np.random.default_rng(31 + K)
+    B0, M, B1 = 2, 5, 3
+    A = rng.integers(-128, 128, size=(B0, M, B1, K)).astype(np.int64)
+    B = rng.integers(-128, 128, size=(B0, K, B1, N)).astype(np.int64)
+    acc = np.einsum("bmhk,bkhn->bmhn", A, B)
+    out = orc.matmul_int8_nd(A, B, None, None, out_shape=acc.shape, right_transpose=True, left_transpose=True,
+                             output_transpose=True, hdim_is_batch=True, chip=chip, multipliers=(57,), rshifts=(12,),
+                             out_zp=1)
+    assert np.array_equal(out.astype(np.int64), _half_up(acc, 57, 12, 1))
+
+
+def test_matmul_int8_nd_hdim_is_batch_cv18xx_layout(orc):
+    """MatMul.cpp:60: CV18xx (B0, B1, M, K) x (B0, K, B1, N) = (B0, B1, M, N): only the right operand is transposed."""
+    rng = np.random.default_rng(41)
+    B0, B1, M, K, N = 2, 3, 4, 16, 5
+    A = rng.integers(-128, 128, size=(B0, B1, M, K)).astype(np.int64)
+    B = rng.integers(-128, 128, size=(B0, K, B1, N)).astype(np.int64)
+    acc = np.einsum("bhmk,bkhn->bhmn", A, B)
+    out = orc.matmul_int8_nd(A, B, None, None, out_shape=acc.shape, right_transpose=True, hdim_is_batch=True, cv18xx=True,
+                             out_kind=1)
+    assert np.array_equal(out.astype(np.int64), acc)

@@ -724,6 +724,55 @@ static int check_i8_attr(const mi_i8mm_attr *a, const char *who) {
   return MI_SUCCESS;
 }
 
+// The scalar part of the requantization of tpu::MatMulOp::inference (MatMul.cpp:636-727) as a device descriptor; the
+// caller adds per-channel / per-batch arrays.
+static void fill_i8_rq(const mi_i8mm_attr *attr, mi_requant_desc *rq) {
+  memset(rq, 0, sizeof(*rq));
+  rq->chip = attr->chip;
+  rq->out_dtype = attr->out_dtype;
+  rq->quant_mode = attr->quant_mode;
+  rq->multiplier = attr->multipliers && attr->n_multipliers > 0 ? (int32_t)attr->multipliers[0] : 1;
+  rq->shift = attr->rshifts && attr->n_rshifts > 0 ? (int32_t)attr->rshifts[0] : 0;
+  if (attr->chip == MI_CHIP_CV18XX) {
+    // MatMul.cpp:638-664: per-batch multiplier/rshift, half away from zero, no zero point
+    rq->round_mode = MI_ROUND_HALF_AWAY_FROM_ZERO;
+    rq->zp = 0;
+  } else if (attr->quant_mode == MI_RQ_ONLY_SCALE) {
+    // MatMul.cpp:683-691: (int32)roundf(acc * (float)out_scales[0]) + zero point
+    rq->round_mode = MI_ROUND_HALF_AWAY_FROM_ZERO;
+    rq->zp = (int32_t)attr->out_zp;
+    rq->only_scale = (float)attr->out_scale;
+  } else if (attr->quant_mode == MI_RQ_MULTIPLIER_SHIFT) {
+    // MatMul.cpp:708-726: default rounding of applyMultiplierAndRShift is half up (MathUtils.h:178-181)
+    rq->round_mode = MI_ROUND_HALF_UP;
+    rq->zp = (int32_t)attr->out_zp;
+  } else {
+    // MatMul.cpp:696-707: MultiplyByQuantizedMultiplier(acc, mult, -rshift), half away from zero
+    rq->round_mode = MI_ROUND_HALF_AWAY_FROM_ZERO;
+    rq->zp = (int32_t)attr->out_zp;
+  }
+}
+
+static void bytes_to_floats(const void *ho, int out_dtype, int64_t n, float *y) {
+  switch (out_dtype) {
+  case MI_DT_I8:
+    for (int64_t i = 0; i < n; ++i) y[i] = (float)((const int8_t *)ho)[i];
+    break;
+  case MI_DT_U8:
+    for (int64_t i = 0; i < n; ++i) y[i] = (float)((const uint8_t *)ho)[i];
+    break;
+  case MI_DT_I16:
+    for (int64_t i = 0; i < n; ++i) y[i] = (float)((const int16_t *)ho)[i];
+    break;
+  case MI_DT_U16:
+    for (int64_t i = 0; i < n; ++i) y[i] = (float)((const uint16_t *)ho)[i];
+    break;
+  default:
+    for (int64_t i = 0; i < n; ++i) y[i] = (float)((const int32_t *)ho)[i];
+    break;
+  }
+}
+
 }  // namespace mi
 
 extern "C" {
@@ -810,41 +859,18 @@ int mi_i8mm_inference(const mi_i8mm_attr *attr, mi_infer_param *p) {
     h->has_bias = attr->right_is_weight;  // weights' bias is constant; otherwise re-upload each call
   }
   mi_requant_desc rq;
-  memset(&rq, 0, sizeof(rq));
   const mi_requant_desc *rqp = nullptr;
   if (attr->out_dtype != MI_DT_I32) {
     rqp = &rq;
-    rq.chip = attr->chip;
-    rq.out_dtype = attr->out_dtype;
-    rq.quant_mode = attr->quant_mode;
-    rq.multiplier = attr->multipliers && attr->n_multipliers > 0 ? (int32_t)attr->multipliers[0] : 1;
-    rq.shift = attr->rshifts && attr->n_rshifts > 0 ? (int32_t)attr->rshifts[0] : 0;
-    if (attr->chip == MI_CHIP_CV18XX) {
-      // MatMul.cpp:638-664: per-batch (here: one) multiplier/rshift, half away from zero, no zero point
-      rq.round_mode = MI_ROUND_HALF_AWAY_FROM_ZERO;
-      rq.zp = 0;
-    } else if (attr->quant_mode == MI_RQ_ONLY_SCALE) {
-      // MatMul.cpp:683-691: (int32)roundf(acc * (float)out_scales[0]) + zero point
-      rq.round_mode = MI_ROUND_HALF_AWAY_FROM_ZERO;
-      rq.zp = (int32_t)attr->out_zp;
-      rq.only_scale = (float)attr->out_scale;
-    } else if (attr->quant_mode == MI_RQ_MULTIPLIER_SHIFT) {
-      // MatMul.cpp:708-726: default rounding of applyMultiplierAndRShift is half up (MathUtils.h:178-181)
-      rq.round_mode = MI_ROUND_HALF_UP;
-      rq.zp = (int32_t)attr->out_zp;
-      if (attr->fuse_rq) {
-        MI_REQUIRE(multi, MI_BAD_ARGUMENT, "mi_i8mm_inference: fuse_rq needs the multi operand");
-        if (!h->has_multi) {
-          if ((rc = floats_to_i32_dev(multi, N, h->d_multi, h->stream)))
-            return rc;
-          h->has_multi = attr->right_is_weight;
-        }
-        rq.d_multiplier = (const int32_t *)h->d_multi.ptr;
+    fill_i8_rq(attr, &rq);
+    if (attr->chip != MI_CHIP_CV18XX && attr->quant_mode == MI_RQ_MULTIPLIER_SHIFT && attr->fuse_rq) {
+      MI_REQUIRE(multi, MI_BAD_ARGUMENT, "mi_i8mm_inference: fuse_rq needs the multi operand");
+      if (!h->has_multi) {
+        if ((rc = floats_to_i32_dev(multi, N, h->d_multi, h->stream)))
+          return rc;
+        h->has_multi = attr->right_is_weight;
       }
-    } else {
-      // MatMul.cpp:696-707: MultiplyByQuantizedMultiplier(acc, mult, -rshift), half away from zero
-      rq.round_mode = MI_ROUND_HALF_AWAY_FROM_ZERO;
-      rq.zp = (int32_t)attr->out_zp;
+      rq.d_multiplier = (const int32_t *)h->d_multi.ptr;
     }
   }
   const int64_t relu_limit = attr->relu_limit > 0.0 ? (int64_t)floor(attr->relu_limit) : -1;
@@ -855,25 +881,7 @@ int mi_i8mm_inference(const mi_i8mm_attr *attr, mi_infer_param *p) {
     return rc;
   MI_HIP(hipMemcpyAsync(h->h_out.ptr, h->d_out.ptr, (size_t)M * N * osz, hipMemcpyDeviceToHost, h->stream));
   MI_HIP(hipStreamSynchronize(h->stream));
-  float *y = p->outputs[0];
-  const void *ho = h->h_out.ptr;
-  switch (attr->out_dtype) {
-  case MI_DT_I8:
-    for (int64_t i = 0; i < M * N; ++i) y[i] = (float)((const int8_t *)ho)[i];
-    break;
-  case MI_DT_U8:
-    for (int64_t i = 0; i < M * N; ++i) y[i] = (float)((const uint8_t *)ho)[i];
-    break;
-  case MI_DT_I16:
-    for (int64_t i = 0; i < M * N; ++i) y[i] = (float)((const int16_t *)ho)[i];
-    break;
-  case MI_DT_U16:
-    for (int64_t i = 0; i < M * N; ++i) y[i] = (float)((const uint16_t *)ho)[i];
-    break;
-  default:
-    for (int64_t i = 0; i < M * N; ++i) y[i] = (float)((const int32_t *)ho)[i];
-    break;
-  }
+  bytes_to_floats(h->h_out.ptr, attr->out_dtype, M * N, p->outputs[0]);
   return MI_SUCCESS;
 }
 
@@ -883,12 +891,29 @@ struct I8BatchHandle {
   std::vector<void *> per_batch;
 };
 
+// a MatMul whose operands or output MatMul::run transposes: everything in one handle, nothing cached between calls
+// (these are matmuls of two activations)
+struct I8NdHandle {
+  uint32_t magic = 0x18D18D18u;
+  mi::DevBuf d_a, d_a2, d_b, d_b2, d_acc, d_acc2, d_out, d_bias, d_multi, d_mult_b, d_rs_b;
+  mi::Pinned h_a, h_b, h_out;
+  hipStream_t stream = nullptr;
+  ~I8NdHandle() {
+    if (stream) {
+      mi::release_stream_workspaces(stream);
+      (void)hipStreamDestroy(stream);
+    }
+  }
+};
+
 void mi_i8mm_deinit(mi_infer_param *p) {
   if (!p || !p->handle)
     return;
   I8Handle *h = (I8Handle *)p->handle;
   if (h->magic == 0x18181818u) {
     delete h;
+  } else if (h->magic == 0x18D18D18u) {
+    delete (I8NdHandle *)p->handle;
   } else if (h->magic == 0x18B18B18u) {
     I8BatchHandle *bh = (I8BatchHandle *)p->handle;
     for (void *one : bh->per_batch)
@@ -974,26 +999,155 @@ int mi_matmul_parse_param(const mi_matmul_shapes *sh, int right_transpose, int c
   return MI_SUCCESS;
 }
 
+// tpu.MatMul with left_transpose, output_transpose or hdim_is_batch: the operands are re-laid on the device as
+// MatMul::run does on the host (lib/Support/Dnnl/MatMul.cpp:167-201), every batch's product leaves as int32
+// accumulators, the output is re-laid (:228-238) and requantized in one pass over the flat result, per-channel operands
+// indexed by the output's last dimension (MatMul.cpp:666-668).
+static int i8mm_inference_relaid(const mi_i8mm_attr *attr, const mi_matmul_shapes *shapes, const mi_matmul_param &mp,
+                                 mi_infer_param *p) {
+  const int64_t B = mp.batch, BL = mp.batch_low, FB = B * BL, M = mp.M, K = mp.K, N = mp.N;
+  const int64_t a_num = FB * M * K, b_num = FB * K * N, o_num = FB * M * N;
+  MI_REQUIRE(shapes->o_dims >= 1, MI_BAD_ARGUMENT, "mi_i8mm_inference_nd: output shape missing");
+  const int64_t n_last = shapes->o_shape[shapes->o_dims - 1];
+  I8NdHandle *h = (I8NdHandle *)p->handle;
+  if (!h) {
+    MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_i8mm_inference_nd: no GPU visible");
+    h = new (std::nothrow) I8NdHandle();
+    MI_REQUIRE(h, MI_HIP_ERROR, "mi_i8mm_inference_nd: out of host memory");
+    hipError_t e = hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+      delete h;
+      return hip_fail(e, "hipStreamCreateWithFlags", __FILE__, __LINE__);
+    }
+    p->handle = h;
+  }
+  MI_REQUIRE(h->magic == 0x18D18D18u, MI_BAD_ARGUMENT, "mi_i8mm_inference_nd: the handle belongs to another op");
+  if (o_num == 0)
+    return MI_SUCCESS;
+  const int osz = out_elem_size(attr->out_dtype);
+  int rc;
+  if ((rc = h->h_a.reserve((size_t)a_num)) || (rc = h->d_a.reserve((size_t)a_num)) ||
+      (rc = h->h_b.reserve((size_t)b_num)) || (rc = h->d_b.reserve((size_t)b_num)) ||
+      (rc = h->d_acc.reserve((size_t)o_num * 4)) || (rc = h->h_out.reserve((size_t)o_num * 4)) ||
+      (rc = h->d_out.reserve((size_t)o_num * osz)))
+    return rc;
+  int a_unsigned = 0, b_unsigned = 0;
+  if ((rc = floats_to_bytes(p->inputs[0], a_num, (uint8_t *)h->h_a.ptr, &a_unsigned, "mi_i8mm_inference_nd")) ||
+      (rc = floats_to_bytes(p->inputs[1], b_num, (uint8_t *)h->h_b.ptr, &b_unsigned, "mi_i8mm_inference_nd")))
+    return rc;
+  MI_HIP(hipMemcpyAsync(h->d_a.ptr, h->h_a.ptr, (size_t)a_num, hipMemcpyHostToDevice, h->stream));
+  MI_HIP(hipMemcpyAsync(h->d_b.ptr, h->h_b.ptr, (size_t)b_num, hipMemcpyHostToDevice, h->stream));
+  const uint8_t *pa = (const uint8_t *)h->d_a.ptr, *pb = (const uint8_t *)h->d_b.ptr;
+  if (mp.left_transpose) {
+    if ((rc = h->d_a2.reserve((size_t)a_num)))
+      return rc;
+    rc = mp.hdim_is_batch ? permute_launch(h->d_a.ptr, h->d_a2.ptr, 1, 1, B, M, BL, K, h->stream)
+                          : permute_launch(h->d_a.ptr, h->d_a2.ptr, 1, 0, 1, B, K, M, h->stream);
+    if (rc)
+      return rc;
+    pa = (const uint8_t *)h->d_a2.ptr;
+  }
+  int gemm_rt = mp.right_transpose;  // [N, K] per batch is the layout the kernels read
+  if (mp.right_transpose && mp.hdim_is_batch) {
+    if ((rc = h->d_b2.reserve((size_t)b_num)) ||
+        (rc = permute_launch(h->d_b.ptr, h->d_b2.ptr, 1, 1, B, K, BL, N, h->stream)))
+      return rc;
+    pb = (const uint8_t *)h->d_b2.ptr;
+    gemm_rt = 0;  // the re-laid operand is [batch, batch_low, K, N]
+  }
+  const float *bias = p->n_inputs > 2 ? p->inputs[2] : nullptr;
+  const float *multi = p->n_inputs > 3 ? p->inputs[3] : nullptr;
+  if (bias && (rc = floats_to_i32_dev(bias, N, h->d_bias, h->stream)))
+    return rc;
+  const int64_t relu_limit = attr->relu_limit > 0.0 ? (int64_t)floor(attr->relu_limit) : -1;
+  int32_t *acc = (int32_t *)h->d_acc.ptr;
+  for (int64_t b = 0; b < FB; ++b) {
+    rc = i8mm_launch(pa + b * M * K, a_unsigned, pb + b * K * N, b_unsigned, gemm_rt,
+                     bias ? (const int32_t *)h->d_bias.ptr : nullptr, M, K, N, attr->input_zp, attr->right_zp,
+                     attr->do_relu, relu_limit, nullptr, nullptr, acc + b * M * N, h->stream);
+    if (rc)
+      return rc;
+  }
+  if (mp.output_transpose) {
+    if ((rc = h->d_acc2.reserve((size_t)o_num * 4)))
+      return rc;
+    rc = mp.hdim_is_batch ? permute_launch(acc, h->d_acc2.ptr, 4, 1, B, BL, M, N, h->stream)
+                          : permute_launch(acc, h->d_acc2.ptr, 4, 0, B, BL, M, N, h->stream);
+    if (rc)
+      return rc;
+    acc = (int32_t *)h->d_acc2.ptr;
+  }
+  const void *result = acc;
+  if (attr->out_dtype != MI_DT_I32) {
+    mi_requant_desc rq;
+    fill_i8_rq(attr, &rq);
+    int64_t outer = 1, channels = 1, inner = o_num;
+    if (attr->chip == MI_CHIP_CV18XX) {
+      if (FB > 1 && attr->n_multipliers == FB && attr->n_rshifts == FB) {  // MatMul.cpp:645-647: one pair per batch
+        std::vector<int32_t> mb((size_t)FB), rb((size_t)FB);
+        for (int64_t b = 0; b < FB; ++b) {
+          mb[(size_t)b] = (int32_t)attr->multipliers[b];
+          rb[(size_t)b] = (int32_t)attr->rshifts[b];
+        }
+        if ((rc = h->d_mult_b.reserve((size_t)FB * 4)) || (rc = h->d_rs_b.reserve((size_t)FB * 4)))
+          return rc;
+        MI_HIP(hipMemcpy(h->d_mult_b.ptr, mb.data(), (size_t)FB * 4, hipMemcpyHostToDevice));
+        MI_HIP(hipMemcpy(h->d_rs_b.ptr, rb.data(), (size_t)FB * 4, hipMemcpyHostToDevice));
+        rq.d_multiplier = (const int32_t *)h->d_mult_b.ptr;
+        rq.d_shift = (const int32_t *)h->d_rs_b.ptr;
+        channels = FB;
+        inner = M * N;
+      }
+    } else if (attr->quant_mode == MI_RQ_MULTIPLIER_SHIFT && attr->fuse_rq) {
+      MI_REQUIRE(multi, MI_BAD_ARGUMENT, "mi_i8mm_inference_nd: fuse_rq needs the multi operand");
+      MI_REQUIRE(n_last > 0 && o_num % n_last == 0, MI_BAD_ARGUMENT, "mi_i8mm_inference_nd: bad output shape");
+      if ((rc = floats_to_i32_dev(multi, n_last, h->d_multi, h->stream)))
+        return rc;
+      rq.d_multiplier = (const int32_t *)h->d_multi.ptr;
+      outer = o_num / n_last;
+      channels = n_last;
+      inner = 1;
+    }
+    if ((rc = requant_launch(acc, h->d_out.ptr, outer, channels, inner, 0, &rq, h->stream)))
+      return rc;
+    result = h->d_out.ptr;
+  }
+  MI_HIP(hipMemcpyAsync(h->h_out.ptr, result, (size_t)o_num * osz, hipMemcpyDeviceToHost, h->stream));
+  MI_HIP(hipStreamSynchronize(h->stream));
+  bytes_to_floats(h->h_out.ptr, attr->out_dtype, o_num, p->outputs[0]);
+  return MI_SUCCESS;
+}
+
 int mi_i8mm_inference_nd(const mi_i8mm_attr *attr, const mi_matmul_shapes *shapes, mi_infer_param *p) {
   MI_REQUIRE(attr && shapes && p, MI_BAD_ARGUMENT, "mi_i8mm_inference_nd: null argument");
-  MI_REQUIRE(!shapes->left_transpose && !shapes->output_transpose && !shapes->hdim_is_batch, MI_UNSUPPORTED,
-             "mi_i8mm_inference_nd: left_transpose, output_transpose and hdim_is_batch are not handled");
   mi_matmul_param mp;
   int rc = mi_matmul_parse_param(shapes, attr->right_transpose, attr->chip, &mp);
   if (rc)
     return rc;
   const int64_t batch = mp.batch * mp.batch_low;
-  int64_t a_num = 1, b_num = 1;
+  int64_t a_num = 1, b_num = 1, o_num = 1;
   for (int i = 0; i < shapes->a_dims; ++i)
     a_num *= shapes->a_shape[i];
   for (int i = 0; i < shapes->b_dims; ++i)
     b_num *= shapes->b_shape[i];
-  MI_REQUIRE(a_num == batch * mp.M * mp.K && b_num == batch * mp.K * mp.N, MI_UNSUPPORTED,
+  for (int i = 0; i < shapes->o_dims; ++i)
+    o_num *= shapes->o_shape[i];
+  MI_REQUIRE(a_num == batch * mp.M * mp.K && b_num == batch * mp.K * mp.N && o_num == batch * mp.M * mp.N,
+             MI_UNSUPPORTED,
              "mi_i8mm_inference_nd: the operands do not hold exactly one matrix per batch (broadcast batches are not "
              "handled)");
   MI_REQUIRE(p->inputs && p->n_inputs >= 2 && p->inputs[0] && p->inputs[1] && p->outputs && p->n_outputs >= 1 &&
                  p->outputs[0],
              MI_BAD_ARGUMENT, "mi_i8mm_inference_nd: null input or output");
+  if (mp.left_transpose || mp.output_transpose || mp.hdim_is_batch) {
+    mi_i8mm_attr one = *attr;
+    one.M = mp.M;
+    one.K = mp.K;
+    one.N = mp.N;
+    if ((rc = check_i8_attr(&one, "mi_i8mm_inference_nd")))
+      return rc;
+    return i8mm_inference_relaid(attr, shapes, mp, p);
+  }
   I8BatchHandle *bh = (I8BatchHandle *)p->handle;
   if (!bh) {
     bh = new I8BatchHandle;

@@ -38,6 +38,45 @@ __global__ void transpose_bytes_kernel(const uint8_t *__restrict__ src, uint8_t 
   }
 }
 
+// The two layout changes MatMul::run applies to operands and outputs (lib/Support/Dnnl/MatMul.cpp:167-239).  One
+// thread per destination element; T = uint8_t (operands) or int32_t (accumulators).
+// mode 0, tensor_hw_transpose: src [NC, H, W] -> dst [NC, W, H];  mode 1, tensor_hc_transpose: src [N, C, H, W] ->
+// dst [N, H, C, W]
+template <typename T>
+__global__ void permute_kernel(const T *__restrict__ src, T *__restrict__ dst, int64_t total, int mode, int64_t C,
+                               int64_t H, int64_t W) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total)
+    return;
+  if (mode == 0) {
+    const int64_t h = i % H, w = (i / H) % W, nc = i / (H * W);
+    dst[i] = src[nc * H * W + h * W + w];
+  } else {
+    const int64_t w = i % W, c = (i / W) % C, h = (i / (W * C)) % H, n = i / (W * C * H);
+    dst[i] = src[((n * C + c) * H + h) * W + w];
+  }
+}
+
+int permute_launch(const void *d_src, void *d_dst, int elem_bytes, int mode, int64_t n, int64_t c, int64_t h,
+                   int64_t w, hipStream_t stream) {
+  MI_REQUIRE(d_src && d_dst && d_src != d_dst && (elem_bytes == 1 || elem_bytes == 4) && (mode == 0 || mode == 1) &&
+                 n >= 0 && c >= 0 && h >= 0 && w >= 0,
+             MI_BAD_ARGUMENT, "permute_launch: bad argument");
+  const int64_t total = n * c * h * w;
+  if (total == 0)
+    return MI_SUCCESS;
+  const dim3 grid((unsigned)((total + 255) / 256));
+  MI_REQUIRE((total + 255) / 256 < (1ll << 31), MI_BAD_ARGUMENT, "permute_launch: tensor too large");
+  if (elem_bytes == 1)
+    permute_kernel<uint8_t><<<grid, dim3(256), 0, stream>>>((const uint8_t *)d_src, (uint8_t *)d_dst, total, mode, c,
+                                                            h, w);
+  else
+    permute_kernel<int32_t><<<grid, dim3(256), 0, stream>>>((const int32_t *)d_src, (int32_t *)d_dst, total, mode, c,
+                                                            h, w);
+  MI_HIP(hipGetLastError());
+  return MI_SUCCESS;
+}
+
 // dst = src ^ 0x80 per byte: an unsigned operand u becomes the signed value u - 128 the matrix cores take
 __global__ void flip_bytes_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t n) {
   const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 16;

@@ -163,6 +163,10 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
                 const int32_t *d_bias, int64_t M, int64_t K, int64_t N, int64_t input_zp, int64_t right_zp,
                 int do_relu, int64_t relu_limit, const mi_requant_desc *rq, void *d_out, int32_t *d_acc,
                 hipStream_t stream);
+// tensor_hw_transpose (mode 0: [n * c, h, w] -> [n * c, w, h]) / tensor_hc_transpose (mode 1: [n, c, h, w] ->
+// [n, h, c, w]) of 1- or 4-byte elements
+int permute_launch(const void *d_src, void *d_dst, int elem_bytes, int mode, int64_t n, int64_t c, int64_t h,
+                   int64_t w, hipStream_t stream);
 int requant_launch(const int32_t *d_in, void *d_out, int64_t outer, int64_t channels, int64_t inner,
                    int64_t input_zp, const mi_requant_desc *rq, hipStream_t stream);
 }  // namespace mi

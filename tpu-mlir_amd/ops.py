@@ -214,18 +214,24 @@ class MatMulInt8:
             self.param.c.handle = p.c.handle
         return y
 
-    def inference_nd(self, x, right, bias=None, multi=None):
+    def inference_nd(self, x, right, bias=None, multi=None, *, out_shape=None, left_transpose=False,
+                     output_transpose=False, hdim_is_batch=False):
         """Operands of any rank (mi_i8mm_inference_nd): numpy.matmul's shapes, with the right operand stored
-        [.., N, K] under right_transpose.  Keeps its own handle (one per batch inside the library)."""
+        [.., N, K] under right_transpose.  Keeps its own handle (one per batch inside the library).  With
+        left_transpose, output_transpose or hdim_is_batch (the layouts of MatMul.cpp:58-62) out_shape must be given."""
         x, right = _f32(x), _f32(right)
         n = right.shape[-2] if self.attr.right_transpose else (right.shape[-1] if right.ndim > 1 else None)
-        if right.ndim == 1:
+        if out_shape is not None:
+            o_shape = tuple(int(v) for v in out_shape)
+        elif left_transpose or output_transpose or hdim_is_batch:
+            raise clib.BackendError(clib.MI_BAD_ARGUMENT, "inference_nd: transposed layouts need out_shape")
+        elif right.ndim == 1:
             o_shape = tuple(x.shape[:-1])
         elif right.ndim == 2 or x.ndim == 1:
             o_shape = tuple(x.shape[:-1]) + (n,) if x.ndim > 1 else tuple(right.shape[:-2]) + (n,)
         else:
             o_shape = tuple(np.broadcast_shapes(x.shape[:-2], right.shape[:-2])) + (x.shape[-2], n)
-        sh = _matmul_shapes(x.shape, right.shape, o_shape)
+        sh = _matmul_shapes(x.shape, right.shape, o_shape, left_transpose, output_transpose, hdim_is_batch)
         y = np.empty(o_shape, dtype=np.float32)
         p = _Param([x, right, _f32(bias), _f32(multi), None], [y])
         p.c.handle = getattr(self, "_nd_handle", None)
