@@ -37,8 +37,7 @@ def test_argument_errors_need_no_gpu():
                      (dict(w_transpose=False, weight_bits=8), clib.MI_UNSUPPORTED),   # untransposed: 4-bit only
                      (dict(w_transpose=False, q_group_size=3), clib.MI_UNSUPPORTED),  # groups run along N there
                      (dict(weight_bits=3), clib.MI_UNSUPPORTED),
-                     (dict(q_group_size=48), clib.MI_BAD_ARGUMENT),      # K % g != 0
-                     (dict(q_group_size=16), clib.MI_UNSUPPORTED)):      # group size the kernels do not handle
+                     (dict(q_group_size=48), clib.MI_BAD_ARGUMENT)):     # K % g != 0
         args = dict(K=128, N=4, weight_bits=4, q_group_size=0)
         args.update(kw)
         op = M.A16MatMul(**args)

@@ -169,6 +169,38 @@ def test_w8a16_device_level(orc, M, K, N, g, signed):
     _check_against_oracle(orc, cfg, out, pre)
 
 
+PLAIN_GROUP_CASES = [  # (bits, M, K, N, g, signed): group sizes outside 32 / 64 / whole k-tiles
+    (4, 1, 192, 40, 96, False), (4, 3, 256, 33, 16, False), (4, 5, 120, 20, 24, False), (4, 2, 1024, 64, 8, False),
+    (4, 2, 40, 9, 5, False),     # odd group: the odd element of a byte takes the even element's group
+    (8, 1, 160, 17, 16, True), (8, 4, 240, 24, 48, False), (8, 2, 80, 10, 40, True), (8, 6, 72, 5, 9, False),
+]
+
+
+@pytest.mark.parametrize("bits,M,K,N,g,signed", PLAIN_GROUP_CASES)
+def test_group_sizes_outside_the_tiled_layout(orc, bits, M, K, N, g, signed):
+    """Any q_group_size that divides K is taken: the weight then stays as stored and a plain fp32 kernel dequantizes
+    element by element (A16MatMul.cpp:172-231)."""
+    cfg = (S.w4a16(M, K, N, g, seed=K + g, bias=(N % 2 == 0)) if bits == 4
+           else S.w8a16(M, K, N, g, seed=K + g, signed=signed, bias=(N % 2 == 0)))
+    out, pre = _run_device(cfg)
+    _check_against_oracle(orc, cfg, out, pre)
+
+
+def test_group_size_outside_the_tiled_layout_operator_level_f16(orc):
+    cfg = S.w4a16(3, 96, 12, 24, seed=77, bias=True)
+    x = orc.F16(S.bf16_to_f32(cfg["x"]))
+    scale = orc.F16(S.bf16_to_f32(cfg["scale"]))
+    w = cfg["weight"].astype(np.float32)
+    z = cfg["zp"].astype(np.float32)
+    b = S.bf16_to_f32(cfg["bias"])
+    op = M_.A16MatMul(K=96, N=12, weight_bits=4, q_group_size=24, out_dtype=clib.DT_F16).init(w, scale, z, b)
+    y = op.inference(x)
+    op.deinit()
+    want, _ = orc.a16matmul(x, w, scale, z, b, M=3, K=96, N=12, weight_bits=4, q_group_size=24, out_dtype=orc.OUT_F16)
+    assert np.array_equal(orc.F16(y), y)
+    assert np.max(np.abs(y - want)) <= 2.0 ** -10 * np.max(np.abs(want))
+
+
 def test_operator_level_matches_oracle(orc):
     # the interpreter's calling convention: float-expanded operands, init once, inference twice, deinit
     cfg = S.w4a16(4, 1024, 256, 128, seed=11, bias=True)

@@ -741,6 +741,16 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
     MI_REQUIRE(n == 1, MI_UNSUPPORTED, "mi_a16mm_launch_group: untransposed weights are launched one set at a time");
     return a16_kn_launch(w, d_x, M, d_ys ? d_ys[0] : nullptr, d_y32s ? d_y32s[0] : nullptr, stream);
   }
+  if (w && w->plain) {  // a group size outside the tiled layout: one launch per weight set
+    for (int i = 0; i < n; ++i) {
+      MI_REQUIRE(ws[i] && ws[i]->plain && ws[i]->K == w->K, MI_BAD_ARGUMENT,
+                 "mi_a16mm_launch_group: the weight sets must agree in K, bit width, group size, data type and chip");
+      const int rc = a16_plain_launch(ws[i], d_x, M, d_ys ? d_ys[i] : nullptr, d_y32s ? d_y32s[i] : nullptr, stream);
+      if (rc != MI_SUCCESS)
+        return rc;
+    }
+    return MI_SUCCESS;
+  }
   int64_t total_rb = 0;
   SkinnyArgs a;
   for (int i = 0; i < MAX_SEG; ++i) {

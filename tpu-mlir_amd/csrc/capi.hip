@@ -196,9 +196,6 @@ int mi_a16_weight_create(mi_a16_weight **out, const mi_a16_weight_desc *d, const
   MI_REQUIRE(d->K % 8 == 0, MI_UNSUPPORTED, "mi_a16_weight_create: K must be a multiple of 8");
   MI_REQUIRE(d->q_group_size == 0 || (d->q_group_size > 0 && d->K % d->q_group_size == 0), MI_BAD_ARGUMENT,
              "mi_a16_weight_create: K is not a multiple of q_group_size");
-  MI_REQUIRE(group_size_supported(d->weight_bits, d->q_group_size, d->K), MI_UNSUPPORTED,
-             "mi_a16_weight_create: group size not handled (4-bit: 32, 64 or a multiple of 128; 8-bit: 32 or a "
-             "multiple of 64)");
   MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_a16_weight_create: no GPU visible");
   mi_a16_weight *w = new (std::nothrow) mi_a16_weight();
   MI_REQUIRE(w, MI_HIP_ERROR, "mi_a16_weight_create: out of host memory");
@@ -209,9 +206,12 @@ int mi_a16_weight_create(mi_a16_weight **out, const mi_a16_weight_desc *d, const
   w->G = d->q_group_size ? (int)(d->K / d->q_group_size) : 1;
   w->dtype = d->dtype;
   w->chip = d->chip;
-  int rc = a16_pack(w, weight, d->weight_signed, scale, zp, bias);
+  // group sizes of 32, 64 or whole k-tiles are packed for the tiled kernels; any other stays as stored (a16_plain.hip)
+  int rc = group_size_supported(d->weight_bits, d->q_group_size, d->K)
+               ? a16_pack(w, weight, d->weight_signed, scale, zp, bias)
+               : a16_plain_create(w, weight, d->weight_signed, scale, zp, bias);
   if (rc != MI_SUCCESS) {
-    delete w;
+    mi_a16_weight_destroy(w);
     return rc;
   }
   *out = w;
@@ -274,7 +274,9 @@ int mi_a16_weight_export(const mi_a16_weight *w, void *blob, size_t capacity) {
   uint8_t *p = (uint8_t *)blob;
   memcpy(p, &h, sizeof(h));
   p += sizeof(h);
-  MI_REQUIRE(!w->kn, MI_UNSUPPORTED, "mi_a16_weight_export: an untransposed weight has no packed form");
+  MI_REQUIRE(!w->kn && !w->plain, MI_UNSUPPORTED,
+             "mi_a16_weight_export: a weight kept as stored (untransposed, or a group size outside the tiled layout) "
+             "has no packed form");
   MI_HIP(hipMemcpy(p, w->qweight, h.packed_bytes, hipMemcpyDeviceToHost));
   p += h.packed_bytes;
   if (w->bits == 4) {
@@ -485,8 +487,7 @@ int mi_a16mm_init(const mi_a16mm_attr *attr, mi_infer_param *p) {
   }
   const int g = attr->q_group_size;
   MI_REQUIRE(g == 0 || (g > 0 && K % g == 0), MI_BAD_ARGUMENT, "mi_a16mm_init: K is not a multiple of q_group_size");
-  MI_REQUIRE(K % 8 == 0 && group_size_supported(attr->weight_bits, g, K), MI_UNSUPPORTED,
-             "mi_a16mm_init: shape / group size not handled");
+  MI_REQUIRE(K % 8 == 0, MI_UNSUPPORTED, "mi_a16mm_init: K must be a multiple of 8");
   const int64_t G = g ? K / g : 1;
 
   // float-expanded operands -> native storage

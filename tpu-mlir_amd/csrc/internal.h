@@ -100,6 +100,10 @@ struct mi_a16_weight {
   bool kn = false;
   void *kn_w = nullptr;
   float *kn_scale = nullptr, *kn_zp = nullptr;
+  // w_transpose = true with a group size the tiled layout does not take (a16_plain.hip): the weight as stored,
+  // [N][K * bits / 8], in kn_w, widened scale / zero point [N][G] in kn_scale / kn_zp
+  bool plain = false;
+  int plain_signed = 0;
 };
 
 namespace mi {
@@ -109,6 +113,10 @@ void a16_free(mi_a16_weight *w);
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                hipStream_t stream);
 int a16_kn_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32, hipStream_t st);
+int a16_plain_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
+                     hipStream_t st);
+int a16_plain_create(mi_a16_weight *w, const void *weight, int weight_signed, const uint16_t *scale,
+                     const uint8_t *zp, const float *bias);
 // a caller-provided scratch area that a launch must make do with (instead of the stream's growable buffer)
 struct A16Scratch {
   void *ptr;
