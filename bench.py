@@ -316,6 +316,30 @@ def bench_single_matmuls(pkg, S, torch, steps=60):
     return out
 
 
+def bench_f16_prefill_forms(pkg, S, torch, clib, launches=10):
+    """W4 g128 prefill on f16 activations, 4096 x 4096: the exact kernel (the reference's unrounded fp32 weights) beside
+    the tolerance form (weights rounded to f16 first, mi_a16mm_launch_tol: about 2e-3 of the output RMS away from the
+    reference at the worst output).  The tolerance form is opt-in and offered for f16 only."""
+    K = N = 4096
+    cfg = S.w4a16(1, K, N, 128, seed=31)
+    scale16 = np.ascontiguousarray(S.bf16_to_f32(cfg["scale"]).astype(np.float16)).view(np.uint16)  # bf16 values fit f16
+    w = pkg.A16Weight(cfg["weight"], scale16, cfg["zp"], None, K=K, N=N, weight_bits=4, q_group_size=128,
+                      dtype=clib.DT_F16)
+    out = []
+    for M in (2048, 4096):
+        x = torch.randn((M, K), device="cuda").to(torch.float16)
+        y = torch.empty((M, N), dtype=torch.float16, device="cuda")
+        rec = {"M": M, "K": K, "N": N}
+        for label, tol in (("exact", False), ("tolerance", True)):
+            sec = _time_launches(torch, lambda: pkg.a16mm_launch(w, x, y, tolerance=tol), launches, warmup=2)
+            rec[label + "_us"] = round(sec * 1e6, 1)
+            rec[label + "_TFLOPs"] = round(2.0 * M * N * K / sec / 1e12, 1)
+        rec["tolerance_frac_f16_peak"] = round(rec["tolerance_TFLOPs"] / BF16_PEAK_TFLOPS, 4)
+        out.append(rec)
+    w.destroy()
+    return out
+
+
 def bench_dynamic_quant(pkg, S, torch, steps=40):
     """tpu.A16MatMul with dynamic integer activation quantization (activation quantizer + integer product per call),
     weights rotating through HBM; launches replayed from a HIP graph."""
@@ -631,6 +655,7 @@ def main():
             rm = bench_chain(pkg, S, torch, m, 40, 5, args.layers, cm, grouped=not args.no_group)
             ex["chain_M%d_GBps" % m] = round(rm["chain_bytes"] / (rm["gpu_s"] / 40) / 1e9, 1)
         ex["single_matmuls"] = bench_single_matmuls(pkg, S, torch)
+        ex["prefill_f16_exact_vs_tolerance"] = bench_f16_prefill_forms(pkg, S, torch, clib)
         ex["dynamic_quant"] = bench_dynamic_quant(pkg, S, torch)
         ex["int8_256x1024x1024"] = bench_int8(pkg, S, torch, clib, 1024, 40, 5, M=256, graph=True)
         ex["f8_matmul"] = bench_f8_matmul(pkg, torch, clib)

@@ -272,6 +272,17 @@ int mi_a16mm_launch_noalloc(const mi_a16_weight *w, const uint16_t *d_x, int64_t
  * are added in the reference's order -- results are bit-identical to the reference's. */
 int mi_a16mm_dq_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                        void *stream);
+/* mi_a16mm_launch in its TOLERANCE form, for many activation rows (prefill) in F16 mode: every 4-bit weight is first
+ * rounded to f16, w16 = round_to_nearest_even((q - zp) * scale), and the product is an f16 MFMA GEMM with fp32
+ * accumulation.  The reference (A16MatMul.cpp:172-208) multiplies the UNROUNDED fp32 weights, which mi_a16mm_launch
+ * reproduces; this entry point differs from it by at most 2^-12 relative per weight (about 2e-3 of the output RMS at
+ * the worst output, inside the 1e-2 * RMS the comparison tolerates) and runs faster from about 2048 rows on.  It is
+ * never taken implicitly.  MI_UNSUPPORTED unless the set is 4-bit, f16, in the tiled layout with K % 128 == 0 and
+ * q_group_size 0 or 128 * 2^k; bf16 sets are refused because bf16-rounded weights leave that tolerance.  No
+ * counterpart in the reference. */
+int mi_a16mm_launch_tol(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
+                        void *stream);
+
 /* The same branch for any dq_type it names (A16MatMul.cpp:51-61).  MI_DQ_INT is mi_a16mm_dq_launch.  MI_DQ_F8E4M3:
  * the 8-bit weight bytes are E4M3 codes (f8e4m3_to_f32, lib/Support/Float8.cpp:140-191), activations are divided by
  * amax / 448 and rounded to E4M3 (F8E4M3(src, step, true), Float8.cpp:259-261); group products are fp32 sums of the

@@ -1,0 +1,104 @@
+"""The tolerance form of the W4A16 product (mi_a16mm_launch_tol): weights rounded to the 16-bit activation type before
+the multiply.  Checked against its own definition -- float64 product of the activations with round16((q - zp) * scale),
+the rounding taken from the oracle's (pinned) converters -- to the bound the exact kernels are held to, and against the
+reference's arithmetic (the oracle's A16MatMul) to the comparison tolerance of 1e-2 * RMS, with the measured distance
+printed."""
+import numpy as np
+import pytest
+
+from helpers import pkg, f32_valued_a16
+
+pytestmark = pytest.mark.gpu
+
+M_ = pkg()
+S = pkg("synth")
+clib = pkg("clib")
+cmp = pkg("compare")
+
+
+def _run(cfg, dtype, tolerance=True):
+    import torch
+    tdt = torch.bfloat16 if dtype == clib.DT_BF16 else torch.float16
+    w = M_.A16Weight(cfg["weight"], cfg["scale16"], cfg["zp"], cfg["bias_f32"], K=cfg["K"], N=cfg["N"], weight_bits=4,
+                     q_group_size=cfg["g"], dtype=dtype)
+    x = torch.from_numpy(cfg["x16"].view(np.int16)).cuda().view(tdt)
+    y32 = torch.empty((cfg["M"], cfg["N"]), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_launch(w, x, y_f32=y32, tolerance=tolerance)
+    torch.cuda.synchronize()
+    out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    pre = y32.cpu().numpy()
+    w.destroy()
+    return out, pre
+
+
+def _operands(orc, M, K, N, g, dtype, seed):
+    cfg = S.w4a16(M, K, N, g, seed=seed, bias=(N % 3 != 0))
+    x, wq, scale, zp, bias = f32_valued_a16(cfg)
+    if dtype == clib.DT_F16:     # the same values where f16 holds them, else rounded to f16
+        x, scale = orc.F16(x), orc.F16(scale)
+        cfg["x16"] = orc.f32_to_f16(x)
+        cfg["scale16"] = orc.f32_to_f16(scale)
+    else:
+        cfg["x16"], cfg["scale16"] = cfg["x"], cfg["scale"]
+    cfg["bias_f32"] = bias
+    return cfg, x, wq, scale, zp, bias
+
+
+TOL_CASES = [  # (M, K, N, g, dtype)
+    (256, 512, 128, 128, "f16"), (300, 1024, 200, 0, "f16"), (64, 256, 48, 256, "f16"), (17, 384, 136, 128, "f16"),
+    (513, 640, 272, 128, "f16"), (1024, 4096, 1024, 128, "f16"),
+]
+
+
+@pytest.mark.parametrize("M,K,N,g,dt", TOL_CASES)
+def test_tolerance_form_matches_its_definition_and_stays_inside_the_comparison_tolerance(orc, M, K, N, g, dt):
+    dtype = clib.DT_F16 if dt == "f16" else clib.DT_BF16
+    cfg, x, wq, scale, zp, bias = _operands(orc, M, K, N, g, dtype, seed=M + K + N)
+    out, pre = _run(cfg, dtype)
+    # definition: w16 = round16((q - zp) * scale), product and bias in float64
+    G = K // g if g else 1
+    q = cfg["q"].astype(np.float32).reshape(N, G, K // G)
+    w32 = ((q - zp.reshape(N, G, 1)) * scale.reshape(N, G, 1)).astype(np.float32).reshape(N, K)
+    w16 = orc.F16(w32) if dtype == clib.DT_F16 else orc.BF16(w32)
+    want_pre = x.astype(np.float64) @ w16.astype(np.float64).T
+    if bias is not None:
+        want_pre = want_pre + bias.astype(np.float64)
+    err = cmp.max_abs_over_rms(pre, want_pre.astype(np.float32))
+    assert err <= 2e-5, "fp32 pre-round max-abs/RMS against the definition %.3g" % err
+    to16 = orc.f32_to_f16 if dtype == clib.DT_F16 else orc.f32_to_bf16
+    assert np.array_equal(out, to16(pre))            # outputs: the reference rounding of the kernel's own fp32 value
+    # distance to the reference's arithmetic (unrounded fp32 weights): the fp32 results before output rounding within
+    # the comparison tolerance of 1e-2 * RMS; on the 16-bit outputs a rounding flip of the largest output alone is
+    # worth 2^-8 (bf16) of it, so what can hold there is a few ulps
+    want, want_pre = orc.a16matmul(x, wq, scale, zp, bias, M=M, K=K, N=N, weight_bits=4, q_group_size=g,
+                                   out_dtype=orc.OUT_F16 if dtype == clib.DT_F16 else orc.OUT_BF16,
+                                   gemm_kind=orc.GEMM_F64ACC)
+    rms = float(np.sqrt(np.mean(want_pre.astype(np.float64) ** 2)))
+    dist32 = float(np.max(np.abs(pre.astype(np.float64) - want_pre))) / rms
+    got = orc.F16(pre) if dtype == clib.DT_F16 else orc.BF16(pre)
+    dist16 = float(np.max(np.abs(got.astype(np.float64) - want))) / rms
+    ulp16 = 2.0 ** (-11 if dtype == clib.DT_F16 else -8)
+    one_ulp = float(np.max(np.abs(want_pre))) * ulp16 / rms
+    print("tolerance form %s M=%d K=%d N=%d g=%d: fp32 max-abs/RMS to the reference %.3e (bound 1e-2); 16-bit outputs "
+          "%.3e (one ulp of the largest output = %.3e RMS), differing %.2f%%"
+          % (dt, M, K, N, g, dist32, dist16, one_ulp, 100.0 * (got != want).mean()))
+    assert dist32 <= 1e-2
+    assert dist16 <= max(1e-2, 2 * one_ulp)
+
+
+def test_tolerance_form_refuses_other_weight_sets():
+    import torch
+    cfg = S.w8a16(4, 256, 32, 0, seed=3)
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=256, N=32, weight_bits=8, q_group_size=0)
+    x = torch.zeros((4, 256), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(clib.BackendError) as e:
+        M_.a16mm_launch(w, x, tolerance=True)
+    assert e.value.code == clib.MI_UNSUPPORTED
+    w.destroy()
+    for g in (64, 128):                            # bf16 weight sets (rounding them to bf16 leaves the tolerance)
+        cfg = S.w4a16(4, 256, 32, g, seed=3)
+        w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=256, N=32, weight_bits=4, q_group_size=g)
+        with pytest.raises(clib.BackendError) as e:
+            M_.a16mm_launch(w, x, tolerance=True)
+        assert e.value.code == clib.MI_UNSUPPORTED
+        w.destroy()

@@ -19,7 +19,7 @@ EXPORTS = [
     "mi_a16mm_init", "mi_a16mm_inference", "mi_a16mm_deinit",
     "mi_a16_weight_create", "mi_a16_weight_create_kn", "mi_a16_weight_destroy", "mi_a16_weight_bytes", "mi_a16mm_launch",
     "mi_a16mm_launch_noalloc",
-    "mi_a16mm_launch_group", "mi_a16mm_dq_launch", "mi_a16mm_dq_type_launch", "mi_matmul_dq_launch",
+    "mi_a16mm_launch_group", "mi_a16mm_launch_tol", "mi_a16mm_dq_launch", "mi_a16mm_dq_type_launch", "mi_matmul_dq_launch",
     "mi_matmul_dq_inference", "mi_f8mm_inference", "mi_f8mm_launch", "mi_f8mm_e5m2_launch",
     "mi_a16_weight_export_size", "mi_a16_weight_export", "mi_a16_weight_import", "mi_a16_quantize", "mi_llm_unpack",
     "mi_a16_to_group",
@@ -196,6 +196,7 @@ def lib():
         L.mi_a16_weight_create_kn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_a16mm_launch_noalloc.argtypes = L.mi_a16mm_launch.argtypes
+        L.mi_a16mm_launch_tol.argtypes = L.mi_a16mm_launch.argtypes
         L.mi_top_a16_weight_create.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                                C.c_void_p, C.c_void_p, C.c_void_p]
         L.mi_top_a16_weight_destroy.argtypes = [C.c_void_p]

@@ -414,6 +414,12 @@ int mi_a16mm_dq_type_launch(const mi_a16_weight *w, int dq_type, const uint16_t 
   return a16_dq_launch(w, dq_type, d_x, M, d_y, d_y_f32, (hipStream_t)stream);
 }
 
+int mi_a16mm_launch_tol(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
+                        void *stream) {
+  MI_REQUIRE(w, MI_BAD_ARGUMENT, "mi_a16mm_launch_tol: null weight set");
+  return a16_tol_launch(w, d_x, M, d_y, d_y_f32, (hipStream_t)stream);
+}
+
 int mi_a16mm_launch_group(const mi_a16_weight *const *w, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_y,
                           float *const *d_y_f32, void *stream) {
   return a16_launch_group(w, n, d_x, M, d_y, d_y_f32, (hipStream_t)stream);

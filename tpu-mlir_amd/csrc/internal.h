@@ -113,6 +113,10 @@ void a16_free(mi_a16_weight *w);
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                hipStream_t stream);
 int a16_kn_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32, hipStream_t st);
+// tolerance form of the tiled product (a16_tol.hip): weights rounded to the 16-bit type before the multiply
+bool a16_tol_applicable(const mi_a16_weight *w);
+int a16_tol_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
+                   hipStream_t stream);
 int a16_plain_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                      hipStream_t st);
 int a16_plain_create(mi_a16_weight *w, const void *weight, int weight_signed, const uint16_t *scale,

@@ -538,11 +538,12 @@ def a16mm_dq_launch(w, x, y=None, y_f32=None, stream=None, dq_type=clib.DQ_INT):
     return y
 
 
-def a16mm_launch(w, x, y=None, y_f32=None, stream=None, no_alloc=False):
+def a16mm_launch(w, x, y=None, y_f32=None, stream=None, no_alloc=False, tolerance=False):
     """y[M,N] = round16(x[M,K] @ dequant(W)^T + bias) on the current stream.  x, y: torch CUDA tensors of the
     weight set's 16-bit type; y_f32 (optional float32 CUDA tensor) receives the fp32 result before rounding.
     no_alloc: through mi_a16mm_launch_noalloc (the library allocates nothing; pass y yourself to keep torch from
-    allocating it here)."""
+    allocating it here).  tolerance: through mi_a16mm_launch_tol (4-bit weights rounded to the 16-bit type before
+    the multiply: not the reference's arithmetic, see the header)."""
     import torch
     tdt = torch.float16 if w.dtype == DT_F16 else torch.bfloat16
     if not (x.is_cuda and x.dtype == tdt and x.is_contiguous() and x.shape[-1] == w.K):
@@ -556,6 +557,8 @@ def a16mm_launch(w, x, y=None, y_f32=None, stream=None, no_alloc=False):
                                   and y_f32.numel() == M * w.N):
         raise clib.BackendError(clib.MI_BAD_ARGUMENT, "a16mm_launch: bad y_f32 tensor")
     fn = clib.lib().mi_a16mm_launch_noalloc if no_alloc else clib.lib().mi_a16mm_launch
+    if tolerance:
+        fn = clib.lib().mi_a16mm_launch_tol
     check(fn(w.handle, _dptr(x), M, _dptr(y), _dptr(y_f32), _stream_ptr(stream)))
     return y
 
