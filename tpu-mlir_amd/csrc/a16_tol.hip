@@ -2,9 +2,9 @@
 // first -- w16 = round16((q - zp) * scale), one rounding to nearest even of the exact fp32 product -- and the product is
 // a plain 16-bit MFMA GEMM with fp32 accumulation.  The exact kernel (a16_gemm.hip) keeps the reference's unrounded
 // fp32 weights by folding scale and zero point per group in fp32, which costs about as many vector instructions as
-// MFMA cycles; this one trades that for one relative error of at most 2^-12 per weight (f16; the bf16 instance exists
-// for measurement only, see a16_tol_applicable).  It is never chosen by the library on its own: a caller asks for it by
-// name (mi_a16mm_launch_tol).
+// MFMA cycles; this one trades that for one relative error of at most 2^-12 per weight (f16 only, see
+// a16_tol_applicable).  It is never chosen by the library on its own: a caller asks for it by name
+// (mi_a16mm_launch_tol).
 //
 // 256 x 128 outputs per workgroup, 4 waves (2 x 2), each wave 128 rows x 64 channels as 4 x 2 MFMA 32x32x16 blocks
 // (128 fp32 accumulators per lane).  Activations: 64 K elements (128 bytes per row) per stage through a 4-stage,
@@ -13,9 +13,7 @@
 // (channel, kq) owning 16 bytes = four words of eight consecutive K each) the B fragment of a 32-channel block and
 // k-step is word j of lane slot (channel % 16, kq) of one of two neighbouring tiles, so a lane loads its two slots
 // (kq = lane / 32 and that + 2) of a K tile with two 16-byte requests, two K tiles ahead, and unpacks one word per
-// k-step: nibbles to bytes (3 instructions per word), bytes to float (1 each), one fma with the group's scale and
-// -zp * scale, one packed conversion per pair.  That is 23 vector instructions per fragment against the four MFMAs
-// (128 matrix-pipe cycles) that share it.
+// k-step (about 20 vector instructions per fragment against the four MFMAs, 128 matrix-pipe cycles, that share it).
 #include <climits>
 
 #include "a16_common.cuh"
@@ -53,44 +51,24 @@ struct TolArgs {
   int k_tiles, G, row_blocks, group_shift, chip;
 };
 
-template <int DT>
-__device__ __forceinline__ f32x16 tol_mfma(typename Half16<DT>::vec8 a, typename Half16<DT>::vec8 b, f32x16 c) {
-  if constexpr (DT == MI_DT_F16)
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
 
 // one packed word (eight K-consecutive weights of a channel; element 2p in nibble p, element 2p+1 in nibble 4+p)
-// -> eight 16-bit weights round16((q - zp) * s).  f16: the nibbles become the f16 numbers 16 + q in pairs (one
-// and-or each), and one mixed-precision fma per weight forms (16 + q) * s - (16 + zp) * s in fp32 -- exact, 16
-// significant bits at most -- and rounds it to f16 once.  bf16: nibbles to bytes, bytes to float, fma, packed conversion.
-// nzs = -(16 + zp) * s for f16, -zp * s for bf16.
-template <int DT>
-__device__ __forceinline__ typename Half16<DT>::vec8 tol_dequant(uint32_t d, float s, float nzs, uint32_t magic) {
-  using H = Half16<DT>;
-  if constexpr (DT == MI_DT_F16) {
-    const f16x8 q16 = unpack_nibbles<MI_DT_F16>(d, magic);
-    f16x8 w;
+// -> eight f16 weights round((q - zp) * s): the nibbles become the f16 numbers 16 + q in pairs (one and-or each), and
+// one mixed-precision fma per weight forms (16 + q) * s + nzs, nzs = -(16 + zp) * s, in fp32 -- exact, 16 significant
+// bits at most -- and rounds it to f16 once.
+__device__ __forceinline__ f16x8 tol_dequant(uint32_t d, float s, float nzs, uint32_t magic) {
+  const f16x8 q16 = unpack_nibbles<MI_DT_F16>(d, magic);
+  f16x8 w;
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
-      w[e] = (_Float16)fmaf((float)q16[e], s, nzs);
-    return w;
-  } else {
-    const uint32_t ev = d & 0x0F0F0F0Fu;         // nibbles 0, 2, 4, 6 in bytes 0..3
-    const uint32_t od = (d >> 4) & 0x0F0F0F0Fu;  // nibbles 1, 3, 5, 7
-    u32x4 b;
-    b[0] = H::pack2(fmaf((float)(ev & 0xffu), s, nzs), fmaf((float)((ev >> 16) & 0xffu), s, nzs));   // nibbles 0, 4
-    b[1] = H::pack2(fmaf((float)(od & 0xffu), s, nzs), fmaf((float)((od >> 16) & 0xffu), s, nzs));   // nibbles 1, 5
-    b[2] = H::pack2(fmaf((float)((ev >> 8) & 0xffu), s, nzs), fmaf((float)(ev >> 24), s, nzs));      // nibbles 2, 6
-    b[3] = H::pack2(fmaf((float)((od >> 8) & 0xffu), s, nzs), fmaf((float)(od >> 24), s, nzs));      // nibbles 3, 7
-    return __builtin_bit_cast(typename H::vec8, b);
-  }
+  for (int e = 0; e < 8; ++e)
+    w[e] = (_Float16)fmaf((float)q16[e], s, nzs);
+  return w;
 }
 
 // GPT: quantization groups per K tile (1: a group is one or more whole tiles, group of tile kt = kt >> group_shift)
-template <int DT, int GPT>
+template <int GPT>
 __global__ __launch_bounds__(256, 1) void a16_tol_kernel(TolArgs a, int tiles_m, int tiles_n, int per_xcd) {
+  constexpr int DT = MI_DT_F16;  // f16 only: bf16-rounded weights leave the comparison tolerance (a16_tol_applicable)
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -197,8 +175,8 @@ __global__ __launch_bounds__(256, 1) void a16_tol_kernel(TolArgs a, int tiles_m,
       const int u = GPT == 1 ? 0 : (s8 * GPT) / 8;
       const uint32_t szv = szw[rs][jb][u];
       const float s = H::to_f32((uint16_t)(szv >> 16));
-      const float nzs = -((DT == MI_DT_F16 ? H::OFFSET : 0.0f) + (float)(szv & 0xffu)) * s;
-      fb[jb] = tol_dequant<DT>(word, s, nzs, nib_magic);
+      const float nzs = -(H::OFFSET + (float)(szv & 0xffu)) * s;
+      fb[jb] = tol_dequant(word, s, nzs, nib_magic);
     }
   };
 
@@ -268,7 +246,8 @@ __global__ __launch_bounds__(256, 1) void a16_tol_kernel(TolArgs a, int tiles_m,
           for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-              acc[i][j] = tol_mfma<DT>(__builtin_bit_cast(vec8, fa[cur][i]), fb[cur][j], acc[i][j]);
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(vec8, fa[cur][i]), fb[cur][j],
+                                                                 acc[i][j], 0, 0, 0);
         }
       }
     }
@@ -311,7 +290,7 @@ __global__ __launch_bounds__(256, 1) void a16_tol_kernel(TolArgs a, int tiles_m,
       uint16_t hv[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e)
-        hv[e] = a.chip == MI_CHIP_CV18XX ? round_out16<DT, MI_CHIP_CV18XX>(v[e]) : round_out16<DT, MI_CHIP_BM168X>(v[e]);
+        hv[e] = round_out16<DT, MI_CHIP_BM168X>(v[e]);  // f16: the same on every chip
       if (vec_ok) {
         if (a.y32) {
           *(f32x4 *)(a.y32 + o) = f32x4{v[0], v[1], v[2], v[3]};
@@ -382,16 +361,10 @@ int a16_tol_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint1
   const int per_xcd = (int)((tiles_m * tiles_n + 7) / 8);
   const size_t lds_bytes = (size_t)TOL_NST * TOL_STAGE_BYTES;
   const dim3 grid((unsigned)(per_xcd * 8)), block(256);
-  static LdsLimitOnce once_bf16, once_f16;
-  if (w->dtype == MI_DT_F16) {
-    auto kfn = a16_tol_kernel<MI_DT_F16, 1>;
-    once_f16.ensure((const void *)kfn, (int)lds_bytes);
-    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
-  } else {
-    auto kfn = a16_tol_kernel<MI_DT_BF16, 1>;
-    once_bf16.ensure((const void *)kfn, (int)lds_bytes);
-    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
-  }
+  static LdsLimitOnce once;
+  auto kfn = a16_tol_kernel<1>;
+  once.ensure((const void *)kfn, (int)lds_bytes);
+  kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;
 }
