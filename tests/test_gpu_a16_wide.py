@@ -1,5 +1,7 @@
-"""The tolerance form of the W4A16 product (mi_a16mm_launch_tol): weights rounded to the 16-bit activation type before
-the multiply.  Checked against its own definition -- float64 product of the activations with round16((q - zp) * scale),
+"""The wide-tile A16 product (csrc/a16_wide.hip).  8-bit weight sets with one scale per channel take it by themselves
+from a few hundred rows on -- the reference rounds 8-bit weights to the activation type itself, so it is checked
+against the oracle like every other A16 kernel.  For 4-bit sets it is the tolerance form (mi_a16mm_launch_tol): weights
+rounded to the 16-bit activation type before the multiply.  Checked against its own definition -- float64 product of the activations with round16((q - zp) * scale),
 the rounding taken from the oracle's (pinned) converters -- to the bound the exact kernels are held to, and against the
 reference's arithmetic (the oracle's A16MatMul) to the comparison tolerance of 1e-2 * RMS, with the measured distance
 printed."""
@@ -102,3 +104,46 @@ def test_tolerance_form_refuses_other_weight_sets():
             M_.a16mm_launch(w, x, tolerance=True)
         assert e.value.code == clib.MI_UNSUPPORTED
         w.destroy()
+
+
+W8_WIDE_CASES = [  # (M, K, N, signed, dtype)
+    (256, 512, 128, True, "bf16"), (300, 1024, 200, False, "bf16"), (40, 64, 48, True, "f16"), (513, 192, 272, False, "f16"),
+    (512, 4096, 1024, True, "bf16"), (1, 128, 16, True, "bf16"),
+]
+
+
+@pytest.mark.parametrize("M,K,N,signed,dt", W8_WIDE_CASES)
+def test_w8_per_channel_on_wide_tiles_against_oracle(orc, plan, M, K, N, signed, dt):
+    """fp32 result within 2e-5 * RMS of the oracle's float64 accumulation; outputs the reference rounding of the
+    kernel's own fp32 values, at most one ulp from the oracle's on fewer than 0.5 % of them."""
+    import torch
+    plan(a16_wide_min_m=1)          # every row count through the wide tiles
+    dtype = clib.DT_F16 if dt == "f16" else clib.DT_BF16
+    cfg = S.w8a16(M, K, N, 0, seed=M + K + N, signed=signed, bias=(N % 2 == 0))
+    x, wq, scale, zp, bias = f32_valued_a16(cfg)
+    x16, scale16 = cfg["x"], cfg["scale"]
+    if dtype == clib.DT_F16:
+        x, scale = orc.F16(x), orc.F16(scale)
+        x16, scale16 = orc.f32_to_f16(x), orc.f32_to_f16(scale)
+    tdt = torch.float16 if dtype == clib.DT_F16 else torch.bfloat16
+    w = M_.A16Weight(cfg["weight"], scale16, cfg["zp"], bias, K=K, N=N, weight_bits=8, q_group_size=0, dtype=dtype)
+    xd = torch.from_numpy(x16.view(np.int16)).cuda().view(tdt)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_launch(w, xd, y_f32=y32)
+    torch.cuda.synchronize()
+    out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    pre = y32.cpu().numpy()
+    w.destroy()
+    want, want_pre = orc.a16matmul(x, wq, scale, zp, bias, M=M, K=K, N=N, weight_bits=8, q_group_size=0,
+                                   out_dtype=orc.OUT_F16 if dtype == clib.DT_F16 else orc.OUT_BF16,
+                                   gemm_kind=orc.GEMM_F64ACC)
+    err = cmp.max_abs_over_rms(pre, want_pre)
+    assert err <= 2e-5, "fp32 pre-round max-abs/RMS %.3g" % err
+    to16 = orc.f32_to_f16 if dtype == clib.DT_F16 else orc.f32_to_bf16
+    assert np.array_equal(out, to16(pre))
+    got = orc.F16(pre) if dtype == clib.DT_F16 else orc.BF16(pre)
+    rms = float(np.sqrt(np.mean(want_pre.astype(np.float64) ** 2)))
+    differ = got != want
+    assert differ.mean() < 5e-3
+    ulp16 = 2.0 ** (-10 if dtype == clib.DT_F16 else -7)
+    assert np.all(np.abs(got - want)[differ] <= np.maximum(np.abs(want[differ]) * ulp16, 4e-5 * rms))

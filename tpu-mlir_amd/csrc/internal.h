@@ -26,6 +26,7 @@ typedef struct mi_internal_plan {
   int i8_ring;                       // 3 / 4 / 5: LDS ring stages of the large kernel
   int dq_waves;                      // 8 / 16
   int f8_tile;                       // 256 / 128 / 64
+  int a16_wide_min_m;                // > 0: 8-bit per-channel sets take the wide tiles from this many rows on; -1: never
 } mi_internal_plan;
 void mi_internal_set_plan(const mi_internal_plan *p);  // null: back to the heuristics
 }
@@ -113,7 +114,11 @@ void a16_free(mi_a16_weight *w);
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                hipStream_t stream);
 int a16_kn_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32, hipStream_t st);
-// tolerance form of the tiled product (a16_tol.hip): weights rounded to the 16-bit type before the multiply
+// wide-tile product (a16_wide.hip), weights rounded to the 16-bit type before the multiply: the reference's arithmetic
+// for 8-bit per-channel sets (taken from a few hundred rows on), the opt-in tolerance form for 4-bit f16 sets
+bool a16_wide8_applicable(const mi_a16_weight *w, int64_t M);
+int a16_wide_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
+                    hipStream_t stream);
 bool a16_tol_applicable(const mi_a16_weight *w);
 int a16_tol_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                    hipStream_t stream);
