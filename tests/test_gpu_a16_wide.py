@@ -147,3 +147,32 @@ def test_w8_per_channel_on_wide_tiles_against_oracle(orc, plan, M, K, N, signed,
     assert differ.mean() < 5e-3
     ulp16 = 2.0 ** (-10 if dtype == clib.DT_F16 else -7)
     assert np.all(np.abs(got - want)[differ] <= np.maximum(np.abs(want[differ]) * ulp16, 4e-5 * rms))
+
+
+def test_tolerance_form_at_prefill_size_on_sampled_channels(orc):
+    """cfg3's shape in F16 mode (M = 2048, 4096 x 4096, groups of 128): 160 sampled channels against the definition
+    (2e-5 * RMS) and against the reference arithmetic (bound 1e-2 * RMS, figure printed); every output the reference
+    rounding of the kernel's own fp32 value; two runs bit-identical."""
+    import torch
+    M, K, N, g = 2048, 4096, 4096, 128
+    cfg, x, wq, scale, zp, bias = _operands(orc, M, K, N, g, clib.DT_F16, seed=2048)
+    out, pre = _run(cfg, clib.DT_F16)
+    out2, pre2 = _run(cfg, clib.DT_F16)
+    assert np.array_equal(out, out2) and np.array_equal(pre, pre2)
+    assert np.array_equal(out, orc.f32_to_f16(pre))
+    rng = np.random.default_rng(7)
+    pick = np.unique(np.r_[0:32, N - 32:N, rng.integers(0, N, size=96)])
+    G = K // g
+    q = cfg["q"][pick].astype(np.float32).reshape(len(pick), G, g)
+    w32 = ((q - zp[pick].reshape(len(pick), G, 1)) * scale[pick].reshape(len(pick), G, 1)).astype(np.float32)
+    w32 = w32.reshape(len(pick), K)
+    b = 0.0 if bias is None else bias[pick].astype(np.float64)
+    want_def = x.astype(np.float64) @ orc.F16(w32).astype(np.float64).T + b
+    want_ref = x.astype(np.float64) @ w32.astype(np.float64).T + b          # the reference: unrounded fp32 weights
+    rms = float(np.sqrt(np.mean(want_ref ** 2)))
+    err_def = float(np.max(np.abs(pre[:, pick] - want_def))) / rms
+    err_ref = float(np.max(np.abs(pre[:, pick] - want_ref))) / rms
+    print("tolerance form f16 M=%d %dx%d g=%d: to its definition %.3e, to the reference arithmetic %.3e of the RMS "
+          "(%d x %d sampled outputs)" % (M, N, K, g, err_def, err_ref, M, len(pick)))
+    assert err_def <= 2e-5
+    assert err_ref <= 1e-2
