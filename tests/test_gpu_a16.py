@@ -72,6 +72,7 @@ W4_CASES = [  # (M, K, N, g)
     (3, 512, 48, 32), (2, 1024, 100, 256), (5, 384, 33, 0),            # other group sizes, ragged N
     (1, 200, 16, 0), (7, 136, 20, 0),                                  # K not a multiple of the tile
     (40, 512, 64, 128),                                                # M > 16: several row blocks of x
+    (5, 4096, 272, 128), (7, 2048, 100, 64), (6, 1024, 48, 32), (8, 512, 40, 0),   # five to eight rows (decode, MR = 8)
 ]
 
 
@@ -138,6 +139,19 @@ def test_prefill_gemm_full_width_and_f16_mode(orc, plan):
     assert np.array_equal(out, orc.f32_to_f16(pre))
 
 
+@pytest.mark.parametrize("bits,M,K,N,g", [(4, 5, 4096, 272, 128), (4, 7, 2048, 100, 64), (4, 6, 1024, 48, 32),
+                                           (4, 8, 512, 40, 0), (8, 8, 4096, 1024, 0), (8, 5, 512, 40, 64),
+                                           (8, 7, 256, 24, 32)])
+def test_decode_kernel_with_five_to_eight_rows(orc, plan, bits, M, K, N, g):
+    """The eight-row instance of the decode kernel is taken where it was measured to pay (4-bit, K >= 4096, M >= 7);
+    here every shape it can handle goes through it."""
+    plan(a16_decode_rows8=1)
+    cfg = (S.w4a16(M, K, N, g, seed=M + K + N, bias=True) if bits == 4
+           else S.w8a16(M, K, N, g, seed=M + K, signed=(g == 0), bias=True))
+    out, pre = _run_device(cfg)
+    _check_against_oracle(orc, cfg, out, pre)
+
+
 @pytest.mark.parametrize("M,K,N,g", W4_CASES)
 def test_w4a16_device_level(orc, M, K, N, g):
     cfg = S.w4a16(M, K, N, g, seed=M + K + N, bias=(N % 3 == 0))
@@ -159,6 +173,7 @@ W8_CASES = [  # (M, K, N, g, signed)
     (1, 4096, 11008, 0, True), (32, 4096, 1024, 0, True),   # per-channel symmetric MLP up-projection
     (4, 1024, 96, 128, False), (2, 512, 40, 32, False), (3, 256, 24, 64, False),
     (1, 200, 17, 0, True),
+    (8, 4096, 1024, 0, True), (5, 512, 40, 64, False), (7, 256, 24, 32, False),     # five to eight rows
 ]
 
 

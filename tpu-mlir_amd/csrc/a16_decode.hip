@@ -1,4 +1,4 @@
-// W4A16 / W8A16 matmul for gfx950, decode (at most four activation rows): the kernel behind the GEMV numbers.
+// W4A16 / W8A16 matmul for gfx950, decode (at most eight activation rows): the kernel behind the GEMV numbers.
 //
 // Same packed weights, same arithmetic and the same results as the skinny kernel of a16_kernels.hip; what differs is
 // everything around the arithmetic.  At decode sizes a launch lives for a few microseconds, and a workgroup's fixed
@@ -15,9 +15,12 @@
 //     has arrived.
 //   * Tiles are multiplied two at a time -- two independent MFMA chains -- with the LDS reads of both issued before
 //     the wave waits for the weights: with two waves per SIMD there is little else to hide latencies behind.
-//   * Only lanes 0..15 hold live output rows (rows 0..3 of the 16 x 16 MFMA block): they alone take part in the
-//     cross-wave sum: one 16-byte LDS write per lane, the kernel's one barrier, and wave 0 adds the partial sums in
-//     wave order and stores the 64 outputs (their addresses were settled in the prologue).
+//   * Only lanes 0..15 hold live output rows (rows 0..3 of the 16 x 16 MFMA block; with five to eight activation rows
+//     lanes 16..31 hold rows 4..7 as well): they alone take part in the cross-wave sum: one 16-byte LDS write per
+//     lane, the kernel's one barrier, and wave 0 adds the partial sums in wave order and stores the outputs (their
+//     addresses were settled in the prologue).
+//   * Eight rows cost eight times the activation slice per wave: that instance (MR = 8) exists for the 8-wave shapes
+//     whose slice is one request per lane and row (K up to 4096 at 4 bits), at two workgroups per CU.
 // Arithmetic (see a16_kernels.hip): 4-bit  acc += scale * (sum a (16 + q) - (16 + zp) * sum a)  per group, in fp32;
 // 8-bit  weights rounded to the 16-bit type exactly as the reference does, accumulated directly.
 #include <climits>
@@ -34,7 +37,7 @@ __device__ __forceinline__ float dpp_f32(float v) {
 }
 
 constexpr int DEC_MAX_SEG = 4;
-constexpr int DEC_MAX_ROWS = 4;
+constexpr int DEC_MAX_ROWS = 8;
 
 struct DecodeArgs {
   const uint8_t *x;                 // activations [M, K], 16-bit
@@ -66,9 +69,11 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
   constexpr int XROW = XL * 64 * 16;             // bytes of LDS per row (padded to whole requests)
   constexpr int UNIT_CHUNKS = CPT / GPT;         // chunks per quantization group inside a tile
   constexpr int UNITS = TPW * GPT;
-  constexpr int S_BYTES = BITS == 4 ? UNITS * 16 : 0;  // per unit: the sums of rows 0..3
+  constexpr int SROWS = MR > 4 ? 8 : 4;          // rows whose activation sums are kept per unit
+  constexpr int RQ = MR > 4 ? 2 : 1;             // quarter-waves (16 lanes, four rows each) that hold live rows
+  constexpr int S_BYTES = BITS == 4 ? UNITS * SROWS * 4 : 0;
   constexpr int WAVE_LDS = MR * XROW + S_BYTES;
-  constexpr int RED_BYTES = WAVES * 256;         // partial sums of the final reduction
+  constexpr int RED_BYTES = WAVES * RQ * 256;    // partial sums of the final reduction
   static_assert(TPW % 2 == 0, "tiles are taken two at a time");
   static_assert(KSTEPS_PER_UNIT >= 1 && UNIT_CHUNKS >= 1, "at most one group per MFMA k-step");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -142,7 +147,7 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
 
   // ---- this wave's activations: LDS slice, group sums, fragments
   uint8_t *xs = smem + RED_BYTES + wave * WAVE_LDS;          // [MR][XROW]
-  float *s_lds = reinterpret_cast<float *>(xs + MR * XROW);  // [UNITS][4]
+  float *s_lds = reinterpret_cast<float *>(xs + MR * XROW);  // [UNITS][SROWS]
 #pragma unroll
   for (int r = 0; r < MR; ++r)
 #pragma unroll
@@ -162,7 +167,7 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
         if constexpr (UNIT_CHUNKS >= 16)
           part += dpp_f32<0x140>(part);   // row_mirror: the other half row
         if ((q % UNIT_CHUNKS) == 0 && q < XCHUNKS)
-          s_lds[(q / UNIT_CHUNKS) * 4 + r] = part;
+          s_lds[(q / UNIT_CHUNKS) * SROWS + r] = part;
       }
     }
   // The fragments below are other lanes' chunks of this wave's own slice: order the wave's LDS writes before its
@@ -185,11 +190,12 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
     const float sc = H::to_f32((uint16_t)(szw >> 16));
     const float c = H::OFFSET + (float)(szw & 0xffu);
     if constexpr (MR == 1) {  // one live row: register 0
-      const float S0 = s_lds[unit * 4];
+      const float S0 = s_lds[unit * SROWS];
       const float t = fmaf(-c, S0, P[0]);
       acc[0] = fmaf(sc, live ? t : 0.0f, acc[0]);
     } else {
-      const f32x4 S = *(const f32x4 *)(s_lds + unit * 4);
+      // register i of a lane is row 4 * kq + i: rows 0..3 in the first quarter-wave, 4..7 in the second
+      const f32x4 S = *(const f32x4 *)(s_lds + unit * SROWS + (MR > 4 ? 4 * (kq & 1) : 0));
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const float t = fmaf(-c, S[i], P[i]);
@@ -249,26 +255,31 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
     }
   }
 
-  // ---- cross-wave sum.  Rows 0..3 of the block live in lanes 0..15 (register i = row i): 256 bytes per wave, one
+  // ---- cross-wave sum.  Rows 0..3 of the block live in lanes 0..15 (register i = row i), rows 4..7 in lanes 16..31
+  // when MR = 8: 256 bytes per wave and quarter-wave, one
   // barrier (the only one of the kernel), and wave 0 adds the WAVES partial sums in wave order and stores.  (Letting
   // the wave that arrives last do this, behind an LDS ticket instead of the barrier, was measured: the barrier that
   // then has to publish the cleared ticket costs more than it saves, 8.2 against 6.8 us at K = 11008.)
-  f32x4 *red = reinterpret_cast<f32x4 *>(smem);  // [WAVES][16]
-  if (kq == 0)
-    red[wave * 16 + col] = acc;
+  f32x4 *red = reinterpret_cast<f32x4 *>(smem);  // [WAVES][RQ][16]
+  if (kq < RQ)
+    red[(wave * RQ + kq) * 16 + col] = acc;
   __syncthreads();
   if (wave == 0) {
-    // lane (col, kq) finishes row kq of channel col
+    // lane (col, kq) finishes row kq of channel col (and row kq + 4 when eight rows are live)
     const float *redf = reinterpret_cast<const float *>(smem);
-    float v = 0.0f;
 #pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv)
-      v += redf[(wv * 16 + col) * 4 + kq];
-    if (kq < a.M && n < n_end) {
-      v += bias_v;
-      if (y32)
-        y32[o] = v;
-      y[o] = (a.chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+    for (int h2 = 0; h2 < RQ; ++h2) {
+      float v = 0.0f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv)
+        v += redf[((wv * RQ + h2) * 16 + col) * 4 + kq];
+      if (kq + 4 * h2 < a.M && n < n_end) {
+        v += bias_v;
+        const int64_t oo = o + (int64_t)(4 * h2) * n_cols;
+        if (y32)
+          y32[oo] = v;
+        y[oo] = (a.chip == MI_CHIP_CV18XX) ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+      }
     }
   }
 #undef MI_SEL
@@ -277,13 +288,14 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
 // ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
-constexpr size_t DEC_MAX_LDS = 40 * 1024;  // keeps four workgroups on a CU
+constexpr size_t DEC_MAX_LDS = 40 * 1024;   // keeps four workgroups on a CU (up to four rows)
+constexpr size_t DEC_MAX_LDS8 = 76 * 1024;  // eight rows: two workgroups on a CU
 
 static size_t decode_lds_bytes(int bits, int gpt, int waves, int tpw, int mr) {
   const int cpt = (bits == 4 ? W4_TILE_K : W8_TILE_K) / 8;
   const int xl = (tpw * cpt + 63) / 64;
-  const size_t wave_lds = (size_t)mr * xl * 64 * 16 + (bits == 4 ? (size_t)tpw * gpt * 16 : 0);
-  return (size_t)waves * 256 + (size_t)waves * wave_lds;
+  const size_t wave_lds = (size_t)mr * xl * 64 * 16 + (bits == 4 ? (size_t)tpw * gpt * (mr > 4 ? 32 : 16) : 0);
+  return (size_t)waves * 256 * (mr > 4 ? 2 : 1) + (size_t)waves * wave_lds;
 }
 
 struct DecodePlan {
@@ -316,14 +328,23 @@ static DecodePlan decode_plan(const mi_a16_weight *w, int64_t M) {
     return p;  // K too long for one round of requests
   if (p.waves == 16 && p.tpw < 6)
     p.tpw = 6;  // the instantiated set
-  p.mr = M == 1 ? 1 : 4;
-  p.ok = decode_lds_bytes(w->bits, p.gpt, p.waves, p.tpw, p.mr) <= DEC_MAX_LDS;
+  p.mr = M == 1 ? 1 : M <= 4 ? 4 : 8;
+  // eight rows: one request per lane and row only (K up to 4096 at 4 bits), on the 8-wave instances, and only where
+  // it was measured ahead of the skinny kernel (us, skinny / this): 4096 x 4096 M = 5: 5.30 / 5.42, M = 8: 5.73 / 5.39;
+  // 11008 x 4096 M = 5: 9.79 / 9.84, M = 8: 11.00 / 9.84; 6144 x 2048 M = 8: 5.60 / 5.83
+  const bool rows8_pays = plan().a16_decode_rows8 ? plan().a16_decode_rows8 > 0 : (w->bits == 4 && M >= 7 && w->K >= 4096);
+  p.ok = decode_lds_bytes(w->bits, p.gpt, p.waves, p.tpw, p.mr) <= (p.mr > 4 ? DEC_MAX_LDS8 : DEC_MAX_LDS) &&
+         (p.mr <= 4 || (p.waves == 8 && rows8_pays));
   return p;
 }
 
 template <int BITS, int DT, int GPT, int W, int T, int MR>
 static void launch_decode_instance(const DecodeArgs &a, int row_blocks, size_t lds_bytes, hipStream_t st) {
-  auto kfn = a16_decode_kernel<BITS, DT, GPT, W, T, MR>;  // at most 40 KiB of LDS: inside the default limit
+  auto kfn = a16_decode_kernel<BITS, DT, GPT, W, T, MR>;
+  if constexpr (MR > 4) {  // up to 76 KiB of LDS: above the default limit (40 KiB otherwise: inside it)
+    static LdsLimitOnce once;
+    once.ensure((const void *)kfn, (int)DEC_MAX_LDS8);
+  }
   kfn<<<dim3((unsigned)row_blocks), dim3(W * 64), lds_bytes, st>>>(a);
 }
 
@@ -333,8 +354,12 @@ static bool launch_decode_shape(const DecodeArgs &a, const DecodePlan &p, int ro
   if (p.waves == W && p.tpw == T) {                                               \
     if (p.mr == 1)                                                                \
       launch_decode_instance<BITS, DT, GPT, W, T, 1>(a, row_blocks, lds, st);     \
-    else                                                                          \
+    else if (p.mr == 4)                                                           \
       launch_decode_instance<BITS, DT, GPT, W, T, 4>(a, row_blocks, lds, st);     \
+    else if constexpr (W == 8)                                                    \
+      launch_decode_instance<BITS, DT, GPT, W, T, 8>(a, row_blocks, lds, st);     \
+    else                                                                          \
+      return false;                                                               \
     return true;                                                                  \
   }
   MI_DEC_CASE(8, 2)

@@ -26,6 +26,7 @@ typedef struct mi_internal_plan {
   int i8_ring;                       // 3 / 4 / 5: LDS ring stages of the large kernel
   int dq_waves;                      // 8 / 16
   int f8_tile;                       // 256 / 128 / 64
+  int a16_decode_rows8;              // 1: five to eight rows always take the decode kernel where it can; -1: never
   int a16_wide_min_m;                // > 0: 8-bit per-channel sets take the wide tiles from this many rows on; -1: never
 } mi_internal_plan;
 void mi_internal_set_plan(const mi_internal_plan *p);  // null: back to the heuristics
