@@ -428,6 +428,16 @@ def bench_mfma_kernels(pkg, S, torch, clib, launches=10):
     out["w4_g128_prefill_M2048_4096x4096"] = {"us": round(sec * 1e6, 2),
                                               "TFLOPs": round(2.0 * 2048 * N * K / sec / 1e12, 1)}
     w.destroy()
+    # the wide-tile kernel: W8 per-channel prefill (cfg4, M = 512) and the f16 tolerance form of the W4 product
+    K, N = 4096, 11008
+    cfg = S.w8a16(1, K, N, 0, seed=31)
+    w = pkg.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=K, N=N, weight_bits=8, q_group_size=0)
+    x = _dev_bf16(torch, S.bf16_round(np.random.default_rng(5).standard_normal((512, K), dtype=np.float32)))
+    y = torch.empty((512, N), dtype=torch.bfloat16, device="cuda")
+    sec = _time_launches(torch, lambda: pkg.a16mm_launch(w, x, y), launches, warmup=2)
+    out["w8_pc_prefill_M512_11008x4096"] = {"us": round(sec * 1e6, 2), "TFLOPs": round(2.0 * 512 * N * K / sec / 1e12, 1)}
+    w.destroy()
+    out["prefill_f16_exact_vs_tolerance"] = bench_f16_prefill_forms(pkg, S, torch, clib, launches=launches)
     out["f8_matmul"] = bench_f8_matmul(pkg, torch, clib, steps=launches, shapes=((4096, 4096, 4096),))
     return out
 
