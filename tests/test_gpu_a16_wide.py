@@ -176,3 +176,46 @@ def test_tolerance_form_at_prefill_size_on_sampled_channels(orc):
           "(%d x %d sampled outputs)" % (M, N, K, g, err_def, err_ref, M, len(pick)))
     assert err_def <= 2e-5
     assert err_ref <= 1e-2
+
+
+ROWS32_CASES = [  # (M, K, N, signed, dtype): 8-bit, one scale per channel, up to 32 rows
+    (32, 4096, 1024, True, "bf16"), (17, 512, 40, False, "bf16"), (24, 1024, 200, True, "f16"), (32, 64, 16, True, "bf16"),
+    (9, 448, 33, False, "bf16"), (1, 128, 64, True, "f16"), (31, 11008, 96, True, "bf16"),
+]
+
+
+@pytest.mark.parametrize("M,K,N,signed,dt", ROWS32_CASES)
+def test_w8_per_channel_up_to_32_rows_against_oracle(orc, plan, M, K, N, signed, dt):
+    """The 32-row kernel (csrc/a16_rows32.hip; taken by itself for 17 to 32 rows, here for every row count it can
+    handle): fp32 result within 2e-5 * RMS of the oracle, outputs the reference rounding of the kernel's fp32 values."""
+    import torch
+    plan(a16_rows32_min_m=1)
+    dtype = clib.DT_F16 if dt == "f16" else clib.DT_BF16
+    cfg = S.w8a16(M, K, N, 0, seed=M + K + N, signed=signed, bias=(N % 2 == 0))
+    x, wq, scale, zp, bias = f32_valued_a16(cfg)
+    x16, scale16 = cfg["x"], cfg["scale"]
+    if dtype == clib.DT_F16:
+        x, scale = orc.F16(x), orc.F16(scale)
+        x16, scale16 = orc.f32_to_f16(x), orc.f32_to_f16(scale)
+    tdt = torch.float16 if dtype == clib.DT_F16 else torch.bfloat16
+    w = M_.A16Weight(cfg["weight"], scale16, cfg["zp"], bias, K=K, N=N, weight_bits=8, q_group_size=0, dtype=dtype)
+    xd = torch.from_numpy(x16.view(np.int16)).cuda().view(tdt)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_launch(w, xd, y_f32=y32)
+    torch.cuda.synchronize()
+    out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    pre = y32.cpu().numpy()
+    w.destroy()
+    want, want_pre = orc.a16matmul(x, wq, scale, zp, bias, M=M, K=K, N=N, weight_bits=8, q_group_size=0,
+                                   out_dtype=orc.OUT_F16 if dtype == clib.DT_F16 else orc.OUT_BF16,
+                                   gemm_kind=orc.GEMM_F64ACC)
+    err = cmp.max_abs_over_rms(pre, want_pre)
+    assert err <= 2e-5, "fp32 pre-round max-abs/RMS %.3g" % err
+    to16 = orc.f32_to_f16 if dtype == clib.DT_F16 else orc.f32_to_bf16
+    assert np.array_equal(out, to16(pre))
+    got = orc.F16(pre) if dtype == clib.DT_F16 else orc.BF16(pre)
+    rms = float(np.sqrt(np.mean(want_pre.astype(np.float64) ** 2)))
+    differ = got != want
+    assert differ.mean() < 5e-3
+    ulp16 = 2.0 ** (-10 if dtype == clib.DT_F16 else -7)
+    assert np.all(np.abs(got - want)[differ] <= np.maximum(np.abs(want[differ]) * ulp16, 4e-5 * rms))

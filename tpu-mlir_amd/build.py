@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libtpumlir_amd.so")
-SOURCES = ["a16_kernels.hip", "a16_decode.hip", "a16_gemm.hip", "a16_kn.hip", "a16_plain.hip", "a16_wide.hip", "top_a16.hip", "i8_kernels.hip", "cast_kernels.hip", "quant_kernels.hip", "dq_kernels.hip", "f8_kernels.hip", "workspace.hip", "capi.hip", "module.hip", "bench_kernels.hip"]
+SOURCES = ["a16_kernels.hip", "a16_decode.hip", "a16_gemm.hip", "a16_kn.hip", "a16_plain.hip", "a16_wide.hip", "a16_rows32.hip", "top_a16.hip", "i8_kernels.hip", "cast_kernels.hip", "quant_kernels.hip", "dq_kernels.hip", "f8_kernels.hip", "workspace.hip", "capi.hip", "module.hip", "bench_kernels.hip"]
 # packed fp32 VALU ops are switched off for every device translation unit
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -777,6 +777,14 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
   MI_REQUIRE(total_rb < (1ll << 31), MI_BAD_ARGUMENT, "mi_a16mm_launch: too many output channels for one launch");
   if (M == 0)
     return MI_SUCCESS;
+  if (a16_rows32_applicable(w, M)) {  // 8-bit, one scale per channel, 17 to 32 rows: one set per launch
+    for (int i = 0; i < n; ++i) {
+      const int rc = a16_rows32_launch(ws[i], d_x, M, d_ys[i], d_y32s ? d_y32s[i] : nullptr, stream);
+      if (rc != MI_SUCCESS)
+        return rc;
+    }
+    return MI_SUCCESS;
+  }
   if (a16_wide8_applicable(w, M)) {  // 8-bit, one scale per channel, many rows: the wide tiles, one set per launch
     for (int i = 0; i < n; ++i) {
       const int rc = a16_wide_launch(ws[i], d_x, M, d_ys[i], d_y32s ? d_y32s[i] : nullptr, stream);
