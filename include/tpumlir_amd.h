@@ -116,7 +116,9 @@ typedef struct mi_a16_weight_desc {
   int64_t K, N;
   int weight_bits;     /* 4: weight is uint8 [N,K/2], even k in the low nibble; 8: [N,K] */
   int weight_signed;   /* 8-bit only: bytes are int8 */
-  int q_group_size;    /* 0 = per channel */
+  int q_group_size;    /* 0 = per channel; any size that divides K (32, 64 and multiples of the 128- / 64-element
+                        * weight tile are packed for the MFMA kernels, other sizes are kept as stored and served by
+                        * a plain fp32 kernel) */
   int dtype;           /* MI_DT_BF16 / MI_DT_F16: type of activations, scales and outputs */
   int chip;
 } mi_a16_weight_desc;
