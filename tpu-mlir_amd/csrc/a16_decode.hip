@@ -56,8 +56,14 @@ struct DecodeArgs {
   int n_cols[DEC_MAX_SEG];          // N of the set (row stride of its outputs)
 };
 
+// The leading scalar arguments -- what stands between kernel entry and the first requests: the activations, the four
+// sets' packed weights, rows and K tiles (mk = M | k_tiles << 8), the sets' first row blocks -- are 14 dwords, which
+// this file is compiled to have preloaded into SGPRs at wave launch (-amdgpu-kernarg-preload-count): the kernel starts
+// requesting without a round trip to the argument buffer.  Everything needed later comes from the record `a`.
 template <int BITS, int DT, int GPT, int WAVES, int TPW, int MR>
-__global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
+__global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(const uint8_t *x, const uint8_t *qw0, const uint8_t *qw1,
+                                                                const uint8_t *qw2, const uint8_t *qw3, uint32_t mk,
+                                                                int rb1, int rb2, int rb3, DecodeArgs a) {
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
   constexpr int TILE_K = BITS == 4 ? W4_TILE_K : W8_TILE_K;
@@ -83,10 +89,10 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
   const int col = lane & 15, kq = lane >> 4;
 
   // ---- which weight set: everything scalar, selected (not indexed: an index would go back to memory)
-  const int s1 = rb >= a.rb_begin[1], s2 = rb >= a.rb_begin[2], s3 = rb >= a.rb_begin[3];
-#define MI_SEL(f) (s3 ? a.f[3] : s2 ? a.f[2] : s1 ? a.f[1] : a.f[0])
-  const uint8_t *qw = MI_SEL(qw) + (int64_t)rb * a.k_tiles * 1024;
-  const int k_tiles = a.k_tiles;
+  const int s1 = rb >= rb1, s2 = rb >= rb2, s3 = rb >= rb3;
+  const int M = (int)(mk & 0xffu), k_tiles = (int)(mk >> 8);
+  const uint8_t *qw = (s3 ? qw3 : s2 ? qw2 : s1 ? qw1 : qw0) + (int64_t)rb * k_tiles * 1024;
+  const uint32_t x_row_bytes = (uint32_t)k_tiles * (TILE_K * 2);
   const uint32_t lane16 = (uint32_t)lane * 16u;
 
   // ---- requests.  First this wave's slice of the activation rows (cache hits for all but the first workgroups; it
@@ -102,22 +108,35 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
     const uint32_t off = (uint32_t)(kt * TILE_K + (q % CPT) * 8) * 2u;
 #pragma unroll
     for (int r = 0; r < MR; ++r) {
-      const int row = r < a.M ? r : a.M - 1;
-      xv[r][ld] = *(const u32x4 *)(a.x + ((uint32_t)row * (uint32_t)a.x_row_bytes + off));
+      const int row = r < M ? r : M - 1;
+      xv[r][ld] = *(const u32x4 *)(x + ((uint32_t)row * x_row_bytes + off));
     }
   }
   u32x4 w[TPW];
-  uint32_t szv[TPW][GPT];
-  float nzv[TPW][GPT];
-  const uint8_t *szp = MI_SEL(sz) + (int64_t)rb * a.G * (BITS == 4 ? 64 : 32);
-  const uint8_t *nzp = nullptr;
-  if constexpr (BITS == 8)
-    nzp = MI_SEL(nz) + (int64_t)rb * a.G * 64;
 #pragma unroll
   for (int p = 0; p < TPW; ++p) {
     int kt = wave + p * WAVES;
     kt = kt < k_tiles ? kt : k_tiles - 1;  // past the end: a harmless re-load, never multiplied
     w[p] = *(const u32x4 *)(qw + ((uint32_t)kt * 1024u + lane16));
+  }
+  // Everything up to here depends on the preloaded arguments only; what follows reads the argument record.  Keep the
+  // two apart, or the wait for the record ends up in front of the requests above: the record's fields are selected by
+  // compares of their own (on a copy of the row block number the compiler cannot see through), after this point.
+  int rb_late = rb, wave_late = wave;
+  asm volatile("" : "+s"(rb_late), "+s"(wave_late) : : "memory");
+  const int t1 = rb_late >= rb1, t2 = rb_late >= rb2, t3 = rb_late >= rb3;
+#undef MI_SEL
+#define MI_SEL(f) (t3 ? a.f[3] : t2 ? a.f[2] : t1 ? a.f[1] : a.f[0])
+  uint32_t szv[TPW][GPT];
+  float nzv[TPW][GPT];
+  const uint8_t *szp = MI_SEL(sz) + (int64_t)rb_late * a.G * (BITS == 4 ? 64 : 32);
+  const uint8_t *nzp = nullptr;
+  if constexpr (BITS == 8)
+    nzp = MI_SEL(nz) + (int64_t)rb_late * a.G * 64;
+#pragma unroll
+  for (int p = 0; p < TPW; ++p) {
+    int kt = wave_late + p * WAVES;
+    kt = kt < k_tiles ? kt : k_tiles - 1;
 #pragma unroll
     for (int u = 0; u < GPT; ++u) {
       uint32_t gi = GPT == 1 ? (uint32_t)(kt >> a.group_shift) : (uint32_t)(kt * GPT + u);
@@ -176,7 +195,7 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-  const int row_ld = col < a.M ? col : a.M - 1;  // output rows past M repeat the last row; they are never stored
+  const int row_ld = col < M ? col : M - 1;  // output rows past M repeat the last row; they are never stored
   const int row_x = row_ld < MR ? row_ld : MR - 1;
   const uint8_t *xfp = xs + row_x * XROW + kq * 16;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -273,7 +292,7 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(DecodeArgs a) {
 #pragma unroll
       for (int wv = 0; wv < WAVES; ++wv)
         v += redf[((wv * RQ + h2) * 16 + col) * 4 + kq];
-      if (kq + 4 * h2 < a.M && n < n_end) {
+      if (kq + 4 * h2 < M && n < n_end) {
         v += bias_v;
         const int64_t oo = o + (int64_t)(4 * h2) * n_cols;
         if (y32)
@@ -345,7 +364,9 @@ static void launch_decode_instance(const DecodeArgs &a, int row_blocks, size_t l
     static LdsLimitOnce once;
     once.ensure((const void *)kfn, (int)DEC_MAX_LDS8);
   }
-  kfn<<<dim3((unsigned)row_blocks), dim3(W * 64), lds_bytes, st>>>(a);
+  kfn<<<dim3((unsigned)row_blocks), dim3(W * 64), lds_bytes, st>>>(a.x, a.qw[0], a.qw[1], a.qw[2], a.qw[3],
+                                                                     (uint32_t)a.M | ((uint32_t)a.k_tiles << 8),
+                                                                     a.rb_begin[1], a.rb_begin[2], a.rb_begin[3], a);
 }
 
 template <int BITS, int DT, int GPT>
