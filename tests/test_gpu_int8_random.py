@@ -1,0 +1,56 @@
+"""GPU parity of the INT8 tpu.MatMul path on seeded random shapes (any M, K, N; either weight orientation; signed
+or unsigned operands with zero points; ReLU; the Q31 per-channel requantization of the headline configuration):
+bit-exact against exact int64 arithmetic and the oracle's MultiplyByQuantizedMultiplier."""
+import numpy as np
+import pytest
+
+from helpers import pkg
+
+pytestmark = pytest.mark.gpu
+
+M_ = pkg()
+S = pkg("synth")
+clib = pkg("clib")
+
+
+def _draw_cases(seed, count):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        M = int(rng.choice([1, 2, 5, 16, 31, 64, 100, 128, 129, 255, 256, 300, 513]))
+        K = int(rng.integers(1, 1500)) if rng.integers(0, 2) else 64 * int(rng.integers(1, 24))
+        N = int(rng.integers(1, 900)) if rng.integers(0, 2) else 16 * int(rng.integers(1, 56))
+        cases.append((i, M, K, N, bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), bool(rng.integers(0, 2)),
+                      bool(rng.integers(0, 2)), bool(rng.integers(0, 2))))
+    return cases
+
+
+@pytest.mark.parametrize("i,M,K,N,rt,a_unsigned,b_unsigned,relu,requant", _draw_cases(77001, 48))
+def test_random_shape_int8_matmul(orc, i, M, K, N, rt, a_unsigned, b_unsigned, relu, requant):
+    import torch
+    c = S.int8_matmul(M, K, N, seed=500 + i, right_transpose=rt)
+    a = c["a"].view(np.uint8) if a_unsigned else c["a"]
+    b = c["b"].view(np.uint8) if b_unsigned else c["b"]
+    izp = 7 if a_unsigned else -3
+    rzp = 128 if b_unsigned else 0
+    dev = lambda t: torch.from_numpy(np.ascontiguousarray(t)).cuda()
+    rq = None
+    if requant:
+        rq = M_.RequantDesc(clib.RQ_QDM, clib.ROUND_HALF_AWAY_FROM_ZERO, out_dtype=clib.DT_I8,
+                            multiplier=dev(c["mult"]), shift=dev(c["shift"]), zp=0)
+    acc = torch.empty((M, N), dtype=torch.int32, device="cuda")
+    out = M_.i8mm_launch(dev(a), dev(b), dev(c["bias"]), right_transpose=rt, input_zp=izp, right_zp=rzp,
+                         do_relu=relu, rq=rq, acc=acc)
+    torch.cuda.synchronize()
+    b2 = (b.T if rt else b).astype(np.int64) - rzp
+    acc64 = (a.astype(np.int64) - izp) @ b2 + c["bias"].astype(np.int64)
+    if relu:  # on the accumulator, before requantization (MatMul.cpp:391 hands do_relu to the matmul itself)
+        acc64 = np.maximum(acc64, 0)
+    assert np.array_equal(acc.cpu().numpy().astype(np.int64), acc64)
+    if requant:
+        v = orc.mbqm(acc64.astype(np.int32), np.broadcast_to(c["mult"], acc64.shape),
+                     -np.broadcast_to(c["shift"], acc64.shape), orc.HALF_AWAY_FROM_ZERO).astype(np.int64)
+        want = np.clip(v, -128, 127)
+    else:
+        want = acc64
+    assert np.array_equal(out.cpu().numpy().astype(np.int64), want)
