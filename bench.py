@@ -340,6 +340,43 @@ def bench_f16_prefill_forms(pkg, S, torch, clib, launches=10):
     return out
 
 
+def bench_bf16_prefill_two_term(pkg, S, torch, clib, launches=10):
+    """W4 g128 prefill on bf16 activations, 4096 x 4096: the exact kernel the library takes (per-group fp32 fold) beside
+    the other exact form, each weight as the sum of two bf16 numbers and two MFMAs per fragment on the wide tiles.  The
+    library never picks the second by itself; it is selected here through the library's internal planning hook (the one
+    the tests use), which is not part of the C ABI."""
+    import ctypes
+    names = ("a16_waves", "a16_tpw", "a16_rows", "a16_xlds", "a16_no_gemm", "a16_no_decode", "a16_gemm_min_m",
+             "a16_gemm_splits", "a16_gemm_tile", "a16_gemm_rows", "i8_tile", "i8_mid_ring", "i8_ring", "dq_waves", "f8_tile",
+             "a16_decode_rows8", "a16_rows32_min_m", "a16_wide_min_m", "a16_wide4_min_m")
+
+    class Plan(ctypes.Structure):
+        _fields_ = [(n, ctypes.c_int) for n in names]
+
+    hook = clib.lib().mi_internal_set_plan
+    hook.argtypes, hook.restype = [ctypes.c_void_p], None
+    K = N = 4096
+    cfg = S.w4a16(1, K, N, 128, seed=31)
+    w = pkg.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=K, N=N, weight_bits=4, q_group_size=128)
+    out = []
+    try:
+        for M in (2048, 4096):
+            x = torch.randn((M, K), device="cuda").to(torch.bfloat16)
+            y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+            rec = {"M": M, "K": K, "N": N}
+            for label, mode in (("fold", -1), ("two_term", 1)):
+                p = Plan(a16_wide4_min_m=mode)
+                hook(ctypes.byref(p))
+                sec = _time_launches(torch, lambda: pkg.a16mm_launch(w, x, y), launches, warmup=2)
+                rec[label + "_us"] = round(sec * 1e6, 1)
+                rec[label + "_TFLOPs"] = round(2.0 * M * N * K / sec / 1e12, 1)
+            out.append(rec)
+    finally:
+        hook(None)
+        w.destroy()
+    return out
+
+
 def bench_dynamic_quant(pkg, S, torch, steps=40):
     """tpu.A16MatMul with dynamic integer activation quantization (activation quantizer + integer product per call),
     weights rotating through HBM; launches replayed from a HIP graph."""
@@ -666,6 +703,7 @@ def main():
             ex["chain_M%d_GBps" % m] = round(rm["chain_bytes"] / (rm["gpu_s"] / 40) / 1e9, 1)
         ex["single_matmuls"] = bench_single_matmuls(pkg, S, torch)
         ex["prefill_f16_exact_vs_tolerance"] = bench_f16_prefill_forms(pkg, S, torch, clib)
+        ex["prefill_bf16_fold_vs_two_term"] = bench_bf16_prefill_two_term(pkg, S, torch, clib)
         ex["dynamic_quant"] = bench_dynamic_quant(pkg, S, torch)
         ex["int8_256x1024x1024"] = bench_int8(pkg, S, torch, clib, 1024, 40, 5, M=256, graph=True)
         ex["f8_matmul"] = bench_f8_matmul(pkg, torch, clib)

@@ -219,3 +219,40 @@ def test_w8_per_channel_up_to_32_rows_against_oracle(orc, plan, M, K, N, signed,
     assert differ.mean() < 5e-3
     ulp16 = 2.0 ** (-10 if dtype == clib.DT_F16 else -7)
     assert np.all(np.abs(got - want)[differ] <= np.maximum(np.abs(want[differ]) * ulp16, 4e-5 * rms))
+
+
+TWO_TERM_CASES = [  # (M, K, N, g, dtype)
+    (256, 512, 128, 128, "bf16"), (300, 1024, 200, 0, "bf16"), (40, 128, 48, 128, "f16"), (513, 256, 272, 256, "f16"),
+    (512, 4096, 1024, 128, "bf16"), (1, 128, 16, 128, "bf16"), (700, 2048, 520, 512, "bf16"), (260, 1536, 136, 128, "f16"),
+]
+
+
+@pytest.mark.parametrize("M,K,N,g,dt", TWO_TERM_CASES)
+def test_w4_exact_two_term_form_on_wide_tiles_against_oracle(orc, plan, M, K, N, g, dt):
+    """Each 4-bit weight as the sum of two 16-bit numbers, two MFMAs per fragment: the reference's arithmetic (no
+    weight is rounded), held to the exact kernels' bounds."""
+    import torch
+    plan(a16_wide4_min_m=1)
+    dtype = clib.DT_F16 if dt == "f16" else clib.DT_BF16
+    cfg = S.w4a16(M, K, N, g, seed=M + K + N, bias=(N % 2 == 0))
+    x, wq, scale, zp, bias = f32_valued_a16(cfg)
+    x16, scale16 = cfg["x"], cfg["scale"]
+    if dtype == clib.DT_F16:
+        x, scale = orc.F16(x), orc.F16(scale)
+        x16, scale16 = orc.f32_to_f16(x), orc.f32_to_f16(scale)
+    tdt = torch.float16 if dtype == clib.DT_F16 else torch.bfloat16
+    w = M_.A16Weight(cfg["weight"], scale16, cfg["zp"], bias, K=K, N=N, weight_bits=4, q_group_size=g, dtype=dtype)
+    xd = torch.from_numpy(x16.view(np.int16)).cuda().view(tdt)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_launch(w, xd, y_f32=y32)
+    torch.cuda.synchronize()
+    out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    pre = y32.cpu().numpy()
+    w.destroy()
+    want, want_pre = orc.a16matmul(x, wq, scale, zp, bias, M=M, K=K, N=N, weight_bits=4, q_group_size=g,
+                                   out_dtype=orc.OUT_F16 if dtype == clib.DT_F16 else orc.OUT_BF16,
+                                   gemm_kind=orc.GEMM_F64ACC)
+    err = cmp.max_abs_over_rms(pre, want_pre)
+    assert err <= 2e-5, "fp32 pre-round max-abs/RMS %.3g" % err
+    to16 = orc.f32_to_f16 if dtype == clib.DT_F16 else orc.f32_to_bf16
+    assert np.array_equal(out, to16(pre))

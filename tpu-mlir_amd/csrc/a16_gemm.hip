@@ -479,20 +479,40 @@ static int launch_gemm_instance(GemmArgs &a, hipStream_t st, const A16Scratch *f
 
 template <int BITS, int DT, int GPT>
 static int launch_gemm_shape(GemmArgs &a, hipStream_t st, const A16Scratch *fixed) {
-  // 128 x 256 blocks when they fill the chip, else 128 x 128
-  int64_t big = 0;
-  for (int i = 0; i < a.n_seg; ++i)
+  // Output block shape.  With at least 160 of the widest blocks no K split is made and the time of a launch is set by
+  // how the blocks divide among the 256 CUs: one 128 x 256 or 128 x 128 workgroup per CU, two 64 x 128 ones (which
+  // overlap).  Measured at K = 4096, 4-bit g = 128, in us: 94 per round of 128 x 256 blocks, 50.5 per round of
+  // 128 x 128, 35 for the first 256 blocks of 64 x 128 and 24.5 for each further 256 -- all three grow alike with K, so
+  // the cheapest by this count is taken (11008 x 4096: M = 768 187 -> 128 us, M = 1024 188 -> 152, M = 1536 281 -> 230;
+  // 4096 x 4096: M = 1280 98 -> 78, M = 3072 187 -> 155).  Below that, where K is split: wide blocks never, 64 rows up
+  // to M = 640 (measured).
+  int64_t big = 0, t128 = 0, t64 = 0;
+  for (int i = 0; i < a.n_seg; ++i) {
     big += ((a.M + 127) / 128) * ((a.seg[i].N + 255) / 256);
+    t128 += ((a.M + 127) / 128) * ((a.seg[i].N + 127) / 128);
+    t64 += ((a.M + 63) / 64) * ((a.seg[i].N + 127) / 128);
+  }
   const int tile = plan().a16_gemm_tile;
   constexpr bool fits = !(BITS == 4 && GPT == 4);  // 32-wide groups: a 256-column block's scale|zp words overflow LDS
-  const bool wide = fits && (tile ? tile == 256 : big >= 192);
+  int rows = plan().a16_gemm_rows;
+  bool wide = fits && tile == 256;
+  if (tile == 0 && rows == 0 && big >= 160) {
+    const double c_wide = fits ? 94.0 * (double)((big + 255) / 256) : 1e30;
+    const double c_128 = 50.5 * (double)((t128 + 255) / 256);
+    const double c_64 = 35.0 + 24.5 * (double)((t64 + 255) / 256 - 1);
+    if (c_wide <= c_128 && c_wide <= c_64)
+      wide = true;
+    else
+      rows = c_128 <= c_64 ? 128 : 64;
+  }
   if constexpr (fits) {
     if (wide)
       return launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 4>(a, st, fixed);
   }
   (void)wide;
   // few rows: shorter blocks waste fewer MFMAs on rows that do not exist
-  const int rows = plan().a16_gemm_rows ? plan().a16_gemm_rows : (a.M <= 16 ? 16 : a.M <= 32 ? 32 : a.M <= 640 ? 64 : 128);  // measured: 64-row blocks win up to there
+  if (rows == 0)
+    rows = a.M <= 16 ? 16 : a.M <= 32 ? 32 : a.M <= 640 ? 64 : 128;  // measured: 64-row blocks win up to there
   if (rows == 16)
     return launch_gemm_instance<BITS, DT, GPT, 1, 8, 1, 1>(a, st, fixed);
   if (rows == 32)

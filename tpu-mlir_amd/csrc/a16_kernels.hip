@@ -785,9 +785,11 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
     }
     return MI_SUCCESS;
   }
-  if (a16_wide8_applicable(w, M)) {  // 8-bit, one scale per channel, many rows: the wide tiles, one set per launch
+  // 8-bit, one scale per channel, or 4-bit in the exact two-term form; many rows: the wide tiles, one set per launch
+  const bool wide4 = a16_wide4_applicable(w, M);
+  if (wide4 || a16_wide8_applicable(w, M)) {
     for (int i = 0; i < n; ++i) {
-      const int rc = a16_wide_launch(ws[i], d_x, M, d_ys[i], d_y32s ? d_y32s[i] : nullptr, stream);
+      const int rc = a16_wide_launch(ws[i], d_x, M, d_ys[i], d_y32s ? d_y32s[i] : nullptr, stream, wide4);
       if (rc != MI_SUCCESS)
         return rc;
     }

@@ -77,6 +77,28 @@ __device__ __forceinline__ f16x8 tol_dequant(uint32_t d, float s, float nzs, uin
   return w;
 }
 
+// The exact form for 4-bit weights, either 16-bit type: the weight w = (q - zp) * s has at most 4 + 11 significant bits,
+// so it IS the sum of two 16-bit numbers, hi = round16(w) and lo = w - hi (exact, a handful of bits), and
+// sum a * w = sum a * hi + sum a * lo with every product exact in the fp32 accumulator: two MFMAs per fragment and no
+// per-group fold.  w itself comes out of one fp32 fma, exactly: (16 + q) * s - (16 + zp) * s.
+template <int DT>
+__device__ __forceinline__ void two_term_dequant(uint32_t d, float s, float nzs, uint32_t magic,
+                                                 typename Half16<DT>::vec8 &hi, typename Half16<DT>::vec8 &lo) {
+  using H = Half16<DT>;
+  const u32x4 q2 = __builtin_bit_cast(u32x4, unpack_nibbles<DT>(d, magic));
+  u32x4 hb, lb;
+#pragma unroll
+  for (int pr = 0; pr < 4; ++pr) {
+    const float w0 = fmaf(H::to_f32((uint16_t)(q2[pr] & 0xffffu)), s, nzs);
+    const float w1 = fmaf(H::to_f32((uint16_t)(q2[pr] >> 16)), s, nzs);
+    const uint32_t hp = H::pack2(w0, w1);
+    hb[pr] = hp;
+    lb[pr] = H::pack2(w0 - H::to_f32((uint16_t)(hp & 0xffffu)), w1 - H::to_f32((uint16_t)(hp >> 16)));
+  }
+  hi = __builtin_bit_cast(typename H::vec8, hb);
+  lo = __builtin_bit_cast(typename H::vec8, lb);
+}
+
 // GPT: quantization groups per K tile (1: a group is one or more whole tiles, group of tile kt = kt >> group_shift)
 // Weight-side loads the compiler does not know to be loads: it would otherwise guard their first use with waits of its
 // own, and at the head of the main loop those come out as "wait for everything", which drains the activation ring.
@@ -106,9 +128,11 @@ __device__ __forceinline__ f32x16 wide_mfma(typename Half16<DT>::vec8 a, typenam
 
 // BITS == 4: f16 only, groups of whole 128-K tiles (group of tile kt = kt >> group_shift).  BITS == 8: one scale per
 // channel, either 16-bit type.
-template <int BITS, int DT>
+// TT (4-bit only): the exact two-term form instead of weights rounded once.
+template <int BITS, int DT, bool TT>
 __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m, int tiles_n, int per_xcd) {
-  static_assert(BITS == 8 || DT == MI_DT_F16, "4-bit weights rounded to bf16 leave the comparison tolerance");
+  static_assert(BITS == 8 || DT == MI_DT_F16 || TT, "4-bit weights rounded to bf16 leave the comparison tolerance");
+  static_assert(BITS == 4 || !TT, "8-bit weights are rounded to the 16-bit type by the reference itself");
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
   constexpr int WL = TolW<BITS>::WL, WRING = TolW<BITS>::RING, UNIT_ST = TolW<BITS>::UNIT_ST;
@@ -237,7 +261,7 @@ __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m
   // B fragments of k-step su (0 .. 4 * UNIT_ST - 1) of the weight tile in ring slot rs.  Even k-steps take their
   // eight K elements from slot kq = h, odd ones from slot h + 2; 4-bit: word su / 2 of the slot, 8-bit: words
   // 2 * (su / 2) and the next.
-  auto make_b = [&](vec8 (&fb)[2], int rs, int su) {
+  auto make_b = [&](vec8 (&fb)[2], vec8 (&fl)[2], int rs, int su) {
 #pragma unroll
     for (int jb = 0; jb < 2; ++jb) {
       if constexpr (BITS == 4) {
@@ -245,7 +269,10 @@ __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m
         const uint32_t szv = szw[rs][jb][0];
         const float s = H::to_f32((uint16_t)(szv >> 16));
         const float nzs = -(H::OFFSET + (float)(szv & 0xffu)) * s;
-        fb[jb] = tol_dequant(word, s, nzs, nib_magic);
+        if constexpr (TT)
+          two_term_dequant<DT>(word, s, nzs, nib_magic, fb[jb], fl[jb]);
+        else if constexpr (DT == MI_DT_F16)
+          fb[jb] = tol_dequant(word, s, nzs, nib_magic);
       } else {
         const int j = su >> 1;
         fb[jb] = dequant_bytes<DT>(wq[rs][jb][su & 1][2 * j], wq[rs][jb][su & 1][2 * j + 1], s8[jb], nz8[jb]);
@@ -274,12 +301,12 @@ __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m
     issue_part(2, part);
   issue_part(TOL_NST - 1, 0);
   u32x4 fa[2][4];
-  vec8 fb[2][2];
+  vec8 fb[2][2], fl[2][2];  // B fragments of this and the next k-step (fl: the low terms of the two-term form)
   __builtin_amdgcn_s_waitcnt(tol_waitcnt_vm((TOL_NST - 2) * TOL_LOADS + TOL_PART + WL));  // stage 0 landed
   __builtin_amdgcn_s_barrier();
   w_arrived(0);
   read_frags(fa[0], 0, 0);
-  make_b(fb[0], 0, 0);
+  make_b(fb[0], fl[0], 0, 0);
 
   // ---- main loop over weight tiles, a ring's worth at a time so that the weight ring is indexed statically.  One
   // stage = 4 k-steps of 8 MFMAs; the barrier sits before the last k-step of a stage (see the INT8 large-tile kernel):
@@ -305,7 +332,7 @@ __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m
           if (ks + 1 < TOL_KS) {
             issue_part(st + TOL_NST - 1, ks + 1);
             read_frags(fa[nxt], st, ks + 1);
-            make_b(fb[nxt], rs, su + 1);
+            make_b(fb[nxt], fl[nxt], rs, su + 1);
           } else {
             __builtin_amdgcn_s_waitcnt(TOL_WAITCNT_LGKM0);
             // 8-bit: the weight tile of the next stage went out one stage ago, after that stage's last part; the
@@ -317,10 +344,10 @@ __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m
             issue_part(st + TOL_NST, 0);
             read_frags(fa[nxt], st + 1, 0);
             if (hs + 1 < UNIT_ST) {
-              make_b(fb[nxt], rs, su + 1);
+              make_b(fb[nxt], fl[nxt], rs, su + 1);
             } else {
               w_arrived((rs + 1) % WRING);  // requested early enough for the wait above to cover it
-              make_b(fb[nxt], (rs + 1) % WRING, 0);
+              make_b(fb[nxt], fl[nxt], (rs + 1) % WRING, 0);
             }
           }
 #pragma unroll
@@ -328,6 +355,13 @@ __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m
 #pragma unroll
             for (int j = 0; j < 2; ++j)
               acc[i][j] = wide_mfma<DT>(__builtin_bit_cast(vec8, fa[cur][i]), fb[cur][j], acc[i][j]);
+          if constexpr (TT) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+              for (int j = 0; j < 2; ++j)
+                acc[i][j] = wide_mfma<DT>(__builtin_bit_cast(vec8, fa[cur][i]), fl[cur][j], acc[i][j]);
+          }
         }
       }
     }
@@ -406,6 +440,23 @@ bool a16_tol_applicable(const mi_a16_weight *w) {
   return (tpg & (tpg - 1)) == 0 || tpg >= w->k_tiles;
 }
 
+// 4-bit weight sets in the tiled layout with groups of whole tiles, either 16-bit type: the exact two-term form on the
+// wide tiles.
+bool a16_wide4_applicable(const mi_a16_weight *w, int64_t M) {
+  if (!w || !w->qweight || w->kn || w->plain || w->bits != 4 || (w->K % W4_TILE_K) != 0)
+    return false;
+  if (w->g != 0) {
+    if (w->g % W4_TILE_K != 0)
+      return false;
+    const int tpg = w->g / W4_TILE_K;
+    if ((tpg & (tpg - 1)) != 0 && tpg < w->k_tiles)
+      return false;
+  }
+  if (plan().a16_wide4_min_m != 0)
+    return plan().a16_wide4_min_m > 0 && M >= plan().a16_wide4_min_m;
+  return false;
+}
+
 // 8-bit weight sets with one scale per channel: the wide tiles are the reference's arithmetic, and faster than the
 // tiled kernel once there are enough 256 x 128 tiles to occupy the chip.  Measured, bf16, tiled / wide in us:
 //   11008 x 4096   M = 256 (86 tiles): 76.5 / 69.6   M = 384 (172): 110.1 / 73.8   M = 512: 111.7 / 75.7   M = 2048: 323.6 / 224.9
@@ -420,7 +471,7 @@ bool a16_wide8_applicable(const mi_a16_weight *w, int64_t M) {
 }
 
 int a16_wide_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
-                    hipStream_t stream) {
+                    hipStream_t stream, bool two_term) {
   MI_REQUIRE(M >= 0 && M < (1ll << 31), MI_BAD_ARGUMENT, "mi_a16mm_launch: M out of range");
   if (M == 0)
     return MI_SUCCESS;
@@ -455,17 +506,25 @@ int a16_wide_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
   const int per_xcd = (int)((tiles_m * tiles_n + 7) / 8);
   const size_t lds_bytes = (size_t)TOL_NST * TOL_STAGE_BYTES;
   const dim3 grid((unsigned)(per_xcd * 8)), block(256);
-  static LdsLimitOnce once4, once8b, once8h;
-  if (w->bits == 4) {
-    auto kfn = a16_wide_kernel<4, MI_DT_F16>;
+  static LdsLimitOnce once4, once8b, once8h, once4tb, once4th;
+  if (w->bits == 4 && two_term && w->dtype == MI_DT_BF16) {
+    auto kfn = a16_wide_kernel<4, MI_DT_BF16, true>;
+    once4tb.ensure((const void *)kfn, (int)lds_bytes);
+    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
+  } else if (w->bits == 4 && two_term) {
+    auto kfn = a16_wide_kernel<4, MI_DT_F16, true>;
+    once4th.ensure((const void *)kfn, (int)lds_bytes);
+    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
+  } else if (w->bits == 4) {
+    auto kfn = a16_wide_kernel<4, MI_DT_F16, false>;
     once4.ensure((const void *)kfn, (int)lds_bytes);
     kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
   } else if (w->dtype == MI_DT_F16) {
-    auto kfn = a16_wide_kernel<8, MI_DT_F16>;
+    auto kfn = a16_wide_kernel<8, MI_DT_F16, false>;
     once8h.ensure((const void *)kfn, (int)lds_bytes);
     kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
   } else {
-    auto kfn = a16_wide_kernel<8, MI_DT_BF16>;
+    auto kfn = a16_wide_kernel<8, MI_DT_BF16, false>;
     once8b.ensure((const void *)kfn, (int)lds_bytes);
     kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
   }
@@ -478,7 +537,7 @@ int a16_tol_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint1
   MI_REQUIRE(a16_tol_applicable(w), MI_UNSUPPORTED,
              "mi_a16mm_launch_tol: 4-bit f16 weight sets with K a multiple of 128 and groups of 128 * 2^k or one per "
              "channel only (bf16 weights rounded to bf16 leave the comparison tolerance)");
-  return a16_wide_launch(w, d_x, M, d_y, d_y32, stream);
+  return a16_wide_launch(w, d_x, M, d_y, d_y32, stream, false);
 }
 
 }  // namespace mi

@@ -29,6 +29,7 @@ typedef struct mi_internal_plan {
   int a16_decode_rows8;              // 1: five to eight rows always take the decode kernel where it can; -1: never
   int a16_rows32_min_m;              // > 0: 8-bit per-channel sets take the 32-row kernel from this many rows (to 32); -1: never
   int a16_wide_min_m;                // > 0: 8-bit per-channel sets take the wide tiles from this many rows on; -1: never
+  int a16_wide4_min_m;               // > 0: 4-bit sets take the exact two-term wide tiles from this many rows on; -1: never
 } mi_internal_plan;
 void mi_internal_set_plan(const mi_internal_plan *p);  // null: back to the heuristics
 }
@@ -117,14 +118,16 @@ int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t 
                hipStream_t stream);
 int a16_kn_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32, hipStream_t st);
 // wide-tile product (a16_wide.hip), weights rounded to the 16-bit type before the multiply: the reference's arithmetic
-// for 8-bit per-channel sets (taken from a few hundred rows on), the opt-in tolerance form for 4-bit f16 sets
+// for 8-bit per-channel sets (taken from a few hundred rows on), the opt-in tolerance form for 4-bit f16 sets; and the
+// exact two-term form for 4-bit sets (each weight as the sum of two 16-bit numbers, two MFMAs per fragment)
 // 8-bit per-channel sets, 9 to 32 rows (a16_rows32.hip)
 bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M);
 int a16_rows32_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                       hipStream_t stream);
 bool a16_wide8_applicable(const mi_a16_weight *w, int64_t M);
+bool a16_wide4_applicable(const mi_a16_weight *w, int64_t M);
 int a16_wide_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
-                    hipStream_t stream);
+                    hipStream_t stream, bool two_term);
 bool a16_tol_applicable(const mi_a16_weight *w);
 int a16_tol_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                    hipStream_t stream);
