@@ -1,0 +1,89 @@
+"""GPU parity of the 32-row kernel (csrc/a16_rows32.hip) on 4-bit weight sets: the exact kernels' arithmetic, held to
+their bounds -- fp32 result within 2e-5 * RMS(output) of the oracle's float64 accumulation, outputs the reference
+rounding of the kernel's own fp32 values.  The plan sends every row count the kernel can handle through it (by itself
+the library takes it for 17 to 32 rows, and from 13 on large sets); single sets and sibling sets sharing a launch."""
+import numpy as np
+import pytest
+
+from helpers import pkg, f32_valued_a16
+
+pytestmark = pytest.mark.gpu
+
+M_ = pkg()
+S = pkg("synth")
+clib = pkg("clib")
+cmp = pkg("compare")
+
+ROWS32_W4_CASES = [  # (M, K, N, g, dtype)
+    (17, 512, 64, 128, "bf16"), (32, 1024, 200, 0, "bf16"), (9, 128, 48, 128, "f16"), (24, 256, 272, 256, "f16"),
+    (32, 4096, 1024, 128, "bf16"), (1, 128, 16, 128, "bf16"), (20, 2048, 520, 512, "bf16"), (31, 1536, 136, 64, "f16"),
+    (18, 1920, 100, 64, "bf16"), (32, 3200, 40, 128, "bf16"), (25, 1152, 33, 0, "f16"),
+]
+
+
+@pytest.mark.parametrize("M,K,N,g,dt", ROWS32_W4_CASES)
+def test_w4_up_to_32_rows_against_oracle(orc, plan, M, K, N, g, dt):
+    import torch
+    plan(a16_rows32_min_m=1)
+    dtype = clib.DT_F16 if dt == "f16" else clib.DT_BF16
+    cfg = S.w4a16(M, K, N, g, seed=M + K + N, bias=(N % 2 == 0))
+    x, wq, scale, zp, bias = f32_valued_a16(cfg)
+    x16, scale16 = cfg["x"], cfg["scale"]
+    if dtype == clib.DT_F16:
+        x, scale = orc.F16(x), orc.F16(scale)
+        x16, scale16 = orc.f32_to_f16(x), orc.f32_to_f16(scale)
+    tdt = torch.float16 if dtype == clib.DT_F16 else torch.bfloat16
+    w = M_.A16Weight(cfg["weight"], scale16, cfg["zp"], bias, K=K, N=N, weight_bits=4, q_group_size=g, dtype=dtype)
+    xd = torch.from_numpy(x16.view(np.int16)).cuda().view(tdt)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_launch(w, xd, y_f32=y32)
+    torch.cuda.synchronize()
+    out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    pre = y32.cpu().numpy()
+    w.destroy()
+    want, want_pre = orc.a16matmul(x, wq, scale, zp, bias, M=M, K=K, N=N, weight_bits=4, q_group_size=g,
+                                   out_dtype=orc.OUT_F16 if dtype == clib.DT_F16 else orc.OUT_BF16,
+                                   gemm_kind=orc.GEMM_F64ACC)
+    err = cmp.max_abs_over_rms(pre, want_pre)
+    assert err <= 2e-5, "fp32 pre-round max-abs/RMS %.3g" % err
+    to16 = orc.f32_to_f16 if dtype == clib.DT_F16 else orc.f32_to_bf16
+    assert np.array_equal(out, to16(pre))
+
+
+@pytest.mark.parametrize("M,K,Ns,g,dt", [(20, 512, (100, 64, 33), 128, "bf16"), (32, 1024, (48, 272), 64, "bf16"),
+                                        (17, 256, (16, 40, 96, 130), 0, "f16")])
+def test_w4_sibling_sets_share_a_launch(orc, plan, M, K, Ns, g, dt):
+    """q/k/v-style groups, channel counts that are not multiples of 32 included: each set's output against the oracle."""
+    import torch
+    plan(a16_rows32_min_m=1)
+    dtype = clib.DT_F16 if dt == "f16" else clib.DT_BF16
+    tdt = torch.float16 if dtype == clib.DT_F16 else torch.bfloat16
+    cfgs = [S.w4a16(M, K, N, g, seed=7 * i + N, bias=(i % 2 == 0)) for i, N in enumerate(Ns)]
+    x16 = cfgs[0]["x"]
+    xf = S.bf16_to_f32(x16)
+    if dtype == clib.DT_F16:
+        xf = orc.F16(xf)
+        x16 = orc.f32_to_f16(xf)
+    ws, refs = [], []
+    for cfg in cfgs:
+        _, wq, scale, zp, bias = f32_valued_a16(cfg)
+        scale16 = cfg["scale"]
+        if dtype == clib.DT_F16:
+            scale = orc.F16(scale)
+            scale16 = orc.f32_to_f16(scale)
+        ws.append(M_.A16Weight(cfg["weight"], scale16, cfg["zp"], bias, K=K, N=cfg["N"], weight_bits=4, q_group_size=g,
+                               dtype=dtype))
+        refs.append(orc.a16matmul(xf, wq, scale, zp, bias, M=M, K=K, N=cfg["N"], weight_bits=4, q_group_size=g,
+                                  out_dtype=orc.OUT_F16 if dtype == clib.DT_F16 else orc.OUT_BF16,
+                                  gemm_kind=orc.GEMM_F64ACC))
+    xd = torch.from_numpy(x16.view(np.int16)).cuda().view(tdt)
+    y32s = [torch.empty((M, N), dtype=torch.float32, device="cuda") for N in Ns]
+    ys = M_.a16mm_launch_group(ws, xd, ys_f32=y32s)
+    torch.cuda.synchronize()
+    to16 = orc.f32_to_f16 if dtype == clib.DT_F16 else orc.f32_to_bf16
+    for y, y32, (want, want_pre) in zip(ys, y32s, refs):
+        pre = y32.cpu().numpy()
+        assert cmp.max_abs_over_rms(pre, want_pre) <= 2e-5
+        assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), to16(pre))
+    for w in ws:
+        w.destroy()

@@ -777,13 +777,15 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
   MI_REQUIRE(total_rb < (1ll << 31), MI_BAD_ARGUMENT, "mi_a16mm_launch: too many output channels for one launch");
   if (M == 0)
     return MI_SUCCESS;
-  if (a16_rows32_applicable(w, M)) {  // 8-bit, one scale per channel, 17 to 32 rows: one set per launch
-    for (int i = 0; i < n; ++i) {
-      const int rc = a16_rows32_launch(ws[i], d_x, M, d_ys[i], d_y32s ? d_y32s[i] : nullptr, stream);
-      if (rc != MI_SUCCESS)
-        return rc;
-    }
-    return MI_SUCCESS;
+  {  // a few tens of rows: one workgroup per 32 channels over the whole K
+    int64_t blocks = 0;
+    for (int i = 0; i < n; ++i)
+      blocks += (ws[i]->N + 31) / 32;
+    bool all = true;
+    for (int i = 0; i < n; ++i)
+      all = all && a16_rows32_applicable(ws[i], M, blocks);
+    if (all)
+      return a16_rows32_launch_group(ws, n, d_x, M, d_ys, d_y32s, stream);
   }
   // 8-bit, one scale per channel, or 4-bit in the exact two-term form; many rows: the wide tiles, one set per launch
   const bool wide4 = a16_wide4_applicable(w, M);

@@ -1,14 +1,21 @@
-// W8A16 matmul, one scale per channel, for 17 to 32 activation rows: too many rows for the decode / skinny kernels (which
-// re-read the weights once per 16 rows), too few for output tiles that share the activations through LDS.  HBM-bound on
-// the weights: a workgroup owns 32 output channels over the whole K, its eight waves take the 64-K weight tiles
+// W8A16 / W4A16 matmul for a few tens of activation rows (up to 32): too many rows for the decode / skinny kernels
+// (which re-read the weights once per 16 rows), too few for output tiles that share the activations through LDS.
+// HBM-bound on the weights: a workgroup owns 32 output channels over the whole K, its eight waves take the weight tiles
 // round-robin, and every wave multiplies ALL activation rows (one 32 x 32 MFMA block: rows past M repeat the last row
-// and are never stored) against its tiles.  The 8-bit weights are dequantized in registers exactly as the reference
-// does it -- w16 = round16((q - zp) * scale), A16MatMul.cpp:209-231 -- from the packed layout (lane slot = 16 bytes;
-// a lane's two slots of a tile hold its four k-steps' fragments, see a16_wide.hip); the activation fragments come
-// straight from L2, 16 bytes per lane and k-step (a row's 128 bytes of a tile are read by its two lanes in four
-// requests).  Requests run ahead of the arithmetic in a register ring -- weights two tiles ahead (they come from HBM),
-// activations one (they come from L2) -- through loads the compiler does not track, under explicit counts.  The eight
-// partial 32 x 32 blocks are summed once through LDS, in wave order, two accumulator registers per wave.
+// and are never stored) against its tiles.  Weights come straight from the packed layout into registers (lane slot =
+// 16 bytes; a lane's two slots of a tile hold its k-steps' fragments, see a16_wide.hip), two tiles ahead, through loads
+// the compiler does not track, under explicit counts.  Activations: every workgroup reads all of x from L2, which is
+// what this kernel's time grows with, so they are requested in whole cache lines -- a wave's requests go direct to
+// LDS, eight rows x 128 bytes each, into the wave's own two-slot ring (16-byte chunks XOR-swizzled by row), one
+// 64-K piece ahead -- and the MFMA fragments are read back from there (fragments requested straight from L2, 32
+// bytes of each of 32 rows per request, cost 26 instead of 17 us at 11008 x 4096, M = 32).  No barrier in the loop:
+// a wave reads only what it requested itself.  The eight partial 32 x 32 blocks are summed once through LDS, in wave
+// order, two accumulator registers per wave.
+//   8-bit, one scale per channel: dequantized in registers exactly as the reference does it,
+//     w16 = round16((q - zp) * scale), A16MatMul.cpp:209-231.
+//   4-bit: the exact kernels' arithmetic (a16_kernels.hip): per weight tile P = sum a (16 + q) and S = sum a by MFMA
+//     (S against ones: it comes out in the accumulator layout, and the matrix unit is idle here anyway), then
+//     acc += scale * (P - (16 + zp) * S) in fp32.
 #include <climits>
 
 #include "a16_common.cuh"
@@ -17,6 +24,8 @@
 namespace mi {
 
 typedef __attribute__((ext_vector_type(16))) float r32_f32x16;
+typedef const __attribute__((address_space(1))) void *r32_gptr_t;
+typedef __attribute__((address_space(3))) void *r32_lptr_t;
 
 struct Rows32Args {
   const uint8_t *x;      // [M][K] 16-bit
@@ -54,7 +63,10 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
   constexpr int WAVES = 8;
-  __shared__ float red[WAVES][16][64];  // 32 KiB: partial blocks, [wave][register][lane]
+  // 64 KiB: per wave a ring of two activation tiles (32 rows x 128 bytes, 16-byte chunks XOR-swizzled by row); after
+  // the loop the first 32 KiB hold the partial blocks, [wave][register][lane]
+  __shared__ __attribute__((aligned(16))) uint8_t smem[WAVES * 2 * 4096];
+  float (*red)[16][64] = reinterpret_cast<float (*)[16][64]>(smem);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c32 = lane & 31, h = lane >> 5;
@@ -68,8 +80,17 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
   // The compiler knows these two as loads and would wait for them where they are first used -- inside the loop, as a
   // wait for everything, since it does not count the requests below.  Used here, they are waited for here.
   asm volatile("" : "+v"(sc), "+v"(nz));
-  const int row = c32 < a.M ? c32 : a.M - 1;
-  const uint8_t *xp = a.x + (int64_t)row * a.K * 2 + h * 16;
+  // activations, direct to LDS: request i of a tile covers rows 8 i .. 8 i + 7 whole (lane l: row 8 i + l / 8,
+  // position l % 8, which holds the row's chunk (position ^ row % 8)): eight full cache lines per request
+  const uint8_t *xg[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 8 * i + (lane >> 3);
+    const int rr = r < a.M ? r : a.M - 1;  // rows past M repeat the last row; never stored
+    xg[i] = a.x + (int64_t)rr * a.K * 2 + (((lane & 7) ^ (r & 7)) << 4);
+  }
+  uint8_t *xs = smem + wave * 8192;
+  const uint8_t *xf = xs + c32 * 128;  // this lane's fragment row; chunk c sits at position c ^ (c32 & 7)
 
   // this wave's tiles: wave, wave + 8, ...; `count` of them (the same for every lane)
   const int count = (a.k_tiles - wave + WAVES - 1) / WAVES;
@@ -78,12 +99,11 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
     return wave + ii * WAVES;
   };
   u32x4 w[3][2];   // weight ring: [tile % 3][slot kq = h, h + 2]
-  u32x4 xa[2][4];  // activation ring: [tile % 2][k-step]
   auto issue_x = [&](int i, int rs) {
-    const uint8_t *p = xp + (int64_t)tile_of(i) * 128;
+    const int64_t koff = (int64_t)tile_of(i) * 128;
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
-      xa[rs][s] = r32_load16(p + 32 * s);
+    for (int q = 0; q < 4; ++q)
+      __builtin_amdgcn_global_load_lds((r32_gptr_t)(xg[q] + koff), (r32_lptr_t)(xs + rs * 4096 + q * 1024), 16, 0, 0);
   };
   auto issue_w = [&](int i, int rs) {
     const uint8_t *p = wp + (int64_t)tile_of(i) * 1024;
@@ -113,12 +133,16 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
         __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(8));
         r32_arrived(w[u % 3][0]);
         r32_arrived(w[u % 3][1]);
+        asm volatile("" ::: "memory");  // the tile's activations are in LDS from here on, not before
+        u32x4 fa[4];
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          fa[s] = *(const u32x4 *)(xf + (u % 2) * 4096 + (((2 * s + h) ^ (c32 & 7)) << 4));
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-          r32_arrived(xa[u % 2][s]);
           const int j = s >> 1;
           const vec8 b = dequant_bytes<DT>(w[u % 3][s & 1][2 * j], w[u % 3][s & 1][2 * j + 1], sc, nz);
-          acc = r32_mfma<DT>(__builtin_bit_cast(vec8, xa[u % 2][s]), b, acc);
+          acc = r32_mfma<DT>(__builtin_bit_cast(vec8, fa[s]), b, acc);
         }
       }
     }
@@ -126,6 +150,7 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
   }
 
   // ---- cross-wave sum, in wave order.  Register r of lane l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
+  __syncthreads();  // the partial blocks overlay the activation rings: every wave is done with its tiles
 #pragma unroll
   for (int r = 0; r < 16; ++r)
     red[wave][r][lane] = acc[r];
@@ -149,44 +174,302 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
   }
 }
 
-// 8-bit, one scale per channel, K a whole number of tiles: taken for 17 to 32 rows.  Measured, bf16, the kernels
-// otherwise taken (skinny up to 16 rows, tiled + split-K above) / this one, in us:
-//   11008 x 4096   M = 9: 15.7 / 15.1   M = 16: 22.2 / 18.6   M = 17: 28.4 / 18.3   M = 24: 28.8 / 22.2   M = 32: 29.1 / 26.6
-//   4096 x 4096    M = 9:  6.5 /  8.4   M = 16:  7.6 / 10.0   M = 17: 14.5 / 10.2   M = 24: 15.0 / 12.0   M = 32: 15.3 / 14.3
-// Its time grows with the rows: every workgroup reads all of the activations (M * K * 2 bytes, from L2).
-bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M) {
-  if (!w || !w->qweight || w->kn || w->plain || w->bits != 8 || w->g != 0 || (w->K % W8_TILE_K) != 0)
-    return false;
-  if (plan().a16_rows32_min_m != 0)
-    return plan().a16_rows32_min_m > 0 && M >= plan().a16_rows32_min_m && M <= 32;
-  return M >= 17 && M <= 32;
+// 4-bit weights; groups of whole 128-K tiles (group of tile kt = kt >> group_shift; 31: one group per channel) or,
+// GPT = 2, of 64.  A step of the loop is half a weight tile: 64 K elements, four MFMA k-steps, one activation piece.
+constexpr int R32_MAX_SETS = 4;
+// Sibling weight sets on one input (q/k/v, gate/up: same K, group size and type) share a launch: their 32-channel
+// blocks are numbered one set after the other, and a workgroup tells its set by three scalar compares.
+struct Rows32W4Args {
+  const uint8_t *x;                     // [M][K] 16-bit
+  int64_t K;
+  int M, k_tiles, G, group_shift, chip;
+  int block_begin[R32_MAX_SETS];        // first workgroup of each set (unused slots: INT_MAX)
+  const uint8_t *qw[R32_MAX_SETS];      // packed tiles [row_blocks][k_tiles][1024]
+  const uint32_t *sz[R32_MAX_SETS];     // scale|zp words [row_blocks][G][16]
+  const float *bias[R32_MAX_SETS];      // [N] or null
+  uint16_t *y[R32_MAX_SETS];            // [M][N]
+  float *y32[R32_MAX_SETS];             // [M][N] or null
+  int64_t N[R32_MAX_SETS];
+  int row_blocks[R32_MAX_SETS];
+};
+
+__device__ __forceinline__ uint32_t r32_load4(const void *p) {
+  uint32_t v;
+  asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+  return v;
 }
 
-int a16_rows32_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
-                      hipStream_t stream) {
+template <int DT, int GPT>
+__global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
+  using H = Half16<DT>;
+  using vec8 = typename H::vec8;
+  constexpr int WAVES = 8;
+  constexpr int WL = 2 + GPT;  // weight-side requests per tile
+  __shared__ __attribute__((aligned(16))) uint8_t smem[WAVES * 2 * 4096];
+  float (*red)[16][64] = reinterpret_cast<float (*)[16][64]>(smem);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c32 = lane & 31, h = lane >> 5;
+  // which weight set: selected, not indexed (a runtime index would move the argument block to scratch memory)
+  const int bid = blockIdx.x;
+  const int t1 = bid >= a.block_begin[1], t2 = bid >= a.block_begin[2], t3 = bid >= a.block_begin[3];
+#define R32_SEL(f) (t3 ? a.f[3] : t2 ? a.f[2] : t1 ? a.f[1] : a.f[0])
+  const int lb = bid - R32_SEL(block_begin);  // the set's own 32-channel block
+  const int64_t set_n = R32_SEL(N);
+  const int set_rbs = R32_SEL(row_blocks);
+  const int64_t n = (int64_t)lb * 32 + c32;
+
+  int64_t rb = (int64_t)lb * 2 + (c32 >> 4);
+  rb = rb < set_rbs ? rb : set_rbs - 1;  // channels past N repeat the last row block; never stored
+  const uint8_t *wp = R32_SEL(qw) + rb * a.k_tiles * 1024 + (uint32_t)((h * 16 + (c32 & 15)) * 16);
+  const uint32_t *szp = R32_SEL(sz) + rb * a.G * 16 + (c32 & 15);
+  const uint8_t *xg[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 8 * i + (lane >> 3);
+    const int rr = r < a.M ? r : a.M - 1;
+    xg[i] = a.x + (int64_t)rr * a.K * 2 + (((lane & 7) ^ (r & 7)) << 4);
+  }
+  uint8_t *xs = smem + wave * 8192;
+  const uint8_t *xf = xs + c32 * 128;
+
+  const int count = (a.k_tiles - wave + WAVES - 1) / WAVES;  // this wave's tiles: wave, wave + 8, ...
+  auto tile_of = [&](int i) {  // past the end: the wave's last tile again (a harmless re-load, never multiplied)
+    const int ii = i < count ? i : count - 1;
+    return wave + ii * WAVES;
+  };
+  u32x4 w[3][2];         // weight ring: [tile % 3][slot kq = h, h + 2]
+  uint32_t szw[3][GPT];  // the tile's scale|zp words
+  auto issue_x = [&](int i, int p) {  // piece p (K elements 64 p .. 64 p + 63) of the wave's i-th tile
+    const int64_t koff = (int64_t)tile_of(i) * 256 + p * 128;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      __builtin_amdgcn_global_load_lds((r32_gptr_t)(xg[q] + koff), (r32_lptr_t)(xs + p * 4096 + q * 1024), 16, 0, 0);
+  };
+  auto issue_w = [&](int i, int rs) {
+    const int kt = tile_of(i);
+    const uint8_t *p = wp + (int64_t)kt * 1024;
+    w[rs][0] = r32_load16(p);
+    w[rs][1] = r32_load16(p + 512);
+#pragma unroll
+    for (int u = 0; u < GPT; ++u)
+      szw[rs][u] = r32_load4(szp + (GPT == 1 ? (kt >> a.group_shift) : kt * GPT + u) * 16);
+  };
+
+  r32_f32x16 acc, P, S;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    acc[r] = P[r] = S[r] = 0.f;
+  const u32x4 ones_bits = {H::ONE2, H::ONE2, H::ONE2, H::ONE2};
+  const vec8 ones = __builtin_bit_cast(vec8, ones_bits);
+  uint32_t nib_magic = H::NIB_MAGIC2;
+  asm volatile("" : "+v"(nib_magic));  // keep it in a VGPR (see and_or)
+
+  if (count > 0) {
+    // Request order, kept by the loop: w(0) w(1) x(0,0) | x(0,1) w(2) | x(1,0) | x(1,1) w(3) | x(2,0) | ...  A piece
+    // is multiplied when all but the 4 + WL youngest requests have landed: the next piece and one tile of weights.
+    issue_w(0, 0);
+    issue_w(1, 1);
+    issue_x(0, 0);
+    for (int t0 = 0; t0 < count; t0 += 3) {  // three tiles per trip: the weight ring indexed statically
+#pragma unroll
+      for (int u = 0; u < 3; ++u) {
+        const int t = t0 + u;
+        if (t >= count)
+          break;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          if (p == 0) {
+            issue_x(t, 1);
+            issue_w(t + 2, (u + 2) % 3);
+          } else {
+            issue_x(t + 1, 0);
+          }
+          __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(4 + WL));
+          asm volatile("" ::: "memory");  // the piece is in LDS from here on, not before
+          if (p == 0) {
+            r32_arrived(w[u][0]);
+            r32_arrived(w[u][1]);
+#pragma unroll
+            for (int g = 0; g < GPT; ++g)
+              r32_arrived(szw[u][g]);
+          }
+          u32x4 fa[4];
+#pragma unroll
+          for (int s = 0; s < 4; ++s)
+            fa[s] = *(const u32x4 *)(xf + p * 4096 + (((2 * s + h) ^ (c32 & 7)) << 4));
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            // k-step 4 p + s of the tile: word 2 p + s / 2 of slot (h for even, h + 2 for odd k-steps)
+            const vec8 b = unpack_nibbles<DT>(w[u][s & 1][2 * p + (s >> 1)], nib_magic);
+            P = r32_mfma<DT>(__builtin_bit_cast(vec8, fa[s]), b, P);
+            S = r32_mfma<DT>(__builtin_bit_cast(vec8, fa[s]), ones, S);
+          }
+          if (GPT == 2 || p == 1) {  // end of a quantization group (or of the tile: the same words again next tile)
+            const uint32_t szv = szw[u][GPT == 2 ? p : 0];
+            const float sc = H::to_f32((uint16_t)(szv >> 16));
+            const float c = H::OFFSET + (float)(szv & 0xffu);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              acc[r] = fmaf(sc, fmaf(-c, S[r], P[r]), acc[r]);
+              P[r] = S[r] = 0.f;
+            }
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(0));  // the re-loads issued past the end
+  }
+
+  // ---- cross-wave sum, in wave order (see a16_rows32_kernel)
+  __syncthreads();  // the partial blocks overlay the activation rings: every wave is done with its pieces
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    red[wave][r][lane] = acc[r];
+  __syncthreads();
+  const float *biasp = R32_SEL(bias);
+  float *y32 = R32_SEL(y32);
+  uint16_t *y = R32_SEL(y);
+  const float bias_v = (biasp && n < set_n) ? biasp[n] : 0.f;
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int r = wave * 2 + q;
+    float v = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv)
+      v += red[wv][r][lane];
+    const int orow = 8 * (r >> 2) + 4 * h + (r & 3);
+    if (orow < a.M && n < set_n) {
+      v += bias_v;
+      const int64_t o = (int64_t)orow * set_n + n;
+      if (y32)
+        y32[o] = v;
+      y[o] = a.chip == MI_CHIP_CV18XX ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+    }
+  }
+#undef R32_SEL
+}
+
+// Weight sets in the tiled layout whose K is a whole number of tiles: 8-bit with one scale per channel; 4-bit with
+// groups of 64, of 128 * 2^k, or one per channel.  `blocks`: 32-channel blocks of the whole launch (all sibling sets).
+// Taken for 17 to 32 rows -- unless K is long and the blocks cover only part of the chip, where every workgroup's read
+// of all the activations outweighs the rest -- and below that from where it was measured ahead.  bf16, the kernels
+// otherwise taken (decode / skinny up to 16 rows, tiled + split-K above) / this one, in us:
+//   8-bit  11008 x 4096   M = 6: 14.7 / 14.5   M = 8: 16.2 / 14.4   M = 12: 17.6 / 14.5   M = 16: 22.4 / 15.1   M = 17: 29.0 / 15.2   M = 32: 29.3 / 17.2
+//   8-bit  4096 x 4096    M = 8:  6.5 /  7.9   M = 16:  7.6 /  8.4   M = 17: 14.7 /  8.4   M = 24: 14.9 /  9.2   M = 32: 15.1 /  9.8
+//   4-bit  11008 x 4096   M = 8: 10.1 / 13.3   M = 12: 13.0 / 13.2   M = 16: 14.6 / 13.6   M = 17: 17.2 / 13.3   M = 32: 17.8 / 14.3
+//   4-bit  4096 x 4096    M = 12: 6.4 /  7.5   M = 16:  7.0 /  7.6   M = 17: 11.9 /  7.6   M = 32: 12.5 /  8.2
+//   4-bit  4096 x 11008   M = 16: 14.4 / 14.7  M = 17: 16.4 / 14.7   M = 24: 16.9 / 16.3   M = 32: 16.9 / 18.2
+//   4-bit  6144 x 2048, groups of 64   M = 12: 6.3 / 6.0   M = 16: 6.9 / 6.0   M = 17: 10.6 / 6.0   M = 32: 11.6 / 6.3
+bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
+  if (!w || !w->qweight || w->kn || w->plain)
+    return false;
+  if (w->bits == 8) {
+    if (w->g != 0 || (w->K % W8_TILE_K) != 0)
+      return false;
+  } else {
+    if ((w->K % W4_TILE_K) != 0)
+      return false;
+    if (w->g != 0 && w->g != 64) {
+      if (w->g % W4_TILE_K != 0)
+        return false;
+      const int tpg = w->g / W4_TILE_K;
+      if ((tpg & (tpg - 1)) != 0 && tpg < w->k_tiles)
+        return false;
+    }
+  }
+  if (plan().a16_rows32_min_m != 0)
+    return plan().a16_rows32_min_m > 0 && M >= plan().a16_rows32_min_m && M <= 32;
+  if (M > 32)
+    return false;
+  if (M >= 17)
+    return !(w->K > 8192 && blocks < 256 && M > 24);
+  return w->bits == 8 ? (M >= 8 && blocks >= 256) : (M >= 13 && blocks >= 192);
+}
+
+// ws[0..n): sibling weight sets on one input -- same K, width, group size, type and chip (checked by the caller), each
+// acceptable to a16_rows32_applicable
+int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
+                            float *const *d_y32s, hipStream_t stream) {
   MI_REQUIRE(M >= 1 && M <= 32, MI_BAD_ARGUMENT, "mi_a16mm_launch: M out of range for this kernel");
-  MI_REQUIRE(d_x && d_y, MI_BAD_ARGUMENT, "mi_a16mm_launch: null activation or output pointer");
-  Rows32Args a;
-  a.x = (const uint8_t *)d_x;
-  a.qw = (const uint8_t *)w->qweight;
-  a.sc8 = (const uint16_t *)w->scale_t;
-  a.nz8 = (const float *)w->nzs_t;
-  a.bias = w->bias;
-  a.y = d_y;
-  a.y32 = d_y32;
-  a.N = w->N;
-  a.K = w->K;
-  a.M = (int)M;
-  a.k_tiles = (int)w->k_tiles;
-  a.row_blocks = (int)w->row_blocks;
-  a.chip = w->chip;
-  const int64_t blocks = (w->N + 31) / 32;
-  MI_REQUIRE(blocks < (1ll << 31), MI_BAD_ARGUMENT, "mi_a16mm_launch: too many output channels");
-  const dim3 grid((unsigned)blocks), block(512);
-  if (w->dtype == MI_DT_F16)
-    a16_rows32_kernel<MI_DT_F16><<<grid, block, 0, stream>>>(a);
-  else
-    a16_rows32_kernel<MI_DT_BF16><<<grid, block, 0, stream>>>(a);
+  MI_REQUIRE(d_x, MI_BAD_ARGUMENT, "mi_a16mm_launch: null activation pointer");
+  const mi_a16_weight *w = ws[0];
+  const bool f16 = w->dtype == MI_DT_F16;
+  const dim3 block(512);
+  if (w->bits == 8) {  // one set per launch
+    for (int i = 0; i < n; ++i) {
+      const mi_a16_weight *v = ws[i];
+      MI_REQUIRE(d_ys[i], MI_BAD_ARGUMENT, "mi_a16mm_launch: null output pointer");
+      const int64_t blocks = (v->N + 31) / 32;
+      MI_REQUIRE(blocks < (1ll << 31), MI_BAD_ARGUMENT, "mi_a16mm_launch: too many output channels");
+      Rows32Args a;
+      a.x = (const uint8_t *)d_x;
+      a.qw = (const uint8_t *)v->qweight;
+      a.sc8 = (const uint16_t *)v->scale_t;
+      a.nz8 = (const float *)v->nzs_t;
+      a.bias = v->bias;
+      a.y = d_ys[i];
+      a.y32 = d_y32s ? d_y32s[i] : nullptr;
+      a.N = v->N;
+      a.K = v->K;
+      a.M = (int)M;
+      a.k_tiles = (int)v->k_tiles;
+      a.row_blocks = (int)v->row_blocks;
+      a.chip = v->chip;
+      if (f16)
+        a16_rows32_kernel<MI_DT_F16><<<dim3((unsigned)blocks), block, 0, stream>>>(a);
+      else
+        a16_rows32_kernel<MI_DT_BF16><<<dim3((unsigned)blocks), block, 0, stream>>>(a);
+    }
+    MI_HIP(hipGetLastError());
+    return MI_SUCCESS;
+  }
+  for (int i0 = 0; i0 < n; i0 += R32_MAX_SETS) {  // 4-bit: up to four sets per launch
+    const int cnt = (n - i0) < R32_MAX_SETS ? (n - i0) : R32_MAX_SETS;
+    Rows32W4Args a;
+    a.x = (const uint8_t *)d_x;
+    a.K = w->K;
+    a.M = (int)M;
+    a.k_tiles = (int)w->k_tiles;
+    a.G = w->G;
+    a.chip = w->chip;
+    a.group_shift = 0;
+    const int tpg = w->g == 0 ? (int)w->k_tiles : w->g / W4_TILE_K;  // tiles per group (0: groups of 64)
+    if (tpg >= w->k_tiles)
+      a.group_shift = 31;
+    else
+      while ((1 << a.group_shift) < tpg)
+        ++a.group_shift;
+    int64_t blocks = 0;
+    for (int j = 0; j < R32_MAX_SETS; ++j) {
+      const mi_a16_weight *v = ws[i0 + (j < cnt ? j : 0)];
+      a.block_begin[j] = j < cnt ? (int)blocks : INT_MAX;
+      a.qw[j] = (const uint8_t *)v->qweight;
+      a.sz[j] = (const uint32_t *)v->sz_t;
+      a.bias[j] = v->bias;
+      a.y[j] = d_ys[i0 + (j < cnt ? j : 0)];
+      a.y32[j] = d_y32s ? d_y32s[i0 + (j < cnt ? j : 0)] : nullptr;
+      a.N[j] = v->N;
+      a.row_blocks[j] = (int)v->row_blocks;
+      if (j < cnt) {
+        MI_REQUIRE(a.y[j], MI_BAD_ARGUMENT, "mi_a16mm_launch: null output pointer");
+        blocks += (v->N + 31) / 32;
+        MI_REQUIRE(blocks < (1ll << 30), MI_BAD_ARGUMENT, "mi_a16mm_launch: too many output channels");
+      }
+    }
+    const dim3 grid((unsigned)blocks);
+    if (w->g == 64) {
+      if (f16)
+        a16_rows32_w4_kernel<MI_DT_F16, 2><<<grid, block, 0, stream>>>(a);
+      else
+        a16_rows32_w4_kernel<MI_DT_BF16, 2><<<grid, block, 0, stream>>>(a);
+    } else {
+      if (f16)
+        a16_rows32_w4_kernel<MI_DT_F16, 1><<<grid, block, 0, stream>>>(a);
+      else
+        a16_rows32_w4_kernel<MI_DT_BF16, 1><<<grid, block, 0, stream>>>(a);
+    }
+  }
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;
 }

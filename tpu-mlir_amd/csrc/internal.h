@@ -120,10 +120,10 @@ int a16_kn_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16
 // wide-tile product (a16_wide.hip), weights rounded to the 16-bit type before the multiply: the reference's arithmetic
 // for 8-bit per-channel sets (taken from a few hundred rows on), the opt-in tolerance form for 4-bit f16 sets; and the
 // exact two-term form for 4-bit sets (each weight as the sum of two 16-bit numbers, two MFMAs per fragment)
-// 8-bit per-channel sets, 9 to 32 rows (a16_rows32.hip)
-bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M);
-int a16_rows32_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
-                      hipStream_t stream);
+// up to 32 rows, one workgroup per 32 channels over the whole K (a16_rows32.hip)
+bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks);
+int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
+                            float *const *d_y32s, hipStream_t stream);
 bool a16_wide8_applicable(const mi_a16_weight *w, int64_t M);
 bool a16_wide4_applicable(const mi_a16_weight *w, int64_t M);
 int a16_wide_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
