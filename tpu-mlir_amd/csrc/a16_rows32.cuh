@@ -1,0 +1,68 @@
+// For the kernels for a few tens of activation rows (a16_rows32.hip): argument records, the 32 x 32 x 16 MFMA,
+// loads the compiler does not track (their arrival is covered by the kernels' own request counts), wait encodings.
+#pragma once
+#include "a16_common.cuh"
+#include "internal.h"
+
+namespace mi {
+
+typedef __attribute__((ext_vector_type(16))) float r32_f32x16;
+typedef const __attribute__((address_space(1))) void *r32_gptr_t;
+typedef __attribute__((address_space(3))) void *r32_lptr_t;
+
+__device__ __forceinline__ u32x4 r32_load16(const void *p) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+template <typename T>
+__device__ __forceinline__ void r32_arrived(T &v) {
+  asm volatile("" : "+v"(v));
+}
+constexpr int r32_waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
+
+template <int DT>
+__device__ __forceinline__ r32_f32x16 r32_mfma(typename Half16<DT>::vec8 a, typename Half16<DT>::vec8 b, r32_f32x16 c) {
+  if constexpr (DT == MI_DT_F16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ uint32_t r32_load4(const void *p) {
+  uint32_t v;
+  asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+
+// 8-bit weights, one scale per channel: one weight set per launch
+struct Rows32Args {
+  const uint8_t *x;      // [M][K] 16-bit
+  const uint8_t *qw;     // packed tiles [row_blocks][k_tiles][1024]
+  const uint16_t *sc8;   // scale bits [row_blocks][16]
+  const float *nz8;      // -zp' * scale [row_blocks][16]
+  const float *bias;     // [N] or null
+  uint16_t *y;           // [M][N]
+  float *y32;            // [M][N] or null
+  int64_t N, K;
+  int M, k_tiles, row_blocks, chip;
+};
+
+constexpr int R32_MAX_SETS = 4;
+// Sibling weight sets on one input (q/k/v, gate/up: same K, group size and type) share a launch: their 32-channel
+// blocks are numbered one set after the other, and a workgroup tells its set by three scalar compares.
+struct Rows32W4Args {
+  const uint8_t *x;                     // [M][K] 16-bit
+  int64_t K;
+  int M, k_tiles, G, group_shift, chip;
+  int block_begin[R32_MAX_SETS];        // first workgroup of each set (unused slots: INT_MAX)
+  const uint8_t *qw[R32_MAX_SETS];      // packed tiles [row_blocks][k_tiles][1024]
+  const uint32_t *sz[R32_MAX_SETS];     // scale|zp words [row_blocks][G][16]
+  const float *bias[R32_MAX_SETS];      // [N] or null
+  uint16_t *y[R32_MAX_SETS];            // [M][N]
+  float *y32[R32_MAX_SETS];             // [M][N] or null
+  int64_t N[R32_MAX_SETS];
+  int row_blocks[R32_MAX_SETS];
+};
+
+}  // namespace mi

@@ -18,45 +18,9 @@
 //     acc += scale * (P - (16 + zp) * S) in fp32.
 #include <climits>
 
-#include "a16_common.cuh"
-#include "internal.h"
+#include "a16_rows32.cuh"
 
 namespace mi {
-
-typedef __attribute__((ext_vector_type(16))) float r32_f32x16;
-typedef const __attribute__((address_space(1))) void *r32_gptr_t;
-typedef __attribute__((address_space(3))) void *r32_lptr_t;
-
-struct Rows32Args {
-  const uint8_t *x;      // [M][K] 16-bit
-  const uint8_t *qw;     // packed tiles [row_blocks][k_tiles][1024]
-  const uint16_t *sc8;   // scale bits [row_blocks][16]
-  const float *nz8;      // -zp' * scale [row_blocks][16]
-  const float *bias;     // [N] or null
-  uint16_t *y;           // [M][N]
-  float *y32;            // [M][N] or null
-  int64_t N, K;
-  int M, k_tiles, row_blocks, chip;
-};
-
-__device__ __forceinline__ u32x4 r32_load16(const void *p) {
-  u32x4 v;
-  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-  return v;
-}
-template <typename T>
-__device__ __forceinline__ void r32_arrived(T &v) {
-  asm volatile("" : "+v"(v));
-}
-constexpr int r32_waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
-
-template <int DT>
-__device__ __forceinline__ r32_f32x16 r32_mfma(typename Half16<DT>::vec8 a, typename Half16<DT>::vec8 b, r32_f32x16 c) {
-  if constexpr (DT == MI_DT_F16)
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
 
 template <int DT>
 __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
@@ -147,6 +111,13 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
       }
     }
     __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(0));  // the re-loads issued past the end
+    // Their destination registers stay taken until here: named as read after the wait, or the compiler, which does not
+    // know of requests on their way, hands those registers to whatever follows and the late data lands on top of it.
+#pragma unroll
+    for (int rs = 0; rs < 3; ++rs) {
+      r32_arrived(w[rs][0]);
+      r32_arrived(w[rs][1]);
+    }
   }
 
   // ---- cross-wave sum, in wave order.  Register r of lane l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
@@ -176,29 +147,6 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
 
 // 4-bit weights; groups of whole 128-K tiles (group of tile kt = kt >> group_shift; 31: one group per channel) or,
 // GPT = 2, of 64.  A step of the loop is half a weight tile: 64 K elements, four MFMA k-steps, one activation piece.
-constexpr int R32_MAX_SETS = 4;
-// Sibling weight sets on one input (q/k/v, gate/up: same K, group size and type) share a launch: their 32-channel
-// blocks are numbered one set after the other, and a workgroup tells its set by three scalar compares.
-struct Rows32W4Args {
-  const uint8_t *x;                     // [M][K] 16-bit
-  int64_t K;
-  int M, k_tiles, G, group_shift, chip;
-  int block_begin[R32_MAX_SETS];        // first workgroup of each set (unused slots: INT_MAX)
-  const uint8_t *qw[R32_MAX_SETS];      // packed tiles [row_blocks][k_tiles][1024]
-  const uint32_t *sz[R32_MAX_SETS];     // scale|zp words [row_blocks][G][16]
-  const float *bias[R32_MAX_SETS];      // [N] or null
-  uint16_t *y[R32_MAX_SETS];            // [M][N]
-  float *y32[R32_MAX_SETS];             // [M][N] or null
-  int64_t N[R32_MAX_SETS];
-  int row_blocks[R32_MAX_SETS];
-};
-
-__device__ __forceinline__ uint32_t r32_load4(const void *p) {
-  uint32_t v;
-  asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-  return v;
-}
-
 template <int DT, int GPT>
 __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
   using H = Half16<DT>;
@@ -319,6 +267,15 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
       }
     }
     __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(0));  // the re-loads issued past the end
+    // (their destination registers stay taken until here, see a16_rows32_kernel)
+#pragma unroll
+    for (int rs = 0; rs < 3; ++rs) {
+      r32_arrived(w[rs][0]);
+      r32_arrived(w[rs][1]);
+#pragma unroll
+      for (int g = 0; g < GPT; ++g)
+        r32_arrived(szw[rs][g]);
+    }
   }
 
   // ---- cross-wave sum, in wave order (see a16_rows32_kernel)

@@ -367,6 +367,11 @@ __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m
     }
   }
   __builtin_amdgcn_s_waitcnt(tol_waitcnt_vm(0));  // drain the re-loads issued past the end before the workgroup may exit
+  // The weight ring's registers stay taken until here: named as read after the wait, or the compiler, which does not
+  // know of requests on their way, hands those registers to the epilogue and the late data lands on top of it.
+#pragma unroll
+  for (int rs = 0; rs < WRING; ++rs)
+    w_arrived(rs);
 
   // ---- epilogue.  Register r of lane l in block (i, j) is row 8*(r/4) + 4*(l/32) + (r%4), column l%32.  Each wave
   // passes one 32 x 64 strip at a time through its own LDS region and re-reads it so that a lane owns 8 consecutive
