@@ -1,7 +1,7 @@
 """GPU parity of the 32-row kernel (csrc/a16_rows32.hip) on 4-bit weight sets: the exact kernels' arithmetic, held to
 their bounds -- fp32 result within 2e-5 * RMS(output) of the oracle's float64 accumulation, outputs the reference
 rounding of the kernel's own fp32 values.  The plan sends every row count the kernel can handle through it (by itself
-the library takes it for 17 to 32 rows, and from 13 on large sets); single sets and sibling sets sharing a launch."""
+the library takes it for 17 to 32 rows, and from fewer on large sets); single sets and sibling sets sharing a launch."""
 import numpy as np
 import pytest
 

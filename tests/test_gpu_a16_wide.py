@@ -186,7 +186,7 @@ ROWS32_CASES = [  # (M, K, N, signed, dtype): 8-bit, one scale per channel, up t
 
 @pytest.mark.parametrize("M,K,N,signed,dt", ROWS32_CASES)
 def test_w8_per_channel_up_to_32_rows_against_oracle(orc, plan, M, K, N, signed, dt):
-    """The 32-row kernel (csrc/a16_rows32.hip; taken by itself for 17 to 32 rows and from 8 on large sets, here for every row count it can
+    """The 32-row kernel (csrc/a16_rows32.hip; taken by itself for 17 to 32 rows and from fewer on large sets, here for every row count it can
     handle): fp32 result within 2e-5 * RMS of the oracle, outputs the reference rounding of the kernel's fp32 values."""
     import torch
     plan(a16_rows32_min_m=1)

@@ -22,7 +22,9 @@
 
 namespace mi {
 
-template <int DT>
+// NQ: 8-row requests per activation piece, ceil(M / 8): rows from 8 NQ on are never requested (their LDS rows hold
+// whatever was there, and so do their outputs, which are never stored)
+template <int DT, int NQ>
 __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
@@ -46,9 +48,9 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
   asm volatile("" : "+v"(sc), "+v"(nz));
   // activations, direct to LDS: request i of a tile covers rows 8 i .. 8 i + 7 whole (lane l: row 8 i + l / 8,
   // position l % 8, which holds the row's chunk (position ^ row % 8)): eight full cache lines per request
-  const uint8_t *xg[4];
+  const uint8_t *xg[NQ];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < NQ; ++i) {
     const int r = 8 * i + (lane >> 3);
     const int rr = r < a.M ? r : a.M - 1;  // rows past M repeat the last row; never stored
     xg[i] = a.x + (int64_t)rr * a.K * 2 + (((lane & 7) ^ (r & 7)) << 4);
@@ -66,7 +68,7 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
   auto issue_x = [&](int i, int rs) {
     const int64_t koff = (int64_t)tile_of(i) * 128;
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
+    for (int q = 0; q < NQ; ++q)
       __builtin_amdgcn_global_load_lds((r32_gptr_t)(xg[q] + koff), (r32_lptr_t)(xs + rs * 4096 + q * 1024), 16, 0, 0);
   };
   auto issue_w = [&](int i, int rs) {
@@ -94,7 +96,7 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
           break;
         issue_x(t + 1, (u + 1) % 2);
         issue_w(t + 2, (u + 2) % 3);
-        __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(8));
+        __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(NQ + 4));
         r32_arrived(w[u % 3][0]);
         r32_arrived(w[u % 3][1]);
         asm volatile("" ::: "memory");  // the tile's activations are in LDS from here on, not before
@@ -147,7 +149,7 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
 
 // 4-bit weights; groups of whole 128-K tiles (group of tile kt = kt >> group_shift; 31: one group per channel) or,
 // GPT = 2, of 64.  A step of the loop is half a weight tile: 64 K elements, four MFMA k-steps, one activation piece.
-template <int DT, int GPT>
+template <int DT, int GPT, int NQ>
 __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
@@ -171,9 +173,9 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
   rb = rb < set_rbs ? rb : set_rbs - 1;  // channels past N repeat the last row block; never stored
   const uint8_t *wp = R32_SEL(qw) + rb * a.k_tiles * 1024 + (uint32_t)((h * 16 + (c32 & 15)) * 16);
   const uint32_t *szp = R32_SEL(sz) + rb * a.G * 16 + (c32 & 15);
-  const uint8_t *xg[4];
+  const uint8_t *xg[NQ];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < NQ; ++i) {
     const int r = 8 * i + (lane >> 3);
     const int rr = r < a.M ? r : a.M - 1;
     xg[i] = a.x + (int64_t)rr * a.K * 2 + (((lane & 7) ^ (r & 7)) << 4);
@@ -191,7 +193,7 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
   auto issue_x = [&](int i, int p) {  // piece p (K elements 64 p .. 64 p + 63) of the wave's i-th tile
     const int64_t koff = (int64_t)tile_of(i) * 256 + p * 128;
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
+    for (int q = 0; q < NQ; ++q)
       __builtin_amdgcn_global_load_lds((r32_gptr_t)(xg[q] + koff), (r32_lptr_t)(xs + p * 4096 + q * 1024), 16, 0, 0);
   };
   auto issue_w = [&](int i, int rs) {
@@ -233,7 +235,7 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
           } else {
             issue_x(t + 1, 0);
           }
-          __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(4 + WL));
+          __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(NQ + WL));
           asm volatile("" ::: "memory");  // the piece is in LDS from here on, not before
           if (p == 0) {
             r32_arrived(w[u][0]);
@@ -312,12 +314,12 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
 // Taken for 17 to 32 rows -- unless K is long and the blocks cover only part of the chip, where every workgroup's read
 // of all the activations outweighs the rest -- and below that from where it was measured ahead.  bf16, the kernels
 // otherwise taken (decode / skinny up to 16 rows, tiled + split-K above) / this one, in us:
-//   8-bit  11008 x 4096   M = 6: 14.7 / 14.5   M = 8: 16.2 / 14.4   M = 12: 17.6 / 14.5   M = 16: 22.4 / 15.1   M = 17: 29.0 / 15.2   M = 32: 29.3 / 17.2
-//   8-bit  4096 x 4096    M = 8:  6.5 /  7.9   M = 16:  7.6 /  8.4   M = 17: 14.7 /  8.4   M = 24: 14.9 /  9.2   M = 32: 15.1 /  9.8
-//   4-bit  11008 x 4096   M = 8: 10.1 / 13.3   M = 12: 13.0 / 13.2   M = 16: 14.6 / 13.6   M = 17: 17.2 / 13.3   M = 32: 17.8 / 14.3
-//   4-bit  4096 x 4096    M = 12: 6.4 /  7.5   M = 16:  7.0 /  7.6   M = 17: 11.9 /  7.6   M = 32: 12.5 /  8.2
-//   4-bit  4096 x 11008   M = 16: 14.4 / 14.7  M = 17: 16.4 / 14.7   M = 24: 16.9 / 16.3   M = 32: 16.9 / 18.2
-//   4-bit  6144 x 2048, groups of 64   M = 12: 6.3 / 6.0   M = 16: 6.9 / 6.0   M = 17: 10.6 / 6.0   M = 32: 11.6 / 6.3
+//   8-bit  11008 x 4096   M = 4: 10.9 / 13.2   M = 8: 15.8 / 13.4   M = 12: 17.2 / 13.9   M = 16: 22.2 / 14.4   M = 17: 28.5 / 14.9   M = 32: 29.3 / 17.5
+//   8-bit  4096 x 4096    M = 8:  6.6 /  7.1   M = 16:  7.7 /  8.0   M = 17: 14.6 /  8.1   M = 24: 14.9 /  8.9   M = 32: 15.4 /  9.7
+//   4-bit  11008 x 4096   M = 8:  9.9 / 11.8   M = 9: 11.3 / 12.4   M = 12: 13.1 / 12.3   M = 16: 14.6 / 12.7   M = 17: 17.1 / 13.1   M = 32: 17.8 / 15.3
+//   4-bit  4096 x 4096    M = 12: 6.3 /  7.4   M = 16:  7.0 /  7.5   M = 17: 11.8 /  7.6   M = 32: 12.5 /  8.4
+//   4-bit  4096 x 11008   M = 4: 11.8 / 13.3   M = 8: 14.2 / 13.2   M = 16: 14.5 / 13.9   M = 17: 16.3 / 14.5   M = 24: 16.6 / 16.3   M = 32: 16.9 / 18.5
+//   4-bit  6144 x 2048, groups of 64   M = 9: 5.6 / 6.0   M = 12: 6.2 / 6.1   M = 16: 6.9 / 6.2   M = 17: 10.6 / 6.2   M = 32: 11.6 / 6.6
 bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
   if (!w || !w->qweight || w->kn || w->plain)
     return false;
@@ -341,7 +343,9 @@ bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
     return false;
   if (M >= 17)
     return !(w->K > 8192 && blocks < 256 && M > 24);
-  return w->bits == 8 ? (M >= 8 && blocks >= 256) : (M >= 13 && blocks >= 192);
+  if (w->bits == 8)
+    return M >= 8 && blocks >= 256;
+  return (M >= 12 && (blocks >= 192 || w->K > 8192)) || (M >= 8 && w->K > 8192);
 }
 
 // ws[0..n): sibling weight sets on one input -- same K, width, group size, type and chip (checked by the caller), each
@@ -353,6 +357,7 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
   const mi_a16_weight *w = ws[0];
   const bool f16 = w->dtype == MI_DT_F16;
   const dim3 block(512);
+  const int nq = (int)((M + 7) / 8);  // 8-row requests per activation piece
   if (w->bits == 8) {  // one set per launch
     for (int i = 0; i < n; ++i) {
       const mi_a16_weight *v = ws[i];
@@ -373,10 +378,23 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
       a.k_tiles = (int)v->k_tiles;
       a.row_blocks = (int)v->row_blocks;
       a.chip = v->chip;
-      if (f16)
-        a16_rows32_kernel<MI_DT_F16><<<dim3((unsigned)blocks), block, 0, stream>>>(a);
+      const dim3 grid8((unsigned)blocks);
+#define MI_R32_8(NQ_)                                                     \
+  {                                                                       \
+    if (f16)                                                              \
+      a16_rows32_kernel<MI_DT_F16, NQ_><<<grid8, block, 0, stream>>>(a);  \
+    else                                                                  \
+      a16_rows32_kernel<MI_DT_BF16, NQ_><<<grid8, block, 0, stream>>>(a); \
+  }
+      if (nq == 1)
+        MI_R32_8(1)
+      else if (nq == 2)
+        MI_R32_8(2)
+      else if (nq == 3)
+        MI_R32_8(3)
       else
-        a16_rows32_kernel<MI_DT_BF16><<<dim3((unsigned)blocks), block, 0, stream>>>(a);
+        MI_R32_8(4)
+#undef MI_R32_8
     }
     MI_HIP(hipGetLastError());
     return MI_SUCCESS;
@@ -415,17 +433,30 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
       }
     }
     const dim3 grid((unsigned)blocks);
-    if (w->g == 64) {
-      if (f16)
-        a16_rows32_w4_kernel<MI_DT_F16, 2><<<grid, block, 0, stream>>>(a);
-      else
-        a16_rows32_w4_kernel<MI_DT_BF16, 2><<<grid, block, 0, stream>>>(a);
-    } else {
-      if (f16)
-        a16_rows32_w4_kernel<MI_DT_F16, 1><<<grid, block, 0, stream>>>(a);
-      else
-        a16_rows32_w4_kernel<MI_DT_BF16, 1><<<grid, block, 0, stream>>>(a);
-    }
+#define MI_R32_4(GPT_, NQ_)                                                      \
+  {                                                                              \
+    if (f16)                                                                     \
+      a16_rows32_w4_kernel<MI_DT_F16, GPT_, NQ_><<<grid, block, 0, stream>>>(a);  \
+    else                                                                         \
+      a16_rows32_w4_kernel<MI_DT_BF16, GPT_, NQ_><<<grid, block, 0, stream>>>(a); \
+  }
+#define MI_R32_4Q(GPT_) \
+  {                     \
+    if (nq == 1)        \
+      MI_R32_4(GPT_, 1) \
+    else if (nq == 2)   \
+      MI_R32_4(GPT_, 2) \
+    else if (nq == 3)   \
+      MI_R32_4(GPT_, 3) \
+    else                \
+      MI_R32_4(GPT_, 4) \
+  }
+    if (w->g == 64)
+      MI_R32_4Q(2)
+    else
+      MI_R32_4Q(1)
+#undef MI_R32_4Q
+#undef MI_R32_4
   }
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;
