@@ -197,12 +197,12 @@ def test_cast_of_special_values(orc):
 
 
 @pytest.mark.parametrize("chip", [clib.CHIP_BM168X, clib.CHIP_CV18XX])
-@pytest.mark.parametrize("M,K", [(1, 256), (5, 256), (40, 256), (48, 4096)])
+@pytest.mark.parametrize("M,K", [(1, 256), (5, 256), (20, 256), (40, 256), (48, 4096)])
 def test_a16_epilogue_rounding_of_special_values(orc, plan, chip, M, K):
     """The 16-bit output rounding inside the A16MatMul kernels: zero activations make every output equal its bias, and
     the bias carries the special values -- through the skinny kernel (M = 1 with the activations staged in LDS, M = 5
-    without), the tiled kernel (M = 40) and the split-K finishing pass (M = 48 at K = 4096), in the BM168x and CV18xx
-    flavours of the bf16 rounding, and in f16 mode."""
+    without), the 32-row kernel (M = 20), the tiled kernel (M = 40) and the split-K finishing pass (M = 48 at
+    K = 4096), in the BM168x and CV18xx flavours of the bf16 rounding, and in f16 mode."""
     import torch
     plan(a16_gemm_min_m=17)
     N = 32
@@ -241,3 +241,30 @@ def test_a16_epilogue_rounding_of_special_values(orc, plan, chip, M, K):
         got16 = y16.view(torch.int16).cpu().numpy().view(np.uint16)
         assert np.array_equal(got16, orc.f32_to_f16(sum32))
         w16.destroy()
+
+
+@pytest.mark.parametrize("chip", [clib.CHIP_BM168X, clib.CHIP_CV18XX])
+@pytest.mark.parametrize("path,bits,M,K,g", [("rows32", 8, 20, 256, 0), ("wide", 8, 300, 256, 0), ("plain", 4, 3, 96, 24),
+                                            ("plain", 8, 2, 80, 40), ("two_term", 4, 260, 256, 128)])
+def test_a16_epilogue_rounding_in_the_other_kernels(orc, plan, chip, path, bits, M, K, g):
+    """The same check (zero activations, special values in the bias) through the kernels with epilogues of their own:
+    the 8-bit 32-row kernel, the wide tiles (8-bit, and the 4-bit two-term form) and the plain kernel for odd group
+    sizes; BM168x and CV18xx flavours of the bf16 rounding."""
+    import torch
+    plan(a16_wide_min_m=1 if path == "wide" else 0, a16_wide4_min_m=1 if path == "two_term" else 0)
+    N = 32
+    cfg = S.w4a16(M, K, N, g, seed=45) if bits == 4 else S.w8a16(M, K, N, g, seed=45, signed=(g == 0))
+    bias = np.resize(SPECIAL_BITS, N).view(np.float32).copy()
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], bias, K=K, N=N, weight_bits=bits, q_group_size=g, chip=chip)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_launch(w, torch.zeros((M, K), dtype=torch.bfloat16, device="cuda"), y_f32=y32)
+    torch.cuda.synchronize()
+    pre = y32.cpu().numpy().view(np.uint32)
+    got = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    w.destroy()
+    nan = np.isnan(bias)
+    with np.errstate(invalid="ignore"):
+        sum32 = np.broadcast_to(np.float32(0.0) + bias, (M, N)).copy()
+    assert np.array_equal(pre[:, ~nan], sum32.view(np.uint32)[:, ~nan])
+    assert np.all(np.isnan(pre.view(np.float32)[:, nan]))
+    assert np.array_equal(got, orc.f32_to_bf16(sum32, cv18xx=(chip == clib.CHIP_CV18XX)))
