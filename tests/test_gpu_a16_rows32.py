@@ -87,3 +87,40 @@ def test_w4_sibling_sets_share_a_launch(orc, plan, M, K, Ns, g, dt):
         assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), to16(pre))
     for w in ws:
         w.destroy()
+
+
+ROWS32_W8_GROUPED = [  # (M, K, N, g, dtype): 8-bit weights with quantization groups of 64 * 2^k along K
+    (20, 512, 64, 64, "bf16"), (32, 1024, 200, 128, "bf16"), (17, 4096, 96, 256, "bf16"), (9, 448, 33, 64, "f16"),
+    (31, 1536, 40, 512, "f16"), (24, 11008, 48, 64, "bf16"), (1, 64, 16, 64, "bf16"),
+]
+
+
+@pytest.mark.parametrize("M,K,N,g,dt", ROWS32_W8_GROUPED)
+def test_w8_grouped_up_to_32_rows_against_oracle(orc, plan, M, K, N, g, dt):
+    """The reference's 8-bit arithmetic with groups (weights rounded to the 16-bit type, A16MatMul.cpp:209-231): the
+    tile's scale and zero-point term travel with the weights."""
+    import torch
+    plan(a16_rows32_min_m=1)
+    dtype = clib.DT_F16 if dt == "f16" else clib.DT_BF16
+    cfg = S.w8a16(M, K, N, g, seed=M + K + N, signed=False, bias=(N % 2 == 0))
+    x, wq, scale, zp, bias = f32_valued_a16(cfg)
+    x16, scale16 = cfg["x"], cfg["scale"]
+    if dtype == clib.DT_F16:
+        x, scale = orc.F16(x), orc.F16(scale)
+        x16, scale16 = orc.f32_to_f16(x), orc.f32_to_f16(scale)
+    tdt = torch.float16 if dtype == clib.DT_F16 else torch.bfloat16
+    w = M_.A16Weight(cfg["weight"], scale16, cfg["zp"], bias, K=K, N=N, weight_bits=8, q_group_size=g, dtype=dtype)
+    xd = torch.from_numpy(x16.view(np.int16)).cuda().view(tdt)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_launch(w, xd, y_f32=y32)
+    torch.cuda.synchronize()
+    out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    pre = y32.cpu().numpy()
+    w.destroy()
+    want, want_pre = orc.a16matmul(x, wq, scale, zp, bias, M=M, K=K, N=N, weight_bits=8, q_group_size=g,
+                                   out_dtype=orc.OUT_F16 if dtype == clib.DT_F16 else orc.OUT_BF16,
+                                   gemm_kind=orc.GEMM_F64ACC)
+    err = cmp.max_abs_over_rms(pre, want_pre)
+    assert err <= 2e-5, "fp32 pre-round max-abs/RMS %.3g" % err
+    to16 = orc.f32_to_f16 if dtype == clib.DT_F16 else orc.f32_to_bf16
+    assert np.array_equal(out, to16(pre))

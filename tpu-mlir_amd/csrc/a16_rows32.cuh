@@ -29,18 +29,24 @@ __device__ __forceinline__ r32_f32x16 r32_mfma(typename Half16<DT>::vec8 a, type
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
+__device__ __forceinline__ uint32_t r32_load2(const void *p) {  // 16 bits, zero-extended
+  uint32_t v;
+  asm volatile("global_load_ushort %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
 __device__ __forceinline__ uint32_t r32_load4(const void *p) {
   uint32_t v;
   asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
   return v;
 }
 
-// 8-bit weights, one scale per channel: one weight set per launch
+// 8-bit weights: one weight set per launch
 struct Rows32Args {
   const uint8_t *x;      // [M][K] 16-bit
   const uint8_t *qw;     // packed tiles [row_blocks][k_tiles][1024]
-  const uint16_t *sc8;   // scale bits [row_blocks][16]
-  const float *nz8;      // -zp' * scale [row_blocks][16]
+  const uint16_t *sc8;   // scale bits [row_blocks][G][16]
+  const float *nz8;      // -zp' * scale [row_blocks][G][16]
+  int G, group_shift;    // groups along K; group of 64-K tile kt = kt >> group_shift (31: one scale per channel)
   const float *bias;     // [N] or null
   uint16_t *y;           // [M][N]
   float *y32;            // [M][N] or null

@@ -24,7 +24,9 @@ namespace mi {
 
 // NQ: 8-row requests per activation piece, ceil(M / 8): rows from 8 NQ on are never requested (their LDS rows hold
 // whatever was there, and so do their outputs, which are never stored)
-template <int DT, int NQ>
+// GRP: quantization groups of 64 * 2^k along K (scale and -zp' * scale travel with each weight tile) instead of one
+// scale per channel
+template <int DT, int NQ, bool GRP>
 __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
@@ -41,11 +43,17 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
   int64_t rb = (int64_t)blockIdx.x * 2 + (c32 >> 4);
   rb = rb < a.row_blocks ? rb : a.row_blocks - 1;  // channels past N repeat the last row block; never stored
   const uint8_t *wp = a.qw + rb * a.k_tiles * 1024 + (uint32_t)((h * 16 + (c32 & 15)) * 16);
-  float sc = H::to_f32(a.sc8[rb * 16 + (c32 & 15)]);
-  float nz = a.nz8[rb * 16 + (c32 & 15)];
-  // The compiler knows these two as loads and would wait for them where they are first used -- inside the loop, as a
-  // wait for everything, since it does not count the requests below.  Used here, they are waited for here.
-  asm volatile("" : "+v"(sc), "+v"(nz));
+  constexpr int WL = GRP ? 4 : 2;  // weight-side requests per tile
+  const uint16_t *scp = a.sc8 + rb * a.G * 16 + (c32 & 15);
+  const float *nzp = a.nz8 + rb * a.G * 16 + (c32 & 15);
+  float sc = 0.f, nz = 0.f;
+  if constexpr (!GRP) {
+    sc = H::to_f32(scp[0]);
+    nz = nzp[0];
+    // The compiler knows these two as loads and would wait for them where they are first used -- inside the loop, as
+    // a wait for everything, since it does not count the requests below.  Used here, they are waited for here.
+    asm volatile("" : "+v"(sc), "+v"(nz));
+  }
   // activations, direct to LDS: request i of a tile covers rows 8 i .. 8 i + 7 whole, eight full cache lines (lane l:
   // row 8 i + l / 8, position l % 8, which holds the row's chunk (position ^ (row / 2) % 8) -- the swizzle under which
   // the fragment reads below are free of bank conflicts by the counters; with row % 8 they showed 40 % conflict cycles)
@@ -66,6 +74,7 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
     return wave + ii * WAVES;
   };
   u32x4 w[3][2];   // weight ring: [tile % 3][slot kq = h, h + 2]
+  uint32_t scw[3], nzw[3];  // GRP: the tile's scale bits and -zp' * scale
   auto issue_x = [&](int i, int rs) {
     const int64_t koff = (int64_t)tile_of(i) * 128;
 #pragma unroll
@@ -73,9 +82,15 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
       __builtin_amdgcn_global_load_lds((r32_gptr_t)(xg[q] + koff), (r32_lptr_t)(xs + rs * 4096 + q * 1024), 16, 0, 0);
   };
   auto issue_w = [&](int i, int rs) {
-    const uint8_t *p = wp + (int64_t)tile_of(i) * 1024;
+    const int kt = tile_of(i);
+    const uint8_t *p = wp + (int64_t)kt * 1024;
     w[rs][0] = r32_load16(p);
     w[rs][1] = r32_load16(p + 512);
+    if constexpr (GRP) {
+      const int gi = kt >> a.group_shift;
+      scw[rs] = r32_load2(scp + gi * 16);
+      nzw[rs] = r32_load4(nzp + gi * 16);
+    }
   };
 
   r32_f32x16 acc;
@@ -85,7 +100,7 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
 
   if (count > 0) {
     // Request order, kept by the loop: ... x(t), w(t+1) | x(t+1), w(t+2) | ...  Tile t is multiplied when all but
-    // the 8 youngest requests have landed: w(t+1) (2) and this iteration's x(t+1), w(t+2) (6) may still be on their way.
+    // the NQ + 2 WL youngest requests have landed: w(t+1) and this iteration's x(t+1), w(t+2) may still be on their way.
     issue_w(0, 0);
     issue_x(0, 0);
     issue_w(1, 1);
@@ -97,9 +112,15 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
           break;
         issue_x(t + 1, (u + 1) % 2);
         issue_w(t + 2, (u + 2) % 3);
-        __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(NQ + 4));
+        __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(NQ + 2 * WL));
         r32_arrived(w[u % 3][0]);
         r32_arrived(w[u % 3][1]);
+        if constexpr (GRP) {
+          r32_arrived(scw[u % 3]);
+          r32_arrived(nzw[u % 3]);
+          sc = H::to_f32((uint16_t)scw[u % 3]);
+          nz = __builtin_bit_cast(float, nzw[u % 3]);
+        }
         asm volatile("" ::: "memory");  // the tile's activations are in LDS from here on, not before
         u32x4 fa[4];
 #pragma unroll
@@ -120,6 +141,10 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
     for (int rs = 0; rs < 3; ++rs) {
       r32_arrived(w[rs][0]);
       r32_arrived(w[rs][1]);
+      if constexpr (GRP) {
+        r32_arrived(scw[rs]);
+        r32_arrived(nzw[rs]);
+      }
     }
   }
 
@@ -310,8 +335,8 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
 #undef R32_SEL
 }
 
-// Weight sets in the tiled layout whose K is a whole number of tiles: 8-bit with one scale per channel; 4-bit with
-// groups of 64, of 128 * 2^k, or one per channel.  `blocks`: 32-channel blocks of the whole launch (all sibling sets).
+// Weight sets in the tiled layout whose K is a whole number of tiles: 8-bit with one scale per channel or groups of
+// 64 * 2^k; 4-bit with groups of 64, of 128 * 2^k, or one per channel.  `blocks`: 32-channel blocks of the whole launch (all sibling sets).
 // Taken for 17 to 32 rows -- unless K is long and the blocks cover only part of the chip, where every workgroup's read
 // of all the activations outweighs the rest -- and below that from where it was measured ahead.  bf16, the kernels
 // otherwise taken (decode / skinny up to 16 rows, tiled + split-K above) / this one, in us:
@@ -325,8 +350,15 @@ bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
   if (!w || !w->qweight || w->kn || w->plain)
     return false;
   if (w->bits == 8) {
-    if (w->g != 0 || (w->K % W8_TILE_K) != 0)
+    if ((w->K % W8_TILE_K) != 0)
       return false;
+    if (w->g != 0) {  // groups of 64 * 2^k (or one spanning K)
+      if (w->g % W8_TILE_K != 0)
+        return false;
+      const int tpg = w->g / W8_TILE_K;
+      if ((tpg & (tpg - 1)) != 0 && tpg < w->k_tiles)
+        return false;
+    }
   } else {
     if ((w->K % W4_TILE_K) != 0)
       return false;
@@ -379,13 +411,28 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
       a.k_tiles = (int)v->k_tiles;
       a.row_blocks = (int)v->row_blocks;
       a.chip = v->chip;
+      a.G = v->G;
+      a.group_shift = 31;
+      const bool grp = v->g != 0 && v->g / W8_TILE_K < v->k_tiles;
+      if (grp) {
+        a.group_shift = 0;
+        while ((1 << a.group_shift) < v->g / W8_TILE_K)
+          ++a.group_shift;
+      }
       const dim3 grid8((unsigned)blocks);
-#define MI_R32_8(NQ_)                                                     \
-  {                                                                       \
-    if (f16)                                                              \
-      a16_rows32_kernel<MI_DT_F16, NQ_><<<grid8, block, 0, stream>>>(a);  \
-    else                                                                  \
-      a16_rows32_kernel<MI_DT_BF16, NQ_><<<grid8, block, 0, stream>>>(a); \
+#define MI_R32_8G(NQ_, GRP_)                                                    \
+  {                                                                             \
+    if (f16)                                                                    \
+      a16_rows32_kernel<MI_DT_F16, NQ_, GRP_><<<grid8, block, 0, stream>>>(a);  \
+    else                                                                        \
+      a16_rows32_kernel<MI_DT_BF16, NQ_, GRP_><<<grid8, block, 0, stream>>>(a); \
+  }
+#define MI_R32_8(NQ_)       \
+  {                         \
+    if (grp)                \
+      MI_R32_8G(NQ_, true)  \
+    else                    \
+      MI_R32_8G(NQ_, false) \
   }
       if (nq == 1)
         MI_R32_8(1)
@@ -396,6 +443,7 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
       else
         MI_R32_8(4)
 #undef MI_R32_8
+#undef MI_R32_8G
     }
     MI_HIP(hipGetLastError());
     return MI_SUCCESS;
