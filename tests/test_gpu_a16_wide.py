@@ -178,6 +178,43 @@ def test_tolerance_form_at_prefill_size_on_sampled_channels(orc):
     assert err_ref <= 1e-2
 
 
+W8_WIDE_GROUPED_CASES = [  # (M, K, N, g, dtype): quantization groups of 64 * 2^k along K
+    (256, 512, 128, 64, "bf16"), (300, 1024, 200, 128, "bf16"), (40, 192, 48, 64, "f16"), (513, 1024, 272, 256, "f16"),
+    (512, 4096, 1024, 64, "bf16"), (1, 128, 16, 64, "bf16"), (130, 2048, 520, 512, "bf16"), (64, 256, 136, 256, "f16"),
+]
+
+
+@pytest.mark.parametrize("M,K,N,g,dt", W8_WIDE_GROUPED_CASES)
+def test_w8_grouped_on_wide_tiles_against_oracle(orc, plan, M, K, N, g, dt):
+    """8-bit weight sets with one scale and zero point per group of 64 * 2^k inputs: the tile's pairs travel with its
+    weights.  Same bounds as the per-channel cases."""
+    import torch
+    plan(a16_wide_min_m=1)
+    dtype = clib.DT_F16 if dt == "f16" else clib.DT_BF16
+    cfg = S.w8a16(M, K, N, g, seed=M + K + N, bias=(N % 2 == 0))
+    x, wq, scale, zp, bias = f32_valued_a16(cfg)
+    x16, scale16 = cfg["x"], cfg["scale"]
+    if dtype == clib.DT_F16:
+        x, scale = orc.F16(x), orc.F16(scale)
+        x16, scale16 = orc.f32_to_f16(x), orc.f32_to_f16(scale)
+    tdt = torch.float16 if dtype == clib.DT_F16 else torch.bfloat16
+    w = M_.A16Weight(cfg["weight"], scale16, cfg["zp"], bias, K=K, N=N, weight_bits=8, q_group_size=g, dtype=dtype)
+    xd = torch.from_numpy(x16.view(np.int16)).cuda().view(tdt)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_launch(w, xd, y_f32=y32)
+    torch.cuda.synchronize()
+    out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    pre = y32.cpu().numpy()
+    w.destroy()
+    want, want_pre = orc.a16matmul(x, wq, scale, zp, bias, M=M, K=K, N=N, weight_bits=8, q_group_size=g,
+                                   out_dtype=orc.OUT_F16 if dtype == clib.DT_F16 else orc.OUT_BF16,
+                                   gemm_kind=orc.GEMM_F64ACC)
+    err = cmp.max_abs_over_rms(pre, want_pre)
+    assert err <= 2e-5, "fp32 pre-round max-abs/RMS %.3g" % err
+    to16 = orc.f32_to_f16 if dtype == clib.DT_F16 else orc.f32_to_bf16
+    assert np.array_equal(out, to16(pre))
+
+
 ROWS32_CASES = [  # (M, K, N, signed, dtype): 8-bit, one scale per channel, up to 32 rows
     (32, 4096, 1024, True, "bf16"), (17, 512, 40, False, "bf16"), (24, 1024, 200, True, "f16"), (32, 64, 16, True, "bf16"),
     (9, 448, 33, False, "bf16"), (1, 128, 64, True, "f16"), (31, 11008, 96, True, "bf16"),

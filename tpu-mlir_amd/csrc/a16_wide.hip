@@ -54,7 +54,7 @@ struct TolArgs {
   const uint8_t *x;      // [M][K] 16-bit
   const uint8_t *qw;     // packed tiles [row_blocks][k_tiles][1024]
   const uint32_t *sz;    // 4-bit: scale|zp words [row_blocks][G][16]
-  const uint16_t *sc8;   // 8-bit: scale bits [row_blocks][1][16] and -zp' * scale [row_blocks][1][16]
+  const uint16_t *sc8;   // 8-bit: scale bits [row_blocks][G][16] and -zp' * scale [row_blocks][G][16]
   const float *nz8;
   const float *bias;     // [N] or null
   uint16_t *y;           // [M][N]
@@ -108,6 +108,11 @@ __device__ __forceinline__ u32x4 wide_load16(const void *p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
   return v;
 }
+__device__ __forceinline__ uint32_t wide_load2(const void *p) {  // 16 bits, zero-extended
+  uint32_t v;
+  asm volatile("global_load_ushort %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
 __device__ __forceinline__ uint32_t wide_load4(const void *p) {
   uint32_t v;
   asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
@@ -129,13 +134,16 @@ __device__ __forceinline__ f32x16 wide_mfma(typename Half16<DT>::vec8 a, typenam
 // BITS == 4: f16 only, groups of whole 128-K tiles (group of tile kt = kt >> group_shift).  BITS == 8: one scale per
 // channel, either 16-bit type.
 // TT (4-bit only): the exact two-term form instead of weights rounded once.
-template <int BITS, int DT, bool TT>
+// GRP (8-bit only): quantization groups of 64 * 2^k along K; the tile's scales and zero-point terms travel with its
+// weights.
+template <int BITS, int DT, bool TT, bool GRP = false>
 __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m, int tiles_n, int per_xcd) {
   static_assert(BITS == 8 || DT == MI_DT_F16 || TT, "4-bit weights rounded to bf16 leave the comparison tolerance");
   static_assert(BITS == 4 || !TT, "8-bit weights are rounded to the 16-bit type by the reference itself");
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
-  constexpr int WL = TolW<BITS>::WL, WRING = TolW<BITS>::RING, UNIT_ST = TolW<BITS>::UNIT_ST;
+  static_assert(BITS == 8 || !GRP, "4-bit groups ride the scale|zp words");
+  constexpr int WL = TolW<BITS>::WL + (GRP ? 4 : 0), WRING = TolW<BITS>::RING, UNIT_ST = TolW<BITS>::UNIT_ST;
   constexpr int GPT = 1;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -194,13 +202,20 @@ __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m
   u32x4 wq[WRING][2][2];       // [ring][column block][slot: kq = h, h + 2]
   uint32_t szw[WRING][2][GPT];
   float s8[2], nz8[2];         // 8-bit: the lane's per-channel scale and -zp' * scale
+  const uint16_t *sc8base[2];  // ... or, with groups, where the tiles' pairs come from, and their ring
+  const float *nz8base[2];
+  uint32_t scw[WRING][2], nzw[WRING][2];
   if constexpr (BITS == 8) {
 #pragma unroll
     for (int jb = 0; jb < 2; ++jb) {
       int64_t rb = n_base / 16 + wn * 4 + jb * 2 + (c32 >> 4);
       rb = rb < a.row_blocks ? rb : a.row_blocks - 1;
-      s8[jb] = H::to_f32(a.sc8[rb * 16 + (c32 & 15)]);
-      nz8[jb] = a.nz8[rb * 16 + (c32 & 15)];
+      sc8base[jb] = a.sc8 + rb * a.G * 16 + (c32 & 15);
+      nz8base[jb] = a.nz8 + rb * a.G * 16 + (c32 & 15);
+      if constexpr (!GRP) {
+        s8[jb] = H::to_f32(sc8base[jb][0]);
+        nz8[jb] = nz8base[jb][0];
+      }
     }
   }
   // the weight-side requests one stage makes, WL of them, for weight tile kt into ring slot rs.  4-bit: column block
@@ -213,6 +228,10 @@ __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m
       wide_arrived(wq[rs][jb][1]);
       if constexpr (BITS == 4)
         wide_arrived(szw[rs][jb][0]);
+      if constexpr (GRP) {
+        wide_arrived(scw[rs][jb]);
+        wide_arrived(nzw[rs][jb]);
+      }
     }
   };
   auto issue_w = [&](int kt, int rs, int half) {
@@ -228,6 +247,14 @@ __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m
         const uint8_t *p = wbase[jb] + (int64_t)ktc * 1024;
         wq[rs][jb][0] = wide_load16(p);
         wq[rs][jb][1] = wide_load16(p + 512);
+      }
+      if constexpr (GRP) {
+        const int gi = ktc >> a.group_shift;
+#pragma unroll
+        for (int jb = 0; jb < 2; ++jb) {
+          scw[rs][jb] = wide_load2(sc8base[jb] + gi * 16);
+          nzw[rs][jb] = wide_load4(nz8base[jb] + gi * 16);
+        }
       }
     }
   };
@@ -275,7 +302,11 @@ __global__ __launch_bounds__(256, 1) void a16_wide_kernel(TolArgs a, int tiles_m
           fb[jb] = tol_dequant(word, s, nzs, nib_magic);
       } else {
         const int j = su >> 1;
-        fb[jb] = dequant_bytes<DT>(wq[rs][jb][su & 1][2 * j], wq[rs][jb][su & 1][2 * j + 1], s8[jb], nz8[jb]);
+        if constexpr (GRP)
+          fb[jb] = dequant_bytes<DT>(wq[rs][jb][su & 1][2 * j], wq[rs][jb][su & 1][2 * j + 1],
+                                     H::to_f32((uint16_t)scw[rs][jb]), __builtin_bit_cast(float, nzw[rs][jb]));
+        else
+          fb[jb] = dequant_bytes<DT>(wq[rs][jb][su & 1][2 * j], wq[rs][jb][su & 1][2 * j + 1], s8[jb], nz8[jb]);
       }
     }
   };
@@ -462,13 +493,23 @@ bool a16_wide4_applicable(const mi_a16_weight *w, int64_t M) {
   return false;
 }
 
-// 8-bit weight sets with one scale per channel: the wide tiles are the reference's arithmetic, and faster than the
-// tiled kernel once there are enough 256 x 128 tiles to occupy the chip.  Measured, bf16, tiled / wide in us:
-//   11008 x 4096   M = 256 (86 tiles): 76.5 / 69.6   M = 384 (172): 110.1 / 73.8   M = 512: 111.7 / 75.7   M = 2048: 323.6 / 224.9
-//   4096 x 4096    M = 512 (64 tiles): 47.9 / 65.5   M = 1024 (128): 66.6 / 68.8   M = 2048 (256): 110.5 / 78.9
+// 8-bit weight sets with one scale per channel or per group of 64 * 2^k inputs: the wide tiles are the reference's
+// arithmetic, and faster than the tiled kernel once there are enough 256 x 128 tiles to occupy the chip.  Measured,
+// bf16, tiled / wide in us:
+//   per channel  11008 x 4096   M = 256 (86 tiles): 76.5 / 69.6   M = 384 (172): 110.1 / 73.8   M = 512: 111.7 / 75.7   M = 2048: 323.6 / 224.9
+//                4096 x 4096    M = 512 (64 tiles): 47.9 / 65.5   M = 1024 (128): 66.6 / 68.8   M = 2048 (256): 110.5 / 78.9
+//   groups of 64 11008 x 4096   M = 256: 74.1 / 78.1   M = 384: 104.9 / 81.1   M = 512: 104.1 / 79.2   M = 2048: 359.4 / 235.5
+//                4096 x 11008   M = 1024 (128 tiles): 159.4 / 180.3   M = 2048 (256): 252.3 / 210.4
 bool a16_wide8_applicable(const mi_a16_weight *w, int64_t M) {
-  if (!w || !w->qweight || w->kn || w->plain || w->bits != 8 || w->g != 0 || (w->K % W8_TILE_K) != 0)
+  if (!w || !w->qweight || w->kn || w->plain || w->bits != 8 || (w->K % W8_TILE_K) != 0)
     return false;
+  if (w->g != 0) {  // groups of 64 * 2^k (or one spanning K)
+    if (w->g % W8_TILE_K != 0)
+      return false;
+    const int tpg = w->g / W8_TILE_K;
+    if ((tpg & (tpg - 1)) != 0 && tpg < w->k_tiles)
+      return false;
+  }
   if (plan().a16_wide_min_m != 0)
     return plan().a16_wide_min_m > 0 && M >= plan().a16_wide_min_m;
   const int64_t tiles = ((M + TOL_M - 1) / TOL_M) * ((w->N + TOL_N - 1) / TOL_N);
@@ -498,14 +539,14 @@ int a16_wide_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
   a.row_blocks = (int)w->row_blocks;
   a.chip = w->chip;
   a.group_shift = 0;
-  if (w->bits == 4) {
-    const int tpg = w->g == 0 ? (int)w->k_tiles : w->g / W4_TILE_K;
-    if (tpg >= w->k_tiles)
-      a.group_shift = 31;
-    else
-      while ((1 << a.group_shift) < tpg)
-        ++a.group_shift;
-  }
+  const int tile_k = w->bits == 4 ? W4_TILE_K : W8_TILE_K;
+  const int tpg = w->g == 0 ? (int)w->k_tiles : w->g / tile_k;  // weight tiles per group
+  if (tpg >= w->k_tiles)
+    a.group_shift = 31;
+  else
+    while ((1 << a.group_shift) < tpg)
+      ++a.group_shift;
+  const bool grp8 = w->bits == 8 && tpg < w->k_tiles;
   const int64_t tiles_m = (M + TOL_M - 1) / TOL_M, tiles_n = (w->N + TOL_N - 1) / TOL_N;
   MI_REQUIRE(tiles_m * tiles_n < (1ll << 30), MI_BAD_ARGUMENT, "mi_a16mm_launch: too many output tiles");
   const int per_xcd = (int)((tiles_m * tiles_n + 7) / 8);
@@ -523,6 +564,16 @@ int a16_wide_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
   } else if (w->bits == 4) {
     auto kfn = a16_wide_kernel<4, MI_DT_F16, false>;
     once4.ensure((const void *)kfn, (int)lds_bytes);
+    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
+  } else if (grp8 && w->dtype == MI_DT_F16) {
+    auto kfn = a16_wide_kernel<8, MI_DT_F16, false, true>;
+    static LdsLimitOnce once;
+    once.ensure((const void *)kfn, (int)lds_bytes);
+    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
+  } else if (grp8) {
+    auto kfn = a16_wide_kernel<8, MI_DT_BF16, false, true>;
+    static LdsLimitOnce once;
+    once.ensure((const void *)kfn, (int)lds_bytes);
     kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
   } else if (w->dtype == MI_DT_F16) {
     auto kfn = a16_wide_kernel<8, MI_DT_F16, false>;
