@@ -348,7 +348,7 @@ def bench_bf16_prefill_two_term(pkg, S, torch, clib, launches=10):
     import ctypes
     names = ("a16_waves", "a16_tpw", "a16_rows", "a16_xlds", "a16_no_gemm", "a16_no_decode", "a16_gemm_min_m",
              "a16_gemm_splits", "a16_gemm_tile", "a16_gemm_rows", "i8_tile", "i8_mid_ring", "i8_ring", "dq_waves", "f8_tile",
-             "a16_decode_rows8", "a16_rows32_min_m", "a16_wide_min_m", "a16_wide4_min_m")
+             "a16_decode_rows8", "a16_rows32_min_m", "a16_wide_min_m", "a16_wide4_min_m", "a16_rows32_split")
 
     class Plan(ctypes.Structure):
         _fields_ = [(n, ctypes.c_int) for n in names]

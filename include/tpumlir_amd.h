@@ -252,12 +252,14 @@ int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
 /* mi_a16mm_launch for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid it).  No counterpart in the reference.  Same arguments, same kernels, bit-identical results;
  * it calls no hipMalloc / hipFree or allocating library routine.  The only scratch memory the product needs -- the
- * fp32 partial-sum slabs of a K-split tiled launch (more than 16 rows, few output blocks) -- lives in a 16 MiB device
- * array inside the library (one copy per GPU, held until the process ends) instead of the stream's growable buffer.
- * A product whose slabs need more (k_splits * M * N * 4 bytes; e.g. M = 128, N = 4096 with 4 splits is 8 MiB) is
- * refused with MI_BAD_ARGUMENT and a message that says so.  The slabs need no clearing (every element read is written
- * by the same launch), but every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two
- * streams, two threads) race -- serialize them. */
+ * fp32 partial sums of K-split launches (tiled kernel: more than 32 rows, few output blocks; 32-row kernel: long K,
+ * few channels) -- lives in a 16 MiB device array inside the library (one copy per GPU, held until the process ends)
+ * instead of the stream's growable buffer.  A product whose slabs need more than 16 MiB - 1 KiB (tiled kernel:
+ * k_splits * M * N * 4 bytes; e.g. M = 128, N = 4096 with 4 splits is 8 MiB) is refused with MI_BAD_ARGUMENT and a
+ * message that says so.  The slabs need no clearing (every element read is written by the same launch); the array's
+ * first KiB holds the 32-row kernel's arrival counters, which start as zeros and which every launch leaves at zero.
+ * Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two threads)
+ * race -- serialize them. */
 int mi_a16mm_launch_noalloc(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                             void *stream);
 

@@ -24,7 +24,7 @@ class _InternalPlan(__import__("ctypes").Structure):
     """Mirror of mi_internal_plan (csrc/internal.h): kernel-selection overrides, zero = the library's heuristic."""
     _fields_ = [(n, __import__("ctypes").c_int) for n in (
         "a16_waves", "a16_tpw", "a16_rows", "a16_xlds", "a16_no_gemm", "a16_no_decode", "a16_gemm_min_m", "a16_gemm_splits",
-        "a16_gemm_tile", "a16_gemm_rows", "i8_tile", "i8_mid_ring", "i8_ring", "dq_waves", "f8_tile", "a16_decode_rows8", "a16_rows32_min_m", "a16_wide_min_m", "a16_wide4_min_m")]
+        "a16_gemm_tile", "a16_gemm_rows", "i8_tile", "i8_mid_ring", "i8_ring", "dq_waves", "f8_tile", "a16_decode_rows8", "a16_rows32_min_m", "a16_wide_min_m", "a16_wide4_min_m", "a16_rows32_split")]
 
 
 @pytest.fixture

@@ -124,3 +124,48 @@ def test_w8_grouped_up_to_32_rows_against_oracle(orc, plan, M, K, N, g, dt):
     assert err <= 2e-5, "fp32 pre-round max-abs/RMS %.3g" % err
     to16 = orc.f32_to_f16 if dtype == clib.DT_F16 else orc.f32_to_bf16
     assert np.array_equal(out, to16(pre))
+
+
+SPLIT_CASES = [  # (bits, M, K, N, g, parts, dtype): the K of a 32-channel block shared by `parts` workgroups
+    (4, 32, 4096, 1024, 128, 2, "bf16"), (4, 17, 4096, 520, 128, 4, "bf16"), (4, 24, 384, 100, 128, 4, "f16"),
+    (4, 32, 11008, 96, 64, 4, "bf16"), (4, 9, 128, 33, 0, 2, "bf16"), (8, 32, 4096, 1024, 0, 2, "bf16"),
+    (8, 20, 11008, 200, 64, 4, "bf16"), (8, 31, 192, 40, 64, 4, "f16"), (8, 12, 64, 16, 0, 2, "f16"),
+]
+
+
+@pytest.mark.parametrize("bits,M,K,N,g,parts,dt", SPLIT_CASES)
+def test_k_split_over_workgroups_against_oracle_and_repeatable(orc, plan, bits, M, K, N, g, parts, dt):
+    """Launches with few 32-channel blocks share each block's K between 2 or 4 workgroups; the last to arrive sums the
+    partial blocks in part order.  Three launches in a row (the counters have to be back at zero each time) give the
+    same bits, within the exact kernels' bounds of the oracle; K short enough that some waves get no tile included."""
+    import torch
+    plan(a16_rows32_min_m=1, a16_rows32_split=parts)
+    dtype = clib.DT_F16 if dt == "f16" else clib.DT_BF16
+    cfg = (S.w4a16(M, K, N, g, seed=M + K + N, bias=(N % 2 == 0)) if bits == 4
+           else S.w8a16(M, K, N, g, seed=M + K + N, signed=False, bias=(N % 2 == 0)))
+    x, wq, scale, zp, bias = f32_valued_a16(cfg)
+    x16, scale16 = cfg["x"], cfg["scale"]
+    if dtype == clib.DT_F16:
+        x, scale = orc.F16(x), orc.F16(scale)
+        x16, scale16 = orc.f32_to_f16(x), orc.f32_to_f16(scale)
+    tdt = torch.float16 if dtype == clib.DT_F16 else torch.bfloat16
+    w = M_.A16Weight(cfg["weight"], scale16, cfg["zp"], bias, K=K, N=N, weight_bits=bits, q_group_size=g, dtype=dtype)
+    xd = torch.from_numpy(x16.view(np.int16)).cuda().view(tdt)
+    runs = []
+    for _ in range(3):
+        y32 = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        y = M_.a16mm_launch(w, xd, y_f32=y32)
+        torch.cuda.synchronize()
+        runs.append((y.view(torch.int16).cpu().numpy().view(np.uint16), y32.cpu().numpy()))
+    w.destroy()
+    out, pre = runs[0]
+    for o, p in runs[1:]:
+        assert np.array_equal(o, out) and np.array_equal(p, pre)
+    want, want_pre = orc.a16matmul(x, wq, scale, zp, bias, M=M, K=K, N=N, weight_bits=bits, q_group_size=g,
+                                   out_dtype=orc.OUT_F16 if dtype == clib.DT_F16 else orc.OUT_BF16,
+                                   gemm_kind=orc.GEMM_F64ACC)
+    err = cmp.max_abs_over_rms(pre, want_pre)
+    assert err <= 2e-5, "fp32 pre-round max-abs/RMS %.3g" % err
+    to16 = orc.f32_to_f16 if dtype == clib.DT_F16 else orc.f32_to_bf16
+    assert np.array_equal(out, to16(pre))
+

@@ -44,6 +44,27 @@ def test_no_alloc_launch_matches_the_allocating_one(plan):
         assert torch.equal(f_new.view(torch.int32), f_ref.view(torch.int32)), rows
         assert float(f_ref.abs().max()) > 0
     w.destroy()
+    # the 32-row kernel's K split (long K, few channels): partial blocks and arrival counters in the same array
+    K, N, g = 8192, 1024, 128
+    cfg = S.w4a16(32, K, N, g, seed=33, bias=True)
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], S.bf16_to_f32(cfg["bias"]), K=K, N=N, weight_bits=4,
+                     q_group_size=g)
+    x_all = _bf16(torch, cfg["x"])
+    for rows in (32, 20, 32):
+        x = x_all[:rows].contiguous()
+        y_ref = torch.empty((rows, N), dtype=torch.bfloat16, device="cuda")
+        f_ref = torch.empty((rows, N), dtype=torch.float32, device="cuda")
+        y_new, f_new = torch.empty_like(y_ref), torch.empty_like(f_ref)
+        M_.a16mm_launch(w, x, y=y_ref, y_f32=f_ref)
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        M_.a16mm_launch(w, x, y=y_new, y_f32=f_new, no_alloc=True)
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() == before
+        assert torch.equal(y_new.view(torch.int16), y_ref.view(torch.int16)), rows
+        assert torch.equal(f_new.view(torch.int32), f_ref.view(torch.int32)), rows
+        assert float(f_ref.abs().max()) > 0
+    w.destroy()
     # slabs beyond the fixed array are refused with a message that says so: M = 640, N = 4096 split four ways along K
     # needs 40 MiB (the split count is pinned through the library's internal plan so that the case does not depend
     # on the heuristics)

@@ -617,10 +617,13 @@ int a16_gemm_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t 
 }  // namespace mi
 
 // ------------------------------------------------------------------------------------------------
-// A launch that allocates nothing: mi_a16mm_launch with the split-K slabs in a fixed device array.
+// A launch that allocates nothing: mi_a16mm_launch with the partial sums of K-split launches in a fixed device array.
 // ------------------------------------------------------------------------------------------------
 namespace {
 constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)16 << 20;
+// The array's first bytes: the 32-row kernel's K-split counters.  They start as zeros (the array has no initializer)
+// and every launch leaves them so; no partial sum is ever put there.
+constexpr size_t NOALLOC_COUNTER_BYTES = 1024;
 constexpr int NOALLOC_MAX_DEVICES = 64;
 // Each GPU the library runs on holds its own copy of this array, at its own address, until the process ends.  In
 // host code the name below is only a handle for hipGetSymbolAddress, never a device address.
@@ -641,6 +644,7 @@ extern "C" int mi_a16mm_launch_noalloc(const mi_a16_weight *w, const uint16_t *d
     MI_REQUIRE(ptr, MI_HIP_ERROR, "mi_a16mm_launch_noalloc: the scratch array has no address on this device");
     __atomic_store_n(&g_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
   }
-  const A16Scratch fixed = {ptr, NOALLOC_SCRATCH_BYTES};
+  const A16Scratch fixed = {(unsigned char *)ptr + NOALLOC_COUNTER_BYTES, NOALLOC_SCRATCH_BYTES - NOALLOC_COUNTER_BYTES,
+                            (unsigned *)ptr};
   return a16_launch_group(&w, 1, d_x, M, &d_y, d_y_f32 ? &d_y_f32 : nullptr, (hipStream_t)stream, &fixed);
 }

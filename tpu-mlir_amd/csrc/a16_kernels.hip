@@ -785,7 +785,7 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
     for (int i = 0; i < n; ++i)
       all = all && a16_rows32_applicable(ws[i], M, blocks);
     if (all)
-      return a16_rows32_launch_group(ws, n, d_x, M, d_ys, d_y32s, stream);
+      return a16_rows32_launch_group(ws, n, d_x, M, d_ys, d_y32s, stream, fixed);
   }
   // 8-bit, one scale per channel, or 4-bit in the exact two-term form; many rows: the wide tiles, one set per launch
   const bool wide4 = a16_wide4_applicable(w, M);

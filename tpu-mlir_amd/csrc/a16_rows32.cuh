@@ -40,6 +40,56 @@ __device__ __forceinline__ uint32_t r32_load4(const void *p) {
   return v;
 }
 
+// K split over 2^shift workgroups per 32-channel block (adjacent in launch order), for launches whose blocks would
+// leave most of the chip idle.  Each workgroup leaves its 32 x 32 partial block in `part`; the one to arrive last at
+// the block's counter adds them up in part order (so the result does not depend on who that is), stores the outputs
+// and puts the counter back to zero for the next launch.
+constexpr int R32_SPLIT_MAX_WGS = 256;          // workgroups of a split launch, at most
+constexpr int R32_SPLIT_COUNTER_BYTES = 1024;   // one counter per block of a split launch
+struct Rows32Split {
+  int shift;           // 0: no split, nothing below is touched
+  float *part;         // [workgroup][16 registers][64 lanes]
+  unsigned *counters;  // [block], zero between launches
+};
+
+// The workgroup's sums -- v[q] is register 2 wave + q of the block (NV = 2) -- joined with the other K parts'.  False: another workgroup will finish this block.  flag: one int of LDS nobody else uses.
+// The partial sums and the counter are device-scope relaxed atomics -- stores that write through and loads that look
+// past this XCD's L2 -- ordered by waiting for them: a release / acquire fence at device scope would write back and
+// invalidate the whole L2 once per wave (measured: 80 us for 256 workgroups instead of 8).
+template <int NV>
+__device__ __forceinline__ bool r32_join_parts(float (&v)[NV], const Rows32Split &sp, int wave, int lane, int *flag) {
+  const int parts = 1 << sp.shift;
+  const int64_t block = blockIdx.x >> sp.shift;
+  constexpr int SLAB = NV * 512;  // floats per workgroup
+  float *slab = sp.part + block * parts * SLAB;
+  const int idx = wave * 128 + lane;  // + 64 q + 1024 j
+  float *mine = slab + (blockIdx.x & (parts - 1)) * SLAB + idx;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+    __hip_atomic_store(mine + (k >> 1) * 1024 + (k & 1) * 64, v[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(0));  // this wave's partial sums are out before the count below says so
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned before = __hip_atomic_fetch_add(sp.counters + block, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int last = before == (unsigned)(parts - 1);
+    if (last)
+      __hip_atomic_store(sp.counters + block, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *flag = last;
+  }
+  __syncthreads();  // the loads below are issued after the count has come back
+  if (!*flag)
+    return false;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+    v[k] = 0.f;
+  for (int p = 0; p < parts; ++p)
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+      v[k] += __hip_atomic_load(slab + p * SLAB + idx + (k >> 1) * 1024 + (k & 1) * 64, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_AGENT);
+  return true;
+}
+
 // 8-bit weights: one weight set per launch
 struct Rows32Args {
   const uint8_t *x;      // [M][K] 16-bit
@@ -52,6 +102,7 @@ struct Rows32Args {
   float *y32;            // [M][N] or null
   int64_t N, K;
   int M, k_tiles, row_blocks, chip;
+  Rows32Split split;
 };
 
 constexpr int R32_MAX_SETS = 4;
@@ -69,6 +120,7 @@ struct Rows32W4Args {
   float *y32[R32_MAX_SETS];             // [M][N] or null
   int64_t N[R32_MAX_SETS];
   int row_blocks[R32_MAX_SETS];
+  Rows32Split split;
 };
 
 }  // namespace mi

@@ -38,9 +38,10 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c32 = lane & 31, h = lane >> 5;
-  const int64_t n = (int64_t)blockIdx.x * 32 + c32;
+  const int bid = blockIdx.x >> a.split.shift;  // the 32-channel block; its K part: the low bits
+  const int64_t n = (int64_t)bid * 32 + c32;
 
-  int64_t rb = (int64_t)blockIdx.x * 2 + (c32 >> 4);
+  int64_t rb = (int64_t)bid * 2 + (c32 >> 4);
   rb = rb < a.row_blocks ? rb : a.row_blocks - 1;  // channels past N repeat the last row block; never stored
   const uint8_t *wp = a.qw + rb * a.k_tiles * 1024 + (uint32_t)((h * 16 + (c32 & 15)) * 16);
   constexpr int WL = GRP ? 4 : 2;  // weight-side requests per tile
@@ -67,11 +68,13 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
   uint8_t *xs = smem + wave * 8192;
   const uint8_t *xf = xs + c32 * 128;  // this lane's fragment row; chunk c sits at position c ^ (c32 / 2) % 8
 
-  // this wave's tiles: wave, wave + 8, ...; `count` of them (the same for every lane)
-  const int count = (a.k_tiles - wave + WAVES - 1) / WAVES;
+  // this wave's tiles: first, first + stride, ... (the waves of all K parts of the block take the tiles round-robin);
+  // `count` of them (the same for every lane)
+  const int first = (blockIdx.x & ((1 << a.split.shift) - 1)) * WAVES + wave, stride = WAVES << a.split.shift;
+  const int count = (a.k_tiles - first + stride - 1) / stride;
   auto tile_of = [&](int i) {  // past the end: the wave's last tile again (a harmless re-load, never multiplied)
     const int ii = i < count ? i : count - 1;
-    return wave + ii * WAVES;
+    return first + ii * stride;
   };
   u32x4 w[3][2];   // weight ring: [tile % 3][slot kq = h, h + 2]
   uint32_t scw[3], nzw[3];  // GRP: the tile's scale bits and -zp' * scale
@@ -155,20 +158,24 @@ __global__ __launch_bounds__(512) void a16_rows32_kernel(Rows32Args a) {
     red[wave][r][lane] = acc[r];
   __syncthreads();
   const float bias_v = (a.bias && n < a.N) ? a.bias[n] : 0.f;
+  float v[2] = {0.f, 0.f};
+#pragma unroll
+  for (int q = 0; q < 2; ++q)
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv)
+      v[q] += red[wv][wave * 2 + q][lane];
+  if (a.split.shift != 0 && !r32_join_parts(v, a.split, wave, lane, reinterpret_cast<int *>(smem + 32768)))
+    return;
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
     const int r = wave * 2 + q;
-    float v = 0.f;
-#pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv)
-      v += red[wv][r][lane];
     const int orow = 8 * (r >> 2) + 4 * h + (r & 3);
     if (orow < a.M && n < a.N) {
-      v += bias_v;
+      const float o32 = v[q] + bias_v;
       const int64_t o = (int64_t)orow * a.N + n;
       if (a.y32)
-        a.y32[o] = v;
-      a.y[o] = a.chip == MI_CHIP_CV18XX ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+        a.y32[o] = o32;
+      a.y[o] = a.chip == MI_CHIP_CV18XX ? round_out16<DT, MI_CHIP_CV18XX>(o32) : round_out16<DT, MI_CHIP_BM168X>(o32);
     }
   }
 }
@@ -187,7 +194,7 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c32 = lane & 31, h = lane >> 5;
   // which weight set: selected, not indexed (a runtime index would move the argument block to scratch memory)
-  const int bid = blockIdx.x;
+  const int bid = blockIdx.x >> a.split.shift;  // the launch's 32-channel block; its K part: the low bits
   const int t1 = bid >= a.block_begin[1], t2 = bid >= a.block_begin[2], t3 = bid >= a.block_begin[3];
 #define R32_SEL(f) (t3 ? a.f[3] : t2 ? a.f[2] : t1 ? a.f[1] : a.f[0])
   const int lb = bid - R32_SEL(block_begin);  // the set's own 32-channel block
@@ -209,10 +216,12 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
   uint8_t *xs = smem + wave * 8192;
   const uint8_t *xf = xs + c32 * 128;
 
-  const int count = (a.k_tiles - wave + WAVES - 1) / WAVES;  // this wave's tiles: wave, wave + 8, ...
+  // this wave's tiles: first, first + stride, ... (see a16_rows32_kernel)
+  const int first = (blockIdx.x & ((1 << a.split.shift) - 1)) * WAVES + wave, stride = WAVES << a.split.shift;
+  const int count = (a.k_tiles - first + stride - 1) / stride;
   auto tile_of = [&](int i) {  // past the end: the wave's last tile again (a harmless re-load, never multiplied)
     const int ii = i < count ? i : count - 1;
-    return wave + ii * WAVES;
+    return first + ii * stride;
   };
   u32x4 w[3][2];         // weight ring: [tile % 3][slot kq = h, h + 2]
   uint32_t szw[3][GPT];  // the tile's scale|zp words
@@ -316,20 +325,24 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
   float *y32 = R32_SEL(y32);
   uint16_t *y = R32_SEL(y);
   const float bias_v = (biasp && n < set_n) ? biasp[n] : 0.f;
+  float v[2] = {0.f, 0.f};
+#pragma unroll
+  for (int q = 0; q < 2; ++q)
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv)
+      v[q] += red[wv][wave * 2 + q][lane];
+  if (a.split.shift != 0 && !r32_join_parts(v, a.split, wave, lane, reinterpret_cast<int *>(smem + 32768)))
+    return;
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
     const int r = wave * 2 + q;
-    float v = 0.f;
-#pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv)
-      v += red[wv][r][lane];
     const int orow = 8 * (r >> 2) + 4 * h + (r & 3);
     if (orow < a.M && n < set_n) {
-      v += bias_v;
+      const float o32 = v[q] + bias_v;
       const int64_t o = (int64_t)orow * set_n + n;
       if (y32)
-        y32[o] = v;
-      y[o] = a.chip == MI_CHIP_CV18XX ? round_out16<DT, MI_CHIP_CV18XX>(v) : round_out16<DT, MI_CHIP_BM168X>(v);
+        y32[o] = o32;
+      y[o] = a.chip == MI_CHIP_CV18XX ? round_out16<DT, MI_CHIP_CV18XX>(o32) : round_out16<DT, MI_CHIP_BM168X>(o32);
     }
   }
 #undef R32_SEL
@@ -337,9 +350,9 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
 
 // Weight sets in the tiled layout whose K is a whole number of tiles: 8-bit with one scale per channel or groups of
 // 64 * 2^k; 4-bit with groups of 64, of 128 * 2^k, or one per channel.  `blocks`: 32-channel blocks of the whole launch (all sibling sets).
-// Taken for 17 to 32 rows -- unless K is long and the blocks cover only part of the chip, where every workgroup's read
-// of all the activations outweighs the rest -- and below that from where it was measured ahead.  bf16, the kernels
-// otherwise taken (decode / skinny up to 16 rows, tiled + split-K above) / this one, in us:
+// Taken for 17 to 32 rows, and below that from where it was measured ahead.  bf16, the kernels otherwise taken
+// (decode / skinny up to 16 rows, tiled + split-K above) / this one without K split, in us (with the split, which
+// the long-K cases on part of the chip need to stay ahead: the table at rows32_split_shift):
 //   8-bit  11008 x 4096   M = 4: 10.9 / 13.2   M = 8: 15.8 / 13.4   M = 12: 17.2 / 13.9   M = 16: 22.2 / 14.4   M = 17: 28.5 / 14.9   M = 32: 29.3 / 17.5
 //   8-bit  4096 x 4096    M = 8:  6.6 /  7.1   M = 16:  7.7 /  8.0   M = 17: 14.6 /  8.1   M = 24: 14.9 /  8.9   M = 32: 15.4 /  9.7
 //   4-bit  11008 x 4096   M = 8:  9.9 / 11.8   M = 9: 11.3 / 12.4   M = 12: 13.1 / 12.3   M = 16: 14.6 / 12.7   M = 17: 17.1 / 13.1   M = 32: 17.8 / 15.3
@@ -375,16 +388,60 @@ bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
   if (M > 32)
     return false;
   if (M >= 17)
-    return !(w->K > 8192 && blocks < 256 && M > 24);
+    return true;
   if (w->bits == 8)
-    return M >= 8 && blocks >= 256;
-  return (M >= 12 && (blocks >= 192 || w->K > 8192)) || (M >= 8 && w->K > 8192);
+    return M >= 8 && (blocks >= 256 || w->K >= 8192);
+  return (M >= 12 && (blocks >= 192 || w->K >= 8192)) || (M >= 8 && w->K >= 8192 && blocks >= 64);
+}
+
+// K parts per 32-channel block of a launch of `blocks` blocks over K: doubled while the launch stays within one
+// workgroup per CU and every wave keeps five 64-K steps or more (four for 8-bit weights from 24 rows on).  Measured,
+// bf16, M = 32, 1 / 2 / 4 parts in us (two workgroups per CU, 512 in all, lose to 256):
+//   4-bit  4096 x 11008 (128 blocks)  18.7 / 14.3 / 15.7      2048 x 11008 (64)  17.9 / 13.1 / 10.7
+//   4-bit  4096 x 8192  (128)         13.8 / 11.1 / 13.2      1024 x 8192 (32)   12.9 / 10.0 /  8.5
+//   4-bit  4096 x 4096  (128)          8.7 /  8.9             2048 x 4096 (64)    7.2 /  7.6 /  8.0
+//   8-bit  4096 x 11008, groups of 64 (128)  23.6 / 17.0 / 19.2      2048 x 8192 (64)  14.8 / 11.8 / 9.6
+//   8-bit  4096 x 4096  (128)          9.8 /  9.1 (M = 17: 8.1 / 8.3)
+static int rows32_split_shift(const mi_a16_weight *w, int64_t M, int64_t blocks) {
+  const int forced = plan().a16_rows32_split;
+  if (forced == 1 || forced == 2 || forced == 4)
+    return blocks * forced <= R32_SPLIT_MAX_WGS ? (forced >> 1) : 0;
+  const int64_t steps = w->K / 64, per_wave = (w->bits == 8 && M >= 24) ? 4 : 5;
+  int shift = 0;
+  while (shift < 2 && (blocks << (shift + 1)) <= 256 && steps >= per_wave * (8 << (shift + 1)))
+    ++shift;
+  return shift;
+}
+
+// Scratch for a split launch: counters (zero between launches) and the partial blocks, in the caller's fixed area or
+// in the stream's own buffer (counters first), allocated and cleared when the stream first needs it.
+static int rows32_split_scratch(hipStream_t stream, int shift, const A16Scratch *fixed, Rows32Split *out) {
+  out->shift = shift;
+  out->part = nullptr;
+  out->counters = nullptr;
+  if (shift == 0)
+    return MI_SUCCESS;
+  constexpr size_t part_bytes = (size_t)R32_SPLIT_MAX_WGS * 4096;
+  if (fixed) {
+    MI_REQUIRE(fixed->counters && fixed->bytes >= part_bytes, MI_BAD_ARGUMENT,
+               "the fixed scratch area is too small for a K-split launch of the 32-row kernel");
+    out->counters = fixed->counters;
+    out->part = (float *)fixed->ptr;
+    return MI_SUCCESS;
+  }
+  void *p = nullptr;
+  const int rc = stream_workspace(stream, WS_ROWS32_SPLIT, R32_SPLIT_COUNTER_BYTES + part_bytes, &p, /*zero_fresh=*/true);
+  if (rc != MI_SUCCESS)
+    return rc;
+  out->counters = (unsigned *)p;
+  out->part = (float *)((uint8_t *)p + R32_SPLIT_COUNTER_BYTES);
+  return MI_SUCCESS;
 }
 
 // ws[0..n): sibling weight sets on one input -- same K, width, group size, type and chip (checked by the caller), each
 // acceptable to a16_rows32_applicable
 int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
-                            float *const *d_y32s, hipStream_t stream) {
+                            float *const *d_y32s, hipStream_t stream, const A16Scratch *fixed) {
   MI_REQUIRE(M >= 1 && M <= 32, MI_BAD_ARGUMENT, "mi_a16mm_launch: M out of range for this kernel");
   MI_REQUIRE(d_x, MI_BAD_ARGUMENT, "mi_a16mm_launch: null activation pointer");
   const mi_a16_weight *w = ws[0];
@@ -419,7 +476,10 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
         while ((1 << a.group_shift) < v->g / W8_TILE_K)
           ++a.group_shift;
       }
-      const dim3 grid8((unsigned)blocks);
+      const int rc = rows32_split_scratch(stream, rows32_split_shift(v, M, blocks), fixed, &a.split);
+      if (rc != MI_SUCCESS)
+        return rc;
+      const dim3 grid8((unsigned)(blocks << a.split.shift));
 #define MI_R32_8G(NQ_, GRP_)                                                    \
   {                                                                             \
     if (f16)                                                                    \
@@ -481,7 +541,10 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
         MI_REQUIRE(blocks < (1ll << 30), MI_BAD_ARGUMENT, "mi_a16mm_launch: too many output channels");
       }
     }
-    const dim3 grid((unsigned)blocks);
+    const int rc = rows32_split_scratch(stream, rows32_split_shift(w, M, blocks), fixed, &a.split);
+    if (rc != MI_SUCCESS)
+      return rc;
+    const dim3 grid((unsigned)(blocks << a.split.shift));
 #define MI_R32_4(GPT_, NQ_)                                                      \
   {                                                                              \
     if (f16)                                                                     \

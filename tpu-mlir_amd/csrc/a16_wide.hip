@@ -516,6 +516,21 @@ bool a16_wide8_applicable(const mi_a16_weight *w, int64_t M) {
   return tiles > 128;
 }
 
+// One launch of instance KFN; the instance's LDS limit is raised once (all instances share a function type, so the
+// record is per template argument, not per type).
+struct WideLaunch {
+  TolArgs a;
+  int tiles_m, tiles_n, per_xcd;
+  hipStream_t stream;
+};
+template <auto KFN>
+static void wide_go(const WideLaunch &l) {
+  static LdsLimitOnce once;
+  constexpr size_t lds_bytes = (size_t)TOL_NST * TOL_STAGE_BYTES;
+  once.ensure((const void *)KFN, (int)lds_bytes);
+  KFN<<<dim3((unsigned)(l.per_xcd * 8)), dim3(256), lds_bytes, l.stream>>>(l.a, l.tiles_m, l.tiles_n, l.per_xcd);
+}
+
 int a16_wide_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                     hipStream_t stream, bool two_term) {
   MI_REQUIRE(M >= 0 && M < (1ll << 31), MI_BAD_ARGUMENT, "mi_a16mm_launch: M out of range");
@@ -550,40 +565,16 @@ int a16_wide_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
   const int64_t tiles_m = (M + TOL_M - 1) / TOL_M, tiles_n = (w->N + TOL_N - 1) / TOL_N;
   MI_REQUIRE(tiles_m * tiles_n < (1ll << 30), MI_BAD_ARGUMENT, "mi_a16mm_launch: too many output tiles");
   const int per_xcd = (int)((tiles_m * tiles_n + 7) / 8);
-  const size_t lds_bytes = (size_t)TOL_NST * TOL_STAGE_BYTES;
-  const dim3 grid((unsigned)(per_xcd * 8)), block(256);
-  static LdsLimitOnce once4, once8b, once8h, once4tb, once4th;
-  if (w->bits == 4 && two_term && w->dtype == MI_DT_BF16) {
-    auto kfn = a16_wide_kernel<4, MI_DT_BF16, true>;
-    once4tb.ensure((const void *)kfn, (int)lds_bytes);
-    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
-  } else if (w->bits == 4 && two_term) {
-    auto kfn = a16_wide_kernel<4, MI_DT_F16, true>;
-    once4th.ensure((const void *)kfn, (int)lds_bytes);
-    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
-  } else if (w->bits == 4) {
-    auto kfn = a16_wide_kernel<4, MI_DT_F16, false>;
-    once4.ensure((const void *)kfn, (int)lds_bytes);
-    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
-  } else if (grp8 && w->dtype == MI_DT_F16) {
-    auto kfn = a16_wide_kernel<8, MI_DT_F16, false, true>;
-    static LdsLimitOnce once;
-    once.ensure((const void *)kfn, (int)lds_bytes);
-    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
-  } else if (grp8) {
-    auto kfn = a16_wide_kernel<8, MI_DT_BF16, false, true>;
-    static LdsLimitOnce once;
-    once.ensure((const void *)kfn, (int)lds_bytes);
-    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
-  } else if (w->dtype == MI_DT_F16) {
-    auto kfn = a16_wide_kernel<8, MI_DT_F16, false>;
-    once8h.ensure((const void *)kfn, (int)lds_bytes);
-    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
-  } else {
-    auto kfn = a16_wide_kernel<8, MI_DT_BF16, false>;
-    once8b.ensure((const void *)kfn, (int)lds_bytes);
-    kfn<<<grid, block, lds_bytes, stream>>>(a, (int)tiles_m, (int)tiles_n, per_xcd);
-  }
+  const bool f16 = w->dtype == MI_DT_F16;
+  const WideLaunch l{a, (int)tiles_m, (int)tiles_n, per_xcd, stream};
+  if (w->bits == 4 && two_term)
+    f16 ? wide_go<a16_wide_kernel<4, MI_DT_F16, true>>(l) : wide_go<a16_wide_kernel<4, MI_DT_BF16, true>>(l);
+  else if (w->bits == 4)
+    wide_go<a16_wide_kernel<4, MI_DT_F16, false>>(l);  // the tolerance form: f16 only (a16_tol_applicable)
+  else if (grp8)
+    f16 ? wide_go<a16_wide_kernel<8, MI_DT_F16, false, true>>(l) : wide_go<a16_wide_kernel<8, MI_DT_BF16, false, true>>(l);
+  else
+    f16 ? wide_go<a16_wide_kernel<8, MI_DT_F16, false>>(l) : wide_go<a16_wide_kernel<8, MI_DT_BF16, false>>(l);
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;
 }

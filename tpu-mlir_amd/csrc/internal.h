@@ -27,9 +27,10 @@ typedef struct mi_internal_plan {
   int dq_waves;                      // 8 / 16
   int f8_tile;                       // 256 / 128 / 64
   int a16_decode_rows8;              // 1: five to eight rows always take the decode kernel where it can; -1: never
-  int a16_rows32_min_m;              // > 0: 8-bit per-channel sets take the 32-row kernel from this many rows (to 32); -1: never
-  int a16_wide_min_m;                // > 0: 8-bit per-channel sets take the wide tiles from this many rows on; -1: never
+  int a16_rows32_min_m;              // > 0: sets it can handle take the 32-row kernel from this many rows (to 32); -1: never
+  int a16_wide_min_m;                // > 0: 8-bit sets take the wide tiles from this many rows on; -1: never
   int a16_wide4_min_m;               // > 0: 4-bit sets take the exact two-term wide tiles from this many rows on; -1: never
+  int a16_rows32_split;              // 1 / 2 / 4: K parts per 32-channel block of the 32-row kernel
 } mi_internal_plan;
 void mi_internal_set_plan(const mi_internal_plan *p);  // null: back to the heuristics
 }
@@ -117,13 +118,20 @@ void a16_free(mi_a16_weight *w);
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                hipStream_t stream);
 int a16_kn_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32, hipStream_t st);
-// wide-tile product (a16_wide.hip), weights rounded to the 16-bit type before the multiply: the reference's arithmetic
-// for 8-bit per-channel sets (taken from a few hundred rows on), the opt-in tolerance form for 4-bit f16 sets; and the
-// exact two-term form for 4-bit sets (each weight as the sum of two 16-bit numbers, two MFMAs per fragment)
-// up to 32 rows, one workgroup per 32 channels over the whole K (a16_rows32.hip)
+// a caller-provided scratch area that a launch must make do with (instead of the stream's growable buffer)
+struct A16Scratch {
+  void *ptr;           // partial sums of K-split launches; contents are whatever the last launch left
+  size_t bytes;
+  unsigned *counters;  // 256 of them, zero between launches (the 32-row kernel's K split)
+};
+// up to 32 rows, one workgroup per 32 channels over the whole K, or over a part of it where the blocks are few
+// (a16_rows32.hip: the partial blocks then pass through `fixed`, or else the stream's scratch buffer).
 bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks);
 int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
-                            float *const *d_y32s, hipStream_t stream);
+                            float *const *d_y32s, hipStream_t stream, const A16Scratch *fixed);
+// wide-tile product (a16_wide.hip), weights rounded to the 16-bit type before the multiply: the reference's arithmetic
+// for 8-bit sets (taken from a few hundred rows on), the opt-in tolerance form for 4-bit f16 sets; and the exact
+// two-term form for 4-bit sets (each weight as the sum of two 16-bit numbers, two MFMAs per fragment)
 bool a16_wide8_applicable(const mi_a16_weight *w, int64_t M);
 bool a16_wide4_applicable(const mi_a16_weight *w, int64_t M);
 int a16_wide_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
@@ -135,11 +143,6 @@ int a16_plain_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uin
                      hipStream_t st);
 int a16_plain_create(mi_a16_weight *w, const void *weight, int weight_signed, const uint16_t *scale,
                      const uint8_t *zp, const float *bias);
-// a caller-provided scratch area that a launch must make do with (instead of the stream's growable buffer)
-struct A16Scratch {
-  void *ptr;
-  size_t bytes;
-};
 // decode kernel (a16_decode.hip): at most four rows, K a whole number of tiles.  Returns false, having launched
 // nothing, when the shape is not its own; the general kernels then take it.
 bool a16_decode_launch(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
@@ -154,8 +157,10 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
 
 // library-owned scratch, one buffer per (device, stream, purpose) (workspace.hip); contents are whatever the last
 // user left
-enum { WS_SPLIT_K = 0, WS_DYNAMIC_QUANT = 1, WS_F8_TRANSPOSE = 2 };
-int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out);
+enum { WS_SPLIT_K = 0, WS_DYNAMIC_QUANT = 1, WS_F8_TRANSPOSE = 2, WS_ROWS32_SPLIT = 3 };
+// zero_fresh: a newly allocated buffer starts as zeros (for users that leave their counters at zero, and always ask
+// for the same size)
+int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out, bool zero_fresh = false);
 // frees every buffer of a stream (current and retired); for owners of private streams, right before hipStreamDestroy
 void release_stream_workspaces(hipStream_t st);
 

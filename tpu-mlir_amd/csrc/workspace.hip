@@ -26,7 +26,7 @@ std::mutex g_mutex;
 std::map<std::tuple<int, hipStream_t, int>, Buf> g_bufs;
 }  // namespace
 
-int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out) {
+int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out, bool zero_fresh) {
   int dev = 0;
   MI_HIP(hipGetDevice(&dev));
   std::lock_guard<std::mutex> lock(g_mutex);
@@ -40,6 +40,13 @@ int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out) {
     const size_t want = (bytes + 255) & ~(size_t)255;
     void *fresh = nullptr;
     MI_HIP(hipMalloc(&fresh, want));
+    if (zero_fresh) {  // on the stream, ahead of the first kernel to use it (the stream is not being captured)
+      const hipError_t e = hipMemsetAsync(fresh, 0, want, st);
+      if (e != hipSuccess) {
+        (void)hipFree(fresh);
+        MI_HIP(e);
+      }
+    }
     if (b.ptr)
       b.retired.push_back(b.ptr);
     b.ptr = fresh;
