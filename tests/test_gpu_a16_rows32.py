@@ -169,3 +169,38 @@ def test_k_split_over_workgroups_against_oracle_and_repeatable(orc, plan, bits, 
     to16 = orc.f32_to_f16 if dtype == clib.DT_F16 else orc.f32_to_bf16
     assert np.array_equal(out, to16(pre))
 
+
+
+def test_k_split_launch_replays_from_a_graph(orc):
+    """A K-split launch of the 32-row kernel (4096 x 11008, M = 32: two workgroups per 32-channel block by the
+    library's own rule) captured into a graph after one eager run on the stream: four replays with eager launches of
+    another row count between them all give the eager result -- the arrival counters are back at zero every time."""
+    import torch
+    M, K, N, g = 32, 11008, 4096, 128
+    cfg = S.w4a16(M, K, N, g, seed=5)
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=K, N=N, weight_bits=4, q_group_size=g)
+    st = torch.cuda.Stream()
+    x = torch.from_numpy(cfg["x"].view(np.int16)).cuda().view(torch.bfloat16)
+    y_eager = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    y_graph = torch.empty_like(y_eager)
+    y_other = torch.empty((20, N), dtype=torch.bfloat16, device="cuda")
+    M_.a16mm_launch(w, x, y=y_eager, stream=st)                 # eager: the stream gets its scratch buffer
+    st.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=st):
+        M_.a16mm_launch(w, x, y=y_graph, stream=st)
+    torch.cuda.synchronize()
+    for rep in range(4):
+        y_graph.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_graph.view(torch.int16), y_eager.view(torch.int16)), rep
+        M_.a16mm_launch(w, x[:20].contiguous(), y=y_other, stream=st)
+        torch.cuda.synchronize()
+    x32, wq, scale, zp, _ = f32_valued_a16(cfg)
+    want, _ = orc.a16matmul(x32, wq, scale, zp, None, M=M, K=K, N=N, weight_bits=4, q_group_size=g,
+                            out_dtype=orc.OUT_BF16, gemm_kind=orc.GEMM_F64ACC)
+    got = S.bf16_to_f32(y_eager.view(torch.int16).cpu().numpy().view(np.uint16))
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    assert float(np.max(np.abs(got - want))) <= 1e-2 * rms
+    w.destroy()
