@@ -356,6 +356,8 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
 //   8-bit  11008 x 4096   M = 4: 10.9 / 13.2   M = 8: 15.8 / 13.4   M = 12: 17.2 / 13.9   M = 16: 22.2 / 14.4   M = 17: 28.5 / 14.9   M = 32: 29.3 / 17.5
 //   8-bit  4096 x 4096    M = 8:  6.6 /  7.1   M = 16:  7.7 /  8.0   M = 17: 14.6 /  8.1   M = 24: 14.9 /  8.9   M = 32: 15.4 /  9.7
 //   4-bit  11008 x 4096   M = 8:  9.9 / 11.8   M = 9: 11.3 / 12.4   M = 12: 13.1 / 12.3   M = 16: 14.6 / 12.7   M = 17: 17.1 / 13.1   M = 32: 17.8 / 15.3
+//   4-bit  22016 x 4096   M = 7: 17.0 / 18.6   M = 8: 19.5 / 16.9   M = 11: 19.0 / 17.1
+//   8-bit  11008 x 4096   M = 5: 14.5 / 13.0   M = 7: 15.1 / 12.9      8-bit  4096 x 11008   M = 5: 12.8 / 12.7   M = 6: 20.8 / 12.6
 //   4-bit  4096 x 4096    M = 12: 6.3 /  7.4   M = 16:  7.0 /  7.5   M = 17: 11.8 /  7.6   M = 32: 12.5 /  8.4
 //   4-bit  4096 x 11008   M = 4: 11.8 / 13.3   M = 8: 14.2 / 13.2   M = 16: 14.5 / 13.9   M = 17: 16.3 / 14.5   M = 24: 16.6 / 16.3   M = 32: 16.9 / 18.5
 //   4-bit  6144 x 2048, groups of 64   M = 9: 5.6 / 6.0   M = 12: 6.2 / 6.1   M = 16: 6.9 / 6.2   M = 17: 10.6 / 6.2   M = 32: 11.6 / 6.6
@@ -389,9 +391,9 @@ bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
     return false;
   if (M >= 17)
     return true;
-  if (w->bits == 8)
-    return M >= 8 && (blocks >= 256 || w->K >= 8192);
-  return (M >= 12 && (blocks >= 192 || w->K >= 8192)) || (M >= 8 && w->K >= 8192 && blocks >= 64);
+  if (w->bits == 8)  // from five rows on: below, the decode kernel (up to four rows) is ahead
+    return M >= 5 && (blocks >= 256 || w->K >= 8192);
+  return (M >= 12 && (blocks >= 192 || w->K >= 8192)) || (M >= 8 && (blocks >= 512 || (w->K >= 8192 && blocks >= 64)));
 }
 
 // K parts per 32-channel block of a launch of `blocks` blocks over K: doubled while the launch stays within one

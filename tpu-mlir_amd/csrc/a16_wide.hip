@@ -512,8 +512,11 @@ bool a16_wide8_applicable(const mi_a16_weight *w, int64_t M) {
   }
   if (plan().a16_wide_min_m != 0)
     return plan().a16_wide_min_m > 0 && M >= plan().a16_wide_min_m;
+  // ... and enough rows to fill half a tile's 256: a wide set (22016 x 4096: 172 tiles already at one row) otherwise
+  // sent its decode launches here -- 62 us instead of 18 at M = 1.  22016 x 4096, others / wide in us: M = 64: 52.5 /
+  // 67.8   M = 128: 76.1 / 69.0   M = 160: 103.7 / 69.6; 65536 x 4096: M = 128: 130 / 168   M = 160: 227 / 161
   const int64_t tiles = ((M + TOL_M - 1) / TOL_M) * ((w->N + TOL_N - 1) / TOL_N);
-  return tiles > 128;
+  return M > 128 && tiles > 128;
 }
 
 // One launch of instance KFN; the instance's LDS limit is raised once (all instances share a function type, so the
