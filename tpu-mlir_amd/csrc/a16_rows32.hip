@@ -391,9 +391,29 @@ bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
     return false;
   if (M >= 17)
     return true;
-  if (w->bits == 8)  // from five rows on: below, the decode kernel (up to four rows) is ahead
-    return M >= 5 && (blocks >= 256 || w->K >= 8192);
-  return (M >= 12 && (blocks >= 192 || w->K >= 8192)) || (M >= 8 && (blocks >= 512 || (w->K >= 8192 && blocks >= 64)));
+  // Below 17 rows the decode kernel (up to four or eight rows) and the skinny kernel are tuned for K = 4096 and a
+  // number of 16-channel blocks that fills the CUs evenly; this kernel's time hardly moves with M, K or N.  From a sweep
+  // over 15 shapes and M = 1 ... 16 (others / this one, us):
+  //   8-bit  5120 x 5120    M = 1:  9.2 /  8.2   M = 4: 13.0 /  8.2   M = 16: 20.5 /  8.7
+  //   8-bit  6656 x 6656    M = 2: 15.5 / 11.8   M = 8: 17.4 / 11.7      8-bit  8192 x 8192   M = 2: 19.4 / 16.5   M = 6: 25.8 / 16.5
+  //   8-bit  4096 x 4096    M = 5:  6.3 /  7.4   M = 16: 7.9 /  7.6      8-bit  6144 x 2048   M = 8:  6.7 /  6.2   M = 16: 7.9 / 6.2
+  //   4-bit  5120 x 5120    M = 3:  8.8 /  8.3   M = 4: 11.7 /  8.4   M = 16: 19.8 /  8.6
+  //   4-bit  13824 x 5120   M = 4: 22.4 / 13.8   M = 8: 15.8 / 13.9      4-bit  8192 x 8192   M = 5: 13.2 / 12.3   M = 6: 15.7 / 12.7
+  //   4-bit  4096 x 11008   M = 5: 11.1 / 11.9   M = 6: 13.8 / 11.6      4-bit  32000 x 4096  M = 8: 20.8 / 22.5 (tiled kernel ahead)
+  const bool long_k = w->K >= 8192, mid_k = w->K > 4096 && w->K < 8192;
+  if (w->bits == 8) {
+    if (M >= 5)
+      return blocks >= 160 || long_k;
+    // K past 4096: from two rows, and at one row where the decode kernel's 16-channel blocks fall badly on the CUs
+    // (8192 x 8192 M = 1: 17.4 / 15.7; 5120 x 13824: 20.0 / 17.8; but 28672 x 8192: 48.7 / 49.8)
+    return w->K > 4096 && blocks >= 128 && (M >= 2 || (blocks >= 160 && blocks <= 512));
+  }
+  if (long_k && M >= 3 && (blocks >= 160 || (M >= 6 && blocks >= 64)))  // 28672 x 8192 M = 4: 44.1 / 36.0
+    return true;
+  if (mid_k && blocks >= 128 && M >= 4)
+    return true;
+  // very wide sets are the tiled kernel's from 8 rows on (32000 x 4096 M = 12: 20.7 / 23.1)
+  return (M >= 12 && ((blocks >= 192 && blocks <= 768) || long_k)) || (M >= 8 && blocks >= 512 && blocks <= 768);
 }
 
 // K parts per 32-channel block of a launch of `blocks` blocks over K: doubled while the launch stays within one
