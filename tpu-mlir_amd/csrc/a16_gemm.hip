@@ -505,6 +505,31 @@ static int launch_gemm_shape(GemmArgs &a, hipStream_t st, const A16Scratch *fixe
     else
       rows = c_128 <= c_64 ? 128 : 64;
   }
+  // Below that count (where K may be split), from a sweep over nine shapes and M = 17 ... 512, in us:
+  //   sets of very few columns (up to 16 blocks of 64 x 128 in all) take 16- or 32-row blocks for the workgroups'
+  //   sake (1024 x 8192, 4-bit, M = 64: 16.3 -> 13.5; 8-bit, M = 33: 17.0 -> 14.6);
+  //   8-bit weights come through registers, which taller blocks re-read less often: 128 rows from M = 96 where that
+  //   still leaves 32 blocks, 128 x 256 from M = 192 when K or N goes past 4096 (11008 x 4096 M = 128: 50.6 -> 42.4,
+  //   M = 256: 74.1 -> 64.1; 4096 x 11008 M = 384: 119.6 -> 72.1; 8192 x 8192 M = 256: 94.4 -> 68.0; 5120 x 5120
+  //   M = 512: 83.0 -> 57.3; 4096 x 4096 M = 384: 45.1 -> 38.5 with 128 x 128, 128 x 256 no better);
+  //   4-bit: 64-row blocks up to M = 640 at K = 4096 (measured), 128 rows from M = 256 when K is longer and 64 such
+  //   blocks exist (4096 x 11008 M = 384: 71.2 -> 62.8; 8192 x 8192 M = 512: 110.5 -> 97.9; 5120 x 5120 M = 256:
+  //   37.0 -> 30.7; but 1024 x 8192 M = 256: 18.4 with 64 rows, 22.6 with 128)
+  if (tile == 0 && rows == 0 && !wide && a.M > 32) {
+    bool n_past_4096 = false;
+    for (int i = 0; i < a.n_seg; ++i)
+      n_past_4096 = n_past_4096 || a.seg[i].N > 4096;
+    if (t64 <= 16) {
+      rows = a.M <= 64 ? 16 : 32;
+    } else if constexpr (BITS == 8) {
+      if (a.M >= 96 && t128 >= 32) {
+        rows = 128;
+        wide = fits && a.M >= 192 && a.K >= 4096 && (a.K > 4096 || n_past_4096);
+      }
+    } else if (a.K > 4096 && a.M >= 256 && t128 >= 64) {
+      rows = 128;
+    }
+  }
   if constexpr (fits) {
     if (wide)
       return launch_gemm_instance<BITS, DT, GPT, 2, 4, 4, 4>(a, st, fixed);
