@@ -54,3 +54,17 @@ def test_random_shape_int8_matmul(orc, i, M, K, N, rt, a_unsigned, b_unsigned, r
     else:
         want = acc64
     assert np.array_equal(out.cpu().numpy().astype(np.int64), want)
+
+
+@pytest.mark.parametrize("i,M,K,N,rt,a_unsigned,b_unsigned,relu,requant", [
+    (0, 1, 128, 32, True, False, False, False, True), (1, 32, 4096, 1024, True, False, False, False, True),
+    (2, 17, 640, 200, False, True, False, True, True), (3, 5, 256, 33, True, False, True, False, False),
+    (4, 31, 1152, 900, False, True, True, True, True), (5, 8, 11008, 96, True, False, False, False, True),
+    (6, 2, 384, 1, True, True, False, False, False), (7, 24, 2048, 4096, True, False, False, True, True),
+])
+def test_int8_matmul_with_few_rows(orc, plan, i, M, K, N, rt, a_unsigned, b_unsigned, relu, requant):
+    """Up to 32 rows with K a multiple of 128 take the streaming kernel (a workgroup per 32 output columns, operands
+    straight from memory, the K order inside a tile permuted alike for both): forced here, same checks as above, either
+    operand unsigned with its zero point, column counts that are not multiples of 32."""
+    plan(i8_tile=32)
+    test_random_shape_int8_matmul(orc, 200 + i, M, K, N, rt, a_unsigned, b_unsigned, relu, requant)

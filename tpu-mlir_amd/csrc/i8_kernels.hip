@@ -878,6 +878,98 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Few rows (M <= 32): the product is a stream over the right operand, HBM-bound.  A workgroup owns 32 output
+// columns over the whole K; its eight waves take the 128-byte K tiles round-robin, each multiplies all rows (one
+// 32 x 32 MFMA block; rows past M repeat the last row and are never stored) against its tiles, operands straight from
+// global memory into registers one tile ahead; the eight partial blocks are summed once through LDS.  A lane's 64
+// contiguous bytes of its row of a tile feed four MFMAs, 16 bytes each: the K order inside a tile is permuted the same
+// way for both operands, which a dot product does not see.  Requires K % 128 == 0.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(512) void i8_rows32_kernel(I8Args a) {
+  constexpr int WAVES = 8;
+  __shared__ int32_t red[WAVES][16][64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c32 = lane & 31, h = lane >> 5;
+  const int64_t n = (int64_t)blockIdx.x * 32 + c32;
+  const int64_t nb = n < a.N ? n : a.N - 1;  // columns past N repeat the last one; never stored
+  const int64_t ma = c32 < a.M ? c32 : a.M - 1;
+  const uint8_t *pb = a.B + nb * a.K + h * 64;
+  const uint8_t *pa = a.A + ma * a.K + h * 64;
+  const uint32_t fa = (uint32_t)a.a_flip * 0x01010101u, fb = (uint32_t)a.b_flip * 0x01010101u;
+  const int k_tiles = (int)(a.K / 128);
+  const int count = (k_tiles - wave + WAVES - 1) / WAVES;  // this wave's tiles: wave, wave + 8, ...
+
+  i32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    acc[r] = 0;
+  u32x4 xa[2][4], xb[2][4];
+  auto load_tile = [&](int i, int slot) {
+    const int64_t off = (int64_t)(wave + (i < count ? i : count - 1) * WAVES) * 128;  // past the end: a re-load
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      xb[slot][j] = *(const u32x4 *)(pb + off + j * 16);
+      xa[slot][j] = *(const u32x4 *)(pa + off + j * 16);
+    }
+  };
+  if (count > 0) {
+    load_tile(0, 0);
+    for (int t0 = 0; t0 < count; t0 += 2) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        if (t0 + u >= count)
+          break;
+        load_tile(t0 + u + 1, u ^ 1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          u32x4 va = xa[u][j], vb = xb[u][j];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            va[e] ^= fa;
+            vb[e] ^= fb;
+          }
+          acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, va), __builtin_bit_cast(i32x4, vb), acc,
+                                                      0, 0, 0);
+        }
+      }
+    }
+  }
+  // cross-wave sum, in wave order.  Register r of lane l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    red[wave][r][lane] = acc[r];
+  __syncthreads();
+  const int32_t bias_n = (a.bias && n < a.N) ? a.bias[n] : 0;
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int r = wave * 2 + q;
+    int32_t v = 0;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv)
+      v += red[wv][r][lane];
+    const int64_t m = 8 * (r >> 2) + 4 * h + (r & 3);
+    if (m < a.M && n < a.N) {
+      v += bias_n;
+      if (a.row_term)
+        v += a.row_term[m];
+      if (a.do_relu) {
+        v = v > 0 ? v : 0;
+        if (a.relu_limit > 0 && v > a.relu_limit)
+          v = (int32_t)a.relu_limit;
+      }
+      const int64_t o = m * a.N + n;
+      if (a.acc_out)
+        a.acc_out[o] = v;
+      if (a.has_rq)
+        store_out(a.out, o, requant_one(v, n, a.rq), a.rq.out_dtype);
+      else if (a.out)
+        ((int32_t *)a.out)[o] = v;
+    }
+  }
+}
+
 static RequantParams make_rq(const mi_requant_desc *rq) {
   RequantParams p;
   p.mult = rq->d_multiplier;
@@ -993,8 +1085,17 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
   const int64_t tiles_large = ((M + LM - 1) / LM) * ((N + LN - 1) / LN);
   const bool large_ok = (K % 128) == 0 && M >= 128 && N >= 128, mid_ok = (K % 64) == 0;
   const int tile_pick = plan().i8_tile ? plan().i8_tile : (large_ok && tiles_large >= 144 ? 256 : 128);  // measured crossover
-  const bool large = large_ok && tile_pick == 256;
-  const bool mid = !large && mid_ok && tile_pick > 0;
+  // up to 32 rows: the streaming kernel (plan: i8_tile = 32 asks for it, any other value rules it out).  Every
+  // workgroup of it reads all of the left operand, so it is taken where that is little beside its 32 columns of the
+  // right one, or where the 64 x 64 tiles are too few and too long.  Measured, 64 x 64 tiles / this one in us (launches
+  // issued one by one, about 10 us apart at best):  4096 x 11008 (N x K) M = 1: 36.3 / 16.7   M = 32: 36.4 / 28.8;
+  // 8192 x 8192 M = 1: 30.0 / 18.7   M = 32: 31.5 / 25.7;  11008 x 4096 M = 4: 17.5 / 17.9   M = 32: 18.4 / 25.3;
+  // 32000 x 4096 M = 1: 32.9 / 31.2   M = 8: 33.6 / 37.2
+  const bool few_fits = M <= 32 && (K % 128) == 0;
+  const bool few_pays = M * N <= 45056 || (N <= 8192 && (M <= 24 || K > 4096));
+  const bool few = few_fits && (plan().i8_tile == 32 || (plan().i8_tile == 0 && few_pays));
+  const bool large = !few && large_ok && tile_pick == 256;
+  const bool mid = !few && !large && mid_ok && tile_pick > 0;
   uint8_t *a_signed = nullptr, *b_signed = nullptr;
   if (large || mid) {
     // direct-to-LDS loads cannot flip sign bits on the way: unsigned operands are rewritten once (after the
@@ -1062,6 +1163,9 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
       MI_LARGE(EPI_GENERIC)
 #undef MI_LARGE_I
 #undef MI_LARGE
+  } else if (few) {
+    MI_REQUIRE((N + 31) / 32 < (1ll << 31), MI_BAD_ARGUMENT, "i8 matmul: too many output columns");
+    i8_rows32_kernel<<<dim3((unsigned)((N + 31) / 32)), dim3(512), 0, stream>>>(a);
   } else {
     dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
     i8_gemm_kernel<<<grid, dim3(256), 0, stream>>>(a);

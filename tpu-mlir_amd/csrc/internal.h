@@ -21,7 +21,7 @@ typedef struct mi_internal_plan {
   int a16_gemm_splits;               // > 0: number of K splits of the tiled kernel
   int a16_gemm_tile;                 // 128 / 256: columns per output block
   int a16_gemm_rows;                 // 16 / 32 / 64 / 128: rows per output block
-  int i8_tile;                       // 256 / 128 / -1 (register-staged kernel)
+  int i8_tile;                       // 256 / 128 / 32 (streaming kernel for up to 32 rows) / -1 (register-staged kernel)
   int i8_mid_ring;                   // 4 / 8 (128-tiles), 64 (64-tiles)
   int i8_ring;                       // 3 / 4 / 5: LDS ring stages of the large kernel
   int dq_waves;                      // 8 / 16
