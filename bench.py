@@ -153,9 +153,13 @@ def bench_int8(pkg, S, torch, clib, n, steps, warmup, M=None, graph=False):
     else:
         sec = _time_launches(torch, run, steps, warmup=warmup)
     tops = 2.0 * M * n * n / sec / 1e12
-    return {"workload": "int8_requant_gemm_M%d_N%d_K%d_qdm_per_channel" % (M, n, n), "tops": round(tops, 2),
-            "us_per_launch": round(sec * 1e6, 2), "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4),
-            "dtype": "int8*int8->int32->int8"}
+    rec = {"workload": "int8_requant_gemm_M%d_N%d_K%d_qdm_per_channel" % (M, n, n), "tops": round(tops, 2),
+           "us_per_launch": round(sec * 1e6, 2), "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4),
+           "dtype": "int8*int8->int32->int8"}
+    if M <= 32:  # a stream over the right operand (one buffer here: it stays in the 256 MB memory-side cache)
+        rec["right_operand_GBps"] = round(n * n / sec / 1e9, 1)
+        rec["right_operand"] = "one %d MB buffer, cache-resident" % (n * n // 1000000)
+    return rec
 
 
 def _time_launches(torch, fn, steps, warmup=5):
@@ -769,6 +773,7 @@ def main():
         ex["prefill_bf16_fold_vs_two_term"] = bench_bf16_prefill_two_term(pkg, S, torch, clib)
         ex["dynamic_quant"] = bench_dynamic_quant(pkg, S, torch)
         ex["int8_256x1024x1024"] = bench_int8(pkg, S, torch, clib, 1024, 40, 5, M=256, graph=True)
+        ex["int8_1x4096x4096"] = bench_int8(pkg, S, torch, clib, 4096, 40, 5, M=1, graph=True)
         ex["f8_matmul"] = bench_f8_matmul(pkg, torch, clib)
         ex["operator_boundary"] = bench_operator_boundary(pkg, S)
         ex["device_resident_block"] = bench_module_block(pkg, S, clib, cfgs)
