@@ -68,3 +68,21 @@ def test_int8_matmul_with_few_rows(orc, plan, i, M, K, N, rt, a_unsigned, b_unsi
     operand unsigned with its zero point, column counts that are not multiples of 32."""
     plan(i8_tile=32)
     test_random_shape_int8_matmul(orc, 200 + i, M, K, N, rt, a_unsigned, b_unsigned, relu, requant)
+
+
+def test_int8_few_rows_k_split_is_repeatable(orc, plan):
+    """2048 x 8192 (N x K) with one and with 20 rows: 64 column blocks and a long K, so two workgroups share each
+    block's K and the last to arrive adds the two partial blocks.  Three launches in a row give the same bits (the counters are back at zero
+    each time), equal to exact integer arithmetic."""
+    import torch
+    plan(i8_tile=32)
+    K, N = 8192, 2048
+    c = S.int8_matmul(20, K, N, seed=77, right_transpose=True)
+    dev = lambda t: torch.from_numpy(np.ascontiguousarray(t)).cuda()
+    a, b, bias = dev(c["a"]), dev(c["b"]), dev(c["bias"])
+    want = c["a"].astype(np.int64) @ c["b"].astype(np.int64).T + c["bias"].astype(np.int64)
+    for rows in (20, 1, 20):
+        acc = torch.empty((rows, N), dtype=torch.int32, device="cuda")
+        M_.i8mm_launch(a[:rows].contiguous(), b, bias, right_transpose=True, acc=acc)
+        torch.cuda.synchronize()
+        assert np.array_equal(acc.cpu().numpy().astype(np.int64), want[:rows]), rows

@@ -44,8 +44,6 @@ __device__ __forceinline__ uint32_t r32_load4(const void *p) {
 // leave most of the chip idle.  Each workgroup leaves its 32 x 32 partial block in `part`; the one to arrive last at
 // the block's counter adds them up in part order (so the result does not depend on who that is), stores the outputs
 // and puts the counter back to zero for the next launch.
-constexpr int R32_SPLIT_MAX_WGS = 256;          // workgroups of a split launch, at most
-constexpr int R32_SPLIT_COUNTER_BYTES = 1024;   // one counter per block of a split launch
 struct Rows32Split {
   int shift;           // 0: no split, nothing below is touched
   float *part;         // [workgroup][16 registers][64 lanes]

@@ -158,6 +158,10 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
 // library-owned scratch, one buffer per (device, stream, purpose) (workspace.hip); contents are whatever the last
 // user left
 enum { WS_SPLIT_K = 0, WS_DYNAMIC_QUANT = 1, WS_F8_TRANSPOSE = 2, WS_ROWS32_SPLIT = 3 };
+// WS_ROWS32_SPLIT, shared by the few-row kernels that split K over workgroups (A16 and INT8): arrival counters, then
+// one 32 x 32 block of partial sums per workgroup.  Always asked for at this one size, so it is never re-allocated.
+constexpr int R32_SPLIT_MAX_WGS = 256;          // workgroups of a split launch, at most
+constexpr int R32_SPLIT_COUNTER_BYTES = 1024;   // one counter per block of a split launch
 // zero_fresh: a newly allocated buffer starts as zeros (for users that leave their counters at zero, and always ask
 // for the same size)
 int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out, bool zero_fresh = false);
