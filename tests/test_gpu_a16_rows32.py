@@ -204,3 +204,30 @@ def test_k_split_launch_replays_from_a_graph(orc):
     rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
     assert float(np.max(np.abs(got - want))) <= 1e-2 * rms
     w.destroy()
+
+
+def test_k_split_launch_captured_before_any_eager_run(orc):
+    """A stream that is captured into a graph before it ever ran a K-split launch has no scratch buffer, and none can
+    be allocated during capture: the launch then goes out unsplit, and the replay is still right."""
+    import torch
+    M, K, N, g = 24, 11008, 1024, 128
+    cfg = S.w4a16(M, K, N, g, seed=6)
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=K, N=N, weight_bits=4, q_group_size=g)
+    st = torch.cuda.Stream()
+    x = torch.from_numpy(cfg["x"].view(np.int16)).cuda().view(torch.bfloat16)
+    y_graph = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=st):
+        M_.a16mm_launch(w, x, y=y_graph, stream=st)
+    for _ in range(2):
+        y_graph.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+    x32, wq, scale, zp, _ = f32_valued_a16(cfg)
+    want, _ = orc.a16matmul(x32, wq, scale, zp, None, M=M, K=K, N=N, weight_bits=4, q_group_size=g,
+                            out_dtype=orc.OUT_BF16, gemm_kind=orc.GEMM_F64ACC)
+    got = S.bf16_to_f32(y_graph.view(torch.int16).cpu().numpy().view(np.uint16))
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    assert float(np.max(np.abs(got - want))) <= 1e-2 * rms
+    w.destroy()

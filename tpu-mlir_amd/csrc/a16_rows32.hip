@@ -453,8 +453,10 @@ static int rows32_split_scratch(hipStream_t stream, int shift, const A16Scratch 
   }
   void *p = nullptr;
   const int rc = stream_workspace(stream, WS_ROWS32_SPLIT, R32_SPLIT_COUNTER_BYTES + part_bytes, &p, /*zero_fresh=*/true);
-  if (rc != MI_SUCCESS)
-    return rc;
+  if (rc != MI_SUCCESS) {  // no scratch (the stream is being captured before it ever had one): one workgroup per block
+    out->shift = 0;
+    return MI_SUCCESS;
+  }
   out->counters = (unsigned *)p;
   out->part = (float *)((uint8_t *)p + R32_SPLIT_COUNTER_BYTES);
   return MI_SUCCESS;
