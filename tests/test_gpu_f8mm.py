@@ -310,3 +310,22 @@ def test_e5m2_matmul_operator_level_and_rejections(orc):
     with pytest.raises(clib.BackendError) as e:
         M_.matmul_f8(af, bf, None, right_transpose=True, f8_type=7)
     assert e.value.code == clib.MI_BAD_ARGUMENT
+
+
+FEW_ROW_CASES = [  # (M, K, N, right_transpose, relu, per_channel, bias): up to 32 rows, K a multiple of 128
+    (1, 128, 32, True, False, False, False), (5, 512, 100, False, False, False, True), (32, 4096, 256, True, False, True, True),
+    (17, 1024, 200, True, True, True, True), (24, 11008, 64, True, False, False, True), (31, 8192, 33, False, True, True, False),
+]
+
+
+@pytest.mark.parametrize("M,K,N,rt,relu,per_channel,bias", FEW_ROW_CASES)
+def test_f8_matmul_with_few_rows(orc, plan, M, K, N, rt, relu, per_channel, bias):
+    """The streaming kernel for up to 32 rows (a workgroup per 32 columns, waves split K, with long K and few columns
+    several workgroups per block): the bounds of the tiled kernels."""
+    test_f8_matmul_device_level(orc, plan, M, K, N, rt, relu, per_channel, bias, "32")
+
+
+@pytest.mark.parametrize("M,K,N,rt,relu,bias", [(1, 128, 32, True, False, False), (20, 1024, 100, False, True, True),
+                                                (32, 8192, 64, True, False, True)])
+def test_e5m2_matmul_with_few_rows(orc, plan, M, K, N, rt, relu, bias):
+    test_e5m2_matmul_device_level(orc, plan, M, K, N, rt, relu, bias, "32")

@@ -44,6 +44,10 @@ struct F8Args {
   double step;          // one scale: (double)(float)(1 / scale)
   float inv_step;       // one scale: fl32(1 / step)
   const double *scales; // per channel [N], or null
+  // few-row kernel only: K shared by 2^split_shift workgroups per 32-column block (0: none of the below is touched)
+  int split_shift;
+  float *part;          // [workgroup][16 registers][64 lanes]
+  unsigned *counters;   // [block], zero between launches
 };
 
 __device__ __forceinline__ u32x4 f8_load_chunk(const uint8_t *base, int64_t row, int64_t rows, int64_t k, int64_t K,
@@ -157,6 +161,38 @@ __global__ __launch_bounds__(256) void f8_gemm_kernel(F8Args a) {
 
 // epilogue of a wave's 64 x 64 block: register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of its
 // 32 x 32 block (i, j)
+// One output: bias added by the caller; ReLU, the fp32 side output, the requantization and the store.
+template <int FMT>
+__device__ __forceinline__ void f8_finish_one(const F8Args &a, int64_t o, float v, double step, double inv_step) {
+  if (a.do_relu) {  // post_relu, lib/Support/Dnnl/DnnlUtils.cpp:15-25
+    v = v > 0.0f ? v : 0.0f;
+    if (a.relu_limit > 0.0f && v > a.relu_limit)
+      v = a.relu_limit;
+  }
+  if (a.acc_out)
+    a.acc_out[o] = v;
+  if constexpr (FMT == F8_FMT_E5M2) {
+    f8_store_e5m2(a, o, v);
+    return;
+  }
+  // F8E4M3(v, step, true): the quotient in double, narrowed to fp32, rounded to E4M3 (Float8.cpp:259-261).
+  // v * (1 / step) is within two double ulps of that quotient, so the narrowing can come out differently
+  // only when the 29 bits it drops sit next to the halfway pattern; only then is the division carried out.
+  double qd = (double)v * inv_step;
+  const int32_t low = (int32_t)((uint32_t)__double_as_longlong(qd) & 0x1fffffffu);
+  if (low >= 0x10000000 - 4 && low <= 0x10000000 + 4)
+    qd = (double)v / step;
+  const uint32_t code = f8e4m3_from_f32((float)qd);
+  if (a.out_kind == MI_F8_OUT_CODES)
+    ((uint8_t *)a.out)[o] = (uint8_t)code;
+  else if (a.out_kind == MI_F8_OUT_F32)
+    ((float *)a.out)[o] = f8e4m3_to_f32(code);
+  else if (a.out_kind == MI_F8_OUT_BF16)  // exact: E4M3 values fit both 16-bit types
+    ((uint16_t *)a.out)[o] = (uint16_t)(__float_as_uint(f8e4m3_to_f32(code)) >> 16);
+  else
+    ((uint16_t *)a.out)[o] = __builtin_bit_cast(uint16_t, (_Float16)f8e4m3_to_f32(code));
+}
+
 template <int FMT>
 __device__ __forceinline__ void f8_epilogue(const F8Args &a, const f32x16 (&acc)[2][2], int64_t m0, int64_t n0, int lane) {
 #pragma unroll
@@ -171,37 +207,8 @@ __device__ __forceinline__ void f8_epilogue(const F8Args &a, const f32x16 (&acc)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int64_t m = m0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (n_ok && m < a.M) {
-          float v = acc[i][j][r] + bias_n;
-          if (a.do_relu) {  // post_relu, lib/Support/Dnnl/DnnlUtils.cpp:15-25
-            v = v > 0.0f ? v : 0.0f;
-            if (a.relu_limit > 0.0f && v > a.relu_limit)
-              v = a.relu_limit;
-          }
-          const int64_t o = m * a.N + n;
-          if (a.acc_out)
-            a.acc_out[o] = v;
-          if constexpr (FMT == F8_FMT_E5M2) {
-            f8_store_e5m2(a, o, v);
-            continue;
-          }
-          // F8E4M3(v, step, true): the quotient in double, narrowed to fp32, rounded to E4M3 (Float8.cpp:259-261).
-          // v * (1 / step) is within two double ulps of that quotient, so the narrowing can come out differently
-          // only when the 29 bits it drops sit next to the halfway pattern; only then is the division carried out.
-          double qd = (double)v * inv_step;
-          const int32_t low = (int32_t)((uint32_t)__double_as_longlong(qd) & 0x1fffffffu);
-          if (low >= 0x10000000 - 4 && low <= 0x10000000 + 4)
-            qd = (double)v / step;
-          const uint32_t code = f8e4m3_from_f32((float)qd);
-          if (a.out_kind == MI_F8_OUT_CODES)
-            ((uint8_t *)a.out)[o] = (uint8_t)code;
-          else if (a.out_kind == MI_F8_OUT_F32)
-            ((float *)a.out)[o] = f8e4m3_to_f32(code);
-          else if (a.out_kind == MI_F8_OUT_BF16)  // exact: E4M3 values fit both 16-bit types
-            ((uint16_t *)a.out)[o] = (uint16_t)(__float_as_uint(f8e4m3_to_f32(code)) >> 16);
-          else
-            ((uint16_t *)a.out)[o] = __builtin_bit_cast(uint16_t, (_Float16)f8e4m3_to_f32(code));
-        }
+        if (n_ok && m < a.M)
+          f8_finish_one<FMT>(a, m * a.N + n, acc[i][j][r] + bias_n, step, inv_step);
       }
     }
   }
@@ -606,6 +613,112 @@ __global__ __launch_bounds__(256, 1) void f8_gemm_large_kernel(F8Args a, int til
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Few rows (M <= 32): a stream over the right operand, HBM-bound; the INT8 few-row kernel (i8_kernels.hip) on F8
+// codes.  A workgroup owns 32 output columns, its eight waves take the 128-byte K tiles round-robin (with the waves of
+// the block's other K parts, when K is split over workgroups), each multiplies all rows against its tiles, operands
+// straight from memory into MFMA fragments one tile ahead (a lane's 64 contiguous bytes of its row feed two K = 64
+// MFMAs; the K order inside a tile is permuted alike for both operands).  Partial sums are added in wave order, then in
+// part order: fp32 sums in another order than the tiled kernels', inside the same bound.  Requires K % 128 == 0.
+// ------------------------------------------------------------------------------------------------
+template <int FMT>
+__global__ __launch_bounds__(512) void f8_rows32_kernel(F8Args a) {
+  constexpr int WAVES = 8;
+  __shared__ float red[WAVES][16][64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c32 = lane & 31, h = lane >> 5;
+  const int parts = 1 << a.split_shift, part = blockIdx.x & (parts - 1);
+  const int64_t block = blockIdx.x >> a.split_shift;
+  const int64_t n = block * 32 + c32;
+  const int64_t nb = n < a.N ? n : a.N - 1;  // columns past N repeat the last one; never stored
+  const int64_t ma = c32 < a.M ? c32 : a.M - 1;
+  const uint8_t *pb = a.B + nb * a.K + h * 64;
+  const uint8_t *pa = a.A + ma * a.K + h * 64;
+  const int k_tiles = (int)(a.K / 128);
+  const int first = part * WAVES + wave, stride = WAVES << a.split_shift;
+  const int count = (k_tiles - first + stride - 1) / stride;
+
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    acc[r] = 0.0f;
+  u32x4 xa[2][4], xb[2][4];
+  auto load_tile = [&](int i, int slot) {
+    const int64_t off = (int64_t)(first + (i < count ? i : count - 1) * stride) * 128;  // past the end: a re-load
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      xb[slot][j] = *(const u32x4 *)(pb + off + j * 16);
+      xa[slot][j] = *(const u32x4 *)(pa + off + j * 16);
+    }
+  };
+  if (count > 0) {
+    load_tile(0, 0);
+    for (int t0 = 0; t0 < count; t0 += 2) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        if (t0 + u >= count)
+          break;
+        load_tile(t0 + u + 1, u ^ 1);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const u32x4 a0 = xa[u][2 * j], a1 = xa[u][2 * j + 1], b0 = xb[u][2 * j], b1 = xb[u][2 * j + 1];
+          const i32x8 fa = {(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
+          const i32x8 fb = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+          acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa, fb, acc, FMT, FMT, 0, 0, 0, 0);
+        }
+      }
+    }
+  }
+  // cross-wave sum, in wave order.  Register r of lane l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    red[wave][r][lane] = acc[r];
+  __syncthreads();
+  float sum[2] = {0.0f, 0.0f};
+#pragma unroll
+  for (int q = 0; q < 2; ++q)
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv)
+      sum[q] += red[wv][wave * 2 + q][lane];
+  if (a.split_shift != 0) {
+    // the block's other K parts: see i8_rows32_kernel (device-scope relaxed atomics ordered by waiting for them)
+    __shared__ int last_flag;
+    float *slab = a.part + block * parts * 1024;
+    const int idx = wave * 128 + lane;
+    __hip_atomic_store(slab + part * 1024 + idx, sum[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(slab + part * 1024 + idx + 64, sum[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(f8_waitcnt_vm(0));
+    __syncthreads();
+    if (tid == 0) {
+      const unsigned before = __hip_atomic_fetch_add(a.counters + block, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int last = before == (unsigned)(parts - 1);
+      if (last)
+        __hip_atomic_store(a.counters + block, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      last_flag = last;
+    }
+    __syncthreads();
+    if (!last_flag)
+      return;
+    sum[0] = sum[1] = 0.0f;
+    for (int p = 0; p < parts; ++p) {
+      sum[0] += __hip_atomic_load(slab + p * 1024 + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      sum[1] += __hip_atomic_load(slab + p * 1024 + idx + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  const bool n_ok = n < a.N;
+  const float bias_n = (a.bias && n_ok) ? a.bias[n] : 0.0f;
+  const double step = (a.scales && n_ok) ? 1.0 / a.scales[n] : a.step;
+  const double inv_step = 1.0 / step;
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int r = wave * 2 + q;
+    const int64_t m = 8 * (r >> 2) + 4 * h + (r & 3);
+    if (n_ok && m < a.M)
+      f8_finish_one<FMT>(a, m * a.N + n, sum[q] + bias_n, step, inv_step);
+  }
+}
+
 __global__ void f8_transpose_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t K, int64_t N) {
   // [K, N] -> [N, K], 32 x 32 tiles through LDS
   __shared__ uint8_t tile[32][33];
@@ -660,7 +773,38 @@ int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, con
   a.step = (double)(float)(1 / out_scale);  // MatMul.cpp:613-615 into the float parameter of Float8.cpp:267
   a.inv_step = (float)(1.0 / a.step);
   a.scales = d_out_scales;
+  a.split_shift = 0;
+  a.part = nullptr;
+  a.counters = nullptr;
   const bool e5m2 = f8_type == MI_F8_E5M2;
+  {  // up to 32 rows: the streaming kernel, by the INT8 product's rule (same bytes per element; plan: f8_tile = 32
+     // asks for it, any other value rules it out).  4096 x 4096 (N x K) M = 1: 15.2 us on 64 x 64 tiles, 4096 x 11008: 38.7
+    const bool few_pays = M * N <= 45056 || (N <= 8192 && (M <= 24 || K > 4096));
+    if (M <= 32 && (K % 128) == 0 && (plan().f8_tile == 32 || (plan().f8_tile == 0 && few_pays))) {
+      const int64_t blocks = (N + 31) / 32;
+      MI_REQUIRE(blocks < (1ll << 29), MI_BAD_ARGUMENT, "mi_f8mm_launch: too many output columns");
+      while (a.split_shift < 2 && (blocks << (a.split_shift + 1)) <= R32_SPLIT_MAX_WGS &&
+             K / 128 >= (32 << (a.split_shift + 1)))
+        ++a.split_shift;
+      if (a.split_shift != 0) {
+        void *p = nullptr;
+        if (stream_workspace(stream, WS_ROWS32_SPLIT, R32_SPLIT_COUNTER_BYTES + (size_t)R32_SPLIT_MAX_WGS * 4096, &p,
+                             /*zero_fresh=*/true) == MI_SUCCESS) {
+          a.counters = (unsigned *)p;
+          a.part = (float *)((uint8_t *)p + R32_SPLIT_COUNTER_BYTES);
+        } else {
+          a.split_shift = 0;  // no scratch (the stream is being captured before it ever had one)
+        }
+      }
+      const dim3 grid((unsigned)(blocks << a.split_shift));
+      if (e5m2)
+        f8_rows32_kernel<F8_FMT_E5M2><<<grid, dim3(512), 0, stream>>>(a);
+      else
+        f8_rows32_kernel<F8_FMT_E4M3><<<grid, dim3(512), 0, stream>>>(a);
+      MI_HIP(hipGetLastError());
+      return MI_SUCCESS;
+    }
+  }
   const int64_t tiles_m = (M + F8_BM - 1) / F8_BM, tiles_n = (N + F8_BN - 1) / F8_BN;
   if ((K % F8_BK) == 0 && tiles_m * tiles_n < (int64_t(1) << 30)) {
     const int tiles = (int)(tiles_m * tiles_n), per_xcd = (tiles + 7) / 8;

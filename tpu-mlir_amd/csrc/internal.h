@@ -25,7 +25,7 @@ typedef struct mi_internal_plan {
   int i8_mid_ring;                   // 4 / 8 (128-tiles), 64 (64-tiles)
   int i8_ring;                       // 3 / 4 / 5: LDS ring stages of the large kernel
   int dq_waves;                      // 8 / 16
-  int f8_tile;                       // 256 / 128 / 64
+  int f8_tile;                       // 256 / 128 / 64 / 32 (streaming kernel for up to 32 rows)
   int a16_decode_rows8;              // 1: five to eight rows always take the decode kernel where it can; -1: never
   int a16_rows32_min_m;              // > 0: sets it can handle take the 32-row kernel from this many rows (to 32); -1: never
   int a16_wide_min_m;                // > 0: 8-bit sets take the wide tiles from this many rows on; -1: never
