@@ -344,100 +344,6 @@ def bench_f16_prefill_forms(pkg, S, torch, clib, launches=10):
     return out
 
 
-def bench_bf16_prefill_two_term(pkg, S, torch, clib, launches=10):
-    """W4 g128 prefill on bf16 activations, 4096 x 4096: the exact kernel the library takes (per-group fp32 fold) beside
-    the other exact form, each weight as the sum of two bf16 numbers and two MFMAs per fragment on the wide tiles.  The
-    library never picks the second by itself; it is selected here through the library's internal planning hook (the one
-    the tests use), which is not part of the C ABI."""
-    import ctypes
-    names = ("a16_waves", "a16_tpw", "a16_rows", "a16_xlds", "a16_no_gemm", "a16_no_decode", "a16_gemm_min_m",
-             "a16_gemm_splits", "a16_gemm_tile", "a16_gemm_rows", "i8_tile", "i8_mid_ring", "i8_ring", "dq_waves", "f8_tile",
-             "a16_decode_rows8", "a16_rows32_min_m", "a16_wide_min_m", "a16_wide4_min_m", "a16_rows32_split")
-
-    class Plan(ctypes.Structure):
-        _fields_ = [(n, ctypes.c_int) for n in names]
-
-    hook = clib.lib().mi_internal_set_plan
-    hook.argtypes, hook.restype = [ctypes.c_void_p], None
-    K = N = 4096
-    cfg = S.w4a16(1, K, N, 128, seed=31)
-    w = pkg.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=K, N=N, weight_bits=4, q_group_size=128)
-    out = []
-    try:
-        for M in (2048, 4096):
-            x = torch.randn((M, K), device="cuda").to(torch.bfloat16)
-            y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
-            rec = {"M": M, "K": K, "N": N}
-            for label, mode in (("fold", -1), ("two_term", 1)):
-                p = Plan(a16_wide4_min_m=mode)
-                hook(ctypes.byref(p))
-                sec = _time_launches(torch, lambda: pkg.a16mm_launch(w, x, y), launches, warmup=2)
-                rec[label + "_us"] = round(sec * 1e6, 1)
-                rec[label + "_TFLOPs"] = round(2.0 * M * N * K / sec / 1e12, 1)
-            out.append(rec)
-    finally:
-        hook(None)
-        w.destroy()
-    return out
-
-
-def dispatch_sweep(pkg, S, torch, clib):
-    """The kernel the library picks by itself, timed beside the same launch with the 32-row kernel ruled out and forced
-    (through the internal planning hook), for 1 to 16 activation rows over a set of weight shapes: the table the row
-    thresholds of a16_rows32_applicable are read from.  Weights rotate through more than 256 MB; launches replay from
-    a HIP graph.  Prints one line per shape, 'M:default/without/forced' in us, '!' where the default is more than 7 %
-    behind the better of the other two."""
-    import ctypes
-    names = ("a16_waves", "a16_tpw", "a16_rows", "a16_xlds", "a16_no_gemm", "a16_no_decode", "a16_gemm_min_m",
-             "a16_gemm_splits", "a16_gemm_tile", "a16_gemm_rows", "i8_tile", "i8_mid_ring", "i8_ring", "dq_waves", "f8_tile",
-             "a16_decode_rows8", "a16_rows32_min_m", "a16_wide_min_m", "a16_wide4_min_m", "a16_rows32_split")
-
-    class Plan(ctypes.Structure):
-        _fields_ = [(n, ctypes.c_int) for n in names]
-
-    hook = clib.lib().mi_internal_set_plan
-    hook.argtypes, hook.restype = [ctypes.c_void_p], None
-    shapes = ((8192, 8192), (8192, 28672), (11008, 4096), (14336, 4096), (5120, 5120), (5120, 13824), (13824, 5120),
-              (6656, 6656), (4096, 14336), (4096, 4096), (4096, 11008), (8192, 1024), (2048, 6144), (3072, 3072),
-              (4096, 32000))
-    flagged = 0
-    try:
-        for bits in (4, 8):
-            for K, N in shapes:
-                g = 128 if bits == 4 else 0
-                cfg = S.w4a16(1, K, N, g, seed=31) if bits == 4 else S.w8a16(1, K, N, g, seed=31, signed=False)
-                copies = max(1, min(8, int(300e6 // (N * K * bits // 8)) + 1))
-                ws = [pkg.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=K, N=N, weight_bits=bits,
-                                    q_group_size=g) for _ in range(copies)]
-                cells = []
-                for M in (1, 2, 3, 4, 5, 6, 8, 10, 12, 16):
-                    x = torch.randn((M, K), device="cuda").to(torch.bfloat16)
-                    y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
-                    t = []
-                    for mode in (0, -1, 1):
-                        hook(ctypes.byref(Plan(a16_rows32_min_m=mode)))
-                        graph, stream = torch.cuda.CUDAGraph(), torch.cuda.Stream()
-                        with torch.cuda.stream(stream):
-                            for w in ws:
-                                pkg.a16mm_launch(w, x, y)
-                            stream.synchronize()
-                            with torch.cuda.graph(graph, stream=stream):
-                                for w in ws:
-                                    pkg.a16mm_launch(w, x, y)
-                        t.append(_time_launches(torch, graph.replay, 3) / copies * 1e6)
-                        del graph
-                    bad = t[0] > 1.07 * min(t[1], t[2])
-                    flagged += bad
-                    cells.append("%d:%.1f/%.1f/%.1f%s" % (M, t[0], t[1], t[2], "!" if bad else ""))
-                print("W%d K%d N%d blocks%d" % (bits, K, N, (N + 31) // 32), " ".join(cells), flush=True)
-                for w in ws:
-                    w.destroy()
-                torch.cuda.empty_cache()
-    finally:
-        hook(None)
-    print(json.dumps({"dispatch_sweep_cells_flagged": flagged}), flush=True)
-
-
 def bench_dynamic_quant(pkg, S, torch, steps=40):
     """tpu.A16MatMul with dynamic integer activation quantization (activation quantizer + integer product per call),
     weights rotating through HBM; launches replayed from a HIP graph."""
@@ -670,9 +576,6 @@ def main():
     ap.add_argument("--only-mfma", action="store_true",
                     help="run only the three MFMA-bound kernels (INT8 4096^3, W4A16 prefill M=2048, F8 4096^3), a few "
                          "launches each, and print their figures: the command for hardware-counter profiles")
-    ap.add_argument("--dispatch-sweep", action="store_true",
-                    help="time the library's own kernel choice for 1 to 16 rows over a set of weight shapes beside the "
-                         "alternatives, print the table and exit (a tuning aid, not a bench line)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; every GPU box of this run has one. Use --gpus 1.")
@@ -695,9 +598,6 @@ def main():
 
     if args.only_mfma:
         print(json.dumps({"only_mfma": bench_mfma_kernels(pkg, S, torch, clib)}), flush=True)
-        return
-    if args.dispatch_sweep:
-        dispatch_sweep(pkg, S, torch, clib)
         return
 
     M = args.batch
@@ -770,7 +670,6 @@ def main():
             ex["chain_M%d_GBps" % m] = round(rm["chain_bytes"] / (rm["gpu_s"] / 40) / 1e9, 1)
         ex["single_matmuls"] = bench_single_matmuls(pkg, S, torch)
         ex["prefill_f16_exact_vs_tolerance"] = bench_f16_prefill_forms(pkg, S, torch, clib)
-        ex["prefill_bf16_fold_vs_two_term"] = bench_bf16_prefill_two_term(pkg, S, torch, clib)
         ex["dynamic_quant"] = bench_dynamic_quant(pkg, S, torch)
         ex["int8_256x1024x1024"] = bench_int8(pkg, S, torch, clib, 1024, 40, 5, M=256, graph=True)
         ex["int8_1x4096x4096"] = bench_int8(pkg, S, torch, clib, 4096, 40, 5, M=1, graph=True)

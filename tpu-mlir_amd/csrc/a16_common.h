@@ -1,7 +1,7 @@
 // Shared by the A16MatMul kernels (skinny/decode and tiled/prefill): vector types, the traits of the two 16-bit float
 // types, and the in-register dequantization of packed weights.
 #pragma once
-#include "device_math.cuh"
+#include "device_math.h"
 #include "internal.h"
 
 namespace mi {

@@ -25,7 +25,7 @@
 // 8-bit  weights rounded to the 16-bit type exactly as the reference does, accumulated directly.
 #include <climits>
 
-#include "a16_common.cuh"
+#include "a16_common.h"
 #include "internal.h"
 
 namespace mi {

@@ -15,7 +15,7 @@
 #include <climits>
 #include <cstdint>
 
-#include "a16_common.cuh"
+#include "a16_common.h"
 #include "internal.h"
 
 namespace mi {

@@ -27,7 +27,7 @@
 
 #include <type_traits>
 
-#include "a16_common.cuh"
+#include "a16_common.h"
 #include "internal.h"
 
 namespace mi {

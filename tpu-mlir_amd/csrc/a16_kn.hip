@@ -9,7 +9,7 @@
 // K-slices per workgroup, partial sums joined through LDS.
 #include <vector>
 
-#include "a16_common.cuh"
+#include "a16_common.h"
 #include "internal.h"
 
 namespace mi {

@@ -10,7 +10,7 @@
 
 #include <vector>
 
-#include "a16_common.cuh"
+#include "a16_common.h"
 #include "internal.h"
 
 namespace mi {

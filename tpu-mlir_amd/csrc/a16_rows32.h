@@ -1,7 +1,7 @@
 // For the kernels for a few tens of activation rows (a16_rows32.hip): argument records, the 32 x 32 x 16 MFMA,
 // loads the compiler does not track (their arrival is covered by the kernels' own request counts), wait encodings.
 #pragma once
-#include "a16_common.cuh"
+#include "a16_common.h"
 #include "internal.h"
 
 namespace mi {

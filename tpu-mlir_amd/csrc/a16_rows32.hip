@@ -18,7 +18,7 @@
 //     acc += scale * (P - (16 + zp) * S) in fp32.
 #include <climits>
 
-#include "a16_rows32.cuh"
+#include "a16_rows32.h"
 
 namespace mi {
 

@@ -20,7 +20,7 @@
 // fragment per k-step (16 to 20 vector instructions against the four MFMAs, 128 matrix-pipe cycles, that share it).
 #include <climits>
 
-#include "a16_common.cuh"
+#include "a16_common.h"
 #include "internal.h"
 
 namespace mi {

@@ -2,7 +2,7 @@
 // (f32 / bf16 / f16 / int8 / uint8 / int16 / uint16 / int32), following lib/Dialect/Tpu/Interfaces/Common/Cast.cpp:38-200
 // with requant()/dequant() of lib/Support/CastUtils.cpp:15-46 (BM168x branches).  HBM-bound: one read and one write
 // per element, 16 elements per thread.
-#include "device_math.cuh"
+#include "device_math.h"
 #include "internal.h"
 
 namespace mi {

@@ -28,7 +28,7 @@
 //   F8E4M3  both operands widened to bf16 (exact) and multiplied on v_mfma_f32_16x16x32_bf16: the reference's group
 //           product is an f32 matmul whose summation order its library chooses, so parity is to fp32 rounding of the
 //           group sums; the fp8 instruction itself loses about 2^-14 of a sum to operand alignment and is not used.
-#include "a16_common.cuh"
+#include "a16_common.h"
 #include "internal.h"
 
 #include <type_traits>

@@ -18,7 +18,7 @@
 // no summation order either; tests bound the fp32 value and count the differing codes.
 #include <cstdlib>
 
-#include "device_math.cuh"
+#include "device_math.h"
 #include "internal.h"
 
 namespace mi {

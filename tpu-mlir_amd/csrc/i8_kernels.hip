@@ -8,7 +8,7 @@
 // and uint8 operands are re-biased to int8 (x ^ 0x80, zero point - 128) while they are staged into LDS.
 #include <stdlib.h>
 
-#include "device_math.cuh"
+#include "device_math.h"
 #include "internal.h"
 
 namespace mi {

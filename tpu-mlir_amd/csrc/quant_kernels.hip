@@ -7,7 +7,7 @@
 //                                                                    that both the reads and the writes coalesce
 // Every float operation is the reference's (same order, IEEE division and roundf, no contraction), so the codes, zero
 // points and scale bit patterns are identical to the CPU result.
-#include "device_math.cuh"
+#include "device_math.h"
 #include "internal.h"
 
 #pragma clang fp contract(off)
