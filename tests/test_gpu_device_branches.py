@@ -155,6 +155,36 @@ def test_q31_epilogue_at_the_ends_of_the_int32_range(orc, plan, tile):
     assert np.array_equal(out2.cpu().numpy().astype(np.int64), want2)
 
 
+def test_q31_short_form_at_its_accumulator_bound(orc, plan):
+    """The 256-tile kernel takes a short form of the Q31 / half-away epilogue when every bias is below 2^29 in
+    magnitude, K <= 32768 and the output zero point is zero: accumulators then stay below 2^30 and the rounding sum
+    fits int32.  This drives it to that bound: K = 32768 rows of -128 against -128 (2^29) plus a bias of 2^29 - 1, the
+    largest multiplier and right shifts up to 31, both signs; a bias of 2^29 in one column block must take the long
+    form and still be exact."""
+    import torch
+    plan(i8_tile=256)
+    M, K, N = 256, 32768, 512
+    a = np.full((M, K), -128, np.int8)
+    a[1::2] = 127                                                        # odd rows: large negative sums
+    b = np.full((N, K), -128, np.int8)
+    bias = np.where(np.arange(N) % 2 == 0, 2**29 - 1, -(2**29 - 1)).astype(np.int32)
+    bias[256:] = np.where(np.arange(256) % 2 == 0, 2**29, -2**29)      # second column tile: not small, long form
+    shift = (np.arange(N) % 31 + 1).astype(np.int32)
+    shift[:4] = 31
+    mult = np.full(N, 2**31 - 1, np.int32)
+    mult[5::7] = 1 << 30
+    rq = M_.RequantDesc(clib.RQ_QDM, clib.ROUND_HALF_AWAY_FROM_ZERO, out_dtype=clib.DT_I8, multiplier=_dev(mult),
+                        shift=_dev(shift))
+    out = M_.i8mm_launch(_dev(a), _dev(b), _dev(bias), right_transpose=True, rq=rq)
+    torch.cuda.synchronize()
+    acc = (a.astype(np.int64)[:, :1] * b.astype(np.int64)[:, :1].T) * K + bias.astype(np.int64)   # constant rows
+    assert acc.max() == 2**30 - 1 and np.abs(acc).max() < 2**31
+    acc = acc.astype(np.int32)
+    want = _sat(orc.mbqm(acc, np.broadcast_to(mult, acc.shape), np.broadcast_to(-shift, acc.shape),
+                         clib.ROUND_HALF_AWAY_FROM_ZERO).astype(np.int64), -128, 127)
+    assert np.array_equal(out.cpu().numpy().astype(np.int64), want)
+
+
 # f32 bit patterns that ordinary activations never produce, with the reference's bf16 (BM168x) and f16 answers written
 # out by hand from lib/Support/Float16.cpp (:524-526, :550-601, :626-627; f16: :652-714)
 SPECIAL_BITS = np.array([

@@ -288,13 +288,16 @@ __global__ __launch_bounds__(256) void i8_gemm_kernel(I8Args a) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Large-tile kernel: 256x256 outputs per workgroup, 4 waves (2x2), each wave 128x128 as 4x4 MFMA 32x32x32 blocks
-// (256 int32 accumulators per lane).  K advances 64 bytes per stage through a 4-stage LDS ring (32 KiB per stage)
-// that is filled by direct-to-LDS 16-byte loads: no staging registers and no LDS store instructions.  The 16-byte
-// chunks of a row are XOR-swizzled with (row >> 2) & 3 so that the fragment reads (32 consecutive rows, one
-// chunk) hit distinct banks.  Requires K % 64 == 0; rows past M/N are clamped (their results are never stored).
-// Workgroups are renumbered so that the 32 (or so) workgroups that land on one XCD cover a compact block of
-// output tiles and share their A/B panels through that XCD's L2.
+// Large-tile kernel: 256x256 outputs per workgroup, 8 waves (2 x 4, two per SIMD so that one wave's waits run under
+// the other's MFMAs), each wave 128 x 64 as 4 x 2 MFMA 32x32x32 blocks (128 int32 accumulators per lane).  K advances
+// 64 bytes per stage through a 5-stage LDS ring (32 KiB per stage, all 160 KiB) that is filled by direct-to-LDS
+// 16-byte loads: no staging registers and no LDS store instructions.  Two stages are requested together, the two
+// 64-byte halves of every 128-byte line back to back, so that the vector cache asks L2 for each line once (measured:
+// half-line requests a stage apart reach half the L2 bandwidth of whole lines).  The 16-byte chunks of a row are
+// XOR-swizzled with (row >> 2) & 3 so that the fragment reads (32 consecutive rows, one chunk) hit distinct banks.
+// Requires K % 128 == 0; rows past M/N are clamped (their results are never stored).  Workgroups are renumbered so
+// that the 32 (or so) workgroups that land on one XCD cover a compact block of output tiles and share their A/B
+// panels through that XCD's L2.
 // ------------------------------------------------------------------------------------------------
 constexpr int LM = 256, LN = 256;
 enum { EPI_INT32 = 0, EPI_Q31_HALF_AWAY = 1, EPI_GENERIC = 2 };
@@ -588,18 +591,19 @@ __global__ __launch_bounds__(256) void i8_gemm_mid_kernel(I8Args a, int tiles_m,
   }
 }
 
-// LK_ = bytes of K per stage (64 or 128), NST = stages in the LDS ring (NST * 512 * LK_ bytes)
-template <int EPI, int LK_, int NST>
-__global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int tiles_m, int tiles_n, int per_xcd) {
-  constexpr int CH = LK_ / 16;                // 16-byte chunks per row
-  constexpr int KS = LK_ / 32;                // MFMA k-steps per stage
-  constexpr int LOADS = LM * CH / 256;        // direct-to-LDS instructions per operand, stage and wave
-  constexpr int LPS = 2 * LOADS;              // loads per thread and stage
-  constexpr int STAGE_BYTES = (LM + LN) * LK_;
+constexpr int LARGE_LDS_BYTES = 5 * (LM + LN) * 64;  // the whole 160 KiB
+
+template <int EPI>
+__global__ __launch_bounds__(512, 1) void i8_gemm_large_kernel(I8Args a, int tiles_m, int tiles_n, int per_xcd) {
+  constexpr int LK = 64, CH = LK / 16, KS = LK / 32, NST = 5;
+  constexpr int LOADS = LM * CH / 512;  // direct-to-LDS instructions per operand, stage and wave
+  constexpr int LPS = 2 * LOADS;        // loads per thread and stage
+  constexpr int STAGE_BYTES = (LM + LN) * LK;
+  static_assert(NST * STAGE_BYTES == LARGE_LDS_BYTES, "ring size");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave >> 2, wn = wave & 3;
 
   // workgroup -> tile: hardware deals workgroups round-robin over the 8 XCDs; give each XCD a contiguous range of
   // the tile order, and order tiles in groups of 4 tile-rows (column-major inside a group)
@@ -616,51 +620,60 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
 
   // Row swizzle: the 16-byte chunk c of row r is stored at position c ^ sw(r) so that 16 consecutive rows reading
   // the same logical chunk touch 16 different 16-byte bank groups.
-  auto sw = [](int row) { return LK_ == 64 ? ((row >> 2) & 3) : ((row >> 1) & 7); };
+  auto sw = [](int row) { return (row >> 2) & 3; };
 
-  // direct-to-LDS load plan: instruction i of wave w fills slots [(i*4+w)*64, +64) of an operand's stage;
-  // slot s is row s / CH, position s % CH
-  const uint8_t *ga[LOADS], *gb[LOADS];
+  // direct-to-LDS load plan: instruction i of wave w fills slots [(i*8+w)*64, +64) of an operand's stage; slot s is
+  // row s / CH, position s % CH.  A lane's address is a uniform tile base plus a 32-bit offset (rows past the matrix
+  // re-read the last row; their results are never stored).
+  const uint8_t *Abase = a.A + m_base * a.K, *Bbase = a.B + n_base * a.K;
+  uint32_t va[LOADS], vb[LOADS];
 #pragma unroll
   for (int i = 0; i < LOADS; ++i) {
-    const int slot = (i * 4 + wave) * 64 + lane;
+    const int slot = (i * 8 + wave) * 64 + lane;
     const int row = slot / CH, pos = slot % CH;
     const int chunk = pos ^ sw(row);
     int64_t ra = m_base + row, rb = n_base + row;
-    ra = ra < a.M ? ra : a.M - 1;  // rows past the matrix re-read the last row; their results are never stored
+    ra = ra < a.M ? ra : a.M - 1;
     rb = rb < a.N ? rb : a.N - 1;
-    ga[i] = a.A + ra * a.K + chunk * 16;
-    gb[i] = a.B + rb * a.K + chunk * 16;
+    va[i] = (uint32_t)((ra - m_base) * a.K + chunk * 16);
+    vb[i] = (uint32_t)((rb - n_base) * a.K + chunk * 16);
   }
-  const int kt_total = (int)(a.K / LK_);
-  // A stage is requested in KS parts (one per MFMA batch) so that its direct-to-LDS instructions are spread over a
-  // whole stage's worth of MFMAs instead of queueing up behind one batch.
-  constexpr int PART = LOADS / KS;
-  static_assert(PART * KS == LOADS, "loads per operand must split evenly over the k-steps");
-  auto issue_part = [&](int kt, int part) {
-    const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 1) * LK_;  // past the end: harmless re-load
-    uint8_t *sa = lds + (kt % NST) * STAGE_BYTES, *sb = sa + LM * LK_;
+  const int kt_total = (int)(a.K / LK);
+  // Stages 2p and 2p+1 are requested together, one operand (half = 0: A, 1: B) per call: each line's first 64 bytes
+  // go to stage 2p's buffer and its second 64 bytes, with the very next instruction, to stage 2p+1's.
+  auto issue_pair = [&](int p, int half) {
+    const int kt = 2 * p;
+    const int64_t koff = (int64_t)(kt < kt_total ? kt : kt_total - 2) * LK;  // past the end: harmless re-load
+    uint8_t *s0 = lds + (kt % NST) * STAGE_BYTES + half * (LM * LK);
+    uint8_t *s1 = lds + ((kt + 1) % NST) * STAGE_BYTES + half * (LM * LK);
+    const uint8_t *pg = (half ? Bbase : Abase) + koff;
 #pragma unroll
-    for (int i = part * PART; i < (part + 1) * PART; ++i) {
-      __builtin_amdgcn_global_load_lds((gptr_t)(ga[i] + koff), (lptr_t)(sa + (i * 4 + wave) * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_t)(gb[i] + koff), (lptr_t)(sb + (i * 4 + wave) * 1024), 16, 0, 0);
+    for (int i = 0; i < LOADS; ++i) {
+      const uint32_t v = half ? vb[i] : va[i];
+      __builtin_amdgcn_global_load_lds((gptr_t)(pg + v), (lptr_t)(s0 + (i * 8 + wave) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(pg + v + LK), (lptr_t)(s1 + (i * 8 + wave) * 1024), 16, 0, 0);
     }
   };
 
-  i32x16 acc[4][4];
+  i32x16 acc[4][2];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         acc[i][j][r] = 0;
-  // The accumulators start from the per-column bias instead of zero, so the epilogue has no bias to add.  Lane l of block (i, j) holds column 32 j + l % 32, rows 8 (r/4) + 4 (l/32) + r % 4.
+  // The accumulators start from the per-column bias instead of zero, so the epilogue has no bias to add.  Lane l of
+  // block (i, j) holds column 32 j + l % 32, rows 8 (r/4) + 4 (l/32) + r % 4.
+  // small_bias: every bias of this wave's 64 columns is below 2^29 in magnitude; with K <= 32768 every accumulator
+  // then stays below 2^30, which the short form of the requantization relies on.
+  bool small_bias = true;
   if (a.bias) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int64_t n = n_base + wn * 128 + j * 32 + (lane & 31);
+    for (int j = 0; j < 2; ++j) {
+      const int64_t n = n_base + wn * 64 + j * 32 + (lane & 31);
       const int32_t b = a.bias[n < a.N ? n : a.N - 1];
+      small_bias = small_bias && (b > -(1 << 29)) && (b < (1 << 29));
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -671,106 +684,89 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
 
   // fragment addressing: lane reads row (lane & 31) of a 32-row block, logical chunk ks*2 + (lane >> 5)
   const int frow = lane & 31, fhalf = lane >> 5;
-  int a_off[4], b_off[4];  // byte offsets of the row inside a stage (without the chunk position)
-  int a_sw[4], b_sw[4];
+  int a_addr[4][KS], b_addr[2][KS];  // byte offsets inside a stage
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int ra = wm * 128 + i * 32 + frow, rb = wn * 128 + i * 32 + frow;
-    a_off[i] = ra * LK_;
-    b_off[i] = LM * LK_ + rb * LK_;
-    a_sw[i] = sw(ra);
-    b_sw[i] = sw(rb);
-  }
-
-  auto read_frags = [&](i32x4 (&fa)[4], i32x4 (&fb)[4], int kt, int ks) {
-    const uint8_t *st = lds + (kt % NST) * STAGE_BYTES;
+  for (int ks = 0; ks < KS; ++ks) {
     const int c = ks * 2 + fhalf;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      fa[i] = *(const i32x4 *)(st + a_off[i] + ((c ^ a_sw[i]) << 4));
-      fb[i] = *(const i32x4 *)(st + b_off[i] + ((c ^ b_sw[i]) << 4));
+      const int ra = wm * 128 + i * 32 + frow;
+      a_addr[i][ks] = ra * LK + ((c ^ sw(ra)) << 4);
     }
-  };
-  // One batch: the 16 MFMAs of k-step `cur` with, pinned between them in this order, the 8 fragment reads of the
-  // next k-step (in the order the next batch consumes them) and one part of a future stage's loads.  The explicit
-  // scheduling barriers keep the compiler from clumping the memory instructions at the head of the batch, where
-  // they would hold up MFMA issue.
-  auto batch = [&](const i32x4 (&ca)[4], const i32x4 (&cb)[4], i32x4 (&na)[4], i32x4 (&nb)[4], int rkt, int rks,
-                   int lkt, int lpart) {
-    const uint8_t *st = lds + (rkt % NST) * STAGE_BYTES;
-    const int c = rks * 2 + fhalf;
-    const int64_t koff = (int64_t)(lkt < kt_total ? lkt : kt_total - 1) * LK_;  // past the end: harmless re-load
-    uint8_t *sa = lds + (lkt % NST) * STAGE_BYTES, *sb = sa + LM * LK_;
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      const int i = t >> 2, j = t & 3;
+    for (int j = 0; j < 2; ++j) {
+      const int rb = wn * 64 + j * 32 + frow;
+      b_addr[j][ks] = LM * LK + rb * LK + ((c ^ sw(rb)) << 4);
+    }
+  }
+  // One batch: the 8 MFMAs of one k-step with, pinned between them, the 6 fragment reads of the next k-step (in the
+  // order the next batch consumes them) and, in two batches of four, one operand's requests for a future pair of
+  // stages.  The scheduling barriers keep the compiler from clumping the memory instructions at the head of the batch.
+  auto batch = [&](const i32x4 (&ca)[4], const i32x4 (&cb)[2], i32x4 (&na)[4], i32x4 (&nb)[2], int rkt, int rks,
+                   int lpair, int lhalf) {
+    const uint8_t *st = lds + (rkt % NST) * STAGE_BYTES;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const int i = t >> 1, j = t & 1;
       acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ca[i], cb[j], acc[i][j], 0, 0, 0);
       if (t == 0)
-        na[0] = *(const i32x4 *)(st + a_off[0] + ((c ^ a_sw[0]) << 4));
-      else if (t <= 4)
-        nb[t - 1] = *(const i32x4 *)(st + b_off[t - 1] + ((c ^ b_sw[t - 1]) << 4));
-      else if (t <= 7)
-        na[t - 4] = *(const i32x4 *)(st + a_off[t - 4] + ((c ^ a_sw[t - 4]) << 4));
-      if (t >= 8) {
-        constexpr int SLOTS = 8, N_LD = 2 * PART;  // loads of this part, spread over the last 8 MFMAs
-        const int q0 = (t - 8) * N_LD / SLOTS, q1 = (t - 7) * N_LD / SLOTS;
-#pragma unroll
-        for (int q = q0; q < q1; ++q) {
-          const int li = lpart * PART + (q >> 1);
-          if (q & 1)
-            __builtin_amdgcn_global_load_lds((gptr_t)(gb[li] + koff), (lptr_t)(sb + (li * 4 + wave) * 1024), 16, 0,
-                                             0);
-          else
-            __builtin_amdgcn_global_load_lds((gptr_t)(ga[li] + koff), (lptr_t)(sa + (li * 4 + wave) * 1024), 16, 0,
-                                             0);
-        }
-      }
+        na[0] = *(const i32x4 *)(st + a_addr[0][rks]);
+      else if (t == 1)
+        nb[0] = *(const i32x4 *)(st + b_addr[0][rks]);
+      else if (t == 2)
+        nb[1] = *(const i32x4 *)(st + b_addr[1][rks]);
+      else if (t <= 5)
+        na[t - 2] = *(const i32x4 *)(st + a_addr[t - 2][rks]);
+      if (t == 6 && lhalf >= 0)
+        issue_pair(lpair, lhalf);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // Software pipeline.  Stage s lives in ring buffer s % NST.  Each batch of 16 MFMAs (one k-step) runs with the
-  // next batch's fragment reads in flight (two fragment register sets alternate) and with one part of a future
-  // stage's loads slotted between its MFMAs.  The one barrier per stage sits before the LAST batch of stage kt: by
-  // then every wave has received that stage's last fragments (lgkmcnt(0)) and its own share of stage kt+1 (vmcnt),
-  // so after the barrier buffer kt % NST is free and stage kt+1 is complete.  Stage kt+NST is then requested in
-  // parts: part 0 in this last batch, parts 1.. in the first KS-1 batches of stage kt+1; it is needed NST-2 full
-  // stages after its last part went out.  A bare s_barrier is used: __syncthreads() carries a fence that would
-  // drain every outstanding load (vmcnt(0)).
-  static_assert(NST >= 3, "the spread-out stage requests need two stages of slack");
-#pragma unroll
-  for (int s = 0; s < NST - 1; ++s)
-#pragma unroll
-    for (int part = 0; part < KS; ++part)
-      issue_part(s, part);
-  issue_part(NST - 1, 0);
-  i32x4 fa[2][4], fb[2][4];
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm((NST - 2) * LPS + 2 * PART));  // stage 0 landed
+  // Software pipeline.  Stage s lives in ring buffer s % 5.  Each batch runs with the next batch's fragment reads in
+  // flight (two fragment register sets alternate).  One barrier per stage, before the stage's LAST batch: by then
+  // every wave has received that stage's last fragments (lgkmcnt(0)) and its own share of the next stage (vmcnt), so
+  // after the barrier the stage's buffer is free and the next stage is complete.  The pair of stages (2p+4, 2p+5)
+  // takes the buffers of stages 2p-1 and 2p, both free after the barrier of stage 2p: it is requested in the two
+  // batches that follow that barrier and is needed two and a half stages later.  A bare s_barrier is used:
+  // __syncthreads() carries a fence that would drain every outstanding load (vmcnt(0)).
+  issue_pair(0, 0);
+  issue_pair(0, 1);
+  issue_pair(1, 0);
+  issue_pair(1, 1);
+  i32x4 fa[2][4], fb[2][2];
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * LPS));  // stages 0 and 1 landed
   __builtin_amdgcn_s_barrier();
-  read_frags(fa[0], fb[0], 0, 0);
-  for (int kt = 0; kt < kt_total; ++kt) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      if (ks + 1 < KS) {
-        batch(fa[ks & 1], fb[ks & 1], fa[(ks + 1) & 1], fb[(ks + 1) & 1], kt, ks + 1, kt + NST - 1, ks + 1);
-      } else {
-        __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm((NST - 2) * LPS));  // this thread's share of stage kt+1 landed
-        __builtin_amdgcn_s_barrier();
-        batch(fa[ks & 1], fb[ks & 1], fa[(ks + 1) & 1], fb[(ks + 1) & 1], kt + 1, 0, kt + NST, 0);
-      }
-    }
+  for (int i = 0; i < 4; ++i)
+    fa[0][i] = *(const i32x4 *)(lds + a_addr[i][0]);
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+    fb[0][j] = *(const i32x4 *)(lds + b_addr[j][0]);
+  const int pairs = kt_total / 2;
+  for (int p = 0; p < pairs; ++p) {
+    batch(fa[0], fb[0], fa[1], fb[1], 2 * p, 1, 0, -1);
+    __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * LPS));  // everything but the newest pair of stages
+    __builtin_amdgcn_s_barrier();
+    batch(fa[1], fb[1], fa[0], fb[0], 2 * p + 1, 0, p + 2, 0);
+    batch(fa[0], fb[0], fa[1], fb[1], 2 * p + 1, 1, p + 2, 1);
+    __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * LPS));
+    __builtin_amdgcn_s_barrier();
+    batch(fa[1], fb[1], fa[0], fb[0], 2 * p + 2, 0, 0, -1);
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // drain the re-loads issued past the end before the workgroup may exit
 
   // Epilogue.  Register r of lane l in block (i, j) is row 8*(r/4) + 4*(l/32) + (r%4), column l%32 -- a layout
-  // that would store 32-byte row fragments.  Each wave instead passes one 32 x 128 strip at a time through its own
-  // LDS region (row stride 132 dwords) and re-reads it so that a lane owns 16 consecutive columns of a row: the
+  // that would store 32-byte row fragments.  Each wave instead passes one 32 x 64 strip at a time through its own
+  // LDS region (row stride 68 dwords) and re-reads it so that a lane owns 16 consecutive columns of a row: the
   // per-column requant parameters are then loaded once per lane and the int8 result leaves as 16-byte stores.
   __syncthreads();  // every wave is done with the stage buffers
-  int32_t *strip = reinterpret_cast<int32_t *>(lds) + wave * (32 * 132);
-  const int cc = lane & 7, rsub = lane >> 3;  // column chunk (16 columns) and row within a group of 8 rows
-  const int64_t n0 = n_base + wn * 128 + cc * 16;
+  constexpr int SS = 68;
+  int32_t *strip = reinterpret_cast<int32_t *>(lds) + wave * (32 * SS);
+  const int cc = lane & 3, rsub = lane >> 2;  // column chunk (16 columns) and row within a group of 16 rows
+  const int64_t n0 = n_base + wn * 64 + cc * 16;
   const bool vec_ok = (a.N % 16) == 0 && n0 + 16 <= a.N;
   // relu (and its optional upper limit) is one clamp, applied only when asked for
   const int32_t relu_hi = (a.relu_limit > 0 && a.relu_limit < INT32_MAX) ? (int32_t)a.relu_limit : INT32_MAX;
@@ -785,26 +781,66 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
       p_zp[e] = (a.rq.zp ? a.rq.zp[n] : a.rq.zp_s) + 128;  // +128: saturate as unsigned, flip the sign bits after
     }
   }
+  // The short form of the Q31 requantization: with every accumulator below 2^30 in magnitude (small biases, K up to
+  // 32768, no per-row term) t = round(x * mult / 2^31) is below 2^30 too and t + 2^(s-1) - (t < 0) cannot leave
+  // int32, so the rounding shift is an add and an arithmetic shift; with a zero output zero point the saturation is
+  // one clamp and the bytes are picked by two permutes.  The workgroup-uniform conditions are tested here, the
+  // bias one per wave.
+  const bool short_form = EPI == EPI_Q31_HALF_AWAY && !a.row_term && !a.do_relu && !a.acc_out && a.K <= 32768 &&
+                          !a.rq.zp && a.rq.zp_s == 0 && __builtin_amdgcn_ballot_w64(!small_bias) == 0;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
-        strip[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * 132 + j * 32 + (lane & 31)] = acc[i][j][r];
+        strip[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * SS + j * 32 + (lane & 31)] = acc[i][j][r];
     // same-wave LDS traffic is ordered; the compiler waits on lgkmcnt before the reads below
 #pragma unroll 1
-    for (int it = 0; it < 4; ++it) {  // kept rolled: unrolling it spills registers
-      const int row = it * 8 + rsub;
+    for (int it = 0; it < 2; ++it) {  // kept rolled: unrolling it spills registers
+      const int row = it * 16 + rsub;
       const int64_t m = m_base + wm * 128 + i * 32 + row;
       int32_t v[16];
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
-        const i32x4 t = *(const i32x4 *)(strip + row * 132 + cc * 16 + q4 * 4);
+        const i32x4 t = *(const i32x4 *)(strip + row * SS + cc * 16 + q4 * 4);
         v[q4 * 4 + 0] = t[0];
         v[q4 * 4 + 1] = t[1];
         v[q4 * 4 + 2] = t[2];
         v[q4 * 4 + 3] = t[3];
+      }
+      const bool live = m < a.M && n0 < a.N;
+      const int64_t o = m * a.N + n0;
+      if constexpr (EPI == EPI_Q31_HALF_AWAY) {
+        if (short_form) {
+          uint32_t packed[4];
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            int32_t q[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const int e = q4 * 4 + u;
+              const int64_t p = (int64_t)v[e] * (int64_t)p_mult[e] + (1ll << 30);
+              const int32_t t = (int32_t)(p >> 31);
+              q[u] = med3_i32((t + p_half[e] + (t >> 31)) >> p_shift[e], -128, 127);
+            }
+            // low bytes of the four clamped values
+            const uint32_t lo = __builtin_amdgcn_perm((uint32_t)q[1], (uint32_t)q[0], 0x0c0c0400u);
+            const uint32_t hi = __builtin_amdgcn_perm((uint32_t)q[3], (uint32_t)q[2], 0x04000c0cu);
+            packed[q4] = lo | hi;
+          }
+          if (live) {
+            int8_t *out = (int8_t *)a.out;
+            if (vec_ok) {
+              *(u32x4 *)(out + o) = u32x4{packed[0], packed[1], packed[2], packed[3]};
+            } else {
+              for (int e = 0; e < 16; ++e)
+                if (n0 + e < a.N)
+                  out[o + e] = (int8_t)((packed[e >> 2] >> (8 * (e & 3))) & 0xff);
+            }
+          }
+          continue;
+        }
       }
       if (a.row_term) {  // per-row term of a nonzero right zero point
         const int32_t rt = a.row_term[m < a.M ? m : a.M - 1];
@@ -817,8 +853,6 @@ __global__ __launch_bounds__(256, 1) void i8_gemm_large_kernel(I8Args a, int til
         for (int e = 0; e < 16; ++e)
           v[e] = med3_i32(v[e], 0, relu_hi);
       }
-      const bool live = m < a.M && n0 < a.N;
-      const int64_t o = m * a.N + n0;
       if (a.acc_out && live) {
         if (vec_ok) {
 #pragma unroll
@@ -1179,23 +1213,12 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
   } else if (large) {
     const int tiles_m = (int)((M + LM - 1) / LM), tiles_n = (int)((N + LN - 1) / LN);
     const int per_xcd = (tiles_m * tiles_n + 7) / 8;
-    const int ring = plan().i8_ring ? plan().i8_ring : 4;
-    const size_t lds_bytes = (size_t)(ring == 5 ? 5 : ring == 3 ? 3 : 4) * 32 * 1024;
     dim3 grid((unsigned)(per_xcd * 8));
-#define MI_LARGE_I(E, LK_, NST)                                                                             \
-  {                                                                                                         \
-    static LdsLimitOnce lds_limit;                                                                          \
-    lds_limit.ensure((const void *)i8_gemm_large_kernel<E, LK_, NST>, 160 * 1024);                          \
-    i8_gemm_large_kernel<E, LK_, NST><<<grid, dim3(256), lds_bytes, stream>>>(a, tiles_m, tiles_n, per_xcd);\
-  }
-#define MI_LARGE(E)         \
-  {                         \
-    if (ring == 5)          \
-      MI_LARGE_I(E, 64, 5)  \
-    else if (ring == 3)     \
-      MI_LARGE_I(E, 64, 3)  \
-    else                    \
-      MI_LARGE_I(E, 64, 4)  \
+#define MI_LARGE(E)                                                                                                \
+  {                                                                                                                \
+    static LdsLimitOnce lds_limit;                                                                                 \
+    lds_limit.ensure((const void *)i8_gemm_large_kernel<E>, LARGE_LDS_BYTES);                                      \
+    i8_gemm_large_kernel<E><<<grid, dim3(512), LARGE_LDS_BYTES, stream>>>(a, tiles_m, tiles_n, per_xcd);           \
   }
     if (epi == EPI_INT32)
       MI_LARGE(EPI_INT32)
@@ -1203,7 +1226,6 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
       MI_LARGE(EPI_Q31_HALF_AWAY)
     else
       MI_LARGE(EPI_GENERIC)
-#undef MI_LARGE_I
 #undef MI_LARGE
   } else if (few) {
     const int64_t blocks = (N + 31) / 32;

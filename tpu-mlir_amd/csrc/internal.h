@@ -23,7 +23,7 @@ typedef struct mi_internal_plan {
   int a16_gemm_rows;                 // 16 / 32 / 64 / 128: rows per output block
   int i8_tile;                       // 256 / 128 / 32 (streaming kernel for up to 32 rows) / -1 (register-staged kernel)
   int i8_mid_ring;                   // 4 / 8 (128-tiles), 64 (64-tiles)
-  int i8_ring;                       // 3 / 4 / 5: LDS ring stages of the large kernel
+  int i8_ring;                       // not read any more (the large kernel has one ring form); kept so that the record keeps its layout
   int dq_waves;                      // 8 / 16
   int f8_tile;                       // 256 / 128 / 64 / 32 (streaming kernel for up to 32 rows)
   int a16_decode_rows8;              // 1: five to eight rows always take the decode kernel where it can; -1: never
