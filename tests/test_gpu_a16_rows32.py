@@ -208,7 +208,9 @@ def test_k_split_launch_replays_from_a_graph(orc):
 
 def test_k_split_launch_captured_before_any_eager_run(orc):
     """A stream that is captured into a graph before it ever ran a K-split launch has no scratch buffer, and none can
-    be allocated during capture: the launch then goes out unsplit, and the replay is still right."""
+    be allocated during capture.  Whether a launch is split depends on its shape alone (an unsplit launch adds the
+    partial sums in another order), so the capture is refused with an error, as the tiled kernel's K split refuses it;
+    after one eager run on the stream the same capture works and replays the eager bits."""
     import torch
     M, K, N, g = 24, 11008, 1024, 128
     cfg = S.w4a16(M, K, N, g, seed=6)
@@ -216,7 +218,16 @@ def test_k_split_launch_captured_before_any_eager_run(orc):
     st = torch.cuda.Stream()
     x = torch.from_numpy(cfg["x"].view(np.int16)).cuda().view(torch.bfloat16)
     y_graph = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    y_eager = torch.empty_like(y_graph)
     torch.cuda.synchronize()
+    refused = torch.cuda.CUDAGraph()
+    with pytest.raises(clib.BackendError) as err:
+        with torch.cuda.graph(refused, stream=st):
+            M_.a16mm_launch(w, x, y=y_graph, stream=st)
+    assert "eagerly" in str(err.value)
+    torch.cuda.synchronize()
+    M_.a16mm_launch(w, x, y=y_eager, stream=st)
+    st.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=st):
         M_.a16mm_launch(w, x, y=y_graph, stream=st)
@@ -224,6 +235,7 @@ def test_k_split_launch_captured_before_any_eager_run(orc):
         y_graph.zero_()
         graph.replay()
         torch.cuda.synchronize()
+        assert torch.equal(y_graph.view(torch.int16), y_eager.view(torch.int16))
     x32, wq, scale, zp, _ = f32_valued_a16(cfg)
     want, _ = orc.a16matmul(x32, wq, scale, zp, None, M=M, K=K, N=N, weight_bits=4, q_group_size=g,
                             out_dtype=orc.OUT_BF16, gemm_kind=orc.GEMM_F64ACC)

@@ -1,6 +1,14 @@
-"""mi_a16mm_launch_noalloc: the launch that allocates nothing must give exactly what mi_a16mm_launch gives.
+"""mi_a16mm_launch_noalloc: the launch that allocates nothing must give exactly what mi_a16mm_launch gives, and must
+really allocate nothing.
+
+"Allocates nothing" is checked three ways, none of which looks at torch's own allocator (which the library does not
+use): the library's count of scratch-buffer allocations does not move, the device's free memory (hipMemGetInfo) does
+not shrink, and the K-split shapes run on a fresh stream that never sees the allocating entry point (so no scratch
+buffer exists for it) -- eagerly and captured into a HIP graph, where an allocation is impossible.
 
 Collected last on purpose (the file name sorts after every other test file)."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -17,57 +25,118 @@ def _bf16(torch, a):
     return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda().view(torch.bfloat16)
 
 
-def test_no_alloc_launch_matches_the_allocating_one(plan):
-    """Two calls in a row through the C ABI, the second with a smaller input: a K-split tiled launch whose partial
-    sums sit in the library's fixed scratch array (M = 96, then M = 40 which leaves most of the first call's slabs
-    behind in it), against mi_a16mm_launch on the same operands -- bit for bit, 16-bit outputs and the fp32 side
-    output.  Then the paths that need no scratch at all (decode, M = 1) and the refusal of a product whose slabs
-    exceed the array."""
+def _allocations():
+    fn = clib.lib().mi_internal_workspace_allocations
+    fn.restype = ctypes.c_long
+    return fn()
+
+
+class _NothingAllocated:
+    """with _NothingAllocated(torch): the library's scratch allocations and the device's free memory stay put."""
+
+    def __init__(self, torch):
+        self.torch = torch
+
+    def __enter__(self):
+        self.torch.cuda.synchronize()
+        self.count = _allocations()
+        self.free = self.torch.cuda.mem_get_info()[0]
+
+    def __exit__(self, *exc):
+        self.torch.cuda.synchronize()
+        if exc[0] is None:
+            assert _allocations() == self.count, "the library allocated a scratch buffer"
+            assert self.torch.cuda.mem_get_info()[0] >= self.free, "device memory was taken during the call"
+        return False
+
+
+def _weights(K, N, g, rows, seed):
+    cfg = S.w4a16(rows, K, N, g, seed=seed, bias=True)
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], S.bf16_to_f32(cfg["bias"]), K=K, N=N, weight_bits=4,
+                     q_group_size=g)
+    return cfg, w
+
+
+@pytest.mark.parametrize("K,N,g,row_counts,seed", [
+    (4096, 1024, 128, (96, 40, 1), 31),    # tiled kernel with K split (M = 96, then M = 40 over the first call's slabs), decode
+    (8192, 1024, 128, (32, 20, 32), 33),   # the 32-row kernel's K split: partial blocks and arrival counters
+])
+def test_no_alloc_launch_matches_the_allocating_one(K, N, g, row_counts, seed):
+    """The no-alloc entry point runs on a fresh stream that never sees the allocating one (no scratch buffer of the
+    library exists for that stream, so a call that secretly used one would have to allocate it, which the guard
+    sees); the allocating entry point runs on the default stream and both are compared bit for bit, 16-bit outputs and
+    the fp32 side output.  The second call of each pair has fewer rows, so it runs over what the first left in the
+    fixed array."""
     import torch
-    K, N, g = 4096, 1024, 128
-    cfg = S.w4a16(96, K, N, g, seed=31, bias=True)
-    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], S.bf16_to_f32(cfg["bias"]), K=K, N=N, weight_bits=4,
-                     q_group_size=g)
+    cfg, w = _weights(K, N, g, max(row_counts), seed)
     x_all = _bf16(torch, cfg["x"])
-    for rows in (96, 40, 1):
+    fresh = torch.cuda.Stream()
+    with torch.cuda.stream(fresh):             # the runtime's own first-use set-up of a stream is not the library's
+        torch.zeros(16, device="cuda").add_(1)
+    for rows in row_counts:
         x = x_all[:rows].contiguous()
         y_ref = torch.empty((rows, N), dtype=torch.bfloat16, device="cuda")
         f_ref = torch.empty((rows, N), dtype=torch.float32, device="cuda")
         y_new, f_new = torch.empty_like(y_ref), torch.empty_like(f_ref)
+        # the allocating entry point on the default stream first: the kernels' code is on the device afterwards, and
+        # the scratch buffer it makes belongs to THAT stream, not to the fresh one
         M_.a16mm_launch(w, x, y=y_ref, y_f32=f_ref)
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated()
-        M_.a16mm_launch(w, x, y=y_new, y_f32=f_new, no_alloc=True)
+        with _NothingAllocated(torch):
+            with torch.cuda.stream(fresh):
+                M_.a16mm_launch(w, x, y=y_new, y_f32=f_new, no_alloc=True)
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
         assert torch.equal(y_new.view(torch.int16), y_ref.view(torch.int16)), rows
         assert torch.equal(f_new.view(torch.int32), f_ref.view(torch.int32)), rows
         assert float(f_ref.abs().max()) > 0
     w.destroy()
-    # the 32-row kernel's K split (long K, few channels): partial blocks and arrival counters in the same array
-    K, N, g = 8192, 1024, 128
-    cfg = S.w4a16(32, K, N, g, seed=33, bias=True)
-    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], S.bf16_to_f32(cfg["bias"]), K=K, N=N, weight_bits=4,
-                     q_group_size=g)
-    x_all = _bf16(torch, cfg["x"])
-    for rows in (32, 20, 32):
-        x = x_all[:rows].contiguous()
-        y_ref = torch.empty((rows, N), dtype=torch.bfloat16, device="cuda")
-        f_ref = torch.empty((rows, N), dtype=torch.float32, device="cuda")
-        y_new, f_new = torch.empty_like(y_ref), torch.empty_like(f_ref)
-        M_.a16mm_launch(w, x, y=y_ref, y_f32=f_ref)
+
+
+def test_no_alloc_launch_under_graph_capture_on_a_fresh_stream():
+    """A K-split launch captured into a HIP graph on a stream that never ran anything: the allocating entry point has
+    to refuse (its scratch buffer would have to be allocated during capture), the no-alloc one is captured, and every
+    replay -- with eager work of the same library in between -- gives the eager result bit for bit."""
+    import torch
+    K, N, g, rows = 4096, 1024, 128, 96
+    cfg, w = _weights(K, N, g, rows, 35)
+    x = _bf16(torch, cfg["x"])
+    y_ref = torch.empty((rows, N), dtype=torch.bfloat16, device="cuda")
+    f_ref = torch.empty((rows, N), dtype=torch.float32, device="cuda")
+    M_.a16mm_launch(w, x, y=y_ref, y_f32=f_ref)
+    torch.cuda.synchronize()
+    y_cap, f_cap = torch.zeros_like(y_ref), torch.zeros_like(f_ref)
+
+    refused = torch.cuda.Stream()
+    g0 = torch.cuda.CUDAGraph()
+    with pytest.raises(clib.BackendError):
+        with torch.cuda.graph(g0, stream=refused):
+            M_.a16mm_launch(w, x, y=y_cap, y_f32=f_cap)
+    torch.cuda.synchronize()
+
+    fresh = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with _NothingAllocated(torch):
+        with torch.cuda.graph(graph, stream=fresh):
+            M_.a16mm_launch(w, x, y=y_cap, y_f32=f_cap, no_alloc=True)
+    other = torch.empty_like(y_ref)
+    for replay in range(3):
+        y_cap.zero_()
+        f_cap.zero_()
+        with _NothingAllocated(torch):
+            graph.replay()
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated()
-        M_.a16mm_launch(w, x, y=y_new, y_f32=f_new, no_alloc=True)
+        assert torch.equal(y_cap.view(torch.int16), y_ref.view(torch.int16)), replay
+        assert torch.equal(f_cap.view(torch.int32), f_ref.view(torch.int32)), replay
+        M_.a16mm_launch(w, x[:40].contiguous(), y=other[:40])   # eager work between the replays
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
-        assert torch.equal(y_new.view(torch.int16), y_ref.view(torch.int16)), rows
-        assert torch.equal(f_new.view(torch.int32), f_ref.view(torch.int32)), rows
-        assert float(f_ref.abs().max()) > 0
     w.destroy()
-    # slabs beyond the fixed array are refused with a message that says so: M = 640, N = 4096 split four ways along K
-    # needs 40 MiB (the split count is pinned through the library's internal plan so that the case does not depend
-    # on the heuristics)
+
+
+def test_no_alloc_launch_refuses_what_does_not_fit(plan):
+    """Slabs beyond the fixed array are refused with a message that says so: M = 640, N = 4096 split four ways along K
+    needs 40 MiB (the split count is pinned through the library's internal plan so that the case does not depend on
+    the heuristics)."""
+    import torch
     plan(a16_gemm_splits=4)
     cfg = S.w4a16(1, 4096, 4096, 128, seed=32)
     wb = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=4096, N=4096, weight_bits=4, q_group_size=128)

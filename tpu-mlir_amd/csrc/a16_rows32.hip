@@ -452,11 +452,12 @@ static int rows32_split_scratch(hipStream_t stream, int shift, const A16Scratch 
     return MI_SUCCESS;
   }
   void *p = nullptr;
+  // Whether a launch is split is a function of its shape alone (the partial sums of a split launch are added in another
+  // order than an unsplit one's): a stream that is being captured before it ever ran such a shape gets the error, as
+  // from the tiled kernel's K split, not a differently rounded result.
   const int rc = stream_workspace(stream, WS_ROWS32_SPLIT, R32_SPLIT_COUNTER_BYTES + part_bytes, &p, /*zero_fresh=*/true);
-  if (rc != MI_SUCCESS) {  // no scratch (the stream is being captured before it ever had one): one workgroup per block
-    out->shift = 0;
-    return MI_SUCCESS;
-  }
+  if (rc != MI_SUCCESS)
+    return rc;
   out->counters = (unsigned *)p;
   out->part = (float *)((uint8_t *)p + R32_SPLIT_COUNTER_BYTES);
   return MI_SUCCESS;

@@ -8,14 +8,20 @@
 #include <string>
 #include <vector>
 
+#include <atomic>
+
 #include "internal.h"
 
 namespace mi {
 
 static thread_local std::string g_last_error;
-static mi_internal_plan g_plan = {};
+// The override record is published as a pointer to an immutable copy, so a launch on one thread reads either the old
+// record or the new one, never a mixture.  Superseded copies are not freed (a launch may still be reading one); the hook
+// is a test and tuning aid, called a handful of times per process.
+static const mi_internal_plan g_no_plan = {};
+static std::atomic<const mi_internal_plan *> g_plan{&g_no_plan};
 
-const mi_internal_plan &plan() { return g_plan; }
+const mi_internal_plan &plan() { return *g_plan.load(std::memory_order_acquire); }
 
 void set_error(const std::string &msg) { g_last_error = msg; }
 
@@ -167,7 +173,10 @@ using namespace mi;
 
 extern "C" {
 
-void mi_internal_set_plan(const mi_internal_plan *p) { g_plan = p ? *p : mi_internal_plan{}; }
+void mi_internal_set_plan(const mi_internal_plan *p) {
+  g_plan.store(p ? new mi_internal_plan(*p) : &g_no_plan, std::memory_order_release);
+}
+long mi_internal_workspace_allocations(void) { return mi::workspace_allocations(); }
 
 const char *mi_version(void) { return "tpumlir_amd 0.1 (gfx950)"; }
 const char *mi_last_error(void) { return g_last_error.c_str(); }

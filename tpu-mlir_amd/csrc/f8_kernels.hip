@@ -788,13 +788,14 @@ int f8mm_launch(const uint8_t *d_a, const uint8_t *d_b, int right_transpose, con
         ++a.split_shift;
       if (a.split_shift != 0) {
         void *p = nullptr;
-        if (stream_workspace(stream, WS_ROWS32_SPLIT, R32_SPLIT_COUNTER_BYTES + (size_t)R32_SPLIT_MAX_WGS * 4096, &p,
-                             /*zero_fresh=*/true) == MI_SUCCESS) {
-          a.counters = (unsigned *)p;
-          a.part = (float *)((uint8_t *)p + R32_SPLIT_COUNTER_BYTES);
-        } else {
-          a.split_shift = 0;  // no scratch (the stream is being captured before it ever had one)
-        }
+        // (a stream under capture that never ran such a shape gets the error: an unsplit launch would add the partial
+        // sums in another order)
+        const int rc = stream_workspace(stream, WS_ROWS32_SPLIT, R32_SPLIT_COUNTER_BYTES + (size_t)R32_SPLIT_MAX_WGS * 4096,
+                                        &p, /*zero_fresh=*/true);
+        if (rc != MI_SUCCESS)
+          return rc;
+        a.counters = (unsigned *)p;
+        a.part = (float *)((uint8_t *)p + R32_SPLIT_COUNTER_BYTES);
       }
       const dim3 grid((unsigned)(blocks << a.split_shift));
       if (e5m2)

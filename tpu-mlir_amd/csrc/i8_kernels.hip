@@ -1241,12 +1241,10 @@ int i8mm_launch(const void *d_a, int a_unsigned, const void *d_b, int b_unsigned
       void *p = nullptr;
       const int rc = stream_workspace(stream, WS_ROWS32_SPLIT,
                                       R32_SPLIT_COUNTER_BYTES + (size_t)R32_SPLIT_MAX_WGS * 4096, &p, /*zero_fresh=*/true);
-      if (rc == MI_SUCCESS) {
-        a.counters = (unsigned *)p;
-        a.part = (int32_t *)((uint8_t *)p + R32_SPLIT_COUNTER_BYTES);
-      } else {
-        a.split_shift = 0;  // no scratch (the stream is being captured before it ever had one): one workgroup per block
-      }
+      if (rc != MI_SUCCESS)  // (a stream under capture that never ran such a shape: the caller runs it eagerly first)
+        return rc;
+      a.counters = (unsigned *)p;
+      a.part = (int32_t *)((uint8_t *)p + R32_SPLIT_COUNTER_BYTES);
     }
     i8_rows32_kernel<<<dim3((unsigned)(blocks << a.split_shift)), dim3(512), 0, stream>>>(a);
   } else {

@@ -10,7 +10,8 @@
 
 // Kernel-selection overrides for the test-suite and for tuning runs: one process-wide record that the launch paths
 // consult in place of their heuristics wherever a field is non-zero.  Not part of the C ABI (the public header does
-// not declare it): the tests bind mi_internal_set_plan by name.  Not thread safe; set it while nothing is launching.
+// not declare it): the tests bind mi_internal_set_plan by name.  A launch reads the record that was current when it
+// started (the record is swapped as a whole); production code never calls the hook.
 extern "C" {
 typedef struct mi_internal_plan {
   int a16_waves, a16_tpw, a16_rows;  // skinny kernel instance (waves per workgroup, tiles per wave and round, row blocks)
@@ -33,6 +34,9 @@ typedef struct mi_internal_plan {
   int a16_rows32_split;              // 1 / 2 / 4: K parts per 32-channel block of the 32-row kernel
 } mi_internal_plan;
 void mi_internal_set_plan(const mi_internal_plan *p);  // null: back to the heuristics
+// device allocations the library's per-stream scratch buffers have made since it was loaded (for the tests of the entry
+// point that must allocate nothing)
+long mi_internal_workspace_allocations(void);
 }
 
 namespace mi {
@@ -165,6 +169,7 @@ constexpr int R32_SPLIT_COUNTER_BYTES = 1024;   // one counter per block of a sp
 // zero_fresh: a newly allocated buffer starts as zeros (for users that leave their counters at zero, and always ask
 // for the same size)
 int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out, bool zero_fresh = false);
+long workspace_allocations();
 // frees every buffer of a stream (current and retired); for owners of private streams, right before hipStreamDestroy
 void release_stream_workspaces(hipStream_t st);
 

@@ -24,6 +24,7 @@ struct Buf {
 };
 std::mutex g_mutex;
 std::map<std::tuple<int, hipStream_t, int>, Buf> g_bufs;
+long g_allocations = 0;  // hipMalloc calls made here since the library was loaded (read by the tests)
 }  // namespace
 
 int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out, bool zero_fresh) {
@@ -40,6 +41,7 @@ int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out, bool
     const size_t want = (bytes + 255) & ~(size_t)255;
     void *fresh = nullptr;
     MI_HIP(hipMalloc(&fresh, want));
+    ++g_allocations;
     if (zero_fresh) {  // on the stream, ahead of the first kernel to use it (the stream is not being captured)
       const hipError_t e = hipMemsetAsync(fresh, 0, want, st);
       if (e != hipSuccess) {
@@ -54,6 +56,11 @@ int stream_workspace(hipStream_t st, int purpose, size_t bytes, void **out, bool
   }
   *out = b.ptr;
   return MI_SUCCESS;
+}
+
+long workspace_allocations() {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  return g_allocations;
 }
 
 void release_stream_workspaces(hipStream_t st) {
