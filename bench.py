@@ -483,6 +483,41 @@ def bench_operator_boundary(pkg, S, steps=200):
             "GBps_algorithmic": round(S.w4_gemv_bytes(1, K, N, 128) / sec / 1e9, 1)}
 
 
+def bench_operator_boundary_int8(pkg, S, clib, steps=100):
+    """The quantized tpu.MatMul of cfg1 (256 x 1024 x 1024, int8 weights on the right) through the reference's operator
+    interface: float32-expanded host tensors in and out (1 MiB each way), per-channel multipliers with one common right
+    shift (the fused BM168x requantization, MatMul.cpp:708-716).  Times the C entry point with a prepared parameter
+    block; includes the float <-> 8-bit conversions and both transfers, so it is NOT a roofline figure."""
+    import ctypes
+    M, K, N = 256, 1024, 1024
+    c = S.int8_matmul(M, K, N, seed=9, right_transpose=False, qdm=False)
+    x = c["a"].astype(np.float32)
+    right = c["b"].astype(np.float32)
+    bias = c["bias"].astype(np.float32)
+    multi = c["mult"].astype(np.float32)
+    op = pkg.MatMulInt8(K, N, quant_mode=clib.RQ_MULTIPLIER_SHIFT, fuse_rq=True, multipliers=[1],
+                        rshifts=[int(c["shift"][0])], out_dtype=clib.DT_I8, right_is_weight=True)
+    op.init(x, right, bias, multi)
+    want = op.inference(x)
+    y = np.empty((M, N), dtype=np.float32)
+    fp = ctypes.POINTER(ctypes.c_float)
+    ins = (fp * 5)(x.ctypes.data_as(fp), right.ctypes.data_as(fp), bias.ctypes.data_as(fp), multi.ctypes.data_as(fp), None)
+    outs = (fp * 1)(y.ctypes.data_as(fp))
+    prm = clib.InferParam(ins, 5, outs, 1, op.param.c.handle)
+    op.attr.M = M
+    fn, a_ref, p_ref = clib.lib().mi_i8mm_inference, ctypes.byref(op.attr), ctypes.byref(prm)
+    for _ in range(10):
+        fn(a_ref, p_ref)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        rc = fn(a_ref, p_ref)
+    sec = (time.perf_counter() - t0) / steps
+    assert rc == 0 and np.array_equal(y, want)
+    op.deinit()
+    return {"case": "tpu.MatMul int8 inference, float32 host tensors, 256x1024x1024, fused per-channel requant",
+            "us_per_call": round(sec * 1e6, 1), "host_bytes_per_call": int(4 * (M * K + M * N))}
+
+
 def bench_module_block(pkg, S, clib, cfgs, steps=50):
     """The decode block as a device-resident op list (float32 in through set_tensor, Cast to bf16, the seven
     matmuls chained q/k/v <- x, o <- q, gate/up <- o, down <- gate, float32 out through get_tensor): wall time of
@@ -675,6 +710,7 @@ def main():
         ex["int8_1x4096x4096"] = bench_int8(pkg, S, torch, clib, 4096, 40, 5, M=1, graph=True)
         ex["f8_matmul"] = bench_f8_matmul(pkg, torch, clib)
         ex["operator_boundary"] = bench_operator_boundary(pkg, S)
+        ex["operator_boundary_int8"] = bench_operator_boundary_int8(pkg, S, clib)
         ex["device_resident_block"] = bench_module_block(pkg, S, clib, cfgs)
         line["extras"] = ex
     if not args.no_cpu_baseline:

@@ -208,6 +208,40 @@ def test_operator_level_against_oracle(orc):
     op.deinit()
 
 
+def test_operator_boundary_recognises_the_8_bit_type_of_its_float_operands():
+    """The interpreter hands 8-bit tensors over as floats.  The boundary turns them into bytes, in 16-element vector
+    steps and a scalar tail: int8 values, uint8 values (up to 255), lengths that are not multiples of 16, and the
+    refusals -- a value of each sign's far end in one tensor, a fraction, NaN, infinity, anything outside [-128, 255],
+    wherever in the tensor (vector part or tail) it sits."""
+    rng = np.random.default_rng(21)
+    M, K, N = 3, 37, 5                                                   # 111 activations: six vector steps and a tail
+    b = rng.integers(-128, 128, size=(K, N)).astype(np.float32)
+    for lo, hi in ((-128, 128), (0, 256)):
+        a = rng.integers(lo, hi, size=(M, K)).astype(np.float32)
+        a[0, 0], a[-1, -1] = lo, hi - 1                                  # the ends of the type, first and last element
+        op = M_.MatMulInt8(K=K, N=N, out_dtype=clib.DT_I32, right_is_weight=False)
+        want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+        assert np.array_equal(op.inference(a, b), want), (lo, hi)
+        op.deinit()
+    good = rng.integers(0, 100, size=(M, K)).astype(np.float32)
+    for pos in (0, 17, M * K - 1):                                       # first vector, a middle one, the scalar tail
+        for value in (0.5, -128.5, 256.0, -129.0, 1e10, np.nan, np.inf, -np.inf):
+            a = good.copy()
+            a.reshape(-1)[pos] = value
+            op = M_.MatMulInt8(K=K, N=N, out_dtype=clib.DT_I32, right_is_weight=False)
+            with pytest.raises(clib.BackendError) as e:
+                op.inference(a, b)
+            assert e.value.code == clib.MI_UNSUPPORTED, (pos, value)
+            op.deinit()
+    a = good.copy()
+    a.reshape(-1)[3], a.reshape(-1)[M * K - 2] = -1.0, 200.0             # int8 and uint8 values in one tensor
+    op = M_.MatMulInt8(K=K, N=N, out_dtype=clib.DT_I32, right_is_weight=False)
+    with pytest.raises(clib.BackendError) as e:
+        op.inference(a, b)
+    assert e.value.code == clib.MI_UNSUPPORTED
+    op.deinit()
+
+
 @pytest.mark.parametrize("rmode", [clib.ROUND_HALF_AWAY_FROM_ZERO, clib.ROUND_HALF_UP, clib.ROUND_HALF_TO_EVEN])
 def test_requant_ops_against_oracle(orc, rmode):
     rng = np.random.default_rng(5)

@@ -1,6 +1,9 @@
 // C ABI of libtpumlir_amd.so: operator-level entry points (float-expanded host operands, as the reference
 // interpreter hands them over) and device-level launches.  See include/tpumlir_amd.h for the contract.
 #include <math.h>
+#if defined(__SSE2__)
+#include <emmintrin.h>
+#endif
 #include <string.h>
 
 #include <algorithm>
@@ -138,6 +141,12 @@ static unsigned stage_grid(int64_t n) {
 }
 // calls with at most this many elements on a side go through the pinned buffers
 constexpr int64_t SMALL_CALL_ELEMS = 1 << 16;
+// the quantized MatMul's 8-bit operand and its result travel the same way up to this many bytes
+constexpr size_t SMALL_I8_CALL_BYTES = (size_t)1 << 20;
+__global__ __launch_bounds__(256) void copy16_kernel(const uint4 *in, uint4 *out, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+    out[i] = in[i];
+}
 
 struct A16Handle {
   uint32_t magic = 0xA16A16u;
@@ -646,6 +655,7 @@ struct I8Handle {
   uint32_t magic = 0x18181818u;
   int64_t K = 0, N = 0;
   bool right_cached = false;
+  bool right_pre_transposed = false;  // a [K, N] weight is kept as [N, K]
   int right_unsigned = 0;
   DevBuf d_a, d_b, d_bias, d_multi, d_out;
   Pinned h_a, h_b, h_out;
@@ -672,21 +682,48 @@ static int out_elem_size(int dt) {
   }
 }
 
-// float-expanded 8-bit integers -> bytes; reports whether they are int8 or uint8 valued
+// float-expanded 8-bit integers -> bytes; reports whether they are int8 or uint8 valued.  A call of the operator spends
+// its time here and in the expansion of the result, not on the GPU, so the loop is written with SSE2 intrinsics (every
+// x86-64 host has them; left to the auto-vectorizer the same loop came out scalar in this translation unit, five times
+// slower).  Per element: truncate to int and convert back (stands in for truncf; NaN compares unequal), check the
+// range on the integer, take the low byte.  Bytes past the last multiple of 16 go through the scalar form.
 static int floats_to_bytes(const float *src, int64_t n, uint8_t *dst, int *is_unsigned, const char *who) {
-  float lo = 0.f, hi = 0.f;
-  bool whole = true;  // integer valued and inside [-128, 255] (false for NaN and infinities as well)
-  for (int64_t i = 0; i < n; ++i) {
-    const float v = src[i];
-    whole &= (v >= -128.f) & (v <= 255.f) & (v == truncf(v));
-    lo = v < lo ? v : lo;
-    hi = v > hi ? v : hi;
+  int bad = 0, any_neg = 0, any_big = 0;
+  int64_t i = 0;
+#if defined(__SSE2__)
+  __m128i vbad = _mm_setzero_si128(), vneg = _mm_setzero_si128(), vbig = _mm_setzero_si128();
+  const __m128i c128 = _mm_set1_epi32(128), c383 = _mm_set1_epi32(383 - 0x7fffffff - 1), sign = _mm_set1_epi32(-0x7fffffff - 1);
+  const __m128i c127 = _mm_set1_epi32(127), lowbyte = _mm_set1_epi32(0xff);
+  for (; i + 16 <= n; i += 16) {
+    __m128i q[4];
+    for (int u = 0; u < 4; ++u) {
+      const __m128 v = _mm_loadu_ps(src + i + 4 * u);
+      const __m128i iv = _mm_cvttps_epi32(v);  // out of range and NaN give INT_MIN, caught by the range check
+      vbad = _mm_or_si128(vbad, _mm_castps_si128(_mm_cmpneq_ps(_mm_cvtepi32_ps(iv), v)));
+      // unsigned (iv + 128) > 383, as a signed compare on both sides flipped
+      vbad = _mm_or_si128(vbad, _mm_cmpgt_epi32(_mm_xor_si128(_mm_add_epi32(iv, c128), sign), c383));
+      vneg = _mm_or_si128(vneg, iv);                        // sign bit: some value below zero
+      vbig = _mm_or_si128(vbig, _mm_sub_epi32(c127, iv));   // sign bit: some value above 127
+      q[u] = _mm_and_si128(iv, lowbyte);
+    }
+    _mm_storeu_si128((__m128i *)(dst + i), _mm_packus_epi16(_mm_packs_epi32(q[0], q[1]), _mm_packs_epi32(q[2], q[3])));
   }
-  MI_REQUIRE(whole && !(lo < 0.f && hi > 127.f), MI_UNSUPPORTED,
+  bad = _mm_movemask_epi8(vbad) != 0;
+  any_neg = (_mm_movemask_ps(_mm_castsi128_ps(vneg)) != 0);
+  any_big = (_mm_movemask_ps(_mm_castsi128_ps(vbig)) != 0);
+#endif
+  for (; i < n; ++i) {
+    const float v = src[i];
+    const bool in_range = v >= -128.f && v <= 255.f;  // false for NaN
+    const int32_t iv = in_range ? (int32_t)v : 0;
+    bad |= !in_range || (float)iv != v;
+    any_neg |= iv < 0;
+    any_big |= iv > 127;
+    dst[i] = (uint8_t)iv;
+  }
+  MI_REQUIRE(!bad && !(any_neg && any_big), MI_UNSUPPORTED,
              std::string(who) + ": operand does not hold the values of one 8-bit integer type");
-  for (int64_t i = 0; i < n; ++i)
-    dst[i] = (uint8_t)(int)src[i];
-  *is_unsigned = hi > 127.f;
+  *is_unsigned = any_big;
   return MI_SUCCESS;
 }
 
@@ -711,6 +748,19 @@ static int upload_right(I8Handle *h, const mi_i8mm_attr *attr, const float *righ
     return rc;
   if ((rc = h->d_b.reserve((size_t)n)))
     return rc;
+  h->right_pre_transposed = false;
+  if (attr->right_is_weight && !attr->right_transpose) {
+    // a [K, N] weight is laid out [N, K] once, here, instead of on every call (the kernels read both operands along K)
+    DevBuf tmp;
+    if ((rc = tmp.reserve((size_t)n)))
+      return rc;
+    MI_HIP(hipMemcpyAsync(tmp.ptr, h->h_b.ptr, (size_t)n, hipMemcpyHostToDevice, h->stream));
+    if ((rc = permute_launch(tmp.ptr, h->d_b.ptr, 1, 0, 1, 1, attr->K, attr->N, h->stream)))
+      return rc;
+    MI_HIP(hipStreamSynchronize(h->stream));  // tmp is freed on return
+    h->right_pre_transposed = true;
+    return MI_SUCCESS;
+  }
   MI_HIP(hipMemcpyAsync(h->d_b.ptr, h->h_b.ptr, (size_t)n, hipMemcpyHostToDevice, h->stream));
   return MI_SUCCESS;
 }
@@ -864,7 +914,11 @@ int mi_i8mm_inference(const mi_i8mm_attr *attr, mi_infer_param *p) {
   int a_unsigned = 0;
   if ((rc = floats_to_bytes(p->inputs[0], M * K, (uint8_t *)h->h_a.ptr, &a_unsigned, "mi_i8mm_inference")))
     return rc;
-  MI_HIP(hipMemcpyAsync(h->d_a.ptr, h->h_a.ptr, (size_t)M * K, hipMemcpyHostToDevice, h->stream));
+  if ((size_t)M * K <= SMALL_I8_CALL_BYTES && ((size_t)M * K) % 16 == 0)  // read over the bus by a kernel: no copy command
+    copy16_kernel<<<dim3(stage_grid(M * K / 16)), dim3(256), 0, h->stream>>>((const uint4 *)h->h_a.ptr,
+                                                                              (uint4 *)h->d_a.ptr, M * K / 16);
+  else
+    MI_HIP(hipMemcpyAsync(h->d_a.ptr, h->h_a.ptr, (size_t)M * K, hipMemcpyHostToDevice, h->stream));
   if (!h->right_cached && (rc = upload_right(h, attr, p->inputs[1])))
     return rc;
   const float *bias = p->n_inputs > 2 ? p->inputs[2] : nullptr;
@@ -890,12 +944,20 @@ int mi_i8mm_inference(const mi_i8mm_attr *attr, mi_infer_param *p) {
     }
   }
   const int64_t relu_limit = attr->relu_limit > 0.0 ? (int64_t)floor(attr->relu_limit) : -1;
-  rc = i8mm_launch(h->d_a.ptr, a_unsigned, h->d_b.ptr, h->right_unsigned, attr->right_transpose,
+  // a small result goes to the pinned host buffer through a copy kernel's 16-byte stores over the bus (no copy command;
+  // the matmul's own epilogue may store single bytes, which the bus takes one at a time)
+  const bool out_direct = false;
+  const bool out_by_kernel = (size_t)M * N * osz <= SMALL_I8_CALL_BYTES && ((size_t)M * N * osz) % 16 == 0;
+  rc = i8mm_launch(h->d_a.ptr, a_unsigned, h->d_b.ptr, h->right_unsigned, attr->right_transpose || h->right_pre_transposed,
                    bias ? (const int32_t *)h->d_bias.ptr : nullptr, M, K, N, attr->input_zp, attr->right_zp,
-                   attr->do_relu, relu_limit, rqp, h->d_out.ptr, nullptr, h->stream);
+                   attr->do_relu, relu_limit, rqp, out_direct ? h->h_out.ptr : h->d_out.ptr, nullptr, h->stream);
   if (rc)
     return rc;
-  MI_HIP(hipMemcpyAsync(h->h_out.ptr, h->d_out.ptr, (size_t)M * N * osz, hipMemcpyDeviceToHost, h->stream));
+  if (out_by_kernel)
+    copy16_kernel<<<dim3(stage_grid(M * N * osz / 16)), dim3(256), 0, h->stream>>>((const uint4 *)h->d_out.ptr,
+                                                                                 (uint4 *)h->h_out.ptr, M * N * osz / 16);
+  else
+    MI_HIP(hipMemcpyAsync(h->h_out.ptr, h->d_out.ptr, (size_t)M * N * osz, hipMemcpyDeviceToHost, h->stream));
   MI_HIP(hipStreamSynchronize(h->stream));
   bytes_to_floats(h->h_out.ptr, attr->out_dtype, M * N, p->outputs[0]);
   return MI_SUCCESS;
