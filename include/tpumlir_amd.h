@@ -56,8 +56,11 @@ enum {
 /* storage types */
 enum { MI_DT_BF16 = 0, MI_DT_F16 = 1, MI_DT_I8 = 2, MI_DT_U8 = 3, MI_DT_I16 = 4, MI_DT_U16 = 5, MI_DT_I32 = 6 };
 /* chip family: selects the bf16 rounding flavour and the CV18xx requant branches
- * (module::isCV18xx(), lib/Support/Float16.cpp:769-774, lib/Support/MathUtils.cpp:538-562) */
-enum { MI_CHIP_BM168X = 0, MI_CHIP_CV18XX = 1 };
+ * (module::isCV18xx(), lib/Support/Float16.cpp:769-774, lib/Support/MathUtils.cpp:538-562).  MI_CHIP_BM168X stands for
+ * the BM1684X and BM1690 families; MI_CHIP_BM1684 for every other non-CV18xx chip: the same arithmetic everywhere, and
+ * the one place the reference tells them apart on this path is parseParam's K / N swap of a transposed right operand
+ * under hdim_is_batch (module::isBM1684XFamily() || module::isBM1690Family(), MatMul.cpp:66-71), which it does not take. */
+enum { MI_CHIP_BM168X = 0, MI_CHIP_CV18XX = 1, MI_CHIP_BM1684 = 2 };
 
 /* ---- library ---------------------------------------------------------------- */
 const char *mi_version(void);

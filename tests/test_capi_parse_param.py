@@ -28,7 +28,8 @@ def test_parse_param_matches_oracle_on_every_flag(orc):
             for lt in (False, True):
                 for ot in (False, True):
                     for hd in (False, True):
-                        for chip, ochip in ((clib.CHIP_BM168X, orc.CHIP_BM1684X), (clib.CHIP_CV18XX, orc.CHIP_CV18XX)):
+                        for chip, ochip in ((clib.CHIP_BM168X, orc.CHIP_BM1684X), (clib.CHIP_CV18XX, orc.CHIP_CV18XX),
+                                            (clib.CHIP_BM1684, orc.CHIP_OTHER)):
                             kw = dict(right_transpose=rt, left_transpose=lt, output_transpose=ot, hdim_is_batch=hd)
                             try:
                                 want = orc.matmul_parse_param(a, b, o, chip=ochip, **kw)
@@ -37,3 +38,15 @@ def test_parse_param_matches_oracle_on_every_flag(orc):
                                     m.matmul_parse_param(a, b, o, chip=chip, **kw)
                                 continue
                             assert m.matmul_parse_param(a, b, o, chip=chip, **kw) == want, (a, b, o, kw, chip)
+
+
+def test_parse_param_tells_bm1684_from_the_bm1684x_family():
+    """MatMul.cpp:63-72: under hdim_is_batch a transposed right operand (B0, K, B1, N) gives K = shape[-3],
+    N = shape[-1]; only the BM1684X / BM1690 families swap the two."""
+    m = pkg()
+    clib = pkg("clib")
+    a, b, o = (2, 5, 3, 6), (2, 6, 3, 7), (2, 5, 3, 7)
+    kw = dict(right_transpose=True, hdim_is_batch=True)
+    plain = m.matmul_parse_param(a, b, o, chip=clib.CHIP_BM1684, **kw)
+    swapped = m.matmul_parse_param(a, b, o, chip=clib.CHIP_BM168X, **kw)
+    assert (plain["K"], plain["N"]) == (6, 7) and (swapped["K"], swapped["N"]) == (7, 6)

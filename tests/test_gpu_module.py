@@ -319,13 +319,54 @@ def test_get_tensor_scales_uniform_quantized_tensors():
     c = rng.integers(-32768, 32768, size=n).astype(np.float32)
     m.set_quant("a", 0.0123, -7).set_quant("b", 0.37, 131).set_quant("c", 1.7e-3, 5)
     for name, v in (("a", a), ("b", b), ("c", c), ("plain", a)):
-        m.set_tensor(name, v)
+        m.set_tensor_from_int(name, v)                                   # the stored integers themselves
     assert np.array_equal(m.get_tensor("a"), (a - np.float32(-7)) * np.float32(0.0123))
     assert np.array_equal(m.get_tensor("b"), (b - np.float32(131)) * np.float32(0.37))
     assert np.array_equal(m.get_tensor("c"), (c.astype(np.float64) * 1.7e-3).astype(np.float32))  # no zero point
     assert np.array_equal(m.get_tensor("plain"), a)
     for name, v in (("a", a), ("b", b), ("c", c)):
         assert np.array_equal(m.get_tensor_raw(name), v)
+    # set_tensor on a uniform-quantized 8-bit tensor takes REAL values and quantizes them the way
+    # ModuleInterpreter::setTensor does (host/ModuleInterpreter.cpp:1341-1348): p * (float)(1 / scale) + (float)zp,
+    # half away from zero, saturated; a tensor without quantization parameters and a 16-bit one take the values as given
+    real = (rng.standard_normal(n) * 2).astype(np.float32)
+    real[:4] = [1e6, -1e6, 0.0123 * 2.5, -0.0123 * 2.5]                  # both saturations and both ties
+    for name, (scale, zp), lo, hi in (("a", (0.0123, -7), -128, 127), ("b", (0.37, 131), 0, 255)):
+        m.set_tensor(name, real)
+        d = real * np.float32(1.0 / scale) + np.float32(zp)
+        want = np.clip(np.sign(d) * np.floor(np.abs(d) + np.float32(0.5)), lo, hi)
+        assert np.array_equal(m.get_tensor_raw(name), want), name
+    m.set_tensor("plain", a)
+    assert np.array_equal(m.get_tensor_raw("plain"), a)
+    # the name lists and the quantization summary of pymlir.module (pymlir.cpp:112, :116-119)
+    assert m.all_tensor_names == ["a", "b", "c", "plain"] and m.input_names == ["a", "b", "c", "plain"]
+    assert m.output_names == []
+    assert m.get_tensor_qinfo("a") == ("I8", 0.0123, -7, "[300]")
+    assert m.get_tensor_qinfo("plain") == ("I8", 1.0, 0, "[300]")
+    assert m.get_tensor_qinfo("nowhere") == ("NA", 1.0, 0, "[]")
+    every = m.get_all_tensor()
+    assert sorted(every) == ["a", "b", "c", "plain"] and np.array_equal(every["plain"], a)
     with pytest.raises(clib.BackendError):
         m.add_tensor("f", clib.ST_F32, (4,)).set_quant("f", 1.0, 0)
+    m.destroy()
+
+
+def test_hook_lists_and_name_lists_of_a_block():
+    """before_invoke / after_invoke append callables that run in the order added, clear_hooks removes them all
+    (pymodule.cpp:71-82); input_names / output_names follow from which op writes and reads what."""
+    M, K = 1, 512
+    m, _, _ = _decoder_like_module(M, K)
+    assert m.input_names == ["x"]
+    assert sorted(m.output_names) == ["down", "k", "up", "v"]           # what no later op reads
+    m.set_tensor("x", np.ones((M, K), dtype=np.float32))
+    calls = []
+    m.before_invoke(lambda n: calls.append(("b1", n)))
+    m.before_invoke(lambda n: calls.append(("b2", n)))
+    m.after_invoke(lambda n: calls.append(("a1", n)))
+    m.invoke()
+    assert calls[:3] == [("b1", "xb"), ("b2", "xb"), ("a1", "xb")] and len(calls) == 3 * 8
+    calls.clear()
+    m.clear_hooks()
+    m.invoke()
+    assert calls == []
     m.destroy()

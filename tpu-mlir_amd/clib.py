@@ -10,7 +10,7 @@ ROUND_HALF_AWAY_FROM_ZERO, ROUND_HALF_UP, ROUND_HALF_DOWN, ROUND_HALF_TO_EVEN = 
 ROUND_TOWARDS_ZERO, ROUND_UP, ROUND_DOWN = 6, 8, 9
 RQ_TFLITE_LSHIFT, RQ_TFLITE, RQ_MULTIPLIER_SHIFT, RQ_ONLY_SHIFT, RQ_QDM, RQ_ONLY_SCALE = 0, 1, 2, 3, 4, 5
 DT_BF16, DT_F16, DT_I8, DT_U8, DT_I16, DT_U16, DT_I32 = range(7)
-CHIP_BM168X, CHIP_CV18XX = 0, 1
+CHIP_BM168X, CHIP_CV18XX, CHIP_BM1684 = 0, 1, 2
 ST_F32, ST_BF16, ST_F16, ST_I8, ST_U8, ST_I16, ST_U16, ST_I32, ST_U32, ST_F8E4M3, ST_F8E5M2 = range(11)
 
 # every symbol include/tpumlir_amd.h declares

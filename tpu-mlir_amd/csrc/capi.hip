@@ -1412,7 +1412,8 @@ int cast_scalars(const mi_cast_attr *a, float *inv_scale, float *scale) {
                    (f8_in && wide_out && !a->in_quant && !a->out_quant),
                MI_UNSUPPORTED, "mi_cast: an 8-bit float casts from and to F32 / F16 only");
   }
-  MI_REQUIRE(a->chip == MI_CHIP_BM168X || a->chip == MI_CHIP_CV18XX, MI_BAD_ARGUMENT, "mi_cast: unknown chip");
+  MI_REQUIRE(a->chip == MI_CHIP_BM168X || a->chip == MI_CHIP_CV18XX || a->chip == MI_CHIP_BM1684, MI_BAD_ARGUMENT,
+             "mi_cast: unknown chip");
   MI_REQUIRE(a->num_elem >= 0, MI_BAD_ARGUMENT, "mi_cast: negative element count");
   *inv_scale = 1.0f;
   *scale = (float)a->scale;

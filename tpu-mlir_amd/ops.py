@@ -707,13 +707,36 @@ class Module:
     def __init__(self):
         self.handle = C.c_void_p()
         self.shapes = {}
+        self.types = {}          # name -> clib.ST_*
+        self.quant = {}          # name -> (scale, zero point) of a uniform-quantized tensor
+        self._produced = []      # output tensor of every op, in program order
+        self._consumed = set()
+        self._before, self._after = [], []
         check(clib.lib().mi_module_create(C.byref(self.handle)))
 
     def add_tensor(self, name, storage_type, shape):
         n = int(np.prod(shape))
         check(clib.lib().mi_module_add_tensor(self.handle, name.encode(), storage_type, n))
         self.shapes[name] = tuple(shape)
+        self.types[name] = storage_type
         return self
+
+    def _op(self, inputs, output):
+        self._produced.append(output)
+        self._consumed.update(inputs)
+
+    # the name lists of pymlir.module (bindings/pymlir/pymlir.cpp:116-119)
+    @property
+    def all_tensor_names(self):
+        return list(self.shapes)
+
+    @property
+    def input_names(self):
+        return [n for n in self.shapes if n not in self._produced]
+
+    @property
+    def output_names(self):
+        return [n for n in self._produced if n not in self._consumed]
 
     def add_a16matmul(self, input, output, weight, scale_bits, zp, bias=None, *, K, N, weight_bits, q_group_size,
                       dtype=DT_BF16, chip=CHIP_BM168X, dq_type=clib.DQ_NONE):
@@ -725,6 +748,7 @@ class Module:
         check(clib.lib().mi_module_add_a16matmul_dq(self.handle, input.encode(), output.encode(), C.byref(desc),
                                                     int(dq_type), weight.ctypes.data, scale_bits.ctypes.data,
                                                     zp.ctypes.data, None if bias is None else bias.ctypes.data))
+        self._op([input], output)
         return self
 
     def add_matmul_int8(self, input, output, right, bias=None, *, K, N, right_transpose=False, input_zp=0, right_zp=0,
@@ -747,6 +771,7 @@ class Module:
                               None if bias is None else bias.ctypes.data, input_zp, right_zp, int(do_relu),
                               int(relu_limit), int(quant_mode is not None), rq)
         check(clib.lib().mi_module_add_matmul_int8(self.handle, input.encode(), output.encode(), C.byref(d)))
+        self._op([input], output)
         return self
 
     def add_requant(self, input, output, *, outer=1, channels, inner=1, input_zp=0, quant_mode,
@@ -764,6 +789,7 @@ class Module:
                 setattr(rq, name, int(v))
         d = clib.ModuleRqDesc(outer, channels, inner, input_zp, rq)
         check(clib.lib().mi_module_add_requant(self.handle, input.encode(), output.encode(), C.byref(d)))
+        self._op([input], output)
         return self
 
     def add_matmul_dq(self, left, right, output, *, K, N, right_transpose=False, q_group_size, dq_type=clib.DQ_INT8):
@@ -771,6 +797,7 @@ class Module:
         DQ_F8E4M3 / DQ_F4)."""
         check(clib.lib().mi_module_add_matmul_dq(self.handle, left.encode(), right.encode(), output.encode(), K, N,
                                                  int(right_transpose), q_group_size, dq_type))
+        self._op([left, right], output)
         return self
 
     def add_cast(self, input, output, *, in_type, out_type, in_quant=False, out_quant=False, scale=1.0, zero_point=0,
@@ -778,9 +805,24 @@ class Module:
         attr = clib.CastAttr(0, in_type, out_type, int(in_quant), int(out_quant), float(scale), int(zero_point),
                              clib.ST_F32 if expressed is None else expressed, round_mode, CHIP_BM168X)
         check(clib.lib().mi_module_add_cast(self.handle, input.encode(), output.encode(), C.byref(attr)))
+        self._op([input], output)
         return self
 
     def set_tensor(self, name, data):
+        """ModuleInterpreter::setTensor (host/ModuleInterpreter.cpp:1313-1362) with is_integer = false: real values
+        for a uniform-quantized 8-bit tensor are quantized on the way in, p * (float)(1 / scale) + (float)zp, rounded
+        half away from zero and saturated (to_int8 / to_uint8); every other tensor takes the values as they are."""
+        data = _f32(data)
+        if name in self.quant and self.types.get(name) in (clib.ST_I8, clib.ST_U8):
+            scale, zp = self.quant[name]
+            d = data * np.float32(1.0 / scale) + np.float32(zp)
+            q = np.sign(d) * np.floor(np.abs(d) + np.float32(0.5))
+            lo, hi = (-128, 127) if self.types[name] == clib.ST_I8 else (0, 255)
+            data = np.ascontiguousarray(np.clip(q, lo, hi), dtype=np.float32)
+        check(clib.lib().mi_module_set_tensor(self.handle, name.encode(), data.ctypes.data, data.size))
+
+    def set_tensor_from_int(self, name, data):
+        """setTensor with is_integer = true (pymodule.cpp:96-101): the stored integer values themselves."""
         data = _f32(data)
         check(clib.lib().mi_module_set_tensor(self.handle, name.encode(), data.ctypes.data, data.size))
 
@@ -801,9 +843,29 @@ class Module:
         check(clib.lib().mi_module_get_tensor_raw(self.handle, name.encode(), out.ctypes.data, out.size))
         return out
 
+    def get_all_tensor(self):
+        """py_module::getAllTensor (pymodule.cpp:56-69): every tensor as get_tensor gives it.  After plan_memory()
+        intermediates share one arena, so only inputs, marked outputs and the tensors still live hold their values."""
+        return {name: self.get_tensor(name) for name in self.shapes}
+
     def set_quant(self, name, scale, zero_point=0):
         check(clib.lib().mi_module_set_quant(self.handle, name.encode(), C.c_double(scale), C.c_int64(zero_point)))
+        self.quant[name] = (float(scale), int(zero_point))
         return self
+
+    _QINFO_NAMES = {clib.ST_F32: "F32", clib.ST_BF16: "BF16", clib.ST_F16: "F16", clib.ST_I8: "I8", clib.ST_U8: "U8",
+                    clib.ST_I16: "I16", clib.ST_U16: "U16", clib.ST_I32: "I32", clib.ST_U32: "U32",
+                    clib.ST_F8E4M3: "F8E4M3", clib.ST_F8E5M2: "F8E5M2"}
+
+    def get_tensor_qinfo(self, name):
+        """py_module::format_tensor_qinfo (pymodule.cpp:117-136; ModuleInterpreter::getTensorQuantInfo,
+        host/ModuleInterpreter.cpp:1436-1500): (dtype, scale, zero point, shape string); an unknown name gives
+        ("NA", 1.0, 0, "[]"), a tensor without quantization parameters scale 1 and zero point 0."""
+        if name not in self.shapes:
+            return ("NA", 1.0, 0, "[]")
+        scale, zp = self.quant.get(name, (1.0, 0))
+        return (self._QINFO_NAMES.get(self.types[name], "NA"), scale, zp,
+                "[" + ", ".join(str(int(v)) for v in self.shapes[name]) + "]")
 
     def mark_output(self, name):
         check(clib.lib().mi_module_mark_output(self.handle, name.encode()))
@@ -822,6 +884,24 @@ class Module:
         nullf = C.cast(None, clib.MODULE_HOOK)
         check(clib.lib().mi_module_set_hooks(self.handle, self._hooks[0] or nullf, self._hooks[1] or nullf, None))
         return self
+
+    # pymlir.module's hook interface (pymodule.cpp:71-82): any number of callables each way, run in the order added
+    def _install_hook_lists(self):
+        before = (lambda n: [f(n) for f in self._before]) if self._before else None
+        after = (lambda n: [f(n) for f in self._after]) if self._after else None
+        return self.set_hooks(before, after)
+
+    def before_invoke(self, func):
+        self._before.append(func)
+        return self._install_hook_lists()
+
+    def after_invoke(self, func):
+        self._after.append(func)
+        return self._install_hook_lists()
+
+    def clear_hooks(self):
+        self._before, self._after = [], []
+        return self.set_hooks(None, None)
 
     def invoke_at(self, name):
         check(clib.lib().mi_module_invoke_at(self.handle, name.encode()))
