@@ -355,3 +355,34 @@ def test_grouped_launch_through_the_tiled_kernel(orc, bits, M, K, Ns, g):
             _check_against_oracle(orc, c, y.view(torch.int16).cpu().numpy().view(np.uint16), f.cpu().numpy())
     for w in ws:
         w.destroy()
+
+
+@pytest.mark.parametrize("M,K,N,g,splits,f16", [
+    (130, 4096, 512, 128, 0, False),    # two whole chunks of 16 stages
+    (100, 4480, 272, 128, 0, False),    # 35 stages: 16 + 16 + 3, ragged N
+    (64, 2560, 256, 256, 0, False),     # a group spans two stages
+    (48, 2304, 256, 0, 0, False),       # per channel: one group for all 18 stages
+    (96, 4224, 256, 128, 2, False),     # K split: 17 + 16 stages, each with its own chunks
+    (70, 6144, 300, 128, 3, True),      # f16 operands, three splits of 16 stages
+])
+def test_widest_block_takes_the_zero_point_term_out_of_the_loop(orc, plan, M, K, N, g, splits, f16):
+    """The 128 x 256 block adds scale * P per group and subtracts the zero-point term every 16 stages through a small
+    bf16-piece matrix product; whole chunks, a short last chunk, groups longer than a stage and K splits all have to
+    agree with the oracle to the bound of every other kernel."""
+    plan(a16_gemm_tile=256, a16_gemm_min_m=17, a16_gemm_splits=splits)
+    cfg = S.w4a16(M, K, N, g, seed=M + K + N, bias=(N % 3 == 0))
+    if not f16:
+        out, pre = _run_device(cfg)
+        _check_against_oracle(orc, cfg, out, pre)
+        return
+    xf = orc.F16(S.bf16_to_f32(cfg["x"]))
+    sf = orc.F16(S.bf16_to_f32(cfg["scale"]))
+    cfg16 = dict(cfg)
+    cfg16["x"] = orc.f32_to_f16(xf)
+    cfg16["scale"] = orc.f32_to_f16(sf)
+    out, pre = _run_device(cfg16, dtype=clib.DT_F16)
+    want, want_pre = orc.a16matmul(xf, cfg["weight"].astype(np.float32), sf, cfg["zp"].astype(np.float32),
+                                   S.bf16_to_f32(cfg["bias"]) if cfg.get("bias") is not None else None,
+                                   M=M, K=K, N=N, weight_bits=4, q_group_size=g, out_dtype=orc.OUT_F16)
+    assert cmp.max_abs_over_rms(pre, want_pre) <= 2e-5
+    assert np.array_equal(out, orc.f32_to_f16(pre))

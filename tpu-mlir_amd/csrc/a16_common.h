@@ -27,6 +27,11 @@ struct Half16<MI_DT_BF16> {
   static __device__ __forceinline__ f32x4 mfma(vec8 a, vec8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
+  // acc + both halves of a packed pair, in fp32
+  static __device__ __forceinline__ float dot2_ones(uint32_t pair, float acc) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair), __builtin_bit_cast(bf16x2_t, ONE2), acc, false);
+  }
   static __device__ __forceinline__ float to_f32(uint16_t h) { return bf16_bits_to_f32(h); }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
@@ -46,6 +51,12 @@ struct Half16<MI_DT_F16> {
   static constexpr uint32_t ONE2 = 0x3C003C00u;
   static __device__ __forceinline__ f32x4 mfma(vec8 a, vec8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  // (conversions and adds: the packed f16 dot product gave NaN sums here where the bf16 one is exact)
+  static __device__ __forceinline__ float dot2_ones(uint32_t pair, float acc) {
+    typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+    const f16x2_t h = __builtin_bit_cast(f16x2_t, pair);
+    return acc + ((float)h[0] + (float)h[1]);
   }
   static __device__ __forceinline__ float to_f32(uint16_t h) { return f16_bits_to_f32(h); }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {

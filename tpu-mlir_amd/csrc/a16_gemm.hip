@@ -10,6 +10,9 @@
 // Arithmetic is that of the skinny kernel (see a16_kernels.hip), per quantization group:
 //   4-bit: P = sum_k a_k (16 + q_k) by MFMA, S = sum_k a_k by one more MFMA against ones, then
 //          acc += scale * (P - (16 + zp) * S) in fp32.
+//          The widest block (128 x 256) takes the second term out of the loop: acc += scale * P per group, and every
+//          16 groups one small matrix product subtracts sum_g S[m, g] * (scale * (16 + zp))[g, n], exact to fp32
+//          (see "correction" below).
 //   8-bit: the weight is rounded to the 16-bit type exactly as the reference does, and the MFMA accumulates directly.
 #include <algorithm>
 #include <climits>
@@ -27,6 +30,12 @@ constexpr int GEMM_KS = 128;     // K per LDS stage (one 4-bit weight tile, two 
 constexpr int GEMM_NST = 3;      // LDS ring depth
 constexpr int GEMM_WAVES = 8;
 constexpr int waitcnt_vm_only(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
+constexpr int WAITCNT_LGKM0 = 0xC07F;  // lgkmcnt(0), every other counter untouched
+constexpr int HOIST_CHUNK = 16;        // stages per zero-point correction (the K of its MFMA)
+template <int BITS, int GPT, int TM, int TN>
+constexpr bool gemm_hoists() {
+  return BITS == 4 && GPT == 1 && TM == 4 && TN == 4;
+}
 
 
 // One weight set of a launch.  Sibling sets on one input (q/k/v, gate/up: same K, width, group size and type) share a
@@ -56,6 +65,7 @@ struct GemmArgs {
   int64_t K;
   int k_tiles, G;
   int tiles_per_group;  // GPT == 1: weight tiles that share one group (g / TILE_K; k_tiles when per channel)
+  uint32_t tpg_magic;   // ceil(2^32 / tiles_per_group): tile / tiles_per_group == umulhi(tile, magic) for tile < 2^16
   int chip;
   int tiles_m, per_xcd;
   // split K: each output block is computed by k_splits workgroups over kt_per_split stages each; workgroup `split`
@@ -90,8 +100,11 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
   constexpr int XL = X_BYTES / 16 / (GEMM_WAVES * 64);  // activation direct-to-LDS instructions per thread and stage
   constexpr int WL = W_BYTES / 1024 / GEMM_WAVES;        // weight tiles each wave requests per stage
   constexpr int LPS = XL + WL + (WLDS ? GPT : 0);        // direct-to-LDS instructions per thread and stage
+  // 4-bit, one group per stage, widest block: the zero-point term leaves the loop (HOIST_CHUNK stages at a time)
+  constexpr bool HOIST = gemm_hoists<BITS, GPT, TM, TN>();
+  constexpr int SUMS_BYTES = HOIST ? HOIST_CHUNK * GM * 4 : 0;  // S of the last HOIST_CHUNK stages: [slot][row] fp32
   static_assert(!WLDS || (GN / 16) % GEMM_WAVES == 0, "weight tiles split evenly over the waves");
-  static_assert(GEMM_NST * STAGE_BYTES <= 160 * 1024, "LDS ring exceeds 160 KiB");
+  static_assert(GEMM_NST * STAGE_BYTES + SUMS_BYTES <= 160 * 1024, "LDS ring exceeds 160 KiB");
   static_assert(KSTEPS_PER_UNIT >= 1, "at most one group per MFMA k-step");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
@@ -178,6 +191,7 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
                                          (lptr_t)(st + X_BYTES + W_BYTES + (wave * GPT + u) * 256), 4, 0, 0);
     }
   };
+  const int sum_off = ((wm * TM + wn) * 16 + col) * (GEMM_KS * 2);  // HOIST: the row this lane sums (see Sq)
   int a_off[TM];  // byte offset of this lane's fragment row inside a stage
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -245,10 +259,21 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
   auto compute_stage = [&](const WStage &s, int kt) {
     const uint8_t *st = lds + (kt % GEMM_NST) * STAGE_BYTES;
     f32x4 P[TM][TN], S[TM];
+    float sq0 = 0.f, sq1 = 0.f;  // HOIST: sums of this lane's k-quarter of the row it adds up (see sum_off)
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       const bool first = (ks % KSTEPS_PER_UNIT) == 0;
       vec8 af[TM];
+      if constexpr (HOIST) {
+        // row sums: the WN waves of a row strip split its TM 16-row blocks among them; a wave reads the MFMA fragment
+        // of its block once more and adds the 8 values of every lane up (packed dot products against ones, fp32)
+        static_assert(TM == WN, "one 16-row block of the strip per wave");
+        const u32x4 v = *(const u32x4 *)(st + sum_off + (((ks * 4 + kq) ^ col) << 4));
+        sq0 = H::dot2_ones(v[0], sq0);
+        sq1 = H::dot2_ones(v[1], sq1);
+        sq0 = H::dot2_ones(v[2], sq0);
+        sq1 = H::dot2_ones(v[3], sq1);
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
         const int row15 = col;  // (wm*TM*16 + i*16 + col) & 15
@@ -262,7 +287,10 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
           bf[j] = unpack_nibbles<DT>(s.w[j][0][ks], nib_magic);
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-          S[i] = H::mfma(af[i], ones, first ? zero4 : S[i]);
+          if constexpr (!HOIST)
+            S[i] = H::mfma(af[i], ones, first ? zero4 : S[i]);
+          else
+            (void)S;
 #pragma unroll
           for (int j = 0; j < TN; ++j)
             P[i][j] = H::mfma(af[i], bf[j], first ? zero4 : P[i][j]);
@@ -272,12 +300,20 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
 #pragma unroll
           for (int j = 0; j < TN; ++j) {
             const float sc = H::to_f32((uint16_t)(s.sz[j][u] >> 16));
-            const float c = H::OFFSET + (float)(s.sz[j][u] & 0xffu);
+            if constexpr (HOIST) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+              for (int i = 0; i < TM; ++i)
 #pragma unroll
-              for (int r = 0; r < 4; ++r)
-                acc[i][j][r] = fmaf(sc, fmaf(-c, S[i][r], P[i][j][r]), acc[i][j][r]);
+                for (int r = 0; r < 4; ++r)
+                  acc[i][j][r] = fmaf(sc, P[i][j][r], acc[i][j][r]);
+            } else {
+              const float c = H::OFFSET + (float)(s.sz[j][u] & 0xffu);
+#pragma unroll
+              for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                  acc[i][j][r] = fmaf(sc, fmaf(-c, S[i][r], P[i][j][r]), acc[i][j][r]);
+            }
           }
         }
       } else {
@@ -293,6 +329,102 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
 #pragma unroll
           for (int j = 0; j < TN; ++j)
             acc[i][j] = H::mfma(af[i], bf[j], acc[i][j]);
+      }
+    }
+    if constexpr (HOIST) {
+      // the four k-quarters of a row sit 16 lanes apart: two lane-block swaps add them up (after the first, blocks
+      // 0|1 and 2|3 of the two registers hold each other's halves; after the second, so do the wave's halves)
+      float ta = sq0 + sq1, tb = ta;
+      asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(ta), "+v"(tb));
+      ta += tb;
+      tb = ta;
+      asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(ta), "+v"(tb));
+      // into the stage's slot of the sums area (the four k-quarters store alike)
+      ((float *)(lds + GEMM_NST * STAGE_BYTES))[(kt % HOIST_CHUNK) * GM + (wm * TM + wn) * 16 + col] = ta + tb;
+    }
+  };
+
+  // ---- correction (HOIST): after stages [c0, c0 + n) the accumulators hold sum_g scale_g * P_g; what is missing is
+  //   - sum_g S[m, g] * (scale * (16 + zp))[g, n],
+  // a [rows x n] by [n x columns] product.  Both factors are fp32 values; each is cut into bf16 pieces that add up to
+  // it exactly (S: three pieces of 8 bits; scale * (16 + zp) has at most 16 significant bits: two pieces), and the
+  // pieces go through the K = 16 bf16 MFMA, whose products are exact and whose sums are fp32.  The piece of lowest
+  // order (third of S times second of the other factor, 2^-24 of the term) is left out.
+  auto correct = [&](int c0, int n) {
+    if constexpr (HOIST) {
+      typedef short s16x4 __attribute__((ext_vector_type(4)));
+      // the other factor first (global loads, answered by L2: the same words went through the ring moments ago).
+      // Lane (column, k-quarter) takes the words of its column for stages 4 * kq ... 4 * kq + 3 of the chunk.
+      uint32_t szw[TN][4];
+      {
+        uint32_t gofs[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int u = 4 * kq + e;
+          const uint32_t tile = (uint32_t)(kt0 + c0 + (u < n ? u : n - 1));  // past the chunk: a valid word, unused
+          uint32_t gi = a.tiles_per_group == 1 ? tile : __umulhi(tile, a.tpg_magic);
+          gi = gi < (uint32_t)a.G ? gi : (uint32_t)a.G - 1;
+          gofs[e] = gi * 16 + col;
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          int64_t rb = n_base / 16 + (wn * TN + j);
+          rb = rb < sg.row_blocks ? rb : sg.row_blocks - 1;
+          const uint32_t *base = sg.sz_t + rb * a.G * 16;  // wave-uniform
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            szw[j][e] = base[gofs[e]];
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);  // this wave's sums are written
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      const float *sums = (const float *)(lds + GEMM_NST * STAGE_BYTES);
+      s16x4 bh[TN], bm[TN];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        uint32_t h[4], m[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float sc = H::to_f32((uint16_t)(szw[j][e] >> 16));
+          const float v = -sc * (H::OFFSET + (float)(szw[j][e] & 0xffu));  // exact: 11 + 5 bits at most
+          h[e] = __builtin_bit_cast(uint32_t, v) & 0xffff0000u;
+          m[e] = __builtin_bit_cast(uint32_t, v - __builtin_bit_cast(float, h[e]));
+        }
+        const u32x2 hp = {__builtin_amdgcn_perm(h[1], h[0], 0x07060302u), __builtin_amdgcn_perm(h[3], h[2], 0x07060302u)};
+        const u32x2 mp = {__builtin_amdgcn_perm(m[1], m[0], 0x07060302u), __builtin_amdgcn_perm(m[3], m[2], 0x07060302u)};
+        bh[j] = __builtin_bit_cast(s16x4, hp);
+        bm[j] = __builtin_bit_cast(s16x4, mp);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        uint32_t h[4], m[4], l[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int u = 4 * kq + e;
+          float v = sums[u * GM + wm * TM * 16 + i * 16 + col];
+          v = u < n ? v : 0.0f;
+          h[e] = __builtin_bit_cast(uint32_t, v) & 0xffff0000u;
+          const float r1 = v - __builtin_bit_cast(float, h[e]);
+          m[e] = __builtin_bit_cast(uint32_t, r1) & 0xffff0000u;
+          l[e] = __builtin_bit_cast(uint32_t, r1 - __builtin_bit_cast(float, m[e]));
+        }
+        const u32x2 hp = {__builtin_amdgcn_perm(h[1], h[0], 0x07060302u), __builtin_amdgcn_perm(h[3], h[2], 0x07060302u)};
+        const u32x2 mp = {__builtin_amdgcn_perm(m[1], m[0], 0x07060302u), __builtin_amdgcn_perm(m[3], m[2], 0x07060302u)};
+        const u32x2 lp = {__builtin_amdgcn_perm(l[1], l[0], 0x07060302u), __builtin_amdgcn_perm(l[3], l[2], 0x07060302u)};
+        const s16x4 ah = __builtin_bit_cast(s16x4, hp), am = __builtin_bit_cast(s16x4, mp),
+                    al = __builtin_bit_cast(s16x4, lp);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          f32x4 t = acc[i][j];
+          t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(al, bh[j], t, 0, 0, 0);  // smallest terms first
+          t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(am, bm[j], t, 0, 0, 0);
+          t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ah, bm[j], t, 0, 0, 0);
+          t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(am, bh[j], t, 0, 0, 0);
+          t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ah, bh[j], t, 0, 0, 0);
+          acc[i][j] = t;
+        }
       }
     }
   };
@@ -317,6 +449,12 @@ __global__ __launch_bounds__(GEMM_WAVES * 64, 2) void a16_gemm_kernel(GemmArgs a
       load_w(nxt, kt + 1);
     issue_x(kt + GEMM_NST - 1);
     compute_stage(cur, kt);
+    if constexpr (HOIST) {
+      // the readers of a chunk's sums are through with them before they reach the next stage's barrier, and the next
+      // sums are written after it
+      if ((kt + 1) % HOIST_CHUNK == 0 || kt + 1 == kt_total)
+        correct(kt - kt % HOIST_CHUNK, kt % HOIST_CHUNK + 1);
+    }
   };
   int kt = 0;
   for (; kt + 1 < kt_total; kt += 2) {
@@ -453,7 +591,8 @@ static int launch_gemm_instance(GemmArgs &a, hipStream_t st, const A16Scratch *f
   a.per_xcd = (a.tiles_total * a.k_splits + 7) / 8;
   auto kfn = a16_gemm_kernel<BITS, DT, GPT, WM, WN, TM, TN>;
   const size_t lds_bytes =
-      (size_t)GEMM_NST * ((GM < 32 ? 32 : GM) * GEMM_KS * 2 + (BITS == 4 ? (GN / 16) * 1024 + GEMM_WAVES * GPT * 256 : 0));
+      (size_t)GEMM_NST * ((GM < 32 ? 32 : GM) * GEMM_KS * 2 + (BITS == 4 ? (GN / 16) * 1024 + GEMM_WAVES * GPT * 256 : 0)) +
+      (gemm_hoists<BITS, GPT, TM, TN>() ? HOIST_CHUNK * GM * 4 : 0);
   static LdsLimitOnce lds_limit;
   lds_limit.ensure((const void *)kfn, 160 * 1024);
   kfn<<<dim3((unsigned)(a.per_xcd * 8)), dim3(GEMM_WAVES * 64), lds_bytes, st>>>(a);
@@ -481,7 +620,8 @@ template <int BITS, int DT, int GPT>
 static int launch_gemm_shape(GemmArgs &a, hipStream_t st, const A16Scratch *fixed) {
   // Output block shape.  With at least 160 of the widest blocks no K split is made and the time of a launch is set by
   // how the blocks divide among the 256 CUs: one 128 x 256 or 128 x 128 workgroup per CU, two 64 x 128 ones (which
-  // overlap).  Measured at K = 4096, 4-bit g = 128, in us: 94 per round of 128 x 256 blocks, 50.5 per round of
+  // overlap).  Measured at K = 4096, 4-bit g = 128, in us: 94 per round of 128 x 256 blocks (82 where the zero-point
+  // term is taken out of the loop: 4-bit, groups of at least 128), 50.5 per round of
   // 128 x 128, 35 for the first 256 blocks of 64 x 128 and 24.5 for each further 256 -- all three grow alike with K, so
   // the cheapest by this count is taken (11008 x 4096: M = 768 187 -> 128 us, M = 1024 188 -> 152, M = 1536 281 -> 230;
   // 4096 x 4096: M = 1280 98 -> 78, M = 3072 187 -> 155).  Below that, where K is split: wide blocks never, 64 rows up
@@ -494,10 +634,11 @@ static int launch_gemm_shape(GemmArgs &a, hipStream_t st, const A16Scratch *fixe
   }
   const int tile = plan().a16_gemm_tile;
   constexpr bool fits = !(BITS == 4 && GPT == 4);  // 32-wide groups: a 256-column block's scale|zp words overflow LDS
+  constexpr bool hoists = gemm_hoists<BITS, GPT, 4, 4>();
   int rows = plan().a16_gemm_rows;
   bool wide = fits && tile == 256;
   if (tile == 0 && rows == 0 && big >= 160) {
-    const double c_wide = fits ? 94.0 * (double)((big + 255) / 256) : 1e30;
+    const double c_wide = fits ? (hoists ? 82.0 : 94.0) * (double)((big + 255) / 256) : 1e30;
     const double c_128 = 50.5 * (double)((t128 + 255) / 256);
     const double c_64 = 35.0 + 24.5 * (double)((t64 + 255) / 256 - 1);
     if (c_wide <= c_128 && c_wide <= c_64)
@@ -612,6 +753,7 @@ int a16_gemm_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t 
     a.tiles_per_group = w->g / tile_k;
   else
     gpt = tile_k / w->g;
+  a.tpg_magic = a.tiles_per_group > 1 ? (uint32_t)(((uint64_t(1) << 32) + a.tiles_per_group - 1) / a.tiles_per_group) : 0;
   const bool f16 = w->dtype == MI_DT_F16;
   int rc = MI_SUCCESS;
 #define MI_GEMM(BITS_, GPT_)                                             \
