@@ -59,6 +59,9 @@ def build_chain(pkg, S, torch, M, n_layers, cfgs):
     return layers, acts, outs
 
 
+# steps captured into one HIP graph at most (4 launches each; a 32-layer decoder's graph holds 32 steps' worth per token)
+MAX_STEPS_PER_GRAPH = 256
+
 # sibling projections that read the same activations go out as one grouped launch
 CHAIN_GROUPS = [("q_proj", "k_proj", "v_proj"), ("o_proj",), ("gate_proj", "up_proj"), ("down_proj",)]
 
@@ -81,12 +84,12 @@ def run_chain(pkg, mats, acts, outs, grouped=True):
 
 def bench_chain(pkg, S, torch, M, steps, warmup, n_layers, cfgs, grouped=True, graph_steps=None):
     """Times exactly `steps` steps (one step = the seven matmuls of one layer).  The launches are replayed from HIP
-    graphs: one graph holds the steps of all n_layers weight copies back to back (as a decoder's graph holds its
-    layers), a second one the steps % n_layers left over, so that a graph launch's own cost is spread over several
-    steps as it is in a real decode step.  graph_steps: steps per graph when that is not n_layers (the weight copies are
-    then used round-robin)."""
+    graphs, as few as possible: one graph holds up to MAX_STEPS_PER_GRAPH steps back to back, step i on weight copy
+    i % n_layers (as a decoder's graph holds all of its layers), a second one the steps left over, so that a graph
+    launch's own cost is spread over many steps as it is in a real decode step.  graph_steps: steps per graph when
+    that is to be something else."""
     layers, acts, outs = build_chain(pkg, S, torch, M, n_layers, cfgs)
-    per_graph = graph_steps or n_layers
+    per_graph = graph_steps or min(steps, MAX_STEPS_PER_GRAPH)
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         for mats in layers:  # eager pass first: loads the code objects before capture
@@ -102,8 +105,9 @@ def bench_chain(pkg, S, torch, M, steps, warmup, n_layers, cfgs, grouped=True, g
 
         full = capture(per_graph)
         rest = capture(steps % per_graph) if steps % per_graph else None
-        for i in range(max(1, warmup // per_graph)):
-            full.replay()
+        warm = capture(min(max(warmup, 1), per_graph))
+        for i in range(max(1, -(-warmup // per_graph))):
+            warm.replay()
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         stream.synchronize()
         torch.cuda.synchronize()
@@ -268,6 +272,22 @@ def bench_read_ceiling(pkg, torch, sizes, steps=60, pool_mb=1024):
         out[int(nbytes)] = {"us": round(best * 1e6, 2), "GBps": round(nbytes / best / 1e9, 1)}
     del pool
     return out
+
+
+def bench_launch_floor(pkg, torch, launch_bytes, replays=20, copies=16):
+    """What one step's launches cost when their kernels touch no memory: the same grids as the read-only ceiling's
+    launches (one per entry of launch_bytes), every wave returning at once, replayed from a HIP graph that holds
+    `copies` such steps.  Returns microseconds per step and per launch."""
+    pool = torch.empty(max(launch_bytes), dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+
+    def run():
+        for _ in range(copies):
+            for b in launch_bytes:
+                pkg.bench_read_launch(pool, b, sink, chunks_per_wave=0)
+    sec = _time_graph(torch, run, replays) / copies
+    return {"us_per_step": round(sec * 1e6, 2), "us_per_launch": round(sec * 1e6 / len(launch_bytes), 2),
+            "launches_per_step": len(launch_bytes)}
 
 
 def bench_single_matmuls(pkg, S, torch, steps=60):
@@ -659,7 +679,8 @@ def main():
                                "down 4096x11008)" % M,
                    "bytes_per_step": r["chain_bytes"], "launches_per_step": r["launches_per_step"],
                    "weight_copies": args.layers, "resident_weight_mb": round(r["weight_set_mb"], 1),
-                   "launch": ("one HIP graph replay per %d steps (one per weight copy); " % args.layers) +
+                   "launch": ("one HIP graph replay per %d steps (step i on weight copy i %% %d); "
+                              % (min(args.steps, MAX_STEPS_PER_GRAPH), args.layers)) +
                              ("q/k/v and gate/up each as one grouped launch" if not args.no_group
                               else "one launch per matmul"),
                    "timing": "value: host wall clock around the timed region; roofline: HIP events on the launch stream"},
@@ -690,6 +711,8 @@ def main():
     if not args.no_extras:
         ex = {}
         ex["read_ceiling"] = {str(k): v for k, v in ceil.items()}
+        # the step's launches with kernels that touch no memory: what remains of a step when no byte moves
+        ex["launch_floor_us"] = bench_launch_floor(pkg, torch, launch_bytes)
         if not args.no_int8:
             ex["int8_context"] = bench_int8_context(pkg, S, torch, clib, args.int8_size)
         # the same chain with one weight copy (101 MB: resident in the 256 MB cache after the first pass)

@@ -563,7 +563,8 @@ int mi_top_a16mm_launch(const mi_top_a16_weight *w, const float *d_x, int64_t M,
 /* Streams `bytes` (rounded down to whole KiB chunks) from d_src with one 16-byte load per lane, every wave requesting
  * chunks_per_wave (2, 4 or 8) chunks before it consumes any, and writes nothing (d_sink: 4 writable bytes, never
  * written for ordinary data).  The launch time of this kernel is the ceiling for any single launch that has to move
- * the same bytes from HBM; the benchmark reports the decode kernels against it. */
+ * the same bytes from HBM; the benchmark reports the decode kernels against it.  chunks_per_wave == 0 launches the grid
+ * of the 4-chunk form with every wave returning at once: the time of a launch that touches no memory. */
 int mi_bench_read_launch(const void *d_src, size_t bytes, int chunks_per_wave, void *d_sink, void *stream);
 
 #ifdef __cplusplus

@@ -34,14 +34,17 @@ __global__ __launch_bounds__(256) void bench_read_kernel(const u32x4 *__restrict
 extern "C" int mi_bench_read_launch(const void *d_src, size_t bytes, int chunks_per_wave, void *d_sink, void *stream) {
   using namespace mi;
   MI_REQUIRE(d_src && d_sink, MI_BAD_ARGUMENT, "mi_bench_read_launch: null pointer");
-  MI_REQUIRE(chunks_per_wave == 2 || chunks_per_wave == 4 || chunks_per_wave == 8, MI_BAD_ARGUMENT,
-             "mi_bench_read_launch: chunks_per_wave must be 2, 4 or 8");
-  const int64_t n_waves = (int64_t)(bytes / 1024) / chunks_per_wave;  // whole chunks only
+  MI_REQUIRE(chunks_per_wave == 0 || chunks_per_wave == 2 || chunks_per_wave == 4 || chunks_per_wave == 8,
+             MI_BAD_ARGUMENT, "mi_bench_read_launch: chunks_per_wave must be 0, 2, 4 or 8");
+  // 0: the grid of the 4-chunk launch, every wave of which returns at once (what a launch costs before it moves a byte)
+  const int64_t n_waves = (int64_t)(bytes / 1024) / (chunks_per_wave ? chunks_per_wave : 4);  // whole chunks only
   if (n_waves == 0)
     return MI_SUCCESS;
   const dim3 grid((unsigned)((n_waves + 3) / 4)), block(256);
   hipStream_t st = (hipStream_t)stream;
-  if (chunks_per_wave == 2)
+  if (chunks_per_wave == 0)
+    bench_read_kernel<4><<<grid, block, 0, st>>>((const u32x4 *)d_src, (uint32_t *)d_sink, 0);
+  else if (chunks_per_wave == 2)
     bench_read_kernel<2><<<grid, block, 0, st>>>((const u32x4 *)d_src, (uint32_t *)d_sink, n_waves);
   else if (chunks_per_wave == 4)
     bench_read_kernel<4><<<grid, block, 0, st>>>((const u32x4 *)d_src, (uint32_t *)d_sink, n_waves);
