@@ -539,7 +539,10 @@ typedef struct mi_top_a16mm_attr {
   int64_t K, N;
   int weight_bits;      /* 4 or 8 */
   int q_group_size;     /* < 1: one group per K elements (A16MatMul.cpp:88-91) */
-  int right_transpose;  /* 1 = weight stored [N, K] (4-bit: [N, K/2] bytes); 0 is MI_UNSUPPORTED */
+  int right_transpose;  /* 1 = weight stored [N, K] (4-bit: [N, K/2] bytes), scale / zp [N, K / group];
+                         * 0 = weight stored [K, N] and dequantized as ONE FLAT ARRAY, as MatMul::dequant_weight does:
+                         * element k * N + n in byte (k * N + n) / (8 / bits), group (k * N + n) / group size,
+                         * scale / zp hold N * K / group entries (the group size must divide N * K) */
 } mi_top_a16mm_attr;
 /* Replaces top::A16MatMulOp::inference (lib/Dialect/Top/Interfaces/A16MatMul.cpp:82-102), whose init and deinit are
  * empty (:76-80): inputs = {input, weight, scale, zp, bias|NULL}, all f32 (weight: packed bytes 0..255 as floats);
@@ -548,8 +551,8 @@ typedef struct mi_top_a16mm_attr {
  * first call uploads the weight operands and stores a handle in p->handle; later calls assume the same weights. */
 int mi_top_a16mm_inference(const mi_top_a16mm_attr *attr, mi_infer_param *p);
 void mi_top_a16mm_deinit(mi_infer_param *p);
-/* device level: weight = uint8 [N, K * bits / 8], scale / zp = float [N, G] (G = K / group), bias = float [N] or NULL,
- * all HOST arrays; d_x float [M, K] (16-byte aligned), d_y float [M, N]; asynchronous on stream */
+/* device level: weight = uint8 [N, K * bits / 8], scale / zp = float [N, G] (G = K / group) -- with right_transpose == 0
+ * the flat [K, N] form described at mi_top_a16mm_attr -- bias = float [N] or NULL, all HOST arrays; d_x float [M, K] (16-byte aligned), d_y float [M, N]; asynchronous on stream */
 typedef struct mi_top_a16_weight mi_top_a16_weight;
 int mi_top_a16_weight_create(mi_top_a16_weight **out, int64_t K, int64_t N, int weight_bits, int q_group_size,
                              int right_transpose, const uint8_t *weight, const float *scale, const float *zp,

@@ -64,10 +64,48 @@ def test_top_a16matmul_refuses_what_it_does_not_handle():
     m = pkg()
     clib = pkg("clib")
     cfg, x, scale, zp, bias = _top_operands(4, 1, 64, 8, 0, seed=2)
-    with pytest.raises(clib.BackendError) as e:
-        m.TopA16MatMul(K=64, N=8, weight_bits=4, q_group_size=0, right_transpose=False).inference(
+    with pytest.raises(clib.BackendError) as e:     # [N, K] storage: a group of 24 does not divide K = 64
+        m.TopA16MatMul(K=64, N=8, weight_bits=4, q_group_size=24).inference(
             x, cfg["weight"].astype(np.float32), scale, zp, bias)
     assert e.value.code == clib.MI_UNSUPPORTED
+    with pytest.raises(clib.BackendError) as e:     # [K, N] storage: 64 * 8 / 48 is not a whole number of groups
+        m.TopA16MatMul(K=64, N=8, weight_bits=4, q_group_size=48, right_transpose=False).inference(
+            x, cfg["weight"].astype(np.float32), scale, zp, bias)
+    assert e.value.code == clib.MI_UNSUPPORTED
+
+
+@pytest.mark.parametrize("bits,M,K,N,g", [(4, 1, 512, 256, 64), (4, 5, 384, 96, 32), (4, 3, 64, 48, 0),
+                                          (4, 2, 128, 40, 16),     # groups of 16 columns; 40 = 2.5 groups per row
+                                          (8, 1, 1024, 128, 128), (8, 6, 256, 130, 65)])
+def test_top_a16matmul_untransposed_weight_against_oracle(orc, bits, M, K, N, g):
+    """right_transpose == false: the weight is [K, N] and the reference dequantizes it as one flat array
+    (lib/Support/Dnnl/MatMul.cpp:29-40): element k * N + n, byte (k * N + n) / (8 / bits), group (k * N + n) / g.
+    Against the oracle on random operands, and bit for bit on one-hot rows (single products)."""
+    import torch
+    m = pkg()
+    rng = np.random.default_rng(bits * 1000 + K + N)
+    ge = g if g >= 1 else K                                        # A16MatMul.cpp:88-91
+    n_groups = N * K // ge
+    wbytes = rng.integers(0, 256, size=N * K * bits // 8, dtype=np.uint8)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    scale = (np.abs(rng.standard_normal(n_groups)) * 0.01 + 1e-4).astype(np.float32)
+    zp = (rng.integers(0, 1 << bits, size=n_groups) + 0.7).astype(np.float32)   # fractional: (int) truncates it
+    bias = rng.standard_normal(N).astype(np.float32)
+    wf = wbytes.astype(np.float32)
+    ref = orc.top_a16matmul(x, wf, scale, zp, bias, M=M, K=K, N=N, weight_bits=bits, q_group_size=g,
+                            right_transpose=False)
+    op = m.TopA16MatMul(K=K, N=N, weight_bits=bits, q_group_size=g, right_transpose=False)
+    y = op.inference(x, wf, scale, zp, bias)
+    op.deinit()
+    rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+    assert float(np.max(np.abs(y.astype(np.float64) - ref))) <= TOP_TOL * rms
+    w = m.TopA16Weight(wbytes, scale, zp, None, K=K, N=N, weight_bits=bits, q_group_size=g, right_transpose=False)
+    eye = torch.eye(K, dtype=torch.float32, device="cuda")
+    got = m.top_a16mm_launch(w, eye)
+    torch.cuda.synchronize()
+    expect = orc.dequant_weight(wf, scale, zp, weight_len=N * K, q_group_size=ge, weight_bits=bits).reshape(K, N)
+    assert np.array_equal(got.cpu().numpy(), expect)
+    w.destroy()
 
 
 @pytest.mark.parametrize("a,b,rt", [((3, 64, 128), (3, 128, 96), False), ((2, 2, 33, 64), (2, 2, 40, 64), True),

@@ -8,6 +8,11 @@
 // One wave per output channel: its row of the [N, K] weight is read exactly once per group of MR activation rows, in
 // 4- or 8-byte pieces that make a wave's load contiguous.  HBM-bound on the weights for few rows; this op is the
 // reference stage, not the hot path, and is not tuned further.
+//
+// right_transpose == false: the weight is [K, N] and dequant_weight walks it FLAT (MatMul.cpp:29-40): element
+// e = k * N + n sits in byte e / (8 / bits), and its group is e / q_group_size, so groups run along N inside a row k
+// (and across rows when the group does not divide N).  top_a16_kn_kernel follows that indexing literally: one thread
+// per output column, the k loop in order.
 #include <math.h>
 
 #include <climits>
@@ -92,6 +97,37 @@ __global__ __launch_bounds__(256) void top_a16_kernel(TopA16Args a) {
   }
 }
 
+template <int BITS, int MR>
+__global__ __launch_bounds__(256) void top_a16_kn_kernel(TopA16Args a) {
+  const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (n >= a.N)
+    return;
+  const int m0 = blockIdx.y * MR;
+  float acc[MR];
+#pragma unroll
+  for (int r = 0; r < MR; ++r)
+    acc[r] = 0.f;
+  for (int64_t k = 0; k < a.K; ++k) {
+    const int64_t e = k * a.N + n;
+    int q;
+    if constexpr (BITS == 4)
+      q = (a.w[e >> 1] >> (4 * (int)(e & 1))) & 0xF;
+    else
+      q = a.w[e];
+    const int64_t gi = e / a.g;
+    const float wq = (float)(q - a.zp[gi]) * a.scale[gi];
+#pragma unroll
+    for (int r = 0; r < MR; ++r) {
+      const int row = m0 + r < a.M ? m0 + r : a.M - 1;
+      acc[r] = fmaf(a.x[(int64_t)row * a.K + k], wq, acc[r]);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < MR; ++r)
+    if (m0 + r < a.M)
+      a.y[(int64_t)(m0 + r) * a.N + n] = acc[r] + (a.bias ? a.bias[n] : 0.f);
+}
+
 }  // namespace mi
 
 using namespace mi;
@@ -103,6 +139,7 @@ struct mi_top_a16_weight {
   float *bias = nullptr;
   int64_t K = 0, N = 0;
   int bits = 0, g = 0, G = 0;
+  bool kn = false;  // [K, N] storage, flat groups (right_transpose == false)
 };
 
 extern "C" {
@@ -113,21 +150,30 @@ int mi_top_a16_weight_create(mi_top_a16_weight **out, int64_t K, int64_t N, int 
   MI_REQUIRE(out && weight && scale && zp, MI_BAD_ARGUMENT, "mi_top_a16_weight_create: null argument");
   *out = nullptr;
   MI_REQUIRE(weight_bits == 4 || weight_bits == 8, MI_UNSUPPORTED, "mi_top_a16_weight_create: weight_bits");
-  MI_REQUIRE(right_transpose, MI_UNSUPPORTED,
-             "mi_top_a16_weight_create: only right_transpose weights ([N, K]) are handled");
-  MI_REQUIRE(K > 0 && N > 0 && K % 8 == 0, MI_UNSUPPORTED, "mi_top_a16_weight_create: K must be a multiple of 8");
+  MI_REQUIRE(K > 0 && N > 0, MI_BAD_ARGUMENT, "mi_top_a16_weight_create: bad shape");
   const int g = q_group_size < 1 ? (int)K : q_group_size;  // A16MatMul.cpp:88-91
-  MI_REQUIRE(K % g == 0 && g % 8 == 0, MI_UNSUPPORTED,
-             "mi_top_a16_weight_create: the group size must divide K and be a multiple of 8");
-  const int64_t G = K / g;
+  int64_t G = 0;     // groups per weight row ([N, K] storage)
+  int64_t n_groups;  // scale / zero-point entries in all
+  if (right_transpose) {
+    MI_REQUIRE(K % 8 == 0, MI_UNSUPPORTED, "mi_top_a16_weight_create: K must be a multiple of 8");
+    MI_REQUIRE(K % g == 0 && g % 8 == 0, MI_UNSUPPORTED,
+               "mi_top_a16_weight_create: the group size must divide K and be a multiple of 8");
+    G = K / g;
+    n_groups = N * G;
+  } else {
+    MI_REQUIRE((N * K) % g == 0 && (N * K) % (8 / weight_bits) == 0, MI_UNSUPPORTED,
+               "mi_top_a16_weight_create: [K, N] storage: the group size must divide N * K");
+    n_groups = N * K / g;
+  }
   mi_top_a16_weight *t = new mi_top_a16_weight;
   t->K = K;
   t->N = N;
   t->bits = weight_bits;
   t->g = g;
   t->G = (int)G;
-  std::vector<int32_t> zi((size_t)(N * G));
-  for (int64_t i = 0; i < N * G; ++i)
+  t->kn = !right_transpose;
+  std::vector<int32_t> zi((size_t)n_groups);
+  for (int64_t i = 0; i < n_groups; ++i)
     zi[(size_t)i] = (int)zp[i];  // (int)(zp_i), MatMul.cpp:36
   const size_t wbytes = (size_t)(N * K * weight_bits / 8);
   auto fail = [&](hipError_t e, const char *what) {
@@ -138,17 +184,17 @@ int mi_top_a16_weight_create(mi_top_a16_weight **out, int64_t K, int64_t N, int 
   hipError_t e;
   if ((e = hipMalloc(&t->w, wbytes)) != hipSuccess)
     return fail(e, "hipMalloc");
-  if ((e = hipMalloc((void **)&t->scale, (size_t)(N * G) * 4)) != hipSuccess)
+  if ((e = hipMalloc((void **)&t->scale, (size_t)n_groups * 4)) != hipSuccess)
     return fail(e, "hipMalloc");
-  if ((e = hipMalloc((void **)&t->zp, (size_t)(N * G) * 4)) != hipSuccess)
+  if ((e = hipMalloc((void **)&t->zp, (size_t)n_groups * 4)) != hipSuccess)
     return fail(e, "hipMalloc");
   if (bias && (e = hipMalloc((void **)&t->bias, (size_t)N * 4)) != hipSuccess)
     return fail(e, "hipMalloc");
   if ((e = hipMemcpy(t->w, weight, wbytes, hipMemcpyHostToDevice)) != hipSuccess)
     return fail(e, "hipMemcpy");
-  if ((e = hipMemcpy(t->scale, scale, (size_t)(N * G) * 4, hipMemcpyHostToDevice)) != hipSuccess)
+  if ((e = hipMemcpy(t->scale, scale, (size_t)n_groups * 4, hipMemcpyHostToDevice)) != hipSuccess)
     return fail(e, "hipMemcpy");
-  if ((e = hipMemcpy(t->zp, zi.data(), (size_t)(N * G) * 4, hipMemcpyHostToDevice)) != hipSuccess)
+  if ((e = hipMemcpy(t->zp, zi.data(), (size_t)n_groups * 4, hipMemcpyHostToDevice)) != hipSuccess)
     return fail(e, "hipMemcpy");
   if (bias && (e = hipMemcpy(t->bias, bias, (size_t)N * 4, hipMemcpyHostToDevice)) != hipSuccess)
     return fail(e, "hipMemcpy");
@@ -189,7 +235,20 @@ int mi_top_a16mm_launch(const mi_top_a16_weight *t, const float *d_x, int64_t M,
   MI_REQUIRE(gy <= 65535 && (t->N + 3) / 4 <= INT32_MAX, MI_UNSUPPORTED, "mi_top_a16mm_launch: too many rows");
   const dim3 grid((unsigned)((t->N + 3) / 4), (unsigned)gy), block(256);
   hipStream_t st = (hipStream_t)stream;
-  if (t->bits == 4) {
+  if (t->kn) {
+    const dim3 grid_kn((unsigned)((t->N + 255) / 256), (unsigned)gy);
+    if (t->bits == 4) {
+      if (mr == 1)
+        top_a16_kn_kernel<4, 1><<<grid_kn, block, 0, st>>>(a);
+      else
+        top_a16_kn_kernel<4, 4><<<grid_kn, block, 0, st>>>(a);
+    } else {
+      if (mr == 1)
+        top_a16_kn_kernel<8, 1><<<grid_kn, block, 0, st>>>(a);
+      else
+        top_a16_kn_kernel<8, 4><<<grid_kn, block, 0, st>>>(a);
+    }
+  } else if (t->bits == 4) {
     if (mr == 1)
       top_a16_kernel<4, 1><<<grid, block, 0, st>>>(a);
     else
