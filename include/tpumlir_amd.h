@@ -99,8 +99,10 @@ typedef struct mi_a16mm_attr {
   int out_dtype;        /* MI_DT_BF16, or MI_DT_F16 when module::isF16Modes() */
   int chip;             /* MI_CHIP_* */
   int dynamic_quant;    /* MI_DQ_*: module::isDynamicQuantize() and getDqType().  MI_DQ_INT, MI_DQ_F8E4M3 (8-bit
-                         * weights) and MI_DQ_F4 (4-bit weights) with K % 128 == 0 and groups of 32, 64 or k*128 (integer
-                         * codes in 8-bit weights: up to 512) are handled; anything else is MI_UNSUPPORTED */
+                         * weights) and MI_DQ_F4 (4-bit weights) are handled for every group size that divides K (integer
+                         * codes in 8-bit weights: groups of up to 512, where the reference's f32 group product stops being
+                         * exact; no group beyond 32768): K % 128 == 0 with groups of 32, 64 or k*128 on MFMA kernels,
+                         * everything else on a plain kernel in the reference's order.  Anything else is MI_UNSUPPORTED */
 } mi_a16mm_attr;
 
 /* Replaces tpu::A16MatMulOp::init (A16MatMul.cpp:16-18).  inputs = {input, weight, scale, zp, bias|NULL}.

@@ -97,15 +97,64 @@ def test_dynamic_int_operator_level(orc):
 
 def test_dynamic_int_rejects_what_it_does_not_handle():
     import torch
-    for cfg, bits in ((S.w4a16(1, 192, 16, 64, seed=1), 4),        # K is not a multiple of 128
-                      (S.w8a16(1, 1024, 16, 1024, seed=1), 8)):    # 8-bit group too long to stay exact
-        w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=cfg["K"], N=16, weight_bits=bits,
-                         q_group_size=cfg["g"])
-        x = torch.zeros((1, cfg["K"]), dtype=torch.bfloat16, device="cuda")
-        with pytest.raises(clib.BackendError) as e:
-            M_.a16mm_dq_launch(w, x)
-        assert e.value.code == clib.MI_UNSUPPORTED
-        w.destroy()
+    cfg, bits = S.w8a16(1, 1024, 16, 1024, seed=1), 8              # 8-bit group too long to stay exact
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=cfg["K"], N=16, weight_bits=bits,
+                     q_group_size=cfg["g"])
+    x = torch.zeros((1, cfg["K"]), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(clib.BackendError) as e:
+        M_.a16mm_dq_launch(w, x)
+    assert e.value.code == clib.MI_UNSUPPORTED
+    w.destroy()
+
+
+PLAIN_CASES = [  # (bits, M, K, N, g, bias, dq): shapes outside the fragment kernels' layout
+    (4, 1, 192, 16, 64, False, "INT"),       # K is not a multiple of 128 (tiled weight, padded last tile)
+    (4, 5, 320, 100, 32, True, "INT"),
+    (4, 3, 384, 48, 96, True, "INT"),        # a group size the tiled layout does not take (weight kept as stored)
+    (4, 2, 240, 20, 24, False, "INT"),
+    (4, 300, 64, 260, 16, True, "INT"),      # many rows, more than one block of 256 channels
+    (8, 4, 192, 40, 64, True, "INT"),        # 8-bit, tiled, K % 128 != 0
+    (8, 2, 480, 24, 160, False, "INT"),      # 8-bit kept as stored
+    (4, 3, 192, 16, 64, True, "F4"), (4, 2, 384, 40, 96, False, "F4"),
+    (8, 3, 192, 16, 64, True, "F8"), (8, 2, 480, 24, 160, False, "F8"),
+]
+
+
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("bits,M,K,N,g,bias,dq", PLAIN_CASES)
+def test_dynamic_quantization_outside_the_fragment_layout(orc, bits, M, K, N, g, bias, dq, signed):
+    """K that is not a multiple of 128 and group sizes other than 32, 64 or whole tiles run through one plain kernel
+    in the reference's own order (A16MatMul.cpp:93-160): bit for bit against the oracle, whose float-code products
+    are double sums in k order just as the kernel's are."""
+    import torch
+    if signed and (bits == 4 or dq != "INT"):
+        pytest.skip("signed storage exists for 8-bit integer weights only")
+    if bits == 4:
+        cfg = S.w4a16(M, K, N, g, seed=M + K + N, bias=bias)
+    else:
+        cfg = S.w8a16(M, K, N, g, seed=M + K + N, bias=bias, signed=signed)
+        if not signed:
+            cfg["zp"] = np.random.default_rng(M + N).integers(0, 256 if dq == "INT" else 4, size=cfg["zp"].shape).astype(np.uint8)
+    if dq == "F8":   # weight bytes are E4M3 codes: keep them finite
+        wq = cfg["weight"].copy()
+        wq[(wq & 0x7f) == 0x7f] = 0x3a
+        cfg["weight"] = wq
+    dq_type = {"INT": clib.DQ_INT, "F4": clib.DQ_F4, "F8": clib.DQ_F8E4M3}[dq]
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"],
+                     None if cfg.get("bias") is None else S.bf16_to_f32(cfg["bias"]),
+                     K=K, N=N, weight_bits=bits, q_group_size=g)
+    x = torch.from_numpy(cfg["x"].view(np.int16)).cuda().view(torch.bfloat16)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.a16mm_dq_launch(w, x, y_f32=y32, dq_type=dq_type)
+    torch.cuda.synchronize()
+    out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    pre = y32.cpu().numpy()
+    w.destroy()
+    xf, wf, sf, zf, bf = f32_valued_a16(cfg)
+    want, want_pre = orc.a16matmul_dynamic(xf, wf, sf, zf, bf, M=M, K=K, N=N, weight_bits=bits, q_group_size=g,
+                                           dq_type={"INT": orc.DQ_INT, "F4": orc.DQ_F4, "F8": orc.DQ_F8E4M3}[dq])
+    assert np.array_equal(pre.view(np.uint32), want_pre.view(np.uint32))
+    assert np.array_equal(out, orc.f32_to_bf16(want))
 
 
 # ---- tpu.MatMul with both operands quantized (MatMul.cpp:447-597) ------------------------------------------------

@@ -558,18 +558,210 @@ int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_
   return MI_SUCCESS;
 }
 
+// ---- the same operation for shapes the fragment kernels above do not take: K that is not a multiple of 128, group
+// sizes other than 32, 64 or whole tiles, weights kept as stored.  A workgroup takes one activation row and 256
+// output channels and walks the groups in order, as A16MatMul.cpp:93-160 does: the row's codes of a group are formed
+// once into LDS (:98-132), every thread then adds code * (weight - zp) over the group for its channel -- integer codes
+// in int32 (exact, the launcher bounds the group), the float code types in double in k order, which is what the
+// checker of this path does as well -- and accumulates prod * (amax / imax) * scale, the bias after group 0, with
+// every fp32 operation rounded separately.  About completeness, not speed.
+struct DqPlainArgs {
+  const uint16_t *x;
+  uint16_t *y;
+  float *y32;
+  const float *bias;
+  int64_t M, K, N;
+  int g, G, bits, chip;
+  float imax;
+  // weights kept as stored: [N][K * bits / 8] bytes, float scale / zp [N][G]
+  const uint8_t *pw;
+  const float *pscale, *pzp;
+  int plain_signed;
+  // tiled weights (see a16_common.h): 16-byte lane slots, scale|zp words (4-bit) or scale + (-zp' * scale) (8-bit)
+  const uint32_t *qw;
+  const uint32_t *sz_t;
+  const uint16_t *scale_t;
+  const float *nzs_t;
+  int64_t k_tiles;
+};
+
+template <int DT, int FLAV>
+__global__ __launch_bounds__(256) void dq_plain_kernel(DqPlainArgs a) {
+  using H = Half16<DT>;
+  extern __shared__ float dqp_codes[];  // the group's codes, then four floats for the row maximum
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t m = blockIdx.y;
+  const int64_t n = (int64_t)blockIdx.x * 256 + tid;
+  const bool live = n < a.N;
+  const int64_t nn = live ? n : a.N - 1;
+  const int64_t rb = nn >> 4;
+  const int c = (int)(nn & 15);
+  float *wmax = dqp_codes + a.g;
+  float out = 0.0f;
+  for (int gi = 0; gi < a.G; ++gi) {
+    const int64_t k_base = (int64_t)gi * a.g;
+    const int len = (int)((a.K - k_base) < a.g ? (a.K - k_base) : a.g);
+    float amax = (float)1e-8;  // :98-108
+    for (int k = tid; k < len; k += 256) {
+      const float v = fabsf(H::to_f32(a.x[m * a.K + k_base + k]));
+      amax = amax > v ? amax : v;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float other = __shfl_xor(amax, o, 64);
+      amax = amax > other ? amax : other;
+    }
+    __syncthreads();  // the previous group's codes and maxima have been read
+    if (lane == 0)
+      wmax[wave] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+    const float step = amax / a.imax;
+    for (int k = tid; k < len; k += 256) {  // :109-132
+      const float v = H::to_f32(a.x[m * a.K + k_base + k]);
+      float code;
+      if constexpr (FLAV == FLAV_INT)
+        code = roundf(v / amax * a.imax);
+      else if constexpr (FLAV == FLAV_F8)
+        code = f8e4m3_to_f32(f8e4m3_from_f32(v / step));
+      else
+        code = f8e4m3_to_f32(f4_code_as_f8(f4e2m1_from_f32(v / step)));
+      dqp_codes[k] = code;
+    }
+    __syncthreads();
+    // this channel's scale and zero point of the group
+    float sc, zp;
+    if (a.pw) {
+      sc = a.pscale[nn * a.G + gi];
+      zp = a.pzp[nn * a.G + gi];
+    } else if (a.bits == 4) {
+      const uint32_t word = a.sz_t[(rb * a.G + gi) * 16 + c];
+      sc = H::to_f32((uint16_t)(word >> 16));
+      zp = (float)(word & 0xffu);
+    } else {
+      sc = H::to_f32(a.scale_t[(rb * a.G + gi) * 16 + c]);
+      const float nzs = a.nzs_t[(rb * a.G + gi) * 16 + c];
+      zp = sc != 0.0f ? rintf(-nzs / sc) : 0.0f;  // exact: nzs is -(zp') * scale without rounding (stored-byte domain)
+    }
+    int isum = 0;
+    double dsum = 0.0;
+    for (int k = 0; k < len; ++k) {
+      const int64_t kk = k_base + k;
+      int q;  // the stored code: a nibble, or a byte in the domain the zero point above belongs to
+      if (a.pw) {
+        if (a.bits == 4) {
+          const uint32_t b = a.pw[nn * (a.K / 2) + (kk >> 1)];
+          q = (int)((kk & 1) ? (b >> 4) : (b & 0xFu));
+        } else {
+          const uint32_t b = a.pw[nn * a.K + kk];
+          q = a.plain_signed ? (int)(int8_t)b : (int)b;
+        }
+      } else if (a.bits == 4) {
+        const int64_t kt = kk >> 7;
+        const int in_tile = (int)(kk & 127), j = in_tile >> 5, kq = (in_tile >> 3) & 3, e = in_tile & 7;
+        const uint32_t d = a.qw[((rb * a.k_tiles + kt) * 64 + kq * 16 + c) * 4 + j];
+        q = (int)((d >> ((e & 1) ? 16 + 4 * (e >> 1) : 4 * (e >> 1))) & 0xFu);
+      } else {
+        const int64_t kt = kk >> 6;
+        const int in_tile = (int)(kk & 63), h = in_tile >> 5, kq = (in_tile >> 3) & 3, e = in_tile & 7;
+        q = (int)((const uint8_t *)a.qw)[((rb * a.k_tiles + kt) * 64 + kq * 16 + c) * 16 + h * 8 + e];
+      }
+      if constexpr (FLAV == FLAV_INT) {
+        isum += (int)dqp_codes[k] * (q - (int)zp);
+      } else {
+        const float wv = FLAV == FLAV_F8 ? f8e4m3_to_f32((uint32_t)q) : f8e4m3_to_f32(f4_code_as_f8((uint32_t)q));
+        const float wz = wv - zp;
+        dsum += (double)dqp_codes[k] * (double)wz;
+      }
+    }
+    const float prod = FLAV == FLAV_INT ? (float)isum : (float)dsum;
+    // :143-150, every operation rounded on its own: plain operators under this file's contract(off) -- the runtime
+    // header's __fmul_rn / __fadd_rn are compiled with contraction allowed and fuse once inlined
+    float t = prod * step;
+    t = t * sc;
+    out = out + t;
+    if (gi == 0 && a.bias)
+      out = out + a.bias[nn];
+  }
+  if (live) {
+    const int64_t o = m * a.N + n;
+    if (a.y32)
+      a.y32[o] = out;
+    a.y[o] = a.chip == MI_CHIP_CV18XX ? round_out16<DT, MI_CHIP_CV18XX>(out) : round_out16<DT, MI_CHIP_BM168X>(out);
+  }
+}
+
+static int a16_dq_plain_launch(const mi_a16_weight *w, int dq_type, float imax, const uint16_t *d_x, int64_t M,
+                               uint16_t *d_y, float *d_y32, hipStream_t stream) {
+  MI_REQUIRE(!w->kn, MI_UNSUPPORTED, "mi_a16mm_dq_launch: untransposed weights have no dynamic-quantization form");
+  MI_REQUIRE(w->g >= 1 && w->g <= 32768, MI_UNSUPPORTED,
+             "mi_a16mm_dq_launch: groups of more than 32768 inputs are not handled");
+  MI_REQUIRE(M <= 65535, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: M out of range for this group size / K");
+  DqPlainArgs a;
+  a.x = d_x;
+  a.y = d_y;
+  a.y32 = d_y32;
+  a.bias = w->bias;
+  a.M = M;
+  a.K = w->K;
+  a.N = w->N;
+  a.g = w->g;
+  a.G = w->G;
+  a.bits = w->bits;
+  a.chip = w->chip;
+  a.imax = imax;
+  a.pw = w->plain ? (const uint8_t *)w->kn_w : nullptr;
+  a.pscale = w->kn_scale;
+  a.pzp = w->kn_zp;
+  a.plain_signed = w->plain_signed;
+  a.qw = (const uint32_t *)w->qweight;
+  a.sz_t = w->sz_t;
+  a.scale_t = w->scale_t;
+  a.nzs_t = w->nzs_t;
+  a.k_tiles = w->k_tiles;
+  const dim3 grid((unsigned)((w->N + 255) / 256), (unsigned)M), block(256);
+  const size_t lds = ((size_t)w->g + 4) * sizeof(float);
+  const bool f16 = w->dtype == MI_DT_F16;
+#define MI_DQP_RUN(DT_, FLAV_)                                                        \
+  {                                                                                   \
+    static LdsLimitOnce lds_limit;                                                    \
+    lds_limit.ensure((const void *)dq_plain_kernel<DT_, FLAV_>, 160 * 1024);          \
+    dq_plain_kernel<DT_, FLAV_><<<grid, block, lds, stream>>>(a);                     \
+  }
+  if (dq_type == MI_DQ_F8E4M3) {
+    if (f16)
+      MI_DQP_RUN(MI_DT_F16, FLAV_F8)
+    else
+      MI_DQP_RUN(MI_DT_BF16, FLAV_F8)
+  } else if (dq_type == MI_DQ_F4) {
+    if (f16)
+      MI_DQP_RUN(MI_DT_F16, FLAV_F4)
+    else
+      MI_DQP_RUN(MI_DT_BF16, FLAV_F4)
+  } else {
+    if (f16)
+      MI_DQP_RUN(MI_DT_F16, FLAV_INT)
+    else
+      MI_DQP_RUN(MI_DT_BF16, FLAV_INT)
+  }
+#undef MI_DQP_RUN
+  MI_HIP(hipGetLastError());
+  return MI_SUCCESS;
+}
+
 int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32,
                   hipStream_t stream) {
   MI_REQUIRE(M >= 0 && M <= 65535 * 16, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: M out of range");
-  MI_REQUIRE(w && w->qweight && (M == 0 || (d_x && d_y)), MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: null argument");
+  MI_REQUIRE(w && (w->qweight || w->plain) && (M == 0 || (d_x && d_y)), MI_BAD_ARGUMENT,
+             "mi_a16mm_dq_launch: null argument");
   MI_REQUIRE(w->g != 0, MI_BAD_ARGUMENT, "mi_a16mm_dq_launch: dynamic quantization needs a group size (A16MatMul.cpp:42)");
   const int g = w->g;
   const int bits = w->bits;
   // A16MatMul.cpp:51-91: F8E4M3 codes are read from 8-bit, F4 codes from 4-bit weights
   MI_REQUIRE(dq_type == MI_DQ_INT || (dq_type == MI_DQ_F8E4M3 && bits == 8) || (dq_type == MI_DQ_F4 && bits == 4),
              MI_UNSUPPORTED, "mi_a16mm_dq_launch: dq_type must be MI_DQ_INT, MI_DQ_F8E4M3 (8-bit weights) or MI_DQ_F4 (4-bit)");
-  MI_REQUIRE((w->K % 128) == 0 && (g == 32 || g == 64 || g % 128 == 0), MI_UNSUPPORTED,
-             "mi_a16mm_dq_launch: K must be a multiple of 128 and the group size 32, 64 or a multiple of 128");
+  // whole 128-wide tiles and groups of 32, 64 or whole tiles take the fragment kernels, everything else the plain one
+  const bool fragments = !w->plain && !w->kn && (w->K % 128) == 0 && (g == 32 || g == 64 || g % 128 == 0);
   // imax: (1 << (weight_bits - 1)) - 1, get_f8e4m3_max() or get_f4e2m1_max(), A16MatMul.cpp:51-61.  The reference's f32
   // group product is exact only while the sums of integer codes stay below 2^24; E2M1 products are quarter units up
   // to 36 (15 with a zero point), E4M3 sums are rounded by the reference as well
@@ -589,6 +781,8 @@ int a16_dq_launch(const mi_a16_weight *w, int dq_type, const uint16_t *d_x, int6
              "mi_a16mm_dq_launch: group too long for the group sums to stay exact in the reference's f32 product");
   if (M == 0)
     return MI_SUCCESS;
+  if (!fragments)
+    return a16_dq_plain_launch(w, dq_type, imax, d_x, M, d_y, d_y32, stream);
   const int64_t m_blocks = (M + 15) / 16, rows_padded = m_blocks * 16;
   const int G = w->G;
   // codes, scales and code sums of this call: the stream's scratch buffer
