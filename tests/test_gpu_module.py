@@ -212,13 +212,24 @@ def test_dynamic_quant_a16matmul_in_a_module(orc, dq, bits):
         y, _ = orc.a16matmul_dynamic(h, w, s, z, None, M=M, K=N, N=128, weight_bits=bits, q_group_size=g, dq_type=odq)
         assert np.array_equal(m.get_tensor("h"), h), rep
         assert np.array_equal(m.get_tensor("y"), y), rep
-    # shapes the dynamic kernels do not handle are refused when the op is added
-    bad = S.w4a16(M, 192, 16, 64, seed=1)  # K is not a multiple of 128
+    # a shape outside the fragment kernels' layout (K is not a multiple of 128) runs on the plain kernel
+    odd = S.w4a16(M, 192, 16, 64, seed=1)
     m2 = M_.Module()
     m2.add_tensor("a", clib.ST_BF16, (M, 192)).add_tensor("b", clib.ST_BF16, (M, 16))
+    m2.add_a16matmul("a", "b", odd["weight"], odd["scale"], odd["zp"], None, K=192, N=16, weight_bits=4,
+                     q_group_size=64, dq_type=clib.DQ_INT)
+    xa, w, s, z, _ = f32_valued_a16(odd)
+    m2.set_tensor("a", xa)
+    m2.invoke()
+    want, _ = orc.a16matmul_dynamic(xa, w, s, z, None, M=M, K=192, N=16, weight_bits=4, q_group_size=64)
+    assert np.array_equal(m2.get_tensor("b"), want)
+    # what the dynamic kernels do not handle is refused when the op is added: an 8-bit group too long to stay exact
+    bad = S.w8a16(M, 1024, 16, 1024, seed=1)
+    m3 = M_.Module()
+    m3.add_tensor("a", clib.ST_BF16, (M, 1024)).add_tensor("b", clib.ST_BF16, (M, 16))
     with pytest.raises(clib.BackendError) as e:
-        m2.add_a16matmul("a", "b", bad["weight"], bad["scale"], bad["zp"], None, K=192, N=16, weight_bits=4,
-                         q_group_size=64, dq_type=clib.DQ_INT)
+        m3.add_a16matmul("a", "b", bad["weight"], bad["scale"], bad["zp"], None, K=1024, N=16, weight_bits=8,
+                         q_group_size=1024, dq_type=clib.DQ_INT)
     assert e.value.code == clib.MI_UNSUPPORTED
 
 
