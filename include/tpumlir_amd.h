@@ -159,7 +159,9 @@ int mi_a16_weight_import(mi_a16_weight **out, const void *blob, size_t size);
  * sums, rescaled and added in group order.  No bias, no relu (the reference applies none on this branch).  Integer
  * types and F4: results are bit-identical to the reference's while its f32 group product is exact (group * imax^2
  * < 2^24 in code units), which is checked.  F8E4M3: exact products, fp32 group sums -- agreement to the fp32 rounding
- * of a group sum, whose order the reference leaves to its matmul library.  K must be a multiple of 64, the group size 32 or a multiple of 64. */
+ * of a group sum, whose order the reference leaves to its matmul library.  With K a multiple of 64 and groups of 32 or
+ * whole 64-element tiles the products run on MFMA kernels; every other K and group size (a last group cut short by K
+ * included) on a plain kernel that follows the reference's loop order. */
 typedef struct mi_matmul_dq_attr {
   int64_t M, K, N;
   int right_transpose;  /* right operand stored [N, K] instead of [K, N] */

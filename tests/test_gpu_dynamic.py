@@ -183,6 +183,36 @@ def test_matmul_dynamic_device_level(orc, M, K, N, g, rt, dq):
     assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), orc.f32_to_bf16(want))
 
 
+MM_PLAIN_CASES = [  # (M, K, N, g, right_transpose, dq_type): outside the fragment kernels' layout
+    (3, 200, 20, 64, True, "DQ_INT8"),       # K is not a multiple of 64; the last group has 8 elements
+    (5, 192, 300, 48, False, "DQ_INT8"),     # groups of 48, more than one block of 256 columns
+    (2, 100, 16, -1, False, "DQ_INT4"),      # one group spanning an odd K
+    (4, 96, 24, 24, True, "DQ_INT4"),
+    (3, 160, 20, 40, False, "DQ_F4"), (2, 200, 16, 64, True, "DQ_F4"),
+    (3, 160, 20, 40, True, "DQ_F8E4M3"), (2, 200, 16, 64, False, "DQ_F8E4M3"),
+]
+
+
+@pytest.mark.parametrize("M,K,N,g,rt,dq", MM_PLAIN_CASES)
+def test_matmul_dynamic_outside_the_fragment_layout(orc, M, K, N, g, rt, dq):
+    """K that is not a multiple of 64, odd group sizes and a last group cut short by K (MatMul.cpp:467-583 as
+    written) run on a plain kernel in the reference's order; bit for bit against the oracle for every code type (its
+    float-code products are double sums in k order, as the kernel's are)."""
+    import torch
+    rng = np.random.default_rng(M + K + N)
+    lb = S.bf16_round((rng.standard_normal((M, K)) * rng.uniform(0.2, 3.0, size=(M, 1))).astype(np.float32))
+    rb = S.bf16_round(rng.standard_normal((N, K) if rt else (K, N)).astype(np.float32))
+    left = torch.from_numpy(lb.view(np.int16)).cuda().view(torch.bfloat16)
+    right = torch.from_numpy(rb.view(np.int16)).cuda().view(torch.bfloat16)
+    y32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    y = M_.matmul_dq_launch(left, right, right_transpose=rt, q_group_size=g, dq_type=getattr(clib, dq), y_f32=y32)
+    torch.cuda.synchronize()
+    kw = dict(imax=127 if dq == "DQ_INT8" else 7) if dq.startswith("DQ_INT") else dict(dq_type=getattr(orc, dq))
+    want, want_pre = orc.matmul_dynamic(S.bf16_to_f32(lb), S.bf16_to_f32(rb), right_transpose=rt, q_group_size=g, **kw)
+    assert np.array_equal(y32.cpu().numpy().view(np.uint32), want_pre.view(np.uint32))
+    assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), orc.f32_to_bf16(want))
+
+
 def test_matmul_dynamic_operator_level_and_rejections(orc):
     rng = np.random.default_rng(77)
     M, K, N, g = 6, 256, 40, 64
@@ -194,9 +224,9 @@ def test_matmul_dynamic_operator_level_and_rejections(orc):
     with pytest.raises(clib.BackendError) as e:
         M_.matmul_dq(left, right, q_group_size=g, dq_type=clib.DQ_INT)   # A16MatMul's name for its integer types
     assert e.value.code == clib.MI_UNSUPPORTED
-    with pytest.raises(clib.BackendError) as e:
-        M_.matmul_dq(left, right, q_group_size=48)
-    assert e.value.code == clib.MI_UNSUPPORTED
+    y48 = M_.matmul_dq(left, right, q_group_size=48)           # 256 = 5 * 48 + 16: a short last group, plain kernel
+    want48, _ = orc.matmul_dynamic(left, right, q_group_size=48)
+    assert np.array_equal(y48, want48)
     with pytest.raises(clib.BackendError) as e:  # 2048 x 127^2 >= 2^24: outside the reference's exact range
         M_.matmul_dq(np.zeros((1, 2048), np.float32), np.zeros((2048, 4), np.float32), q_group_size=2048)
     assert e.value.code == clib.MI_UNSUPPORTED

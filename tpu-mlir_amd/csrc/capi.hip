@@ -1633,8 +1633,6 @@ int mi_matmul_dq_inference(const mi_matmul_dq_attr *a, mi_infer_param *p) {
   MI_REQUIRE(a->out_dtype == MI_DT_BF16 || a->out_dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_matmul_dq_inference: out_dtype");
   const int64_t g = a->q_group_size == -1 ? a->K : a->q_group_size;
   MI_REQUIRE(g > 0, MI_BAD_ARGUMENT, "mi_matmul_dq_inference: dynamic quantization needs a group size");
-  MI_REQUIRE((a->K % 64) == 0 && (g == 32 || (g % 64) == 0) && (a->K % g) == 0, MI_UNSUPPORTED,
-             "mi_matmul_dq_inference: K must be a multiple of 64 and the group size 32 or a multiple of 64");
   if (a->M == 0)
     return MI_SUCCESS;
   MI_REQUIRE(mi_device_count() > 0, MI_HIP_ERROR, "mi_matmul_dq_inference: no GPU visible");

@@ -460,6 +460,141 @@ __global__ __launch_bounds__(DQ_WAVES * 64) void dq2_gemm_kernel(Dq2Args a) {
   }
 }
 
+// ---- tpu.MatMul with both operands quantized, for shapes the fragment kernels do not take (K that is not a multiple
+// of 64, groups other than 32 or whole 64-element tiles, a last group cut short by K): MatMul.cpp:467-583 as
+// written.  A workgroup takes one left row and 256 output columns; per group the row's codes are formed once into
+// LDS, every thread finds its column's abs-max, then adds code * code over the group (int32 for the integer types,
+// double in k order for the float code types, as the checker of this path does) and accumulates
+// prod * (lmax / imax) * (rmax / imax), every fp32 operation rounded on its own.
+struct Dq2PlainArgs {
+  const uint16_t *left, *right;  // [M][K]; [N][K] (right_transpose) or [K][N]
+  uint16_t *y;
+  float *y32;
+  int64_t M, K, N;
+  int g, G, right_transpose;
+  float imax;
+};
+
+template <int DT, int FLAV>
+__device__ __forceinline__ float dq_code_value(float v, float amax, float imax, float step) {
+  if constexpr (FLAV == FLAV_INT)
+    return roundf(v / amax * imax);
+  else if constexpr (FLAV == FLAV_F8)
+    return f8e4m3_to_f32(f8e4m3_from_f32(v / step));
+  else
+    return f8e4m3_to_f32(f4_code_as_f8(f4e2m1_from_f32(v / step)));
+}
+
+template <int DT, int FLAV>
+__global__ __launch_bounds__(256) void dq2_plain_kernel(Dq2PlainArgs a) {
+  using H = Half16<DT>;
+  extern __shared__ float dqp_codes[];  // the left row's codes of the group, then four floats for its maximum
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t m = blockIdx.y;
+  const int64_t n = (int64_t)blockIdx.x * 256 + tid;
+  const bool live = n < a.N;
+  const int64_t nn = live ? n : a.N - 1;
+  float *wmax = dqp_codes + a.g;
+  float out = 0.0f;
+  for (int gi = 0; gi < a.G; ++gi) {
+    const int64_t k_base = (int64_t)gi * a.g;
+    const int len = (int)((a.K - k_base) < a.g ? (a.K - k_base) : a.g);
+    float lmax = (float)1e-8;  // :478-505
+    for (int k = tid; k < len; k += 256) {
+      const float v = fabsf(H::to_f32(a.left[m * a.K + k_base + k]));
+      lmax = lmax > v ? lmax : v;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float other = __shfl_xor(lmax, o, 64);
+      lmax = lmax > other ? lmax : other;
+    }
+    __syncthreads();  // the previous group's codes and maxima have been read
+    if (lane == 0)
+      wmax[wave] = lmax;
+    __syncthreads();
+    lmax = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+    const float lstep = lmax / a.imax;
+    for (int k = tid; k < len; k += 256)
+      dqp_codes[k] = dq_code_value<DT, FLAV>(H::to_f32(a.left[m * a.K + k_base + k]), lmax, a.imax, lstep);
+    __syncthreads();
+    float rmax = (float)1e-8;
+    for (int k = 0; k < len; ++k) {
+      const int64_t kk = k_base + k;
+      const float v = fabsf(H::to_f32(a.right_transpose ? a.right[nn * a.K + kk] : a.right[kk * a.N + nn]));
+      rmax = rmax > v ? rmax : v;
+    }
+    const float rstep = rmax / a.imax;
+    int isum = 0;
+    double dsum = 0.0;
+    for (int k = 0; k < len; ++k) {
+      const int64_t kk = k_base + k;
+      const float rv = H::to_f32(a.right_transpose ? a.right[nn * a.K + kk] : a.right[kk * a.N + nn]);
+      const float rc = dq_code_value<DT, FLAV>(rv, rmax, a.imax, rstep);
+      if constexpr (FLAV == FLAV_INT)
+        isum += (int)dqp_codes[k] * (int)rc;
+      else
+        dsum += (double)dqp_codes[k] * (double)rc;
+    }
+    const float prod = FLAV == FLAV_INT ? (float)isum : (float)dsum;
+    float t = prod * lstep;  // :576-582, left to right
+    t = t * rstep;
+    out = out + t;
+  }
+  if (live) {
+    const int64_t o = m * a.N + n;
+    if (a.y32)
+      a.y32[o] = out;
+    a.y[o] = round_out16<DT, MI_CHIP_BM168X>(out);
+  }
+}
+
+static int matmul_dq_plain_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M,
+                                  int64_t K, int64_t N, int64_t g, int dq_type, float imax, bool f16, uint16_t *d_y,
+                                  float *d_y32, hipStream_t stream) {
+  MI_REQUIRE(g <= 32768, MI_UNSUPPORTED, "mi_matmul_dq_launch: groups of more than 32768 inputs are not handled");
+  MI_REQUIRE(M <= 65535, MI_BAD_ARGUMENT, "mi_matmul_dq_launch: M out of range for this group size / K");
+  Dq2PlainArgs a;
+  a.left = d_left;
+  a.right = d_right;
+  a.y = d_y;
+  a.y32 = d_y32;
+  a.M = M;
+  a.K = K;
+  a.N = N;
+  a.g = (int)g;
+  a.G = (int)((K + g - 1) / g);
+  a.right_transpose = right_transpose;
+  a.imax = imax;
+  const dim3 grid((unsigned)((N + 255) / 256), (unsigned)M), block(256);
+  const size_t lds = ((size_t)g + 4) * sizeof(float);
+#define MI_DQ2P_RUN(DT_, FLAV_)                                                        \
+  {                                                                                    \
+    static LdsLimitOnce lds_limit;                                                     \
+    lds_limit.ensure((const void *)dq2_plain_kernel<DT_, FLAV_>, 160 * 1024);          \
+    dq2_plain_kernel<DT_, FLAV_><<<grid, block, lds, stream>>>(a);                     \
+  }
+  if (dq_type == MI_DQ_F8E4M3) {
+    if (f16)
+      MI_DQ2P_RUN(MI_DT_F16, FLAV_F8)
+    else
+      MI_DQ2P_RUN(MI_DT_BF16, FLAV_F8)
+  } else if (dq_type == MI_DQ_F4) {
+    if (f16)
+      MI_DQ2P_RUN(MI_DT_F16, FLAV_F4)
+    else
+      MI_DQ2P_RUN(MI_DT_BF16, FLAV_F4)
+  } else {
+    if (f16)
+      MI_DQ2P_RUN(MI_DT_F16, FLAV_INT)
+    else
+      MI_DQ2P_RUN(MI_DT_BF16, FLAV_INT)
+  }
+#undef MI_DQ2P_RUN
+  MI_HIP(hipGetLastError());
+  return MI_SUCCESS;
+}
+
 int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_transpose, int64_t M, int64_t K,
                      int64_t N, int q_group_size, int dq_type, int dtype, uint16_t *d_y, float *d_y32,
                      hipStream_t stream) {
@@ -480,13 +615,15 @@ int matmul_dq_launch(const uint16_t *d_left, const uint16_t *d_right, int right_
   MI_REQUIRE(dtype == MI_DT_BF16 || dtype == MI_DT_F16, MI_UNSUPPORTED, "mi_matmul_dq_launch: dtype");
   const int64_t g = q_group_size == -1 ? K : q_group_size;  // MatMul.cpp:465-466
   MI_REQUIRE(g > 0, MI_BAD_ARGUMENT, "mi_matmul_dq_launch: dynamic quantization needs a group size");
-  MI_REQUIRE((K % 64) == 0 && (g == 32 || (g % 64) == 0) && (K % g) == 0, MI_UNSUPPORTED,
-             "mi_matmul_dq_launch: K must be a multiple of 64, the group size 32 or a multiple of 64, K a multiple of "
-             "the group size");
+  // whole 64-element tiles and groups of 32 or whole tiles take the fragment kernels, everything else the plain one
+  const bool fragments = (K % 64) == 0 && (g == 32 || (g % 64) == 0) && (K % g) == 0;
   MI_REQUIRE(g * peak < (1 << 24), MI_UNSUPPORTED,
              "mi_matmul_dq_launch: group too long for the group sums to stay exact in the reference's f32 product");
   if (M == 0)
     return MI_SUCCESS;
+  if (!fragments)
+    return matmul_dq_plain_launch(d_left, d_right, right_transpose, M, K, N, g, dq_type, imax, dtype == MI_DT_F16, d_y,
+                                  d_y32, stream);
   const int G = (int)(K / g);
   const int64_t k_tiles = K / 64;
   const int64_t m_blocks = (M + 15) / 16, n_blocks = (N + 15) / 16;
