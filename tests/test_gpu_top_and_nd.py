@@ -64,14 +64,44 @@ def test_top_a16matmul_refuses_what_it_does_not_handle():
     m = pkg()
     clib = pkg("clib")
     cfg, x, scale, zp, bias = _top_operands(4, 1, 64, 8, 0, seed=2)
-    with pytest.raises(clib.BackendError) as e:     # [N, K] storage: a group of 24 does not divide K = 64
-        m.TopA16MatMul(K=64, N=8, weight_bits=4, q_group_size=24).inference(
+    with pytest.raises(clib.BackendError) as e:     # [N, K] storage: 64 * 8 / 48 is not a whole number of groups
+        m.TopA16MatMul(K=64, N=8, weight_bits=4, q_group_size=48).inference(
             x, cfg["weight"].astype(np.float32), scale, zp, bias)
     assert e.value.code == clib.MI_UNSUPPORTED
     with pytest.raises(clib.BackendError) as e:     # [K, N] storage: 64 * 8 / 48 is not a whole number of groups
         m.TopA16MatMul(K=64, N=8, weight_bits=4, q_group_size=48, right_transpose=False).inference(
             x, cfg["weight"].astype(np.float32), scale, zp, bias)
     assert e.value.code == clib.MI_UNSUPPORTED
+
+
+@pytest.mark.parametrize("bits,M,K,N,g", [(4, 2, 100, 24, 20), (4, 3, 66, 10, 12), (8, 2, 37, 9, 37), (8, 5, 90, 20, 36),
+                                          (4, 1, 96, 8, 64)])     # 64 does not divide K = 96 but divides N * K: groups cross rows
+def test_top_a16matmul_odd_shapes_of_the_transposed_weight(orc, bits, M, K, N, g):
+    """[N, K] weights with K that is not a multiple of 8, groups that are not, groups that cross rows: the flat kernel,
+    against the oracle and bit for bit on one-hot rows."""
+    import torch
+    m = pkg()
+    rng = np.random.default_rng(bits * 1000 + K + N)
+    n_groups = N * K // g
+    wbytes = rng.integers(0, 256, size=N * K * bits // 8, dtype=np.uint8)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    scale = (np.abs(rng.standard_normal(n_groups)) * 0.01 + 1e-4).astype(np.float32)
+    zp = (rng.integers(0, 1 << bits, size=n_groups) + 0.7).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    wf = wbytes.astype(np.float32)
+    ref = orc.top_a16matmul(x, wf, scale, zp, bias, M=M, K=K, N=N, weight_bits=bits, q_group_size=g)
+    op = m.TopA16MatMul(K=K, N=N, weight_bits=bits, q_group_size=g)
+    y = op.inference(x, wf, scale, zp, bias)
+    op.deinit()
+    rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+    assert float(np.max(np.abs(y.astype(np.float64) - ref))) <= TOP_TOL * rms
+    w = m.TopA16Weight(wbytes, scale, zp, None, K=K, N=N, weight_bits=bits, q_group_size=g)
+    eye = torch.eye(K, dtype=torch.float32, device="cuda")
+    got = m.top_a16mm_launch(w, eye)
+    torch.cuda.synchronize()
+    expect = orc.dequant_weight(wf, scale, zp, weight_len=N * K, q_group_size=g, weight_bits=bits).reshape(N, K).T
+    assert np.array_equal(got.cpu().numpy(), expect)
+    w.destroy()
 
 
 @pytest.mark.parametrize("bits,M,K,N,g", [(4, 1, 512, 256, 64), (4, 5, 384, 96, 32), (4, 3, 64, 48, 0),

@@ -12,7 +12,8 @@
 // right_transpose == false: the weight is [K, N] and dequant_weight walks it FLAT (MatMul.cpp:29-40): element
 // e = k * N + n sits in byte e / (8 / bits), and its group is e / q_group_size, so groups run along N inside a row k
 // (and across rows when the group does not divide N).  top_a16_kn_kernel follows that indexing literally: one thread
-// per output column, the k loop in order.
+// per output column, the k loop in order.  The same kernel, with e = n * K + k, takes the [N, K] weights the wave
+// kernel does not: K that is not a multiple of 8, groups that are not, groups that do not divide K.
 #include <math.h>
 
 #include <climits>
@@ -31,6 +32,7 @@ struct TopA16Args {
   float *y;             // [M][N]
   int64_t K, N;
   int M, G, g;
+  int flat_nk;  // flat kernel only: 1 = element (n, k) is n * K + k ([N, K] storage), 0 = k * N + n
 };
 
 template <int BITS, int MR>
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(256) void top_a16_kn_kernel(TopA16Args a) {
   for (int r = 0; r < MR; ++r)
     acc[r] = 0.f;
   for (int64_t k = 0; k < a.K; ++k) {
-    const int64_t e = k * a.N + n;
+    const int64_t e = a.flat_nk ? n * a.K + k : k * a.N + n;
     int q;
     if constexpr (BITS == 4)
       q = (a.w[e >> 1] >> (4 * (int)(e & 1))) & 0xF;
@@ -139,7 +141,8 @@ struct mi_top_a16_weight {
   float *bias = nullptr;
   int64_t K = 0, N = 0;
   int bits = 0, g = 0, G = 0;
-  bool kn = false;  // [K, N] storage, flat groups (right_transpose == false)
+  bool kn = false;  // the flat kernel: [K, N] storage (right_transpose == false), or [N, K] storage it alone takes
+  bool flat_nk = false;
 };
 
 extern "C" {
@@ -154,15 +157,13 @@ int mi_top_a16_weight_create(mi_top_a16_weight **out, int64_t K, int64_t N, int 
   const int g = q_group_size < 1 ? (int)K : q_group_size;  // A16MatMul.cpp:88-91
   int64_t G = 0;     // groups per weight row ([N, K] storage)
   int64_t n_groups;  // scale / zero-point entries in all
-  if (right_transpose) {
-    MI_REQUIRE(K % 8 == 0, MI_UNSUPPORTED, "mi_top_a16_weight_create: K must be a multiple of 8");
-    MI_REQUIRE(K % g == 0 && g % 8 == 0, MI_UNSUPPORTED,
-               "mi_top_a16_weight_create: the group size must divide K and be a multiple of 8");
+  const bool wave_kernel = right_transpose && K % 8 == 0 && K % g == 0 && g % 8 == 0;
+  if (wave_kernel) {
     G = K / g;
     n_groups = N * G;
   } else {
     MI_REQUIRE((N * K) % g == 0 && (N * K) % (8 / weight_bits) == 0, MI_UNSUPPORTED,
-               "mi_top_a16_weight_create: [K, N] storage: the group size must divide N * K");
+               "mi_top_a16_weight_create: the group size must divide N * K (the weight is dequantized as one flat array)");
     n_groups = N * K / g;
   }
   mi_top_a16_weight *t = new mi_top_a16_weight;
@@ -171,7 +172,8 @@ int mi_top_a16_weight_create(mi_top_a16_weight **out, int64_t K, int64_t N, int 
   t->bits = weight_bits;
   t->g = g;
   t->G = (int)G;
-  t->kn = !right_transpose;
+  t->kn = !wave_kernel;
+  t->flat_nk = !wave_kernel && right_transpose;
   std::vector<int32_t> zi((size_t)n_groups);
   for (int64_t i = 0; i < n_groups; ++i)
     zi[(size_t)i] = (int)zp[i];  // (int)(zp_i), MatMul.cpp:36
@@ -217,7 +219,8 @@ int mi_top_a16mm_launch(const mi_top_a16_weight *t, const float *d_x, int64_t M,
   MI_REQUIRE(M >= 0 && M <= INT32_MAX / 2, MI_BAD_ARGUMENT, "mi_top_a16mm_launch: bad M");
   if (M == 0)
     return MI_SUCCESS;
-  MI_REQUIRE(((uintptr_t)d_x & 15) == 0, MI_BAD_ARGUMENT, "mi_top_a16mm_launch: activations must be 16-byte aligned");
+  MI_REQUIRE(t->kn || ((uintptr_t)d_x & 15) == 0, MI_BAD_ARGUMENT,
+             "mi_top_a16mm_launch: activations must be 16-byte aligned");
   TopA16Args a;
   a.w = (const uint8_t *)t->w;
   a.scale = t->scale;
@@ -230,6 +233,7 @@ int mi_top_a16mm_launch(const mi_top_a16_weight *t, const float *d_x, int64_t M,
   a.M = (int)M;
   a.G = t->G;
   a.g = t->g;
+  a.flat_nk = t->flat_nk;
   const int mr = M == 1 ? 1 : 4;
   const int64_t gy = (M + mr - 1) / mr;
   MI_REQUIRE(gy <= 65535 && (t->N + 3) / 4 <= INT32_MAX, MI_UNSUPPORTED, "mi_top_a16mm_launch: too many rows");
