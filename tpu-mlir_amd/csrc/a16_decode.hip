@@ -10,9 +10,9 @@
 //     compares against the sets' first row blocks; the host has pre-subtracted each set's offset from its pointers,
 //     so every address is `pointer of the set + global row block * stride` with no per-set index arithmetic.
 //   * A wave loads ITS slice of the activation rows (one 16-byte request per lane and row for the usual shapes),
-//     parks it in its own corner of LDS, forms the per-group activation sums with cross-lane (DPP) adds, and reads the
-//     MFMA A fragments back, all by itself (no workgroup barrier): a wave starts multiplying as soon as ITS data
-//     has arrived.
+//     parks it in its own corner of LDS, forms the per-group activation sums (one row: cross-lane DPP adds; more
+//     rows: an MFMA against ones beside each product MFMA), and reads the MFMA A fragments back, all by itself (no
+//     workgroup barrier): a wave starts multiplying as soon as ITS data has arrived.
 //   * Tiles are multiplied two at a time -- two independent MFMA chains -- with the LDS reads of both issued before
 //     the wave waits for the weights: with two waves per SIMD there is little else to hide latencies behind.
 //   * Only lanes 0..15 hold live output rows (rows 0..3 of the 16 x 16 MFMA block; with five to eight activation rows
@@ -77,7 +77,12 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(const uint8_t *x
   constexpr int UNITS = TPW * GPT;
   constexpr int SROWS = MR > 4 ? 8 : 4;          // rows whose activation sums are kept per unit
   constexpr int RQ = MR > 4 ? 2 : 1;             // quarter-waves (16 lanes, four rows each) that hold live rows
-  constexpr int S_BYTES = BITS == 4 ? UNITS * SROWS * 4 : 0;
+  // more than one row: the activation sums come from one more MFMA per k-step (against ones: they land in the
+  // accumulator layout the fold reads) instead of vector adds, DPP and a trip through LDS for every row -- the matrix
+  // unit is idle here, the vector unit is not (chain M = 7: 45.9 -> 44.2 us per step, M = 8: 49.0 -> 48.2, M = 4:
+  // 35.4 -> 34.6, three runs each way)
+  constexpr bool SUM_MFMA = BITS == 4 && MR > 1;
+  constexpr int S_BYTES = (BITS == 4 && !SUM_MFMA) ? UNITS * SROWS * 4 : 0;
   constexpr int WAVE_LDS = MR * XROW + S_BYTES;
   constexpr int RED_BYTES = WAVES * RQ * 256;    // partial sums of the final reduction
   static_assert(TPW % 2 == 0, "tiles are taken two at a time");
@@ -173,7 +178,7 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(const uint8_t *x
     for (int ld = 0; ld < XL; ++ld) {
       const int q = ld * 64 + lane;
       *(u32x4 *)(xs + r * XROW + q * 16) = xv[r][ld];
-      if constexpr (BITS == 4) {
+      if constexpr (BITS == 4 && !SUM_MFMA) {
         float part = 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -205,10 +210,16 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(const uint8_t *x
   // Tiles are taken two at a time: the A fragments and activation sums of both are read from LDS before the wave
   // waits for the weights, and the two tiles' MFMA chains are independent, so one chain's latency hides behind the
   // other's unpacking.
-  auto fold4 = [&](const f32x4 &P, int unit, uint32_t szw, bool live) {
+  auto fold4 = [&](const f32x4 &P, const f32x4 &Sm, int unit, uint32_t szw, bool live) {
     const float sc = H::to_f32((uint16_t)(szw >> 16));
     const float c = H::OFFSET + (float)(szw & 0xffu);
-    if constexpr (MR == 1) {  // one live row: register 0
+    if constexpr (SUM_MFMA) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float t = fmaf(-c, Sm[i], P[i]);
+        acc[i] = fmaf(sc, live ? t : 0.0f, acc[i]);
+      }
+    } else if constexpr (MR == 1) {  // one live row: register 0
       const float S0 = s_lds[unit * SROWS];
       const float t = fmaf(-c, S0, P[0]);
       acc[0] = fmaf(sc, live ? t : 0.0f, acc[0]);
@@ -235,15 +246,19 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(const uint8_t *x
         xf[b][j] = *(const u32x4 *)(xfp + ((pb + b) * CPT + 4 * j) * 16);
     }
     if constexpr (BITS == 4) {
-      f32x4 P[NB];
+      f32x4 P[NB], Sm[NB];
+      const u32x4 ones_bits = {H::ONE2, H::ONE2, H::ONE2, H::ONE2};
 #pragma unroll
       for (int b = 0; b < NB; ++b)
-        P[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+        P[b] = Sm[b] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int j = 0; j < KSTEPS; ++j) {
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
+        for (int b = 0; b < NB; ++b) {
           P[b] = H::mfma(__builtin_bit_cast(vec8, xf[b][j]), unpack_nibbles<DT>(w[pb + b][j], nib_magic), P[b]);
+          if constexpr (SUM_MFMA)
+            Sm[b] = H::mfma(__builtin_bit_cast(vec8, xf[b][j]), __builtin_bit_cast(vec8, ones_bits), Sm[b]);
+        }
         if ((j + 1) % KSTEPS_PER_UNIT == 0) {
           const int u = j / KSTEPS_PER_UNIT;
 #pragma unroll
@@ -252,8 +267,8 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(const uint8_t *x
             // the three dead registers are handed to the next fragment's unpacking while the matrix unit has yet to
             // write them (observed: fragments overwritten by late MFMA results).
             asm volatile("" ::"v"(P[b]));
-            fold4(P[b], (pb + b) * GPT + u, szv[pb + b][u], live[b]);
-            P[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+            fold4(P[b], Sm[b], (pb + b) * GPT + u, szv[pb + b][u], live[b]);
+            P[b] = Sm[b] = f32x4{0.f, 0.f, 0.f, 0.f};
           }
         }
       }
@@ -313,7 +328,7 @@ constexpr size_t DEC_MAX_LDS8 = 76 * 1024;  // eight rows: two workgroups on a C
 static size_t decode_lds_bytes(int bits, int gpt, int waves, int tpw, int mr) {
   const int cpt = (bits == 4 ? W4_TILE_K : W8_TILE_K) / 8;
   const int xl = (tpw * cpt + 63) / 64;
-  const size_t wave_lds = (size_t)mr * xl * 64 * 16 + (bits == 4 ? (size_t)tpw * gpt * (mr > 4 ? 32 : 16) : 0);
+  const size_t wave_lds = (size_t)mr * xl * 64 * 16 + ((bits == 4 && mr == 1) ? (size_t)tpw * gpt * 16 : 0);
   return (size_t)waves * 256 * (mr > 4 ? 2 : 1) + (size_t)waves * wave_lds;
 }
 
