@@ -18,6 +18,11 @@ ROWS32_W4_CASES = [  # (M, K, N, g, dtype)
     (17, 512, 64, 128, "bf16"), (32, 1024, 200, 0, "bf16"), (9, 128, 48, 128, "f16"), (24, 256, 272, 256, "f16"),
     (32, 4096, 1024, 128, "bf16"), (1, 128, 16, 128, "bf16"), (20, 2048, 520, 512, "bf16"), (31, 1536, 136, 64, "f16"),
     (18, 1920, 100, 64, "bf16"), (32, 3200, 40, 128, "bf16"), (25, 1152, 33, 0, "f16"),
+    # up to 16 rows (the 16 x 16 x 32 form: activations a tile ahead up to 8 rows, piece by piece above): one tile, a
+    # ragged number of tiles per wave, two groups per tile, per-channel scales, channel counts off the 32-block
+    (8, 1152, 48, 128, "bf16"), (5, 4096, 72, 128, "f16"), (16, 1920, 100, 64, "bf16"), (12, 2048, 264, 64, "f16"),
+    (3, 8192, 64, 0, "bf16"), (13, 3200, 40, 128, "bf16"), (16, 128, 33, 128, "f16"), (7, 256, 16, 256, "bf16"),
+    (2, 128, 48, 64, "f16"), (10, 1024, 520, 512, "bf16"),
 ]
 
 
@@ -51,7 +56,8 @@ def test_w4_up_to_32_rows_against_oracle(orc, plan, M, K, N, g, dt):
 
 
 @pytest.mark.parametrize("M,K,Ns,g,dt", [(20, 512, (100, 64, 33), 128, "bf16"), (32, 1024, (48, 272), 64, "bf16"),
-                                        (17, 256, (16, 40, 96, 130), 0, "f16")])
+                                        (17, 256, (16, 40, 96, 130), 0, "f16"), (8, 1152, (100, 64, 33), 128, "f16"),
+                                        (14, 512, (48, 272), 64, "bf16"), (4, 4096, (16, 40, 96, 130), 128, "bf16")])
 def test_w4_sibling_sets_share_a_launch(orc, plan, M, K, Ns, g, dt):
     """q/k/v-style groups, channel counts that are not multiples of 32 included: each set's output against the oracle."""
     import torch
@@ -130,6 +136,7 @@ SPLIT_CASES = [  # (bits, M, K, N, g, parts, dtype): the K of a 32-channel block
     (4, 32, 4096, 1024, 128, 2, "bf16"), (4, 17, 4096, 520, 128, 4, "bf16"), (4, 24, 384, 100, 128, 4, "f16"),
     (4, 32, 11008, 96, 64, 4, "bf16"), (4, 9, 128, 33, 0, 2, "bf16"), (8, 32, 4096, 1024, 0, 2, "bf16"),
     (8, 20, 11008, 200, 64, 4, "bf16"), (8, 31, 192, 40, 64, 4, "f16"), (8, 12, 64, 16, 0, 2, "f16"),
+    (4, 8, 11008, 96, 128, 2, "bf16"), (4, 16, 4096, 520, 64, 4, "f16"), (4, 6, 384, 100, 128, 4, "bf16"),
 ]
 
 

@@ -348,9 +348,220 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
 #undef R32_SEL
 }
 
+// 4-bit weights, up to 16 rows: the same streaming design on the 16 x 16 x 32 MFMA.  With at most 16 rows the
+// 32 x 32 x 16 instruction spends half of its rows on nothing and takes twice the matrix-pipe time per weight element;
+// here a wave multiplies its tile's two 16-channel row blocks separately (lane (channel, k-quarter) holds exactly the
+// B fragments of its slot of a packed tile, as in the decode kernel), one activation-sum MFMA serves both, and a lane
+// carries 8 accumulators instead of 16 (plus 12 instead of 32 for the group's products and sums).
+template <int DT, int GPT, int NQ>
+__global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
+  using H = Half16<DT>;
+  using vec8 = typename H::vec8;
+  static_assert(NQ == 1 || NQ == 2, "up to 16 rows");
+  constexpr int WAVES = 8;
+  constexpr int WL = 2 + 2 * GPT;  // weight-side requests per tile: two row blocks' slots and their scale|zp words
+  constexpr int SLOT_ROWS = 8 * NQ, SLOT = SLOT_ROWS * 128;  // an activation piece: the rows that exist x 64 K
+  // Up to 8 rows a wave asks for a tile's activations a whole tile ahead (XR = 2 tiles in LDS); with 16 rows, piece by
+  // piece as the 32-row kernels do (4096 x 4096, 16 rows: 6.8 against 7.3 us that way round; 8 rows: 6.5 against 6.3).
+  constexpr int XR = NQ == 1 ? 2 : 1, WR = 3;  // activation ring in LDS and weight ring in registers, in tiles
+  constexpr int RING_BYTES = WAVES * XR * 2 * SLOT, RED_BYTES = WAVES * 8 * 256;
+  // The partial sums have a place of their own behind the rings (48 KiB in all): no barrier before they are written,
+  // and a request into a ring that is still on its way when a wave leaves the loop has nothing to land on.
+  constexpr int FLAG_AT = RING_BYTES + RED_BYTES;
+  __shared__ __attribute__((aligned(16))) uint8_t smem[FLAG_AT + 16];
+  float (*red)[8][64] = reinterpret_cast<float (*)[8][64]>(smem + RING_BYTES);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, kq = lane >> 4;
+  const int bid = blockIdx.x >> a.split.shift;  // the launch's 32-channel block; its K part: the low bits
+  const int t1 = bid >= a.block_begin[1], t2 = bid >= a.block_begin[2], t3 = bid >= a.block_begin[3];
+#define R32_SEL(f) (t3 ? a.f[3] : t2 ? a.f[2] : t1 ? a.f[1] : a.f[0])
+  const int lb = bid - R32_SEL(block_begin);  // the set's own 32-channel block
+  const int64_t set_n = R32_SEL(N);
+  const int set_rbs = R32_SEL(row_blocks);
+
+  const uint8_t *wp[2];
+  const uint32_t *szp[2];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    int64_t rb = (int64_t)lb * 2 + b;
+    rb = rb < set_rbs ? rb : set_rbs - 1;  // a row block past N repeats the last one; never stored
+    wp[b] = R32_SEL(qw) + rb * a.k_tiles * 1024 + (uint32_t)(lane * 16);
+    szp[b] = R32_SEL(sz) + rb * a.G * 16 + col;
+  }
+  const uint8_t *xg[NQ];
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) {
+    const int r = 8 * i + (lane >> 3);
+    const int rr = r < a.M ? r : a.M - 1;
+    xg[i] = a.x + (int64_t)rr * a.K * 2 + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+  }
+  uint8_t *xs = smem + wave * (XR * 2 * SLOT);
+  const int frow = col & (SLOT_ROWS - 1);  // fragment rows past the slot re-read a row that exists; never stored
+  const uint8_t *xf = xs + frow * 128;
+
+  // this wave's tiles: first, first + stride, ... (see a16_rows32_kernel)
+  const int first = (blockIdx.x & ((1 << a.split.shift) - 1)) * WAVES + wave, stride = WAVES << a.split.shift;
+  const int count = (a.k_tiles - first + stride - 1) / stride;
+  auto tile_of = [&](int i) { return first + i * stride; };
+  u32x4 w[WR][2];            // weight ring: [tile % WR][row block]: the lane's four k-steps of 8 nibbles
+  uint32_t szw[WR][2][GPT];  // the tile's scale|zp words
+  // A request past the wave's last tile keeps the static request count the waits rely on.  For weights it moves
+  // nothing: all lanes ask for the same 16 bytes at the start of the buffer (one cache line, resident after the first
+  // time).  For activations it repeats the wave's last tile: with a request of that one-address kind as the wave's
+  // last one into LDS, the partial sums that overlay the rings after the loop came out overwritten.
+  const uint8_t *w_idle = R32_SEL(qw);
+  const uint32_t *sz_idle = R32_SEL(sz);
+  auto issue_x = [&](int i, int p) {  // piece p (K elements 64 p .. 64 p + 63) of the wave's i-th tile
+    const int64_t koff = (int64_t)tile_of(i < count ? i : count - 1) * 256 + p * 128;
+    uint8_t *slot = xs + ((i % XR) * 2 + p) * SLOT;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q)
+      __builtin_amdgcn_global_load_lds((r32_gptr_t)(xg[q] + koff), (r32_lptr_t)(slot + q * 1024), 16, 0, 0);
+  };
+  auto issue_w = [&](int i, int rs) {
+    const bool real = i < count;
+    const int kt = tile_of(i);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      w[rs][b] = r32_load16(real ? wp[b] + (int64_t)kt * 1024 : w_idle);
+#pragma unroll
+      for (int u = 0; u < GPT; ++u)
+        szw[rs][b][u] = r32_load4(real ? szp[b] + (GPT == 1 ? (kt >> a.group_shift) : kt * GPT + u) * 16 : sz_idle);
+    }
+  };
+
+  f32x4 acc[2], P[2], S;
+#pragma unroll
+  for (int b = 0; b < 2; ++b)
+    acc[b] = P[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  S = f32x4{0.f, 0.f, 0.f, 0.f};
+  const u32x4 ones_bits = {H::ONE2, H::ONE2, H::ONE2, H::ONE2};
+  const vec8 ones = __builtin_bit_cast(vec8, ones_bits);
+  uint32_t nib_magic = H::NIB_MAGIC2;
+  asm volatile("" : "+v"(nib_magic));  // keep it in a VGPR (see and_or)
+
+  if (count > 0) {
+    // Requests, oldest first.  The counter retires in order, so a wait for an activation piece is a wait for every
+    // request before it.
+    //   XR = 2:  w(0) x(0) w(1) | x(1) w(2) | x(2) w(3) | ...      the wait at tile t leaves w(t + 1), x(t + 1), w(t + 2)
+    //   XR = 1:  w(0) w(1) x(0,0) | x(0,1) w(2) | x(1,0) | x(1,1) w(3) | ...   as in a16_rows32_w4_kernel
+    issue_w(0, 0);
+    if (XR == 2) {
+      issue_x(0, 0);
+      issue_x(0, 1);
+    }
+    issue_w(1, 1);
+    if (XR == 1)
+      issue_x(0, 0);
+    for (int t0 = 0; t0 < count; t0 += WR) {
+#pragma unroll
+      for (int u = 0; u < WR; ++u) {
+        const int t = t0 + u;
+        if (t >= count)
+          break;
+        const uint8_t *xt = xf + (t % XR) * (2 * SLOT);
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          if (XR == 2) {
+            if (p == 0) {
+              issue_x(t + 1, 0);
+              issue_x(t + 1, 1);
+              issue_w(t + 2, (u + 2) % WR);
+              __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(2 * NQ + 2 * WL));
+            }
+          } else {
+            if (p == 0) {
+              issue_x(t, 1);
+              issue_w(t + 2, (u + 2) % WR);
+            } else {
+              issue_x(t + 1, 0);
+            }
+            __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(NQ + WL));
+          }
+          asm volatile("" ::: "memory");  // the piece is in LDS from here on, not before
+          if (p == 0) {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+              r32_arrived(w[u][b]);
+#pragma unroll
+              for (int g = 0; g < GPT; ++g)
+                r32_arrived(szw[u][b][g]);
+            }
+          }
+          u32x4 fa[2];
+#pragma unroll
+          for (int s = 0; s < 2; ++s)
+            fa[s] = *(const u32x4 *)(xt + p * SLOT + (((4 * s + kq) ^ ((frow >> 1) & 7)) << 4));
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {  // k-step 2 p + s of the tile
+            const vec8 af = __builtin_bit_cast(vec8, fa[s]);
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+              P[b] = H::mfma(af, unpack_nibbles<DT>(w[u][b][2 * p + s], nib_magic), P[b]);
+            S = H::mfma(af, ones, S);
+          }
+          if (GPT == 2 || p == 1) {  // end of a quantization group (or of the tile: the same words again next tile)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+              const uint32_t szv = szw[u][b][GPT == 2 ? p : 0];
+              const float sc = H::to_f32((uint16_t)(szv >> 16));
+              const float c = H::OFFSET + (float)(szv & 0xffu);
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                acc[b][i] = fmaf(sc, fmaf(-c, S[i], P[b][i]), acc[b][i]);
+              P[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+            S = f32x4{0.f, 0.f, 0.f, 0.f};
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(r32_waitcnt_vm(0));  // the idle requests issued past the end
+#pragma unroll
+    for (int rs = 0; rs < WR; ++rs)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        r32_arrived(w[rs][b]);
+#pragma unroll
+        for (int g = 0; g < GPT; ++g)
+          r32_arrived(szw[rs][b][g]);
+      }
+  }
+
+  // ---- cross-wave sum, in wave order: register 4 b + i of a lane is row 4 kq + i of channel 16 b + col
+#pragma unroll
+  for (int b = 0; b < 2; ++b)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      red[wave][4 * b + i][lane] = acc[b][i];
+  __syncthreads();
+  float v[2] = {0.f, 0.f};  // wave w finishes register w; the second slot only fills the K-split record
+#pragma unroll
+  for (int wv = 0; wv < WAVES; ++wv)
+    v[0] += red[wv][wave][lane];
+  if (a.split.shift != 0 && !r32_join_parts(v, a.split, wave, lane, reinterpret_cast<int *>(smem + FLAG_AT)))
+    return;
+  const int b = wave >> 2, i = wave & 3;
+  const int orow = 4 * kq + i;
+  const int64_t n = (int64_t)lb * 32 + b * 16 + col;
+  if (orow < a.M && n < set_n) {
+    const float *biasp = R32_SEL(bias);
+    float *y32 = R32_SEL(y32);
+    uint16_t *y = R32_SEL(y);
+    const float o32 = v[0] + (biasp ? biasp[n] : 0.f);
+    const int64_t o = (int64_t)orow * set_n + n;
+    if (y32)
+      y32[o] = o32;
+    y[o] = a.chip == MI_CHIP_CV18XX ? round_out16<DT, MI_CHIP_CV18XX>(o32) : round_out16<DT, MI_CHIP_BM168X>(o32);
+  }
+#undef R32_SEL
+}
+
 // Weight sets in the tiled layout whose K is a whole number of tiles: 8-bit with one scale per channel or groups of
 // 64 * 2^k; 4-bit with groups of 64, of 128 * 2^k, or one per channel.  `blocks`: 32-channel blocks of the whole launch (all sibling sets).
-// Taken for 17 to 32 rows, and below that from where it was measured ahead.  bf16, the kernels otherwise taken
+// Taken for 17 to 32 rows, and below that from where it was measured ahead (the 4-bit figures up to 16 rows are of
+// the 32 x 32 x 16 form; the 16 x 16 x 32 form that runs there now has its own table below).  bf16, the kernels otherwise taken
 // (decode / skinny up to 16 rows, tiled + split-K above) / this one without K split, in us (with the split, which
 // the long-K cases on part of the chip need to stay ahead: the table at rows32_split_shift):
 //   8-bit  11008 x 4096   M = 4: 10.9 / 13.2   M = 8: 15.8 / 13.4   M = 12: 17.2 / 13.9   M = 16: 22.2 / 14.4   M = 17: 28.5 / 14.9   M = 32: 29.3 / 17.5
@@ -397,9 +608,6 @@ bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
   //   8-bit  5120 x 5120    M = 1:  9.2 /  8.2   M = 4: 13.0 /  8.2   M = 16: 20.5 /  8.7
   //   8-bit  6656 x 6656    M = 2: 15.5 / 11.8   M = 8: 17.4 / 11.7      8-bit  8192 x 8192   M = 2: 19.4 / 16.5   M = 6: 25.8 / 16.5
   //   8-bit  4096 x 4096    M = 5:  6.3 /  7.4   M = 16: 7.9 /  7.6      8-bit  6144 x 2048   M = 8:  6.7 /  6.2   M = 16: 7.9 / 6.2
-  //   4-bit  5120 x 5120    M = 3:  8.8 /  8.3   M = 4: 11.7 /  8.4   M = 16: 19.8 /  8.6
-  //   4-bit  13824 x 5120   M = 4: 22.4 / 13.8   M = 8: 15.8 / 13.9      4-bit  8192 x 8192   M = 5: 13.2 / 12.3   M = 6: 15.7 / 12.7
-  //   4-bit  4096 x 11008   M = 5: 11.1 / 11.9   M = 6: 13.8 / 11.6      4-bit  32000 x 4096  M = 8: 20.8 / 22.5 (tiled kernel ahead)
   const bool long_k = w->K >= 8192, mid_k = w->K > 4096 && w->K < 8192;
   if (w->bits == 8) {
     if (M >= 5)
@@ -408,12 +616,34 @@ bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
     // (8192 x 8192 M = 1: 17.4 / 15.7; 5120 x 13824: 20.0 / 17.8; but 28672 x 8192: 48.7 / 49.8)
     return w->K > 4096 && blocks >= 128 && (M >= 2 || (blocks >= 160 && blocks <= 512));
   }
-  if (long_k && M >= 3 && (blocks >= 160 || (M >= 6 && blocks >= 64)))  // 28672 x 8192 M = 4: 44.1 / 36.0
+  // 4-bit, up to 16 rows: the 16 x 16 x 32 form of this kernel.  Others / this one, us, bf16, groups of 128:
+  //   28672 x 8192  M = 2: 31.2 / 26.7   M = 4: 39.7 / 26.6      8192 x 8192   M = 2: 12.4 / 10.6   M = 3: 13.8 / 10.2   M = 8: 15.7 / 10.9
+  //   4096 x 11008  M = 2:  9.8 /  9.9   M = 3: 10.6 /  9.8   M = 4: 11.8 / 10.3   M = 8: 14.5 / 10.3
+  //   5120 x 5120   M = 2:  8.1 /  6.8   M = 8: 14.2 /  7.3       13824 x 5120  M = 2: 13.5 / 11.6   M = 8: 16.6 / 12.2
+  if (long_k && ((M >= 2 && blocks >= 160) || (M >= 3 && blocks >= 64)))
     return true;
-  if (mid_k && blocks >= 128 && M >= 4)
+  if (mid_k && blocks >= 128 && M >= 2)
     return true;
-  // very wide sets are the tiled kernel's from 8 rows on (32000 x 4096 M = 12: 20.7 / 23.1)
-  return (M >= 12 && ((blocks >= 192 && blocks <= 768) || long_k)) || (M >= 8 && blocks >= 512 && blocks <= 768);
+  if (long_k || mid_k)
+    return false;
+  // K up to 4096: the decode kernel's four- and eight-row forms (1 to 4, 7 and 8 rows) stay ahead on launches of up to
+  // two workgroups per CU.
+  //   22016 x 4096  M = 4: 12.4 / 14.2   M = 5: 17.0 / 14.3   M = 7: 16.2 / 14.1   M = 8: 20.0 / 14.0   M = 16: 19.1 / 16.1
+  //   32000 x 4096  M = 4: 15.0 / 17.4   M = 5: 22.4 / 17.4   M = 8: 21.2 / 17.4   M = 12: 20.9 / 19.0   M = 16: 20.4 / 19.5
+  //   11008 x 4096  M = 5:  9.8 /  9.6   M = 8:  9.0 /  9.8   M = 9: 11.2 / 10.4   M = 12: 12.8 / 10.6   M = 16: 14.5 / 11.2
+  //    8192 x 4096  M = 5:  7.6 /  6.8   M = 8:  6.8 /  7.0   M = 9:  8.5 /  7.3   M = 12:  9.6 /  7.4   M = 16: 11.0 /  7.6
+  //    4096 x 4096  M = 8:  4.8 /  6.1   M = 12: 6.4 /  6.6   M = 14: 6.5 /  6.6   M = 16:  7.0 /  6.7
+  //    2048 x 4096  M = 8:  4.2 /  5.3   M = 10: 5.5 /  5.6   M = 12: 5.9 /  5.6   M = 16:  6.5 /  5.6
+  //    6144 x 2048, groups of 64   M = 5: 5.1 / 5.1   M = 7: 5.4 / 5.1   M = 8: 5.6 / 5.1   M = 12: 6.2 / 5.4   M = 16: 6.9 / 5.4
+  if (blocks > 1024)
+    return false;
+  if (M >= 16 || (M >= 12 && blocks <= 96))
+    return true;
+  if (M >= 9 && blocks >= 192)
+    return true;
+  if (M >= 7)
+    return blocks >= 512 || (blocks >= 192 && w->K <= 2048);
+  return M >= 5 && blocks >= 256;
 }
 
 // K parts per 32-channel block of a launch of `blocks` blocks over K: doubled while the launch stays within one
@@ -577,16 +807,23 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
     else                                                                         \
       a16_rows32_w4_kernel<MI_DT_BF16, GPT_, NQ_><<<grid, block, 0, stream>>>(a); \
   }
-#define MI_R32_4Q(GPT_) \
-  {                     \
-    if (nq == 1)        \
-      MI_R32_4(GPT_, 1) \
-    else if (nq == 2)   \
-      MI_R32_4(GPT_, 2) \
-    else if (nq == 3)   \
-      MI_R32_4(GPT_, 3) \
-    else                \
-      MI_R32_4(GPT_, 4) \
+#define MI_R16_4(GPT_, NQ_)                                                      \
+  {                                                                              \
+    if (f16)                                                                     \
+      a16_rows16_w4_kernel<MI_DT_F16, GPT_, NQ_><<<grid, block, 0, stream>>>(a);  \
+    else                                                                         \
+      a16_rows16_w4_kernel<MI_DT_BF16, GPT_, NQ_><<<grid, block, 0, stream>>>(a); \
+  }
+#define MI_R32_4Q(GPT_)  /* up to 16 rows: the 16 x 16 x 32 form */ \
+  {                       \
+    if (nq == 1)          \
+      MI_R16_4(GPT_, 1)   \
+    else if (nq == 2)     \
+      MI_R16_4(GPT_, 2)   \
+    else if (nq == 3)     \
+      MI_R32_4(GPT_, 3)   \
+    else                  \
+      MI_R32_4(GPT_, 4)   \
   }
     if (w->g == 64)
       MI_R32_4Q(2)
@@ -594,6 +831,7 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
       MI_R32_4Q(1)
 #undef MI_R32_4Q
 #undef MI_R32_4
+#undef MI_R16_4
   }
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;
