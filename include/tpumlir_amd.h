@@ -263,7 +263,10 @@ int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint
  * few channels) -- lives in a 16 MiB device array inside the library (one copy per GPU, held until the process ends)
  * instead of the stream's growable buffer.  A product whose slabs need more than 16 MiB - 1 KiB (tiled kernel:
  * k_splits * M * N * 4 bytes; e.g. M = 128, N = 4096 with 4 splits is 8 MiB) is refused with MI_BAD_ARGUMENT and a
- * message that says so.  The slabs need no clearing (every element read is written by the same launch); the array's
+ * message that says so.  One exception to both: where mi_a16mm_launch cuts K in 2 to 4 parts for speed alone (the
+ * widest output block of large 4-bit products, e.g. M = 1024 at 4096 x 4096) and those slabs would not fit, this entry
+ * point runs the product unsplit instead of refusing it -- the same result up to the order of the fp32 partial sums,
+ * as between two K splits of mi_a16mm_launch itself.  The slabs need no clearing (every element read is written by the same launch); the array's
  * first KiB holds the 32-row kernel's arrival counters, which start as zeros and which every launch leaves at zero.
  * Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two threads)
  * race -- serialize them. */

@@ -128,7 +128,9 @@ def _exact_properties(torch, cfg, w, M):
 
 # (label, bits, K, N, g, Ms): every BASELINE configuration / M not already run at full size elsewhere
 FULL_SIZE = [
-    ("cfg3 W4 g128 4096x4096 prefill", 4, 4096, 4096, 128, (1024,)),
+    ("cfg3 W4 g128 4096x4096 prefill", 4, 4096, 4096, 128, (640, 1024)),   # the widest block with K in 3 and 2 parts
+    ("W4 g128 gate/up 11008x4096 prefill", 4, 4096, 11008, 128, (256, 1024)),  # ... in 2 parts: one round, three rounds
+    ("W4 g128 down 4096x11008 prefill", 4, 11008, 4096, 128, (512,)),          # ... in 4 parts
     ("cfg4 W8 per-channel 11008x4096", 8, 4096, 11008, 0, (32, 512)),
     ("cfg5 W4 g128 q_proj 4096x4096", 4, 4096, 4096, 128, (8, 32)),
     ("cfg5 W4 g128 gate/up 11008x4096", 4, 4096, 11008, 128, (8, 32)),

@@ -75,6 +75,7 @@ struct GemmArgs {
   int k_splits, kt_per_split;
   float *slab;
   int64_t slab_stride;
+  int want_splits;  // host side only: K splits chosen with the block shape (0: the launch's own rule)
 };
 
 // WM x WN waves, each TM x TN MFMA tiles of 16 x 16:  GM = WM * TM * 16 rows, GN = WN * TN * 16 columns.
@@ -570,16 +571,23 @@ static int launch_gemm_instance(GemmArgs &a, hipStream_t st, const A16Scratch *f
   // split K when the output blocks alone leave most of the 256 CUs idle: enough workgroups for one per CU, at least
   // four stages each
   const int kt_all = (int)(a.K / GEMM_KS);
+  a.slab_stride = (acc_elems + 3) & ~(int64_t)3;  // slabs stay 16-byte aligned
   int splits = 1;
-  if (plan().a16_gemm_splits > 0)
+  if (plan().a16_gemm_splits > 0) {
     splits = plan().a16_gemm_splits;
-  else if (tiles < 160 && n4)
+  } else if (a.want_splits > 0) {
+    // a split made for speed, not for want of workgroups: the caller's fixed scratch area may be too small for it, and
+    // then the product runs unsplit (same result up to the order of the fp32 partial sums)
+    splits = n4 ? a.want_splits : 1;
+    if (fixed && (size_t)splits * a.slab_stride * sizeof(float) > fixed->bytes)
+      splits = 1;
+  } else if (tiles < 160 && n4) {
     splits = std::min(std::max(256 / (int)tiles, 1), std::max(kt_all / 4, 1));
+  }
   splits = std::max(1, std::min(splits, kt_all));
   a.kt_per_split = (kt_all + splits - 1) / splits;
   a.k_splits = (kt_all + a.kt_per_split - 1) / a.kt_per_split;  // no empty split
   a.slab = nullptr;
-  a.slab_stride = (acc_elems + 3) & ~(int64_t)3;  // slabs stay 16-byte aligned
   if (a.k_splits > 1) {
     MI_REQUIRE(n4, MI_BAD_ARGUMENT, "a16 split-K product: N must be a multiple of 4");
     // fp32 partial sums, one slab per split: the caller's fixed scratch, or the stream's own buffer.  Every element a
@@ -645,7 +653,39 @@ static int launch_gemm_shape(GemmArgs &a, hipStream_t st, const A16Scratch *fixe
   constexpr bool hoists = gemm_hoists<BITS, GPT, 4, 4>();
   int rows = plan().a16_gemm_rows;
   bool wide = fits && tile == 256;
-  if (tile == 0 && rows == 0 && big >= 160) {
+  a.want_splits = 0;
+  // Where the widest block takes the zero-point term out of its loop (4-bit, groups of at least 128) and K >= 4096 it
+  // is the fastest shape per output, and what is left to choose is how its workgroups fill the 256 CUs: one such
+  // block keeps a CU for 85 us per 4096 of K, so a launch of `big` blocks takes ceil(big / 256) rounds of that, and
+  // cutting K in s parts gives s times the workgroups, each 1 / s as long, plus a pass over the fp32 partial sums
+  // (4 us + 10 bytes per output at 5 TB/s for two parts).  Measured, us, unsplit / split (best other shape):
+  //   4096 x 4096    M = 640: 80 / 44 in three parts (55)   M = 1024: 87 / 55 (60)   M = 3072: 171 / 154   M = 2048: 96 / 103
+  //   11008 x 4096   M = 256: 81 / 52 (55)   M = 1024: 170 / 145 (177)   M = 1536: 252 / 233   M = 2048: 256 / 279
+  //   4096 x 11008   M = 512: 184 / 70 in four parts (78)   M = 1024: 192 / 116 (144)   M = 3072: 388 / 328
+  //   8192 x 8192    M = 256: 148 / 55 in four parts (62)   M = 1280: 289 / 237   M = 2048: 313 / 328
+  // but 4096 x 4096 M = 512: 39 in four parts against 38 from 64-row blocks, 4096 x 11008 M = 256: 60 against 47.
+  bool decided = false;
+  if constexpr (hoists && fits) {
+    if (tile == 0 && rows == 0 && plan().a16_gemm_splits == 0 && a.K >= 4096) {
+      double outputs = 0;
+      for (int i = 0; i < a.n_seg; ++i)
+        outputs += (double)a.M * (double)a.seg[i].N;
+      if (big >= 160) {
+        const double r1 = (double)((big + 255) / 256), r2 = (double)((2 * big + 255) / 256) / 2.0;
+        const double saved = (r1 - r2) * 85.0 * (double)a.K / 4096.0, pass = 4.0 + outputs * 10.0 / 5e6;
+        wide = decided = true;
+        a.want_splits = saved > pass ? 2 : 1;
+      } else {
+        const int s = (int)std::min<int64_t>(4, 256 / big);
+        const bool rows_fill = a.M >= 256 && a.M * 5 >= ((a.M + 127) / 128) * 128 * 4;  // at most a fifth of the rows idle
+        if (rows_fill && big * s >= 160 && (t64 > 256 || (a.K >= 8192 && t64 >= 192))) {
+          wide = decided = true;
+          a.want_splits = s;
+        }
+      }
+    }
+  }
+  if (!decided && tile == 0 && rows == 0 && big >= 160) {
     const double c_wide = fits ? (hoists ? 82.0 : 94.0) * (double)((big + 255) / 256) : 1e30;
     const double c_128 = 50.5 * (double)((t128 + 255) / 256);
     const double c_64 = 35.0 + 24.5 * (double)((t64 + 255) / 256 - 1);
@@ -664,7 +704,7 @@ static int launch_gemm_shape(GemmArgs &a, hipStream_t st, const A16Scratch *fixe
   //   4-bit: 64-row blocks up to M = 640 at K = 4096 (measured), 128 rows from M = 256 when K is longer and 64 such
   //   blocks exist (4096 x 11008 M = 384: 71.2 -> 62.8; 8192 x 8192 M = 512: 110.5 -> 97.9; 5120 x 5120 M = 256:
   //   37.0 -> 30.7; but 1024 x 8192 M = 256: 18.4 with 64 rows, 22.6 with 128)
-  if (tile == 0 && rows == 0 && !wide && a.M > 32) {
+  if (!decided && tile == 0 && rows == 0 && !wide && a.M > 32) {
     bool n_past_4096 = false;
     for (int i = 0; i < a.n_seg; ++i)
       n_past_4096 = n_past_4096 || a.seg[i].N > 4096;
