@@ -311,7 +311,8 @@ def bench_single_matmuls(pkg, S, torch, steps=60):
             with torch.cuda.graph(g_, stream=stream):
                 for w in ws:
                     pkg.a16mm_launch(w, x, y)
-        sec = _time_launches(torch, g_.replay, max(3, steps // copies)) / copies
+        # prefill launches are timed warm: the first ten milliseconds after a pause read 5-15 % slow on this machine
+        sec = _time_launches(torch, g_.replay, max(3, steps // copies), warmup=5 if M <= 32 else 40) / copies
         nbytes = S.w4_gemv_bytes(M, K, N, g) if bits == 4 else S.w8_gemv_bytes(M, K, N, g)
         rec = {"case": tag, "bits": bits, "M": M, "K": K, "N": N, "g": g, "us": round(sec * 1e6, 2)}
         if M <= 32:
