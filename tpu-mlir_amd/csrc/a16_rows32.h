@@ -15,6 +15,17 @@ __device__ __forceinline__ u32x4 r32_load16(const void *p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
   return v;
 }
+// the same from a wave-uniform base (two SGPRs) plus a lane's 32-bit byte offset: no vector arithmetic per request
+__device__ __forceinline__ u32x4 r32_load16(const void *base, uint32_t lane_off) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(lane_off), "s"(base) : "memory");
+  return v;
+}
+__device__ __forceinline__ uint32_t r32_load4(const void *base, uint32_t lane_off) {
+  uint32_t v;
+  asm volatile("global_load_dword %0, %1, %2" : "=v"(v) : "v"(lane_off), "s"(base) : "memory");
+  return v;
+}
 template <typename T>
 __device__ __forceinline__ void r32_arrived(T &v) {
   asm volatile("" : "+v"(v));

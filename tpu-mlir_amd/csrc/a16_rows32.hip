@@ -385,21 +385,24 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
   const int64_t set_n = R32_SEL(N);
   const int set_rbs = R32_SEL(row_blocks);
 
-  const uint8_t *wp[2];
-  const uint32_t *szp[2];
+  // Every request is a wave-uniform base (scalar arithmetic) plus a lane offset that never changes: the lane's 16
+  // bytes of a 1 KiB weight slot, its channel's word of a group's 16 scale|zp words, its 16 bytes of an activation row.
+  const uint8_t *wp[2];    // the row blocks' first tiles
+  const uint32_t *szp[2];  // ... and first groups
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
     int64_t rb = (int64_t)lb * 2 + b;
     rb = rb < set_rbs ? rb : set_rbs - 1;  // a row block past N repeats the last one; never stored
-    wp[b] = R32_SEL(qw) + rb * a.k_tiles * 1024 + (uint32_t)(lane * 16);
-    szp[b] = R32_SEL(sz) + rb * a.G * 16 + col;
+    wp[b] = R32_SEL(qw) + rb * a.k_tiles * 1024;
+    szp[b] = R32_SEL(sz) + rb * a.G * 16;
   }
-  const uint8_t *xg[NQ];
+  const uint32_t w_lane = (uint32_t)lane * 16, sz_lane = (uint32_t)col * 4;
+  uint32_t x_lane[NQ];
 #pragma unroll
   for (int i = 0; i < NQ; ++i) {
     const int r = 8 * i + (lane >> 3);
     const int rr = r < a.M ? r : a.M - 1;
-    xg[i] = a.x + (int64_t)rr * a.K * 2 + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+    x_lane[i] = (uint32_t)rr * (uint32_t)a.K * 2 + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
   }
   uint8_t *xs = smem + wave * (XR * 2 * SLOT);
   const int frow = col & (SLOT_ROWS - 1);  // fragment rows past the slot re-read a row that exists; never stored
@@ -411,28 +414,28 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
   auto tile_of = [&](int i) { return first + i * stride; };
   u32x4 w[WR][2];            // weight ring: [tile % WR][row block]: the lane's four k-steps of 8 nibbles
   uint32_t szw[WR][2][GPT];  // the tile's scale|zp words
-  // A request past the wave's last tile keeps the static request count the waits rely on.  For weights it moves
-  // nothing: all lanes ask for the same 16 bytes at the start of the buffer (one cache line, resident after the first
-  // time).  For activations it repeats the wave's last tile: with a request of that one-address kind as the wave's
-  // last one into LDS, the partial sums that overlay the rings after the loop came out overwritten.
+  // A request past the wave's last tile keeps the static request count the waits rely on.  For weights it moves next
+  // to nothing: the first KiB of the buffer again and again (resident after the first time).  For activations it
+  // repeats the wave's last tile: with every lane of the wave's *last* request into LDS asking for one and the same 16
+  // bytes, the partial sums that then overlaid the rings came out overwritten.
   const uint8_t *w_idle = R32_SEL(qw);
   const uint32_t *sz_idle = R32_SEL(sz);
   auto issue_x = [&](int i, int p) {  // piece p (K elements 64 p .. 64 p + 63) of the wave's i-th tile
-    const int64_t koff = (int64_t)tile_of(i < count ? i : count - 1) * 256 + p * 128;
+    const uint8_t *base = a.x + ((int64_t)tile_of(i < count ? i : count - 1) * 256 + p * 128);
     uint8_t *slot = xs + ((i % XR) * 2 + p) * SLOT;
 #pragma unroll
     for (int q = 0; q < NQ; ++q)
-      __builtin_amdgcn_global_load_lds((r32_gptr_t)(xg[q] + koff), (r32_lptr_t)(slot + q * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((r32_gptr_t)(base + x_lane[q]), (r32_lptr_t)(slot + q * 1024), 16, 0, 0);
   };
   auto issue_w = [&](int i, int rs) {
     const bool real = i < count;
     const int kt = tile_of(i);
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-      w[rs][b] = r32_load16(real ? wp[b] + (int64_t)kt * 1024 : w_idle);
+      w[rs][b] = r32_load16(real ? wp[b] + (int64_t)kt * 1024 : w_idle, w_lane);
 #pragma unroll
       for (int u = 0; u < GPT; ++u)
-        szw[rs][b][u] = r32_load4(real ? szp[b] + (GPT == 1 ? (kt >> a.group_shift) : kt * GPT + u) * 16 : sz_idle);
+        szw[rs][b][u] = r32_load4(real ? szp[b] + (GPT == 1 ? (kt >> a.group_shift) : kt * GPT + u) * 16 : sz_idle, sz_lane);
     }
   };
 
