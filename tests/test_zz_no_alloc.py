@@ -154,3 +154,35 @@ def test_no_alloc_launch_refuses_what_does_not_fit(plan):
     assert err.value.code == clib.MI_BAD_ARGUMENT and "scratch" in str(err.value)
     torch.cuda.synchronize()
     wb.destroy()
+
+
+def test_no_alloc_launch_drops_a_split_made_for_speed_alone():
+    """M = 640 at 4096 x 4096: the allocating entry point cuts K in three for the widest output block (31 MiB of fp32
+    slabs), which the fixed array cannot hold; the no-alloc one runs the same product unsplit -- not refused, nothing
+    allocated, the same fp32 result up to the order of the partial sums (2e-5 of the output RMS, the bound every A16
+    kernel is held to against the oracle) and 16-bit outputs at most one ulp apart (the fp32 bound next to zero)."""
+    import torch
+    K, N, g, rows = 4096, 4096, 128, 640
+    cfg, w = _weights(K, N, g, rows, 36)
+    x = _bf16(torch, cfg["x"])
+    y_ref = torch.empty((rows, N), dtype=torch.bfloat16, device="cuda")
+    f_ref = torch.empty((rows, N), dtype=torch.float32, device="cuda")
+    M_.a16mm_launch(w, x, y=y_ref, y_f32=f_ref)
+    torch.cuda.synchronize()
+    y_new, f_new = torch.empty_like(y_ref), torch.empty_like(f_ref)
+    fresh = torch.cuda.Stream()
+    with torch.cuda.stream(fresh):
+        torch.zeros(16, device="cuda").add_(1)
+    with _NothingAllocated(torch):
+        with torch.cuda.stream(fresh):
+            M_.a16mm_launch(w, x, y=y_new, y_f32=f_new, no_alloc=True)
+    torch.cuda.synchronize()
+    a, b = f_new.cpu().numpy().astype(np.float64), f_ref.cpu().numpy().astype(np.float64)
+    rms = float(np.sqrt(np.mean(b * b)))
+    assert rms > 0 and float(np.max(np.abs(a - b))) <= 2e-5 * rms
+    assert not np.array_equal(a, b), "the allocating entry point was expected to cut K here (another summation order)"
+    ya = S.bf16_to_f32(y_new.view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)
+    yb = S.bf16_to_f32(y_ref.view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)
+    one_ulp = 2.0 ** -7 * np.maximum(np.abs(ya), np.abs(yb))  # of the larger neighbour; outputs next to zero: the fp32 bound
+    assert bool(np.all(np.abs(ya - yb) <= one_ulp + 2e-5 * rms))
+    w.destroy()
