@@ -708,6 +708,8 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
   MI_REQUIRE(M >= 1 && M <= 32, MI_BAD_ARGUMENT, "mi_a16mm_launch: M out of range for this kernel");
   MI_REQUIRE(d_x, MI_BAD_ARGUMENT, "mi_a16mm_launch: null activation pointer");
   const mi_a16_weight *w = ws[0];
+  // a lane's offset into the activations is kept in 32 bits by the 16-row form
+  MI_REQUIRE(w->K < (int64_t(1) << 26), MI_BAD_ARGUMENT, "mi_a16mm_launch: K too large for this kernel");
   const bool f16 = w->dtype == MI_DT_F16;
   const dim3 block(512);
   const int nq = (int)((M + 7) / 8);  // 8-row requests per activation piece
