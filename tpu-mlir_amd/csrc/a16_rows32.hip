@@ -581,7 +581,7 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
 //   4-bit  4096 x 11008   M = 4: 11.8 / 13.3   M = 8: 14.2 / 13.2   M = 16: 14.5 / 13.9   M = 17: 16.3 / 14.5   M = 24: 16.6 / 16.3   M = 32: 16.9 / 18.5
 //   4-bit  6144 x 2048, groups of 64   M = 9: 5.6 / 6.0   M = 12: 6.2 / 6.1   M = 16: 6.9 / 6.2   M = 17: 10.6 / 6.2   M = 32: 11.6 / 6.6
 bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
-  if (!w || !w->qweight || w->kn || w->plain)
+  if (!w || !w->qweight || w->kn || w->plain || w->K >= (int64_t(1) << 26))
     return false;
   if (w->bits == 8) {
     if ((w->K % W8_TILE_K) != 0)
