@@ -250,7 +250,8 @@ int mi_llm_unpack(int mode, int bits, const int32_t *qweight, const int32_t *qze
 int mi_a16_to_group(const uint16_t *scale, int64_t scale_num, const uint8_t *zp, int64_t zp_num, int64_t K,
                     uint16_t *scale_out, uint8_t *zp_out);
 
-/* y[M,N] = round(x[M,K] * dequant(W)^T + bias).  d_x/d_y are DEVICE pointers to bf16/f16 bit patterns;
+/* y[M,N] = round(x[M,K] * dequant(W)^T + bias).  d_x/d_y are DEVICE pointers to bf16/f16 bit patterns (d_x 16-byte
+ * aligned for weight sets in the tiled layout, i.e. every set but those with odd group sizes or w_transpose = false);
  * d_y_f32 (optional DEVICE pointer, may be NULL) receives the fp32 result before output rounding.
  * Asynchronous on `stream` (a hipStream_t, NULL = default stream). */
 int mi_a16mm_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,

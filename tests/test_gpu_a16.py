@@ -386,3 +386,22 @@ def test_widest_block_takes_the_zero_point_term_out_of_the_loop(orc, plan, M, K,
                                    M=M, K=K, N=N, weight_bits=4, q_group_size=g, out_dtype=orc.OUT_F16)
     assert cmp.max_abs_over_rms(pre, want_pre) <= 2e-5
     assert np.array_equal(out, orc.f32_to_f16(pre))
+
+
+def test_misaligned_activations_are_refused():
+    """The kernels of the tiled layout read activations 16 bytes at a time: a pointer that is not 16-byte aligned (a
+    view that starts one element into a buffer) is refused with a message, not launched."""
+    import torch
+    K, N = 256, 64
+    cfg = S.w4a16(2, K, N, 128, seed=5)
+    w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], None, K=K, N=N, weight_bits=4, q_group_size=128)
+    buf = torch.zeros(2 * K + 8, dtype=torch.bfloat16, device="cuda")
+    x = buf[1:1 + 2 * K].view(2, K)
+    assert x.data_ptr() % 16 == 2
+    with pytest.raises(clib.BackendError) as err:
+        M_.a16mm_launch(w, x)
+    assert err.value.code == clib.MI_BAD_ARGUMENT and "aligned" in str(err.value)
+    y = M_.a16mm_launch(w, buf[8:8 + 2 * K].view(2, K))   # the same values 16 bytes in: taken
+    torch.cuda.synchronize()
+    assert tuple(y.shape) == (2, N)
+    w.destroy()

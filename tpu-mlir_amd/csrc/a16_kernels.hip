@@ -751,6 +751,9 @@ int a16_launch_group(const mi_a16_weight *const *ws, int n, const uint16_t *d_x,
     }
     return MI_SUCCESS;
   }
+  // the kernels of the tiled layout read the activations 16 bytes at a time (rows are whole multiples: K % 8 == 0)
+  MI_REQUIRE(M == 0 || ((uintptr_t)d_x & 15) == 0, MI_BAD_ARGUMENT,
+             "mi_a16mm_launch: the activation pointer must be 16-byte aligned");
   int64_t total_rb = 0;
   SkinnyArgs a;
   for (int i = 0; i < MAX_SEG; ++i) {
