@@ -2,7 +2,7 @@
 // interpreter hands them over) and device-level launches.  See include/tpumlir_amd.h for the contract.
 #include <math.h>
 #if defined(__SSE2__)
-#include <emmintrin.h>
+#include <immintrin.h>
 #endif
 #include <string.h>
 
@@ -687,10 +687,60 @@ static int out_elem_size(int dt) {
 // x86-64 host has them; left to the auto-vectorizer the same loop came out scalar in this translation unit, five times
 // slower).  Per element: truncate to int and convert back (stands in for truncf; NaN compares unequal), check the
 // range on the integer, take the low byte.  Bytes past the last multiple of 16 go through the scalar form.
+#if defined(__SSE2__)
+// The same loop eight floats at a time where the host has AVX2 (checked once at run time; the translation unit is not
+// compiled for it): 32 values per pass, bytes put back in order after the two in-lane packs.  Returns the number of
+// values done (a multiple of 32); the flags are ORed into.
+__attribute__((target("avx2"))) static int64_t floats_to_bytes_avx2(const float *src, int64_t n, uint8_t *dst, int *bad,
+                                                                    int *any_neg, int *any_big) {
+  __m256i vbad = _mm256_setzero_si256(), vneg = _mm256_setzero_si256(), vbig = _mm256_setzero_si256();
+  const __m256i c128 = _mm256_set1_epi32(128), c383 = _mm256_set1_epi32(383 - 0x7fffffff - 1);
+  const __m256i sign = _mm256_set1_epi32(-0x7fffffff - 1), c127 = _mm256_set1_epi32(127), lowbyte = _mm256_set1_epi32(0xff);
+  const __m256i order = _mm256_setr_epi32(0, 4, 1, 5, 2, 6, 3, 7);
+  int64_t i = 0;
+  for (; i + 32 <= n; i += 32) {
+    __m256i q[4];
+    for (int u = 0; u < 4; ++u) {
+      const __m256 v = _mm256_loadu_ps(src + i + 8 * u);
+      const __m256i iv = _mm256_cvttps_epi32(v);
+      vbad = _mm256_or_si256(vbad, _mm256_castps_si256(_mm256_cmp_ps(_mm256_cvtepi32_ps(iv), v, _CMP_NEQ_UQ)));
+      vbad = _mm256_or_si256(vbad, _mm256_cmpgt_epi32(_mm256_xor_si256(_mm256_add_epi32(iv, c128), sign), c383));
+      vneg = _mm256_or_si256(vneg, iv);
+      vbig = _mm256_or_si256(vbig, _mm256_sub_epi32(c127, iv));
+      q[u] = _mm256_and_si256(iv, lowbyte);
+    }
+    const __m256i packed = _mm256_packus_epi16(_mm256_packs_epi32(q[0], q[1]), _mm256_packs_epi32(q[2], q[3]));
+    _mm256_storeu_si256((__m256i *)(dst + i), _mm256_permutevar8x32_epi32(packed, order));
+  }
+  *bad |= _mm256_movemask_epi8(vbad) != 0;
+  *any_neg |= _mm256_movemask_ps(_mm256_castsi256_ps(vneg)) != 0;
+  *any_big |= _mm256_movemask_ps(_mm256_castsi256_ps(vbig)) != 0;
+  return i;
+}
+__attribute__((target("avx2"))) static int64_t i8_to_floats_avx2(const int8_t *src, int64_t n, float *y, bool is_unsigned) {
+  int64_t i = 0;
+  for (; i + 16 <= n; i += 16) {
+    const __m128i b = _mm_loadu_si128((const __m128i *)(src + i));
+    const __m128i hi = _mm_unpackhi_epi64(b, b);
+    const __m256i lo32 = is_unsigned ? _mm256_cvtepu8_epi32(b) : _mm256_cvtepi8_epi32(b);
+    const __m256i hi32 = is_unsigned ? _mm256_cvtepu8_epi32(hi) : _mm256_cvtepi8_epi32(hi);
+    _mm256_storeu_ps(y + i, _mm256_cvtepi32_ps(lo32));
+    _mm256_storeu_ps(y + i + 8, _mm256_cvtepi32_ps(hi32));
+  }
+  return i;
+}
+static bool host_has_avx2() {
+  static const bool yes = __builtin_cpu_supports("avx2");
+  return yes;
+}
+#endif
+
 static int floats_to_bytes(const float *src, int64_t n, uint8_t *dst, int *is_unsigned, const char *who) {
   int bad = 0, any_neg = 0, any_big = 0;
   int64_t i = 0;
 #if defined(__SSE2__)
+  if (host_has_avx2())
+    i = floats_to_bytes_avx2(src, n, dst, &bad, &any_neg, &any_big);
   __m128i vbad = _mm_setzero_si128(), vneg = _mm_setzero_si128(), vbig = _mm_setzero_si128();
   const __m128i c128 = _mm_set1_epi32(128), c383 = _mm_set1_epi32(383 - 0x7fffffff - 1), sign = _mm_set1_epi32(-0x7fffffff - 1);
   const __m128i c127 = _mm_set1_epi32(127), lowbyte = _mm_set1_epi32(0xff);
@@ -708,9 +758,9 @@ static int floats_to_bytes(const float *src, int64_t n, uint8_t *dst, int *is_un
     }
     _mm_storeu_si128((__m128i *)(dst + i), _mm_packus_epi16(_mm_packs_epi32(q[0], q[1]), _mm_packs_epi32(q[2], q[3])));
   }
-  bad = _mm_movemask_epi8(vbad) != 0;
-  any_neg = (_mm_movemask_ps(_mm_castsi128_ps(vneg)) != 0);
-  any_big = (_mm_movemask_ps(_mm_castsi128_ps(vbig)) != 0);
+  bad |= _mm_movemask_epi8(vbad) != 0;
+  any_neg |= (_mm_movemask_ps(_mm_castsi128_ps(vneg)) != 0);
+  any_big |= (_mm_movemask_ps(_mm_castsi128_ps(vbig)) != 0);
 #endif
   for (; i < n; ++i) {
     const float v = src[i];
@@ -820,12 +870,17 @@ static void fill_i8_rq(const mi_i8mm_attr *attr, mi_requant_desc *rq) {
 }
 
 static void bytes_to_floats(const void *ho, int out_dtype, int64_t n, float *y) {
+  int64_t i0 = 0;
+#if defined(__SSE2__)
+  if ((out_dtype == MI_DT_I8 || out_dtype == MI_DT_U8) && host_has_avx2())
+    i0 = i8_to_floats_avx2((const int8_t *)ho, n, y, out_dtype == MI_DT_U8);
+#endif
   switch (out_dtype) {
   case MI_DT_I8:
-    for (int64_t i = 0; i < n; ++i) y[i] = (float)((const int8_t *)ho)[i];
+    for (int64_t i = i0; i < n; ++i) y[i] = (float)((const int8_t *)ho)[i];
     break;
   case MI_DT_U8:
-    for (int64_t i = 0; i < n; ++i) y[i] = (float)((const uint8_t *)ho)[i];
+    for (int64_t i = i0; i < n; ++i) y[i] = (float)((const uint8_t *)ho)[i];
     break;
   case MI_DT_I16:
     for (int64_t i = 0; i < n; ++i) y[i] = (float)((const int16_t *)ho)[i];
