@@ -209,12 +209,12 @@ def test_operator_level_against_oracle(orc):
 
 
 def test_operator_boundary_recognises_the_8_bit_type_of_its_float_operands():
-    """The interpreter hands 8-bit tensors over as floats.  The boundary turns them into bytes, in 16-element vector
-    steps and a scalar tail: int8 values, uint8 values (up to 255), lengths that are not multiples of 16, and the
-    refusals -- a value of each sign's far end in one tensor, a fraction, NaN, infinity, anything outside [-128, 255],
-    wherever in the tensor (vector part or tail) it sits."""
+    """The interpreter hands 8-bit tensors over as floats.  The boundary turns them into bytes, in 32-element vector
+    steps where the host has AVX2, 16-element ones for what is left (or for everything), and a scalar tail: int8
+    values, uint8 values (up to 255), lengths that are not multiples of 16, and the refusals -- a value of each sign's
+    far end in one tensor, a fraction, NaN, infinity, anything outside [-128, 255], wherever in the tensor it sits."""
     rng = np.random.default_rng(21)
-    M, K, N = 3, 37, 5                                                   # 111 activations: six vector steps and a tail
+    M, K, N = 3, 41, 5                                   # 123 activations: 96 in 32-steps, 16 in a 16-step, a tail of 11
     b = rng.integers(-128, 128, size=(K, N)).astype(np.float32)
     for lo, hi in ((-128, 128), (0, 256)):
         a = rng.integers(lo, hi, size=(M, K)).astype(np.float32)
@@ -224,7 +224,7 @@ def test_operator_boundary_recognises_the_8_bit_type_of_its_float_operands():
         assert np.array_equal(op.inference(a, b), want), (lo, hi)
         op.deinit()
     good = rng.integers(0, 100, size=(M, K)).astype(np.float32)
-    for pos in (0, 17, M * K - 1):                                       # first vector, a middle one, the scalar tail
+    for pos in (0, 17, 70, 100, M * K - 1):              # first vector, middle ones, the 16-step, the scalar tail
         for value in (0.5, -128.5, 256.0, -129.0, 1e10, np.nan, np.inf, -np.inf):
             a = good.copy()
             a.reshape(-1)[pos] = value
