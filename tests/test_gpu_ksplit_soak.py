@@ -37,10 +37,11 @@ def _soak(torch, stream, launch, other, out):
             pytest.fail("replay %d of %d differs from the first result in %d elements" % (rep, REPLAYS, bad))
 
 
-def test_a16_four_part_split_replays_bit_identically(plan):
+@pytest.mark.parametrize("M", [32, 12])   # the 32-row kernel; the 16-row form (its partial sums in an LDS area of their own)
+def test_a16_four_part_split_replays_bit_identically(plan, M):
     import torch
     plan(a16_rows32_min_m=1, a16_rows32_split=4)
-    M, K, N, g = 32, 8192, 1024, 128
+    K, N, g = 8192, 1024, 128
     cfg = S.w4a16(M, K, N, g, seed=91, bias=True)
     w = M_.A16Weight(cfg["weight"], cfg["scale"], cfg["zp"], S.bf16_to_f32(cfg["bias"]), K=K, N=N, weight_bits=4,
                      q_group_size=g)
