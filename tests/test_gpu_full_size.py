@@ -161,13 +161,15 @@ GROUPED = [("cfg5 grouped q/k/v 3 x 4096x4096", 4096, (4096, 4096, 4096)),
 def test_grouped_sibling_launches_at_full_size(orc, label, K, Ns):
     """The launches behind the headline decode number: q/k/v and gate/up as one grouped launch each, M = 1 / 8 / 32 and
     two row counts in between (from 12 rows on a grouped launch of this size takes the 32-row kernel).  Every set's
-    output against the oracle (sampled channels), and -- where one launch per set runs the same kernel instance (up
-    to 8 rows) -- bit-identical to separate launches."""
+    output against the oracle (sampled channels), and -- up to 8 rows -- bit-identical to separate launches, whichever
+    of the decode, skinny and 16-row streaming kernels the grouped launch and each single one take (at 5 rows q/k/v
+    grouped takes the streaming kernel and a set alone the skinny one; at 8 rows gate/up grouped the streaming kernel
+    and a set alone the decode kernel): the three deal the K tiles to their waves, fold and sum alike."""
     import torch
     g = 128
     cfgs = [S.w4a16(32, K, N, g, seed=60 + i, bias=(i == 1)) for i, N in enumerate(Ns)]
     ws = [_weight(c) for c in cfgs]
-    for M in (1, 8, 16, 24, 32):
+    for M in (1, 5, 8, 16, 24, 32):
         x_bits = cfgs[0]["x"][:M]
         x = _bf16(torch, x_bits)
         f32s = [torch.empty((M, N), dtype=torch.float32, device="cuda") for N in Ns]
