@@ -617,8 +617,10 @@ def cpu_baseline_chain(S, M, cfgs, budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    # the first milliseconds after a pause run at lower clocks (200 steps after 20: 3770-3860 GB/s; 1000 after 100:
+    # 4030-4040; 2000 after 200: 4057): the defaults time a 26 ms stretch of a loop that is already running
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--batch", type=int, default=1, help="activation rows M of the decode chain")
     ap.add_argument("--layers", type=int, default=4, help="distinct weight copies rotated through (4 x 101 MB); one "
                     "HIP graph replay covers one step on each of them")

@@ -107,12 +107,52 @@ __global__ void pack_qparams_kernel(const uint16_t *__restrict__ scale, const ui
     nzs_t[idx] = -(float)((int)z + zp_bias) * Half16<DT>::to_f32(s);
 }
 
+// sz_t [rb][G][16] -> the decode kernel's order [rb][waves][16][tpw * gpt]: word p * gpt + u of wave w and channel c
+// is the group of tile w + p * waves (clamped to the last tile: such a word is never used), sub-group u
+__global__ void pack_sz_dec_kernel(const uint32_t *__restrict__ sz_t, uint32_t *__restrict__ sz_dec, int G, int k_tiles,
+                                   int waves, int tpw, int gpt, int group_shift, int64_t total) {
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total)
+    return;
+  const int nw = tpw * gpt;
+  const int j = (int)(idx % nw);
+  int64_t t = idx / nw;
+  const int c = (int)(t & 15);
+  t >>= 4;
+  const int w = (int)(t % waves);
+  const int64_t rb = t / waves;
+  int kt = w + (j / gpt) * waves;
+  kt = kt < k_tiles ? kt : k_tiles - 1;
+  const int gi = gpt == 1 ? (kt >> group_shift) : kt * gpt + j % gpt;
+  sz_dec[idx] = sz_t[(rb * G + gi) * 16 + c];
+}
+
+// The decode kernel's copy of a 4-bit set's scale|zp words (derived from sz_t, so a set uploaded from a blob gets it
+// too); nothing to do for sets the decode kernel cannot take.
+int a16_build_sz_dec(mi_a16_weight *w) {
+  int dw = 0, dt = 0, dg = 1, dshift = 0;
+  if (w->bits != 4 || !w->sz_t || w->sz_dec || !a16_decode_geometry(w, &dw, &dt, &dg, &dshift))
+    return MI_SUCCESS;
+  const int64_t total = w->row_blocks * dw * 16 * dt * dg;
+  MI_HIP(hipMalloc((void **)&w->sz_dec, (size_t)total * 4));
+  w->bytes += (size_t)total * 4;
+  w->dec_waves = dw;
+  w->dec_tpw = dt;
+  pack_sz_dec_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256)>>>(w->sz_t, w->sz_dec, w->G, (int)w->k_tiles, dw,
+                                                                          dt, dg, dshift, total);
+  MI_HIP(hipGetLastError());
+  MI_HIP(hipDeviceSynchronize());
+  return MI_SUCCESS;
+}
+
 void a16_free(mi_a16_weight *w) {
   if (!w)
     return;
   (void)hipFree(w->qweight);
   (void)hipFree(w->scale_t);
   (void)hipFree(w->sz_t);
+  (void)hipFree(w->sz_dec);
+  w->sz_dec = nullptr;
   (void)hipFree(w->nzs_t);
   (void)hipFree(w->bias);
   (void)hipFree(w->kn_w);
@@ -201,7 +241,10 @@ int a16_pack(mi_a16_weight *w, const void *h_weight, int weight_signed, const ui
   PACK_HIP(hipDeviceSynchronize());
 #undef PACK_HIP
   cleanup();
-  return MI_SUCCESS;
+  const int rc = a16_build_sz_dec(w);
+  if (rc != MI_SUCCESS)
+    a16_free(w);
+  return rc;
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -357,6 +357,8 @@ int mi_a16_weight_import(mi_a16_weight **out, const void *blob, size_t size) {
     rc = upload((void **)&w->nzs_t, h.qparam_entries * 4);
   if (rc == MI_SUCCESS && h.has_bias)
     rc = upload((void **)&w->bias, (size_t)h.N * 4);
+  if (rc == MI_SUCCESS)
+    rc = a16_build_sz_dec(w);
   if (rc != MI_SUCCESS) {
     a16_free(w);
     delete w;

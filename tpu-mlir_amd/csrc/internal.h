@@ -98,6 +98,11 @@ struct mi_a16_weight {
   void *qweight = nullptr;
   // 4-bit: [row_blocks][G][16] u32 = scale bit pattern (bf16/f16) << 16 | zero point
   uint32_t *sz_t = nullptr;
+  // 4-bit, K a whole number of tiles that the decode kernel can take: the same words in the order its waves want them,
+  // [row_blocks][dec_waves][16 channels][dec_tpw tiles x groups per tile] -- a lane's words for all of its tiles in one
+  // piece (a copy: 4 bytes per channel and tile, 6 % on top of the weights)
+  uint32_t *sz_dec = nullptr;
+  int dec_waves = 0, dec_tpw = 0;
   // 8-bit: [row_blocks][G][16] scale bit patterns
   uint16_t *scale_t = nullptr;
   // 8-bit: [row_blocks][G][16] float, -(zp + bias_of_unsigned_storage) * scale (exact in f32)
@@ -119,6 +124,7 @@ namespace mi {
 int a16_pack(mi_a16_weight *w, const void *h_weight, int weight_signed, const uint16_t *h_scale,
              const uint8_t *h_zp, const float *h_bias);
 void a16_free(mi_a16_weight *w);
+int a16_build_sz_dec(mi_a16_weight *w);
 int a16_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y_f32,
                hipStream_t stream);
 int a16_kn_launch(const mi_a16_weight *w, const uint16_t *d_x, int64_t M, uint16_t *d_y, float *d_y32, hipStream_t st);
@@ -149,6 +155,8 @@ int a16_plain_create(mi_a16_weight *w, const void *weight, int weight_signed, co
                      const uint8_t *zp, const float *bias);
 // decode kernel (a16_decode.hip): at most four rows, K a whole number of tiles.  Returns false, having launched
 // nothing, when the shape is not its own; the general kernels then take it.
+// the decode kernel's division of a set's K among its waves (a function of the set alone); false: not one it can take
+bool a16_decode_geometry(const mi_a16_weight *w, int *waves, int *tpw, int *gpt, int *group_shift);
 bool a16_decode_launch(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
                        float *const *d_y32s, hipStream_t stream);
 // tiled MFMA GEMM for many activation rows (prefill)
