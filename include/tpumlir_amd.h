@@ -141,7 +141,9 @@ void mi_a16_weight_destroy(mi_a16_weight *w);
  * export).  A plain fp32 kernel serves it: the converter never emits this form, so it is built for completeness. */
 int mi_a16_weight_create_kn(mi_a16_weight **out, const mi_a16_weight_desc *desc, const uint8_t *weight,
                             const float *scale, const float *zp, const float *bias);
-/* HBM bytes held by the packed set */
+/* HBM bytes held by the packed set: the tile-ordered weights, the per-group scale / zero-point tables and, for 4-bit
+ * sets, a second copy of those tables in the order the decode kernel reads them (4 bytes per channel and 128 K
+ * elements, 6 % of the weights; derived on the device, not part of the blob below) */
 size_t mi_a16_weight_bytes(const mi_a16_weight *w);
 
 /* The packed set as one relocatable blob (header + the tile-ordered arrays exactly as they sit in HBM): the
