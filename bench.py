@@ -61,6 +61,10 @@ def build_chain(pkg, S, torch, M, n_layers, cfgs):
 
 # steps captured into one HIP graph at most (4 launches each; a 32-layer decoder's graph holds 32 steps' worth per token)
 MAX_STEPS_PER_GRAPH = 256
+# Before the W warm-up steps the timed graph is replayed for this long, untimed: a GPU that has idled for a few
+# milliseconds (graph capture is host work) runs its first milliseconds at lower clocks, and a decode loop is a
+# loop that is already running.  The read-only ceiling the result is compared with gets the same treatment.
+PREROLL_S = 0.02
 
 # sibling projections that read the same activations go out as one grouped launch
 CHAIN_GROUPS = [("q_proj", "k_proj", "v_proj"), ("o_proj",), ("gate_proj", "up_proj"), ("down_proj",)]
@@ -106,6 +110,11 @@ def bench_chain(pkg, S, torch, M, steps, warmup, n_layers, cfgs, grouped=True, g
         full = capture(per_graph)
         rest = capture(steps % per_graph) if steps % per_graph else None
         warm = capture(min(max(warmup, 1), per_graph))
+        t_end = time.perf_counter() + PREROLL_S
+        while time.perf_counter() < t_end:
+            for _ in range(4):
+                full.replay()
+            stream.synchronize()
         for i in range(max(1, -(-warmup // per_graph))):
             warm.replay()
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -166,10 +175,16 @@ def bench_int8(pkg, S, torch, clib, n, steps, warmup, M=None, graph=False):
     return rec
 
 
-def _time_launches(torch, fn, steps, warmup=5):
-    """Average device time of fn() (which enqueues on the current stream), by HIP events, in seconds."""
+def _time_launches(torch, fn, steps, warmup=5, preroll_s=0.0):
+    """Average device time of fn() (which enqueues on the current stream), by HIP events, in seconds.  preroll_s: fn is
+    first repeated for that long, untimed (see PREROLL_S)."""
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
+        t_end = time.perf_counter() + preroll_s
+        while preroll_s and time.perf_counter() < t_end:
+            for _ in range(4):
+                fn()
+            stream.synchronize()
         for _ in range(warmup):
             fn()
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -237,7 +252,7 @@ def cpu_baseline_int8(S, budget_s=8.0):
                                       "scalar requantization loop)" % (passes, el)}
 
 
-def _time_graph(torch, fn, replays, warmup=2):
+def _time_graph(torch, fn, replays, warmup=2, preroll_s=0.0):
     """Average device time of one fn() when fn's launches are replayed from a HIP graph (fn runs eagerly first, so
     that whatever it allocates on its stream exists before the capture): a launch of a few microseconds issued from
     Python would otherwise be timed by the host's call rate."""
@@ -248,7 +263,7 @@ def _time_graph(torch, fn, replays, warmup=2):
         stream.synchronize()
         with torch.cuda.graph(g_, stream=stream):
             fn()
-    return _time_launches(torch, g_.replay, replays, warmup=warmup)
+    return _time_launches(torch, g_.replay, replays, warmup=warmup, preroll_s=preroll_s)
 
 
 def bench_read_ceiling(pkg, torch, sizes, steps=60, pool_mb=1024):
@@ -267,7 +282,7 @@ def bench_read_ceiling(pkg, torch, sizes, steps=60, pool_mb=1024):
             def run():
                 for c in range(copies):
                     pkg.bench_read_launch(pool[c * stride:], nbytes, sink, chunks_per_wave=cpw)
-            sec = _time_graph(torch, run, max(3, steps // copies)) / copies
+            sec = _time_graph(torch, run, max(3, steps // copies), preroll_s=PREROLL_S / 2) / copies
             best = sec if best is None else min(best, sec)
         out[int(nbytes)] = {"us": round(best * 1e6, 2), "GBps": round(nbytes / best / 1e9, 1)}
     del pool
@@ -686,7 +701,11 @@ def main():
                               % (min(args.steps, MAX_STEPS_PER_GRAPH), args.layers)) +
                              ("q/k/v and gate/up each as one grouped launch" if not args.no_group
                               else "one launch per matmul"),
-                   "timing": "value: host wall clock around the timed region; roofline: HIP events on the launch stream"},
+                   "timing": "value: host wall clock around the timed region; roofline: HIP events on the launch stream",
+                   "preroll_ms": PREROLL_S * 1e3,
+                   "preroll": "the timed graph is replayed for preroll_ms, untimed, before the warm-up steps (and the "
+                              "read-only ceiling's launches for half as long before each of its timings): the first "
+                              "milliseconds after an idle stretch run at lower clocks"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of this command
