@@ -175,7 +175,7 @@ def bench_int8(pkg, S, torch, clib, n, steps, warmup, M=None, graph=False):
     return rec
 
 
-def _time_launches(torch, fn, steps, warmup=5, preroll_s=0.0):
+def _time_launches(torch, fn, steps, warmup=5, preroll_s=PREROLL_S / 2):
     """Average device time of fn() (which enqueues on the current stream), by HIP events, in seconds.  preroll_s: fn is
     first repeated for that long, untimed (see PREROLL_S)."""
     stream = torch.cuda.Stream()
@@ -252,7 +252,7 @@ def cpu_baseline_int8(S, budget_s=8.0):
                                       "scalar requantization loop)" % (passes, el)}
 
 
-def _time_graph(torch, fn, replays, warmup=2, preroll_s=0.0):
+def _time_graph(torch, fn, replays, warmup=2, preroll_s=PREROLL_S / 2):
     """Average device time of one fn() when fn's launches are replayed from a HIP graph (fn runs eagerly first, so
     that whatever it allocates on its stream exists before the capture): a launch of a few microseconds issued from
     Python would otherwise be timed by the host's call rate."""
@@ -282,7 +282,7 @@ def bench_read_ceiling(pkg, torch, sizes, steps=60, pool_mb=1024):
             def run():
                 for c in range(copies):
                     pkg.bench_read_launch(pool[c * stride:], nbytes, sink, chunks_per_wave=cpw)
-            sec = _time_graph(torch, run, max(3, steps // copies), preroll_s=PREROLL_S / 2) / copies
+            sec = _time_graph(torch, run, max(3, steps // copies)) / copies
             best = sec if best is None else min(best, sec)
         out[int(nbytes)] = {"us": round(best * 1e6, 2), "GBps": round(nbytes / best / 1e9, 1)}
     del pool
@@ -704,8 +704,9 @@ def main():
                    "timing": "value: host wall clock around the timed region; roofline: HIP events on the launch stream",
                    "preroll_ms": PREROLL_S * 1e3,
                    "preroll": "the timed graph is replayed for preroll_ms, untimed, before the warm-up steps (and the "
-                              "read-only ceiling's launches for half as long before each of its timings): the first "
-                              "milliseconds after an idle stretch run at lower clocks"},
+                              "launches of the read-only ceiling and of every figure under extras for half as long "
+                              "before each of their timings): the first milliseconds after an idle stretch run at "
+                              "lower clocks"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of this command
