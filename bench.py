@@ -118,16 +118,14 @@ def bench_chain(pkg, S, torch, M, steps, warmup, n_layers, cfgs, grouped=True, g
         for i in range(max(1, -(-warmup // per_graph))):
             warm.replay()
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        stream.synchronize()
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
         ev0.record(stream)
+        t0 = time.perf_counter()
         for i in range(steps // per_graph):
             full.replay()
         if rest is not None:
             rest.replay()
         ev1.record(stream)
-        stream.synchronize()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
     wall_s = t1 - t0
