@@ -124,6 +124,7 @@ struct Rows32W4Args {
   int block_begin[R32_MAX_SETS];        // first workgroup of each set (unused slots: INT_MAX)
   const uint8_t *qw[R32_MAX_SETS];      // packed tiles [row_blocks][k_tiles][1024]
   const uint32_t *sz[R32_MAX_SETS];     // scale|zp words [row_blocks][G][16]
+  const uint32_t *szd[R32_MAX_SETS];    // the 16-row form, where it can: the decode kernel's copy [row_blocks][8][16][4]
   const float *bias[R32_MAX_SETS];      // [N] or null
   uint16_t *y[R32_MAX_SETS];            // [M][N]
   float *y32[R32_MAX_SETS];             // [M][N] or null

@@ -358,13 +358,16 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
 // here a wave multiplies its tile's two 16-channel row blocks separately (lane (channel, k-quarter) holds exactly the
 // B fragments of its slot of a packed tile, as in the decode kernel), one activation-sum MFMA serves both, and a lane
 // carries 8 accumulators instead of 16 (plus 12 instead of 32 for the group's products and sums).
-template <int DT, int GPT, int NQ>
+// SZD: the wave's scale|zp words for all of its tiles (at most 4 / GPT of them, K not split over workgroups) come
+// from the decode kernel's copy of them, which deals the tiles to eight waves the same way: two requests up front
+// instead of two per tile.
+template <int DT, int GPT, int NQ, bool SZD>
 __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
   static_assert(NQ == 1 || NQ == 2, "up to 16 rows");
   constexpr int WAVES = 8;
-  constexpr int WL = 2 + 2 * GPT;  // weight-side requests per tile: two row blocks' slots and their scale|zp words
+  constexpr int WL = SZD ? 2 : 2 + 2 * GPT;  // weight-side requests per tile: two row blocks' slots (and their scale|zp words)
   constexpr int SLOT_ROWS = 8 * NQ, SLOT = SLOT_ROWS * 128;  // an activation piece: the rows that exist x 64 K
   // Up to 8 rows a wave asks for a tile's activations a whole tile ahead (XR = 2 tiles in LDS); with 16 rows, piece by
   // piece as the 32-row kernels do (4096 x 4096, 16 rows: 6.8 against 7.3 us that way round; 8 rows: 6.5 against 6.3).
@@ -435,9 +438,11 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       w[rs][b] = r32_load16(real ? wp[b] + (int64_t)kt * 1024 : w_idle, w_lane);
+      if constexpr (!SZD) {
 #pragma unroll
-      for (int u = 0; u < GPT; ++u)
-        szw[rs][b][u] = r32_load4(real ? szp[b] + (GPT == 1 ? (kt >> a.group_shift) : kt * GPT + u) * 16 : sz_idle, sz_lane);
+        for (int u = 0; u < GPT; ++u)
+          szw[rs][b][u] = r32_load4(real ? szp[b] + (GPT == 1 ? (kt >> a.group_shift) : kt * GPT + u) * 16 : sz_idle, sz_lane);
+      }
     }
   };
 
@@ -451,7 +456,17 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
   uint32_t nib_magic = H::NIB_MAGIC2;
   asm volatile("" : "+v"(nib_magic));  // keep it in a VGPR (see and_or)
 
+  u32x4 szall[2];  // SZD: word GPT * i + u = tile i, group u of the tile
   if (count > 0) {
+    if constexpr (SZD) {
+      const uint32_t *szd = R32_SEL(szd);
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        int64_t rb = (int64_t)lb * 2 + b;
+        rb = rb < set_rbs ? rb : set_rbs - 1;
+        szall[b] = r32_load16(szd + (rb * WAVES + wave) * 64, (uint32_t)col * 16);  // the oldest requests: every wait covers them
+      }
+    }
     // Requests, oldest first.  The counter retires in order, so a wait for an activation piece is a wait for every
     // request before it.
     //   XR = 2:  w(0) x(0) w(1) | x(1) w(2) | x(2) w(3) | ...      the wait at tile t leaves w(t + 1), x(t + 1), w(t + 2)
@@ -494,9 +509,13 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
               r32_arrived(w[u][b]);
+              if constexpr (SZD) {
+                r32_arrived(szall[b]);
+              } else {
 #pragma unroll
-              for (int g = 0; g < GPT; ++g)
-                r32_arrived(szw[u][b][g]);
+                for (int g = 0; g < GPT; ++g)
+                  r32_arrived(szw[u][b][g]);
+              }
             }
           }
           u32x4 fa[2];
@@ -514,7 +533,13 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
           if (GPT == 2 || p == 1) {  // end of a quantization group (or of the tile: the same words again next tile)
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
-              const uint32_t szv = szw[u][b][GPT == 2 ? p : 0];
+              uint32_t szv;
+              if constexpr (SZD) {
+                const int j = GPT == 2 ? 2 * t + p : t;  // 0 .. 3, the same for the whole wave
+                szv = j == 0 ? szall[b][0] : j == 1 ? szall[b][1] : j == 2 ? szall[b][2] : szall[b][3];
+              } else {
+                szv = szw[u][b][GPT == 2 ? p : 0];
+              }
               const float sc = H::to_f32((uint16_t)(szv >> 16));
               const float c = H::OFFSET + (float)(szv & 0xffu);
 #pragma unroll
@@ -533,9 +558,11 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
 #pragma unroll
       for (int b = 0; b < 2; ++b) {
         r32_arrived(w[rs][b]);
+        if constexpr (!SZD) {
 #pragma unroll
-        for (int g = 0; g < GPT; ++g)
-          r32_arrived(szw[rs][b][g]);
+          for (int g = 0; g < GPT; ++g)
+            r32_arrived(szw[rs][b][g]);
+        }
       }
   }
 
@@ -792,11 +819,14 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
       while ((1 << a.group_shift) < tpg)
         ++a.group_shift;
     int64_t blocks = 0;
+    bool szd_ok = M <= 16;  // the 16-row form reads the decode kernel's copy of the scale|zp words where the two deal alike
     for (int j = 0; j < R32_MAX_SETS; ++j) {
       const mi_a16_weight *v = ws[i0 + (j < cnt ? j : 0)];
       a.block_begin[j] = j < cnt ? (int)blocks : INT_MAX;
       a.qw[j] = (const uint8_t *)v->qweight;
       a.sz[j] = (const uint32_t *)v->sz_t;
+      a.szd[j] = v->sz_dec;
+      szd_ok = szd_ok && v->sz_dec && v->dec_waves == 8 && v->dec_tpw * (v->g == 64 ? 2 : 1) == 4;
       a.bias[j] = v->bias;
       a.y[j] = d_ys[i0 + (j < cnt ? j : 0)];
       a.y32[j] = d_y32s ? d_y32s[i0 + (j < cnt ? j : 0)] : nullptr;
@@ -812,6 +842,7 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
     if (rc != MI_SUCCESS)
       return rc;
     const dim3 grid((unsigned)(blocks << a.split.shift));
+    szd_ok = szd_ok && a.split.shift == 0;
 #define MI_R32_4(GPT_, NQ_)                                                      \
   {                                                                              \
     if (f16)                                                                     \
@@ -819,12 +850,19 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
     else                                                                         \
       a16_rows32_w4_kernel<MI_DT_BF16, GPT_, NQ_><<<grid, block, 0, stream>>>(a); \
   }
-#define MI_R16_4(GPT_, NQ_)                                                      \
-  {                                                                              \
-    if (f16)                                                                     \
-      a16_rows16_w4_kernel<MI_DT_F16, GPT_, NQ_><<<grid, block, 0, stream>>>(a);  \
-    else                                                                         \
-      a16_rows16_w4_kernel<MI_DT_BF16, GPT_, NQ_><<<grid, block, 0, stream>>>(a); \
+#define MI_R16_4S(GPT_, NQ_, SZD_)                                                     \
+  {                                                                                    \
+    if (f16)                                                                           \
+      a16_rows16_w4_kernel<MI_DT_F16, GPT_, NQ_, SZD_><<<grid, block, 0, stream>>>(a);  \
+    else                                                                               \
+      a16_rows16_w4_kernel<MI_DT_BF16, GPT_, NQ_, SZD_><<<grid, block, 0, stream>>>(a); \
+  }
+#define MI_R16_4(GPT_, NQ_)       \
+  {                               \
+    if (szd_ok)                   \
+      MI_R16_4S(GPT_, NQ_, true)  \
+    else                          \
+      MI_R16_4S(GPT_, NQ_, false) \
   }
 #define MI_R32_4Q(GPT_)  /* up to 16 rows: the 16 x 16 x 32 form */ \
   {                       \
@@ -844,6 +882,7 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
 #undef MI_R32_4Q
 #undef MI_R32_4
 #undef MI_R16_4
+#undef MI_R16_4S
   }
   MI_HIP(hipGetLastError());
   return MI_SUCCESS;
