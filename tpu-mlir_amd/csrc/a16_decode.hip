@@ -61,12 +61,18 @@ struct DecodeArgs {
 // sets' packed weights, rows and K tiles (mk = M | k_tiles << 8), the sets' first row blocks -- are 14 dwords, which
 // this file is compiled to have preloaded into SGPRs at wave launch (-amdgpu-kernarg-preload-count): the kernel starts
 // requesting without a round trip to the argument buffer.  Everything needed later comes from the record `a`.
-template <int BITS, int DT, int GPT, int WAVES, int TPW, int MR>
+template <int BITS, int DT, int GPT_, int WAVES, int TPW, int MR>
 __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(const uint8_t *x, const uint8_t *qw0, const uint8_t *qw1,
                                                                 const uint8_t *qw2, const uint8_t *qw3, uint32_t mk,
                                                                 int rb1, int rb2, int rb3, DecodeArgs a) {
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
+  // GPT_ = 0 (8-bit weights only): one group spans all of K -- per-channel quantization -- so a lane asks for its
+  // channel's scale and folded zero point once, not once per tile (11008 x 4096 per-channel: 10.11 -> 9.96 us at M = 1,
+  // 10.33 -> 10.23 at M = 4; 4096 x 4096: 6.03 -> 6.08 and 6.30 -> 6.14; three interleaved runs each way)
+  constexpr bool PER_CHANNEL = GPT_ == 0;
+  constexpr int GPT = PER_CHANNEL ? 1 : GPT_;
+  static_assert(!PER_CHANNEL || BITS == 8, "the 4-bit words are merged per lane already");
   constexpr int TILE_K = BITS == 4 ? W4_TILE_K : W8_TILE_K;
   constexpr int KSTEPS = TILE_K / 32;
   constexpr int KSTEPS_PER_UNIT = KSTEPS / GPT;
@@ -163,6 +169,13 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(const uint8_t *x
   } else {
     const uint8_t *szp = MI_SEL(sz) + (int64_t)rb_late * a.G * 32;
     const uint8_t *nzp = MI_SEL(nz) + (int64_t)rb_late * a.G * 64;
+    if constexpr (PER_CHANNEL) {
+      const uint32_t s0 = *(const uint16_t *)(szp + (uint32_t)col * 2u);
+      const float z0 = *(const float *)(nzp + (uint32_t)col * 4u);
+#pragma unroll
+      for (int p = 0; p < TPW; ++p)
+        szv[p][0] = s0, nzv[p][0] = z0;
+    } else
 #pragma unroll
     for (int p = 0; p < TPW; ++p) {
       int kt = wave_late + p * WAVES;
@@ -509,7 +522,9 @@ bool a16_decode_launch(const mi_a16_weight *const *ws, int n, const uint16_t *d_
       MI_DEC(4, 4)
     }
   } else {
-    if (p.gpt == 1) {
+    if (p.gpt == 1 && a.group_shift == 31) {
+      MI_DEC(8, 0)
+    } else if (p.gpt == 1) {
       MI_DEC(8, 1)
     } else if (p.gpt == 2) {
       MI_DEC(8, 2)
