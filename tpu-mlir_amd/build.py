@@ -1,5 +1,6 @@
 """Builds libtpumlir_amd.so (HIP kernels + C ABI) in-tree for gfx950 with hipcc."""
 import os
+import re
 import subprocess
 import sys
 
@@ -19,6 +20,26 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-u
 EXTRA_FLAGS = {"a16_decode.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"],
                "bench_kernels.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=6"]}
 
+# Kernels that keep load requests in flight across their loop (issued by inline asm, waited for by hand-counted
+# s_waitcnt) must not spill: the compiler takes a requested register for loaded, may store it to scratch and hand the
+# register on, and the data then lands on the register's next user; and a spill's own memory instruction moves the
+# count the waits rely on.  These files are compiled with the resource report on, and a spilling instance of such a
+# kernel fails the build.
+NO_SPILL = {"a16_rows32.hip": ("rows32", "rows16"), "a16_wide.hip": ("wide",), "i8_kernels.hip": ("rows32",),
+            "f8_kernels.hip": ("rows32",)}
+REPORT_FLAG = "-Rpass-analysis=kernel-resource-usage"
+
+
+def _spilling_kernels(report, name_parts):
+    """Names of the kernels in a resource report whose name holds one of name_parts and that use scratch memory."""
+    bad = []
+    for block in re.split(r"remark:\s+Function Name: ", report)[1:]:
+        name = block.split()[0]
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", block)
+        if any(part in name for part in name_parts) and m and int(m.group(1)) > 0:
+            bad.append("%s (%s bytes/lane)" % (name, m.group(1)))
+    return bad
+
 
 def build_library(verbose=False):
     os.makedirs(LIB_DIR, exist_ok=True)
@@ -26,7 +47,8 @@ def build_library(verbose=False):
     procs = []
     for src in SOURCES:
         obj = os.path.join(LIB_DIR, src.replace(".hip", ".o"))
-        cmd = ["hipcc", *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = ["hipcc", *FLAGS, *EXTRA_FLAGS.get(src, []), *([REPORT_FLAG] if src in NO_SPILL else []), "-c",
+               os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
@@ -37,6 +59,11 @@ def build_library(verbose=False):
         out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l)
         if p.returncode != 0:
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, out))
+        if src in NO_SPILL:
+            bad = _spilling_kernels(out, NO_SPILL[src])
+            if bad:
+                raise RuntimeError("%s: kernels with requests in flight must not spill:\n  %s" % (src, "\n  ".join(bad)))
+            out = "\n".join(l for l in out.splitlines() if REPORT_FLAG not in l)
         if verbose and out.strip():
             print(out)
     cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]

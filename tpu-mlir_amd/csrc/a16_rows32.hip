@@ -353,11 +353,15 @@ __global__ __launch_bounds__(512) void a16_rows32_w4_kernel(Rows32W4Args a) {
 #undef R32_SEL
 }
 
-// 4-bit weights, up to 16 rows: the same streaming design on the 16 x 16 x 32 MFMA.  With at most 16 rows the
-// 32 x 32 x 16 instruction spends half of its rows on nothing and takes twice the matrix-pipe time per weight element;
-// here a wave multiplies its tile's two 16-channel row blocks separately (lane (channel, k-quarter) holds exactly the
-// B fragments of its slot of a packed tile, as in the decode kernel), one activation-sum MFMA serves both, and a lane
-// carries 8 accumulators instead of 16 (plus 12 instead of 32 for the group's products and sums).
+// 4-bit weights: the same streaming design on the 16 x 16 x 32 MFMA.  With at most 16 rows the 32 x 32 x 16
+// instruction spends half of its rows on nothing and takes twice the matrix-pipe time per weight element; here a wave
+// multiplies its tile's two 16-channel row blocks separately (lane (channel, k-quarter) holds exactly the B fragments
+// of its slot of a packed tile, as in the decode kernel), one activation-sum MFMA serves both, and a lane carries 8
+// accumulators instead of 16 (plus 12 instead of 32 for the group's products and sums).
+// From 17 rows (NQ = 3, 4) the activations are two 16-row tiles against the same unpacked weights: per 64 K twelve
+// 16-cycle instructions where the 32 x 32 x 16 form issues eight of 32 cycles, the sums being one of three instead of
+// one of two (decode chain, us per step, 32 x 32 form / this: M = 17 53.0 / 49.5, M = 24 54.9 / 53.0, M = 32
+// 58.9 / 57.3).  With two groups per tile those instances need more than 128 registers and stay with the 32 x 32 form.
 // SZD: the wave's scale|zp words for all of its tiles (at most 4 / GPT of them, K not split over workgroups) come
 // from the decode kernel's copy of them, which deals the tiles to eight waves the same way: two requests up front
 // instead of two per tile.
@@ -365,19 +369,25 @@ template <int DT, int GPT, int NQ, bool SZD>
 __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
   using H = Half16<DT>;
   using vec8 = typename H::vec8;
-  static_assert(NQ == 1 || NQ == 2, "up to 16 rows");
+  static_assert(NQ >= 1 && NQ <= 4, "up to 32 rows");
+  constexpr int RT = NQ > 2 ? 2 : 1;  // 16-row tiles of the activations
+  constexpr int NR = 8 * RT;          // accumulators of a lane: [row tile][row block][4]
   constexpr int WAVES = 8;
   constexpr int WL = SZD ? 2 : 2 + 2 * GPT;  // weight-side requests per tile: two row blocks' slots (and their scale|zp words)
   constexpr int SLOT_ROWS = 8 * NQ, SLOT = SLOT_ROWS * 128;  // an activation piece: the rows that exist x 64 K
   // Up to 8 rows a wave asks for a tile's activations a whole tile ahead (XR = 2 tiles in LDS); with 16 rows, piece by
   // piece as the 32-row kernels do (4096 x 4096, 16 rows: 6.8 against 7.3 us that way round; 8 rows: 6.5 against 6.3).
   constexpr int XR = NQ == 1 ? 2 : 1, WR = 3;  // activation ring in LDS and weight ring in registers, in tiles
-  constexpr int RING_BYTES = WAVES * XR * 2 * SLOT, RED_BYTES = WAVES * 8 * 256;
-  // The partial sums have a place of their own behind the rings (48 KiB in all): no barrier before they are written,
-  // and a request into a ring that is still on its way when a wave leaves the loop has nothing to land on.
-  constexpr int FLAG_AT = RING_BYTES + RED_BYTES;
+  constexpr int RING_BYTES = WAVES * XR * 2 * SLOT, RED_BYTES = WAVES * NR * 256;
+  // Up to 16 rows the partial sums have a place of their own behind the rings (48 KiB in all): no barrier before they
+  // are written, and a request into a ring that is still on its way when a wave leaves the loop has nothing to land on.
+  // Beyond (rings of 48 or 64 KiB, 32 KiB of partial sums) they overlay the rings behind a barrier, as in the 32-row
+  // kernels, so that two workgroups still fit a CU.
+  constexpr bool OVERLAY = RT == 2;
+  constexpr int RED_AT = OVERLAY ? 0 : RING_BYTES;
+  constexpr int FLAG_AT = OVERLAY ? (RING_BYTES > RED_BYTES ? RING_BYTES : RED_BYTES) : RING_BYTES + RED_BYTES;
   __shared__ __attribute__((aligned(16))) uint8_t smem[FLAG_AT + 16];
-  float (*red)[8][64] = reinterpret_cast<float (*)[8][64]>(smem + RING_BYTES);
+  float (*red)[NR][64] = reinterpret_cast<float (*)[NR][64]>(smem + RED_AT);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, kq = lane >> 4;
@@ -408,8 +418,12 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
     x_lane[i] = (uint32_t)rr * (uint32_t)a.K * 2 + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
   }
   uint8_t *xs = smem + wave * (XR * 2 * SLOT);
-  const int frow = col & (SLOT_ROWS - 1);  // fragment rows past the slot re-read a row that exists; never stored
-  const uint8_t *xf = xs + frow * 128;
+  int frow[RT];  // the lane's row of each row tile; rows past the slot re-read a row that exists and are never stored
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int rows_here = SLOT_ROWS - 16 * rt < 16 ? SLOT_ROWS - 16 * rt : 16;  // 8 or 16
+    frow[rt] = 16 * rt + (col & (rows_here - 1));
+  }
 
   // this wave's tiles: first, first + stride, ... (see a16_rows32_kernel; a run of consecutive tiles per wave instead
   // was 5-10 % slower: 4096 x 4096, 8 rows: 6.1 -> 6.5 us).  The decode kernel deals its tiles the same way, and the
@@ -446,11 +460,14 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
     }
   };
 
-  f32x4 acc[2], P[2], S;
+  f32x4 acc[RT][2], P[RT][2], S[RT];
 #pragma unroll
-  for (int b = 0; b < 2; ++b)
-    acc[b] = P[b] = f32x4{0.f, 0.f, 0.f, 0.f};
-  S = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+      acc[rt][b] = P[rt][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    S[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
   const u32x4 ones_bits = {H::ONE2, H::ONE2, H::ONE2, H::ONE2};
   const vec8 ones = __builtin_bit_cast(vec8, ones_bits);
   uint32_t nib_magic = H::NIB_MAGIC2;
@@ -485,7 +502,7 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
         const int t = t0 + u;
         if (t >= count)
           break;
-        const uint8_t *xt = xf + (t % XR) * (2 * SLOT);
+        const uint8_t *xt = xs + (t % XR) * (2 * SLOT);
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
           if (XR == 2) {
@@ -518,17 +535,26 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
               }
             }
           }
-          u32x4 fa[2];
+          u32x4 fa[RT][2];
 #pragma unroll
-          for (int s = 0; s < 2; ++s)
-            fa[s] = *(const u32x4 *)(xt + p * SLOT + (((4 * s + kq) ^ ((frow >> 1) & 7)) << 4));
+          for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+              fa[rt][s] = *(const u32x4 *)(xt + p * SLOT + frow[rt] * 128 + (((4 * s + kq) ^ ((frow[rt] >> 1) & 7)) << 4));
 #pragma unroll
           for (int s = 0; s < 2; ++s) {  // k-step 2 p + s of the tile
-            const vec8 af = __builtin_bit_cast(vec8, fa[s]);
+            vec8 bf[2];
 #pragma unroll
             for (int b = 0; b < 2; ++b)
-              P[b] = H::mfma(af, unpack_nibbles<DT>(w[u][b][2 * p + s], nib_magic), P[b]);
-            S = H::mfma(af, ones, S);
+              bf[b] = unpack_nibbles<DT>(w[u][b][2 * p + s], nib_magic);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+              const vec8 af = __builtin_bit_cast(vec8, fa[rt][s]);
+#pragma unroll
+              for (int b = 0; b < 2; ++b)
+                P[rt][b] = H::mfma(af, bf[b], P[rt][b]);
+              S[rt] = H::mfma(af, ones, S[rt]);
+            }
           }
           if (GPT == 2 || p == 1) {  // end of a quantization group (or of the tile: the same words again next tile)
 #pragma unroll
@@ -543,11 +569,16 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
               const float sc = H::to_f32((uint16_t)(szv >> 16));
               const float c = H::OFFSET + (float)(szv & 0xffu);
 #pragma unroll
-              for (int i = 0; i < 4; ++i)
-                acc[b][i] = fmaf(sc, fmaf(-c, S[i], P[b][i]), acc[b][i]);
-              P[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+              for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                  acc[rt][b][i] = fmaf(sc, fmaf(-c, S[rt][i], P[rt][b][i]), acc[rt][b][i]);
+                P[rt][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+              }
             }
-            S = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+              S[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
           }
         }
       }
@@ -566,31 +597,42 @@ __global__ __launch_bounds__(512, 4) void a16_rows16_w4_kernel(Rows32W4Args a) {
       }
   }
 
-  // ---- cross-wave sum, in wave order: register 4 b + i of a lane is row 4 kq + i of channel 16 b + col
+  // ---- cross-wave sum, in wave order: register 8 rt + 4 b + i of a lane is row 16 rt + 4 kq + i of channel 16 b + col
+  if constexpr (OVERLAY)
+    __syncthreads();  // the partial sums overlay the rings: every wave is done with its pieces
 #pragma unroll
-  for (int b = 0; b < 2; ++b)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      red[wave][4 * b + i][lane] = acc[b][i];
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        red[wave][8 * rt + 4 * b + i][lane] = acc[rt][b][i];
   __syncthreads();
-  float v[2] = {0.f, 0.f};  // wave w finishes register w; the second slot only fills the K-split record
+  // one row tile: wave w finishes register w (the second slot only fills the K-split record); two: 2 w and 2 w + 1
+  float v[2] = {0.f, 0.f};
 #pragma unroll
-  for (int wv = 0; wv < WAVES; ++wv)
-    v[0] += red[wv][wave][lane];
+  for (int q = 0; q < RT; ++q)
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv)
+      v[q] += red[wv][RT * wave + q][lane];
   if (a.split.shift != 0 && !r32_join_parts(v, a.split, wave, lane, reinterpret_cast<int *>(smem + FLAG_AT)))
     return;
-  const int b = wave >> 2, i = wave & 3;
-  const int orow = 4 * kq + i;
-  const int64_t n = (int64_t)lb * 32 + b * 16 + col;
-  if (orow < a.M && n < set_n) {
-    const float *biasp = R32_SEL(bias);
-    float *y32 = R32_SEL(y32);
-    uint16_t *y = R32_SEL(y);
-    const float o32 = v[0] + (biasp ? biasp[n] : 0.f);
-    const int64_t o = (int64_t)orow * set_n + n;
-    if (y32)
-      y32[o] = o32;
-    y[o] = a.chip == MI_CHIP_CV18XX ? round_out16<DT, MI_CHIP_CV18XX>(o32) : round_out16<DT, MI_CHIP_BM168X>(o32);
+  const float *biasp = R32_SEL(bias);
+  float *y32 = R32_SEL(y32);
+  uint16_t *y = R32_SEL(y);
+#pragma unroll
+  for (int q = 0; q < RT; ++q) {
+    const int reg = RT * wave + q;
+    const int b = (reg >> 2) & 1, i = reg & 3;
+    const int orow = 16 * (reg >> 3) + 4 * kq + i;
+    const int64_t n = (int64_t)lb * 32 + b * 16 + col;
+    if (orow < a.M && n < set_n) {
+      const float o32 = v[q] + (biasp ? biasp[n] : 0.f);
+      const int64_t o = (int64_t)orow * set_n + n;
+      if (y32)
+        y32[o] = o32;
+      y[o] = a.chip == MI_CHIP_CV18XX ? round_out16<DT, MI_CHIP_CV18XX>(o32) : round_out16<DT, MI_CHIP_BM168X>(o32);
+    }
   }
 #undef R32_SEL
 }
@@ -819,7 +861,7 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
       while ((1 << a.group_shift) < tpg)
         ++a.group_shift;
     int64_t blocks = 0;
-    bool szd_ok = M <= 16;  // the 16-row form reads the decode kernel's copy of the scale|zp words where the two deal alike
+    bool szd_ok = true;  // the 16-row form reads the decode kernel's copy of the scale|zp words where the two deal alike
     for (int j = 0; j < R32_MAX_SETS; ++j) {
       const mi_a16_weight *v = ws[i0 + (j < cnt ? j : 0)];
       a.block_begin[j] = j < cnt ? (int)blocks : INT_MAX;
@@ -864,22 +906,28 @@ int a16_rows32_launch_group(const mi_a16_weight *const *ws, int n, const uint16_
     else                          \
       MI_R16_4S(GPT_, NQ_, false) \
   }
-#define MI_R32_4Q(GPT_)  /* up to 16 rows: the 16 x 16 x 32 form */ \
-  {                       \
-    if (nq == 1)          \
-      MI_R16_4(GPT_, 1)   \
-    else if (nq == 2)     \
-      MI_R16_4(GPT_, 2)   \
-    else if (nq == 3)     \
-      MI_R32_4(GPT_, 3)   \
-    else                  \
-      MI_R32_4(GPT_, 4)   \
-  }
-    if (w->g == 64)
-      MI_R32_4Q(2)
-    else
-      MI_R32_4Q(1)
-#undef MI_R32_4Q
+    // The 16 x 16 x 32 form everywhere but from 17 rows with groups of 64: those instances do not fit 128 registers,
+    // and a kernel whose requests are in flight across the loop must not spill -- the compiler takes a requested
+    // register for loaded, stores it and hands it on, and the data then lands on its next user.
+    if (w->g == 64) {
+      if (nq == 1)
+        MI_R16_4(2, 1)
+      else if (nq == 2)
+        MI_R16_4(2, 2)
+      else if (nq == 3)
+        MI_R32_4(2, 3)
+      else
+        MI_R32_4(2, 4)
+    } else {
+      if (nq == 1)
+        MI_R16_4(1, 1)
+      else if (nq == 2)
+        MI_R16_4(1, 2)
+      else if (nq == 3)
+        MI_R16_4(1, 3)
+      else
+        MI_R16_4(1, 4)
+    }
 #undef MI_R32_4
 #undef MI_R16_4
 #undef MI_R16_4S
