@@ -131,7 +131,8 @@ FULL_SIZE = [
     ("cfg3 W4 g128 4096x4096 prefill", 4, 4096, 4096, 128, (640, 1024)),   # the widest block with K in 3 and 2 parts
     ("W4 g128 gate/up 11008x4096 prefill", 4, 4096, 11008, 128, (256, 1024)),  # ... in 2 parts: one round, three rounds
     ("W4 g128 down 4096x11008 prefill", 4, 11008, 4096, 128, (512,)),          # ... in 4 parts
-    ("cfg4 W8 per-channel 11008x4096", 8, 4096, 11008, 0, (32, 512)),
+    ("cfg4 W8 per-channel 11008x4096", 8, 4096, 11008, 0, (6, 32, 512)),   # 6 rows: the decode kernel's eight-row form
+    ("W8 g128 9216x2048", 8, 2048, 9216, 128, (5, 8)),                     # ... with groups
     ("cfg5 W4 g128 q_proj 4096x4096", 4, 4096, 4096, 128, (8, 32)),
     ("cfg5 W4 g128 gate/up 11008x4096", 4, 4096, 11008, 128, (8, 32)),
     ("cfg5 W4 g128 down 4096x11008", 4, 11008, 4096, 128, (1, 8, 32)),

@@ -408,7 +408,22 @@ bool a16_decode_geometry(const mi_a16_weight *w, int *waves, int *tpw, int *gpt,
   return true;
 }
 
-static DecodePlan decode_plan(const mi_a16_weight *w, int64_t M) {
+// 8-bit weights, 5 to 8 rows, K up to 4096: between one and one and a half workgroups of the 32-row kernel per CU
+// (blocks32: 32-channel blocks of the whole launch) that kernel's second, mostly empty round costs a third more, and
+// this kernel's eight-row form is ahead.  32-row kernel / this one, us, per-channel scales unless noted:
+//   4096 x 9216 (288 blocks)  M = 5: 11.8 / 10.3   M = 8: 11.8 / 10.4      4096 x 11008 (344)  M = 5 ... 8: 12.5 / 11.1
+//   4096 x 12288, groups of 128 (384)  14.4 / 13.1      2048 x 11008  8.2 / 7.7      3072 x 11008  10.1 / 9.2
+//   4096 x 8192 (256)  8.8 / 8.8      4096 x 13312 (416)  13.9 / 14.4      4096 x 6144 (192)  7.7 / 7.9
+bool a16_decode_rows8_w8(const mi_a16_weight *w, int64_t M, int64_t blocks32) {
+  if (!w || w->bits != 8 || M < 5 || M > 8 || plan().a16_decode_rows8 != 0 || plan().a16_no_decode)
+    return false;
+  int waves = 0, tpw = 0, gpt = 0, shift = 0;
+  if (w->K < 2048 || w->K > 4096 || blocks32 <= 256 || blocks32 > 400 || !a16_decode_geometry(w, &waves, &tpw, &gpt, &shift))
+    return false;
+  return waves == 8 && decode_lds_bytes(8, gpt, waves, tpw, 8) <= DEC_MAX_LDS8;
+}
+
+static DecodePlan decode_plan(const mi_a16_weight *w, int64_t M, int64_t blocks32) {
   DecodePlan p = {8, 0, 0, 1, false};
   int shift = 0;
   if (M < 1 || M > DEC_MAX_ROWS || !a16_decode_geometry(w, &p.waves, &p.tpw, &p.gpt, &shift))
@@ -419,7 +434,8 @@ static DecodePlan decode_plan(const mi_a16_weight *w, int64_t M) {
   // eight rows: one request per lane and row only (K up to 4096 at 4 bits), on the 8-wave instances, and only where
   // it was measured ahead of the skinny kernel (us, skinny / this): 4096 x 4096 M = 5: 5.30 / 5.42, M = 8: 5.73 / 5.39;
   // 11008 x 4096 M = 5: 9.79 / 9.84, M = 8: 11.00 / 9.84; 6144 x 2048 M = 8: 5.60 / 5.83
-  const bool rows8_pays = plan().a16_decode_rows8 ? plan().a16_decode_rows8 > 0 : (w->bits == 4 && M >= 7 && w->K >= 4096);
+  const bool rows8_pays = plan().a16_decode_rows8 ? plan().a16_decode_rows8 > 0
+                                                  : ((w->bits == 4 && M >= 7 && w->K >= 4096) || a16_decode_rows8_w8(w, M, blocks32));
   p.ok = decode_lds_bytes(w->bits, p.gpt, p.waves, p.tpw, p.mr) <= (p.mr > 4 ? DEC_MAX_LDS8 : DEC_MAX_LDS) &&
          (p.mr <= 4 || (p.waves == 8 && rows8_pays));
   return p;
@@ -467,7 +483,10 @@ bool a16_decode_launch(const mi_a16_weight *const *ws, int n, const uint16_t *d_
   const mi_a16_weight *w = ws[0];
   if (n < 1 || n > DEC_MAX_SEG)
     return false;
-  const DecodePlan p = decode_plan(w, M);
+  int64_t blocks32 = 0;
+  for (int i = 0; i < n; ++i)
+    blocks32 += (ws[i]->N + 31) / 32;
+  const DecodePlan p = decode_plan(w, M, blocks32);
   if (!p.ok)
     return false;
   DecodeArgs a;

@@ -690,7 +690,7 @@ bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
   const bool long_k = w->K >= 8192, mid_k = w->K > 4096 && w->K < 8192;
   if (w->bits == 8) {
     if (M >= 5)
-      return blocks >= 160 || long_k;
+      return (blocks >= 160 || long_k) && !a16_decode_rows8_w8(w, M, blocks);
     // K past 4096: from two rows, and at one row where the decode kernel's 16-channel blocks fall badly on the CUs
     // (8192 x 8192 M = 1: 17.4 / 15.7; 5120 x 13824: 20.0 / 17.8; but 28672 x 8192: 48.7 / 49.8)
     return w->K > 4096 && blocks >= 128 && (M >= 2 || (blocks >= 160 && blocks <= 512));

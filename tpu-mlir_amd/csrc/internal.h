@@ -157,6 +157,9 @@ int a16_plain_create(mi_a16_weight *w, const void *weight, int weight_signed, co
 // nothing, when the shape is not its own; the general kernels then take it.
 // the decode kernel's division of a set's K among its waves (a function of the set alone); false: not one it can take
 bool a16_decode_geometry(const mi_a16_weight *w, int *waves, int *tpw, int *gpt, int *group_shift);
+// 8-bit weights, 5 to 8 rows: true where the decode kernel's eight-row form is ahead of the 32-row kernel (blocks32:
+// 32-channel blocks of the whole launch); the 32-row kernel leaves such launches alone
+bool a16_decode_rows8_w8(const mi_a16_weight *w, int64_t M, int64_t blocks32);
 bool a16_decode_launch(const mi_a16_weight *const *ws, int n, const uint16_t *d_x, int64_t M, uint16_t *const *d_ys,
                        float *const *d_y32s, hipStream_t stream);
 // tiled MFMA GEMM for many activation rows (prefill)
