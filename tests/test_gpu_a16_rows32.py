@@ -18,6 +18,7 @@ ROWS32_W4_CASES = [  # (M, K, N, g, dtype)
     (17, 512, 64, 128, "bf16"), (32, 1024, 200, 0, "bf16"), (9, 128, 48, 128, "f16"), (24, 256, 272, 256, "f16"),
     (32, 4096, 1024, 128, "bf16"), (1, 128, 16, 128, "bf16"), (20, 2048, 520, 512, "bf16"), (31, 1536, 136, 64, "f16"),
     (18, 1920, 100, 64, "bf16"), (32, 3200, 40, 128, "bf16"), (25, 1152, 33, 0, "f16"),
+    # (above: 17 to 32 rows -- two 16-row tiles on the 16 x 16 x 32 form, the 32 x 32 x 16 kernel with groups of 64)
     # up to 16 rows (the 16 x 16 x 32 form: activations a tile ahead up to 8 rows, piece by piece above): one tile, a
     # ragged number of tiles per wave, two groups per tile, per-channel scales, channel counts off the 32-block
     (8, 1152, 48, 128, "bf16"), (5, 4096, 72, 128, "f16"), (16, 1920, 100, 64, "bf16"), (12, 2048, 264, 64, "f16"),
