@@ -357,6 +357,32 @@ def test_grouped_launch_through_the_tiled_kernel(orc, bits, M, K, Ns, g):
         w.destroy()
 
 
+@pytest.mark.parametrize("M,g", [(6, 0), (8, 128)])
+def test_grouped_8bit_sets_at_five_to_eight_rows(orc, M, g):
+    """Two 8-bit sibling sets whose 289 32-channel blocks together fall where the decode kernel's eight-row form is
+    taken by the library's own rule (each set alone, 145 and 144 blocks, does not): one grouped launch, every output
+    against the oracle; then each set alone, which takes another kernel, against the oracle as well."""
+    torch = _torch()
+    K, Ns = 2048, (4640, 4608)
+    cfgs = [S.w8a16(M, K, N, g, seed=70 + i, bias=(i == 0)) for i, N in enumerate(Ns)]
+    for c in cfgs:
+        c["x"] = cfgs[0]["x"]
+    x = torch.from_numpy(cfgs[0]["x"].view(np.int16)).cuda().view(torch.bfloat16)
+    ws = [M_.A16Weight(c["weight"], c["scale"], c["zp"], None if c.get("bias") is None else S.bf16_to_f32(c["bias"]),
+                       K=K, N=c["N"], weight_bits=8, q_group_size=c["g"]) for c in cfgs]
+    f32s = [torch.empty((M, c["N"]), dtype=torch.float32, device="cuda") for c in cfgs]
+    ys = M_.a16mm_launch_group(ws, x, ys_f32=f32s)
+    torch.cuda.synchronize()
+    for c, y, f in zip(cfgs, ys, f32s):
+        _check_against_oracle(orc, c, y.view(torch.int16).cpu().numpy().view(np.uint16), f.cpu().numpy())
+    for w, c in zip(ws, cfgs):
+        f1 = torch.empty((M, c["N"]), dtype=torch.float32, device="cuda")
+        y1 = M_.a16mm_launch(w, x, y_f32=f1)
+        torch.cuda.synchronize()
+        _check_against_oracle(orc, c, y1.view(torch.int16).cpu().numpy().view(np.uint16), f1.cpu().numpy())
+        w.destroy()
+
+
 @pytest.mark.parametrize("M,K,N,g,splits,f16", [
     (130, 4096, 512, 128, 0, False),    # two whole chunks of 16 stages
     (100, 4480, 272, 128, 0, False),    # 35 stages: 16 + 16 + 3, ragged N
