@@ -129,7 +129,10 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(const uint8_t *x
   for (int p = 0; p < TPW; ++p) {
     int kt = wave + p * WAVES;
     kt = kt < k_tiles ? kt : k_tiles - 1;  // past the end: a harmless re-load, never multiplied
-    w[p] = *(const u32x4 *)(qw + ((uint32_t)kt * 1024u + lane16));
+    // (non-temporal: every weight byte is read once, by this wave -- decode chain, 4 x 1024 steps, two interleaved
+    // pairs: M = 1 25.85 -> 24.8 us per step, M = 4 31.1 -> 30.0; the same hint on the weight requests of the 16- and
+    // 32-row kernels bought nothing at 8 rows and lost at 16 and more)
+    w[p] = __builtin_nontemporal_load((const u32x4 *)(qw + ((uint32_t)kt * 1024u + lane16)));
   }
   // Everything up to here depends on the preloaded arguments only; what follows reads the argument record.  Keep the
   // two apart, or the wait for the record ends up in front of the requests above: the record's fields are selected by
@@ -150,14 +153,14 @@ __global__ __launch_bounds__(WAVES * 64) void a16_decode_kernel(const uint8_t *x
     uint32_t words[NW];
 #pragma unroll
     for (int j = 0; j + 4 <= NW; j += 4) {
-      const u32x4 t = *(const u32x4 *)(szp + j * 4);
+      const u32x4 t = __builtin_nontemporal_load((const u32x4 *)(szp + j * 4));
       words[j] = t[0];
       words[j + 1] = t[1];
       words[j + 2] = t[2];
       words[j + 3] = t[3];
     }
     if constexpr (NW % 4 == 2) {
-      const u32x2 t = *(const u32x2 *)(szp + (NW - 2) * 4);
+      const u32x2 t = __builtin_nontemporal_load((const u32x2 *)(szp + (NW - 2) * 4));
       words[NW - 2] = t[0];
       words[NW - 1] = t[1];
     }

@@ -20,7 +20,7 @@ __global__ __launch_bounds__(256) void bench_read_kernel(const u32x4 *__restrict
   u32x4 v[CPW];
 #pragma unroll
   for (int u = 0; u < CPW; ++u)
-    v[u] = p[u * 64];
+    v[u] = __builtin_nontemporal_load(p + u * 64);  // as the decode kernel reads its weights: used once
   uint32_t acc = 0;
 #pragma unroll
   for (int u = 0; u < CPW; ++u)
