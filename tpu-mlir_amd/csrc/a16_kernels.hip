@@ -431,7 +431,7 @@ __global__ __launch_bounds__(WAVES * 64) void a16_skinny_kernel(SkinnyArgs a) {
     const uint32_t woff = (uint32_t)kt * 1024u + lane16;
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      t.w[r] = *(const u32x4 *)(wq[r] + woff);
+      t.w[r] = __builtin_nontemporal_load((const u32x4 *)(wq[r] + woff));
 #pragma unroll
     for (int u = 0; u < GPT; ++u) {
       const uint32_t gi = (uint32_t)unit_group(kt, u);
