@@ -28,7 +28,7 @@ from __graft_entry__ import load_package  # noqa: E402
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, AMD's published figure
 INT8_PEAK_TOPS = 5000.0      # dense INT8 MFMA
 BF16_PEAK_TFLOPS = 2500.0    # dense bf16 MFMA
-HBM_TRAFFIC_RATIO = 1.020    # measured HBM bytes / algorithmic bytes of the decode chain (see roofline.traffic_source)
+HBM_TRAFFIC_RATIO = 1.022    # measured HBM bytes / algorithmic bytes of the decode chain (see roofline.traffic_source)
 
 
 def _dev_bf16(torch, bits):
