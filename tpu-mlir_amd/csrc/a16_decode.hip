@@ -436,9 +436,12 @@ static DecodePlan decode_plan(const mi_a16_weight *w, int64_t M, int64_t blocks3
   p.mr = M == 1 ? 1 : M <= 4 ? 4 : 8;
   // eight rows: one request per lane and row only (K up to 4096 at 4 bits), on the 8-wave instances, and only where
   // it was measured ahead of the skinny kernel (us, skinny / this): 4096 x 4096 M = 5: 5.30 / 5.42, M = 8: 5.73 / 5.39;
-  // 11008 x 4096 M = 5: 9.79 / 9.84, M = 8: 11.00 / 9.84; 6144 x 2048 M = 8: 5.60 / 5.83
+  // 11008 x 4096 M = 8: 11.00 / 9.84; 6144 x 2048 M = 8: 5.60 / 5.83; at 5 and 6 rows from 256 32-channel blocks on
+  // (8192 x 4096 M = 5: 7.2 / 6.4, 11008 x 4096: 9.3 / 8.5, 22016 x 4096: 15.9 / 14.7; the table at
+  // a16_rows32_applicable has the 16-row streaming kernel beside them)
   const bool rows8_pays = plan().a16_decode_rows8 ? plan().a16_decode_rows8 > 0
-                                                  : ((w->bits == 4 && M >= 7 && w->K >= 4096) || a16_decode_rows8_w8(w, M, blocks32));
+                                                  : ((w->bits == 4 && w->K >= 4096 && (M >= 7 || (M >= 5 && blocks32 >= 256))) ||
+                                                     a16_decode_rows8_w8(w, M, blocks32));
   p.ok = decode_lds_bytes(w->bits, p.gpt, p.waves, p.tpw, p.mr) <= (p.mr > 4 ? DEC_MAX_LDS8 : DEC_MAX_LDS) &&
          (p.mr <= 4 || (p.waves == 8 && rows8_pays));
   return p;

@@ -714,15 +714,26 @@ bool a16_rows32_applicable(const mi_a16_weight *w, int64_t M, int64_t blocks) {
   //    4096 x 4096  M = 8:  4.8 /  6.1   M = 12: 6.4 /  6.6   M = 14: 6.5 /  6.6   M = 16:  7.0 /  6.7
   //    2048 x 4096  M = 8:  4.2 /  5.3   M = 10: 5.5 /  5.6   M = 12: 5.9 /  5.6   M = 16:  6.5 /  5.6
   //    6144 x 2048, groups of 64   M = 5: 5.1 / 5.1   M = 7: 5.4 / 5.1   M = 8: 5.6 / 5.1   M = 12: 6.2 / 5.4   M = 16: 6.9 / 5.4
+  // With the weights of the decode and skinny kernels requested non-temporally (weights streaming from HBM, 330 MB
+  // of copies in rotation; skinny / eight-row decode / this one):
+  //   16384 x 4096  M = 5: 11.6 / 11.0 / 12.2   M = 7: 12.6 / 11.1 / 11.4      22016 x 4096  M = 5: 15.9 / 14.7 / 15.7   M = 7: 17.2 / 15.0 / 14.9
+  //   11008 x 4096  M = 5:  9.3 /  8.5 /  9.2   M = 8: 10.7 /  8.7 /  9.5       8192 x 4096  M = 5:  7.2 /  6.4 /  6.7   M = 8:  8.3 /  6.7 /  6.7
+  //    6144 x 4096  M = 5:  6.9 /  6.1 /  6.0   M = 8:  7.8 /  6.4 /  6.1      16384 x 2048  M = 5:  7.2 /  8.2 /  7.0   M = 8:  8.3 /  8.2 /  7.1
   if (blocks > 1024)
     return false;
   if (M >= 16 || (M >= 12 && blocks <= 96))
     return true;
   if (M >= 9 && blocks >= 192)
     return true;
-  if (M >= 7)
-    return blocks >= 512 || (blocks >= 192 && w->K <= 2048);
-  return M >= 5 && blocks >= 256;
+  if (M < 5 || M >= 9)
+    return false;
+  if (w->K <= 2048)  // the decode kernel's eight-row form does not pay there
+    return M >= 7 ? blocks >= 192 : blocks >= 256;
+  // 5 to 8 rows, 2048 < K <= 4096: this kernel below one workgroup per CU, the decode kernel's eight-row form from
+  // there on (5 and 6 rows) or up to two per CU (7 and 8 rows)
+  if (blocks >= 160 && blocks < 256)
+    return true;
+  return M >= 7 && blocks >= 512;
 }
 
 // K parts per 32-channel block of a launch of `blocks` blocks over K: doubled while the launch stays within one
