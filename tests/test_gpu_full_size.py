@@ -164,8 +164,8 @@ def test_grouped_sibling_launches_at_full_size(orc, label, K, Ns):
     two row counts in between (from 12 rows on a grouped launch of this size takes the 32-row kernel).  Every set's
     output against the oracle (sampled channels), and -- up to 8 rows -- bit-identical to separate launches, whichever
     of the decode, skinny and 16-row streaming kernels the grouped launch and each single one take (at 5 rows q/k/v
-    grouped takes the streaming kernel and a set alone the skinny one; at 8 rows gate/up grouped the streaming kernel
-    and a set alone the decode kernel): the three deal the K tiles to their waves, fold and sum alike."""
+    grouped takes the decode kernel's eight-row form and a set alone the skinny one; at 8 rows gate/up grouped the
+    streaming kernel and a set alone the decode kernel): the three deal the K tiles to their waves, fold and sum alike."""
     import torch
     g = 128
     cfgs = [S.w4a16(32, K, N, g, seed=60 + i, bias=(i == 1)) for i, N in enumerate(Ns)]
