@@ -919,24 +919,45 @@ __global__ __launch_bounds__(512, 1) void i8_gemm_large_kernel(I8Args a, int til
 // ------------------------------------------------------------------------------------------------
 // Few rows (M <= 32): the product is a stream over the right operand, HBM-bound.  A workgroup owns 32 output
 // columns over the whole K; its eight waves take the 128-byte K tiles round-robin, each multiplies all rows (one
-// 32 x 32 MFMA block; rows past M repeat the last row and are never stored) against its tiles, operands straight from
-// global memory into registers one tile ahead; the eight partial blocks are summed once through LDS.  A lane's 64
-// contiguous bytes of its row of a tile feed four MFMAs, 16 bytes each: the K order inside a tile is permuted the same
-// way for both operands, which a dot product does not see.  Requires K % 128 == 0.
+// 32 x 32 MFMA block; rows past M repeat the last row and are never stored) against its tiles; the eight partial
+// blocks are summed once through LDS.  A lane's 64 bytes of its row of a tile feed four MFMAs, 16 bytes each: the K
+// order inside a tile is permuted the same way for both operands, which a dot product does not see.
+// The right operand -- the stream -- is requested in whole cache lines straight into LDS: eight rows x 128 bytes per
+// request into the wave's own two-tile ring (XOR-swizzled; a wave reads only what it requested, so no barrier), and
+// the MFMA fragments are read back from there.  Asked for as fragments (16 bytes of each of 64 half rows per
+// request) every line was fetched in eight pieces, which the CU's L1 served at a third of this rate.  The left
+// operand (rows past M repeat, so few distinct lines) comes straight into registers, one tile ahead, by loads the
+// compiler does not track; both are waited for by request count.  Requires K % 128 == 0.
 // ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ u32x4 i8_load16_untracked(const void *p) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
 __global__ __launch_bounds__(512) void i8_rows32_kernel(I8Args a) {
   constexpr int WAVES = 8;
-  __shared__ int32_t red[WAVES][16][64];
+  constexpr int RING_BYTES = WAVES * 2 * 4096;  // per wave: two tiles of 32 rows x 128 bytes of the right operand
+  __shared__ __attribute__((aligned(16))) uint8_t smem[RING_BYTES];
+  int32_t (*red)[16][64] = reinterpret_cast<int32_t (*)[16][64]>(smem);  // overlays the rings after the loop
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c32 = lane & 31, h = lane >> 5;
   const int parts = 1 << a.split_shift, part = blockIdx.x & (parts - 1);
   const int64_t block = blockIdx.x >> a.split_shift;
   const int64_t n = block * 32 + c32;
-  const int64_t nb = n < a.N ? n : a.N - 1;  // columns past N repeat the last one; never stored
   const int64_t ma = c32 < a.M ? c32 : a.M - 1;
-  const uint8_t *pb = a.B + nb * a.K + h * 64;
   const uint8_t *pa = a.A + ma * a.K + h * 64;
+  // request q of a tile: rows 8 q + lane / 8 of the block, the lane's 16-byte chunk (lane % 8, swizzled by the row)
+  const uint8_t *pb[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int r = 8 * q + (lane >> 3);
+    int64_t nb = block * 32 + r;
+    nb = nb < a.N ? nb : a.N - 1;  // columns past N repeat the last one; never stored
+    pb[q] = a.B + nb * a.K + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+  }
+  uint8_t *ring = smem + wave * 8192;
+  const uint8_t *bfrag = ring + c32 * 128;
   const uint32_t fa = (uint32_t)a.a_flip * 0x01010101u, fb = (uint32_t)a.b_flip * 0x01010101u;
   const int k_tiles = (int)(a.K / 128);
   // this wave's tiles: first, first + stride, ... (the waves of all K parts of the block take the tiles round-robin)
@@ -947,26 +968,33 @@ __global__ __launch_bounds__(512) void i8_rows32_kernel(I8Args a) {
 #pragma unroll
   for (int r = 0; r < 16; ++r)
     acc[r] = 0;
-  u32x4 xa[2][4], xb[2][4];
-  auto load_tile = [&](int i, int slot) {
+  u32x4 xa[2][4];
+  auto issue_tile = [&](int i, int slot) {  // eight requests: four into LDS, four into registers
     const int64_t off = (int64_t)(first + (i < count ? i : count - 1) * stride) * 128;  // past the end: a re-load
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      xb[slot][j] = *(const u32x4 *)(pb + off + j * 16);
-      xa[slot][j] = *(const u32x4 *)(pa + off + j * 16);
-    }
+    for (int q = 0; q < 4; ++q)
+      __builtin_amdgcn_global_load_lds((gptr_t)(pb[q] + off), (lptr_t)(ring + slot * 4096 + q * 1024), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      xa[slot][j] = i8_load16_untracked(pa + off + j * 16);
   };
   if (count > 0) {
-    load_tile(0, 0);
+    issue_tile(0, 0);
     for (int t0 = 0; t0 < count; t0 += 2) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         if (t0 + u >= count)
           break;
-        load_tile(t0 + u + 1, u ^ 1);
+        issue_tile(t0 + u + 1, u ^ 1);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(8));  // all but the tile just asked for
+        asm volatile("" ::: "memory");              // the tile is in LDS from here on, not before
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          asm volatile("" : "+v"(xa[u][j]));        // ... and in its registers
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          u32x4 va = xa[u][j], vb = xb[u][j];
+          u32x4 va = xa[u][j];
+          u32x4 vb = *(const u32x4 *)(bfrag + u * 4096 + (((4 * h + j) ^ ((c32 >> 1) & 7)) << 4));
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             va[e] ^= fa;
@@ -977,7 +1005,14 @@ __global__ __launch_bounds__(512) void i8_rows32_kernel(I8Args a) {
         }
       }
     }
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // the re-loads issued past the end
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        asm volatile("" : "+v"(xa[u][j]));  // their registers stay taken until here
   }
+  __syncthreads();  // the partial blocks overlay the rings: every wave is done with its tiles
   // cross-wave sum, in wave order.  Register r of lane l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
 #pragma unroll
   for (int r = 0; r < 16; ++r)
