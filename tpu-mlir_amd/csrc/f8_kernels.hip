@@ -616,25 +616,43 @@ __global__ __launch_bounds__(256, 1) void f8_gemm_large_kernel(F8Args a, int til
 // ------------------------------------------------------------------------------------------------
 // Few rows (M <= 32): a stream over the right operand, HBM-bound; the INT8 few-row kernel (i8_kernels.hip) on F8
 // codes.  A workgroup owns 32 output columns, its eight waves take the 128-byte K tiles round-robin (with the waves of
-// the block's other K parts, when K is split over workgroups), each multiplies all rows against its tiles, operands
-// straight from memory into MFMA fragments one tile ahead (a lane's 64 contiguous bytes of its row feed two K = 64
-// MFMAs; the K order inside a tile is permuted alike for both operands).  Partial sums are added in wave order, then in
-// part order: fp32 sums in another order than the tiled kernels', inside the same bound.  Requires K % 128 == 0.
+// the block's other K parts, when K is split over workgroups), each multiplies all rows against its tiles (a lane's 64
+// bytes of its row feed two K = 64 MFMAs; the K order inside a tile is permuted alike for both operands).  As there,
+// the right operand comes in whole cache lines through the wave's own two-tile LDS ring and the left one straight into
+// registers by untracked loads, one tile ahead, both waited for by request count.  Partial sums are added in wave
+// order, then in part order: fp32 sums in another order than the tiled kernels', inside the same bound.  Requires
+// K % 128 == 0.
 // ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ u32x4 f8_load16_untracked(const void *p) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
 template <int FMT>
 __global__ __launch_bounds__(512) void f8_rows32_kernel(F8Args a) {
   constexpr int WAVES = 8;
-  __shared__ float red[WAVES][16][64];
+  constexpr int RING_BYTES = WAVES * 2 * 4096;  // per wave: two tiles of 32 rows x 128 bytes of the right operand
+  __shared__ __attribute__((aligned(16))) uint8_t smem[RING_BYTES];
+  float (*red)[16][64] = reinterpret_cast<float (*)[16][64]>(smem);  // overlays the rings after the loop
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c32 = lane & 31, h = lane >> 5;
   const int parts = 1 << a.split_shift, part = blockIdx.x & (parts - 1);
   const int64_t block = blockIdx.x >> a.split_shift;
   const int64_t n = block * 32 + c32;
-  const int64_t nb = n < a.N ? n : a.N - 1;  // columns past N repeat the last one; never stored
   const int64_t ma = c32 < a.M ? c32 : a.M - 1;
-  const uint8_t *pb = a.B + nb * a.K + h * 64;
   const uint8_t *pa = a.A + ma * a.K + h * 64;
+  // request q of a tile: rows 8 q + lane / 8 of the block, the lane's 16-byte chunk (lane % 8, swizzled by the row)
+  const uint8_t *pb[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int r = 8 * q + (lane >> 3);
+    int64_t nb = block * 32 + r;
+    nb = nb < a.N ? nb : a.N - 1;  // columns past N repeat the last one; never stored
+    pb[q] = a.B + nb * a.K + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+  }
+  uint8_t *ring = smem + wave * 8192;
+  const uint8_t *bfrag = ring + c32 * 128;
   const int k_tiles = (int)(a.K / 128);
   const int first = part * WAVES + wave, stride = WAVES << a.split_shift;
   const int count = (k_tiles - first + stride - 1) / stride;
@@ -643,33 +661,48 @@ __global__ __launch_bounds__(512) void f8_rows32_kernel(F8Args a) {
 #pragma unroll
   for (int r = 0; r < 16; ++r)
     acc[r] = 0.0f;
-  u32x4 xa[2][4], xb[2][4];
-  auto load_tile = [&](int i, int slot) {
+  u32x4 xa[2][4];
+  auto issue_tile = [&](int i, int slot) {  // eight requests: four into LDS, four into registers
     const int64_t off = (int64_t)(first + (i < count ? i : count - 1) * stride) * 128;  // past the end: a re-load
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      xb[slot][j] = *(const u32x4 *)(pb + off + j * 16);
-      xa[slot][j] = *(const u32x4 *)(pa + off + j * 16);
-    }
+    for (int q = 0; q < 4; ++q)
+      __builtin_amdgcn_global_load_lds((f8_gptr_t)(pb[q] + off), (f8_lptr_t)(ring + slot * 4096 + q * 1024), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      xa[slot][j] = f8_load16_untracked(pa + off + j * 16);
   };
   if (count > 0) {
-    load_tile(0, 0);
+    issue_tile(0, 0);
     for (int t0 = 0; t0 < count; t0 += 2) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         if (t0 + u >= count)
           break;
-        load_tile(t0 + u + 1, u ^ 1);
+        issue_tile(t0 + u + 1, u ^ 1);
+        __builtin_amdgcn_s_waitcnt(f8_waitcnt_vm(8));  // all but the tile just asked for
+        asm volatile("" ::: "memory");                 // the tile is in LDS from here on, not before
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          asm volatile("" : "+v"(xa[u][j]));           // ... and in its registers
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-          const u32x4 a0 = xa[u][2 * j], a1 = xa[u][2 * j + 1], b0 = xb[u][2 * j], b1 = xb[u][2 * j + 1];
+          const u32x4 a0 = xa[u][2 * j], a1 = xa[u][2 * j + 1];
+          const u32x4 b0 = *(const u32x4 *)(bfrag + u * 4096 + (((4 * h + 2 * j) ^ ((c32 >> 1) & 7)) << 4));
+          const u32x4 b1 = *(const u32x4 *)(bfrag + u * 4096 + (((4 * h + 2 * j + 1) ^ ((c32 >> 1) & 7)) << 4));
           const i32x8 fa = {(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
           const i32x8 fb = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
           acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa, fb, acc, FMT, FMT, 0, 0, 0, 0);
         }
       }
     }
+    __builtin_amdgcn_s_waitcnt(f8_waitcnt_vm(0));  // the re-loads issued past the end
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        asm volatile("" : "+v"(xa[u][j]));  // their registers stay taken until here
   }
+  __syncthreads();  // the partial blocks overlay the rings: every wave is done with its tiles
   // cross-wave sum, in wave order.  Register r of lane l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
 #pragma unroll
   for (int r = 0; r < 16; ++r)
